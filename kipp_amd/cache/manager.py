@@ -1,0 +1,239 @@
+"""The cache manager: pages of keys and values for every request, per group of
+layers, and slots of fixed-size state.
+
+Runs of the layer order with the same need (heads, head size, window) form a
+group; a group has its own pool of pages, its own block table for every
+request, and one key and one value tensor for each of its runs, laid out
+[page][kv head][slot in page][head_dim].  A group with a window gives pages
+back as soon as the window has passed them; every group gives all pages back
+when the request ends.  Mixers that keep state of fixed size get a slot per
+request instead: a row of a tensor [slots, ...], zeroed when claimed.
+
+A step is transactional (/root/reference/src/kipp.c:3616-3635, 4043-4072): `reserve`
+claims the pages of every entry of the step or none.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Sequence, Tuple
+
+from .needs import KVNeed, StateNeed
+from .pool import PagePool
+
+
+class OutOfPages(RuntimeError):
+    """A step needs more pages than are free; nothing was changed."""
+
+
+class OutOfSlots(RuntimeError):
+    """Every request slot is taken."""
+
+
+@dataclass
+class KVCacheView:
+    """What a mixer sees of the cache in one run."""
+    group: int
+    k: object
+    v: object
+    page_size: int
+    writable: bool = True
+
+
+@dataclass
+class RequestCache:
+    id: object
+    slot: int
+    length: int = 0
+    tokens: List[int] = field(default_factory=list)
+    tables: List[List[int]] = field(default_factory=list)   # per group: page id per block, -1 once given back
+    adopted: List[int] = field(default_factory=list)        # per group: leading pages taken from the index
+    adopted_tokens: int = 0
+
+
+class CacheGroup:
+    def __init__(self, index: int, need: KVNeed, runs: List[int], num_pages: int, page_size: int):
+        self.index = index
+        self.need = need
+        self.runs = runs
+        self.page_size = page_size
+        self.pool = PagePool(num_pages, page_size)
+        self.k: Dict[int, object] = {}
+        self.v: Dict[int, object] = {}
+
+    def bytes_per_token(self, element_size: int) -> int:
+        return 2 * len(self.runs) * self.need.num_kv_heads * self.need.head_dim * element_size
+
+
+class CacheManager:
+    def __init__(self, kv_needs: Sequence[Optional[KVNeed]], state_needs: Sequence[Optional[StateNeed]],
+                 page_size: int, num_pages: int, max_requests: int, max_position: int,
+                 runtime=None, share_prefixes: bool = True):
+        """`kv_needs[r]` / `state_needs[r]`: what run r of the layer order keeps
+        (None: nothing).  `num_pages` is the size of every group's pool.  With
+        `runtime` None no device memory is made (bookkeeping only)."""
+        self.page_size = page_size
+        self.max_requests = max_requests
+        self.max_position = max_position
+        self.max_blocks = (max_position + page_size - 1) // page_size
+        self.rt = runtime
+        self.groups: List[CacheGroup] = []
+        self.run_group: Dict[int, Tuple[int, int]] = {}
+        by_need: Dict[KVNeed, CacheGroup] = {}
+        for run, need in enumerate(kv_needs):
+            if need is None:
+                continue
+            group = by_need.get(need)
+            if group is None:
+                group = CacheGroup(len(self.groups), need, [], num_pages, page_size)
+                by_need[need] = group
+                self.groups.append(group)
+            group.runs.append(run)
+        self.state_needs = {r: n for r, n in enumerate(state_needs) if n is not None}
+        self.states: Dict[int, object] = {}
+        # content sharing needs every token of the prefix to be in pages that are kept
+        self.share = share_prefixes and not self.state_needs and all(g.need.window is None for g in self.groups)
+        self.free_slots = list(range(max_requests - 1, -1, -1))
+        self.requests: Dict[object, RequestCache] = {}
+        if runtime is not None:
+            self._allocate_device()
+
+    # -- device memory -----------------------------------------------------------
+    def _allocate_device(self) -> None:
+        import torch
+        rt = self.rt
+        for g in self.groups:
+            shape = (g.pool.num_pages, g.need.num_kv_heads, self.page_size, g.need.head_dim)
+            for run in g.runs:
+                # zeroed: masked slots must hold finite values
+                g.k[run] = torch.zeros(shape, dtype=rt.cache_dtype, device=rt.device)
+                g.v[run] = torch.zeros(shape, dtype=rt.cache_dtype, device=rt.device)
+        for run, need in self.state_needs.items():
+            dtype = {"float32": torch.float32, "bfloat16": torch.bfloat16}[need.dtype]
+            self.states[run] = torch.zeros((self.max_requests,) + tuple(need.shape), dtype=dtype, device=rt.device)
+
+    def view(self, run: int, reads_run: Optional[int] = None) -> Optional[KVCacheView]:
+        """The cache of `run`, or of `reads_run` read-only."""
+        src = run if reads_run is None else reads_run
+        for g in self.groups:
+            if src in g.runs:
+                return KVCacheView(g.index, g.k.get(src), g.v.get(src), self.page_size, writable=reads_run is None)
+        return None
+
+    def state(self, run: int):
+        return self.states.get(run)
+
+    # -- requests ------------------------------------------------------------------
+    def open(self, request_id, prompt: Optional[Sequence[int]] = None) -> RequestCache:
+        """Claim a slot (its state zeroed) and, where sharing is on and `prompt`
+        is given, adopt the pages of its longest known beginning."""
+        if request_id in self.requests:
+            raise ValueError(f"request {request_id!r} is already open")
+        if not self.free_slots:
+            raise OutOfSlots(f"all {self.max_requests} request slots are taken")
+        slot = self.free_slots.pop()
+        for tensor in self.states.values():
+            tensor[slot].zero_()
+        req = RequestCache(request_id, slot, tables=[[] for _ in self.groups], adopted=[0 for _ in self.groups])
+        if self.share and prompt is not None and self.groups:
+            matches = [g.pool.prefix_match(prompt) for g in self.groups]
+            keep = min(len(pages) for pages, _ in matches)
+            for g, (pages, _) in zip(self.groups, matches):
+                for page in pages[keep:]:
+                    g.pool.release(page)
+                req.tables[g.index] = list(pages[:keep])
+                req.adopted[g.index] = keep
+            req.adopted_tokens = keep * self.page_size
+            req.length = req.adopted_tokens
+            req.tokens = [int(t) for t in prompt[:req.length]]
+        self.requests[request_id] = req
+        return req
+
+    def pages_needed(self, req: RequestCache, new_length: int) -> List[int]:
+        """Pages each group still has to claim so that positions < new_length have one."""
+        blocks = (new_length + self.page_size - 1) // self.page_size
+        return [max(0, blocks - len(req.tables[g.index])) for g in self.groups]
+
+    def free_pages(self) -> List[int]:
+        return [g.pool.free_count for g in self.groups]
+
+    def reserve(self, entries: Sequence[Tuple[RequestCache, int]]) -> None:
+        """Claim the pages that every (request, number of new tokens) of a step
+        needs, in every group; all or nothing."""
+        claimed: List[Tuple[RequestCache, int, int]] = []
+        for req, n_new in entries:
+            new_length = req.length + n_new
+            if n_new <= 0:
+                self._rollback(claimed)
+                raise ValueError("a step entry needs at least one token")
+            if new_length > self.max_position:
+                self._rollback(claimed)
+                raise ValueError(f"request {req.id!r}: {new_length} tokens exceed the model's {self.max_position} positions")
+            for g, need in zip(self.groups, self.pages_needed(req, new_length)):
+                for _ in range(need):
+                    page = g.pool.alloc()
+                    if page is None:
+                        self._rollback(claimed)
+                        raise OutOfPages(f"group {g.index}: no free page for request {req.id!r}")
+                    req.tables[g.index].append(page)
+                    claimed.append((req, g.index, page))
+
+    def _rollback(self, claimed) -> None:
+        for req, gi, page in reversed(claimed):
+            popped = req.tables[gi].pop()
+            assert popped == page
+            self.groups[gi].pool.release(page)
+
+    def commit(self, req: RequestCache, tokens: Sequence[int]) -> None:
+        """The step ran: the request now holds `tokens` more.  Pages that a
+        window has passed are given back."""
+        req.tokens.extend(int(t) for t in tokens)
+        req.length += len(tokens)
+        for g in self.groups:
+            window = g.need.window
+            if window is None:
+                continue
+            first_needed = max(0, req.length - window + 1)
+            table = req.tables[g.index]
+            for block in range(min(first_needed // self.page_size, len(table))):
+                if table[block] >= 0:
+                    g.pool.release(table[block])
+                    table[block] = -1
+
+    def close(self, request_id) -> None:
+        """The request ended: publish its full pages where sharing is on, give
+        every page and the slot back."""
+        req = self.requests.pop(request_id)
+        for g in self.groups:
+            table = req.tables[g.index]
+            if self.share:
+                parent = 0
+                for block in range(req.length // self.page_size):
+                    chunk = req.tokens[block * self.page_size:(block + 1) * self.page_size]
+                    if block < req.adopted[g.index] or g.pool.content[table[block]] is not None:
+                        parent = g.pool._hash(parent, chunk)
+                    else:
+                        parent = g.pool.seal(table[block], parent, chunk)
+            for page in table:
+                if page >= 0:
+                    g.pool.release(page)
+            table.clear()
+        self.free_slots.append(req.slot)
+
+    def check(self) -> None:
+        """Invariants over pools and tables: a held page is held exactly as often
+        as tables name it; nothing is lost."""
+        for g in self.groups:
+            g.pool.check()
+            counts = [0] * g.pool.num_pages
+            for req in self.requests.values():
+                for page in req.tables[g.index]:
+                    if page >= 0:
+                        counts[page] += 1
+            for page in range(g.pool.num_pages):
+                if counts[page] != g.pool.ref[page]:
+                    raise AssertionError(f"group {g.index} page {page}: named {counts[page]} times, held {g.pool.ref[page]} times")
+        slots = [r.slot for r in self.requests.values()]
+        if len(set(slots)) != len(slots) or set(slots) & set(self.free_slots):
+            raise AssertionError("a slot is held twice or both held and free")
+        if len(slots) + len(self.free_slots) != self.max_requests:
+            raise AssertionError("a slot was lost")

@@ -1,0 +1,223 @@
+"""Python bindings of the HIP kernels: shape and type checks on the host, then
+one launch on torch's current stream.  Every function fails loudly when its
+library cannot be built or loaded, or when there is no GPU; there is no CPU
+path behind any of them.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from . import build
+
+F32, BF16 = 0, 1
+_CODE = {torch.float32: F32, torch.bfloat16: BF16}
+
+_c_int, _c_float, _c_size, _c_ptr = ctypes.c_int, ctypes.c_float, ctypes.c_size_t, ctypes.c_void_p
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _code(t: torch.Tensor) -> int:
+    try:
+        return _CODE[t.dtype]
+    except KeyError:
+        raise KernelError(f"kernels take float32 or bfloat16 tensors, got {t.dtype}") from None
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return _c_ptr(t.data_ptr()) if t is not None else _c_ptr(0)
+
+
+def _stream():
+    return _c_ptr(torch.cuda.current_stream().cuda_stream)
+
+
+def _need(cond: bool, msg: str) -> None:
+    if not cond:
+        raise KernelError(msg)
+
+
+def _dev(*tensors: Optional[torch.Tensor]) -> None:
+    for t in tensors:
+        if t is None:
+            continue
+        _need(t.is_cuda, "kernel operand is not on the GPU (there is no CPU path)")
+        _need(t.is_contiguous(), "kernel operand is not contiguous")
+
+
+def _i32(t: torch.Tensor, name: str) -> None:
+    _need(t.dtype == torch.int32, f"{name} must be int32, got {t.dtype}")
+
+
+_sigs_set = set()
+
+
+def _fn(lib_name: str, fn_name: str, argtypes, defines=None):
+    lib = build.library(lib_name, defines)
+    fn = getattr(lib, fn_name)
+    key = (lib._name, fn_name)
+    if key not in _sigs_set:
+        fn.argtypes = argtypes
+        fn.restype = _c_int
+        _sigs_set.add(key)
+    return fn
+
+
+def _check(rc: int, what: str) -> None:
+    if rc != 0:
+        raise KernelError(f"{what}: launch failed or arguments refused (code {rc})")
+
+
+# --------------------------------------------------------------------------- elementwise
+
+def embed(table: torch.Tensor, tokens: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    _dev(table, tokens, out)
+    _i32(tokens, "tokens")
+    n, hidden = out.shape
+    _need(table.dim() == 2 and table.shape[1] == hidden, "embed: table width differs from output width")
+    _need(tokens.numel() == n and out.dtype == torch.float32, "embed: one float32 output row per token")
+    fn = _fn("elementwise", "kipp_embed", [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr])
+    _check(fn(_ptr(table), _code(table), _ptr(tokens), _ptr(out), n, hidden, _stream()), "embed")
+    return out
+
+
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor,
+            delta: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out = rmsnorm(x [+ delta]) * weight; with `delta`, x += delta in place."""
+    _dev(x, weight, out, delta)
+    rows, width = x.shape
+    _need(x.dtype == torch.float32 and weight.dtype == torch.float32, "rmsnorm: x and weight are float32")
+    _need(weight.numel() == width and out.shape == x.shape, "rmsnorm: shapes differ")
+    if delta is not None:
+        _need(delta.shape == x.shape, "rmsnorm: delta shape differs from x")
+    fn = _fn("elementwise", "kipp_rmsnorm",
+             [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_float, _c_ptr])
+    _check(fn(_ptr(x), _ptr(delta), _code(delta) if delta is not None else F32, _ptr(weight), _ptr(out),
+              _code(out), rows, width, float(eps), _stream()), "rmsnorm")
+    return out
+
+
+def residual_add(x: torch.Tensor, delta: torch.Tensor) -> torch.Tensor:
+    _dev(x, delta)
+    _need(x.dtype == torch.float32 and x.shape == delta.shape, "residual_add: float32 x and a delta of its shape")
+    fn = _fn("elementwise", "kipp_residual_add", [_c_ptr, _c_ptr, _c_int, _c_size, _c_ptr])
+    _check(fn(_ptr(x), _ptr(delta), _code(delta), x.numel(), _stream()), "residual_add")
+    return x
+
+
+def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[t, i] = silu(gate_up[t, i]) * gate_up[t, inner + i]."""
+    _dev(gate_up, out)
+    rows, inner = out.shape
+    _need(gate_up.shape == (rows, 2 * inner), "swiglu: input must be [rows, 2 * inner]")
+    fn = _fn("elementwise", "kipp_swiglu", [_c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_int, _c_ptr])
+    _check(fn(_ptr(gate_up), _code(gate_up), _ptr(out), _code(out), rows, inner, _stream()), "swiglu")
+    return out
+
+
+def cast(src: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    _dev(src, out)
+    _need(src.numel() == out.numel(), "cast: sizes differ")
+    fn = _fn("elementwise", "kipp_cast", [_c_ptr, _c_int, _c_ptr, _c_int, _c_size, _c_ptr])
+    _check(fn(_ptr(src), _code(src), _ptr(out), _code(out), src.numel(), _stream()), "cast")
+    return out
+
+
+def gather_rows(x: torch.Tensor, index: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    _dev(x, index, out)
+    _i32(index, "index")
+    _need(x.dtype == torch.float32 and out.dtype == torch.float32, "gather_rows: float32 rows")
+    _need(out.shape == (index.numel(), x.shape[1]), "gather_rows: output shape")
+    fn = _fn("elementwise", "kipp_gather_rows", [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr])
+    _check(fn(_ptr(x), _ptr(index), _ptr(out), index.numel(), x.shape[1], _stream()), "gather_rows")
+    return out
+
+
+# --------------------------------------------------------------------------- attention
+
+def qk_norm_rope_kv_write(qkv: torch.Tensor, q_out: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                          positions: torch.Tensor, seq_of_token: torch.Tensor, block_table: torch.Tensor,
+                          n_q: int, n_kv: int, head_dim: int,
+                          q_norm_w: Optional[torch.Tensor], k_norm_w: Optional[torch.Tensor], eps: float,
+                          inv_freq: Optional[torch.Tensor], rotary_dim: int, write_kv: bool = True) -> torch.Tensor:
+    """Per-head norm of q and k, rotation at each token's position, q to `q_out`
+    and k, v into their pages.  Caches are [pages, n_kv, page, head_dim]."""
+    _dev(qkv, q_out, k_cache, v_cache, positions, seq_of_token, block_table, q_norm_w, k_norm_w, inv_freq)
+    for t, name in ((positions, "positions"), (seq_of_token, "seq_of_token"), (block_table, "block_table")):
+        _i32(t, name)
+    n = qkv.shape[0]
+    _need(qkv.shape == (n, (n_q + 2 * n_kv) * head_dim), "qk_norm_rope: qkv must be [tokens, (n_q + 2 n_kv) d]")
+    _need(q_out.shape == (n, n_q * head_dim), "qk_norm_rope: q_out must be [tokens, n_q d]")
+    _need(k_cache.shape == v_cache.shape and k_cache.dim() == 4 and k_cache.shape[1] == n_kv
+          and k_cache.shape[3] == head_dim and k_cache.dtype == v_cache.dtype,
+          "qk_norm_rope: caches must be [pages, n_kv, page, d] of one type")
+    _need(positions.numel() == n and seq_of_token.numel() == n, "qk_norm_rope: one position and sequence per token")
+    _need(block_table.dim() == 2, "qk_norm_rope: block_table is [sequences, blocks]")
+    for w in (q_norm_w, k_norm_w):
+        if w is not None:
+            _need(w.dtype == torch.float32 and w.numel() == head_dim, "qk_norm_rope: norm weight is float32 [d]")
+    if inv_freq is not None:
+        _need(inv_freq.dtype == torch.float32 and inv_freq.numel() == rotary_dim // 2 and rotary_dim % 2 == 0
+              and 0 < rotary_dim <= head_dim, "qk_norm_rope: inv_freq is float32 [rotary_dim / 2]")
+    fn = _fn("rope_kv", "kipp_qk_norm_rope_kv",
+             [_c_ptr, _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int,
+              _c_ptr, _c_ptr, _c_float, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr])
+    _check(fn(_ptr(qkv), _code(qkv), _ptr(q_out), _code(q_out), _ptr(k_cache), _ptr(v_cache), _code(k_cache),
+              _ptr(positions), _ptr(seq_of_token), _ptr(block_table), block_table.shape[1],
+              _ptr(q_norm_w), _ptr(k_norm_w), float(eps), _ptr(inv_freq), int(rotary_dim),
+              n, n_q, n_kv, head_dim, k_cache.shape[2], 1 if write_kv else 0, _stream()), "qk_norm_rope_kv_write")
+    return q_out
+
+
+def paged_attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
+                            positions: torch.Tensor, seq_of_token: torch.Tensor, block_table: torch.Tensor,
+                            n_q: int, n_kv: int, head_dim: int, scale: float, window: int = 0) -> torch.Tensor:
+    _dev(q, k_cache, v_cache, out, positions, seq_of_token, block_table)
+    for t, name in ((positions, "positions"), (seq_of_token, "seq_of_token"), (block_table, "block_table")):
+        _i32(t, name)
+    n = q.shape[0]
+    _need(q.shape == (n, n_q * head_dim) and out.shape == q.shape, "attention: q and out are [tokens, n_q d]")
+    _need(k_cache.shape == v_cache.shape and k_cache.dim() == 4 and k_cache.shape[1] == n_kv
+          and k_cache.shape[3] == head_dim and k_cache.dtype == v_cache.dtype,
+          "attention: caches must be [pages, n_kv, page, d] of one type")
+    _need(positions.numel() == n and seq_of_token.numel() == n and block_table.dim() == 2,
+          "attention: one position and sequence per token, block_table [sequences, blocks]")
+    fn = _fn("attention_generic", "kipp_paged_attention_generic",
+             [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int,
+              _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_ptr])
+    _check(fn(_ptr(q), _code(q), _ptr(k_cache), _ptr(v_cache), _code(k_cache), _ptr(out), _code(out),
+              _ptr(positions), _ptr(seq_of_token), _ptr(block_table), block_table.shape[1],
+              n, n_q, n_kv, head_dim, k_cache.shape[2], float(scale), int(window), _stream()),
+           "paged_attention_generic")
+    return out
+
+
+# --------------------------------------------------------------------------- matrix products
+
+def gemm_f32(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[M,N] = x[M,K] . w[N,K]^T in true float32 (w float32 or bfloat16)."""
+    _dev(x, w, out)
+    _need(x.dtype == torch.float32 and out.dtype == torch.float32, "gemm_f32: x and out are float32")
+    m, k = x.shape
+    n = w.shape[0]
+    _need(w.shape == (n, k) and out.shape == (m, n), "gemm_f32: shapes do not match [M,K] x [N,K] -> [M,N]")
+    fn = _fn("gemm_f32", "kipp_gemm_f32", [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_int, _c_ptr])
+    _check(fn(_ptr(x), _ptr(w), _code(w), _ptr(out), m, n, k, _stream()), "gemm_f32")
+    return out
+
+
+# --------------------------------------------------------------------------- sampling
+
+def argmax(logits: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    _dev(logits, out)
+    _i32(out, "argmax output")
+    _need(logits.dtype == torch.float32 and logits.dim() == 2 and out.numel() == logits.shape[0],
+          "argmax: float32 [rows, vocab] and one int32 per row")
+    fn = _fn("sampling", "kipp_argmax", [_c_ptr, _c_ptr, _c_int, _c_int, _c_ptr])
+    _check(fn(_ptr(logits), _ptr(out), logits.shape[0], logits.shape[1], _stream()), "argmax")
+    return out

@@ -1,0 +1,84 @@
+"""The engine: a model, its cache manager, and ONE step function.
+
+`step(entries)` runs exactly the tokens it is given, as one batch, from the
+cache that earlier steps left: portions of prompts beside single decoded
+tokens, cut anywhere.  It returns the float32 logits at the wanted places in
+the order of the entries and of their `want` lists
+(/root/reference/src/kipp.c:3984-4082 is the reference's batched call; there
+one row per item, here any places).
+"""
+from __future__ import annotations
+
+from typing import List, Optional, Sequence
+
+import torch
+
+from ..cache import CacheManager, OutOfPages
+from ..runtime import Runtime
+from .batch import StepEntry, build_batch
+from .model import Model, load_model
+
+
+class Engine:
+    def __init__(self, model: Model, page_size: int = 16, num_pages: Optional[int] = None,
+                 max_tokens: Optional[int] = None, max_requests: int = 64, share_prefixes: bool = True):
+        """The pool of every cache group has `num_pages` pages, or as many as
+        hold `max_tokens` tokens."""
+        if num_pages is None:
+            if max_tokens is None:
+                raise ValueError("give num_pages or max_tokens")
+            num_pages = (max_tokens + page_size - 1) // page_size
+        self.model = model
+        self.rt: Runtime = model.rt
+        self.vocab_size = model.spec.vocab_size
+        self.cache = CacheManager(model.kv_needs(), model.state_needs(), page_size, num_pages, max_requests,
+                                  model.spec.max_position, runtime=self.rt, share_prefixes=share_prefixes)
+
+    @classmethod
+    def from_folder(cls, model_dir: str, dtype: str = "bfloat16", device: str = "cuda:0", **kw) -> "Engine":
+        return cls(load_model(model_dir, Runtime(dtype, device)), **kw)
+
+    # -- requests ---------------------------------------------------------------------
+    def open(self, request_id, prompt: Optional[Sequence[int]] = None):
+        return self.cache.open(request_id, prompt)
+
+    def close(self, request_id) -> None:
+        self.cache.close(request_id)
+
+    def length(self, request_id) -> int:
+        return self.cache.requests[request_id].length
+
+    # -- the step ---------------------------------------------------------------------
+    def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+        """Run one batch.  Requests not yet open are opened.  Raises OutOfPages
+        (nothing changed) when the pools cannot hold the step."""
+        if not entries:
+            return None
+        seen = set()
+        requests = []
+        for e in entries:
+            if e.request in seen:
+                raise ValueError(f"request {e.request!r} appears twice in one step")
+            seen.add(e.request)
+            if len(e.tokens) == 0:
+                raise ValueError(f"request {e.request!r}: an entry needs at least one token")
+            for t in e.tokens:
+                if not 0 <= int(t) < self.vocab_size:
+                    raise ValueError(f"request {e.request!r}: token {t} is outside the vocabulary of {self.vocab_size}")
+        opened = []
+        try:
+            for e in entries:
+                if e.request not in self.cache.requests:
+                    self.cache.open(e.request)
+                    opened.append(e.request)
+                requests.append(self.cache.requests[e.request])
+            self.cache.reserve([(r, len(e.tokens)) for r, e in zip(requests, entries)])
+        except Exception:
+            for rid in opened:
+                self.cache.close(rid)
+            raise
+        batch = build_batch(entries, requests, len(self.cache.groups), self.rt.device)
+        logits = self.model.forward(batch, self.cache)
+        for r, e in zip(requests, entries):
+            self.cache.commit(r, e.tokens)
+        return logits

@@ -1,0 +1,35 @@
+"""Block arrangements: how the parts of one layer are put together.
+
+Interface of a block:
+
+    roles: tuple of (role, category) the arrangement needs in LayerSpec.parts
+    forward(x, pending, batch, cache, state) -> (x, pending)
+        x        float32 [tokens, hidden], the residual stream (updated in place)
+        pending  a delta not yet added to x (or None); the block adds it inside
+                 its first norm and hands its own last delta on the same way,
+                 so that residual add and norm are one kernel
+"""
+from __future__ import annotations
+
+from .base import build_part, register
+
+
+@register("block", "pre_norm")
+class PreNormBlock:
+    """x += mixer(mixer_norm(x)); x += ffn(ffn_norm(x))
+    (/root/reference/docs/ARCHITECTURE.md:77-92)."""
+
+    roles = (("mixer_norm", "norm"), ("mixer", "mixer"), ("ffn_norm", "norm"), ("ffn", "feed_forward"))
+
+    def __init__(self, layer_spec, runtime):
+        self.rt = runtime
+        self.parts = {role: build_part(cat, layer_spec.part(role), runtime) for role, cat in self.roles}
+        self.mixer = self.parts["mixer"]
+
+    def forward(self, x, pending, batch, cache, state):
+        act = self.rt.act_dtype
+        norm1, norm2 = self.parts["mixer_norm"], self.parts["ffn_norm"]
+        h = norm1.forward(x, act) if pending is None else norm1.add_forward(x, pending, act)
+        delta = self.mixer.forward(h, batch, cache, state)
+        h = norm2.add_forward(x, delta, act)
+        return x, self.parts["ffn"].forward(h, batch)

@@ -1,0 +1,42 @@
+"""Feed-forward parts.  Interface:
+
+    params(spec) -> {local name: ParamSpec}
+    load(tensors)
+    forward(x, batch) -> delta      x [tokens, hidden] activation type,
+                                    delta float32 [tokens, hidden]
+"""
+from __future__ import annotations
+
+from .base import ParamSpec, register
+
+
+@register("feed_forward", "gated_mlp")
+class GatedMLP:
+    """delta = W_down (silu(W_gate x) * (W_up x))  (/root/reference/src/kipp.c:2633-2653)."""
+
+    def __init__(self, spec, runtime):
+        self.spec = spec
+        self.rt = runtime
+        self.w_gate_up = self.w_down = None
+
+    @staticmethod
+    def params(spec):
+        return {
+            "gate_proj.weight": ParamSpec((spec.intermediate_size, spec.hidden_size)),
+            "up_proj.weight": ParamSpec((spec.intermediate_size, spec.hidden_size)),
+            "down_proj.weight": ParamSpec((spec.hidden_size, spec.intermediate_size)),
+        }
+
+    def load(self, tensors):
+        import torch
+        g, u = tensors["gate_proj.weight"], tensors["up_proj.weight"]
+        if g.dtype != u.dtype:
+            g, u = g.float(), u.float()
+        self.w_gate_up = torch.cat([g, u], dim=0).contiguous()
+        self.w_down = tensors["down_proj.weight"]
+
+    def forward(self, x, batch=None):
+        rt = self.rt
+        gate_up = rt.linear(x, self.w_gate_up)
+        act = rt.ops.swiglu(gate_up, rt.empty((x.shape[0], self.spec.intermediate_size), rt.act_dtype))
+        return rt.linear(act, self.w_down)

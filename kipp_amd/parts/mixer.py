@@ -1,0 +1,87 @@
+"""Token mixers.  Interface of a mixer:
+
+    params(spec) -> {local name: ParamSpec}
+    load(tensors)
+    cache_need() -> KVNeed or None      what it keeps per token, in pages
+    state_need() -> StateNeed or None   what it keeps per request, of fixed size
+    forward(x, batch, cache, state) -> delta
+        x      [tokens, hidden] in the activation type (the normed residual)
+        batch  the step's StepBatch (positions, sequence of each token, tables)
+        cache  the KVCacheView of this run (None if cache_need() is None)
+        state  tensor [slots, ...] of this run (None if state_need() is None)
+        delta  float32 [tokens, hidden], added to the residual by the block
+"""
+from __future__ import annotations
+
+import math
+
+from ..cache.needs import KVNeed
+from .base import ParamSpec, build_part, register
+
+
+@register("mixer", "attention")
+class Attention:
+    """Causal grouped-query attention with optional per-head q/k RMSNorm, a
+    rotary position part and an optional window, over the paged cache
+    (/root/reference/src/kipp.c:2950-2993).  Query head h reads key/value head
+    h // (n_q / n_kv)."""
+
+    def __init__(self, spec, runtime):
+        self.spec = spec
+        self.rt = runtime
+        self.position = build_part("position", spec.position, runtime)
+        self.scale = spec.scale if spec.scale is not None else 1.0 / math.sqrt(spec.head_dim)
+        self.w_qkv = self.w_o = self.q_norm = self.k_norm = None
+
+    @staticmethod
+    def params(spec):
+        p = {
+            "q_proj.weight": ParamSpec((spec.q_dim, spec.hidden_size)),
+            "k_proj.weight": ParamSpec((spec.kv_dim, spec.hidden_size)),
+            "v_proj.weight": ParamSpec((spec.kv_dim, spec.hidden_size)),
+            "o_proj.weight": ParamSpec((spec.hidden_size, spec.q_dim)),
+        }
+        if spec.qk_norm_eps is not None:
+            p["q_norm.weight"] = ParamSpec((spec.head_dim,), "float", ("one_plus_normal", 0.05))
+            p["k_norm.weight"] = ParamSpec((spec.head_dim,), "float", ("one_plus_normal", 0.05))
+        return p
+
+    @staticmethod
+    def placement(spec):
+        return {"q_norm.weight": "float32", "k_norm.weight": "float32"}
+
+    def load(self, tensors):
+        import torch
+        q, k, v = tensors["q_proj.weight"], tensors["k_proj.weight"], tensors["v_proj.weight"]
+        if not (q.dtype == k.dtype == v.dtype):
+            q, k, v = (t.float() for t in (q, k, v))
+        # rows concatenated: one product serves q, k and v; no output element changes
+        self.w_qkv = torch.cat([q, k, v], dim=0).contiguous()
+        self.w_o = tensors["o_proj.weight"]
+        if self.spec.qk_norm_eps is not None:
+            self.q_norm = tensors["q_norm.weight"]
+            self.k_norm = tensors["k_norm.weight"]
+
+    def cache_need(self):
+        s = self.spec
+        return KVNeed(num_kv_heads=s.num_kv_heads, head_dim=s.head_dim, window=s.window)
+
+    def state_need(self):
+        return None
+
+    def forward(self, x, batch, cache, state=None):
+        s, rt = self.spec, self.rt
+        n = x.shape[0]
+        qkv = rt.linear(x, self.w_qkv)
+        inv_freq, rotary_dim = self.position.rotary_table()
+        table = batch.block_tables[cache.group]
+        q = rt.ops.qk_norm_rope_kv_write(
+            qkv, rt.empty((n, s.q_dim), rt.act_dtype), cache.k, cache.v,
+            batch.positions, batch.seq_of_token, table, s.num_heads, s.num_kv_heads, s.head_dim,
+            self.q_norm, self.k_norm, s.qk_norm_eps if s.qk_norm_eps is not None else 0.0,
+            inv_freq, rotary_dim, write_kv=cache.writable)
+        out = rt.ops.paged_attention_generic(
+            q, cache.k, cache.v, rt.empty((n, s.q_dim), rt.act_dtype),
+            batch.positions, batch.seq_of_token, table, s.num_heads, s.num_kv_heads, s.head_dim,
+            self.scale, s.window or 0)
+        return rt.linear(out, self.w_o)

@@ -1,0 +1,59 @@
+"""Position-encoding parts.  A position part is owned by a mixer, which applies
+it inside its own kernel; the interface is what that kernel needs:
+
+    rotary_table() -> (inv_freq float32 [rotary_dim / 2] on the device, rotary_dim)
+                      or (None, 0) when the part does not rotate
+
+A rotary part of another kind (scaled frequencies, another base) only has to
+produce its own table; pairing "half" rotates dim i with dim i + rotary_dim/2.
+"""
+from __future__ import annotations
+
+import torch
+
+from .base import register
+
+
+@register("position", "none")
+class NoPosition:
+    def __init__(self, spec, runtime):
+        self.spec = spec
+
+    @staticmethod
+    def params(spec):
+        return {}
+
+    def load(self, tensors):
+        pass
+
+    def rotary_table(self):
+        return None, 0
+
+
+@register("position", "rope")
+class Rope:
+    """inv_freq[i] = theta^(-2i / rotary_dim), angle = float32(pos) * inv_freq[i]
+    (/root/reference/src/kipp.c:2368-2382).  The table is computed once in
+    float64 and rounded to float32; the angle product is float32."""
+
+    def __init__(self, spec, runtime):
+        if spec.pairing != "half":
+            raise ValueError(f"rope pairing {spec.pairing!r} is not implemented (only 'half')")
+        self.spec = spec
+        self.rotary_dim = spec.head_dim if spec.rotary_dim is None else spec.rotary_dim
+        self.inv_freq = self.frequencies().to(device=runtime.device, dtype=torch.float32)
+
+    def frequencies(self) -> torch.Tensor:
+        half = self.rotary_dim // 2
+        i = torch.arange(half, dtype=torch.float64)
+        return torch.pow(torch.tensor(float(self.spec.theta), dtype=torch.float64), -(2.0 * i) / self.rotary_dim)
+
+    @staticmethod
+    def params(spec):
+        return {}
+
+    def load(self, tensors):
+        pass
+
+    def rotary_table(self):
+        return self.inv_freq, self.rotary_dim

@@ -1,0 +1,72 @@
+"""The device side that parts share: which GPU, which precision, how a tensor
+is placed, and the matrix product.
+
+dtype "bfloat16": weights stay as stored (bfloat16; a tensor stored in 32-bit
+stays 32-bit), activations between kernels are bfloat16, while the residual
+stream, norms, softmax, rotation and every accumulation are float32.
+dtype "float32": everything is widened to float32 and every product is a true
+32-bit one (no matrix-core or reduced-precision mode).
+"""
+from __future__ import annotations
+
+import torch
+
+from .csrc import ops
+
+DTYPES = {"bfloat16": torch.bfloat16, "float32": torch.float32}
+
+
+class Runtime:
+    def __init__(self, dtype: str = "bfloat16", device: str = "cuda:0"):
+        if dtype not in DTYPES:
+            raise ValueError(f"dtype must be one of {sorted(DTYPES)}, got {dtype!r}")
+        if not torch.cuda.is_available():
+            raise RuntimeError("no GPU visible: kipp_amd runs on a gfx950 GPU only and has no CPU path")
+        self.dtype = dtype
+        self.device = torch.device(device)
+        self.act_dtype = DTYPES[dtype]
+        self.cache_dtype = DTYPES[dtype]
+        self.ops = ops
+        self._mm_out_f32 = None
+        torch.backends.cuda.matmul.allow_tf32 = False
+
+    # -- placement -----------------------------------------------------------
+    def stored_dtype(self, stored: torch.dtype, kind: str) -> torch.dtype:
+        """Type a tensor has on the device, from its type in the file."""
+        if kind == "int":
+            return torch.int32
+        if self.dtype == "float32":
+            return torch.float32
+        if stored == torch.bfloat16:
+            return torch.bfloat16
+        return torch.float32  # float32 stays, float16 widens exactly
+
+    def place(self, t: torch.Tensor, kind: str = "float", force: torch.dtype | None = None) -> torch.Tensor:
+        target = force or self.stored_dtype(t.dtype, kind)
+        return t.to(device=self.device, dtype=target).contiguous()
+
+    def empty(self, shape, dtype) -> torch.Tensor:
+        return torch.empty(shape, dtype=dtype, device=self.device)
+
+    # -- matrix product ------------------------------------------------------
+    def linear(self, x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+        """float32 [M, N] = x [M, K] . w [N, K]^T."""
+        m = x.shape[0]
+        n = w.shape[0]
+        if w.dtype == torch.float32:
+            if x.dtype != torch.float32:
+                x = self.ops.cast(x, self.empty(x.shape, torch.float32))
+            return self.ops.gemm_f32(x, w, self.empty((m, n), torch.float32))
+        if x.dtype != torch.bfloat16:
+            x = self.ops.cast(x, self.empty(x.shape, torch.bfloat16))
+        # bfloat16 x bfloat16 with float32 accumulation: the library product
+        if self._mm_out_f32 is None:
+            try:
+                torch.mm(x[:1], w[:1].t(), out_dtype=torch.float32)
+                self._mm_out_f32 = True
+            except (RuntimeError, TypeError):
+                self._mm_out_f32 = False
+        if self._mm_out_f32:
+            return torch.mm(x, w.t(), out_dtype=torch.float32)
+        y = torch.mm(x, w.t())
+        return self.ops.cast(y, self.empty((m, n), torch.float32))

@@ -1,0 +1,142 @@
+"""Shared by the GPU tests: schedules of steps, replay through the engine's
+step function, comparison with the plain implementation."""
+from __future__ import annotations
+
+import random
+from typing import Dict, List, Sequence, Tuple
+
+import numpy as np
+
+from tests.plain import qwen3_plain as plain
+
+# Tolerances, fixed before any run.  float32 engine against the float64 plain
+# implementation: rounding of float32 sums only.  bfloat16 engine against the
+# plain implementation on the same (already rounded) weights: activations are
+# rounded to 8 bits of mantissa a few times per layer.
+NMSE_F32 = 1e-10
+NMSE_BF16 = 1e-3
+
+
+def random_tokens(seed: int, n: int, vocab: int) -> List[int]:
+    rng = random.Random(seed)
+    return [rng.randrange(vocab) for _ in range(n)]
+
+
+def plain_logits(folder: str, tokens: Sequence[int]) -> np.ndarray:
+    cfg, weights = plain.load_folder(folder)
+    return plain.forward_whole(cfg, weights, list(tokens))
+
+
+Step = Tuple[List[Tuple[str, int]], List[str]]   # ([(request, number of next tokens)], [requests that end])
+
+
+def replay(engine, requests: Dict[str, Sequence[int]], steps: Sequence[Step]) -> Dict[str, np.ndarray]:
+    """Feed `steps` through engine.step, asking for the logits of every token;
+    returns {request: [tokens fed, vocab]}."""
+    from kipp_amd.engine import StepEntry
+    fed = {r: 0 for r in requests}
+    rows: Dict[str, List[np.ndarray]] = {r: [] for r in requests}
+    for entries, ends in steps:
+        batch = []
+        for rid, n in entries:
+            toks = list(requests[rid][fed[rid]:fed[rid] + n])
+            assert len(toks) == n, f"schedule feeds more tokens of {rid} than it has"
+            batch.append(StepEntry(rid, toks, list(range(n))))
+        logits = engine.step(batch)
+        out = logits.float().cpu().numpy()
+        at = 0
+        for rid, n in entries:
+            rows[rid].append(out[at:at + n])
+            at += n
+            fed[rid] += n
+        for rid in ends:
+            engine.close(rid)
+        engine.cache.check()
+    return {r: np.concatenate(v, axis=0) for r, v in rows.items() if v}
+
+
+def whole(requests) -> List[Step]:
+    return [([(rid, len(toks))], [rid]) for rid, toks in requests.items()]
+
+
+def tail_one_by_one(requests, tail: int = 32) -> List[Step]:
+    steps: List[Step] = []
+    for rid, toks in requests.items():
+        head = max(1, len(toks) - tail)
+        steps.append(([(rid, head)], []))
+        for i in range(head, len(toks)):
+            steps.append(([(rid, 1)], [rid] if i == len(toks) - 1 else []))
+        if head == len(toks):
+            steps[-1] = (steps[-1][0], [rid])
+    return steps
+
+
+def changing_portions(requests, sizes=(5, 16, 2, 7, 3, 2, 33, 2, 11)) -> List[Step]:
+    steps: List[Step] = []
+    for rid, toks in requests.items():
+        at, i = 0, 0
+        while at < len(toks):
+            n = min(sizes[i % len(sizes)], len(toks) - at)
+            if len(toks) - at - n == 1:   # never leave a single token as a "portion" by accident
+                n += 1
+            at += n
+            i += 1
+            steps.append(([(rid, n)], [rid] if at == len(toks) else []))
+    return steps
+
+
+def mixed(requests, seed: int, max_live: int = 4, prefill_portion=(2, 9), decode_tail: int = 12) -> List[Step]:
+    """Up to `max_live` requests at a time; each is fed in portions until
+    `decode_tail` tokens are left, then one token a step; portions of some stand
+    beside single tokens of others; a request is sometimes left out of a step."""
+    rng = random.Random(seed)
+    waiting = list(requests)
+    live: List[str] = []
+    fed = {r: 0 for r in requests}
+    steps: List[Step] = []
+    while waiting or live:
+        while waiting and len(live) < max_live:
+            live.append(waiting.pop(0))
+        entries, ends = [], []
+        for rid in list(live):
+            left = len(requests[rid]) - fed[rid]
+            if len(live) > 1 and rng.random() < 0.2:
+                continue   # left out of this step, goes on later
+            if left > decode_tail:
+                n = min(rng.randint(*prefill_portion), left - decode_tail)
+                if n < 2:
+                    n = min(2, left)
+            else:
+                n = 1
+            entries.append((rid, n))
+            fed[rid] += n
+            if fed[rid] == len(requests[rid]):
+                ends.append(rid)
+                live.remove(rid)
+        if entries:
+            steps.append((entries, ends))
+    return steps
+
+
+def peak_pages(requests, steps: Sequence[Step], page: int) -> int:
+    """The most pages that live requests hold at any time under `steps`."""
+    fed: Dict[str, int] = {}
+    peak = 0
+    for entries, ends in steps:
+        for rid, n in entries:
+            fed[rid] = fed.get(rid, 0) + n
+        peak = max(peak, sum(-(-n // page) for n in fed.values()))
+        for rid in ends:
+            del fed[rid]
+    return peak
+
+
+def assert_close(got: np.ndarray, ref: np.ndarray, tol: float, what: str) -> None:
+    assert got.shape == ref.shape, f"{what}: shape {got.shape} vs {ref.shape}"
+    assert np.isfinite(got).all(), f"{what}: non-finite logits"
+    worst, worst_at = 0.0, -1
+    for i in range(ref.shape[0]):
+        e = plain.nmse(got[i], ref[i])
+        if e > worst:
+            worst, worst_at = e, i
+    assert worst <= tol, f"{what}: NMSE {worst:.3e} at position {worst_at} exceeds {tol:.1e}"

@@ -1,0 +1,60 @@
+"""The engine against the plain implementation: whole sequences, decoding one
+by one, portions of changing size and mixed batches with few pages, in float32
+and in bfloat16, for both tiny configurations."""
+import numpy as np
+import pytest
+
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+PAGE = {"a": 16, "b": 8}
+LENGTHS = {"a": [1, 17, 40, 64], "b": [7, 33, 61, 100]}
+
+
+def _engine(model_folders, key, dtype, num_pages=None, max_tokens=512, **kw):
+    from kipp_amd.engine import Engine
+    return Engine.from_folder(model_folders[(key, dtype)], dtype=dtype, page_size=PAGE[key],
+                              num_pages=num_pages, max_tokens=None if num_pages else max_tokens, **kw)
+
+
+def _requests(key, cfg, seed=0):
+    return {f"r{i}": H.random_tokens(seed * 100 + i, n, cfg["vocab_size"]) for i, n in enumerate(LENGTHS[key])}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("key", ["a", "b"])
+@pytest.mark.parametrize("cut", ["whole", "tail", "portions", "mixed"])
+def test_cuttings_match_plain(model_folders, tiny_configs, key, dtype, cut):
+    cfg = tiny_configs[key]
+    requests = _requests(key, cfg)
+    tol = H.NMSE_F32 if dtype == "float32" else H.NMSE_BF16
+    if cut == "mixed":
+        more = {f"s{i}": H.random_tokens(900 + i, n, cfg["vocab_size"]) for i, n in enumerate(LENGTHS[key])}
+        requests = {**requests, **more}
+        steps = H.mixed(requests, seed=5)
+        # exactly as many pages as the live requests hold at the peak: freed pages are used again
+        pages = H.peak_pages(requests, steps, PAGE[key])
+        assert pages < sum(-(-len(t) // PAGE[key]) for t in requests.values())
+        engine = _engine(model_folders, key, dtype, num_pages=pages, share_prefixes=False)
+    else:
+        engine = _engine(model_folders, key, dtype, share_prefixes=False)
+        steps = {"whole": H.whole, "tail": H.tail_one_by_one, "portions": H.changing_portions}[cut](requests)
+    got = H.replay(engine, requests, steps)
+    for rid, toks in requests.items():
+        ref = H.plain_logits(model_folders[(key, dtype)], toks)
+        H.assert_close(got[rid], ref, tol, f"{key}/{dtype}/{cut}/{rid}")
+    assert engine.cache.free_pages() == [g.pool.num_pages for g in engine.cache.groups]
+
+
+@pytest.mark.parametrize("key", ["a", "b"])
+def test_float32_cuttings_are_bitwise_equal(model_folders, tiny_configs, key):
+    """In float32 every reduction runs in an order fixed by the token's own
+    position, so the logits do not depend on the cutting at all."""
+    cfg = tiny_configs[key]
+    requests = _requests(key, cfg, seed=3)
+    base = H.replay(_engine(model_folders, key, "float32", share_prefixes=False), requests, H.whole(requests))
+    for maker in (H.tail_one_by_one, H.changing_portions, lambda r: H.mixed(r, seed=11)):
+        got = H.replay(_engine(model_folders, key, "float32", share_prefixes=False), requests, maker(requests))
+        for rid in requests:
+            assert np.array_equal(got[rid], base[rid]), f"{key}/{rid}: bits differ between cuttings"

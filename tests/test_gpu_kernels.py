@@ -1,0 +1,259 @@
+"""Each HIP kernel alone against a plain float64 reference, at sizes other
+than the engine tests use (ragged widths, odd head counts, several head sizes)."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from tests.plain import qwen3_plain as plain
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+def _ops():
+    from kipp_amd.csrc import ops
+    return ops
+
+
+def _t(a, dtype=torch.float32):
+    return torch.tensor(np.asarray(a), dtype=dtype, device=DEV).contiguous()
+
+
+def _rel(got, ref):
+    return plain.nmse(got, ref)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_embed(dtype):
+    ops = _ops()
+    rng = np.random.default_rng(0)
+    table = torch.tensor(rng.normal(size=(301, 72)), dtype=dtype)
+    tokens = rng.integers(0, 301, size=19)
+    out = ops.embed(table.to(DEV), _t(tokens, torch.int32), torch.empty(19, 72, device=DEV))
+    assert torch.equal(out.cpu(), table.float()[tokens])
+
+
+@pytest.mark.parametrize("width,rows", [(2, 1), (72, 5), (2560, 3), (5000, 2)])
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+def test_rmsnorm(width, rows, out_dtype):
+    ops = _ops()
+    rng = np.random.default_rng(width)
+    x = rng.normal(size=(rows, width)).astype(np.float32)
+    w = (1 + 0.1 * rng.normal(size=width)).astype(np.float32)
+    eps = 1e-5
+    ref = plain.rms_norm(x, w, eps)
+    got = ops.rmsnorm(_t(x), _t(w), eps, torch.empty(rows, width, dtype=out_dtype, device=DEV))
+    tol = 1e-12 if out_dtype == torch.float32 else 1e-5
+    assert _rel(got.float().cpu().numpy(), ref) < tol
+    # with the residual add fused in: x is updated in place
+    delta = rng.normal(size=(rows, width)).astype(np.float32)
+    xd = _t(x)
+    got = ops.rmsnorm(xd, _t(w), eps, torch.empty(rows, width, dtype=out_dtype, device=DEV), delta=_t(delta))
+    assert np.array_equal(xd.cpu().numpy(), x + delta)
+    assert _rel(got.float().cpu().numpy(), plain.rms_norm(x + delta, w, eps)) < tol
+
+
+def test_rmsnorm_reference_vector():
+    # /root/reference/tests/kipp_test.c:88-96: x=[3,4], w=1, eps=0 -> x / sqrt(12.5)
+    ops = _ops()
+    got = ops.rmsnorm(_t([[3.0, 4.0]]), _t([1.0, 1.0]), 0.0, torch.empty(1, 2, device=DEV)).cpu().numpy()[0]
+    assert np.allclose(got, np.array([3.0, 4.0]) / math.sqrt(12.5), rtol=1e-6)
+
+
+@pytest.mark.parametrize("inner,rows", [(1, 1), (200, 7), (9728, 2)])
+def test_swiglu(inner, rows):
+    ops = _ops()
+    rng = np.random.default_rng(inner)
+    gu = (3 * rng.normal(size=(rows, 2 * inner))).astype(np.float32)
+    ref = plain.silu(gu[:, :inner].astype(np.float64)) * gu[:, inner:]
+    got = ops.swiglu(_t(gu), torch.empty(rows, inner, device=DEV))
+    assert _rel(got.cpu().numpy(), ref) < 1e-12
+    # /root/reference/tests/kipp_test.c:130-132
+    got = ops.swiglu(_t([[0.0, 1.0, 5.0, 2.0]]), torch.empty(1, 2, device=DEV)).cpu().numpy()[0]
+    assert abs(got[0]) < 1e-7 and abs(got[1] - 1.4621172) < 1e-6
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 1, 1), (3, 2, 3), (5, 77, 130), (64, 64, 16), (130, 509, 80), (17, 200, 2560)])
+@pytest.mark.parametrize("wdtype", [torch.float32, torch.bfloat16])
+def test_gemm_f32(m, n, k, wdtype):
+    ops = _ops()
+    rng = np.random.default_rng(m * 1000 + n)
+    x = rng.normal(size=(m, k)).astype(np.float32)
+    w = torch.tensor(rng.normal(size=(n, k)), dtype=wdtype)
+    ref = x.astype(np.float64) @ w.double().numpy().T
+    got = ops.gemm_f32(_t(x), w.to(DEV), torch.empty(m, n, device=DEV))
+    assert _rel(got.cpu().numpy(), ref) < 1e-12
+    # integer-valued inputs: float32 sums are exact, so any tiling fault shows at tolerance 0
+    xi = rng.integers(-3, 4, size=(m, k)).astype(np.float32)
+    wi = rng.integers(-3, 4, size=(n, k)).astype(np.float32)
+    got = ops.gemm_f32(_t(xi), _t(wi).to(wdtype), torch.empty(m, n, device=DEV))
+    assert np.array_equal(got.cpu().numpy(), xi @ wi.T)
+
+
+def test_gemm_f32_reference_vector():
+    # /root/reference/tests/kipp_test.c:98-108
+    ops = _ops()
+    got = ops.gemm_f32(_t([[2.0, -1.0, 0.5]]), _t([[1, 2, 3], [-1, 0.5, 0]]), torch.empty(1, 2, device=DEV))
+    assert np.allclose(got.cpu().numpy(), [[1.5, -2.5]])
+
+
+def test_gemm_f32_rows_do_not_depend_on_the_batch():
+    ops = _ops()
+    rng = np.random.default_rng(5)
+    x = rng.normal(size=(150, 333)).astype(np.float32)
+    w = rng.normal(size=(90, 333)).astype(np.float32)
+    full = ops.gemm_f32(_t(x), _t(w), torch.empty(150, 90, device=DEV)).cpu().numpy()
+    for lo, hi in [(0, 1), (63, 66), (149, 150), (70, 133)]:
+        part = ops.gemm_f32(_t(x[lo:hi]), _t(w), torch.empty(hi - lo, 90, device=DEV)).cpu().numpy()
+        assert np.array_equal(part, full[lo:hi])
+
+
+def _paged_setup(rng, seq_lens, n_kv, d, page, dtype, extra_pages=3):
+    """Random caches and a scrambled page table for sequences of the given lengths."""
+    blocks = [-(-n // page) for n in seq_lens]
+    total = sum(blocks) + extra_pages
+    perm = rng.permutation(total)
+    max_blocks = max(blocks)
+    table = np.zeros((len(seq_lens), max_blocks), dtype=np.int32)
+    at = 0
+    for s, b in enumerate(blocks):
+        table[s, :b] = perm[at:at + b]
+        at += b
+    k = torch.tensor(rng.normal(size=(total, n_kv, page, d)) + 0.5, dtype=dtype)
+    v = torch.tensor(rng.normal(size=(total, n_kv, page, d)) + 1.0, dtype=dtype)  # a DC offset in V
+    return table, k, v
+
+
+def _gather(cache, table_row, n, page):
+    out = []
+    for s in range(n):
+        out.append(cache[table_row[s // page], :, s % page, :].double().numpy())
+    return np.stack(out)  # [n, n_kv, d]
+
+
+@pytest.mark.parametrize("n_q,n_kv,d,page", [(4, 2, 16, 16), (6, 3, 48, 8), (5, 1, 80, 4), (8, 8, 128, 16), (2, 1, 256, 32)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("window", [0, 37])
+def test_paged_attention_generic(n_q, n_kv, d, page, dtype, window):
+    ops = _ops()
+    rng = np.random.default_rng(n_q * 100 + d + window)
+    seq_lens = [1, 70, 130, 33]              # tokens in the cache after this step
+    q_lens = [1, 1, 21, 33]                  # of which the last q_len are this step's queries
+    table, k, v = _paged_setup(rng, seq_lens, n_kv, d, page, dtype)
+    positions, seq_of = [], []
+    for s, (n, ql) in enumerate(zip(seq_lens, q_lens)):
+        positions += list(range(n - ql, n))
+        seq_of += [s] * ql
+    t = len(positions)
+    q = torch.tensor(rng.normal(size=(t, n_q * d)), dtype=dtype)
+    scale = 1.0 / math.sqrt(d)
+    out = ops.paged_attention_generic(q.to(DEV), k.to(DEV), v.to(DEV), torch.empty(t, n_q * d, dtype=dtype, device=DEV),
+                                      _t(positions, torch.int32), _t(seq_of, torch.int32), _t(table, torch.int32),
+                                      n_q, n_kv, d, scale, window)
+    ref = np.zeros((t, n_q, d))
+    qd = q.double().numpy().reshape(t, n_q, d)
+    for i, (pos, s) in enumerate(zip(positions, seq_of)):
+        ks, vs = _gather(k, table[s], pos + 1, page), _gather(v, table[s], pos + 1, page)
+        lo = max(0, pos - window + 1) if window else 0
+        for h in range(n_q):
+            g = h // (n_q // n_kv)
+            p = plain.softmax((ks[lo:, g] @ qd[i, h]) * scale)
+            ref[i, h] = p @ vs[lo:, g]
+    tol = 1e-11 if dtype == torch.float32 else 2e-5
+    assert _rel(out.float().cpu().numpy().reshape(t, n_q, d), ref) < tol
+
+
+def test_attention_reference_vector():
+    # /root/reference/tests/kipp_test.c:135-175: 2 tokens, 32 query heads over 8 key/value heads,
+    # q = k = 0, v0 = 1, v1 = 3 -> token 0 gives 1.0, token 1 gives 2.0
+    ops = _ops()
+    n_q, n_kv, d, page = 32, 8, 128, 16
+    k = torch.zeros(1, n_kv, page, d, device=DEV)
+    v = torch.zeros(1, n_kv, page, d, device=DEV)
+    v[0, :, 0, :] = 1.0
+    v[0, :, 1, :] = 3.0
+    q = torch.zeros(2, n_q * d, device=DEV)
+    out = ops.paged_attention_generic(q, k, v, torch.empty_like(q), _t([0, 1], torch.int32), _t([0, 0], torch.int32),
+                                      _t([[0]], torch.int32), n_q, n_kv, d, 1 / math.sqrt(d), 0).cpu().numpy()
+    assert np.allclose(out[0], 1.0) and np.allclose(out[1], 2.0)
+
+
+@pytest.mark.parametrize("n_q,n_kv,d,page,rotary", [(4, 2, 16, 16, 16), (3, 1, 48, 8, 48), (8, 2, 128, 16, 128), (2, 2, 64, 4, 32)])
+@pytest.mark.parametrize("mode", ["f32", "bf16"])
+@pytest.mark.parametrize("norm", [True, False])
+def test_qk_norm_rope_kv_write(n_q, n_kv, d, page, rotary, mode, norm):
+    ops = _ops()
+    rng = np.random.default_rng(d + n_q)
+    seq_lens, q_lens = [40, 9, 1], [7, 9, 1]
+    cdt = torch.float32 if mode == "f32" else torch.bfloat16
+    table, k, v = _paged_setup(rng, seq_lens, n_kv, d, page, cdt)
+    k0, v0 = k.clone(), v.clone()
+    positions, seq_of = [], []
+    for s, (n, ql) in enumerate(zip(seq_lens, q_lens)):
+        positions += list(range(n - ql, n))
+        seq_of += [s] * ql
+    t = len(positions)
+    qkv = rng.normal(size=(t, (n_q + 2 * n_kv) * d)).astype(np.float32)
+    qw = (1 + 0.1 * rng.normal(size=d)).astype(np.float32)
+    kw = (1 + 0.1 * rng.normal(size=d)).astype(np.float32)
+    eps, theta = 1e-5, 10000.0
+    half = rotary // 2
+    inv_freq = np.power(np.float64(theta), -(2.0 * np.arange(half)) / rotary).astype(np.float32)
+    kd, vd = k.to(DEV), v.to(DEV)
+    q_out = ops.qk_norm_rope_kv_write(
+        _t(qkv), torch.empty(t, n_q * d, dtype=cdt, device=DEV), kd, vd,
+        _t(positions, torch.int32), _t(seq_of, torch.int32), _t(table, torch.int32), n_q, n_kv, d,
+        _t(qw) if norm else None, _t(kw) if norm else None, eps, _t(inv_freq), rotary)
+
+    def ref_heads(x, n_heads, w):
+        x = x.astype(np.float64)
+        if norm:
+            x = plain.head_norm(x, n_heads, d, w, eps)
+        xh = x.reshape(t, n_heads, d)
+        rot = plain.rope(xh[..., :rotary].reshape(t, n_heads * rotary), n_heads, rotary, positions, theta)
+        xh = np.concatenate([rot.reshape(t, n_heads, rotary), xh[..., rotary:]], axis=-1)
+        return xh
+    q_ref = ref_heads(qkv[:, :n_q * d], n_q, qw)
+    k_ref = ref_heads(qkv[:, n_q * d:(n_q + n_kv) * d], n_kv, kw)
+    v_ref = qkv[:, (n_q + n_kv) * d:].reshape(t, n_kv, d)
+    tol = 1e-11 if mode == "f32" else 1e-5
+    assert _rel(q_out.float().cpu().numpy().reshape(t, n_q, d), q_ref) < tol
+    kc, vc = kd.cpu(), vd.cpu()
+    touched = torch.zeros(k.shape[0], page, dtype=torch.bool)
+    for i, (pos, s) in enumerate(zip(positions, seq_of)):
+        pg, slot = table[s, pos // page], pos % page
+        touched[pg, slot] = True
+        assert _rel(kc[pg, :, slot, :].float().numpy(), k_ref[i]) < tol
+        assert _rel(vc[pg, :, slot, :].float().numpy(), v_ref[i]) < (1e-14 if mode == "f32" else 1e-5)
+    # every slot that no token of the step maps to is untouched
+    keep = ~touched[:, None, :, None].expand_as(k)
+    assert torch.equal(kc[keep], k0[keep]) and torch.equal(vc[keep], v0[keep])
+
+
+def test_rope_reference_vector():
+    # /root/reference/tests/kipp_test.c:110-123: d=4, pos 1, theta 1e4, x=[1,2,3,4]:
+    # pair (0,2) turns by 1.0, pair (1,3) by 0.01
+    ops = _ops()
+    k = torch.zeros(1, 1, 4, 16, device=DEV)
+    v = torch.zeros_like(k)
+    x = np.zeros((1, 3 * 16), dtype=np.float32)
+    x[0, :4] = [1, 2, 3, 4]
+    inv_freq = np.array([1.0, 0.01], dtype=np.float32)
+    q = ops.qk_norm_rope_kv_write(_t(x), torch.empty(1, 16, device=DEV), k, v, _t([1], torch.int32), _t([0], torch.int32),
+                                  _t([[0]], torch.int32), 1, 1, 16, None, None, 0.0, _t(inv_freq), 4).cpu().numpy()[0]
+    c, s, c2, s2 = math.cos(1.0), math.sin(1.0), math.cos(0.01), math.sin(0.01)
+    assert np.allclose(q[:4], [c - 3 * s, 2 * c2 - 4 * s2, 3 * c + s, 4 * c2 + 2 * s2], rtol=1e-6)
+
+
+@pytest.mark.parametrize("vocab,rows", [(1, 1), (509, 3), (151936, 2)])
+def test_argmax(vocab, rows):
+    ops = _ops()
+    rng = np.random.default_rng(vocab)
+    logits = rng.normal(size=(rows, vocab)).astype(np.float32)
+    if vocab > 10:
+        logits[0, 7] = logits[0, vocab - 3] = 50.0   # a tie: the lowest index wins
+    got = ops.argmax(_t(logits), torch.empty(rows, dtype=torch.int32, device=DEV)).cpu().numpy()
+    assert np.array_equal(got, np.argmax(logits, axis=1))
