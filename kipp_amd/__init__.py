@@ -9,3 +9,8 @@ sampling/  greedy and temperature sampling
 csrc/      hand-written HIP kernels for gfx950 and their build
 """
 __version__ = "0.1.0"
+
+
+def generate(*args, **kwargs):
+    from .generation import generate as _generate
+    return _generate(*args, **kwargs)

@@ -82,3 +82,20 @@ class Engine:
         for r, e in zip(requests, entries):
             self.cache.commit(r, e.tokens)
         return logits
+
+    # -- token choice -------------------------------------------------------------------
+    def choose(self, logits: torch.Tensor, requests: Sequence[object]) -> List[int]:
+        """One token for each row of `logits`; `requests[i]` carries the row's
+        sampling parameters, generator and recent tokens.  Greedy rows are
+        chosen on the device; rows with a temperature go through the sampler."""
+        from ..sampling import sample
+        rows = logits.shape[0]
+        if rows != len(requests):
+            raise ValueError("one request for each row of logits")
+        picked = self.rt.ops.argmax(logits, self.rt.empty((rows,), torch.int32)).cpu().tolist()
+        for i, req in enumerate(requests):
+            params = req.params
+            if params.greedy and not params.changes_logits:
+                continue
+            picked[i] = sample(logits[i].cpu().numpy(), params, req.rng, list(req.recent))
+        return picked

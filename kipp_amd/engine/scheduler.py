@@ -1,0 +1,246 @@
+"""The scheduler above the step function: it admits requests, cuts prompts
+into portions under a token budget, decodes, finishes and frees.
+
+Policy (the reference's server loop lifted out of its HTTP code,
+/root/reference/src/kipp_server.c:1623-1893 admission, :1900-2125 stepping):
+
+* Waiting requests are admitted strictly in arrival order; the first that does
+  not fit blocks those behind it.
+* A request is refused at `add` if its prompt plus `max_new_tokens` exceeds the
+  model's positions, or if it could never fit the page pool even alone.
+* Pages are reserved at admission: a request is admitted only if every pool
+  still has its worst-case need plus what every running request may still
+  claim.  So pages never run out in the middle of a generation; when they are
+  short, requests wait (pressure delays, never corrupts).
+* One step = one call of the step function: every decoding request gives its
+  one next token first, then the remaining token budget goes to portions of
+  prompts in arrival order; the last portion of a prompt asks for the logits of
+  its last place.
+* A sampled stop token ends the request and is neither kept nor fed back;
+  reaching `max_new_tokens` ends it without running the last token.
+"""
+from __future__ import annotations
+
+import time
+from collections import deque
+from dataclasses import dataclass, field
+from typing import Deque, Dict, List, Optional, Sequence, Tuple
+
+from ..sampling import SampleParams, XorShift64Star
+from .batch import StepEntry
+
+RECENT_WINDOW = 64  # tokens the penalties look back over (/root/reference/src/kipp_server.c:848)
+
+
+class RequestRefused(ValueError):
+    """The request can never run on this engine."""
+
+
+@dataclass
+class Request:
+    id: object
+    prompt: Sequence[int]
+    max_new_tokens: int
+    params: SampleParams = field(default_factory=SampleParams)
+    seed: int = 1
+    stop_tokens: Tuple[int, ...] = ()
+    # progress
+    state: str = "waiting"          # waiting, prefill, decode, finished
+    fed: int = 0                    # prompt tokens already in the cache
+    output: List[int] = field(default_factory=list)
+    next_token: Optional[int] = None
+    finish_reason: Optional[str] = None
+    rng: Optional[XorShift64Star] = None
+    recent: Deque[int] = field(default_factory=lambda: deque(maxlen=RECENT_WINDOW))
+    arrived: float = 0.0
+    first_token_at: Optional[float] = None
+    finished_at: Optional[float] = None
+
+    @property
+    def budget_tokens(self) -> int:
+        """Most tokens the cache will ever hold for it: the last sampled token is never run."""
+        return len(self.prompt) + max(0, self.max_new_tokens - 1)
+
+
+@dataclass
+class SchedulerStats:
+    requests: int = 0
+    refused: int = 0
+    finished: int = 0
+    prompt_tokens: int = 0
+    generated_tokens: int = 0
+    prefix_tokens_reused: int = 0
+    steps: int = 0
+    waits_for_pages: int = 0
+
+
+class Scheduler:
+    def __init__(self, engine, max_step_tokens: int = 2048, prefill_chunk: int = 512, max_running: int = 64):
+        if max_step_tokens < 1 or prefill_chunk < 1 or max_running < 1:
+            raise ValueError("budgets must be positive")
+        self.engine = engine
+        self.cache = engine.cache
+        self.max_step_tokens = max_step_tokens
+        self.prefill_chunk = prefill_chunk
+        self.max_running = min(max_running, self.cache.max_requests)
+        self.waiting: Deque[Request] = deque()
+        self.running: List[Request] = []
+        self.finished: Dict[object, Request] = {}
+        self.stats = SchedulerStats()
+
+    # -- page arithmetic -----------------------------------------------------------
+    def _pages(self, tokens: int) -> int:
+        return -(-tokens // self.cache.page_size)
+
+    def _still_to_claim(self, req: Request) -> List[int]:
+        """Pages a running request may still claim in each group."""
+        rc = self.cache.requests[req.id]
+        return self.cache.pages_needed(rc, req.budget_tokens)
+
+    # -- interface -------------------------------------------------------------------
+    def add(self, req: Request) -> None:
+        if len(req.prompt) == 0:
+            raise RequestRefused(f"request {req.id!r}: empty prompt")
+        if req.max_new_tokens < 0:
+            raise RequestRefused(f"request {req.id!r}: max_new_tokens must be >= 0")
+        if len(req.prompt) + req.max_new_tokens > self.cache.max_position:
+            self.stats.refused += 1
+            raise RequestRefused(
+                f"request {req.id!r}: prompt {len(req.prompt)} + max_new_tokens {req.max_new_tokens} "
+                f"exceeds the model's {self.cache.max_position} positions")
+        if any(self._pages(req.budget_tokens) > g.pool.num_pages for g in self.cache.groups):
+            self.stats.refused += 1
+            raise RequestRefused(f"request {req.id!r}: needs {self._pages(req.budget_tokens)} pages, more than the pool has")
+        for t in req.prompt:
+            if not 0 <= int(t) < self.engine.vocab_size:
+                self.stats.refused += 1
+                raise RequestRefused(f"request {req.id!r}: token {t} is outside the vocabulary")
+        req.params.validate()
+        if not req.params.greedy:
+            req.rng = XorShift64Star(req.seed if req.seed != 0 else 1)   # 0 mapped to 1 (kipp_server.c:1852-1862)
+        req.state = "waiting"
+        req.arrived = time.monotonic()
+        self.waiting.append(req)
+        self.stats.requests += 1
+
+    def cancel(self, request_id) -> None:
+        for req in list(self.waiting):
+            if req.id == request_id:
+                self.waiting.remove(req)
+                self._finish(req, "cancelled", opened=False)
+                return
+        for req in self.running:
+            if req.id == request_id:
+                self._finish(req, "cancelled")
+                return
+
+    @property
+    def idle(self) -> bool:
+        return not self.waiting and not self.running
+
+    # -- admission ---------------------------------------------------------------------
+    def _admit(self) -> None:
+        while self.waiting and len(self.running) < self.max_running:
+            req = self.waiting[0]
+            rc = self.cache.open(req.id, req.prompt)       # adopts the longest known beginning
+            need = self.cache.pages_needed(rc, req.budget_tokens)
+            promised = [0] * len(self.cache.groups)
+            for other in self.running:
+                for g, n in enumerate(self._still_to_claim(other)):
+                    promised[g] += n
+            free = self.cache.free_pages()
+            if any(need[g] + promised[g] > free[g] for g in range(len(free))):
+                self.cache.close(req.id)                   # undo; stays first in line
+                self.stats.waits_for_pages += 1
+                return
+            self.waiting.popleft()
+            req.fed = rc.length
+            self.stats.prefix_tokens_reused += rc.length
+            req.state = "prefill"
+            self.running.append(req)
+
+    # -- one step ------------------------------------------------------------------------
+    def plan(self) -> List[Tuple[Request, List[int], List[int]]]:
+        """(request, tokens, want) of the next step: decode tokens first, then
+        portions of prompts in arrival order while the token budget lasts."""
+        budget = self.max_step_tokens
+        plan = []
+        for req in self.running:
+            if req.state == "decode" and budget > 0:
+                plan.append((req, [req.next_token], [0]))
+                budget -= 1
+        for req in self.running:
+            if req.state != "prefill" or budget <= 0:
+                continue
+            left = len(req.prompt) - req.fed
+            n = min(self.prefill_chunk, left, budget)
+            tokens = [int(t) for t in req.prompt[req.fed:req.fed + n]]
+            plan.append((req, tokens, [n - 1] if n == left else []))
+            budget -= n
+        return plan
+
+    def step(self) -> List[Tuple[object, int]]:
+        """Admit, run one batch, sample.  Returns the (request id, token) pairs
+        produced by this step."""
+        self._admit()
+        plan = self.plan()
+        if not plan:
+            return []
+        entries = [StepEntry(req.id, tokens, want) for req, tokens, want in plan]
+        logits = self.engine.step(entries)
+        self.stats.steps += 1
+        produced: List[Tuple[object, int]] = []
+        sampling = [req for req, _, want in plan if want]
+        for req, tokens, want in plan:
+            if req.state == "prefill":
+                req.fed += len(tokens)
+                self.stats.prompt_tokens += len(tokens)
+        if sampling:
+            chosen = self.engine.choose(logits, sampling)
+            for req, token in zip(sampling, chosen):
+                self._accept(req, int(token), produced)
+        return produced
+
+    def _accept(self, req: Request, token: int, produced) -> None:
+        if req.max_new_tokens == 0:
+            self._finish(req, "length")
+            return
+        if token in req.stop_tokens:
+            self._finish(req, "stop")                      # not kept, not fed back
+            return
+        now = time.monotonic()
+        if req.first_token_at is None:
+            req.first_token_at = now
+        req.output.append(token)
+        req.recent.append(token)
+        produced.append((req.id, token))
+        self.stats.generated_tokens += 1
+        if len(req.output) >= req.max_new_tokens:
+            self._finish(req, "length")
+            return
+        req.next_token = token
+        req.state = "decode"
+
+    def _finish(self, req: Request, reason: str, opened: bool = True) -> None:
+        req.state = "finished"
+        req.finish_reason = reason
+        req.finished_at = time.monotonic()
+        if req in self.running:
+            self.running.remove(req)
+        if opened and req.id in self.cache.requests:
+            self.engine.close(req.id)
+        self.finished[req.id] = req
+        self.stats.finished += 1
+
+    def run(self, max_steps: Optional[int] = None) -> Dict[object, Request]:
+        """Step until every request has finished."""
+        steps = 0
+        while not self.idle:
+            before = (len(self.waiting), len(self.running), self.stats.steps)
+            self.step()
+            steps += 1
+            if max_steps is not None and steps >= max_steps:
+                break
+            if not self.running and self.waiting and (len(self.waiting), 0, self.stats.steps) == before:
+                raise RuntimeError("scheduler stalled: a waiting request cannot be admitted although nothing is running")
+        return self.finished

@@ -16,6 +16,20 @@ from .csrc import ops
 DTYPES = {"bfloat16": torch.bfloat16, "float32": torch.float32}
 
 
+def device_dtype(stored: torch.dtype, kind: str, compute: str) -> torch.dtype:
+    """Type a tensor has on the device, from its type in the file: integer
+    tables are int32; under float32 every real tensor is widened; under bfloat16
+    a bfloat16 tensor stays bfloat16, a tensor stored in 32-bit stays 32-bit and
+    float16 is widened (exactly) to float32."""
+    if kind == "int":
+        return torch.int32
+    if compute == "float32":
+        return torch.float32
+    if stored == torch.bfloat16:
+        return torch.bfloat16
+    return torch.float32
+
+
 class Runtime:
     def __init__(self, dtype: str = "bfloat16", device: str = "cuda:0"):
         if dtype not in DTYPES:
@@ -32,14 +46,7 @@ class Runtime:
 
     # -- placement -----------------------------------------------------------
     def stored_dtype(self, stored: torch.dtype, kind: str) -> torch.dtype:
-        """Type a tensor has on the device, from its type in the file."""
-        if kind == "int":
-            return torch.int32
-        if self.dtype == "float32":
-            return torch.float32
-        if stored == torch.bfloat16:
-            return torch.bfloat16
-        return torch.float32  # float32 stays, float16 widens exactly
+        return device_dtype(stored, kind, self.dtype)
 
     def place(self, t: torch.Tensor, kind: str = "float", force: torch.dtype | None = None) -> torch.Tensor:
         target = force or self.stored_dtype(t.dtype, kind)

@@ -128,7 +128,7 @@ def load_folder(model_dir):
     return config, {name: t.float().numpy().astype(DTYPE) for name, t in tensors.items()}
 
 
-def forward_whole(config, weights, tokens, kv_round=None, return_hidden=False):
+def forward_whole(config, weights, tokens, kv_round=None, return_hidden=False, position_offset=0):
     """Logits [len(tokens), vocab] of one whole sequence.
     Layer order of /root/reference/src/kipp.c:2588-2655 (cpu_forward): input norm, q/k/v,
     per-head q and k norm, rotation, attention, output projection and residual,
@@ -136,13 +136,14 @@ def forward_whole(config, weights, tokens, kv_round=None, return_hidden=False):
     (:2657-2661), here for every position, not only the last.
     `kv_round`: a function applied to keys and values before attention (the
     reference rounds them to bfloat16 there, :2614-2615; the float32 engine keeps
-    them in float32, so its reference passes None)."""
+    them in float32, so its reference passes None).  `position_offset` shifts every
+    position (the result must not change: only distances count)."""
     n_q = config["num_attention_heads"]
     n_kv = config["num_key_value_heads"]
     d = config.get("head_dim") or config["hidden_size"] // n_q
     eps = config["rms_norm_eps"]
     theta = config["rope_theta"]
-    positions = np.arange(len(tokens))
+    positions = np.arange(len(tokens)) + position_offset
     x = embed(weights["model.embed_tokens.weight"], tokens)
     for layer in range(config["num_hidden_layers"]):
         p = f"model.layers.{layer}."

@@ -1,0 +1,140 @@
+"""Through the entry points: greedy generation, temperature sampling, the
+command line, and trace replay as a user runs it."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+from tests import helpers as H
+from tests.plain import qwen3_plain as plain
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _follows_plain_argmax(folder, prompt, output, margin):
+    """Teacher-forced: every generated token is the plain implementation's
+    argmax at its step (or within `margin` of it, for reduced precision)."""
+    cfg, weights = plain.load_folder(folder)
+    logits = plain.forward_whole(cfg, weights, list(prompt) + list(output))
+    for i, tok in enumerate(output):
+        row = logits[len(prompt) - 1 + i]
+        assert row[tok] >= row.max() - margin, f"token {i}: chose {tok} ({row[tok]:.5f}), plain argmax {row.argmax()} ({row.max():.5f})"
+
+
+@pytest.mark.parametrize("key,dtype,margin", [("a", "float32", 1e-5), ("b", "float32", 1e-5), ("a", "bfloat16", 0.03), ("b", "bfloat16", 0.03)])
+def test_greedy_generation_through_the_entry_point(model_folders, tiny_configs, key, dtype, margin):
+    from kipp_amd import generate
+    vocab = tiny_configs[key]["vocab_size"]
+    prompts = [H.random_tokens(40 + i, n, vocab) for i, n in enumerate([1, 9, 40, 23])]
+    outputs = generate(model_folders[(key, dtype)], prompts, max_new_tokens=16, dtype=dtype,
+                       page_size=16 if key == "a" else 8, prefill_chunk=16, max_step_tokens=24)
+    assert [len(o) for o in outputs] == [16] * 4
+    for prompt, out in zip(prompts, outputs):
+        _follows_plain_argmax(model_folders[(key, dtype)], prompt, out, margin)
+
+
+def test_long_decoding_matches_plain(model_folders, tiny_configs):
+    """100 tokens decoded one by one after a short prompt, every logits row compared."""
+    from kipp_amd.engine import Engine, StepEntry
+    folder = model_folders[("b", "float32")]
+    engine = Engine.from_folder(folder, dtype="float32", page_size=8, max_tokens=256)
+    toks = H.random_tokens(77, 3, 509)
+    rows = [engine.step([StepEntry("d", toks, [2])])]
+    for _ in range(100):
+        nxt = int(engine.choose(rows[-1], [type("R", (), {"params": __import__("kipp_amd.sampling", fromlist=["x"]).SampleParams(), "rng": None, "recent": []})()])[0])
+        toks.append(nxt)
+        rows.append(engine.step([StepEntry("d", [nxt], [0])]))
+    got = np.concatenate([r.cpu().numpy() for r in rows])
+    ref = H.plain_logits(folder, toks)[2:]
+    H.assert_close(got, ref, H.NMSE_F32, "long decode")
+
+
+def test_first_tokens_of_a_sequence(model_folders):
+    """Positions 0, 1, 2 each as a step of their own: the empty-cache edge."""
+    from kipp_amd.engine import Engine, StepEntry
+    for dtype, tol in (("float32", H.NMSE_F32), ("bfloat16", H.NMSE_BF16)):
+        folder = model_folders[("a", dtype)]
+        engine = Engine.from_folder(folder, dtype=dtype, page_size=16, max_tokens=64)
+        toks = [200, 3, 77]
+        got = np.concatenate([engine.step([StepEntry("f", [t], [0])]).float().cpu().numpy() for t in toks])
+        H.assert_close(got, H.plain_logits(folder, toks), tol, f"first tokens {dtype}")
+
+
+def test_temperature_sampling_is_seeded(model_folders, tiny_configs):
+    from kipp_amd import generate
+    folder = model_folders[("b", "bfloat16")]
+    prompts = [H.random_tokens(5, 7, 509), H.random_tokens(6, 33, 509), H.random_tokens(7, 61, 509)]
+    kw = dict(max_new_tokens=12, temperature=0.8, seed=11, dtype="bfloat16", page_size=8, prefill_chunk=16)
+    a, b = generate(folder, prompts, **kw), generate(folder, prompts, **kw)
+    c = generate(folder, prompts, **dict(kw, seed=12))
+    assert a == b and a != c and all(len(o) == 12 for o in a)
+    top1 = generate(folder, prompts, **dict(kw, top_k=1))
+    assert top1 == generate(folder, prompts, **dict(kw, temperature=0.0))
+
+
+def test_command_line(model_folders):
+    folder = model_folders[("a", "float32")]
+    run = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "kipp"), "--model", folder, "--dtype", "float32",
+                          "--tokens", "5,17,3,99", "--decode", "6", "--top", "3"], capture_output=True, text=True, timeout=300)
+    assert run.returncode == 0, run.stderr
+    lines = run.stdout.strip().splitlines()
+    assert lines[0].startswith("generated\t") and len(lines[0].split("\t")[1].split()) == 6
+    generated = [int(t) for t in lines[0].split("\t")[1].split()]
+    _follows_plain_argmax(folder, [5, 17, 3, 99], generated, 1e-5)
+    table = [l.split("\t") for l in lines[1:4]]
+    assert [r[0] for r in table] == ["1", "2", "3"] and float(table[0][2]) >= float(table[1][2]) >= float(table[2][2])
+    # the table is of the last evaluated position: the prompt plus all but the last generated token
+    ref = H.plain_logits(folder, [5, 17, 3, 99] + generated[:-1])[-1]
+    assert int(table[0][1]) == int(ref.argmax()) and abs(float(table[0][2]) - ref.max()) < 1e-4
+    assert "KIPP_METRIC backend=hip-float32 prefill_tokens=4" in run.stderr and "decode_tokens=5" in run.stderr
+
+
+def _trace(requests, steps):
+    fed = {r: 0 for r in requests}
+    lines = []
+    for i, (entries, ends) in enumerate(steps):
+        es = []
+        for rid, n in entries:
+            es.append({"id": rid, "tokens": list(requests[rid][fed[rid]:fed[rid] + n]), "want": list(range(n))})
+            fed[rid] += n
+        lines.append(json.dumps({"step": i, "entries": es, "end": ends}))
+    return lines
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run(model_folders, tiny_configs, tmp_path, dtype):
+    folder = model_folders[("b", dtype)]
+    requests = {f"r{i}": H.random_tokens(300 + i, n, 509) for i, n in enumerate([70, 33, 100, 7, 61, 90])}
+    steps = H.mixed(requests, seed=9)
+    # --max-tokens: live requests' counts, each rounded up to 64
+    fed, peak = {}, 0
+    for entries, ends in steps:
+        for rid, n in entries:
+            fed[rid] = fed.get(rid, 0) + n
+        peak = max(peak, sum(-(-n // 64) * 64 for n in fed.values()))
+        for rid in ends:
+            del fed[rid]
+    out = tmp_path / "out"
+    proc = subprocess.Popen([os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype, "--out", str(out),
+                             "--max-tokens", str(peak)], stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True)
+    for i, line in enumerate(_trace(requests, steps)):
+        proc.stdin.write(line + "\n")
+        proc.stdin.flush()
+        assert proc.stdout.readline().strip() == f"done {i}"
+    proc.stdin.close()
+    assert proc.wait(timeout=60) == 0
+    rows = {r: [] for r in requests}
+    for i, (entries, _) in enumerate(steps):
+        data = np.fromfile(out / f"{i}.f32", dtype="<f4").reshape(-1, 509)
+        at = 0
+        for rid, n in entries:
+            rows[rid].append(data[at:at + n])
+            at += n
+        assert at == data.shape[0]
+    tol = H.NMSE_F32 if dtype == "float32" else H.NMSE_BF16
+    for rid, toks in requests.items():
+        H.assert_close(np.concatenate(rows[rid]), H.plain_logits(folder, toks), tol, f"trace {dtype} {rid}")

@@ -1,0 +1,179 @@
+"""The scheduler's decisions, with the real cache manager and a step function
+that computes nothing (the next token is a function of the tokens fed)."""
+import numpy as np
+import pytest
+
+from kipp_amd.cache import CacheManager, KVNeed
+from kipp_amd.engine.scheduler import Request, RequestRefused, Scheduler
+from kipp_amd.sampling import SampleParams
+
+VOCAB = 50
+
+
+class FakeEngine:
+    """Keeps the cache bookkeeping of the real engine; 'logits' are one-hot at
+    (sum of the request's tokens so far) % VOCAB."""
+
+    def __init__(self, num_pages=8, page_size=4, max_requests=4, max_position=64, share=True):
+        self.cache = CacheManager([KVNeed(1, 16)], [None], page_size, num_pages, max_requests, max_position,
+                                  runtime=None, share_prefixes=share)
+        self.vocab_size = VOCAB
+        self.calls = []
+
+    def step(self, entries):
+        reqs = []
+        for e in entries:
+            if e.request not in self.cache.requests:
+                self.cache.open(e.request)
+            reqs.append(self.cache.requests[e.request])
+        self.cache.reserve([(r, len(e.tokens)) for r, e in zip(reqs, entries)])
+        rows = []
+        for r, e in zip(reqs, entries):
+            self.cache.commit(r, e.tokens)
+            for w in e.want:
+                row = np.zeros(VOCAB, dtype=np.float32)
+                row[sum(r.tokens[:r.length - len(e.tokens) + w + 1]) % VOCAB] = 1.0
+                rows.append(row)
+        self.calls.append([(e.request, len(e.tokens), list(e.want)) for e in entries])
+        self.cache.check()
+        return np.stack(rows) if rows else None
+
+    def choose(self, logits, requests):
+        return [int(np.argmax(row)) for row in logits]
+
+    def close(self, rid):
+        self.cache.close(rid)
+
+
+def expected_output(prompt, n, stop=()):
+    toks, out = list(prompt), []
+    for _ in range(n):
+        t = sum(toks) % VOCAB
+        if t in stop:
+            break
+        out.append(t)
+        toks.append(t)
+    return out
+
+
+def test_one_request_prefill_in_portions_then_decode():
+    eng = FakeEngine(num_pages=16)
+    s = Scheduler(eng, max_step_tokens=8, prefill_chunk=5)
+    prompt = list(range(1, 13))
+    s.add(Request("a", prompt, 4))
+    done = s.run()
+    assert done["a"].output == expected_output(prompt, 4) and done["a"].finish_reason == "length"
+    # portions of 5, 5, 2 (the last asks for its last place), then single tokens; the 4th token is never run
+    assert eng.calls == [[("a", 5, [])], [("a", 5, [])], [("a", 2, [1])], [("a", 1, [0])], [("a", 1, [0])], [("a", 1, [0])]]
+    assert eng.cache.free_pages() == [16] and s.stats.generated_tokens == 4 and s.stats.prompt_tokens == 12
+
+
+def test_decode_tokens_come_first_and_the_budget_is_kept():
+    eng = FakeEngine(num_pages=40, max_requests=4, share=False)
+    s = Scheduler(eng, max_step_tokens=6, prefill_chunk=4)
+    s.add(Request("a", [1, 2, 3], 6))
+    s.step()                                              # a: whole prompt, first token
+    s.add(Request("b", list(range(10)), 2))
+    s.add(Request("c", list(range(5)), 2))
+    s.step()
+    assert eng.calls[-1] == [("a", 1, [0]), ("b", 4, []), ("c", 1, [])]   # 1 + 4 + 1 = budget 6
+    for call in eng.calls:
+        assert sum(n for _, n, _ in call) <= 6
+    s.run()
+    assert s.finished["b"].output == expected_output(list(range(10)), 2)
+    assert s.finished["c"].output == expected_output(list(range(5)), 2)
+    assert s.finished["a"].output == expected_output([1, 2, 3], 6)
+
+
+def test_stop_token_is_neither_kept_nor_fed_back():
+    prompt = [3, 4]
+    chain = expected_output(prompt, 5)
+    stop = chain[2]
+    eng = FakeEngine()
+    s = Scheduler(eng)
+    s.add(Request("a", prompt, 10, stop_tokens=(stop,)))
+    done = s.run()
+    assert done["a"].output == chain[:2] and done["a"].finish_reason == "stop"
+    assert sum(n for call in eng.calls for _, n, _ in call) == len(prompt) + 2   # the stop token was not run
+
+
+def test_refusals():
+    s = Scheduler(FakeEngine(num_pages=4, max_position=64))
+    with pytest.raises(RequestRefused, match="positions"):
+        s.add(Request("a", [1] * 60, 10))
+    with pytest.raises(RequestRefused, match="pages"):
+        s.add(Request("b", [1] * 20, 4))                  # 23 tokens need 6 pages, the pool has 4
+    with pytest.raises(RequestRefused, match="vocabulary"):
+        s.add(Request("c", [VOCAB], 1))
+    with pytest.raises(RequestRefused, match="empty"):
+        s.add(Request("d", [], 1))
+    with pytest.raises(ValueError, match="top_p"):
+        s.add(Request("e", [1], 1, SampleParams(temperature=1.0, top_p=0.0)))
+    assert s.stats.refused == 3 and s.idle
+
+
+def test_when_pages_run_out_requests_wait_in_order_and_nothing_is_corrupted():
+    # 6 pages of 4 tokens.  a and b need 3 pages each at worst; c must wait although a slot is free.
+    eng = FakeEngine(num_pages=6, max_requests=4, share=False)
+    s = Scheduler(eng, max_step_tokens=64, prefill_chunk=64)
+    pa, pb, pc, pd = [1] * 6, [2] * 7, [3] * 5, [4]
+    s.add(Request("a", pa, 6))                            # budget 11 tokens -> 3 pages
+    s.add(Request("b", pb, 5))                            # budget 11 -> 3 pages
+    s.add(Request("c", pc, 3))                            # budget 7 -> 2 pages
+    s.add(Request("d", pd, 1))                            # 1 page, but behind c: strict arrival order
+    s.step()
+    assert [r.id for r in s.running] == ["a", "b"] and [r.id for r in s.waiting] == ["c", "d"]
+    assert s.stats.waits_for_pages >= 1
+    while "b" not in s.finished:
+        s.step()
+        assert all(f >= 0 for f in eng.cache.free_pages())
+    s.step()
+    assert "c" in [r.id for r in s.running] + list(s.finished)
+    done = s.run()
+    for rid, prompt, n in (("a", pa, 6), ("b", pb, 5), ("c", pc, 3), ("d", pd, 1)):
+        assert done[rid].output == expected_output(prompt, n), rid
+    assert eng.cache.free_pages() == [6]
+
+
+def test_reservation_counts_what_running_requests_may_still_claim():
+    eng = FakeEngine(num_pages=5, share=False)
+    s = Scheduler(eng, max_step_tokens=64, prefill_chunk=64)
+    s.add(Request("a", [1, 2], 11))                       # holds 1 page now, may grow to 3
+    s.step()
+    s.add(Request("b", [5] * 9, 1))                       # needs 3 pages; 4 are free, but 2 are promised to a
+    s.step()
+    assert [r.id for r in s.waiting] == ["b"]
+    done = s.run()
+    assert done["a"].output == expected_output([1, 2], 11) and done["b"].output == expected_output([5] * 9, 1)
+
+
+def test_known_beginnings_are_adopted():
+    eng = FakeEngine(num_pages=12, share=True)
+    s = Scheduler(eng)
+    prompt = list(range(1, 15))
+    s.add(Request("a", prompt, 2))
+    s.run()
+    s.add(Request("b", prompt[:10] + [40, 41], 2))
+    done = s.run()
+    assert s.stats.prefix_tokens_reused == 8              # two full pages of four
+    assert eng.calls[-2] == [("b", 4, [3])]               # only the rest of the prompt is run
+    assert done["b"].output == expected_output(prompt[:10] + [40, 41], 2)
+
+
+def test_cancel_and_zero_new_tokens():
+    eng = FakeEngine()
+    s = Scheduler(eng)
+    s.add(Request("a", [1, 2, 3], 5))
+    s.add(Request("z", [1, 2, 3], 0))
+    s.step()
+    s.cancel("a")
+    s.run()
+    assert s.finished["a"].finish_reason == "cancelled" and s.finished["z"].output == []
+    assert eng.cache.free_pages() == [8]
+
+
+def test_temperature_requests_get_their_own_generator():
+    s = Scheduler(FakeEngine())
+    r = Request("a", [1], 1, SampleParams(temperature=0.8), seed=0)
+    s.add(r)
+    assert r.rng is not None and r.rng.state == 1         # 0 is mapped to 1
