@@ -1,0 +1,279 @@
+// Decode attention over the paged cache, bfloat16, split over the keys.
+//
+// One query token per sequence.  A workgroup (4 waves) takes one sequence, one
+// key/value head and one split of SPLIT keys; the GROUP query heads that share
+// the key/value head are computed together, so every key and value is read
+// once for all of them (/root/reference/metal/kipp_kernels.metal:517-626 plays this
+// role in the reference, with 1024-key splits and no sharing across heads).
+//
+//   scores   S^T[key][head] = K . Q^T on the matrix cores: the A operand of
+//            v_mfma_f32_16x16x32_bf16 is a block of 16 key rows read straight
+//            from global memory (16 bytes a lane), B holds the GROUP queries;
+//   softmax  over the split's keys in float32, in LDS, base 2;
+//   values   lanes own 8 columns of a value row; 16 lanes read one row (256 B
+//            at head size 128), the 16 lane groups of the workgroup take every
+//            16th key; products in float32 FMA, summed over the groups in LDS.
+//
+// Split boundaries are multiples of SPLIT in absolute key index, and the merge
+// (attention_decode_reduce_kernel) adds the splits in index order, so the result
+// for a token does not depend on the batch it is in.  A sequence that needs
+// one split only is written normalised at once.
+//
+// Compile-time: HEAD_DIM (multiple of 16, <= 256), GROUP (query heads per
+// key/value head, <= 16).
+#include "common.h"
+#include <math.h>
+
+#ifndef HEAD_DIM
+#error "compile with -DHEAD_DIM=<head size>"
+#endif
+#ifndef GROUP
+#error "compile with -DGROUP=<query heads per key/value head>"
+#endif
+
+#define SPLIT 256
+#define WAVES 4
+#define THREADS (WAVES * KIPP_WAVE)
+#define KSTEPS ((HEAD_DIM + 31) / 32)          // MFMA steps of 32 over the head size
+#define CHUNKS (HEAD_DIM / 8)                  // 16-byte chunks of a row
+#define CHUNKS_PER_LANE ((CHUNKS + 15) / 16)
+#define BLOCKS_PER_WAVE (SPLIT / 16 / WAVES)   // 16-key blocks a wave scores
+#define KEYS_PER_GROUP (SPLIT / 16)            // keys a lane group multiplies with values
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+union Frag {
+    uint4 u;
+    bf16x8 v;
+    bf16_t h[8];
+};
+
+__global__ void __launch_bounds__(THREADS) attention_decode_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
+    bf16_t* __restrict__ out, float* __restrict__ part_acc, float* __restrict__ part_ml,
+    const int32_t* __restrict__ rows, const int32_t* __restrict__ positions, const int32_t* __restrict__ seq_of_token,
+    const int32_t* __restrict__ block_table, int max_blocks, int n_q, int n_kv, int page, float scale_log2e,
+    int window, int max_splits) {
+    __shared__ float s_scores[GROUP][SPLIT + 4];
+    __shared__ float s_red[WAVES][GROUP][HEAD_DIM];
+    __shared__ float s_m[GROUP], s_l[GROUP];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int l16 = lane & 15, h = lane >> 4;
+    const int kvh = blockIdx.y;
+    const int row = rows[blockIdx.z];                 // row of this query token in the batch
+    const int pos = positions[row];
+    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+    const int first_split = lo / SPLIT, last_split = pos / SPLIT;
+    const int split = first_split + blockIdx.x;
+    if (split > last_split) return;                   // the grid covers the longest sequence
+    const int n_splits = last_split - first_split + 1;
+    const int base = split * SPLIT;
+    const int32_t* table = block_table + (size_t)seq_of_token[row] * max_blocks;
+
+    // ---- the GROUP queries as B operand: lane (slot l16, quarter h) holds q[slot][32 t + 8 h .. + 7]
+    Frag qf[KSTEPS];
+#pragma unroll
+    for (int t = 0; t < KSTEPS; ++t) {
+        qf[t].u = make_uint4(0, 0, 0, 0);
+        const int dcol = 32 * t + 8 * h;
+        if (l16 < GROUP && dcol < HEAD_DIM)
+            qf[t].u = *(const uint4*)(q + ((size_t)row * n_q + (size_t)kvh * GROUP + l16) * HEAD_DIM + dcol);
+    }
+
+    // ---- scores: each wave takes BLOCKS_PER_WAVE blocks of 16 keys
+    Frag kf[BLOCKS_PER_WAVE][KSTEPS];
+#pragma unroll
+    for (int b = 0; b < BLOCKS_PER_WAVE; ++b) {
+        const int s = base + (wave * BLOCKS_PER_WAVE + b) * 16 + l16;
+        const bool valid = s >= lo && s <= pos;
+        const bf16_t* k_row = nullptr;
+        if (valid) k_row = k_cache + (((size_t)table[s / page] * n_kv + kvh) * page + s % page) * HEAD_DIM;
+#pragma unroll
+        for (int t = 0; t < KSTEPS; ++t) {
+            const int dcol = 32 * t + 8 * h;
+            kf[b][t].u = make_uint4(0, 0, 0, 0);
+            if (valid && dcol < HEAD_DIM) kf[b][t].u = *(const uint4*)(k_row + dcol);
+        }
+    }
+    // ---- values are asked for now, so that they arrive while the scores are worked on
+    Frag vf[KEYS_PER_GROUP][CHUNKS_PER_LANE];
+    const int kg = wave * 4 + h;                      // this lane group's keys: base + kg + 16 i
+#pragma unroll
+    for (int i = 0; i < KEYS_PER_GROUP; ++i) {
+        const int s = base + kg + 16 * i;
+        const bool valid = s >= lo && s <= pos;
+        const bf16_t* v_row = nullptr;
+        if (valid) v_row = v_cache + (((size_t)table[s / page] * n_kv + kvh) * page + s % page) * HEAD_DIM;
+#pragma unroll
+        for (int c = 0; c < CHUNKS_PER_LANE; ++c) {
+            const int chunk = l16 + 16 * c;
+            vf[i][c].u = make_uint4(0, 0, 0, 0);
+            if (valid && chunk < CHUNKS) vf[i][c].u = *(const uint4*)(v_row + chunk * 8);
+        }
+    }
+#pragma unroll
+    for (int b = 0; b < BLOCKS_PER_WAVE; ++b) {
+        f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int t = 0; t < KSTEPS; ++t) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[b][t].v, qf[t].v, acc, 0, 0, 0);
+        // acc[v] = S^T[key 4 h + v][slot l16]
+        if (l16 < GROUP) {
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int kl = (wave * BLOCKS_PER_WAVE + b) * 16 + 4 * h + v;
+                const int s = base + kl;
+                s_scores[l16][kl] = (s >= lo && s <= pos) ? acc[v] * scale_log2e : -INFINITY;
+            }
+        }
+    }
+    __syncthreads();
+
+    // ---- softmax over the split's keys, one head per wave at a time
+    for (int g = wave; g < GROUP; g += WAVES) {
+        float sc[SPLIT / KIPP_WAVE];
+        float m = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < SPLIT / KIPP_WAVE; ++i) {
+            sc[i] = s_scores[g][lane + KIPP_WAVE * i];
+            m = fmaxf(m, sc[i]);
+        }
+        m = wave_max(m);
+        float l = 0.0f;
+#pragma unroll
+        for (int i = 0; i < SPLIT / KIPP_WAVE; ++i) {
+            const float p = exp2f(sc[i] - m);          // -inf gives 0
+            s_scores[g][lane + KIPP_WAVE * i] = p;
+            l += p;
+        }
+        l = wave_sum(l);
+        if (lane == 0) {
+            s_m[g] = m;
+            s_l[g] = l;
+        }
+    }
+    __syncthreads();
+
+    // ---- values: acc[g][c][j] += p[g][key] * v[key][8 chunk + j]
+    float acc[GROUP][CHUNKS_PER_LANE][8];
+#pragma unroll
+    for (int g = 0; g < GROUP; ++g)
+#pragma unroll
+        for (int c = 0; c < CHUNKS_PER_LANE; ++c)
+#pragma unroll
+            for (int j = 0; j < 8; ++j) acc[g][c][j] = 0.0f;
+#pragma unroll
+    for (int i = 0; i < KEYS_PER_GROUP; ++i) {
+        const int kl = kg + 16 * i;
+        float p[GROUP];
+#pragma unroll
+        for (int g = 0; g < GROUP; ++g) p[g] = s_scores[g][kl];
+#pragma unroll
+        for (int c = 0; c < CHUNKS_PER_LANE; ++c) {
+            float vv[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) vv[j] = bf16_to_f32(vf[i][c].h[j]);
+#pragma unroll
+            for (int g = 0; g < GROUP; ++g)
+#pragma unroll
+                for (int j = 0; j < 8; ++j) acc[g][c][j] = fmaf(p[g], vv[j], acc[g][c][j]);
+        }
+    }
+    // sum the four lane groups of the wave, then the waves
+#pragma unroll
+    for (int g = 0; g < GROUP; ++g)
+#pragma unroll
+        for (int c = 0; c < CHUNKS_PER_LANE; ++c)
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                float a = acc[g][c][j];
+                a += __shfl_xor(a, 16, KIPP_WAVE);
+                a += __shfl_xor(a, 32, KIPP_WAVE);
+                acc[g][c][j] = a;
+            }
+    if (h == 0) {
+#pragma unroll
+        for (int g = 0; g < GROUP; ++g)
+#pragma unroll
+            for (int c = 0; c < CHUNKS_PER_LANE; ++c) {
+                const int chunk = l16 + 16 * c;
+                if (chunk < CHUNKS) {
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) s_red[wave][g][chunk * 8 + j] = acc[g][c][j];
+                }
+            }
+    }
+    __syncthreads();
+    for (int idx = tid; idx < GROUP * HEAD_DIM; idx += THREADS) {
+        const int g = idx / HEAD_DIM, dcol = idx % HEAD_DIM;
+        float a = 0.0f;
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w) a += s_red[w][g][dcol];
+        const int head = kvh * GROUP + g;
+        if (n_splits == 1) {
+            out[((size_t)row * n_q + head) * HEAD_DIM + dcol] = f32_to_bf16(a / s_l[g]);
+        } else {
+            const size_t slot = ((size_t)blockIdx.z * n_q + head) * max_splits + blockIdx.x;
+            part_acc[slot * HEAD_DIM + dcol] = a;
+            if (dcol == 0) {
+                part_ml[slot * 2] = s_m[g];
+                part_ml[slot * 2 + 1] = s_l[g];
+            }
+        }
+    }
+}
+
+// Merge the splits of every (token, head) in index order:
+// m* = max m_s, out = sum_s acc_s 2^(m_s - m*) / sum_s l_s 2^(m_s - m*)
+// (/root/reference/metal/kipp_kernels.metal:741-779).
+__global__ void attention_decode_reduce_kernel(
+    const float* __restrict__ part_acc, const float* __restrict__ part_ml, bf16_t* __restrict__ out,
+    const int32_t* __restrict__ rows, const int32_t* __restrict__ positions, int n_q, int window, int max_splits) {
+    const int head = blockIdx.x, item = blockIdx.y;
+    const int row = rows[item];
+    const int pos = positions[row];
+    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+    const int n_splits = pos / SPLIT - lo / SPLIT + 1;
+    if (n_splits == 1) return;
+    const size_t slot0 = ((size_t)item * n_q + head) * max_splits;
+    float m = -INFINITY;
+    for (int s = 0; s < n_splits; ++s) m = fmaxf(m, part_ml[(slot0 + s) * 2]);
+    float denom = 0.0f;
+    for (int s = 0; s < n_splits; ++s) denom += part_ml[(slot0 + s) * 2 + 1] * exp2f(part_ml[(slot0 + s) * 2] - m);
+    for (int dcol = threadIdx.x; dcol < HEAD_DIM; dcol += blockDim.x) {
+        float a = 0.0f;
+        for (int s = 0; s < n_splits; ++s)
+            a += part_acc[(slot0 + s) * HEAD_DIM + dcol] * exp2f(part_ml[(slot0 + s) * 2] - m);
+        out[((size_t)row * n_q + head) * HEAD_DIM + dcol] = f32_to_bf16(a / denom);
+    }
+}
+
+extern "C" {
+
+int kipp_attention_decode_split() { return SPLIT; }
+
+// `rows[i]` is the batch row of the i-th decode token.  `grid_splits` is how
+// many splits the launch covers (at least those of the longest sequence);
+// `part_acc` holds n_items * n_q * max_splits * HEAD_DIM floats, `part_ml`
+// n_items * n_q * max_splits * 2.
+int kipp_attention_decode(const void* q, const void* k_cache, const void* v_cache, void* out, float* part_acc,
+                          float* part_ml, const int32_t* rows, const int32_t* positions, const int32_t* seq_of_token,
+                          const int32_t* block_table, int max_blocks, int n_items, int n_q, int n_kv, int head_dim,
+                          int page, float scale, int window, int grid_splits, int max_splits, hipStream_t stream) {
+    if (n_items <= 0) return 0;
+    if (head_dim != HEAD_DIM || n_kv <= 0 || n_q != n_kv * GROUP) return -1;
+    if (grid_splits <= 0 || grid_splits > max_splits) return -3;
+    const float scale_log2e = scale * 1.4426950408889634f;
+    hipLaunchKernelGGL(attention_decode_kernel, dim3(grid_splits, n_kv, n_items), dim3(THREADS), 0, stream,
+                       (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, part_acc, part_ml,
+                       rows, positions, seq_of_token, block_table, max_blocks, n_q, n_kv, page, scale_log2e, window,
+                       max_splits);
+    int rc = KIPP_LAUNCH_CHECK();
+    if (rc != 0 || grid_splits == 1) return rc;
+    hipLaunchKernelGGL(attention_decode_reduce_kernel, dim3(n_q, n_items), dim3(HEAD_DIM >= 64 ? 64 : HEAD_DIM), 0,
+                       stream, part_acc, part_ml, (bf16_t*)out, rows, positions, n_q, window, max_splits);
+    return KIPP_LAUNCH_CHECK();
+}
+
+}  // extern "C"

@@ -1,0 +1,240 @@
+// Prefill attention over the paged cache, bfloat16: causal grouped-query
+// attention for portions of prompts (two tokens and more), with the online
+// softmax of flash attention and both products on the matrix cores
+// (/root/reference/metal/kipp_kernels.metal:1380-1611 plays this role in the reference).
+//
+// A workgroup (4 waves) takes 128 consecutive query rows of one sequence and
+// one query head; a wave owns 32 of them.  Keys and values of the sequence are
+// streamed through LDS in tiles of 64 positions, found through the block table
+// (the portion may start at any position; keys 0..pos are in the cache, this
+// step's own keys included).
+//
+//   S^T = K Q^T   v_mfma_f32_32x32x16_bf16, A = key tile from LDS, B = the wave's
+//                 queries held in registers.  In the result a lane holds 16
+//                 keys of ONE query (its column), so the row statistics of the
+//                 softmax are per lane plus one exchange with lane ^ 32.
+//   O^T = V^T P^T A = value tile stored transposed in LDS, B = the probabilities
+//                 straight from the S^T registers (the contraction index of the
+//                 instruction is a dummy, so the key order a lane happens to
+//                 hold is simply used for both operands).  O^T again has the
+//                 query as its column: rescaling needs no exchange at all.
+//
+// Softmax in float32, base 2; probabilities are rounded to bfloat16 for the
+// second product, the row sum is taken from the float32 values.
+//
+// Compile-time: HEAD_DIM (multiple of 16, <= 256).
+#include "common.h"
+#include <math.h>
+
+#ifndef HEAD_DIM
+#error "compile with -DHEAD_DIM=<head size>"
+#endif
+
+#define BM 128
+#define BN 64
+#define WAVES 4
+#define THREADS (WAVES * KIPP_WAVE)
+#define QSTEPS (HEAD_DIM / 16)                 // contraction steps of S^T
+#define DP (((HEAD_DIM + 31) / 32) * 32)       // value columns rounded up to the 32-row tile of O^T
+#define DTILES (DP / 32)
+#define K_PITCH (HEAD_DIM + 8)                 // bf16 elements per key row in LDS
+#define V_PITCH (BN + 4)                       // bf16 elements per value column in LDS
+#define DCHUNKS (HEAD_DIM / 8)
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+
+union Frag {
+    uint4 u;
+    uint2 d[2];
+    bf16x8 v;
+    bf16_t h[8];
+};
+
+__device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
+    return (uint32_t)f32_to_bf16(a) | ((uint32_t)f32_to_bf16(b) << 16);
+}
+
+__global__ void __launch_bounds__(THREADS) attention_prefill_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
+    bf16_t* __restrict__ out, const int32_t* __restrict__ item_seq, const int32_t* __restrict__ item_tile,
+    const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len, const int32_t* __restrict__ positions,
+    const int32_t* __restrict__ block_table, int max_blocks, int n_q, int n_kv, int page, float scale_log2e,
+    int window) {
+    __shared__ __attribute__((aligned(16))) bf16_t Ks[BN * K_PITCH];
+    __shared__ __attribute__((aligned(16))) bf16_t Vt[DP * V_PITCH];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int l32 = lane & 31, hh = lane >> 5;
+    const int head = blockIdx.y;
+    const int kvh = head / (n_q / n_kv);
+    const int seq = item_seq[blockIdx.x];
+    const int tile_row0 = item_tile[blockIdx.x] * BM;           // first row of the tile within the portion
+    const int row0 = q_start[seq] + tile_row0;                  // ... within the batch
+    const int rows_in_tile = min(BM, q_len[seq] - tile_row0);
+    const int pos0 = positions[row0];                           // position of the tile's first query
+    const int last_pos = pos0 + rows_in_tile - 1;
+    const int32_t* table = block_table + (size_t)seq * max_blocks;
+
+    const int my_row = wave * 32 + l32;                         // this lane's query within the tile
+    const bool wave_active = wave * 32 < rows_in_tile;
+    const bool row_valid = my_row < rows_in_tile;
+    const int my_pos = pos0 + my_row;
+    const int my_lo = window > 0 ? max(0, my_pos - window + 1) : 0;
+
+    // the wave's queries as B operand: lane (query l32, half hh) holds q[16 t + 8 hh .. + 7]
+    Frag qf[QSTEPS];
+#pragma unroll
+    for (int t = 0; t < QSTEPS; ++t) {
+        qf[t].u = make_uint4(0, 0, 0, 0);
+        if (row_valid) qf[t].u = *(const uint4*)(q + ((size_t)(row0 + my_row) * n_q + head) * HEAD_DIM + 16 * t + 8 * hh);
+    }
+
+    f32x16 o[DTILES];
+#pragma unroll
+    for (int dt = 0; dt < DTILES; ++dt)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) o[dt][v] = 0.0f;
+    float m_run = -INFINITY, l_run = 0.0f;
+
+    // value rows beyond the head size stay zero for the whole kernel
+    if (DP > HEAD_DIM) {
+        for (int i = tid; i < (DP - HEAD_DIM) * V_PITCH; i += THREADS) Vt[HEAD_DIM * V_PITCH + i] = 0;
+    }
+
+    const int tile_lo = (window > 0 ? max(0, pos0 - window + 1) : 0) / BN;
+    const int tile_hi = last_pos / BN;
+    for (int kt = tile_lo; kt <= tile_hi; ++kt) {
+        const int key0 = kt * BN;
+        __syncthreads();   // the tile before has been read by every wave
+        // ---- keys: [key][d], 16 bytes a thread
+        for (int c = tid; c < BN * DCHUNKS; c += THREADS) {
+            const int key = c / DCHUNKS, chunk = c % DCHUNKS;
+            const int s = key0 + key;
+            uint4 val = make_uint4(0, 0, 0, 0);
+            if (s <= last_pos)
+                val = *(const uint4*)(k_cache + (((size_t)table[s / page] * n_kv + kvh) * page + s % page) * HEAD_DIM + chunk * 8);
+            *(uint4*)(Ks + key * K_PITCH + chunk * 8) = val;
+        }
+        // ---- values, transposed: [d][key]; a thread takes two keys and 8 columns
+        for (int c = tid; c < (BN / 2) * DCHUNKS; c += THREADS) {
+            const int pair = c % (BN / 2), chunk = c / (BN / 2);
+            Frag a, b;
+            a.u = make_uint4(0, 0, 0, 0);
+            b.u = make_uint4(0, 0, 0, 0);
+            const int s = key0 + 2 * pair;
+            if (s <= last_pos)
+                a.u = *(const uint4*)(v_cache + (((size_t)table[s / page] * n_kv + kvh) * page + s % page) * HEAD_DIM + chunk * 8);
+            if (s + 1 <= last_pos)
+                b.u = *(const uint4*)(v_cache + (((size_t)table[(s + 1) / page] * n_kv + kvh) * page + (s + 1) % page) * HEAD_DIM + chunk * 8);
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                *(uint32_t*)(Vt + (chunk * 8 + j) * V_PITCH + 2 * pair) = (uint32_t)a.h[j] | ((uint32_t)b.h[j] << 16);
+        }
+        __syncthreads();
+        if (!wave_active) continue;
+
+        // ---- S^T = K Q^T for the two 32-key halves of the tile
+        f32x16 s_acc[2];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) s_acc[j][v] = 0.0f;
+#pragma unroll
+            for (int t = 0; t < QSTEPS; ++t) {
+                Frag kf;
+                kf.u = *(const uint4*)(Ks + (32 * j + l32) * K_PITCH + 16 * t + 8 * hh);
+                s_acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf.v, qf[t].v, s_acc[j], 0, 0, 0);
+            }
+        }
+        // ---- mask and online softmax; register v of half j is key 32 j + 8 (v / 4) + 4 hh + v % 4
+        float m_tile = -INFINITY;
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int s = key0 + 32 * j + 8 * (v / 4) + 4 * hh + (v % 4);
+                const float x = (s <= my_pos && s >= my_lo) ? s_acc[j][v] * scale_log2e : -INFINITY;
+                s_acc[j][v] = x;
+                m_tile = fmaxf(m_tile, x);
+            }
+        m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, KIPP_WAVE));
+        const float m_new = fmaxf(m_run, m_tile);
+        const float m_use = m_new == -INFINITY ? 0.0f : m_new;   // a row with nothing visible yet
+        const float alpha = exp2f(m_run - m_use);
+        float l_tile = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const float p = exp2f(s_acc[j][v] - m_use);
+                s_acc[j][v] = p;
+                l_tile += p;
+            }
+        l_tile += __shfl_xor(l_tile, 32, KIPP_WAVE);
+        l_run = l_run * alpha + l_tile;
+        m_run = m_new;
+#pragma unroll
+        for (int dt = 0; dt < DTILES; ++dt)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) o[dt][v] *= alpha;
+        // ---- O^T += V^T P^T; step st of half j uses registers 8 st .. 8 st + 7, which are the keys
+        //      32 j + 16 st + {4 hh .. 4 hh + 3} and 32 j + 16 st + 8 + {4 hh .. 4 hh + 3}
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int st = 0; st < 2; ++st) {
+                Frag pf;
+                pf.u.x = pack_bf16(s_acc[j][8 * st + 0], s_acc[j][8 * st + 1]);
+                pf.u.y = pack_bf16(s_acc[j][8 * st + 2], s_acc[j][8 * st + 3]);
+                pf.u.z = pack_bf16(s_acc[j][8 * st + 4], s_acc[j][8 * st + 5]);
+                pf.u.w = pack_bf16(s_acc[j][8 * st + 6], s_acc[j][8 * st + 7]);
+#pragma unroll
+                for (int dt = 0; dt < DTILES; ++dt) {
+                    Frag vf;
+                    const bf16_t* col = Vt + (32 * dt + l32) * V_PITCH + 32 * j + 16 * st + 4 * hh;
+                    vf.d[0] = *(const uint2*)(col);
+                    vf.d[1] = *(const uint2*)(col + 8);
+                    o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf.v, pf.v, o[dt], 0, 0, 0);
+                }
+            }
+    }
+    if (!row_valid) return;
+    // O^T register v of tile dt is column 32 dt + 8 (v / 4) + 4 hh + v % 4 of this lane's query
+    const float inv = 1.0f / l_run;
+    bf16_t* o_row = out + ((size_t)(row0 + my_row) * n_q + head) * HEAD_DIM;
+#pragma unroll
+    for (int dt = 0; dt < DTILES; ++dt)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const int dcol = 32 * dt + 8 * g + 4 * hh;
+            if (dcol < HEAD_DIM) {
+                uint2 w;
+                w.x = pack_bf16(o[dt][4 * g + 0] * inv, o[dt][4 * g + 1] * inv);
+                w.y = pack_bf16(o[dt][4 * g + 2] * inv, o[dt][4 * g + 3] * inv);
+                *(uint2*)(o_row + dcol) = w;
+            }
+        }
+}
+
+extern "C" {
+
+int kipp_attention_prefill_rows() { return BM; }
+
+// `item_seq[i]`, `item_tile[i]`: sequence (row of the block table) and 128-row
+// tile of its portion for work item i.
+int kipp_attention_prefill(const void* q, const void* k_cache, const void* v_cache, void* out,
+                           const int32_t* item_seq, const int32_t* item_tile, const int32_t* q_start,
+                           const int32_t* q_len, const int32_t* positions, const int32_t* block_table, int max_blocks,
+                           int n_items, int n_q, int n_kv, int head_dim, int page, float scale, int window,
+                           hipStream_t stream) {
+    if (n_items <= 0) return 0;
+    if (head_dim != HEAD_DIM || n_kv <= 0 || n_q % n_kv) return -1;
+    const float scale_log2e = scale * 1.4426950408889634f;
+    hipLaunchKernelGGL(attention_prefill_kernel, dim3(n_items, n_q), dim3(THREADS), 0, stream, (const bf16_t*)q,
+                       (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, item_seq, item_tile, q_start, q_len,
+                       positions, block_table, max_blocks, n_q, n_kv, page, scale_log2e, window);
+    return KIPP_LAUNCH_CHECK();
+}
+
+}  // extern "C"

@@ -162,11 +162,13 @@ def loaded_libraries() -> Dict[str, str]:
     return {k: v._name for k, v in _loaded.items()}
 
 
-def clean_stale() -> None:
-    """Remove libraries in the in-tree folder whose hash no longer matches a source."""
+def clean_stale(keep: Iterable[Tuple[str, Optional[dict]]] = ()) -> None:
+    """Remove left-over temporary files from the in-tree folder and, when `keep`
+    is given, every library that is not the current build of one of its entries."""
     folder = os.path.join(HERE, "_lib")
     if not os.path.isdir(folder):
         return
+    wanted = {os.path.basename(library_path(name, defines)[0]) for name, defines in keep}
     for f in os.listdir(folder):
-        if f.endswith(".tmp"):
+        if f.endswith(".tmp") or (wanted and f.endswith(".so") and f not in wanted):
             os.remove(os.path.join(folder, f))

@@ -14,20 +14,22 @@ __global__ void embed_kernel(const TW* __restrict__ table, const int32_t* __rest
 }
 
 // One workgroup per row.  If `delta` is given, x += delta first and the sum is
-// written back (the residual add of the block before), then
+// written back (the residual add of the block before); `delta` may come in
+// `parts` slabs [parts, rows, width] that are added in order (a product whose
+// contraction was split over workgroups), then
 // y = x * rsqrt(mean(x^2) + eps) * w   (/root/reference/src/kipp.c:2221-2231:
 // eps inside the root, (x * scale) * w).
 template <typename TD, typename TO>
 __global__ void rmsnorm_kernel(float* __restrict__ x, const TD* __restrict__ delta,
                                const float* __restrict__ weight, TO* __restrict__ out,
-                               int width, float eps) {
+                               int width, float eps, int parts, size_t part_stride) {
     __shared__ float scratch[16];
     const size_t base = (size_t)blockIdx.x * width;
     float ss = 0.0f;
     for (int i = threadIdx.x; i < width; i += blockDim.x) {
         float v = x[base + i];
         if (delta != nullptr) {
-            v += load_f(delta, base + i);
+            for (int p = 0; p < parts; ++p) v += load_f(delta, p * part_stride + base + i);
             x[base + i] = v;
         }
         ss += v * v;
@@ -41,9 +43,13 @@ __global__ void rmsnorm_kernel(float* __restrict__ x, const TD* __restrict__ del
 
 // x += delta (the last residual add when no norm follows in the same kernel).
 template <typename TD>
-__global__ void residual_add_kernel(float* __restrict__ x, const TD* __restrict__ delta, size_t n) {
+__global__ void residual_add_kernel(float* __restrict__ x, const TD* __restrict__ delta, size_t n, int parts) {
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) x[i] += load_f(delta, i);
+    if (i < n) {
+        float v = x[i];
+        for (int p = 0; p < parts; ++p) v += load_f(delta, p * n + i);
+        x[i] = v;
+    }
 }
 
 // out[t, i] = silu(gu[t, i]) * gu[t, inner + i], silu(z) = z / (1 + exp(-z))
@@ -87,11 +93,11 @@ int kipp_embed(const void* table, int table_dtype, const int32_t* tokens, float*
     return KIPP_LAUNCH_CHECK();
 }
 
-int kipp_rmsnorm(float* x, const void* delta, int delta_dtype, const float* weight, void* out, int out_dtype,
+int kipp_rmsnorm(float* x, const void* delta, int delta_dtype, int parts, const float* weight, void* out, int out_dtype,
                  int rows, int width, float eps, hipStream_t stream) {
     if (rows <= 0) return 0;
     dim3 grid(rows), block(width >= 2048 ? 512 : 256);
-#define KIPP_RN(TD, TO) hipLaunchKernelGGL((rmsnorm_kernel<TD, TO>), grid, block, 0, stream, x, (const TD*)delta, weight, (TO*)out, width, eps)
+#define KIPP_RN(TD, TO) hipLaunchKernelGGL((rmsnorm_kernel<TD, TO>), grid, block, 0, stream, x, (const TD*)delta, weight, (TO*)out, width, eps, parts, (size_t)rows * width)
     if (delta_dtype == KIPP_BF16) {
         if (out_dtype == KIPP_BF16) KIPP_RN(bf16_t, bf16_t); else KIPP_RN(bf16_t, float);
     } else {
@@ -101,13 +107,13 @@ int kipp_rmsnorm(float* x, const void* delta, int delta_dtype, const float* weig
     return KIPP_LAUNCH_CHECK();
 }
 
-int kipp_residual_add(float* x, const void* delta, int delta_dtype, size_t n, hipStream_t stream) {
+int kipp_residual_add(float* x, const void* delta, int delta_dtype, int parts, size_t n, hipStream_t stream) {
     if (n == 0) return 0;
     dim3 grid((unsigned)((n + 255) / 256)), block(256);
     if (delta_dtype == KIPP_BF16)
-        hipLaunchKernelGGL(residual_add_kernel<bf16_t>, grid, block, 0, stream, x, (const bf16_t*)delta, n);
+        hipLaunchKernelGGL(residual_add_kernel<bf16_t>, grid, block, 0, stream, x, (const bf16_t*)delta, n, parts);
     else
-        hipLaunchKernelGGL(residual_add_kernel<float>, grid, block, 0, stream, x, (const float*)delta, n);
+        hipLaunchKernelGGL(residual_add_kernel<float>, grid, block, 0, stream, x, (const float*)delta, n, parts);
     return KIPP_LAUNCH_CHECK();
 }
 

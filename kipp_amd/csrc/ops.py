@@ -88,25 +88,30 @@ def embed(table: torch.Tensor, tokens: torch.Tensor, out: torch.Tensor) -> torch
 
 def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor,
             delta: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """out = rmsnorm(x [+ delta]) * weight; with `delta`, x += delta in place."""
+    """out = rmsnorm(x [+ delta]) * weight; with `delta`, x += delta in place.
+    `delta` is [rows, width] or, in slabs that are added in order, [parts, rows, width]."""
     _dev(x, weight, out, delta)
     rows, width = x.shape
     _need(x.dtype == torch.float32 and weight.dtype == torch.float32, "rmsnorm: x and weight are float32")
     _need(weight.numel() == width and out.shape == x.shape, "rmsnorm: shapes differ")
+    parts = 1
     if delta is not None:
-        _need(delta.shape == x.shape, "rmsnorm: delta shape differs from x")
+        _need(tuple(delta.shape[-2:]) == tuple(x.shape) and delta.dim() in (2, 3), "rmsnorm: delta shape differs from x")
+        parts = delta.shape[0] if delta.dim() == 3 else 1
     fn = _fn("elementwise", "kipp_rmsnorm",
-             [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_float, _c_ptr])
-    _check(fn(_ptr(x), _ptr(delta), _code(delta) if delta is not None else F32, _ptr(weight), _ptr(out),
+             [_c_ptr, _c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_float, _c_ptr])
+    _check(fn(_ptr(x), _ptr(delta), _code(delta) if delta is not None else F32, parts, _ptr(weight), _ptr(out),
               _code(out), rows, width, float(eps), _stream()), "rmsnorm")
     return out
 
 
 def residual_add(x: torch.Tensor, delta: torch.Tensor) -> torch.Tensor:
     _dev(x, delta)
-    _need(x.dtype == torch.float32 and x.shape == delta.shape, "residual_add: float32 x and a delta of its shape")
-    fn = _fn("elementwise", "kipp_residual_add", [_c_ptr, _c_ptr, _c_int, _c_size, _c_ptr])
-    _check(fn(_ptr(x), _ptr(delta), _code(delta), x.numel(), _stream()), "residual_add")
+    _need(x.dtype == torch.float32 and tuple(delta.shape[-2:]) == tuple(x.shape) and delta.dim() in (2, 3),
+          "residual_add: float32 x and a delta of its shape (or slabs of it)")
+    parts = delta.shape[0] if delta.dim() == 3 else 1
+    fn = _fn("elementwise", "kipp_residual_add", [_c_ptr, _c_ptr, _c_int, _c_int, _c_size, _c_ptr])
+    _check(fn(_ptr(x), _ptr(delta), _code(delta), parts, x.numel(), _stream()), "residual_add")
     return x
 
 
@@ -197,7 +202,111 @@ def paged_attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
     return out
 
 
+def _attn_common(q, k_cache, v_cache, out, n_q, n_kv, head_dim, what):
+    n = q.shape[0]
+    _need(q.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and k_cache.dtype == torch.bfloat16
+          and v_cache.dtype == torch.bfloat16, f"{what}: bfloat16 queries, caches and output")
+    _need(q.shape == (n, n_q * head_dim) and out.shape == q.shape, f"{what}: q and out are [tokens, n_q d]")
+    _need(k_cache.shape == v_cache.shape and k_cache.dim() == 4 and k_cache.shape[1] == n_kv
+          and k_cache.shape[3] == head_dim, f"{what}: caches must be [pages, n_kv, page, d]")
+    _need(head_dim % 16 == 0 and 0 < head_dim <= 256 and n_q % n_kv == 0, f"{what}: head size or head counts refused")
+
+
+DECODE_SPLIT = 256      # keys per workgroup of the decode kernel (checked against the library at load)
+PREFILL_ROWS = 128      # query rows per workgroup of the prefill kernel
+
+
+def attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
+                     rows: torch.Tensor, positions: torch.Tensor, seq_of_token: torch.Tensor, block_table: torch.Tensor,
+                     n_q: int, n_kv: int, head_dim: int, scale: float, window: int, max_context: int,
+                     workspace: tuple, grid_splits: Optional[int] = None) -> torch.Tensor:
+    """Attention of single query tokens (batch rows `rows`) over their pages.
+    `max_context`: the longest context among them (sizes the grid); `workspace`:
+    (part_acc, part_ml) float32 buffers from `attention_decode_workspace`."""
+    _dev(q, k_cache, v_cache, out, rows, positions, seq_of_token, block_table, *workspace)
+    for t, name in ((rows, "rows"), (positions, "positions"), (seq_of_token, "seq_of_token"), (block_table, "block_table")):
+        _i32(t, name)
+    _attn_common(q, k_cache, v_cache, out, n_q, n_kv, head_dim, "attention_decode")
+    group = n_q // n_kv
+    _need(group <= 16, "attention_decode: more than 16 query heads per key/value head are refused")
+    n_items = rows.numel()
+    part_acc, part_ml = workspace
+    max_splits = part_ml.numel() // max(1, n_items * n_q * 2)
+    span = min(max_context, window) if window else max_context
+    need = (span + DECODE_SPLIT - 1) // DECODE_SPLIT + (1 if window else 0)
+    grid = grid_splits if grid_splits is not None else max(1, min(need, max_splits))
+    _need(part_acc.dtype == torch.float32 and part_ml.dtype == torch.float32
+          and part_acc.numel() >= n_items * n_q * max_splits * head_dim and need <= max_splits,
+          "attention_decode: workspace too small for this context")
+    defines = {"HEAD_DIM": head_dim, "GROUP": group}
+    fn = _fn("attention_decode", "kipp_attention_decode",
+             [_c_ptr] * 10 + [_c_int] * 6 + [_c_float, _c_int, _c_int, _c_int, _c_ptr], defines)
+    _check(fn(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(part_acc), _ptr(part_ml), _ptr(rows),
+              _ptr(positions), _ptr(seq_of_token), _ptr(block_table), block_table.shape[1], n_items, n_q, n_kv,
+              head_dim, k_cache.shape[2], float(scale), int(window), grid, max_splits, _stream()), "attention_decode")
+    return out
+
+
+def attention_decode_workspace(n_items: int, n_q: int, head_dim: int, max_context: int, device) -> tuple:
+    max_splits = (max_context + DECODE_SPLIT - 1) // DECODE_SPLIT + 1
+    return (torch.empty(n_items * n_q * max_splits * head_dim, dtype=torch.float32, device=device),
+            torch.empty(n_items * n_q * max_splits * 2, dtype=torch.float32, device=device))
+
+
+def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
+                      item_seq: torch.Tensor, item_tile: torch.Tensor, q_start: torch.Tensor, q_len: torch.Tensor,
+                      positions: torch.Tensor, block_table: torch.Tensor, n_q: int, n_kv: int, head_dim: int,
+                      scale: float, window: int = 0) -> torch.Tensor:
+    """Attention of prompt portions: work item i is the `item_tile[i]`-th tile
+    of PREFILL_ROWS query rows of sequence `item_seq[i]`."""
+    _dev(q, k_cache, v_cache, out, item_seq, item_tile, q_start, q_len, positions, block_table)
+    for t, name in ((item_seq, "item_seq"), (item_tile, "item_tile"), (q_start, "q_start"), (q_len, "q_len"),
+                    (positions, "positions"), (block_table, "block_table")):
+        _i32(t, name)
+    _attn_common(q, k_cache, v_cache, out, n_q, n_kv, head_dim, "attention_prefill")
+    _need(item_seq.numel() == item_tile.numel(), "attention_prefill: one tile index per work item")
+    fn = _fn("attention_prefill", "kipp_attention_prefill",
+             [_c_ptr] * 10 + [_c_int] * 6 + [_c_float, _c_int, _c_ptr], {"HEAD_DIM": head_dim})
+    _check(fn(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(item_seq), _ptr(item_tile), _ptr(q_start),
+              _ptr(q_len), _ptr(positions), _ptr(block_table), block_table.shape[1], item_seq.numel(), n_q, n_kv,
+              head_dim, k_cache.shape[2], float(scale), int(window), _stream()), "attention_prefill")
+    return out
+
+
 # --------------------------------------------------------------------------- matrix products
+
+SKINNY_MAX_ROWS = 64
+
+
+def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[parts, M, N] (float32 slabs that add up to x . w^T) for M <= 64 rows of
+    bfloat16 x against bfloat16 w [N, K]; parts = out.shape[0] splits K."""
+    _dev(x, w, out)
+    m, k = x.shape
+    n = w.shape[0]
+    _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and out.dtype == torch.float32,
+          "gemm_skinny: bfloat16 operands, float32 output")
+    _need(w.shape == (n, k) and out.dim() == 3 and tuple(out.shape[1:]) == (m, n), "gemm_skinny: shapes do not match")
+    _need(m <= SKINNY_MAX_ROWS and k % 8 == 0, "gemm_skinny: at most 64 rows and K a multiple of 8")
+    fn = _fn("gemm_skinny", "kipp_gemm_skinny", [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr])
+    _check(fn(_ptr(x), _ptr(w), _ptr(out), m, n, k, out.shape[0], _stream()), "gemm_skinny")
+    return out
+
+
+def gemm_skinny_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[M, I] (bfloat16) = silu(x . w_gate^T) * (x . w_up^T), w_gate_up = [gate; up] of [2 I, K]."""
+    _dev(x, w_gate_up, out)
+    m, k = x.shape
+    two_inner = w_gate_up.shape[0]
+    _need(x.dtype == torch.bfloat16 and w_gate_up.dtype == torch.bfloat16 and out.dtype == torch.bfloat16,
+          "gemm_skinny_swiglu: bfloat16 operands and output")
+    _need(w_gate_up.shape == (two_inner, k) and two_inner % 2 == 0 and out.shape == (m, two_inner // 2),
+          "gemm_skinny_swiglu: shapes do not match")
+    _need(m <= SKINNY_MAX_ROWS and k % 8 == 0, "gemm_skinny_swiglu: at most 64 rows and K a multiple of 8")
+    fn = _fn("gemm_skinny", "kipp_gemm_skinny_swiglu", [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr])
+    _check(fn(_ptr(x), _ptr(w_gate_up), _ptr(out), m, two_inner, k, _stream()), "gemm_skinny_swiglu")
+    return out
+
 
 def gemm_f32(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     """out[M,N] = x[M,K] . w[N,K]^T in true float32 (w float32 or bfloat16)."""

@@ -1,0 +1,44 @@
+"""Which libraries a model needs, and the list that `build()` compiles ahead
+of time (the sizes of the benchmark, of the tests and of the smoke run)."""
+from __future__ import annotations
+
+from typing import Iterable, List, Optional, Tuple
+
+Spec = Tuple[str, Optional[dict]]
+
+GENERIC: List[Spec] = [(name, None) for name in
+                       ("elementwise", "rope_kv", "attention_generic", "gemm_f32", "gemm_skinny", "sampling")]
+
+
+def attention_variants(head_dim: int, group: int) -> List[Spec]:
+    out: List[Spec] = [("attention_prefill", {"HEAD_DIM": head_dim})]
+    if group <= 16:
+        out.append(("attention_decode", {"HEAD_DIM": head_dim, "GROUP": group}))
+    return out
+
+
+def model_variants(spec, dtype: str) -> List[Spec]:
+    """Everything the model `spec` launches under `dtype`."""
+    out = list(GENERIC)
+    if dtype == "bfloat16":
+        for layer in spec.layers:
+            for _, part in layer.parts:
+                if getattr(part, "kind", None) == "attention":
+                    for v in attention_variants(part.head_dim, part.num_heads // part.num_kv_heads):
+                        if v not in out:
+                            out.append(v)
+    return out
+
+
+# (head_dim, query heads per key/value head) of the benchmark shape, the tiny
+# configurations, the toy model of the tests and the kernel tests
+PREBUILT_ATTENTION = [(128, 4), (16, 2), (32, 4), (16, 3), (48, 3), (64, 1), (32, 16), (256, 4), (80, 3), (256, 2), (16, 1)]
+
+
+def prebuilt() -> List[Spec]:
+    out = list(GENERIC)
+    for head_dim, group in PREBUILT_ATTENTION:
+        for v in attention_variants(head_dim, group):
+            if v not in out:
+                out.append(v)
+    return out

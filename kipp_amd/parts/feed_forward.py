@@ -7,6 +7,8 @@
 """
 from __future__ import annotations
 
+import torch
+
 from .base import ParamSpec, register
 
 
@@ -28,7 +30,6 @@ class GatedMLP:
         }
 
     def load(self, tensors):
-        import torch
         g, u = tensors["gate_proj.weight"], tensors["up_proj.weight"]
         if g.dtype != u.dtype:
             g, u = g.float(), u.float()
@@ -37,6 +38,11 @@ class GatedMLP:
 
     def forward(self, x, batch=None):
         rt = self.rt
-        gate_up = rt.linear(x, self.w_gate_up)
-        act = rt.ops.swiglu(gate_up, rt.empty((x.shape[0], self.spec.intermediate_size), rt.act_dtype))
-        return rt.linear(act, self.w_down)
+        rows, inner = x.shape[0], self.spec.intermediate_size
+        act = rt.empty((rows, inner), rt.act_dtype)
+        if (self.w_gate_up.dtype == x.dtype == torch.bfloat16 and rows <= rt.ops.SKINNY_MAX_ROWS
+                and x.shape[1] % 8 == 0):
+            rt.ops.gemm_skinny_swiglu(x, self.w_gate_up, act)      # both products and the activation in one kernel
+        else:
+            rt.ops.swiglu(rt.linear(x, self.w_gate_up), act)
+        return rt.linear(act, self.w_down, slabs=True)

@@ -80,8 +80,30 @@ class Attention:
             batch.positions, batch.seq_of_token, table, s.num_heads, s.num_kv_heads, s.head_dim,
             self.q_norm, self.k_norm, s.qk_norm_eps if s.qk_norm_eps is not None else 0.0,
             inv_freq, rotary_dim, write_kv=cache.writable)
-        out = rt.ops.paged_attention_generic(
-            q, cache.k, cache.v, rt.empty((n, s.q_dim), rt.act_dtype),
-            batch.positions, batch.seq_of_token, table, s.num_heads, s.num_kv_heads, s.head_dim,
-            self.scale, s.window or 0)
-        return rt.linear(out, self.w_o)
+        out = rt.empty((n, s.q_dim), rt.act_dtype)
+        group = s.num_heads // s.num_kv_heads
+        if rt.dtype == "bfloat16" and group <= 16:
+            if batch.n_prefill_items:
+                rt.ops.attention_prefill(q, cache.k, cache.v, out, batch.prefill_seq, batch.prefill_tile, batch.q_start,
+                                         batch.q_len, batch.positions, table, s.num_heads, s.num_kv_heads, s.head_dim,
+                                         self.scale, s.window or 0)
+            if batch.n_decode:
+                rt.ops.attention_decode(q, cache.k, cache.v, out, batch.decode_rows, batch.positions, batch.seq_of_token,
+                                        table, s.num_heads, s.num_kv_heads, s.head_dim, self.scale, s.window or 0,
+                                        batch.max_decode_ctx, self._workspace(batch))
+        else:
+            # the float32 path, and group sizes the split kernel refuses
+            rt.ops.paged_attention_generic(q, cache.k, cache.v, out, batch.positions, batch.seq_of_token, table,
+                                           s.num_heads, s.num_kv_heads, s.head_dim, self.scale, s.window or 0)
+        return rt.linear(out, self.w_o, slabs=True)
+
+    def _workspace(self, batch):
+        """Partial results of the split decode kernel, kept while they are large enough."""
+        s = self.spec
+        key = (batch.n_decode, batch.max_decode_ctx)
+        ws = batch.host.get("decode_workspace")
+        if ws is None or ws[0] != key:
+            ws = (key, self.rt.ops.attention_decode_workspace(batch.n_decode, s.num_heads, s.head_dim,
+                                                              batch.max_decode_ctx, self.rt.device))
+            batch.host["decode_workspace"] = ws
+        return ws[1]

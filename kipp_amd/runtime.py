@@ -56,8 +56,11 @@ class Runtime:
         return torch.empty(shape, dtype=dtype, device=self.device)
 
     # -- matrix product ------------------------------------------------------
-    def linear(self, x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
-        """float32 [M, N] = x [M, K] . w [N, K]^T."""
+    def linear(self, x: torch.Tensor, w: torch.Tensor, slabs: bool = False) -> torch.Tensor:
+        """float32 [M, N] = x [M, K] . w [N, K]^T.  With `slabs` the result may come
+        as [parts, M, N] whose sum over parts is the product (few rows against a
+        weight with few output rows: the contraction is split over workgroups and
+        the consumer adds the slabs in order)."""
         m = x.shape[0]
         n = w.shape[0]
         if w.dtype == torch.float32:
@@ -66,6 +69,15 @@ class Runtime:
             return self.ops.gemm_f32(x, w, self.empty((m, n), torch.float32))
         if x.dtype != torch.bfloat16:
             x = self.ops.cast(x, self.empty(x.shape, torch.bfloat16))
+        k = x.shape[1]
+        if m <= self.ops.SKINNY_MAX_ROWS and k % 8 == 0:
+            # few rows: our own kernel streams the weight once
+            parts = 1
+            if slabs:
+                tiles, steps = (n + 15) // 16, (k + 31) // 32
+                parts = max(1, min(-(-768 // tiles), steps // 32))
+            y = self.ops.gemm_skinny(x, w, self.empty((parts, m, n), torch.float32))
+            return y if slabs and parts > 1 else y[0]
         # bfloat16 x bfloat16 with float32 accumulation: the library product
         if self._mm_out_f32 is None:
             try:

@@ -257,3 +257,154 @@ def test_argmax(vocab, rows):
         logits[0, 7] = logits[0, vocab - 3] = 50.0   # a tie: the lowest index wins
     got = ops.argmax(_t(logits), torch.empty(rows, dtype=torch.int32, device=DEV)).cpu().numpy()
     assert np.array_equal(got, np.argmax(logits, axis=1))
+
+
+# ----------------------------------------------------------------------------- bfloat16 kernels
+
+def _attention_reference(q, k, v, table, positions, seq_of, n_q, n_kv, d, page, window):
+    t = len(positions)
+    scale = 1.0 / math.sqrt(d)
+    ref = np.zeros((t, n_q, d))
+    qd = q.double().numpy().reshape(t, n_q, d)
+    cache = {}
+    for i, (pos, s) in enumerate(zip(positions, seq_of)):
+        if s not in cache or cache[s][0].shape[0] < pos + 1:
+            n = max(p for p, ss in zip(positions, seq_of) if ss == s) + 1
+            cache[s] = (_gather(k, table[s], n, page), _gather(v, table[s], n, page))
+        ks, vs = cache[s]
+        lo = max(0, pos - window + 1) if window else 0
+        for h in range(n_q):
+            g = h // (n_q // n_kv)
+            p = plain.softmax((ks[lo:pos + 1, g] @ qd[i, h]) * scale)
+            ref[i, h] = p @ vs[lo:pos + 1, g]
+    return ref
+
+
+@pytest.mark.parametrize("n_q,n_kv,d,page", [(32, 8, 128, 16), (6, 2, 48, 8), (4, 4, 64, 4), (16, 1, 32, 16), (8, 2, 256, 32), (2, 1, 16, 16)])
+@pytest.mark.parametrize("window", [0, 300])
+def test_attention_decode(n_q, n_kv, d, page, window):
+    ops = _ops()
+    rng = np.random.default_rng(n_q * 7 + d + window)
+    seq_lens = [1, 70, 300, 700, 256, 257, 513]
+    table, k, v = _paged_setup(rng, seq_lens, n_kv, d, page, torch.bfloat16)
+    # a batch in which the decode tokens are not the first rows: rows 1, 3, 4, ... of a larger batch
+    t = len(seq_lens) + 3
+    rows = [1, 3, 4, 5, 7, 8, 9]
+    positions = [0] * t
+    seq_of = [0] * t
+    for r, (s, n) in zip(rows, enumerate(seq_lens)):
+        positions[r], seq_of[r] = n - 1, s
+    q = torch.tensor(rng.normal(size=(t, n_q * d)), dtype=torch.bfloat16)
+    out = torch.zeros(t, n_q * d, dtype=torch.bfloat16, device=DEV)
+    ws = ops.attention_decode_workspace(len(rows), n_q, d, max(seq_lens), DEV)
+    ops.attention_decode(q.to(DEV), k.to(DEV), v.to(DEV), out, _t(rows, torch.int32), _t(positions, torch.int32),
+                         _t(seq_of, torch.int32), _t(table, torch.int32), n_q, n_kv, d, 1 / math.sqrt(d), window,
+                         max(seq_lens), ws)
+    ref = _attention_reference(q[rows], k, v, table, [positions[r] for r in rows], [seq_of[r] for r in rows],
+                               n_q, n_kv, d, page, window)
+    got = out.float().cpu().numpy().reshape(t, n_q, d)
+    assert _rel(got[rows], ref) < 1e-5
+    untouched = [r for r in range(t) if r not in rows]
+    assert not got[untouched].any()
+
+
+@pytest.mark.parametrize("n_q,n_kv,d,page", [(32, 8, 128, 16), (6, 2, 48, 8), (4, 4, 64, 4), (3, 1, 80, 16), (2, 1, 256, 32), (2, 2, 16, 8)])
+@pytest.mark.parametrize("window", [0, 100])
+def test_attention_prefill(n_q, n_kv, d, page, window):
+    ops = _ops()
+    rng = np.random.default_rng(n_q * 11 + d + window)
+    seq_lens = [130, 64, 300, 5, 257]      # tokens in the cache after this step
+    q_lens = [130, 2, 100, 5, 129]         # this step's portion of each
+    table, k, v = _paged_setup(rng, seq_lens, n_kv, d, page, torch.bfloat16)
+    positions, seq_of, q_start = [], [], []
+    for s, (n, ql) in enumerate(zip(seq_lens, q_lens)):
+        q_start.append(len(positions))
+        positions += list(range(n - ql, n))
+        seq_of += [s] * ql
+    t = len(positions)
+    items = [(s, tile) for s, ql in enumerate(q_lens) for tile in range(-(-ql // ops.PREFILL_ROWS))]
+    q = torch.tensor(rng.normal(size=(t, n_q * d)), dtype=torch.bfloat16)
+    out = ops.attention_prefill(q.to(DEV), k.to(DEV), v.to(DEV), torch.zeros(t, n_q * d, dtype=torch.bfloat16, device=DEV),
+                                _t([i[0] for i in items], torch.int32), _t([i[1] for i in items], torch.int32),
+                                _t(q_start, torch.int32), _t(q_lens, torch.int32), _t(positions, torch.int32),
+                                _t(table, torch.int32), n_q, n_kv, d, 1 / math.sqrt(d), window)
+    ref = _attention_reference(q, k, v, table, positions, seq_of, n_q, n_kv, d, page, window)
+    got = out.float().cpu().numpy().reshape(t, n_q, d)
+    for i in range(t):
+        assert _rel(got[i], ref[i]) < 2e-5, f"row {i}: position {positions[i]} of sequence {seq_of[i]}"
+
+
+@pytest.mark.parametrize("kernel", ["decode", "prefill"])
+def test_one_far_key_among_hundreds_decides(kernel):
+    """Random values would hide a key that is skipped or read from the wrong
+    page: here one far key has by far the largest score, so the output must be
+    its value row."""
+    ops = _ops()
+    n_q, n_kv, d, page = 8, 2, 128, 16
+    rng = np.random.default_rng(3)
+    n = 777
+    for far in (0, 15, 16, 255, 256, 511, 640, 776):
+        table, k, v = _paged_setup(rng, [n], n_kv, d, page, torch.bfloat16)
+        qv = rng.normal(size=(1, n_q * d))
+        q = torch.tensor(qv, dtype=torch.bfloat16)
+        kk = k.clone()
+        for g in range(n_kv):   # the far key of head g points along query head 4 g
+            kk[table[0, far // page], g, far % page, :] = 6.0 * q[0].reshape(n_q, d)[4 * g]
+        if kernel == "decode":
+            ws = ops.attention_decode_workspace(1, n_q, d, n, DEV)
+            out = ops.attention_decode(q.to(DEV), kk.to(DEV), v.to(DEV), torch.zeros(1, n_q * d, dtype=torch.bfloat16, device=DEV),
+                                       _t([0], torch.int32), _t([n - 1], torch.int32), _t([0], torch.int32),
+                                       _t(table, torch.int32), n_q, n_kv, d, 1 / math.sqrt(d), 0, n, ws)
+        else:
+            q2 = torch.cat([torch.zeros(1, n_q * d, dtype=torch.bfloat16), q])
+            out = ops.attention_prefill(q2.to(DEV), kk.to(DEV), v.to(DEV), torch.zeros(2, n_q * d, dtype=torch.bfloat16, device=DEV),
+                                        _t([0], torch.int32), _t([0], torch.int32), _t([0], torch.int32), _t([2], torch.int32),
+                                        _t([n - 2, n - 1], torch.int32), _t(table, torch.int32), n_q, n_kv, d,
+                                        1 / math.sqrt(d), 0)[1:]
+        got = out.float().cpu().numpy().reshape(n_q, d)
+        for g in range(n_kv):
+            want = v[table[0, far // page], g, far % page, :].float().numpy()
+            assert np.abs(got[4 * g] - want).max() < 0.02, f"far key {far}, head {4 * g}"
+
+
+@pytest.mark.parametrize("m", [1, 8, 16, 17, 33, 64])
+@pytest.mark.parametrize("n,k,parts", [(16, 8, 1), (77, 80, 1), (2560, 200, 3), (509, 2560, 2), (6144, 2560, 1)])
+def test_gemm_skinny(m, n, k, parts):
+    ops = _ops()
+    rng = np.random.default_rng(m + n)
+    x = torch.tensor(rng.normal(size=(m, k)), dtype=torch.bfloat16)
+    w = torch.tensor(rng.normal(size=(n, k)), dtype=torch.bfloat16)
+    out = ops.gemm_skinny(x.to(DEV), w.to(DEV), torch.full((parts, m, n), 7.0, device=DEV))
+    ref = x.double().numpy() @ w.double().numpy().T
+    assert _rel(out.sum(dim=0).cpu().numpy(), ref) < 1e-11
+    xi = torch.tensor(rng.integers(-3, 4, size=(m, k)), dtype=torch.bfloat16)
+    wi = torch.tensor(rng.integers(-3, 4, size=(n, k)), dtype=torch.bfloat16)
+    out = ops.gemm_skinny(xi.to(DEV), wi.to(DEV), torch.empty(parts, m, n, device=DEV)).sum(dim=0)
+    assert np.array_equal(out.cpu().numpy(), xi.float().numpy() @ wi.float().numpy().T)
+
+
+@pytest.mark.parametrize("m,inner,k", [(1, 16, 32), (8, 200, 80), (64, 9728, 2560), (5, 77, 8)])
+def test_gemm_skinny_swiglu(m, inner, k):
+    ops = _ops()
+    rng = np.random.default_rng(m + inner)
+    x = torch.tensor(rng.normal(size=(m, k)), dtype=torch.bfloat16)
+    w = torch.tensor(rng.normal(size=(2 * inner, k)) / math.sqrt(k), dtype=torch.bfloat16)
+    out = ops.gemm_skinny_swiglu(x.to(DEV), w.to(DEV), torch.empty(m, inner, dtype=torch.bfloat16, device=DEV))
+    gu = x.double().numpy() @ w.double().numpy().T
+    ref = plain.silu(gu[:, :inner]) * gu[:, inner:]
+    assert _rel(out.float().cpu().numpy(), ref) < 1e-5
+
+
+def test_rmsnorm_adds_slabs_in_order():
+    ops = _ops()
+    rng = np.random.default_rng(8)
+    x = rng.normal(size=(3, 80)).astype(np.float32)
+    parts = rng.normal(size=(4, 3, 80)).astype(np.float32)
+    w = np.ones(80, dtype=np.float32)
+    xd = _t(x)
+    got = ops.rmsnorm(xd, _t(w), 1e-6, torch.empty(3, 80, device=DEV), delta=_t(parts))
+    total = x.copy()
+    for p in parts:
+        total = total + p
+    assert np.array_equal(xd.cpu().numpy(), total)
+    assert _rel(got.cpu().numpy(), plain.rms_norm(total, w, 1e-6)) < 1e-12
