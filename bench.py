@@ -1,0 +1,189 @@
+"""Decode and prefill throughput of the Qwen3-4B-shaped model with random
+bfloat16 weights on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+One JSON line: `value` is decoded tokens a second at batch 8 (a step is one
+decode step of the whole batch, tokens chosen greedily on the device and fed
+back), with the prefill of one 2,048-token prompt, the decode step's HBM
+roofline and the batch-1 / batch-64 points beside it.  Peaks are MI355X's
+published ones: HBM 8 TB/s, dense bf16 MFMA 2.5 PFLOP/s.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+PEAK_FLOPS = {"bf16": 2.5e15, "fp16": 2.5e15, "fp8": 5.0e15, "fp32": 157.3e12}
+PREFILL_TOKENS = 2048
+
+
+def log(msg):
+    print(f"bench: {msg}", file=sys.stderr, flush=True)
+
+
+def model_numbers(cfg, layers):
+    """Weight elements a decode step reads and flops per token of the products."""
+    h, q, kv, i, v = cfg.hidden_size, cfg.q_dim, cfg.kv_dim, cfg.intermediate_size, cfg.vocab_size
+    per_layer = h * (q + 2 * kv) + q * h + 3 * h * i
+    head = v * h
+    kv_bytes_per_token = layers * 2 * kv * 2
+    return per_layer, head, kv_bytes_per_token
+
+
+def prefill_flops(cfg, layers, n):
+    per_layer, head, _ = model_numbers(cfg, layers)
+    gemm = 2.0 * n * per_layer * layers + 2.0 * head          # the head runs on one row
+    attn = layers * 4.0 * cfg.q_dim * (n * (n + 1) / 2.0)     # causal half of QK^T and PV
+    return gemm + attn
+
+
+def fill(engine, ids, prompt_len, vocab, seed, chunk=2048):
+    """Put a random prompt of `prompt_len` tokens into the cache for every id;
+    returns the first decode token of each (greedy)."""
+    import torch
+    from kipp_amd.engine import StepEntry
+    gen = torch.Generator().manual_seed(seed)
+    first = {}
+    for rid in ids:
+        toks = torch.randint(0, vocab, (prompt_len,), generator=gen).tolist()
+        for at in range(0, prompt_len, chunk):
+            part = toks[at:at + chunk]
+            last = at + chunk >= prompt_len
+            logits = engine.step([StepEntry(rid, part, [len(part) - 1] if last else [])])
+        first[rid] = int(logits.argmax(dim=-1)[0])
+    return first
+
+
+def decode_run(engine, ids, tokens, steps, warmup):
+    """`warmup` untimed and `steps` timed decode steps of all `ids` together."""
+    import torch
+    from kipp_amd.engine import StepEntry
+    cur = [tokens[r] for r in ids]
+
+    def one():
+        nonlocal cur
+        logits = engine.step([StepEntry(r, [t], [0]) for r, t in zip(ids, cur)])
+        cur = engine.rt.ops.argmax(logits, engine.rt.empty((len(ids),), torch.int32)).cpu().tolist()
+    for _ in range(warmup):
+        one()
+    torch.cuda.synchronize()
+    start = time.perf_counter()
+    for _ in range(steps):
+        one()
+    torch.cuda.synchronize()
+    return time.perf_counter() - start
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--shape", default="qwen3-4b")
+    ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the shape has (named in config)")
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--prompt", type=int, default=2048)
+    ap.add_argument("--points", default="1,64", help="further decode batch sizes")
+    ap.add_argument("--no-prefill", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench: this engine runs on one GPU; --gpus {args.gpus} is not supported")
+        return 2
+
+    import torch
+    from kipp_amd.config import parse_config, shape_config
+    from kipp_amd.engine import Engine, StepEntry, random_model
+    from kipp_amd.runtime import Runtime
+
+    config = shape_config(args.shape)
+    full_layers = config["num_hidden_layers"]
+    layers = args.layers or full_layers
+    config["num_hidden_layers"] = layers
+    _, cfg = parse_config(config)
+    context = cfg.max_position_embeddings
+    points = [int(b) for b in args.points.split(",") if b]
+    batches = sorted(set([args.batch] + points))
+    max_batch = max(batches)
+    page = 16
+    log(f"building {args.shape} ({layers} of {full_layers} layers) with random bfloat16 weights on the device ...")
+    t0 = time.perf_counter()
+    rt = Runtime("bfloat16")
+    model = random_model(config, seed=0, runtime=rt)
+    tokens_per_request = args.prompt + args.warmup + args.steps + 8
+    engine = Engine(model, page_size=page, num_pages=max_batch * (-(-tokens_per_request // page)) + 4,
+                    max_requests=max_batch, share_prefixes=False)
+    torch.cuda.synchronize()
+    log(f"model and cache ready in {time.perf_counter() - t0:.1f} s")
+
+    per_layer, head, kv_per_token = model_numbers(cfg, layers)
+    weight_bytes = 2.0 * (per_layer * layers + head)
+
+    # ---- prefill of one 2,048-token prompt (logits of the last place)
+    prefill = None
+    if not args.no_prefill:
+        gen = torch.Generator().manual_seed(1)
+        times = []
+        for i in range(5):
+            toks = torch.randint(0, cfg.vocab_size, (PREFILL_TOKENS,), generator=gen).tolist()
+            torch.cuda.synchronize()
+            start = time.perf_counter()
+            engine.step([StepEntry("prefill", toks, [PREFILL_TOKENS - 1])])
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - start)
+            engine.close("prefill")
+        best = sorted(times[1:])[len(times[1:]) // 2]
+        flops = prefill_flops(cfg, layers, PREFILL_TOKENS)
+        prefill = {"value": round(PREFILL_TOKENS / best, 1), "tokens": PREFILL_TOKENS, "ms": round(best * 1e3, 3),
+                   "frac": round(flops / best / PEAK_FLOPS["bf16"], 4)}
+        log(f"prefill {PREFILL_TOKENS} tokens: {best * 1e3:.2f} ms, {PREFILL_TOKENS / best:.0f} tok/s")
+
+    # ---- decode at every batch size; the requests of the largest batch are filled once
+    ids = [f"d{i}" for i in range(max_batch)]
+    log(f"filling {max_batch} requests with {args.prompt}-token prompts ...")
+    t0 = time.perf_counter()
+    first = fill(engine, ids, args.prompt, cfg.vocab_size, seed=2)
+    log(f"filled in {time.perf_counter() - t0:.1f} s")
+    results = {}
+    for b in batches:
+        steps = args.steps if b == args.batch else max(8, args.steps // 2)
+        warmup = args.warmup if b == args.batch else max(2, args.warmup // 2)
+        before = engine.length(ids[0])
+        seconds = decode_run(engine, ids[:b], first, steps, warmup)
+        ctx_mid = before + warmup + steps / 2.0
+        results[b] = {"tok_s": b * steps / seconds, "ms": seconds / steps * 1e3, "steps": steps, "warmup": warmup,
+                      "bytes": weight_bytes + b * ctx_mid * kv_per_token}
+        log(f"decode batch {b}: {seconds / steps * 1e3:.3f} ms/step, {b * steps / seconds:.0f} tok/s, "
+            f"{results[b]['bytes'] / (seconds / steps) / 1e9:.0f} GB/s")
+        # the requests beyond this batch keep their caches; the first ones simply go on
+
+    main_r = results[args.batch]
+    achieved = main_r["bytes"] / (main_r["ms"] / 1e3) / 1e9
+    line = {
+        "metric": "decode tok/s at batch 8 (Qwen3-4B-shaped, bf16, random weights)",
+        "value": round(main_r["tok_s"], 1), "unit": "tok/s", "n_gpus": 1, "steps": main_r["steps"],
+        "warmup": main_r["warmup"], "ms_per_step": round(main_r["ms"], 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"model": args.shape, "layers": layers, "layers_of_shape": full_layers, "hidden": cfg.hidden_size,
+                   "q_heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
+                   "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size, "tied": cfg.tie_word_embeddings,
+                   "global_batch": args.batch, "seq_len": context, "prompt_tokens": args.prompt, "kv_page": page,
+                   "parallelism": "none", "weights": "random N(0,0.02) seed 0"},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4)},
+        "points": {f"decode_b{b}": round(results[b]["tok_s"], 1) for b in batches if b != args.batch},
+    }
+    if prefill is not None:
+        line["prefill"] = prefill
+    print(json.dumps(line), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

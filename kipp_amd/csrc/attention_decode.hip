@@ -58,8 +58,10 @@ __global__ void __launch_bounds__(THREADS) attention_decode_kernel(
     __shared__ float s_scores[GROUP][SPLIT + 4];
     __shared__ float s_red[WAVES][GROUP][HEAD_DIM];
     __shared__ float s_m[GROUP], s_l[GROUP];
+    __shared__ int s_page[SPLIT + 2];                 // page of every key of the split (any page size)
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l16 = lane & 15, h = lane >> 4;
     const int kvh = blockIdx.y;
     const int row = rows[blockIdx.z];                 // row of this query token in the batch
@@ -72,47 +74,45 @@ __global__ void __launch_bounds__(THREADS) attention_decode_kernel(
     const int base = split * SPLIT;
     const int32_t* table = block_table + (size_t)seq_of_token[row] * max_blocks;
 
+    // Pages first, once, into LDS: the loads of keys and values below then depend on
+    // nothing that is still in flight and can all be issued back to back.  Keys beyond
+    // the query's position read the last valid page (finite values, masked later).
+    if (tid < SPLIT) s_page[tid] = table[min(base + tid, pos) / page];
+    __syncthreads();
+
     // ---- the GROUP queries as B operand: lane (slot l16, quarter h) holds q[slot][32 t + 8 h .. + 7]
     Frag qf[KSTEPS];
 #pragma unroll
     for (int t = 0; t < KSTEPS; ++t) {
-        qf[t].u = make_uint4(0, 0, 0, 0);
-        const int dcol = 32 * t + 8 * h;
-        if (l16 < GROUP && dcol < HEAD_DIM)
-            qf[t].u = *(const uint4*)(q + ((size_t)row * n_q + (size_t)kvh * GROUP + l16) * HEAD_DIM + dcol);
+        const int dcol = min(32 * t + 8 * h, HEAD_DIM - 8);
+        qf[t].u = *(const uint4*)(q + ((size_t)row * n_q + (size_t)kvh * GROUP + min(l16, GROUP - 1)) * HEAD_DIM + dcol);
     }
 
-    // ---- scores: each wave takes BLOCKS_PER_WAVE blocks of 16 keys
+    // ---- scores: each wave takes BLOCKS_PER_WAVE blocks of 16 keys; every load is unconditional
     Frag kf[BLOCKS_PER_WAVE][KSTEPS];
 #pragma unroll
     for (int b = 0; b < BLOCKS_PER_WAVE; ++b) {
-        const int s = base + (wave * BLOCKS_PER_WAVE + b) * 16 + l16;
-        const bool valid = s >= lo && s <= pos;
-        const bf16_t* k_row = nullptr;
-        if (valid) k_row = k_cache + (((size_t)table[s / page] * n_kv + kvh) * page + s % page) * HEAD_DIM;
+        const int kl = (wave * BLOCKS_PER_WAVE + b) * 16 + l16;
+        const int s = min(base + kl, pos);
+        const bf16_t* k_row = k_cache + (((size_t)s_page[kl] * n_kv + kvh) * page + s % page) * HEAD_DIM;
 #pragma unroll
-        for (int t = 0; t < KSTEPS; ++t) {
-            const int dcol = 32 * t + 8 * h;
-            kf[b][t].u = make_uint4(0, 0, 0, 0);
-            if (valid && dcol < HEAD_DIM) kf[b][t].u = *(const uint4*)(k_row + dcol);
-        }
+        for (int t = 0; t < KSTEPS; ++t) kf[b][t].u = *(const uint4*)(k_row + min(32 * t + 8 * h, HEAD_DIM - 8));
     }
     // ---- values are asked for now, so that they arrive while the scores are worked on
     Frag vf[KEYS_PER_GROUP][CHUNKS_PER_LANE];
     const int kg = wave * 4 + h;                      // this lane group's keys: base + kg + 16 i
 #pragma unroll
     for (int i = 0; i < KEYS_PER_GROUP; ++i) {
-        const int s = base + kg + 16 * i;
-        const bool valid = s >= lo && s <= pos;
-        const bf16_t* v_row = nullptr;
-        if (valid) v_row = v_cache + (((size_t)table[s / page] * n_kv + kvh) * page + s % page) * HEAD_DIM;
+        const int kl = kg + 16 * i;
+        const int s = min(base + kl, pos);
+        const bf16_t* v_row = v_cache + (((size_t)s_page[kl] * n_kv + kvh) * page + s % page) * HEAD_DIM;
 #pragma unroll
-        for (int c = 0; c < CHUNKS_PER_LANE; ++c) {
-            const int chunk = l16 + 16 * c;
-            vf[i][c].u = make_uint4(0, 0, 0, 0);
-            if (valid && chunk < CHUNKS) vf[i][c].u = *(const uint4*)(v_row + chunk * 8);
-        }
+        for (int c = 0; c < CHUNKS_PER_LANE; ++c) vf[i][c].u = *(const uint4*)(v_row + min(l16 + 16 * c, CHUNKS - 1) * 8);
     }
+    // operands that reach beyond the head size or the group were read from clamped addresses: zero them
+#pragma unroll
+    for (int t = 0; t < KSTEPS; ++t)
+        if (32 * t + 8 * h >= HEAD_DIM || l16 >= GROUP) qf[t].u = make_uint4(0, 0, 0, 0);
 #pragma unroll
     for (int b = 0; b < BLOCKS_PER_WAVE; ++b) {
         f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};

@@ -40,6 +40,9 @@
 #define K_PITCH (HEAD_DIM + 8)                 // bf16 elements per key row in LDS
 #define V_PITCH (BN + 4)                       // bf16 elements per value column in LDS
 #define DCHUNKS (HEAD_DIM / 8)
+#define K_LOADS ((BN * DCHUNKS + THREADS - 1) / THREADS)
+#define V_TASKS (((BN / 2) * DCHUNKS + THREADS - 1) / THREADS)
+#define MAX_PAGES 2048
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
@@ -63,6 +66,7 @@ __global__ void __launch_bounds__(THREADS) attention_prefill_kernel(
     int window) {
     __shared__ __attribute__((aligned(16))) bf16_t Ks[BN * K_PITCH];
     __shared__ __attribute__((aligned(16))) bf16_t Vt[DP * V_PITCH];
+    __shared__ int s_page[MAX_PAGES];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int l32 = lane & 31, hh = lane >> 5;
@@ -104,34 +108,69 @@ __global__ void __launch_bounds__(THREADS) attention_prefill_kernel(
 
     const int tile_lo = (window > 0 ? max(0, pos0 - window + 1) : 0) / BN;
     const int tile_hi = last_pos / BN;
+
+    // The pages of the keys this workgroup reads, once, into LDS: the loads of a tile then
+    // depend on nothing in flight and are issued back to back.  (A sequence with more pages
+    // than fit is read through the table in global memory instead.)
+    const int first_block = (tile_lo * BN) / page, last_block = last_pos / page;
+    const bool pages_in_lds = last_block - first_block < MAX_PAGES;
+    if (pages_in_lds)
+        for (int i = tid; i <= last_block - first_block; i += THREADS) s_page[i] = table[first_block + i];
+    __syncthreads();
+    auto page_of = [&](int s) {   // s is clamped to the last key of the portion: beyond it the values are masked
+        const int block = min(s, last_pos) / page;
+        return pages_in_lds ? s_page[block - first_block] : table[block];
+    };
+
+    // registers for one tile: keys (K_LOADS 16-byte chunks a thread), values (2 chunks for each of V_TASKS key pairs)
+    uint4 k_reg[K_LOADS];
+    Frag v_reg[V_TASKS][2];
+    auto fetch_tile = [&](int key0) {
+#pragma unroll
+        for (int i = 0; i < K_LOADS; ++i) {
+            const int c = min(tid + i * THREADS, BN * DCHUNKS - 1);
+            const int key = c / DCHUNKS, chunk = c % DCHUNKS;
+            const int s = min(key0 + key, last_pos);
+            k_reg[i] = *(const uint4*)(k_cache + (((size_t)page_of(s) * n_kv + kvh) * page + s % page) * HEAD_DIM + chunk * 8);
+        }
+#pragma unroll
+        for (int i = 0; i < V_TASKS; ++i) {
+            const int c = min(tid + i * THREADS, (BN / 2) * DCHUNKS - 1);
+            const int pair = c % (BN / 2), chunk = c / (BN / 2);
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                const int s = min(key0 + 2 * pair + e, last_pos);
+                v_reg[i][e].u = *(const uint4*)(v_cache + (((size_t)page_of(s) * n_kv + kvh) * page + s % page) * HEAD_DIM + chunk * 8);
+            }
+        }
+    };
+    auto store_tile = [&]() {
+        // keys: [key][d]; values transposed: [d][key], two keys to a 32-bit word
+#pragma unroll
+        for (int i = 0; i < K_LOADS; ++i) {
+            const int c = tid + i * THREADS;
+            if (c < BN * DCHUNKS) *(uint4*)(Ks + (c / DCHUNKS) * K_PITCH + (c % DCHUNKS) * 8) = k_reg[i];
+        }
+#pragma unroll
+        for (int i = 0; i < V_TASKS; ++i) {
+            const int c = tid + i * THREADS;
+            if (c < (BN / 2) * DCHUNKS) {
+                const int pair = c % (BN / 2), chunk = c / (BN / 2);
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    *(uint32_t*)(Vt + (chunk * 8 + j) * V_PITCH + 2 * pair) =
+                        (uint32_t)v_reg[i][0].h[j] | ((uint32_t)v_reg[i][1].h[j] << 16);
+            }
+        }
+    };
+
+    fetch_tile(tile_lo * BN);
     for (int kt = tile_lo; kt <= tile_hi; ++kt) {
         const int key0 = kt * BN;
         __syncthreads();   // the tile before has been read by every wave
-        // ---- keys: [key][d], 16 bytes a thread
-        for (int c = tid; c < BN * DCHUNKS; c += THREADS) {
-            const int key = c / DCHUNKS, chunk = c % DCHUNKS;
-            const int s = key0 + key;
-            uint4 val = make_uint4(0, 0, 0, 0);
-            if (s <= last_pos)
-                val = *(const uint4*)(k_cache + (((size_t)table[s / page] * n_kv + kvh) * page + s % page) * HEAD_DIM + chunk * 8);
-            *(uint4*)(Ks + key * K_PITCH + chunk * 8) = val;
-        }
-        // ---- values, transposed: [d][key]; a thread takes two keys and 8 columns
-        for (int c = tid; c < (BN / 2) * DCHUNKS; c += THREADS) {
-            const int pair = c % (BN / 2), chunk = c / (BN / 2);
-            Frag a, b;
-            a.u = make_uint4(0, 0, 0, 0);
-            b.u = make_uint4(0, 0, 0, 0);
-            const int s = key0 + 2 * pair;
-            if (s <= last_pos)
-                a.u = *(const uint4*)(v_cache + (((size_t)table[s / page] * n_kv + kvh) * page + s % page) * HEAD_DIM + chunk * 8);
-            if (s + 1 <= last_pos)
-                b.u = *(const uint4*)(v_cache + (((size_t)table[(s + 1) / page] * n_kv + kvh) * page + (s + 1) % page) * HEAD_DIM + chunk * 8);
-#pragma unroll
-            for (int j = 0; j < 8; ++j)
-                *(uint32_t*)(Vt + (chunk * 8 + j) * V_PITCH + 2 * pair) = (uint32_t)a.h[j] | ((uint32_t)b.h[j] << 16);
-        }
+        store_tile();
         __syncthreads();
+        if (kt < tile_hi) fetch_tile(key0 + BN);   // on its way while this tile is worked on
         if (!wave_active) continue;
 
         // ---- S^T = K Q^T for the two 32-key halves of the tile

@@ -41,6 +41,62 @@ __global__ void rmsnorm_kernel(float* __restrict__ x, const TD* __restrict__ del
     }
 }
 
+// The same for widths that are a multiple of 4 and at most 1024 * CH: the row stays in
+// registers between the sum of squares and the scaling (one read of x, 16-byte accesses).
+__device__ __forceinline__ float4 load4(const float* p, size_t i4) { return ((const float4*)p)[i4]; }
+__device__ __forceinline__ float4 load4(const bf16_t* p, size_t i4) {
+    const uint2 r = ((const uint2*)p)[i4];
+    return make_float4(__uint_as_float(r.x << 16), __uint_as_float(r.x & 0xffff0000u),
+                       __uint_as_float(r.y << 16), __uint_as_float(r.y & 0xffff0000u));
+}
+__device__ __forceinline__ void store4(float* p, size_t i4, float4 v) { ((float4*)p)[i4] = v; }
+__device__ __forceinline__ void store4(bf16_t* p, size_t i4, float4 v) {
+    uint2 r;
+    r.x = (uint32_t)f32_to_bf16(v.x) | ((uint32_t)f32_to_bf16(v.y) << 16);
+    r.y = (uint32_t)f32_to_bf16(v.z) | ((uint32_t)f32_to_bf16(v.w) << 16);
+    ((uint2*)p)[i4] = r;
+}
+
+template <typename TD, typename TO, int CH>
+__global__ void __launch_bounds__(256) rmsnorm_rows_kernel(float* __restrict__ x, const TD* __restrict__ delta,
+                                                           const float* __restrict__ weight, TO* __restrict__ out,
+                                                           int width, float eps, int parts, size_t part_stride) {
+    __shared__ float scratch[16];
+    const int n4 = width / 4;
+    const size_t base4 = (size_t)blockIdx.x * n4;
+    float4 v[CH];
+    float ss = 0.0f;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const int i = threadIdx.x + c * 256;
+        v[c] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        if (i < n4) {
+            v[c] = load4(x, base4 + i);
+            if (delta != nullptr) {
+                for (int p = 0; p < parts; ++p) {
+                    const float4 d = load4(delta, p * (part_stride / 4) + base4 + i);
+                    v[c].x += d.x;
+                    v[c].y += d.y;
+                    v[c].z += d.z;
+                    v[c].w += d.w;
+                }
+                store4(x, base4 + i, v[c]);
+            }
+        }
+        ss += v[c].x * v[c].x + v[c].y * v[c].y + v[c].z * v[c].z + v[c].w * v[c].w;
+    }
+    ss = block_sum(ss, scratch);
+    const float scale = 1.0f / sqrtf(ss / (float)width + eps);
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const int i = threadIdx.x + c * 256;
+        if (i < n4) {
+            const float4 w = load4(weight, (size_t)i);
+            store4(out, base4 + i, make_float4(v[c].x * scale * w.x, v[c].y * scale * w.y, v[c].z * scale * w.z, v[c].w * scale * w.w));
+        }
+    }
+}
+
 // x += delta (the last residual add when no norm follows in the same kernel).
 template <typename TD>
 __global__ void residual_add_kernel(float* __restrict__ x, const TD* __restrict__ delta, size_t n, int parts) {
@@ -80,6 +136,24 @@ __global__ void gather_rows_kernel(const float* __restrict__ x, const int32_t* _
     for (int i = threadIdx.x; i < width; i += blockDim.x) out[dst + i] = x[src + i];
 }
 
+template <typename TD, typename TO>
+static void launch_rmsnorm(float* x, const void* delta, const float* weight, void* out, int rows, int width, float eps,
+                           int parts, hipStream_t stream) {
+    const size_t stride = (size_t)rows * width;
+    const int n4 = width / 4;
+    if ((width & 3) == 0 && n4 <= 256 * 8) {
+#define KIPP_RV(CH) hipLaunchKernelGGL((rmsnorm_rows_kernel<TD, TO, CH>), dim3(rows), dim3(256), 0, stream, x, (const TD*)delta, weight, (TO*)out, width, eps, parts, stride)
+        if (n4 <= 256) KIPP_RV(1);
+        else if (n4 <= 512) KIPP_RV(2);
+        else if (n4 <= 1024) KIPP_RV(4);
+        else KIPP_RV(8);
+#undef KIPP_RV
+    } else {
+        hipLaunchKernelGGL((rmsnorm_kernel<TD, TO>), dim3(rows), dim3(width >= 2048 ? 512 : 256), 0, stream, x,
+                           (const TD*)delta, weight, (TO*)out, width, eps, parts, stride);
+    }
+}
+
 extern "C" {
 
 int kipp_embed(const void* table, int table_dtype, const int32_t* tokens, float* out,
@@ -96,14 +170,13 @@ int kipp_embed(const void* table, int table_dtype, const int32_t* tokens, float*
 int kipp_rmsnorm(float* x, const void* delta, int delta_dtype, int parts, const float* weight, void* out, int out_dtype,
                  int rows, int width, float eps, hipStream_t stream) {
     if (rows <= 0) return 0;
-    dim3 grid(rows), block(width >= 2048 ? 512 : 256);
-#define KIPP_RN(TD, TO) hipLaunchKernelGGL((rmsnorm_kernel<TD, TO>), grid, block, 0, stream, x, (const TD*)delta, weight, (TO*)out, width, eps, parts, (size_t)rows * width)
     if (delta_dtype == KIPP_BF16) {
-        if (out_dtype == KIPP_BF16) KIPP_RN(bf16_t, bf16_t); else KIPP_RN(bf16_t, float);
+        if (out_dtype == KIPP_BF16) launch_rmsnorm<bf16_t, bf16_t>(x, delta, weight, out, rows, width, eps, parts, stream);
+        else launch_rmsnorm<bf16_t, float>(x, delta, weight, out, rows, width, eps, parts, stream);
     } else {
-        if (out_dtype == KIPP_BF16) KIPP_RN(float, bf16_t); else KIPP_RN(float, float);
+        if (out_dtype == KIPP_BF16) launch_rmsnorm<float, bf16_t>(x, delta, weight, out, rows, width, eps, parts, stream);
+        else launch_rmsnorm<float, float>(x, delta, weight, out, rows, width, eps, parts, stream);
     }
-#undef KIPP_RN
     return KIPP_LAUNCH_CHECK();
 }
 

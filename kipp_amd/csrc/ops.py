@@ -278,18 +278,26 @@ def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
 SKINNY_MAX_ROWS = 64
 
 
-def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
-    """out[parts, M, N] (float32 slabs that add up to x . w^T) for M <= 64 rows of
-    bfloat16 x against bfloat16 w [N, K]; parts = out.shape[0] splits K."""
-    _dev(x, w, out)
+def gemm_skinny_ok(m: int, k: int) -> bool:
+    """Shapes the few-rows kernel takes: at most 64 rows, K a multiple of 8 and at least 32."""
+    return 0 < m <= SKINNY_MAX_ROWS and k % 8 == 0 and k >= 32
+
+
+def gemm_skinny(x: torch.Tensor, w: torch.Tensor, max_parts: int = 1) -> torch.Tensor:
+    """float32 [parts, M, N] whose sum over parts is x . w^T, for M <= 64 rows of
+    bfloat16 x against bfloat16 w [N, K].  parts <= max_parts is chosen from the
+    shape (1 when the weight has many rows)."""
+    _dev(x, w)
     m, k = x.shape
     n = w.shape[0]
-    _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and out.dtype == torch.float32,
-          "gemm_skinny: bfloat16 operands, float32 output")
-    _need(w.shape == (n, k) and out.dim() == 3 and tuple(out.shape[1:]) == (m, n), "gemm_skinny: shapes do not match")
-    _need(m <= SKINNY_MAX_ROWS and k % 8 == 0, "gemm_skinny: at most 64 rows and K a multiple of 8")
+    _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm_skinny: bfloat16 operands")
+    _need(w.shape == (n, k), "gemm_skinny: shapes do not match")
+    _need(gemm_skinny_ok(m, k), "gemm_skinny: at most 64 rows, K a multiple of 8 and at least 32")
+    lib = build.library("gemm_skinny")
+    parts = lib.kipp_gemm_skinny_parts(n, k, int(max_parts))
+    out = torch.empty((parts, m, n), dtype=torch.float32, device=x.device)
     fn = _fn("gemm_skinny", "kipp_gemm_skinny", [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr])
-    _check(fn(_ptr(x), _ptr(w), _ptr(out), m, n, k, out.shape[0], _stream()), "gemm_skinny")
+    _check(fn(_ptr(x), _ptr(w), _ptr(out), m, n, k, int(max_parts), _stream()), "gemm_skinny")
     return out
 
 
@@ -302,7 +310,7 @@ def gemm_skinny_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tens
           "gemm_skinny_swiglu: bfloat16 operands and output")
     _need(w_gate_up.shape == (two_inner, k) and two_inner % 2 == 0 and out.shape == (m, two_inner // 2),
           "gemm_skinny_swiglu: shapes do not match")
-    _need(m <= SKINNY_MAX_ROWS and k % 8 == 0, "gemm_skinny_swiglu: at most 64 rows and K a multiple of 8")
+    _need(gemm_skinny_ok(m, k), "gemm_skinny_swiglu: at most 64 rows, K a multiple of 8 and at least 32")
     fn = _fn("gemm_skinny", "kipp_gemm_skinny_swiglu", [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr])
     _check(fn(_ptr(x), _ptr(w_gate_up), _ptr(out), m, two_inner, k, _stream()), "gemm_skinny_swiglu")
     return out

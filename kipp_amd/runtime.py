@@ -69,15 +69,10 @@ class Runtime:
             return self.ops.gemm_f32(x, w, self.empty((m, n), torch.float32))
         if x.dtype != torch.bfloat16:
             x = self.ops.cast(x, self.empty(x.shape, torch.bfloat16))
-        k = x.shape[1]
-        if m <= self.ops.SKINNY_MAX_ROWS and k % 8 == 0:
+        if self.ops.gemm_skinny_ok(m, x.shape[1]):
             # few rows: our own kernel streams the weight once
-            parts = 1
-            if slabs:
-                tiles, steps = (n + 15) // 16, (k + 31) // 32
-                parts = max(1, min(-(-768 // tiles), steps // 32))
-            y = self.ops.gemm_skinny(x, w, self.empty((parts, m, n), torch.float32))
-            return y if slabs and parts > 1 else y[0]
+            y = self.ops.gemm_skinny(x, w, max_parts=8 if slabs else 1)
+            return y if y.shape[0] > 1 else y[0]
         # bfloat16 x bfloat16 with float32 accumulation: the library product
         if self._mm_out_f32 is None:
             try:

@@ -368,22 +368,35 @@ def test_one_far_key_among_hundreds_decides(kernel):
 
 
 @pytest.mark.parametrize("m", [1, 8, 16, 17, 33, 64])
-@pytest.mark.parametrize("n,k,parts", [(16, 8, 1), (77, 80, 1), (2560, 200, 3), (509, 2560, 2), (6144, 2560, 1)])
-def test_gemm_skinny(m, n, k, parts):
+@pytest.mark.parametrize("n,k,max_parts", [(16, 32, 1), (77, 80, 1), (2560, 200, 8), (2560, 9728, 8), (509, 2560, 2), (6144, 2560, 1),
+                                           (40, 4096, 8)])
+def test_gemm_skinny(m, n, k, max_parts):
     ops = _ops()
     rng = np.random.default_rng(m + n)
     x = torch.tensor(rng.normal(size=(m, k)), dtype=torch.bfloat16)
     w = torch.tensor(rng.normal(size=(n, k)), dtype=torch.bfloat16)
-    out = ops.gemm_skinny(x.to(DEV), w.to(DEV), torch.full((parts, m, n), 7.0, device=DEV))
+    out = ops.gemm_skinny(x.to(DEV), w.to(DEV), max_parts)
+    assert 1 <= out.shape[0] <= max_parts and tuple(out.shape[1:]) == (m, n)
     ref = x.double().numpy() @ w.double().numpy().T
     assert _rel(out.sum(dim=0).cpu().numpy(), ref) < 1e-11
     xi = torch.tensor(rng.integers(-3, 4, size=(m, k)), dtype=torch.bfloat16)
     wi = torch.tensor(rng.integers(-3, 4, size=(n, k)), dtype=torch.bfloat16)
-    out = ops.gemm_skinny(xi.to(DEV), wi.to(DEV), torch.empty(parts, m, n, device=DEV)).sum(dim=0)
+    out = ops.gemm_skinny(xi.to(DEV), wi.to(DEV), max_parts).sum(dim=0)
     assert np.array_equal(out.cpu().numpy(), xi.float().numpy() @ wi.float().numpy().T)
 
 
-@pytest.mark.parametrize("m,inner,k", [(1, 16, 32), (8, 200, 80), (64, 9728, 2560), (5, 77, 8)])
+def test_gemm_skinny_refuses_what_it_cannot_do():
+    ops = _ops()
+    x = torch.zeros(2, 8, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(ops.KernelError):
+        ops.gemm_skinny(x, torch.zeros(16, 8, dtype=torch.bfloat16, device=DEV))        # K below 32
+    with pytest.raises(ops.KernelError):
+        ops.gemm_skinny(torch.zeros(65, 64, dtype=torch.bfloat16, device=DEV), torch.zeros(16, 64, dtype=torch.bfloat16, device=DEV))
+    with pytest.raises(ops.KernelError):
+        ops.gemm_skinny(torch.zeros(2, 36, dtype=torch.bfloat16, device=DEV), torch.zeros(16, 36, dtype=torch.bfloat16, device=DEV))
+
+
+@pytest.mark.parametrize("m,inner,k", [(1, 16, 32), (8, 200, 80), (64, 9728, 2560), (5, 77, 40), (33, 100, 2560)])
 def test_gemm_skinny_swiglu(m, inner, k):
     ops = _ops()
     rng = np.random.default_rng(m + inner)
