@@ -17,6 +17,8 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 from typing import Dict, List, Optional, Sequence, Tuple
 
+import numpy as np
+
 from .needs import KVNeed, StateNeed
 from .pool import PagePool
 
@@ -48,6 +50,7 @@ class RequestCache:
     tables: List[List[int]] = field(default_factory=list)   # per group: page id per block, -1 once given back
     adopted: List[int] = field(default_factory=list)        # per group: leading pages taken from the index
     adopted_tokens: int = 0
+    rows: List[np.ndarray] = field(default_factory=list)    # per group: the table as the device sees it (int32, given-back pages 0)
 
 
 class CacheGroup:
@@ -133,7 +136,8 @@ class CacheManager:
         slot = self.free_slots.pop()
         for tensor in self.states.values():
             tensor[slot].zero_()
-        req = RequestCache(request_id, slot, tables=[[] for _ in self.groups], adopted=[0 for _ in self.groups])
+        req = RequestCache(request_id, slot, tables=[[] for _ in self.groups], adopted=[0 for _ in self.groups],
+                           rows=[np.zeros(self.max_blocks, dtype=np.int32) for _ in self.groups])
         if self.share and prompt is not None and self.groups:
             matches = [g.pool.prefix_match(prompt) for g in self.groups]
             keep = min(len(pages) for pages, _ in matches)
@@ -141,6 +145,7 @@ class CacheManager:
                 for page in pages[keep:]:
                     g.pool.release(page)
                 req.tables[g.index] = list(pages[:keep])
+                req.rows[g.index][:keep] = pages[:keep]
                 req.adopted[g.index] = keep
             req.adopted_tokens = keep * self.page_size
             req.length = req.adopted_tokens
@@ -174,6 +179,7 @@ class CacheManager:
                     if page is None:
                         self._rollback(claimed)
                         raise OutOfPages(f"group {g.index}: no free page for request {req.id!r}")
+                    req.rows[g.index][len(req.tables[g.index])] = page
                     req.tables[g.index].append(page)
                     claimed.append((req, g.index, page))
 
@@ -181,6 +187,7 @@ class CacheManager:
         for req, gi, page in reversed(claimed):
             popped = req.tables[gi].pop()
             assert popped == page
+            req.rows[gi][len(req.tables[gi])] = 0
             self.groups[gi].pool.release(page)
 
     def commit(self, req: RequestCache, tokens: Sequence[int]) -> None:
@@ -198,6 +205,7 @@ class CacheManager:
                 if table[block] >= 0:
                     g.pool.release(table[block])
                     table[block] = -1
+                    req.rows[g.index][block] = 0
 
     def close(self, request_id) -> None:
         """The request ended: publish its full pages where sharing is on, give

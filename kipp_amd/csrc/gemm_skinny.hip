@@ -5,7 +5,8 @@
 //
 // A wave owns 16 rows of W and a slice of K.  It keeps a ring of DEPTH steps
 // (32 columns each) in registers: while the matrix core works on step s, the
-// loads of steps s+1 .. s+DEPTH are on their way.  The 4 waves of a workgroup
+// loads of steps s+1 .. s+DEPTH are on their way (plain loads: streaming hints made this
+// access pattern slower in measurements).  The 4 waves of a workgroup
 // are KW slices of K times 4/KW row tiles; slices are added in LDS in slice
 // order.  `parts` > 1 splits K over workgroups as well (for products with few
 // output rows): part p writes its own [M, N] slab and the consumer adds the
@@ -35,7 +36,7 @@ union Frag {
 template <int MT, bool SWIGLU, int KW, int DEPTH>
 __global__ void __launch_bounds__(THREADS) gemm_skinny_kernel(
     const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, float* __restrict__ Y, bf16_t* __restrict__ act,
-    int M, int N, int K, int steps_per_part) {
+    int M, int N, int K) {
     constexpr int NT = SWIGLU ? 2 : 1;
     constexpr int TW = WAVES / KW;                   // row tiles of a workgroup
     __shared__ float red[KW > 1 ? WAVES : 1][NT][MT][256];
@@ -46,12 +47,15 @@ __global__ void __launch_bounds__(THREADS) gemm_skinny_kernel(
     const int n0 = (blockIdx.x * TW + tile_in_wg) * 16;
     const int part = blockIdx.y;
     const int inner = SWIGLU ? N / 2 : N;            // rows of one of the stacked matrices
-    const int full_steps = K / 32;                   // steps of 32 columns; a rest of 8, 16 or 24 comes last
-    const int part_begin = min(full_steps, part * steps_per_part);
-    const int part_end = min(full_steps, part_begin + steps_per_part);
-    const int per_slice = (part_end - part_begin + KW - 1) / KW;
-    const int s_begin = min(part_end, part_begin + slice * per_slice);
-    const int s_end = min(part_end, s_begin + per_slice);
+    // The contraction in groups of DEPTH steps of 32 columns.  Groups are dealt out evenly to
+    // the gridDim.y * KW slices; what is left beyond the last whole group (fewer than DEPTH
+    // steps and a rest of 8, 16 or 24 columns) goes to the very last slice.
+    const int full_steps = K / 32;
+    const int groups = full_steps / DEPTH;
+    const int slices = (int)gridDim.y * KW;
+    const int my_slice = part * KW + slice;
+    const int g_begin = (int)((long long)groups * my_slice / slices);
+    const int g_end = (int)((long long)groups * (my_slice + 1) / slices);
 
     const bool row_ok = n0 + l16 < inner;
     const int row = row_ok ? n0 + l16 : 0;           // clamped: the loads stay in bounds, the result is dropped
@@ -69,12 +73,11 @@ __global__ void __launch_bounds__(THREADS) gemm_skinny_kernel(
         for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
 
     Frag wf[DEPTH][NT], xf[DEPTH][MT];
-    // A step beyond the slice reads the slice's last step again (in bounds) and is never used.
     // No value is touched between its load and its product: the loads stay in flight.
-    auto fetch = [&](int u, int s) {
-        const int k = 32 * min(s, s_end - 1);
+    auto fetch = [&](int u, int step) {
+        const int k = 32 * step;
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) wf[u][nt].u = __builtin_nontemporal_load((const u32x4*)(w_row[nt] + k));
+        for (int nt = 0; nt < NT; ++nt) wf[u][nt].u = *(const u32x4*)(w_row[nt] + k);
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) xf[u][mt].u = *(const u32x4*)(x_row[mt] + k);
     };
@@ -86,47 +89,40 @@ __global__ void __launch_bounds__(THREADS) gemm_skinny_kernel(
                 acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u][nt].v, xf[u][mt].v, acc[nt][mt], 0, 0, 0);
     };
 
-    if (s_begin < s_end) {
+    if (g_begin < g_end) {
 #pragma unroll
-        for (int u = 0; u < DEPTH; ++u) fetch(u, s_begin + u);
-        int s = s_begin;
-        for (; s + 2 * DEPTH <= s_end; s += DEPTH) {     // every step used and every step fetched is inside the slice
+        for (int u = 0; u < DEPTH; ++u) fetch(u, g_begin * DEPTH + u);
+        for (int g = g_begin; g + 1 < g_end; ++g) {      // while step s is multiplied, step s + DEPTH is fetched
 #pragma unroll
             for (int u = 0; u < DEPTH; ++u) {
                 multiply(u);
-                fetch(u, s + DEPTH + u);
+                fetch(u, (g + 1) * DEPTH + u);
             }
         }
 #pragma unroll
-        for (int u = 0; u < DEPTH; ++u) {
-            if (s + u < s_end) multiply(u);
-            fetch(u, s + DEPTH + u);
-        }
-        s += DEPTH;
-#pragma unroll
-        for (int u = 0; u < DEPTH; ++u)
-            if (s + u < s_end) multiply(u);
+        for (int u = 0; u < DEPTH; ++u) multiply(u);
     }
-    // the rest of K beyond the last full step, by the wave that owns the end of the contraction
-    if ((K & 31) != 0 && part == (int)gridDim.y - 1 && slice == KW - 1) {
-        const int k = 32 * full_steps;
-        const bool ok = k + 8 * h < K;
-        Frag w_t[NT], x_t[MT];
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-            w_t[nt].u = (u32x4){0u, 0u, 0u, 0u};
-            if (ok) w_t[nt].u = *(const u32x4*)(w_row[nt] + k);
+    // what is left of K, by the last slice: whole steps one at a time, then the rest with a mask
+    if (my_slice == slices - 1) {
+        for (int step = groups * DEPTH; step < full_steps; ++step) {
+            fetch(0, step);
+            multiply(0);
         }
+        if ((K & 31) != 0) {
+            const int k = 32 * full_steps;
+            const bool ok = k + 8 * h < K;
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-            x_t[mt].u = (u32x4){0u, 0u, 0u, 0u};
-            if (ok) x_t[mt].u = *(const u32x4*)(x_row[mt] + k);
+            for (int nt = 0; nt < NT; ++nt) {
+                wf[0][nt].u = (u32x4){0u, 0u, 0u, 0u};
+                if (ok) wf[0][nt].u = *(const u32x4*)(w_row[nt] + k);
+            }
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                xf[0][mt].u = (u32x4){0u, 0u, 0u, 0u};
+                if (ok) xf[0][mt].u = *(const u32x4*)(x_row[mt] + k);
+            }
+            multiply(0);
         }
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt)
-                acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_t[nt].v, x_t[mt].v, acc[nt][mt], 0, 0, 0);
     }
     // tokens beyond M and rows beyond N were computed from clamped addresses and are dropped below
 
@@ -189,14 +185,12 @@ template <bool SWIGLU, int KW>
 static int launch_kw(const bf16_t* X, const bf16_t* W, float* Y, bf16_t* act, int M, int N, int K, int parts,
                      hipStream_t stream) {
     const int inner = SWIGLU ? N / 2 : N;
-    const int full_steps = K / 32;
-    const int steps_per_part = (full_steps + parts - 1) / parts;
     const int tiles = (inner + 15) / 16;
     constexpr int TW = WAVES / KW;
     dim3 grid((tiles + TW - 1) / TW, parts), block(THREADS);
     const int mt = (M + 15) / 16;
 #define KIPP_SK(MT, D) \
-    hipLaunchKernelGGL((gemm_skinny_kernel<MT, SWIGLU, KW, D>), grid, block, 0, stream, X, W, Y, act, M, N, K, steps_per_part)
+    hipLaunchKernelGGL((gemm_skinny_kernel<MT, SWIGLU, KW, D>), grid, block, 0, stream, X, W, Y, act, M, N, K)
     switch (mt) {
         case 1: KIPP_SK(1, 8); break;
         case 2: KIPP_SK(2, 8); break;
@@ -219,13 +213,14 @@ static int launch(const bf16_t* X, const bf16_t* W, float* Y, bf16_t* act, int M
     }
 }
 
-// How the contraction is split: `kw` slices inside a workgroup and `parts`
-// across workgroups, so that about 1500 waves stream the weight and each has
-// at least 16 steps.  A function of the shape only, never of the data.
-static void plan(int tiles, int total_steps, int max_parts, int* kw, int* parts) {
-    int want = (1536 + tiles - 1) / tiles;                 // slices per tile to reach ~1536 waves
-    const int by_steps = total_steps / 16 > 0 ? total_steps / 16 : 1;
-    if (want > by_steps) want = by_steps;
+// How the contraction is split: `kw` slices inside a workgroup and `parts` across workgroups,
+// so that about 2500 waves stream the weight (short products gain more from many waves than
+// from long pipelines) and each slice has at least one whole group of 8 steps.  A function of
+// the shape only, never of the data.
+static void plan(int tiles, int K, int max_parts, int* kw, int* parts) {
+    const int groups = K / 32 / 8 > 0 ? K / 32 / 8 : 1;
+    int want = (2560 + tiles - 1) / tiles;
+    if (want > groups) want = groups;
     if (want >= 4) {
         *kw = 4;
         *parts = want / 4;
@@ -245,7 +240,7 @@ extern "C" {
 // Slabs the product of this shape comes in when the caller allows up to `max_parts`.
 int kipp_gemm_skinny_parts(int N, int K, int max_parts) {
     int kw, parts;
-    plan((N + 15) / 16, (K + 31) / 32, max_parts, &kw, &parts);
+    plan((N + 15) / 16, K, max_parts, &kw, &parts);
     return parts;
 }
 
@@ -255,7 +250,7 @@ int kipp_gemm_skinny(const void* X, const void* W, float* Y, int M, int N, int K
     if (M <= 0 || N <= 0) return 0;
     if (M > 64 || K <= 0 || (K & 7) || max_parts <= 0) return -1;
     int kw, parts;
-    plan((N + 15) / 16, (K + 31) / 32, max_parts, &kw, &parts);
+    plan((N + 15) / 16, K, max_parts, &kw, &parts);
     return launch<false>((const bf16_t*)X, (const bf16_t*)W, Y, nullptr, M, N, K, parts, kw, stream);
 }
 
@@ -264,7 +259,7 @@ int kipp_gemm_skinny_swiglu(const void* X, const void* W, void* act, int M, int 
     if (M <= 0 || two_inner <= 0) return 0;
     if (M > 64 || K <= 0 || (K & 7) || (two_inner & 1)) return -1;
     int kw, parts;
-    plan((two_inner / 2 + 15) / 16, (K + 31) / 32, 1, &kw, &parts);
+    plan((two_inner / 2 + 15) / 16, K, 1, &kw, &parts);
     return launch<true>((const bf16_t*)X, (const bf16_t*)W, nullptr, (bf16_t*)act, M, two_inner, K, 1, kw, stream);
 }
 

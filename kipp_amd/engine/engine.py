@@ -16,12 +16,14 @@ import torch
 from ..cache import CacheManager, OutOfPages
 from ..runtime import Runtime
 from .batch import StepEntry, build_batch
+from .graphs import DecodeGraphs
 from .model import Model, load_model
 
 
 class Engine:
     def __init__(self, model: Model, page_size: int = 16, num_pages: Optional[int] = None,
-                 max_tokens: Optional[int] = None, max_requests: int = 64, share_prefixes: bool = True):
+                 max_tokens: Optional[int] = None, max_requests: int = 64, share_prefixes: bool = True,
+                 use_graphs: bool = True):
         """The pool of every cache group has `num_pages` pages, or as many as
         hold `max_tokens` tokens."""
         if num_pages is None:
@@ -33,6 +35,7 @@ class Engine:
         self.vocab_size = model.spec.vocab_size
         self.cache = CacheManager(model.kv_needs(), model.state_needs(), page_size, num_pages, max_requests,
                                   model.spec.max_position, runtime=self.rt, share_prefixes=share_prefixes)
+        self.graphs = DecodeGraphs(self) if use_graphs else None
 
     @classmethod
     def from_folder(cls, model_dir: str, dtype: str = "bfloat16", device: str = "cuda:0", **kw) -> "Engine":
@@ -77,8 +80,11 @@ class Engine:
             for rid in opened:
                 self.cache.close(rid)
             raise
-        batch = build_batch(entries, requests, len(self.cache.groups), self.rt.device)
-        logits = self.model.forward(batch, self.cache)
+        if self.graphs is not None and self.graphs.applies(entries):
+            logits = self.graphs.run(entries, requests)     # a static buffer: read it before the next step
+        else:
+            batch = build_batch(entries, requests, len(self.cache.groups), self.rt.device)
+            logits = self.model.forward(batch, self.cache)
         for r, e in zip(requests, entries):
             self.cache.commit(r, e.tokens)
         return logits

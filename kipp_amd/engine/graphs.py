@@ -1,0 +1,136 @@
+"""Decode steps as HIP graphs.
+
+A step in which every entry brings one token launches a few hundred small
+kernels; recorded once into a HIP graph and replayed, the launches cost the
+host almost nothing.  A graph is kept for each (number of entries, context
+bucket): shapes, grids and buffer addresses of a decode step depend on nothing
+else.  What changes from step to step (tokens, positions, slots, block
+tables) lives in one static int32 buffer that is overwritten before a replay.
+
+A graph holds our own kernels only: nothing that reads back to the host, no
+library call, no memset node.  A model with a part that does not declare
+`graph_safe`, or a step that went to a library product, runs eagerly instead.
+"""
+from __future__ import annotations
+
+import gc
+import weakref
+from typing import Dict, Optional, Sequence, Tuple
+
+import numpy as np
+import torch
+
+from .batch import StepBatch
+
+CONTEXT_BUCKET = 1024
+
+
+class DecodeGraph:
+    def __init__(self, engine, n_seqs: int, max_context: int):
+        cache = engine.cache
+        rt = engine.rt
+        self.n = n = n_seqs
+        self.groups = len(cache.groups)
+        self.max_blocks = cache.max_blocks
+        self.max_context = max_context
+        table_ints = self.groups * n * self.max_blocks
+        # [tokens | positions | ctx_len | slots | tables | arange | ones]
+        self.layout = {"tokens": 0, "positions": n, "ctx_len": 2 * n, "slots": 3 * n, "tables": 4 * n}
+        var_ints = 4 * n + table_ints
+        total = var_ints + 2 * n
+        self.var_ints = var_ints
+        self.host = torch.zeros(total, dtype=torch.int32).pin_memory()
+        self.host_np = self.host.numpy()
+        self.host_np[var_ints:var_ints + n] = np.arange(n, dtype=np.int32)
+        self.host_np[var_ints + n:] = 1
+        self.dev = torch.zeros(total, dtype=torch.int32, device=rt.device)
+        self.dev.copy_(self.host)
+        d = self.dev
+        arange = d[var_ints:var_ints + n]
+        ones = d[var_ints + n:]
+        tables = {g: d[4 * n + g * n * self.max_blocks:4 * n + (g + 1) * n * self.max_blocks].view(n, self.max_blocks)
+                  for g in range(self.groups)}
+        self.batch = StepBatch(
+            n_tokens=n, n_seqs=n, n_want=n, tokens=d[0:n], positions=d[n:2 * n], seq_of_token=arange, q_start=arange,
+            q_len=ones, ctx_len=d[2 * n:3 * n], slots=d[3 * n:4 * n], want_rows=arange, block_tables=tables,
+            decode_rows=arange, prefill_seq=d[0:0], prefill_tile=d[0:0], n_decode=n, n_prefill_items=0,
+            max_decode_ctx=max_context, max_q_len=1, max_ctx_len=max_context,
+            host={"q_start": list(range(n)), "q_len": [1] * n})
+        self.graph: Optional[torch.cuda.CUDAGraph] = None
+        self.logits: Optional[torch.Tensor] = None
+        self.copied: Optional[torch.cuda.Event] = None
+
+    def fill(self, entries, requests) -> None:
+        n, h = self.n, self.host_np
+        if self.copied is not None:
+            self.copied.synchronize()     # the copy of the step before has left the pinned buffer
+        h[0:n] = [int(e.tokens[0]) for e in entries]
+        lengths = np.fromiter((r.length for r in requests), dtype=np.int32, count=n)
+        h[n:2 * n] = lengths
+        h[2 * n:3 * n] = lengths + 1
+        h[3 * n:4 * n] = [r.slot for r in requests]
+        at = 4 * n
+        for g in range(self.groups):
+            block = h[at:at + n * self.max_blocks].reshape(n, self.max_blocks)
+            for i, r in enumerate(requests):
+                block[i] = r.rows[g]
+            at += n * self.max_blocks
+        self.dev[:self.var_ints].copy_(self.host[:self.var_ints], non_blocking=True)
+        self.copied = torch.cuda.Event()
+        self.copied.record()
+
+    def run(self, engine, entries, requests) -> torch.Tensor:
+        self.fill(entries, requests)
+        if self.graph is None:
+            # the first step with this shape runs eagerly (it also makes every workspace the
+            # kernels keep); if nothing in it went to a library, the same launches are then
+            # recorded for the steps to come
+            before = engine.rt.library_products
+            logits = engine.model.forward(self.batch, engine.cache)
+            if engine.rt.library_products != before:
+                return logits
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            # nothing may be freed on the device while the stream records: the collector stays
+            # off until the recording ends (it runs once before, inside torch.cuda.graph)
+            was_enabled = gc.isenabled()
+            gc.disable()
+            try:
+                with torch.cuda.graph(graph):
+                    self.logits = engine.model.forward(self.batch, engine.cache)
+            finally:
+                if was_enabled:
+                    gc.enable()
+            self.graph = graph
+            return logits
+        self.graph.replay()
+        return self.logits.clone()        # the graph's own output buffer is overwritten by the next replay
+
+
+class DecodeGraphs:
+    """The graphs of one engine, made when a shape is first seen."""
+
+    def __init__(self, engine):
+        self._engine = weakref.ref(engine)     # no cycle: an engine and its graphs go away together, at once
+        self.graphs: Dict[Tuple[int, int], DecodeGraph] = {}
+        model = engine.model
+        self.possible = all(getattr(b, "graph_safe", False) for b in model.blocks) and all(
+            getattr(p, "graph_safe", False) for p in (model.embedding, model.final_norm, model.head))
+        self.replays = 0
+
+    def applies(self, entries: Sequence) -> bool:
+        return (self.possible and 0 < len(entries) <= 64
+                and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries))
+
+    def run(self, entries, requests) -> torch.Tensor:
+        engine = self._engine()
+        cache = engine.cache
+        longest = max(r.length for r in requests) + 1
+        bucket = min(-(-longest // CONTEXT_BUCKET) * CONTEXT_BUCKET, max(cache.max_position, 1))
+        key = (len(entries), bucket)
+        graph = self.graphs.get(key)
+        if graph is None:
+            graph = self.graphs[key] = DecodeGraph(engine, len(entries), bucket)
+        if graph.graph is not None:
+            self.replays += 1
+        return graph.run(engine, entries, requests)

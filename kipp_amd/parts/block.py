@@ -25,6 +25,7 @@ class PreNormBlock:
         self.rt = runtime
         self.parts = {role: build_part(cat, layer_spec.part(role), runtime) for role, cat in self.roles}
         self.mixer = self.parts["mixer"]
+        self.graph_safe = all(getattr(part, "graph_safe", False) for part in self.parts.values())
 
     def forward(self, x, pending, batch, cache, state):
         act = self.rt.act_dtype

@@ -8,6 +8,8 @@ from .base import ParamSpec, register
 class Embedding:
     """x[t] = E[token_t], widened to float32, no scaling (/root/reference/src/kipp.c:2579-2585)."""
 
+    graph_safe = True   # forward launches kernels only: no host reads, no data-dependent launches
+
     def __init__(self, spec, runtime):
         self.spec = spec
         self.rt = runtime
@@ -29,6 +31,8 @@ class Embedding:
 class Head:
     """logits = W x, float32, no bias (/root/reference/src/kipp.c:2660-2661).  A tied
     head has no tensor of its own and uses the embedding table."""
+
+    graph_safe = True   # forward launches kernels only: no host reads, no data-dependent launches
 
     def __init__(self, spec, runtime):
         self.spec = spec

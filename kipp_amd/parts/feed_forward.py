@@ -16,6 +16,8 @@ from .base import ParamSpec, register
 class GatedMLP:
     """delta = W_down (silu(W_gate x) * (W_up x))  (/root/reference/src/kipp.c:2633-2653)."""
 
+    graph_safe = True   # forward launches kernels only: no host reads, no data-dependent launches
+
     def __init__(self, spec, runtime):
         self.spec = spec
         self.rt = runtime

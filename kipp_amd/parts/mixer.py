@@ -26,6 +26,8 @@ class Attention:
     (/root/reference/src/kipp.c:2950-2993).  Query head h reads key/value head
     h // (n_q / n_kv)."""
 
+    graph_safe = True   # forward launches kernels only: no host reads, no data-dependent launches
+
     def __init__(self, spec, runtime):
         self.spec = spec
         self.rt = runtime

@@ -14,6 +14,8 @@ from .base import ParamSpec, register
 class RMSNorm:
     """y = x * rsqrt(mean(x^2) + eps) * w  (/root/reference/src/kipp.c:2221-2231)."""
 
+    graph_safe = True   # forward launches kernels only: no host reads, no data-dependent launches
+
     def __init__(self, spec, runtime):
         self.spec = spec
         self.rt = runtime

@@ -16,6 +16,7 @@ from .base import register
 
 @register("position", "none")
 class NoPosition:
+    graph_safe = True   # forward launches kernels only: no host reads, no data-dependent launches
     def __init__(self, spec, runtime):
         self.spec = spec
 
@@ -35,6 +36,8 @@ class Rope:
     """inv_freq[i] = theta^(-2i / rotary_dim), angle = float32(pos) * inv_freq[i]
     (/root/reference/src/kipp.c:2368-2382).  The table is computed once in
     float64 and rounded to float32; the angle product is float32."""
+
+    graph_safe = True   # forward launches kernels only: no host reads, no data-dependent launches
 
     def __init__(self, spec, runtime):
         if spec.pairing != "half":

@@ -42,6 +42,7 @@ class Runtime:
         self.cache_dtype = DTYPES[dtype]
         self.ops = ops
         self._mm_out_f32 = None
+        self.library_products = 0   # calls that went to the library (they stay out of HIP graphs)
         torch.backends.cuda.matmul.allow_tf32 = False
 
     # -- placement -----------------------------------------------------------
@@ -74,6 +75,7 @@ class Runtime:
             y = self.ops.gemm_skinny(x, w, max_parts=8 if slabs else 1)
             return y if y.shape[0] > 1 else y[0]
         # bfloat16 x bfloat16 with float32 accumulation: the library product
+        self.library_products += 1
         if self._mm_out_f32 is None:
             try:
                 torch.mm(x[:1], w[:1].t(), out_dtype=torch.float32)
