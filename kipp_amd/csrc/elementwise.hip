@@ -111,13 +111,16 @@ __global__ void residual_add_kernel(float* __restrict__ x, const TD* __restrict_
 // out[t, i] = silu(gu[t, i]) * gu[t, inner + i], silu(z) = z / (1 + exp(-z))
 // (/root/reference/src/kipp.c:2402, 2644-2648).
 template <typename TI, typename TO>
-__global__ void swiglu_kernel(const TI* __restrict__ gu, TO* __restrict__ out, int inner, size_t total) {
+__global__ void swiglu_kernel(const TI* __restrict__ gu, TO* __restrict__ out, int inner, size_t total, int parts) {
     size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= total) return;
     size_t t = idx / inner;
     int i = (int)(idx - t * inner);
-    float g = load_f(gu, t * 2 * (size_t)inner + i);
-    float u = load_f(gu, t * 2 * (size_t)inner + inner + i);
+    float g = 0.0f, u = 0.0f;
+    for (int p = 0; p < parts; ++p) {   // slabs of a split product, in order
+        g += load_f(gu, (p * total + t * (size_t)inner) * 2 + i);
+        u += load_f(gu, (p * total + t * (size_t)inner) * 2 + inner + i);
+    }
     store_f(out, idx, g / (1.0f + expf(-g)) * u);
 }
 
@@ -190,11 +193,11 @@ int kipp_residual_add(float* x, const void* delta, int delta_dtype, int parts, s
     return KIPP_LAUNCH_CHECK();
 }
 
-int kipp_swiglu(const void* gu, int in_dtype, void* out, int out_dtype, int rows, int inner, hipStream_t stream) {
+int kipp_swiglu(const void* gu, int in_dtype, int parts, void* out, int out_dtype, int rows, int inner, hipStream_t stream) {
     size_t total = (size_t)rows * inner;
     if (total == 0) return 0;
     dim3 grid((unsigned)((total + 255) / 256)), block(256);
-#define KIPP_SW(TI, TO) hipLaunchKernelGGL((swiglu_kernel<TI, TO>), grid, block, 0, stream, (const TI*)gu, (TO*)out, inner, total)
+#define KIPP_SW(TI, TO) hipLaunchKernelGGL((swiglu_kernel<TI, TO>), grid, block, 0, stream, (const TI*)gu, (TO*)out, inner, total, parts)
     if (in_dtype == KIPP_BF16) {
         if (out_dtype == KIPP_BF16) KIPP_SW(bf16_t, bf16_t); else KIPP_SW(bf16_t, float);
     } else {

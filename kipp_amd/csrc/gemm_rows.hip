@@ -1,0 +1,192 @@
+// Matrix product for a few dozen rows (decode at larger batches):
+// Y[M, N] = X[M, K] . W[N, K]^T, bfloat16 operands, float32 accumulation,
+// M <= 64.  Like the few-rows kernel it is bound by reading W once, but here
+// the rows of X are too many to fetch per wave: every wave would read as much
+// of X from L2 as of W from HBM.  So the TW waves of a workgroup share one
+// range of K and stage X through LDS in chunks of 256 columns (double
+// buffered, one barrier a chunk), while each wave streams its own 16 rows of W
+// through a ring of 8 steps in registers.
+//
+// K is split over `parts` workgroups (grid.y): part p writes slab p of
+// Y[parts, M, N]; the consumer adds the slabs in order.
+//
+// v_mfma_f32_16x16x32_bf16: A = W tile (lane: row l % 16, k = 8 (l / 16) + j),
+// B = X^T from LDS (lane: token l % 16, same k), D: lane holds features
+// 4 (l / 16) + v of token l % 16.
+#include "common.h"
+
+#define DEPTH 8                       // steps of 32 columns in one chunk
+#define CHUNK (32 * DEPTH)            // columns of X staged at a time
+#define X_PITCH (CHUNK + 8)           // bf16 elements per staged row (the pad spreads the banks)
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+
+union Frag {
+    u32x4 u;
+    bf16x8 v;
+};
+
+template <int MT, int TW>
+__global__ void __launch_bounds__(TW * KIPP_WAVE) gemm_rows_kernel(
+    const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, float* __restrict__ Y, int M, int N, int K) {
+    constexpr int THREADS = TW * KIPP_WAVE;
+    constexpr int UNITS = MT * 16 * (CHUNK / 8);              // 16-byte units of one staged chunk
+    constexpr int XR = (UNITS + THREADS - 1) / THREADS;       // units a thread moves
+    __shared__ __attribute__((aligned(16))) bf16_t xs[2][MT * 16 * X_PITCH];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l16 = lane & 15, h = lane >> 4;
+    const int n0 = (blockIdx.x * TW + wave) * 16;
+    const int part = blockIdx.y, parts = gridDim.y;
+    const int groups = K / CHUNK;                              // whole chunks; the rest of K goes to the last part
+    const int g_begin = (int)((long long)groups * part / parts);
+    const int g_end = (int)((long long)groups * (part + 1) / parts);
+
+    const int row = min(n0 + l16, N - 1);                      // clamped: in bounds, dropped at the store
+    const bf16_t* w_row = W + (size_t)row * K + 8 * h;
+
+    // the units of X this thread stages: unit -> (row, 8-column chunk)
+    const bf16_t* x_src[XR];
+    int x_dst[XR];
+#pragma unroll
+    for (int i = 0; i < XR; ++i) {
+        const int unit = min(tid + i * THREADS, UNITS - 1);
+        const int r = unit / (CHUNK / 8), c = unit % (CHUNK / 8);
+        x_src[i] = X + (size_t)min(r, M - 1) * K + c * 8;
+        x_dst[i] = r * X_PITCH + c * 8;
+    }
+
+    f32x4 acc[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[mt] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
+    Frag wf[DEPTH];
+    u32x4 xr[XR];
+
+    auto fetch_w = [&](int u, int step) { wf[u].u = *(const u32x4*)(w_row + 32 * step); };
+    auto fetch_x = [&](int g) {
+#pragma unroll
+        for (int i = 0; i < XR; ++i) xr[i] = *(const u32x4*)(x_src[i] + (size_t)g * CHUNK);
+    };
+    auto stage_x = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < XR; ++i)
+            if (tid + i * THREADS < UNITS) *(u32x4*)(xs[buf] + x_dst[i]) = xr[i];
+    };
+    auto multiply = [&](int u, int buf) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            Frag xf;
+            xf.u = *(const u32x4*)(xs[buf] + (mt * 16 + l16) * X_PITCH + 32 * u + 8 * h);
+            acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u].v, xf.v, acc[mt], 0, 0, 0);
+        }
+    };
+
+    if (g_begin < g_end) {
+#pragma unroll
+        for (int u = 0; u < DEPTH; ++u) fetch_w(u, g_begin * DEPTH + u);
+        fetch_x(g_begin);
+        stage_x(0);
+        __syncthreads();
+        for (int g = g_begin; g < g_end; ++g) {
+            const int buf = (g - g_begin) & 1;
+            const bool more = g + 1 < g_end;
+            if (more) fetch_x(g + 1);
+#pragma unroll
+            for (int u = 0; u < DEPTH; ++u) {
+                multiply(u, buf);
+                if (more) fetch_w(u, (g + 1) * DEPTH + u);
+            }
+            if (more) stage_x(buf ^ 1);
+            __syncthreads();
+        }
+    }
+    // the rest of K (fewer than 256 columns), by the last part, straight from global memory
+    if (part == parts - 1) {
+        for (int k = groups * CHUNK; k < K; k += 32) {
+            const bool ok = k + 8 * h < K;
+            Frag w_t;
+            w_t.u = (u32x4){0u, 0u, 0u, 0u};
+            if (ok) w_t.u = *(const u32x4*)(w_row + k);
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                Frag x_t;
+                x_t.u = (u32x4){0u, 0u, 0u, 0u};
+                if (ok) x_t.u = *(const u32x4*)(X + (size_t)min(16 * mt + l16, M - 1) * K + 8 * h + k);
+                acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_t.v, x_t.v, acc[mt], 0, 0, 0);
+            }
+        }
+    }
+    const int n = n0 + 4 * h;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        const int token = 16 * mt + l16;
+        if (token >= M) continue;
+        float* y = Y + ((size_t)part * M + token) * N + n;
+        if (n + 3 < N && (N & 3) == 0) {
+            *(float4*)y = make_float4(acc[mt][0], acc[mt][1], acc[mt][2], acc[mt][3]);
+        } else {
+#pragma unroll
+            for (int v = 0; v < 4; ++v)
+                if (n + v < N) y[v] = acc[mt][v];
+        }
+    }
+}
+
+// Waves per workgroup and parts of K, from the shape only: about 640 workgroups,
+// each part at least one whole chunk, at most `max_parts` slabs.
+static void plan(int N, int K, int max_parts, int* tw, int* parts) {
+    const int tiles = (N + 15) / 16;
+    const int groups = K / CHUNK > 0 ? K / CHUNK : 1;
+    *tw = tiles >= 4096 ? 8 : 4;
+    const int wgs = (tiles + *tw - 1) / *tw;
+    int p = (640 + wgs - 1) / wgs;
+    if (p > groups) p = groups;
+    if (p > max_parts) p = max_parts;
+    *parts = p < 1 ? 1 : p;
+}
+
+extern "C" {
+
+int kipp_gemm_rows_parts(int N, int K, int max_parts) {
+    int tw, parts;
+    plan(N, K, max_parts, &tw, &parts);
+    return parts;
+}
+
+// Y: float32 [parts, M, N] with parts = kipp_gemm_rows_parts(N, K, max_parts).
+// M <= 64, K a multiple of 8.
+int kipp_gemm_rows(const void* X, const void* W, float* Y, int M, int N, int K, int max_parts, hipStream_t stream) {
+    if (M <= 0 || N <= 0) return 0;
+    if (M > 64 || K <= 0 || (K & 7) || max_parts <= 0) return -1;
+    int tw, parts;
+    plan(N, K, max_parts, &tw, &parts);
+    const int tiles = (N + 15) / 16;
+    dim3 grid((tiles + tw - 1) / tw, parts), block(tw * KIPP_WAVE);
+    const int mt = (M + 15) / 16;
+#define KIPP_GR(MT, TW) \
+    hipLaunchKernelGGL((gemm_rows_kernel<MT, TW>), grid, block, 0, stream, (const bf16_t*)X, (const bf16_t*)W, Y, M, N, K)
+    if (tw == 8) {
+        switch (mt) {
+            case 1: KIPP_GR(1, 8); break;
+            case 2: KIPP_GR(2, 8); break;
+            case 3: KIPP_GR(3, 8); break;
+            case 4: KIPP_GR(4, 8); break;
+            default: return -1;
+        }
+    } else {
+        switch (mt) {
+            case 1: KIPP_GR(1, 4); break;
+            case 2: KIPP_GR(2, 4); break;
+            case 3: KIPP_GR(3, 4); break;
+            case 4: KIPP_GR(4, 4); break;
+            default: return -1;
+        }
+    }
+#undef KIPP_GR
+    return KIPP_LAUNCH_CHECK();
+}
+
+}  // extern "C"

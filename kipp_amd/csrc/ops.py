@@ -116,12 +116,14 @@ def residual_add(x: torch.Tensor, delta: torch.Tensor) -> torch.Tensor:
 
 
 def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
-    """out[t, i] = silu(gate_up[t, i]) * gate_up[t, inner + i]."""
+    """out[t, i] = silu(gate_up[t, i]) * gate_up[t, inner + i]; `gate_up` is
+    [rows, 2 inner] or slabs [parts, rows, 2 inner] that are added in order."""
     _dev(gate_up, out)
     rows, inner = out.shape
-    _need(gate_up.shape == (rows, 2 * inner), "swiglu: input must be [rows, 2 * inner]")
-    fn = _fn("elementwise", "kipp_swiglu", [_c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_int, _c_ptr])
-    _check(fn(_ptr(gate_up), _code(gate_up), _ptr(out), _code(out), rows, inner, _stream()), "swiglu")
+    _need(tuple(gate_up.shape[-2:]) == (rows, 2 * inner) and gate_up.dim() in (2, 3), "swiglu: input must be [rows, 2 * inner]")
+    parts = gate_up.shape[0] if gate_up.dim() == 3 else 1
+    fn = _fn("elementwise", "kipp_swiglu", [_c_ptr, _c_int, _c_int, _c_ptr, _c_int, _c_int, _c_int, _c_ptr])
+    _check(fn(_ptr(gate_up), _code(gate_up), parts, _ptr(out), _code(out), rows, inner, _stream()), "swiglu")
     return out
 
 
@@ -155,8 +157,10 @@ def qk_norm_rope_kv_write(qkv: torch.Tensor, q_out: torch.Tensor, k_cache: torch
     _dev(qkv, q_out, k_cache, v_cache, positions, seq_of_token, block_table, q_norm_w, k_norm_w, inv_freq)
     for t, name in ((positions, "positions"), (seq_of_token, "seq_of_token"), (block_table, "block_table")):
         _i32(t, name)
-    n = qkv.shape[0]
-    _need(qkv.shape == (n, (n_q + 2 * n_kv) * head_dim), "qk_norm_rope: qkv must be [tokens, (n_q + 2 n_kv) d]")
+    n = qkv.shape[-2]
+    parts = qkv.shape[0] if qkv.dim() == 3 else 1
+    _need(tuple(qkv.shape[-2:]) == (n, (n_q + 2 * n_kv) * head_dim) and qkv.dim() in (2, 3),
+          "qk_norm_rope: qkv must be [tokens, (n_q + 2 n_kv) d], or slabs of it")
     _need(q_out.shape == (n, n_q * head_dim), "qk_norm_rope: q_out must be [tokens, n_q d]")
     _need(k_cache.shape == v_cache.shape and k_cache.dim() == 4 and k_cache.shape[1] == n_kv
           and k_cache.shape[3] == head_dim and k_cache.dtype == v_cache.dtype,
@@ -171,11 +175,11 @@ def qk_norm_rope_kv_write(qkv: torch.Tensor, q_out: torch.Tensor, k_cache: torch
               and 0 < rotary_dim <= head_dim, "qk_norm_rope: inv_freq is float32 [rotary_dim / 2]")
     fn = _fn("rope_kv", "kipp_qk_norm_rope_kv",
              [_c_ptr, _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int,
-              _c_ptr, _c_ptr, _c_float, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr])
+              _c_ptr, _c_ptr, _c_float, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr])
     _check(fn(_ptr(qkv), _code(qkv), _ptr(q_out), _code(q_out), _ptr(k_cache), _ptr(v_cache), _code(k_cache),
               _ptr(positions), _ptr(seq_of_token), _ptr(block_table), block_table.shape[1],
               _ptr(q_norm_w), _ptr(k_norm_w), float(eps), _ptr(inv_freq), int(rotary_dim),
-              n, n_q, n_kv, head_dim, k_cache.shape[2], 1 if write_kv else 0, _stream()), "qk_norm_rope_kv_write")
+              n, n_q, n_kv, head_dim, k_cache.shape[2], 1 if write_kv else 0, parts, _stream()), "qk_norm_rope_kv_write")
     return q_out
 
 
@@ -298,6 +302,24 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, max_parts: int = 1) -> torch.T
     out = torch.empty((parts, m, n), dtype=torch.float32, device=x.device)
     fn = _fn("gemm_skinny", "kipp_gemm_skinny", [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr])
     _check(fn(_ptr(x), _ptr(w), _ptr(out), m, n, k, int(max_parts), _stream()), "gemm_skinny")
+    return out
+
+
+def gemm_rows(x: torch.Tensor, w: torch.Tensor, max_parts: int = 1) -> torch.Tensor:
+    """float32 [parts, M, N] whose sum over parts is x . w^T, for 16 < M <= 64 rows
+    (any M <= 64 is taken): the rows of x are staged through LDS and shared by
+    the waves of a workgroup."""
+    _dev(x, w)
+    m, k = x.shape
+    n = w.shape[0]
+    _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm_rows: bfloat16 operands")
+    _need(w.shape == (n, k), "gemm_rows: shapes do not match")
+    _need(0 < m <= SKINNY_MAX_ROWS and k % 8 == 0, "gemm_rows: at most 64 rows and K a multiple of 8")
+    lib = build.library("gemm_rows")
+    parts = lib.kipp_gemm_rows_parts(n, k, int(max_parts))
+    out = torch.empty((parts, m, n), dtype=torch.float32, device=x.device)
+    fn = _fn("gemm_rows", "kipp_gemm_rows", [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr])
+    _check(fn(_ptr(x), _ptr(w), _ptr(out), m, n, k, int(max_parts), _stream()), "gemm_rows")
     return out
 
 

@@ -2,7 +2,8 @@
 // values into the paged cache, in one pass over the projection output.
 //
 // Input row layout of `qkv`: [n_q heads | n_kv key heads | n_kv value heads],
-// each head `d` wide.  One wave handles one head of one token.
+// each head `d` wide; `qkv` may come in `parts` slabs [parts, tokens, width] that are added
+// in order (a product whose contraction was split over workgroups).  One wave handles one head of one token.
 //   norm   u_j *= rsqrt(mean(u^2) + eps) * w_j, the same w for every head
 //          (/root/reference/src/kipp.c:2480-2500), before the rotation;
 //   rotary (u_i, u_{i+r/2}) <- (u_i c - u_{i+r/2} s, u_{i+r/2} c + u_i s),
@@ -21,7 +22,7 @@ __global__ void qk_norm_rope_kv_kernel(
     const int32_t* __restrict__ block_table, int max_blocks,
     const float* __restrict__ q_norm_w, const float* __restrict__ k_norm_w, float eps,
     const float* __restrict__ inv_freq, int rotary_dim,
-    int n_q, int n_kv, int d, int page, int n_slots) {
+    int n_q, int n_kv, int d, int page, int n_slots, int parts, size_t part_stride) {
     __shared__ float buf[HEADS_PER_BLOCK][MAX_D];
     const int wave = threadIdx.x / KIPP_WAVE;
     const int lane = threadIdx.x & (KIPP_WAVE - 1);
@@ -39,8 +40,11 @@ __global__ void qk_norm_rope_kv_kernel(
 #pragma unroll
     for (int c = 0; c < MAX_D / KIPP_WAVE; ++c) {
         const int e = lane + c * KIPP_WAVE;
-        vals[c] = e < d ? load_f(src, e) : 0.0f;
-        ss += vals[c] * vals[c];
+        float v = 0.0f;
+        if (e < d)
+            for (int p = 0; p < parts; ++p) v += load_f(src, p * part_stride + e);   // slabs of a split product, in order
+        vals[c] = v;
+        ss += v * v;
     }
     const float* norm_w = kind == 0 ? q_norm_w : (kind == 1 ? k_norm_w : nullptr);
     if (norm_w != nullptr) {
@@ -103,7 +107,7 @@ extern "C" int kipp_qk_norm_rope_kv(
     const void* qkv, int in_dtype, void* q_out, int q_dtype, void* k_cache, void* v_cache, int cache_dtype,
     const int32_t* positions, const int32_t* seq_of_token, const int32_t* block_table, int max_blocks,
     const float* q_norm_w, const float* k_norm_w, float eps, const float* inv_freq, int rotary_dim,
-    int n_tokens, int n_q, int n_kv, int d, int page, int write_kv, hipStream_t stream) {
+    int n_tokens, int n_q, int n_kv, int d, int page, int write_kv, int parts, hipStream_t stream) {
     if (n_tokens <= 0) return 0;
     if (d > MAX_D || d <= 0 || rotary_dim > d || (rotary_dim & 1)) return -1;
     const int n_slots = write_kv ? n_q + 2 * n_kv : n_q;
@@ -111,7 +115,8 @@ extern "C" int kipp_qk_norm_rope_kv(
 #define KIPP_RK(TI, TO, TC)                                                                                  \
     hipLaunchKernelGGL((qk_norm_rope_kv_kernel<TI, TO, TC>), grid, block, 0, stream, (const TI*)qkv,         \
                        (TO*)q_out, (TC*)k_cache, (TC*)v_cache, positions, seq_of_token, block_table,         \
-                       max_blocks, q_norm_w, k_norm_w, eps, inv_freq, rotary_dim, n_q, n_kv, d, page, n_slots)
+                       max_blocks, q_norm_w, k_norm_w, eps, inv_freq, rotary_dim, n_q, n_kv, d, page, n_slots, parts,      \
+                       (size_t)n_tokens * (n_q + 2 * n_kv) * d)
     if (in_dtype == KIPP_F32 && q_dtype == KIPP_F32 && cache_dtype == KIPP_F32) KIPP_RK(float, float, float);
     else if (in_dtype == KIPP_F32 && q_dtype == KIPP_BF16 && cache_dtype == KIPP_BF16) KIPP_RK(float, bf16_t, bf16_t);
     else if (in_dtype == KIPP_BF16 && q_dtype == KIPP_BF16 && cache_dtype == KIPP_BF16) KIPP_RK(bf16_t, bf16_t, bf16_t);

@@ -7,7 +7,7 @@ from typing import Iterable, List, Optional, Tuple
 Spec = Tuple[str, Optional[dict]]
 
 GENERIC: List[Spec] = [(name, None) for name in
-                       ("elementwise", "rope_kv", "attention_generic", "gemm_f32", "gemm_skinny", "sampling")]
+                       ("elementwise", "rope_kv", "attention_generic", "gemm_f32", "gemm_skinny", "gemm_rows", "sampling")]
 
 
 def attention_variants(head_dim: int, group: int) -> List[Spec]:

@@ -74,7 +74,7 @@ class Attention:
     def forward(self, x, batch, cache, state=None):
         s, rt = self.spec, self.rt
         n = x.shape[0]
-        qkv = rt.linear(x, self.w_qkv)
+        qkv = rt.linear(x, self.w_qkv, slabs=True)
         inv_freq, rotary_dim = self.position.rotary_table()
         table = batch.block_tables[cache.group]
         q = rt.ops.qk_norm_rope_kv_write(

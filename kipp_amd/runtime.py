@@ -71,8 +71,11 @@ class Runtime:
         if x.dtype != torch.bfloat16:
             x = self.ops.cast(x, self.empty(x.shape, torch.bfloat16))
         if self.ops.gemm_skinny_ok(m, x.shape[1]):
-            # few rows: our own kernel streams the weight once
-            y = self.ops.gemm_skinny(x, w, max_parts=8 if slabs else 1)
+            # few rows: our own kernels stream the weight once
+            if m <= 16:
+                y = self.ops.gemm_skinny(x, w, max_parts=8 if slabs else 1)
+            else:
+                y = self.ops.gemm_rows(x, w, max_parts=16 if slabs else 1)
             return y if y.shape[0] > 1 else y[0]
         # bfloat16 x bfloat16 with float32 accumulation: the library product
         self.library_products += 1

@@ -385,6 +385,47 @@ def test_gemm_skinny(m, n, k, max_parts):
     assert np.array_equal(out.cpu().numpy(), xi.float().numpy() @ wi.float().numpy().T)
 
 
+@pytest.mark.parametrize("m", [1, 17, 32, 33, 64])
+@pytest.mark.parametrize("n,k,max_parts", [(16, 32, 1), (77, 80, 4), (2560, 264, 8), (2560, 9728, 16), (509, 2560, 2), (6144, 2560, 16),
+                                           (70000, 512, 1)])
+def test_gemm_rows(m, n, k, max_parts):
+    ops = _ops()
+    rng = np.random.default_rng(m + n)
+    x = torch.tensor(rng.normal(size=(m, k)), dtype=torch.bfloat16)
+    w = torch.tensor(rng.normal(size=(n, k)), dtype=torch.bfloat16)
+    out = ops.gemm_rows(x.to(DEV), w.to(DEV), max_parts)
+    assert 1 <= out.shape[0] <= max_parts and tuple(out.shape[1:]) == (m, n)
+    ref = x.double().numpy() @ w.double().numpy().T
+    assert _rel(out.sum(dim=0).cpu().numpy(), ref) < 1e-11
+    xi = torch.tensor(rng.integers(-3, 4, size=(m, k)), dtype=torch.bfloat16)
+    wi = torch.tensor(rng.integers(-3, 4, size=(n, k)), dtype=torch.bfloat16)
+    out = ops.gemm_rows(xi.to(DEV), wi.to(DEV), max_parts).sum(dim=0)
+    assert np.array_equal(out.cpu().numpy(), xi.float().numpy() @ wi.float().numpy().T)
+
+
+def test_consumers_add_slabs_in_order():
+    """The rotary kernel and SwiGLU take a product that comes in slabs."""
+    ops = _ops()
+    rng = np.random.default_rng(12)
+    n_q, n_kv, d, page, t = 4, 2, 32, 8, 5
+    slabs = rng.normal(size=(3, t, (n_q + 2 * n_kv) * d)).astype(np.float32)
+    whole = slabs[0] + slabs[1] + slabs[2]
+    table = np.arange(4, dtype=np.int32).reshape(1, 4)
+    inv_freq = np.power(1e4, -(2.0 * np.arange(d // 2)) / d).astype(np.float32)
+    outs = []
+    for qkv in (slabs, whole):
+        k, v = torch.zeros(4, n_kv, page, d, device=DEV), torch.zeros(4, n_kv, page, d, device=DEV)
+        q = ops.qk_norm_rope_kv_write(_t(qkv), torch.empty(t, n_q * d, device=DEV), k, v, _t(np.arange(t), torch.int32),
+                                      _t(np.zeros(t), torch.int32), _t(table, torch.int32), n_q, n_kv, d,
+                                      _t(np.ones(d)), _t(np.ones(d)), 1e-6, _t(inv_freq), d)
+        outs.append((q.cpu(), k.cpu(), v.cpu()))
+    assert all(torch.equal(a, b) for a, b in zip(*outs))
+    gu = rng.normal(size=(4, 6, 2 * 40)).astype(np.float32)
+    a = ops.swiglu(_t(gu), torch.empty(6, 40, device=DEV)).cpu()
+    b = ops.swiglu(_t(gu[0] + gu[1] + gu[2] + gu[3]), torch.empty(6, 40, device=DEV)).cpu()
+    assert torch.equal(a, b)
+
+
 def test_gemm_skinny_refuses_what_it_cannot_do():
     ops = _ops()
     x = torch.zeros(2, 8, dtype=torch.bfloat16, device=DEV)
