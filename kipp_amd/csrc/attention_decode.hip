@@ -77,7 +77,8 @@ __global__ void __launch_bounds__(THREADS) attention_decode_kernel(
     // Pages first, once, into LDS: the loads of keys and values below then depend on
     // nothing that is still in flight and can all be issued back to back.  Keys beyond
     // the query's position read the last valid page (finite values, masked later).
-    if (tid < SPLIT) s_page[tid] = table[min(base + tid, pos) / page];
+    const int page_shift = __builtin_ctz(page);          // the page size is a power of two (checked by the launcher)
+    if (tid < SPLIT) s_page[tid] = table[min(base + tid, pos) >> page_shift];
     __syncthreads();
 
     // ---- the GROUP queries as B operand: lane (slot l16, quarter h) holds q[slot][32 t + 8 h .. + 7]
@@ -94,7 +95,7 @@ __global__ void __launch_bounds__(THREADS) attention_decode_kernel(
     for (int b = 0; b < BLOCKS_PER_WAVE; ++b) {
         const int kl = (wave * BLOCKS_PER_WAVE + b) * 16 + l16;
         const int s = min(base + kl, pos);
-        const bf16_t* k_row = k_cache + (((size_t)s_page[kl] * n_kv + kvh) * page + s % page) * HEAD_DIM;
+        const bf16_t* k_row = k_cache + (((size_t)s_page[kl] * n_kv + kvh) * page + (s & (page - 1))) * HEAD_DIM;
 #pragma unroll
         for (int t = 0; t < KSTEPS; ++t) kf[b][t].u = *(const uint4*)(k_row + min(32 * t + 8 * h, HEAD_DIM - 8));
     }
@@ -105,7 +106,7 @@ __global__ void __launch_bounds__(THREADS) attention_decode_kernel(
     for (int i = 0; i < KEYS_PER_GROUP; ++i) {
         const int kl = kg + 16 * i;
         const int s = min(base + kl, pos);
-        const bf16_t* v_row = v_cache + (((size_t)s_page[kl] * n_kv + kvh) * page + s % page) * HEAD_DIM;
+        const bf16_t* v_row = v_cache + (((size_t)s_page[kl] * n_kv + kvh) * page + (s & (page - 1))) * HEAD_DIM;
 #pragma unroll
         for (int c = 0; c < CHUNKS_PER_LANE; ++c) vf[i][c].u = *(const uint4*)(v_row + min(l16 + 16 * c, CHUNKS - 1) * 8);
     }
@@ -264,6 +265,7 @@ int kipp_attention_decode(const void* q, const void* k_cache, const void* v_cach
     if (n_items <= 0) return 0;
     if (head_dim != HEAD_DIM || n_kv <= 0 || n_q != n_kv * GROUP) return -1;
     if (grid_splits <= 0 || grid_splits > max_splits) return -3;
+    if (page <= 0 || (page & (page - 1))) return -4;   // pages of a power of two only
     const float scale_log2e = scale * 1.4426950408889634f;
     hipLaunchKernelGGL(attention_decode_kernel, dim3(grid_splits, n_kv, n_items), dim3(THREADS), 0, stream,
                        (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, part_acc, part_ml,

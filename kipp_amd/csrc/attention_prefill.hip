@@ -42,23 +42,35 @@
 #define DCHUNKS (HEAD_DIM / 8)
 #define K_LOADS ((BN * DCHUNKS + THREADS - 1) / THREADS)
 #define V_TASKS (((BN / 2) * DCHUNKS + THREADS - 1) / THREADS)
-#define MAX_PAGES 2048
+#define MAX_PAGES 4096
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+
 union Frag {
-    uint4 u;
-    uint2 d[2];
+    u32x4 u;
     bf16x8 v;
-    bf16_t h[8];
 };
 
+
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+
+// two floats to two bfloat16 (round to nearest even) in one 32-bit word: the conversion
+// instruction of gfx950
 __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
-    return (uint32_t)f32_to_bf16(a) | ((uint32_t)f32_to_bf16(b) << 16);
+    union {
+        bf16x2 v;
+        uint32_t u;
+    } r;
+    r.v = __builtin_convertvector((f32x2){a, b}, bf16x2);
+    return r.u;
 }
 
-__global__ void __launch_bounds__(THREADS) attention_prefill_kernel(
+__global__ void __launch_bounds__(THREADS, 2) attention_prefill_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     bf16_t* __restrict__ out, const int32_t* __restrict__ item_seq, const int32_t* __restrict__ item_tile,
     const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len, const int32_t* __restrict__ positions,
@@ -70,10 +82,16 @@ __global__ void __launch_bounds__(THREADS) attention_prefill_kernel(
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int l32 = lane & 31, hh = lane >> 5;
-    const int head = blockIdx.y;
+    // Work = (item, head), items sorted by the host from the longest key range to the
+    // shortest.  The first half of the grid takes the work in that order, the second half
+    // from the light end: workgroups that come to share a compute unit (k and k + half, when
+    // the whole grid is resident at once) then carry about the same load together.
+    const int total = gridDim.x, half = (total + 1) / 2;
+    const int work = (int)blockIdx.x < half ? (int)blockIdx.x : total - 1 - ((int)blockIdx.x - half);
+    const int item = work / n_q, head = work % n_q;
     const int kvh = head / (n_q / n_kv);
-    const int seq = item_seq[blockIdx.x];
-    const int tile_row0 = item_tile[blockIdx.x] * BM;           // first row of the tile within the portion
+    const int seq = item_seq[item];
+    const int tile_row0 = item_tile[item] * BM;                 // first row of the tile within the portion
     const int row0 = q_start[seq] + tile_row0;                  // ... within the batch
     const int rows_in_tile = min(BM, q_len[seq] - tile_row0);
     const int pos0 = positions[row0];                           // position of the tile's first query
@@ -90,8 +108,8 @@ __global__ void __launch_bounds__(THREADS) attention_prefill_kernel(
     Frag qf[QSTEPS];
 #pragma unroll
     for (int t = 0; t < QSTEPS; ++t) {
-        qf[t].u = make_uint4(0, 0, 0, 0);
-        if (row_valid) qf[t].u = *(const uint4*)(q + ((size_t)(row0 + my_row) * n_q + head) * HEAD_DIM + 16 * t + 8 * hh);
+        qf[t].u = (u32x4){0u, 0u, 0u, 0u};
+        if (row_valid) qf[t].u = *(const u32x4*)(q + ((size_t)(row0 + my_row) * n_q + head) * HEAD_DIM + 16 * t + 8 * hh);
     }
 
     f32x16 o[DTILES];
@@ -110,28 +128,28 @@ __global__ void __launch_bounds__(THREADS) attention_prefill_kernel(
     const int tile_hi = last_pos / BN;
 
     // The pages of the keys this workgroup reads, once, into LDS: the loads of a tile then
-    // depend on nothing in flight and are issued back to back.  (A sequence with more pages
-    // than fit is read through the table in global memory instead.)
-    const int first_block = (tile_lo * BN) / page, last_block = last_pos / page;
-    const bool pages_in_lds = last_block - first_block < MAX_PAGES;
-    if (pages_in_lds)
-        for (int i = tid; i <= last_block - first_block; i += THREADS) s_page[i] = table[first_block + i];
+    // depend on nothing in flight and are issued back to back.  The page size is a power of
+    // two and the table row fits s_page (both checked by the launcher).
+    const int page_shift = __builtin_ctz(page);
+    const int first_block = (tile_lo * BN) >> page_shift, last_block = last_pos >> page_shift;
+    for (int i = tid; i <= last_block - first_block; i += THREADS) s_page[i] = table[first_block + i];
     __syncthreads();
-    auto page_of = [&](int s) {   // s is clamped to the last key of the portion: beyond it the values are masked
-        const int block = min(s, last_pos) / page;
-        return pages_in_lds ? s_page[block - first_block] : table[block];
+    // address of key s of this sequence and head; s is clamped to the last key of the portion
+    // (beyond it the scores are masked, the values only have to be finite)
+    auto row_offset = [&](int s) -> size_t {
+        const int sc = min(s, last_pos);
+        return (((size_t)s_page[(sc >> page_shift) - first_block] * n_kv + kvh) * page + (sc & (page - 1))) * HEAD_DIM;
     };
 
     // registers for one tile: keys (K_LOADS 16-byte chunks a thread), values (2 chunks for each of V_TASKS key pairs)
-    uint4 k_reg[K_LOADS];
+    Frag k_reg[K_LOADS];
     Frag v_reg[V_TASKS][2];
     auto fetch_tile = [&](int key0) {
 #pragma unroll
         for (int i = 0; i < K_LOADS; ++i) {
             const int c = min(tid + i * THREADS, BN * DCHUNKS - 1);
             const int key = c / DCHUNKS, chunk = c % DCHUNKS;
-            const int s = min(key0 + key, last_pos);
-            k_reg[i] = *(const uint4*)(k_cache + (((size_t)page_of(s) * n_kv + kvh) * page + s % page) * HEAD_DIM + chunk * 8);
+            k_reg[i].u = *(const u32x4*)(k_cache + row_offset(key0 + key) + chunk * 8);
         }
 #pragma unroll
         for (int i = 0; i < V_TASKS; ++i) {
@@ -139,8 +157,7 @@ __global__ void __launch_bounds__(THREADS) attention_prefill_kernel(
             const int pair = c % (BN / 2), chunk = c / (BN / 2);
 #pragma unroll
             for (int e = 0; e < 2; ++e) {
-                const int s = min(key0 + 2 * pair + e, last_pos);
-                v_reg[i][e].u = *(const uint4*)(v_cache + (((size_t)page_of(s) * n_kv + kvh) * page + s % page) * HEAD_DIM + chunk * 8);
+                v_reg[i][e].u = *(const u32x4*)(v_cache + row_offset(key0 + 2 * pair + e) + chunk * 8);
             }
         }
     };
@@ -149,7 +166,7 @@ __global__ void __launch_bounds__(THREADS) attention_prefill_kernel(
 #pragma unroll
         for (int i = 0; i < K_LOADS; ++i) {
             const int c = tid + i * THREADS;
-            if (c < BN * DCHUNKS) *(uint4*)(Ks + (c / DCHUNKS) * K_PITCH + (c % DCHUNKS) * 8) = k_reg[i];
+            if (c < BN * DCHUNKS) *(u32x4*)(Ks + (c / DCHUNKS) * K_PITCH + (c % DCHUNKS) * 8) = k_reg[i].u;
         }
 #pragma unroll
         for (int i = 0; i < V_TASKS; ++i) {
@@ -157,9 +174,11 @@ __global__ void __launch_bounds__(THREADS) attention_prefill_kernel(
             if (c < (BN / 2) * DCHUNKS) {
                 const int pair = c % (BN / 2), chunk = c / (BN / 2);
 #pragma unroll
-                for (int j = 0; j < 8; ++j)
+                for (int j = 0; j < 8; ++j) {
+                    const uint32_t a = v_reg[i][0].u[j >> 1], b = v_reg[i][1].u[j >> 1];
                     *(uint32_t*)(Vt + (chunk * 8 + j) * V_PITCH + 2 * pair) =
-                        (uint32_t)v_reg[i][0].h[j] | ((uint32_t)v_reg[i][1].h[j] << 16);
+                        (j & 1) ? (a >> 16) | (b & 0xffff0000u) : (a & 0xffffu) | (b << 16);
+                }
             }
         }
     };
@@ -182,41 +201,51 @@ __global__ void __launch_bounds__(THREADS) attention_prefill_kernel(
 #pragma unroll
             for (int t = 0; t < QSTEPS; ++t) {
                 Frag kf;
-                kf.u = *(const uint4*)(Ks + (32 * j + l32) * K_PITCH + 16 * t + 8 * hh);
+                kf.u = *(const u32x4*)(Ks + (32 * j + l32) * K_PITCH + 16 * t + 8 * hh);
                 s_acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf.v, qf[t].v, s_acc[j], 0, 0, 0);
             }
         }
-        // ---- mask and online softmax; register v of half j is key 32 j + 8 (v / 4) + 4 hh + v % 4
+        // ---- online softmax in base 2; register v of half j is key 32 j + 8 (v / 4) + 4 hh + v % 4.
+        //      The scale is folded into the exponent: p = 2^(s c - m c), one FMA and one exp a key.
+        //      Only tiles that touch the diagonal (or a window's edge) pay for a mask.
+        const bool masked = key0 + BN - 1 > pos0 + wave * 32 || window > 0;
+        if (masked) {
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int s = key0 + 32 * j + 8 * (v / 4) + 4 * hh + (v % 4);
+                    if (s > my_pos || s < my_lo) s_acc[j][v] = -INFINITY;
+                }
+        }
         float m_tile = -INFINITY;
 #pragma unroll
         for (int j = 0; j < 2; ++j)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int s = key0 + 32 * j + 8 * (v / 4) + 4 * hh + (v % 4);
-                const float x = (s <= my_pos && s >= my_lo) ? s_acc[j][v] * scale_log2e : -INFINITY;
-                s_acc[j][v] = x;
-                m_tile = fmaxf(m_tile, x);
-            }
+            for (int v = 0; v < 16; ++v) m_tile = fmaxf(m_tile, s_acc[j][v]);
         m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, KIPP_WAVE));
-        const float m_new = fmaxf(m_run, m_tile);
-        const float m_use = m_new == -INFINITY ? 0.0f : m_new;   // a row with nothing visible yet
-        const float alpha = exp2f(m_run - m_use);
+        const float m_new = fmaxf(m_run, m_tile);                 // raw scores; scale_log2e > 0 keeps the order
+        const float m_use = m_new == -INFINITY ? 0.0f : m_new;    // a row with nothing visible yet
+        const float m_scaled = m_use * scale_log2e;
+        const float alpha = __builtin_amdgcn_exp2f(m_run * scale_log2e - m_scaled);
         float l_tile = 0.0f;
 #pragma unroll
         for (int j = 0; j < 2; ++j)
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
-                const float p = exp2f(s_acc[j][v] - m_use);
+                const float p = __builtin_amdgcn_exp2f(fmaf(s_acc[j][v], scale_log2e, -m_scaled));   // -inf gives 0
                 s_acc[j][v] = p;
                 l_tile += p;
             }
         l_tile += __shfl_xor(l_tile, 32, KIPP_WAVE);
         l_run = l_run * alpha + l_tile;
         m_run = m_new;
+        if (__any(alpha != 1.0f)) {                               // the maximum moved for some query of the wave
 #pragma unroll
-        for (int dt = 0; dt < DTILES; ++dt)
+            for (int dt = 0; dt < DTILES; ++dt)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) o[dt][v] *= alpha;
+                for (int v = 0; v < 16; ++v) o[dt][v] *= alpha;
+        }
         // ---- O^T += V^T P^T; step st of half j uses registers 8 st .. 8 st + 7, which are the keys
         //      32 j + 16 st + {4 hh .. 4 hh + 3} and 32 j + 16 st + 8 + {4 hh .. 4 hh + 3}
 #pragma unroll
@@ -224,16 +253,16 @@ __global__ void __launch_bounds__(THREADS) attention_prefill_kernel(
 #pragma unroll
             for (int st = 0; st < 2; ++st) {
                 Frag pf;
-                pf.u.x = pack_bf16(s_acc[j][8 * st + 0], s_acc[j][8 * st + 1]);
-                pf.u.y = pack_bf16(s_acc[j][8 * st + 2], s_acc[j][8 * st + 3]);
-                pf.u.z = pack_bf16(s_acc[j][8 * st + 4], s_acc[j][8 * st + 5]);
-                pf.u.w = pack_bf16(s_acc[j][8 * st + 6], s_acc[j][8 * st + 7]);
+                pf.u = (u32x4){pack_bf16(s_acc[j][8 * st + 0], s_acc[j][8 * st + 1]),
+                               pack_bf16(s_acc[j][8 * st + 2], s_acc[j][8 * st + 3]),
+                               pack_bf16(s_acc[j][8 * st + 4], s_acc[j][8 * st + 5]),
+                               pack_bf16(s_acc[j][8 * st + 6], s_acc[j][8 * st + 7])};
 #pragma unroll
                 for (int dt = 0; dt < DTILES; ++dt) {
                     Frag vf;
                     const bf16_t* col = Vt + (32 * dt + l32) * V_PITCH + 32 * j + 16 * st + 4 * hh;
-                    vf.d[0] = *(const uint2*)(col);
-                    vf.d[1] = *(const uint2*)(col + 8);
+                    const u32x2 lo = *(const u32x2*)(col), hi = *(const u32x2*)(col + 8);
+                    vf.u = (u32x4){lo[0], lo[1], hi[0], hi[1]};
                     o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf.v, pf.v, o[dt], 0, 0, 0);
                 }
             }
@@ -248,10 +277,8 @@ __global__ void __launch_bounds__(THREADS) attention_prefill_kernel(
         for (int g = 0; g < 4; ++g) {
             const int dcol = 32 * dt + 8 * g + 4 * hh;
             if (dcol < HEAD_DIM) {
-                uint2 w;
-                w.x = pack_bf16(o[dt][4 * g + 0] * inv, o[dt][4 * g + 1] * inv);
-                w.y = pack_bf16(o[dt][4 * g + 2] * inv, o[dt][4 * g + 3] * inv);
-                *(uint2*)(o_row + dcol) = w;
+                *(u32x2*)(o_row + dcol) = (u32x2){pack_bf16(o[dt][4 * g + 0] * inv, o[dt][4 * g + 1] * inv),
+                                                  pack_bf16(o[dt][4 * g + 2] * inv, o[dt][4 * g + 3] * inv)};
             }
         }
 }
@@ -261,7 +288,7 @@ extern "C" {
 int kipp_attention_prefill_rows() { return BM; }
 
 // `item_seq[i]`, `item_tile[i]`: sequence (row of the block table) and 128-row
-// tile of its portion for work item i.
+// tile of its portion for work item i; best sorted from the longest key range to the shortest.
 int kipp_attention_prefill(const void* q, const void* k_cache, const void* v_cache, void* out,
                            const int32_t* item_seq, const int32_t* item_tile, const int32_t* q_start,
                            const int32_t* q_len, const int32_t* positions, const int32_t* block_table, int max_blocks,
@@ -269,8 +296,10 @@ int kipp_attention_prefill(const void* q, const void* k_cache, const void* v_cac
                            hipStream_t stream) {
     if (n_items <= 0) return 0;
     if (head_dim != HEAD_DIM || n_kv <= 0 || n_q % n_kv) return -1;
+    if (page <= 0 || (page & (page - 1))) return -4;   // pages of a power of two only
+    if (max_blocks > MAX_PAGES) return -5;             // the table row is staged in LDS
     const float scale_log2e = scale * 1.4426950408889634f;
-    hipLaunchKernelGGL(attention_prefill_kernel, dim3(n_items, n_q), dim3(THREADS), 0, stream, (const bf16_t*)q,
+    hipLaunchKernelGGL(attention_prefill_kernel, dim3(n_items * n_q), dim3(THREADS), 0, stream, (const bf16_t*)q,
                        (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, item_seq, item_tile, q_start, q_len,
                        positions, block_table, max_blocks, n_q, n_kv, page, scale_log2e, window);
     return KIPP_LAUNCH_CHECK();

@@ -214,6 +214,16 @@ def _attn_common(q, k_cache, v_cache, out, n_q, n_kv, head_dim, what):
     _need(k_cache.shape == v_cache.shape and k_cache.dim() == 4 and k_cache.shape[1] == n_kv
           and k_cache.shape[3] == head_dim, f"{what}: caches must be [pages, n_kv, page, d]")
     _need(head_dim % 16 == 0 and 0 < head_dim <= 256 and n_q % n_kv == 0, f"{what}: head size or head counts refused")
+    page = k_cache.shape[2]
+    _need(page > 0 and page & (page - 1) == 0, f"{what}: the page size must be a power of two (the generic kernel takes any)")
+
+
+PREFILL_MAX_BLOCKS = 4096   # table entries of one sequence the prefill kernel stages in LDS
+
+
+def attention_fast_ok(n_q: int, n_kv: int, page: int, max_blocks: int = 0) -> bool:
+    """Whether the matrix-core attention kernels take this geometry."""
+    return n_q // n_kv <= 16 and page > 0 and page & (page - 1) == 0 and max_blocks <= PREFILL_MAX_BLOCKS
 
 
 DECODE_SPLIT = 256      # keys per workgroup of the decode kernel (checked against the library at load)
@@ -269,6 +279,7 @@ def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
         _i32(t, name)
     _attn_common(q, k_cache, v_cache, out, n_q, n_kv, head_dim, "attention_prefill")
     _need(item_seq.numel() == item_tile.numel(), "attention_prefill: one tile index per work item")
+    _need(block_table.shape[1] <= PREFILL_MAX_BLOCKS, "attention_prefill: more pages per sequence than the kernel stages")
     fn = _fn("attention_prefill", "kipp_attention_prefill",
              [_c_ptr] * 10 + [_c_int] * 6 + [_c_float, _c_int, _c_ptr], {"HEAD_DIM": head_dim})
     _check(fn(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(item_seq), _ptr(item_tile), _ptr(q_start),

@@ -72,12 +72,16 @@ def build_batch(entries: Sequence[StepEntry], requests: Sequence[object], n_grou
     n_seqs = len(entries)
     decode_rows = [q_start[i] for i in range(n_seqs) if q_len[i] == 1]
     decode_ctx = [ctx_len[i] for i in range(n_seqs) if q_len[i] == 1]
-    prefill_seq, prefill_tile = [], []
+    items = []
     for i in range(n_seqs):
         if q_len[i] > 1:
+            start = ctx_len[i] - q_len[i]
             for tile in range((q_len[i] + PREFILL_TILE - 1) // PREFILL_TILE):
-                prefill_seq.append(i)
-                prefill_tile.append(tile)
+                keys = start + min((tile + 1) * PREFILL_TILE, q_len[i])     # keys the tile's last row sees
+                items.append((-keys, i, tile))
+    items.sort()                                                          # longest key range first
+    prefill_seq = [i for _, i, _ in items]
+    prefill_tile = [t for _, _, t in items]
     max_blocks = max(1, max(len(req.tables[g]) for req in requests for g in range(n_groups)) if n_groups else 1)
     tables = []
     for g in range(n_groups):

@@ -83,8 +83,7 @@ class Attention:
             self.q_norm, self.k_norm, s.qk_norm_eps if s.qk_norm_eps is not None else 0.0,
             inv_freq, rotary_dim, write_kv=cache.writable)
         out = rt.empty((n, s.q_dim), rt.act_dtype)
-        group = s.num_heads // s.num_kv_heads
-        if rt.dtype == "bfloat16" and group <= 16:
+        if rt.dtype == "bfloat16" and rt.ops.attention_fast_ok(s.num_heads, s.num_kv_heads, cache.page_size, table.shape[1]):
             if batch.n_prefill_items:
                 rt.ops.attention_prefill(q, cache.k, cache.v, out, batch.prefill_seq, batch.prefill_tile, batch.q_start,
                                          batch.q_len, batch.positions, table, s.num_heads, s.num_kv_heads, s.head_dim,
@@ -94,7 +93,7 @@ class Attention:
                                         table, s.num_heads, s.num_kv_heads, s.head_dim, self.scale, s.window or 0,
                                         batch.max_decode_ctx, self._workspace(batch))
         else:
-            # the float32 path, and group sizes the split kernel refuses
+            # the float32 path, and geometries the matrix-core kernels refuse (groups above 16, odd page sizes)
             rt.ops.paged_attention_generic(q, cache.k, cache.v, out, batch.positions, batch.seq_of_token, table,
                                            s.num_heads, s.num_kv_heads, s.head_dim, self.scale, s.window or 0)
         return rt.linear(out, self.w_o, slabs=True)
