@@ -190,6 +190,17 @@ class CacheManager:
             req.rows[gi][len(req.tables[gi])] = 0
             self.groups[gi].pool.release(page)
 
+    def trim(self, req: RequestCache) -> None:
+        """Give back pages that were claimed for a step that did not happen."""
+        blocks = (req.length + self.page_size - 1) // self.page_size
+        for g in self.groups:
+            table = req.tables[g.index]
+            while len(table) > blocks:
+                page = table.pop()
+                req.rows[g.index][len(table)] = 0
+                if page >= 0:
+                    g.pool.release(page)
+
     def commit(self, req: RequestCache, tokens: Sequence[int]) -> None:
         """The step ran: the request now holds `tokens` more.  Pages that a
         window has passed are given back."""

@@ -68,6 +68,9 @@ class Engine:
             for t in e.tokens:
                 if not 0 <= int(t) < self.vocab_size:
                     raise ValueError(f"request {e.request!r}: token {t} is outside the vocabulary of {self.vocab_size}")
+            for w in e.want:
+                if not 0 <= int(w) < len(e.tokens):
+                    raise ValueError(f"request {e.request!r}: wanted place {w} is not among its {len(e.tokens)} tokens")
         opened = []
         try:
             for e in entries:
@@ -80,11 +83,18 @@ class Engine:
             for rid in opened:
                 self.cache.close(rid)
             raise
-        if self.graphs is not None and self.graphs.applies(entries):
-            logits = self.graphs.run(entries, requests)     # a static buffer: read it before the next step
-        else:
-            batch = build_batch(entries, requests, len(self.cache.groups), self.rt.device)
-            logits = self.model.forward(batch, self.cache)
+        try:
+            if self.graphs is not None and self.graphs.applies(entries):
+                logits = self.graphs.run(entries, requests)
+            else:
+                batch = build_batch(entries, requests, len(self.cache.groups), self.rt.device)
+                logits = self.model.forward(batch, self.cache)
+        except Exception:
+            for r in requests:                  # the step did not happen: its pages go back
+                self.cache.trim(r)
+            for rid in opened:
+                self.cache.close(rid)
+            raise
         for r, e in zip(requests, entries):
             self.cache.commit(r, e.tokens)
         return logits
