@@ -371,3 +371,23 @@ def argmax(logits: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     fn = _fn("sampling", "kipp_argmax", [_c_ptr, _c_ptr, _c_int, _c_int, _c_ptr])
     _check(fn(_ptr(logits), _ptr(out), logits.shape[0], logits.shape[1], _stream()), "argmax")
     return out
+
+
+def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
+           min_p: torch.Tensor, uniform: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """One token for each row of float32 logits: greedy where temperature <= 0,
+    else temperature sampling with top-k (0: off), min-p (0: off) and top-p, using
+    the row's uniform draw in [0, 1) (float64) made on the host."""
+    _dev(logits, temperature, top_k, top_p, min_p, uniform, out)
+    _i32(top_k, "top_k")
+    _i32(out, "sample output")
+    rows = logits.shape[0]
+    _need(logits.dtype == torch.float32 and logits.dim() == 2, "sample: float32 [rows, vocab]")
+    _need(temperature.dtype == torch.float32 and top_p.dtype == torch.float32 and min_p.dtype == torch.float32
+          and uniform.dtype == torch.float64, "sample: float32 parameters and float64 draws")
+    _need(all(t.numel() == rows for t in (temperature, top_k, top_p, min_p, uniform, out)), "sample: one value per row")
+    _need(logits.shape[1] < (1 << 24), "sample: the vocabulary must be below 2^24")
+    fn = _fn("sampling", "kipp_sample", [_c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr])
+    _check(fn(_ptr(logits), rows, logits.shape[1], _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(min_p),
+              _ptr(uniform), _ptr(out), _stream()), "sample")
+    return out

@@ -51,3 +51,193 @@ extern "C" int kipp_argmax(const float* logits, int32_t* out, int rows, int voca
     hipLaunchKernelGGL(argmax_kernel, dim3(rows), dim3(1024), 0, stream, logits, out, vocab);
     return KIPP_LAUNCH_CHECK();
 }
+
+// ---------------------------------------------------------------------------------------
+// Temperature sampling with top-k, min-p and top-p, one workgroup per row, with the
+// meaning of the host sampler (/root/reference/src/kipp.c:3433-3559): scale by 1/T,
+// keep candidates within 20 of the maximum, order them by descending logit (ties: lower
+// id first), cut to the k first, drop what is below min_p times the top weight, keep
+// the shortest prefix whose mass reaches top_p of the total, and take the first
+// candidate whose cumulative mass exceeds u times the kept mass, u drawn on the host.
+//
+// Nothing is sorted.  A candidate's place in the order is its 64-bit key
+// (monotone image of the scaled logit above the inverted index), and every question
+// ("which key is the k-th", "where does the cumulative mass reach x") is answered by
+// walking down the key one byte at a time with a 256-bin histogram of counts or of
+// masses.  Masses are weights exp(l - max) in 44-bit fixed point, added with integer
+// atomics: the sums are exact and do not depend on the order of the additions.
+
+#define SAMPLE_THREADS 1024
+#define MASS_SCALE 17592186044416.0f   // 2^44
+
+__device__ __forceinline__ uint32_t float_order(float x) {
+    const uint32_t b = __float_as_uint(x);
+    return (b & 0x80000000u) ? ~b : (b | 0x80000000u);   // larger float, larger integer
+}
+
+struct SampleRow {
+    const float* row;
+    int vocab;
+    float inv_t, scaled_max, cutoff;
+    unsigned long long key_floor;   // candidates of the top-k cut have key >= key_floor
+    double min_weight;              // ... and weight >= min_weight (0: no min-p)
+
+    __device__ __forceinline__ bool member(int i, unsigned long long* key, float* weight) const {
+        const float scaled = row[i] * inv_t;
+        if (!(scaled >= cutoff)) return false;
+        *key = ((unsigned long long)float_order(scaled) << 32) | (uint32_t)(0xffffffffu - (uint32_t)i);
+        if (*key < key_floor) return false;
+        *weight = expf(scaled - scaled_max);
+        return (double)*weight >= min_weight;
+    }
+};
+
+// Walk down the key bytes.  With MASS the measure of a candidate is its fixed-point weight,
+// else 1.  Finds the first candidate in key order (descending) at which the running measure
+// reaches `target` (STRICT: exceeds it).  Returns its key; *before gets the measure of the
+// candidates ahead of it, *own its own measure.  If the target is beyond the total, the
+// last candidate is returned.
+template <bool MASS, bool STRICT>
+__device__ unsigned long long descend(const SampleRow& r, double target, unsigned long long* hist,
+                                      unsigned long long* shared, double* before, double* own) {
+    unsigned long long prefix = 0;      // the key bytes fixed so far, right-aligned
+    double ahead = 0.0;
+    for (int level = 7; level >= 0; --level) {
+        if (level == 3) {               // byte 3 is the top byte of the inverted index: always 0xff (vocab < 2^24)
+            prefix = (prefix << 8) | 0xffull;
+            continue;
+        }
+        for (int b = threadIdx.x; b < 256; b += blockDim.x) hist[b] = 0;
+        __syncthreads();
+        for (int i = threadIdx.x; i < r.vocab; i += blockDim.x) {
+            unsigned long long key;
+            float w;
+            if (!r.member(i, &key, &w)) continue;
+            if (level < 7 && (key >> (8 * (level + 1))) != prefix) continue;
+            const unsigned long long m = MASS ? (unsigned long long)(w * MASS_SCALE) : 1ull;
+            atomicAdd(&hist[(key >> (8 * level)) & 0xff], m);
+        }
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            int chosen = -1, lowest = 0;
+            double run = ahead;
+            for (int b = 255; b >= 0; --b) {
+                if (hist[b] == 0) continue;
+                lowest = b;
+                const double next = run + (double)hist[b];
+                if (STRICT ? next > target : next >= target) {
+                    chosen = b;
+                    break;
+                }
+                run = next;
+            }
+            if (chosen < 0) {           // the target lies beyond everything: the last candidate
+                chosen = lowest;
+                run -= (double)hist[lowest];
+            }
+            shared[0] = (unsigned long long)chosen;
+            shared[1] = (unsigned long long)__double_as_longlong(run);
+            shared[2] = hist[chosen];
+        }
+        __syncthreads();
+        prefix = (prefix << 8) | shared[0];
+        ahead = __longlong_as_double((long long)shared[1]);
+        *own = (double)shared[2];
+        __syncthreads();
+    }
+    *before = ahead;
+    return prefix;
+}
+
+__global__ void __launch_bounds__(SAMPLE_THREADS) sample_kernel(
+    const float* __restrict__ logits, int vocab, const float* __restrict__ temperature, const int32_t* __restrict__ top_k,
+    const float* __restrict__ top_p, const float* __restrict__ min_p, const double* __restrict__ uniform,
+    int32_t* __restrict__ out) {
+    __shared__ unsigned long long hist[256];
+    __shared__ unsigned long long shared[4];
+    __shared__ float best_v[16];
+    __shared__ int best_i[16];
+    const int rowi = blockIdx.x;
+    const float* row = logits + (size_t)rowi * vocab;
+    // ---- the maximum, the lowest index among equals
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
+        const float v = row[i];
+        if (v > bv || (bi == 0x7fffffff && !(v != v))) {
+            bv = v;
+            bi = i;
+        }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(bv, off, KIPP_WAVE);
+        const int oi = __shfl_xor(bi, off, KIPP_WAVE);
+        if (ov > bv || (ov == bv && oi < bi)) {
+            bv = ov;
+            bi = oi;
+        }
+    }
+    if ((threadIdx.x & 63) == 0) {
+        best_v[threadIdx.x >> 6] = bv;
+        best_i[threadIdx.x >> 6] = bi;
+    }
+    __syncthreads();
+    bv = best_v[0];
+    bi = best_i[0];
+    for (int w = 1; w < SAMPLE_THREADS / KIPP_WAVE; ++w)
+        if (best_v[w] > bv || (best_v[w] == bv && best_i[w] < bi)) {
+            bv = best_v[w];
+            bi = best_i[w];
+        }
+    if (bi == 0x7fffffff) bi = 0;
+    const float t = temperature[rowi];
+    if (!(t > 0.0f)) {                      // greedy
+        if (threadIdx.x == 0) out[rowi] = bi;
+        return;
+    }
+    SampleRow r;
+    r.row = row;
+    r.vocab = vocab;
+    r.inv_t = 1.0f / t;
+    r.scaled_max = bv * r.inv_t;
+    r.cutoff = r.scaled_max - 20.0f;
+    r.key_floor = 0;
+    r.min_weight = 0.0;
+    double before, own;
+    // ---- top-k: the key of the k-th candidate is the floor of what stays
+    const int k = top_k[rowi];
+    if (k > 0) r.key_floor = descend<false, false>(r, (double)k, hist, shared, &before, &own);
+    // ---- min-p relative to the top weight, which is exp(0) = 1
+    const float mp = min_p[rowi];
+    if (mp > 0.0f) r.min_weight = (double)mp;
+    // ---- top-p: the shortest prefix whose mass reaches top_p of the total
+    for (int b = threadIdx.x; b < 4; b += blockDim.x) shared[b] = 0;
+    __syncthreads();
+    unsigned long long mine = 0;
+    for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
+        unsigned long long key;
+        float w;
+        if (r.member(i, &key, &w)) mine += (unsigned long long)(w * MASS_SCALE);
+    }
+    atomicAdd(&shared[3], mine);
+    __syncthreads();
+    const double total = (double)shared[3];
+    __syncthreads();
+    const unsigned long long last = descend<true, false>(r, (double)top_p[rowi] * total, hist, shared, &before, &own);
+    if (last > r.key_floor) r.key_floor = last;
+    const double kept = before + own;
+    // ---- the draw
+    const unsigned long long pick = descend<true, true>(r, uniform[rowi] * kept, hist, shared, &before, &own);
+    if (threadIdx.x == 0) out[rowi] = (int32_t)(0xffffffffu - (uint32_t)(pick & 0xffffffffu));
+}
+
+extern "C" int kipp_sample(const float* logits, int rows, int vocab, const float* temperature, const int32_t* top_k,
+                           const float* top_p, const float* min_p, const double* uniform, int32_t* out,
+                           hipStream_t stream) {
+    if (rows <= 0) return 0;
+    if (vocab <= 0 || vocab >= (1 << 24)) return -1;
+    hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(SAMPLE_THREADS), 0, stream, logits, vocab, temperature, top_k,
+                       top_p, min_p, uniform, out);
+    return KIPP_LAUNCH_CHECK();
+}

@@ -32,6 +32,10 @@ class Engine:
             num_pages = (max_tokens + page_size - 1) // page_size
         self.model = model
         self.rt: Runtime = model.rt
+        # what this model launches is compiled now, all at once, if it is not built yet
+        from ..csrc import build
+        from ..csrc.variants import model_variants
+        build.build_all(model_variants(model.spec, self.rt.dtype))
         self.vocab_size = model.spec.vocab_size
         self.cache = CacheManager(model.kv_needs(), model.state_needs(), page_size, num_pages, max_requests,
                                   model.spec.max_position, runtime=self.rt, share_prefixes=share_prefixes)
@@ -102,16 +106,33 @@ class Engine:
     # -- token choice -------------------------------------------------------------------
     def choose(self, logits: torch.Tensor, requests: Sequence[object]) -> List[int]:
         """One token for each row of `logits`; `requests[i]` carries the row's
-        sampling parameters, generator and recent tokens.  Greedy rows are
-        chosen on the device; rows with a temperature go through the sampler."""
+        sampling parameters, generator and recent tokens.  Rows are chosen on the
+        device in one launch (greedy and temperature rows alike; the uniform draw
+        of a temperature row comes from its request's generator on the host).
+        Only rows whose logits are changed first (bias, penalties) go through the
+        host sampler."""
         from ..sampling import sample
         rows = logits.shape[0]
         if rows != len(requests):
             raise ValueError("one request for each row of logits")
-        picked = self.rt.ops.argmax(logits, self.rt.empty((rows,), torch.int32)).cpu().tolist()
+        on_host = [i for i, r in enumerate(requests) if r.params.changes_logits]
+        temperature, top_k, top_p, min_p, uniform = [], [], [], [], []
         for i, req in enumerate(requests):
-            params = req.params
-            if params.greedy and not params.changes_logits:
-                continue
-            picked[i] = sample(logits[i].cpu().numpy(), params, req.rng, list(req.recent))
+            p = req.params
+            sampled = not p.greedy and i not in on_host
+            if sampled:
+                p.validate()
+            temperature.append(float(p.temperature) if sampled else 0.0)
+            top_k.append(int(p.top_k) if sampled else 0)
+            top_p.append(float(p.top_p) if sampled else 1.0)
+            min_p.append(float(p.min_p) if sampled else 0.0)
+            uniform.append(req.rng.uniform() if sampled else 0.0)
+        dev = self.rt.device
+        f32 = lambda v: torch.tensor(v, dtype=torch.float32, device=dev)
+        picked = self.rt.ops.sample(logits, f32(temperature), torch.tensor(top_k, dtype=torch.int32, device=dev),
+                                    f32(top_p), f32(min_p), torch.tensor(uniform, dtype=torch.float64, device=dev),
+                                    self.rt.empty((rows,), torch.int32)).cpu().tolist()
+        for i in on_host:
+            req = requests[i]
+            picked[i] = sample(logits[i].cpu().numpy(), req.params, req.rng, list(req.recent))
         return picked

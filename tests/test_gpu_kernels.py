@@ -462,3 +462,46 @@ def test_rmsnorm_adds_slabs_in_order():
         total = total + p
     assert np.array_equal(xd.cpu().numpy(), total)
     assert _rel(got.cpu().numpy(), plain.rms_norm(total, w, 1e-6)) < 1e-12
+
+
+@pytest.mark.parametrize("vocab", [509, 151936])
+def test_device_sampler_agrees_with_the_host_sampler(vocab):
+    """Same logits, same parameters, same uniform draw: the same token."""
+    from kipp_amd.sampling import SampleParams, XorShift64Star, sample
+    ops = _ops()
+    rng = np.random.default_rng(vocab)
+    cases = []
+    for temperature in (0.0, 0.3, 0.8, 1.5):
+        for top_k in (0, 1, 5, 40):
+            for top_p in (1.0, 0.9, 0.3, 1e-6):
+                for min_p in (0.0, 0.05, 0.5):
+                    cases.append((temperature, top_k, top_p, min_p))
+    cases = cases[:: 3 if vocab > 1000 else 1]
+    rows = len(cases)
+    logits = (rng.normal(size=(rows, vocab)) * rng.choice([0.3, 2.0, 6.0], size=(rows, 1))).astype(np.float32)
+    logits[::2, 17] = logits[::2, 400] = logits[::2].max(axis=1) + 0.25    # two equal maxima: the lower id comes first
+    logits[1::4, 100:140] = -30.0                                           # many equal values far below
+    seeds = rng.integers(1, 2 ** 62, size=rows)
+    uniforms = [XorShift64Star(int(s)).uniform() for s in seeds]
+    got = ops.sample(_t(logits), _t([c[0] for c in cases]), _t([c[1] for c in cases], torch.int32),
+                     _t([c[2] for c in cases]), _t([c[3] for c in cases]), _t(uniforms, torch.float64),
+                     torch.empty(rows, dtype=torch.int32, device=DEV)).cpu().tolist()
+    for i, (temperature, top_k, top_p, min_p) in enumerate(cases):
+        want = sample(logits[i], SampleParams(temperature=temperature, top_k=top_k, top_p=top_p, min_p=min_p),
+                      XorShift64Star(int(seeds[i])))
+        assert got[i] == want, f"row {i}: T={temperature} top_k={top_k} top_p={top_p} min_p={min_p}: {got[i]} != {want}"
+
+
+def test_device_sampler_follows_the_distribution():
+    ops = _ops()
+    from kipp_amd.sampling import XorShift64Star
+    logits = np.array([0.0, 3.0, -1.0, 2.5, 1.0, -40.0], dtype=np.float32)
+    n = 4000
+    r = XorShift64Star(5)
+    u = [r.uniform() for _ in range(n)]
+    got = ops.sample(_t(np.tile(logits, (n, 1))), _t([0.7] * n), _t([0] * n, torch.int32), _t([1.0] * n), _t([0.0] * n),
+                     _t(u, torch.float64), torch.empty(n, dtype=torch.int32, device=DEV)).cpu().numpy()
+    p = np.exp((logits[:5] - logits.max()) / 0.7)
+    p /= p.sum()
+    counts = np.bincount(got, minlength=6)
+    assert np.abs(counts[:5] / n - p).max() < 0.03 and counts[5] == 0
