@@ -14,10 +14,10 @@
 //            at head size 128), the 16 lane groups of the workgroup take every
 //            16th key; products in float32 FMA, summed over the groups in LDS.
 //
-// Split boundaries are multiples of SPLIT in absolute key index, and the merge
-// (attention_decode_reduce_kernel) adds the splits in index order, so the result
-// for a token does not depend on the batch it is in.  A sequence that needs
-// one split only is written normalised at once.
+// Split boundaries are multiples of SPLIT in absolute key index, and the merge (done by
+// the workgroup of a token and head that finishes last) adds the splits in index order,
+// so the result for a token does not depend on the batch it is in.  A sequence that
+// needs one split only is written normalised at once.
 //
 // Compile-time: HEAD_DIM (multiple of 16, <= 256), GROUP (query heads per
 // key/value head, <= 16).
@@ -43,15 +43,16 @@
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+
 union Frag {
-    uint4 u;
+    u32x4 u;
     bf16x8 v;
-    bf16_t h[8];
 };
 
 __global__ void __launch_bounds__(THREADS) attention_decode_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
-    bf16_t* __restrict__ out, float* __restrict__ part_acc, float* __restrict__ part_ml,
+    bf16_t* __restrict__ out, float* __restrict__ part_acc, float* __restrict__ part_ml, uint32_t* __restrict__ arrived,
     const int32_t* __restrict__ rows, const int32_t* __restrict__ positions, const int32_t* __restrict__ seq_of_token,
     const int32_t* __restrict__ block_table, int max_blocks, int n_q, int n_kv, int page, float scale_log2e,
     int window, int max_splits) {
@@ -86,7 +87,7 @@ __global__ void __launch_bounds__(THREADS) attention_decode_kernel(
 #pragma unroll
     for (int t = 0; t < KSTEPS; ++t) {
         const int dcol = min(32 * t + 8 * h, HEAD_DIM - 8);
-        qf[t].u = *(const uint4*)(q + ((size_t)row * n_q + (size_t)kvh * GROUP + min(l16, GROUP - 1)) * HEAD_DIM + dcol);
+        qf[t].u = *(const u32x4*)(q + ((size_t)row * n_q + (size_t)kvh * GROUP + min(l16, GROUP - 1)) * HEAD_DIM + dcol);
     }
 
     // ---- scores: each wave takes BLOCKS_PER_WAVE blocks of 16 keys; every load is unconditional
@@ -97,7 +98,7 @@ __global__ void __launch_bounds__(THREADS) attention_decode_kernel(
         const int s = min(base + kl, pos);
         const bf16_t* k_row = k_cache + (((size_t)s_page[kl] * n_kv + kvh) * page + (s & (page - 1))) * HEAD_DIM;
 #pragma unroll
-        for (int t = 0; t < KSTEPS; ++t) kf[b][t].u = *(const uint4*)(k_row + min(32 * t + 8 * h, HEAD_DIM - 8));
+        for (int t = 0; t < KSTEPS; ++t) kf[b][t].u = *(const u32x4*)(k_row + min(32 * t + 8 * h, HEAD_DIM - 8));
     }
     // ---- values are asked for now, so that they arrive while the scores are worked on
     Frag vf[KEYS_PER_GROUP][CHUNKS_PER_LANE];
@@ -108,12 +109,12 @@ __global__ void __launch_bounds__(THREADS) attention_decode_kernel(
         const int s = min(base + kl, pos);
         const bf16_t* v_row = v_cache + (((size_t)s_page[kl] * n_kv + kvh) * page + (s & (page - 1))) * HEAD_DIM;
 #pragma unroll
-        for (int c = 0; c < CHUNKS_PER_LANE; ++c) vf[i][c].u = *(const uint4*)(v_row + min(l16 + 16 * c, CHUNKS - 1) * 8);
+        for (int c = 0; c < CHUNKS_PER_LANE; ++c) vf[i][c].u = *(const u32x4*)(v_row + min(l16 + 16 * c, CHUNKS - 1) * 8);
     }
     // operands that reach beyond the head size or the group were read from clamped addresses: zero them
 #pragma unroll
     for (int t = 0; t < KSTEPS; ++t)
-        if (32 * t + 8 * h >= HEAD_DIM || l16 >= GROUP) qf[t].u = make_uint4(0, 0, 0, 0);
+        if (32 * t + 8 * h >= HEAD_DIM || l16 >= GROUP) qf[t].u = (u32x4){0u, 0u, 0u, 0u};
 #pragma unroll
     for (int b = 0; b < BLOCKS_PER_WAVE; ++b) {
         f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -174,7 +175,8 @@ __global__ void __launch_bounds__(THREADS) attention_decode_kernel(
         for (int c = 0; c < CHUNKS_PER_LANE; ++c) {
             float vv[8];
 #pragma unroll
-            for (int j = 0; j < 8; ++j) vv[j] = bf16_to_f32(vf[i][c].h[j]);
+            for (int j = 0; j < 8; ++j)
+                vv[j] = __uint_as_float((j & 1) ? (vf[i][c].u[j >> 1] & 0xffff0000u) : (vf[i][c].u[j >> 1] << 16));
 #pragma unroll
             for (int g = 0; g < GROUP; ++g)
 #pragma unroll
@@ -223,29 +225,36 @@ __global__ void __launch_bounds__(THREADS) attention_decode_kernel(
             }
         }
     }
-}
-
-// Merge the splits of every (token, head) in index order:
-// m* = max m_s, out = sum_s acc_s 2^(m_s - m*) / sum_s l_s 2^(m_s - m*)
-// (/root/reference/metal/kipp_kernels.metal:741-779).
-__global__ void attention_decode_reduce_kernel(
-    const float* __restrict__ part_acc, const float* __restrict__ part_ml, bf16_t* __restrict__ out,
-    const int32_t* __restrict__ rows, const int32_t* __restrict__ positions, int n_q, int window, int max_splits) {
-    const int head = blockIdx.x, item = blockIdx.y;
-    const int row = rows[item];
-    const int pos = positions[row];
-    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
-    const int n_splits = pos / SPLIT - lo / SPLIT + 1;
     if (n_splits == 1) return;
-    const size_t slot0 = ((size_t)item * n_q + head) * max_splits;
-    float m = -INFINITY;
-    for (int s = 0; s < n_splits; ++s) m = fmaxf(m, part_ml[(slot0 + s) * 2]);
-    float denom = 0.0f;
-    for (int s = 0; s < n_splits; ++s) denom += part_ml[(slot0 + s) * 2 + 1] * exp2f(part_ml[(slot0 + s) * 2] - m);
-    for (int dcol = threadIdx.x; dcol < HEAD_DIM; dcol += blockDim.x) {
-        float a = 0.0f;
-        for (int s = 0; s < n_splits; ++s)
-            a += part_acc[(slot0 + s) * HEAD_DIM + dcol] * exp2f(part_ml[(slot0 + s) * 2] - m);
+
+    // ---- the workgroup that arrives last merges the splits of this (token, key/value head),
+    //      in split order: m* = max m_s, out = sum_s acc_s 2^(m_s - m*) / sum_s l_s 2^(m_s - m*)
+    //      (/root/reference/metal/kipp_kernels.metal:741-779 does this in a kernel of its own).
+    __shared__ uint32_t s_ticket;
+    __threadfence();                                   // this split's partial result is visible device-wide ...
+    __syncthreads();
+    uint32_t* counter = arrived + (size_t)blockIdx.z * n_kv + kvh;
+    if (tid == 0) s_ticket = atomicAdd(counter, 1u);   // ... before its arrival is counted
+    __syncthreads();
+    if (s_ticket != (uint32_t)(n_splits - 1)) return;
+    if (tid == 0) *counter = 0;                        // ready for the next launch
+    __threadfence();
+    for (int idx = tid; idx < GROUP * HEAD_DIM; idx += THREADS) {
+        const int g = idx / HEAD_DIM, dcol = idx % HEAD_DIM;
+        const int head = kvh * GROUP + g;
+        const size_t slot0 = ((size_t)blockIdx.z * n_q + head) * max_splits;
+        // partial results of other workgroups are read past this compute unit's cache
+        float m = -INFINITY;
+        for (int sp = 0; sp < n_splits; ++sp)
+            m = fmaxf(m, __hip_atomic_load(part_ml + (slot0 + sp) * 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+        float denom = 0.0f, a = 0.0f;
+        for (int sp = 0; sp < n_splits; ++sp) {
+            const float ms = __hip_atomic_load(part_ml + (slot0 + sp) * 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const float ls = __hip_atomic_load(part_ml + (slot0 + sp) * 2 + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const float w = exp2f(ms - m);
+            denom += ls * w;
+            a += __hip_atomic_load(part_acc + (slot0 + sp) * HEAD_DIM + dcol, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) * w;
+        }
         out[((size_t)row * n_q + head) * HEAD_DIM + dcol] = f32_to_bf16(a / denom);
     }
 }
@@ -257,9 +266,10 @@ int kipp_attention_decode_split() { return SPLIT; }
 // `rows[i]` is the batch row of the i-th decode token.  `grid_splits` is how
 // many splits the launch covers (at least those of the longest sequence);
 // `part_acc` holds n_items * n_q * max_splits * HEAD_DIM floats, `part_ml`
-// n_items * n_q * max_splits * 2.
+// n_items * n_q * max_splits * 2, `arrived` n_items * n_kv counters that are zero
+// before the first launch (every launch leaves them zero again).
 int kipp_attention_decode(const void* q, const void* k_cache, const void* v_cache, void* out, float* part_acc,
-                          float* part_ml, const int32_t* rows, const int32_t* positions, const int32_t* seq_of_token,
+                          float* part_ml, uint32_t* arrived, const int32_t* rows, const int32_t* positions, const int32_t* seq_of_token,
                           const int32_t* block_table, int max_blocks, int n_items, int n_q, int n_kv, int head_dim,
                           int page, float scale, int window, int grid_splits, int max_splits, hipStream_t stream) {
     if (n_items <= 0) return 0;
@@ -269,12 +279,8 @@ int kipp_attention_decode(const void* q, const void* k_cache, const void* v_cach
     const float scale_log2e = scale * 1.4426950408889634f;
     hipLaunchKernelGGL(attention_decode_kernel, dim3(grid_splits, n_kv, n_items), dim3(THREADS), 0, stream,
                        (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, part_acc, part_ml,
-                       rows, positions, seq_of_token, block_table, max_blocks, n_q, n_kv, page, scale_log2e, window,
+                       arrived, rows, positions, seq_of_token, block_table, max_blocks, n_q, n_kv, page, scale_log2e, window,
                        max_splits);
-    int rc = KIPP_LAUNCH_CHECK();
-    if (rc != 0 || grid_splits == 1) return rc;
-    hipLaunchKernelGGL(attention_decode_reduce_kernel, dim3(n_q, n_items), dim3(HEAD_DIM >= 64 ? 64 : HEAD_DIM), 0,
-                       stream, part_acc, part_ml, (bf16_t*)out, rows, positions, n_q, window, max_splits);
     return KIPP_LAUNCH_CHECK();
 }
 

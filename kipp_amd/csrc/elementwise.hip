@@ -64,36 +64,57 @@ __global__ void __launch_bounds__(256) rmsnorm_rows_kernel(float* __restrict__ x
     __shared__ float scratch[16];
     const int n4 = width / 4;
     const size_t base4 = (size_t)blockIdx.x * n4;
-    float4 v[CH];
+    float4 v[CH], w[CH];
     float ss = 0.0f;
+    // every load is issued before anything is added: the kernel is a few round trips to memory long
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
         const int i = threadIdx.x + c * 256;
         v[c] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        w[c] = v[c];
         if (i < n4) {
             v[c] = load4(x, base4 + i);
-            if (delta != nullptr) {
-                for (int p = 0; p < parts; ++p) {
-                    const float4 d = load4(delta, p * (part_stride / 4) + base4 + i);
-                    v[c].x += d.x;
-                    v[c].y += d.y;
-                    v[c].z += d.z;
-                    v[c].w += d.w;
-                }
-                store4(x, base4 + i, v[c]);
-            }
+            w[c] = load4(weight, (size_t)i);
         }
-        ss += v[c].x * v[c].x + v[c].y * v[c].y + v[c].z * v[c].z + v[c].w * v[c].w;
     }
+    if (delta != nullptr) {
+        for (int p0 = 0; p0 < parts; p0 += 4) {
+            float4 d[CH][4];
+#pragma unroll
+            for (int c = 0; c < CH; ++c) {
+                const int i = threadIdx.x + c * 256;
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    d[c][q] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                    if (i < n4 && p0 + q < parts) d[c][q] = load4(delta, (p0 + q) * (part_stride / 4) + base4 + i);
+                }
+            }
+#pragma unroll
+            for (int c = 0; c < CH; ++c)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {   // slabs in order
+                    v[c].x += d[c][q].x;
+                    v[c].y += d[c][q].y;
+                    v[c].z += d[c][q].z;
+                    v[c].w += d[c][q].w;
+                }
+        }
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            const int i = threadIdx.x + c * 256;
+            if (i < n4) store4(x, base4 + i, v[c]);
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < CH; ++c) ss += v[c].x * v[c].x + v[c].y * v[c].y + v[c].z * v[c].z + v[c].w * v[c].w;
     ss = block_sum(ss, scratch);
     const float scale = 1.0f / sqrtf(ss / (float)width + eps);
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
         const int i = threadIdx.x + c * 256;
-        if (i < n4) {
-            const float4 w = load4(weight, (size_t)i);
-            store4(out, base4 + i, make_float4(v[c].x * scale * w.x, v[c].y * scale * w.y, v[c].z * scale * w.z, v[c].w * scale * w.w));
-        }
+        if (i < n4)
+            store4(out, base4 + i, make_float4(v[c].x * scale * w[c].x, v[c].y * scale * w[c].y, v[c].z * scale * w[c].z,
+                                               v[c].w * scale * w[c].w));
     }
 }
 

@@ -45,10 +45,82 @@ __global__ void __launch_bounds__(1024) argmax_kernel(const float* __restrict__ 
     }
 }
 
-extern "C" int kipp_argmax(const float* logits, int32_t* out, int rows, int vocab, hipStream_t stream) {
+// The same in two stages for large vocabularies: ARGMAX_CHUNKS workgroups a row each find the
+// best of their stretch, then one workgroup a row picks among them (again the lowest index
+// among equals: stretches are in index order).
+#define ARGMAX_CHUNKS 32
+
+__global__ void __launch_bounds__(256) argmax_chunks_kernel(const float* __restrict__ logits, float* __restrict__ part_v,
+                                                            int32_t* __restrict__ part_i, int vocab) {
+    __shared__ float best_v[4];
+    __shared__ int best_i[4];
+    const float* row = logits + (size_t)blockIdx.y * vocab;
+    const int per = (vocab + ARGMAX_CHUNKS - 1) / ARGMAX_CHUNKS;
+    const int begin = blockIdx.x * per, end = min(vocab, begin + per);
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int i = begin + threadIdx.x; i < end; i += blockDim.x) {
+        const float v = row[i];
+        if (v > bv || (bi == 0x7fffffff && !(v != v))) {
+            bv = v;
+            bi = i;
+        }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(bv, off, KIPP_WAVE);
+        const int oi = __shfl_xor(bi, off, KIPP_WAVE);
+        if (ov > bv || (ov == bv && oi < bi)) {
+            bv = ov;
+            bi = oi;
+        }
+    }
+    if ((threadIdx.x & 63) == 0) {
+        best_v[threadIdx.x >> 6] = bv;
+        best_i[threadIdx.x >> 6] = bi;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < 4; ++w)
+            if (best_v[w] > bv || (best_v[w] == bv && best_i[w] < bi)) {
+                bv = best_v[w];
+                bi = best_i[w];
+            }
+        part_v[blockIdx.y * ARGMAX_CHUNKS + blockIdx.x] = bv;
+        part_i[blockIdx.y * ARGMAX_CHUNKS + blockIdx.x] = bi;
+    }
+}
+
+__global__ void argmax_pick_kernel(const float* __restrict__ part_v, const int32_t* __restrict__ part_i,
+                                   int32_t* __restrict__ out) {
+    float bv = part_v[blockIdx.x * ARGMAX_CHUNKS + threadIdx.x];
+    int bi = part_i[blockIdx.x * ARGMAX_CHUNKS + threadIdx.x];
+#pragma unroll
+    for (int off = ARGMAX_CHUNKS / 2; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(bv, off, KIPP_WAVE);
+        const int oi = __shfl_xor(bi, off, KIPP_WAVE);
+        if (ov > bv || (ov == bv && oi < bi)) {
+            bv = ov;
+            bi = oi;
+        }
+    }
+    if (threadIdx.x == 0) out[blockIdx.x] = bi == 0x7fffffff ? 0 : bi;
+}
+
+extern "C" int kipp_argmax_scratch_floats(int rows) { return rows * ARGMAX_CHUNKS * 2; }
+
+// `scratch`: kipp_argmax_scratch_floats(rows) 4-byte words, used when the vocabulary is large.
+extern "C" int kipp_argmax(const float* logits, int32_t* out, int rows, int vocab, float* scratch, hipStream_t stream) {
     if (rows <= 0) return 0;
     if (vocab <= 0) return -1;
-    hipLaunchKernelGGL(argmax_kernel, dim3(rows), dim3(1024), 0, stream, logits, out, vocab);
+    if (vocab < 16384 || scratch == nullptr) {
+        hipLaunchKernelGGL(argmax_kernel, dim3(rows), dim3(1024), 0, stream, logits, out, vocab);
+        return KIPP_LAUNCH_CHECK();
+    }
+    float* part_v = scratch;
+    int32_t* part_i = (int32_t*)(scratch + (size_t)rows * ARGMAX_CHUNKS);
+    hipLaunchKernelGGL(argmax_chunks_kernel, dim3(ARGMAX_CHUNKS, rows), dim3(256), 0, stream, logits, part_v, part_i, vocab);
+    hipLaunchKernelGGL(argmax_pick_kernel, dim3(rows), dim3(ARGMAX_CHUNKS), 0, stream, part_v, part_i, out);
     return KIPP_LAUNCH_CHECK();
 }
 
