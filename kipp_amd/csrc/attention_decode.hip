@@ -14,10 +14,10 @@
 //            at head size 128), the 16 lane groups of the workgroup take every
 //            16th key; products in float32 FMA, summed over the groups in LDS.
 //
-// Split boundaries are multiples of SPLIT in absolute key index, and the merge (done by
-// the workgroup of a token and head that finishes last) adds the splits in index order,
-// so the result for a token does not depend on the batch it is in.  A sequence that
-// needs one split only is written normalised at once.
+// Split boundaries are multiples of SPLIT in absolute key index, and the merge
+// (attention_decode_reduce_kernel) adds the splits in index order, so the result
+// for a token does not depend on the batch it is in.  A sequence that needs
+// one split only is written normalised at once.
 //
 // Compile-time: HEAD_DIM (multiple of 16, <= 256), GROUP (query heads per
 // key/value head, <= 16).
@@ -52,7 +52,7 @@ union Frag {
 
 __global__ void __launch_bounds__(THREADS) attention_decode_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
-    bf16_t* __restrict__ out, float* __restrict__ part_acc, float* __restrict__ part_ml, uint32_t* __restrict__ arrived,
+    bf16_t* __restrict__ out, float* __restrict__ part_acc, float* __restrict__ part_ml,
     const int32_t* __restrict__ rows, const int32_t* __restrict__ positions, const int32_t* __restrict__ seq_of_token,
     const int32_t* __restrict__ block_table, int max_blocks, int n_q, int n_kv, int page, float scale_log2e,
     int window, int max_splits) {
@@ -225,36 +225,41 @@ __global__ void __launch_bounds__(THREADS) attention_decode_kernel(
             }
         }
     }
-    if (n_splits == 1) return;
+}
 
-    // ---- the workgroup that arrives last merges the splits of this (token, key/value head),
-    //      in split order: m* = max m_s, out = sum_s acc_s 2^(m_s - m*) / sum_s l_s 2^(m_s - m*)
-    //      (/root/reference/metal/kipp_kernels.metal:741-779 does this in a kernel of its own).
-    __shared__ uint32_t s_ticket;
-    __threadfence();                                   // this split's partial result is visible device-wide ...
-    __syncthreads();
-    uint32_t* counter = arrived + (size_t)blockIdx.z * n_kv + kvh;
-    if (tid == 0) s_ticket = atomicAdd(counter, 1u);   // ... before its arrival is counted
-    __syncthreads();
-    if (s_ticket != (uint32_t)(n_splits - 1)) return;
-    if (tid == 0) *counter = 0;                        // ready for the next launch
-    __threadfence();
-    for (int idx = tid; idx < GROUP * HEAD_DIM; idx += THREADS) {
-        const int g = idx / HEAD_DIM, dcol = idx % HEAD_DIM;
-        const int head = kvh * GROUP + g;
-        const size_t slot0 = ((size_t)blockIdx.z * n_q + head) * max_splits;
-        // partial results of other workgroups are read past this compute unit's cache
-        float m = -INFINITY;
-        for (int sp = 0; sp < n_splits; ++sp)
-            m = fmaxf(m, __hip_atomic_load(part_ml + (slot0 + sp) * 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-        float denom = 0.0f, a = 0.0f;
-        for (int sp = 0; sp < n_splits; ++sp) {
-            const float ms = __hip_atomic_load(part_ml + (slot0 + sp) * 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            const float ls = __hip_atomic_load(part_ml + (slot0 + sp) * 2 + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            const float w = exp2f(ms - m);
-            denom += ls * w;
-            a += __hip_atomic_load(part_acc + (slot0 + sp) * HEAD_DIM + dcol, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) * w;
+// Merge the splits of every (token, head) in index order:
+// m* = max m_s, out = sum_s acc_s 2^(m_s - m*) / sum_s l_s 2^(m_s - m*)
+// (/root/reference/metal/kipp_kernels.metal:741-779).
+__global__ void attention_decode_reduce_kernel(
+    const float* __restrict__ part_acc, const float* __restrict__ part_ml, bf16_t* __restrict__ out,
+    const int32_t* __restrict__ rows, const int32_t* __restrict__ positions, int n_q, int window, int max_splits) {
+    const int head = blockIdx.x, item = blockIdx.y;
+    const int row = rows[item];
+    const int pos = positions[row];
+    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+    const int n_splits = pos / SPLIT - lo / SPLIT + 1;
+    if (n_splits == 1) return;
+    const size_t slot0 = ((size_t)item * n_q + head) * max_splits;
+    // the (m, l) pairs of all splits, one a lane, so that they arrive together
+    const int lane = threadIdx.x & 63;
+    float m = -INFINITY;
+    for (int s0 = 0; s0 < n_splits; s0 += KIPP_WAVE)
+        if (s0 + lane < n_splits) m = fmaxf(m, part_ml[(slot0 + s0 + lane) * 2]);
+    m = wave_max(m);
+    float denom = 0.0f;
+    for (int s = 0; s < n_splits; ++s) denom += part_ml[(slot0 + s) * 2 + 1] * exp2f(part_ml[(slot0 + s) * 2] - m);
+    for (int dcol = threadIdx.x; dcol < HEAD_DIM; dcol += blockDim.x) {
+        float a = 0.0f;
+        int s = 0;
+        for (; s + 4 <= n_splits; s += 4) {       // four loads in flight; added in split order
+            const float a0 = part_acc[(slot0 + s) * HEAD_DIM + dcol], a1 = part_acc[(slot0 + s + 1) * HEAD_DIM + dcol];
+            const float a2 = part_acc[(slot0 + s + 2) * HEAD_DIM + dcol], a3 = part_acc[(slot0 + s + 3) * HEAD_DIM + dcol];
+            a += a0 * exp2f(part_ml[(slot0 + s) * 2] - m);
+            a += a1 * exp2f(part_ml[(slot0 + s + 1) * 2] - m);
+            a += a2 * exp2f(part_ml[(slot0 + s + 2) * 2] - m);
+            a += a3 * exp2f(part_ml[(slot0 + s + 3) * 2] - m);
         }
+        for (; s < n_splits; ++s) a += part_acc[(slot0 + s) * HEAD_DIM + dcol] * exp2f(part_ml[(slot0 + s) * 2] - m);
         out[((size_t)row * n_q + head) * HEAD_DIM + dcol] = f32_to_bf16(a / denom);
     }
 }
@@ -266,10 +271,9 @@ int kipp_attention_decode_split() { return SPLIT; }
 // `rows[i]` is the batch row of the i-th decode token.  `grid_splits` is how
 // many splits the launch covers (at least those of the longest sequence);
 // `part_acc` holds n_items * n_q * max_splits * HEAD_DIM floats, `part_ml`
-// n_items * n_q * max_splits * 2, `arrived` n_items * n_kv counters that are zero
-// before the first launch (every launch leaves them zero again).
+// n_items * n_q * max_splits * 2.
 int kipp_attention_decode(const void* q, const void* k_cache, const void* v_cache, void* out, float* part_acc,
-                          float* part_ml, uint32_t* arrived, const int32_t* rows, const int32_t* positions, const int32_t* seq_of_token,
+                          float* part_ml, const int32_t* rows, const int32_t* positions, const int32_t* seq_of_token,
                           const int32_t* block_table, int max_blocks, int n_items, int n_q, int n_kv, int head_dim,
                           int page, float scale, int window, int grid_splits, int max_splits, hipStream_t stream) {
     if (n_items <= 0) return 0;
@@ -279,8 +283,12 @@ int kipp_attention_decode(const void* q, const void* k_cache, const void* v_cach
     const float scale_log2e = scale * 1.4426950408889634f;
     hipLaunchKernelGGL(attention_decode_kernel, dim3(grid_splits, n_kv, n_items), dim3(THREADS), 0, stream,
                        (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, part_acc, part_ml,
-                       arrived, rows, positions, seq_of_token, block_table, max_blocks, n_q, n_kv, page, scale_log2e, window,
+                       rows, positions, seq_of_token, block_table, max_blocks, n_q, n_kv, page, scale_log2e, window,
                        max_splits);
+    int rc = KIPP_LAUNCH_CHECK();
+    if (rc != 0 || grid_splits == 1) return rc;
+    hipLaunchKernelGGL(attention_decode_reduce_kernel, dim3(n_q, n_items), dim3(HEAD_DIM >= 64 ? 64 : HEAD_DIM), 0,
+                       stream, part_acc, part_ml, (bf16_t*)out, rows, positions, n_q, window, max_splits);
     return KIPP_LAUNCH_CHECK();
 }
 

@@ -244,31 +244,27 @@ def attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
     group = n_q // n_kv
     _need(group <= 16, "attention_decode: more than 16 query heads per key/value head are refused")
     n_items = rows.numel()
-    part_acc, part_ml, arrived = workspace
+    part_acc, part_ml = workspace
     max_splits = part_ml.numel() // max(1, n_items * n_q * 2)
     span = min(max_context, window) if window else max_context
     need = (span + DECODE_SPLIT - 1) // DECODE_SPLIT + (1 if window else 0)
     grid = grid_splits if grid_splits is not None else max(1, min(need, max_splits))
-    _need(part_acc.dtype == torch.float32 and part_ml.dtype == torch.float32 and arrived.dtype == torch.int32
-          and part_acc.numel() >= n_items * n_q * max_splits * head_dim and need <= max_splits
-          and arrived.numel() >= n_items * n_kv, "attention_decode: workspace too small for this context")
+    _need(part_acc.dtype == torch.float32 and part_ml.dtype == torch.float32
+          and part_acc.numel() >= n_items * n_q * max_splits * head_dim and need <= max_splits,
+          "attention_decode: workspace too small for this context")
     defines = {"HEAD_DIM": head_dim, "GROUP": group}
     fn = _fn("attention_decode", "kipp_attention_decode",
-             [_c_ptr] * 11 + [_c_int] * 6 + [_c_float, _c_int, _c_int, _c_int, _c_ptr], defines)
-    _check(fn(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(part_acc), _ptr(part_ml), _ptr(arrived), _ptr(rows),
+             [_c_ptr] * 10 + [_c_int] * 6 + [_c_float, _c_int, _c_int, _c_int, _c_ptr], defines)
+    _check(fn(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(part_acc), _ptr(part_ml), _ptr(rows),
               _ptr(positions), _ptr(seq_of_token), _ptr(block_table), block_table.shape[1], n_items, n_q, n_kv,
               head_dim, k_cache.shape[2], float(scale), int(window), grid, max_splits, _stream()), "attention_decode")
     return out
 
 
 def attention_decode_workspace(n_items: int, n_q: int, head_dim: int, max_context: int, device) -> tuple:
-    """Partial results of the splits and the arrival counters (zero; every launch
-    leaves them zero).  One workspace serves launches that follow one another on a
-    stream, not launches that overlap."""
     max_splits = (max_context + DECODE_SPLIT - 1) // DECODE_SPLIT + 1
     return (torch.empty(n_items * n_q * max_splits * head_dim, dtype=torch.float32, device=device),
-            torch.empty(n_items * n_q * max_splits * 2, dtype=torch.float32, device=device),
-            torch.zeros(n_items * n_q, dtype=torch.int32, device=device))
+            torch.empty(n_items * n_q * max_splits * 2, dtype=torch.float32, device=device))
 
 
 def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
