@@ -505,3 +505,38 @@ def test_device_sampler_follows_the_distribution():
     p /= p.sum()
     counts = np.bincount(got, minlength=6)
     assert np.abs(counts[:5] / n - p).max() < 0.03 and counts[5] == 0
+
+
+@pytest.mark.parametrize("kernel", ["generic", "decode", "prefill"])
+def test_window_edge(kernel):
+    """With a window of W the key at pos - W + 1 is the oldest one seen and the key at pos - W is
+    not: each of the two is given by far the largest score in turn."""
+    ops = _ops()
+    n_q, n_kv, d, page, window = 8, 2, 128, 16, 300
+    rng = np.random.default_rng(9)
+    n = 700
+    for offset, seen in ((window - 1, True), (window, False)):
+        table, k, v = _paged_setup(rng, [n], n_kv, d, page, torch.bfloat16)
+        q = torch.tensor(rng.normal(size=(1, n_q * d)), dtype=torch.bfloat16)
+        far = n - 1 - offset
+        kk = k.clone()
+        for g in range(n_kv):
+            kk[table[0, far // page], g, far % page, :] = 6.0 * q[0].reshape(n_q, d)[4 * g]
+        args = dict(n_q=n_q, n_kv=n_kv, head_dim=d, scale=1 / math.sqrt(d), window=window)
+        i32 = lambda x: _t(x, torch.int32)
+        if kernel == "generic":
+            out = ops.paged_attention_generic(q.to(DEV), kk.to(DEV), v.to(DEV), torch.zeros(1, n_q * d, dtype=torch.bfloat16, device=DEV),
+                                              i32([n - 1]), i32([0]), i32(table), **args)
+        elif kernel == "decode":
+            ws = ops.attention_decode_workspace(1, n_q, d, n, DEV)
+            out = ops.attention_decode(q.to(DEV), kk.to(DEV), v.to(DEV), torch.zeros(1, n_q * d, dtype=torch.bfloat16, device=DEV),
+                                       i32([0]), i32([n - 1]), i32([0]), i32(table), max_context=n, workspace=ws, **args)
+        else:
+            q2 = torch.cat([torch.zeros(1, n_q * d, dtype=torch.bfloat16), q])
+            out = ops.attention_prefill(q2.to(DEV), kk.to(DEV), v.to(DEV), torch.zeros(2, n_q * d, dtype=torch.bfloat16, device=DEV),
+                                        i32([0]), i32([0]), i32([0]), i32([2]), i32([n - 2, n - 1]), i32(table), **args)[1:]
+        got = out.float().cpu().numpy().reshape(n_q, d)
+        for g in range(n_kv):
+            want = v[table[0, far // page], g, far % page, :].float().numpy()
+            close = np.abs(got[4 * g] - want).max() < 0.02
+            assert close == seen, f"{kernel}: key at distance {offset} (window {window}) seen={close}, expected {seen}"
