@@ -51,6 +51,7 @@ class RequestCache:
     adopted: List[int] = field(default_factory=list)        # per group: leading pages taken from the index
     adopted_tokens: int = 0
     rows: List[np.ndarray] = field(default_factory=list)    # per group: the table as the device sees it (int32, given-back pages 0)
+    table_version: int = 0                                  # counts changes of `rows`
 
 
 class CacheGroup:
@@ -146,6 +147,7 @@ class CacheManager:
                     g.pool.release(page)
                 req.tables[g.index] = list(pages[:keep])
                 req.rows[g.index][:keep] = pages[:keep]
+                req.table_version += 1
                 req.adopted[g.index] = keep
             req.adopted_tokens = keep * self.page_size
             req.length = req.adopted_tokens
@@ -165,8 +167,13 @@ class CacheManager:
         """Claim the pages that every (request, number of new tokens) of a step
         needs, in every group; all or nothing."""
         claimed: List[Tuple[RequestCache, int, int]] = []
+        page_size = self.page_size
         for req, n_new in entries:
             new_length = req.length + n_new
+            if n_new > 0 and new_length <= self.max_position:
+                blocks = (new_length + page_size - 1) // page_size
+                if all(len(t) >= blocks for t in req.tables):
+                    continue                                  # every position already has its page
             if n_new <= 0:
                 self._rollback(claimed)
                 raise ValueError("a step entry needs at least one token")
@@ -180,6 +187,7 @@ class CacheManager:
                         self._rollback(claimed)
                         raise OutOfPages(f"group {g.index}: no free page for request {req.id!r}")
                     req.rows[g.index][len(req.tables[g.index])] = page
+                    req.table_version += 1
                     req.tables[g.index].append(page)
                     claimed.append((req, g.index, page))
 
@@ -188,6 +196,7 @@ class CacheManager:
             popped = req.tables[gi].pop()
             assert popped == page
             req.rows[gi][len(req.tables[gi])] = 0
+            req.table_version += 1
             self.groups[gi].pool.release(page)
 
     def trim(self, req: RequestCache) -> None:
@@ -198,6 +207,7 @@ class CacheManager:
             while len(table) > blocks:
                 page = table.pop()
                 req.rows[g.index][len(table)] = 0
+                req.table_version += 1
                 if page >= 0:
                     g.pool.release(page)
 
@@ -217,6 +227,7 @@ class CacheManager:
                     g.pool.release(table[block])
                     table[block] = -1
                     req.rows[g.index][block] = 0
+                    req.table_version += 1
 
     def close(self, request_id) -> None:
         """The request ended: publish its full pages where sharing is on, give

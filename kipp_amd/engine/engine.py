@@ -69,12 +69,12 @@ class Engine:
             seen.add(e.request)
             if len(e.tokens) == 0:
                 raise ValueError(f"request {e.request!r}: an entry needs at least one token")
-            for t in e.tokens:
-                if not 0 <= int(t) < self.vocab_size:
-                    raise ValueError(f"request {e.request!r}: token {t} is outside the vocabulary of {self.vocab_size}")
-            for w in e.want:
-                if not 0 <= int(w) < len(e.tokens):
-                    raise ValueError(f"request {e.request!r}: wanted place {w} is not among its {len(e.tokens)} tokens")
+            if min(e.tokens) < 0 or max(e.tokens) >= self.vocab_size:
+                bad = [t for t in e.tokens if not 0 <= int(t) < self.vocab_size][0]
+                raise ValueError(f"request {e.request!r}: token {bad} is outside the vocabulary of {self.vocab_size}")
+            if e.want and (min(e.want) < 0 or max(e.want) >= len(e.tokens)):
+                bad = [w for w in e.want if not 0 <= int(w) < len(e.tokens)][0]
+                raise ValueError(f"request {e.request!r}: wanted place {bad} is not among its {len(e.tokens)} tokens")
         opened = []
         try:
             for e in entries:

@@ -59,23 +59,31 @@ class DecodeGraph:
         self.graph: Optional[torch.cuda.CUDAGraph] = None
         self.logits: Optional[torch.Tensor] = None
         self.copied: Optional[torch.cuda.Event] = None
+        self.row_marks = [None] * n
 
     def fill(self, entries, requests) -> None:
         n, h = self.n, self.host_np
         if self.copied is not None:
             self.copied.synchronize()     # the copy of the step before has left the pinned buffer
-        h[0:n] = [int(e.tokens[0]) for e in entries]
-        lengths = np.fromiter((r.length for r in requests), dtype=np.int32, count=n)
+        h[0:n] = [e.tokens[0] for e in entries]
+        lengths = [r.length for r in requests]
         h[n:2 * n] = lengths
-        h[2 * n:3 * n] = lengths + 1
+        h[2 * n:3 * n] = h[n:2 * n] + 1
         h[3 * n:4 * n] = [r.slot for r in requests]
-        at = 4 * n
-        for g in range(self.groups):
-            block = h[at:at + n * self.max_blocks].reshape(n, self.max_blocks)
-            for i, r in enumerate(requests):
-                block[i] = r.rows[g]
-            at += n * self.max_blocks
-        self.dev[:self.var_ints].copy_(self.host[:self.var_ints], non_blocking=True)
+        # a row of a block table changes only when its request got a page (or another request
+        # took the row): only then is it written again, and only then are the tables copied
+        changed = False
+        for i, r in enumerate(requests):
+            mark = (r.id, r.table_version)
+            if self.row_marks[i] != mark:
+                self.row_marks[i] = mark
+                changed = True
+                at = 4 * n + i * self.max_blocks
+                for g in range(self.groups):
+                    h[at:at + self.max_blocks] = r.rows[g]
+                    at += n * self.max_blocks
+        upto = self.var_ints if changed else 4 * n
+        self.dev[:upto].copy_(self.host[:upto], non_blocking=True)
         self.copied = torch.cuda.Event()
         self.copied.record()
 

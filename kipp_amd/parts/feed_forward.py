@@ -45,5 +45,5 @@ class GatedMLP:
         if self.w_gate_up.dtype == x.dtype == torch.bfloat16 and rows <= 16 and rt.ops.gemm_skinny_ok(rows, x.shape[1]):
             rt.ops.gemm_skinny_swiglu(x, self.w_gate_up, act)      # both products and the activation in one kernel
         else:
-            rt.ops.swiglu(rt.linear(x, self.w_gate_up, slabs=True), act)
+            rt.ops.swiglu(rt.linear(x, self.w_gate_up, slabs=True, low_precision_out=True), act)
         return rt.linear(act, self.w_down, slabs=True)

@@ -57,11 +57,13 @@ class Runtime:
         return torch.empty(shape, dtype=dtype, device=self.device)
 
     # -- matrix product ------------------------------------------------------
-    def linear(self, x: torch.Tensor, w: torch.Tensor, slabs: bool = False) -> torch.Tensor:
+    def linear(self, x: torch.Tensor, w: torch.Tensor, slabs: bool = False, low_precision_out: bool = False) -> torch.Tensor:
         """float32 [M, N] = x [M, K] . w [N, K]^T.  With `slabs` the result may come
         as [parts, M, N] whose sum over parts is the product (few rows against a
         weight with few output rows: the contraction is split over workgroups and
-        the consumer adds the slabs in order)."""
+        the consumer adds the slabs in order).  With `low_precision_out` a large
+        bfloat16 product may be returned in bfloat16 (for a consumer that rounds to
+        bfloat16 anyway and is bound by reading it)."""
         m = x.shape[0]
         n = w.shape[0]
         if w.dtype == torch.float32:
@@ -85,6 +87,8 @@ class Runtime:
                 self._mm_out_f32 = True
             except (RuntimeError, TypeError):
                 self._mm_out_f32 = False
+        if low_precision_out:
+            return torch.mm(x, w.t())
         if self._mm_out_f32:
             return torch.mm(x, w.t(), out_dtype=torch.float32)
         y = torch.mm(x, w.t())

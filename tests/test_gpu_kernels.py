@@ -63,7 +63,7 @@ def test_rmsnorm_reference_vector():
     assert np.allclose(got, np.array([3.0, 4.0]) / math.sqrt(12.5), rtol=1e-6)
 
 
-@pytest.mark.parametrize("inner,rows", [(1, 1), (200, 7), (9728, 2)])
+@pytest.mark.parametrize("inner,rows", [(1, 1), (200, 7), (9728, 2), (204, 3)])
 def test_swiglu(inner, rows):
     ops = _ops()
     rng = np.random.default_rng(inner)
@@ -71,6 +71,10 @@ def test_swiglu(inner, rows):
     ref = plain.silu(gu[:, :inner].astype(np.float64)) * gu[:, inner:]
     got = ops.swiglu(_t(gu), torch.empty(rows, inner, device=DEV))
     assert _rel(got.cpu().numpy(), ref) < 1e-12
+    gub = torch.tensor(gu).bfloat16()
+    refb = plain.silu(gub[:, :inner].double().numpy()) * gub[:, inner:].double().numpy()
+    got = ops.swiglu(gub.to(DEV), torch.empty(rows, inner, dtype=torch.bfloat16, device=DEV))
+    assert _rel(got.float().cpu().numpy(), refb) < 1e-5
     # /root/reference/tests/kipp_test.c:130-132
     got = ops.swiglu(_t([[0.0, 1.0, 5.0, 2.0]]), torch.empty(1, 2, device=DEV)).cpu().numpy()[0]
     assert abs(got[0]) < 1e-7 and abs(got[1] - 1.4621172) < 1e-6
