@@ -211,6 +211,21 @@ class CacheManager:
                 if page >= 0:
                     g.pool.release(page)
 
+    def truncate(self, req: RequestCache, length: int) -> None:
+        """Keep only the first `length` tokens of the request; pages above them go
+        back (/root/reference/src/kipp.c:3739-3774).  Pages adopted from the index are
+        shared and complete, so a request is never cut below them; a windowed group
+        or a state slot cannot be rolled back."""
+        if not 0 <= length <= req.length:
+            raise ValueError(f"cannot truncate {req.length} tokens to {length}")
+        if self.state_needs or any(g.need.window is not None for g in self.groups):
+            raise NotImplementedError("truncation needs every group to keep all keys and no per-request state")
+        if length < req.adopted_tokens:
+            raise ValueError(f"cannot truncate below the {req.adopted_tokens} adopted tokens")
+        req.length = length
+        del req.tokens[length:]
+        self.trim(req)
+
     def commit(self, req: RequestCache, tokens: Sequence[int]) -> None:
         """The step ran: the request now holds `tokens` more.  Pages that a
         window has passed are given back."""

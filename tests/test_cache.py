@@ -164,6 +164,37 @@ def test_prefix_adoption_through_the_manager():
     m.check()
 
 
+def test_truncate_gives_back_the_pages_above_and_never_the_adopted_ones():
+    # /root/reference/src/kipp.c:3739-3774: only the private tail is released
+    m = _manager()
+    toks = list(range(30))
+    a = m.open("a")
+    m.reserve([(a, 30)])
+    m.commit(a, toks)
+    assert m.free_pages() == [4]
+    m.truncate(a, 9)                                      # into the third page
+    assert a.length == 9 and a.tokens == toks[:9] and len([p for p in a.tables[0] if p >= 0]) == 3
+    assert m.free_pages() == [9]
+    m.check()
+    m.reserve([(a, 8)])
+    m.commit(a, toks[9:17])
+    m.close("a")                                          # publishes four full pages of the new timeline
+    b = m.open("b", toks)
+    assert b.length == 16
+    with pytest.raises(ValueError):
+        m.truncate(b, 12)                                 # adopted pages are shared
+    with pytest.raises(ValueError):
+        m.truncate(b, 17)
+    m.truncate(b, 16)
+    m.close("b")
+    assert m.free_pages() == [12]
+    m.check()
+    for other in (_manager(window=6, share=False), _manager(states=True)):
+        r = other.open("r")
+        with pytest.raises(NotImplementedError):
+            other.truncate(r, 0)
+
+
 def test_slots():
     m = _manager(states=True, max_requests=2)
     a, b = m.open("a"), m.open("b")

@@ -1,0 +1,131 @@
+"""The session interface, after the reference's gates for its cached path
+(/root/reference/tests/kipp_test.c:2488-2730, 1684-2026): every check there that
+does not need the pinned checkpoint, against the plain implementation."""
+import numpy as np
+import pytest
+
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def model(model_folders):
+    from kipp_amd.api import Model
+    m = Model.open(model_folders[("b", "float32")], dtype="float32", kv_pool_blocks=64, page_tokens=8)
+    yield m
+    assert not m.sessions
+    m.close()
+
+
+@pytest.fixture(scope="module")
+def reference(model_folders):
+    toks = H.random_tokens(50, 96, 509)            # three pages and more
+    return toks, H.plain_logits(model_folders[("b", "float32")], toks)
+
+
+def test_cached_decode_equals_recompute_at_every_position(model, reference):
+    toks, ref = reference
+    s = model.session_create(len(toks))
+    for i, t in enumerate(toks[:40]):
+        H.assert_close(s.eval([t])[None], ref[i:i + 1], H.NMSE_F32, f"position {i}")
+    assert s.get_info().length == 40
+    s.destroy()
+
+
+def test_multi_token_prefill_equals_token_by_token_and_rows_are_bitwise(model, reference):
+    toks, ref = reference
+    a, b = model.session_create(96), model.session_create(96)
+    whole = a.eval_n(toks, 96)
+    H.assert_close(whole, ref, H.NMSE_F32, "eval_n")
+    singles = np.stack([b.eval([t]) for t in toks])
+    assert np.array_equal(whole, singles)          # rows reproduce single-token evaluation bit for bit
+    a.destroy()
+    b.destroy()
+
+
+def test_capacity_and_argument_checks(model, reference):
+    from kipp_amd.api import ERROR_ARGUMENT, ERROR_RANGE, KippError
+    toks, _ = reference
+    for bad in (0, 257):
+        with pytest.raises(KippError) as e:
+            model.session_create(bad)
+        assert e.value.code == ERROR_RANGE
+    s = model.session_create(10)
+    with pytest.raises(KippError) as e:
+        s.eval([])
+    assert e.value.code == ERROR_ARGUMENT
+    s.eval(toks[:10])                              # exactly the capacity
+    with pytest.raises(KippError) as e:
+        s.eval([1])
+    assert e.value.code == ERROR_RANGE and s.length == 10
+    with pytest.raises(KippError) as e:
+        s.eval_n(toks[:0] + [1], 2)
+    t = model.session_create(4)
+    with pytest.raises(KippError):
+        t.eval([509])                              # outside the vocabulary
+    assert t.length == 0
+    with pytest.raises(KippError):
+        model.close()                              # sessions are alive
+    s.destroy()
+    t.destroy()
+    s.destroy()                                    # twice is harmless
+
+
+def test_reset_truncate_resume_and_independence(model, reference):
+    toks, ref = reference
+    s, other = model.session_create(96), model.session_create(96)
+    other.eval(H.random_tokens(7, 30, 509))        # a neighbour must not disturb s
+    s.eval(toks[:70])
+    s.truncate(37)                                 # in the middle of a page
+    assert s.length == 37
+    other.eval([3])
+    H.assert_close(s.eval_n(toks[37:60], 23), ref[37:60], H.NMSE_F32, "truncate and resume")
+    s.reset()
+    assert s.length == 0
+    H.assert_close(s.eval_n(toks[:20], 20), ref[:20], H.NMSE_F32, "after reset")
+    from kipp_amd.api import KippError
+    with pytest.raises(KippError):
+        s.truncate(21)
+    s.destroy()
+    other.destroy()
+
+
+def test_batch_of_sessions_equals_isolated_and_rejects_duplicates(model, reference):
+    from kipp_amd.api import KippError
+    toks, ref = reference
+    a, b, c = (model.session_create(96) for _ in range(3))
+    a.eval(toks[:33])
+    b.eval(toks[:7])
+    got = model.eval_batch([(a, toks[33:34]), (b, toks[7:40]), (c, toks[:61])])
+    for row, upto in zip(got, (34, 40, 61)):
+        H.assert_close(row[None], ref[upto - 1:upto], H.NMSE_F32, f"batch item ending at {upto}")
+    with pytest.raises(KippError):
+        model.eval_batch([(a, [1]), (a, [2])])
+    assert a.length == 34
+    for s in (a, b, c):
+        s.destroy()
+
+
+def test_published_prefix_is_adopted_and_a_small_pool_fails_cleanly(model_folders, reference):
+    from kipp_amd.api import ERROR_RANGE, KippError, Model
+    toks, ref = reference
+    m = Model.open(model_folders[("b", "float32")], dtype="float32", kv_pool_blocks=13, page_tokens=8)
+    a = m.session_create(96)
+    a.eval(toks[:70])
+    a.destroy()                                    # publishes 8 full pages
+    b = m.session_create(96)
+    assert b.match_prefix(toks) == 64
+    H.assert_close(b.eval_n(toks[64:90], 26), ref[64:90], H.NMSE_F32, "adopted prefix")
+    assert m.kv_pool_stats().reused_pages_total >= 8
+    c = m.session_create(96)                       # 12 of 13 pages are held: a long prompt cannot fit
+    with pytest.raises(KippError) as e:
+        c.eval(toks[:30])
+    assert e.value.code == ERROR_RANGE and c.length == 0
+    H.assert_close(b.eval_n(toks[90:96], 6), ref[90:96], H.NMSE_F32, "neighbour unharmed")
+    c.eval(toks[:8])                               # one page still fits
+    for s in (b, c):
+        s.destroy()
+    stateless = m.eval(toks[:20])
+    H.assert_close(stateless[None], ref[19:20], H.NMSE_F32, "stateless evaluation")
+    m.close()
