@@ -52,6 +52,9 @@ class RequestCache:
     adopted_tokens: int = 0
     rows: List[np.ndarray] = field(default_factory=list)    # per group: the table as the device sees it (int32, given-back pages 0)
     table_version: int = 0                                  # counts changes of `rows`
+    publish_early: bool = False                             # full pages are published as soon as they are committed
+    published: int = 0                                      # leading blocks that are adopted or published
+    chain: int = 0                                          # chained hash after `published` blocks
 
 
 class CacheGroup:
@@ -127,9 +130,15 @@ class CacheManager:
         return self.states.get(run)
 
     # -- requests ------------------------------------------------------------------
-    def open(self, request_id, prompt: Optional[Sequence[int]] = None) -> RequestCache:
+    def open(self, request_id, prompt: Optional[Sequence[int]] = None, publish_early: bool = False) -> RequestCache:
         """Claim a slot (its state zeroed) and, where sharing is on and `prompt`
-        is given, adopt the pages of its longest known beginning."""
+        is given, adopt the pages of its longest known beginning.
+
+        The reference publishes a session's pages when it ends, which keeps
+        truncation sound (/root/reference/src/kipp.c:3647-3670).  A request that
+        will never be truncated may set `publish_early`: its pages are published
+        as soon as they are full, so that requests running beside it can adopt
+        them; it can then no longer be cut below them."""
         if request_id in self.requests:
             raise ValueError(f"request {request_id!r} is already open")
         if not self.free_slots:
@@ -152,8 +161,16 @@ class CacheManager:
             req.adopted_tokens = keep * self.page_size
             req.length = req.adopted_tokens
             req.tokens = [int(t) for t in prompt[:req.length]]
+            req.published, req.chain = keep, matches[0][1] if keep == len(matches[0][0]) else self._chain(req.tokens)
+        req.publish_early = publish_early and self.share
         self.requests[request_id] = req
         return req
+
+    def _chain(self, tokens: Sequence[int]) -> int:
+        parent = 0
+        for block in range(len(tokens) // self.page_size):
+            parent = self.groups[0].pool._hash(parent, tokens[block * self.page_size:(block + 1) * self.page_size])
+        return parent
 
     def pages_needed(self, req: RequestCache, new_length: int) -> List[int]:
         """Pages each group still has to claim so that positions < new_length have one."""
@@ -220,8 +237,9 @@ class CacheManager:
             raise ValueError(f"cannot truncate {req.length} tokens to {length}")
         if self.state_needs or any(g.need.window is not None for g in self.groups):
             raise NotImplementedError("truncation needs every group to keep all keys and no per-request state")
-        if length < req.adopted_tokens:
-            raise ValueError(f"cannot truncate below the {req.adopted_tokens} adopted tokens")
+        floor = max(req.adopted_tokens, req.published * self.page_size)
+        if length < floor:
+            raise ValueError(f"cannot truncate below the {floor} adopted or published tokens")
         req.length = length
         del req.tokens[length:]
         self.trim(req)
@@ -231,6 +249,13 @@ class CacheManager:
         window has passed are given back."""
         req.tokens.extend(int(t) for t in tokens)
         req.length += len(tokens)
+        if req.publish_early:
+            while (req.published + 1) * self.page_size <= req.length:
+                block = req.published
+                chunk = req.tokens[block * self.page_size:(block + 1) * self.page_size]
+                for g in self.groups:
+                    h = g.pool.seal(req.tables[g.index][block], req.chain, chunk)
+                req.chain, req.published = h, block + 1
         for g in self.groups:
             window = g.need.window
             if window is None:

@@ -103,6 +103,118 @@ __global__ void qk_norm_rope_kv_kernel(
     }
 }
 
+// The same for head sizes of 128 and 256 rotated over their whole width: element
+// i and its partner i + d/2 then lie in the same lane (lane i % 64 holds elements
+// i % 64 + 64 c), so nothing passes through LDS; a wave takes several heads of one
+// token, four at a time with all their loads issued first, and computes the
+// token's sines and cosines once for all of them.
+template <int NC, bool SLABS, typename TI, typename TO, typename TC>
+__global__ void __launch_bounds__(HEADS_PER_BLOCK * KIPP_WAVE) qk_norm_rope_kv_regs_kernel(
+    const TI* __restrict__ qkv, TO* __restrict__ q_out, TC* __restrict__ k_cache, TC* __restrict__ v_cache,
+    const int32_t* __restrict__ positions, const int32_t* __restrict__ seq_of_token,
+    const int32_t* __restrict__ block_table, int max_blocks,
+    const float* __restrict__ q_norm_w, const float* __restrict__ k_norm_w, float eps,
+    const float* __restrict__ inv_freq, int n_q, int n_kv, int page, int n_slots, int parts, size_t part_stride) {
+    constexpr int D = NC * KIPP_WAVE, HC = NC / 2, BATCH = 4;
+    const int wave = threadIdx.x / KIPP_WAVE;
+    const int lane = threadIdx.x & (KIPP_WAVE - 1);
+    const int t = blockIdx.y;
+    const int waves = gridDim.x * HEADS_PER_BLOCK;
+    const int pos = positions[t];
+    const size_t row = (size_t)t * (n_q + 2 * n_kv) * D;
+
+    float cs[HC], sn[HC], qw[NC], kw[NC];
+#pragma unroll
+    for (int c = 0; c < HC; ++c) {
+        cs[c] = 1.0f;
+        sn[c] = 0.0f;
+        if (inv_freq != nullptr) {
+            const float angle = (float)pos * inv_freq[lane + c * KIPP_WAVE];
+            cs[c] = cosf(angle);
+            sn[c] = sinf(angle);
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+        qw[c] = q_norm_w != nullptr ? q_norm_w[lane + c * KIPP_WAVE] : 1.0f;
+        kw[c] = k_norm_w != nullptr ? k_norm_w[lane + c * KIPP_WAVE] : 1.0f;
+    }
+    size_t cache_row = 0;
+    if (n_slots > n_q) {
+        const int page_id = block_table[(size_t)seq_of_token[t] * max_blocks + pos / page];
+        cache_row = (size_t)page_id * n_kv * page + pos % page;
+    }
+
+    for (int s0 = blockIdx.x * HEADS_PER_BLOCK + wave; s0 < n_slots; s0 += waves * BATCH) {
+        float v[BATCH][NC];
+#pragma unroll
+        for (int u = 0; u < BATCH; ++u) {
+            const int slot = min(s0 + u * waves, n_slots - 1);
+            const TI* src = qkv + row + (size_t)slot * D + lane;
+#pragma unroll
+            for (int c = 0; c < NC; ++c) {
+                v[u][c] = load_f(src, c * KIPP_WAVE);
+                if (SLABS)
+                    for (int p = 1; p < parts; ++p) v[u][c] += load_f(src, p * part_stride + c * KIPP_WAVE);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < BATCH; ++u) {
+            const int slot = s0 + u * waves;
+            if (slot >= n_slots) break;
+            const int kind = slot < n_q ? 0 : (slot < n_q + n_kv ? 1 : 2);
+            if (kind != 2) {
+                if ((kind == 0 ? q_norm_w : k_norm_w) != nullptr) {
+                    float ss = 0.0f;
+#pragma unroll
+                    for (int c = 0; c < NC; ++c) ss += v[u][c] * v[u][c];
+                    ss = wave_sum(ss);
+                    const float scale = 1.0f / sqrtf(ss / (float)D + eps);
+#pragma unroll
+                    for (int c = 0; c < NC; ++c) v[u][c] *= scale * (kind == 0 ? qw[c] : kw[c]);
+                }
+#pragma unroll
+                for (int c = 0; c < HC; ++c) {
+                    const float a = v[u][c], b = v[u][c + HC];
+                    v[u][c] = a * cs[c] - b * sn[c];
+                    v[u][c + HC] = b * cs[c] + a * sn[c];
+                }
+            }
+            if (kind == 0) {
+                TO* dst = q_out + ((size_t)t * n_q + slot) * D + lane;
+#pragma unroll
+                for (int c = 0; c < NC; ++c) store_f(dst, c * KIPP_WAVE, v[u][c]);
+            } else {
+                const int head = kind == 1 ? slot - n_q : slot - n_q - n_kv;
+                TC* dst = (kind == 1 ? k_cache : v_cache) + (cache_row + (size_t)head * page) * D + lane;
+#pragma unroll
+                for (int c = 0; c < NC; ++c) store_f(dst, c * KIPP_WAVE, v[u][c]);
+            }
+        }
+    }
+}
+
+template <typename TI, typename TO, typename TC>
+static void launch_regs(const void* qkv, void* q_out, void* k_cache, void* v_cache, const int32_t* positions,
+                        const int32_t* seq_of_token, const int32_t* block_table, int max_blocks, const float* q_norm_w,
+                        const float* k_norm_w, float eps, const float* inv_freq, int n_tokens, int n_q, int n_kv, int d,
+                        int page, int n_slots, int parts, hipStream_t stream) {
+    // few tokens: a wave for every head; many: a workgroup for a token
+    const int per_token = n_tokens >= 256 ? 1 : (n_slots + HEADS_PER_BLOCK - 1) / HEADS_PER_BLOCK;
+    dim3 grid(per_token, n_tokens), block(HEADS_PER_BLOCK * KIPP_WAVE);
+    const size_t stride = (size_t)n_tokens * (n_q + 2 * n_kv) * d;
+#define KIPP_RR(NC, SLABS)                                                                                          \
+    hipLaunchKernelGGL((qk_norm_rope_kv_regs_kernel<NC, SLABS, TI, TO, TC>), grid, block, 0, stream, (const TI*)qkv, \
+                       (TO*)q_out, (TC*)k_cache, (TC*)v_cache, positions, seq_of_token, block_table, max_blocks,     \
+                       q_norm_w, k_norm_w, eps, inv_freq, n_q, n_kv, page, n_slots, parts, stride)
+    if (d == 128) {
+        if (parts > 1) KIPP_RR(2, true); else KIPP_RR(2, false);
+    } else {
+        if (parts > 1) KIPP_RR(4, true); else KIPP_RR(4, false);
+    }
+#undef KIPP_RR
+}
+
 extern "C" int kipp_qk_norm_rope_kv(
     const void* qkv, int in_dtype, void* q_out, int q_dtype, void* k_cache, void* v_cache, int cache_dtype,
     const int32_t* positions, const int32_t* seq_of_token, const int32_t* block_table, int max_blocks,
@@ -111,6 +223,17 @@ extern "C" int kipp_qk_norm_rope_kv(
     if (n_tokens <= 0) return 0;
     if (d > MAX_D || d <= 0 || rotary_dim > d || (rotary_dim & 1)) return -1;
     const int n_slots = write_kv ? n_q + 2 * n_kv : n_q;
+    if ((d == 128 || d == 256) && (inv_freq == nullptr || rotary_dim == d)) {
+#define KIPP_RL(TI, TO, TC)                                                                                        \
+    launch_regs<TI, TO, TC>(qkv, q_out, k_cache, v_cache, positions, seq_of_token, block_table, max_blocks, q_norm_w, \
+                            k_norm_w, eps, inv_freq, n_tokens, n_q, n_kv, d, page, n_slots, parts, stream)
+        if (in_dtype == KIPP_F32 && q_dtype == KIPP_F32 && cache_dtype == KIPP_F32) KIPP_RL(float, float, float);
+        else if (in_dtype == KIPP_F32 && q_dtype == KIPP_BF16 && cache_dtype == KIPP_BF16) KIPP_RL(float, bf16_t, bf16_t);
+        else if (in_dtype == KIPP_BF16 && q_dtype == KIPP_BF16 && cache_dtype == KIPP_BF16) KIPP_RL(bf16_t, bf16_t, bf16_t);
+        else return -2;
+#undef KIPP_RL
+        return KIPP_LAUNCH_CHECK();
+    }
     dim3 grid((n_slots + HEADS_PER_BLOCK - 1) / HEADS_PER_BLOCK, n_tokens), block(HEADS_PER_BLOCK * KIPP_WAVE);
 #define KIPP_RK(TI, TO, TC)                                                                                  \
     hipLaunchKernelGGL((qk_norm_rope_kv_kernel<TI, TO, TC>), grid, block, 0, stream, (const TI*)qkv,         \

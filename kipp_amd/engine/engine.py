@@ -46,8 +46,8 @@ class Engine:
         return cls(load_model(model_dir, Runtime(dtype, device)), **kw)
 
     # -- requests ---------------------------------------------------------------------
-    def open(self, request_id, prompt: Optional[Sequence[int]] = None):
-        return self.cache.open(request_id, prompt)
+    def open(self, request_id, prompt: Optional[Sequence[int]] = None, publish_early: bool = False):
+        return self.cache.open(request_id, prompt, publish_early)
 
     def close(self, request_id) -> None:
         self.cache.close(request_id)

@@ -6,6 +6,9 @@ Policy (the reference's server loop lifted out of its HTTP code,
 
 * Waiting requests are admitted strictly in arrival order; the first that does
   not fit blocks those behind it.
+* Requests publish their full pages as they go.  A waiting request whose prompt
+  begins like that of a request still running its prompt waits until those pages
+  are published and then adopts them instead of computing them again.
 * A request is refused at `add` if its prompt plus `max_new_tokens` exceeds the
   model's positions, or if it could never fit the page pool even alone.
 * Pages are reserved at admission: a request is admitted only if every pool
@@ -25,6 +28,8 @@ import time
 from collections import deque
 from dataclasses import dataclass, field
 from typing import Deque, Dict, List, Optional, Sequence, Tuple
+
+import numpy as np
 
 from ..sampling import SampleParams, XorShift64Star
 from .batch import StepEntry
@@ -72,6 +77,7 @@ class SchedulerStats:
     prefix_tokens_reused: int = 0
     steps: int = 0
     waits_for_pages: int = 0
+    waits_for_prefix: int = 0
 
 
 class Scheduler:
@@ -87,6 +93,7 @@ class Scheduler:
         self.running: List[Request] = []
         self.finished: Dict[object, Request] = {}
         self.stats = SchedulerStats()
+        self._common: Dict[Tuple[object, object], int] = {}
 
     # -- page arithmetic -----------------------------------------------------------
     def _pages(self, tokens: int) -> int:
@@ -139,10 +146,31 @@ class Scheduler:
         return not self.waiting and not self.running
 
     # -- admission ---------------------------------------------------------------------
+    def _worth_waiting(self, req: Request) -> bool:
+        """Is a running request about to publish pages that `req` could adopt?"""
+        if not self.cache.share:
+            return False
+        page = self.cache.page_size
+        for other in self.running:
+            if other.state != "prefill":
+                continue
+            key = (req.id, other.id)
+            if key not in self._common:
+                n = min(len(req.prompt) - 1, len(other.prompt))
+                a, b = np.asarray(req.prompt[:n]), np.asarray(other.prompt[:n])
+                differ = np.nonzero(a != b)[0]
+                self._common[key] = (int(differ[0]) if len(differ) else n) // page
+            if self._common[key] > other.fed // page:
+                return True
+        return False
+
     def _admit(self) -> None:
         while self.waiting and len(self.running) < self.max_running:
             req = self.waiting[0]
-            rc = self.cache.open(req.id, req.prompt)       # adopts the longest known beginning
+            if self._worth_waiting(req):
+                self.stats.waits_for_prefix += 1
+                return
+            rc = self.cache.open(req.id, req.prompt, publish_early=True)   # adopts the longest known beginning
             need = self.cache.pages_needed(rc, req.budget_tokens)
             promised = [0] * len(self.cache.groups)
             for other in self.running:
@@ -231,6 +259,7 @@ class Scheduler:
             self.engine.close(req.id)
         self.finished[req.id] = req
         self.stats.finished += 1
+        self._common = {k: v for k, v in self._common.items() if req.id not in k}
 
     def run(self, max_steps: Optional[int] = None) -> Dict[object, Request]:
         """Step until every request has finished."""

@@ -1,0 +1,148 @@
+"""Serving workloads through the scheduler, with random weights made on the
+device: requests of many lengths under continuous batching with prompts cut into
+portions, and requests that share a long beginning (paged prefix reuse).
+
+    python -m kipp_amd.workloads continuous    [--shape qwen3-8b]  [--requests 32] ...
+    python -m kipp_amd.workloads shared-prefix [--shape qwen3-32b] [--requests 8]  ...
+
+One JSON line: generated tokens a second over the whole run, prompt tokens a
+second, time to the first token, and what the cache reused.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import sys
+import time
+
+
+def log(msg: str) -> None:
+    print(f"workload: {msg}", file=sys.stderr, flush=True)
+
+
+def build_engine(shape: str, layers, context: int, pool_tokens: int, max_requests: int, seed: int = 1):
+    import torch
+    from .config import shape_config
+    from .engine import Engine, random_model
+    from .runtime import Runtime
+    config = shape_config(shape)
+    full = config["num_hidden_layers"]
+    if layers:
+        config["num_hidden_layers"] = min(layers, full)
+    config["max_position_embeddings"] = max(context, 64)
+    rt = Runtime("bfloat16", "cuda:0")
+    start = time.perf_counter()
+    model = random_model(config, seed, rt)
+    torch.cuda.synchronize()
+    log(f"{shape}: {config['num_hidden_layers']} of {full} layers made in {time.perf_counter() - start:.1f} s, "
+        f"{torch.cuda.memory_allocated() / 2**30:.1f} GiB")
+    engine = Engine(model, page_size=16, max_tokens=pool_tokens, max_requests=max_requests)
+    return engine, config, full
+
+
+def continuous_prompts(n: int, low: int, high: int, vocab: int, seed: int):
+    import torch
+    gen = torch.Generator().manual_seed(seed)
+    lengths = torch.randint(low, high + 1, (n,), generator=gen).tolist()
+    return [torch.randint(0, vocab, (length,), generator=gen).tolist() for length in lengths]
+
+
+def shared_prefix_prompts(n: int, prefix: int, suffix: int, vocab: int, seed: int):
+    import torch
+    gen = torch.Generator().manual_seed(seed)
+    head = torch.randint(0, vocab, (prefix,), generator=gen).tolist()
+    return [head + torch.randint(0, vocab, (suffix,), generator=gen).tolist() for _ in range(n)]
+
+
+def serve(engine, prompts, new_tokens: int, chunk: int, max_step_tokens: int):
+    """All requests arrive at once; runs until every one has finished."""
+    import torch
+    from .engine.scheduler import Request, Scheduler
+    sched = Scheduler(engine, max_step_tokens=max_step_tokens, prefill_chunk=chunk, max_running=len(prompts))
+    for i, prompt in enumerate(prompts):
+        sched.add(Request(i, prompt, new_tokens))
+    torch.cuda.synchronize()
+    start = time.perf_counter()
+    last = start
+    while not sched.idle:
+        sched.step()
+        now = time.perf_counter()
+        if now - last > 20:
+            log(f"step {sched.stats.steps}: {sched.stats.prompt_tokens} prompt tokens run, "
+                f"{sched.stats.generated_tokens} generated, {len(sched.running)} running, {len(sched.waiting)} waiting")
+            last = now
+    torch.cuda.synchronize()
+    seconds = time.perf_counter() - start
+    done = sched.finished
+    first = [r.first_token_at - r.arrived for r in done.values() if r.first_token_at is not None]
+    return sched, seconds, first
+
+
+def main(argv=None) -> int:
+    ap = argparse.ArgumentParser(prog="python -m kipp_amd.workloads", description=__doc__,
+                                 formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("workload", choices=["continuous", "shared-prefix"])
+    ap.add_argument("--shape", default=None, help="a name under kipp_amd/config/shapes (default: qwen3-8b / qwen3-32b)")
+    ap.add_argument("--layers", type=int, default=0, help="fewer layers than the shape has (0: all)")
+    ap.add_argument("--requests", type=int, default=None)
+    ap.add_argument("--new", type=int, default=None, help="tokens generated for each request")
+    ap.add_argument("--min-prompt", type=int, default=512)
+    ap.add_argument("--max-prompt", type=int, default=4096)
+    ap.add_argument("--prefix", type=int, default=6000)
+    ap.add_argument("--suffix", type=int, default=500)
+    ap.add_argument("--prefill-chunk", type=int, default=512)
+    ap.add_argument("--max-step-tokens", type=int, default=2048)
+    ap.add_argument("--context", type=int, default=None)
+    ap.add_argument("--seed", type=int, default=1)
+    ap.add_argument("--no-sharing", action="store_true", help="shared-prefix: compute every prompt in full, for comparison")
+    args = ap.parse_args(argv)
+
+    import torch
+    if not torch.cuda.is_available():
+        print("workload: no GPU", file=sys.stderr)
+        return 1
+    cont = args.workload == "continuous"
+    shape = args.shape or ("qwen3-8b" if cont else "qwen3-32b")
+    n = args.requests or (32 if cont else 8)
+    new = args.new or (128 if cont else 256)
+    context = args.context or (8192 if cont else 16384)
+    longest = args.max_prompt if cont else args.prefix + args.suffix
+    if longest + new > context:
+        print(f"workload: prompt {longest} + {new} new tokens exceed the context {context}", file=sys.stderr)
+        return 1
+    per_request = -(-(longest + new) // 64) * 64
+    engine, config, full_layers = build_engine(shape, args.layers, context, n * per_request, n, args.seed)
+    if args.no_sharing:
+        engine.cache.share = False
+    vocab = config["vocab_size"]
+    if cont:
+        prompts = continuous_prompts(n, args.min_prompt, args.max_prompt, vocab, args.seed)
+    else:
+        prompts = shared_prefix_prompts(n, args.prefix, args.suffix, vocab, args.seed)
+
+    warm = [p[:args.prefill_chunk + 3] for p in prompts[:2]]            # other tokens: nothing of it is adopted later
+    serve(engine, [[(t + 1) % vocab for t in p] for p in warm], 4, args.prefill_chunk, args.max_step_tokens)
+    sched, seconds, first = serve(engine, prompts, new, args.prefill_chunk, args.max_step_tokens)
+    st = sched.stats
+    prompt_tokens = sum(len(p) for p in prompts)
+    out = {
+        "workload": args.workload, "value": st.generated_tokens / seconds, "unit": "generated tokens/s",
+        "seconds": seconds, "requests": n, "generated_tokens": st.generated_tokens,
+        "prompt_tokens": prompt_tokens, "prompt_tokens_run": st.prompt_tokens,
+        "prefix_tokens_reused": st.prefix_tokens_reused,
+        "total_tokens_per_s": (prompt_tokens + st.generated_tokens) / seconds,
+        "steps": st.steps, "first_token_s_mean": sum(first) / max(1, len(first)), "first_token_s_max": max(first or [0.0]),
+        "dtype": "bf16", "data": "synthetic uniform-random tokens, random weights",
+        "config": {"model": shape, "layers": config["num_hidden_layers"], "layers_full": full_layers,
+                   "hidden": config["hidden_size"], "intermediate": config["intermediate_size"],
+                   "heads": config["num_attention_heads"], "kv_heads": config["num_key_value_heads"],
+                   "head_dim": config["head_dim"], "vocab": vocab, "context": context,
+                   "prefill_chunk": args.prefill_chunk, "max_step_tokens": args.max_step_tokens,
+                   "new_tokens": new, "kv_page": 16, "sharing": not args.no_sharing},
+    }
+    print(json.dumps(out), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

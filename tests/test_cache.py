@@ -195,6 +195,33 @@ def test_truncate_gives_back_the_pages_above_and_never_the_adopted_ones():
             other.truncate(r, 0)
 
 
+def test_early_publication_lets_a_neighbour_adopt_pages_of_a_running_request():
+    m = _manager()
+    toks = list(range(30))
+    a = m.open("a", toks, publish_early=True)
+    m.reserve([(a, 9)])
+    m.commit(a, toks[:9])                                 # two full pages are published at once
+    b = m.open("b", toks, publish_early=True)
+    assert b.length == 8 and b.tables[0] == a.tables[0][:2]
+    with pytest.raises(ValueError):
+        m.truncate(a, 7)                                  # published pages can no longer be cut
+    m.truncate(a, 8)
+    m.reserve([(a, 5), (b, 5)])                           # both compute the fourth page themselves
+    m.commit(a, toks[8:13])
+    m.commit(b, toks[8:13])
+    assert a.published == 3 and b.published == 3 and a.tables[0][2] != b.tables[0][2]
+    m.check()
+    c = m.open("c", toks)
+    assert c.length == 12 and c.tables[0][2] == a.tables[0][2]   # the first of the two copies is the indexed one
+    for r in "abc":
+        m.close(r)
+    assert m.free_pages() == [12]
+    m.check()
+    d = m.open("d", toks)                                 # published pages outlive their requests
+    assert d.length == 12
+    m.close("d")
+
+
 def test_slots():
     m = _manager(states=True, max_requests=2)
     a, b = m.open("a"), m.open("b")

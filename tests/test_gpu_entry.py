@@ -37,6 +37,29 @@ def test_greedy_generation_through_the_entry_point(model_folders, tiny_configs, 
         _follows_plain_argmax(model_folders[(key, dtype)], prompt, out, margin)
 
 
+@pytest.mark.parametrize("dtype,margin", [("float32", 1e-5), ("bfloat16", 0.03)])
+def test_requests_that_begin_alike_share_pages_and_still_follow_plain(model_folders, dtype, margin):
+    """Four requests with a common beginning of five pages arrive together: the
+    later ones adopt the pages the first one publishes while it is still
+    running, and every generated token is still the plain argmax."""
+    from kipp_amd.engine import Engine
+    from kipp_amd.engine.scheduler import Request, Scheduler
+    folder = model_folders[("b", dtype)]
+    common = H.random_tokens(61, 43, 509)
+    prompts = [common + H.random_tokens(62 + i, n, 509) for i, n in enumerate([5, 1, 17, 9])]
+    engine = Engine.from_folder(folder, dtype=dtype, page_size=8, max_tokens=4 * 128)
+    sched = Scheduler(engine, max_step_tokens=24, prefill_chunk=10)
+    for i, prompt in enumerate(prompts):
+        sched.add(Request(i, prompt, 12))
+    done = sched.run()
+    assert sched.stats.prefix_tokens_reused == 3 * 40 and sched.stats.prompt_tokens == sum(map(len, prompts)) - 120
+    for i, prompt in enumerate(prompts):
+        assert len(done[i].output) == 12
+        _follows_plain_argmax(folder, prompt, done[i].output, margin)
+    engine.cache.check()
+    assert engine.cache.free_pages() == [64]
+
+
 def test_long_decoding_matches_plain(model_folders, tiny_configs):
     """100 tokens decoded one by one after a short prompt, every logits row compared."""
     from kipp_amd.engine import Engine, StepEntry

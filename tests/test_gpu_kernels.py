@@ -185,7 +185,8 @@ def test_attention_reference_vector():
     assert np.allclose(out[0], 1.0) and np.allclose(out[1], 2.0)
 
 
-@pytest.mark.parametrize("n_q,n_kv,d,page,rotary", [(4, 2, 16, 16, 16), (3, 1, 48, 8, 48), (8, 2, 128, 16, 128), (2, 2, 64, 4, 32)])
+@pytest.mark.parametrize("n_q,n_kv,d,page,rotary", [(4, 2, 16, 16, 16), (3, 1, 48, 8, 48), (8, 2, 128, 16, 128), (2, 2, 64, 4, 32),
+                                                  (5, 1, 256, 16, 256), (9, 3, 128, 8, 128), (4, 2, 128, 16, 64)])
 @pytest.mark.parametrize("mode", ["f32", "bf16"])
 @pytest.mark.parametrize("norm", [True, False])
 def test_qk_norm_rope_kv_write(n_q, n_kv, d, page, rotary, mode, norm):
@@ -408,22 +409,23 @@ def test_gemm_rows(m, n, k, max_parts):
 
 
 def test_consumers_add_slabs_in_order():
-    """The rotary kernel and SwiGLU take a product that comes in slabs."""
+    """The rotary kernels and SwiGLU take a product that comes in slabs."""
     ops = _ops()
     rng = np.random.default_rng(12)
-    n_q, n_kv, d, page, t = 4, 2, 32, 8, 5
-    slabs = rng.normal(size=(3, t, (n_q + 2 * n_kv) * d)).astype(np.float32)
-    whole = slabs[0] + slabs[1] + slabs[2]
-    table = np.arange(4, dtype=np.int32).reshape(1, 4)
-    inv_freq = np.power(1e4, -(2.0 * np.arange(d // 2)) / d).astype(np.float32)
-    outs = []
-    for qkv in (slabs, whole):
-        k, v = torch.zeros(4, n_kv, page, d, device=DEV), torch.zeros(4, n_kv, page, d, device=DEV)
-        q = ops.qk_norm_rope_kv_write(_t(qkv), torch.empty(t, n_q * d, device=DEV), k, v, _t(np.arange(t), torch.int32),
-                                      _t(np.zeros(t), torch.int32), _t(table, torch.int32), n_q, n_kv, d,
-                                      _t(np.ones(d)), _t(np.ones(d)), 1e-6, _t(inv_freq), d)
-        outs.append((q.cpu(), k.cpu(), v.cpu()))
-    assert all(torch.equal(a, b) for a, b in zip(*outs))
+    for d in (32, 128):                                    # through LDS, and in registers
+        n_q, n_kv, page, t = 4, 2, 8, 5
+        slabs = rng.normal(size=(3, t, (n_q + 2 * n_kv) * d)).astype(np.float32)
+        whole = slabs[0] + slabs[1] + slabs[2]
+        table = np.arange(4, dtype=np.int32).reshape(1, 4)
+        inv_freq = np.power(1e4, -(2.0 * np.arange(d // 2)) / d).astype(np.float32)
+        outs = []
+        for qkv in (slabs, whole):
+            k, v = torch.zeros(4, n_kv, page, d, device=DEV), torch.zeros(4, n_kv, page, d, device=DEV)
+            q = ops.qk_norm_rope_kv_write(_t(qkv), torch.empty(t, n_q * d, device=DEV), k, v, _t(np.arange(t), torch.int32),
+                                          _t(np.zeros(t), torch.int32), _t(table, torch.int32), n_q, n_kv, d,
+                                          _t(np.ones(d)), _t(np.ones(d)), 1e-6, _t(inv_freq), d)
+            outs.append((q.cpu(), k.cpu(), v.cpu()))
+        assert all(torch.equal(a, b) for a, b in zip(*outs))
     gu = rng.normal(size=(4, 6, 2 * 40)).astype(np.float32)
     a = ops.swiglu(_t(gu), torch.empty(6, 40, device=DEV)).cpu()
     b = ops.swiglu(_t(gu[0] + gu[1] + gu[2] + gu[3]), torch.empty(6, 40, device=DEV)).cpu()

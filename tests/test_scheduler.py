@@ -160,6 +160,24 @@ def test_known_beginnings_are_adopted():
     assert done["b"].output == expected_output(prompt[:10] + [40, 41], 2)
 
 
+def test_requests_that_begin_alike_wait_for_the_first_and_adopt_its_pages():
+    eng = FakeEngine(num_pages=32, page_size=4, max_requests=4, share=True)
+    s = Scheduler(eng, max_step_tokens=16, prefill_chunk=6)
+    common = list(range(1, 22))                            # five full pages and one token
+    prompts = {"a": common + [30, 31], "b": common + [40], "c": [9] + common, "d": common[:9] + [45, 46, 47]}
+    for rid, prompt in prompts.items():
+        s.add(Request(rid, prompt, 3))
+    done = s.run()
+    for rid, prompt in prompts.items():
+        assert done[rid].output == expected_output(prompt, 3), rid
+    # b waited until a had published the five pages they share, c (another first token) shares nothing,
+    # d shares two pages
+    assert s.stats.prefix_tokens_reused == 20 + 8 and s.stats.waits_for_prefix > 0
+    assert s.stats.prompt_tokens == sum(len(p) for p in prompts.values()) - 28
+    assert all(("b", n, w) not in call for call in eng.calls[:3] for n in range(8) for w in ([], [0]))
+    assert eng.cache.free_pages() == [32]
+
+
 def test_cancel_and_zero_new_tokens():
     eng = FakeEngine()
     s = Scheduler(eng)
