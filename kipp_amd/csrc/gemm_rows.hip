@@ -28,7 +28,10 @@ union Frag {
     bf16x8 v;
 };
 
-template <int MT, int TW>
+// TILED: W in the streaming layout [tile of 16 rows][step of 32 columns][lane][8 values]
+// (rows padded to whole tiles with zeros, K a multiple of 32), in which a wave's load is
+// one contiguous KB.
+template <int MT, int TW, bool TILED>
 __global__ void __launch_bounds__(TW * KIPP_WAVE) gemm_rows_kernel(
     const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, float* __restrict__ Y, int M, int N, int K) {
     constexpr int THREADS = TW * KIPP_WAVE;
@@ -46,7 +49,8 @@ __global__ void __launch_bounds__(TW * KIPP_WAVE) gemm_rows_kernel(
     const int g_end = (int)((long long)groups * (part + 1) / parts);
 
     const int row = min(n0 + l16, N - 1);                      // clamped: in bounds, dropped at the store
-    const bf16_t* w_row = W + (size_t)row * K + 8 * h;
+    const bf16_t* w_row = TILED ? W + (size_t)min(n0 >> 4, (N + 15) / 16 - 1) * (K / 32) * 512 + lane * 8
+                                : W + (size_t)row * K + 8 * h;
 
     // the units of X this thread stages: unit -> (row, 8-column chunk)
     const bf16_t* x_src[XR];
@@ -65,7 +69,7 @@ __global__ void __launch_bounds__(TW * KIPP_WAVE) gemm_rows_kernel(
     Frag wf[DEPTH];
     u32x4 xr[XR];
 
-    auto fetch_w = [&](int u, int step) { wf[u].u = *(const u32x4*)(w_row + 32 * step); };
+    auto fetch_w = [&](int u, int step) { wf[u].u = *(const u32x4*)(w_row + (TILED ? 512 : 32) * step); };
     auto fetch_x = [&](int g) {
 #pragma unroll
         for (int i = 0; i < XR; ++i) xr[i] = *(const u32x4*)(x_src[i] + (size_t)g * CHUNK);
@@ -109,7 +113,7 @@ __global__ void __launch_bounds__(TW * KIPP_WAVE) gemm_rows_kernel(
             const bool ok = k + 8 * h < K;
             Frag w_t;
             w_t.u = (u32x4){0u, 0u, 0u, 0u};
-            if (ok) w_t.u = *(const u32x4*)(w_row + k);
+            if (ok) w_t.u = *(const u32x4*)(w_row + (TILED ? 16 * k : k));
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
                 Frag x_t;
@@ -157,17 +161,25 @@ int kipp_gemm_rows_parts(int N, int K, int max_parts) {
 }
 
 // Y: float32 [parts, M, N] with parts = kipp_gemm_rows_parts(N, K, max_parts).
-// M <= 64, K a multiple of 8.
-int kipp_gemm_rows(const void* X, const void* W, float* Y, int M, int N, int K, int max_parts, hipStream_t stream) {
+// M <= 64, K a multiple of 8; `tiled`: W in the streaming layout (K a multiple of 32).
+int kipp_gemm_rows(const void* X, const void* W, float* Y, int M, int N, int K, int max_parts, int tiled,
+                   hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
-    if (M > 64 || K <= 0 || (K & 7) || max_parts <= 0) return -1;
+    if (M > 64 || K <= 0 || (K & 7) || max_parts <= 0 || (tiled && (K & 31))) return -1;
     int tw, parts;
     plan(N, K, max_parts, &tw, &parts);
     const int tiles = (N + 15) / 16;
     dim3 grid((tiles + tw - 1) / tw, parts), block(tw * KIPP_WAVE);
     const int mt = (M + 15) / 16;
-#define KIPP_GR(MT, TW) \
-    hipLaunchKernelGGL((gemm_rows_kernel<MT, TW>), grid, block, 0, stream, (const bf16_t*)X, (const bf16_t*)W, Y, M, N, K)
+#define KIPP_GR(MT, TW)                                                                                             \
+    do {                                                                                                            \
+        if (tiled)                                                                                                  \
+            hipLaunchKernelGGL((gemm_rows_kernel<MT, TW, true>), grid, block, 0, stream, (const bf16_t*)X,          \
+                               (const bf16_t*)W, Y, M, N, K);                                                       \
+        else                                                                                                        \
+            hipLaunchKernelGGL((gemm_rows_kernel<MT, TW, false>), grid, block, 0, stream, (const bf16_t*)X,         \
+                               (const bf16_t*)W, Y, M, N, K);                                                       \
+    } while (0)
     if (tw == 8) {
         switch (mt) {
             case 1: KIPP_GR(1, 8); break;

@@ -16,6 +16,13 @@
 // B = X^T (lane: token l % 16, same k), D: lane holds features 4 (l / 16) + v of
 // token l % 16, i.e. 16 contiguous bytes of a Y row.
 //
+// TILED: W comes in the streaming layout, in which the 1 KB that a wave reads in
+// one step (16 rows x 32 columns) is contiguous: [tile of 16 rows][step of 32
+// columns][lane][8 values], lane l holding row l % 16, columns 8 (l / 16) .. + 7 of
+// the step; rows are padded to whole tiles with zeros and K is a multiple of 32.
+// Every request then covers full memory lines, which a compute unit issues at a
+// bounded rate: the same kernel streams a fifth faster than from [N, K] rows.
+//
 // With SWIGLU the weight is [gate rows; up rows] ([2 I, K]); a wave computes the
 // gate tile and the matching up tile together and writes
 // silu(gate) * up as bfloat16 [M, I]  (/root/reference/src/kipp.c:2644-2648).
@@ -33,7 +40,7 @@ union Frag {
     bf16x8 v;
 };
 
-template <int MT, bool SWIGLU, int KW, int DEPTH>
+template <int MT, bool SWIGLU, int KW, int DEPTH, bool TILED>
 __global__ void __launch_bounds__(THREADS) gemm_skinny_kernel(
     const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, float* __restrict__ Y, bf16_t* __restrict__ act,
     int M, int N, int K) {
@@ -60,8 +67,16 @@ __global__ void __launch_bounds__(THREADS) gemm_skinny_kernel(
     const bool row_ok = n0 + l16 < inner;
     const int row = row_ok ? n0 + l16 : 0;           // clamped: the loads stay in bounds, the result is dropped
     const bf16_t* w_row[NT];
-    w_row[0] = W + (size_t)row * K + 8 * h;
-    if (SWIGLU) w_row[NT - 1] = W + (size_t)(inner + row) * K + 8 * h;
+    if (TILED) {
+        // tiles of one stacked matrix; a tile index beyond them (the grid is rounded up) is clamped and dropped
+        const int inner_tiles = (inner + 15) / 16;
+        const size_t tile = (size_t)min(n0 >> 4, inner_tiles - 1);
+        w_row[0] = W + tile * full_steps * 512 + lane * 8;
+        if (SWIGLU) w_row[NT - 1] = W + (inner_tiles + tile) * full_steps * 512 + lane * 8;
+    } else {
+        w_row[0] = W + (size_t)row * K + 8 * h;
+        if (SWIGLU) w_row[NT - 1] = W + (size_t)(inner + row) * K + 8 * h;
+    }
     const bf16_t* x_row[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) x_row[mt] = X + (size_t)min(16 * mt + l16, M - 1) * K + 8 * h;
@@ -77,7 +92,7 @@ __global__ void __launch_bounds__(THREADS) gemm_skinny_kernel(
     auto fetch = [&](int u, int step) {
         const int k = 32 * step;
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) wf[u][nt].u = *(const u32x4*)(w_row[nt] + k);
+        for (int nt = 0; nt < NT; ++nt) wf[u][nt].u = *(const u32x4*)(w_row[nt] + (TILED ? 512 * step : k));
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) xf[u][mt].u = *(const u32x4*)(x_row[mt] + k);
     };
@@ -108,7 +123,7 @@ __global__ void __launch_bounds__(THREADS) gemm_skinny_kernel(
             fetch(0, step);
             multiply(0);
         }
-        if ((K & 31) != 0) {
+        if (!TILED && (K & 31) != 0) {
             const int k = 32 * full_steps;
             const bool ok = k + 8 * h < K;
 #pragma unroll
@@ -181,7 +196,7 @@ __global__ void __launch_bounds__(THREADS) gemm_skinny_kernel(
     }
 }
 
-template <bool SWIGLU, int KW>
+template <bool SWIGLU, int KW, bool TILED>
 static int launch_kw(const bf16_t* X, const bf16_t* W, float* Y, bf16_t* act, int M, int N, int K, int parts,
                      hipStream_t stream) {
     const int inner = SWIGLU ? N / 2 : N;
@@ -190,7 +205,7 @@ static int launch_kw(const bf16_t* X, const bf16_t* W, float* Y, bf16_t* act, in
     dim3 grid((tiles + TW - 1) / TW, parts), block(THREADS);
     const int mt = (M + 15) / 16;
 #define KIPP_SK(MT, D) \
-    hipLaunchKernelGGL((gemm_skinny_kernel<MT, SWIGLU, KW, D>), grid, block, 0, stream, X, W, Y, act, M, N, K)
+    hipLaunchKernelGGL((gemm_skinny_kernel<MT, SWIGLU, KW, D, TILED>), grid, block, 0, stream, X, W, Y, act, M, N, K)
     switch (mt) {
         case 1: KIPP_SK(1, 8); break;
         case 2: KIPP_SK(2, 8); break;
@@ -204,13 +219,18 @@ static int launch_kw(const bf16_t* X, const bf16_t* W, float* Y, bf16_t* act, in
 
 template <bool SWIGLU>
 static int launch(const bf16_t* X, const bf16_t* W, float* Y, bf16_t* act, int M, int N, int K, int parts, int kw,
-                  hipStream_t stream) {
+                  int tiled, hipStream_t stream) {
+    if (tiled && (K & 31)) return -1;
+#define KIPP_KW(KW)                                                                          \
+    return tiled ? launch_kw<SWIGLU, KW, true>(X, W, Y, act, M, N, K, parts, stream)         \
+                 : launch_kw<SWIGLU, KW, false>(X, W, Y, act, M, N, K, parts, stream)
     switch (kw) {
-        case 1: return launch_kw<SWIGLU, 1>(X, W, Y, act, M, N, K, parts, stream);
-        case 2: return launch_kw<SWIGLU, 2>(X, W, Y, act, M, N, K, parts, stream);
-        case 4: return launch_kw<SWIGLU, 4>(X, W, Y, act, M, N, K, parts, stream);
+        case 1: KIPP_KW(1);
+        case 2: KIPP_KW(2);
+        case 4: KIPP_KW(4);
         default: return -1;
     }
+#undef KIPP_KW
 }
 
 // How the contraction is split: `kw` slices inside a workgroup and `parts` across workgroups,
@@ -245,22 +265,25 @@ int kipp_gemm_skinny_parts(int N, int K, int max_parts) {
 }
 
 // Y: float32 [parts, M, N] with parts = kipp_gemm_skinny_parts(N, K, max_parts).
-// K must be a multiple of 8 (16-byte loads), M <= 64.
-int kipp_gemm_skinny(const void* X, const void* W, float* Y, int M, int N, int K, int max_parts, hipStream_t stream) {
+// K must be a multiple of 8 (16-byte loads), M <= 64.  `tiled`: W is in the
+// streaming layout (K a multiple of 32), else [N, K] rows.
+int kipp_gemm_skinny(const void* X, const void* W, float* Y, int M, int N, int K, int max_parts, int tiled,
+                     hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
     if (M > 64 || K <= 0 || (K & 7) || max_parts <= 0) return -1;
     int kw, parts;
     plan((N + 15) / 16, K, max_parts, &kw, &parts);
-    return launch<false>((const bf16_t*)X, (const bf16_t*)W, Y, nullptr, M, N, K, parts, kw, stream);
+    return launch<false>((const bf16_t*)X, (const bf16_t*)W, Y, nullptr, M, N, K, parts, kw, tiled, stream);
 }
 
-// W: [2 I, K] = [gate; up]; act: bfloat16 [M, I].
-int kipp_gemm_skinny_swiglu(const void* X, const void* W, void* act, int M, int two_inner, int K, hipStream_t stream) {
+// W: [2 I, K] = [gate; up] (tiled: the tiles of gate, then those of up); act: bfloat16 [M, I].
+int kipp_gemm_skinny_swiglu(const void* X, const void* W, void* act, int M, int two_inner, int K, int tiled,
+                            hipStream_t stream) {
     if (M <= 0 || two_inner <= 0) return 0;
     if (M > 64 || K <= 0 || (K & 7) || (two_inner & 1)) return -1;
     int kw, parts;
     plan((two_inner / 2 + 15) / 16, K, 1, &kw, &parts);
-    return launch<true>((const bf16_t*)X, (const bf16_t*)W, nullptr, (bf16_t*)act, M, two_inner, K, 1, kw, stream);
+    return launch<true>((const bf16_t*)X, (const bf16_t*)W, nullptr, (bf16_t*)act, M, two_inner, K, 1, kw, tiled, stream);
 }
 
 }  // extern "C"

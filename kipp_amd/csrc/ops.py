@@ -298,10 +298,40 @@ def gemm_skinny_ok(m: int, k: int) -> bool:
     return 0 < m <= SKINNY_MAX_ROWS and k % 8 == 0 and k >= 32
 
 
-def gemm_skinny(x: torch.Tensor, w: torch.Tensor, max_parts: int = 1) -> torch.Tensor:
+def tile_weight(w: torch.Tensor, split: int = 1) -> torch.Tensor:
+    """The streaming layout of a bfloat16 matrix [N, K], K a multiple of 32: the
+    1 KB a wave reads in one step (16 rows x 32 columns) is contiguous,
+    [tile of 16 rows][step of 32 columns][lane][8 values] with lane l holding row
+    l % 16 and columns 8 (l / 16) .. + 7 of the step.  `split` stacked matrices of
+    N / split rows are each padded to whole tiles with zero rows."""
+    _need(w.dim() == 2 and w.dtype == torch.bfloat16, "tile_weight: a bfloat16 matrix")
+    n, k = w.shape
+    _need(k % 32 == 0 and split >= 1 and n % split == 0, "tile_weight: K a multiple of 32, N a multiple of split")
+    inner = n // split
+    tiles = (inner + 15) // 16
+    blocks = []
+    for i in range(split):
+        block = w[i * inner:(i + 1) * inner]
+        if inner % 16:
+            block = torch.cat([block, torch.zeros((tiles * 16 - inner, k), dtype=w.dtype, device=w.device)])
+        blocks.append(block.view(tiles, 16, k // 32, 4, 8).permute(0, 2, 3, 1, 4))
+    return torch.cat(blocks).contiguous().view(-1)
+
+
+def _tiles_ok(tiles, n: int, k: int, split: int, what: str) -> int:
+    if tiles is None:
+        return 0
+    inner_tiles = (n // split + 15) // 16
+    _need(tiles.dtype == torch.bfloat16 and tiles.is_contiguous() and k % 32 == 0
+          and tiles.numel() == split * inner_tiles * 16 * k, f"{what}: the tiled weight does not match [N, K]")
+    return 1
+
+
+def gemm_skinny(x: torch.Tensor, w: torch.Tensor, max_parts: int = 1, tiles: torch.Tensor = None) -> torch.Tensor:
     """float32 [parts, M, N] whose sum over parts is x . w^T, for M <= 64 rows of
     bfloat16 x against bfloat16 w [N, K].  parts <= max_parts is chosen from the
-    shape (1 when the weight has many rows)."""
+    shape (1 when the weight has many rows).  With `tiles` (tile_weight(w)) the
+    weight is streamed from that layout."""
     _dev(x, w)
     m, k = x.shape
     n = w.shape[0]
@@ -311,12 +341,13 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, max_parts: int = 1) -> torch.T
     lib = build.library("gemm_skinny")
     parts = lib.kipp_gemm_skinny_parts(n, k, int(max_parts))
     out = torch.empty((parts, m, n), dtype=torch.float32, device=x.device)
-    fn = _fn("gemm_skinny", "kipp_gemm_skinny", [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr])
-    _check(fn(_ptr(x), _ptr(w), _ptr(out), m, n, k, int(max_parts), _stream()), "gemm_skinny")
+    tiled = _tiles_ok(tiles, n, k, 1, "gemm_skinny")
+    fn = _fn("gemm_skinny", "kipp_gemm_skinny", [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr])
+    _check(fn(_ptr(x), _ptr(tiles if tiled else w), _ptr(out), m, n, k, int(max_parts), tiled, _stream()), "gemm_skinny")
     return out
 
 
-def gemm_rows(x: torch.Tensor, w: torch.Tensor, max_parts: int = 1) -> torch.Tensor:
+def gemm_rows(x: torch.Tensor, w: torch.Tensor, max_parts: int = 1, tiles: torch.Tensor = None) -> torch.Tensor:
     """float32 [parts, M, N] whose sum over parts is x . w^T, for 16 < M <= 64 rows
     (any M <= 64 is taken): the rows of x are staged through LDS and shared by
     the waves of a workgroup."""
@@ -329,13 +360,15 @@ def gemm_rows(x: torch.Tensor, w: torch.Tensor, max_parts: int = 1) -> torch.Ten
     lib = build.library("gemm_rows")
     parts = lib.kipp_gemm_rows_parts(n, k, int(max_parts))
     out = torch.empty((parts, m, n), dtype=torch.float32, device=x.device)
-    fn = _fn("gemm_rows", "kipp_gemm_rows", [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr])
-    _check(fn(_ptr(x), _ptr(w), _ptr(out), m, n, k, int(max_parts), _stream()), "gemm_rows")
+    tiled = _tiles_ok(tiles, n, k, 1, "gemm_rows")
+    fn = _fn("gemm_rows", "kipp_gemm_rows", [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr])
+    _check(fn(_ptr(x), _ptr(tiles if tiled else w), _ptr(out), m, n, k, int(max_parts), tiled, _stream()), "gemm_rows")
     return out
 
 
-def gemm_skinny_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
-    """out[M, I] (bfloat16) = silu(x . w_gate^T) * (x . w_up^T), w_gate_up = [gate; up] of [2 I, K]."""
+def gemm_skinny_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor, tiles: torch.Tensor = None) -> torch.Tensor:
+    """out[M, I] (bfloat16) = silu(x . w_gate^T) * (x . w_up^T), w_gate_up = [gate; up] of [2 I, K];
+    `tiles` = tile_weight(w_gate_up, split=2)."""
     _dev(x, w_gate_up, out)
     m, k = x.shape
     two_inner = w_gate_up.shape[0]
@@ -344,8 +377,9 @@ def gemm_skinny_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tens
     _need(w_gate_up.shape == (two_inner, k) and two_inner % 2 == 0 and out.shape == (m, two_inner // 2),
           "gemm_skinny_swiglu: shapes do not match")
     _need(gemm_skinny_ok(m, k), "gemm_skinny_swiglu: at most 64 rows, K a multiple of 8 and at least 32")
-    fn = _fn("gemm_skinny", "kipp_gemm_skinny_swiglu", [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr])
-    _check(fn(_ptr(x), _ptr(w_gate_up), _ptr(out), m, two_inner, k, _stream()), "gemm_skinny_swiglu")
+    tiled = _tiles_ok(tiles, two_inner, k, 2, "gemm_skinny_swiglu")
+    fn = _fn("gemm_skinny", "kipp_gemm_skinny_swiglu", [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr])
+    _check(fn(_ptr(x), _ptr(tiles if tiled else w_gate_up), _ptr(out), m, two_inner, k, tiled, _stream()), "gemm_skinny_swiglu")
     return out
 
 

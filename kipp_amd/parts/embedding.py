@@ -44,7 +44,7 @@ class Head:
         return {} if spec.tied else {"weight": ParamSpec((spec.vocab_size, spec.hidden_size))}
 
     def load(self, tensors, embedding=None):
-        self.weight = embedding.weight if self.spec.tied else tensors["weight"]
+        self.weight = self.rt.weight(embedding.weight if self.spec.tied else tensors["weight"])
 
     def forward(self, x):
         return self.rt.linear(x, self.weight)

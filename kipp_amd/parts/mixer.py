@@ -58,8 +58,8 @@ class Attention:
         if not (q.dtype == k.dtype == v.dtype):
             q, k, v = (t.float() for t in (q, k, v))
         # rows concatenated: one product serves q, k and v; no output element changes
-        self.w_qkv = torch.cat([q, k, v], dim=0).contiguous()
-        self.w_o = tensors["o_proj.weight"]
+        self.w_qkv = self.rt.weight(torch.cat([q, k, v], dim=0).contiguous())
+        self.w_o = self.rt.weight(tensors["o_proj.weight"])
         if self.spec.qk_norm_eps is not None:
             self.q_norm = tensors["q_norm.weight"]
             self.k_norm = tensors["k_norm.weight"]

@@ -30,8 +30,27 @@ def device_dtype(stored: torch.dtype, kind: str, compute: str) -> torch.dtype:
     return torch.float32
 
 
+class Weight:
+    """A matrix [N, K] as the products want it: `rows` as stored, for the library
+    product and the 32-bit kernels, and `tiles`, the same values in the layout
+    that the few-rows kernels stream fastest (None where that layout does not
+    apply).  `split` stacked matrices share the tensor."""
+    __slots__ = ("rows", "tiles", "split")
+
+    def __init__(self, rows: torch.Tensor, tiles: torch.Tensor | None = None, split: int = 1):
+        self.rows, self.tiles, self.split = rows, tiles, split
+
+    @property
+    def shape(self):
+        return self.rows.shape
+
+    @property
+    def dtype(self):
+        return self.rows.dtype
+
+
 class Runtime:
-    def __init__(self, dtype: str = "bfloat16", device: str = "cuda:0"):
+    def __init__(self, dtype: str = "bfloat16", device: str = "cuda:0", stream_layout: bool = True):
         if dtype not in DTYPES:
             raise ValueError(f"dtype must be one of {sorted(DTYPES)}, got {dtype!r}")
         if not torch.cuda.is_available():
@@ -41,6 +60,7 @@ class Runtime:
         self.act_dtype = DTYPES[dtype]
         self.cache_dtype = DTYPES[dtype]
         self.ops = ops
+        self.stream_layout = stream_layout   # keep a second copy of bfloat16 matrices in the streaming layout
         self._mm_out_f32 = None
         self.library_products = 0   # calls that went to the library (they stay out of HIP graphs)
         torch.backends.cuda.matmul.allow_tf32 = False
@@ -56,14 +76,31 @@ class Runtime:
     def empty(self, shape, dtype) -> torch.Tensor:
         return torch.empty(shape, dtype=dtype, device=self.device)
 
+    def weight(self, w: torch.Tensor, split: int = 1) -> Weight:
+        """A matrix on the device, made ready for `linear`.  A bfloat16 matrix whose
+        K is a multiple of 32 gets a copy in the streaming layout: decode reads every
+        weight once a step and is bound by that read, which is a fifth faster from
+        that layout; many-row products go to the library, which needs the rows.
+        The price is the matrix held twice."""
+        tiles = None
+        if self.stream_layout and w.dtype == torch.bfloat16 and w.dim() == 2 and w.shape[1] % 32 == 0 \
+                and w.shape[0] % split == 0:
+            tiles = self.ops.tile_weight(w, split)
+        return Weight(w, tiles, split)
+
     # -- matrix product ------------------------------------------------------
-    def linear(self, x: torch.Tensor, w: torch.Tensor, slabs: bool = False, low_precision_out: bool = False) -> torch.Tensor:
+    def linear(self, x: torch.Tensor, w, slabs: bool = False, low_precision_out: bool = False) -> torch.Tensor:
         """float32 [M, N] = x [M, K] . w [N, K]^T.  With `slabs` the result may come
         as [parts, M, N] whose sum over parts is the product (few rows against a
         weight with few output rows: the contraction is split over workgroups and
         the consumer adds the slabs in order).  With `low_precision_out` a large
         bfloat16 product may be returned in bfloat16 (for a consumer that rounds to
         bfloat16 anyway and is bound by reading it)."""
+        tiles = None
+        if isinstance(w, Weight):
+            # stacked matrices that fill whole tiles lie in the layout of one matrix
+            whole = w.split == 1 or (w.rows.shape[0] // w.split) % 16 == 0
+            w, tiles = w.rows, (w.tiles if whole else None)
         m = x.shape[0]
         n = w.shape[0]
         if w.dtype == torch.float32:
@@ -75,9 +112,9 @@ class Runtime:
         if self.ops.gemm_skinny_ok(m, x.shape[1]):
             # few rows: our own kernels stream the weight once
             if m <= 16:
-                y = self.ops.gemm_skinny(x, w, max_parts=8 if slabs else 1)
+                y = self.ops.gemm_skinny(x, w, max_parts=8 if slabs else 1, tiles=tiles)
             else:
-                y = self.ops.gemm_rows(x, w, max_parts=8 if slabs else 1)
+                y = self.ops.gemm_rows(x, w, max_parts=8 if slabs else 1, tiles=tiles)
             return y if y.shape[0] > 1 else y[0]
         # bfloat16 x bfloat16 with float32 accumulation: the library product
         self.library_products += 1

@@ -388,6 +388,27 @@ def test_gemm_skinny(m, n, k, max_parts):
     wi = torch.tensor(rng.integers(-3, 4, size=(n, k)), dtype=torch.bfloat16)
     out = ops.gemm_skinny(xi.to(DEV), wi.to(DEV), max_parts).sum(dim=0)
     assert np.array_equal(out.cpu().numpy(), xi.float().numpy() @ wi.float().numpy().T)
+    if k % 32 == 0:      # the same product from the streaming layout: the same sums in the same order
+        wd = w.to(DEV)
+        assert torch.equal(ops.gemm_skinny(x.to(DEV), wd, max_parts, tiles=ops.tile_weight(wd)),
+                           ops.gemm_skinny(x.to(DEV), wd, max_parts))
+
+
+def test_tile_weight_layout():
+    ops = _ops()
+    w = torch.arange(20 * 64, dtype=torch.float32).reshape(20, 64).bfloat16()          # 20 rows: the second tile is padded
+    t = ops.tile_weight(w.to(DEV)).cpu().view(2, 2, 64, 8)                               # [tile][step][lane][8]
+    for tile, step, lane in [(0, 0, 0), (0, 1, 17), (1, 0, 3), (1, 1, 63), (1, 0, 4)]:
+        row, col = 16 * tile + lane % 16, 32 * step + 8 * (lane // 16)
+        want = w[row, col:col + 8] if row < 20 else torch.zeros(8, dtype=torch.bfloat16)
+        assert torch.equal(t[tile, step, lane], want)
+    two = ops.tile_weight(w.to(DEV), split=2).cpu().view(2, 2, 64, 8)                    # 10 + 10 rows, each padded to a tile
+    assert torch.equal(two[1, 1, 16 + 9], w[10 + 9, 32 + 8:32 + 16]) and not two[1, 0, 10].any()
+    with pytest.raises(ops.KernelError):
+        ops.tile_weight(torch.zeros(16, 40, dtype=torch.bfloat16, device=DEV))
+    with pytest.raises(ops.KernelError):
+        ops.gemm_skinny(torch.zeros(2, 64, dtype=torch.bfloat16, device=DEV), torch.zeros(20, 64, dtype=torch.bfloat16, device=DEV),
+                        tiles=torch.zeros(16 * 64, dtype=torch.bfloat16, device=DEV))   # tiles of another matrix
 
 
 @pytest.mark.parametrize("m", [1, 17, 32, 33, 64])
@@ -406,6 +427,10 @@ def test_gemm_rows(m, n, k, max_parts):
     wi = torch.tensor(rng.integers(-3, 4, size=(n, k)), dtype=torch.bfloat16)
     out = ops.gemm_rows(xi.to(DEV), wi.to(DEV), max_parts).sum(dim=0)
     assert np.array_equal(out.cpu().numpy(), xi.float().numpy() @ wi.float().numpy().T)
+    if k % 32 == 0:
+        wd = w.to(DEV)
+        assert torch.equal(ops.gemm_rows(x.to(DEV), wd, max_parts, tiles=ops.tile_weight(wd)),
+                           ops.gemm_rows(x.to(DEV), wd, max_parts))
 
 
 def test_consumers_add_slabs_in_order():
@@ -443,7 +468,7 @@ def test_gemm_skinny_refuses_what_it_cannot_do():
         ops.gemm_skinny(torch.zeros(2, 36, dtype=torch.bfloat16, device=DEV), torch.zeros(16, 36, dtype=torch.bfloat16, device=DEV))
 
 
-@pytest.mark.parametrize("m,inner,k", [(1, 16, 32), (8, 200, 80), (64, 9728, 2560), (5, 77, 40), (33, 100, 2560)])
+@pytest.mark.parametrize("m,inner,k", [(1, 16, 32), (8, 200, 80), (64, 9728, 2560), (5, 77, 40), (33, 100, 2560), (7, 77, 96)])
 def test_gemm_skinny_swiglu(m, inner, k):
     ops = _ops()
     rng = np.random.default_rng(m + inner)
@@ -453,6 +478,11 @@ def test_gemm_skinny_swiglu(m, inner, k):
     gu = x.double().numpy() @ w.double().numpy().T
     ref = plain.silu(gu[:, :inner]) * gu[:, inner:]
     assert _rel(out.float().cpu().numpy(), ref) < 1e-5
+    if k % 32 == 0:
+        wd = w.to(DEV)
+        tiled = ops.gemm_skinny_swiglu(x.to(DEV), wd, torch.empty(m, inner, dtype=torch.bfloat16, device=DEV),
+                                       tiles=ops.tile_weight(wd, split=2))
+        assert torch.equal(tiled, out)
 
 
 def test_rmsnorm_adds_slabs_in_order():
