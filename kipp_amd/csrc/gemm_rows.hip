@@ -139,17 +139,29 @@ __global__ void __launch_bounds__(TW * KIPP_WAVE) gemm_rows_kernel(
     }
 }
 
-// Waves per workgroup and parts of K, from the shape only: about 640 workgroups,
-// each part at least one whole chunk, at most `max_parts` slabs.
+// Waves per workgroup (4 or 8, each with 16 rows of W) and parts of K, from the shape
+// only.  A compute unit draws a bounded number of bytes a second, so the workgroups
+// run in rounds of 256 and a round costs what one workgroup reads plus a fixed start;
+// the plan takes the cheapest rounds, with a small charge for every slab the consumer
+// has to add and every part at least one whole chunk.
 static void plan(int N, int K, int max_parts, int* tw, int* parts) {
     const int tiles = (N + 15) / 16;
     const int groups = K / CHUNK > 0 ? K / CHUNK : 1;
-    *tw = tiles >= 4096 ? 8 : 4;
-    const int wgs = (tiles + *tw - 1) / *tw;
-    int p = (640 + wgs - 1) / wgs;
-    if (p > groups) p = groups;
-    if (p > max_parts) p = max_parts;
-    *parts = p < 1 ? 1 : p;
+    double best = 1e300;
+    *tw = 4;
+    *parts = 1;
+    for (int t = 4; t <= 8; t *= 2) {
+        const int cols = (tiles + t - 1) / t;
+        for (int p = 1; p <= max_parts && p <= groups; ++p) {
+            const int rounds = (cols * p + 255) / 256;
+            const double cost = rounds * (t * (double)K / p + 150.0 * t) * (1.0 + 0.02 * p);
+            if (cost < best * 0.999) {
+                best = cost;
+                *tw = t;
+                *parts = p;
+            }
+        }
+    }
 }
 
 extern "C" {

@@ -233,26 +233,32 @@ static int launch(const bf16_t* X, const bf16_t* W, float* Y, bf16_t* act, int M
 #undef KIPP_KW
 }
 
-// How the contraction is split: `kw` slices inside a workgroup and `parts` across workgroups,
-// so that about 2500 waves stream the weight (short products gain more from many waves than
-// from long pipelines) and each slice has at least one whole group of 8 steps.  A function of
-// the shape only, never of the data.
+// How the contraction is split: `kw` slices inside a workgroup and `parts` across
+// workgroups.  A compute unit draws a bounded number of bytes a second however many
+// waves ask, so what counts is that all 256 of them stream all the time: the
+// workgroups run in rounds of 256, and a round costs what one workgroup reads plus
+// a fixed start.  The plan takes the split with the cheapest rounds (each slice at
+// least one whole group of 8 steps, a small charge for every slab the consumer has
+// to add).  A function of the shape only, never of the data.
 static void plan(int tiles, int K, int max_parts, int* kw, int* parts) {
     const int groups = K / 32 / 8 > 0 ? K / 32 / 8 : 1;
-    int want = (2560 + tiles - 1) / tiles;
-    if (want > groups) want = groups;
-    if (want >= 4) {
-        *kw = 4;
-        *parts = want / 4;
-    } else if (want >= 2) {
-        *kw = 2;
-        *parts = 1;
-    } else {
-        *kw = 1;
-        *parts = 1;
+    const double start = 300.0;                       // a workgroup's fixed cost, in columns of its rows
+    double best = 1e300;
+    *kw = 1;
+    *parts = 1;
+    for (int k = 4; k >= 1; k /= 2) {
+        const int tw = WAVES / k;
+        const int cols = (tiles + tw - 1) / tw;
+        for (int p = 1; p <= max_parts && k * p <= groups; ++p) {
+            const int rounds = (cols * p + 255) / 256;
+            const double cost = rounds * (tw * (double)K / p + start) * (1.0 + 0.02 * p);
+            if (cost < best * 0.999) {
+                best = cost;
+                *kw = k;
+                *parts = p;
+            }
+        }
     }
-    if (*parts > max_parts) *parts = max_parts;
-    if (*parts < 1) *parts = 1;
 }
 
 extern "C" {

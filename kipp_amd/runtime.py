@@ -114,7 +114,7 @@ class Runtime:
             if m <= 16:
                 y = self.ops.gemm_skinny(x, w, max_parts=8 if slabs else 1, tiles=tiles)
             else:
-                y = self.ops.gemm_rows(x, w, max_parts=8 if slabs else 1, tiles=tiles)
+                y = self.ops.gemm_rows(x, w, max_parts=12 if slabs else 1, tiles=tiles)
             return y if y.shape[0] > 1 else y[0]
         # bfloat16 x bfloat16 with float32 accumulation: the library product
         self.library_products += 1
