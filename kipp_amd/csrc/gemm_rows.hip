@@ -36,7 +36,8 @@ __global__ void __launch_bounds__(TW * KIPP_WAVE) gemm_rows_kernel(
     const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, float* __restrict__ Y, int M, int N, int K) {
     constexpr int THREADS = TW * KIPP_WAVE;
     constexpr int UNITS = MT * 16 * (CHUNK / 8);              // 16-byte units of one staged chunk
-    constexpr int XR = (UNITS + THREADS - 1) / THREADS;       // units a thread moves
+    constexpr int XR = UNITS / THREADS;                        // units a thread moves
+    static_assert(UNITS % THREADS == 0, "every thread stages the same number of units");
     __shared__ __attribute__((aligned(16))) bf16_t xs[2][MT * 16 * X_PITCH];
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -57,7 +58,7 @@ __global__ void __launch_bounds__(TW * KIPP_WAVE) gemm_rows_kernel(
     int x_dst[XR];
 #pragma unroll
     for (int i = 0; i < XR; ++i) {
-        const int unit = min(tid + i * THREADS, UNITS - 1);
+        const int unit = tid + i * THREADS;
         const int r = unit / (CHUNK / 8), c = unit % (CHUNK / 8);
         x_src[i] = X + (size_t)min(r, M - 1) * K + c * 8;
         x_dst[i] = r * X_PITCH + c * 8;
@@ -76,8 +77,7 @@ __global__ void __launch_bounds__(TW * KIPP_WAVE) gemm_rows_kernel(
     };
     auto stage_x = [&](int buf) {
 #pragma unroll
-        for (int i = 0; i < XR; ++i)
-            if (tid + i * THREADS < UNITS) *(u32x4*)(xs[buf] + x_dst[i]) = xr[i];
+        for (int i = 0; i < XR; ++i) *(u32x4*)(xs[buf] + x_dst[i]) = xr[i];
     };
     auto multiply = [&](int u, int buf) {
 #pragma unroll
@@ -88,24 +88,29 @@ __global__ void __launch_bounds__(TW * KIPP_WAVE) gemm_rows_kernel(
         }
     };
 
+    // The last chunk stands outside the loop, so that inside it every load has a fixed
+    // place in the order of the loads in flight and no wait covers more than it must.
     if (g_begin < g_end) {
+        fetch_x(g_begin);                             // asked for first: needed first
 #pragma unroll
         for (int u = 0; u < DEPTH; ++u) fetch_w(u, g_begin * DEPTH + u);
-        fetch_x(g_begin);
         stage_x(0);
         __syncthreads();
-        for (int g = g_begin; g < g_end; ++g) {
-            const int buf = (g - g_begin) & 1;
-            const bool more = g + 1 < g_end;
-            if (more) fetch_x(g + 1);
+        int buf = 0;
+        for (int g = g_begin; g + 1 < g_end; ++g) {
+            fetch_x(g + 1);
 #pragma unroll
             for (int u = 0; u < DEPTH; ++u) {
                 multiply(u, buf);
-                if (more) fetch_w(u, (g + 1) * DEPTH + u);
+                fetch_w(u, (g + 1) * DEPTH + u);
+                __builtin_amdgcn_sched_barrier(0);    // keep the load here: the compiler would gather all eight after the products
             }
-            if (more) stage_x(buf ^ 1);
+            stage_x(buf ^ 1);
             __syncthreads();
+            buf ^= 1;
         }
+#pragma unroll
+        for (int u = 0; u < DEPTH; ++u) multiply(u, buf);
     }
     // the rest of K (fewer than 256 columns), by the last part, straight from global memory
     if (part == parts - 1) {
