@@ -19,6 +19,15 @@
 // for a token does not depend on the batch it is in.  A sequence that needs
 // one split only is written normalised at once.
 //
+// FUSED: the kernel starts from the output of the QKV projection instead of from
+// finished queries.  Each workgroup norms and rotates the GROUP queries of its
+// key/value head itself (a wave a head, element i and its rotation partner
+// i + d/2 in one lane, as in the rotary kernel), and the workgroup of the split
+// that holds the token's own position does the same for the new key, takes the
+// new value, writes both into the cache and uses them from LDS.  A decode step
+// then needs no rotary kernel.  Head sizes that are multiples of 128, rotated
+// over their whole width.
+//
 // Compile-time: HEAD_DIM (multiple of 16, <= 256), GROUP (query heads per
 // key/value head, <= 16).
 #include "common.h"
@@ -50,13 +59,32 @@ union Frag {
     bf16x8 v;
 };
 
+#define FUSED_OK ((HEAD_DIM % 128) == 0)
+#define NC (HEAD_DIM / KIPP_WAVE)              // elements of a head a lane holds when a wave takes a head
+#define JOBS ((GROUP + 2 + WAVES - 1) / WAVES)  // heads a wave prepares: GROUP queries, the new key, the new value
+#define MAX_SLABS 4                            // slabs of the projection the fused kernel adds
+
+// What the fused kernel needs beside the attention itself.
+struct Projected {
+    const float* qkv;        // [parts][tokens][(n_q + 2 n_kv) HEAD_DIM], slabs added in order
+    int parts;
+    size_t part_stride;
+    const float* q_norm_w;   // null: no norm
+    const float* k_norm_w;
+    float eps;
+    const float* inv_freq;   // null: no rotation
+    int write_kv;            // 0: the cache is another layer's, keys and values are already there
+};
+
+template <bool FUSED>
 __global__ void __launch_bounds__(THREADS) attention_decode_kernel(
-    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
+    const bf16_t* __restrict__ q, bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache,
     bf16_t* __restrict__ out, float* __restrict__ part_acc, float* __restrict__ part_ml,
     const int32_t* __restrict__ rows, const int32_t* __restrict__ positions, const int32_t* __restrict__ seq_of_token,
     const int32_t* __restrict__ block_table, int max_blocks, int n_q, int n_kv, int page, float scale_log2e,
-    int window, int max_splits) {
+    int window, int max_splits, Projected pj) {
     __shared__ float s_scores[GROUP][SPLIT + 4];
+    __shared__ __attribute__((aligned(16))) bf16_t s_new[FUSED ? GROUP + 2 : 1][HEAD_DIM];
     __shared__ float s_red[WAVES][GROUP][HEAD_DIM];
     __shared__ float s_m[GROUP], s_l[GROUP];
     __shared__ int s_page[SPLIT + 2];                 // page of every key of the split (any page size)
@@ -79,15 +107,60 @@ __global__ void __launch_bounds__(THREADS) attention_decode_kernel(
     // nothing that is still in flight and can all be issued back to back.  Keys beyond
     // the query's position read the last valid page (finite values, masked later).
     const int page_shift = __builtin_ctz(page);          // the page size is a power of two (checked by the launcher)
-    if (tid < SPLIT) s_page[tid] = table[min(base + tid, pos) >> page_shift];
+    int my_page = 0;
+    if (tid < SPLIT) my_page = table[min(base + tid, pos) >> page_shift];
+
+    // ---- fused: ask for the projected heads this wave prepares, and for what their norm and
+    // rotation need, before the keys and values are asked for: they are wanted first
+    const bool owner = FUSED && pj.write_kv && split == last_split;   // this workgroup holds the token's own position
+#if FUSED_OK
+    float raw[JOBS][NC], norm_q[NC], norm_k[NC], freq[NC / 2];
+    if (FUSED) {
+        const size_t width = (size_t)(n_q + 2 * n_kv) * HEAD_DIM;
+        int last_slab = pj.parts - 1;
+        asm volatile("" : "+s"(last_slab));          // opaque: every slab load below is issued, none waits for a branch
+#pragma unroll
+        for (int jj = 0; jj < JOBS; ++jj) {
+            const int j = wave + jj * WAVES;
+            const bool valid = j < GROUP || (owner && j < GROUP + 2);
+            const int slot = !valid ? 0 : (j < GROUP ? kvh * GROUP + j : (j == GROUP ? n_q + kvh : n_q + n_kv + kvh));
+            const float* src = pj.qkv + (size_t)row * width + (size_t)slot * HEAD_DIM + lane;
+            // every slab is asked for before any is used, then they are added in order.  A slab index
+            // beyond `parts` reads the last slab again and enters with the factor 0: no branch, so no
+            // load can be moved behind one and waited for on its own
+            float slab[NC][MAX_SLABS];
+#pragma unroll
+            for (int c = 0; c < NC; ++c)
+#pragma unroll
+                for (int p = 0; p < MAX_SLABS; ++p)
+                    slab[c][p] = src[(size_t)min(p, last_slab) * pj.part_stride + c * KIPP_WAVE];
+#pragma unroll
+            for (int c = 0; c < NC; ++c) {
+                raw[jj][c] = slab[c][0];
+#pragma unroll
+                for (int p = 1; p < MAX_SLABS; ++p) raw[jj][c] += (p <= last_slab ? 1.0f : 0.0f) * slab[c][p];
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+            norm_q[c] = pj.q_norm_w != nullptr ? pj.q_norm_w[lane + c * KIPP_WAVE] : 1.0f;
+            norm_k[c] = pj.k_norm_w != nullptr ? pj.k_norm_w[lane + c * KIPP_WAVE] : 1.0f;
+        }
+#pragma unroll
+        for (int c = 0; c < NC / 2; ++c) freq[c] = pj.inv_freq != nullptr ? pj.inv_freq[lane + c * KIPP_WAVE] : 0.0f;
+    }
+#endif
+    if (tid < SPLIT) s_page[tid] = my_page;
     __syncthreads();
 
     // ---- the GROUP queries as B operand: lane (slot l16, quarter h) holds q[slot][32 t + 8 h .. + 7]
     Frag qf[KSTEPS];
+    if (!FUSED) {
 #pragma unroll
-    for (int t = 0; t < KSTEPS; ++t) {
-        const int dcol = min(32 * t + 8 * h, HEAD_DIM - 8);
-        qf[t].u = *(const u32x4*)(q + ((size_t)row * n_q + (size_t)kvh * GROUP + min(l16, GROUP - 1)) * HEAD_DIM + dcol);
+        for (int t = 0; t < KSTEPS; ++t) {
+            const int dcol = min(32 * t + 8 * h, HEAD_DIM - 8);
+            qf[t].u = *(const u32x4*)(q + ((size_t)row * n_q + (size_t)kvh * GROUP + min(l16, GROUP - 1)) * HEAD_DIM + dcol);
+        }
     }
 
     // ---- scores: each wave takes BLOCKS_PER_WAVE blocks of 16 keys; every load is unconditional
@@ -111,6 +184,76 @@ __global__ void __launch_bounds__(THREADS) attention_decode_kernel(
 #pragma unroll
         for (int c = 0; c < CHUNKS_PER_LANE; ++c) vf[i][c].u = *(const u32x4*)(v_row + min(l16 + 16 * c, CHUNKS - 1) * 8);
     }
+#if FUSED_OK
+    if (FUSED) {
+        // norm (/root/reference/src/kipp.c:2480-2500), rotation (kipp.c:2368-2382), in the arithmetic of
+        // the rotary kernel; the keys and values asked for above are on their way meanwhile
+        float cs[NC / 2], sn[NC / 2];
+#pragma unroll
+        for (int c = 0; c < NC / 2; ++c) {
+            cs[c] = 1.0f;
+            sn[c] = 0.0f;
+            if (pj.inv_freq != nullptr) {
+                const float angle = (float)pos * freq[c];
+                cs[c] = cosf(angle);
+                sn[c] = sinf(angle);
+            }
+        }
+        const int own_slot = pos - base;             // the token's own key within this split (owner only)
+#pragma unroll
+        for (int jj = 0; jj < JOBS; ++jj) {
+            const int j = wave + jj * WAVES;
+            if (!(j < GROUP || (owner && j < GROUP + 2))) continue;
+            if (j <= GROUP) {
+                if ((j < GROUP ? pj.q_norm_w : pj.k_norm_w) != nullptr) {
+                    float ss = 0.0f;
+#pragma unroll
+                    for (int c = 0; c < NC; ++c) ss += raw[jj][c] * raw[jj][c];
+                    ss = wave_sum(ss);
+                    const float r = 1.0f / sqrtf(ss / (float)HEAD_DIM + pj.eps);
+#pragma unroll
+                    for (int c = 0; c < NC; ++c) raw[jj][c] *= r * (j < GROUP ? norm_q[c] : norm_k[c]);
+                }
+#pragma unroll
+                for (int c = 0; c < NC / 2; ++c) {
+                    const float a = raw[jj][c], b = raw[jj][c + NC / 2];
+                    raw[jj][c] = a * cs[c] - b * sn[c];
+                    raw[jj][c + NC / 2] = b * cs[c] + a * sn[c];
+                }
+            }
+            bf16_t* dst = nullptr;
+            if (j >= GROUP)
+                dst = (j == GROUP ? k_cache : v_cache) +
+                      (((size_t)s_page[own_slot] * n_kv + kvh) * page + (pos & (page - 1))) * HEAD_DIM;
+#pragma unroll
+            for (int c = 0; c < NC; ++c) {
+                const bf16_t bits = f32_to_bf16(raw[jj][c]);
+                s_new[j][lane + c * KIPP_WAVE] = bits;
+                if (dst != nullptr) dst[lane + c * KIPP_WAVE] = bits;
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int t = 0; t < KSTEPS; ++t)
+            qf[t].u = *(const u32x4*)(&s_new[min(l16, GROUP - 1)][min(32 * t + 8 * h, HEAD_DIM - 8)]);
+        if (owner) {                                  // the token's own key and value come from LDS, not from the cache
+#pragma unroll
+            for (int b = 0; b < BLOCKS_PER_WAVE; ++b)
+                if ((wave * BLOCKS_PER_WAVE + b) * 16 + l16 == own_slot) {
+#pragma unroll
+                    for (int t = 0; t < KSTEPS; ++t)
+                        kf[b][t].u = *(const u32x4*)(&s_new[GROUP][min(32 * t + 8 * h, HEAD_DIM - 8)]);
+                }
+#pragma unroll
+            for (int i = 0; i < KEYS_PER_GROUP; ++i)
+                if (kg + 16 * i == own_slot) {
+#pragma unroll
+                    for (int c = 0; c < CHUNKS_PER_LANE; ++c)
+                        vf[i][c].u = *(const u32x4*)(&s_new[GROUP + 1][min(l16 + 16 * c, CHUNKS - 1) * 8]);
+                }
+        }
+    }
+#endif
     // operands that reach beyond the head size or the group were read from clamped addresses: zero them
 #pragma unroll
     for (int t = 0; t < KSTEPS; ++t)
@@ -281,15 +424,49 @@ int kipp_attention_decode(const void* q, const void* k_cache, const void* v_cach
     if (grid_splits <= 0 || grid_splits > max_splits) return -3;
     if (page <= 0 || (page & (page - 1))) return -4;   // pages of a power of two only
     const float scale_log2e = scale * 1.4426950408889634f;
-    hipLaunchKernelGGL(attention_decode_kernel, dim3(grid_splits, n_kv, n_items), dim3(THREADS), 0, stream,
-                       (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, part_acc, part_ml,
+    hipLaunchKernelGGL(attention_decode_kernel<false>, dim3(grid_splits, n_kv, n_items), dim3(THREADS), 0, stream,
+                       (const bf16_t*)q, (bf16_t*)k_cache, (bf16_t*)v_cache, (bf16_t*)out, part_acc, part_ml,
                        rows, positions, seq_of_token, block_table, max_blocks, n_q, n_kv, page, scale_log2e, window,
-                       max_splits);
+                       max_splits, Projected{});
     int rc = KIPP_LAUNCH_CHECK();
     if (rc != 0 || grid_splits == 1) return rc;
     hipLaunchKernelGGL(attention_decode_reduce_kernel, dim3(n_q, n_items), dim3(HEAD_DIM >= 64 ? 64 : HEAD_DIM), 0,
                        stream, part_acc, part_ml, (bf16_t*)out, rows, positions, n_q, window, max_splits);
     return KIPP_LAUNCH_CHECK();
+}
+
+// 1 if this build has the fused kernel (head sizes that are multiples of 128).
+int kipp_attention_decode_fused_ok() { return FUSED_OK ? 1 : 0; }
+int kipp_attention_decode_fused_slabs() { return MAX_SLABS; }
+
+// The same from the output of the QKV projection: `qkv` float32 [parts][tokens][(n_q + 2 n_kv) head_dim];
+// norm weights and `inv_freq` may be null (no norm, no rotation; a rotation covers the whole head);
+// with `write_kv` the token's key and value are written into the cache as well.
+int kipp_attention_decode_fused(const float* qkv, int parts, int n_tokens, const float* q_norm_w, const float* k_norm_w,
+                                float eps, const float* inv_freq, int write_kv, void* k_cache, void* v_cache, void* out,
+                                float* part_acc, float* part_ml, const int32_t* rows, const int32_t* positions,
+                                const int32_t* seq_of_token, const int32_t* block_table, int max_blocks, int n_items,
+                                int n_q, int n_kv, int head_dim, int page, float scale, int window, int grid_splits,
+                                int max_splits, hipStream_t stream) {
+#if FUSED_OK
+    if (n_items <= 0) return 0;
+    if (head_dim != HEAD_DIM || n_kv <= 0 || n_q != n_kv * GROUP || parts <= 0 || parts > MAX_SLABS) return -1;
+    if (grid_splits <= 0 || grid_splits > max_splits) return -3;
+    if (page <= 0 || (page & (page - 1))) return -4;
+    const float scale_log2e = scale * 1.4426950408889634f;
+    Projected pj{qkv, parts, (size_t)n_tokens * (n_q + 2 * n_kv) * HEAD_DIM, q_norm_w, k_norm_w, eps, inv_freq, write_kv};
+    hipLaunchKernelGGL(attention_decode_kernel<true>, dim3(grid_splits, n_kv, n_items), dim3(THREADS), 0, stream,
+                       (const bf16_t*)nullptr, (bf16_t*)k_cache, (bf16_t*)v_cache, (bf16_t*)out, part_acc, part_ml,
+                       rows, positions, seq_of_token, block_table, max_blocks, n_q, n_kv, page, scale_log2e, window,
+                       max_splits, pj);
+    int rc = KIPP_LAUNCH_CHECK();
+    if (rc != 0 || grid_splits == 1) return rc;
+    hipLaunchKernelGGL(attention_decode_reduce_kernel, dim3(n_q, n_items), dim3(HEAD_DIM >= 64 ? 64 : HEAD_DIM), 0,
+                       stream, part_acc, part_ml, (bf16_t*)out, rows, positions, n_q, window, max_splits);
+    return KIPP_LAUNCH_CHECK();
+#else
+    return -5;
+#endif
 }
 
 }  // extern "C"

@@ -112,6 +112,7 @@ __global__ void __launch_bounds__(THREADS) gemm_skinny_kernel(
             for (int u = 0; u < DEPTH; ++u) {
                 multiply(u);
                 fetch(u, (g + 1) * DEPTH + u);
+                __builtin_amdgcn_sched_barrier(0);    // keep the loads here: the compiler would gather them after the products
             }
         }
 #pragma unroll

@@ -261,6 +261,66 @@ def attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
     return out
 
 
+DECODE_FUSED_SLABS = 4
+
+
+def attention_decode_fused_ok(head_dim: int, rotary_dim: int, rotates: bool, slabs: int = 1) -> bool:
+    """Can decode attention start from the QKV projection's output?  Head sizes that
+    are multiples of 128, rotated over their whole width (or not at all), a
+    projection in at most 4 slabs."""
+    return head_dim % 128 == 0 and head_dim <= 256 and (not rotates or rotary_dim == head_dim) and slabs <= DECODE_FUSED_SLABS
+
+
+def attention_decode_fused(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
+                           rows: torch.Tensor, positions: torch.Tensor, seq_of_token: torch.Tensor,
+                           block_table: torch.Tensor, n_q: int, n_kv: int, head_dim: int,
+                           q_norm_w: Optional[torch.Tensor], k_norm_w: Optional[torch.Tensor], eps: float,
+                           inv_freq: Optional[torch.Tensor], rotary_dim: int, write_kv: bool, scale: float, window: int,
+                           max_context: int, workspace: tuple, grid_splits: Optional[int] = None) -> torch.Tensor:
+    """Decode attention straight from the QKV projection: per-head q/k RMSNorm,
+    rotation, the write of the token's key and value into its page and the
+    attention over the pages in one kernel (plus the merge of the splits).
+    `qkv`: float32 [tokens, width] or slabs [parts, tokens, width]."""
+    _dev(qkv, k_cache, v_cache, out, rows, positions, seq_of_token, block_table, *workspace)
+    for t, name in ((rows, "rows"), (positions, "positions"), (seq_of_token, "seq_of_token"), (block_table, "block_table")):
+        _i32(t, name)
+    _need(qkv.dtype == torch.float32 and qkv.dim() in (2, 3) and qkv.is_contiguous(), "attention_decode_fused: float32 qkv")
+    parts = qkv.shape[0] if qkv.dim() == 3 else 1
+    n_tokens = qkv.shape[-2]
+    _need(qkv.shape[-1] == (n_q + 2 * n_kv) * head_dim, "attention_decode_fused: qkv width is not (n_q + 2 n_kv) head_dim")
+    _need(attention_decode_fused_ok(head_dim, rotary_dim, inv_freq is not None, parts),
+          "attention_decode_fused: head size a multiple of 128, rotated over its whole width, at most 4 slabs")
+    _need(out.shape == (n_tokens, n_q * head_dim) and out.dtype == torch.bfloat16 and out.is_contiguous(),
+          "attention_decode_fused: out is bfloat16 [tokens, n_q head_dim]")
+    _need(k_cache.dtype == torch.bfloat16 and k_cache.shape == v_cache.shape and k_cache.shape[1] == n_kv
+          and k_cache.shape[3] == head_dim and n_q % n_kv == 0, "attention_decode_fused: cache shape")
+    for w, name in ((q_norm_w, "q_norm_w"), (k_norm_w, "k_norm_w")):
+        _need(w is None or (w.dtype == torch.float32 and w.numel() == head_dim), f"attention_decode_fused: {name} float32 [head_dim]")
+    _need(inv_freq is None or (inv_freq.dtype == torch.float32 and inv_freq.numel() == head_dim // 2),
+          "attention_decode_fused: inv_freq float32 [head_dim / 2]")
+    group = n_q // n_kv
+    _need(group <= 16, "attention_decode_fused: more than 16 query heads per key/value head are refused")
+    n_items = rows.numel()
+    part_acc, part_ml = workspace
+    max_splits = part_ml.numel() // max(1, n_items * n_q * 2)
+    span = min(max_context, window) if window else max_context
+    need = (span + DECODE_SPLIT - 1) // DECODE_SPLIT + (1 if window else 0)
+    grid = grid_splits if grid_splits is not None else max(1, min(need, max_splits))
+    _need(part_acc.dtype == torch.float32 and part_ml.dtype == torch.float32
+          and part_acc.numel() >= n_items * n_q * max_splits * head_dim and need <= max_splits,
+          "attention_decode_fused: workspace too small for this context")
+    defines = {"HEAD_DIM": head_dim, "GROUP": group}
+    fn = _fn("attention_decode", "kipp_attention_decode_fused",
+             [_c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_float, _c_ptr, _c_int] + [_c_ptr] * 9 + [_c_int] * 6
+             + [_c_float, _c_int, _c_int, _c_int, _c_ptr], defines)
+    null = lambda t: _ptr(t) if t is not None else None
+    _check(fn(_ptr(qkv), parts, n_tokens, null(q_norm_w), null(k_norm_w), float(eps), null(inv_freq), 1 if write_kv else 0,
+              _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(part_acc), _ptr(part_ml), _ptr(rows), _ptr(positions),
+              _ptr(seq_of_token), _ptr(block_table), block_table.shape[1], n_items, n_q, n_kv, head_dim,
+              k_cache.shape[2], float(scale), int(window), grid, max_splits, _stream()), "attention_decode_fused")
+    return out
+
+
 def attention_decode_workspace(n_items: int, n_q: int, head_dim: int, max_context: int, device) -> tuple:
     max_splits = (max_context + DECODE_SPLIT - 1) // DECODE_SPLIT + 1
     return (torch.empty(n_items * n_q * max_splits * head_dim, dtype=torch.float32, device=device),

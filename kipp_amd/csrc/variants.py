@@ -32,7 +32,7 @@ def model_variants(spec, dtype: str) -> List[Spec]:
 
 # (head_dim, query heads per key/value head) of the shapes under config/shapes,
 # the tiny configurations, the toy model of the tests and the kernel tests
-PREBUILT_ATTENTION = [(128, 4), (128, 8), (16, 2), (32, 4), (16, 3), (48, 3), (64, 1), (32, 16), (256, 4), (80, 3), (256, 2), (16, 1)]
+PREBUILT_ATTENTION = [(128, 4), (128, 8), (128, 16), (128, 1), (16, 2), (32, 4), (16, 3), (48, 3), (64, 1), (32, 16), (256, 4), (80, 3), (256, 2), (16, 1)]
 
 
 def prebuilt() -> List[Spec]:

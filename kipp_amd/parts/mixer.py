@@ -77,13 +77,24 @@ class Attention:
         qkv = rt.linear(x, self.w_qkv, slabs=True)
         inv_freq, rotary_dim = self.position.rotary_table()
         table = batch.block_tables[cache.group]
+        eps = s.qk_norm_eps if s.qk_norm_eps is not None else 0.0
+        fast = rt.dtype == "bfloat16" and rt.ops.attention_fast_ok(s.num_heads, s.num_kv_heads, cache.page_size, table.shape[1])
+        if fast and not batch.n_prefill_items and batch.n_decode == n \
+                and rt.ops.attention_decode_fused_ok(s.head_dim, rotary_dim, inv_freq is not None,
+                                                     qkv.shape[0] if qkv.dim() == 3 else 1):
+            # single tokens only: norm, rotation, cache write and attention are one kernel
+            out = rt.empty((n, s.q_dim), rt.act_dtype)
+            rt.ops.attention_decode_fused(qkv, cache.k, cache.v, out, batch.decode_rows, batch.positions,
+                                          batch.seq_of_token, table, s.num_heads, s.num_kv_heads, s.head_dim,
+                                          self.q_norm, self.k_norm, eps, inv_freq, rotary_dim, cache.writable,
+                                          self.scale, s.window or 0, batch.max_decode_ctx, self._workspace(batch))
+            return rt.linear(out, self.w_o, slabs=True)
         q = rt.ops.qk_norm_rope_kv_write(
             qkv, rt.empty((n, s.q_dim), rt.act_dtype), cache.k, cache.v,
             batch.positions, batch.seq_of_token, table, s.num_heads, s.num_kv_heads, s.head_dim,
-            self.q_norm, self.k_norm, s.qk_norm_eps if s.qk_norm_eps is not None else 0.0,
-            inv_freq, rotary_dim, write_kv=cache.writable)
+            self.q_norm, self.k_norm, eps, inv_freq, rotary_dim, write_kv=cache.writable)
         out = rt.empty((n, s.q_dim), rt.act_dtype)
-        if rt.dtype == "bfloat16" and rt.ops.attention_fast_ok(s.num_heads, s.num_kv_heads, cache.page_size, table.shape[1]):
+        if fast:
             if batch.n_prefill_items:
                 rt.ops.attention_prefill(q, cache.k, cache.v, out, batch.prefill_seq, batch.prefill_tile, batch.q_start,
                                          batch.q_len, batch.positions, table, s.num_heads, s.num_kv_heads, s.head_dim,

@@ -313,6 +313,47 @@ def test_attention_decode(n_q, n_kv, d, page, window):
     assert not got[untouched].any()
 
 
+@pytest.mark.parametrize("n_q,n_kv,d,page", [(32, 8, 128, 16), (8, 1, 128, 8), (16, 1, 128, 16), (3, 3, 128, 4), (8, 2, 256, 32), (4, 2, 256, 16)])
+@pytest.mark.parametrize("window,norm,slabs,write_kv", [(0, True, 1, True), (300, True, 3, True), (0, False, 2, True), (0, True, 1, False)])
+def test_attention_decode_from_the_projection(n_q, n_kv, d, page, window, norm, slabs, write_kv):
+    """Decode attention that starts from the QKV projection's output: the same bits
+    in the attention output and in the cache as the rotary kernel followed by the
+    attention kernel, at split edges (256, 257, 513) and for the first token."""
+    ops = _ops()
+    rng = np.random.default_rng(n_q * 5 + d + window + slabs)
+    seq_lens = [1, 70, 300, 700, 256, 257, 513]
+    table, k, v = _paged_setup(rng, seq_lens, n_kv, d, page, torch.bfloat16)
+    t = len(seq_lens)
+    rows = list(range(t))
+    positions = [n - 1 for n in seq_lens]
+    seq_of = list(range(t))
+    width = (n_q + 2 * n_kv) * d
+    qkv = _t(rng.normal(size=(slabs, t, width)).astype(np.float32))
+    if slabs == 1:
+        qkv = qkv[0]
+    qw = _t((1 + 0.1 * rng.normal(size=d)).astype(np.float32)) if norm else None
+    kw = _t((1 + 0.1 * rng.normal(size=d)).astype(np.float32)) if norm else None
+    inv_freq = _t(np.power(1e6, -(2.0 * np.arange(d // 2)) / d).astype(np.float32))
+    args = (_t(positions, torch.int32), _t(seq_of, torch.int32), _t(table, torch.int32))
+    ws = ops.attention_decode_workspace(t, n_q, d, max(seq_lens), DEV)
+    # two kernels
+    k1, v1 = k.to(DEV), v.to(DEV)
+    q = ops.qk_norm_rope_kv_write(qkv, torch.empty(t, n_q * d, dtype=torch.bfloat16, device=DEV), k1, v1, *args, n_q, n_kv, d,
+                                  qw, kw, 1e-6, inv_freq, d, write_kv=write_kv)
+    want = ops.attention_decode(q, k1, v1, torch.zeros(t, n_q * d, dtype=torch.bfloat16, device=DEV), _t(rows, torch.int32),
+                                *args, n_q, n_kv, d, 1 / math.sqrt(d), window, max(seq_lens), ws)
+    # one kernel
+    k2, v2 = k.to(DEV), v.to(DEV)
+    got = ops.attention_decode_fused(qkv, k2, v2, torch.zeros(t, n_q * d, dtype=torch.bfloat16, device=DEV),
+                                     _t(rows, torch.int32), *args, n_q, n_kv, d, qw, kw, 1e-6, inv_freq, d, write_kv,
+                                     1 / math.sqrt(d), window, max(seq_lens), ws)
+    assert torch.equal(k1, k2) and torch.equal(v1, v2)
+    assert write_kv != torch.equal(k2.cpu(), k)            # the cache changed exactly when it was to be written
+    assert torch.equal(got, want)
+    assert not ops.attention_decode_fused_ok(64, 64, True) and not ops.attention_decode_fused_ok(128, 64, True)
+    assert ops.attention_decode_fused_ok(128, 64, False)
+
+
 @pytest.mark.parametrize("n_q,n_kv,d,page", [(32, 8, 128, 16), (6, 2, 48, 8), (4, 4, 64, 4), (3, 1, 80, 16), (2, 1, 256, 32), (2, 2, 16, 8)])
 @pytest.mark.parametrize("window", [0, 100])
 def test_attention_prefill(n_q, n_kv, d, page, window):
