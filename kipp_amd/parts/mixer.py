@@ -74,14 +74,14 @@ class Attention:
     def forward(self, x, batch, cache, state=None):
         s, rt = self.spec, self.rt
         n = x.shape[0]
-        qkv = rt.linear(x, self.w_qkv, slabs=True)
         inv_freq, rotary_dim = self.position.rotary_table()
         table = batch.block_tables[cache.group]
         eps = s.qk_norm_eps if s.qk_norm_eps is not None else 0.0
         fast = rt.dtype == "bfloat16" and rt.ops.attention_fast_ok(s.num_heads, s.num_kv_heads, cache.page_size, table.shape[1])
-        if fast and not batch.n_prefill_items and batch.n_decode == n \
-                and rt.ops.attention_decode_fused_ok(s.head_dim, rotary_dim, inv_freq is not None,
-                                                     qkv.shape[0] if qkv.dim() == 3 else 1):
+        fused = fast and not batch.n_prefill_items and batch.n_decode == n \
+            and rt.ops.attention_decode_fused_ok(s.head_dim, rotary_dim, inv_freq is not None)
+        qkv = rt.linear(x, self.w_qkv, slabs=rt.ops.DECODE_FUSED_SLABS if fused else True)
+        if fused:
             # single tokens only: norm, rotation, cache write and attention are one kernel
             out = rt.empty((n, s.q_dim), rt.act_dtype)
             rt.ops.attention_decode_fused(qkv, cache.k, cache.v, out, batch.decode_rows, batch.positions,

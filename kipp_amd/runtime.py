@@ -93,7 +93,8 @@ class Runtime:
         """float32 [M, N] = x [M, K] . w [N, K]^T.  With `slabs` the result may come
         as [parts, M, N] whose sum over parts is the product (few rows against a
         weight with few output rows: the contraction is split over workgroups and
-        the consumer adds the slabs in order).  With `low_precision_out` a large
+        the consumer adds the slabs in order); an integer is the most slabs the
+        consumer takes.  With `low_precision_out` a large
         bfloat16 product may be returned in bfloat16 (for a consumer that rounds to
         bfloat16 anyway and is bound by reading it)."""
         tiles = None
@@ -111,10 +112,11 @@ class Runtime:
             x = self.ops.cast(x, self.empty(x.shape, torch.bfloat16))
         if self.ops.gemm_skinny_ok(m, x.shape[1]):
             # few rows: our own kernels stream the weight once
+            most = 0 if slabs is False else (None if slabs is True else int(slabs))
             if m <= 16:
-                y = self.ops.gemm_skinny(x, w, max_parts=8 if slabs else 1, tiles=tiles)
+                y = self.ops.gemm_skinny(x, w, max_parts=1 if most == 0 else (most or 8), tiles=tiles)
             else:
-                y = self.ops.gemm_rows(x, w, max_parts=12 if slabs else 1, tiles=tiles)
+                y = self.ops.gemm_rows(x, w, max_parts=1 if most == 0 else (most or 12), tiles=tiles)
             return y if y.shape[0] > 1 else y[0]
         # bfloat16 x bfloat16 with float32 accumulation: the library product
         self.library_products += 1
