@@ -72,7 +72,8 @@ struct Projected {
     const float* q_norm_w;   // null: no norm
     const float* k_norm_w;
     float eps;
-    const float* inv_freq;   // null: no rotation
+    const float* inv_freq;   // null (and angles null): no rotation
+    const float* angles;     // [tokens][HEAD_DIM]: cosines then sines of every token's angles, or null: computed here
     int write_kv;            // 0: the cache is another layer's, keys and values are already there
 };
 
@@ -114,7 +115,7 @@ __global__ void __launch_bounds__(THREADS) attention_decode_kernel(
     // rotation need, before the keys and values are asked for: they are wanted first
     const bool owner = FUSED && pj.write_kv && split == last_split;   // this workgroup holds the token's own position
 #if FUSED_OK
-    float raw[JOBS][NC], norm_q[NC], norm_k[NC], freq[NC / 2];
+    float raw[JOBS][NC], norm_q[NC], norm_k[NC], freq[NC / 2], cs[NC / 2], sn[NC / 2];
     if (FUSED) {
         const size_t width = (size_t)(n_q + 2 * n_kv) * HEAD_DIM;
         int last_slab = pj.parts - 1;
@@ -147,7 +148,17 @@ __global__ void __launch_bounds__(THREADS) attention_decode_kernel(
             norm_k[c] = pj.k_norm_w != nullptr ? pj.k_norm_w[lane + c * KIPP_WAVE] : 1.0f;
         }
 #pragma unroll
-        for (int c = 0; c < NC / 2; ++c) freq[c] = pj.inv_freq != nullptr ? pj.inv_freq[lane + c * KIPP_WAVE] : 0.0f;
+        for (int c = 0; c < NC / 2; ++c) {
+            freq[c] = 0.0f;
+            cs[c] = 1.0f;
+            sn[c] = 0.0f;
+            if (pj.angles != nullptr) {
+                cs[c] = pj.angles[(size_t)row * HEAD_DIM + lane + c * KIPP_WAVE];
+                sn[c] = pj.angles[(size_t)row * HEAD_DIM + HEAD_DIM / 2 + lane + c * KIPP_WAVE];
+            } else if (pj.inv_freq != nullptr) {
+                freq[c] = pj.inv_freq[lane + c * KIPP_WAVE];
+            }
+        }
     }
 #endif
     if (tid < SPLIT) s_page[tid] = my_page;
@@ -188,12 +199,9 @@ __global__ void __launch_bounds__(THREADS) attention_decode_kernel(
     if (FUSED) {
         // norm (/root/reference/src/kipp.c:2480-2500), rotation (kipp.c:2368-2382), in the arithmetic of
         // the rotary kernel; the keys and values asked for above are on their way meanwhile
-        float cs[NC / 2], sn[NC / 2];
+        if (pj.angles == nullptr && pj.inv_freq != nullptr) {
 #pragma unroll
-        for (int c = 0; c < NC / 2; ++c) {
-            cs[c] = 1.0f;
-            sn[c] = 0.0f;
-            if (pj.inv_freq != nullptr) {
+            for (int c = 0; c < NC / 2; ++c) {
                 const float angle = (float)pos * freq[c];
                 cs[c] = cosf(angle);
                 sn[c] = sinf(angle);
@@ -440,10 +448,12 @@ int kipp_attention_decode_fused_ok() { return FUSED_OK ? 1 : 0; }
 int kipp_attention_decode_fused_slabs() { return MAX_SLABS; }
 
 // The same from the output of the QKV projection: `qkv` float32 [parts][tokens][(n_q + 2 n_kv) head_dim];
-// norm weights and `inv_freq` may be null (no norm, no rotation; a rotation covers the whole head);
+// norm weights, `inv_freq` and `angles` may be null (no norm; no rotation if both are null; a rotation covers
+// the whole head; `angles` [tokens][head_dim] holds every token's cosines, then sines);
 // with `write_kv` the token's key and value are written into the cache as well.
 int kipp_attention_decode_fused(const float* qkv, int parts, int n_tokens, const float* q_norm_w, const float* k_norm_w,
-                                float eps, const float* inv_freq, int write_kv, void* k_cache, void* v_cache, void* out,
+                                float eps, const float* inv_freq, const float* angles, int write_kv, void* k_cache,
+                                void* v_cache, void* out,
                                 float* part_acc, float* part_ml, const int32_t* rows, const int32_t* positions,
                                 const int32_t* seq_of_token, const int32_t* block_table, int max_blocks, int n_items,
                                 int n_q, int n_kv, int head_dim, int page, float scale, int window, int grid_splits,
@@ -454,7 +464,8 @@ int kipp_attention_decode_fused(const float* qkv, int parts, int n_tokens, const
     if (grid_splits <= 0 || grid_splits > max_splits) return -3;
     if (page <= 0 || (page & (page - 1))) return -4;
     const float scale_log2e = scale * 1.4426950408889634f;
-    Projected pj{qkv, parts, (size_t)n_tokens * (n_q + 2 * n_kv) * HEAD_DIM, q_norm_w, k_norm_w, eps, inv_freq, write_kv};
+    Projected pj{qkv, parts, (size_t)n_tokens * (n_q + 2 * n_kv) * HEAD_DIM, q_norm_w, k_norm_w, eps, inv_freq, angles,
+                 write_kv};
     hipLaunchKernelGGL(attention_decode_kernel<true>, dim3(grid_splits, n_kv, n_items), dim3(THREADS), 0, stream,
                        (const bf16_t*)nullptr, (bf16_t*)k_cache, (bf16_t*)v_cache, (bf16_t*)out, part_acc, part_ml,
                        rows, positions, seq_of_token, block_table, max_blocks, n_q, n_kv, page, scale_log2e, window,

@@ -147,14 +147,35 @@ def gather_rows(x: torch.Tensor, index: torch.Tensor, out: torch.Tensor) -> torc
 
 # --------------------------------------------------------------------------- attention
 
+def _angles_ok(angles, n_tokens: int, rotary_dim: int, what: str) -> None:
+    if angles is not None:
+        _need(angles.dtype == torch.float32 and angles.is_contiguous() and tuple(angles.shape) == (n_tokens, rotary_dim),
+              f"{what}: angles are float32 [tokens, rotary_dim]")
+
+
+def rotary_angles(positions: torch.Tensor, inv_freq: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[t] = [cos(float32(pos_t) * inv_freq[i]) for i | sin(...) for i], float32 [tokens, 2 * len(inv_freq)]:
+    the angles of a step, made once for every layer that rotates with these frequencies."""
+    _dev(positions, inv_freq, out)
+    _i32(positions, "positions")
+    half = inv_freq.numel()
+    _need(inv_freq.dtype == torch.float32 and out.dtype == torch.float32 and out.is_contiguous()
+          and tuple(out.shape) == (positions.numel(), 2 * half), "rotary_angles: out is float32 [tokens, 2 * len(inv_freq)]")
+    fn = _fn("rope_kv", "kipp_rotary_angles", [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr])
+    _check(fn(_ptr(positions), _ptr(inv_freq), _ptr(out), positions.numel(), half, _stream()), "rotary_angles")
+    return out
+
+
 def qk_norm_rope_kv_write(qkv: torch.Tensor, q_out: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                           positions: torch.Tensor, seq_of_token: torch.Tensor, block_table: torch.Tensor,
                           n_q: int, n_kv: int, head_dim: int,
                           q_norm_w: Optional[torch.Tensor], k_norm_w: Optional[torch.Tensor], eps: float,
-                          inv_freq: Optional[torch.Tensor], rotary_dim: int, write_kv: bool = True) -> torch.Tensor:
+                          inv_freq: Optional[torch.Tensor], rotary_dim: int, write_kv: bool = True,
+                          angles: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Per-head norm of q and k, rotation at each token's position, q to `q_out`
-    and k, v into their pages.  Caches are [pages, n_kv, page, head_dim]."""
-    _dev(qkv, q_out, k_cache, v_cache, positions, seq_of_token, block_table, q_norm_w, k_norm_w, inv_freq)
+    and k, v into their pages.  Caches are [pages, n_kv, page, head_dim].  With
+    `angles` (rotary_angles) the cosines and sines are read, not computed."""
+    _dev(qkv, q_out, k_cache, v_cache, positions, seq_of_token, block_table, q_norm_w, k_norm_w, inv_freq, angles)
     for t, name in ((positions, "positions"), (seq_of_token, "seq_of_token"), (block_table, "block_table")):
         _i32(t, name)
     n = qkv.shape[-2]
@@ -173,12 +194,13 @@ def qk_norm_rope_kv_write(qkv: torch.Tensor, q_out: torch.Tensor, k_cache: torch
     if inv_freq is not None:
         _need(inv_freq.dtype == torch.float32 and inv_freq.numel() == rotary_dim // 2 and rotary_dim % 2 == 0
               and 0 < rotary_dim <= head_dim, "qk_norm_rope: inv_freq is float32 [rotary_dim / 2]")
+    _angles_ok(angles, n, rotary_dim, "qk_norm_rope")
     fn = _fn("rope_kv", "kipp_qk_norm_rope_kv",
              [_c_ptr, _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int,
-              _c_ptr, _c_ptr, _c_float, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr])
+              _c_ptr, _c_ptr, _c_float, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr])
     _check(fn(_ptr(qkv), _code(qkv), _ptr(q_out), _code(q_out), _ptr(k_cache), _ptr(v_cache), _code(k_cache),
               _ptr(positions), _ptr(seq_of_token), _ptr(block_table), block_table.shape[1],
-              _ptr(q_norm_w), _ptr(k_norm_w), float(eps), _ptr(inv_freq), int(rotary_dim),
+              _ptr(q_norm_w), _ptr(k_norm_w), float(eps), _ptr(inv_freq), _ptr(angles), int(rotary_dim),
               n, n_q, n_kv, head_dim, k_cache.shape[2], 1 if write_kv else 0, parts, _stream()), "qk_norm_rope_kv_write")
     return q_out
 
@@ -276,14 +298,16 @@ def attention_decode_fused(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: to
                            block_table: torch.Tensor, n_q: int, n_kv: int, head_dim: int,
                            q_norm_w: Optional[torch.Tensor], k_norm_w: Optional[torch.Tensor], eps: float,
                            inv_freq: Optional[torch.Tensor], rotary_dim: int, write_kv: bool, scale: float, window: int,
-                           max_context: int, workspace: tuple, grid_splits: Optional[int] = None) -> torch.Tensor:
+                           max_context: int, workspace: tuple, grid_splits: Optional[int] = None,
+                           angles: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Decode attention straight from the QKV projection: per-head q/k RMSNorm,
     rotation, the write of the token's key and value into its page and the
     attention over the pages in one kernel (plus the merge of the splits).
     `qkv`: float32 [tokens, width] or slabs [parts, tokens, width]."""
-    _dev(qkv, k_cache, v_cache, out, rows, positions, seq_of_token, block_table, *workspace)
+    _dev(qkv, k_cache, v_cache, out, rows, positions, seq_of_token, block_table, angles, *workspace)
     for t, name in ((rows, "rows"), (positions, "positions"), (seq_of_token, "seq_of_token"), (block_table, "block_table")):
         _i32(t, name)
+    _angles_ok(angles, qkv.shape[-2], head_dim, "attention_decode_fused")
     _need(qkv.dtype == torch.float32 and qkv.dim() in (2, 3) and qkv.is_contiguous(), "attention_decode_fused: float32 qkv")
     parts = qkv.shape[0] if qkv.dim() == 3 else 1
     n_tokens = qkv.shape[-2]
@@ -311,10 +335,11 @@ def attention_decode_fused(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: to
           "attention_decode_fused: workspace too small for this context")
     defines = {"HEAD_DIM": head_dim, "GROUP": group}
     fn = _fn("attention_decode", "kipp_attention_decode_fused",
-             [_c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_float, _c_ptr, _c_int] + [_c_ptr] * 9 + [_c_int] * 6
+             [_c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_float, _c_ptr, _c_ptr, _c_int] + [_c_ptr] * 9 + [_c_int] * 6
              + [_c_float, _c_int, _c_int, _c_int, _c_ptr], defines)
     null = lambda t: _ptr(t) if t is not None else None
-    _check(fn(_ptr(qkv), parts, n_tokens, null(q_norm_w), null(k_norm_w), float(eps), null(inv_freq), 1 if write_kv else 0,
+    _check(fn(_ptr(qkv), parts, n_tokens, null(q_norm_w), null(k_norm_w), float(eps), null(inv_freq), null(angles),
+              1 if write_kv else 0,
               _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(part_acc), _ptr(part_ml), _ptr(rows), _ptr(positions),
               _ptr(seq_of_token), _ptr(block_table), block_table.shape[1], n_items, n_q, n_kv, head_dim,
               k_cache.shape[2], float(scale), int(window), grid, max_splits, _stream()), "attention_decode_fused")

@@ -8,6 +8,8 @@
 //          (/root/reference/src/kipp.c:2480-2500), before the rotation;
 //   rotary (u_i, u_{i+r/2}) <- (u_i c - u_{i+r/2} s, u_{i+r/2} c + u_i s),
 //          angle = float(pos) * inv_freq[i]  (kipp.c:2368-2382); dims >= r pass;
+//          with `angles` ([tokens][r]: r/2 cosines, then r/2 sines, made once a step by
+//          rotary_angles_kernel for all layers) the kernel reads them instead of computing them;
 //   write  key/value row of position pos goes to page table[pos / page], slot
 //          pos % page; cache layout [page][kv head][slot][d].
 #include "common.h"
@@ -21,7 +23,7 @@ __global__ void qk_norm_rope_kv_kernel(
     const int32_t* __restrict__ positions, const int32_t* __restrict__ seq_of_token,
     const int32_t* __restrict__ block_table, int max_blocks,
     const float* __restrict__ q_norm_w, const float* __restrict__ k_norm_w, float eps,
-    const float* __restrict__ inv_freq, int rotary_dim,
+    const float* __restrict__ inv_freq, const float* __restrict__ angles, int rotary_dim,
     int n_q, int n_kv, int d, int page, int n_slots, int parts, size_t part_stride) {
     __shared__ float buf[HEADS_PER_BLOCK][MAX_D];
     const int wave = threadIdx.x / KIPP_WAVE;
@@ -64,7 +66,7 @@ __global__ void qk_norm_rope_kv_kernel(
     __syncthreads();
     // Barriers stay outside the conditions: waves of one workgroup hold heads
     // of different kinds.
-    const bool rotate = kind != 2 && inv_freq != nullptr;
+    const bool rotate = kind != 2 && (inv_freq != nullptr || angles != nullptr);
     const int half = rotary_dim / 2;
     float lo[MAX_D / 2 / KIPP_WAVE], hi[MAX_D / 2 / KIPP_WAVE];
 #pragma unroll
@@ -72,8 +74,15 @@ __global__ void qk_norm_rope_kv_kernel(
         const int i = lane + c * KIPP_WAVE;
         lo[c] = hi[c] = 0.0f;
         if (rotate && i < half) {
-            const float angle = (float)pos * inv_freq[i];
-            const float cs = cosf(angle), sn = sinf(angle);
+            float cs, sn;
+            if (angles != nullptr) {
+                cs = angles[(size_t)t * rotary_dim + i];
+                sn = angles[(size_t)t * rotary_dim + half + i];
+            } else {
+                const float angle = (float)pos * inv_freq[i];
+                cs = cosf(angle);
+                sn = sinf(angle);
+            }
             const float a = buf[wave][i], b = buf[wave][i + half];
             lo[c] = a * cs - b * sn;
             hi[c] = b * cs + a * sn;
@@ -114,7 +123,8 @@ __global__ void __launch_bounds__(HEADS_PER_BLOCK * KIPP_WAVE) qk_norm_rope_kv_r
     const int32_t* __restrict__ positions, const int32_t* __restrict__ seq_of_token,
     const int32_t* __restrict__ block_table, int max_blocks,
     const float* __restrict__ q_norm_w, const float* __restrict__ k_norm_w, float eps,
-    const float* __restrict__ inv_freq, int n_q, int n_kv, int page, int n_slots, int parts, size_t part_stride) {
+    const float* __restrict__ inv_freq, const float* __restrict__ angles, int n_q, int n_kv, int page, int n_slots,
+    int parts, size_t part_stride) {
     constexpr int D = NC * KIPP_WAVE, HC = NC / 2, BATCH = 4;
     const int wave = threadIdx.x / KIPP_WAVE;
     const int lane = threadIdx.x & (KIPP_WAVE - 1);
@@ -128,7 +138,10 @@ __global__ void __launch_bounds__(HEADS_PER_BLOCK * KIPP_WAVE) qk_norm_rope_kv_r
     for (int c = 0; c < HC; ++c) {
         cs[c] = 1.0f;
         sn[c] = 0.0f;
-        if (inv_freq != nullptr) {
+        if (angles != nullptr) {
+            cs[c] = angles[(size_t)t * D + lane + c * KIPP_WAVE];
+            sn[c] = angles[(size_t)t * D + D / 2 + lane + c * KIPP_WAVE];
+        } else if (inv_freq != nullptr) {
             const float angle = (float)pos * inv_freq[lane + c * KIPP_WAVE];
             cs[c] = cosf(angle);
             sn[c] = sinf(angle);
@@ -197,8 +210,8 @@ __global__ void __launch_bounds__(HEADS_PER_BLOCK * KIPP_WAVE) qk_norm_rope_kv_r
 template <typename TI, typename TO, typename TC>
 static void launch_regs(const void* qkv, void* q_out, void* k_cache, void* v_cache, const int32_t* positions,
                         const int32_t* seq_of_token, const int32_t* block_table, int max_blocks, const float* q_norm_w,
-                        const float* k_norm_w, float eps, const float* inv_freq, int n_tokens, int n_q, int n_kv, int d,
-                        int page, int n_slots, int parts, hipStream_t stream) {
+                        const float* k_norm_w, float eps, const float* inv_freq, const float* angles, int n_tokens,
+                        int n_q, int n_kv, int d, int page, int n_slots, int parts, hipStream_t stream) {
     // few tokens: a wave for every head; many: a workgroup for a token
     const int per_token = n_tokens >= 256 ? 1 : (n_slots + HEADS_PER_BLOCK - 1) / HEADS_PER_BLOCK;
     dim3 grid(per_token, n_tokens), block(HEADS_PER_BLOCK * KIPP_WAVE);
@@ -206,7 +219,7 @@ static void launch_regs(const void* qkv, void* q_out, void* k_cache, void* v_cac
 #define KIPP_RR(NC, SLABS)                                                                                          \
     hipLaunchKernelGGL((qk_norm_rope_kv_regs_kernel<NC, SLABS, TI, TO, TC>), grid, block, 0, stream, (const TI*)qkv, \
                        (TO*)q_out, (TC*)k_cache, (TC*)v_cache, positions, seq_of_token, block_table, max_blocks,     \
-                       q_norm_w, k_norm_w, eps, inv_freq, n_q, n_kv, page, n_slots, parts, stride)
+                       q_norm_w, k_norm_w, eps, inv_freq, angles, n_q, n_kv, page, n_slots, parts, stride)
     if (d == 128) {
         if (parts > 1) KIPP_RR(2, true); else KIPP_RR(2, false);
     } else {
@@ -215,18 +228,39 @@ static void launch_regs(const void* qkv, void* q_out, void* k_cache, void* v_cac
 #undef KIPP_RR
 }
 
+// angles[t][i] = cos(float(pos_t) * inv_freq[i]), angles[t][half + i] = sin(...): once a step, for every
+// layer that rotates with these frequencies.
+__global__ void rotary_angles_kernel(const int32_t* __restrict__ positions, const float* __restrict__ inv_freq,
+                                     float* __restrict__ angles, int n_tokens, int half) {
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= n_tokens * half) return;
+    const int t = idx / half, i = idx % half;
+    const float angle = (float)positions[t] * inv_freq[i];
+    angles[(size_t)t * 2 * half + i] = cosf(angle);
+    angles[(size_t)t * 2 * half + half + i] = sinf(angle);
+}
+
+extern "C" int kipp_rotary_angles(const int32_t* positions, const float* inv_freq, float* angles, int n_tokens, int half,
+                                  hipStream_t stream) {
+    if (n_tokens <= 0 || half <= 0) return 0;
+    const int total = n_tokens * half;
+    hipLaunchKernelGGL(rotary_angles_kernel, dim3((total + 255) / 256), dim3(256), 0, stream, positions, inv_freq, angles,
+                       n_tokens, half);
+    return KIPP_LAUNCH_CHECK();
+}
+
 extern "C" int kipp_qk_norm_rope_kv(
     const void* qkv, int in_dtype, void* q_out, int q_dtype, void* k_cache, void* v_cache, int cache_dtype,
     const int32_t* positions, const int32_t* seq_of_token, const int32_t* block_table, int max_blocks,
-    const float* q_norm_w, const float* k_norm_w, float eps, const float* inv_freq, int rotary_dim,
+    const float* q_norm_w, const float* k_norm_w, float eps, const float* inv_freq, const float* angles, int rotary_dim,
     int n_tokens, int n_q, int n_kv, int d, int page, int write_kv, int parts, hipStream_t stream) {
     if (n_tokens <= 0) return 0;
     if (d > MAX_D || d <= 0 || rotary_dim > d || (rotary_dim & 1)) return -1;
     const int n_slots = write_kv ? n_q + 2 * n_kv : n_q;
-    if ((d == 128 || d == 256) && (inv_freq == nullptr || rotary_dim == d)) {
+    if ((d == 128 || d == 256) && ((inv_freq == nullptr && angles == nullptr) || rotary_dim == d)) {
 #define KIPP_RL(TI, TO, TC)                                                                                        \
     launch_regs<TI, TO, TC>(qkv, q_out, k_cache, v_cache, positions, seq_of_token, block_table, max_blocks, q_norm_w, \
-                            k_norm_w, eps, inv_freq, n_tokens, n_q, n_kv, d, page, n_slots, parts, stream)
+                            k_norm_w, eps, inv_freq, angles, n_tokens, n_q, n_kv, d, page, n_slots, parts, stream)
         if (in_dtype == KIPP_F32 && q_dtype == KIPP_F32 && cache_dtype == KIPP_F32) KIPP_RL(float, float, float);
         else if (in_dtype == KIPP_F32 && q_dtype == KIPP_BF16 && cache_dtype == KIPP_BF16) KIPP_RL(float, bf16_t, bf16_t);
         else if (in_dtype == KIPP_BF16 && q_dtype == KIPP_BF16 && cache_dtype == KIPP_BF16) KIPP_RL(bf16_t, bf16_t, bf16_t);
@@ -238,7 +272,7 @@ extern "C" int kipp_qk_norm_rope_kv(
 #define KIPP_RK(TI, TO, TC)                                                                                  \
     hipLaunchKernelGGL((qk_norm_rope_kv_kernel<TI, TO, TC>), grid, block, 0, stream, (const TI*)qkv,         \
                        (TO*)q_out, (TC*)k_cache, (TC*)v_cache, positions, seq_of_token, block_table,         \
-                       max_blocks, q_norm_w, k_norm_w, eps, inv_freq, rotary_dim, n_q, n_kv, d, page, n_slots, parts,      \
+                       max_blocks, q_norm_w, k_norm_w, eps, inv_freq, angles, rotary_dim, n_q, n_kv, d, page, n_slots, parts,      \
                        (size_t)n_tokens * (n_q + 2 * n_kv) * d)
     if (in_dtype == KIPP_F32 && q_dtype == KIPP_F32 && cache_dtype == KIPP_F32) KIPP_RK(float, float, float);
     else if (in_dtype == KIPP_F32 && q_dtype == KIPP_BF16 && cache_dtype == KIPP_BF16) KIPP_RK(float, bf16_t, bf16_t);

@@ -40,6 +40,7 @@ class StepBatch:
     max_q_len: int = 0
     max_ctx_len: int = 0
     host: dict = field(default_factory=dict)
+    step_cache: dict = field(default_factory=dict)   # device values of this forward that parts share; emptied by every forward
 
 
 PREFILL_TILE = 128   # query rows of one work item of the prefill attention kernel

@@ -84,6 +84,7 @@ class Model:
     def forward(self, batch, cache) -> Optional[torch.Tensor]:
         """Run the batch's tokens through every run of the order; float32 logits
         [wanted, vocab] at `batch.want_rows`, or None if nothing is wanted."""
+        batch.step_cache.clear()
         x = self.embedding.forward(batch.tokens)
         pending = None
         for index, run in enumerate(self.spec.order):

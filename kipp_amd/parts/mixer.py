@@ -75,6 +75,7 @@ class Attention:
         s, rt = self.spec, self.rt
         n = x.shape[0]
         inv_freq, rotary_dim = self.position.rotary_table()
+        angles = self.position.angles(batch) if hasattr(self.position, "angles") and hasattr(batch, "step_cache") else None
         table = batch.block_tables[cache.group]
         eps = s.qk_norm_eps if s.qk_norm_eps is not None else 0.0
         fast = rt.dtype == "bfloat16" and rt.ops.attention_fast_ok(s.num_heads, s.num_kv_heads, cache.page_size, table.shape[1])
@@ -87,12 +88,13 @@ class Attention:
             rt.ops.attention_decode_fused(qkv, cache.k, cache.v, out, batch.decode_rows, batch.positions,
                                           batch.seq_of_token, table, s.num_heads, s.num_kv_heads, s.head_dim,
                                           self.q_norm, self.k_norm, eps, inv_freq, rotary_dim, cache.writable,
-                                          self.scale, s.window or 0, batch.max_decode_ctx, self._workspace(batch))
+                                          self.scale, s.window or 0, batch.max_decode_ctx, self._workspace(batch),
+                                          angles=angles)
             return rt.linear(out, self.w_o, slabs=True)
         q = rt.ops.qk_norm_rope_kv_write(
             qkv, rt.empty((n, s.q_dim), rt.act_dtype), cache.k, cache.v,
             batch.positions, batch.seq_of_token, table, s.num_heads, s.num_kv_heads, s.head_dim,
-            self.q_norm, self.k_norm, eps, inv_freq, rotary_dim, write_kv=cache.writable)
+            self.q_norm, self.k_norm, eps, inv_freq, rotary_dim, write_kv=cache.writable, angles=angles)
         out = rt.empty((n, s.q_dim), rt.act_dtype)
         if fast:
             if batch.n_prefill_items:

@@ -3,6 +3,11 @@ it inside its own kernel; the interface is what that kernel needs:
 
     rotary_table() -> (inv_freq float32 [rotary_dim / 2] on the device, rotary_dim)
                       or (None, 0) when the part does not rotate
+    angles(batch)  -> float32 [tokens, rotary_dim] (cosines, then sines) of the
+                      batch's positions, or None; optional: a mixer computes
+                      the angles itself from `inv_freq` where it is missing.
+                      Parts with the same frequencies share one table a step
+                      (`batch.step_cache`, emptied at the start of every forward).
 
 A rotary part of another kind (scaled frequencies, another base) only has to
 produce its own table; pairing "half" rotates dim i with dim i + rotary_dim/2.
@@ -30,6 +35,9 @@ class NoPosition:
     def rotary_table(self):
         return None, 0
 
+    def angles(self, batch):
+        return None
+
 
 @register("position", "rope")
 class Rope:
@@ -43,6 +51,7 @@ class Rope:
         if spec.pairing != "half":
             raise ValueError(f"rope pairing {spec.pairing!r} is not implemented (only 'half')")
         self.spec = spec
+        self.rt = runtime
         self.rotary_dim = spec.head_dim if spec.rotary_dim is None else spec.rotary_dim
         self.inv_freq = self.frequencies().to(device=runtime.device, dtype=torch.float32)
 
@@ -60,3 +69,12 @@ class Rope:
 
     def rotary_table(self):
         return self.inv_freq, self.rotary_dim
+
+    def angles(self, batch):
+        key = ("rotary_angles", float(self.spec.theta), self.rotary_dim)
+        table = batch.step_cache.get(key)
+        if table is None:
+            table = self.rt.ops.rotary_angles(batch.positions, self.inv_freq,
+                                              self.rt.empty((batch.n_tokens, self.rotary_dim), torch.float32))
+            batch.step_cache[key] = table
+        return table

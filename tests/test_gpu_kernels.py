@@ -213,6 +213,18 @@ def test_qk_norm_rope_kv_write(n_q, n_kv, d, page, rotary, mode, norm):
         _t(positions, torch.int32), _t(seq_of, torch.int32), _t(table, torch.int32), n_q, n_kv, d,
         _t(qw) if norm else None, _t(kw) if norm else None, eps, _t(inv_freq), rotary)
 
+    # the same with the angles of the step made beforehand: the same bits
+    k2, v2 = k.to(DEV), v.to(DEV)
+    table_of_angles = ops.rotary_angles(_t(positions, torch.int32), _t(inv_freq), torch.empty(t, rotary, device=DEV))
+    q2 = ops.qk_norm_rope_kv_write(
+        _t(qkv), torch.empty(t, n_q * d, dtype=cdt, device=DEV), k2, v2,
+        _t(positions, torch.int32), _t(seq_of, torch.int32), _t(table, torch.int32), n_q, n_kv, d,
+        _t(qw) if norm else None, _t(kw) if norm else None, eps, None, rotary, angles=table_of_angles)
+    assert torch.equal(q2, q_out) and torch.equal(k2, kd) and torch.equal(v2, vd)
+    want = np.float32(np.array(positions, dtype=np.float32)[:, None] * inv_freq[None, :]).astype(np.float64)
+    got_angles = table_of_angles.cpu().numpy()
+    assert np.abs(got_angles[:, :half] - np.cos(want)).max() < 1e-6 and np.abs(got_angles[:, half:] - np.sin(want)).max() < 1e-6
+
     def ref_heads(x, n_heads, w):
         x = x.astype(np.float64)
         if norm:
@@ -348,6 +360,12 @@ def test_attention_decode_from_the_projection(n_q, n_kv, d, page, window, norm, 
                                      _t(rows, torch.int32), *args, n_q, n_kv, d, qw, kw, 1e-6, inv_freq, d, write_kv,
                                      1 / math.sqrt(d), window, max(seq_lens), ws)
     assert torch.equal(k1, k2) and torch.equal(v1, v2)
+    k3, v3 = k.to(DEV), v.to(DEV)
+    angles = ops.rotary_angles(args[0], inv_freq, torch.empty(t, d, device=DEV))
+    again = ops.attention_decode_fused(qkv, k3, v3, torch.zeros(t, n_q * d, dtype=torch.bfloat16, device=DEV),
+                                       _t(rows, torch.int32), *args, n_q, n_kv, d, qw, kw, 1e-6, None, d, write_kv,
+                                       1 / math.sqrt(d), window, max(seq_lens), ws, angles=angles)
+    assert torch.equal(again, got) and torch.equal(k3, k2) and torch.equal(v3, v2)
     assert write_kv != torch.equal(k2.cpu(), k)            # the cache changed exactly when it was to be written
     assert torch.equal(got, want)
     assert not ops.attention_decode_fused_ok(64, 64, True) and not ops.attention_decode_fused_ok(128, 64, True)
