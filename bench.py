@@ -62,15 +62,27 @@ def fill(engine, ids, prompt_len, vocab, seed, chunk=2048):
 
 
 def decode_run(engine, ids, tokens, steps, warmup):
-    """`warmup` untimed and `steps` timed decode steps of all `ids` together."""
+    """`warmup` untimed and `steps` timed decode steps of all `ids` together, as the
+    scheduler runs them: tokens are chosen greedily on the device and feed the next
+    step from there; the host reads them one step behind, while that step runs."""
     import torch
     from kipp_amd.engine import StepEntry
-    cur = [tokens[r] for r in ids]
+    from kipp_amd.sampling import SampleParams
+
+    class Greedy:
+        params, rng, recent = SampleParams(), None, ()
+    rows = [Greedy()] * len(ids)
+    logits = engine.step([StepEntry(r, [tokens[r]], [0]) for r in ids])
+    picks = engine.choose(logits, rows, wait=False)
+    entries = [StepEntry(r, [0], [0]) for r in ids]
 
     def one():
-        nonlocal cur
-        logits = engine.step([StepEntry(r, [t], [0]) for r, t in zip(ids, cur)])
-        cur = engine.rt.ops.argmax(logits, engine.rt.empty((len(ids),), torch.int32)).cpu().tolist()
+        nonlocal picks
+        logits = engine.step(entries, device_tokens=picks.device)
+        ahead = engine.choose(logits, rows, wait=False)
+        for r, t in zip(ids, picks.result()):
+            engine.commit(r, [t])                    # what the step just launched was fed
+        picks = ahead
     for _ in range(warmup):
         one()
     torch.cuda.synchronize()

@@ -85,7 +85,9 @@ def main(argv=None) -> int:
     backend = f"hip-{args.dtype}"
     print(f"kipp: evaluating {len(tokens)} token{'s' if len(tokens) != 1 else ''} on {backend}", file=sys.stderr)
 
-    sched = Scheduler(engine, max_step_tokens=args.max_step_tokens, prefill_chunk=args.prefill_chunk, max_running=1)
+    # no running ahead: the logits printed at the end are those of the last token that counts
+    sched = Scheduler(engine, max_step_tokens=args.max_step_tokens, prefill_chunk=args.prefill_chunk, max_running=1,
+                      lookahead=False)
     params = SampleParams(temperature=args.temperature, top_p=args.top_p, top_k=args.top_k, min_p=args.min_p)
     req = Request("cli", tokens, max(args.decode, 0), params, seed=args.seed, stop_tokens=stops)
     sched.add(req)
@@ -94,8 +96,8 @@ def main(argv=None) -> int:
     last = {}
     inner_step = engine.step
 
-    def keeping_step(entries):
-        logits = inner_step(entries)
+    def keeping_step(entries, **kw):
+        logits = inner_step(entries, **kw)
         if logits is not None:
             last["row"] = logits[-1]
         return logits

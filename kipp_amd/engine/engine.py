@@ -40,6 +40,7 @@ class Engine:
         self.cache = CacheManager(model.kv_needs(), model.state_needs(), page_size, num_pages, max_requests,
                                   model.spec.max_position, runtime=self.rt, share_prefixes=share_prefixes)
         self.graphs = DecodeGraphs(self) if use_graphs else None
+        self._uncommitted = {}      # request -> tokens of a step run from device_tokens and not recorded yet
 
     @classmethod
     def from_folder(cls, model_dir: str, dtype: str = "bfloat16", device: str = "cuda:0", **kw) -> "Engine":
@@ -50,22 +51,38 @@ class Engine:
         return self.cache.open(request_id, prompt, publish_early)
 
     def close(self, request_id) -> None:
+        self._uncommitted.pop(request_id, None)     # a step that was never recorded leaves nothing behind
         self.cache.close(request_id)
 
     def length(self, request_id) -> int:
         return self.cache.requests[request_id].length
 
     # -- the step ---------------------------------------------------------------------
-    def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+    def step(self, entries: Sequence[StepEntry], device_tokens: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
         """Run one batch.  Requests not yet open are opened.  Raises OutOfPages
-        (nothing changed) when the pools cannot hold the step."""
+        (nothing changed) when the pools cannot hold the step.
+
+        With `device_tokens` (int32 [entries] on the device) every entry brings one
+        token that the host does not know yet, for instance the choice of the step
+        before, which is still running: the step reads entry i's token from
+        `device_tokens[i]` (the values in `entries` are ignored), and what the
+        cache records is put off until `commit(request, tokens)` tells it, which
+        must happen before the request's next step."""
         if not entries:
             return None
+        if device_tokens is not None:
+            if self.graphs is None or not self.graphs.applies(entries):
+                raise ValueError("tokens on the device need a step of single tokens that is replayed as a graph")
+            if device_tokens.dtype != torch.int32 or device_tokens.numel() != len(entries) \
+                    or device_tokens.device != self.rt.device:
+                raise ValueError("device_tokens must be int32 [entries] on the engine's device")
         seen = set()
         requests = []
         for e in entries:
             if e.request in seen:
                 raise ValueError(f"request {e.request!r} appears twice in one step")
+            if e.request in self._uncommitted:
+                raise ValueError(f"request {e.request!r}: the tokens of its last step are not recorded yet (commit)")
             seen.add(e.request)
             if len(e.tokens) == 0:
                 raise ValueError(f"request {e.request!r}: an entry needs at least one token")
@@ -89,7 +106,7 @@ class Engine:
             raise
         try:
             if self.graphs is not None and self.graphs.applies(entries):
-                logits = self.graphs.run(entries, requests)
+                logits = self.graphs.run(entries, requests, device_tokens)
             else:
                 batch = build_batch(entries, requests, len(self.cache.groups), self.rt.device)
                 logits = self.model.forward(batch, self.cache)
@@ -99,40 +116,79 @@ class Engine:
             for rid in opened:
                 self.cache.close(rid)
             raise
-        for r, e in zip(requests, entries):
-            self.cache.commit(r, e.tokens)
+        if device_tokens is None:
+            for r, e in zip(requests, entries):
+                self.cache.commit(r, e.tokens)
+        else:
+            for r in requests:
+                self._uncommitted[r.id] = 1
         return logits
 
+    def commit(self, request_id, tokens: Sequence[int]) -> None:
+        """The tokens of a step that ran from `device_tokens` are known now."""
+        if self._uncommitted.pop(request_id, 0) != len(tokens):
+            raise ValueError(f"request {request_id!r} has no step of {len(tokens)} tokens waiting to be recorded")
+        self.cache.commit(self.cache.requests[request_id], tokens)
+
     # -- token choice -------------------------------------------------------------------
-    def choose(self, logits: torch.Tensor, requests: Sequence[object]) -> List[int]:
+    def choose(self, logits: torch.Tensor, requests: Sequence[object], wait: bool = True):
         """One token for each row of `logits`; `requests[i]` carries the row's
         sampling parameters, generator and recent tokens.  Rows are chosen on the
         device in one launch (greedy and temperature rows alike; the uniform draw
         of a temperature row comes from its request's generator on the host).
         Only rows whose logits are changed first (bias, penalties) go through the
-        host sampler."""
+        host sampler.  With `wait` false the choice is not waited for: the result
+        is a `Picks` whose `device` tensor can feed the next step at once and whose
+        `result()` gives the tokens when the host needs them."""
         from ..sampling import sample
         rows = logits.shape[0]
         if rows != len(requests):
             raise ValueError("one request for each row of logits")
         on_host = [i for i, r in enumerate(requests) if r.params.changes_logits]
-        temperature, top_k, top_p, min_p, uniform = [], [], [], [], []
-        for i, req in enumerate(requests):
-            p = req.params
-            sampled = not p.greedy and i not in on_host
-            if sampled:
-                p.validate()
-            temperature.append(float(p.temperature) if sampled else 0.0)
-            top_k.append(int(p.top_k) if sampled else 0)
-            top_p.append(float(p.top_p) if sampled else 1.0)
-            min_p.append(float(p.min_p) if sampled else 0.0)
-            uniform.append(req.rng.uniform() if sampled else 0.0)
-        dev = self.rt.device
-        f32 = lambda v: torch.tensor(v, dtype=torch.float32, device=dev)
-        picked = self.rt.ops.sample(logits, f32(temperature), torch.tensor(top_k, dtype=torch.int32, device=dev),
-                                    f32(top_p), f32(min_p), torch.tensor(uniform, dtype=torch.float64, device=dev),
-                                    self.rt.empty((rows,), torch.int32)).cpu().tolist()
+        if on_host and not wait:
+            raise ValueError("rows whose logits are changed on the host cannot be chosen without waiting")
+        picked = self.rt.empty((rows,), torch.int32)
+        if all(r.params.greedy for r in requests):
+            self.rt.ops.argmax(logits, picked)
+        else:
+            # all parameters in one pinned buffer and one copy: [temperature | top_p | min_p | top_k | uniform (8 bytes)]
+            pack = torch.empty(rows * 24, dtype=torch.uint8).pin_memory()
+            f32 = pack[:rows * 12].view(torch.float32)
+            i32 = pack[rows * 12:rows * 16].view(torch.int32)
+            f64 = pack[rows * 16:].view(torch.float64)
+            for i, req in enumerate(requests):
+                p = req.params
+                sampled = not p.greedy and i not in on_host
+                if sampled:
+                    p.validate()
+                f32[i] = float(p.temperature) if sampled else 0.0
+                f32[rows + i] = float(p.top_p) if sampled else 1.0
+                f32[2 * rows + i] = float(p.min_p) if sampled else 0.0
+                i32[i] = int(p.top_k) if sampled else 0
+                f64[i] = req.rng.uniform() if sampled else 0.0
+            dev = pack.to(self.rt.device, non_blocking=True)
+            d32 = dev[:rows * 12].view(torch.float32)
+            self.rt.ops.sample(logits, d32[:rows], dev[rows * 12:rows * 16].view(torch.int32), d32[rows:2 * rows],
+                               d32[2 * rows:], dev[rows * 16:].view(torch.float64), picked)
+        if not wait:
+            return Picks(picked)
+        out = picked.cpu().tolist()
         for i in on_host:
             req = requests[i]
-            picked[i] = sample(logits[i].cpu().numpy(), req.params, req.rng, list(req.recent))
-        return picked
+            out[i] = sample(logits[i].cpu().numpy(), req.params, req.rng, list(req.recent))
+        return out
+
+
+class Picks:
+    """Tokens chosen on the device and on their way to the host."""
+
+    def __init__(self, device: torch.Tensor):
+        self.device = device
+        self.host = torch.empty(device.shape, dtype=device.dtype).pin_memory()
+        self.host.copy_(device, non_blocking=True)
+        self.ready = torch.cuda.Event()
+        self.ready.record()
+
+    def result(self) -> List[int]:
+        self.ready.synchronize()
+        return self.host.tolist()

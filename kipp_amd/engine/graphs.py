@@ -61,11 +61,11 @@ class DecodeGraph:
         self.copied: Optional[torch.cuda.Event] = None
         self.row_marks = [None] * n
 
-    def fill(self, entries, requests) -> None:
+    def fill(self, entries, requests, device_tokens=None) -> None:
         n, h = self.n, self.host_np
         if self.copied is not None:
             self.copied.synchronize()     # the copy of the step before has left the pinned buffer
-        h[0:n] = [e.tokens[0] for e in entries]
+        h[0:n] = 0 if device_tokens is not None else [e.tokens[0] for e in entries]
         lengths = [r.length for r in requests]
         h[n:2 * n] = lengths
         h[2 * n:3 * n] = h[n:2 * n] + 1
@@ -86,9 +86,11 @@ class DecodeGraph:
         self.dev[:upto].copy_(self.host[:upto], non_blocking=True)
         self.copied = torch.cuda.Event()
         self.copied.record()
+        if device_tokens is not None:
+            self.dev[:n].copy_(device_tokens)     # on the device, after the copy above: the tokens the host does not know
 
-    def run(self, engine, entries, requests) -> torch.Tensor:
-        self.fill(entries, requests)
+    def run(self, engine, entries, requests, device_tokens=None) -> torch.Tensor:
+        self.fill(entries, requests, device_tokens)
         if self.graph is None:
             # the first step with this shape runs eagerly (it also makes every workspace the
             # kernels keep); if nothing in it went to a library, the same launches are then
@@ -130,7 +132,7 @@ class DecodeGraphs:
         return (self.possible and 0 < len(entries) <= 64
                 and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries))
 
-    def run(self, entries, requests) -> torch.Tensor:
+    def run(self, entries, requests, device_tokens=None) -> torch.Tensor:
         engine = self._engine()
         cache = engine.cache
         longest = max(r.length for r in requests) + 1
@@ -141,4 +143,4 @@ class DecodeGraphs:
             graph = self.graphs[key] = DecodeGraph(engine, len(entries), bucket)
         if graph.graph is not None:
             self.replays += 1
-        return graph.run(engine, entries, requests)
+        return graph.run(engine, entries, requests, device_tokens)

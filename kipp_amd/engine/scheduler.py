@@ -21,6 +21,11 @@ Policy (the reference's server loop lifted out of its HTTP code,
   its last place.
 * A sampled stop token ends the request and is neither kept nor fed back;
   reaching `max_new_tokens` ends it without running the last token.
+* While every running request decodes and none waits, the scheduler runs one step
+  ahead of what it knows (`lookahead`): the next step is launched with the tokens
+  still on the device, and the tokens of the step before are read while it runs,
+  so the GPU never waits for the host.  A request that a stop token ends has then
+  run one step in vain; its cache goes back whole.  The tokens are the same.
 """
 from __future__ import annotations
 
@@ -80,10 +85,29 @@ class SchedulerStats:
     waits_for_prefix: int = 0
 
 
+class _PicksRows:
+    """Some rows of a choice that is still on its way."""
+
+    def __init__(self, picks, rows):
+        self.picks, self.rows = picks, list(rows)
+
+    @property
+    def device(self):
+        return self.picks.device[self.rows]
+
+    def result(self):
+        chosen = self.picks.result()
+        return [chosen[i] for i in self.rows]
+
+
 class Scheduler:
-    def __init__(self, engine, max_step_tokens: int = 2048, prefill_chunk: int = 512, max_running: int = 64):
+    def __init__(self, engine, max_step_tokens: int = 2048, prefill_chunk: int = 512, max_running: int = 64,
+                 lookahead: bool = True):
         if max_step_tokens < 1 or prefill_chunk < 1 or max_running < 1:
             raise ValueError("budgets must be positive")
+        # running ahead needs an engine that takes a step's tokens from the device
+        self.lookahead = lookahead and getattr(engine, "graphs", None) is not None
+        self._ahead = None          # (requests, Picks) of the step launched last, its choice not yet read
         self.engine = engine
         self.cache = engine.cache
         self.max_step_tokens = max_step_tokens
@@ -131,6 +155,7 @@ class Scheduler:
         self.stats.requests += 1
 
     def cancel(self, request_id) -> None:
+        self._drain()
         for req in list(self.waiting):
             if req.id == request_id:
                 self.waiting.remove(req)
@@ -209,23 +234,82 @@ class Scheduler:
 
     def step(self) -> List[Tuple[object, int]]:
         """Admit, run one batch, sample.  Returns the (request id, token) pairs
-        produced by this step."""
+        that became known in this step."""
+        if self._ahead is not None:
+            if not self.waiting:
+                return self._step_ahead()
+            produced = self._drain()                       # someone waits: back to steps that may bring prompts
+        else:
+            produced = []
         self._admit()
         plan = self.plan()
         if not plan:
-            return []
+            return produced
         entries = [StepEntry(req.id, tokens, want) for req, tokens, want in plan]
         logits = self.engine.step(entries)
         self.stats.steps += 1
-        produced: List[Tuple[object, int]] = []
         sampling = [req for req, _, want in plan if want]
         for req, tokens, want in plan:
             if req.state == "prefill":
                 req.fed += len(tokens)
                 self.stats.prompt_tokens += len(tokens)
         if sampling:
+            if self._may_run_ahead(plan, sampling):
+                self._ahead = (sampling, self.engine.choose(logits, sampling, wait=False))
+                return produced
             chosen = self.engine.choose(logits, sampling)
             for req, token in zip(sampling, chosen):
+                self._accept(req, int(token), produced)
+        return produced
+
+    # -- one step ahead --------------------------------------------------------------------
+    def _may_run_ahead(self, plan, sampling) -> bool:
+        return (self.lookahead and not self.waiting and len(sampling) == len(plan) == len(self.running)
+                and all(req.state == "decode" and not req.params.changes_logits for req in sampling)
+                and self.engine.graphs.applies([StepEntry(req.id, [0], [0]) for req in sampling]))
+
+    def _step_ahead(self) -> List[Tuple[object, int]]:
+        """The step launched last has not told its tokens yet.  Launch the next one
+        from them where they are, then read them and settle the last step."""
+        reqs, picks = self._ahead
+        # requests that the length ends with the token still on its way need no further step
+        go_on = [i for i, req in enumerate(reqs) if len(req.output) + 1 < req.max_new_tokens]
+        nxt = None
+        if go_on:
+            cont = [reqs[i] for i in go_on]
+            tokens = picks.device if len(go_on) == len(reqs) else picks.device[go_on]
+            logits = self.engine.step([StepEntry(req.id, [0], [0]) for req in cont], device_tokens=tokens.contiguous())
+            self.stats.steps += 1
+            nxt = (cont, self.engine.choose(logits, cont, wait=False))
+        produced: List[Tuple[object, int]] = []
+        chosen = picks.result()
+        for req, token in zip(reqs, chosen):
+            self._accept(req, int(token), produced)
+        if nxt is not None:
+            cont, ahead = nxt
+            alive = []
+            for i, req in enumerate(cont):
+                if req.state == "decode":
+                    self.engine.commit(req.id, [req.next_token])   # what the step just launched was fed
+                    alive.append(i)
+            # a request that its token has just ended ran that step in vain: its row is left out from here on
+            if len(alive) == len(cont):
+                self._ahead = nxt
+            elif alive:
+                self._ahead = ([cont[i] for i in alive], _PicksRows(ahead, alive))
+            else:
+                self._ahead = None
+        else:
+            self._ahead = None
+        return produced
+
+    def _drain(self) -> List[Tuple[object, int]]:
+        """Read the tokens of the step launched last and go back to knowing everything."""
+        produced: List[Tuple[object, int]] = []
+        if self._ahead is not None:
+            reqs, picks = self._ahead
+            self._ahead = None
+            for req, token in zip(reqs, picks.result()):
                 self._accept(req, int(token), produced)
         return produced
 

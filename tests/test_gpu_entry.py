@@ -60,6 +60,47 @@ def test_requests_that_begin_alike_share_pages_and_still_follow_plain(model_fold
     assert engine.cache.free_pages() == [64]
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_running_one_step_ahead_changes_nothing(model_folders, dtype):
+    """The scheduler launches a decode step before it has read the tokens of the
+    step before.  Same tokens as when it waits for every step: greedy and seeded
+    temperature requests, different lengths, a stop token that ends a request one
+    step late, a request that arrives in the middle; every page comes back."""
+    from kipp_amd.engine import Engine
+    from kipp_amd.engine.scheduler import Request, Scheduler
+    from kipp_amd.sampling import SampleParams
+    folder = model_folders[("a", dtype)]
+    prompts = [H.random_tokens(90 + i, n, 256) for i, n in enumerate([5, 17, 33, 2, 9])]
+
+    def run(lookahead, stop_of_first=()):
+        engine = Engine.from_folder(folder, dtype=dtype, page_size=16, max_tokens=5 * 128, share_prefixes=False)
+        sched = Scheduler(engine, max_step_tokens=64, prefill_chunk=16, lookahead=lookahead)
+        for i, prompt in enumerate(prompts[:4]):
+            params = SampleParams(temperature=0.9, top_k=40, top_p=0.95) if i % 2 else SampleParams()
+            sched.add(Request(i, prompt, [40, 7, 23, 31][i], params=params, seed=11 + i,
+                              stop_tokens=tuple(stop_of_first) if i == 0 else ()))
+        steps = 0
+        while not sched.idle:
+            sched.step()
+            steps += 1
+            if steps == 12:
+                sched.add(Request(4, prompts[4], 15))          # arrives while the others decode
+        engine.cache.check()
+        assert engine.cache.free_pages() == [40] and not engine._uncommitted
+        return {rid: (r.output, r.finish_reason) for rid, r in sched.finished.items()}, sched.stats
+
+    plainly, _ = run(False)
+    ahead, stats = run(True)
+    assert ahead == plainly and [len(ahead[i][0]) for i in range(5)] == [40, 7, 23, 31, 15]
+    # end request 0 early by a stop token it is known to produce: one step late, nothing else changes
+    stop = plainly[0][0][20]
+    first = plainly[0][0].index(stop)
+    stopped, _ = run(True, stop_of_first=[stop])
+    assert stopped[0] == (plainly[0][0][:first], "stop")
+    assert all(stopped[i] == plainly[i] for i in range(1, 5))
+    assert run(False, stop_of_first=[stop])[0] == stopped
+
+
 def test_long_decoding_matches_plain(model_folders, tiny_configs):
     """100 tokens decoded one by one after a short prompt, every logits row compared."""
     from kipp_amd.engine import Engine, StepEntry
