@@ -47,3 +47,47 @@ def test_benchmark_layer_sizes_match_plain(real_folder, real_reference, dtype):
             if dtype == "float32":
                 assert np.array_equal(got[rid].argmax(axis=1), refs[rid].argmax(axis=1))
         del engine
+
+
+@pytest.fixture(scope="module")
+def long_folder(tmp_path_factory):
+    """Head size 128 and a long context on a narrow model: decoding runs through the
+    fused attention kernel and the recorded graphs, over many splits of the keys."""
+    from kipp_amd.config import shape_config
+    from kipp_amd.weights import write_random_model
+    cfg = shape_config("tiny-a")
+    cfg.update(hidden_size=96, num_attention_heads=4, num_key_value_heads=1, head_dim=128, intermediate_size=160,
+               vocab_size=311, num_hidden_layers=2, max_position_embeddings=2304, tie_word_embeddings=False)
+    folder = str(tmp_path_factory.mktemp("long") / "narrow-long")
+    write_random_model(folder, cfg, seed=5, dtype="bfloat16")
+    return folder
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decoding_across_a_graph_bucket_and_many_splits(long_folder, dtype):
+    """A prompt of 1,000 tokens in portions, then 60 tokens one by one: the context
+    passes 1,024 (another recorded graph) and split edges; two more requests decode
+    beside it, one of them ending early so that the batch shrinks; every row against
+    the plain implementation."""
+    from kipp_amd.engine import Engine, StepEntry
+    cfg, weights = plain.load_folder(long_folder)
+    seqs = {"long": H.random_tokens(31, 1060, 311), "mid": H.random_tokens(32, 300, 311), "short": H.random_tokens(33, 40, 311)}
+    refs = {k: plain.forward_whole(cfg, weights, v) for k, v in seqs.items()}
+    tol = H.NMSE_F32 if dtype == "float32" else H.NMSE_BF16
+    engine = Engine.from_folder(long_folder, dtype=dtype, page_size=16, max_tokens=1088 + 320 + 64, max_requests=3,
+                                share_prefixes=False)
+    fed = {"long": 1000, "mid": 240, "short": 10}
+    for rid, n in fed.items():                                  # prompts in portions of 300
+        for at in range(0, n, 300):
+            engine.step([StepEntry(rid, seqs[rid][at:min(at + 300, n)], [])])
+    got = {rid: [] for rid in seqs}
+    for _ in range(60):
+        live = [rid for rid in seqs if fed[rid] < len(seqs[rid])]
+        logits = engine.step([StepEntry(rid, [seqs[rid][fed[rid]]], [0]) for rid in live]).cpu().numpy()
+        for row, rid in zip(logits, live):
+            got[rid].append(row)
+            fed[rid] += 1
+    assert engine.graphs.replays > 40 and len(engine.graphs.graphs) >= 3     # 3 and 2 requests, contexts below and above 1,024
+    for rid in seqs:
+        first = {"long": 1000, "mid": 240, "short": 10}[rid]
+        H.assert_close(np.stack(got[rid]), refs[rid][first:fed[rid]], tol, f"long context/{dtype}/{rid}")
