@@ -1,7 +1,8 @@
 """The framework is open: a mixer with state of its own, a windowed attention
-layer, a layer named twice and a layer that reads another layer's cache are
-defined HERE, registered, built and stepped without a change to the
-framework's files.  None of this is a model of anyone's."""
+layer, a layer named twice, a layer that reads another layer's cache, a
+feed-forward with routing and another position encoding are defined HERE,
+registered, built and stepped without a change to the framework's files.
+None of this is a model of anyone's."""
 from dataclasses import dataclass
 
 import numpy as np
@@ -176,3 +177,151 @@ def test_window_pages_return_early_and_slots_start_from_zero(toy_folder):
     again = H.random_tokens(10, 12, VOCAB)
     got = engine.step([StepEntry("x", again, list(range(12)))]).cpu().numpy()
     H.assert_close(got, _plain_toy(weights, again), H.NMSE_F32, "slot reuse")
+
+
+# ---------------------------------------------------------------------------------------------------
+# A feed-forward with routing and another position encoding, again defined here only.
+
+EXPERTS, R_INNER, STRETCH = 3, 24, 4.0
+
+
+@dataclass(frozen=True)
+class RoutedSpec:
+    hidden_size: int
+    experts: int
+    inner: int
+    prefix: str = ""
+    kind: str = "toy_routed"
+
+
+@dataclass(frozen=True)
+class StretchedRopeSpec:
+    head_dim: int
+    theta: float
+    stretch: float
+    kind: str = "toy_stretched_rope"
+
+
+def _register_routed():
+    from kipp_amd.config import register_architecture
+    from kipp_amd.config.specs import (AttentionSpec, EmbeddingSpec, HeadSpec, LayerRun, LayerSpec, ModelSpec, RMSNormSpec)
+    from kipp_amd.parts import ParamSpec, register
+
+    @register("feed_forward", "toy_routed")
+    class RoutedFFN:
+        """Every token goes to the one expert its router logit is largest for;
+        delta = p * W2_e silu(W1_e x) with p the softmax weight of that expert
+        (router logits and softmax in float32)."""
+
+        def __init__(self, spec, runtime):
+            self.spec, self.rt = spec, runtime
+
+        @staticmethod
+        def params(spec):
+            out = {"router.weight": ParamSpec((spec.experts, spec.hidden_size))}
+            for e in range(spec.experts):
+                out[f"experts.{e}.w1.weight"] = ParamSpec((spec.inner, spec.hidden_size))
+                out[f"experts.{e}.w2.weight"] = ParamSpec((spec.hidden_size, spec.inner))
+            return out
+
+        def load(self, tensors):
+            self.t = tensors
+
+        def forward(self, x, batch=None):
+            logits = self.rt.linear(x, self.t["router.weight"])
+            weight, expert = torch.softmax(logits.float(), dim=-1).max(dim=-1)
+            delta = torch.zeros(x.shape, dtype=torch.float32, device=x.device)
+            for e in range(self.spec.experts):
+                rows = (expert == e).nonzero().flatten()
+                if rows.numel():
+                    h = torch.nn.functional.silu(self.rt.linear(x[rows].contiguous(), self.t[f"experts.{e}.w1.weight"]))
+                    delta[rows] = self.rt.linear(h.to(x.dtype).contiguous(), self.t[f"experts.{e}.w2.weight"]) * weight[rows, None]
+            return delta
+
+    @register("position", "toy_stretched_rope")
+    class StretchedRope:
+        """Rotation with every frequency divided by `stretch`.  It gives the mixer its
+        table of frequencies and nothing else: the mixer computes the angles itself."""
+
+        def __init__(self, spec, runtime):
+            i = torch.arange(spec.head_dim // 2, dtype=torch.float64)
+            freq = torch.pow(torch.tensor(float(spec.theta), dtype=torch.float64), -(2.0 * i) / spec.head_dim) / spec.stretch
+            self.inv_freq, self.head_dim = freq.to(device=runtime.device, dtype=torch.float32), spec.head_dim
+
+        @staticmethod
+        def params(spec):
+            return {}
+
+        def load(self, tensors):
+            pass
+
+        def rotary_table(self):
+            return self.inv_freq, self.head_dim
+
+    class RoutedConfig:
+        def __init__(self, d):
+            self.d = d
+
+        def to_dict(self):
+            return dict(self.d)
+
+        def model_spec(self):
+            def layer(i):
+                p = f"layers.{i}."
+                attn = AttentionSpec(HIDDEN, HEADS, KV, D, position=StretchedRopeSpec(D, THETA, STRETCH), qk_norm_eps=None,
+                                     prefix=p + "attn.")
+                return LayerSpec(block="pre_norm", parts=(
+                    ("mixer_norm", RMSNormSpec(HIDDEN, EPS, p + "n1.")), ("mixer", attn),
+                    ("ffn_norm", RMSNormSpec(HIDDEN, EPS, p + "n2.")), ("ffn", RoutedSpec(HIDDEN, EXPERTS, R_INNER, p + "moe."))))
+            layers = (layer(0), layer(1))
+            return ModelSpec("ToyRoutedForTests", HIDDEN, VOCAB, 256, EmbeddingSpec(VOCAB, HIDDEN, "embed."), layers,
+                             (LayerRun(0), LayerRun(1)), RMSNormSpec(HIDDEN, EPS, "norm."), HeadSpec(VOCAB, HIDDEN, True))
+
+    register_architecture("ToyRoutedForTests", RoutedConfig)
+
+
+def _plain_routed(w, tokens):
+    t = len(tokens)
+    pos = np.arange(t) / STRETCH                        # dividing the frequencies is dividing the positions
+    x = plain.embed(w["embed.weight"], tokens)
+    for i in range(2):
+        p = f"layers.{i}."
+        n = plain.rms_norm(x, w[p + "n1.weight"], EPS)
+        q = plain.rope(plain.linear(n, w[p + "attn.q_proj.weight"]), HEADS, D, pos, THETA)
+        k = plain.rope(plain.linear(n, w[p + "attn.k_proj.weight"]), KV, D, pos, THETA)
+        v = plain.linear(n, w[p + "attn.v_proj.weight"])
+        x = x + plain.linear(plain.causal_gqa(q, k, v, HEADS, KV, D), w[p + "attn.o_proj.weight"])
+        n = plain.rms_norm(x, w[p + "n2.weight"], EPS)
+        probs = plain.softmax(plain.linear(n, w[p + "moe.router.weight"]))
+        delta = np.zeros_like(x)
+        for row in range(t):
+            e = int(probs[row].argmax())
+            h = plain.silu(plain.linear(n[row:row + 1], w[p + f"moe.experts.{e}.w1.weight"]))
+            delta[row] = probs[row, e] * plain.linear(h, w[p + f"moe.experts.{e}.w2.weight"])[0]
+        x = x + delta
+    return plain.linear(plain.rms_norm(x, w["norm.weight"], EPS), w["embed.weight"])
+
+
+@pytest.mark.parametrize("cut", ["whole", "portions", "mixed"])
+def test_routed_feed_forward_and_another_position_encoding(tmp_path, cut):
+    from kipp_amd.config import unregister_architecture
+    from kipp_amd.engine import Engine
+    from kipp_amd.parts import unregister
+    from kipp_amd.weights import write_random_model
+    _register_routed()
+    try:
+        folder = write_random_model(str(tmp_path / "routed"), {"architectures": ["ToyRoutedForTests"]}, seed=8, dtype="float32")
+        _, weights = plain.load_folder(folder)
+        requests = {f"r{i}": H.random_tokens(20 + i, n, VOCAB) for i, n in enumerate([7, 45, 30])}
+        steps = {"whole": H.whole, "portions": H.changing_portions, "mixed": lambda r: H.mixed(r, seed=5)}[cut](requests)
+        engine = Engine.from_folder(folder, dtype="float32", page_size=8, num_pages=H.peak_pages(requests, steps, 8),
+                                    max_requests=4)
+        assert engine.graphs is None or not engine.graphs.possible          # parts that do not declare graph_safe run eagerly
+        got = H.replay(engine, requests, steps)
+        for rid, toks in requests.items():
+            H.assert_close(got[rid], _plain_routed(weights, toks), H.NMSE_F32, f"routed/{cut}/{rid}")
+        assert engine.cache.free_pages() == [engine.cache.groups[0].pool.num_pages]
+    finally:
+        unregister_architecture("ToyRoutedForTests")
+        unregister("feed_forward", "toy_routed")
+        unregister("position", "toy_stretched_rope")
