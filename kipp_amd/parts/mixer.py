@@ -19,6 +19,9 @@ from ..cache.needs import KVNeed
 from .base import ParamSpec, build_part, register
 
 
+FUSED_DECODE_ROWS = 16   # up to this many single tokens take the fused decode attention
+
+
 @register("mixer", "attention")
 class Attention:
     """Causal grouped-query attention with optional per-head q/k RMSNorm, a
@@ -79,11 +82,13 @@ class Attention:
         table = batch.block_tables[cache.group]
         eps = s.qk_norm_eps if s.qk_norm_eps is not None else 0.0
         fast = rt.dtype == "bfloat16" and rt.ops.attention_fast_ok(s.num_heads, s.num_kv_heads, cache.page_size, table.shape[1])
-        fused = fast and not batch.n_prefill_items and batch.n_decode == n \
+        # a few single tokens: norm, rotation, cache write and attention in one kernel.  (With many rows the
+        # attention is bound by reading the cache, and the fused kernel's lower occupancy costs more there
+        # than the rotary kernel it saves.)
+        fused = fast and not batch.n_prefill_items and batch.n_decode == n and n <= FUSED_DECODE_ROWS \
             and rt.ops.attention_decode_fused_ok(s.head_dim, rotary_dim, inv_freq is not None)
         qkv = rt.linear(x, self.w_qkv, slabs=rt.ops.DECODE_FUSED_SLABS if fused else True)
         if fused:
-            # single tokens only: norm, rotation, cache write and attention are one kernel
             out = rt.empty((n, s.q_dim), rt.act_dtype)
             rt.ops.attention_decode_fused(qkv, cache.k, cache.v, out, batch.decode_rows, batch.positions,
                                           batch.seq_of_token, table, s.num_heads, s.num_kv_heads, s.head_dim,
