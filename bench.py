@@ -102,6 +102,7 @@ def main():
     ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the shape has (named in config)")
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--prompt", type=int, default=2048)
+    ap.add_argument("--context", type=int, default=None, help="context length (default: the shape's)")
     ap.add_argument("--points", default="1,64", help="further decode batch sizes")
     ap.add_argument("--no-prefill", action="store_true")
     args = ap.parse_args()
@@ -118,6 +119,8 @@ def main():
     full_layers = config["num_hidden_layers"]
     layers = args.layers or full_layers
     config["num_hidden_layers"] = layers
+    if args.context:
+        config["max_position_embeddings"] = args.context
     _, cfg = parse_config(config)
     context = cfg.max_position_embeddings
     points = [int(b) for b in args.points.split(",") if b]
