@@ -4,11 +4,13 @@ prompt, generate `--decode` tokens, print the final top-N logits and one
 KIPP_METRIC line.  The prompt is token ids (this engine has no tokenizer).
 
     python -m kipp_amd.cli --model DIR --tokens 5,17,3 --decode 16
+    python -m kipp_amd.cli --model DIR --ppl tokens.u32 --ppl-window 512
     python -m kipp_amd.cli --write-random DIR --random tiny-a --seed-weights 7
 """
 from __future__ import annotations
 
 import argparse
+import math
 import struct
 import sys
 import time
@@ -31,6 +33,7 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--model", help="model folder (config.json, model.safetensors)")
     ap.add_argument("--tokens", help="prompt as token ids: 5,17,3")
     ap.add_argument("--tokens-file", help="prompt as little-endian uint32 token ids")
+    ap.add_argument("--backend", default="hip", help="explicit backend; this engine has one, hip, and never falls back")
     ap.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16",
                     help="execution path (default bfloat16; float32 is the true 32-bit path)")
     ap.add_argument("--decode", type=int, default=0, help="greedy/sampled tokens to generate")
@@ -40,6 +43,9 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--min-p", type=float, default=0.0, help="min prob vs top, 0 <= F <= 1 (0 = off)")
     ap.add_argument("--seed", type=int, default=1, help="nonzero sampling seed (default 1)")
     ap.add_argument("--top", type=int, default=10, help="final top-N logits to print (default 10)")
+    ap.add_argument("--ppl", metavar="FILE", help="perplexity over a little-endian uint32 token file")
+    ap.add_argument("--ppl-window", type=int, default=512, help="tokens of one window; each starts from an empty context")
+    ap.add_argument("--ppl-limit", type=int, default=0, help="score at most this many tokens of the file (0 = all)")
     ap.add_argument("--stop-token", type=int, action="append", default=None,
                     help="token that ends decoding (default: eos_token_id of config.json)")
     ap.add_argument("--page", type=int, default=16, help="tokens per cache page")
@@ -53,8 +59,58 @@ def build_parser() -> argparse.ArgumentParser:
     return ap
 
 
+def run_perplexity(args) -> int:
+    """Windows of `--ppl-window` tokens that do not overlap, each from an empty
+    context, no burn-in; a window of W tokens scores its W - 1 targets
+    (/root/reference/src/kipp_cli.c:646-801: the protocol and the lines printed)."""
+    import torch
+    from .engine import Engine, StepEntry
+    with open(args.ppl, "rb") as f:
+        raw = f.read()
+    if len(raw) % 4:
+        raise SystemExit(f"kipp: ppl: '{args.ppl}' is not a uint32 token file")
+    stream = list(struct.unpack(f"<{len(raw) // 4}I", raw))
+    if args.ppl_limit:
+        stream = stream[:args.ppl_limit]
+    if len(stream) < 2:
+        raise SystemExit("kipp: ppl: need at least two tokens to score")
+    window = args.ppl_window
+    engine = Engine.from_folder(args.model, dtype=args.dtype, page_size=args.page,
+                                num_pages=args.kv_pages or -(-window // args.page), max_requests=1, share_prefixes=False)
+    if not 2 <= window <= engine.model.spec.max_position:
+        raise SystemExit(f"kipp: --ppl-window must be between 2 and {engine.model.spec.max_position}")
+    for index, token in enumerate(stream):
+        if not 0 <= token < engine.vocab_size:
+            raise SystemExit(f"kipp: ppl: token {index} is out of range")
+    windows = -(-len(stream) // window)
+    nll, scored = 0.0, 0
+    torch.cuda.synchronize()
+    started = time.perf_counter()
+    for w in range(windows):
+        tokens = stream[w * window:(w + 1) * window]
+        if len(tokens) < 2:
+            break                                      # a tail of one token has nothing to score
+        for at in range(0, len(tokens), args.prefill_chunk):
+            chunk = tokens[at:at + args.prefill_chunk]
+            rows = [r for r in range(len(chunk)) if at + r + 1 < len(tokens)]
+            logits = engine.step([StepEntry("ppl", chunk, rows)])
+            if rows:
+                targets = torch.tensor([tokens[at + r + 1] for r in rows], device=logits.device)
+                wide = logits.double()
+                nll += float((torch.logsumexp(wide, dim=-1) - wide.gather(1, targets[:, None])[:, 0]).sum())
+                scored += len(rows)
+        engine.close("ppl")
+        print(f"ppl: window {w + 1}/{windows} ppl={math.exp(nll / scored):.4f}", file=sys.stderr)
+    torch.cuda.synchronize()
+    print(f"KIPP_PPL backend=hip-{args.dtype} tokens={len(stream)} scored={scored} window={window} nll={nll:.9f} "
+          f"ppl={math.exp(nll / scored):.6f} seconds={time.perf_counter() - started:.3f}", file=sys.stderr)
+    return 0
+
+
 def main(argv=None) -> int:
     args = build_parser().parse_args(argv)
+    if args.backend != "hip":
+        raise SystemExit(f"kipp: backend {args.backend!r} is not built into this engine (only hip)")
     if args.write_random:
         from .config import shape_config
         from .weights import write_random_model
@@ -65,6 +121,8 @@ def main(argv=None) -> int:
         return 0
     if not args.model:
         raise SystemExit("kipp: --model is required")
+    if args.ppl:
+        return run_perplexity(args)
     if not 1 <= args.top <= 100:
         raise SystemExit("kipp: --top must be between 1 and 100")
     if args.seed == 0:

@@ -157,6 +157,35 @@ def test_command_line(model_folders):
     assert "KIPP_METRIC backend=hip-float32 prefill_tokens=4" in run.stderr and "decode_tokens=5" in run.stderr
 
 
+def test_command_line_perplexity(model_folders, tmp_path):
+    """--ppl: windows that do not overlap, each from an empty context, a window of W
+    tokens scores W - 1 targets; against the plain implementation."""
+    import struct
+    folder = model_folders[("b", "float32")]
+    stream = H.random_tokens(55, 75, 509)
+    path = tmp_path / "tokens.u32"
+    path.write_bytes(struct.pack("<75I", *stream))
+    run = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "kipp"), "--model", folder, "--dtype", "float32", "--page", "8",
+                          "--ppl", str(path), "--ppl-window", "32", "--prefill-chunk", "10"], capture_output=True, text=True, timeout=300)
+    assert run.returncode == 0, run.stderr
+    nll, scored = 0.0, 0
+    for at in range(0, 75, 32):
+        tokens = stream[at:at + 32]
+        logits = H.plain_logits(folder, tokens)
+        for r in range(len(tokens) - 1):
+            row = logits[r]
+            nll += row.max() + np.log(np.exp(row - row.max()).sum()) - row[tokens[r + 1]]
+            scored += 1
+    line = [l for l in run.stderr.splitlines() if l.startswith("KIPP_PPL")][0]
+    fields = dict(f.split("=") for f in line.split()[1:])
+    assert fields["backend"] == "hip-float32" and int(fields["tokens"]) == 75 and int(fields["scored"]) == scored == 72
+    assert abs(float(fields["nll"]) - nll) < 1e-3 and abs(float(fields["ppl"]) - np.exp(nll / scored)) < 1e-3
+    assert "ppl: window 3/3" in run.stderr
+    bad = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "kipp"), "--model", folder, "--backend", "metal", "--tokens", "1"],
+                         capture_output=True, text=True, timeout=300)
+    assert bad.returncode != 0 and "only hip" in bad.stderr
+
+
 def _trace(requests, steps):
     fed = {r: 0 for r in requests}
     lines = []
