@@ -29,12 +29,23 @@ def _code(t: torch.Tensor) -> int:
         raise KernelError(f"kernels take float32 or bfloat16 tensors, got {t.dtype}") from None
 
 
+# The helpers below run a few hundred times in a step that is not replayed as a graph, so they
+# are kept cheap: plain integers for pointers, the raw stream handle, one dictionary lookup for a
+# kernel's entry point.
+
 def _ptr(t: Optional[torch.Tensor]):
-    return _c_ptr(t.data_ptr()) if t is not None else _c_ptr(0)
+    return t.data_ptr() if t is not None else None
+
+
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_raw_device = getattr(torch._C, "_cuda_getDevice", None)
 
 
 def _stream():
-    return _c_ptr(torch.cuda.current_stream().cuda_stream)
+    """torch's current stream of the current device (also the one a graph is recorded on)."""
+    if _raw_stream is not None and _raw_device is not None:
+        return _raw_stream(_raw_device())
+    return torch.cuda.current_stream().cuda_stream
 
 
 def _need(cond: bool, msg: str) -> None:
@@ -44,27 +55,26 @@ def _need(cond: bool, msg: str) -> None:
 
 def _dev(*tensors: Optional[torch.Tensor]) -> None:
     for t in tensors:
-        if t is None:
-            continue
-        _need(t.is_cuda, "kernel operand is not on the GPU (there is no CPU path)")
-        _need(t.is_contiguous(), "kernel operand is not contiguous")
+        if t is not None and not (t.is_cuda and t.is_contiguous()):
+            raise KernelError("kernel operand is not on the GPU (there is no CPU path)" if not t.is_cuda
+                              else "kernel operand is not contiguous")
 
 
 def _i32(t: torch.Tensor, name: str) -> None:
     _need(t.dtype == torch.int32, f"{name} must be int32, got {t.dtype}")
 
 
-_sigs_set = set()
+_entry_points = {}
 
 
 def _fn(lib_name: str, fn_name: str, argtypes, defines=None):
-    lib = build.library(lib_name, defines)
-    fn = getattr(lib, fn_name)
-    key = (lib._name, fn_name)
-    if key not in _sigs_set:
+    key = (lib_name, fn_name, tuple(sorted(defines.items())) if defines else None)
+    fn = _entry_points.get(key)
+    if fn is None:
+        fn = getattr(build.library(lib_name, defines), fn_name)
         fn.argtypes = argtypes
         fn.restype = _c_int
-        _sigs_set.add(key)
+        _entry_points[key] = fn
     return fn
 
 
