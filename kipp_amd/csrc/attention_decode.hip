@@ -32,6 +32,7 @@
 // key/value head, <= 16).
 #include "common.h"
 #include <math.h>
+#include <type_traits>
 
 #ifndef HEAD_DIM
 #error "compile with -DHEAD_DIM=<head size>"
@@ -378,17 +379,243 @@ __global__ void __launch_bounds__(THREADS) attention_decode_kernel(
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// The same attention for long contexts.  A workgroup takes a long range of keys (BIG) and walks
+// it in blocks of SUB keys with a running maximum and sum per head; while block i is worked on,
+// the keys and values of block i + 1 are on their way into a second set of registers.  Against
+// the kernel above this saves page lookups, partial results and merge work per key, which pays
+// from several thousand keys on (measured: a sixth faster at 30,000 keys); at a few thousand
+// keys the kernel above, which has more bytes in flight, is faster.  Partial results have the
+// same layout, and the same merge kernel adds the ranges in order.
+#define SUB 128
+#define BIG 1024
+#ifndef STREAM_FROM
+#define STREAM_FROM 8192                         // keys from which the launcher takes this kernel
+#endif
+#define SUB_BLOCKS_PER_WAVE (SUB / 16 / WAVES)   // 16-key blocks of a sub-block that a wave scores
+#define SUB_KEYS_PER_GROUP (SUB / 16)            // keys of a sub-block that a lane group multiplies with values
+
+__global__ void __launch_bounds__(THREADS) attention_decode_stream_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
+    bf16_t* __restrict__ out, float* __restrict__ part_acc, float* __restrict__ part_ml,
+    const int32_t* __restrict__ rows, const int32_t* __restrict__ positions, const int32_t* __restrict__ seq_of_token,
+    const int32_t* __restrict__ block_table, int max_blocks, int n_q, int n_kv, int page, float scale_log2e,
+    int window, int max_splits) {
+    __shared__ float s_scores[GROUP][SUB + 4];
+    __shared__ float s_red[WAVES][GROUP][HEAD_DIM];
+    __shared__ float s_m[GROUP], s_l[GROUP], s_alpha[GROUP];
+    __shared__ int s_page[BIG];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l16 = lane & 15, h = lane >> 4;
+    const int kvh = blockIdx.y;
+    const int row = rows[blockIdx.z];
+    const int pos = positions[row];
+    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+    const int first_split = lo / BIG, last_split = pos / BIG;
+    const int split = first_split + blockIdx.x;
+    if (split > last_split) return;
+    const int n_splits = last_split - first_split + 1;
+    const int base = split * BIG;
+    const int n_sub = (min(BIG, pos + 1 - base) + SUB - 1) / SUB;      // blocks that hold a key up to the query's own
+    const int32_t* table = block_table + (size_t)seq_of_token[row] * max_blocks;
+    const int page_shift = __builtin_ctz(page);
+
+    for (int i = tid; i < n_sub * SUB; i += THREADS) s_page[i] = table[min(base + i, pos) >> page_shift];
+    if (tid < GROUP) {
+        s_m[tid] = -INFINITY;
+        s_l[tid] = 0.0f;
+    }
+    Frag qf[KSTEPS];
+#pragma unroll
+    for (int t = 0; t < KSTEPS; ++t) {
+        const int dcol = min(32 * t + 8 * h, HEAD_DIM - 8);
+        qf[t].u = *(const u32x4*)(q + ((size_t)row * n_q + (size_t)kvh * GROUP + min(l16, GROUP - 1)) * HEAD_DIM + dcol);
+    }
+    __syncthreads();
+
+    Frag kf[2][SUB_BLOCKS_PER_WAVE][KSTEPS], vf[2][SUB_KEYS_PER_GROUP][CHUNKS_PER_LANE];
+    const int kg = wave * 4 + h;                      // this lane group's keys of a sub-block: kg + 16 i
+    auto fetch = [&](auto set, int sub) {
+        constexpr int S = decltype(set)::value;
+        const int first = sub * SUB;
+#pragma unroll
+        for (int b = 0; b < SUB_BLOCKS_PER_WAVE; ++b) {
+            const int kl = first + (wave * SUB_BLOCKS_PER_WAVE + b) * 16 + l16;
+            const int sk = min(base + kl, pos);
+            const bf16_t* k_row = k_cache + (((size_t)s_page[kl] * n_kv + kvh) * page + (sk & (page - 1))) * HEAD_DIM;
+#pragma unroll
+            for (int t = 0; t < KSTEPS; ++t) kf[S][b][t].u = *(const u32x4*)(k_row + min(32 * t + 8 * h, HEAD_DIM - 8));
+        }
+#pragma unroll
+        for (int i = 0; i < SUB_KEYS_PER_GROUP; ++i) {
+            const int kl = first + kg + 16 * i;
+            const int sk = min(base + kl, pos);
+            const bf16_t* v_row = v_cache + (((size_t)s_page[kl] * n_kv + kvh) * page + (sk & (page - 1))) * HEAD_DIM;
+#pragma unroll
+            for (int c = 0; c < CHUNKS_PER_LANE; ++c) vf[S][i][c].u = *(const u32x4*)(v_row + min(l16 + 16 * c, CHUNKS - 1) * 8);
+        }
+    };
+
+    float acc[GROUP][CHUNKS_PER_LANE][8];
+#pragma unroll
+    for (int g = 0; g < GROUP; ++g)
+#pragma unroll
+        for (int c = 0; c < CHUNKS_PER_LANE; ++c)
+#pragma unroll
+            for (int j = 0; j < 8; ++j) acc[g][c][j] = 0.0f;
+#pragma unroll
+    for (int t = 0; t < KSTEPS; ++t)
+        if (32 * t + 8 * h >= HEAD_DIM || l16 >= GROUP) qf[t].u = (u32x4){0u, 0u, 0u, 0u};
+
+    auto work = [&](auto set, int sub) {
+        constexpr int S = decltype(set)::value;
+        const int first = base + sub * SUB;
+        // ---- scores of this sub-block
+#pragma unroll
+        for (int b = 0; b < SUB_BLOCKS_PER_WAVE; ++b) {
+            f32x4 sc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int t = 0; t < KSTEPS; ++t) sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[S][b][t].v, qf[t].v, sc, 0, 0, 0);
+            if (l16 < GROUP) {
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const int kl = (wave * SUB_BLOCKS_PER_WAVE + b) * 16 + 4 * h + v;
+                    const int sk = first + kl;
+                    s_scores[l16][kl] = (sk >= lo && sk <= pos) ? sc[v] * scale_log2e : -INFINITY;
+                }
+            }
+        }
+        __syncthreads();
+        // ---- running maximum and sum, one head per wave at a time
+        for (int g = wave; g < GROUP; g += WAVES) {
+            float sc[SUB / KIPP_WAVE];
+            float m = -INFINITY;
+#pragma unroll
+            for (int i = 0; i < SUB / KIPP_WAVE; ++i) {
+                sc[i] = s_scores[g][lane + KIPP_WAVE * i];
+                m = fmaxf(m, sc[i]);
+            }
+            m = wave_max(m);
+            const float m_old = s_m[g];
+            const float m_new = fmaxf(m_old, m);
+            const float m_use = m_new == -INFINITY ? 0.0f : m_new;     // nothing visible yet: every weight is 0
+            float l = 0.0f;
+#pragma unroll
+            for (int i = 0; i < SUB / KIPP_WAVE; ++i) {
+                const float pw = exp2f(sc[i] - m_use);
+                s_scores[g][lane + KIPP_WAVE * i] = pw;
+                l += pw;
+            }
+            l = wave_sum(l);
+            if (lane == 0) {
+                const float alpha = exp2f(m_old - m_use);                // m_old = -inf gives 0
+                s_alpha[g] = alpha;
+                s_l[g] = s_l[g] * alpha + l;
+                s_m[g] = m_new;
+            }
+        }
+        __syncthreads();
+        // ---- values: what was gathered so far is brought to the new maximum, then this sub-block is added
+        float alpha[GROUP];
+#pragma unroll
+        for (int g = 0; g < GROUP; ++g) alpha[g] = s_alpha[g];
+#pragma unroll
+        for (int g = 0; g < GROUP; ++g)
+#pragma unroll
+            for (int c = 0; c < CHUNKS_PER_LANE; ++c)
+#pragma unroll
+                for (int j = 0; j < 8; ++j) acc[g][c][j] *= alpha[g];
+#pragma unroll
+        for (int i = 0; i < SUB_KEYS_PER_GROUP; ++i) {
+            const int kl = kg + 16 * i;
+            float pw[GROUP];
+#pragma unroll
+            for (int g = 0; g < GROUP; ++g) pw[g] = s_scores[g][kl];
+#pragma unroll
+            for (int c = 0; c < CHUNKS_PER_LANE; ++c) {
+                float vv[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    vv[j] = __uint_as_float((j & 1) ? (vf[S][i][c].u[j >> 1] & 0xffff0000u) : (vf[S][i][c].u[j >> 1] << 16));
+#pragma unroll
+                for (int g = 0; g < GROUP; ++g)
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) acc[g][c][j] = fmaf(pw[g], vv[j], acc[g][c][j]);
+            }
+        }
+        __syncthreads();                              // the scores are overwritten by the next sub-block
+    };
+
+    using Set0 = std::integral_constant<int, 0>;
+    using Set1 = std::integral_constant<int, 1>;
+    fetch(Set0{}, 0);
+    for (int sub = 0; sub < n_sub; sub += 2) {
+        if (sub + 1 < n_sub) fetch(Set1{}, sub + 1);
+        work(Set0{}, sub);
+        if (sub + 1 < n_sub) {
+            if (sub + 2 < n_sub) fetch(Set0{}, sub + 2);
+            work(Set1{}, sub + 1);
+        }
+    }
+
+    // sum the four lane groups of the wave, then the waves
+#pragma unroll
+    for (int g = 0; g < GROUP; ++g)
+#pragma unroll
+        for (int c = 0; c < CHUNKS_PER_LANE; ++c)
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                float a = acc[g][c][j];
+                a += __shfl_xor(a, 16, KIPP_WAVE);
+                a += __shfl_xor(a, 32, KIPP_WAVE);
+                acc[g][c][j] = a;
+            }
+    if (h == 0) {
+#pragma unroll
+        for (int g = 0; g < GROUP; ++g)
+#pragma unroll
+            for (int c = 0; c < CHUNKS_PER_LANE; ++c) {
+                const int chunk = l16 + 16 * c;
+                if (chunk < CHUNKS) {
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) s_red[wave][g][chunk * 8 + j] = acc[g][c][j];
+                }
+            }
+    }
+    __syncthreads();
+    for (int idx = tid; idx < GROUP * HEAD_DIM; idx += THREADS) {
+        const int g = idx / HEAD_DIM, dcol = idx % HEAD_DIM;
+        float a = 0.0f;
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w) a += s_red[w][g][dcol];
+        const int head = kvh * GROUP + g;
+        if (n_splits == 1) {
+            out[((size_t)row * n_q + head) * HEAD_DIM + dcol] = f32_to_bf16(a / s_l[g]);
+        } else {
+            const size_t slot = ((size_t)blockIdx.z * n_q + head) * max_splits + blockIdx.x;
+            part_acc[slot * HEAD_DIM + dcol] = a;
+            if (dcol == 0) {
+                part_ml[slot * 2] = s_m[g];
+                part_ml[slot * 2 + 1] = s_l[g];
+            }
+        }
+    }
+}
+
 // Merge the splits of every (token, head) in index order:
 // m* = max m_s, out = sum_s acc_s 2^(m_s - m*) / sum_s l_s 2^(m_s - m*)
 // (/root/reference/metal/kipp_kernels.metal:741-779).
 __global__ void attention_decode_reduce_kernel(
     const float* __restrict__ part_acc, const float* __restrict__ part_ml, bf16_t* __restrict__ out,
-    const int32_t* __restrict__ rows, const int32_t* __restrict__ positions, int n_q, int window, int max_splits) {
+    const int32_t* __restrict__ rows, const int32_t* __restrict__ positions, int n_q, int window, int max_splits,
+    int split_keys) {
     const int head = blockIdx.x, item = blockIdx.y;
     const int row = rows[item];
     const int pos = positions[row];
     const int lo = window > 0 ? max(0, pos - window + 1) : 0;
-    const int n_splits = pos / SPLIT - lo / SPLIT + 1;
+    const int n_splits = pos / split_keys - lo / split_keys + 1;
     if (n_splits == 1) return;
     const size_t slot0 = ((size_t)item * n_q + head) * max_splits;
     // the (m, l) pairs of all splits, one a lane, so that they arrive together
@@ -432,6 +659,20 @@ int kipp_attention_decode(const void* q, const void* k_cache, const void* v_cach
     if (grid_splits <= 0 || grid_splits > max_splits) return -3;
     if (page <= 0 || (page & (page - 1))) return -4;   // pages of a power of two only
     const float scale_log2e = scale * 1.4426950408889634f;
+    // Long contexts: long ranges of keys walked by each workgroup, if that still gives every compute
+    // unit two workgroups.  A function of the launch's shape, never of the data.
+    const int big_splits = (grid_splits * SPLIT + BIG - 1) / BIG + (window > 0 ? 1 : 0);
+    if (grid_splits * SPLIT >= STREAM_FROM && (long long)n_items * n_kv * big_splits >= 2 * 256 && big_splits <= max_splits) {
+        hipLaunchKernelGGL(attention_decode_stream_kernel, dim3(big_splits, n_kv, n_items), dim3(THREADS), 0, stream,
+                           (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, part_acc,
+                           part_ml, rows, positions, seq_of_token, block_table, max_blocks, n_q, n_kv, page, scale_log2e,
+                           window, max_splits);
+        int rc = KIPP_LAUNCH_CHECK();
+        if (rc != 0 || big_splits == 1) return rc;
+        hipLaunchKernelGGL(attention_decode_reduce_kernel, dim3(n_q, n_items), dim3(HEAD_DIM >= 64 ? 64 : HEAD_DIM), 0,
+                           stream, part_acc, part_ml, (bf16_t*)out, rows, positions, n_q, window, max_splits, BIG);
+        return KIPP_LAUNCH_CHECK();
+    }
     hipLaunchKernelGGL(attention_decode_kernel<false>, dim3(grid_splits, n_kv, n_items), dim3(THREADS), 0, stream,
                        (const bf16_t*)q, (bf16_t*)k_cache, (bf16_t*)v_cache, (bf16_t*)out, part_acc, part_ml,
                        rows, positions, seq_of_token, block_table, max_blocks, n_q, n_kv, page, scale_log2e, window,
@@ -439,7 +680,7 @@ int kipp_attention_decode(const void* q, const void* k_cache, const void* v_cach
     int rc = KIPP_LAUNCH_CHECK();
     if (rc != 0 || grid_splits == 1) return rc;
     hipLaunchKernelGGL(attention_decode_reduce_kernel, dim3(n_q, n_items), dim3(HEAD_DIM >= 64 ? 64 : HEAD_DIM), 0,
-                       stream, part_acc, part_ml, (bf16_t*)out, rows, positions, n_q, window, max_splits);
+                       stream, part_acc, part_ml, (bf16_t*)out, rows, positions, n_q, window, max_splits, SPLIT);
     return KIPP_LAUNCH_CHECK();
 }
 
@@ -473,7 +714,7 @@ int kipp_attention_decode_fused(const float* qkv, int parts, int n_tokens, const
     int rc = KIPP_LAUNCH_CHECK();
     if (rc != 0 || grid_splits == 1) return rc;
     hipLaunchKernelGGL(attention_decode_reduce_kernel, dim3(n_q, n_items), dim3(HEAD_DIM >= 64 ? 64 : HEAD_DIM), 0,
-                       stream, part_acc, part_ml, (bf16_t*)out, rows, positions, n_q, window, max_splits);
+                       stream, part_acc, part_ml, (bf16_t*)out, rows, positions, n_q, window, max_splits, SPLIT);
     return KIPP_LAUNCH_CHECK();
 #else
     return -5;

@@ -35,10 +35,17 @@ def model_variants(spec, dtype: str) -> List[Spec]:
 PREBUILT_ATTENTION = [(128, 4), (128, 8), (128, 16), (128, 1), (16, 2), (32, 4), (16, 3), (48, 3), (64, 1), (32, 16), (256, 4), (80, 3), (256, 2), (16, 1)]
 
 
+# builds of the decode attention in which the kernel for long contexts takes over at 1,024 keys
+# already, so that a kernel test can reach it with contexts it can check
+PREBUILT_EARLY_STREAM = [(128, 4), (48, 3), (16, 2)]
+
+
 def prebuilt() -> List[Spec]:
     out = list(GENERIC)
     for head_dim, group in PREBUILT_ATTENTION:
         for v in attention_variants(head_dim, group):
             if v not in out:
                 out.append(v)
+    for head_dim, group in PREBUILT_EARLY_STREAM:
+        out.append(("attention_decode", {"HEAD_DIM": head_dim, "GROUP": group, "STREAM_FROM": 1024}))
     return out

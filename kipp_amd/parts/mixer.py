@@ -19,7 +19,8 @@ from ..cache.needs import KVNeed
 from .base import ParamSpec, build_part, register
 
 
-FUSED_DECODE_ROWS = 16   # up to this many single tokens take the fused decode attention
+FUSED_DECODE_ROWS = 16      # up to this many single tokens take the fused decode attention ...
+FUSED_DECODE_KEYS = 8192    # ... while their contexts are shorter than this
 
 
 @register("mixer", "attention")
@@ -82,10 +83,11 @@ class Attention:
         table = batch.block_tables[cache.group]
         eps = s.qk_norm_eps if s.qk_norm_eps is not None else 0.0
         fast = rt.dtype == "bfloat16" and rt.ops.attention_fast_ok(s.num_heads, s.num_kv_heads, cache.page_size, table.shape[1])
-        # a few single tokens: norm, rotation, cache write and attention in one kernel.  (With many rows the
-        # attention is bound by reading the cache, and the fused kernel's lower occupancy costs more there
-        # than the rotary kernel it saves.)
+        # a few single tokens: norm, rotation, cache write and attention in one kernel.  (With many rows or
+        # long contexts the attention is bound by reading the cache, and the fused kernel's lower occupancy
+        # costs more there than the rotary kernel it saves.)
         fused = fast and not batch.n_prefill_items and batch.n_decode == n and n <= FUSED_DECODE_ROWS \
+            and batch.max_decode_ctx < FUSED_DECODE_KEYS \
             and rt.ops.attention_decode_fused_ok(s.head_dim, rotary_dim, inv_freq is not None)
         qkv = rt.linear(x, self.w_qkv, slabs=rt.ops.DECODE_FUSED_SLABS if fused else True)
         if fused:

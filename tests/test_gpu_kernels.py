@@ -325,6 +325,48 @@ def test_attention_decode(n_q, n_kv, d, page, window):
     assert not got[untouched].any()
 
 
+@pytest.mark.parametrize("n_q,n_kv,d,page,window", [(32, 8, 128, 16, 0), (32, 8, 128, 16, 1500), (6, 2, 48, 8, 0), (2, 1, 16, 16, 700)])
+def test_attention_decode_of_many_rows(n_q, n_kv, d, page, window):
+    """The kernel that walks long ranges of keys with a running maximum (built here so that it
+    takes over at 1,024 keys instead of 8,192): contexts on both sides of its range and block
+    edges (128, 129, 1024, 1025, 2049), the first token, rows that are not the first of the batch."""
+    ops = _ops()
+    inner = ops._fn
+
+    def early(lib, name, argtypes, defines=None):
+        return inner(lib, name, argtypes, dict(defines, STREAM_FROM=1024) if lib == "attention_decode" else defines)
+    ops._fn = early
+    try:
+        _many_rows(ops, n_q, n_kv, d, page, window)
+    finally:
+        ops._fn = inner
+
+
+def _many_rows(ops, n_q, n_kv, d, page, window):
+    rng = np.random.default_rng(n_q + d + window)
+    n_rows = 512 // n_kv + 8
+    edge = [1, 2, 127, 128, 129, 255, 256, 257, 1023, 1024, 1025, 2047, 2048, 2049, 2300]
+    seq_lens = (edge + [int(x) for x in rng.integers(1, 2300, size=n_rows)])[:n_rows]
+    table, k, v = _paged_setup(rng, seq_lens, n_kv, d, page, torch.bfloat16)
+    t = n_rows + 2
+    rows = list(range(2, t))
+    positions, seq_of = [0] * t, [0] * t
+    for r, (sq, n) in zip(rows, enumerate(seq_lens)):
+        positions[r], seq_of[r] = n - 1, sq
+    q = torch.tensor(rng.normal(size=(t, n_q * d)), dtype=torch.bfloat16)
+    out = torch.zeros(t, n_q * d, dtype=torch.bfloat16, device=DEV)
+    ws = ops.attention_decode_workspace(n_rows, n_q, d, max(seq_lens), DEV)
+    ops.attention_decode(q.to(DEV), k.to(DEV), v.to(DEV), out, _t(rows, torch.int32), _t(positions, torch.int32),
+                         _t(seq_of, torch.int32), _t(table, torch.int32), n_q, n_kv, d, 1 / math.sqrt(d), window,
+                         max(seq_lens), ws)
+    got = out.float().cpu().numpy().reshape(t, n_q, d)
+    check = list(range(len(edge))) + list(range(len(edge), n_rows, 7))        # the plain form is slow: the edges and a sample
+    ref = _attention_reference(q[[rows[i] for i in check]], k, v, table, [positions[rows[i]] for i in check],
+                               [seq_of[rows[i]] for i in check], n_q, n_kv, d, page, window)
+    assert _rel(got[[rows[i] for i in check]], ref) < 1e-5
+    assert not got[:2].any()
+
+
 @pytest.mark.parametrize("n_q,n_kv,d,page", [(32, 8, 128, 16), (8, 1, 128, 8), (16, 1, 128, 16), (3, 3, 128, 4), (8, 2, 256, 32), (4, 2, 256, 16)])
 @pytest.mark.parametrize("window,norm,slabs,write_kv", [(0, True, 1, True), (300, True, 3, True), (0, False, 2, True), (0, True, 1, False)])
 def test_attention_decode_from_the_projection(n_q, n_kv, d, page, window, norm, slabs, write_kv):
