@@ -39,6 +39,7 @@ class StepBatch:
     max_decode_ctx: int = 0
     max_q_len: int = 0
     max_ctx_len: int = 0
+    want_every_row: bool = False         # want_rows is 0, 1, ... n_tokens - 1
     host: dict = field(default_factory=dict)
     step_cache: dict = field(default_factory=dict)   # device values of this forward that parts share; emptied by every forward
 
@@ -109,4 +110,5 @@ def build_batch(entries: Sequence[StepEntry], requests: Sequence[object], n_grou
         decode_rows=t_dec, prefill_seq=t_pfs, prefill_tile=t_pft, n_decode=len(decode_rows),
         n_prefill_items=len(prefill_seq), max_decode_ctx=max(decode_ctx) if decode_ctx else 0,
         max_q_len=max(q_len) if q_len else 0, max_ctx_len=max(ctx_len) if ctx_len else 0,
+        want_every_row=want_rows == list(range(len(tokens))),
         host={"q_start": q_start, "q_len": q_len, "ctx_len": ctx_len})

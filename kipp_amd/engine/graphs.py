@@ -54,7 +54,7 @@ class DecodeGraph:
             n_tokens=n, n_seqs=n, n_want=n, tokens=d[0:n], positions=d[n:2 * n], seq_of_token=arange, q_start=arange,
             q_len=ones, ctx_len=d[2 * n:3 * n], slots=d[3 * n:4 * n], want_rows=arange, block_tables=tables,
             decode_rows=arange, prefill_seq=d[0:0], prefill_tile=d[0:0], n_decode=n, n_prefill_items=0,
-            max_decode_ctx=max_context, max_q_len=1, max_ctx_len=max_context,
+            max_decode_ctx=max_context, max_q_len=1, max_ctx_len=max_context, want_every_row=True,
             host={"q_start": list(range(n)), "q_len": [1] * n})
         self.graph: Optional[torch.cuda.CUDAGraph] = None
         self.logits: Optional[torch.Tensor] = None

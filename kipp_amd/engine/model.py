@@ -94,6 +94,11 @@ class Model:
         if batch.n_want == 0:
             return None
         ops = self.rt.ops
+        if batch.want_every_row:
+            # every row in order (a step of single tokens): no gather, and the last delta is added inside the norm
+            normed = (self.final_norm.forward(x, self.rt.act_dtype) if pending is None
+                      else self.final_norm.add_forward(x, pending, self.rt.act_dtype))
+            return self.head.forward(normed)
         if pending is not None:
             ops.residual_add(x, pending)
         rows = ops.gather_rows(x, batch.want_rows, self.rt.empty((batch.n_want, x.shape[1]), torch.float32))
