@@ -2,7 +2,7 @@
 of time (the sizes of the benchmark, of the tests and of the smoke run)."""
 from __future__ import annotations
 
-from typing import Iterable, List, Optional, Tuple
+from typing import List, Optional, Tuple
 
 Spec = Tuple[str, Optional[dict]]
 

@@ -13,7 +13,7 @@ from typing import List, Optional, Sequence
 
 import torch
 
-from ..cache import CacheManager, OutOfPages
+from ..cache import CacheManager
 from ..runtime import Runtime
 from .batch import StepEntry, build_batch
 from .graphs import DecodeGraphs

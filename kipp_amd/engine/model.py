@@ -3,7 +3,7 @@ and the forward pass over one flattened batch of tokens.
 """
 from __future__ import annotations
 
-from typing import Dict, List, Optional
+from typing import Dict, Optional
 
 import torch
 

@@ -9,7 +9,7 @@ in (0, 1], top_k 0 = off, min_p 0 = off, seed nonzero.
 """
 from __future__ import annotations
 
-from typing import List, Optional, Sequence
+from typing import Optional, Sequence
 
 from .engine import Engine
 from .engine.scheduler import Request, Scheduler

@@ -1,6 +1,5 @@
 """Each part of a layer alone, built from its spec with random weights, against
 the plain implementation; then prefix adoption and the step's error paths."""
-import math
 
 import numpy as np
 import pytest

@@ -5,7 +5,6 @@ wrong head mapping) fails it."""
 import math
 
 import numpy as np
-import pytest
 import torch
 
 from tests.plain import qwen3_plain as P
