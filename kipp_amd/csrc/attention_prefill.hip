@@ -25,6 +25,7 @@
 // Compile-time: HEAD_DIM (multiple of 16, <= 256).
 #include "common.h"
 #include <math.h>
+#include <type_traits>
 
 #ifndef HEAD_DIM
 #error "compile with -DHEAD_DIM=<head size>"
@@ -283,6 +284,240 @@ __global__ void __launch_bounds__(THREADS, 2) attention_prefill_kernel(
         }
 }
 
+// ---------------------------------------------------------------------------------------------
+// The same kernel for head size 128 with the tiles brought into LDS by the memory pipeline
+// itself (global_load_lds_dwordx4: 16 bytes a lane from global memory straight into LDS).
+// No register holds a tile on its way, nothing is packed or transposed by the lanes, and two
+// buffers take turns, so a tile costs one barrier: while tile i is worked on, tile i + 1 lands.
+//
+// Keys and values lie in LDS as in the cache, [key][d], 256 bytes a row.  Row r keeps its
+// 16-byte chunk c at slot c ^ (r % 16) (keys) or c ^ 4 (r % 4) (values): the rows that one
+// matrix-core operand reads at once then fall into different banks.  The lane that fills slot p
+// of row r simply asks for chunk p ^ ... of that row.  The value operand V^T comes out of LDS
+// transposed by ds_read_b64_tr_b16 (within 16 lanes, lane i receives element i % 4 of the
+// 8-byte pieces addressed by lanes i / 4, 4 + i / 4, 8 + i / 4, 12 + i / 4).
+#if HEAD_DIM == 128
+#ifndef PREFILL_DMA
+#define PREFILL_DMA 1                            // 0: head size 128 takes the kernel above as well
+#endif
+#define TILE_BYTES (BN * HEAD_DIM * 2)           // the keys (or the values) of one tile
+#define DMA_LDS_BYTES (2 * TILE_BYTES)           // dynamic LDS: the second tile buffer; the page table lies behind it
+
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+#define LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
+#define GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void*)(p))
+
+__global__ void __launch_bounds__(THREADS, 2) attention_prefill_dma_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
+    bf16_t* __restrict__ out, const int32_t* __restrict__ item_seq, const int32_t* __restrict__ item_tile,
+    const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len, const int32_t* __restrict__ positions,
+    const int32_t* __restrict__ block_table, int max_blocks, int n_q, int n_kv, int page, float scale_log2e,
+    int window) {
+    // the two tile buffers are two objects (one static, one dynamic): the compiler then sees that the loads
+    // into one never touch what is read from the other, and makes no read wait for them
+    __shared__ __attribute__((aligned(1024))) unsigned char tile_a[2 * TILE_BYTES];
+    extern __shared__ __attribute__((aligned(1024))) unsigned char tile_b[];
+    int* s_page = (int*)(tile_b + 2 * TILE_BYTES);
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31, hh = lane >> 5;
+    const int l16 = lane & 15, quarter = lane >> 4;
+    const int total = gridDim.x, half = (total + 1) / 2;
+    const int work = (int)blockIdx.x < half ? (int)blockIdx.x : total - 1 - ((int)blockIdx.x - half);
+    const int item = work / n_q, head = work % n_q;
+    const int kvh = head / (n_q / n_kv);
+    const int seq = item_seq[item];
+    const int tile_row0 = item_tile[item] * BM;
+    const int row0 = q_start[seq] + tile_row0;
+    const int rows_in_tile = min(BM, q_len[seq] - tile_row0);
+    const int pos0 = positions[row0];
+    const int last_pos = pos0 + rows_in_tile - 1;
+    const int32_t* table = block_table + (size_t)seq * max_blocks;
+
+    const int my_row = wave * 32 + l32;
+    const bool wave_active = wave * 32 < rows_in_tile;
+    const bool row_valid = my_row < rows_in_tile;
+    const int my_pos = pos0 + my_row;
+    const int my_lo = window > 0 ? max(0, my_pos - window + 1) : 0;
+
+    Frag qf[QSTEPS];
+#pragma unroll
+    for (int t = 0; t < QSTEPS; ++t) {
+        qf[t].u = (u32x4){0u, 0u, 0u, 0u};
+        if (row_valid) qf[t].u = *(const u32x4*)(q + ((size_t)(row0 + my_row) * n_q + head) * HEAD_DIM + 16 * t + 8 * hh);
+    }
+
+    f32x16 o[DTILES];
+#pragma unroll
+    for (int dt = 0; dt < DTILES; ++dt)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) o[dt][v] = 0.0f;
+    float m_run = -INFINITY, l_run = 0.0f;
+
+    const int tile_lo = (window > 0 ? max(0, pos0 - window + 1) : 0) / BN;
+    const int tile_hi = last_pos / BN;
+    const int page_shift = __builtin_ctz(page);
+    const int first_block = (tile_lo * BN) >> page_shift, last_block = last_pos >> page_shift;
+    for (int i = tid; i <= last_block - first_block; i += THREADS) s_page[i] = table[first_block + i];
+    __syncthreads();
+
+    // A wave brings 16 keys of a tile (and their values): instruction i the rows 4 i + quarter, a lane one
+    // 16-byte slot of a row.  Keys beyond the portion's last read its last row again (masked below).
+    auto issue = [&](int kt, unsigned char* tile) {
+        unsigned char* kdst = tile + wave * (16 * HEAD_DIM * 2);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int r = 16 * wave + 4 * i + quarter;                      // row of the tile
+            const int sc = min(kt * BN + r, last_pos);
+            const size_t at = (((size_t)s_page[(sc >> page_shift) - first_block] * n_kv + kvh) * page + (sc & (page - 1))) * HEAD_DIM;
+            __builtin_amdgcn_global_load_lds(GLOBAL_PTR(k_cache + at + ((l16 ^ (r & 15)) << 3)), LDS_PTR(kdst + 1024 * i), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds(GLOBAL_PTR(v_cache + at + ((l16 ^ (4 * (r & 3))) << 3)),
+                                             LDS_PTR(kdst + TILE_BYTES + 1024 * i), 16, 0, 0);
+        }
+    };
+
+    // a lane's places in the operands.  Keys: row 32 j + l32, chunk 2 t + hh.  Values, transposed read for the
+    // 32 columns of tile dt: this lane gives the address of row 4 hh + l16 / 4 (+ 32 j + 16 st, + 8 for the second
+    // half of the step), columns 32 dt + 16 (quarter % 2) + 4 (l16 % 4) .. + 3
+    const int v_row = 4 * hh + (l16 >> 2);
+    int v_at[DTILES], k_at[QSTEPS];
+#pragma unroll
+    for (int dt = 0; dt < DTILES; ++dt)
+        v_at[dt] = TILE_BYTES + v_row * 256 +
+                   ((((4 * dt + 2 * (quarter & 1) + ((l16 & 3) >> 1)) ^ (4 * (v_row & 3))) << 4) | ((l16 & 1) << 3));
+#pragma unroll
+    for (int t = 0; t < QSTEPS; ++t) k_at[t] = l32 * 256 + (((2 * t + hh) ^ (l32 & 15)) << 4);
+
+    // one tile: `Ks` holds it (keys, then values), the next one goes to `next`
+    auto work_tile = [&](int kt, const unsigned char* Ks, unsigned char* next) {
+        const int key0 = kt * BN;
+        __builtin_amdgcn_s_waitcnt(0x0F70);      // vmcnt(0): this wave's part of the tile is in LDS
+        __syncthreads();                         // every part is; and the other buffer has been read by every wave
+        if (kt < tile_hi) issue(kt + 1, next);
+        if (!wave_active) return;
+
+        // ---- S^T = K Q^T for the two 32-key halves of the tile
+        f32x16 s_acc[2];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) s_acc[j][v] = 0.0f;
+#pragma unroll
+            for (int t = 0; t < QSTEPS; ++t) {
+                Frag kf;
+                kf.u = *(const u32x4*)(Ks + k_at[t] + j * (32 * 256));
+                s_acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf.v, qf[t].v, s_acc[j], 0, 0, 0);
+            }
+        }
+        const bool masked = key0 + BN - 1 > pos0 + wave * 32 || window > 0;
+        if (masked) {
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int s = key0 + 32 * j + 8 * (v / 4) + 4 * hh + (v % 4);
+                    if (s > my_pos || s < my_lo) s_acc[j][v] = -INFINITY;
+                }
+        }
+        float m_tile = -INFINITY;
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) m_tile = fmaxf(m_tile, s_acc[j][v]);
+        m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, KIPP_WAVE));
+        // The exponents are taken against a reference maximum that follows the true one only when some
+        // query's maximum has moved by more than 8 (a weight is then at most 2^8, sums and products stay
+        // far inside float32): what has been gathered is rescaled on few tiles instead of on most.
+        const float m_new = fmaxf(m_run, m_tile);
+        if (__any((m_new - m_run) * scale_log2e > 8.0f)) {           // the first visible key: -inf to finite
+            // 0 at a query's first visible key, 1 where nothing moved or nothing is visible yet
+            const float alpha = m_new == -INFINITY ? 1.0f : __builtin_amdgcn_exp2f((m_run - m_new) * scale_log2e);
+            l_run *= alpha;
+#pragma unroll
+            for (int dt = 0; dt < DTILES; ++dt)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) o[dt][v] *= alpha;
+            m_run = m_new;
+        }
+        const float m_scaled = (m_run == -INFINITY ? 0.0f : m_run) * scale_log2e;   // nothing visible yet: every weight is 0
+        float l_tile = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const float p = __builtin_amdgcn_exp2f(fmaf(s_acc[j][v], scale_log2e, -m_scaled));
+                s_acc[j][v] = p;
+                l_tile += p;
+            }
+        l_tile += __shfl_xor(l_tile, 32, KIPP_WAVE);
+        l_run += l_tile;
+        // ---- O^T += V^T P^T in four steps of 16 keys; the second half of a step lies 8 rows (2,048 bytes)
+        //      further.  The transposed reads are written out: through the intrinsic the compiler makes each wait
+        //      for every load into LDS that is on its way, the next tile's included.  The reads of step s + 1 are
+        //      asked for before step s is multiplied.
+        static_assert(DTILES == 4, "the waits below count eight transposed reads a step");
+        uint32_t v_lds[DTILES];
+#pragma unroll
+        for (int dt = 0; dt < DTILES; ++dt) v_lds[dt] = (uint32_t)(uintptr_t)LDS_PTR(Ks + v_at[dt]);
+        u32x2 vt[2][2 * DTILES];
+#define KIPP_READ_STEP(S, STEP)                                                                                      \
+    _Pragma("unroll") for (int dt = 0; dt < DTILES; ++dt) {                                                          \
+        asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(vt[S][2 * dt]) : "v"(v_lds[dt]), "i"((STEP) * 4096)); \
+        asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2"                                                           \
+                     : "=v"(vt[S][2 * dt + 1])                                                                       \
+                     : "v"(v_lds[dt]), "i"((STEP) * 4096 + 2048));                                                   \
+    }
+#define KIPP_WAIT_STEP(S, N)                                                                                     \
+    asm volatile("s_waitcnt lgkmcnt(" #N ")"                                                                     \
+                 : "+v"(vt[S][0]), "+v"(vt[S][1]), "+v"(vt[S][2]), "+v"(vt[S][3]), "+v"(vt[S][4]), "+v"(vt[S][5]), \
+                   "+v"(vt[S][6]), "+v"(vt[S][7]))
+        auto multiply_step = [&](const u32x2* set, int step) {
+            const int j = step >> 1, st = step & 1;
+            Frag pf;
+            pf.u = (u32x4){pack_bf16(s_acc[j][8 * st + 0], s_acc[j][8 * st + 1]), pack_bf16(s_acc[j][8 * st + 2], s_acc[j][8 * st + 3]),
+                           pack_bf16(s_acc[j][8 * st + 4], s_acc[j][8 * st + 5]), pack_bf16(s_acc[j][8 * st + 6], s_acc[j][8 * st + 7])};
+#pragma unroll
+            for (int dt = 0; dt < DTILES; ++dt) {
+                Frag vf;
+                vf.u = (u32x4){set[2 * dt][0], set[2 * dt][1], set[2 * dt + 1][0], set[2 * dt + 1][1]};
+                o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf.v, pf.v, o[dt], 0, 0, 0);
+            }
+        };
+        KIPP_READ_STEP(0, 0)
+        KIPP_READ_STEP(1, 1)
+        KIPP_WAIT_STEP(0, 8);
+        multiply_step(vt[0], 0);
+        KIPP_READ_STEP(0, 2)
+        KIPP_WAIT_STEP(1, 8);
+        multiply_step(vt[1], 1);
+        KIPP_READ_STEP(1, 3)
+        KIPP_WAIT_STEP(0, 8);
+        multiply_step(vt[0], 2);
+        KIPP_WAIT_STEP(1, 0);
+        multiply_step(vt[1], 3);
+#undef KIPP_READ_STEP
+#undef KIPP_WAIT_STEP
+    };
+    issue(tile_lo, tile_a);
+    for (int kt = tile_lo; kt <= tile_hi; kt += 2) {
+        work_tile(kt, tile_a, tile_b);
+        if (kt + 1 <= tile_hi) work_tile(kt + 1, tile_b, tile_a);
+    }
+    if (!row_valid) return;
+    const float inv = 1.0f / l_run;
+    bf16_t* o_row = out + ((size_t)(row0 + my_row) * n_q + head) * HEAD_DIM;
+#pragma unroll
+    for (int dt = 0; dt < DTILES; ++dt)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const int dcol = 32 * dt + 8 * g + 4 * hh;
+            *(u32x2*)(o_row + dcol) = (u32x2){pack_bf16(o[dt][4 * g + 0] * inv, o[dt][4 * g + 1] * inv),
+                                              pack_bf16(o[dt][4 * g + 2] * inv, o[dt][4 * g + 3] * inv)};
+        }
+}
+#endif  // HEAD_DIM == 128
+
 extern "C" {
 
 int kipp_attention_prefill_rows() { return BM; }
@@ -299,6 +534,20 @@ int kipp_attention_prefill(const void* q, const void* k_cache, const void* v_cac
     if (page <= 0 || (page & (page - 1))) return -4;   // pages of a power of two only
     if (max_blocks > MAX_PAGES) return -5;             // the table row is staged in LDS
     const float scale_log2e = scale * 1.4426950408889634f;
+#if HEAD_DIM == 128 && PREFILL_DMA
+    {
+        static bool prepared = false;
+        if (!prepared) {
+            if (hipFuncSetAttribute((const void*)attention_prefill_dma_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    DMA_LDS_BYTES + MAX_PAGES * 4) != hipSuccess) return -6;
+            prepared = true;
+        }
+        hipLaunchKernelGGL(attention_prefill_dma_kernel, dim3(n_items * n_q), dim3(THREADS), DMA_LDS_BYTES + max_blocks * 4,
+                           stream, (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, item_seq,
+                           item_tile, q_start, q_len, positions, block_table, max_blocks, n_q, n_kv, page, scale_log2e, window);
+        return KIPP_LAUNCH_CHECK();
+    }
+#endif
     hipLaunchKernelGGL(attention_prefill_kernel, dim3(n_items * n_q), dim3(THREADS), 0, stream, (const bf16_t*)q,
                        (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, item_seq, item_tile, q_start, q_len,
                        positions, block_table, max_blocks, n_q, n_kv, page, scale_log2e, window);
