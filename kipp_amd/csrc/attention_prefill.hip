@@ -364,8 +364,31 @@ __global__ void __launch_bounds__(THREADS, 2) attention_prefill_dma_kernel(
 
     // A wave brings 16 keys of a tile (and their values): instruction i the rows 4 i + quarter, a lane one
     // 16-byte slot of a row.  Keys beyond the portion's last read its last row again (masked below).
+    // Where the 16 keys lie in one page and none is beyond the last (all tiles but a portion's last, pages
+    // of 16 keys and more), their rows are one run of memory: a base the whole wave shares plus a lane's own
+    // offset, which never changes.
+    uint32_t k_off[4], v_off[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int r = 4 * i + quarter;
+        k_off[i] = (uint32_t)(r * HEAD_DIM + ((l16 ^ r) << 3)) * 2;
+        v_off[i] = (uint32_t)(r * HEAD_DIM + ((l16 ^ (4 * (r & 3))) << 3)) * 2;
+    }
     auto issue = [&](int kt, unsigned char* tile) {
         unsigned char* kdst = tile + wave * (16 * HEAD_DIM * 2);
+        const int s0 = kt * BN + 16 * wave;                                 // the wave's first key
+        if (page >= 16 && s0 + 15 <= last_pos) {
+            const int pg = __builtin_amdgcn_readfirstlane(s_page[(s0 >> page_shift) - first_block]);
+            const size_t base = (((size_t)pg * n_kv + kvh) * page + (s0 & (page - 1))) * (HEAD_DIM * 2);
+            const unsigned char* kb = (const unsigned char*)k_cache + base;
+            const unsigned char* vb = (const unsigned char*)v_cache + base;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                __builtin_amdgcn_global_load_lds(GLOBAL_PTR(kb + k_off[i]), LDS_PTR(kdst + 1024 * i), 16, 0, 0);
+                __builtin_amdgcn_global_load_lds(GLOBAL_PTR(vb + v_off[i]), LDS_PTR(kdst + TILE_BYTES + 1024 * i), 16, 0, 0);
+            }
+            return;
+        }
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int r = 16 * wave + 4 * i + quarter;                      // row of the tile

@@ -414,7 +414,8 @@ def test_attention_decode_from_the_projection(n_q, n_kv, d, page, window, norm, 
     assert ops.attention_decode_fused_ok(128, 64, False)
 
 
-@pytest.mark.parametrize("n_q,n_kv,d,page", [(32, 8, 128, 16), (6, 2, 48, 8), (4, 4, 64, 4), (3, 1, 80, 16), (2, 1, 256, 32), (2, 2, 16, 8)])
+@pytest.mark.parametrize("n_q,n_kv,d,page", [(32, 8, 128, 16), (6, 2, 48, 8), (4, 4, 64, 4), (3, 1, 80, 16), (2, 1, 256, 32), (2, 2, 16, 8),
+                                             (4, 2, 128, 4), (5, 1, 128, 64)])
 @pytest.mark.parametrize("window", [0, 100])
 def test_attention_prefill(n_q, n_kv, d, page, window):
     ops = _ops()
@@ -438,6 +439,37 @@ def test_attention_prefill(n_q, n_kv, d, page, window):
     got = out.float().cpu().numpy().reshape(t, n_q, d)
     for i in range(t):
         assert _rel(got[i], ref[i]) < 2e-5, f"row {i}: position {positions[i]} of sequence {seq_of[i]}"
+
+
+@pytest.mark.parametrize("rise", [3.0, 40.0, 400.0, -40.0])
+def test_attention_prefill_with_a_moving_maximum(rise):
+    """The head-size-128 kernel takes its exponents against a maximum that follows the true one
+    only after it has moved by 2^8: here every query's scores rise (or fall) along the keys by
+    `rise` in all, in small steps, so the reference is stale on most tiles and renewed on some."""
+    ops = _ops()
+    n_q, n_kv, d, page = 4, 2, 128, 16
+    rng = np.random.default_rng(int(abs(rise)))
+    n, ql = 900, 200
+    table, k, v = _paged_setup(rng, [n], n_kv, d, page, torch.bfloat16)
+    positions = list(range(n - ql, n))
+    q = torch.tensor(rng.normal(size=(ql, n_q * d)), dtype=torch.bfloat16)
+    # a direction every query has the component 1 along: key s gets `rise * s / n * sqrt(d)` of it on top of noise
+    kk = 0.05 * k.clone().float()
+    qq = q.float().reshape(ql, n_q, d).clone()
+    qq[:, :, 0] = 1.0
+    for s_ in range(n):
+        kk[table[0, s_ // page], :, s_ % page, 0] = rise * s_ / n * math.sqrt(d)
+    q, kk = qq.reshape(ql, n_q * d).to(torch.bfloat16), kk.to(torch.bfloat16)
+    items = list(range(-(-ql // ops.PREFILL_ROWS)))
+    out = ops.attention_prefill(q.to(DEV), kk.to(DEV), v.to(DEV), torch.zeros(ql, n_q * d, dtype=torch.bfloat16, device=DEV),
+                                _t([0] * len(items), torch.int32), _t(items, torch.int32), _t([0], torch.int32),
+                                _t([ql], torch.int32), _t(positions, torch.int32), _t(table, torch.int32), n_q, n_kv, d,
+                                1 / math.sqrt(d), 0)
+    ref = _attention_reference(q, kk, v, table, positions, [0] * ql, n_q, n_kv, d, page, 0)
+    got = out.float().cpu().numpy().reshape(ql, n_q, d)
+    assert np.isfinite(got).all()
+    for i in range(ql):
+        assert _rel(got[i], ref[i]) < 2e-5, f"row {i}"
 
 
 @pytest.mark.parametrize("kernel", ["decode", "prefill"])
