@@ -6,7 +6,7 @@ bfloat16 weights on one MI355X.
 One JSON line: `value` is decoded tokens a second at batch 8 (a step is one
 decode step of the whole batch, tokens chosen greedily on the device and fed
 back), with the prefill of one 2,048-token prompt, the decode step's HBM
-roofline and the batch-1 / batch-64 points beside it.  Peaks are MI355X's
+roofline and the batch-1 / batch-64 / batch-128 points beside it.  Peaks are MI355X's
 published ones: HBM 8 TB/s, dense bf16 MFMA 2.5 PFLOP/s.
 """
 import argparse
@@ -103,7 +103,7 @@ def main():
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--prompt", type=int, default=2048)
     ap.add_argument("--context", type=int, default=None, help="context length (default: the shape's)")
-    ap.add_argument("--points", default="1,64", help="further decode batch sizes")
+    ap.add_argument("--points", default="1,64,128", help="further decode batch sizes")
     ap.add_argument("--no-prefill", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:

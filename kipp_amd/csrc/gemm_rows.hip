@@ -1,11 +1,12 @@
 // Matrix product for a few dozen rows (decode at larger batches):
 // Y[M, N] = X[M, K] . W[N, K]^T, bfloat16 operands, float32 accumulation,
-// M <= 64.  Like the few-rows kernel it is bound by reading W once, but here
+// M <= 128.  Like the few-rows kernel it is bound by reading W once, but here
 // the rows of X are too many to fetch per wave: every wave would read as much
 // of X from L2 as of W from HBM.  So the TW waves of a workgroup share one
-// range of K and stage X through LDS in chunks of 256 columns (double
-// buffered, one barrier a chunk), while each wave streams its own 16 rows of W
-// through a ring of 8 steps in registers.
+// range of K and stage X through LDS in chunks of 256 columns (128 from 65
+// rows on, so that two workgroups still fit a compute unit; double buffered,
+// one barrier a chunk), while each wave streams its own 16 rows of W through a
+// ring of one chunk's steps in registers.
 //
 // K is split over `parts` workgroups (grid.y): part p writes slab p of
 // Y[parts, M, N]; the consumer adds the slabs in order.
@@ -15,9 +16,7 @@
 // 4 (l / 16) + v of token l % 16.
 #include "common.h"
 
-#define DEPTH 8                       // steps of 32 columns in one chunk
-#define CHUNK (32 * DEPTH)            // columns of X staged at a time
-#define X_PITCH (CHUNK + 8)           // bf16 elements per staged row (the pad spreads the banks)
+#define MAX_ROWS 128
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
@@ -31,9 +30,12 @@ union Frag {
 // TILED: W in the streaming layout [tile of 16 rows][step of 32 columns][lane][8 values]
 // (rows padded to whole tiles with zeros, K a multiple of 32), in which a wave's load is
 // one contiguous KB.
-template <int MT, int TW, bool TILED>
+// DEPTH: steps of 32 columns in one chunk.
+template <int MT, int TW, bool TILED, int DEPTH>
 __global__ void __launch_bounds__(TW * KIPP_WAVE) gemm_rows_kernel(
     const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, float* __restrict__ Y, int M, int N, int K) {
+    constexpr int CHUNK = 32 * DEPTH;                          // columns of X staged at a time
+    constexpr int X_PITCH = CHUNK + 8;                         // bf16 elements per staged row (the pad spreads the banks)
     constexpr int THREADS = TW * KIPP_WAVE;
     constexpr int UNITS = MT * 16 * (CHUNK / 8);              // 16-byte units of one staged chunk
     constexpr int XR = UNITS / THREADS;                        // units a thread moves
@@ -112,7 +114,7 @@ __global__ void __launch_bounds__(TW * KIPP_WAVE) gemm_rows_kernel(
 #pragma unroll
         for (int u = 0; u < DEPTH; ++u) multiply(u, buf);
     }
-    // the rest of K (fewer than 256 columns), by the last part, straight from global memory
+    // the rest of K (less than a chunk), by the last part, straight from global memory
     if (part == parts - 1) {
         for (int k = groups * CHUNK; k < K; k += 32) {
             const bool ok = k + 8 * h < K;
@@ -149,9 +151,11 @@ __global__ void __launch_bounds__(TW * KIPP_WAVE) gemm_rows_kernel(
 // run in rounds of 256 and a round costs what one workgroup reads plus a fixed start;
 // the plan takes the cheapest rounds, with a small charge for every slab the consumer
 // has to add and every part at least one whole chunk.
-static void plan(int N, int K, int max_parts, int* tw, int* parts) {
+static int chunk_of(int M) { return M > 64 ? 128 : 256; }
+
+static void plan(int M, int N, int K, int max_parts, int* tw, int* parts) {
     const int tiles = (N + 15) / 16;
-    const int groups = K / CHUNK > 0 ? K / CHUNK : 1;
+    const int groups = K / chunk_of(M) > 0 ? K / chunk_of(M) : 1;
     double best = 1e300;
     *tw = 4;
     *parts = 1;
@@ -171,49 +175,52 @@ static void plan(int N, int K, int max_parts, int* tw, int* parts) {
 
 extern "C" {
 
-int kipp_gemm_rows_parts(int N, int K, int max_parts) {
+int kipp_gemm_rows_max_rows() { return MAX_ROWS; }
+
+int kipp_gemm_rows_parts(int M, int N, int K, int max_parts) {
     int tw, parts;
-    plan(N, K, max_parts, &tw, &parts);
+    plan(M, N, K, max_parts, &tw, &parts);
     return parts;
 }
 
-// Y: float32 [parts, M, N] with parts = kipp_gemm_rows_parts(N, K, max_parts).
-// M <= 64, K a multiple of 8; `tiled`: W in the streaming layout (K a multiple of 32).
+// Y: float32 [parts, M, N] with parts = kipp_gemm_rows_parts(M, N, K, max_parts).
+// M <= 128, K a multiple of 8; `tiled`: W in the streaming layout (K a multiple of 32).
 int kipp_gemm_rows(const void* X, const void* W, float* Y, int M, int N, int K, int max_parts, int tiled,
                    hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
-    if (M > 64 || K <= 0 || (K & 7) || max_parts <= 0 || (tiled && (K & 31))) return -1;
+    if (M > MAX_ROWS || K <= 0 || (K & 7) || max_parts <= 0 || (tiled && (K & 31))) return -1;
     int tw, parts;
-    plan(N, K, max_parts, &tw, &parts);
+    plan(M, N, K, max_parts, &tw, &parts);
     const int tiles = (N + 15) / 16;
     dim3 grid((tiles + tw - 1) / tw, parts), block(tw * KIPP_WAVE);
-    const int mt = (M + 15) / 16;
-#define KIPP_GR(MT, TW)                                                                                             \
+    const int mt = (M + 15) / 16;       // from 65 rows on an even number of 16-row tiles is staged (every thread moves whole units)
+#define KIPP_GR(MT, TW, DEPTH)                                                                                      \
     do {                                                                                                            \
         if (tiled)                                                                                                  \
-            hipLaunchKernelGGL((gemm_rows_kernel<MT, TW, true>), grid, block, 0, stream, (const bf16_t*)X,          \
+            hipLaunchKernelGGL((gemm_rows_kernel<MT, TW, true, DEPTH>), grid, block, 0, stream, (const bf16_t*)X,   \
                                (const bf16_t*)W, Y, M, N, K);                                                       \
         else                                                                                                        \
-            hipLaunchKernelGGL((gemm_rows_kernel<MT, TW, false>), grid, block, 0, stream, (const bf16_t*)X,         \
+            hipLaunchKernelGGL((gemm_rows_kernel<MT, TW, false, DEPTH>), grid, block, 0, stream, (const bf16_t*)X,  \
                                (const bf16_t*)W, Y, M, N, K);                                                       \
     } while (0)
-    if (tw == 8) {
-        switch (mt) {
-            case 1: KIPP_GR(1, 8); break;
-            case 2: KIPP_GR(2, 8); break;
-            case 3: KIPP_GR(3, 8); break;
-            case 4: KIPP_GR(4, 8); break;
-            default: return -1;
-        }
-    } else {
-        switch (mt) {
-            case 1: KIPP_GR(1, 4); break;
-            case 2: KIPP_GR(2, 4); break;
-            case 3: KIPP_GR(3, 4); break;
-            case 4: KIPP_GR(4, 4); break;
-            default: return -1;
-        }
+#define KIPP_GR_TW(TW)                    \
+    switch (mt) {                         \
+        case 1: KIPP_GR(1, TW, 8); break; \
+        case 2: KIPP_GR(2, TW, 8); break; \
+        case 3: KIPP_GR(3, TW, 8); break; \
+        case 4: KIPP_GR(4, TW, 8); break; \
+        case 5:                           \
+        case 6: KIPP_GR(6, TW, 4); break; \
+        case 7:                           \
+        case 8: KIPP_GR(8, TW, 4); break; \
+        default: return -1;               \
     }
+    if (tw == 8) {
+        KIPP_GR_TW(8)
+    } else {
+        KIPP_GR_TW(4)
+    }
+#undef KIPP_GR_TW
 #undef KIPP_GR
     return KIPP_LAUNCH_CHECK();
 }

@@ -385,7 +385,13 @@ def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
 
 # --------------------------------------------------------------------------- matrix products
 
-SKINNY_MAX_ROWS = 64
+SKINNY_MAX_ROWS = 64     # rows of the few-rows kernel
+ROWS_MAX_ROWS = 128      # rows of the kernel that stages x through LDS
+
+
+def gemm_rows_ok(m: int, k: int) -> bool:
+    """Shapes our own streaming products take: at most 128 rows, K a multiple of 8 and at least 32."""
+    return 0 < m <= ROWS_MAX_ROWS and k % 8 == 0 and k >= 32
 
 
 def gemm_skinny_ok(m: int, k: int) -> bool:
@@ -443,17 +449,17 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, max_parts: int = 1, tiles: tor
 
 
 def gemm_rows(x: torch.Tensor, w: torch.Tensor, max_parts: int = 1, tiles: torch.Tensor = None) -> torch.Tensor:
-    """float32 [parts, M, N] whose sum over parts is x . w^T, for 16 < M <= 64 rows
-    (any M <= 64 is taken): the rows of x are staged through LDS and shared by
+    """float32 [parts, M, N] whose sum over parts is x . w^T, for 16 < M <= 128 rows
+    (any M <= 128 is taken): the rows of x are staged through LDS and shared by
     the waves of a workgroup."""
     _dev(x, w)
     m, k = x.shape
     n = w.shape[0]
     _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm_rows: bfloat16 operands")
     _need(w.shape == (n, k), "gemm_rows: shapes do not match")
-    _need(0 < m <= SKINNY_MAX_ROWS and k % 8 == 0, "gemm_rows: at most 64 rows and K a multiple of 8")
+    _need(0 < m <= ROWS_MAX_ROWS and k % 8 == 0, "gemm_rows: at most 128 rows and K a multiple of 8")
     lib = build.library("gemm_rows")
-    parts = lib.kipp_gemm_rows_parts(n, k, int(max_parts))
+    parts = lib.kipp_gemm_rows_parts(m, n, k, int(max_parts))
     out = torch.empty((parts, m, n), dtype=torch.float32, device=x.device)
     tiled = _tiles_ok(tiles, n, k, 1, "gemm_rows")
     fn = _fn("gemm_rows", "kipp_gemm_rows", [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr])

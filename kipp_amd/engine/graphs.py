@@ -23,6 +23,7 @@ import torch
 from .batch import StepBatch
 
 CONTEXT_BUCKET = 1024
+MAX_GRAPH_ENTRIES = 128     # rows up to which every product of a step is one of our own kernels (none goes to a library)
 
 
 class DecodeGraph:
@@ -129,7 +130,7 @@ class DecodeGraphs:
         self.replays = 0
 
     def applies(self, entries: Sequence) -> bool:
-        return (self.possible and 0 < len(entries) <= 64
+        return (self.possible and 0 < len(entries) <= MAX_GRAPH_ENTRIES
                 and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries))
 
     def run(self, entries, requests, device_tokens=None) -> torch.Tensor:

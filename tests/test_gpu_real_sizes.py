@@ -91,3 +91,29 @@ def test_decoding_across_a_graph_bucket_and_many_splits(long_folder, dtype):
     for rid in seqs:
         first = {"long": 1000, "mid": 240, "short": 10}[rid]
         H.assert_close(np.stack(got[rid]), refs[rid][first:fed[rid]], tol, f"long context/{dtype}/{rid}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_hundred_requests_decode_together(long_folder, dtype):
+    """More rows than one 64-row product takes: 100 prompts of 3 to 40 tokens enter in one step, then all
+    decode together for 6 steps (the products stage their rows in chunks of 128 columns, the steps are
+    recorded graphs); every tenth request against the plain implementation."""
+    from kipp_amd.engine import Engine, StepEntry
+    cfg, weights = plain.load_folder(long_folder)
+    rng = np.random.default_rng(7)
+    seqs = {f"r{i}": H.random_tokens(100 + i, int(rng.integers(3, 41)) + 6, 311) for i in range(100)}
+    engine = Engine.from_folder(long_folder, dtype=dtype, page_size=16, max_tokens=100 * 64, max_requests=100,
+                                share_prefixes=False)
+    fed = {rid: len(toks) - 6 for rid, toks in seqs.items()}
+    engine.step([StepEntry(rid, seqs[rid][:fed[rid]], []) for rid in seqs])
+    got = {rid: [] for rid in seqs}
+    for _ in range(6):
+        logits = engine.step([StepEntry(rid, [seqs[rid][fed[rid]]], [0]) for rid in seqs]).cpu().numpy()
+        for row, rid in zip(logits, seqs):
+            got[rid].append(row)
+            fed[rid] += 1
+    assert engine.graphs.replays >= 4
+    tol = H.NMSE_F32 if dtype == "float32" else H.NMSE_BF16
+    for rid in list(seqs)[::10]:
+        ref = plain.forward_whole(cfg, weights, seqs[rid])
+        H.assert_close(np.stack(got[rid]), ref[len(seqs[rid]) - 6:], tol, f"hundred together/{dtype}/{rid}")
