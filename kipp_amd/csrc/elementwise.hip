@@ -130,32 +130,38 @@ __global__ void residual_add_kernel(float* __restrict__ x, const TD* __restrict_
 }
 
 // out[t, i] = silu(gu[t, i]) * gu[t, inner + i], silu(z) = z / (1 + exp(-z))
-// (/root/reference/src/kipp.c:2402, 2644-2648).
+// (/root/reference/src/kipp.c:2402, 2644-2648).  `pairs`: the columns of gu come in tiles of 16,
+// 8 gates over the 8 matching ups (the product of a weight in the paired streaming layout):
+// gate i at 16 (i / 8) + i % 8, its up 8 further, rows of 16 ceil(inner / 8) columns.
 template <typename TI, typename TO>
-__global__ void swiglu_kernel(const TI* __restrict__ gu, TO* __restrict__ out, int inner, size_t total, int parts) {
+__global__ void swiglu_kernel(const TI* __restrict__ gu, TO* __restrict__ out, int inner, size_t total, int parts, int pairs) {
     size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= total) return;
     size_t t = idx / inner;
     int i = (int)(idx - t * inner);
+    const size_t width = pairs ? 16 * (size_t)((inner + 7) / 8) : 2 * (size_t)inner;
+    const size_t slab = (total / inner) * width;
+    const size_t at_g = t * width + (pairs ? 16 * (i >> 3) + (i & 7) : i), at_u = at_g + (pairs ? 8 : inner);
     float g = 0.0f, u = 0.0f;
     for (int p = 0; p < parts; ++p) {   // slabs of a split product, in order
-        g += load_f(gu, (p * total + t * (size_t)inner) * 2 + i);
-        u += load_f(gu, (p * total + t * (size_t)inner) * 2 + inner + i);
+        g += load_f(gu, p * slab + at_g);
+        u += load_f(gu, p * slab + at_u);
     }
     store_f(out, idx, g / (1.0f + expf(-g)) * u);
 }
 
 // The same, eight columns a thread with 16-byte accesses (inner a multiple of 8, one slab).
 template <typename TI, typename TO>
-__global__ void swiglu_vec_kernel(const TI* __restrict__ gu, TO* __restrict__ out, int inner, size_t total8) {
+__global__ void swiglu_vec_kernel(const TI* __restrict__ gu, TO* __restrict__ out, int inner, size_t total8, int pairs) {
     const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= total8) return;
     const int per_row = inner / 8;
     const size_t t = idx / per_row;
     const int i4 = (int)(idx - t * per_row) * 2;              // in units of 4 columns
     const size_t row4 = t * 2 * (size_t)inner / 4;
-    const float4 g0 = load4(gu, row4 + i4), g1 = load4(gu, row4 + i4 + 1);
-    const float4 u0 = load4(gu, row4 + inner / 4 + i4), u1 = load4(gu, row4 + inner / 4 + i4 + 1);
+    const size_t g4 = row4 + (pairs ? 2 * i4 : i4), u4 = g4 + (pairs ? 2 : inner / 4);
+    const float4 g0 = load4(gu, g4), g1 = load4(gu, g4 + 1);
+    const float4 u0 = load4(gu, u4), u1 = load4(gu, u4 + 1);
     const size_t o4 = t * (size_t)inner / 4 + i4;
     store4(out, o4, make_float4(g0.x / (1.0f + expf(-g0.x)) * u0.x, g0.y / (1.0f + expf(-g0.y)) * u0.y,
                                 g0.z / (1.0f + expf(-g0.z)) * u0.z, g0.w / (1.0f + expf(-g0.w)) * u0.w));
@@ -232,13 +238,14 @@ int kipp_residual_add(float* x, const void* delta, int delta_dtype, int parts, s
     return KIPP_LAUNCH_CHECK();
 }
 
-int kipp_swiglu(const void* gu, int in_dtype, int parts, void* out, int out_dtype, int rows, int inner, hipStream_t stream) {
+int kipp_swiglu(const void* gu, int in_dtype, int parts, void* out, int out_dtype, int rows, int inner, int pairs,
+                hipStream_t stream) {
     size_t total = (size_t)rows * inner;
     if (total == 0) return 0;
     if (parts == 1 && (inner & 7) == 0) {
         const size_t total8 = total / 8;
         dim3 grid8((unsigned)((total8 + 255) / 256)), block8(256);
-#define KIPP_SV(TI, TO) hipLaunchKernelGGL((swiglu_vec_kernel<TI, TO>), grid8, block8, 0, stream, (const TI*)gu, (TO*)out, inner, total8)
+#define KIPP_SV(TI, TO) hipLaunchKernelGGL((swiglu_vec_kernel<TI, TO>), grid8, block8, 0, stream, (const TI*)gu, (TO*)out, inner, total8, pairs)
         if (in_dtype == KIPP_BF16) {
             if (out_dtype == KIPP_BF16) KIPP_SV(bf16_t, bf16_t); else KIPP_SV(bf16_t, float);
         } else {
@@ -248,7 +255,7 @@ int kipp_swiglu(const void* gu, int in_dtype, int parts, void* out, int out_dtyp
         return KIPP_LAUNCH_CHECK();
     }
     dim3 grid((unsigned)((total + 255) / 256)), block(256);
-#define KIPP_SW(TI, TO) hipLaunchKernelGGL((swiglu_kernel<TI, TO>), grid, block, 0, stream, (const TI*)gu, (TO*)out, inner, total, parts)
+#define KIPP_SW(TI, TO) hipLaunchKernelGGL((swiglu_kernel<TI, TO>), grid, block, 0, stream, (const TI*)gu, (TO*)out, inner, total, parts, pairs)
     if (in_dtype == KIPP_BF16) {
         if (out_dtype == KIPP_BF16) KIPP_SW(bf16_t, bf16_t); else KIPP_SW(bf16_t, float);
     } else {

@@ -125,15 +125,18 @@ def residual_add(x: torch.Tensor, delta: torch.Tensor) -> torch.Tensor:
     return x
 
 
-def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+def swiglu(gate_up: torch.Tensor, out: torch.Tensor, pairs: bool = False) -> torch.Tensor:
     """out[t, i] = silu(gate_up[t, i]) * gate_up[t, inner + i]; `gate_up` is
-    [rows, 2 inner] or slabs [parts, rows, 2 inner] that are added in order."""
+    [rows, 2 inner] or slabs [parts, rows, 2 inner] that are added in order.
+    `pairs`: the columns come in tiles of 16, 8 gates over the 8 matching ups
+    (a product from `tile_weight_pairs`), 16 ceil(inner / 8) of them a row."""
     _dev(gate_up, out)
     rows, inner = out.shape
-    _need(tuple(gate_up.shape[-2:]) == (rows, 2 * inner) and gate_up.dim() in (2, 3), "swiglu: input must be [rows, 2 * inner]")
+    width = 16 * ((inner + 7) // 8) if pairs else 2 * inner
+    _need(tuple(gate_up.shape[-2:]) == (rows, width) and gate_up.dim() in (2, 3), "swiglu: input must be [rows, 2 * inner]")
     parts = gate_up.shape[0] if gate_up.dim() == 3 else 1
-    fn = _fn("elementwise", "kipp_swiglu", [_c_ptr, _c_int, _c_int, _c_ptr, _c_int, _c_int, _c_int, _c_ptr])
-    _check(fn(_ptr(gate_up), _code(gate_up), parts, _ptr(out), _code(out), rows, inner, _stream()), "swiglu")
+    fn = _fn("elementwise", "kipp_swiglu", [_c_ptr, _c_int, _c_int, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr])
+    _check(fn(_ptr(gate_up), _code(gate_up), parts, _ptr(out), _code(out), rows, inner, int(pairs), _stream()), "swiglu")
     return out
 
 
@@ -399,32 +402,51 @@ def gemm_skinny_ok(m: int, k: int) -> bool:
     return 0 < m <= SKINNY_MAX_ROWS and k % 8 == 0 and k >= 32
 
 
-def tile_weight(w: torch.Tensor, split: int = 1) -> torch.Tensor:
+def _tile(block: torch.Tensor) -> torch.Tensor:
+    """[16 t, K] rows -> [tile][step of 32 columns][lane][8 values], lane l = row l % 16, columns 8 (l / 16) .. + 7."""
+    rows, k = block.shape
+    return block.view(rows // 16, 16, k // 32, 4, 8).permute(0, 2, 3, 1, 4).contiguous().view(-1)
+
+
+def _pad_rows(block: torch.Tensor, multiple: int) -> torch.Tensor:
+    rest = -block.shape[0] % multiple
+    return block if not rest else torch.cat([block, torch.zeros((rest, block.shape[1]), dtype=block.dtype, device=block.device)])
+
+
+def tile_weight(w: torch.Tensor) -> torch.Tensor:
     """The streaming layout of a bfloat16 matrix [N, K], K a multiple of 32: the
     1 KB a wave reads in one step (16 rows x 32 columns) is contiguous,
     [tile of 16 rows][step of 32 columns][lane][8 values] with lane l holding row
-    l % 16 and columns 8 (l / 16) .. + 7 of the step.  `split` stacked matrices of
-    N / split rows are each padded to whole tiles with zero rows."""
+    l % 16 and columns 8 (l / 16) .. + 7 of the step.  The rows are padded to
+    whole tiles with zeros."""
     _need(w.dim() == 2 and w.dtype == torch.bfloat16, "tile_weight: a bfloat16 matrix")
-    n, k = w.shape
-    _need(k % 32 == 0 and split >= 1 and n % split == 0, "tile_weight: K a multiple of 32, N a multiple of split")
-    inner = n // split
-    tiles = (inner + 15) // 16
-    blocks = []
-    for i in range(split):
-        block = w[i * inner:(i + 1) * inner]
-        if inner % 16:
-            block = torch.cat([block, torch.zeros((tiles * 16 - inner, k), dtype=w.dtype, device=w.device)])
-        blocks.append(block.view(tiles, 16, k // 32, 4, 8).permute(0, 2, 3, 1, 4))
-    return torch.cat(blocks).contiguous().view(-1)
+    _need(w.shape[1] % 32 == 0, "tile_weight: K a multiple of 32")
+    return _tile(_pad_rows(w, 16))
 
 
-def _tiles_ok(tiles, n: int, k: int, split: int, what: str) -> int:
+def tile_weight_pairs(w_gate_up: torch.Tensor) -> torch.Tensor:
+    """The streaming layout of [gate; up] ([2 I, K]) for the product that ends in
+    SwiGLU: tile t holds gate rows 8 t .. 8 t + 7 over up rows 8 t .. 8 t + 7, so
+    that one tile gives 8 finished outputs (I padded to a multiple of 8 with zeros).
+    As a plain tiled matrix it is the weight with its rows in that order."""
+    _need(w_gate_up.dim() == 2 and w_gate_up.dtype == torch.bfloat16, "tile_weight_pairs: a bfloat16 matrix")
+    two_inner, k = w_gate_up.shape
+    _need(k % 32 == 0 and two_inner % 2 == 0, "tile_weight_pairs: K a multiple of 32, gate and up of equal height")
+    inner = two_inner // 2
+    gate, up = _pad_rows(w_gate_up[:inner], 8), _pad_rows(w_gate_up[inner:], 8)
+    return _tile(torch.cat([gate.view(-1, 8, k), up.view(-1, 8, k)], dim=1).view(-1, k))
+
+
+def pairs_width(inner: int) -> int:
+    """Columns of a product from paired tiles: 16 for every 8 outputs."""
+    return 16 * ((inner + 7) // 8)
+
+
+def _tiles_ok(tiles, n: int, k: int, what: str) -> int:
     if tiles is None:
         return 0
-    inner_tiles = (n // split + 15) // 16
     _need(tiles.dtype == torch.bfloat16 and tiles.is_contiguous() and k % 32 == 0
-          and tiles.numel() == split * inner_tiles * 16 * k, f"{what}: the tiled weight does not match [N, K]")
+          and tiles.numel() == ((n + 15) // 16) * 16 * k, f"{what}: the tiled weight does not match [N, K]")
     return 1
 
 
@@ -442,26 +464,32 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, max_parts: int = 1, tiles: tor
     lib = build.library("gemm_skinny")
     parts = lib.kipp_gemm_skinny_parts(n, k, int(max_parts))
     out = torch.empty((parts, m, n), dtype=torch.float32, device=x.device)
-    tiled = _tiles_ok(tiles, n, k, 1, "gemm_skinny")
+    tiled = _tiles_ok(tiles, n, k, "gemm_skinny")
     fn = _fn("gemm_skinny", "kipp_gemm_skinny", [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr])
     _check(fn(_ptr(x), _ptr(tiles if tiled else w), _ptr(out), m, n, k, int(max_parts), tiled, _stream()), "gemm_skinny")
     return out
 
 
-def gemm_rows(x: torch.Tensor, w: torch.Tensor, max_parts: int = 1, tiles: torch.Tensor = None) -> torch.Tensor:
+def gemm_rows(x: torch.Tensor, w: torch.Tensor, max_parts: int = 1, tiles: torch.Tensor = None,
+              pairs: bool = False) -> torch.Tensor:
     """float32 [parts, M, N] whose sum over parts is x . w^T, for 16 < M <= 128 rows
     (any M <= 128 is taken): the rows of x are staged through LDS and shared by
-    the waves of a workgroup."""
+    the waves of a workgroup.  `pairs`: `tiles` is tile_weight_pairs(w), w = [gate; up];
+    the product then has `pairs_width(inner)` columns in the order of those tiles
+    (what `swiglu(..., pairs=True)` takes)."""
     _dev(x, w)
     m, k = x.shape
     n = w.shape[0]
     _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm_rows: bfloat16 operands")
     _need(w.shape == (n, k), "gemm_rows: shapes do not match")
     _need(0 < m <= ROWS_MAX_ROWS and k % 8 == 0, "gemm_rows: at most 128 rows and K a multiple of 8")
+    if pairs:
+        _need(tiles is not None and n % 2 == 0, "gemm_rows: pairs need the paired tiles of [gate; up]")
+        n = pairs_width(n // 2)
     lib = build.library("gemm_rows")
     parts = lib.kipp_gemm_rows_parts(m, n, k, int(max_parts))
     out = torch.empty((parts, m, n), dtype=torch.float32, device=x.device)
-    tiled = _tiles_ok(tiles, n, k, 1, "gemm_rows")
+    tiled = _tiles_ok(tiles, n, k, "gemm_rows")
     fn = _fn("gemm_rows", "kipp_gemm_rows", [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr])
     _check(fn(_ptr(x), _ptr(tiles if tiled else w), _ptr(out), m, n, k, int(max_parts), tiled, _stream()), "gemm_rows")
     return out
@@ -469,7 +497,7 @@ def gemm_rows(x: torch.Tensor, w: torch.Tensor, max_parts: int = 1, tiles: torch
 
 def gemm_skinny_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor, tiles: torch.Tensor = None) -> torch.Tensor:
     """out[M, I] (bfloat16) = silu(x . w_gate^T) * (x . w_up^T), w_gate_up = [gate; up] of [2 I, K];
-    `tiles` = tile_weight(w_gate_up, split=2)."""
+    `tiles` = tile_weight_pairs(w_gate_up).  The same bits from both layouts."""
     _dev(x, w_gate_up, out)
     m, k = x.shape
     two_inner = w_gate_up.shape[0]
@@ -478,7 +506,7 @@ def gemm_skinny_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tens
     _need(w_gate_up.shape == (two_inner, k) and two_inner % 2 == 0 and out.shape == (m, two_inner // 2),
           "gemm_skinny_swiglu: shapes do not match")
     _need(gemm_skinny_ok(m, k), "gemm_skinny_swiglu: at most 64 rows, K a multiple of 8 and at least 32")
-    tiled = _tiles_ok(tiles, two_inner, k, 2, "gemm_skinny_swiglu")
+    tiled = _tiles_ok(tiles, pairs_width(two_inner // 2), k, "gemm_skinny_swiglu")
     fn = _fn("gemm_skinny", "kipp_gemm_skinny_swiglu", [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr])
     _check(fn(_ptr(x), _ptr(tiles if tiled else w_gate_up), _ptr(out), m, two_inner, k, tiled, _stream()), "gemm_skinny_swiglu")
     return out

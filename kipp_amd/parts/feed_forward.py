@@ -35,16 +35,21 @@ class GatedMLP:
         g, u = tensors["gate_proj.weight"], tensors["up_proj.weight"]
         if g.dtype != u.dtype:
             g, u = g.float(), u.float()
-        self.w_gate_up = self.rt.weight(torch.cat([g, u], dim=0).contiguous(), split=2)
+        self.w_gate_up = self.rt.weight(torch.cat([g, u], dim=0).contiguous(), gate_up=True)
         self.w_down = self.rt.weight(tensors["down_proj.weight"])
 
     def forward(self, x, batch=None):
         rt = self.rt
         rows, inner = x.shape[0], self.spec.intermediate_size
         act = rt.empty((rows, inner), rt.act_dtype)
-        if self.w_gate_up.dtype == x.dtype == torch.bfloat16 and rows <= 16 and rt.ops.gemm_skinny_ok(rows, x.shape[1]):
+        w = self.w_gate_up
+        ours = w.dtype == x.dtype == torch.bfloat16 and rt.ops.gemm_rows_ok(rows, x.shape[1])
+        if ours and rows <= 16:
             # both products and the activation in one kernel
-            rt.ops.gemm_skinny_swiglu(x, self.w_gate_up.rows, act, tiles=self.w_gate_up.tiles)
+            rt.ops.gemm_skinny_swiglu(x, w.rows, act, tiles=w.tiles)
+        elif ours and w.pairs:
+            # streamed from the paired tiles: the columns come out gate tile by gate tile
+            rt.ops.swiglu(rt.ops.gemm_rows(x, w.rows, max_parts=12, tiles=w.tiles, pairs=True), act, pairs=True)
         else:
-            rt.ops.swiglu(rt.linear(x, self.w_gate_up, slabs=True, low_precision_out=True), act)
+            rt.ops.swiglu(rt.linear(x, w, slabs=True, low_precision_out=True), act)
         return rt.linear(act, self.w_down, slabs=True)

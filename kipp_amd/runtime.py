@@ -34,11 +34,12 @@ class Weight:
     """A matrix [N, K] as the products want it: `rows` as stored, for the library
     product and the 32-bit kernels, and `tiles`, the same values in the layout
     that the few-rows kernels stream fastest (None where that layout does not
-    apply).  `split` stacked matrices share the tensor."""
-    __slots__ = ("rows", "tiles", "split")
+    apply).  `pairs`: the matrix is [gate; up] and its tiles hold 8 gate rows over
+    the 8 matching up rows each (for the product that ends in SwiGLU)."""
+    __slots__ = ("rows", "tiles", "pairs")
 
-    def __init__(self, rows: torch.Tensor, tiles: torch.Tensor | None = None, split: int = 1):
-        self.rows, self.tiles, self.split = rows, tiles, split
+    def __init__(self, rows: torch.Tensor, tiles: torch.Tensor | None = None, pairs: bool = False):
+        self.rows, self.tiles, self.pairs = rows, tiles, pairs
 
     @property
     def shape(self):
@@ -76,17 +77,17 @@ class Runtime:
     def empty(self, shape, dtype) -> torch.Tensor:
         return torch.empty(shape, dtype=dtype, device=self.device)
 
-    def weight(self, w: torch.Tensor, split: int = 1) -> Weight:
+    def weight(self, w: torch.Tensor, gate_up: bool = False) -> Weight:
         """A matrix on the device, made ready for `linear`.  A bfloat16 matrix whose
         K is a multiple of 32 gets a copy in the streaming layout: decode reads every
         weight once a step and is bound by that read, which is a fifth faster from
         that layout; many-row products go to the library, which needs the rows.
-        The price is the matrix held twice."""
+        The price is the matrix held twice.  `gate_up`: w is [gate; up] and feeds
+        SwiGLU; its tiles pair gate rows with their up rows."""
         tiles = None
-        if self.stream_layout and w.dtype == torch.bfloat16 and w.dim() == 2 and w.shape[1] % 32 == 0 \
-                and w.shape[0] % split == 0:
-            tiles = self.ops.tile_weight(w, split)
-        return Weight(w, tiles, split)
+        if self.stream_layout and w.dtype == torch.bfloat16 and w.dim() == 2 and w.shape[1] % 32 == 0:
+            tiles = self.ops.tile_weight_pairs(w) if gate_up else self.ops.tile_weight(w)
+        return Weight(w, tiles, gate_up and tiles is not None)
 
     # -- matrix product ------------------------------------------------------
     def linear(self, x: torch.Tensor, w, slabs: bool = False, low_precision_out: bool = False) -> torch.Tensor:
@@ -99,9 +100,8 @@ class Runtime:
         bfloat16 anyway and is bound by reading it)."""
         tiles = None
         if isinstance(w, Weight):
-            # stacked matrices that fill whole tiles lie in the layout of one matrix
-            whole = w.split == 1 or (w.rows.shape[0] // w.split) % 16 == 0
-            w, tiles = w.rows, (w.tiles if whole else None)
+            # paired tiles give the columns in another order: only the feed-forward asks for that
+            w, tiles = w.rows, (None if w.pairs else w.tiles)
         m = x.shape[0]
         n = w.shape[0]
         if w.dtype == torch.float32:

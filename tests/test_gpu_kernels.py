@@ -535,8 +535,12 @@ def test_tile_weight_layout():
         row, col = 16 * tile + lane % 16, 32 * step + 8 * (lane // 16)
         want = w[row, col:col + 8] if row < 20 else torch.zeros(8, dtype=torch.bfloat16)
         assert torch.equal(t[tile, step, lane], want)
-    two = ops.tile_weight(w.to(DEV), split=2).cpu().view(2, 2, 64, 8)                    # 10 + 10 rows, each padded to a tile
-    assert torch.equal(two[1, 1, 16 + 9], w[10 + 9, 32 + 8:32 + 16]) and not two[1, 0, 10].any()
+    # [gate; up] of 10 + 10 rows in pairs: tile 0 = gate rows 0..7 over up rows 0..7, tile 1 = gate 8, 9 (then zeros) over up 8, 9
+    two = ops.tile_weight_pairs(w.to(DEV)).cpu().view(2, 2, 64, 8)
+    assert torch.equal(two[0, 1, 16 + 3], w[3, 32 + 8:32 + 16]) and torch.equal(two[0, 0, 32 + 8 + 5], w[10 + 5, 16:24])
+    assert torch.equal(two[1, 1, 1], w[9, 32:40]) and torch.equal(two[1, 0, 48 + 9], w[10 + 9, 24:32])
+    assert not two[1, 0, 2].any() and not two[1, 1, 8 + 2].any()
+    assert ops.pairs_width(10) == 32 and ops.pairs_width(9728) == 2 * 9728
     with pytest.raises(ops.KernelError):
         ops.tile_weight(torch.zeros(16, 40, dtype=torch.bfloat16, device=DEV))
     with pytest.raises(ops.KernelError):
@@ -615,8 +619,32 @@ def test_gemm_skinny_swiglu(m, inner, k):
     if k % 32 == 0:
         wd = w.to(DEV)
         tiled = ops.gemm_skinny_swiglu(x.to(DEV), wd, torch.empty(m, inner, dtype=torch.bfloat16, device=DEV),
-                                       tiles=ops.tile_weight(wd, split=2))
+                                       tiles=ops.tile_weight_pairs(wd))
         assert torch.equal(tiled, out)
+
+
+@pytest.mark.parametrize("m,inner,k,max_parts", [(17, 16, 32, 1), (40, 77, 96, 4), (64, 9728, 2560, 12), (100, 200, 256, 2), (128, 1001, 512, 3)])
+def test_gate_up_product_from_paired_tiles(m, inner, k, max_parts):
+    """Many rows: the product streamed from the paired tiles has its columns tile by tile (8 gates, 8 ups);
+    the activation kernel reads them so, one slab or several."""
+    ops = _ops()
+    rng = np.random.default_rng(m + inner)
+    x = torch.tensor(rng.normal(size=(m, k)), dtype=torch.bfloat16)
+    w = torch.tensor(rng.normal(size=(2 * inner, k)) / math.sqrt(k), dtype=torch.bfloat16)
+    wd = w.to(DEV)
+    y = ops.gemm_rows(x.to(DEV), wd, max_parts, tiles=ops.tile_weight_pairs(wd), pairs=True)
+    assert y.shape[1:] == (m, ops.pairs_width(inner)) and 1 <= y.shape[0] <= max_parts
+    got = ops.swiglu(y, torch.empty(m, inner, dtype=torch.bfloat16, device=DEV), pairs=True)
+    gu = x.double().numpy() @ w.double().numpy().T
+    ref = plain.silu(gu[:, :inner]) * gu[:, inner:]
+    assert _rel(got.float().cpu().numpy(), ref) < 1e-5
+    # the same columns as the plain product, only in another order
+    plain_y = ops.gemm_rows(x.to(DEV), wd, max_parts).sum(dim=0).cpu()
+    # column c of the paired product: tile c // 16, gate (c % 16 < 8) or up of feature 8 (c // 16) + c % 8
+    cols = [(c, 8 * (c // 16) + c % 8, c % 16 >= 8) for c in range(ops.pairs_width(inner))]
+    keep = [c for c, f, _ in cols if f < inner]
+    order = {c: (inner + f if is_up else f) for c, f, is_up in cols}
+    assert _rel(y.sum(dim=0).cpu().numpy()[:, keep], plain_y.numpy()[:, [order[c] for c in keep]]) < 1e-10
 
 
 def test_rmsnorm_adds_slabs_in_order():
