@@ -524,6 +524,23 @@ def gemm_f32(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tenso
     return out
 
 
+# --------------------------------------------------------------------------- probe
+
+def stream_read(buffer: torch.Tensor, workgroups: int, depth: int = 8) -> int:
+    """Reads `buffer` once with `workgroups` x 4 waves, `depth` 16-byte loads a lane in
+    flight; returns the bytes read (what the grid covers in whole rings)."""
+    _dev(buffer)
+    _need(buffer.is_contiguous() and depth in (4, 8, 16), "stream_read: a contiguous buffer, depth 4, 8 or 16")
+    lib = build.library("probe")
+    fn = lib.kipp_probe_stream_read
+    fn.restype = ctypes.c_longlong
+    fn.argtypes = [_c_ptr, ctypes.c_longlong, _c_int, _c_int, _c_ptr, _c_ptr]
+    sink = torch.zeros(1, dtype=torch.int32, device=buffer.device)
+    got = fn(_ptr(buffer), buffer.numel() * buffer.element_size(), int(workgroups), int(depth), _ptr(sink), _stream())
+    _need(got > 0, "stream_read: buffer too small for this grid")
+    return int(got)
+
+
 # --------------------------------------------------------------------------- sampling
 
 def argmax(logits: torch.Tensor, out: torch.Tensor) -> torch.Tensor:

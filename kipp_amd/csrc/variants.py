@@ -48,4 +48,5 @@ def prebuilt() -> List[Spec]:
                 out.append(v)
     for head_dim, group in PREBUILT_EARLY_STREAM:
         out.append(("attention_decode", {"HEAD_DIM": head_dim, "GROUP": group, "STREAM_FROM": 1024}))
+    out.append(("probe", None))       # the read-bandwidth yardstick of `python -m kipp_amd.workloads hbm`
     return out

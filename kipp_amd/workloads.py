@@ -4,9 +4,12 @@ portions, and requests that share a long beginning (paged prefix reuse).
 
     python -m kipp_amd.workloads continuous    [--shape qwen3-8b]  [--requests 32] ...
     python -m kipp_amd.workloads shared-prefix [--shape qwen3-32b] [--requests 8]  ...
+    python -m kipp_amd.workloads hbm           [--gib 4]
 
 One JSON line: generated tokens a second over the whole run, prompt tokens a
-second, time to the first token, and what the cache reused.
+second, time to the first token, and what the cache reused.  `hbm` is no
+workload but the yardstick for the decode kernels: how fast a kernel that only
+reads gets a large buffer out of memory (best of several grids and ring depths).
 """
 from __future__ import annotations
 
@@ -78,7 +81,45 @@ def serve(engine, prompts, new_tokens: int, chunk: int, max_step_tokens: int):
     return sched, seconds, first
 
 
+def hbm_read(gib: float) -> dict:
+    """Read bandwidth of a buffer far larger than every cache, one pass a launch, over
+    grids of 1 to 8 workgroups a compute unit and rings of 4 to 16 loads a lane."""
+    import torch
+    from .csrc import ops
+    buf = torch.empty(int(gib * 2**30) // 4, dtype=torch.int32, device="cuda:0")
+    buf.fill_(7)
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    best, table = None, []
+    for per_cu in (1, 2, 4, 8):
+        for depth in (4, 8, 16):
+            start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            fastest = 0.0
+            for _ in range(4):
+                start.record()
+                got = ops.stream_read(buf, cus * per_cu, depth)
+                end.record()
+                torch.cuda.synchronize()
+                fastest = max(fastest, got / (start.elapsed_time(end) * 1e-3) / 1e9)
+            table.append({"workgroups_per_cu": per_cu, "depth": depth, "GB_s": round(fastest, 1)})
+            log(f"{per_cu} workgroups a compute unit, {depth} loads a lane in flight: {fastest:7.1f} GB/s")
+            if best is None or fastest > best["GB_s"]:
+                best = table[-1]
+    return {"workload": "hbm read", "GiB": gib, "compute_units": cus, "best": best, "all": table}
+
+
 def main(argv=None) -> int:
+    if argv is None:
+        argv = sys.argv[1:]
+    if argv and argv[0] == "hbm":
+        ap = argparse.ArgumentParser(prog="python -m kipp_amd.workloads hbm")
+        ap.add_argument("--gib", type=float, default=4.0, help="size of the buffer that is read")
+        args = ap.parse_args(argv[1:])
+        import torch
+        if not torch.cuda.is_available():
+            print("workload: no GPU", file=sys.stderr)
+            return 1
+        print(json.dumps(hbm_read(args.gib)), flush=True)
+        return 0
     ap = argparse.ArgumentParser(prog="python -m kipp_amd.workloads", description=__doc__,
                                  formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("workload", choices=["continuous", "shared-prefix"])

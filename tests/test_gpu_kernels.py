@@ -595,6 +595,19 @@ def test_consumers_add_slabs_in_order():
     assert torch.equal(a, b)
 
 
+def test_stream_read_probe_covers_the_buffer():
+    """The bandwidth yardstick reads whole rings only and says how many bytes that was."""
+    ops = _ops()
+    buf = torch.zeros(3 * 2**20 + 5, dtype=torch.int32, device=DEV)
+    for groups, depth in ((8, 4), (32, 8), (5, 16)):
+        got = ops.stream_read(buf, groups, depth)
+        ring = groups * 4 * depth * 1024
+        assert got % ring == 0 and buf.numel() * 4 - ring < got <= buf.numel() * 4
+    with pytest.raises(ops.KernelError):
+        ops.stream_read(torch.zeros(1024, dtype=torch.int32, device=DEV), 64, 8)    # less than two rings a wave
+    torch.cuda.synchronize()
+
+
 def test_gemm_skinny_refuses_what_it_cannot_do():
     ops = _ops()
     x = torch.zeros(2, 8, dtype=torch.bfloat16, device=DEV)
