@@ -131,7 +131,10 @@ def main():
     t0 = time.perf_counter()
     rt = Runtime("bfloat16")
     model = random_model(config, seed=0, runtime=rt)
-    tokens_per_request = args.prompt + args.warmup + args.steps + 8
+    # the first requests take part in every batch size: room for all those steps
+    decoded = sum((args.steps if b == args.batch else max(8, args.steps // 2)) +
+                  (args.warmup if b == args.batch else max(2, args.warmup // 2)) + 1 for b in batches)
+    tokens_per_request = args.prompt + decoded + 8
     engine = Engine(model, page_size=page, num_pages=max_batch * (-(-tokens_per_request // page)) + 4,
                     max_requests=max_batch, share_prefixes=False)
     torch.cuda.synchronize()

@@ -12,6 +12,7 @@ stays in the index until it is taken for new content
 """
 from __future__ import annotations
 
+import math
 from collections import OrderedDict
 from dataclasses import dataclass
 from typing import Dict, List, Optional, Sequence, Tuple
@@ -41,6 +42,19 @@ class PoolStats:
     evicted_pages_total: int
 
 
+def scattered_order(n: int) -> List[int]:
+    """0 .. n-1 in an order in which neighbours lie far apart (steps of about 0.618 n, coprime
+    to n).  A fresh pool hands its pages out in this order: sequences that arrive together and
+    have the same length would otherwise lie at equal distances in memory, a power of two for
+    prompts of 2,048 tokens, and kernels that walk all of them in step would find every sequence's
+    current page in the same memory channel (measured: decode attention of 128 such sequences a
+    fifth slower)."""
+    step = max(1, int(n * 0.6180339887))
+    while math.gcd(step, n) != 1:
+        step += 1
+    return [(i * step) % n for i in range(n)]
+
+
 class PagePool:
     def __init__(self, num_pages: int, page_size: int):
         if num_pages <= 0 or page_size <= 0:
@@ -48,7 +62,7 @@ class PagePool:
         self.num_pages = num_pages
         self.page_size = page_size
         self.ref = [0] * num_pages
-        self.free: "OrderedDict[int, None]" = OrderedDict((i, None) for i in range(num_pages))
+        self.free: "OrderedDict[int, None]" = OrderedDict((i, None) for i in scattered_order(num_pages))
         self.content: List[Optional[Tuple[int, Tuple[int, ...]]]] = [None] * num_pages  # (hash, tokens) if indexed
         self.index: Dict[int, List[int]] = {}
         self.reused_total = 0

@@ -217,17 +217,17 @@ __global__ void __launch_bounds__(THREADS) attention_decode_kernel(
                 if ((j < GROUP ? pj.q_norm_w : pj.k_norm_w) != nullptr) {
                     float ss = 0.0f;
 #pragma unroll
-                    for (int c = 0; c < NC; ++c) ss += raw[jj][c] * raw[jj][c];
+                    for (int c = 0; c < NC; ++c) ss = square_add(ss, raw[jj][c]);
                     ss = wave_sum(ss);
-                    const float r = 1.0f / sqrtf(ss / (float)HEAD_DIM + pj.eps);
+                    const float r = head_norm_scale(ss, (float)HEAD_DIM, pj.eps);
 #pragma unroll
                     for (int c = 0; c < NC; ++c) raw[jj][c] *= r * (j < GROUP ? norm_q[c] : norm_k[c]);
                 }
 #pragma unroll
                 for (int c = 0; c < NC / 2; ++c) {
                     const float a = raw[jj][c], b = raw[jj][c + NC / 2];
-                    raw[jj][c] = a * cs[c] - b * sn[c];
-                    raw[jj][c + NC / 2] = b * cs[c] + a * sn[c];
+                    raw[jj][c] = rotate_lo(a, b, cs[c], sn[c]);
+                    raw[jj][c + NC / 2] = rotate_hi(a, b, cs[c], sn[c]);
                 }
             }
             bf16_t* dst = nullptr;
@@ -604,6 +604,324 @@ __global__ void __launch_bounds__(THREADS) attention_decode_stream_kernel(
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// The same attention with keys and values streamed through LDS by the memory pipeline itself
+// (global_load_lds_dwordx4: 16 bytes a lane straight into LDS, no register in between), for
+// head size 128 and pages that are multiples of 16 keys.
+//
+// Every wave is a stream of its own: it takes every fourth block of 16 keys of the workgroup's
+// range, keeps a ring of RING_STAGES blocks (keys and values, 8 KB a block) in its own part of
+// LDS and, while it works on one block, the next is on its way; no barrier until the waves merge
+// at the end.  The loads therefore never stop while a wave has keys left, where the kernels above
+// load everything, then compute everything (and all workgroups of a launch do so in step).
+//
+//   scores   S^T[key][head] = K . Q^T, v_mfma_f32_16x16x32_bf16, A = the block's keys from LDS;
+//   softmax  online, per wave: a lane holds 4 keys of one head, the lanes of the other key
+//            quarters are two exchanges away; running maximum and sum per head in registers;
+//   values   O^T[d][head] += V^T . P^T, v_mfma_f32_16x16x16_bf16: P^T is the score registers as
+//            they are (rounded to bfloat16), V^T comes out of LDS transposed by
+//            ds_read_b64_tr_b16 (values lie in LDS as in the cache, [key][d]).
+//
+// The launcher takes this kernel from 128 (sequence, key/value head) pairs on (measured: from there it is
+// at least as fast as splitting the keys, merge kernel included, with pages scattered over the pool):
+// a workgroup then walks a sequence's whole context (up to RING_RANGE keys), the partial results
+// and the merge kernel fall away, and in the FUSED form every query is normed and rotated once (by
+// the one workgroup of its key/value head) while the first blocks are on their way; that workgroup
+// also writes the token's key and value into the cache and puts them into the block it has in LDS.
+//
+// LDS layout of a block: key row r at 256 r, its 16-byte chunk c at slot c ^ r (keys) or
+// c ^ 2 (r % 8) (values): the 16 rows a matrix-core operand reads at once then fall into
+// different banks.  The lane that brings slot p of row r simply asks for chunk p ^ r of that row.
+#define RING_OK (HEAD_DIM == 128)
+#define RING_STAGES 2
+#define RING_HALF (16 * HEAD_DIM * 2)                          // bytes of a block's keys (or values)
+#define RING_BYTES (WAVES * RING_STAGES * 2 * RING_HALF)
+#define RING_RANGE (KIPP_WAVE * WAVES * 16)                    // keys of a workgroup at most: a wave holds its blocks' pages one a lane
+#ifndef RING_FROM_PAIRS
+#define RING_FROM_PAIRS 128                                    // sequences x key/value heads from which this kernel is taken
+#endif
+
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+
+#if RING_OK
+__device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
+    union {
+        bf16x2 v;
+        uint32_t u;
+    } r;
+    r.v = __builtin_convertvector((f32x2){a, b}, bf16x2);
+    return r.u;
+}
+
+#define LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
+#define GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void*)(p))
+
+template <bool FUSED>
+__global__ void __launch_bounds__(THREADS, 2) attention_decode_ring_kernel(
+    const bf16_t* __restrict__ q, bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache,
+    bf16_t* __restrict__ out, float* __restrict__ part_acc, float* __restrict__ part_ml,
+    const int32_t* __restrict__ rows, const int32_t* __restrict__ positions, const int32_t* __restrict__ seq_of_token,
+    const int32_t* __restrict__ block_table, int max_blocks, int n_q, int n_kv, int page, float scale_log2e,
+    int window, int max_splits, int range, Projected pj) {
+    extern __shared__ __attribute__((aligned(1024))) unsigned char ring[];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l16 = lane & 15, h = lane >> 4;
+    const int kvh = blockIdx.y;
+    const int row = rows[blockIdx.z];
+    const int pos = positions[row];
+    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+    const int first_split = lo / range, last_split = pos / range;
+    const int split = first_split + blockIdx.x;
+    if (split > last_split) return;
+    const int n_splits = last_split - first_split + 1;
+    const int base = split * range;
+    const int32_t* table = block_table + (size_t)seq_of_token[row] * max_blocks;
+    const int page_shift = __builtin_ctz(page);
+
+    // blocks of 16 keys (absolute index) that hold a visible key of this range; the wave's are every fourth
+    const int kb_lo = max(lo, base) >> 4, kb_hi = min(pos, base + range - 1) >> 4;
+    const int kb_first = kb_lo + wave;
+    const int n_mine = kb_first <= kb_hi ? (kb_hi - kb_first) / WAVES + 1 : 0;
+    // the page of the wave's j-th block in lane j (a block lies within one page)
+    int my_pages = 0;
+    if (lane < n_mine) my_pages = table[((kb_first + WAVES * lane) << 4) >> page_shift];
+
+    unsigned char* my_ring = ring + wave * (RING_STAGES * 2 * RING_HALF);
+    auto issue = [&](int j, int stage) {
+        const int kb = kb_first + WAVES * j;
+        const int pg = __builtin_amdgcn_readlane(my_pages, j);
+        const size_t off = (((size_t)pg * n_kv + kvh) * page + ((kb << 4) & (page - 1))) * HEAD_DIM;
+        const int last = pos - (kb << 4);            // keys beyond the query's own read its row again (masked below)
+        unsigned char* dst = my_ring + stage * (2 * RING_HALF);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int r = 4 * i + h;
+            const bf16_t* src = k_cache + off + (size_t)min(r, last) * HEAD_DIM + ((l16 ^ r) << 3);
+            __builtin_amdgcn_global_load_lds(GLOBAL_PTR(src), LDS_PTR(dst + 1024 * i), 16, 0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int r = 4 * i + h;
+            const bf16_t* src = v_cache + off + (size_t)min(r, last) * HEAD_DIM + ((l16 ^ (2 * (r & 7))) << 3);
+            __builtin_amdgcn_global_load_lds(GLOBAL_PTR(src), LDS_PTR(dst + RING_HALF + 1024 * i), 16, 0, 0);
+        }
+    };
+    if (n_mine > 0) issue(0, 0);
+    if (n_mine > 1) issue(1, 1);
+
+    // ---- the GROUP queries as B operand: lane (slot l16, quarter h) holds q[slot][32 t + 8 h .. + 7]
+    Frag qf[KSTEPS];
+    bf16_t (*s_new)[HEAD_DIM] = (bf16_t(*)[HEAD_DIM])(ring + RING_BYTES);   // FUSED: the GROUP queries, the new key, the new value
+    const bool owner = FUSED && pj.write_kv && split == last_split;        // this workgroup holds the token's own position
+    if (FUSED) {
+        // norm (/root/reference/src/kipp.c:2480-2500) and rotation (kipp.c:2368-2382) of the heads this wave
+        // prepares, in the arithmetic of the rotary kernel: a wave a head, element i and its rotation
+        // partner i + d/2 in one lane; the slabs of the projection are added in order
+        const size_t width = (size_t)(n_q + 2 * n_kv) * HEAD_DIM;
+        int last_slab = pj.parts - 1;
+        asm volatile("" : "+s"(last_slab));          // opaque: every slab load below is issued, none waits for a branch
+        float cs[NC / 2], sn[NC / 2];
+#pragma unroll
+        for (int c = 0; c < NC / 2; ++c) {
+            cs[c] = 1.0f;
+            sn[c] = 0.0f;
+            if (pj.angles != nullptr) {
+                cs[c] = pj.angles[(size_t)row * HEAD_DIM + lane + c * KIPP_WAVE];
+                sn[c] = pj.angles[(size_t)row * HEAD_DIM + HEAD_DIM / 2 + lane + c * KIPP_WAVE];
+            } else if (pj.inv_freq != nullptr) {
+                const float angle = (float)pos * pj.inv_freq[lane + c * KIPP_WAVE];
+                cs[c] = cosf(angle);
+                sn[c] = sinf(angle);
+            }
+        }
+#pragma unroll
+        for (int jj = 0; jj < JOBS; ++jj) {
+            const int j = wave + jj * WAVES;
+            if (!(j < GROUP || (owner && j < GROUP + 2))) continue;
+            const int slot = j < GROUP ? kvh * GROUP + j : (j == GROUP ? n_q + kvh : n_q + n_kv + kvh);
+            const float* src = pj.qkv + (size_t)row * width + (size_t)slot * HEAD_DIM + lane;
+            float slab[NC][MAX_SLABS], raw[NC];
+#pragma unroll
+            for (int c = 0; c < NC; ++c)
+#pragma unroll
+                for (int p = 0; p < MAX_SLABS; ++p)
+                    slab[c][p] = src[(size_t)min(p, last_slab) * pj.part_stride + c * KIPP_WAVE];
+#pragma unroll
+            for (int c = 0; c < NC; ++c) {
+                raw[c] = slab[c][0];
+#pragma unroll
+                for (int p = 1; p < MAX_SLABS; ++p) raw[c] += (p <= last_slab ? 1.0f : 0.0f) * slab[c][p];
+            }
+            if (j <= GROUP) {
+                const float* norm_w = j < GROUP ? pj.q_norm_w : pj.k_norm_w;
+                if (norm_w != nullptr) {
+                    float ss = 0.0f;
+#pragma unroll
+                    for (int c = 0; c < NC; ++c) ss = square_add(ss, raw[c]);
+                    ss = wave_sum(ss);
+                    const float r = head_norm_scale(ss, (float)HEAD_DIM, pj.eps);
+#pragma unroll
+                    for (int c = 0; c < NC; ++c) raw[c] *= r * norm_w[lane + c * KIPP_WAVE];
+                }
+#pragma unroll
+                for (int c = 0; c < NC / 2; ++c) {
+                    const float a = raw[c], b = raw[c + NC / 2];
+                    raw[c] = rotate_lo(a, b, cs[c], sn[c]);
+                    raw[c + NC / 2] = rotate_hi(a, b, cs[c], sn[c]);
+                }
+            }
+            bf16_t* dst = nullptr;
+            if (j >= GROUP)
+                dst = (j == GROUP ? k_cache : v_cache) +
+                      (((size_t)table[pos >> page_shift] * n_kv + kvh) * page + (pos & (page - 1))) * HEAD_DIM;
+#pragma unroll
+            for (int c = 0; c < NC; ++c) {
+                const bf16_t bits = f32_to_bf16(raw[c]);
+                s_new[j][lane + c * KIPP_WAVE] = bits;
+                if (dst != nullptr) dst[lane + c * KIPP_WAVE] = bits;
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int t = 0; t < KSTEPS; ++t) qf[t].u = *(const u32x4*)(&s_new[min(l16, GROUP - 1)][32 * t + 8 * h]);
+    } else {
+#pragma unroll
+        for (int t = 0; t < KSTEPS; ++t)
+            qf[t].u = *(const u32x4*)(q + ((size_t)row * n_q + (size_t)kvh * GROUP + min(l16, GROUP - 1)) * HEAD_DIM + 32 * t + 8 * h);
+    }
+#pragma unroll
+    for (int t = 0; t < KSTEPS; ++t)
+        if (l16 >= GROUP) qf[t].u = (u32x4){0u, 0u, 0u, 0u};
+
+    f32x4 o[HEAD_DIM / 16];
+#pragma unroll
+    for (int b = 0; b < HEAD_DIM / 16; ++b) o[b] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
+    float m_run = -INFINITY, l_run = 0.0f;
+    // a lane's place in the operands: key row l16 of the keys; for the transposed read of the values, the
+    // 8 bytes at row 4 h + l16 / 4, columns 4 (l16 % 4) .. + 3 of a 16-column block
+    const int v_row = 4 * h + (l16 >> 2);
+    uint32_t v_addr[HEAD_DIM / 16];                  // LDS addresses of those 8 bytes in stage 0, one per block of columns
+#pragma unroll
+    for (int b = 0; b < HEAD_DIM / 16; ++b)
+        v_addr[b] = (uint32_t)(uintptr_t)LDS_PTR(my_ring + RING_HALF) + v_row * 256 + 8 * (l16 & 3) + 32 * (b ^ (v_row & 7));
+
+    for (int j = 0; j < n_mine; ++j) {
+        const int stage = j & 1;
+        // the block's 8 loads have landed when at most the next block's 8 are still out
+        if (j + 1 < n_mine) __builtin_amdgcn_s_waitcnt(0x0F78);      // vmcnt(8)
+        else __builtin_amdgcn_s_waitcnt(0x0F70);                     // vmcnt(0)
+        unsigned char* kbuf = my_ring + stage * (2 * RING_HALF);
+        const int kb = kb_first + WAVES * j;
+        if (owner && kb == (pos >> 4)) {
+            // the token's own key and value (the cache row may or may not have them yet): from s_new into the block
+            const int r = pos & 15;
+            if (lane < 16) {
+                *(u32x4*)(kbuf + r * 256 + ((lane ^ r) << 4)) = *(const u32x4*)(&s_new[GROUP][8 * lane]);
+                *(u32x4*)(kbuf + RING_HALF + r * 256 + ((lane ^ (2 * (r & 7))) << 4)) = *(const u32x4*)(&s_new[GROUP + 1][8 * lane]);
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");       // written before the transposed reads below are asked for
+        }
+        f32x4 sc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int t = 0; t < KSTEPS; ++t) {
+            Frag kf;
+            kf.u = *(const u32x4*)(kbuf + l16 * 256 + (((4 * t + h) ^ l16) << 4));
+            sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qf[t].v, sc, 0, 0, 0);
+        }
+        // The values, transposed, are asked for now and arrive during the softmax.  The instruction is
+        // written out: the compiler would make a read through the intrinsic wait for every load into
+        // LDS that is still on its way, the next block's included.
+        s16x4 vt[HEAD_DIM / 16];
+#pragma unroll
+        for (int b = 0; b < HEAD_DIM / 16; ++b)
+            asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(vt[b]) : "v"(v_addr[b] + stage * (2 * RING_HALF)));
+        // sc[v] = S^T[key 4 h + v][head l16]
+        float m_blk = -INFINITY;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const int s = (kb << 4) + 4 * h + v;
+            sc[v] = (s >= lo && s <= pos) ? __fmul_rn(sc[v], scale_log2e) : -INFINITY;   // every rounding spelt out: both forms of the kernel give the same bits
+            m_blk = fmaxf(m_blk, sc[v]);
+        }
+        m_blk = fmaxf(m_blk, __shfl_xor(m_blk, 16, KIPP_WAVE));
+        m_blk = fmaxf(m_blk, __shfl_xor(m_blk, 32, KIPP_WAVE));
+        const float m_new = fmaxf(m_run, m_blk);
+        const float m_use = m_new == -INFINITY ? 0.0f : m_new;       // nothing visible yet: every weight is 0
+        const float alpha = exp2f(__fsub_rn(m_run, m_use));          // m_run = -inf gives 0
+        float l_blk = 0.0f;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            sc[v] = exp2f(__fsub_rn(sc[v], m_use));                  // -inf gives 0
+            l_blk = __fadd_rn(l_blk, sc[v]);
+        }
+        l_blk += __shfl_xor(l_blk, 16, KIPP_WAVE);
+        l_blk += __shfl_xor(l_blk, 32, KIPP_WAVE);
+        l_run = fmaf(l_run, alpha, l_blk);
+        m_run = m_new;
+        union {
+            u32x2 u;
+            s16x4 v;
+        } pb;
+        pb.u = (u32x2){pack_bf16(sc[0], sc[1]), pack_bf16(sc[2], sc[3])};
+        static_assert(HEAD_DIM / 16 == 8, "the wait below names the eight transposed reads");
+        asm volatile("s_waitcnt lgkmcnt(0)"
+                     : "+v"(vt[0]), "+v"(vt[1]), "+v"(vt[2]), "+v"(vt[3]), "+v"(vt[4]), "+v"(vt[5]), "+v"(vt[6]), "+v"(vt[7]));
+        // every read of the stage has come back: the block after next is asked for
+        if (j + 2 < n_mine) issue(j + 2, stage);
+#pragma unroll
+        for (int b = 0; b < HEAD_DIM / 16; ++b) {
+#pragma unroll
+            for (int v = 0; v < 4; ++v) o[b][v] = __fmul_rn(o[b][v], alpha);
+            o[b] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vt[b], pb.v, o[b], 0, 0, 0);
+        }
+    }
+
+    // ---- merge the waves: o[b][v] = O[head l16][16 b + 4 h + v]
+    __syncthreads();                                                 // every ring has been read for the last time
+    float* s_red = (float*)ring;                                     // [WAVES][GROUP][HEAD_DIM]
+    float* s_ml = s_red + WAVES * GROUP * HEAD_DIM;                  // [WAVES][GROUP][2]
+    if (l16 < GROUP) {
+#pragma unroll
+        for (int b = 0; b < HEAD_DIM / 16; ++b)
+            *(f32x4*)(s_red + ((size_t)wave * GROUP + l16) * HEAD_DIM + 16 * b + 4 * h) = o[b];
+        if (h == 0) {
+            s_ml[(wave * GROUP + l16) * 2] = m_run;
+            s_ml[(wave * GROUP + l16) * 2 + 1] = l_run;
+        }
+    }
+    __syncthreads();
+    for (int idx = tid; idx < GROUP * HEAD_DIM; idx += THREADS) {
+        const int g = idx / HEAD_DIM, dcol = idx % HEAD_DIM;
+        float m = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w) m = fmaxf(m, s_ml[(w * GROUP + g) * 2]);
+        float a = 0.0f, l = 0.0f;
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w) {
+            const float f = exp2f(__fsub_rn(s_ml[(w * GROUP + g) * 2], m));    // a wave without keys: 2^-inf = 0
+            a = fmaf(s_red[((size_t)w * GROUP + g) * HEAD_DIM + dcol], f, a);
+            l = fmaf(s_ml[(w * GROUP + g) * 2 + 1], f, l);
+        }
+        const int head = kvh * GROUP + g;
+        if (n_splits == 1) {
+            out[((size_t)row * n_q + head) * HEAD_DIM + dcol] = f32_to_bf16(a / l);
+        } else {
+            const size_t slot = ((size_t)blockIdx.z * n_q + head) * max_splits + blockIdx.x;
+            part_acc[slot * HEAD_DIM + dcol] = a;
+            if (dcol == 0) {
+                part_ml[slot * 2] = m;
+                part_ml[slot * 2 + 1] = l;
+            }
+        }
+    }
+}
+#endif  // RING_OK
+
 // Merge the splits of every (token, head) in index order:
 // m* = max m_s, out = sum_s acc_s 2^(m_s - m*) / sum_s l_s 2^(m_s - m*)
 // (/root/reference/metal/kipp_kernels.metal:741-779).
@@ -642,9 +960,55 @@ __global__ void attention_decode_reduce_kernel(
     }
 }
 
+
+#if RING_OK
+// The kernel that streams through LDS, if it takes this launch (0 if not): whole contexts a workgroup.
+template <bool FUSED>
+static int launch_ring(const bf16_t* q, bf16_t* k_cache, bf16_t* v_cache, bf16_t* out, float* part_acc, float* part_ml,
+                       const int32_t* rows, const int32_t* positions, const int32_t* seq_of_token,
+                       const int32_t* block_table, int max_blocks, int n_items, int n_q, int n_kv, int page,
+                       float scale_log2e, int window, int grid_splits, int max_splits, Projected pj, hipStream_t stream,
+                       int* rc) {
+    if (page % 16 != 0 || (long long)n_items * n_kv < RING_FROM_PAIRS) return 0;
+    const int lds = RING_BYTES + (FUSED ? (GROUP + 2) * HEAD_DIM * 2 : 0);
+    static bool prepared = false;
+    if (!prepared) {
+        if (hipFuncSetAttribute((const void*)attention_decode_ring_kernel<FUSED>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                lds) != hipSuccess) {
+            *rc = -6;
+            return 1;
+        }
+        prepared = true;
+    }
+    const int span = grid_splits * SPLIT;
+    const int range = span < RING_RANGE ? span : RING_RANGE;
+    const int ring_splits = (span + range - 1) / range + (window > 0 ? 1 : 0);   // a window may straddle one more edge
+    if (ring_splits > max_splits) return 0;
+    hipLaunchKernelGGL(attention_decode_ring_kernel<FUSED>, dim3(ring_splits, n_kv, n_items), dim3(THREADS), lds, stream, q,
+                       k_cache, v_cache, out, part_acc, part_ml, rows, positions, seq_of_token, block_table, max_blocks, n_q,
+                       n_kv, page, scale_log2e, window, max_splits, range, pj);
+    *rc = KIPP_LAUNCH_CHECK();
+    if (*rc != 0 || ring_splits == 1) return 1;
+    hipLaunchKernelGGL(attention_decode_reduce_kernel, dim3(n_q, n_items), dim3(HEAD_DIM >= 64 ? 64 : HEAD_DIM), 0, stream,
+                       part_acc, part_ml, out, rows, positions, n_q, window, max_splits, range);
+    *rc = KIPP_LAUNCH_CHECK();
+    return 1;
+}
+#endif
+
 extern "C" {
 
 int kipp_attention_decode_split() { return SPLIT; }
+
+// 1 if a launch of this shape goes to the kernel that streams through LDS (whole contexts a workgroup;
+// its fused form has no limit on the rows).
+int kipp_attention_decode_ring_takes(int n_items, int n_kv, int page) {
+#if RING_OK
+    return page % 16 == 0 && (long long)n_items * n_kv >= RING_FROM_PAIRS ? 1 : 0;
+#else
+    return 0;
+#endif
+}
 
 // `rows[i]` is the batch row of the i-th decode token.  `grid_splits` is how
 // many splits the launch covers (at least those of the longest sequence);
@@ -659,6 +1023,15 @@ int kipp_attention_decode(const void* q, const void* k_cache, const void* v_cach
     if (grid_splits <= 0 || grid_splits > max_splits) return -3;
     if (page <= 0 || (page & (page - 1))) return -4;   // pages of a power of two only
     const float scale_log2e = scale * 1.4426950408889634f;
+#if RING_OK
+    {
+        int rc = 0;
+        if (launch_ring<false>((const bf16_t*)q, (bf16_t*)k_cache, (bf16_t*)v_cache, (bf16_t*)out, part_acc, part_ml, rows,
+                               positions, seq_of_token, block_table, max_blocks, n_items, n_q, n_kv, page, scale_log2e, window,
+                               grid_splits, max_splits, Projected{}, stream, &rc))
+            return rc;
+    }
+#endif
     // Long contexts: long ranges of keys walked by each workgroup, if that still gives every compute
     // unit two workgroups.  A function of the launch's shape, never of the data.
     const int big_splits = (grid_splits * SPLIT + BIG - 1) / BIG + (window > 0 ? 1 : 0);
@@ -707,6 +1080,15 @@ int kipp_attention_decode_fused(const float* qkv, int parts, int n_tokens, const
     const float scale_log2e = scale * 1.4426950408889634f;
     Projected pj{qkv, parts, (size_t)n_tokens * (n_q + 2 * n_kv) * HEAD_DIM, q_norm_w, k_norm_w, eps, inv_freq, angles,
                  write_kv};
+#if RING_OK
+    {
+        int rc = 0;
+        if (launch_ring<true>((const bf16_t*)nullptr, (bf16_t*)k_cache, (bf16_t*)v_cache, (bf16_t*)out, part_acc, part_ml, rows,
+                              positions, seq_of_token, block_table, max_blocks, n_items, n_q, n_kv, page, scale_log2e, window,
+                              grid_splits, max_splits, pj, stream, &rc))
+            return rc;
+    }
+#endif
     hipLaunchKernelGGL(attention_decode_kernel<true>, dim3(grid_splits, n_kv, n_items), dim3(THREADS), 0, stream,
                        (const bf16_t*)nullptr, (bf16_t*)k_cache, (bf16_t*)v_cache, (bf16_t*)out, part_acc, part_ml,
                        rows, positions, seq_of_token, block_table, max_blocks, n_q, n_kv, page, scale_log2e, window,

@@ -27,6 +27,17 @@ __device__ __forceinline__ float load_f(const bf16_t* p, size_t i) { return bf16
 __device__ __forceinline__ void store_f(float* p, size_t i, float v) { p[i] = v; }
 __device__ __forceinline__ void store_f(bf16_t* p, size_t i, float v) { p[i] = f32_to_bf16(v); }
 
+// The per-head norm and the rotation with every rounding spelt out: nothing is left for the
+// compiler to contract one way in one kernel and another way in the next, so whichever kernel
+// prepares a head (the rotary kernels, the fused decode attention) gives the same bits
+// (/root/reference/src/kipp.c:2480-2500, 2368-2382).
+__device__ __forceinline__ float square_add(float ss, float v) { return fmaf(v, v, ss); }
+__device__ __forceinline__ float head_norm_scale(float ss, float width, float eps) {
+    return 1.0f / sqrtf(__fadd_rn(ss / width, eps));
+}
+__device__ __forceinline__ float rotate_lo(float a, float b, float cs, float sn) { return fmaf(a, cs, -__fmul_rn(b, sn)); }
+__device__ __forceinline__ float rotate_hi(float a, float b, float cs, float sn) { return fmaf(b, cs, __fmul_rn(a, sn)); }
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, KIPP_WAVE);

@@ -6,6 +6,7 @@ path behind any of them.
 from __future__ import annotations
 
 import ctypes
+import functools
 from typing import Optional
 
 import torch
@@ -299,6 +300,17 @@ def attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
 DECODE_FUSED_SLABS = 4
 
 
+@functools.lru_cache(maxsize=None)
+def attention_decode_whole_contexts(n_items: int, n_kv: int, head_dim: int, group: int, page: int) -> bool:
+    """Does a decode launch of this shape go to the kernel in which a workgroup walks a
+    sequence's whole context (sequences x key/value heads alone fill the chip)?  Its fused
+    form takes any number of rows."""
+    if head_dim % 16 or group > 16:
+        return False
+    lib = build.library("attention_decode", {"HEAD_DIM": head_dim, "GROUP": group})
+    return bool(lib.kipp_attention_decode_ring_takes(int(n_items), int(n_kv), int(page)))
+
+
 def attention_decode_fused_ok(head_dim: int, rotary_dim: int, rotates: bool, slabs: int = 1) -> bool:
     """Can decode attention start from the QKV projection's output?  Head sizes that
     are multiples of 128, rotated over their whole width (or not at all), a
@@ -388,7 +400,8 @@ def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
 
 # --------------------------------------------------------------------------- matrix products
 
-SKINNY_MAX_ROWS = 64     # rows of the few-rows kernel
+SKINNY_MAX_ROWS = 64     # rows the few-rows kernel takes
+SKINNY_BEST_ROWS = 8     # ... and rows up to which it is the faster one (each wave reads its rows of x itself; beyond, x staged in LDS wins)
 ROWS_MAX_ROWS = 128      # rows of the kernel that stages x through LDS
 
 

@@ -46,12 +46,12 @@ __global__ void qk_norm_rope_kv_kernel(
         if (e < d)
             for (int p = 0; p < parts; ++p) v += load_f(src, p * part_stride + e);   // slabs of a split product, in order
         vals[c] = v;
-        ss += v * v;
+        ss = square_add(ss, v);
     }
     const float* norm_w = kind == 0 ? q_norm_w : (kind == 1 ? k_norm_w : nullptr);
     if (norm_w != nullptr) {
         ss = wave_sum(ss);
-        const float scale = 1.0f / sqrtf(ss / (float)d + eps);
+        const float scale = head_norm_scale(ss, (float)d, eps);
 #pragma unroll
         for (int c = 0; c < MAX_D / KIPP_WAVE; ++c) {
             const int e = lane + c * KIPP_WAVE;
@@ -84,8 +84,8 @@ __global__ void qk_norm_rope_kv_kernel(
                 sn = sinf(angle);
             }
             const float a = buf[wave][i], b = buf[wave][i + half];
-            lo[c] = a * cs - b * sn;
-            hi[c] = b * cs + a * sn;
+            lo[c] = rotate_lo(a, b, cs, sn);
+            hi[c] = rotate_hi(a, b, cs, sn);
         }
     }
     __syncthreads();
@@ -180,17 +180,17 @@ __global__ void __launch_bounds__(HEADS_PER_BLOCK * KIPP_WAVE) qk_norm_rope_kv_r
                 if ((kind == 0 ? q_norm_w : k_norm_w) != nullptr) {
                     float ss = 0.0f;
 #pragma unroll
-                    for (int c = 0; c < NC; ++c) ss += v[u][c] * v[u][c];
+                    for (int c = 0; c < NC; ++c) ss = square_add(ss, v[u][c]);
                     ss = wave_sum(ss);
-                    const float scale = 1.0f / sqrtf(ss / (float)D + eps);
+                    const float scale = head_norm_scale(ss, (float)D, eps);
 #pragma unroll
                     for (int c = 0; c < NC; ++c) v[u][c] *= scale * (kind == 0 ? qw[c] : kw[c]);
                 }
 #pragma unroll
                 for (int c = 0; c < HC; ++c) {
                     const float a = v[u][c], b = v[u][c + HC];
-                    v[u][c] = a * cs[c] - b * sn[c];
-                    v[u][c + HC] = b * cs[c] + a * sn[c];
+                    v[u][c] = rotate_lo(a, b, cs[c], sn[c]);
+                    v[u][c + HC] = rotate_hi(a, b, cs[c], sn[c]);
                 }
             }
             if (kind == 0) {

@@ -37,6 +37,7 @@ PREBUILT_ATTENTION = [(128, 4), (128, 8), (128, 16), (128, 1), (16, 2), (32, 4),
 
 # builds of the decode attention in which the kernel for long contexts takes over at 1,024 keys
 # already, so that a kernel test can reach it with contexts it can check
+PREBUILT_WHOLE_CONTEXTS = [(128, 4), (128, 16)]    # tests: the whole-context decode kernel at few sequences
 PREBUILT_EARLY_STREAM = [(128, 4), (48, 3), (16, 2)]
 
 
@@ -48,5 +49,7 @@ def prebuilt() -> List[Spec]:
                 out.append(v)
     for head_dim, group in PREBUILT_EARLY_STREAM:
         out.append(("attention_decode", {"HEAD_DIM": head_dim, "GROUP": group, "STREAM_FROM": 1024}))
+    for head_dim, group in PREBUILT_WHOLE_CONTEXTS:
+        out.append(("attention_decode", {"HEAD_DIM": head_dim, "GROUP": group, "RING_FROM_PAIRS": 1}))
     out.append(("probe", None))       # the read-bandwidth yardstick of `python -m kipp_amd.workloads hbm`
     return out

@@ -44,7 +44,7 @@ class GatedMLP:
         act = rt.empty((rows, inner), rt.act_dtype)
         w = self.w_gate_up
         ours = w.dtype == x.dtype == torch.bfloat16 and rt.ops.gemm_rows_ok(rows, x.shape[1])
-        if ours and rows <= 16:
+        if ours and rows <= rt.ops.SKINNY_BEST_ROWS:
             # both products and the activation in one kernel
             rt.ops.gemm_skinny_swiglu(x, w.rows, act, tiles=w.tiles)
         elif ours and w.pairs:

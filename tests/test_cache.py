@@ -107,14 +107,29 @@ def test_groups_are_formed_by_need():
     assert m.view(2).group == 1 and m.view(1, reads_run=0).writable is False and m.view(0).writable
 
 
+def test_a_fresh_pool_hands_out_scattered_pages():
+    """Every page once, neighbours far apart: sequences of equal length that arrive together do not
+    end up at equal distances in memory."""
+    from kipp_amd.cache.pool import PagePool, scattered_order
+    for n in (1, 2, 5, 64, 1000, 17028):
+        order = scattered_order(n)
+        assert sorted(order) == list(range(n))
+        if n >= 64:
+            assert min(abs(a - b) for a, b in zip(order, order[1:])) > n // 4
+    pool = PagePool(10, 4)
+    assert [pool.alloc() for _ in range(10)] == scattered_order(10) and pool.alloc() is None
+
+
 def test_reserve_is_all_or_nothing():
     m = _manager(num_pages=5)
     a, b = m.open("a"), m.open("b")
     m.reserve([(a, 9)])                                   # 3 pages
     m.commit(a, list(range(9)))
+    before = [list(t) for t in a.tables]
+    assert len(before[0]) == 3 and len(set(before[0])) == 3
     with pytest.raises(OutOfPages):
         m.reserve([(a, 3), (b, 9)])                       # a: +0 (12 fits 3 pages), b: 3 > 2 free
-    assert m.free_pages() == [2] and a.tables == [[0, 1, 2]] and b.tables == [[]]
+    assert m.free_pages() == [2] and a.tables == before and b.tables == [[]]
     m.check()
     with pytest.raises(ValueError):
         m.reserve([(a, 0)])

@@ -367,13 +367,69 @@ def _many_rows(ops, n_q, n_kv, d, page, window):
     assert not got[:2].any()
 
 
+def _whole_contexts(ops):
+    """The kernels built so that the one in which a workgroup walks a whole context takes every launch
+    it can (head size 128, pages of 16 keys and more), not only those of many sequences."""
+    inner = ops._fn
+
+    def forced(lib, name, argtypes, defines=None):
+        return inner(lib, name, argtypes, dict(defines, RING_FROM_PAIRS=1) if lib == "attention_decode" else defines)
+    return inner, forced
+
+
+@pytest.mark.parametrize("n_q,n_kv,d,page,window", [(32, 8, 128, 16, 0), (32, 8, 128, 16, 300), (16, 1, 128, 32, 0), (16, 1, 128, 16, 5000)])
+def test_attention_decode_over_whole_contexts(n_q, n_kv, d, page, window):
+    """A workgroup a (sequence, key/value head), keys and values streamed through LDS: contexts of one
+    key, at block edges (15, 16, 17, 63, 64, 65), around a stage's and a range's end (4095, 4096, 4097, 8200),
+    rows that are not the first of the batch."""
+    ops = _ops()
+    inner, forced = _whole_contexts(ops)
+    ops._fn = forced
+    try:
+        rng = np.random.default_rng(n_q + page + window)
+        seq_lens = [1, 2, 15, 16, 17, 63, 64, 65, 128, 300, 777, 1024, 2049] + ([4095, 4096, 4097, 8200] if n_kv == 1 else [])
+        table, k, v = _paged_setup(rng, seq_lens, n_kv, d, page, torch.bfloat16)
+        t = len(seq_lens) + 2
+        rows = list(range(2, t))
+        positions, seq_of = [0] * t, [0] * t
+        for r, (sq, n) in zip(rows, enumerate(seq_lens)):
+            positions[r], seq_of[r] = n - 1, sq
+        q = torch.tensor(rng.normal(size=(t, n_q * d)), dtype=torch.bfloat16)
+        out = torch.zeros(t, n_q * d, dtype=torch.bfloat16, device=DEV)
+        ws = ops.attention_decode_workspace(len(rows), n_q, d, max(seq_lens), DEV)
+        ops.attention_decode(q.to(DEV), k.to(DEV), v.to(DEV), out, _t(rows, torch.int32), _t(positions, torch.int32),
+                             _t(seq_of, torch.int32), _t(table, torch.int32), n_q, n_kv, d, 1 / math.sqrt(d), window,
+                             max(seq_lens), ws)
+        ref = _attention_reference(q[rows], k, v, table, [positions[r] for r in rows], [seq_of[r] for r in rows],
+                                   n_q, n_kv, d, page, window)
+        got = out.float().cpu().numpy().reshape(t, n_q, d)
+        for i, r in enumerate(rows):
+            assert _rel(got[r], ref[i]) < 1e-5, f"context of {seq_lens[i]} keys"
+        assert not got[:2].any()
+    finally:
+        ops._fn = inner
+
+
+@pytest.mark.parametrize("whole", [False, True])
 @pytest.mark.parametrize("n_q,n_kv,d,page", [(32, 8, 128, 16), (8, 1, 128, 8), (16, 1, 128, 16), (3, 3, 128, 4), (8, 2, 256, 32), (4, 2, 256, 16)])
 @pytest.mark.parametrize("window,norm,slabs,write_kv", [(0, True, 1, True), (300, True, 3, True), (0, False, 2, True), (0, True, 1, False)])
-def test_attention_decode_from_the_projection(n_q, n_kv, d, page, window, norm, slabs, write_kv):
+def test_attention_decode_from_the_projection(n_q, n_kv, d, page, window, norm, slabs, write_kv, whole):
     """Decode attention that starts from the QKV projection's output: the same bits
     in the attention output and in the cache as the rotary kernel followed by the
-    attention kernel, at split edges (256, 257, 513) and for the first token."""
+    attention kernel, at split edges (256, 257, 513) and for the first token.  `whole`: the
+    kernels in which a workgroup walks a whole context (head size 128, pages of 16 and more)."""
     ops = _ops()
+    if whole and not (d == 128 and page % 16 == 0):
+        pytest.skip("the whole-context kernel takes head size 128 and pages of 16 keys and more")
+    inner, forced = _whole_contexts(ops)
+    ops._fn = forced if whole else inner
+    try:
+        _from_the_projection(ops, n_q, n_kv, d, page, window, norm, slabs, write_kv)
+    finally:
+        ops._fn = inner
+
+
+def _from_the_projection(ops, n_q, n_kv, d, page, window, norm, slabs, write_kv):
     rng = np.random.default_rng(n_q * 5 + d + window + slabs)
     seq_lens = [1, 70, 300, 700, 256, 257, 513]
     table, k, v = _paged_setup(rng, seq_lens, n_kv, d, page, torch.bfloat16)
