@@ -301,14 +301,17 @@ DECODE_FUSED_SLABS = 4
 
 
 @functools.lru_cache(maxsize=None)
-def attention_decode_whole_contexts(n_items: int, n_kv: int, head_dim: int, group: int, page: int) -> bool:
-    """Does a decode launch of this shape go to the kernel in which a workgroup walks a
-    sequence's whole context (sequences x key/value heads alone fill the chip)?  Its fused
-    form takes any number of rows."""
+def attention_decode_streams(n_items: int, n_kv: int, head_dim: int, group: int, page: int, max_context: int,
+                             window: int = 0) -> bool:
+    """Does a decode launch of this shape go to the kernel that streams keys and values
+    through LDS (many sequences: a workgroup a whole context; few sequences with long
+    contexts: long ranges)?  Its fused form takes any number of rows and any context."""
     if head_dim % 16 or group > 16:
         return False
+    span = min(max_context, window) if window else max_context
+    splits = (span + DECODE_SPLIT - 1) // DECODE_SPLIT + (1 if window else 0)
     lib = build.library("attention_decode", {"HEAD_DIM": head_dim, "GROUP": group})
-    return bool(lib.kipp_attention_decode_ring_takes(int(n_items), int(n_kv), int(page)))
+    return bool(lib.kipp_attention_decode_ring_takes(int(n_items), int(n_kv), int(page), int(max(1, splits))))
 
 
 def attention_decode_fused_ok(head_dim: int, rotary_dim: int, rotates: bool, slabs: int = 1) -> bool:

@@ -85,12 +85,12 @@ class Attention:
         fast = rt.dtype == "bfloat16" and rt.ops.attention_fast_ok(s.num_heads, s.num_kv_heads, cache.page_size, table.shape[1])
         # single tokens only: norm, rotation, cache write and attention in one kernel, for a few of them (with
         # more rows or long contexts every split's workgroup would prepare the queries again, which costs more
-        # than the rotary kernel it saves) and again for so many that a workgroup takes a whole context
+        # than the rotary kernel it saves) and wherever the kernel that walks whole contexts or long ranges runs
         fused = fast and not batch.n_prefill_items and batch.n_decode == n \
             and rt.ops.attention_decode_fused_ok(s.head_dim, rotary_dim, inv_freq is not None) \
             and ((n <= FUSED_DECODE_ROWS and batch.max_decode_ctx < FUSED_DECODE_KEYS)
-                 or rt.ops.attention_decode_whole_contexts(n, s.num_kv_heads, s.head_dim, s.num_heads // s.num_kv_heads,
-                                                           cache.page_size))
+                 or rt.ops.attention_decode_streams(n, s.num_kv_heads, s.head_dim, s.num_heads // s.num_kv_heads,
+                                                    cache.page_size, batch.max_decode_ctx, s.window or 0))
         qkv = rt.linear(x, self.w_qkv, slabs=rt.ops.DECODE_FUSED_SLABS if fused else True)
         if fused:
             out = rt.empty((n, s.q_dim), rt.act_dtype)

@@ -410,6 +410,31 @@ def test_attention_decode_over_whole_contexts(n_q, n_kv, d, page, window):
         ops._fn = inner
 
 
+@pytest.mark.parametrize("window", [0, 6000, 8000])
+def test_attention_decode_of_few_long_sequences(window):
+    """Four sequences of several thousand keys: the streaming kernel takes them in ranges of 1,024 keys
+    (what gives 256 workgroups), with the merge kernel behind it; contexts at the ranges' edges.  With a
+    window of 6,000 the ranges would be shorter than that and the split kernel stays."""
+    ops = _ops()
+    n_q, n_kv, d, page = 8, 8, 128, 16
+    assert ops.attention_decode_streams(4, n_kv, d, 1, page, 9000) and not ops.attention_decode_streams(4, n_kv, d, 1, page, 2000)
+    assert ops.attention_decode_streams(4, n_kv, d, 1, page, 9000, 8000) and not ops.attention_decode_streams(4, n_kv, d, 1, page, 9000, 6000)
+    rng = np.random.default_rng(17 + window)
+    seq_lens = [9000, 1024, 1025, 7168]
+    table, k, v = _paged_setup(rng, seq_lens, n_kv, d, page, torch.bfloat16)
+    rows = list(range(4))
+    positions = [n - 1 for n in seq_lens]
+    q = torch.tensor(rng.normal(size=(4, n_q * d)), dtype=torch.bfloat16)
+    out = torch.zeros(4, n_q * d, dtype=torch.bfloat16, device=DEV)
+    ws = ops.attention_decode_workspace(4, n_q, d, max(seq_lens), DEV)
+    ops.attention_decode(q.to(DEV), k.to(DEV), v.to(DEV), out, _t(rows, torch.int32), _t(positions, torch.int32),
+                         _t(rows, torch.int32), _t(table, torch.int32), n_q, n_kv, d, 1 / math.sqrt(d), window, max(seq_lens), ws)
+    ref = _attention_reference(q, k, v, table, positions, rows, n_q, n_kv, d, page, window)
+    got = out.float().cpu().numpy().reshape(4, n_q, d)
+    for i in range(4):
+        assert _rel(got[i], ref[i]) < 1e-5, f"context of {seq_lens[i]} keys"
+
+
 @pytest.mark.parametrize("whole", [False, True])
 @pytest.mark.parametrize("n_q,n_kv,d,page", [(32, 8, 128, 16), (8, 1, 128, 8), (16, 1, 128, 16), (3, 3, 128, 4), (8, 2, 256, 32), (4, 2, 256, 16)])
 @pytest.mark.parametrize("window,norm,slabs,write_kv", [(0, True, 1, True), (300, True, 3, True), (0, False, 2, True), (0, True, 1, False)])
