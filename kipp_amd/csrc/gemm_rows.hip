@@ -30,8 +30,9 @@ union Frag {
 // TILED: W in the streaming layout [tile of 16 rows][step of 32 columns][lane][8 values]
 // (rows padded to whole tiles with zeros, K a multiple of 32), in which a wave's load is
 // one contiguous KB.
-// DEPTH: steps of 32 columns in one chunk.
-template <int MT, int TW, bool TILED, int DEPTH>
+// DEPTH: steps of 32 columns in one chunk.  NTW: 16-row tiles of W a wave streams (every fragment of X
+// read from LDS then serves NTW products, and a workgroup's staging of X serves NTW times the rows).
+template <int MT, int TW, bool TILED, int DEPTH, int NTW>
 __global__ void __launch_bounds__(TW * KIPP_WAVE) gemm_rows_kernel(
     const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, float* __restrict__ Y, int M, int N, int K) {
     constexpr int CHUNK = 32 * DEPTH;                          // columns of X staged at a time
@@ -45,15 +46,17 @@ __global__ void __launch_bounds__(TW * KIPP_WAVE) gemm_rows_kernel(
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l16 = lane & 15, h = lane >> 4;
-    const int n0 = (blockIdx.x * TW + wave) * 16;
+    const int n0 = (blockIdx.x * TW + wave) * (16 * NTW);
     const int part = blockIdx.y, parts = gridDim.y;
     const int groups = K / CHUNK;                              // whole chunks; the rest of K goes to the last part
     const int g_begin = (int)((long long)groups * part / parts);
     const int g_end = (int)((long long)groups * (part + 1) / parts);
 
-    const int row = min(n0 + l16, N - 1);                      // clamped: in bounds, dropped at the store
-    const bf16_t* w_row = TILED ? W + (size_t)min(n0 >> 4, (N + 15) / 16 - 1) * (K / 32) * 512 + lane * 8
-                                : W + (size_t)row * K + 8 * h;
+    const bf16_t* w_row[NTW];                                  // clamped: in bounds, dropped at the store
+#pragma unroll
+    for (int i = 0; i < NTW; ++i)
+        w_row[i] = TILED ? W + (size_t)min((n0 >> 4) + i, (N + 15) / 16 - 1) * (K / 32) * 512 + lane * 8
+                         : W + (size_t)min(n0 + 16 * i + l16, N - 1) * K + 8 * h;
 
     // the units of X this thread stages: unit -> (row, 8-column chunk)
     const bf16_t* x_src[XR];
@@ -66,13 +69,18 @@ __global__ void __launch_bounds__(TW * KIPP_WAVE) gemm_rows_kernel(
         x_dst[i] = r * X_PITCH + c * 8;
     }
 
-    f32x4 acc[MT];
+    f32x4 acc[NTW][MT];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) acc[mt] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
-    Frag wf[DEPTH];
+    for (int i = 0; i < NTW; ++i)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) acc[i][mt] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
+    Frag wf[DEPTH][NTW];
     u32x4 xr[XR];
 
-    auto fetch_w = [&](int u, int step) { wf[u].u = *(const u32x4*)(w_row + (TILED ? 512 : 32) * step); };
+    auto fetch_w = [&](int u, int step) {
+#pragma unroll
+        for (int i = 0; i < NTW; ++i) wf[u][i].u = *(const u32x4*)(w_row[i] + (TILED ? 512 : 32) * step);
+    };
     auto fetch_x = [&](int g) {
 #pragma unroll
         for (int i = 0; i < XR; ++i) xr[i] = *(const u32x4*)(x_src[i] + (size_t)g * CHUNK);
@@ -86,7 +94,8 @@ __global__ void __launch_bounds__(TW * KIPP_WAVE) gemm_rows_kernel(
         for (int mt = 0; mt < MT; ++mt) {
             Frag xf;
             xf.u = *(const u32x4*)(xs[buf] + (mt * 16 + l16) * X_PITCH + 32 * u + 8 * h);
-            acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u].v, xf.v, acc[mt], 0, 0, 0);
+#pragma unroll
+            for (int i = 0; i < NTW; ++i) acc[i][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u][i].v, xf.v, acc[i][mt], 0, 0, 0);
         }
     };
 
@@ -118,55 +127,65 @@ __global__ void __launch_bounds__(TW * KIPP_WAVE) gemm_rows_kernel(
     if (part == parts - 1) {
         for (int k = groups * CHUNK; k < K; k += 32) {
             const bool ok = k + 8 * h < K;
-            Frag w_t;
-            w_t.u = (u32x4){0u, 0u, 0u, 0u};
-            if (ok) w_t.u = *(const u32x4*)(w_row + (TILED ? 16 * k : k));
+            Frag w_t[NTW];
+#pragma unroll
+            for (int i = 0; i < NTW; ++i) {
+                w_t[i].u = (u32x4){0u, 0u, 0u, 0u};
+                if (ok) w_t[i].u = *(const u32x4*)(w_row[i] + (TILED ? 16 * k : k));
+            }
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
                 Frag x_t;
                 x_t.u = (u32x4){0u, 0u, 0u, 0u};
                 if (ok) x_t.u = *(const u32x4*)(X + (size_t)min(16 * mt + l16, M - 1) * K + 8 * h + k);
-                acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_t.v, x_t.v, acc[mt], 0, 0, 0);
+#pragma unroll
+                for (int i = 0; i < NTW; ++i) acc[i][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_t[i].v, x_t.v, acc[i][mt], 0, 0, 0);
             }
         }
     }
-    const int n = n0 + 4 * h;
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-        const int token = 16 * mt + l16;
-        if (token >= M) continue;
-        float* y = Y + ((size_t)part * M + token) * N + n;
-        if (n + 3 < N && (N & 3) == 0) {
-            *(float4*)y = make_float4(acc[mt][0], acc[mt][1], acc[mt][2], acc[mt][3]);
-        } else {
+    for (int i = 0; i < NTW; ++i) {
+        const int n = n0 + 16 * i + 4 * h;
 #pragma unroll
-            for (int v = 0; v < 4; ++v)
-                if (n + v < N) y[v] = acc[mt][v];
+        for (int mt = 0; mt < MT; ++mt) {
+            const int token = 16 * mt + l16;
+            if (token >= M) continue;
+            float* y = Y + ((size_t)part * M + token) * N + n;
+            if (n + 3 < N && (N & 3) == 0) {
+                *(float4*)y = make_float4(acc[i][mt][0], acc[i][mt][1], acc[i][mt][2], acc[i][mt][3]);
+            } else {
+#pragma unroll
+                for (int v = 0; v < 4; ++v)
+                    if (n + v < N) y[v] = acc[i][mt][v];
+            }
         }
     }
 }
 
-// Waves per workgroup (4 or 8, each with 16 rows of W) and parts of K, from the shape
-// only.  A compute unit draws a bounded number of bytes a second, so the workgroups
-// run in rounds of 256 and a round costs what one workgroup reads plus a fixed start;
-// the plan takes the cheapest rounds, with a small charge for every slab the consumer
-// has to add and every part at least one whole chunk.
+// Tiles of 16 rows of W per workgroup (4 or 8 waves with one tile each, or 8 waves with two) and parts of
+// K, from the shape only.  A compute unit draws a bounded number of bytes a second, so the workgroups run
+// in rounds of 256 and a round costs what one workgroup reads, its rows of W and (from L2, at about a
+// quarter of the price a row) all rows of X, plus a fixed start; the plan takes the cheapest rounds, with a
+// small charge for every slab the consumer has to add and every part at least one whole chunk.  (Fitted to
+// sweeps over these splits at 32, 64 and 128 rows: the more rows X has, the larger the workgroups.)
 static int chunk_of(int M) { return M > 64 ? 128 : 256; }
 
-static void plan(int M, int N, int K, int max_parts, int* tw, int* parts) {
+static void plan(int M, int N, int K, int max_parts, int* tw, int* ntw, int* parts) {
     const int tiles = (N + 15) / 16;
     const int groups = K / chunk_of(M) > 0 ? K / chunk_of(M) : 1;
     double best = 1e300;
     *tw = 4;
+    *ntw = 1;
     *parts = 1;
-    for (int t = 4; t <= 8; t *= 2) {
+    for (int t = 4; t <= 16; t *= 2) {
         const int cols = (tiles + t - 1) / t;
         for (int p = 1; p <= max_parts && p <= groups; ++p) {
             const int rounds = (cols * p + 255) / 256;
-            const double cost = rounds * (t * (double)K / p + 150.0 * t) * (1.0 + 0.02 * p);
+            const double cost = rounds * ((t + 0.27 * M / 16.0) * (double)K / p + 150.0 * t) * (1.0 + 0.02 * p);
             if (cost < best * 0.999) {
                 best = cost;
-                *tw = t;
+                *tw = t > 8 ? 8 : t;
+                *ntw = t > 8 ? 2 : 1;
                 *parts = p;
             }
         }
@@ -178,8 +197,8 @@ extern "C" {
 int kipp_gemm_rows_max_rows() { return MAX_ROWS; }
 
 int kipp_gemm_rows_parts(int M, int N, int K, int max_parts) {
-    int tw, parts;
-    plan(M, N, K, max_parts, &tw, &parts);
+    int tw, ntw, parts;
+    plan(M, N, K, max_parts, &tw, &ntw, &parts);
     return parts;
 }
 
@@ -189,36 +208,38 @@ int kipp_gemm_rows(const void* X, const void* W, float* Y, int M, int N, int K, 
                    hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
     if (M > MAX_ROWS || K <= 0 || (K & 7) || max_parts <= 0 || (tiled && (K & 31))) return -1;
-    int tw, parts;
-    plan(M, N, K, max_parts, &tw, &parts);
+    int tw, ntw, parts;
+    plan(M, N, K, max_parts, &tw, &ntw, &parts);
     const int tiles = (N + 15) / 16;
-    dim3 grid((tiles + tw - 1) / tw, parts), block(tw * KIPP_WAVE);
+    dim3 grid((tiles + tw * ntw - 1) / (tw * ntw), parts), block(tw * KIPP_WAVE);
     const int mt = (M + 15) / 16;       // from 65 rows on an even number of 16-row tiles is staged (every thread moves whole units)
-#define KIPP_GR(MT, TW, DEPTH)                                                                                      \
-    do {                                                                                                            \
-        if (tiled)                                                                                                  \
-            hipLaunchKernelGGL((gemm_rows_kernel<MT, TW, true, DEPTH>), grid, block, 0, stream, (const bf16_t*)X,   \
-                               (const bf16_t*)W, Y, M, N, K);                                                       \
-        else                                                                                                        \
-            hipLaunchKernelGGL((gemm_rows_kernel<MT, TW, false, DEPTH>), grid, block, 0, stream, (const bf16_t*)X,  \
-                               (const bf16_t*)W, Y, M, N, K);                                                       \
+#define KIPP_GR(MT, TW, DEPTH, NTW)                                                                                     \
+    do {                                                                                                                \
+        if (tiled)                                                                                                      \
+            hipLaunchKernelGGL((gemm_rows_kernel<MT, TW, true, DEPTH, NTW>), grid, block, 0, stream, (const bf16_t*)X,  \
+                               (const bf16_t*)W, Y, M, N, K);                                                           \
+        else                                                                                                            \
+            hipLaunchKernelGGL((gemm_rows_kernel<MT, TW, false, DEPTH, NTW>), grid, block, 0, stream, (const bf16_t*)X, \
+                               (const bf16_t*)W, Y, M, N, K);                                                           \
     } while (0)
-#define KIPP_GR_TW(TW)                    \
-    switch (mt) {                         \
-        case 1: KIPP_GR(1, TW, 8); break; \
-        case 2: KIPP_GR(2, TW, 8); break; \
-        case 3: KIPP_GR(3, TW, 8); break; \
-        case 4: KIPP_GR(4, TW, 8); break; \
-        case 5:                           \
-        case 6: KIPP_GR(6, TW, 4); break; \
-        case 7:                           \
-        case 8: KIPP_GR(8, TW, 4); break; \
-        default: return -1;               \
+#define KIPP_GR_TW(TW, NTW)                    \
+    switch (mt) {                              \
+        case 1: KIPP_GR(1, TW, 8, NTW); break; \
+        case 2: KIPP_GR(2, TW, 8, NTW); break; \
+        case 3: KIPP_GR(3, TW, 8, NTW); break; \
+        case 4: KIPP_GR(4, TW, 8, NTW); break; \
+        case 5:                                \
+        case 6: KIPP_GR(6, TW, 4, NTW); break; \
+        case 7:                                \
+        case 8: KIPP_GR(8, TW, 4, NTW); break; \
+        default: return -1;                    \
     }
-    if (tw == 8) {
-        KIPP_GR_TW(8)
+    if (tw == 8 && ntw == 2) {
+        KIPP_GR_TW(8, 2)
+    } else if (tw == 8) {
+        KIPP_GR_TW(8, 1)
     } else {
-        KIPP_GR_TW(4)
+        KIPP_GR_TW(4, 1)
     }
 #undef KIPP_GR_TW
 #undef KIPP_GR
