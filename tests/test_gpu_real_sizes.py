@@ -94,15 +94,18 @@ def test_decoding_across_a_graph_bucket_and_many_splits(long_folder, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_a_hundred_requests_decode_together(long_folder, dtype):
-    """More rows than one 64-row product takes: 100 prompts of 3 to 40 tokens enter in one step, then all
-    decode together for 6 steps (the products stage their rows in chunks of 128 columns, the steps are
-    recorded graphs); every tenth request against the plain implementation."""
+@pytest.mark.parametrize("n_requests", [100, 128])
+def test_many_requests_decode_together(long_folder, dtype, n_requests):
+    """More rows than one 64-row product takes: prompts of 3 to 40 tokens enter in one step, then all decode
+    together for 6 steps (the products stage their rows in chunks of 128 columns, the steps are recorded
+    graphs).  With 128 requests (one key/value head each) decode attention is the kernel in which a
+    workgroup walks a whole context, from the projection's output; with 100 the keys are split.  Every
+    tenth request against the plain implementation."""
     from kipp_amd.engine import Engine, StepEntry
     cfg, weights = plain.load_folder(long_folder)
     rng = np.random.default_rng(7)
-    seqs = {f"r{i}": H.random_tokens(100 + i, int(rng.integers(3, 41)) + 6, 311) for i in range(100)}
-    engine = Engine.from_folder(long_folder, dtype=dtype, page_size=16, max_tokens=100 * 64, max_requests=100,
+    seqs = {f"r{i}": H.random_tokens(100 + i, int(rng.integers(3, 41)) + 6, 311) for i in range(n_requests)}
+    engine = Engine.from_folder(long_folder, dtype=dtype, page_size=16, max_tokens=n_requests * 64, max_requests=n_requests,
                                 share_prefixes=False)
     fed = {rid: len(toks) - 6 for rid, toks in seqs.items()}
     engine.step([StepEntry(rid, seqs[rid][:fed[rid]], []) for rid in seqs])
@@ -113,7 +116,9 @@ def test_a_hundred_requests_decode_together(long_folder, dtype):
             got[rid].append(row)
             fed[rid] += 1
     assert engine.graphs.replays >= 4
+    from kipp_amd.csrc import ops
+    assert ops.attention_decode_streams(n_requests, 1, 128, 4, 16, 64) == (n_requests >= 128)
     tol = H.NMSE_F32 if dtype == "float32" else H.NMSE_BF16
     for rid in list(seqs)[::10]:
         ref = plain.forward_whole(cfg, weights, seqs[rid])
-        H.assert_close(np.stack(got[rid]), ref[len(seqs[rid]) - 6:], tol, f"hundred together/{dtype}/{rid}")
+        H.assert_close(np.stack(got[rid]), ref[len(seqs[rid]) - 6:], tol, f"{n_requests} together/{dtype}/{rid}")
