@@ -173,7 +173,13 @@ def main():
         steps = args.steps if b == args.batch else max(8, args.steps // 2)
         warmup = args.warmup if b == args.batch else max(2, args.warmup // 2)
         before = engine.length(ids[0])
-        seconds = decode_run(engine, ids[:b], first, steps, warmup)
+        try:
+            seconds = decode_run(engine, ids[:b], first, steps, warmup)
+        except Exception as exc:          # a further point must not cost the headline: say so and go on
+            if b == args.batch:
+                raise
+            log(f"decode batch {b} failed and is left out: {type(exc).__name__}: {exc}")
+            continue
         ctx_mid = before + warmup + steps / 2.0
         results[b] = {"tok_s": b * steps / seconds, "ms": seconds / steps * 1e3, "steps": steps, "warmup": warmup,
                       "bytes": weight_bytes + b * ctx_mid * kv_per_token}
@@ -195,7 +201,7 @@ def main():
                    "parallelism": "none", "weights": "random N(0,0.02) seed 0"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4)},
-        "points": {f"decode_b{b}": round(results[b]["tok_s"], 1) for b in batches if b != args.batch},
+        "points": {f"decode_b{b}": round(results[b]["tok_s"], 1) for b in batches if b != args.batch and b in results},
     }
     if prefill is not None:
         line["prefill"] = prefill
