@@ -58,3 +58,23 @@ def test_float32_cuttings_are_bitwise_equal(model_folders, tiny_configs, key):
         got = H.replay(_engine(model_folders, key, "float32", share_prefixes=False), requests, maker(requests))
         for rid in requests:
             assert np.array_equal(got[rid], base[rid]), f"{key}/{rid}: bits differ between cuttings"
+
+
+@pytest.mark.parametrize("key", ["a", "b"])
+def test_without_the_streaming_layout(model_folders, tiny_configs, key):
+    """`Runtime(stream_layout=False)` keeps every weight once, as rows: the same kernels read the
+    weights from there (decoding one by one and in a mixed batch), against the plain implementation."""
+    from kipp_amd.engine import Engine
+    from kipp_amd.engine.model import load_model
+    from kipp_amd.runtime import Runtime
+    cfg = tiny_configs[key]
+    requests = _requests(key, cfg, seed=2)
+    folder = model_folders[(key, "bfloat16")]
+    for maker in (H.tail_one_by_one, lambda r: H.mixed(r, seed=9)):
+        steps = maker(requests)
+        engine = Engine(load_model(folder, Runtime("bfloat16", stream_layout=False)), page_size=PAGE[key], max_tokens=512,
+                        share_prefixes=False)
+        assert all(block.parts["ffn"].w_gate_up.tiles is None for block in engine.model.blocks)
+        got = H.replay(engine, requests, steps)
+        for rid, toks in requests.items():
+            H.assert_close(got[rid], H.plain_logits(folder, toks), H.NMSE_BF16, f"{key}/rows only/{rid}")
