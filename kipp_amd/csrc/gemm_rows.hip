@@ -1,10 +1,11 @@
 // Matrix product for a few dozen rows (decode at larger batches):
 // Y[M, N] = X[M, K] . W[N, K]^T, bfloat16 operands, float32 accumulation,
-// M <= 128.  Like the few-rows kernel it is bound by reading W once, but here
+// M <= 256.  Like the few-rows kernel it is bound by reading W once (up to about
+// 128 rows; beyond, the matrix cores' work shows), but here
 // the rows of X are too many to fetch per wave: every wave would read as much
 // of X from L2 as of W from HBM.  So the TW waves of a workgroup share one
 // range of K and stage X through LDS in chunks of 256 columns (128 from 65
-// rows on, so that two workgroups still fit a compute unit; double buffered,
+// rows on, 64 from 129, so that two workgroups still fit a compute unit; double buffered,
 // one barrier a chunk), while each wave streams its own 16 rows of W through a
 // ring of one chunk's steps in registers.
 //
@@ -16,7 +17,7 @@
 // 4 (l / 16) + v of token l % 16.
 #include "common.h"
 
-#define MAX_ROWS 128
+#define MAX_ROWS 256
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
@@ -168,7 +169,7 @@ __global__ void __launch_bounds__(TW * KIPP_WAVE) gemm_rows_kernel(
 // quarter of the price a row) all rows of X, plus a fixed start; the plan takes the cheapest rounds, with a
 // small charge for every slab the consumer has to add and every part at least one whole chunk.  (Fitted to
 // sweeps over these splits at 32, 64 and 128 rows: the more rows X has, the larger the workgroups.)
-static int chunk_of(int M) { return M > 64 ? 128 : 256; }
+static int chunk_of(int M) { return M > 128 ? 64 : (M > 64 ? 128 : 256); }
 
 static void plan(int M, int N, int K, int max_parts, int* tw, int* ntw, int* parts) {
     const int tiles = (N + 15) / 16;
@@ -203,7 +204,7 @@ int kipp_gemm_rows_parts(int M, int N, int K, int max_parts) {
 }
 
 // Y: float32 [parts, M, N] with parts = kipp_gemm_rows_parts(M, N, K, max_parts).
-// M <= 128, K a multiple of 8; `tiled`: W in the streaming layout (K a multiple of 32).
+// M <= 256, K a multiple of 8; `tiled`: W in the streaming layout (K a multiple of 32).
 int kipp_gemm_rows(const void* X, const void* W, float* Y, int M, int N, int K, int max_parts, int tiled,
                    hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
@@ -232,6 +233,14 @@ int kipp_gemm_rows(const void* X, const void* W, float* Y, int M, int N, int K, 
         case 6: KIPP_GR(6, TW, 4, NTW); break; \
         case 7:                                \
         case 8: KIPP_GR(8, TW, 4, NTW); break; \
+        case 9:                                \
+        case 10:                               \
+        case 11:                               \
+        case 12: KIPP_GR(12, TW, 2, NTW); break; \
+        case 13:                               \
+        case 14:                               \
+        case 15:                               \
+        case 16: KIPP_GR(16, TW, 2, NTW); break; \
         default: return -1;                    \
     }
     if (tw == 8 && ntw == 2) {

@@ -405,11 +405,11 @@ def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
 
 SKINNY_MAX_ROWS = 64     # rows the few-rows kernel takes
 SKINNY_BEST_ROWS = 8     # ... and rows up to which it is the faster one (each wave reads its rows of x itself; beyond, x staged in LDS wins)
-ROWS_MAX_ROWS = 128      # rows of the kernel that stages x through LDS
+ROWS_MAX_ROWS = 256      # rows of the kernel that stages x through LDS
 
 
 def gemm_rows_ok(m: int, k: int) -> bool:
-    """Shapes our own streaming products take: at most 128 rows, K a multiple of 8 and at least 32."""
+    """Shapes our own streaming products take: at most 256 rows, K a multiple of 8 and at least 32."""
     return 0 < m <= ROWS_MAX_ROWS and k % 8 == 0 and k >= 32
 
 
@@ -488,8 +488,8 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, max_parts: int = 1, tiles: tor
 
 def gemm_rows(x: torch.Tensor, w: torch.Tensor, max_parts: int = 1, tiles: torch.Tensor = None,
               pairs: bool = False) -> torch.Tensor:
-    """float32 [parts, M, N] whose sum over parts is x . w^T, for 16 < M <= 128 rows
-    (any M <= 128 is taken): the rows of x are staged through LDS and shared by
+    """float32 [parts, M, N] whose sum over parts is x . w^T, for 8 < M <= 256 rows
+    (any M <= 256 is taken): the rows of x are staged through LDS and shared by
     the waves of a workgroup.  `pairs`: `tiles` is tile_weight_pairs(w), w = [gate; up];
     the product then has `pairs_width(inner)` columns in the order of those tiles
     (what `swiglu(..., pairs=True)` takes)."""
@@ -498,7 +498,7 @@ def gemm_rows(x: torch.Tensor, w: torch.Tensor, max_parts: int = 1, tiles: torch
     n = w.shape[0]
     _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm_rows: bfloat16 operands")
     _need(w.shape == (n, k), "gemm_rows: shapes do not match")
-    _need(0 < m <= ROWS_MAX_ROWS and k % 8 == 0, "gemm_rows: at most 128 rows and K a multiple of 8")
+    _need(0 < m <= ROWS_MAX_ROWS and k % 8 == 0, "gemm_rows: at most 256 rows and K a multiple of 8")
     if pairs:
         _need(tiles is not None and n % 2 == 0, "gemm_rows: pairs need the paired tiles of [gate; up]")
         n = pairs_width(n // 2)

@@ -23,7 +23,7 @@ import torch
 from .batch import StepBatch
 
 CONTEXT_BUCKET = 1024
-MAX_GRAPH_ENTRIES = 128     # rows up to which every product of a step is one of our own kernels (none goes to a library)
+MAX_GRAPH_ENTRIES = 256     # rows up to which every product of a step is one of our own kernels (none goes to a library)
 
 
 class DecodeGraph:

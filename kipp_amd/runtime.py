@@ -111,7 +111,7 @@ class Runtime:
         if x.dtype != torch.bfloat16:
             x = self.ops.cast(x, self.empty(x.shape, torch.bfloat16))
         if self.ops.gemm_rows_ok(m, x.shape[1]):
-            # up to 128 rows: our own kernels stream the weight once
+            # up to 256 rows: our own kernels stream the weight once
             most = 0 if slabs is False else (None if slabs is True else int(slabs))
             if m <= self.ops.SKINNY_BEST_ROWS:
                 y = self.ops.gemm_skinny(x, w, max_parts=1 if most == 0 else (most or 8), tiles=tiles)

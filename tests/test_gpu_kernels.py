@@ -629,11 +629,11 @@ def test_tile_weight_layout():
                         tiles=torch.zeros(16 * 64, dtype=torch.bfloat16, device=DEV))   # tiles of another matrix
 
 
-@pytest.mark.parametrize("m", [1, 17, 32, 33, 64, 65, 81, 113, 128])
+@pytest.mark.parametrize("m", [1, 17, 32, 33, 64, 65, 81, 113, 128, 129, 177, 200, 256])
 @pytest.mark.parametrize("n,k,max_parts", [(16, 32, 1), (77, 80, 4), (2560, 264, 8), (2560, 9728, 16), (509, 2560, 2), (6144, 2560, 16),
                                            (70000, 512, 1)])
 def test_gemm_rows(m, n, k, max_parts):
-    """Up to 64 rows x is staged in chunks of 256 columns, from 65 rows on in chunks of 128."""
+    """Up to 64 rows x is staged in chunks of 256 columns, from 65 rows on in chunks of 128, from 129 of 64."""
     ops = _ops()
     rng = np.random.default_rng(m + n)
     x = torch.tensor(rng.normal(size=(m, k)), dtype=torch.bfloat16)

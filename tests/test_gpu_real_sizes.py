@@ -94,7 +94,7 @@ def test_decoding_across_a_graph_bucket_and_many_splits(long_folder, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("n_requests", [100, 128])
+@pytest.mark.parametrize("n_requests", [100, 128, 200])
 def test_many_requests_decode_together(long_folder, dtype, n_requests):
     """More rows than one 64-row product takes: prompts of 3 to 40 tokens enter in one step, then all decode
     together for 6 steps (the products stage their rows in chunks of 128 columns, the steps are recorded
