@@ -101,6 +101,36 @@ def test_running_one_step_ahead_changes_nothing(model_folders, dtype):
     assert run(False, stop_of_first=[stop])[0] == stopped
 
 
+def test_the_scheduler_with_many_requests(model_folders):
+    """150 requests at once (more than one 128-row product and more than the default of running requests):
+    greedy and seeded sampling, lengths of 3 to 20; one step ahead gives what waiting for every step gives,
+    and every page comes back."""
+    from kipp_amd.engine import Engine
+    from kipp_amd.engine.scheduler import Request, Scheduler
+    from kipp_amd.sampling import SampleParams
+    folder = model_folders[("b", "bfloat16")]
+    rng = np.random.default_rng(5)
+    prompts = [H.random_tokens(500 + i, int(rng.integers(2, 30)), 509) for i in range(150)]
+    lengths = [int(rng.integers(3, 21)) for _ in range(150)]
+
+    def run(lookahead):
+        engine = Engine.from_folder(folder, dtype="bfloat16", page_size=8, max_tokens=150 * 64, max_requests=150,
+                                    share_prefixes=False)
+        sched = Scheduler(engine, max_step_tokens=1024, prefill_chunk=64, max_running=150, lookahead=lookahead)
+        for i, prompt in enumerate(prompts):
+            params = SampleParams(temperature=0.8, top_k=50, top_p=0.9, min_p=0.01) if i % 3 == 0 else SampleParams()
+            sched.add(Request(i, prompt, lengths[i], params=params, seed=1000 + i))
+        while not sched.idle:
+            sched.step()
+        engine.cache.check()
+        assert engine.cache.free_pages() == [g.pool.num_pages for g in engine.cache.groups] and not engine._uncommitted
+        return {rid: r.output for rid, r in sched.finished.items()}
+
+    plainly = run(False)
+    ahead = run(True)
+    assert ahead == plainly and [len(ahead[i]) for i in range(150)] == lengths
+
+
 def test_long_decoding_matches_plain(model_folders, tiny_configs):
     """100 tokens decoded one by one after a short prompt, every logits row compared."""
     from kipp_amd.engine import Engine, StepEntry
