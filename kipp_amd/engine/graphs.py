@@ -10,11 +10,17 @@ tables) lives in one static int32 buffer that is overwritten before a replay.
 A graph holds our own kernels only: nothing that reads back to the host, no
 library call, no memset node.  A model with a part that does not declare
 `graph_safe`, or a step that went to a library product, runs eagerly instead.
+
+A shape is recorded when it comes a second time (recording costs the host a
+whole forward pass: under continuous batching the number of decoding requests
+often changes from step to step, and a shape seen once may never return), and
+only the most recently used shapes are kept.
 """
 from __future__ import annotations
 
 import gc
 import weakref
+from collections import OrderedDict
 from typing import Dict, Optional, Sequence, Tuple
 
 import numpy as np
@@ -23,6 +29,7 @@ import torch
 from .batch import StepBatch
 
 CONTEXT_BUCKET = 1024
+MAX_GRAPHS = 48              # shapes kept (each holds its recorded launches and small static buffers)
 MAX_GRAPH_ENTRIES = 256     # rows up to which every product of a step is one of our own kernels (none goes to a library)
 
 
@@ -61,6 +68,7 @@ class DecodeGraph:
         self.logits: Optional[torch.Tensor] = None
         self.copied: Optional[torch.cuda.Event] = None
         self.row_marks = [None] * n
+        self.eager_runs = 0
 
     def fill(self, entries, requests, device_tokens=None) -> None:
         n, h = self.n, self.host_np
@@ -93,12 +101,13 @@ class DecodeGraph:
     def run(self, engine, entries, requests, device_tokens=None) -> torch.Tensor:
         self.fill(entries, requests, device_tokens)
         if self.graph is None:
-            # the first step with this shape runs eagerly (it also makes every workspace the
+            # a shape runs eagerly until it has come twice (that also makes every workspace the
             # kernels keep); if nothing in it went to a library, the same launches are then
             # recorded for the steps to come
             before = engine.rt.library_products
             logits = engine.model.forward(self.batch, engine.cache)
-            if engine.rt.library_products != before:
+            self.eager_runs += 1
+            if engine.rt.library_products != before or self.eager_runs < 2:
                 return logits
             torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()
@@ -123,7 +132,7 @@ class DecodeGraphs:
 
     def __init__(self, engine):
         self._engine = weakref.ref(engine)     # no cycle: an engine and its graphs go away together, at once
-        self.graphs: Dict[Tuple[int, int], DecodeGraph] = {}
+        self.graphs: "OrderedDict[Tuple[int, int], DecodeGraph]" = OrderedDict()
         model = engine.model
         self.possible = all(getattr(b, "graph_safe", False) for b in model.blocks) and all(
             getattr(p, "graph_safe", False) for p in (model.embedding, model.final_norm, model.head))
@@ -142,6 +151,10 @@ class DecodeGraphs:
         graph = self.graphs.get(key)
         if graph is None:
             graph = self.graphs[key] = DecodeGraph(engine, len(entries), bucket)
+            if len(self.graphs) > MAX_GRAPHS:
+                self.graphs.popitem(last=False)        # the shape used longest ago
+        else:
+            self.graphs.move_to_end(key)
         if graph.graph is not None:
             self.replays += 1
         return graph.run(engine, entries, requests, device_tokens)
