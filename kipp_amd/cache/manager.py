@@ -109,14 +109,26 @@ class CacheManager:
         import torch
         rt = self.rt
         for g in self.groups:
-            shape = (g.pool.num_pages, g.need.num_kv_heads, self.page_size, g.need.head_dim)
+            # one page more than the pool hands out: `scratch_page`, where rows that only pad a batch write
+            shape = (g.pool.num_pages + 1, g.need.num_kv_heads, self.page_size, g.need.head_dim)
             for run in g.runs:
                 # zeroed: masked slots must hold finite values
                 g.k[run] = torch.zeros(shape, dtype=rt.cache_dtype, device=rt.device)
                 g.v[run] = torch.zeros(shape, dtype=rt.cache_dtype, device=rt.device)
         for run, need in self.state_needs.items():
             dtype = {"float32": torch.float32, "bfloat16": torch.bfloat16}[need.dtype]
-            self.states[run] = torch.zeros((self.max_requests,) + tuple(need.shape), dtype=dtype, device=rt.device)
+            # one slot more than requests: `scratch_slot`
+            self.states[run] = torch.zeros((self.max_requests + 1,) + tuple(need.shape), dtype=dtype, device=rt.device)
+
+    def scratch_page(self, group: int) -> int:
+        """A page of the group's tensors that no request ever gets: rows that only fill a batch up to a
+        recorded size keep their key and value there."""
+        return self.groups[group].pool.num_pages
+
+    @property
+    def scratch_slot(self) -> int:
+        """The state slot of such rows."""
+        return self.max_requests
 
     def view(self, run: int, reads_run: Optional[int] = None) -> Optional[KVCacheView]:
         """The cache of `run`, or of `reads_run` read-only."""

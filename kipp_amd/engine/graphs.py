@@ -11,6 +11,12 @@ A graph holds our own kernels only: nothing that reads back to the host, no
 library call, no memset node.  A model with a part that does not declare
 `graph_safe`, or a step that went to a library product, runs eagerly instead.
 
+The number of rows is rounded up to one of a few sizes (exact up to 8, then 12, 16, 24, 32,
+48, ... 256), so that a batch whose size changes from step to step still finds its
+graph: the rows that fill up bring token 0 at position 0 of a sequence of their own,
+whose block table names the cache's scratch page and whose state is the scratch slot;
+their logits are dropped.
+
 A shape is recorded when it comes a second time (recording costs the host a
 whole forward pass: under continuous batching the number of decoding requests
 often changes from step to step, and a shape seen once may never return), and
@@ -31,6 +37,16 @@ from .batch import StepBatch
 CONTEXT_BUCKET = 1024
 MAX_GRAPHS = 48              # shapes kept (each holds its recorded launches and small static buffers)
 MAX_GRAPH_ENTRIES = 256     # rows up to which every product of a step is one of our own kernels (none goes to a library)
+
+
+GRAPH_SIZES = [1, 2, 3, 4, 5, 6, 7, 8, 12, 16, 24, 32, 48, 64, 96, 128, 192, 256]
+
+
+def padded_size(n: int) -> int:
+    for size in GRAPH_SIZES:
+        if size >= n:
+            return size
+    raise ValueError(f"{n} rows are more than a recorded step takes")
 
 
 class DecodeGraph:
@@ -69,34 +85,41 @@ class DecodeGraph:
         self.copied: Optional[torch.cuda.Event] = None
         self.row_marks = [None] * n
         self.eager_runs = 0
+        self.scratch_pages = [cache.scratch_page(g) for g in range(self.groups)]
+        self.scratch_slot = cache.scratch_slot
 
     def fill(self, entries, requests, device_tokens=None) -> None:
         n, h = self.n, self.host_np
+        live = len(entries)                  # rows beyond them only fill the batch up to the recorded size
         if self.copied is not None:
             self.copied.synchronize()     # the copy of the step before has left the pinned buffer
-        h[0:n] = 0 if device_tokens is not None else [e.tokens[0] for e in entries]
-        lengths = [r.length for r in requests]
-        h[n:2 * n] = lengths
+        h[0:n] = 0
+        if device_tokens is None:
+            h[0:live] = [e.tokens[0] for e in entries]
+        h[n:n + live] = [r.length for r in requests]
+        h[n + live:2 * n] = 0
         h[2 * n:3 * n] = h[n:2 * n] + 1
-        h[3 * n:4 * n] = [r.slot for r in requests]
+        h[3 * n:3 * n + live] = [r.slot for r in requests]
+        h[3 * n + live:4 * n] = self.scratch_slot
         # a row of a block table changes only when its request got a page (or another request
         # took the row): only then is it written again, and only then are the tables copied
         changed = False
-        for i, r in enumerate(requests):
-            mark = (r.id, r.table_version)
+        for i in range(n):
+            r = requests[i] if i < live else None
+            mark = (r.id, r.table_version) if r is not None else "fills up"
             if self.row_marks[i] != mark:
                 self.row_marks[i] = mark
                 changed = True
                 at = 4 * n + i * self.max_blocks
                 for g in range(self.groups):
-                    h[at:at + self.max_blocks] = r.rows[g]
+                    h[at:at + self.max_blocks] = r.rows[g] if r is not None else self.scratch_pages[g]
                     at += n * self.max_blocks
         upto = self.var_ints if changed else 4 * n
         self.dev[:upto].copy_(self.host[:upto], non_blocking=True)
         self.copied = torch.cuda.Event()
         self.copied.record()
         if device_tokens is not None:
-            self.dev[:n].copy_(device_tokens)     # on the device, after the copy above: the tokens the host does not know
+            self.dev[:live].copy_(device_tokens)  # on the device, after the copy above: the tokens the host does not know
 
     def run(self, engine, entries, requests, device_tokens=None) -> torch.Tensor:
         self.fill(entries, requests, device_tokens)
@@ -108,7 +131,7 @@ class DecodeGraph:
             logits = engine.model.forward(self.batch, engine.cache)
             self.eager_runs += 1
             if engine.rt.library_products != before or self.eager_runs < 2:
-                return logits
+                return logits[:len(entries)]
             torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()
             # nothing may be freed on the device while the stream records: the collector stays
@@ -122,9 +145,9 @@ class DecodeGraph:
                 if was_enabled:
                     gc.enable()
             self.graph = graph
-            return logits
+            return logits[:len(entries)]
         self.graph.replay()
-        return self.logits.clone()        # the graph's own output buffer is overwritten by the next replay
+        return self.logits[:len(entries)].clone()     # the graph's own output buffer is overwritten by the next replay
 
 
 class DecodeGraphs:
@@ -147,10 +170,10 @@ class DecodeGraphs:
         cache = engine.cache
         longest = max(r.length for r in requests) + 1
         bucket = min(-(-longest // CONTEXT_BUCKET) * CONTEXT_BUCKET, max(cache.max_position, 1))
-        key = (len(entries), bucket)
+        key = (padded_size(len(entries)), bucket)
         graph = self.graphs.get(key)
         if graph is None:
-            graph = self.graphs[key] = DecodeGraph(engine, len(entries), bucket)
+            graph = self.graphs[key] = DecodeGraph(engine, key[0], bucket)
             if len(self.graphs) > MAX_GRAPHS:
                 self.graphs.popitem(last=False)        # the shape used longest ago
         else:
