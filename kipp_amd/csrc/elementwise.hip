@@ -118,6 +118,21 @@ __global__ void __launch_bounds__(256) rmsnorm_rows_kernel(float* __restrict__ x
     }
 }
 
+// out[t, :] = rows[t, :] * rsqrt(sum_p sumsq[p, t] / width + eps), sumsq in rows of `stride`: the normalized rows, for a consumer that
+// does not apply the scale itself (rows = bfloat16(x * norm weight), sumsq = partial sums of x^2).
+__global__ void __launch_bounds__(256) scale_rows_kernel(const bf16_t* __restrict__ rows, const float* __restrict__ sumsq,
+                                                         bf16_t* __restrict__ out, int width, int parts, int stride, float eps) {
+    __shared__ float scratch[16];
+    float a = 0.0f;
+    for (int p = threadIdx.x; p < parts; p += 256) a += sumsq[(size_t)p * stride + blockIdx.x];
+    a = block_sum(a, scratch);
+    const float scale = 1.0f / sqrtf(a / (float)width + eps);
+    for (int i = threadIdx.x; i < width; i += 256) {
+        const size_t at = (size_t)blockIdx.x * width + i;
+        out[at] = f32_to_bf16(bf16_to_f32(rows[at]) * scale);
+    }
+}
+
 // x += delta (the last residual add when no norm follows in the same kernel).
 template <typename TD>
 __global__ void residual_add_kernel(float* __restrict__ x, const TD* __restrict__ delta, size_t n, int parts) {
@@ -225,6 +240,15 @@ int kipp_rmsnorm(float* x, const void* delta, int delta_dtype, int parts, const 
         if (out_dtype == KIPP_BF16) launch_rmsnorm<float, bf16_t>(x, delta, weight, out, rows, width, eps, parts, stream);
         else launch_rmsnorm<float, float>(x, delta, weight, out, rows, width, eps, parts, stream);
     }
+    return KIPP_LAUNCH_CHECK();
+}
+
+int kipp_scale_rows(const void* rows, const float* sumsq, void* out, int n_rows, int width, int parts, int stride, float eps,
+                    hipStream_t stream) {
+    if (n_rows <= 0 || width <= 0) return 0;
+    if (parts <= 0 || stride < n_rows) return -1;
+    hipLaunchKernelGGL(scale_rows_kernel, dim3(n_rows), dim3(256), 0, stream, (const bf16_t*)rows, sumsq, (bf16_t*)out, width,
+                       parts, stride, eps);
     return KIPP_LAUNCH_CHECK();
 }
 

@@ -30,6 +30,16 @@
 // up rows, so a wave has 8 outputs: there are twice as many, half as heavy
 // workgroups, which fill the last round of 256 better (9,728 outputs: 4.75
 // rounds instead of 2.4, so 5 % lost instead of 26 %).
+//
+// Two optional ends spare the decode step its norm kernels (a launch costs more than the
+// norm's work there).  `AddNorm`: the product is a delta of the residual stream and is not
+// split over workgroups; the wave that holds a tile's sums adds the residual, writes the new
+// residual, its product with the next norm's weight as bfloat16, and the sum of squares of
+// every row over the tile's 16 columns.  (Split over workgroups, the last to arrive would
+// have to add the slabs: the device-wide fences that takes cost several times the kernel,
+// measured 27 instead of 6 microseconds.)  `RowScale`: X holds such rows; the kernel sums a
+// row's partial sums and multiplies the row of the product by rsqrt(sum / K + eps), which is
+// the product of the normalized row (the scale of a row commutes with the contraction).
 #include "common.h"
 
 #define WAVES 4
@@ -44,10 +54,26 @@ union Frag {
     bf16x8 v;
 };
 
+struct RowScale {               // sumsq == nullptr: none
+    const float* sumsq;         // [parts, stride]: partial sums of squares of the rows X was made from
+    int parts, stride;          // stride: 4, 8 or 16 tokens (the smallest that holds M), so that a lane loads four tokens' sums
+    float inv_width, eps;
+};
+
+struct AddNorm {                // residual == nullptr: none
+    float* residual;            // [M, N], updated in place
+    const float* norm_w;        // [N]
+    bf16_t* rows_out;           // [M, N] = bfloat16(residual * norm_w)
+    float* sumsq_out;           // [ceil(N / 16), stride], stride as in RowScale
+    int stride;
+};
+
+#define SCALE_LOADS 10          // 16-byte loads of partial sums a lane has in flight: 160 sums of 16 tokens, 640 of 4
+
 template <int MT, bool SWIGLU, int KW, int DEPTH, bool TILED>
 __global__ void __launch_bounds__(THREADS) gemm_skinny_kernel(
-    const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, float* __restrict__ Y, bf16_t* __restrict__ act,
-    int M, int N, int K) {
+    const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, float* Y, bf16_t* __restrict__ act,
+    int M, int N, int K, RowScale rs, AddNorm an) {
     constexpr bool PAIRS = SWIGLU && TILED;          // gate and up rows share a tile
     constexpr int NT = SWIGLU && !TILED ? 2 : 1;
     constexpr int TW = WAVES / KW;                   // row tiles of a workgroup
@@ -86,6 +112,46 @@ __global__ void __launch_bounds__(THREADS) gemm_skinny_kernel(
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) x_row[mt] = X + (size_t)min(16 * mt + l16, M - 1) * K + 8 * h;
 
+    // the partial sums of the rows' scales, asked for first, all at once, and added once the first
+    // weights are on their way (up to 16 rows).  A lane loads the sums of four tokens for one index;
+    // stride / 4 lanes side by side cover the tokens, the others take further indices.
+    float4 scale_part[MT == 1 ? SCALE_LOADS : 1];
+    const float* scale_src = nullptr;
+    const int lanes_per_index = MT == 1 ? rs.stride >> 2 : 1;             // 1, 2 or 4
+    const int index_step = KIPP_WAVE / lanes_per_index;
+    const int first_index = lane / lanes_per_index;
+    if (MT == 1 && rs.sumsq != nullptr) {
+        scale_src = rs.sumsq + 4 * (lane % lanes_per_index);
+#pragma unroll
+        for (int i = 0; i < SCALE_LOADS; ++i)   // beyond the last index: read the last again, dropped below
+            scale_part[i] = *(const float4*)(scale_src + (size_t)min(first_index + index_step * i, rs.parts - 1) * rs.stride);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+
+    // what the residual end adds to, asked for first as well (nobody writes these elements before that end does)
+    const bool wide = (N & 3) == 0;                  // a lane's four columns are 16 aligned bytes
+    float res[MT][4], norm_w[4];
+    if (!SWIGLU && an.residual != nullptr) {
+        const int col = min(n0 + 4 * h, wide ? N - 4 : N - 1);
+        if (wide) {
+            const float4 w4 = *(const float4*)(an.norm_w + col);
+            norm_w[0] = w4.x, norm_w[1] = w4.y, norm_w[2] = w4.z, norm_w[3] = w4.w;
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                const float4 r4 = *(const float4*)(an.residual + (size_t)min(16 * mt + l16, M - 1) * N + col);
+                res[mt][0] = r4.x, res[mt][1] = r4.y, res[mt][2] = r4.z, res[mt][3] = r4.w;
+            }
+        } else {
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int c = min(n0 + 4 * h + v, N - 1);
+                norm_w[v] = an.norm_w[c];
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) res[mt][v] = an.residual[(size_t)min(16 * mt + l16, M - 1) * N + c];
+            }
+        }
+    }
+
     f32x4 acc[NT][MT];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
@@ -109,9 +175,50 @@ __global__ void __launch_bounds__(THREADS) gemm_skinny_kernel(
                 acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u][nt].v, xf[u][mt].v, acc[nt][mt], 0, 0, 0);
     };
 
+    // the rows' scales: added up once the first weights have been asked for (asked for first, the partial sums
+    // arrive first, and the weights are on their way meanwhile).  The sum starts from a zero that exists only
+    // after those requests, or the compiler would add before it asks for the weights and the wave would wait idle;
+    // and it stands in the same block as those requests, so that the wait counts them and is not for all of them.
+    float row_scale[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) row_scale[mt] = 1.0f;
+    auto finish_scale = [&]() {
+        if (MT == 1 && scale_src != nullptr) {
+            float t[4];
+            asm volatile("v_mov_b32 %0, 0" : "=v"(t[0]) : : "memory");
+            t[1] = t[2] = t[3] = t[0];
+#pragma unroll
+            for (int i = 0; i < SCALE_LOADS; ++i) {
+                const bool ok = first_index + index_step * i < rs.parts;
+                t[0] += ok ? scale_part[i].x : 0.0f;
+                t[1] += ok ? scale_part[i].y : 0.0f;
+                t[2] += ok ? scale_part[i].z : 0.0f;
+                t[3] += ok ? scale_part[i].w : 0.0f;
+            }
+            for (int p = first_index + index_step * SCALE_LOADS; p < rs.parts; p += index_step) {   // wider rows: the rest one by one
+                const float4 more = *(const float4*)(scale_src + (size_t)p * rs.stride);
+                t[0] += more.x, t[1] += more.y, t[2] += more.z, t[3] += more.w;
+            }
+            // the lanes that hold the same tokens, added pairwise: in the end every lane has its four tokens' totals
+            for (int off = lanes_per_index; off < KIPP_WAVE; off <<= 1)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) t[e] += __shfl_xor(t[e], off, KIPP_WAVE);
+            // token l % 16 sits in lane (l % 16) / 4 (any lane of that remainder would do), element (l % 16) % 4
+            const int from = min(l16 >> 2, lanes_per_index - 1);
+            float mine = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float got = __shfl(t[e], from, KIPP_WAVE);
+                if ((l16 & 3) == e) mine = got;
+            }
+            row_scale[0] = 1.0f / sqrtf(mine * rs.inv_width + rs.eps);
+        }
+    };
+    if (g_begin >= g_end) finish_scale();
     if (g_begin < g_end) {
 #pragma unroll
         for (int u = 0; u < DEPTH; ++u) fetch(u, g_begin * DEPTH + u);
+        finish_scale();
         for (int g = g_begin; g + 1 < g_end; ++g) {      // while step s is multiplied, step s + DEPTH is fetched
 #pragma unroll
             for (int u = 0; u < DEPTH; ++u) {
@@ -148,6 +255,7 @@ __global__ void __launch_bounds__(THREADS) gemm_skinny_kernel(
     // tokens beyond M and rows beyond N were computed from clamped addresses and are dropped below
 
     float sum[NT][MT][4];
+    bool writer = true;                               // this wave holds finished sums
     if (KW > 1) {
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt)
@@ -156,7 +264,7 @@ __global__ void __launch_bounds__(THREADS) gemm_skinny_kernel(
 #pragma unroll
                 for (int v = 0; v < 4; ++v) red[wave][nt][mt][lane * 4 + v] = acc[nt][mt][v];
         __syncthreads();
-        if (slice != 0) return;
+        writer = slice == 0;
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
@@ -164,9 +272,11 @@ __global__ void __launch_bounds__(THREADS) gemm_skinny_kernel(
 #pragma unroll
                 for (int v = 0; v < 4; ++v) {
                     float a = 0.0f;
+                    if (writer) {
 #pragma unroll
-                    for (int w = 0; w < KW; ++w) a += red[tile_in_wg * KW + w][nt][mt][lane * 4 + v];
-                    sum[nt][mt][v] = a;
+                        for (int w = 0; w < KW; ++w) a += red[tile_in_wg * KW + w][nt][mt][lane * 4 + v];
+                    }
+                    sum[nt][mt][v] = a * row_scale[mt];
                 }
     } else {
 #pragma unroll
@@ -174,9 +284,46 @@ __global__ void __launch_bounds__(THREADS) gemm_skinny_kernel(
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-                for (int v = 0; v < 4; ++v) sum[nt][mt][v] = acc[nt][mt][v];
+                for (int v = 0; v < 4; ++v) sum[nt][mt][v] = acc[nt][mt][v] * row_scale[mt];
     }
     const int n = n0 + 4 * h;
+    if (!SWIGLU && an.residual != nullptr) {
+        // ---- the product is a delta of the residual stream (never split over workgroups: the launcher sees to it)
+        if (!writer) return;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const int token = 16 * mt + l16;
+            float x[4], ss = 0.0f;
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                x[v] = res[mt][v] + sum[0][mt][v];
+                if (token < M && n + v < N) ss = fmaf(x[v], x[v], ss);
+            }
+            if (token < M && wide && n + 3 < N) {
+                const size_t at = (size_t)token * N + n;
+                *(float4*)(an.residual + at) = make_float4(x[0], x[1], x[2], x[3]);
+                uint2 packed;
+                packed.x = (uint32_t)f32_to_bf16(x[0] * norm_w[0]) | ((uint32_t)f32_to_bf16(x[1] * norm_w[1]) << 16);
+                packed.y = (uint32_t)f32_to_bf16(x[2] * norm_w[2]) | ((uint32_t)f32_to_bf16(x[3] * norm_w[3]) << 16);
+                *(uint2*)(an.rows_out + at) = packed;
+            } else if (token < M) {
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    if (n + v < N) {
+                        const size_t at = (size_t)token * N + n + v;
+                        an.residual[at] = x[v];
+                        an.rows_out[at] = f32_to_bf16(x[v] * norm_w[v]);
+                    }
+                }
+            }
+            ss += __shfl_xor(ss, 16, KIPP_WAVE);      // the four lane groups hold a tile's 16 columns of a token
+            ss += __shfl_xor(ss, 32, KIPP_WAVE);
+            // tokens beyond M up to the stride get a zero: the consumer loads them with the others
+            if (h == 0 && token < an.stride && n0 < N) an.sumsq_out[(size_t)(n0 >> 4) * an.stride + token] = token < M ? ss : 0.0f;
+        }
+        return;
+    }
+    if (!writer) return;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
         const int token = 16 * mt + l16;
@@ -214,14 +361,16 @@ __global__ void __launch_bounds__(THREADS) gemm_skinny_kernel(
 
 template <bool SWIGLU, int KW, bool TILED>
 static int launch_kw(const bf16_t* X, const bf16_t* W, float* Y, bf16_t* act, int M, int N, int K, int parts,
-                     hipStream_t stream) {
+                     RowScale rs, AddNorm an, hipStream_t stream) {
     const int inner = SWIGLU ? N / 2 : N;
     const int tiles = SWIGLU && TILED ? (inner + 7) / 8 : (inner + 15) / 16;
     constexpr int TW = WAVES / KW;
     dim3 grid((tiles + TW - 1) / TW, parts), block(THREADS);
+    if (an.residual != nullptr && parts != 1) return -1;
+    if (rs.sumsq != nullptr && M > 16) return -1;
     const int mt = (M + 15) / 16;
 #define KIPP_SK(MT, D) \
-    hipLaunchKernelGGL((gemm_skinny_kernel<MT, SWIGLU, KW, D, TILED>), grid, block, 0, stream, X, W, Y, act, M, N, K)
+    hipLaunchKernelGGL((gemm_skinny_kernel<MT, SWIGLU, KW, D, TILED>), grid, block, 0, stream, X, W, Y, act, M, N, K, rs, an)
     switch (mt) {
         case 1: KIPP_SK(1, 8); break;
         case 2: KIPP_SK(2, 8); break;
@@ -235,11 +384,11 @@ static int launch_kw(const bf16_t* X, const bf16_t* W, float* Y, bf16_t* act, in
 
 template <bool SWIGLU>
 static int launch(const bf16_t* X, const bf16_t* W, float* Y, bf16_t* act, int M, int N, int K, int parts, int kw,
-                  int tiled, hipStream_t stream) {
+                  int tiled, RowScale rs, AddNorm an, hipStream_t stream) {
     if (tiled && (K & 31)) return -1;
 #define KIPP_KW(KW)                                                                          \
-    return tiled ? launch_kw<SWIGLU, KW, true>(X, W, Y, act, M, N, K, parts, stream)         \
-                 : launch_kw<SWIGLU, KW, false>(X, W, Y, act, M, N, K, parts, stream)
+    return tiled ? launch_kw<SWIGLU, KW, true>(X, W, Y, act, M, N, K, parts, rs, an, stream)         \
+                 : launch_kw<SWIGLU, KW, false>(X, W, Y, act, M, N, K, parts, rs, an, stream)
     switch (kw) {
         case 1: KIPP_KW(1);
         case 2: KIPP_KW(2);
@@ -286,27 +435,53 @@ int kipp_gemm_skinny_parts(int N, int K, int max_parts) {
     return parts;
 }
 
+// Tokens a row of partial sums has room for: the smallest of 4, 8, 16 that holds M (0: more than 16 rows).
+static int sumsq_stride(int M) { return M <= 4 ? 4 : (M <= 8 ? 8 : (M <= 16 ? 16 : 0)); }
+
+static RowScale row_scale_of(const float* sumsq, int sumsq_parts, int M, int K, float eps) {
+    RowScale rs = {sumsq, sumsq_parts, sumsq != nullptr ? sumsq_stride(M) : 4, 1.0f / (float)K, eps};
+    return rs;
+}
+
+// Width of a row of partial sums for M rows (0: more rows than the fused ends take).
+int kipp_gemm_skinny_sumsq_stride(int M) { return sumsq_stride(M); }
+
 // Y: float32 [parts, M, N] with parts = kipp_gemm_skinny_parts(N, K, max_parts).
 // K must be a multiple of 8 (16-byte loads), M <= 64.  `tiled`: W is in the
 // streaming layout (K a multiple of 32), else [N, K] rows.
+// `sumsq` [sumsq_parts, kipp_gemm_skinny_sumsq_stride(M)] (or null; M <= 16 then): every row of the product is multiplied by
+// rsqrt(sum of the row's sumsq / K + eps).
+// `residual` [M, N] (or null): the product is added to it in place (Y is not written and there is
+// one part), `rows_out` [M, N] = bfloat16(residual * norm_w) and `sumsq_out`
+// [ceil(N / 16), kipp_gemm_skinny_sumsq_stride(M)] = the new residual's sums of squares over each 16 columns
+// (M <= 16 with a residual).
 int kipp_gemm_skinny(const void* X, const void* W, float* Y, int M, int N, int K, int max_parts, int tiled,
-                     hipStream_t stream) {
+                     const float* sumsq, int sumsq_parts, float eps, float* residual, const float* norm_w, void* rows_out,
+                     float* sumsq_out, hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
     if (M > 64 || K <= 0 || (K & 7) || max_parts <= 0) return -1;
+    if (sumsq != nullptr && (sumsq_parts <= 0 || M > 16)) return -1;
+    if (residual != nullptr && (norm_w == nullptr || rows_out == nullptr || sumsq_out == nullptr || M > 16)) return -1;
     int kw, parts;
-    plan((N + 15) / 16, K, max_parts, &kw, &parts);
-    return launch<false>((const bf16_t*)X, (const bf16_t*)W, Y, nullptr, M, N, K, parts, kw, tiled, stream);
+    plan((N + 15) / 16, K, residual != nullptr ? 1 : max_parts, &kw, &parts);
+    AddNorm an = {residual, norm_w, (bf16_t*)rows_out, sumsq_out, sumsq_stride(M)};
+    return launch<false>((const bf16_t*)X, (const bf16_t*)W, Y, nullptr, M, N, K, parts, kw, tiled,
+                         row_scale_of(sumsq, sumsq_parts, M, K, eps), an, stream);
 }
 
 // W: [2 I, K] = [gate; up] (tiled: tiles of 8 gate rows over the 8 matching up rows); act: bfloat16 [M, I].
 // The contraction is cut the same way from both layouts, so both give the same bits.
+// `sumsq`, `sumsq_parts`, `eps`: as above.
 int kipp_gemm_skinny_swiglu(const void* X, const void* W, void* act, int M, int two_inner, int K, int tiled,
-                            hipStream_t stream) {
+                            const float* sumsq, int sumsq_parts, float eps, hipStream_t stream) {
     if (M <= 0 || two_inner <= 0) return 0;
     if (M > 64 || K <= 0 || (K & 7) || (two_inner & 1)) return -1;
+    if (sumsq != nullptr && (sumsq_parts <= 0 || M > 16)) return -1;
     int kw, parts;
     plan((two_inner / 2 + 7) / 8, K, 1, &kw, &parts);
-    return launch<true>((const bf16_t*)X, (const bf16_t*)W, nullptr, (bf16_t*)act, M, two_inner, K, 1, kw, tiled, stream);
+    AddNorm none = {nullptr, nullptr, nullptr, nullptr, 4};
+    return launch<true>((const bf16_t*)X, (const bf16_t*)W, nullptr, (bf16_t*)act, M, two_inner, K, 1, kw, tiled,
+                        row_scale_of(sumsq, sumsq_parts, M, K, eps), none, stream);
 }
 
 }  // extern "C"

@@ -466,11 +466,38 @@ def _tiles_ok(tiles, n: int, k: int, what: str) -> int:
     return 1
 
 
-def gemm_skinny(x: torch.Tensor, w: torch.Tensor, max_parts: int = 1, tiles: torch.Tensor = None) -> torch.Tensor:
+def _row_scale_args(row_scale, m: int, what: str):
+    """(sumsq pointer, parts, eps) of `row_scale` = (sumsq [parts, sumsq_stride(M)] float32, eps), or nulls."""
+    if row_scale is None:
+        return None, 0, 0.0
+    sumsq, eps = row_scale
+    _dev(sumsq)
+    _need(m <= 16 and sumsq.dtype == torch.float32 and sumsq.dim() == 2 and sumsq.shape[1] == sumsq_stride(m)
+          and sumsq.shape[0] > 0 and sumsq.is_contiguous(),
+          f"{what}: row_scale is (float32 [parts, sumsq_stride(M)], eps), for at most 16 rows")
+    return _ptr(sumsq), sumsq.shape[0], float(eps)
+
+
+def sumsq_stride(m: int) -> int:
+    """Width of a row of partial sums for m rows: 4, 8 or 16, the smallest that holds them
+    (the consumer loads four tokens' sums at once); 0 for more than 16 rows."""
+    return 4 if m <= 4 else (8 if m <= 8 else (16 if m <= 16 else 0))
+
+
+def gemm_skinny(x: torch.Tensor, w: torch.Tensor, max_parts: int = 1, tiles: torch.Tensor = None,
+                row_scale=None, add_norm=None):
     """float32 [parts, M, N] whose sum over parts is x . w^T, for M <= 64 rows of
     bfloat16 x against bfloat16 w [N, K].  parts <= max_parts is chosen from the
     shape (1 when the weight has many rows).  With `tiles` (tile_weight(w)) the
-    weight is streamed from that layout."""
+    weight is streamed from that layout.
+
+    `row_scale` = (sumsq [P, sumsq_stride(M)], eps), M <= 16: row t of the product is
+    multiplied by rsqrt(sum(sumsq[:, t]) / K + eps), i.e. x holds rows of an RMS
+    norm that still lack their scale.
+    `add_norm` = (residual float32 [M, N], norm_weight float32 [N]), M <= 16: the product
+    (in one part) is added to `residual` in place by the kernel itself and the
+    call returns (rows, sumsq) instead: rows = bfloat16(residual * norm_weight)
+    and sumsq [ceil(N / 16), sumsq_stride(M)], what `row_scale` of the next product takes."""
     _dev(x, w)
     m, k = x.shape
     n = w.shape[0]
@@ -478,11 +505,38 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, max_parts: int = 1, tiles: tor
     _need(w.shape == (n, k), "gemm_skinny: shapes do not match")
     _need(gemm_skinny_ok(m, k), "gemm_skinny: at most 64 rows, K a multiple of 8 and at least 32")
     lib = build.library("gemm_skinny")
-    parts = lib.kipp_gemm_skinny_parts(n, k, int(max_parts))
-    out = torch.empty((parts, m, n), dtype=torch.float32, device=x.device)
     tiled = _tiles_ok(tiles, n, k, "gemm_skinny")
-    fn = _fn("gemm_skinny", "kipp_gemm_skinny", [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr])
-    _check(fn(_ptr(x), _ptr(tiles if tiled else w), _ptr(out), m, n, k, int(max_parts), tiled, _stream()), "gemm_skinny")
+    sumsq, sumsq_parts, eps = _row_scale_args(row_scale, m, "gemm_skinny")
+    residual = norm_w = rows = sumsq_out = out = None
+    if add_norm is None:
+        parts = lib.kipp_gemm_skinny_parts(n, k, int(max_parts))
+        out = torch.empty((parts, m, n), dtype=torch.float32, device=x.device)
+    else:
+        residual, norm_w = add_norm
+        _dev(residual, norm_w)
+        _need(m <= 16 and residual.dtype == torch.float32 and residual.shape == (m, n) and residual.is_contiguous(),
+              "gemm_skinny: the residual is float32 [M, N], at most 16 rows")
+        _need(norm_w.dtype == torch.float32 and norm_w.numel() == n, "gemm_skinny: the norm weight is float32 [N]")
+        rows = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
+        sumsq_out = torch.empty(((n + 15) // 16, sumsq_stride(m)), dtype=torch.float32, device=x.device)
+    fn = _fn("gemm_skinny", "kipp_gemm_skinny",
+             [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_int, _c_float,
+              _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr])
+    _check(fn(_ptr(x), _ptr(tiles if tiled else w), _ptr(out), m, n, k, int(max_parts), tiled, sumsq, sumsq_parts, eps,
+              _ptr(residual), _ptr(norm_w), _ptr(rows), _ptr(sumsq_out), _stream()), "gemm_skinny")
+    return out if add_norm is None else (rows, sumsq_out)
+
+
+def scale_rows(rows: torch.Tensor, sumsq: torch.Tensor, eps: float, out: torch.Tensor) -> torch.Tensor:
+    """out[t] = rows[t] * rsqrt(sum(sumsq[:, t]) / width + eps), bfloat16: the rows of an RMS norm
+    from what `gemm_skinny(..., add_norm=...)` returns, for a consumer that does not take `row_scale`."""
+    _dev(rows, sumsq, out)
+    m, width = rows.shape
+    _need(rows.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and out.shape == rows.shape
+          and sumsq.dtype == torch.float32 and sumsq.dim() == 2 and sumsq.shape[1] >= m and sumsq.is_contiguous(),
+          "scale_rows: shapes or types differ")
+    fn = _fn("elementwise", "kipp_scale_rows", [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_float, _c_ptr])
+    _check(fn(_ptr(rows), _ptr(sumsq), _ptr(out), m, width, sumsq.shape[0], sumsq.shape[1], float(eps), _stream()), "scale_rows")
     return out
 
 
@@ -511,9 +565,11 @@ def gemm_rows(x: torch.Tensor, w: torch.Tensor, max_parts: int = 1, tiles: torch
     return out
 
 
-def gemm_skinny_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor, tiles: torch.Tensor = None) -> torch.Tensor:
+def gemm_skinny_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor, tiles: torch.Tensor = None,
+                       row_scale=None) -> torch.Tensor:
     """out[M, I] (bfloat16) = silu(x . w_gate^T) * (x . w_up^T), w_gate_up = [gate; up] of [2 I, K];
-    `tiles` = tile_weight_pairs(w_gate_up).  The same bits from both layouts."""
+    `tiles` = tile_weight_pairs(w_gate_up).  The same bits from both layouts.
+    `row_scale`: as in `gemm_skinny` (both products are scaled before the activation)."""
     _dev(x, w_gate_up, out)
     m, k = x.shape
     two_inner = w_gate_up.shape[0]
@@ -523,8 +579,11 @@ def gemm_skinny_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tens
           "gemm_skinny_swiglu: shapes do not match")
     _need(gemm_skinny_ok(m, k), "gemm_skinny_swiglu: at most 64 rows, K a multiple of 8 and at least 32")
     tiled = _tiles_ok(tiles, pairs_width(two_inner // 2), k, "gemm_skinny_swiglu")
-    fn = _fn("gemm_skinny", "kipp_gemm_skinny_swiglu", [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr])
-    _check(fn(_ptr(x), _ptr(tiles if tiled else w_gate_up), _ptr(out), m, two_inner, k, tiled, _stream()), "gemm_skinny_swiglu")
+    sumsq, sumsq_parts, eps = _row_scale_args(row_scale, m, "gemm_skinny_swiglu")
+    fn = _fn("gemm_skinny", "kipp_gemm_skinny_swiglu",
+             [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_int, _c_float, _c_ptr])
+    _check(fn(_ptr(x), _ptr(tiles if tiled else w_gate_up), _ptr(out), m, two_inner, k, tiled, sumsq, sumsq_parts, eps,
+              _stream()), "gemm_skinny_swiglu")
     return out
 
 

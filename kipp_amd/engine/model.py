@@ -94,6 +94,8 @@ class Model:
         if batch.n_want == 0:
             return None
         ops = self.rt.ops
+        if pending is not None and not (batch.want_every_row and getattr(self.final_norm, "fuses_products", False)):
+            pending = self.rt.settle(pending)
         if batch.want_every_row:
             # every row in order (a step of single tokens): no gather, and the last delta is added inside the norm
             normed = (self.final_norm.forward(x, self.rt.act_dtype) if pending is None

@@ -7,7 +7,13 @@ Interface of a block:
         x        float32 [tokens, hidden], the residual stream (updated in place)
         pending  a delta not yet added to x (or None); the block adds it inside
                  its first norm and hands its own last delta on the same way,
-                 so that residual add and norm are one kernel
+                 so that residual add and norm are one kernel.  A delta may
+                 be a product that the runtime has not launched yet
+                 (`Runtime.linear(..., defer=True)`), and a norm may leave its
+                 scale to the product that follows (`ScaledRows`): the block
+                 settles either for a part that does not declare it takes it
+                 (`fuses_products` of a norm, `takes_scaled_rows` of a mixer
+                 or feed-forward).
 """
 from __future__ import annotations
 
@@ -30,7 +36,16 @@ class PreNormBlock:
     def forward(self, x, pending, batch, cache, state):
         act = self.rt.act_dtype
         norm1, norm2 = self.parts["mixer_norm"], self.parts["ffn_norm"]
+        rt, ffn = self.rt, self.parts["ffn"]
+        if pending is not None and not getattr(norm1, "fuses_products", False):
+            pending = rt.settle(pending)
         h = norm1.forward(x, act) if pending is None else norm1.add_forward(x, pending, act)
+        if not getattr(self.mixer, "takes_scaled_rows", False):
+            h = rt.rows_of(h)
         delta = self.mixer.forward(h, batch, cache, state)
+        if not getattr(norm2, "fuses_products", False):
+            delta = rt.settle(delta)
         h = norm2.add_forward(x, delta, act)
-        return x, self.parts["ffn"].forward(h, batch)
+        if not getattr(ffn, "takes_scaled_rows", False):
+            h = rt.rows_of(h)
+        return x, ffn.forward(h, batch)

@@ -3,7 +3,10 @@
     params(spec) -> {local name: ParamSpec}
     load(tensors)
     forward(x, batch) -> delta      x [tokens, hidden] activation type,
-                                    delta float32 [tokens, hidden]
+                                    delta float32 [tokens, hidden] (or slabs of it,
+                                    or a product deferred by `Runtime.linear`)
+
+A feed-forward with `takes_scaled_rows = True` also takes `ScaledRows` for x.
 """
 from __future__ import annotations
 
@@ -17,6 +20,7 @@ class GatedMLP:
     """delta = W_down (silu(W_gate x) * (W_up x))  (/root/reference/src/kipp.c:2633-2653)."""
 
     graph_safe = True   # forward launches kernels only: no host reads, no data-dependent launches
+    takes_scaled_rows = True
 
     def __init__(self, spec, runtime):
         self.spec = spec
@@ -45,11 +49,15 @@ class GatedMLP:
         w = self.w_gate_up
         ours = w.dtype == x.dtype == torch.bfloat16 and rt.ops.gemm_rows_ok(rows, x.shape[1])
         if ours and rows <= rt.ops.SKINNY_BEST_ROWS:
-            # both products and the activation in one kernel
-            rt.ops.gemm_skinny_swiglu(x, w.rows, act, tiles=w.tiles)
-        elif ours and w.pairs:
+            # both products and the activation in one kernel (and the norm's scale, if it was left to us)
+            scaled = hasattr(x, "sumsq")
+            rt.ops.gemm_skinny_swiglu(x.rows if scaled else x, w.rows, act, tiles=w.tiles,
+                                      row_scale=(x.sumsq, x.eps) if scaled else None)
+            return rt.linear(act, self.w_down, slabs=True, defer=True)
+        x = rt.rows_of(x)
+        if ours and w.pairs:
             # streamed from the paired tiles: the columns come out gate tile by gate tile
             rt.ops.swiglu(rt.ops.gemm_rows(x, w.rows, max_parts=12, tiles=w.tiles, pairs=True), act, pairs=True)
         else:
             rt.ops.swiglu(rt.linear(x, w, slabs=True, low_precision_out=True), act)
-        return rt.linear(act, self.w_down, slabs=True)
+        return rt.linear(act, self.w_down, slabs=True, defer=True)

@@ -10,6 +10,10 @@
         cache  the KVCacheView of this run (None if cache_need() is None)
         state  tensor [slots, ...] of this run (None if state_need() is None)
         delta  float32 [tokens, hidden], added to the residual by the block
+               (or slabs of it, or a product deferred by `Runtime.linear`)
+
+A mixer with `takes_scaled_rows = True` passes x on to `Runtime.linear` only,
+which also takes rows whose norm scale is still to be applied.
 """
 from __future__ import annotations
 
@@ -31,6 +35,7 @@ class Attention:
     h // (n_q / n_kv)."""
 
     graph_safe = True   # forward launches kernels only: no host reads, no data-dependent launches
+    takes_scaled_rows = True
 
     def __init__(self, spec, runtime):
         self.spec = spec
@@ -99,7 +104,7 @@ class Attention:
                                           self.q_norm, self.k_norm, eps, inv_freq, rotary_dim, cache.writable,
                                           self.scale, s.window or 0, batch.max_decode_ctx, self._workspace(batch),
                                           angles=angles)
-            return rt.linear(out, self.w_o, slabs=True)
+            return rt.linear(out, self.w_o, slabs=True, defer=True)
         q = rt.ops.qk_norm_rope_kv_write(
             qkv, rt.empty((n, s.q_dim), rt.act_dtype), cache.k, cache.v,
             batch.positions, batch.seq_of_token, table, s.num_heads, s.num_kv_heads, s.head_dim,
@@ -118,7 +123,7 @@ class Attention:
             # the float32 path, and geometries the matrix-core kernels refuse (groups above 16, odd page sizes)
             rt.ops.paged_attention_generic(q, cache.k, cache.v, out, batch.positions, batch.seq_of_token, table,
                                            s.num_heads, s.num_kv_heads, s.head_dim, self.scale, s.window or 0)
-        return rt.linear(out, self.w_o, slabs=True)
+        return rt.linear(out, self.w_o, slabs=True, defer=True)
 
     def _workspace(self, batch):
         """Partial results of the split decode kernel, kept while they are large enough."""

@@ -4,6 +4,11 @@
     load(tensors)                       tensors by local name, already on the device
     forward(x, out_dtype) -> y          x float32 [rows, width]
     add_forward(x, delta, out_dtype)    x += delta in place, then y = norm(x)
+
+A norm with `fuses_products = True` also takes a delta that `Runtime.linear(...,
+defer=True)` has not launched yet and may return `ScaledRows` (its rows without
+their scale, which the product that follows applies); blocks settle both for
+parts that do not say they take them.
 """
 from __future__ import annotations
 
@@ -15,6 +20,7 @@ class RMSNorm:
     """y = x * rsqrt(mean(x^2) + eps) * w  (/root/reference/src/kipp.c:2221-2231)."""
 
     graph_safe = True   # forward launches kernels only: no host reads, no data-dependent launches
+    fuses_products = True
 
     def __init__(self, spec, runtime):
         self.spec = spec
@@ -37,4 +43,9 @@ class RMSNorm:
         return self.rt.ops.rmsnorm(x, self.weight, self.spec.eps, self.rt.empty(x.shape, out_dtype))
 
     def add_forward(self, x, delta, out_dtype):
+        if not hasattr(delta, "shape"):       # a product not launched yet: add and norm ride on it where they can
+            fused = self.rt.product_add_norm(delta, x, self.weight, self.spec.eps) if out_dtype == self.rt.act_dtype else None
+            if fused is not None:
+                return fused
+            delta = delta.run()
         return self.rt.ops.rmsnorm(x, self.weight, self.spec.eps, self.rt.empty(x.shape, out_dtype), delta=delta)

@@ -50,6 +50,40 @@ class Weight:
         return self.rows.dtype
 
 
+class ScaledRows:
+    """Rows of an RMS norm that still lack their scale: `rows` = bfloat16(x * norm
+    weight) and `sumsq` [P, 4 | 8 | 16], partial sums of x^2 whose total gives row t's scale
+    rsqrt(sum(sumsq[:, t]) / width + eps).  A row's scale commutes with a product over
+    the row, so `Runtime.linear` applies it to the product's rows; any other
+    consumer asks `Runtime.rows_of` for the finished rows."""
+    __slots__ = ("rows", "sumsq", "eps")
+
+    def __init__(self, rows: torch.Tensor, sumsq: torch.Tensor, eps: float):
+        self.rows, self.sumsq, self.eps = rows, sumsq, eps
+
+    @property
+    def shape(self):
+        return self.rows.shape
+
+    @property
+    def dtype(self):
+        return self.rows.dtype
+
+
+class Deferred:
+    """A product `x . w^T` that `Runtime.linear(..., defer=True)` has not launched
+    yet: the delta of a mixer or a feed-forward, which a norm that follows may
+    launch together with the residual add (`Runtime.product_add_norm`); `run()`
+    launches it as it is."""
+    __slots__ = ("rt", "x", "w", "slabs")
+
+    def __init__(self, rt, x, w, slabs):
+        self.rt, self.x, self.w, self.slabs = rt, x, w, slabs
+
+    def run(self) -> torch.Tensor:
+        return self.rt.linear(self.x, self.w, slabs=self.slabs)
+
+
 class Runtime:
     def __init__(self, dtype: str = "bfloat16", device: str = "cuda:0", stream_layout: bool = True):
         if dtype not in DTYPES:
@@ -64,6 +98,7 @@ class Runtime:
         self.stream_layout = stream_layout   # keep a second copy of bfloat16 matrices in the streaming layout
         self._mm_out_f32 = None
         self.library_products = 0   # calls that went to the library (they stay out of HIP graphs)
+        self.fuse_norms = True      # few rows: residual add and norm ride on the products around them
         torch.backends.cuda.matmul.allow_tf32 = False
 
     # -- placement -----------------------------------------------------------
@@ -90,14 +125,51 @@ class Runtime:
         return Weight(w, tiles, gate_up and tiles is not None)
 
     # -- matrix product ------------------------------------------------------
-    def linear(self, x: torch.Tensor, w, slabs: bool = False, low_precision_out: bool = False) -> torch.Tensor:
+    def _few_rows(self, m: int, k: int, w) -> bool:
+        """The product goes to the few-rows kernel (the one with the fused ends, which take up to 16 rows)."""
+        return w.dtype == torch.bfloat16 and self.ops.gemm_rows_ok(m, k) and m <= min(self.ops.SKINNY_BEST_ROWS, 16)
+
+    def settle(self, delta):
+        """The tensor of a delta, launched now if it was deferred."""
+        return delta.run() if isinstance(delta, Deferred) else delta
+
+    def rows_of(self, h):
+        """The tensor of norm output, scaled now if the scale was left to a product."""
+        if not isinstance(h, ScaledRows):
+            return h
+        return self.ops.scale_rows(h.rows, h.sumsq, h.eps, self.empty(h.rows.shape, torch.bfloat16))
+
+    def product_add_norm(self, delta: Deferred, x: torch.Tensor, norm_weight: torch.Tensor, eps: float):
+        """x += delta's product, in the product's own kernel, which also prepares the
+        RMS norm of the new x: returns ScaledRows (None if this product has no such
+        kernel: the caller then runs it and norms as usual)."""
+        w = delta.w
+        rows, k = delta.x.shape
+        if not (self.fuse_norms and isinstance(w, Weight) and not w.pairs and delta.x.dtype == torch.bfloat16
+                and self._few_rows(rows, k, w) and x.dtype == torch.float32 and x.is_contiguous()
+                and norm_weight.dtype == torch.float32):
+            return None
+        rows_out, sumsq = self.ops.gemm_skinny(delta.x, w.rows, tiles=w.tiles, add_norm=(x, norm_weight))
+        return ScaledRows(rows_out, sumsq, eps)
+
+    def linear(self, x, w, slabs: bool = False, low_precision_out: bool = False, defer: bool = False):
         """float32 [M, N] = x [M, K] . w [N, K]^T.  With `slabs` the result may come
         as [parts, M, N] whose sum over parts is the product (few rows against a
         weight with few output rows: the contraction is split over workgroups and
         the consumer adds the slabs in order); an integer is the most slabs the
         consumer takes.  With `low_precision_out` a large
         bfloat16 product may be returned in bfloat16 (for a consumer that rounds to
-        bfloat16 anyway and is bound by reading it)."""
+        bfloat16 anyway and is bound by reading it).  `x` may be ScaledRows.  With
+        `defer` the product may come back as a `Deferred` (for a delta of the
+        residual stream, which the next norm launches or `settle` does)."""
+        if defer and self.fuse_norms and not isinstance(x, ScaledRows) and self._few_rows(x.shape[0], x.shape[1], w):
+            return Deferred(self, x, w, slabs)
+        row_scale = None
+        if isinstance(x, ScaledRows):
+            if self._few_rows(x.shape[0], x.shape[1], w):
+                row_scale, x = (x.sumsq, x.eps), x.rows
+            else:
+                x = self.rows_of(x)
         tiles = None
         if isinstance(w, Weight):
             # paired tiles give the columns in another order: only the feed-forward asks for that
@@ -114,7 +186,7 @@ class Runtime:
             # up to 256 rows: our own kernels stream the weight once
             most = 0 if slabs is False else (None if slabs is True else int(slabs))
             if m <= self.ops.SKINNY_BEST_ROWS:
-                y = self.ops.gemm_skinny(x, w, max_parts=1 if most == 0 else (most or 8), tiles=tiles)
+                y = self.ops.gemm_skinny(x, w, max_parts=1 if most == 0 else (most or 8), tiles=tiles, row_scale=row_scale)
             else:
                 y = self.ops.gemm_rows(x, w, max_parts=1 if most == 0 else (most or 12), tiles=tiles)
             return y if y.shape[0] > 1 else y[0]

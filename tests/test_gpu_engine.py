@@ -78,3 +78,37 @@ def test_without_the_streaming_layout(model_folders, tiny_configs, key):
         got = H.replay(engine, requests, steps)
         for rid, toks in requests.items():
             H.assert_close(got[rid], H.plain_logits(folder, toks), H.NMSE_BF16, f"{key}/rows only/{rid}")
+
+
+@pytest.mark.parametrize("key", ["a", "b"])
+def test_norms_in_kernels_of_their_own(model_folders, tiny_configs, key):
+    """With few rows the residual add and the norm ride on the products around them; `fuse_norms =
+    False` gives every norm its own kernel again.  Both against the plain implementation, and the
+    fused engine launches fewer kernels' worth of norms: it never calls the norm kernel with a delta."""
+    from kipp_amd.engine import Engine
+    from kipp_amd.engine.model import load_model
+    from kipp_amd.runtime import Runtime
+    cfg = tiny_configs[key]
+    requests = _requests(key, cfg, seed=4)
+    folder = model_folders[(key, "bfloat16")]
+    steps = H.tail_one_by_one(requests)
+    for fuse in (False, True):
+        rt = Runtime("bfloat16")
+        rt.fuse_norms = fuse
+        calls = {"delta": 0, "plain": 0}
+        inner = rt.ops.rmsnorm
+
+        class Counting:
+            def __getattr__(self, name, ops=rt.ops):
+                return getattr(ops, name)
+
+            @staticmethod
+            def rmsnorm(x, weight, eps, out, delta=None):
+                calls["delta" if delta is not None and x.shape[0] <= 8 else "plain"] += 1
+                return inner(x, weight, eps, out, delta=delta)
+        rt.ops = Counting()
+        engine = Engine(load_model(folder, rt), page_size=PAGE[key], max_tokens=512, share_prefixes=False, use_graphs=False)
+        got = H.replay(engine, requests, steps)
+        for rid, toks in requests.items():
+            H.assert_close(got[rid], H.plain_logits(folder, toks), H.NMSE_BF16, f"{key}/fused norms {fuse}/{rid}")
+        assert (calls["delta"] == 0) == fuse, calls

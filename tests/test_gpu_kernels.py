@@ -608,6 +608,49 @@ def test_gemm_skinny(m, n, k, max_parts):
                            ops.gemm_skinny(x.to(DEV), wd, max_parts))
 
 
+@pytest.mark.parametrize("m", [1, 3, 4, 5, 8, 11, 16])
+@pytest.mark.parametrize("n,k,tiled", [(16, 32, True), (77, 80, False), (2560, 4096, True), (2560, 9728, True),
+                                       (100, 2560, False), (200, 4096, True), (36, 512, True), (5120, 1024, True), (12288, 256, True)])
+def test_gemm_skinny_adds_the_residual_and_prepares_the_norm(m, n, k, tiled):
+    """The product's own kernel adds it to the residual and writes the rows and partial sums that the
+    next product scales its rows by: the chain residual add -> RMS norm -> product without a norm
+    kernel (12,288 columns: more partial sums than a lane asks for at once)."""
+    ops = _ops()
+    rng = np.random.default_rng(m + n + k)
+    x = torch.tensor(rng.normal(size=(m, k)) / math.sqrt(k), dtype=torch.bfloat16)
+    w = torch.tensor(rng.normal(size=(n, k)), dtype=torch.bfloat16)
+    norm_w = torch.tensor(1.0 + 0.1 * rng.normal(size=n), dtype=torch.float32)
+    residual0 = torch.tensor(rng.normal(size=(m, n)) * 3.0, dtype=torch.float32)
+    wd = w.to(DEV)
+    tiles = ops.tile_weight(wd) if tiled else None
+    eps = 1e-3
+    ref_x = residual0.double().numpy() + x.double().numpy() @ w.double().numpy().T
+    residual = residual0.to(DEV)
+    rows, sumsq = ops.gemm_skinny(x.to(DEV), wd, tiles=tiles, add_norm=(residual, norm_w.to(DEV)))
+    assert _rel(residual.cpu().numpy(), ref_x) < 1e-11
+    # the rows are exactly bfloat16(new residual * norm weight), the partial sums add up to the rows' sums of squares
+    assert torch.equal(rows, (residual * norm_w.to(DEV)).bfloat16())
+    assert sumsq.shape == ((n + 15) // 16, ops.sumsq_stride(m))
+    assert np.allclose(sumsq.sum(dim=0)[:m].cpu().numpy(), (residual.double() ** 2).sum(dim=1).cpu().numpy(), rtol=1e-5)
+    assert float(sumsq[:, m:].abs().sum()) == 0.0
+    # the same sums as the product launched alone, in one part, and added afterwards
+    assert torch.equal(residual, residual0.to(DEV) + ops.gemm_skinny(x.to(DEV), wd, 1, tiles=tiles)[0])
+    # the next product, scaled by the rows' norms, against the product of the normalized rows (up to 16 rows)
+    if n % 8 == 0 and n >= 32:
+        n2 = 48
+        w2 = torch.tensor(rng.normal(size=(n2, n)) / math.sqrt(n), dtype=torch.bfloat16)
+        got = ops.gemm_skinny(rows, w2.to(DEV), 4, row_scale=(sumsq, eps)).sum(dim=0)
+        normed = ref_x / np.sqrt((ref_x ** 2).mean(axis=1, keepdims=True) + eps) * norm_w.double().numpy()
+        ref = normed @ w2.double().numpy().T
+        assert _rel(got.cpu().numpy(), ref) < 2e-5
+        # the rows alone, for a consumer that does not scale
+        finished = ops.scale_rows(rows, sumsq, eps, torch.empty_like(rows))
+        assert _rel(finished.float().cpu().numpy(), normed) < 2e-5
+        act = ops.gemm_skinny_swiglu(rows, torch.cat([w2, w2]).to(DEV), torch.empty(m, n2, dtype=torch.bfloat16, device=DEV),
+                                     row_scale=(sumsq, eps))
+        assert _rel(act.float().cpu().numpy(), plain.silu(ref) * ref) < 3e-5
+
+
 def test_tile_weight_layout():
     ops = _ops()
     w = torch.arange(20 * 64, dtype=torch.float32).reshape(20, 64).bfloat16()          # 20 rows: the second tile is padded

@@ -107,7 +107,7 @@ def test_attention_part(dtype, tol, n_q, n_kv, d, hidden, window):
     # step 1 writes the first tokens of every sequence into the pages step 2 will read
     b1.block_tables = {0: b2.block_tables[0]}
     part.forward(x1, b1, view)
-    got = part.forward(x2, b2, view).float().cpu().numpy()
+    got = rt.settle(part.forward(x2, b2, view)).float().cpu().numpy()
     wd = {k: v.double().numpy() for k, v in w.items()}
     at = 0
     for x, n0, n1 in zip(xs, first, second):
@@ -134,7 +134,7 @@ def test_gated_mlp_part(dtype, tol, rows):
     w = _weights(cls, spec, 4, wdt)
     _load(part, cls, spec, w, rt)
     x = torch.randn(rows, 80).to(rt.act_dtype)
-    got = part.forward(x.to(DEV))
+    got = rt.settle(part.forward(x.to(DEV)))        # few rows: the last product comes back not yet launched
     got = got.sum(dim=0) if got.dim() == 3 else got
     wd = {k: v.double().numpy() for k, v in w.items()}
     ref = plain.swiglu_mlp(x.double().numpy(), wd["gate_proj.weight"], wd["up_proj.weight"], wd["down_proj.weight"])
