@@ -118,13 +118,13 @@ __global__ void __launch_bounds__(256) rmsnorm_rows_kernel(float* __restrict__ x
     }
 }
 
-// out[t, :] = rows[t, :] * rsqrt(sum_p sumsq[p, t] / width + eps), sumsq in rows of `stride`: the normalized rows, for a consumer that
+// out[t, :] = rows[t, :] * rsqrt(sum_p sumsq[t, p] / width + eps), sumsq in rows of `stride`: the normalized rows, for a consumer that
 // does not apply the scale itself (rows = bfloat16(x * norm weight), sumsq = partial sums of x^2).
 __global__ void __launch_bounds__(256) scale_rows_kernel(const bf16_t* __restrict__ rows, const float* __restrict__ sumsq,
                                                          bf16_t* __restrict__ out, int width, int parts, int stride, float eps) {
     __shared__ float scratch[16];
     float a = 0.0f;
-    for (int p = threadIdx.x; p < parts; p += 256) a += sumsq[(size_t)p * stride + blockIdx.x];
+    for (int p = threadIdx.x; p < parts; p += 256) a += sumsq[(size_t)blockIdx.x * stride + p];
     a = block_sum(a, scratch);
     const float scale = 1.0f / sqrtf(a / (float)width + eps);
     for (int i = threadIdx.x; i < width; i += 256) {
@@ -246,7 +246,7 @@ int kipp_rmsnorm(float* x, const void* delta, int delta_dtype, int parts, const 
 int kipp_scale_rows(const void* rows, const float* sumsq, void* out, int n_rows, int width, int parts, int stride, float eps,
                     hipStream_t stream) {
     if (n_rows <= 0 || width <= 0) return 0;
-    if (parts <= 0 || stride < n_rows) return -1;
+    if (parts <= 0 || stride < parts) return -1;
     hipLaunchKernelGGL(scale_rows_kernel, dim3(n_rows), dim3(256), 0, stream, (const bf16_t*)rows, sumsq, (bf16_t*)out, width,
                        parts, stride, eps);
     return KIPP_LAUNCH_CHECK();

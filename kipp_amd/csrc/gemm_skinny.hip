@@ -55,8 +55,8 @@ union Frag {
 };
 
 struct RowScale {               // sumsq == nullptr: none
-    const float* sumsq;         // [parts, stride]: partial sums of squares of the rows X was made from
-    int parts, stride;          // stride: 4, 8 or 16 tokens (the smallest that holds M), so that a lane loads four tokens' sums
+    const float* sumsq;         // [M, stride]: `parts` partial sums of squares of each row X was made from
+    int parts, stride;          // stride: parts rounded up to a multiple of 4, so that a lane loads four sums at once
     float inv_width, eps;
 };
 
@@ -64,11 +64,11 @@ struct AddNorm {                // residual == nullptr: none
     float* residual;            // [M, N], updated in place
     const float* norm_w;        // [N]
     bf16_t* rows_out;           // [M, N] = bfloat16(residual * norm_w)
-    float* sumsq_out;           // [ceil(N / 16), stride], stride as in RowScale
+    float* sumsq_out;           // [M, stride]: ceil(N / 16) sums a row, stride as in RowScale
     int stride;
 };
 
-#define SCALE_LOADS 10          // 16-byte loads of partial sums a lane has in flight: 160 sums of 16 tokens, 640 of 4
+#define SCALE_LOADS 10          // 16-byte loads of partial sums a lane has in flight: 160 sums of a row, what 2,560 columns give
 
 template <int MT, bool SWIGLU, int KW, int DEPTH, bool TILED>
 __global__ void __launch_bounds__(THREADS) gemm_skinny_kernel(
@@ -113,25 +113,24 @@ __global__ void __launch_bounds__(THREADS) gemm_skinny_kernel(
     for (int mt = 0; mt < MT; ++mt) x_row[mt] = X + (size_t)min(16 * mt + l16, M - 1) * K + 8 * h;
 
     // the partial sums of the rows' scales, asked for first, all at once, and added once the first
-    // weights are on their way (up to 16 rows).  A lane loads the sums of four tokens for one index;
-    // stride / 4 lanes side by side cover the tokens, the others take further indices.
+    // weights are on their way (up to 16 rows): lane group h takes every fourth run of four sums of token l % 16.
+    // Of the waves that share a tile one does this for all (the one of the second slice; the scale is wanted
+    // after the slices have met in LDS anyway): every load a compute unit issues counts against the weights'.
+    __shared__ float s_scale[KW > 1 ? TW : 1][16];
     float4 scale_part[MT == 1 ? SCALE_LOADS : 1];
     const float* scale_src = nullptr;
-    const int lanes_per_index = MT == 1 ? rs.stride >> 2 : 1;             // 1, 2 or 4
-    const int index_step = KIPP_WAVE / lanes_per_index;
-    const int first_index = lane / lanes_per_index;
-    if (MT == 1 && rs.sumsq != nullptr) {
-        scale_src = rs.sumsq + 4 * (lane % lanes_per_index);
+    if (MT == 1 && rs.sumsq != nullptr && (KW == 1 || slice == 1)) {
+        scale_src = rs.sumsq + (size_t)min(l16, M - 1) * rs.stride;
 #pragma unroll
-        for (int i = 0; i < SCALE_LOADS; ++i)   // beyond the last index: read the last again, dropped below
-            scale_part[i] = *(const float4*)(scale_src + (size_t)min(first_index + index_step * i, rs.parts - 1) * rs.stride);
+        for (int i = 0; i < SCALE_LOADS; ++i)   // beyond the last run: read the last again, dropped below
+            scale_part[i] = *(const float4*)(scale_src + min(4 * (h + 4 * i), rs.stride - 4));
         __builtin_amdgcn_sched_barrier(0);
     }
 
     // what the residual end adds to, asked for first as well (nobody writes these elements before that end does)
     const bool wide = (N & 3) == 0;                  // a lane's four columns are 16 aligned bytes
     float res[MT][4], norm_w[4];
-    if (!SWIGLU && an.residual != nullptr) {
+    if (!SWIGLU && an.residual != nullptr && slice == 0) {       // the wave that will hold the tile's sums
         const int col = min(n0 + 4 * h, wide ? N - 4 : N - 1);
         if (wide) {
             const float4 w4 = *(const float4*)(an.norm_w + col);
@@ -184,34 +183,27 @@ __global__ void __launch_bounds__(THREADS) gemm_skinny_kernel(
     for (int mt = 0; mt < MT; ++mt) row_scale[mt] = 1.0f;
     auto finish_scale = [&]() {
         if (MT == 1 && scale_src != nullptr) {
-            float t[4];
-            asm volatile("v_mov_b32 %0, 0" : "=v"(t[0]) : : "memory");
-            t[1] = t[2] = t[3] = t[0];
+            float t;
+            asm volatile("v_mov_b32 %0, 0" : "=v"(t) : : "memory");
 #pragma unroll
             for (int i = 0; i < SCALE_LOADS; ++i) {
-                const bool ok = first_index + index_step * i < rs.parts;
-                t[0] += ok ? scale_part[i].x : 0.0f;
-                t[1] += ok ? scale_part[i].y : 0.0f;
-                t[2] += ok ? scale_part[i].z : 0.0f;
-                t[3] += ok ? scale_part[i].w : 0.0f;
+                const int p = 4 * (h + 4 * i);
+                t += p < rs.parts ? scale_part[i].x : 0.0f;
+                t += p + 1 < rs.parts ? scale_part[i].y : 0.0f;
+                t += p + 2 < rs.parts ? scale_part[i].z : 0.0f;
+                t += p + 3 < rs.parts ? scale_part[i].w : 0.0f;
             }
-            for (int p = first_index + index_step * SCALE_LOADS; p < rs.parts; p += index_step) {   // wider rows: the rest one by one
-                const float4 more = *(const float4*)(scale_src + (size_t)p * rs.stride);
-                t[0] += more.x, t[1] += more.y, t[2] += more.z, t[3] += more.w;
+            for (int p = 4 * (h + 4 * SCALE_LOADS); p < rs.parts; p += 16) {   // wider rows: the rest one by one
+                const float4 more = *(const float4*)(scale_src + p);
+                t += more.x;
+                t += p + 1 < rs.parts ? more.y : 0.0f;
+                t += p + 2 < rs.parts ? more.z : 0.0f;
+                t += p + 3 < rs.parts ? more.w : 0.0f;
             }
-            // the lanes that hold the same tokens, added pairwise: in the end every lane has its four tokens' totals
-            for (int off = lanes_per_index; off < KIPP_WAVE; off <<= 1)
-#pragma unroll
-                for (int e = 0; e < 4; ++e) t[e] += __shfl_xor(t[e], off, KIPP_WAVE);
-            // token l % 16 sits in lane (l % 16) / 4 (any lane of that remainder would do), element (l % 16) % 4
-            const int from = min(l16 >> 2, lanes_per_index - 1);
-            float mine = 0.0f;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const float got = __shfl(t[e], from, KIPP_WAVE);
-                if ((l16 & 3) == e) mine = got;
-            }
-            row_scale[0] = 1.0f / sqrtf(mine * rs.inv_width + rs.eps);
+            t += __shfl_xor(t, 16, KIPP_WAVE);     // the four lane groups of a token
+            t += __shfl_xor(t, 32, KIPP_WAVE);
+            row_scale[0] = 1.0f / sqrtf(t * rs.inv_width + rs.eps);
+            if (KW > 1 && h == 0) s_scale[tile_in_wg][l16] = row_scale[0];
         }
     };
     if (g_begin >= g_end) finish_scale();
@@ -265,6 +257,7 @@ __global__ void __launch_bounds__(THREADS) gemm_skinny_kernel(
                 for (int v = 0; v < 4; ++v) red[wave][nt][mt][lane * 4 + v] = acc[nt][mt][v];
         __syncthreads();
         writer = slice == 0;
+        if (MT == 1 && rs.sumsq != nullptr) row_scale[0] = s_scale[tile_in_wg][l16];
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
@@ -318,8 +311,7 @@ __global__ void __launch_bounds__(THREADS) gemm_skinny_kernel(
             }
             ss += __shfl_xor(ss, 16, KIPP_WAVE);      // the four lane groups hold a tile's 16 columns of a token
             ss += __shfl_xor(ss, 32, KIPP_WAVE);
-            // tokens beyond M up to the stride get a zero: the consumer loads them with the others
-            if (h == 0 && token < an.stride && n0 < N) an.sumsq_out[(size_t)(n0 >> 4) * an.stride + token] = token < M ? ss : 0.0f;
+            if (h == 0 && token < M && n0 < N) an.sumsq_out[(size_t)token * an.stride + (n0 >> 4)] = ss;
         }
         return;
     }
@@ -435,25 +427,25 @@ int kipp_gemm_skinny_parts(int N, int K, int max_parts) {
     return parts;
 }
 
-// Tokens a row of partial sums has room for: the smallest of 4, 8, 16 that holds M (0: more than 16 rows).
-static int sumsq_stride(int M) { return M <= 4 ? 4 : (M <= 8 ? 8 : (M <= 16 ? 16 : 0)); }
+// Floats of a row of `parts` partial sums: whole runs of four.
+static int sumsq_stride(int parts) { return (parts + 3) / 4 * 4; }
 
-static RowScale row_scale_of(const float* sumsq, int sumsq_parts, int M, int K, float eps) {
-    RowScale rs = {sumsq, sumsq_parts, sumsq != nullptr ? sumsq_stride(M) : 4, 1.0f / (float)K, eps};
+static RowScale row_scale_of(const float* sumsq, int sumsq_parts, int K, float eps) {
+    RowScale rs = {sumsq, sumsq_parts, sumsq_stride(sumsq_parts), 1.0f / (float)K, eps};
     return rs;
 }
 
-// Width of a row of partial sums for M rows (0: more rows than the fused ends take).
-int kipp_gemm_skinny_sumsq_stride(int M) { return sumsq_stride(M); }
+// Floats of a row of the partial sums a product of N columns writes (ceil(N / 16) sums, in whole runs of four).
+int kipp_gemm_skinny_sumsq_stride(int N) { return sumsq_stride((N + 15) / 16); }
 
 // Y: float32 [parts, M, N] with parts = kipp_gemm_skinny_parts(N, K, max_parts).
 // K must be a multiple of 8 (16-byte loads), M <= 64.  `tiled`: W is in the
 // streaming layout (K a multiple of 32), else [N, K] rows.
-// `sumsq` [sumsq_parts, kipp_gemm_skinny_sumsq_stride(M)] (or null; M <= 16 then): every row of the product is multiplied by
+// `sumsq` [M, sumsq_parts rounded up to a multiple of 4] (or null; M <= 16 then): every row of the product is multiplied by
 // rsqrt(sum of the row's sumsq / K + eps).
 // `residual` [M, N] (or null): the product is added to it in place (Y is not written and there is
 // one part), `rows_out` [M, N] = bfloat16(residual * norm_w) and `sumsq_out`
-// [ceil(N / 16), kipp_gemm_skinny_sumsq_stride(M)] = the new residual's sums of squares over each 16 columns
+// [M, kipp_gemm_skinny_sumsq_stride(N)] = every row's sums of squares of the new residual over each 16 columns
 // (M <= 16 with a residual).
 int kipp_gemm_skinny(const void* X, const void* W, float* Y, int M, int N, int K, int max_parts, int tiled,
                      const float* sumsq, int sumsq_parts, float eps, float* residual, const float* norm_w, void* rows_out,
@@ -464,9 +456,9 @@ int kipp_gemm_skinny(const void* X, const void* W, float* Y, int M, int N, int K
     if (residual != nullptr && (norm_w == nullptr || rows_out == nullptr || sumsq_out == nullptr || M > 16)) return -1;
     int kw, parts;
     plan((N + 15) / 16, K, residual != nullptr ? 1 : max_parts, &kw, &parts);
-    AddNorm an = {residual, norm_w, (bf16_t*)rows_out, sumsq_out, sumsq_stride(M)};
+    AddNorm an = {residual, norm_w, (bf16_t*)rows_out, sumsq_out, sumsq_stride((N + 15) / 16)};
     return launch<false>((const bf16_t*)X, (const bf16_t*)W, Y, nullptr, M, N, K, parts, kw, tiled,
-                         row_scale_of(sumsq, sumsq_parts, M, K, eps), an, stream);
+                         row_scale_of(sumsq, sumsq_parts, K, eps), an, stream);
 }
 
 // W: [2 I, K] = [gate; up] (tiled: tiles of 8 gate rows over the 8 matching up rows); act: bfloat16 [M, I].
@@ -481,7 +473,7 @@ int kipp_gemm_skinny_swiglu(const void* X, const void* W, void* act, int M, int 
     plan((two_inner / 2 + 7) / 8, K, 1, &kw, &parts);
     AddNorm none = {nullptr, nullptr, nullptr, nullptr, 4};
     return launch<true>((const bf16_t*)X, (const bf16_t*)W, nullptr, (bf16_t*)act, M, two_inner, K, 1, kw, tiled,
-                        row_scale_of(sumsq, sumsq_parts, M, K, eps), none, stream);
+                        row_scale_of(sumsq, sumsq_parts, K, eps), none, stream);
 }
 
 }  // extern "C"

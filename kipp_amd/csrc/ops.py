@@ -467,21 +467,15 @@ def _tiles_ok(tiles, n: int, k: int, what: str) -> int:
 
 
 def _row_scale_args(row_scale, m: int, what: str):
-    """(sumsq pointer, parts, eps) of `row_scale` = (sumsq [parts, sumsq_stride(M)] float32, eps), or nulls."""
+    """(sumsq pointer, parts, eps) of `row_scale` = (sumsq, parts, eps), sumsq float32 [M, parts rounded up to 4]."""
     if row_scale is None:
         return None, 0, 0.0
-    sumsq, eps = row_scale
+    sumsq, parts, eps = row_scale
     _dev(sumsq)
-    _need(m <= 16 and sumsq.dtype == torch.float32 and sumsq.dim() == 2 and sumsq.shape[1] == sumsq_stride(m)
-          and sumsq.shape[0] > 0 and sumsq.is_contiguous(),
-          f"{what}: row_scale is (float32 [parts, sumsq_stride(M)], eps), for at most 16 rows")
-    return _ptr(sumsq), sumsq.shape[0], float(eps)
-
-
-def sumsq_stride(m: int) -> int:
-    """Width of a row of partial sums for m rows: 4, 8 or 16, the smallest that holds them
-    (the consumer loads four tokens' sums at once); 0 for more than 16 rows."""
-    return 4 if m <= 4 else (8 if m <= 8 else (16 if m <= 16 else 0))
+    _need(m <= 16 and sumsq.dtype == torch.float32 and sumsq.dim() == 2 and parts > 0
+          and tuple(sumsq.shape) == (m, (parts + 3) // 4 * 4) and sumsq.is_contiguous(),
+          f"{what}: row_scale is (float32 [M, parts rounded up to 4], parts, eps), for at most 16 rows")
+    return _ptr(sumsq), int(parts), float(eps)
 
 
 def gemm_skinny(x: torch.Tensor, w: torch.Tensor, max_parts: int = 1, tiles: torch.Tensor = None,
@@ -491,13 +485,14 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, max_parts: int = 1, tiles: tor
     shape (1 when the weight has many rows).  With `tiles` (tile_weight(w)) the
     weight is streamed from that layout.
 
-    `row_scale` = (sumsq [P, sumsq_stride(M)], eps), M <= 16: row t of the product is
-    multiplied by rsqrt(sum(sumsq[:, t]) / K + eps), i.e. x holds rows of an RMS
-    norm that still lack their scale.
+    `row_scale` = (sumsq [M, P rounded up to 4], P, eps), M <= 16: row t of the
+    product is multiplied by rsqrt(sum(sumsq[t, :P]) / K + eps), i.e. x holds rows
+    of an RMS norm that still lack their scale.
     `add_norm` = (residual float32 [M, N], norm_weight float32 [N]), M <= 16: the product
     (in one part) is added to `residual` in place by the kernel itself and the
     call returns (rows, sumsq) instead: rows = bfloat16(residual * norm_weight)
-    and sumsq [ceil(N / 16), sumsq_stride(M)], what `row_scale` of the next product takes."""
+    and sumsq [M, P rounded up to 4] with P = ceil(N / 16) sums a row: (sumsq, P, eps)
+    is the `row_scale` of the next product."""
     _dev(x, w)
     m, k = x.shape
     n = w.shape[0]
@@ -518,7 +513,7 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, max_parts: int = 1, tiles: tor
               "gemm_skinny: the residual is float32 [M, N], at most 16 rows")
         _need(norm_w.dtype == torch.float32 and norm_w.numel() == n, "gemm_skinny: the norm weight is float32 [N]")
         rows = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
-        sumsq_out = torch.empty(((n + 15) // 16, sumsq_stride(m)), dtype=torch.float32, device=x.device)
+        sumsq_out = torch.empty((m, ((n + 15) // 16 + 3) // 4 * 4), dtype=torch.float32, device=x.device)
     fn = _fn("gemm_skinny", "kipp_gemm_skinny",
              [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_int, _c_float,
               _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr])
@@ -527,16 +522,16 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, max_parts: int = 1, tiles: tor
     return out if add_norm is None else (rows, sumsq_out)
 
 
-def scale_rows(rows: torch.Tensor, sumsq: torch.Tensor, eps: float, out: torch.Tensor) -> torch.Tensor:
-    """out[t] = rows[t] * rsqrt(sum(sumsq[:, t]) / width + eps), bfloat16: the rows of an RMS norm
+def scale_rows(rows: torch.Tensor, sumsq: torch.Tensor, parts: int, eps: float, out: torch.Tensor) -> torch.Tensor:
+    """out[t] = rows[t] * rsqrt(sum(sumsq[t, :parts]) / width + eps), bfloat16: the rows of an RMS norm
     from what `gemm_skinny(..., add_norm=...)` returns, for a consumer that does not take `row_scale`."""
     _dev(rows, sumsq, out)
     m, width = rows.shape
     _need(rows.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and out.shape == rows.shape
-          and sumsq.dtype == torch.float32 and sumsq.dim() == 2 and sumsq.shape[1] >= m and sumsq.is_contiguous(),
-          "scale_rows: shapes or types differ")
+          and sumsq.dtype == torch.float32 and sumsq.dim() == 2 and sumsq.shape[0] == m and 0 < parts <= sumsq.shape[1]
+          and sumsq.is_contiguous(), "scale_rows: shapes or types differ")
     fn = _fn("elementwise", "kipp_scale_rows", [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_float, _c_ptr])
-    _check(fn(_ptr(rows), _ptr(sumsq), _ptr(out), m, width, sumsq.shape[0], sumsq.shape[1], float(eps), _stream()), "scale_rows")
+    _check(fn(_ptr(rows), _ptr(sumsq), _ptr(out), m, width, int(parts), sumsq.shape[1], float(eps), _stream()), "scale_rows")
     return out
 
 

@@ -52,7 +52,7 @@ class GatedMLP:
             # both products and the activation in one kernel (and the norm's scale, if it was left to us)
             scaled = hasattr(x, "sumsq")
             rt.ops.gemm_skinny_swiglu(x.rows if scaled else x, w.rows, act, tiles=w.tiles,
-                                      row_scale=(x.sumsq, x.eps) if scaled else None)
+                                      row_scale=x.scale if scaled else None)
             return rt.linear(act, self.w_down, slabs=True, defer=True)
         x = rt.rows_of(x)
         if ours and w.pairs:

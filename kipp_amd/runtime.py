@@ -52,14 +52,19 @@ class Weight:
 
 class ScaledRows:
     """Rows of an RMS norm that still lack their scale: `rows` = bfloat16(x * norm
-    weight) and `sumsq` [P, 4 | 8 | 16], partial sums of x^2 whose total gives row t's scale
-    rsqrt(sum(sumsq[:, t]) / width + eps).  A row's scale commutes with a product over
+    weight) and `sumsq` [M, >= parts], `parts` partial sums of x^2 a row whose total gives
+    row t's scale rsqrt(sum(sumsq[t, :parts]) / width + eps).  A row's scale commutes with a product over
     the row, so `Runtime.linear` applies it to the product's rows; any other
     consumer asks `Runtime.rows_of` for the finished rows."""
-    __slots__ = ("rows", "sumsq", "eps")
+    __slots__ = ("rows", "sumsq", "parts", "eps")
 
-    def __init__(self, rows: torch.Tensor, sumsq: torch.Tensor, eps: float):
-        self.rows, self.sumsq, self.eps = rows, sumsq, eps
+    def __init__(self, rows: torch.Tensor, sumsq: torch.Tensor, parts: int, eps: float):
+        self.rows, self.sumsq, self.parts, self.eps = rows, sumsq, parts, eps
+
+    @property
+    def scale(self):
+        """What the products' `row_scale` takes."""
+        return (self.sumsq, self.parts, self.eps)
 
     @property
     def shape(self):
@@ -137,7 +142,7 @@ class Runtime:
         """The tensor of norm output, scaled now if the scale was left to a product."""
         if not isinstance(h, ScaledRows):
             return h
-        return self.ops.scale_rows(h.rows, h.sumsq, h.eps, self.empty(h.rows.shape, torch.bfloat16))
+        return self.ops.scale_rows(h.rows, h.sumsq, h.parts, h.eps, self.empty(h.rows.shape, torch.bfloat16))
 
     def product_add_norm(self, delta: Deferred, x: torch.Tensor, norm_weight: torch.Tensor, eps: float):
         """x += delta's product, in the product's own kernel, which also prepares the
@@ -150,7 +155,7 @@ class Runtime:
                 and norm_weight.dtype == torch.float32):
             return None
         rows_out, sumsq = self.ops.gemm_skinny(delta.x, w.rows, tiles=w.tiles, add_norm=(x, norm_weight))
-        return ScaledRows(rows_out, sumsq, eps)
+        return ScaledRows(rows_out, sumsq, (w.shape[0] + 15) // 16, eps)
 
     def linear(self, x, w, slabs: bool = False, low_precision_out: bool = False, defer: bool = False):
         """float32 [M, N] = x [M, K] . w [N, K]^T.  With `slabs` the result may come
@@ -167,7 +172,7 @@ class Runtime:
         row_scale = None
         if isinstance(x, ScaledRows):
             if self._few_rows(x.shape[0], x.shape[1], w):
-                row_scale, x = (x.sumsq, x.eps), x.rows
+                row_scale, x = x.scale, x.rows
             else:
                 x = self.rows_of(x)
         tiles = None

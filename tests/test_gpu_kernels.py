@@ -630,24 +630,24 @@ def test_gemm_skinny_adds_the_residual_and_prepares_the_norm(m, n, k, tiled):
     assert _rel(residual.cpu().numpy(), ref_x) < 1e-11
     # the rows are exactly bfloat16(new residual * norm weight), the partial sums add up to the rows' sums of squares
     assert torch.equal(rows, (residual * norm_w.to(DEV)).bfloat16())
-    assert sumsq.shape == ((n + 15) // 16, ops.sumsq_stride(m))
-    assert np.allclose(sumsq.sum(dim=0)[:m].cpu().numpy(), (residual.double() ** 2).sum(dim=1).cpu().numpy(), rtol=1e-5)
-    assert float(sumsq[:, m:].abs().sum()) == 0.0
+    parts = (n + 15) // 16
+    assert sumsq.shape == (m, (parts + 3) // 4 * 4)
+    assert np.allclose(sumsq[:, :parts].sum(dim=1).cpu().numpy(), (residual.double() ** 2).sum(dim=1).cpu().numpy(), rtol=1e-5)
     # the same sums as the product launched alone, in one part, and added afterwards
     assert torch.equal(residual, residual0.to(DEV) + ops.gemm_skinny(x.to(DEV), wd, 1, tiles=tiles)[0])
     # the next product, scaled by the rows' norms, against the product of the normalized rows (up to 16 rows)
     if n % 8 == 0 and n >= 32:
         n2 = 48
         w2 = torch.tensor(rng.normal(size=(n2, n)) / math.sqrt(n), dtype=torch.bfloat16)
-        got = ops.gemm_skinny(rows, w2.to(DEV), 4, row_scale=(sumsq, eps)).sum(dim=0)
+        got = ops.gemm_skinny(rows, w2.to(DEV), 4, row_scale=(sumsq, parts, eps)).sum(dim=0)
         normed = ref_x / np.sqrt((ref_x ** 2).mean(axis=1, keepdims=True) + eps) * norm_w.double().numpy()
         ref = normed @ w2.double().numpy().T
         assert _rel(got.cpu().numpy(), ref) < 2e-5
         # the rows alone, for a consumer that does not scale
-        finished = ops.scale_rows(rows, sumsq, eps, torch.empty_like(rows))
+        finished = ops.scale_rows(rows, sumsq, parts, eps, torch.empty_like(rows))
         assert _rel(finished.float().cpu().numpy(), normed) < 2e-5
         act = ops.gemm_skinny_swiglu(rows, torch.cat([w2, w2]).to(DEV), torch.empty(m, n2, dtype=torch.bfloat16, device=DEV),
-                                     row_scale=(sumsq, eps))
+                                     row_scale=(sumsq, parts, eps))
         assert _rel(act.float().cpu().numpy(), plain.silu(ref) * ref) < 3e-5
 
 
