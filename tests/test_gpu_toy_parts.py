@@ -325,3 +325,127 @@ def test_routed_feed_forward_and_another_position_encoding(tmp_path, cut):
         unregister_architecture("ToyRoutedForTests")
         unregister("feed_forward", "toy_routed")
         unregister("position", "toy_stretched_rope")
+
+
+# ---------------------------------------------------------------------------------------------
+# A norm of another kind between the framework's own parts, in bfloat16: with few rows the framework's
+# products come back not yet launched and its norm leaves its scale to the next product; a norm that
+# knows nothing of either gets tensors, and the parts behind it work as before.
+
+@dataclass(frozen=True)
+class MeanAbsNormSpec:
+    width: int
+    eps: float
+    prefix: str = ""
+    kind: str = "toy_mean_abs"
+
+
+def _register_mean_abs():
+    from kipp_amd.config import register_architecture
+    from kipp_amd.config.specs import (AttentionSpec, EmbeddingSpec, GatedMLPSpec, HeadSpec, LayerRun, LayerSpec, ModelSpec,
+                                       RMSNormSpec, RopeSpec)
+    from kipp_amd.parts import ParamSpec, register
+
+    @register("norm", "toy_mean_abs")
+    class MeanAbsNorm:
+        """y = x / (mean |x| + eps) * w."""
+
+        def __init__(self, spec, runtime):
+            self.spec, self.rt = spec, runtime
+
+        @staticmethod
+        def params(spec):
+            return {"weight": ParamSpec((spec.width,), "float", ("one_plus_normal", 0.05))}
+
+        @staticmethod
+        def placement(spec):
+            return {"weight": "float32"}
+
+        def load(self, tensors):
+            self.weight = tensors["weight"]
+
+        def forward(self, x, out_dtype):
+            return (x / (x.abs().mean(dim=-1, keepdim=True) + self.spec.eps) * self.weight).to(out_dtype)
+
+        def add_forward(self, x, delta, out_dtype):
+            assert isinstance(delta, torch.Tensor), "a norm that does not declare fuses_products gets tensors"
+            x += delta.sum(dim=0) if delta.dim() == 3 else delta
+            return self.forward(x, out_dtype)
+
+    class MeanAbsConfig:
+        def __init__(self, d):
+            self.d = d
+
+        def to_dict(self):
+            return dict(self.d)
+
+        def model_spec(self):
+            def layer(i):
+                p = f"layers.{i}."
+                attn = AttentionSpec(M_HIDDEN, 4, 2, 32, position=RopeSpec(32, THETA), qk_norm_eps=EPS, prefix=p + "attn.")
+                return LayerSpec(block="pre_norm", parts=(
+                    ("mixer_norm", RMSNormSpec(M_HIDDEN, EPS, p + "n1.")), ("mixer", attn),
+                    ("ffn_norm", MeanAbsNormSpec(M_HIDDEN, EPS, p + "n2.")), ("ffn", GatedMLPSpec(M_HIDDEN, M_INNER, prefix=p + "mlp."))))
+            return ModelSpec("ToyMeanAbsForTests", M_HIDDEN, VOCAB, 256, EmbeddingSpec(VOCAB, M_HIDDEN, "embed."),
+                             (layer(0), layer(1)), (LayerRun(0), LayerRun(1)), MeanAbsNormSpec(M_HIDDEN, EPS, "norm."),
+                             HeadSpec(VOCAB, M_HIDDEN, True))
+
+    register_architecture("ToyMeanAbsForTests", MeanAbsConfig)
+
+
+M_HIDDEN, M_INNER = 64, 96
+
+
+def _plain_mean_abs(w, tokens):
+    def mean_abs(x, weight):
+        return x / (np.abs(x).mean(axis=-1, keepdims=True) + EPS) * weight
+    pos = np.arange(len(tokens))
+    x = plain.embed(w["embed.weight"], tokens)
+    for i in range(2):
+        p = f"layers.{i}."
+        n = plain.rms_norm(x, w[p + "n1.weight"], EPS)
+        q = plain.head_norm(plain.linear(n, w[p + "attn.q_proj.weight"]), 4, 32, w[p + "attn.q_norm.weight"], EPS)
+        k = plain.head_norm(plain.linear(n, w[p + "attn.k_proj.weight"]), 2, 32, w[p + "attn.k_norm.weight"], EPS)
+        q, k = plain.rope(q, 4, 32, pos, THETA), plain.rope(k, 2, 32, pos, THETA)
+        v = plain.linear(n, w[p + "attn.v_proj.weight"])
+        x = x + plain.linear(plain.causal_gqa(q, k, v, 4, 2, 32), w[p + "attn.o_proj.weight"])
+        n = mean_abs(x, w[p + "n2.weight"])
+        x = x + plain.swiglu_mlp(n, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+    return plain.linear(mean_abs(x, w["norm.weight"]), w["embed.weight"])
+
+
+@pytest.mark.parametrize("cut", ["tail", "mixed"])
+def test_another_norm_between_products_that_fuse_theirs(tmp_path, cut):
+    from kipp_amd.config import unregister_architecture
+    from kipp_amd.engine import Engine
+    from kipp_amd.parts import unregister
+    from kipp_amd.runtime import Deferred, ScaledRows
+    from kipp_amd.weights import write_random_model
+    _register_mean_abs()
+    try:
+        folder = write_random_model(str(tmp_path / "meanabs"), {"architectures": ["ToyMeanAbsForTests"]}, seed=12, dtype="bfloat16")
+        _, weights = plain.load_folder(folder)
+        requests = {f"r{i}": H.random_tokens(40 + i, n, VOCAB) for i, n in enumerate([37, 52, 44])}
+        steps = {"tail": H.tail_one_by_one, "mixed": lambda r: H.mixed(r, seed=6)}[cut](requests)
+        engine = Engine.from_folder(folder, dtype="bfloat16", page_size=8, max_tokens=256, max_requests=4)
+        # the framework's parts did fuse where they met each other: the second layer's first norm got a product
+        # that was not launched yet and handed rows without their scale to the attention
+        seen = {"deferred": 0, "scaled": 0}
+        norm1, mixer = engine.model.blocks[1].parts["mixer_norm"], engine.model.blocks[1].parts["mixer"]
+        inner_add, inner_mix = norm1.add_forward, mixer.forward
+
+        def add_forward(x, delta, out_dtype):
+            seen["deferred"] += isinstance(delta, Deferred)
+            return inner_add(x, delta, out_dtype)
+
+        def forward(x, *rest):
+            seen["scaled"] += isinstance(x, ScaledRows)
+            return inner_mix(x, *rest)
+        norm1.add_forward, mixer.forward = add_forward, forward
+        got = H.replay(engine, requests, steps)
+        for rid, toks in requests.items():
+            H.assert_close(got[rid], _plain_mean_abs(weights, toks), H.NMSE_BF16, f"mean-abs norm/{cut}/{rid}")
+        assert seen["deferred"] > 0 and seen["scaled"] > 0, seen
+    finally:
+        unregister_architecture("ToyMeanAbsForTests")
+        unregister("norm", "toy_mean_abs")
