@@ -622,8 +622,9 @@ __global__ void __launch_bounds__(THREADS) attention_decode_stream_kernel(
 //            they are (rounded to bfloat16), V^T comes out of LDS transposed by
 //            ds_read_b64_tr_b16 (values lie in LDS as in the cache, [key][d]).
 //
-// The launcher takes this kernel from 128 (sequence, key/value head) pairs on (measured: from there it is
-// at least as fast as splitting the keys, merge kernel included, with pages scattered over the pool):
+// The launcher takes this kernel from 96 (sequence, key/value head) pairs on (measured in the decode step at
+// 2,100 keys: from there it is at least as fast as splitting the keys, merge kernel included, with pages
+// scattered over the pool; at 80 pairs it is a tenth slower):
 // a workgroup then walks a sequence's whole context (up to RING_RANGE keys), the partial results
 // and the merge kernel fall away, and in the FUSED form every query is normed and rotated once (by
 // the one workgroup of its key/value head) while the first blocks are on their way; that workgroup
@@ -640,7 +641,7 @@ __global__ void __launch_bounds__(THREADS) attention_decode_stream_kernel(
 #define RING_BYTES (WAVES * RING_STAGES * 2 * RING_HALF)
 #define RING_RANGE (KIPP_WAVE * WAVES * 16)                    // keys of a workgroup at most: a wave holds its blocks' pages one a lane
 #ifndef RING_FROM_PAIRS
-#define RING_FROM_PAIRS 128                                    // sequences x key/value heads from which this kernel is taken
+#define RING_FROM_PAIRS 96                                    // sequences x key/value heads from which this kernel is taken
 #endif
 
 typedef __attribute__((ext_vector_type(4))) short s16x4;

@@ -94,12 +94,13 @@ def test_decoding_across_a_graph_bucket_and_many_splits(long_folder, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("n_requests", [100, 128, 200])
+@pytest.mark.parametrize("n_requests", [80, 128, 200])
 def test_many_requests_decode_together(long_folder, dtype, n_requests):
     """More rows than one 64-row product takes: prompts of 3 to 40 tokens enter in one step, then all decode
     together for 6 steps (the products stage their rows in chunks of 128 columns, the steps are recorded
-    graphs).  With 128 requests (one key/value head each) decode attention is the kernel in which a
-    workgroup walks a whole context, from the projection's output; with 100 the keys are split.  Every
+    graphs).  From 96 rows on (one key/value head each) decode attention is the kernel in which a
+    workgroup walks a whole context, from the projection's output; with 80 the keys are split in the steps
+    that run as they are, and the recorded steps, filled up to 96 rows, take the other kernel.  Every
     tenth request against the plain implementation."""
     from kipp_amd.engine import Engine, StepEntry
     cfg, weights = plain.load_folder(long_folder)
@@ -117,7 +118,7 @@ def test_many_requests_decode_together(long_folder, dtype, n_requests):
             fed[rid] += 1
     assert engine.graphs.replays >= 4
     from kipp_amd.csrc import ops
-    assert ops.attention_decode_streams(n_requests, 1, 128, 4, 16, 64) == (n_requests >= 128)
+    assert ops.attention_decode_streams(n_requests, 1, 128, 4, 16, 64) == (n_requests >= 96)
     tol = H.NMSE_F32 if dtype == "float32" else H.NMSE_BF16
     for rid in list(seqs)[::10]:
         ref = plain.forward_whole(cfg, weights, seqs[rid])
