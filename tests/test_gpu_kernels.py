@@ -435,8 +435,11 @@ def test_attention_decode_of_few_long_sequences(window):
         assert _rel(got[i], ref[i]) < 1e-5, f"context of {seq_lens[i]} keys"
 
 
-@pytest.mark.parametrize("whole", [False, True])
-@pytest.mark.parametrize("n_q,n_kv,d,page", [(32, 8, 128, 16), (8, 1, 128, 8), (16, 1, 128, 16), (3, 3, 128, 4), (8, 2, 256, 32), (4, 2, 256, 16)])
+_PROJECTION_GEOMETRIES = [(32, 8, 128, 16), (8, 1, 128, 8), (16, 1, 128, 16), (3, 3, 128, 4), (8, 2, 256, 32), (4, 2, 256, 16)]
+
+
+@pytest.mark.parametrize("n_q,n_kv,d,page,whole", [g + (False,) for g in _PROJECTION_GEOMETRIES]
+                         + [g + (True,) for g in _PROJECTION_GEOMETRIES if g[2] == 128 and g[3] % 16 == 0])
 @pytest.mark.parametrize("window,norm,slabs,write_kv", [(0, True, 1, True), (300, True, 3, True), (0, False, 2, True), (0, True, 1, False)])
 def test_attention_decode_from_the_projection(n_q, n_kv, d, page, window, norm, slabs, write_kv, whole):
     """Decode attention that starts from the QKV projection's output: the same bits
@@ -444,8 +447,6 @@ def test_attention_decode_from_the_projection(n_q, n_kv, d, page, window, norm, 
     attention kernel, at split edges (256, 257, 513) and for the first token.  `whole`: the
     kernels in which a workgroup walks a whole context (head size 128, pages of 16 and more)."""
     ops = _ops()
-    if whole and not (d == 128 and page % 16 == 0):
-        pytest.skip("the whole-context kernel takes head size 128 and pages of 16 keys and more")
     inner, forced = _whole_contexts(ops)
     ops._fn = forced if whole else inner
     try:
