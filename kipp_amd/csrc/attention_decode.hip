@@ -964,6 +964,72 @@ __global__ void attention_decode_reduce_kernel(
 }
 
 
+// The same merge for launches of up to MAXS splits: the (m, l) pairs and the partial sums of every split the
+// launch has are asked for at once, before the token's position says how many of them count, so the kernel is
+// two round trips to memory long instead of four.  The same sums in the same order as above.
+template <int MAXS>
+__global__ void __launch_bounds__(KIPP_WAVE) attention_decode_reduce_few_kernel(
+    const float* __restrict__ part_acc, const float* __restrict__ part_ml, bf16_t* __restrict__ out,
+    const int32_t* __restrict__ rows, const int32_t* __restrict__ positions, int n_q, int window, int max_splits,
+    int split_keys, int grid_splits) {
+    constexpr int COLS = (HEAD_DIM + KIPP_WAVE - 1) / KIPP_WAVE;     // columns of a head a lane merges
+    const int head = blockIdx.x, item = blockIdx.y, lane = threadIdx.x;
+    const size_t slot0 = ((size_t)item * n_q + head) * max_splits;
+    float m_s[MAXS], l_s[MAXS], a_s[MAXS][COLS];
+#pragma unroll
+    for (int s = 0; s < MAXS; ++s) {
+        const size_t slot = slot0 + min(s, grid_splits - 1);         // beyond the launch's splits: the last again, dropped below
+        m_s[s] = part_ml[slot * 2];
+        l_s[s] = part_ml[slot * 2 + 1];
+#pragma unroll
+        for (int c = 0; c < COLS; ++c) a_s[s][c] = part_acc[slot * HEAD_DIM + min(lane + KIPP_WAVE * c, HEAD_DIM - 1)];
+    }
+    const int row = rows[item];
+    const int pos = positions[row];
+    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+    const int n_splits = pos / split_keys - lo / split_keys + 1;
+    if (n_splits == 1) return;                                        // written by the attention kernel itself
+    // slots of splits that did not run hold whatever was there before: they are chosen away, never multiplied
+    float m = -INFINITY;
+#pragma unroll
+    for (int s = 0; s < MAXS; ++s) m = fmaxf(m, s < n_splits ? m_s[s] : -INFINITY);
+    float denom = 0.0f, a[COLS];
+#pragma unroll
+    for (int c = 0; c < COLS; ++c) a[c] = 0.0f;
+#pragma unroll
+    for (int s = 0; s < MAXS; ++s) {
+        if (s < n_splits) {
+            const float w = exp2f(m_s[s] - m);
+            denom += l_s[s] * w;
+#pragma unroll
+            for (int c = 0; c < COLS; ++c) a[c] += a_s[s][c] * w;
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < COLS; ++c) {
+        const int dcol = lane + KIPP_WAVE * c;
+        if (dcol < HEAD_DIM) out[((size_t)row * n_q + head) * HEAD_DIM + dcol] = f32_to_bf16(a[c] / denom);
+    }
+}
+
+// The merge of a launch's splits (`grid_splits` of `split_keys` keys each at most).
+static int launch_reduce(const float* part_acc, const float* part_ml, bf16_t* out, const int32_t* rows,
+                         const int32_t* positions, int n_items, int n_q, int window, int max_splits, int split_keys,
+                         int grid_splits, hipStream_t stream) {
+    const dim3 grid(n_q, n_items);
+    if (grid_splits <= 8)
+        hipLaunchKernelGGL(attention_decode_reduce_few_kernel<8>, grid, dim3(KIPP_WAVE), 0, stream, part_acc, part_ml, out,
+                           rows, positions, n_q, window, max_splits, split_keys, grid_splits);
+    else if (grid_splits <= 16)
+        hipLaunchKernelGGL(attention_decode_reduce_few_kernel<16>, grid, dim3(KIPP_WAVE), 0, stream, part_acc, part_ml, out,
+                           rows, positions, n_q, window, max_splits, split_keys, grid_splits);
+    else
+        hipLaunchKernelGGL(attention_decode_reduce_kernel, grid, dim3(HEAD_DIM >= 64 ? 64 : HEAD_DIM), 0, stream, part_acc,
+                           part_ml, out, rows, positions, n_q, window, max_splits, split_keys);
+    return KIPP_LAUNCH_CHECK();
+}
+
+
 #if RING_OK
 // Keys a workgroup of the kernel that streams through LDS walks in a launch of this shape; 0: the launch
 // is not for it.  Many sequences: whole contexts (RING_RANGE keys at most).  Few: ranges that give 256
@@ -1004,9 +1070,7 @@ static int launch_ring(const bf16_t* q, bf16_t* k_cache, bf16_t* v_cache, bf16_t
                        n_kv, page, scale_log2e, window, max_splits, range, pj);
     *rc = KIPP_LAUNCH_CHECK();
     if (*rc != 0 || ring_splits == 1) return 1;
-    hipLaunchKernelGGL(attention_decode_reduce_kernel, dim3(n_q, n_items), dim3(HEAD_DIM >= 64 ? 64 : HEAD_DIM), 0, stream,
-                       part_acc, part_ml, out, rows, positions, n_q, window, max_splits, range);
-    *rc = KIPP_LAUNCH_CHECK();
+    *rc = launch_reduce(part_acc, part_ml, (bf16_t*)out, rows, positions, n_items, n_q, window, max_splits, range, ring_splits, stream);
     return 1;
 }
 #endif
@@ -1057,9 +1121,7 @@ int kipp_attention_decode(const void* q, const void* k_cache, const void* v_cach
                            window, max_splits);
         int rc = KIPP_LAUNCH_CHECK();
         if (rc != 0 || big_splits == 1) return rc;
-        hipLaunchKernelGGL(attention_decode_reduce_kernel, dim3(n_q, n_items), dim3(HEAD_DIM >= 64 ? 64 : HEAD_DIM), 0,
-                           stream, part_acc, part_ml, (bf16_t*)out, rows, positions, n_q, window, max_splits, BIG);
-        return KIPP_LAUNCH_CHECK();
+        return launch_reduce(part_acc, part_ml, (bf16_t*)out, rows, positions, n_items, n_q, window, max_splits, BIG, big_splits, stream);
     }
     hipLaunchKernelGGL(attention_decode_kernel<false>, dim3(grid_splits, n_kv, n_items), dim3(THREADS), 0, stream,
                        (const bf16_t*)q, (bf16_t*)k_cache, (bf16_t*)v_cache, (bf16_t*)out, part_acc, part_ml,
@@ -1067,9 +1129,7 @@ int kipp_attention_decode(const void* q, const void* k_cache, const void* v_cach
                        max_splits, Projected{});
     int rc = KIPP_LAUNCH_CHECK();
     if (rc != 0 || grid_splits == 1) return rc;
-    hipLaunchKernelGGL(attention_decode_reduce_kernel, dim3(n_q, n_items), dim3(HEAD_DIM >= 64 ? 64 : HEAD_DIM), 0,
-                       stream, part_acc, part_ml, (bf16_t*)out, rows, positions, n_q, window, max_splits, SPLIT);
-    return KIPP_LAUNCH_CHECK();
+    return launch_reduce(part_acc, part_ml, (bf16_t*)out, rows, positions, n_items, n_q, window, max_splits, SPLIT, grid_splits, stream);
 }
 
 // 1 if this build has the fused kernel (head sizes that are multiples of 128).
@@ -1110,9 +1170,7 @@ int kipp_attention_decode_fused(const float* qkv, int parts, int n_tokens, const
                        max_splits, pj);
     int rc = KIPP_LAUNCH_CHECK();
     if (rc != 0 || grid_splits == 1) return rc;
-    hipLaunchKernelGGL(attention_decode_reduce_kernel, dim3(n_q, n_items), dim3(HEAD_DIM >= 64 ? 64 : HEAD_DIM), 0,
-                       stream, part_acc, part_ml, (bf16_t*)out, rows, positions, n_q, window, max_splits, SPLIT);
-    return KIPP_LAUNCH_CHECK();
+    return launch_reduce(part_acc, part_ml, (bf16_t*)out, rows, positions, n_items, n_q, window, max_splits, SPLIT, grid_splits, stream);
 #else
     return -5;
 #endif
