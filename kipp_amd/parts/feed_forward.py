@@ -12,6 +12,7 @@ from __future__ import annotations
 
 import torch
 
+from ..runtime import ScaledRows
 from .base import ParamSpec, register
 
 
@@ -50,7 +51,7 @@ class GatedMLP:
         ours = w.dtype == x.dtype == torch.bfloat16 and rt.ops.gemm_rows_ok(rows, x.shape[1])
         if ours and rows <= rt.ops.SKINNY_BEST_ROWS:
             # both products and the activation in one kernel (and the norm's scale, if it was left to us)
-            scaled = hasattr(x, "sumsq")
+            scaled = isinstance(x, ScaledRows)
             rt.ops.gemm_skinny_swiglu(x.rows if scaled else x, w.rows, act, tiles=w.tiles,
                                       row_scale=x.scale if scaled else None)
             return rt.linear(act, self.w_down, slabs=True, defer=True)

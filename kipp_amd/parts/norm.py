@@ -12,6 +12,7 @@ parts that do not say they take them.
 """
 from __future__ import annotations
 
+from ..runtime import Deferred
 from .base import ParamSpec, register
 
 
@@ -43,7 +44,7 @@ class RMSNorm:
         return self.rt.ops.rmsnorm(x, self.weight, self.spec.eps, self.rt.empty(x.shape, out_dtype))
 
     def add_forward(self, x, delta, out_dtype):
-        if not hasattr(delta, "shape"):       # a product not launched yet: add and norm ride on it where they can
+        if isinstance(delta, Deferred):       # a product not launched yet: add and norm ride on it where they can
             fused = self.rt.product_add_norm(delta, x, self.weight, self.spec.eps) if out_dtype == self.rt.act_dtype else None
             if fused is not None:
                 return fused
