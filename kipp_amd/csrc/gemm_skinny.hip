@@ -193,12 +193,18 @@ __global__ void __launch_bounds__(THREADS) gemm_skinny_kernel(
                 t += p + 2 < rs.parts ? scale_part[i].z : 0.0f;
                 t += p + 3 < rs.parts ? scale_part[i].w : 0.0f;
             }
-            for (int p = 4 * (h + 4 * SCALE_LOADS); p < rs.parts; p += 16) {   // wider rows: the rest one by one
-                const float4 more = *(const float4*)(scale_src + p);
-                t += more.x;
-                t += p + 1 < rs.parts ? more.y : 0.0f;
-                t += p + 2 < rs.parts ? more.z : 0.0f;
-                t += p + 3 < rs.parts ? more.w : 0.0f;
+            for (int p0 = 16 * SCALE_LOADS; p0 < rs.parts; p0 += 16 * SCALE_LOADS) {   // wider rows: as many again at a time
+                float4 more[SCALE_LOADS];
+#pragma unroll
+                for (int i = 0; i < SCALE_LOADS; ++i) more[i] = *(const float4*)(scale_src + min(p0 + 4 * (h + 4 * i), rs.stride - 4));
+#pragma unroll
+                for (int i = 0; i < SCALE_LOADS; ++i) {
+                    const int p = p0 + 4 * (h + 4 * i);
+                    t += p < rs.parts ? more[i].x : 0.0f;
+                    t += p + 1 < rs.parts ? more[i].y : 0.0f;
+                    t += p + 2 < rs.parts ? more[i].z : 0.0f;
+                    t += p + 3 < rs.parts ? more[i].w : 0.0f;
+                }
             }
             t += __shfl_xor(t, 16, KIPP_WAVE);     // the four lane groups of a token
             t += __shfl_xor(t, 32, KIPP_WAVE);

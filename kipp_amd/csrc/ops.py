@@ -478,6 +478,11 @@ def _row_scale_args(row_scale, m: int, what: str):
     return _ptr(sumsq), int(parts), float(eps)
 
 
+def gemm_skinny_parts(n: int, k: int, max_parts: int) -> int:
+    """Slabs `gemm_skinny` cuts a product against a weight [n, k] into when it may use up to `max_parts`."""
+    return build.library("gemm_skinny").kipp_gemm_skinny_parts(int(n), int(k), int(max_parts))
+
+
 def gemm_skinny(x: torch.Tensor, w: torch.Tensor, max_parts: int = 1, tiles: torch.Tensor = None,
                 row_scale=None, add_norm=None):
     """float32 [parts, M, N] whose sum over parts is x . w^T, for M <= 64 rows of

@@ -90,6 +90,8 @@ class Deferred:
 
 
 class Runtime:
+    FUSE_NORM_X_BYTES = 40e6    # most bytes of X the workgroups of an unsplit product may read together for the fused norm to pay
+
     def __init__(self, dtype: str = "bfloat16", device: str = "cuda:0", stream_layout: bool = True):
         if dtype not in DTYPES:
             raise ValueError(f"dtype must be one of {sorted(DTYPES)}, got {dtype!r}")
@@ -153,6 +155,14 @@ class Runtime:
         if not (self.fuse_norms and isinstance(w, Weight) and not w.pairs and delta.x.dtype == torch.bfloat16
                 and self._few_rows(rows, k, w) and x.dtype == torch.float32 and x.is_contiguous()
                 and norm_weight.dtype == torch.float32):
+            return None
+        # That kernel is not split over workgroups.  Where the product alone would be, each of its N / 16
+        # workgroups reads all of delta.x instead of a part of it, which costs more than the norm's kernel
+        # once that is some tens of megabytes (measured: 5120 x 8192 and 5120 x 25600 at 8 rows, +5.6 us
+        # each against 4.6 saved; at 4 rows and for narrower weights the fused form wins).
+        most = 1 if delta.slabs is False else (8 if delta.slabs is True else int(delta.slabs))
+        n_out = w.shape[0]
+        if self.ops.gemm_skinny_parts(n_out, k, most) > 1 and ((n_out + 15) // 16) * rows * k * 2 > self.FUSE_NORM_X_BYTES:
             return None
         rows_out, sumsq = self.ops.gemm_skinny(delta.x, w.rows, tiles=w.tiles, add_norm=(x, norm_weight))
         return ScaledRows(rows_out, sumsq, (w.shape[0] + 15) // 16, eps)

@@ -49,6 +49,35 @@ def test_benchmark_layer_sizes_match_plain(real_folder, real_reference, dtype):
         del engine
 
 
+def test_split_products_keep_their_norm_kernels(real_folder, real_reference):
+    """The residual add rides on a product only where that product need not be split over workgroups or
+    reads little of X; with the limit at zero the output and down projections of these sizes (which are
+    split) are launched as they are and every norm has its kernel again.  Both ways against the plain
+    implementation."""
+    from kipp_amd.engine import Engine
+    from kipp_amd.engine.model import load_model
+    from kipp_amd.runtime import Runtime
+    requests, refs = real_reference
+    steps = H.tail_one_by_one(requests, 12)
+    for limit in (0, None):
+        rt = Runtime("bfloat16")
+        if limit is not None:
+            rt.FUSE_NORM_X_BYTES = limit
+        fused = {"yes": 0, "no": 0}
+        inner = rt.product_add_norm
+
+        def counting(delta, x, weight, eps):
+            out = inner(delta, x, weight, eps)
+            fused["no" if out is None else "yes"] += 1
+            return out
+        rt.product_add_norm = counting
+        engine = Engine(load_model(real_folder, rt), page_size=16, max_tokens=512, share_prefixes=False, use_graphs=False)
+        got = H.replay(engine, requests, steps)
+        for rid in requests:
+            H.assert_close(got[rid], refs[rid], H.NMSE_BF16, f"4B sizes/limit {limit}/{rid}")
+        assert (fused["yes"] == 0 and fused["no"] > 0) if limit == 0 else (fused["yes"] > 0 and fused["no"] == 0), fused
+
+
 @pytest.fixture(scope="module")
 def long_folder(tmp_path_factory):
     """Head size 128 and a long context on a narrow model: decoding runs through the
