@@ -328,7 +328,7 @@ def test_routed_feed_forward_and_another_position_encoding(tmp_path, cut):
 
 
 # ---------------------------------------------------------------------------------------------
-# A norm of another kind between the framework's own parts, in bfloat16: with few rows the framework's
+# A norm and a feed-forward of other kinds between the framework's own parts, in bfloat16: with few rows the framework's
 # products come back not yet launched and its norm leaves its scale to the next product; a norm that
 # knows nothing of either gets tensors, and the parts behind it work as before.
 
@@ -338,6 +338,14 @@ class MeanAbsNormSpec:
     eps: float
     prefix: str = ""
     kind: str = "toy_mean_abs"
+
+
+@dataclass(frozen=True)
+class ReluMLPSpec:
+    hidden_size: int
+    inner: int
+    prefix: str = ""
+    kind: str = "toy_relu_mlp"
 
 
 def _register_mean_abs():
@@ -372,6 +380,25 @@ def _register_mean_abs():
             x += delta.sum(dim=0) if delta.dim() == 3 else delta
             return self.forward(x, out_dtype)
 
+    @register("feed_forward", "toy_relu_mlp")
+    class ReluMLP:
+        """delta = W2 relu(W1 x).  It does not declare `takes_scaled_rows`: the block hands it finished rows."""
+
+        def __init__(self, spec, runtime):
+            self.spec, self.rt = spec, runtime
+
+        @staticmethod
+        def params(spec):
+            return {"w1.weight": ParamSpec((spec.inner, spec.hidden_size)), "w2.weight": ParamSpec((spec.hidden_size, spec.inner))}
+
+        def load(self, tensors):
+            self.t = tensors
+
+        def forward(self, x, batch=None):
+            assert isinstance(x, torch.Tensor), "a feed-forward that does not declare takes_scaled_rows gets tensors"
+            h = torch.relu(self.rt.linear(x, self.t["w1.weight"])).to(x.dtype).contiguous()
+            return self.rt.linear(h, self.t["w2.weight"])
+
     class MeanAbsConfig:
         def __init__(self, d):
             self.d = d
@@ -383,11 +410,16 @@ def _register_mean_abs():
             def layer(i):
                 p = f"layers.{i}."
                 attn = AttentionSpec(M_HIDDEN, 4, 2, 32, position=RopeSpec(32, THETA), qk_norm_eps=EPS, prefix=p + "attn.")
+                if i == 2:      # the framework's norm in front of a feed-forward of another kind
+                    return LayerSpec(block="pre_norm", parts=(
+                        ("mixer_norm", RMSNormSpec(M_HIDDEN, EPS, p + "n1.")), ("mixer", attn),
+                        ("ffn_norm", RMSNormSpec(M_HIDDEN, EPS, p + "n2.")), ("ffn", ReluMLPSpec(M_HIDDEN, M_INNER, p + "mlp."))))
                 return LayerSpec(block="pre_norm", parts=(
                     ("mixer_norm", RMSNormSpec(M_HIDDEN, EPS, p + "n1.")), ("mixer", attn),
                     ("ffn_norm", MeanAbsNormSpec(M_HIDDEN, EPS, p + "n2.")), ("ffn", GatedMLPSpec(M_HIDDEN, M_INNER, prefix=p + "mlp."))))
             return ModelSpec("ToyMeanAbsForTests", M_HIDDEN, VOCAB, 256, EmbeddingSpec(VOCAB, M_HIDDEN, "embed."),
-                             (layer(0), layer(1)), (LayerRun(0), LayerRun(1)), MeanAbsNormSpec(M_HIDDEN, EPS, "norm."),
+                             (layer(0), layer(1), layer(2)), (LayerRun(0), LayerRun(1), LayerRun(2)),
+                             MeanAbsNormSpec(M_HIDDEN, EPS, "norm."),
                              HeadSpec(VOCAB, M_HIDDEN, True))
 
     register_architecture("ToyMeanAbsForTests", MeanAbsConfig)
@@ -401,7 +433,7 @@ def _plain_mean_abs(w, tokens):
         return x / (np.abs(x).mean(axis=-1, keepdims=True) + EPS) * weight
     pos = np.arange(len(tokens))
     x = plain.embed(w["embed.weight"], tokens)
-    for i in range(2):
+    for i in range(3):
         p = f"layers.{i}."
         n = plain.rms_norm(x, w[p + "n1.weight"], EPS)
         q = plain.head_norm(plain.linear(n, w[p + "attn.q_proj.weight"]), 4, 32, w[p + "attn.q_norm.weight"], EPS)
@@ -409,6 +441,10 @@ def _plain_mean_abs(w, tokens):
         q, k = plain.rope(q, 4, 32, pos, THETA), plain.rope(k, 2, 32, pos, THETA)
         v = plain.linear(n, w[p + "attn.v_proj.weight"])
         x = x + plain.linear(plain.causal_gqa(q, k, v, 4, 2, 32), w[p + "attn.o_proj.weight"])
+        if i == 2:
+            n = plain.rms_norm(x, w[p + "n2.weight"], EPS)
+            x = x + plain.linear(np.maximum(plain.linear(n, w[p + "mlp.w1.weight"]), 0.0), w[p + "mlp.w2.weight"])
+            continue
         n = mean_abs(x, w[p + "n2.weight"])
         x = x + plain.swiglu_mlp(n, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
     return plain.linear(mean_abs(x, w["norm.weight"]), w["embed.weight"])
@@ -430,7 +466,13 @@ def test_another_norm_between_products_that_fuse_theirs(tmp_path, cut):
         engine = Engine.from_folder(folder, dtype="bfloat16", page_size=8, max_tokens=256, max_requests=4)
         # the framework's parts did fuse where they met each other: the second layer's first norm got a product
         # that was not launched yet and handed rows without their scale to the attention
-        seen = {"deferred": 0, "scaled": 0}
+        seen = {"deferred": 0, "scaled": 0, "finished": 0}
+        inner_rows = engine.model.rt.rows_of
+
+        def rows_of(h):
+            seen["finished"] += isinstance(h, ScaledRows)
+            return inner_rows(h)
+        engine.model.rt.rows_of = rows_of
         norm1, mixer = engine.model.blocks[1].parts["mixer_norm"], engine.model.blocks[1].parts["mixer"]
         inner_add, inner_mix = norm1.add_forward, mixer.forward
 
@@ -445,7 +487,9 @@ def test_another_norm_between_products_that_fuse_theirs(tmp_path, cut):
         got = H.replay(engine, requests, steps)
         for rid, toks in requests.items():
             H.assert_close(got[rid], _plain_mean_abs(weights, toks), H.NMSE_BF16, f"mean-abs norm/{cut}/{rid}")
-        assert seen["deferred"] > 0 and seen["scaled"] > 0, seen
+        # and the block finished the rows of the framework's norm for the feed-forward of another kind
+        assert seen["deferred"] > 0 and seen["scaled"] > 0 and seen["finished"] > 0, seen
     finally:
         unregister_architecture("ToyMeanAbsForTests")
         unregister("norm", "toy_mean_abs")
+        unregister("feed_forward", "toy_relu_mlp")
