@@ -55,6 +55,7 @@ class RequestCache:
     publish_early: bool = False                             # full pages are published as soon as they are committed
     published: int = 0                                      # leading blocks that are adopted or published
     chain: int = 0                                          # chained hash after `published` blocks
+    serial: int = 0                                         # unique among all requests the manager ever opened (ids may come again)
 
 
 class CacheGroup:
@@ -101,6 +102,7 @@ class CacheManager:
         self.share = share_prefixes and not self.state_needs and all(g.need.window is None for g in self.groups)
         self.free_slots = list(range(max_requests - 1, -1, -1))
         self.requests: Dict[object, RequestCache] = {}
+        self._serial = 0
         if runtime is not None:
             self._allocate_device()
 
@@ -158,8 +160,9 @@ class CacheManager:
         slot = self.free_slots.pop()
         for tensor in self.states.values():
             tensor[slot].zero_()
+        self._serial += 1
         req = RequestCache(request_id, slot, tables=[[] for _ in self.groups], adopted=[0 for _ in self.groups],
-                           rows=[np.zeros(self.max_blocks, dtype=np.int32) for _ in self.groups])
+                           rows=[np.zeros(self.max_blocks, dtype=np.int32) for _ in self.groups], serial=self._serial)
         if self.share and prompt is not None and self.groups:
             matches = [g.pool.prefix_match(prompt) for g in self.groups]
             keep = min(len(pages) for pages, _ in matches)

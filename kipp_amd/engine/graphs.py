@@ -106,7 +106,8 @@ class DecodeGraph:
         changed = False
         for i in range(n):
             r = requests[i] if i < live else None
-            mark = (r.id, r.table_version) if r is not None else "fills up"
+            # the serial, not the id: an id that was closed and opened again names another request with other pages
+            mark = (r.serial, r.table_version) if r is not None else "fills up"
             if self.row_marks[i] != mark:
                 self.row_marks[i] = mark
                 changed = True

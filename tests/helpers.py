@@ -2,6 +2,7 @@
 step function, comparison with the plain implementation."""
 from __future__ import annotations
 
+import os
 import random
 from typing import Dict, List, Sequence, Tuple
 
@@ -14,11 +15,13 @@ from tests.plain import qwen3_plain as plain
 # plain implementation on the same (already rounded) weights: activations are
 # rounded to 8 bits of mantissa a few times per layer.
 NMSE_F32 = 1e-10
-NMSE_BF16 = 1e-3
-# Observed (worst position): float32 2e-13 .. 3e-13; bfloat16 2e-5 .. 3e-5 at the tiny sizes and 1e-4 at
-# the benchmark's layer sizes.  The reference's own bound for its GPU backends, 1e-4
-# (/root/reference/tests/kipp_test.c:2733-2743), is for float32 activations; here activations between
-# kernels are bfloat16, each rounding adding about 3e-6.
+# bfloat16, per kind of configuration, about three times the worst value observed over all tests of that kind
+# (worst position of any request): 2e-5 .. 4.3e-5 at the tiny sizes, 1.02e-4 at the benchmark's layer sizes.  The
+# reference's own bound for its GPU backends, 1e-4 (/root/reference/tests/kipp_test.c:2733-2743), is for
+# float32 activations; here activations between kernels are bfloat16, each rounding adding about 3e-6, and
+# more so the wider the layers.
+NMSE_BF16 = {"tiny": 1e-4, "real": 3e-4}
+NMSE_LOG = os.environ.get("KIPP_NMSE_LOG")       # a file that collects "what<TAB>worst NMSE" of every comparison
 
 
 def random_tokens(seed: int, n: int, vocab: int) -> List[int]:
@@ -143,4 +146,7 @@ def assert_close(got: np.ndarray, ref: np.ndarray, tol: float, what: str) -> Non
         e = plain.nmse(got[i], ref[i])
         if e > worst:
             worst, worst_at = e, i
+    if NMSE_LOG:
+        with open(NMSE_LOG, "a") as f:
+            f.write(f"{what}\t{worst:.3e}\t{tol:.1e}\n")
     assert worst <= tol, f"{what}: NMSE {worst:.3e} at position {worst_at} exceeds {tol:.1e}"

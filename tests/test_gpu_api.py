@@ -129,3 +129,46 @@ def test_published_prefix_is_adopted_and_a_small_pool_fails_cleanly(model_folder
     stateless = m.eval(toks[:20])
     H.assert_close(stateless[None], ref[19:20], H.NMSE_F32, "stateless evaluation")
     m.close()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_session_that_is_reset_decodes_over_its_new_pages(model_folders, dtype):
+    """A request id that is closed and opened again names a new request with other pages.  Single-token
+    steps keep their block tables on the device from step to step and copy a row only when it changed:
+    the row of the old request must not serve the new one."""
+    from kipp_amd.api import Model
+    folder = model_folders[("b", dtype)]
+    tol = H.NMSE_F32 if dtype == "float32" else H.NMSE_BF16["tiny"]
+    m = Model.open(folder, dtype=dtype, kv_pool_blocks=64, page_tokens=8)
+    first, second = H.random_tokens(70, 30, 509), H.random_tokens(71, 30, 509)
+    ref_first, ref_second = H.plain_logits(folder, first), H.plain_logits(folder, second)
+    s = m.session_create(64)
+    s.eval(first[:20])
+    for i in range(20, 26):
+        H.assert_close(s.eval([first[i]])[None], ref_first[i:i + 1], tol, f"first timeline, position {i}")
+    pages_before = list(s._req.tables[0])
+    s.reset()
+    s.eval(second[:20])
+    assert list(s._req.tables[0]) != pages_before       # the case the test is for: same id, other pages
+    for i in range(20, 30):
+        H.assert_close(s.eval([second[i]])[None], ref_second[i:i + 1], tol, f"after reset, position {i}")
+    s.destroy()
+    m.close()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_two_generations_on_one_engine(model_folders, dtype):
+    """The second run's requests take rows of recorded steps that the first run's requests held."""
+    from kipp_amd import generate
+    from kipp_amd.engine import Engine
+    from tests.test_gpu_entry import _follows_plain_argmax
+    folder = model_folders[("a", dtype)]
+    engine = Engine.from_folder(folder, dtype=dtype, page_size=16, max_tokens=1024, share_prefixes=False)
+    margin = 1e-5 if dtype == "float32" else 0.03
+    for run in range(3):
+        prompts = [H.random_tokens(300 + 10 * run + i, n, 256) for i, n in enumerate([7 + run, 21, 3])]
+        outputs = generate(engine, prompts, max_new_tokens=12)
+        for prompt, out in zip(prompts, outputs):
+            assert len(out) == 12
+            _follows_plain_argmax(folder, prompt, out, margin)
+    engine.cache.check()

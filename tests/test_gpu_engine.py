@@ -28,7 +28,7 @@ def _requests(key, cfg, seed=0):
 def test_cuttings_match_plain(model_folders, tiny_configs, key, dtype, cut):
     cfg = tiny_configs[key]
     requests = _requests(key, cfg)
-    tol = H.NMSE_F32 if dtype == "float32" else H.NMSE_BF16
+    tol = H.NMSE_F32 if dtype == "float32" else H.NMSE_BF16["tiny"]
     if cut == "mixed":
         more = {f"s{i}": H.random_tokens(900 + i, n, cfg["vocab_size"]) for i, n in enumerate(LENGTHS[key])}
         requests = {**requests, **more}
@@ -77,7 +77,7 @@ def test_without_the_streaming_layout(model_folders, tiny_configs, key):
         assert all(block.parts["ffn"].w_gate_up.tiles is None for block in engine.model.blocks)
         got = H.replay(engine, requests, steps)
         for rid, toks in requests.items():
-            H.assert_close(got[rid], H.plain_logits(folder, toks), H.NMSE_BF16, f"{key}/rows only/{rid}")
+            H.assert_close(got[rid], H.plain_logits(folder, toks), H.NMSE_BF16["tiny"], f"{key}/rows only/{rid}")
 
 
 @pytest.mark.parametrize("key", ["a", "b"])
@@ -110,5 +110,5 @@ def test_norms_in_kernels_of_their_own(model_folders, tiny_configs, key):
         engine = Engine(load_model(folder, rt), page_size=PAGE[key], max_tokens=512, share_prefixes=False, use_graphs=False)
         got = H.replay(engine, requests, steps)
         for rid, toks in requests.items():
-            H.assert_close(got[rid], H.plain_logits(folder, toks), H.NMSE_BF16, f"{key}/fused norms {fuse}/{rid}")
+            H.assert_close(got[rid], H.plain_logits(folder, toks), H.NMSE_BF16["tiny"], f"{key}/fused norms {fuse}/{rid}")
         assert (calls["delta"] == 0) == fuse, calls

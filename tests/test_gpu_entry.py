@@ -150,7 +150,7 @@ def test_long_decoding_matches_plain(model_folders, tiny_configs):
 def test_first_tokens_of_a_sequence(model_folders):
     """Positions 0, 1, 2 each as a step of their own: the empty-cache edge."""
     from kipp_amd.engine import Engine, StepEntry
-    for dtype, tol in (("float32", H.NMSE_F32), ("bfloat16", H.NMSE_BF16)):
+    for dtype, tol in (("float32", H.NMSE_F32), ("bfloat16", H.NMSE_BF16["tiny"])):
         folder = model_folders[("a", dtype)]
         engine = Engine.from_folder(folder, dtype=dtype, page_size=16, max_tokens=64)
         toks = [200, 3, 77]
@@ -258,6 +258,6 @@ def test_trace_run(model_folders, tiny_configs, tmp_path, dtype):
             rows[rid].append(data[at:at + n])
             at += n
         assert at == data.shape[0]
-    tol = H.NMSE_F32 if dtype == "float32" else H.NMSE_BF16
+    tol = H.NMSE_F32 if dtype == "float32" else H.NMSE_BF16["tiny"]
     for rid, toks in requests.items():
         H.assert_close(np.concatenate(rows[rid]), H.plain_logits(folder, toks), tol, f"trace {dtype} {rid}")

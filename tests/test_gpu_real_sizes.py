@@ -36,7 +36,7 @@ def real_reference(real_folder):
 def test_benchmark_layer_sizes_match_plain(real_folder, real_reference, dtype):
     from kipp_amd.engine import Engine
     requests, refs = real_reference
-    tol = H.NMSE_F32 if dtype == "float32" else H.NMSE_BF16
+    tol = H.NMSE_F32 if dtype == "float32" else H.NMSE_BF16["real"]
     for cut, maker in (("whole", H.whole), ("tail", lambda r: H.tail_one_by_one(r, 20)), ("mixed", lambda r: H.mixed(r, seed=4))):
         steps = maker(requests)
         engine = Engine.from_folder(real_folder, dtype=dtype, page_size=16, num_pages=H.peak_pages(requests, steps, 16),
@@ -74,7 +74,7 @@ def test_split_products_keep_their_norm_kernels(real_folder, real_reference):
         engine = Engine(load_model(real_folder, rt), page_size=16, max_tokens=512, share_prefixes=False, use_graphs=False)
         got = H.replay(engine, requests, steps)
         for rid in requests:
-            H.assert_close(got[rid], refs[rid], H.NMSE_BF16, f"4B sizes/limit {limit}/{rid}")
+            H.assert_close(got[rid], refs[rid], H.NMSE_BF16["real"], f"4B sizes/limit {limit}/{rid}")
         assert (fused["yes"] == 0 and fused["no"] > 0) if limit == 0 else (fused["yes"] > 0 and fused["no"] == 0), fused
 
 
@@ -102,7 +102,7 @@ def test_decoding_across_a_graph_bucket_and_many_splits(long_folder, dtype):
     cfg, weights = plain.load_folder(long_folder)
     seqs = {"long": H.random_tokens(31, 1060, 311), "mid": H.random_tokens(32, 300, 311), "short": H.random_tokens(33, 40, 311)}
     refs = {k: plain.forward_whole(cfg, weights, v) for k, v in seqs.items()}
-    tol = H.NMSE_F32 if dtype == "float32" else H.NMSE_BF16
+    tol = H.NMSE_F32 if dtype == "float32" else H.NMSE_BF16["real"]
     engine = Engine.from_folder(long_folder, dtype=dtype, page_size=16, max_tokens=1088 + 320 + 64, max_requests=3,
                                 share_prefixes=False)
     fed = {"long": 1000, "mid": 240, "short": 10}
@@ -148,7 +148,7 @@ def test_many_requests_decode_together(long_folder, dtype, n_requests):
     assert engine.graphs.replays >= 4
     from kipp_amd.csrc import ops
     assert ops.attention_decode_streams(n_requests, 1, 128, 4, 16, 64) == (n_requests >= 96)
-    tol = H.NMSE_F32 if dtype == "float32" else H.NMSE_BF16
+    tol = H.NMSE_F32 if dtype == "float32" else H.NMSE_BF16["real"]
     for rid in list(seqs)[::10]:
         ref = plain.forward_whole(cfg, weights, seqs[rid])
         H.assert_close(np.stack(got[rid]), ref[len(seqs[rid]) - 6:], tol, f"{n_requests} together/{dtype}/{rid}")
@@ -177,7 +177,7 @@ def test_a_batch_whose_size_changes_replays_one_graph(long_folder, dtype):
             got[rid].append(row)
             fed[rid] += 1
     assert len(engine.graphs.graphs) == 1 and engine.graphs.replays >= 11
-    tol = H.NMSE_F32 if dtype == "float32" else H.NMSE_BF16
+    tol = H.NMSE_F32 if dtype == "float32" else H.NMSE_BF16["real"]
     for rid, toks in seqs.items():
         ref = plain.forward_whole(cfg, weights, toks)
         first = len(toks) - 14

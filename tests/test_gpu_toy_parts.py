@@ -486,7 +486,7 @@ def test_another_norm_between_products_that_fuse_theirs(tmp_path, cut):
         norm1.add_forward, mixer.forward = add_forward, forward
         got = H.replay(engine, requests, steps)
         for rid, toks in requests.items():
-            H.assert_close(got[rid], _plain_mean_abs(weights, toks), H.NMSE_BF16, f"mean-abs norm/{cut}/{rid}")
+            H.assert_close(got[rid], _plain_mean_abs(weights, toks), H.NMSE_BF16["tiny"], f"mean-abs norm/{cut}/{rid}")
         # and the block finished the rows of the framework's norm for the feed-forward of another kind
         assert seen["deferred"] > 0 and seen["scaled"] > 0 and seen["finished"] > 0, seen
     finally:
