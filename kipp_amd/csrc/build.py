@@ -1,7 +1,7 @@
 """Compile the HIP sources for gfx950 and load them with ctypes.
 
 Each `.hip` file becomes one shared library under `_lib/`; the file name holds
-a hash of the source, the shared header, the flags and the specialisation
+a hash of the source, the shared headers, the flags and the specialisation
 constants, so a changed source is never served by a stale library.  A library
 is compiled at its first use if it is not there (a line is printed when that
 starts and every few seconds until it ends); `build_all` compiles a list in
@@ -72,7 +72,8 @@ def library_path(name: str, defines: Optional[dict] = None) -> Tuple[str, list, 
         raise BuildError(f"no kernel source {src}")
     tag, dflags = _defines_tag(defines)
     h = hashlib.sha1()
-    for path in (src, os.path.join(HERE, "common.h")):
+    headers = sorted(f for f in os.listdir(HERE) if f.endswith(".h"))
+    for path in [src] + [os.path.join(HERE, f) for f in headers]:
         with open(path, "rb") as f:
             h.update(f.read())
     h.update(" ".join(FLAGS + dflags).encode())

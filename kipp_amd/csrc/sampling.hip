@@ -125,6 +125,49 @@ extern "C" int kipp_argmax(const float* logits, int32_t* out, int rows, int voca
 }
 
 // ---------------------------------------------------------------------------------------
+// The same choice for callers that cannot allocate (declared in no_alloc.h).  The partial
+// results of the two-stage form live in a file-scope device array instead of a buffer the
+// caller brings.  Every GPU holds its own copy of the array at its own address: in host code
+// the array's name is only a stand-in, so its address on the current device is looked up
+// once per device and that pointer is what the kernels get.
+#include "no_alloc.h"
+
+static __device__ __align__(256) unsigned char scratch[KIPP_ARGMAX_STATIC_MAX_ROWS * ARGMAX_CHUNKS * 2 * 4];
+
+#define KIPP_MAX_DEVICES 64
+static void* scratch_of_device[KIPP_MAX_DEVICES];   // the array's address on each device, once looked up
+
+static int static_scratch(float** ptr) {
+    int device = -1;
+    hipError_t err = hipGetDevice(&device);
+    if (err != hipSuccess) return (int)err;
+    if (device < 0 || device >= KIPP_MAX_DEVICES) return -3;
+    void* p = __atomic_load_n(&scratch_of_device[device], __ATOMIC_ACQUIRE);
+    if (p == nullptr) {
+        err = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (err != hipSuccess) return (int)err;
+        if (p == nullptr) return -4;
+        __atomic_store_n(&scratch_of_device[device], p, __ATOMIC_RELEASE);   // two first callers store the same address
+    }
+    *ptr = (float*)p;
+    return 0;
+}
+
+extern "C" int kipp_argmax_static_max_rows(void) { return KIPP_ARGMAX_STATIC_MAX_ROWS; }
+
+extern "C" int kipp_argmax_static(const float* logits, int32_t* out, int rows, int vocab, hipStream_t stream) {
+    if (rows <= 0) return 0;
+    if (vocab <= 0 || logits == nullptr || out == nullptr) return -1;
+    if (rows > KIPP_ARGMAX_STATIC_MAX_ROWS) return -2;      // beyond what the array holds: refused, nothing launched
+    float* ptr = nullptr;
+    const int rc = static_scratch(&ptr);
+    if (rc != 0) return rc;
+    // every slot that the second kernel reads is written by the first one of the same call,
+    // so nothing of an earlier call has to be cleared
+    return kipp_argmax(logits, out, rows, vocab, ptr, stream);
+}
+
+// ---------------------------------------------------------------------------------------
 // Temperature sampling with top-k, min-p and top-p, one workgroup per row, with the
 // meaning of the host sampler (/root/reference/src/kipp.c:3433-3559): scale by 1/T,
 // keep candidates within 20 of the maximum, order them by descending logit (ties: lower
