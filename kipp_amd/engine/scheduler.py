@@ -130,6 +130,12 @@ class Scheduler:
 
     # -- interface -------------------------------------------------------------------
     def add(self, req: Request) -> None:
+        # an id names one request at a time: a second one would fail at admission, stay first in line
+        # and block the queue for good, and its result would replace the first one's
+        if (req.id in self.cache.requests or req.id in self.finished
+                or any(other.id == req.id for other in self.waiting) or any(other.id == req.id for other in self.running)):
+            self.stats.refused += 1
+            raise RequestRefused(f"request id {req.id!r} is already waiting, running, open in the engine, or finished and not collected")
         if len(req.prompt) == 0:
             raise RequestRefused(f"request {req.id!r}: empty prompt")
         if req.max_new_tokens < 0:

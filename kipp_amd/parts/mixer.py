@@ -126,12 +126,13 @@ class Attention:
         return rt.linear(out, self.w_o, slabs=True, defer=True)
 
     def _workspace(self, batch):
-        """Partial results of the split decode kernel, kept while they are large enough."""
+        """Partial results of the split decode kernel, shared by the layers of one geometry and kept
+        while the batch object lives (a recorded step keeps its own)."""
         s = self.spec
-        key = (batch.n_decode, batch.max_decode_ctx)
-        ws = batch.host.get("decode_workspace")
-        if ws is None or ws[0] != key:
-            ws = (key, self.rt.ops.attention_decode_workspace(batch.n_decode, s.num_heads, s.head_dim,
-                                                              batch.max_decode_ctx, self.rt.device))
-            batch.host["decode_workspace"] = ws
-        return ws[1]
+        key = ("decode_workspace", batch.n_decode, batch.max_decode_ctx, s.num_heads, s.head_dim)
+        ws = batch.host.get(key)
+        if ws is None:
+            ws = self.rt.ops.attention_decode_workspace(batch.n_decode, s.num_heads, s.head_dim,
+                                                        batch.max_decode_ctx, self.rt.device)
+            batch.host[key] = ws
+        return ws

@@ -115,7 +115,7 @@ def sample(logits: np.ndarray, params: SampleParams, rng: XorShift64Star | None,
     if params.temperature <= 0.0:
         return best
     params.validate()
-    if rng is None:
+    if rng is None or rng.state == 0:      # /root/reference/src/kipp.c:3477-3480
         raise ValueError("sampling requires a nonzero RNG state")
     inverse_temperature = np.float32(1.0) / np.float32(params.temperature)
     scaled = values * inverse_temperature                      # float32

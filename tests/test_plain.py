@@ -181,3 +181,116 @@ def test_whole_model_closed_form_and_invariants():
     # the reference rounds keys and values to bfloat16; that changes logits a little, not a lot
     rounded = P.forward_whole(cfg, w, tokens, kv_round=P.bf16_round)
     assert 0 < P.nmse(rounded, base) < 1e-4
+
+
+def test_swiglu_vector_and_which_side_goes_through_silu():
+    # /root/reference/tests/kipp_test.c:130-132: gate 1, up 2 -> silu(1) * 2 = 1.4621172, here through 1 x 1 weights
+    one = np.ones((1, 1))
+    assert abs(P.swiglu_mlp(np.array([[1.0]]), one, 2 * one, one)[0, 0] - 1.4621172) < 1e-6
+    # the other way round it would be silu(2) * 1 = 1.7615942
+    assert abs(P.swiglu_mlp(np.array([[1.0]]), 2 * one, one, one)[0, 0] - 1.7615942) < 1e-6
+    # the delta is linear in W_up and not in W_gate
+    rng = np.random.default_rng(5)
+    x, wg, wu, wd = rng.normal(size=(3, 6)), rng.normal(size=(10, 6)), rng.normal(size=(10, 6)), rng.normal(size=(6, 10))
+    base = P.swiglu_mlp(x, wg, wu, wd)
+    assert np.allclose(P.swiglu_mlp(x, wg, 2 * wu, wd), 2 * base, rtol=1e-12)
+    assert not np.allclose(P.swiglu_mlp(x, 2 * wg, wu, wd), 2 * base, rtol=1e-3)
+    # a gate of zero closes the unit whatever the up side holds
+    assert np.array_equal(P.swiglu_mlp(x, np.zeros_like(wg), wu, wd), np.zeros((3, 6)))
+
+
+def test_block_arrangement():
+    """Which norm feeds which half of a block, and that the residual itself is never normed."""
+    cfg, w = _tiny(seed=3)
+    cfg = dict(cfg, num_hidden_layers=1)
+    tokens = [3, 17, 3, 44, 9, 21]
+    p = "model.layers.0."
+    emb = w["model.embed_tokens.weight"][tokens]
+    _, hidden = P.forward_whole(cfg, w, tokens, return_hidden=True)
+    # input_layernorm feeds the attention and nothing else: with its weight at zero q, k and v are zero, so is
+    # the attention's delta, and what is left is x + mlp(norm(x, post_attention_layernorm)) of the plain embedding
+    w_in0 = dict(w)
+    w_in0[p + "input_layernorm.weight"] = np.zeros(24)
+    _, h_in0 = P.forward_whole(cfg, w_in0, tokens, return_hidden=True)
+    mlp_only = emb + P.swiglu_mlp(P.rms_norm(emb, w[p + "post_attention_layernorm.weight"], 1e-5),
+                                  w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+    assert np.allclose(h_in0, mlp_only, rtol=1e-12)
+    # post_attention_layernorm feeds the feed-forward and nothing else: with its weight at zero the feed-forward's
+    # delta is zero (silu(0) * 0), and the hidden state is the one of the same model with a zero down projection
+    w_post0, w_down0 = dict(w), dict(w)
+    w_post0[p + "post_attention_layernorm.weight"] = np.zeros(24)
+    w_down0[p + "mlp.down_proj.weight"] = np.zeros((24, 40))
+    _, h_post0 = P.forward_whole(cfg, w_post0, tokens, return_hidden=True)
+    _, h_down0 = P.forward_whole(cfg, w_down0, tokens, return_hidden=True)
+    assert np.array_equal(h_post0, h_down0) and not np.allclose(h_post0, emb)     # the attention's delta is still there
+    # the feed-forward reads the residual AFTER the attention's delta was added: its own delta differs from the
+    # one it would give on the embedding alone
+    assert not np.allclose(hidden - h_down0, mlp_only - emb, rtol=1e-3)
+    # pre-norm: a norm's weight reaches the residual only through its half's delta.  Scaling post_attention_layernorm
+    # by c is the same as scaling the columns of W_gate and W_up by c (the delta is linear in W_up's input side)
+    w_c, w_cols = dict(w), dict(w)
+    w_c[p + "post_attention_layernorm.weight"] = 1.7 * w[p + "post_attention_layernorm.weight"]
+    w_cols[p + "mlp.gate_proj.weight"] = 1.7 * w[p + "mlp.gate_proj.weight"]
+    w_cols[p + "mlp.up_proj.weight"] = 1.7 * w[p + "mlp.up_proj.weight"]
+    assert np.allclose(P.forward_whole(cfg, w_c, tokens), P.forward_whole(cfg, w_cols, tokens), rtol=1e-12)
+    # ... and scaling input_layernorm by c is the same as scaling W_q, W_k and W_v by c
+    w_c, w_cols = dict(w), dict(w)
+    w_c[p + "input_layernorm.weight"] = 0.6 * w[p + "input_layernorm.weight"]
+    for name in ("q_proj", "k_proj", "v_proj"):
+        w_cols[p + f"self_attn.{name}.weight"] = 0.6 * w[p + f"self_attn.{name}.weight"]
+    assert np.allclose(P.forward_whole(cfg, w_c, tokens), P.forward_whole(cfg, w_cols, tokens), rtol=1e-12)
+    # the final norm is applied once, after the last block, with model.norm.weight
+    assert np.allclose(P.forward_whole(cfg, w, tokens), P.rms_norm(hidden, w["model.norm.weight"], 1e-5)
+                       @ w["model.embed_tokens.weight"].T, rtol=1e-12)
+
+
+def test_q_norm_and_k_norm_are_not_interchangeable():
+    """q_norm.weight belongs to the queries.  With it at zero on the upper half of a head, the upper halves of
+    the (normed) queries vanish, so flipping the sign of those rows of W_q changes nothing (a sign leaves the
+    norm's scale alone), while the same flip in W_k does; were the two weights applied the other way round,
+    it would be the flip in W_q that shows."""
+    cfg, w = _tiny(seed=4)
+    cfg = dict(cfg, num_hidden_layers=1)
+    tokens = [7, 1, 30, 30, 12, 5, 48]
+    p = "model.layers.0.self_attn."
+    rng = np.random.default_rng(6)
+    w = dict(w)
+    w[p + "q_norm.weight"] = np.concatenate([1 + 0.3 * rng.normal(size=8), np.zeros(8)])
+    w[p + "k_norm.weight"] = 1 + 0.3 * rng.normal(size=16)
+    base = P.forward_whole(cfg, w, tokens)
+    upper = np.tile(np.concatenate([np.ones(8), -np.ones(8)]), 3)        # 3 query heads of 16
+    flipped_q, flipped_k = dict(w), dict(w)
+    flipped_q[p + "q_proj.weight"] = w[p + "q_proj.weight"] * upper[:, None]
+    flipped_k[p + "k_proj.weight"] = w[p + "k_proj.weight"] * upper[:16, None]
+    assert np.allclose(P.forward_whole(cfg, flipped_q, tokens), base, rtol=1e-12)
+    assert not np.allclose(P.forward_whole(cfg, flipped_k, tokens), base, rtol=1e-3)
+    # and the mirror image pins k_norm.weight to the keys
+    w[p + "q_norm.weight"], w[p + "k_norm.weight"] = w[p + "k_norm.weight"], w[p + "q_norm.weight"]
+    base = P.forward_whole(cfg, w, tokens)
+    flipped_q, flipped_k = dict(w), dict(w)
+    flipped_q[p + "q_proj.weight"] = w[p + "q_proj.weight"] * upper[:, None]
+    flipped_k[p + "k_proj.weight"] = w[p + "k_proj.weight"] * upper[:16, None]
+    assert np.allclose(P.forward_whole(cfg, flipped_k, tokens), base, rtol=1e-12)
+    assert not np.allclose(P.forward_whole(cfg, flipped_q, tokens), base, rtol=1e-3)
+
+
+def test_the_second_plain_implementation_agrees(model_folders):
+    """Scalar loops over tokens, heads and sources with a running cache, written on its own
+    (`tests/plain/qwen3_loops.py`), against the whole-sequence NumPy form, on both tiny configurations
+    (float32 and bfloat16 files): relative difference below 1e-12 at every logit's scale."""
+    from tests.plain import qwen3_loops as L
+    for (key, dtype), folder in sorted(model_folders.items()):
+        cfg, weights = P.load_folder(folder)
+        cfg2, weights2 = L.read_folder(folder)
+        assert cfg2 == cfg and sorted(weights2) == sorted(weights)
+        assert all(np.array_equal(weights[name], weights2[name]) for name in weights)
+        vocab = cfg["vocab_size"]
+        tokens = [int(t) for t in np.random.default_rng(11).integers(0, vocab, size=19)]
+        a, b = P.forward_whole(cfg, weights, tokens), L.forward(cfg2, weights2, tokens)
+        assert a.shape == b.shape == (19, vocab)
+        assert np.abs(a - b).max() <= 1e-12 * np.abs(a).max(), (key, dtype, np.abs(a - b).max(), np.abs(a).max())
+    # and on the hand-made model of these tests, whose norm weights differ more from one
+    cfg, w = _tiny(seed=9, tied=False)
+    tokens = [3, 17, 3, 44, 9, 21, 0, 49]
+    a, b = P.forward_whole(cfg, w, tokens), L.forward(cfg, w, tokens)
+    assert np.abs(a - b).max() <= 1e-12 * np.abs(a).max()

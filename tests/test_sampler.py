@@ -1,5 +1,5 @@
-"""The host sampler against the vectors of the reference's own tests
-(/root/reference/tests/kipp_test.c:502-694)."""
+"""The host sampler: vectors of its own that show each rule, and then the reference's own sampler
+tests, vector for vector (/root/reference/tests/kipp_test.c:502-540, 586-694)."""
 import numpy as np
 import pytest
 
@@ -78,3 +78,77 @@ def test_distribution_matches_softmax():
     p = np.exp((LOGITS[:5] - LOGITS.max()) / 0.7)
     p /= p.sum()
     assert np.abs(counts[:5] / n - p).max() < 0.012 and counts[5] == 0
+
+
+# ------------------------------------------------------------------------------------------------
+# The reference's own sampler tests, vector for vector, through the interface that carries its
+# names (`kipp_amd.api.sample` / `sample_ex` / `KippError`).
+
+def test_reference_test_sampler():
+    # /root/reference/tests/kipp_test.c:502-540 (test_sampler)
+    from kipp_amd.api import ERROR_ARGUMENT, KippError, sample as kipp_sample
+    logits = np.array([0.1, 4.0, -1.0, 3.5, 0.0, -7.0, 2.0, 1.0], dtype=np.float32)
+    assert kipp_sample(logits, 0.0, 1.0, None) == 1
+    rng = XorShift64Star(42)
+    assert kipp_sample(logits, 1.0, 1.0e-6, rng) == 1
+    first = kipp_sample(logits, 1.0, 0.9, XorShift64Star(42))
+    token = kipp_sample(logits, 1.0, 0.9, XorShift64Star(42))
+    assert token == first and token < 8
+    seen = [0] * 8
+    rng = XorShift64Star(7)
+    for _ in range(200):
+        token = kipp_sample(logits, 1.5, 1.0, rng)
+        assert token < 8
+        seen[token] = 1
+    assert seen[1] and seen[3]
+    assert not seen[5]
+    zero_rng = XorShift64Star(1)
+    zero_rng.state = 0
+    for call in (lambda: kipp_sample(None, 0.0, 1.0, None),
+                 lambda: kipp_sample(logits, 1.0, 0.0, rng),
+                 lambda: kipp_sample(logits, 1.0, 1.5, rng),
+                 lambda: kipp_sample(logits, 1.0, 1.0, zero_rng)):
+        with pytest.raises(KippError) as e:
+            call()
+        assert e.value.code == ERROR_ARGUMENT
+
+
+def test_reference_test_sample_ex():
+    # /root/reference/tests/kipp_test.c:586-647 (test_sample_ex)
+    from kipp_amd.api import ERROR_ARGUMENT, KippError, sample_ex
+    logits = np.array([1.0, 5.0, 2.0, 4.0, 0.0, 3.0], dtype=np.float32)
+    rng = XorShift64Star(99)
+    # greedy over bias-adjusted logits: token 4 is lifted above the rest
+    assert sample_ex(logits, SampleParams(temperature=0.0, top_p=1.0, repetition_penalty=1.0, logit_bias={4: 10.0}), None) == 4
+    # top_k = 1 with temperature always returns the argmax
+    topk = SampleParams(temperature=1.0, top_p=1.0, top_k=1, repetition_penalty=1.0)
+    for _ in range(20):
+        assert sample_ex(logits, topk, rng) == 1
+    # repetition penalty: logit[1] 5.0 / 2 = 2.5, now below logit[3] = 4.0
+    penalized = SampleParams(temperature=0.0, top_p=1.0, repetition_penalty=2.0)
+    assert sample_ex(logits, penalized, None, recent=[1, 1, 1, 1]) == 3
+    # min_p keeps only the dominant token
+    peaked = np.array([10.0, 0.0, 0.0, 0.0], dtype=np.float32)
+    minp = SampleParams(temperature=1.0, top_p=1.0, min_p=0.5, repetition_penalty=1.0)
+    rng = XorShift64Star(7)
+    for _ in range(20):
+        assert sample_ex(peaked, minp, rng) == 0
+    with pytest.raises(KippError) as e:
+        sample_ex(logits, SampleParams(temperature=1.0, top_p=1.0, min_p=1.5, repetition_penalty=1.0), rng)
+    assert e.value.code == ERROR_ARGUMENT
+
+
+def test_reference_test_sample_fast_paths():
+    # /root/reference/tests/kipp_test.c:655-694: a zero-valued bias forces the path that copies the logits; both
+    # paths give the same token from the same generator state and leave the generator in the same state
+    from kipp_amd.api import sample_ex
+    logits = np.array([np.float32((i * 37 + 11) % 29) * np.float32(0.35) - np.float32((i * 13) % 7) for i in range(64)],
+                      dtype=np.float32)
+    for temperature in (0.0, 0.8):
+        for seed in (1, 7, 99, 12345):
+            fast = SampleParams(temperature=temperature, top_p=0.9, top_k=40, repetition_penalty=1.0)
+            slow = SampleParams(temperature=temperature, top_p=0.9, top_k=40, repetition_penalty=1.0, logit_bias={3: 0.0})
+            assert not fast.changes_logits and slow.changes_logits
+            fast_rng, slow_rng = XorShift64Star(seed), XorShift64Star(seed)
+            assert sample_ex(logits, fast, fast_rng) == sample_ex(logits, slow, slow_rng)
+            assert fast_rng.state == slow_rng.state and (fast_rng.state == seed) == (temperature == 0.0)

@@ -195,3 +195,32 @@ def test_temperature_requests_get_their_own_generator():
     r = Request("a", [1], 1, SampleParams(temperature=0.8), seed=0)
     s.add(r)
     assert r.rng is not None and r.rng.state == 1         # 0 is mapped to 1
+
+
+def test_a_request_id_names_one_request_at_a_time():
+    """A second request under an id that is waiting, running, open in the engine or finished and not yet
+    collected is refused at `add`; it never reaches admission, where it would fail on every step and
+    block everyone behind it."""
+    eng = FakeEngine(num_pages=16)
+    sched = Scheduler(eng, max_step_tokens=8, prefill_chunk=4)
+    sched.add(Request("a", [1, 2, 3], 3))
+    with pytest.raises(RequestRefused):
+        sched.add(Request("a", [4, 5], 2))                 # waiting
+    sched.step()
+    assert [r.id for r in sched.running] == ["a"]
+    with pytest.raises(RequestRefused):
+        sched.add(Request("a", [4, 5], 2))                 # running
+    eng.cache.open("session")                              # held by someone else, a session for instance
+    with pytest.raises(RequestRefused):
+        sched.add(Request("session", [4, 5], 2))
+    sched.add(Request("b", [4, 5], 2))                     # the queue is not blocked by the refusals
+    done = sched.run()
+    assert done["a"].output == expected_output([1, 2, 3], 3) and done["b"].output == expected_output([4, 5], 2)
+    with pytest.raises(RequestRefused):
+        sched.add(Request("a", [9], 1))                    # finished, its result not collected yet
+    first = sched.finished.pop("a")
+    sched.add(Request("a", [9], 1))
+    assert sched.run()["a"] is not first and sched.finished["a"].output == expected_output([9], 1)
+    assert sched.stats.refused == 4
+    eng.cache.close("session")
+    eng.cache.check()
