@@ -6,8 +6,19 @@ bfloat16 weights on one MI355X.
 One JSON line: `value` is decoded tokens a second at batch 8 (a step is one
 decode step of the whole batch, tokens chosen greedily on the device and fed
 back), with the prefill of one 2,048-token prompt, the decode step's HBM
-roofline and the batch-1 / batch-64 / batch-128 points beside it.  Peaks are MI355X's
-published ones: HBM 8 TB/s, dense bf16 MFMA 2.5 PFLOP/s.
+roofline and the batch-1 / batch-64 / batch-128 points beside it, then points at
+longer contexts (decode at batch 8 behind 8,192 and 30,720 tokens, a prompt
+portion of 512 tokens behind 4,096 and 16,384).  Peaks are MI355X's published
+ones: HBM 8 TB/s, dense bf16 MFMA 2.5 PFLOP/s.
+
+Protocol (after /root/reference/tools/bench.py:203-221 and
+/root/reference/bench/README.md:62-68): warm-up steps are discarded; the K timed
+steps are run `--repeats` times and the median repeat is the one reported, with
+the median absolute deviation beside it; and the run FAILS, printing no line,
+unless the timed decode steps were replays of recorded graphs made of the
+engine's own kernels (no product went to the library, no attention fell to the
+generic kernel): a number from a slower kernel class would otherwise look like
+any other.
 """
 import argparse
 import json
@@ -93,6 +104,104 @@ def decode_run(engine, ids, tokens, steps, warmup):
     return time.perf_counter() - start
 
 
+class WrongKernelClass(RuntimeError):
+    """The timed steps did not run on the kernels the measurement is about."""
+
+
+def measure_decode(engine, rt, ids, first, steps, warmup, repeats, weight_bytes, kv_per_token):
+    """`repeats` timings of `steps` decode steps (warm-up before the first); the median one is reported.
+    Raises WrongKernelClass unless every timed step was a replay of a recorded graph of our own kernels."""
+    timings = []
+    again = 0
+    rep = 0
+    while rep < repeats:
+        lengths = [engine.length(r) for r in ids]
+        library, generic, replays = rt.library_products, rt.generic_attention_launches, engine.graphs.replays
+        w = warmup if rep == 0 else 0
+        seconds = decode_run(engine, ids, first, steps, w)
+        if rt.library_products != library or rt.generic_attention_launches != generic:
+            raise WrongKernelClass(f"decode batch {len(ids)}: {rt.library_products - library} products went to the library and "
+                                   f"{rt.generic_attention_launches - generic} attention launches to the generic kernel")
+        if engine.graphs.replays - replays < steps and again < 2:
+            again += 1         # the contexts passed into the next bucket, whose graph is recorded now: time these steps again
+            continue
+        if engine.graphs.replays - replays < steps:
+            raise WrongKernelClass(f"decode batch {len(ids)}: only {engine.graphs.replays - replays} of {steps + w + 1} steps "
+                                   f"were replays of a recorded graph")
+        # bytes a step has to read: every weight once and the cache of the live requests (their lengths mid-way)
+        kv_tokens = sum(n + 1 + w + steps / 2.0 for n in lengths)
+        timings.append((seconds / steps, weight_bytes + kv_tokens * kv_per_token))
+        rep += 1
+    per_step = sorted(t for t, _ in timings)
+    median = per_step[len(per_step) // 2]
+    mad = sorted(abs(t - median) for t in per_step)[len(per_step) // 2]
+    nbytes = [b for t, b in timings if t == median][0]
+    return {"tok_s": len(ids) / median, "ms": median * 1e3, "mad_ms": mad * 1e3, "steps": steps, "warmup": warmup,
+            "bytes": nbytes, "repeats": repeats}
+
+
+def long_context_points(model, rt, cfg, layers, args, weight_bytes, kv_per_token):
+    """Decode at batch 8 behind 8,192 and 30,720 tokens and a prompt portion of 512 tokens behind 4,096 and
+    16,384: tokens a second, and the fraction of the roofline (HBM for decode, bf16 MFMA for the portion)."""
+    import torch
+    from kipp_amd.engine import Engine, StepEntry
+    batch, page, top = 8, 16, 30720
+    steps, warmup = max(8, args.steps // 2), max(2, args.warmup // 2)
+    room = top + 2 * (steps * 5 + warmup + 2) + 16
+    engine = Engine(model, page_size=page, num_pages=batch * (-(-room // page)) + 4, max_requests=batch,
+                    share_prefixes=False, max_position=room)
+    ids = [f"long{i}" for i in range(batch)]
+    gen = torch.Generator().manual_seed(3)
+    points, fracs = {}, {}
+    portion_ms = {4096: [], 16384: []}
+    last = {}
+
+    def feed(rid, n, want_last=False):
+        toks = torch.randint(0, cfg.vocab_size, (n,), generator=gen).tolist()
+        return engine.step([StepEntry(rid, toks, [n - 1] if want_last else [])])
+
+    def fill_to(target):
+        for rid in ids:
+            while engine.cache.requests.get(rid) is None or engine.length(rid) < target:
+                have = engine.length(rid) if rid in engine.cache.requests else 0
+                if have in portion_ms and target - have >= 512:
+                    torch.cuda.synchronize()
+                    start = time.perf_counter()
+                    feed(rid, 512)
+                    torch.cuda.synchronize()
+                    portion_ms[have].append((time.perf_counter() - start) * 1e3)
+                    continue
+                n = min(2048, target - have)
+                for mark in portion_ms:              # stop at the places where a portion is timed
+                    if have < mark < have + n:
+                        n = mark - have
+                logits = feed(rid, n, want_last=have + n == target)
+                if have + n == target:
+                    last[rid] = int(logits.argmax(dim=-1)[0])
+
+    for ctx in (8192, top):
+        t0 = time.perf_counter()
+        fill_to(ctx)
+        log(f"{batch} requests filled to {ctx} tokens in {time.perf_counter() - t0:.1f} s")
+        r = measure_decode(engine, rt, ids, last, steps, warmup, 3, weight_bytes, kv_per_token)
+        points[f"decode_b{batch}_ctx{ctx}"] = round(r["tok_s"], 1)
+        fracs[f"decode_b{batch}_ctx{ctx}"] = round(r["bytes"] / (r["ms"] / 1e3) / 1e9 / HBM_PEAK_GBS, 4)
+        log(f"decode batch {batch} behind {ctx} tokens: {r['ms']:.3f} ms/step, {r['tok_s']:.0f} tok/s, "
+            f"{r['bytes'] / (r['ms'] / 1e3) / 1e9:.0f} GB/s")
+        for rid in ids:                              # the tokens of the timed steps are in the cache; go on from a known one
+            last[rid] = 0
+    per_layer, _, _ = model_numbers(cfg, layers)
+    for behind, times in portion_ms.items():
+        if not times:
+            continue
+        ms = sorted(times)[len(times) // 2]
+        flops = 2.0 * 512 * per_layer * layers + layers * 4.0 * cfg.q_dim * (512 * behind + 512 * 513 / 2.0)
+        points[f"prefill512_ctx{behind}"] = round(512 / (ms / 1e3), 1)
+        fracs[f"prefill512_ctx{behind}"] = round(flops / (ms / 1e3) / PEAK_FLOPS["bf16"], 4)
+        log(f"a portion of 512 tokens behind {behind}: {ms:.2f} ms (median of {len(times)}), {512 / (ms / 1e3):.0f} tok/s")
+    return points, fracs
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -105,6 +214,8 @@ def main():
     ap.add_argument("--context", type=int, default=None, help="context length (default: the shape's)")
     ap.add_argument("--points", default="1,64,128", help="further decode batch sizes")
     ap.add_argument("--no-prefill", action="store_true")
+    ap.add_argument("--repeats", type=int, default=5, help="times the K timed steps are run; the median is reported")
+    ap.add_argument("--no-long", action="store_true", help="leave out the points at longer contexts")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -132,7 +243,8 @@ def main():
     rt = Runtime("bfloat16")
     model = random_model(config, seed=0, runtime=rt)
     # the first requests take part in every batch size: room for all those steps
-    decoded = sum((args.steps if b == args.batch else max(8, args.steps // 2)) +
+    repeats = max(1, args.repeats)
+    decoded = sum((repeats + 2) * (args.steps if b == args.batch else max(8, args.steps // 2)) +
                   (args.warmup if b == args.batch else max(2, args.warmup // 2)) + 1 for b in batches)
     tokens_per_request = args.prompt + decoded + 8
     engine = Engine(model, page_size=page, num_pages=max_batch * (-(-tokens_per_request // page)) + 4,
@@ -172,20 +284,29 @@ def main():
     for b in batches:
         steps = args.steps if b == args.batch else max(8, args.steps // 2)
         warmup = args.warmup if b == args.batch else max(2, args.warmup // 2)
-        before = engine.length(ids[0])
         try:
-            seconds = decode_run(engine, ids[:b], first, steps, warmup)
+            results[b] = measure_decode(engine, rt, ids[:b], first, steps, warmup, repeats, weight_bytes, kv_per_token)
         except Exception as exc:          # a further point must not cost the headline: say so and go on
-            if b == args.batch:
+            if b == args.batch or isinstance(exc, WrongKernelClass):
                 raise
             log(f"decode batch {b} failed and is left out: {type(exc).__name__}: {exc}")
             continue
-        ctx_mid = before + warmup + steps / 2.0
-        results[b] = {"tok_s": b * steps / seconds, "ms": seconds / steps * 1e3, "steps": steps, "warmup": warmup,
-                      "bytes": weight_bytes + b * ctx_mid * kv_per_token}
-        log(f"decode batch {b}: {seconds / steps * 1e3:.3f} ms/step, {b * steps / seconds:.0f} tok/s, "
-            f"{results[b]['bytes'] / (seconds / steps) / 1e9:.0f} GB/s")
+        r = results[b]
+        log(f"decode batch {b}: {r['ms']:.3f} ms/step (median of {repeats}, MAD {r['mad_ms']:.3f}), {r['tok_s']:.0f} tok/s, "
+            f"{r['bytes'] / (r['ms'] / 1e3) / 1e9:.0f} GB/s")
         # the requests beyond this batch keep their caches; the first ones simply go on
+
+    # ---- longer contexts, on a cache of their own behind the same weights
+    long_points, long_fracs = {}, {}
+    if not args.no_long:
+        del engine
+        torch.cuda.empty_cache()
+        try:
+            long_points, long_fracs = long_context_points(model, rt, cfg, layers, args, weight_bytes, kv_per_token)
+        except WrongKernelClass:
+            raise
+        except Exception as exc:
+            log(f"the points at longer contexts failed and are left out: {type(exc).__name__}: {exc}")
 
     main_r = results[args.batch]
     achieved = main_r["bytes"] / (main_r["ms"] / 1e3) / 1e9
@@ -202,7 +323,13 @@ def main():
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4)},
         "points": {f"decode_b{b}": round(results[b]["tok_s"], 1) for b in batches if b != args.batch and b in results},
+        "protocol": {"repeats": main_r["repeats"], "reported": "median", "mad_ms_per_step": round(main_r["mad_ms"], 4),
+                     "timed_steps_are_graph_replays_of_own_kernels": True},
     }
+    line["points"].update(long_points)
+    line["points_roofline_frac"] = {f"decode_b{b}": round(results[b]["bytes"] / (results[b]["ms"] / 1e3) / 1e9 / HBM_PEAK_GBS, 4)
+                                    for b in batches if b != args.batch and b in results}
+    line["points_roofline_frac"].update(long_fracs)
     if prefill is not None:
         line["prefill"] = prefill
     print(json.dumps(line), flush=True)

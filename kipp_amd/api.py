@@ -182,15 +182,39 @@ class Session:
         return self.eval_n(tokens, 1)[0]
 
     def eval_n(self, tokens: Sequence[int], rows: int) -> np.ndarray:
-        """Append the tokens; logits [rows, vocab] of the last `rows` of them."""
+        """Append the tokens; logits [rows, vocab] of the last `rows` of them, each row the bits that
+        evaluating its token alone would give (/root/reference/src/kipp.h:190-200: the primitive behind
+        verification, where a greedy choice must not flip).  Under float32 every kernel gives a row the
+        same bits however the tokens are cut, so one step serves.  Under bfloat16 a portion runs through
+        other kernels than a single token does: the tokens before the wanted rows go in as one portion,
+        the wanted ones one by one.  All or nothing: a failure leaves the session as it was."""
+        self._check(tokens)
+        n = len(tokens)
+        if not 1 <= rows <= n:
+            raise KippError(ERROR_ARGUMENT, "rows must be in 1..token_count")
+        if self.model.engine.rt.dtype == "float32" or rows == 1:
+            return self.eval_scored(tokens, rows)
+        before = self.length
+        try:
+            if n > rows:
+                self.model._step([StepEntry(self.id, list(tokens[:n - rows]), [])])
+            out = [self.model._step([StepEntry(self.id, [int(t)], [0])]).float().cpu().numpy() for t in tokens[n - rows:]]
+        except KippError:
+            if self.length != before:
+                self.truncate(before)
+            raise
+        return np.concatenate(out, axis=0)
+
+    def eval_scored(self, tokens: Sequence[int], rows: int) -> np.ndarray:
+        """As `eval_n`, but all tokens go through one step, whose rows agree with single-token evaluation
+        within the precision's tolerance only (/root/reference/src/kipp.h:202-213: for scoring, where the
+        logits feed arithmetic that tolerates it)."""
         self._check(tokens)
         n = len(tokens)
         if not 1 <= rows <= n:
             raise KippError(ERROR_ARGUMENT, "rows must be in 1..token_count")
         logits = self.model._step([StepEntry(self.id, list(tokens), list(range(n - rows, n)))])
         return logits.float().cpu().numpy()
-
-    eval_scored = eval_n   # one kernel path serves both: rows agree with single-token evaluation within rounding
 
     def match_prefix(self, tokens: Sequence[int]) -> int:
         """On a fresh session: adopt the longest published beginning of `tokens`

@@ -59,12 +59,12 @@ class RequestCache:
 
 
 class CacheGroup:
-    def __init__(self, index: int, need: KVNeed, runs: List[int], num_pages: int, page_size: int):
+    def __init__(self, index: int, need: KVNeed, runs: List[int], num_pages: int, page_size: int, page_order=None):
         self.index = index
         self.need = need
         self.runs = runs
         self.page_size = page_size
-        self.pool = PagePool(num_pages, page_size)
+        self.pool = PagePool(num_pages, page_size, order=page_order)
         self.k: Dict[int, object] = {}
         self.v: Dict[int, object] = {}
 
@@ -75,10 +75,11 @@ class CacheGroup:
 class CacheManager:
     def __init__(self, kv_needs: Sequence[Optional[KVNeed]], state_needs: Sequence[Optional[StateNeed]],
                  page_size: int, num_pages: int, max_requests: int, max_position: int,
-                 runtime=None, share_prefixes: bool = True):
+                 runtime=None, share_prefixes: bool = True, page_order=None):
         """`kv_needs[r]` / `state_needs[r]`: what run r of the layer order keeps
         (None: nothing).  `num_pages` is the size of every group's pool.  With
-        `runtime` None no device memory is made (bookkeeping only)."""
+        `runtime` None no device memory is made (bookkeeping only).  `page_order`:
+        the order in which every group's fresh pool hands out its pages (see `PagePool`)."""
         self.page_size = page_size
         self.max_requests = max_requests
         self.max_position = max_position
@@ -92,7 +93,7 @@ class CacheManager:
                 continue
             group = by_need.get(need)
             if group is None:
-                group = CacheGroup(len(self.groups), need, [], num_pages, page_size)
+                group = CacheGroup(len(self.groups), need, [], num_pages, page_size, page_order)
                 by_need[need] = group
                 self.groups.append(group)
             group.runs.append(run)
@@ -159,7 +160,11 @@ class CacheManager:
             raise OutOfSlots(f"all {self.max_requests} request slots are taken")
         slot = self.free_slots.pop()
         for tensor in self.states.values():
-            tensor[slot].zero_()
+            row = tensor[slot]
+            if self.rt is not None and (row.numel() * row.element_size()) % 4 == 0:
+                self.rt.ops.fill_zero(row)
+            else:
+                row.zero_()
         self._serial += 1
         req = RequestCache(request_id, slot, tables=[[] for _ in self.groups], adopted=[0 for _ in self.groups],
                            rows=[np.zeros(self.max_blocks, dtype=np.int32) for _ in self.groups], serial=self._serial)

@@ -56,13 +56,19 @@ def scattered_order(n: int) -> List[int]:
 
 
 class PagePool:
-    def __init__(self, num_pages: int, page_size: int):
+    def __init__(self, num_pages: int, page_size: int, order: Optional[Sequence[int]] = None):
+        """`order`: the order in which a fresh pool hands its pages out (a permutation of
+        0 .. num_pages - 1; default `scattered_order`).  Where a request's pages lie must not change
+        its results; tests run one trace under several orders."""
         if num_pages <= 0 or page_size <= 0:
             raise ValueError("a pool needs at least one page of at least one token")
+        order = scattered_order(num_pages) if order is None else [int(p) for p in order]
+        if sorted(order) != list(range(num_pages)):
+            raise ValueError("the order of a pool's pages must name every page once")
         self.num_pages = num_pages
         self.page_size = page_size
         self.ref = [0] * num_pages
-        self.free: "OrderedDict[int, None]" = OrderedDict((i, None) for i in scattered_order(num_pages))
+        self.free: "OrderedDict[int, None]" = OrderedDict((i, None) for i in order)
         self.content: List[Optional[Tuple[int, Tuple[int, ...]]]] = [None] * num_pages  # (hash, tokens) if indexed
         self.index: Dict[int, List[int]] = {}
         self.reused_total = 0

@@ -143,23 +143,17 @@ def main(argv=None) -> int:
     backend = f"hip-{args.dtype}"
     print(f"kipp: evaluating {len(tokens)} token{'s' if len(tokens) != 1 else ''} on {backend}", file=sys.stderr)
 
-    # no running ahead: the logits printed at the end are those of the last token that counts
+    # no running ahead: the logits printed at the end are those of the last token that counts;
+    # the last logits row is kept for the top-N table
+    last = {}
+
+    def keep_last(requests, logits):
+        last["row"] = logits[-1].clone()
     sched = Scheduler(engine, max_step_tokens=args.max_step_tokens, prefill_chunk=args.prefill_chunk, max_running=1,
-                      lookahead=False)
+                      lookahead=False, on_logits=keep_last)
     params = SampleParams(temperature=args.temperature, top_p=args.top_p, top_k=args.top_k, min_p=args.min_p)
     req = Request("cli", tokens, max(args.decode, 0), params, seed=args.seed, stop_tokens=stops)
     sched.add(req)
-
-    # the last logits row is kept for the top-N table
-    last = {}
-    inner_step = engine.step
-
-    def keeping_step(entries, **kw):
-        logits = inner_step(entries, **kw)
-        if logits is not None:
-            last["row"] = logits[-1]
-        return logits
-    engine.step = keeping_step
 
     torch.cuda.synchronize()
     started = time.perf_counter()

@@ -70,6 +70,12 @@ def load_config(model_dir: str):
     return parse_config(d)
 
 
+def shape_names():
+    """Names of the shapes shipped under config/shapes/."""
+    here = os.path.join(os.path.dirname(__file__), "shapes")
+    return sorted(f[:-5] for f in os.listdir(here) if f.endswith(".json"))
+
+
 def shape_config(name: str) -> dict:
     """config.json dict of a named shape shipped under config/shapes/."""
     here = os.path.join(os.path.dirname(__file__), "shapes")

@@ -190,10 +190,32 @@ __global__ void cast_kernel(const TI* __restrict__ in, TO* __restrict__ out, siz
     if (i < n) store_f(out, i, load_f(in, i));
 }
 
-// rows[i, :] = x[index[i], :]  (float32 rows; used to pick the positions whose
-// logits are wanted before the final norm and the output head).
-__global__ void gather_rows_kernel(const float* __restrict__ x, const int32_t* __restrict__ index,
-                                   float* __restrict__ out, int width) {
+// out = in, 16 bytes a lane and step where both are aligned so, else 4 (whole 4-byte words, copied bit for bit).
+__global__ void __launch_bounds__(256) copy_words_kernel(const uint32_t* __restrict__ in, uint32_t* __restrict__ out,
+                                                         size_t words, int wide) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (wide) {
+        const uint4* in4 = (const uint4*)in;
+        uint4* out4 = (uint4*)out;
+        const size_t quads = words / 4;
+        for (size_t q = i; q < quads; q += stride) out4[q] = in4[q];
+        for (size_t w = quads * 4 + i; w < words; w += stride) out[w] = in[w];
+    } else {
+        for (; i < words; i += stride) out[i] = in[i];
+    }
+}
+
+// words[0 .. n) = 0
+__global__ void __launch_bounds__(256) fill_zero_kernel(uint32_t* __restrict__ out, size_t words) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < words; i += stride) out[i] = 0u;
+}
+
+// rows[i, :] = x[index[i], :]  (rows of 4-byte words, copied bit for bit; used to pick the positions whose
+// logits are wanted before the final norm and the output head, and the tokens of the requests that go on).
+__global__ void gather_rows_kernel(const uint32_t* __restrict__ x, const int32_t* __restrict__ index,
+                                   uint32_t* __restrict__ out, int width) {
     const size_t src = (size_t)index[blockIdx.x] * width;
     const size_t dst = (size_t)blockIdx.x * width;
     for (int i = threadIdx.x; i < width; i += blockDim.x) out[dst + i] = x[src + i];
@@ -302,9 +324,28 @@ int kipp_cast(const void* in, int in_dtype, void* out, int out_dtype, size_t n, 
     return KIPP_LAUNCH_CHECK();
 }
 
-int kipp_gather_rows(const float* x, const int32_t* index, float* out, int rows, int width, hipStream_t stream) {
+int kipp_gather_rows(const void* x, const int32_t* index, void* out, int rows, int width, hipStream_t stream) {
     if (rows <= 0) return 0;
-    hipLaunchKernelGGL(gather_rows_kernel, dim3(rows), dim3(256), 0, stream, x, index, out, width);
+    hipLaunchKernelGGL(gather_rows_kernel, dim3(rows), dim3(width >= 256 ? 256 : 64), 0, stream, (const uint32_t*)x, index,
+                       (uint32_t*)out, width);
+    return KIPP_LAUNCH_CHECK();
+}
+
+// out[0 .. words) = in[0 .. words), 4-byte words
+int kipp_copy_words(const void* in, void* out, size_t words, hipStream_t stream) {
+    if (words == 0) return 0;
+    const int wide = (((uintptr_t)in | (uintptr_t)out) & 15) == 0;
+    const size_t units = wide ? (words + 3) / 4 : words;
+    const unsigned blocks = (unsigned)((units + 255) / 256 < 4096 ? (units + 255) / 256 : 4096);
+    hipLaunchKernelGGL(copy_words_kernel, dim3(blocks), dim3(256), 0, stream, (const uint32_t*)in, (uint32_t*)out, words, wide);
+    return KIPP_LAUNCH_CHECK();
+}
+
+// out[0 .. words) = 0, 4-byte words (a kernel, not a memset: it may be recorded into a graph)
+int kipp_fill_zero(void* out, size_t words, hipStream_t stream) {
+    if (words == 0) return 0;
+    const unsigned blocks = (unsigned)((words + 255) / 256 < 2048 ? (words + 255) / 256 : 2048);
+    hipLaunchKernelGGL(fill_zero_kernel, dim3(blocks), dim3(256), 0, stream, (uint32_t*)out, words);
     return KIPP_LAUNCH_CHECK();
 }
 

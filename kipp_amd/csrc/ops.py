@@ -150,12 +150,33 @@ def cast(src: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
 
 
 def gather_rows(x: torch.Tensor, index: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[i] = x[index[i]] for rows of float32 or int32 [n, width], copied bit for bit."""
     _dev(x, index, out)
     _i32(index, "index")
-    _need(x.dtype == torch.float32 and out.dtype == torch.float32, "gather_rows: float32 rows")
+    _need(x.dtype == out.dtype and x.dtype in (torch.float32, torch.int32) and x.dim() == 2, "gather_rows: rows of float32 or int32")
     _need(out.shape == (index.numel(), x.shape[1]), "gather_rows: output shape")
     fn = _fn("elementwise", "kipp_gather_rows", [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr])
     _check(fn(_ptr(x), _ptr(index), _ptr(out), index.numel(), x.shape[1], _stream()), "gather_rows")
+    return out
+
+
+def copy(src: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out = src, bit for bit, for contiguous tensors of one type and size whose bytes are whole 4-byte words."""
+    _dev(src, out)
+    nbytes = src.numel() * src.element_size()
+    _need(src.dtype == out.dtype and src.numel() == out.numel() and nbytes % 4 == 0, "copy: same type and size, whole words")
+    fn = _fn("elementwise", "kipp_copy_words", [_c_ptr, _c_ptr, _c_size, _c_ptr])
+    _check(fn(_ptr(src), _ptr(out), nbytes // 4, _stream()), "copy")
+    return out
+
+
+def fill_zero(out: torch.Tensor) -> torch.Tensor:
+    """out[...] = 0 by a kernel (no memset node when a graph records it)."""
+    _dev(out)
+    nbytes = out.numel() * out.element_size()
+    _need(nbytes % 4 == 0, "fill_zero: whole 4-byte words")
+    fn = _fn("elementwise", "kipp_fill_zero", [_c_ptr, _c_size, _c_ptr])
+    _check(fn(_ptr(out), nbytes // 4, _stream()), "fill_zero")
     return out
 
 

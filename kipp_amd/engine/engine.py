@@ -23,9 +23,11 @@ from .model import Model, load_model
 class Engine:
     def __init__(self, model: Model, page_size: int = 16, num_pages: Optional[int] = None,
                  max_tokens: Optional[int] = None, max_requests: int = 64, share_prefixes: bool = True,
-                 use_graphs: bool = True):
+                 use_graphs: bool = True, page_order=None, max_position: Optional[int] = None):
         """The pool of every cache group has `num_pages` pages, or as many as
-        hold `max_tokens` tokens."""
+        hold `max_tokens` tokens.  `page_order`: the order in which fresh pools hand
+        out their pages (a permutation; results must not depend on it).  `max_position`:
+        the longest context a request may reach (default: the model's own limit)."""
         if num_pages is None:
             if max_tokens is None:
                 raise ValueError("give num_pages or max_tokens")
@@ -38,7 +40,8 @@ class Engine:
         build.build_all(model_variants(model.spec, self.rt.dtype))
         self.vocab_size = model.spec.vocab_size
         self.cache = CacheManager(model.kv_needs(), model.state_needs(), page_size, num_pages, max_requests,
-                                  model.spec.max_position, runtime=self.rt, share_prefixes=share_prefixes)
+                                  max_position or model.spec.max_position, runtime=self.rt, share_prefixes=share_prefixes,
+                                  page_order=page_order)
         self.graphs = DecodeGraphs(self) if use_graphs else None
         self._uncommitted = {}      # request -> tokens of a step run from device_tokens and not recorded yet
 
@@ -58,9 +61,14 @@ class Engine:
         return self.cache.requests[request_id].length
 
     # -- the step ---------------------------------------------------------------------
-    def step(self, entries: Sequence[StepEntry], device_tokens: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    def step(self, entries: Sequence[StepEntry], device_tokens: Optional[torch.Tensor] = None,
+             borrow: bool = False) -> Optional[torch.Tensor]:
         """Run one batch.  Requests not yet open are opened.  Raises OutOfPages
         (nothing changed) when the pools cannot hold the step.
+
+        With `borrow` the logits may lie in a buffer of the engine's own that a later
+        step overwrites: for a caller that is done with them (has launched what reads
+        them) before it calls `step` again, and saves a copy of [entries, vocab] floats.
 
         With `device_tokens` (int32 [entries] on the device) every entry brings one
         token that the host does not know yet, for instance the choice of the step
@@ -106,7 +114,7 @@ class Engine:
             raise
         try:
             if self.graphs is not None and self.graphs.applies(entries):
-                logits = self.graphs.run(entries, requests, device_tokens)
+                logits = self.graphs.run(entries, requests, device_tokens, borrow)
             else:
                 batch = build_batch(entries, requests, len(self.cache.groups), self.rt.device)
                 logits = self.model.forward(batch, self.cache)

@@ -55,7 +55,9 @@ class DecodeGraph:
         rt = engine.rt
         self.n = n = n_seqs
         self.groups = len(cache.groups)
-        self.max_blocks = cache.max_blocks
+        # a table row is as wide as the contexts of this shape, not as the model's longest possible one:
+        # kernels choose by it what they can do, and it is copied whenever a row changes
+        self.max_blocks = max(1, -(-max_context // cache.page_size))
         self.max_context = max_context
         table_ints = self.groups * n * self.max_blocks
         # [tokens | positions | ctx_len | slots | tables | arange | ones]
@@ -77,9 +79,9 @@ class DecodeGraph:
         self.batch = StepBatch(
             n_tokens=n, n_seqs=n, n_want=n, tokens=d[0:n], positions=d[n:2 * n], seq_of_token=arange, q_start=arange,
             q_len=ones, ctx_len=d[2 * n:3 * n], slots=d[3 * n:4 * n], want_rows=arange, block_tables=tables,
-            decode_rows=arange, prefill_seq=d[0:0], prefill_tile=d[0:0], n_decode=n, n_prefill_items=0,
+            decode_rows=arange, n_decode=n, n_portions=0,
             max_decode_ctx=max_context, max_q_len=1, max_ctx_len=max_context, want_every_row=True,
-            host={"q_start": list(range(n)), "q_len": [1] * n})
+            host={"q_start": list(range(n)), "q_len": [1] * n, "ctx_len": [max_context] * n})
         self.graph: Optional[torch.cuda.CUDAGraph] = None
         self.logits: Optional[torch.Tensor] = None
         self.copied: Optional[torch.cuda.Event] = None
@@ -113,7 +115,7 @@ class DecodeGraph:
                 changed = True
                 at = 4 * n + i * self.max_blocks
                 for g in range(self.groups):
-                    h[at:at + self.max_blocks] = r.rows[g] if r is not None else self.scratch_pages[g]
+                    h[at:at + self.max_blocks] = r.rows[g][:self.max_blocks] if r is not None else self.scratch_pages[g]
                     at += n * self.max_blocks
         upto = self.var_ints if changed else 4 * n
         self.dev[:upto].copy_(self.host[:upto], non_blocking=True)
@@ -122,7 +124,7 @@ class DecodeGraph:
         if device_tokens is not None:
             self.dev[:live].copy_(device_tokens)  # on the device, after the copy above: the tokens the host does not know
 
-    def run(self, engine, entries, requests, device_tokens=None) -> torch.Tensor:
+    def run(self, engine, entries, requests, device_tokens=None, borrow: bool = False) -> torch.Tensor:
         self.fill(entries, requests, device_tokens)
         if self.graph is None:
             # a shape runs eagerly until it has come twice (that also makes every workspace the
@@ -148,7 +150,10 @@ class DecodeGraph:
             self.graph = graph
             return logits[:len(entries)]
         self.graph.replay()
-        return self.logits[:len(entries)].clone()     # the graph's own output buffer is overwritten by the next replay
+        rows = self.logits[:len(entries)]
+        if borrow:
+            return rows                 # the graph's own output buffer: the next replay of this shape overwrites it
+        return engine.rt.ops.copy(rows, engine.rt.empty(rows.shape, rows.dtype))
 
 
 class DecodeGraphs:
@@ -166,7 +171,7 @@ class DecodeGraphs:
         return (self.possible and 0 < len(entries) <= MAX_GRAPH_ENTRIES
                 and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries))
 
-    def run(self, entries, requests, device_tokens=None) -> torch.Tensor:
+    def run(self, entries, requests, device_tokens=None, borrow: bool = False) -> torch.Tensor:
         engine = self._engine()
         cache = engine.cache
         longest = max(r.length for r in requests) + 1
@@ -181,4 +186,4 @@ class DecodeGraphs:
             self.graphs.move_to_end(key)
         if graph.graph is not None:
             self.replays += 1
-        return graph.run(engine, entries, requests, device_tokens)
+        return graph.run(engine, entries, requests, device_tokens, borrow)

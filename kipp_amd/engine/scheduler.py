@@ -85,15 +85,23 @@ class SchedulerStats:
     waits_for_prefix: int = 0
 
 
+def _rows_on_device(engine, tokens, rows):
+    """tokens[rows] (int32 on the device), picked by the engine's own gather kernel."""
+    import torch
+    rt = engine.rt
+    index = torch.tensor(list(rows), dtype=torch.int32).pin_memory().to(rt.device, non_blocking=True)
+    return rt.ops.gather_rows(tokens.view(-1, 1), index, rt.empty((len(rows), 1), torch.int32)).view(-1)
+
+
 class _PicksRows:
     """Some rows of a choice that is still on its way."""
 
-    def __init__(self, picks, rows):
-        self.picks, self.rows = picks, list(rows)
+    def __init__(self, engine, picks, rows):
+        self.engine, self.picks, self.rows = engine, picks, list(rows)
 
     @property
     def device(self):
-        return self.picks.device[self.rows]
+        return _rows_on_device(self.engine, self.picks.device, self.rows)
 
     def result(self):
         chosen = self.picks.result()
@@ -102,9 +110,14 @@ class _PicksRows:
 
 class Scheduler:
     def __init__(self, engine, max_step_tokens: int = 2048, prefill_chunk: int = 512, max_running: int = 64,
-                 lookahead: bool = True):
+                 lookahead: bool = True, on_logits=None):
+        """`on_logits(requests, logits)`: called after every step that asked for logits, before tokens are
+        chosen from them, with the requests whose rows they are, in order, and the float32 tensor
+        [rows, vocab] on the device.  The tensor may be overwritten by the next step: a caller that wants to
+        keep a row copies it."""
         if max_step_tokens < 1 or prefill_chunk < 1 or max_running < 1:
             raise ValueError("budgets must be positive")
+        self.on_logits = on_logits
         # running ahead needs an engine that takes a step's tokens from the device
         self.lookahead = lookahead and getattr(engine, "graphs", None) is not None
         self._ahead = None          # (requests, Picks) of the step launched last, its choice not yet read
@@ -252,9 +265,10 @@ class Scheduler:
         if not plan:
             return produced
         entries = [StepEntry(req.id, tokens, want) for req, tokens, want in plan]
-        logits = self.engine.step(entries)
+        logits = self.engine.step(entries, borrow=True)      # read by `choose` before the next step is launched
         self.stats.steps += 1
         sampling = [req for req, _, want in plan if want]
+        self._tell(sampling, logits)
         for req, tokens, want in plan:
             if req.state == "prefill":
                 req.fed += len(tokens)
@@ -267,6 +281,10 @@ class Scheduler:
             for req, token in zip(sampling, chosen):
                 self._accept(req, int(token), produced)
         return produced
+
+    def _tell(self, requests, logits) -> None:
+        if self.on_logits is not None and logits is not None and requests:
+            self.on_logits(requests, logits)
 
     # -- one step ahead --------------------------------------------------------------------
     def _may_run_ahead(self, plan, sampling) -> bool:
@@ -283,8 +301,9 @@ class Scheduler:
         nxt = None
         if go_on:
             cont = [reqs[i] for i in go_on]
-            tokens = picks.device if len(go_on) == len(reqs) else picks.device[go_on]
-            logits = self.engine.step([StepEntry(req.id, [0], [0]) for req in cont], device_tokens=tokens.contiguous())
+            tokens = picks.device if len(go_on) == len(reqs) else _rows_on_device(self.engine, picks.device, go_on)
+            logits = self.engine.step([StepEntry(req.id, [0], [0]) for req in cont], device_tokens=tokens, borrow=True)
+            self._tell(cont, logits)
             self.stats.steps += 1
             nxt = (cont, self.engine.choose(logits, cont, wait=False))
         produced: List[Tuple[object, int]] = []
@@ -302,7 +321,7 @@ class Scheduler:
             if len(alive) == len(cont):
                 self._ahead = nxt
             elif alive:
-                self._ahead = ([cont[i] for i in alive], _PicksRows(ahead, alive))
+                self._ahead = ([cont[i] for i in alive], _PicksRows(self.engine, ahead, alive))
             else:
                 self._ahead = None
         else:

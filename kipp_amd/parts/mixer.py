@@ -61,6 +61,19 @@ class Attention:
     def placement(spec):
         return {"q_norm.weight": "float32", "k_norm.weight": "float32"}
 
+    @staticmethod
+    def variants(spec, dtype):
+        """The builds of its specialised kernels (one per head size; decode also per number of query heads
+        that share a key/value head).  Under float32, and for more than 16 heads a group, the generic
+        attention kernel runs, which every model has."""
+        if dtype != "bfloat16":
+            return []
+        group = spec.num_heads // spec.num_kv_heads
+        out = [("attention_prefill", {"HEAD_DIM": spec.head_dim})]
+        if group <= 16:
+            out.append(("attention_decode", {"HEAD_DIM": spec.head_dim, "GROUP": group}))
+        return out
+
     def load(self, tensors):
         import torch
         q, k, v = tensors["q_proj.weight"], tensors["k_proj.weight"], tensors["v_proj.weight"]
@@ -87,11 +100,14 @@ class Attention:
         angles = self.position.angles(batch) if hasattr(self.position, "angles") and hasattr(batch, "step_cache") else None
         table = batch.block_tables[cache.group]
         eps = s.qk_norm_eps if s.qk_norm_eps is not None else 0.0
+        # a table row is as wide as the longest context of this step, so what decides is what the step needs
         fast = rt.dtype == "bfloat16" and rt.ops.attention_fast_ok(s.num_heads, s.num_kv_heads, cache.page_size, table.shape[1])
+        if rt.dtype == "bfloat16" and not fast:
+            rt.generic_attention_launches += 1      # the slow kernel class: a measurement must know it ran
         # single tokens only: norm, rotation, cache write and attention in one kernel, for a few of them (with
         # more rows or long contexts every split's workgroup would prepare the queries again, which costs more
         # than the rotary kernel it saves) and wherever the kernel that walks whole contexts or long ranges runs
-        fused = fast and not batch.n_prefill_items and batch.n_decode == n \
+        fused = fast and not batch.n_portions and batch.n_decode == n \
             and rt.ops.attention_decode_fused_ok(s.head_dim, rotary_dim, inv_freq is not None) \
             and ((n <= FUSED_DECODE_ROWS and batch.max_decode_ctx < FUSED_DECODE_KEYS)
                  or rt.ops.attention_decode_streams(n, s.num_kv_heads, s.head_dim, s.num_heads // s.num_kv_heads,
@@ -111,8 +127,9 @@ class Attention:
             self.q_norm, self.k_norm, eps, inv_freq, rotary_dim, write_kv=cache.writable, angles=angles)
         out = rt.empty((n, s.q_dim), rt.act_dtype)
         if fast:
-            if batch.n_prefill_items:
-                rt.ops.attention_prefill(q, cache.k, cache.v, out, batch.prefill_seq, batch.prefill_tile, batch.q_start,
+            if batch.n_portions:
+                item_seq, item_tile = self._prefill_work(batch)
+                rt.ops.attention_prefill(q, cache.k, cache.v, out, item_seq, item_tile, batch.q_start,
                                          batch.q_len, batch.positions, table, s.num_heads, s.num_kv_heads, s.head_dim,
                                          self.scale, s.window or 0)
             if batch.n_decode:
@@ -124,6 +141,26 @@ class Attention:
             rt.ops.paged_attention_generic(q, cache.k, cache.v, out, batch.positions, batch.seq_of_token, table,
                                            s.num_heads, s.num_kv_heads, s.head_dim, self.scale, s.window or 0)
         return rt.linear(out, self.w_o, slabs=True, defer=True)
+
+    def _prefill_work(self, batch):
+        """The work list of the prefill kernel: (entry, tile of its kernel's query rows) for every
+        entry that brings a portion, the longest key range first (the kernel folds the list so that
+        workgroups sharing a compute unit carry about the same load).  Made by the first attention
+        layer of a forward pass and shared by the others of the same tile size."""
+        tile = self.rt.ops.PREFILL_ROWS
+        key = ("attention_prefill_work", tile)
+        work = batch.step_cache.get(key)
+        if work is None:
+            items = []
+            for i, (n, ctx) in enumerate(zip(batch.host["q_len"], batch.host["ctx_len"])):
+                if n > 1:
+                    start = ctx - n
+                    for t in range((n + tile - 1) // tile):
+                        items.append((-(start + min((t + 1) * tile, n)), i, t))    # keys the tile's last row sees
+            items.sort()
+            work = batch.upload([i for _, i, _ in items], [t for _, _, t in items])
+            batch.step_cache[key] = work
+        return work
 
     def _workspace(self, batch):
         """Partial results of the split decode kernel, shared by the layers of one geometry and kept

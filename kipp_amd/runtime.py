@@ -105,6 +105,7 @@ class Runtime:
         self.stream_layout = stream_layout   # keep a second copy of bfloat16 matrices in the streaming layout
         self._mm_out_f32 = None
         self.library_products = 0   # calls that went to the library (they stay out of HIP graphs)
+        self.generic_attention_launches = 0   # bfloat16 attention that fell to the generic kernel (geometry the matrix-core kernels refuse)
         self.fuse_norms = True      # few rows: residual add and norm ride on the products around them
         torch.backends.cuda.matmul.allow_tf32 = False
 

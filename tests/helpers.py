@@ -125,6 +125,50 @@ def mixed(requests, seed: int, max_live: int = 4, prefill_portion=(2, 9), decode
     return steps
 
 
+def busy(requests, seed: int, decode_tail, most_decoding: int = 40, portions_at_once: int = 3,
+         sizes=(2, 5, 33, 16, 7, 130, 3, 61, 290, 2, 24)) -> List[Step]:
+    """Many requests at once: up to `portions_at_once` of them bring the next portion of their prompt
+    (sizes change from portion to portion, down to two tokens), while every request whose prompt is in
+    (up to `most_decoding` of them; the rest are left out of the step and go on later) brings one token.
+    `decode_tail[rid]`: how many of a request's last tokens are fed one by one."""
+    rng = random.Random(seed)
+    waiting = list(requests)
+    prefilling: List[str] = []
+    decoding: List[str] = []
+    fed = {r: 0 for r in requests}
+    steps: List[Step] = []
+    turn = 0
+    while waiting or prefilling or decoding:
+        while waiting and len(prefilling) < portions_at_once:
+            prefilling.append(waiting.pop(0))
+        entries, ends = [], []
+        chosen = decoding if len(decoding) <= most_decoding else rng.sample(decoding, most_decoding)
+        for rid in list(chosen):
+            entries.append((rid, 1))
+            fed[rid] += 1
+            if fed[rid] == len(requests[rid]):
+                ends.append(rid)
+                decoding.remove(rid)
+        for rid in list(prefilling):
+            left = len(requests[rid]) - decode_tail[rid] - fed[rid]
+            n = min(sizes[turn % len(sizes)], left)
+            turn += 1
+            if left - n == 1:
+                n += 1
+            if n == 1:           # a prompt of one token more than its tail: the token joins the single ones
+                n = 1
+            entries.append((rid, n))
+            fed[rid] += n
+            if fed[rid] >= len(requests[rid]) - decode_tail[rid]:
+                prefilling.remove(rid)
+                if fed[rid] == len(requests[rid]):
+                    ends.append(rid)
+                else:
+                    decoding.append(rid)
+        steps.append((entries, ends))
+    return steps
+
+
 def peak_pages(requests, steps: Sequence[Step], page: int) -> int:
     """The most pages that live requests hold at any time under `steps`."""
     fed: Dict[str, int] = {}

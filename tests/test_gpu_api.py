@@ -172,3 +172,34 @@ def test_two_generations_on_one_engine(model_folders, dtype):
             assert len(out) == 12
             _follows_plain_argmax(folder, prompt, out, margin)
     engine.cache.check()
+
+
+def test_eval_n_reproduces_single_tokens_bitwise_and_eval_scored_within_tolerance(model_folders):
+    """/root/reference/src/kipp.h:190-213: `eval_n` rows are the bits of single-token evaluation (so a greedy
+    choice cannot flip between verification and decoding); `eval_scored` may run all rows through kernels
+    that reduce in another order and agrees within tolerance.  Under bfloat16 the two differ."""
+    from kipp_amd.api import Model
+    folder = model_folders[("b", "bfloat16")]
+    toks = H.random_tokens(81, 60, 509)
+    ref = H.plain_logits(folder, toks)
+    m = Model.open(folder, dtype="bfloat16", kv_pool_blocks=64, page_tokens=8)
+    a, b, c = (m.session_create(64) for _ in range(3))
+    exact = a.eval_n(toks, 25)
+    scored = b.eval_scored(toks, 25)
+    c.eval(toks[:35])
+    singles = np.stack([c.eval([t]) for t in toks[35:]])
+    assert np.array_equal(exact, singles)
+    assert not np.array_equal(scored, singles)
+    H.assert_close(scored, ref[35:], H.NMSE_BF16["tiny"], "eval_scored")
+    H.assert_close(exact, ref[35:], H.NMSE_BF16["tiny"], "eval_n")
+    assert a.length == b.length == c.length == 60
+    # all or nothing: 5 tokens that do not fit leave the session as it was, also when some of them ran
+    d = m.session_create(10)
+    d.eval(toks[:8])
+    from kipp_amd.api import KippError
+    with pytest.raises(KippError):
+        d.eval_n(toks[8:13], 3)
+    assert d.length == 8
+    for s in (a, b, c, d):
+        s.destroy()
+    m.close()

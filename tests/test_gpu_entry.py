@@ -92,6 +92,9 @@ def test_running_one_step_ahead_changes_nothing(model_folders, dtype):
     plainly, _ = run(False)
     ahead, stats = run(True)
     assert ahead == plainly and [len(ahead[i][0]) for i in range(5)] == [40, 7, 23, 31, 15]
+    # not only the same as when it waits: the greedy requests follow the plain implementation's argmax
+    for i in (0, 2, 4):
+        _follows_plain_argmax(folder, prompts[i], ahead[i][0], 1e-5 if dtype == "float32" else 0.03)
     # end request 0 early by a stop token it is known to produce: one step late, nothing else changes
     stop = plainly[0][0][20]
     first = plainly[0][0].index(stop)
@@ -229,10 +232,12 @@ def _trace(requests, steps):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_trace_run(model_folders, tiny_configs, tmp_path, dtype):
-    folder = model_folders[("b", dtype)]
-    requests = {f"r{i}": H.random_tokens(300 + i, n, 509) for i, n in enumerate([70, 33, 100, 7, 61, 90])}
-    steps = H.mixed(requests, seed=9)
+@pytest.mark.parametrize("key,page,cut", [("b", 16, "mixed"), ("a", 16, "portions"), ("b", 8, "portions"), ("a", 32, "tail")])
+def test_trace_run(model_folders, tiny_configs, tmp_path, dtype, key, page, cut):
+    folder = model_folders[(key, dtype)]
+    vocab = tiny_configs[key]["vocab_size"]
+    requests = {f"r{i}": H.random_tokens(300 + i, n, vocab) for i, n in enumerate([70, 33, 100, 7, 61, 90])}
+    steps = {"mixed": lambda r: H.mixed(r, seed=9), "portions": H.changing_portions, "tail": H.tail_one_by_one}[cut](requests)
     # --max-tokens: live requests' counts, each rounded up to 64
     fed, peak = {}, 0
     for entries, ends in steps:
@@ -243,7 +248,7 @@ def test_trace_run(model_folders, tiny_configs, tmp_path, dtype):
             del fed[rid]
     out = tmp_path / "out"
     proc = subprocess.Popen([os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype, "--out", str(out),
-                             "--max-tokens", str(peak)], stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True)
+                             "--max-tokens", str(peak), "--page", str(page)], stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True)
     for i, line in enumerate(_trace(requests, steps)):
         proc.stdin.write(line + "\n")
         proc.stdin.flush()
@@ -252,7 +257,7 @@ def test_trace_run(model_folders, tiny_configs, tmp_path, dtype):
     assert proc.wait(timeout=60) == 0
     rows = {r: [] for r in requests}
     for i, (entries, _) in enumerate(steps):
-        data = np.fromfile(out / f"{i}.f32", dtype="<f4").reshape(-1, 509)
+        data = np.fromfile(out / f"{i}.f32", dtype="<f4").reshape(-1, vocab)
         at = 0
         for rid, n in entries:
             rows[rid].append(data[at:at + n])
@@ -260,4 +265,4 @@ def test_trace_run(model_folders, tiny_configs, tmp_path, dtype):
         assert at == data.shape[0]
     tol = H.NMSE_F32 if dtype == "float32" else H.NMSE_BF16["tiny"]
     for rid, toks in requests.items():
-        H.assert_close(np.concatenate(rows[rid]), H.plain_logits(folder, toks), tol, f"trace {dtype} {rid}")
+        H.assert_close(np.concatenate(rows[rid]), H.plain_logits(folder, toks), tol, f"trace {key} page {page} {cut} {dtype} {rid}")

@@ -183,3 +183,61 @@ def test_a_batch_whose_size_changes_replays_one_graph(long_folder, dtype):
         first = len(toks) - 14
         H.assert_close(np.stack(got[rid]), ref[first:first + len(got[rid])], tol, f"changing batch/{dtype}/{rid}")
     engine.cache.check()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_many_decoding_rows_beside_prompt_portions(long_folder, dtype):
+    """Steps that hold 20 to 34 single tokens AND two or three prompt portions of changing size (2 to 290
+    tokens; a few steps pass 256 rows and take the library's product), at head size 128: in bfloat16 one
+    forward pass then runs the rotary kernel, the prefill attention and the split decode attention side
+    by side.  The pool holds exactly what live requests need at the peak, so pages are used again while
+    others are still read.  Every row of every request against the plain implementation."""
+    from kipp_amd.engine import Engine
+    cfg, weights = plain.load_folder(long_folder)
+    rng = np.random.default_rng(3)
+    requests, tail = {}, {}
+    for i in range(70):
+        tail[f"r{i}"] = 25 + (i * 7) % 26
+        requests[f"r{i}"] = H.random_tokens(700 + i, int(rng.integers(4, 200)) + tail[f"r{i}"], 311)
+    steps = H.busy(requests, 1, tail)
+    singles = [sum(1 for _, n in entries if n == 1) for entries, _ in steps]
+    portions = [sum(1 for _, n in entries if n > 1) for entries, _ in steps]
+    assert sum(1 for s, p in zip(singles, portions) if s >= 20 and p >= 2) >= 50 and max(singles) > 32
+    assert sum(1 for entries, _ in steps if sum(n for _, n in entries) > 256) >= 2
+    pages = H.peak_pages(requests, steps, 16)
+    assert pages < 0.6 * sum(-(-len(t) // 16) for t in requests.values())
+    engine = Engine.from_folder(long_folder, dtype=dtype, page_size=16, num_pages=pages, max_requests=64, share_prefixes=False)
+    got = H.replay(engine, requests, steps)
+    tol = H.NMSE_F32 if dtype == "float32" else H.NMSE_BF16["real"]
+    for rid, toks in requests.items():
+        H.assert_close(got[rid], plain.forward_whole(cfg, weights, toks), tol, f"busy/{dtype}/{rid}")
+    assert engine.cache.free_pages() == [pages]
+
+
+def test_a_long_position_limit_keeps_the_matrix_core_kernels(real_folder, real_reference, tmp_path):
+    """A model folder whose config.json allows 40,960 positions (the reference's Qwen3-4B,
+    /root/reference/src/kipp_checkpoints.h:31): block tables are as wide as the contexts of a step, not
+    as that limit, so short contexts decode on the matrix-core attention kernels under recorded graphs,
+    nothing falls to the generic kernel, and the logits match the plain implementation."""
+    import json
+    import os
+    from kipp_amd.engine import Engine
+    folder = str(tmp_path / "long-limit")
+    os.makedirs(folder)
+    with open(os.path.join(real_folder, "config.json")) as f:
+        config = json.load(f)
+    config["max_position_embeddings"] = 40960
+    with open(os.path.join(folder, "config.json"), "w") as f:
+        json.dump(config, f)
+    os.symlink(os.path.join(real_folder, "model.safetensors"), os.path.join(folder, "model.safetensors"))
+    requests, refs = real_reference
+    requests = {rid: requests[rid] for rid in ("p", "q")}
+    steps = H.tail_one_by_one(requests, 20)
+    engine = Engine.from_folder(folder, dtype="bfloat16", page_size=16, max_tokens=512, max_requests=4, share_prefixes=False)
+    assert engine.cache.max_position == 40960
+    got = H.replay(engine, requests, steps)
+    for rid in requests:
+        H.assert_close(got[rid], refs[rid], H.NMSE_BF16["real"], f"long limit/{rid}")
+    assert engine.rt.generic_attention_launches == 0
+    assert engine.graphs.replays >= 30
+    assert all(g.max_blocks <= 1024 // 16 for g in engine.graphs.graphs.values())

@@ -20,7 +20,7 @@ class FakeEngine:
         self.vocab_size = VOCAB
         self.calls = []
 
-    def step(self, entries):
+    def step(self, entries, borrow=False):
         reqs = []
         for e in entries:
             if e.request not in self.cache.requests:
