@@ -34,7 +34,7 @@ class RopeSpec:
     """Rotary position encoding over the first `rotary_dim` dims of a head.
 
     pairing "half": dim i rotates with dim i + rotary_dim/2 (the reference's
-    pairing, /root/reference/src/kipp.c:2368-2382).
+    pairing, /root/reference/src/kipp.c:2368-2382); "interleaved": dim 2i with dim 2i + 1.
     """
     head_dim: int
     theta: float
@@ -48,6 +48,8 @@ class RopeSpec:
             raise ConfigError(f"rotary_dim {rd} must be even and in (0, head_dim={self.head_dim}]")
         if not self.theta > 0:
             raise ConfigError(f"rope theta must be positive, got {self.theta}")
+        if self.pairing not in ("half", "interleaved"):
+            raise ConfigError(f"rope pairing {self.pairing!r} is not one of half, interleaved")
 
 
 @dataclass(frozen=True)
@@ -173,6 +175,7 @@ class ModelSpec:
     final_norm: object
     head: HeadSpec
     stop_tokens: Tuple[int, ...] = field(default_factory=tuple)
+    input_position: Optional[object] = None   # a position part applied to the residual stream after the embedding (None: none)
 
     def __post_init__(self):
         for index, run in enumerate(self.order):

@@ -206,10 +206,12 @@ def qk_norm_rope_kv_write(qkv: torch.Tensor, q_out: torch.Tensor, k_cache: torch
                           n_q: int, n_kv: int, head_dim: int,
                           q_norm_w: Optional[torch.Tensor], k_norm_w: Optional[torch.Tensor], eps: float,
                           inv_freq: Optional[torch.Tensor], rotary_dim: int, write_kv: bool = True,
-                          angles: Optional[torch.Tensor] = None) -> torch.Tensor:
+                          angles: Optional[torch.Tensor] = None, pairing: str = "half") -> torch.Tensor:
     """Per-head norm of q and k, rotation at each token's position, q to `q_out`
     and k, v into their pages.  Caches are [pages, n_kv, page, head_dim].  With
-    `angles` (rotary_angles) the cosines and sines are read, not computed."""
+    `angles` (rotary_angles) the cosines and sines are read, not computed.
+    `pairing`: "half" rotates dim i with dim i + rotary_dim / 2, "interleaved" dim 2i with dim 2i + 1."""
+    _need(pairing in ("half", "interleaved"), f"qk_norm_rope: pairing {pairing!r} is not one of half, interleaved")
     _dev(qkv, q_out, k_cache, v_cache, positions, seq_of_token, block_table, q_norm_w, k_norm_w, inv_freq, angles)
     for t, name in ((positions, "positions"), (seq_of_token, "seq_of_token"), (block_table, "block_table")):
         _i32(t, name)
@@ -232,11 +234,11 @@ def qk_norm_rope_kv_write(qkv: torch.Tensor, q_out: torch.Tensor, k_cache: torch
     _angles_ok(angles, n, rotary_dim, "qk_norm_rope")
     fn = _fn("rope_kv", "kipp_qk_norm_rope_kv",
              [_c_ptr, _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int,
-              _c_ptr, _c_ptr, _c_float, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr])
+              _c_ptr, _c_ptr, _c_float, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr])
     _check(fn(_ptr(qkv), _code(qkv), _ptr(q_out), _code(q_out), _ptr(k_cache), _ptr(v_cache), _code(k_cache),
               _ptr(positions), _ptr(seq_of_token), _ptr(block_table), block_table.shape[1],
               _ptr(q_norm_w), _ptr(k_norm_w), float(eps), _ptr(inv_freq), _ptr(angles), int(rotary_dim),
-              n, n_q, n_kv, head_dim, k_cache.shape[2], 1 if write_kv else 0, parts, _stream()), "qk_norm_rope_kv_write")
+              1 if pairing == "interleaved" else 0, n, n_q, n_kv, head_dim, k_cache.shape[2], 1 if write_kv else 0, parts, _stream()), "qk_norm_rope_kv_write")
     return q_out
 
 

@@ -8,6 +8,8 @@
 //          (/root/reference/src/kipp.c:2480-2500), before the rotation;
 //   rotary (u_i, u_{i+r/2}) <- (u_i c - u_{i+r/2} s, u_{i+r/2} c + u_i s),
 //          angle = float(pos) * inv_freq[i]  (kipp.c:2368-2382); dims >= r pass;
+//          with `interleaved` pair i is (u_{2i}, u_{2i+1}) instead (another pairing that
+//          checkpoints of other families use; the general kernel only);
 //          with `angles` ([tokens][r]: r/2 cosines, then r/2 sines, made once a step by
 //          rotary_angles_kernel for all layers) the kernel reads them instead of computing them;
 //   write  key/value row of position pos goes to page table[pos / page], slot
@@ -23,7 +25,7 @@ __global__ void qk_norm_rope_kv_kernel(
     const int32_t* __restrict__ positions, const int32_t* __restrict__ seq_of_token,
     const int32_t* __restrict__ block_table, int max_blocks,
     const float* __restrict__ q_norm_w, const float* __restrict__ k_norm_w, float eps,
-    const float* __restrict__ inv_freq, const float* __restrict__ angles, int rotary_dim,
+    const float* __restrict__ inv_freq, const float* __restrict__ angles, int rotary_dim, int interleaved,
     int n_q, int n_kv, int d, int page, int n_slots, int parts, size_t part_stride) {
     __shared__ float buf[HEADS_PER_BLOCK][MAX_D];
     const int wave = threadIdx.x / KIPP_WAVE;
@@ -83,7 +85,7 @@ __global__ void qk_norm_rope_kv_kernel(
                 cs = cosf(angle);
                 sn = sinf(angle);
             }
-            const float a = buf[wave][i], b = buf[wave][i + half];
+            const float a = buf[wave][interleaved ? 2 * i : i], b = buf[wave][interleaved ? 2 * i + 1 : i + half];
             lo[c] = rotate_lo(a, b, cs, sn);
             hi[c] = rotate_hi(a, b, cs, sn);
         }
@@ -93,8 +95,8 @@ __global__ void qk_norm_rope_kv_kernel(
     for (int c = 0; c < MAX_D / 2 / KIPP_WAVE; ++c) {
         const int i = lane + c * KIPP_WAVE;
         if (rotate && i < half) {
-            buf[wave][i] = lo[c];
-            buf[wave][i + half] = hi[c];
+            buf[wave][interleaved ? 2 * i : i] = lo[c];
+            buf[wave][interleaved ? 2 * i + 1 : i + half] = hi[c];
         }
     }
     __syncthreads();
@@ -253,11 +255,12 @@ extern "C" int kipp_qk_norm_rope_kv(
     const void* qkv, int in_dtype, void* q_out, int q_dtype, void* k_cache, void* v_cache, int cache_dtype,
     const int32_t* positions, const int32_t* seq_of_token, const int32_t* block_table, int max_blocks,
     const float* q_norm_w, const float* k_norm_w, float eps, const float* inv_freq, const float* angles, int rotary_dim,
-    int n_tokens, int n_q, int n_kv, int d, int page, int write_kv, int parts, hipStream_t stream) {
+    int interleaved, int n_tokens, int n_q, int n_kv, int d, int page, int write_kv, int parts, hipStream_t stream) {
     if (n_tokens <= 0) return 0;
     if (d > MAX_D || d <= 0 || rotary_dim > d || (rotary_dim & 1)) return -1;
     const int n_slots = write_kv ? n_q + 2 * n_kv : n_q;
-    if ((d == 128 || d == 256) && ((inv_freq == nullptr && angles == nullptr) || rotary_dim == d)) {
+    const bool rotates = inv_freq != nullptr || angles != nullptr;
+    if ((d == 128 || d == 256) && (!rotates || (rotary_dim == d && !interleaved))) {
 #define KIPP_RL(TI, TO, TC)                                                                                        \
     launch_regs<TI, TO, TC>(qkv, q_out, k_cache, v_cache, positions, seq_of_token, block_table, max_blocks, q_norm_w, \
                             k_norm_w, eps, inv_freq, angles, n_tokens, n_q, n_kv, d, page, n_slots, parts, stream)
@@ -272,7 +275,7 @@ extern "C" int kipp_qk_norm_rope_kv(
 #define KIPP_RK(TI, TO, TC)                                                                                  \
     hipLaunchKernelGGL((qk_norm_rope_kv_kernel<TI, TO, TC>), grid, block, 0, stream, (const TI*)qkv,         \
                        (TO*)q_out, (TC*)k_cache, (TC*)v_cache, positions, seq_of_token, block_table,         \
-                       max_blocks, q_norm_w, k_norm_w, eps, inv_freq, angles, rotary_dim, n_q, n_kv, d, page, n_slots, parts,      \
+                       max_blocks, q_norm_w, k_norm_w, eps, inv_freq, angles, rotary_dim, interleaved, n_q, n_kv, d, page, n_slots, parts,      \
                        (size_t)n_tokens * (n_q + 2 * n_kv) * d)
     if (in_dtype == KIPP_F32 && q_dtype == KIPP_F32 && cache_dtype == KIPP_F32) KIPP_RK(float, float, float);
     else if (in_dtype == KIPP_F32 && q_dtype == KIPP_BF16 && cache_dtype == KIPP_BF16) KIPP_RK(float, bf16_t, bf16_t);

@@ -31,6 +31,8 @@ def model_variants(spec, dtype: str) -> List[Spec]:
     from ..parts import part_class
     out = list(GENERIC)
     owners = [("embedding", spec.embedding), ("norm", spec.final_norm), ("head", spec.head)]
+    if getattr(spec, "input_position", None) is not None:
+        owners.append(("position", spec.input_position))
     for layer in spec.layers:
         block = part_class("block", layer.block)
         _add(out, getattr(block, "variants", lambda s, d: [])(layer, dtype))

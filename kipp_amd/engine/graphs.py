@@ -164,7 +164,8 @@ class DecodeGraphs:
         self.graphs: "OrderedDict[Tuple[int, int], DecodeGraph]" = OrderedDict()
         model = engine.model
         self.possible = all(getattr(b, "graph_safe", False) for b in model.blocks) and all(
-            getattr(p, "graph_safe", False) for p in (model.embedding, model.final_norm, model.head))
+            getattr(p, "graph_safe", False) for p in (model.embedding, model.final_norm, model.head)
+            + ((model.input_position,) if model.input_position is not None else ()))
         self.replays = 0
 
     def applies(self, entries: Sequence) -> bool:

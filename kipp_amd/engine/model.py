@@ -15,6 +15,8 @@ from ..weights.loader import check_tensors, read_model_tensors
 def _part_specs(spec: ModelSpec):
     """(category, part spec) of every part that owns tensors, in file order."""
     yield "embedding", spec.embedding
+    if spec.input_position is not None:
+        yield "position", spec.input_position
     for layer in spec.layers:
         block_cls = part_class("block", layer.block)
         for role, category in block_cls.roles:
@@ -39,6 +41,8 @@ class Model:
         self.spec = spec
         self.rt = runtime
         self.embedding = build_part("embedding", spec.embedding, runtime)
+        self.input_position = (build_part("position", spec.input_position, runtime)
+                               if spec.input_position is not None else None)
         self.blocks = [build_part("block", layer, runtime) for layer in spec.layers]
         self.final_norm = build_part("norm", spec.final_norm, runtime)
         self.head = build_part("head", spec.head, runtime)
@@ -55,6 +59,8 @@ class Model:
     # -- weights ------------------------------------------------------------------------
     def _owners(self):
         yield "embedding", self.spec.embedding, self.embedding
+        if self.input_position is not None:
+            yield "position", self.spec.input_position, self.input_position
         for layer, block in zip(self.spec.layers, self.blocks):
             for role, category in block.roles:
                 yield category, layer.part(role), block.parts[role]
@@ -86,6 +92,8 @@ class Model:
         [wanted, vocab] at `batch.want_rows`, or None if nothing is wanted."""
         batch.step_cache.clear()
         x = self.embedding.forward(batch.tokens)
+        if self.input_position is not None:
+            x = self.input_position.forward(x, batch)
         pending = None
         for index, run in enumerate(self.spec.order):
             block = self.blocks[run.layer]

@@ -100,6 +100,7 @@ class Attention:
         angles = self.position.angles(batch) if hasattr(self.position, "angles") and hasattr(batch, "step_cache") else None
         table = batch.block_tables[cache.group]
         eps = s.qk_norm_eps if s.qk_norm_eps is not None else 0.0
+        pairing = getattr(self.position, "pairing", "half")
         # a table row is as wide as the longest context of this step, so what decides is what the step needs
         fast = rt.dtype == "bfloat16" and rt.ops.attention_fast_ok(s.num_heads, s.num_kv_heads, cache.page_size, table.shape[1])
         if rt.dtype == "bfloat16" and not fast:
@@ -107,7 +108,7 @@ class Attention:
         # single tokens only: norm, rotation, cache write and attention in one kernel, for a few of them (with
         # more rows or long contexts every split's workgroup would prepare the queries again, which costs more
         # than the rotary kernel it saves) and wherever the kernel that walks whole contexts or long ranges runs
-        fused = fast and not batch.n_portions and batch.n_decode == n \
+        fused = fast and not batch.n_portions and batch.n_decode == n and pairing == "half" \
             and rt.ops.attention_decode_fused_ok(s.head_dim, rotary_dim, inv_freq is not None) \
             and ((n <= FUSED_DECODE_ROWS and batch.max_decode_ctx < FUSED_DECODE_KEYS)
                  or rt.ops.attention_decode_streams(n, s.num_kv_heads, s.head_dim, s.num_heads // s.num_kv_heads,
@@ -124,7 +125,7 @@ class Attention:
         q = rt.ops.qk_norm_rope_kv_write(
             qkv, rt.empty((n, s.q_dim), rt.act_dtype), cache.k, cache.v,
             batch.positions, batch.seq_of_token, table, s.num_heads, s.num_kv_heads, s.head_dim,
-            self.q_norm, self.k_norm, eps, inv_freq, rotary_dim, write_kv=cache.writable, angles=angles)
+            self.q_norm, self.k_norm, eps, inv_freq, rotary_dim, write_kv=cache.writable, angles=angles, pairing=pairing)
         out = rt.empty((n, s.q_dim), rt.act_dtype)
         if fast:
             if batch.n_portions:

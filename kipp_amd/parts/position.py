@@ -3,6 +3,8 @@ it inside its own kernel; the interface is what that kernel needs:
 
     rotary_table() -> (inv_freq float32 [rotary_dim / 2] on the device, rotary_dim)
                       or (None, 0) when the part does not rotate
+    pairing           "half" (dim i turns with dim i + rotary_dim / 2; the default when
+                      the attribute is missing) or "interleaved" (dim 2i with dim 2i + 1)
     angles(batch)  -> float32 [tokens, rotary_dim] (cosines, then sines) of the
                       batch's positions, or None; optional: a mixer computes
                       the angles itself from `inv_freq` where it is missing.
@@ -10,7 +12,16 @@ it inside its own kernel; the interface is what that kernel needs:
                       (`batch.step_cache`, emptied at the start of every forward).
 
 A rotary part of another kind (scaled frequencies, another base) only has to
-produce its own table; pairing "half" rotates dim i with dim i + rotary_dim/2.
+produce its own table.
+
+A position encoding that is no rotation inside a mixer (a learned table, an
+additive code) is a part of the same category that the model applies to the
+residual stream once, after the embedding: `ModelSpec.input_position` names
+its spec, and its interface is
+
+    params(spec), load(tensors)
+    forward(x, batch) -> x          x float32 [tokens, hidden], changed in place or anew;
+                                    batch.positions holds every token's position
 """
 from __future__ import annotations
 
@@ -48,9 +59,10 @@ class Rope:
     graph_safe = True   # forward launches kernels only: no host reads, no data-dependent launches
 
     def __init__(self, spec, runtime):
-        if spec.pairing != "half":
-            raise ValueError(f"rope pairing {spec.pairing!r} is not implemented (only 'half')")
+        if spec.pairing not in ("half", "interleaved"):
+            raise ValueError(f"rope pairing {spec.pairing!r} is not implemented (half, interleaved)")
         self.spec = spec
+        self.pairing = spec.pairing
         self.rt = runtime
         self.rotary_dim = spec.head_dim if spec.rotary_dim is None else spec.rotary_dim
         self.inv_freq = self.frequencies().to(device=runtime.device, dtype=torch.float32)

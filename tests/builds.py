@@ -3,7 +3,7 @@ own small models, and builds of the decode attention whose thresholds are lowere
 reach the kernels for long contexts and many sequences with inputs it can check.  `__graft_entry__.build()`
 compiles them ahead together with the product's own list; a test that finds one missing compiles it then."""
 
-ATTENTION = [(128, 16), (128, 1), (16, 3), (48, 3), (64, 1), (32, 16), (256, 4), (80, 3), (256, 2), (16, 1)]   # (head size, group)
+ATTENTION = [(128, 16), (128, 1), (16, 3), (48, 3), (64, 1), (32, 16), (256, 4), (80, 3), (256, 2), (16, 1), (32, 2), (16, 6)]   # (head size, group)
 EARLY_STREAM = [(128, 4), (48, 3), (16, 2)]      # the kernel for long contexts takes over at 1,024 keys
 WHOLE_CONTEXTS = [(128, 4), (128, 16)]           # the whole-context kernel at few sequences
 

@@ -250,6 +250,43 @@ def test_qk_norm_rope_kv_write(n_q, n_kv, d, page, rotary, mode, norm):
     assert torch.equal(kc[keep], k0[keep]) and torch.equal(vc[keep], v0[keep])
 
 
+@pytest.mark.parametrize("n_q,n_kv,d,rotary", [(4, 2, 16, 16), (3, 1, 48, 32), (2, 1, 128, 128), (2, 2, 256, 64)])
+def test_rotary_pairing_of_neighbours(n_q, n_kv, d, rotary):
+    """pairing "interleaved": pair i is (2i, 2i + 1).  It is the half pairing of a head whose rotated dims are
+    reordered, evens first, then odds: checked against the plain rotation of the reordered head, and head
+    sizes that the half pairing rotates in registers take the general kernel here."""
+    ops = _ops()
+    rng = np.random.default_rng(d)
+    t, page = 11, 8
+    positions = list(range(20, 20 + t))
+    table = np.arange(4, dtype=np.int32)[None, :]
+    k = torch.zeros(4, n_kv, page, d, device=DEV)
+    v = torch.zeros_like(k)
+    qkv = rng.normal(size=(t, (n_q + 2 * n_kv) * d)).astype(np.float32)
+    w = (1 + 0.1 * rng.normal(size=d)).astype(np.float32)
+    inv_freq = np.power(np.float64(300.0), -(2.0 * np.arange(rotary // 2)) / rotary).astype(np.float32)
+    q = ops.qk_norm_rope_kv_write(_t(qkv), torch.empty(t, n_q * d, device=DEV), k, v, _t(positions, torch.int32),
+                                  _t([0] * t, torch.int32), _t(table, torch.int32), n_q, n_kv, d, _t(w), _t(w), 1e-6,
+                                  _t(inv_freq), rotary, pairing="interleaved").cpu().numpy().reshape(t, n_q, d)
+    order = np.concatenate([np.arange(0, rotary, 2), np.arange(1, rotary, 2)])
+
+    def ref(x, heads):
+        xh = plain.head_norm(x.astype(np.float64), heads, d, w, 1e-6).reshape(t, heads, d)
+        rot = plain.rope(xh[..., order].reshape(t, heads * rotary), heads, rotary, positions, 300.0).reshape(t, heads, rotary)
+        out = xh.copy()
+        out[..., order] = rot
+        return out
+    assert _rel(q, ref(qkv[:, :n_q * d], n_q)) < 1e-11
+    k_ref = ref(qkv[:, n_q * d:(n_q + n_kv) * d], n_kv)
+    kc = k.cpu().numpy()
+    for i, pos in enumerate(positions):
+        assert _rel(kc[pos // page, :, pos % page, :], k_ref[i]) < 1e-11
+    with pytest.raises(Exception):
+        ops.qk_norm_rope_kv_write(_t(qkv), torch.empty(t, n_q * d, device=DEV), k, v, _t(positions, torch.int32),
+                                  _t([0] * t, torch.int32), _t(table, torch.int32), n_q, n_kv, d, None, None, 1e-6,
+                                  _t(inv_freq), rotary, pairing="pairs of three")
+
+
 def test_rope_reference_vector():
     # /root/reference/tests/kipp_test.c:110-123: d=4, pos 1, theta 1e4, x=[1,2,3,4]:
     # pair (0,2) turns by 1.0, pair (1,3) by 0.01

@@ -493,3 +493,154 @@ def test_another_norm_between_products_that_fuse_theirs(tmp_path, cut):
         unregister_architecture("ToyMeanAbsForTests")
         unregister("norm", "toy_mean_abs")
         unregister("feed_forward", "toy_relu_mlp")
+
+
+# ---------------------------------------------------------------------------------------------
+# Two attention layers of different geometry in one model (head counts, head sizes, one with a window),
+# rotary encodings of both pairings (one over a part of the head only), and a position encoding that is
+# no rotation at all: a learned table added to the residual stream after the embedding.  In both
+# precisions: under bfloat16 the two geometries take different builds of the attention kernels and
+# different workspaces within one step, and pages that the window has passed go back while the
+# matrix-core kernels read the rest.
+
+G_HIDDEN, G_INNER, G_WINDOW, G_POSITIONS = 64, 80, 13, 96
+
+
+@dataclass(frozen=True)
+class LearnedPositionSpec:
+    positions: int
+    hidden_size: int
+    prefix: str = ""
+    kind: str = "toy_learned_position"
+
+
+def _register_geometries():
+    from kipp_amd.config import register_architecture
+    from kipp_amd.config.specs import (AttentionSpec, EmbeddingSpec, GatedMLPSpec, HeadSpec, LayerRun, LayerSpec, ModelSpec,
+                                       RMSNormSpec, RopeSpec)
+    from kipp_amd.parts import ParamSpec, register
+
+    @register("position", "toy_learned_position")
+    class LearnedPosition:
+        """x[t] += table[position of t]: applied by the model once, after the embedding."""
+
+        def __init__(self, spec, runtime):
+            self.spec, self.rt = spec, runtime
+
+        @staticmethod
+        def params(spec):
+            return {"table.weight": ParamSpec((spec.positions, spec.hidden_size))}
+
+        @staticmethod
+        def placement(spec):
+            return {"table.weight": "float32"}
+
+        def load(self, tensors):
+            self.table = tensors["table.weight"]
+
+        def forward(self, x, batch):
+            return x + self.table[batch.positions.long()]
+
+    class GeometriesConfig:
+        def __init__(self, d):
+            self.d = d
+
+        def to_dict(self):
+            return dict(self.d)
+
+        def model_spec(self):
+            def layer(i, attn):
+                p = f"layers.{i}."
+                return LayerSpec(block="pre_norm", parts=(
+                    ("mixer_norm", RMSNormSpec(G_HIDDEN, EPS, p + "n1.")), ("mixer", attn),
+                    ("ffn_norm", RMSNormSpec(G_HIDDEN, EPS, p + "n2.")), ("ffn", GatedMLPSpec(G_HIDDEN, G_INNER, prefix=p + "mlp."))))
+            wide = AttentionSpec(G_HIDDEN, 4, 2, 32, position=RopeSpec(32, THETA, pairing="interleaved"), qk_norm_eps=EPS,
+                                 prefix="layers.0.attn.")
+            narrow = AttentionSpec(G_HIDDEN, 6, 1, 16, position=RopeSpec(16, 50.0, rotary_dim=8), qk_norm_eps=None,
+                                   window=G_WINDOW, prefix="layers.1.attn.")
+            return ModelSpec("ToyGeometriesForTests", G_HIDDEN, VOCAB, G_POSITIONS, EmbeddingSpec(VOCAB, G_HIDDEN, "embed."),
+                             (layer(0, wide), layer(1, narrow)), (LayerRun(0), LayerRun(1)), RMSNormSpec(G_HIDDEN, EPS, "norm."),
+                             HeadSpec(VOCAB, G_HIDDEN, False, "head."),
+                             input_position=LearnedPositionSpec(G_POSITIONS, G_HIDDEN, "positions."))
+
+    register_architecture("ToyGeometriesForTests", GeometriesConfig)
+
+
+def _rotate(states, n_heads, d, rotary, pos, theta, interleaved):
+    """Rotation over the first `rotary` dims of every head; pair i is (i, i + rotary/2) or (2i, 2i + 1)."""
+    t = states.shape[0]
+    heads = np.array(states, dtype=np.float64).reshape(t, n_heads, d)
+    half = rotary // 2
+    freq = np.power(np.float64(theta), -(2.0 * np.arange(half)) / rotary).astype(np.float32)
+    angle = (np.asarray(pos, dtype=np.float32)[:, None] * freq[None, :]).astype(np.float64)
+    cos, sin = np.cos(angle)[:, None, :], np.sin(angle)[:, None, :]
+    first = np.arange(half) * 2 if interleaved else np.arange(half)
+    second = first + 1 if interleaved else first + half
+    a, b = heads[..., first].copy(), heads[..., second].copy()
+    heads[..., first] = a * cos - b * sin
+    heads[..., second] = b * cos + a * sin
+    return heads.reshape(t, n_heads * d)
+
+
+def _plain_geometries(w, tokens):
+    pos = np.arange(len(tokens))
+    x = plain.embed(w["embed.weight"], tokens) + w["positions.table.weight"][pos]
+    for i, (n_q, n_kv, d, rotary, theta, interleaved, window) in enumerate([(4, 2, 32, 32, THETA, True, None),
+                                                                           (6, 1, 16, 8, 50.0, False, G_WINDOW)]):
+        p = f"layers.{i}."
+        n = plain.rms_norm(x, w[p + "n1.weight"], EPS)
+        q, k = plain.linear(n, w[p + "attn.q_proj.weight"]), plain.linear(n, w[p + "attn.k_proj.weight"])
+        if i == 0:
+            q = plain.head_norm(q, n_q, d, w[p + "attn.q_norm.weight"], EPS)
+            k = plain.head_norm(k, n_kv, d, w[p + "attn.k_norm.weight"], EPS)
+        q, k = _rotate(q, n_q, d, rotary, pos, theta, interleaved), _rotate(k, n_kv, d, rotary, pos, theta, interleaved)
+        v = plain.linear(n, w[p + "attn.v_proj.weight"])
+        x = x + plain.linear(plain.causal_gqa(q, k, v, n_q, n_kv, d, window=window), w[p + "attn.o_proj.weight"])
+        n = plain.rms_norm(x, w[p + "n2.weight"], EPS)
+        x = x + plain.swiglu_mlp(n, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+    return plain.linear(plain.rms_norm(x, w["norm.weight"], EPS), w["head.weight"])
+
+
+def test_the_rotation_of_this_file_is_the_plain_one_where_they_meet():
+    rng = np.random.default_rng(0)
+    x = rng.normal(size=(5, 3 * 16))
+    assert np.allclose(_rotate(x, 3, 16, 16, np.arange(5), 100.0, False), plain.rope(x, 3, 16, np.arange(5), 100.0), rtol=1e-12)
+    # interleaved pairing is the half pairing of the head with its dims reordered (evens first, then odds)
+    order = np.concatenate([np.arange(0, 16, 2), np.arange(1, 16, 2)])
+    xh = x.reshape(5, 3, 16)
+    ref = plain.rope(xh[..., order].reshape(5, 48), 3, 16, np.arange(5), 100.0).reshape(5, 3, 16)
+    got = _rotate(x, 3, 16, 16, np.arange(5), 100.0, True).reshape(5, 3, 16)
+    assert np.allclose(got[..., order], ref, rtol=1e-12)
+    # a rotation over 8 of 16 dims leaves the other 8 alone
+    part = _rotate(x, 3, 16, 8, np.arange(5), 100.0, False).reshape(5, 3, 16)
+    assert np.array_equal(part[..., 8:], xh[..., 8:]) and not np.allclose(part[1:, :, :8], xh[1:, :, :8])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("cut", ["whole", "tail", "portions", "mixed"])
+def test_two_attention_geometries_a_window_and_a_learned_position(tmp_path, dtype, cut):
+    from kipp_amd.config import unregister_architecture
+    from kipp_amd.engine import Engine
+    from kipp_amd.parts import unregister
+    from kipp_amd.weights import write_random_model
+    _register_geometries()
+    try:
+        folder = write_random_model(str(tmp_path / "geometries"), {"architectures": ["ToyGeometriesForTests"]}, seed=14, dtype=dtype)
+        _, weights = plain.load_folder(folder)
+        requests = {f"g{i}": H.random_tokens(60 + i, n, VOCAB) for i, n in enumerate([9, 70, 41, 90, 33])}
+        steps = {"whole": H.whole, "tail": H.tail_one_by_one, "portions": H.changing_portions,
+                 "mixed": lambda r: H.mixed(r, seed=7)}[cut](requests)
+        engine = Engine.from_folder(folder, dtype=dtype, page_size=8, num_pages=H.peak_pages(requests, steps, 8), max_requests=4)
+        cache = engine.cache
+        assert len(cache.groups) == 2 and not cache.share                   # a window: no shared beginnings
+        assert engine.graphs is None or not engine.graphs.possible          # the learned position declares nothing: eager steps
+        got = H.replay(engine, requests, steps)
+        tol = H.NMSE_F32 if dtype == "float32" else H.NMSE_BF16["tiny"]
+        for rid, toks in requests.items():
+            H.assert_close(got[rid], _plain_geometries(weights, toks), tol, f"geometries/{dtype}/{cut}/{rid}")
+        assert cache.free_pages() == [g.pool.num_pages for g in cache.groups]
+        if dtype == "bfloat16":
+            assert engine.rt.generic_attention_launches == 0                # both geometries ran on the matrix-core kernels
+    finally:
+        unregister_architecture("ToyGeometriesForTests")
+        unregister("position", "toy_learned_position")
