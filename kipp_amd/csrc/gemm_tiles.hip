@@ -1,0 +1,437 @@
+// Matrix product for prompt portions (hundreds to thousands of rows):
+// Y[M, N] = X[M, K] . W[N, K]^T, bfloat16 operands, float32 accumulation on
+// v_mfma_f32_32x32x16_bf16, K a multiple of 32.
+//
+// A workgroup of 4 waves (2 x 2) owns a tile of outputs; a wave holds WM x WN accumulator tiles of
+// 32 x 32 (4 x 4: a workgroup tile of 256 x 256 and 256 accumulator registers a lane; also 4 x 2,
+// 2 x 4 and 2 x 2, chosen by the launcher so that the tiles of a product fill the 256 compute units
+// in whole rounds).  It walks K in steps of 32 columns.  The pieces of X and W of a step go from
+// global memory straight into LDS (global_load_lds_dwordx4: no registers, no waiting wave), four
+// steps deep.  In LDS four rows of a piece share 256 bytes, whose sixteen 16-byte slots are permuted
+// by the low bits of the group's index: the 16 lanes that read one operand column together then hit
+// sixteen different slots (no bank conflict is counted), and a wave's DMA instruction still writes
+// one contiguous KB.
+//
+// A wave is alone on its SIMD, so whatever holds up its instruction stream idles the matrix cores.
+// Every other instruction of the walk (the reads of the next operands out of LDS, the DMA of the
+// step four ahead) is therefore placed between two products, a few at a time, and the barrier of a
+// step falls between its two halves.  Measured with the DMA and the reads taken out: the walk
+// takes the same time, i.e. it is bound by the matrix cores' own rate.
+//
+// The result leaves through one of three ends:
+//   slabs   float32 [parts, M, N]: K is split over `parts` workgroups (grid.z) where the tiles
+//           alone would leave compute units idle, and the consumer adds the slabs in order
+//           (the residual add, the rotary kernel: no atomics, the same bits every time);
+//   swiglu  W = [gate; up] ([2 I, K]): a wave's columns are gate rows and the up rows that belong
+//           to them, a lane holds both values of an output, and bfloat16(silu(gate) * up)
+//           [M, I] is all that is written (/root/reference/src/kipp.c:2633-2653);
+//   bf16    bfloat16 [M, N].
+// The bfloat16 ends pass through LDS so that a lane stores 16 bytes of one row.
+//
+// Tiles are handed to the 8 dies of the GPU in blocks: workgroups that run on one die (every
+// eighth one) take tiles that share their rows of W, which that die's L2 then serves.
+#include "common.h"
+
+#define BK 32                                      // columns of a step
+#define STAGES 4
+#define THREADS 256
+#define CHUNKS (BK / 8)                            // 16-byte chunks of a row of a piece
+#define GROUP_ROWS (16 / CHUNKS)                   // rows that share 256 bytes of LDS
+#define INSTR_ROWS (4 * GROUP_ROWS)                // rows one DMA instruction of a wave brings (1 KB)
+#ifndef ABLATE_READS
+#define ABLATE_READS 0                             // measurements only: 1 takes the reads of the operands out
+#endif
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+
+union Frag {
+    u32x4 u;
+    bf16x8 v;
+};
+
+#define LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
+#define GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void*)(p))
+
+enum { END_SLABS = 0, END_SWIGLU = 1, END_BF16 = 2 };
+
+// silu(g) * u with the exponential of the hardware (base 2)
+__device__ __forceinline__ float swiglu_of(float g, float u) {
+    return g / (1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * g)) * u;
+}
+
+// every operand register of a set is tied to the wait for its reads, so that no product moves in front of it
+template <int WM, int WN>
+__device__ __forceinline__ void wait_reads(u32x4 (&fa)[WM], u32x4 (&fb)[WN]) {
+    if constexpr (WM == 4 && WN == 4)
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(fa[0]), "+v"(fa[1]), "+v"(fa[2]), "+v"(fa[3]), "+v"(fb[0]), "+v"(fb[1]), "+v"(fb[2]), "+v"(fb[3]));
+    else if constexpr (WM == 4 && WN == 3)
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(fa[0]), "+v"(fa[1]), "+v"(fa[2]), "+v"(fa[3]), "+v"(fb[0]), "+v"(fb[1]), "+v"(fb[2]));
+    else if constexpr (WM == 2 && WN == 3)
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(fa[0]), "+v"(fa[1]), "+v"(fb[0]), "+v"(fb[1]), "+v"(fb[2]));
+    else if constexpr (WM == 4)
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(fa[0]), "+v"(fa[1]), "+v"(fa[2]), "+v"(fa[3]), "+v"(fb[0]), "+v"(fb[1]));
+    else if constexpr (WN == 4)
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(fa[0]), "+v"(fa[1]), "+v"(fb[0]), "+v"(fb[1]), "+v"(fb[2]), "+v"(fb[3]));
+    else
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(fa[0]), "+v"(fa[1]), "+v"(fb[0]), "+v"(fb[1]));
+}
+
+template <int WM, int WN, int END>
+__global__ void __launch_bounds__(THREADS, 1) gemm_tiles_kernel(
+    const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* __restrict__ Y, int M, int N, int K,
+    int tiles_m, int tiles_n, int parts, int inner, int col_begin, int col_end) {
+    constexpr int TM = 64 * WM, TN = 64 * WN;                     // the workgroup's tile
+    constexpr int X_PIECE = TM * BK * 2, W_PIECE = TN * BK * 2;   // bytes of a step's pieces
+    constexpr int STAGE_BYTES = X_PIECE + W_PIECE;
+    constexpr int LOADS = WM + WN;                                // DMA instructions a wave issues a step
+    constexpr int NM = WM * WN;                                   // products of a half step
+    constexpr int NR = WM + WN;                                   // operand reads of a half step
+    constexpr int OUT_N = END == END_SWIGLU ? TN / 2 : TN;        // output columns of a tile
+    static_assert((WM == 2 || WM == 4) && (WN == 2 || WN == 3 || WN == 4), "wave tiles of 2 or 4 MFMA tiles down, 2 to 4 across");
+    static_assert(WN != 3 || END == END_SLABS, "three tiles across only for the float32 end");
+    static_assert((STAGES - 1) * LOADS < 64, "the wait counts below must fit the counter");
+    extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31, hh = lane >> 5;
+    const int wm = wave >> 1, wn = wave & 1;
+
+    // ---- which tile: workgroups id, id + 8, id + 16, ... run on one die; each die takes a run of
+    //      consecutive tiles, rows of X fastest, so that its tiles share rows of W
+    const int n_tiles = tiles_m * tiles_n;
+    const int id = blockIdx.x;
+    const int per_die = (n_tiles + 7) / 8;
+    const int tile = (id & 7) * per_die + (id >> 3);
+    if ((id >> 3) >= per_die || tile >= n_tiles) return;          // the grid is rounded up to whole dies
+    const int tm = tile % tiles_m, tn = tile / tiles_m;
+    const int part = blockIdx.z;
+    const int steps_all = K / BK;
+    const int s_begin = (int)((long long)steps_all * part / parts);
+    const int nk = (int)((long long)steps_all * (part + 1) / parts) - s_begin;
+
+    // ---- the DMA: a wave brings a quarter of each piece, INSTR_ROWS rows an instruction; a lane brings the
+    //      16 bytes that belong at its place of the KB: group g = 4 i + lane / 16 of GROUP_ROWS rows, slot
+    //      s = lane % 16, which holds chunk s ^ (g % CHUNKS) of the group: row (that / CHUNKS) of the group,
+    //      columns 8 (that % CHUNKS) .. + 7
+    const int q4 = lane >> 4, s16 = lane & 15;
+    const int in_group = s16 ^ (q4 & (CHUNKS - 1));
+    const int lane_row = GROUP_ROWS * q4 + in_group / CHUNKS, col8 = (in_group % CHUNKS) * 8;
+    const unsigned char* x_src[WM];
+    const unsigned char* w_src[WN];
+#pragma unroll
+    for (int i = 0; i < WM; ++i) {
+        const int r = (TM / 4) * wave + INSTR_ROWS * i + lane_row;
+        x_src[i] = (const unsigned char*)(X + (size_t)min(tm * TM + r, M - 1) * K + (size_t)s_begin * BK + col8);
+    }
+#pragma unroll
+    for (int i = 0; i < WN; ++i) {
+        const int r = (TN / 4) * wave + INSTR_ROWS * i + lane_row;    // row of the piece
+        int wr;
+        if (END == END_SWIGLU) {
+            // a wave's 32 WN rows of the piece are 16 WN gate rows, then the 16 WN up rows that belong to them
+            const int half = r / (32 * WN), within = r % (32 * WN);
+            const int c = col_begin + tn * OUT_N + 16 * WN * half + within % (16 * WN);
+            wr = min(c, col_end - 1) + (within >= 16 * WN ? inner : 0);
+        } else {
+            wr = min(col_begin + tn * TN + r, col_end - 1);
+        }
+        w_src[i] = (const unsigned char*)(W + (size_t)wr * K + (size_t)s_begin * BK + col8);
+    }
+    auto issue_one = [&](int step, int stage, int n) {          // DMA instruction n (0 .. LOADS - 1) of a step
+#ifdef ABLATE_DMA
+        return;
+#endif
+        unsigned char* dst = lds + stage * STAGE_BYTES;
+        const size_t at = (size_t)step * (BK * 2);
+        if (n < WM)
+            __builtin_amdgcn_global_load_lds(GLOBAL_PTR(x_src[n < WM ? n : 0] + at), LDS_PTR(dst + wave * (X_PIECE / 4) + 1024 * n), 16, 0, 0);
+        else
+            __builtin_amdgcn_global_load_lds(GLOBAL_PTR(w_src[n < WM ? 0 : n - WM] + at),
+                                             LDS_PTR(dst + X_PIECE + wave * (W_PIECE / 4) + 1024 * (n - WM)), 16, 0, 0);
+    };
+
+    // ---- a lane's place in the operands: row 32 j + l32 of the wave's rows, chunk 2 t + hh of the step
+    int frag_at[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+        const int group = l32 / GROUP_ROWS;
+        frag_at[t] = group * 256 + (((CHUNKS * (l32 % GROUP_ROWS) + 2 * t + hh) ^ (group & (CHUNKS - 1))) << 4);
+    }
+    const int a_base = wm * (X_PIECE / 2), b_base = X_PIECE + wn * (W_PIECE / 2);
+
+    f32x16 acc[WM][WN];
+#pragma unroll
+    for (int i = 0; i < WM; ++i)
+#pragma unroll
+        for (int j = 0; j < WN; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+    // ---- the walk over K.  The operands of a product leave LDS through reads written out by hand (through
+    //      ordinary loads the compiler would make every read wait for all DMA into LDS that is on its way), asked
+    //      for one half step ahead.  Steps beyond the last are asked for again from the last one (into a buffer
+    //      that nobody reads any more), so that the count of loads on their way is the same at every step.
+    u32x4 a[2][WM], b[2][WN];
+    // read R of a half step: the first row operand, every column operand, then the other row operands (the
+    // order in which the products below want them)
+#define KIPP_READ_ONE(T, STEP, KS, R)                                                                              \
+    do {                                                                                                           \
+        const uint32_t st_ = (uint32_t)(uintptr_t)LDS_PTR(lds + ((STEP) % STAGES) * STAGE_BYTES);                  \
+        const uint32_t a_at_ = st_ + a_base + frag_at[KS], b_at_ = st_ + b_base + frag_at[KS];                     \
+        if (!ABLATE_READS) {                                                                                       \
+            if ((R) == 0) asm volatile("ds_read_b128 %0, %1" : "=v"(a[T][0]) : "v"(a_at_));                        \
+            else if ((R) <= WN)                                                                                    \
+                asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(b[T][(R) <= WN ? (R) - 1 : 0]) : "v"(b_at_), "i"(((R) - 1) * 32 * BK * 2)); \
+            else                                                                                                   \
+                asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(a[T][(R) > WN ? (R) - WN : 0]) : "v"(a_at_), "i"(((R) - WN) * 32 * BK * 2)); \
+        }                                                                                                          \
+    } while (0)
+#define KIPP_PRODUCT(T, M_)                                                                         \
+    do {                                                                                            \
+        Frag fa, fb;                                                                                \
+        fa.u = a[T][(M_) / WN];                                                                     \
+        fb.u = b[T][(M_) % WN];                                                                     \
+        acc[(M_) / WN][(M_) % WN] =                                                                 \
+            __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa.v, fb.v, acc[(M_) / WN][(M_) % WN], 0, 0, 0); \
+    } while (0)
+
+#pragma unroll
+    for (int s = 0; s < STAGES; ++s)
+#pragma unroll
+        for (int n = 0; n < LOADS; ++n) issue_one(min(s, nk - 1), s, n);
+    // the loads of steps 1 .. STAGES - 1 may still be on their way
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (((STAGES - 1) * LOADS) & 15) | ((((STAGES - 1) * LOADS) >> 4) << 14));
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < NR; ++r) KIPP_READ_ONE(0, 0, 0, r);
+    for (int kt = 0; kt < nk; ++kt) {
+        // first half: products of columns 0 .. 15 of the step; the operands of the second half arrive meanwhile
+        // (the scheduler may not carry instructions over the marks: the order written here is the order meant)
+        wait_reads<WM, WN>(a[0], b[0]);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int m = 0; m < NM; ++m) {
+            KIPP_PRODUCT(0, m);
+#pragma unroll
+            for (int r = m * NR / NM; r < (m + 1) * NR / NM; ++r) KIPP_READ_ONE(1, kt, 1, r);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // second half: every wave's part of the next step has arrived, and every wave is done with this step's
+        // buffer (its operands are in registers), which the step STAGES ahead is now asked into
+        wait_reads<WM, WN>(a[1], b[1]);
+        __builtin_amdgcn_s_waitcnt(0x0F70 | (((STAGES - 2) * LOADS) & 15) | ((((STAGES - 2) * LOADS) >> 4) << 14));
+        __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+        const int ahead = min(kt + STAGES, nk - 1);
+#pragma unroll
+        for (int m = 0; m < NM; ++m) {
+            KIPP_PRODUCT(1, m);
+            // NR reads of the next step's first operands, then the LOADS DMA instructions, spread over the products
+#pragma unroll
+            for (int x = m * (NR + LOADS) / NM; x < (m + 1) * (NR + LOADS) / NM; ++x) {
+                if (x < NR) KIPP_READ_ONE(0, kt + 1, 0, x);
+                else issue_one(ahead, kt % STAGES, x - NR);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    wait_reads<WM, WN>(a[0], b[0]);
+    __builtin_amdgcn_s_waitcnt(0x0F70);      // nothing may still be on its way into LDS when the buffers are used again
+#undef KIPP_READ_ONE
+#undef KIPP_PRODUCT
+
+    // ---- the ends.  In accumulator tile (i, j) a lane holds column l32 and rows 8 (v / 4) + 4 hh + v % 4.
+    const int row0 = tm * TM + wm * (32 * WM);
+    if (END == END_SLABS) {
+        // a lane stores 4 bytes; the 32 lanes of a half wave 128 bytes of one row
+        float* out = (float*)Y + (size_t)part * M * N;
+        const int col0 = col_begin + tn * TN + wn * (32 * WN);
+#pragma unroll
+        for (int i = 0; i < WM; ++i)
+#pragma unroll
+            for (int j = 0; j < WN; ++j) {
+                const int col = col0 + 32 * j + l32;
+                if (col >= col_end) continue;
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int row = row0 + 32 * i + 8 * (v / 4) + 4 * hh + (v % 4);
+                    if (row < M) out[(size_t)row * N + col] = acc[i][j][v];
+                }
+            }
+        return;
+    }
+    if constexpr (WN == 3) return;
+    // bfloat16 ends: the wave's outputs, 32 rows at a time, go through its own corner of LDS (now free), from
+    // which a lane takes 8 neighbouring columns of one row: 16 bytes a store, whole memory lines a row
+    constexpr int WCOLS = END == END_SWIGLU ? 16 * WN : 32 * WN;   // output columns of a wave
+    constexpr int PITCH = WCOLS + 8;                               // bf16 elements a staged row (the pad spreads the banks)
+    static_assert(32 * PITCH * 2 <= STAGES * STAGE_BYTES / 4, "a wave's staging fits its quarter of LDS");
+    __syncthreads();                                               // every wave is done reading operands
+    bf16_t* stage = (bf16_t*)(lds + wave * (STAGES * STAGE_BYTES / 4));
+    bf16_t* out = (bf16_t*)Y;
+    const int out_width = END == END_SWIGLU ? inner : N;
+    const int col0 = col_begin + tn * OUT_N + wn * WCOLS;
+    constexpr int LANES_PER_ROW = WCOLS / 8, ROWS_PER_PASS = 64 / LANES_PER_ROW;
+#pragma unroll
+    for (int i = 0; i < WM; ++i) {
+#pragma unroll
+        for (int j = 0; j < WCOLS / 32; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int r = 8 * (v / 4) + 4 * hh + (v % 4);
+                const float value = END == END_SWIGLU ? swiglu_of(acc[i][j][v], acc[i][(j + WN / 2) % WN][v]) : acc[i][j][v];
+                stage[r * PITCH + 32 * j + l32] = f32_to_bf16(value);
+            }
+        // (a wave's lanes run in step: what the wave wrote it can read back without a barrier of the workgroup)
+        __builtin_amdgcn_s_waitcnt(0xC07F);                        // lgkmcnt(0): the writes above have landed
+#pragma unroll
+        for (int pass = 0; pass < 32 / ROWS_PER_PASS; ++pass) {
+            const int r = pass * ROWS_PER_PASS + lane / LANES_PER_ROW, c = (lane % LANES_PER_ROW) * 8;
+            const u32x4 v = *(const u32x4*)(stage + r * PITCH + c);
+            const int row = row0 + 32 * i + r, col = col0 + c;
+            if (row < M) {
+                if (col + 8 <= col_end && (out_width & 7) == 0) {
+                    *(u32x4*)(out + (size_t)row * out_width + col) = v;
+                } else {
+                    const bf16_t* e = (const bf16_t*)&v;
+                    for (int k = 0; k < 8; ++k)
+                        if (col + k < col_end) out[(size_t)row * out_width + col + k] = e[k];
+                }
+            }
+        }
+        __builtin_amdgcn_s_waitcnt(0xC07F);                        // the reads are done before the next 32 rows overwrite them
+    }
+}
+
+// How a product is cut: the wave's tile (WM x WN MFMA tiles) and the parts of K, for a range of output columns.
+// The cost of a cut is what its slowest compute unit does: rounds of tiles over the 256 units, each a fixed cost
+// (first data, the stores of the end) plus the steps of its part of K.  Times in microseconds, measured at the
+// benchmark's sizes; smaller wave tiles move more bytes through LDS for the same products and cost more a product.
+struct Cut {
+    int wm, wn, parts;
+    int col_begin, col_end;     // output columns
+};
+
+#define N_SHAPES 5
+static const int kShapes[N_SHAPES][2] = {{4, 4}, {4, 3}, {4, 2}, {2, 4}, {2, 2}};
+static const double kStep[N_SHAPES] = {0.80, 0.62, 0.47, 0.47, 0.27};    // one step of 32 columns of one tile
+static const double kFixed[N_SHAPES] = {13.0, 11.0, 9.0, 9.0, 6.0};      // start and end of a tile
+
+static double cut_cost(int M, int cols, int steps, int end, int shape, int parts) {
+    const int tm = 64 * kShapes[shape][0], tn = end == END_SWIGLU ? 32 * kShapes[shape][1] : 64 * kShapes[shape][1];
+    const long long tiles = (long long)((M + tm - 1) / tm) * ((cols + tn - 1) / tn);
+    const long long rounds = (tiles * parts + 255) / 256;
+    return rounds * (kFixed[shape] + kStep[shape] * ((steps + parts - 1) / parts)) + 1.0 * (parts - 1);
+}
+
+// Up to two cuts, side by side in the output's columns.  The float32 end takes one cut, whose parts of K may be
+// more than one.  The bfloat16 ends cannot split K; where whole rounds of the largest tile leave a rest of tiles
+// that would hold the 256 units for another whole round, the rest of the columns is cut into smaller tiles.
+static int plan(int M, int N, int K, int end, int max_parts, Cut* cuts) {
+    const int steps = K / BK;
+    const int cols = end == END_SWIGLU ? N / 2 : N;
+    double best = 1e30;
+    int n_cuts = 1;
+    for (int s = 0; s < N_SHAPES; ++s) {
+        if (kShapes[s][1] == 3 && end != END_SLABS) continue;
+        for (int parts = 1; parts <= (end == END_SLABS ? max_parts : 1) && parts <= steps; ++parts) {
+            const double cost = cut_cost(M, cols, steps, end, s, parts);
+            if (cost < best - 1e-9) {
+                best = cost;
+                cuts[0] = {kShapes[s][0], kShapes[s][1], parts, 0, cols};
+            }
+        }
+    }
+    if (end != END_SLABS) {
+        // whole rounds of the largest tile first, the rest of the columns in smaller tiles
+        const int tn = end == END_SWIGLU ? 128 : 256;
+        const int tiles_m = (M + 255) / 256;
+        const long long whole = ((long long)tiles_m * (cols / tn)) / 256 * 256;      // tiles of whole rounds
+        const int first_cols = (int)(whole / tiles_m) * tn;
+        if (first_cols > 0 && first_cols < cols) {
+            for (int s = 2; s < N_SHAPES; ++s) {
+                const double cost = cut_cost(M, first_cols, steps, end, 0, 1) + cut_cost(M, cols - first_cols, steps, end, s, 1);
+                if (cost < best - 1e-9) {
+                    best = cost;
+                    n_cuts = 2;
+                    cuts[0] = {4, 4, 1, 0, first_cols};
+                    cuts[1] = {kShapes[s][0], kShapes[s][1], 1, first_cols, cols};
+                }
+            }
+        }
+    }
+    return n_cuts;
+}
+
+template <int WM, int WN, int END>
+static int launch_cut(const void* X, const void* W, void* Y, int M, int N, int K, const Cut& cut, hipStream_t stream) {
+    constexpr int lds_bytes = STAGES * 64 * (WM + WN) * BK * 2;
+    static bool prepared = false;
+    if (!prepared) {
+        if (hipFuncSetAttribute((const void*)gemm_tiles_kernel<WM, WN, END>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                lds_bytes) != hipSuccess)
+            return -6;
+        prepared = true;
+    }
+    const int tm = 64 * WM, tn = END == END_SWIGLU ? 32 * WN : 64 * WN;
+    const int tiles_m = (M + tm - 1) / tm, tiles_n = (cut.col_end - cut.col_begin + tn - 1) / tn;
+    const int per_die = (tiles_m * tiles_n + 7) / 8;
+    hipLaunchKernelGGL((gemm_tiles_kernel<WM, WN, END>), dim3(per_die * 8, 1, cut.parts), dim3(THREADS), lds_bytes, stream,
+                       (const bf16_t*)X, (const bf16_t*)W, Y, M, N, K, tiles_m, tiles_n, cut.parts, N / 2, cut.col_begin,
+                       cut.col_end);
+    return KIPP_LAUNCH_CHECK();
+}
+
+template <int END>
+static int launch_end(const void* X, const void* W, void* Y, int M, int N, int K, const Cut& cut, hipStream_t stream) {
+    if (cut.wm == 4 && cut.wn == 4) return launch_cut<4, 4, END>(X, W, Y, M, N, K, cut, stream);
+    if (cut.wm == 4 && cut.wn == 2) return launch_cut<4, 2, END>(X, W, Y, M, N, K, cut, stream);
+    if (cut.wm == 2 && cut.wn == 4) return launch_cut<2, 4, END>(X, W, Y, M, N, K, cut, stream);
+    if (cut.wm == 2 && cut.wn == 2) return launch_cut<2, 2, END>(X, W, Y, M, N, K, cut, stream);
+    if constexpr (END == END_SLABS) {
+        if (cut.wm == 4 && cut.wn == 3) return launch_cut<4, 3, END>(X, W, Y, M, N, K, cut, stream);
+        if (cut.wm == 2 && cut.wn == 3) return launch_cut<2, 3, END>(X, W, Y, M, N, K, cut, stream);
+    }
+    return -5;
+}
+
+extern "C" {
+
+// parts that kipp_gemm_tiles cuts K into for these sizes when it may use up to `max_parts` (1 for the ends that are not slabs)
+int kipp_gemm_tiles_parts(int M, int N, int K, int end, int max_parts) {
+    if (K <= 0 || (K % BK) || M <= 0 || N <= 0) return -1;
+    Cut cuts[2];
+    plan(M, N, K, end, max_parts, cuts);
+    return cuts[0].parts;
+}
+
+// Y: float32 [parts, M, N] with parts = kipp_gemm_tiles_parts(...) (end 0), bfloat16 [M, N / 2] = silu(gate) * up for
+// W = [gate; up] (end 1), bfloat16 [M, N] (end 2).  K a multiple of 32.  `force`: 0, or 100 wm + 10 wn + parts to take
+// that cut for all columns whatever the plan says (measurements and tests).
+int kipp_gemm_tiles(const void* X, const void* W, void* Y, int M, int N, int K, int end, int max_parts, int force,
+                    hipStream_t stream) {
+    if (M <= 0 || N <= 0) return 0;
+    if (K <= 0 || (K % BK) || max_parts <= 0) return -1;
+    if (end != END_SLABS && end != END_SWIGLU && end != END_BF16) return -3;
+    if (end == END_SWIGLU && (N & 1)) return -4;
+    Cut cuts[2];
+    int n_cuts = plan(M, N, K, end, max_parts, cuts);
+    if (force) {
+        n_cuts = 1;
+        cuts[0] = {force / 100, (force / 10) % 10, force % 10, 0, end == END_SWIGLU ? N / 2 : N};
+    }
+    for (int c = 0; c < n_cuts; ++c) {
+        const Cut& cut = cuts[c];
+        if (cut.parts < 1 || cut.parts > K / BK || (end != END_SLABS && cut.parts != 1)) return -2;
+        const int rc = end == END_SLABS ? launch_end<END_SLABS>(X, W, Y, M, N, K, cut, stream)
+                       : end == END_SWIGLU ? launch_end<END_SWIGLU>(X, W, Y, M, N, K, cut, stream)
+                                           : launch_end<END_BF16>(X, W, Y, M, N, K, cut, stream);
+        if (rc != 0) return rc;
+    }
+    return 0;
+}
+
+}  // extern "C"

@@ -610,6 +610,41 @@ def gemm_skinny_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tens
     return out
 
 
+TILES_END = {"slabs": 0, "swiglu": 1, "bf16": 2}
+
+
+def gemm_tiles_ok(m: int, k: int) -> bool:
+    """Shapes the product for prompt portions takes: K a multiple of 32 (any number of rows; it is built for hundreds)."""
+    return m > 0 and k > 0 and k % 32 == 0
+
+
+def gemm_tiles(x: torch.Tensor, w: torch.Tensor, end: str = "slabs", max_parts: int = 1, force: int = 0) -> torch.Tensor:
+    """x [M, K] . w [N, K]^T on the matrix cores for many rows, bfloat16 operands, float32 accumulation.
+    end "slabs": float32 [parts, M, N] whose sum over parts is the product (parts <= max_parts, chosen from the shape);
+    "swiglu": w = [gate; up] of [2 I, K], the result is bfloat16 [M, I] = silu(x . gate^T) * (x . up^T);
+    "bf16": bfloat16 [M, N].  `force` = 100 wm + 10 wn + parts takes that cut instead of the planned one (tests)."""
+    _dev(x, w)
+    m, k = x.shape
+    n = w.shape[0]
+    _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm_tiles: bfloat16 operands")
+    _need(w.shape == (n, k) and gemm_tiles_ok(m, k), "gemm_tiles: shapes do not match, or K is no multiple of 32")
+    _need(end in TILES_END, f"gemm_tiles: end {end!r} is not one of {sorted(TILES_END)}")
+    code = TILES_END[end]
+    lib = build.library("gemm_tiles")
+    if end == "slabs":
+        parts = force % 10 if force else lib.kipp_gemm_tiles_parts(m, n, k, code, int(max_parts))
+        _need(parts >= 1, "gemm_tiles: no cut for these sizes")
+        out = torch.empty((parts, m, n), dtype=torch.float32, device=x.device)
+    elif end == "swiglu":
+        _need(n % 2 == 0, "gemm_tiles: [gate; up] has an even number of rows")
+        out = torch.empty((m, n // 2), dtype=torch.bfloat16, device=x.device)
+    else:
+        out = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
+    fn = _fn("gemm_tiles", "kipp_gemm_tiles", [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr])
+    _check(fn(_ptr(x), _ptr(w), _ptr(out), m, n, k, code, int(max_parts), int(force), _stream()), "gemm_tiles")
+    return out
+
+
 def gemm_f32(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     """out[M,N] = x[M,K] . w[N,K]^T in true float32 (w float32 or bfloat16)."""
     _dev(x, w, out)

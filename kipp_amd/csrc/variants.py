@@ -17,7 +17,7 @@ from typing import List, Optional, Tuple
 Spec = Tuple[str, Optional[dict]]
 
 GENERIC: List[Spec] = [(name, None) for name in
-                       ("elementwise", "rope_kv", "attention_generic", "gemm_f32", "gemm_skinny", "gemm_rows", "sampling")]
+                       ("elementwise", "rope_kv", "attention_generic", "gemm_f32", "gemm_skinny", "gemm_rows", "gemm_tiles", "sampling")]
 
 
 def _add(out: List[Spec], more) -> None:

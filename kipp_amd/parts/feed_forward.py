@@ -59,6 +59,8 @@ class GatedMLP:
         if ours and w.pairs:
             # streamed from the paired tiles: the columns come out gate tile by gate tile
             rt.ops.swiglu(rt.ops.gemm_rows(x, w.rows, max_parts=12, tiles=w.tiles, pairs=True), act, pairs=True)
+        elif w.dtype == x.dtype == torch.bfloat16 and rows > rt.ops.ROWS_MAX_ROWS:
+            act = rt.gated(x, w, act)       # many rows: both products and the activation, by whichever way is faster
         else:
-            rt.ops.swiglu(rt.linear(x, w, slabs=True, low_precision_out=True), act)
+            rt.ops.swiglu(rt.linear(x, w, slabs=True), act)
         return rt.linear(act, self.w_down, slabs=True, defer=True)

@@ -107,6 +107,11 @@ class Runtime:
         self.library_products = 0   # calls that went to the library (they stay out of HIP graphs)
         self.generic_attention_launches = 0   # bfloat16 attention that fell to the generic kernel (geometry the matrix-core kernels refuse)
         self.fuse_norms = True      # few rows: residual add and norm ride on the products around them
+        # products of more than 256 rows: our own matrix-core kernel or the library's, whichever is faster for the
+        # shape ("auto": both are timed once, at the shape's first use); True / False: always ours / always the library's
+        self.own_prompt_products = "auto"
+        self.prompt_product_choices = {}     # shape -> True (ours) / False (the library's)
+        self.tile_products = 0      # products of more than 256 rows that ran on our own kernel
         torch.backends.cuda.matmul.allow_tf32 = False
 
     # -- placement -----------------------------------------------------------
@@ -168,14 +173,66 @@ class Runtime:
         rows_out, sumsq = self.ops.gemm_skinny(delta.x, w.rows, tiles=w.tiles, add_norm=(x, norm_weight))
         return ScaledRows(rows_out, sumsq, (w.shape[0] + 15) // 16, eps)
 
-    def linear(self, x, w, slabs: bool = False, low_precision_out: bool = False, defer: bool = False):
+    # -- products of prompt portions ------------------------------------------------------------
+    def _ours_is_faster(self, key, ours, library) -> bool:
+        """Which of two ways to compute one product is taken for the shape `key`: decided once, by the
+        switch or by timing both on the operands at hand (three runs each after a first one)."""
+        choice = self.prompt_product_choices.get(key)
+        if choice is None:
+            if self.own_prompt_products != "auto":
+                choice = bool(self.own_prompt_products)
+            else:
+                times = []
+                for run in (ours, library):
+                    run()
+                    begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    begin.record()
+                    for _ in range(3):
+                        run()
+                    end.record()
+                    end.synchronize()
+                    times.append(begin.elapsed_time(end))
+                choice = times[0] <= times[1]
+            self.prompt_product_choices[key] = choice
+        return choice
+
+    def _library_product(self, x, w):
+        """bfloat16 x bfloat16 with float32 accumulation and a float32 result by the library (hipBLASLt through torch.mm)."""
+        if self._mm_out_f32 is None:
+            try:
+                torch.mm(x[:1], w[:1].t(), out_dtype=torch.float32)
+                self._mm_out_f32 = True
+            except (RuntimeError, TypeError):
+                self._mm_out_f32 = False
+        if self._mm_out_f32:
+            return torch.mm(x, w.t(), out_dtype=torch.float32)
+        # a torch without float32 results from bfloat16 products would round deltas of the residual stream
+        raise RuntimeError("this torch cannot return float32 from a bfloat16 product; the library product is not used then")
+
+    def gated(self, x, w: "Weight", act: torch.Tensor) -> torch.Tensor:
+        """act [M, I] (bfloat16) = silu(x . gate^T) * (x . up^T) for many rows, w = [gate; up]: our kernel
+        computes both products and the activation in one pass; after the library's product (float32, so
+        that either way rounds once, after the activation) the activation is a kernel of its own."""
+        m, k = x.shape
+        rows = w.rows
+
+        def ours():
+            return self.ops.gemm_tiles(x, rows, end="swiglu")
+
+        def library():
+            return self.ops.swiglu(self._library_product(x, rows), act)
+        if self.ops.gemm_tiles_ok(m, k) and self._ours_is_faster(("gated", -(-m // 128), rows.shape[0], k), ours, library):
+            self.tile_products += 1
+            return ours()
+        self.library_products += 1
+        return library()
+
+    def linear(self, x, w, slabs: bool = False, defer: bool = False):
         """float32 [M, N] = x [M, K] . w [N, K]^T.  With `slabs` the result may come
         as [parts, M, N] whose sum over parts is the product (few rows against a
         weight with few output rows: the contraction is split over workgroups and
         the consumer adds the slabs in order); an integer is the most slabs the
-        consumer takes.  With `low_precision_out` a large
-        bfloat16 product may be returned in bfloat16 (for a consumer that rounds to
-        bfloat16 anyway and is bound by reading it).  `x` may be ScaledRows.  With
+        consumer takes.  `x` may be ScaledRows.  With
         `defer` the product may come back as a `Deferred` (for a delta of the
         residual stream, which the next norm launches or `settle` does)."""
         if defer and self.fuse_norms and not isinstance(x, ScaledRows) and self._few_rows(x.shape[0], x.shape[1], w):
@@ -206,17 +263,18 @@ class Runtime:
             else:
                 y = self.ops.gemm_rows(x, w, max_parts=1 if most == 0 else (most or 12), tiles=tiles)
             return y if y.shape[0] > 1 else y[0]
-        # bfloat16 x bfloat16 with float32 accumulation: the library product
+        # more than 256 rows (prompt portions): our matrix-core kernel, or the library's product
+        if self.ops.gemm_tiles_ok(m, x.shape[1]):
+            most = 1 if slabs is False else (4 if slabs is True else max(1, min(4, int(slabs))))
+
+            def ours():
+                y = self.ops.gemm_tiles(x, w, end="slabs", max_parts=most)
+                return y if y.shape[0] > 1 else y[0]
+
+            def library():
+                return self._library_product(x, w)
+            if self._ours_is_faster(("linear", -(-m // 128), n, x.shape[1], most), ours, library):
+                self.tile_products += 1
+                return ours()
         self.library_products += 1
-        if self._mm_out_f32 is None:
-            try:
-                torch.mm(x[:1], w[:1].t(), out_dtype=torch.float32)
-                self._mm_out_f32 = True
-            except (RuntimeError, TypeError):
-                self._mm_out_f32 = False
-        if low_precision_out:
-            return torch.mm(x, w.t())
-        if self._mm_out_f32:
-            return torch.mm(x, w.t(), out_dtype=torch.float32)
-        y = torch.mm(x, w.t())
-        return self.ops.cast(y, self.empty((m, n), torch.float32))
+        return self._library_product(x, w)

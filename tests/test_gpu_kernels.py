@@ -733,6 +733,65 @@ def test_gemm_rows(m, n, k, max_parts):
                            ops.gemm_rows(x.to(DEV), wd, max_parts))
 
 
+TILE_CUTS = [0, 441, 442, 421, 243, 221, 224, 431, 232]      # 100 wm + 10 wn + parts; 0: what the launcher plans
+
+
+@pytest.mark.parametrize("force", TILE_CUTS)
+@pytest.mark.parametrize("m,n,k", [(257, 300, 64), (300, 2560, 96), (513, 77, 2560), (1000, 640, 352), (64, 16, 32)])
+def test_gemm_tiles_float32_end(m, n, k, force):
+    """The product for prompt portions, every wave tile and split of K, at sizes that end inside tiles on both
+    sides (and one smaller than any tile): against float64, and exactly on small integers."""
+    ops = _ops()
+    if force % 10 > k // 32:
+        pytest.skip("more parts than steps of K")
+    rng = np.random.default_rng(m + n + force)
+    x = torch.tensor(rng.normal(size=(m, k)), dtype=torch.bfloat16)
+    w = torch.tensor(rng.normal(size=(n, k)), dtype=torch.bfloat16)
+    out = ops.gemm_tiles(x.to(DEV), w.to(DEV), "slabs", max_parts=4, force=force)
+    assert tuple(out.shape[1:]) == (m, n) and (out.shape[0] == force % 10 if force else 1 <= out.shape[0] <= 4)
+    ref = x.double().numpy() @ w.double().numpy().T
+    assert _rel(out.sum(dim=0).cpu().numpy(), ref) < 1e-11
+    xi = torch.tensor(rng.integers(-3, 4, size=(m, k)), dtype=torch.bfloat16)
+    wi = torch.tensor(rng.integers(-3, 4, size=(n, k)), dtype=torch.bfloat16)
+    out = ops.gemm_tiles(xi.to(DEV), wi.to(DEV), "slabs", max_parts=4, force=force).sum(dim=0)
+    assert np.array_equal(out.cpu().numpy(), xi.float().numpy() @ wi.float().numpy().T)
+
+
+@pytest.mark.parametrize("force", [0, 441, 421, 241, 221])
+@pytest.mark.parametrize("m,inner,k", [(257, 150, 64), (600, 9728 // 8, 160), (300, 24, 2560), (2050, 1300, 96)])
+def test_gemm_tiles_swiglu_and_bfloat16_ends(m, inner, k, force):
+    """W = [gate; up]: silu(x . gate^T) * (x . up^T) rounded once, at the end (gate first: the other way round
+    gives another result), also where the launcher cuts the columns into two kinds of tiles; and the plain
+    bfloat16 end.  Widths that are no multiple of 8 take the store of single values."""
+    ops = _ops()
+    rng = np.random.default_rng(m + inner + force)
+    x = torch.tensor(rng.normal(size=(m, k)), dtype=torch.bfloat16)
+    w = torch.tensor(rng.normal(size=(2 * inner, k)) * 0.3, dtype=torch.bfloat16)
+    act = ops.gemm_tiles(x.to(DEV), w.to(DEV), "swiglu", force=force)
+    assert act.dtype == torch.bfloat16 and tuple(act.shape) == (m, inner)
+    both = x.double().numpy() @ w.double().numpy().T
+    ref = plain.silu(both[:, :inner]) * both[:, inner:]
+    assert _rel(act.float().cpu().numpy(), ref) < 2e-5
+    assert _rel(act.float().cpu().numpy(), plain.silu(both[:, inner:]) * both[:, :inner]) > 1e-2
+    rounded = ops.gemm_tiles(x.to(DEV), w.to(DEV), "bf16", force=force)
+    assert rounded.dtype == torch.bfloat16 and _rel(rounded.float().cpu().numpy(), both) < 2e-5
+    # bit for bit what rounding the float32 end gives
+    exact = ops.gemm_tiles(x.to(DEV), w.to(DEV), "slabs", force=force)[0]
+    assert torch.equal(rounded, exact.to(torch.bfloat16))
+
+
+def test_gemm_tiles_refuses_what_it_cannot_do():
+    ops = _ops()
+    x = torch.zeros(300, 40, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(Exception):
+        ops.gemm_tiles(x, torch.zeros(64, 40, dtype=torch.bfloat16, device=DEV))            # K no multiple of 32
+    with pytest.raises(Exception):
+        ops.gemm_tiles(x.float(), torch.zeros(64, 40, device=DEV))                             # float32 operands
+    with pytest.raises(Exception):
+        ops.gemm_tiles(torch.zeros(300, 64, dtype=torch.bfloat16, device=DEV), torch.zeros(63, 64, dtype=torch.bfloat16, device=DEV),
+                       "swiglu")                                                               # an odd number of rows is no [gate; up]
+
+
 def test_consumers_add_slabs_in_order():
     """The rotary kernels and SwiGLU take a product that comes in slabs."""
     ops = _ops()
