@@ -58,6 +58,7 @@ union Frag {
 
 
 typedef __attribute__((ext_vector_type(2))) float f32x2;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
 
 // two floats to two bfloat16 (round to nearest even) in one 32-bit word: the conversion
@@ -76,7 +77,8 @@ __global__ void __launch_bounds__(THREADS, 2) attention_prefill_kernel(
     bf16_t* __restrict__ out, const int32_t* __restrict__ item_seq, const int32_t* __restrict__ item_tile,
     const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len, const int32_t* __restrict__ positions,
     const int32_t* __restrict__ block_table, int max_blocks, int n_q, int n_kv, int page, float scale_log2e,
-    int window) {
+    int window, int tile_rows, const int32_t* __restrict__ item_split, int split_keys, float* __restrict__ part_acc,
+    float* __restrict__ part_ml, int max_splits) {
     __shared__ __attribute__((aligned(16))) bf16_t Ks[BN * K_PITCH];
     __shared__ __attribute__((aligned(16))) bf16_t Vt[DP * V_PITCH];
     __shared__ int s_page[MAX_PAGES];
@@ -92,9 +94,9 @@ __global__ void __launch_bounds__(THREADS, 2) attention_prefill_kernel(
     const int item = work / n_q, head = work % n_q;
     const int kvh = head / (n_q / n_kv);
     const int seq = item_seq[item];
-    const int tile_row0 = item_tile[item] * BM;                 // first row of the tile within the portion
+    const int tile_row0 = item_tile[item] * tile_rows;          // first row of the tile within the portion
     const int row0 = q_start[seq] + tile_row0;                  // ... within the batch
-    const int rows_in_tile = min(BM, q_len[seq] - tile_row0);
+    const int rows_in_tile = min(tile_rows, q_len[seq] - tile_row0);
     const int pos0 = positions[row0];                           // position of the tile's first query
     const int last_pos = pos0 + rows_in_tile - 1;
     const int32_t* table = block_table + (size_t)seq * max_blocks;
@@ -125,14 +127,16 @@ __global__ void __launch_bounds__(THREADS, 2) attention_prefill_kernel(
         for (int i = tid; i < (DP - HEAD_DIM) * V_PITCH; i += THREADS) Vt[HEAD_DIM * V_PITCH + i] = 0;
     }
 
-    const int tile_lo = (window > 0 ? max(0, pos0 - window + 1) : 0) / BN;
-    const int tile_hi = last_pos / BN;
+    // with `split_keys` the keys are cut at multiples of it and this work item takes one cut (windows are not split)
+    const int split = split_keys > 0 ? item_split[item] : 0;
+    const int tile_lo = split_keys > 0 ? split * (split_keys / BN) : (window > 0 ? max(0, pos0 - window + 1) : 0) / BN;
+    const int tile_hi = split_keys > 0 ? min(last_pos / BN, (split + 1) * (split_keys / BN) - 1) : last_pos / BN;
 
     // The pages of the keys this workgroup reads, once, into LDS: the loads of a tile then
     // depend on nothing in flight and are issued back to back.  The page size is a power of
     // two and the table row fits s_page (both checked by the launcher).
     const int page_shift = __builtin_ctz(page);
-    const int first_block = (tile_lo * BN) >> page_shift, last_block = last_pos >> page_shift;
+    const int first_block = (tile_lo * BN) >> page_shift, last_block = min(last_pos, tile_hi * BN + BN - 1) >> page_shift;
     for (int i = tid; i <= last_block - first_block; i += THREADS) s_page[i] = table[first_block + i];
     __syncthreads();
     // address of key s of this sequence and head; s is clamped to the last key of the portion
@@ -269,6 +273,24 @@ __global__ void __launch_bounds__(THREADS, 2) attention_prefill_kernel(
             }
     }
     if (!row_valid) return;
+    if (split_keys > 0) {
+        // one cut of the keys: the sums as they are, with their reference maximum (base 2) and their
+        // denominator; attention_prefill_merge_kernel adds the cuts of a row in order
+        const size_t slot = ((size_t)(row0 + my_row) * n_q + head) * max_splits + split;
+        if (hh == 0) {
+            part_ml[slot * 2] = m_run == -INFINITY ? -INFINITY : m_run * scale_log2e;
+            part_ml[slot * 2 + 1] = l_run;
+        }
+        float* p_row = part_acc + slot * HEAD_DIM;
+#pragma unroll
+        for (int dt = 0; dt < DTILES; ++dt)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int dcol = 32 * dt + 8 * g + 4 * hh;
+                if (dcol < HEAD_DIM) *(f32x4*)(p_row + dcol) = (f32x4){o[dt][4 * g + 0], o[dt][4 * g + 1], o[dt][4 * g + 2], o[dt][4 * g + 3]};
+            }
+        return;
+    }
     // O^T register v of tile dt is column 32 dt + 8 (v / 4) + 4 hh + v % 4 of this lane's query
     const float inv = 1.0f / l_run;
     bf16_t* o_row = out + ((size_t)(row0 + my_row) * n_q + head) * HEAD_DIM;
@@ -312,7 +334,8 @@ __global__ void __launch_bounds__(THREADS, 2) attention_prefill_dma_kernel(
     bf16_t* __restrict__ out, const int32_t* __restrict__ item_seq, const int32_t* __restrict__ item_tile,
     const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len, const int32_t* __restrict__ positions,
     const int32_t* __restrict__ block_table, int max_blocks, int n_q, int n_kv, int page, float scale_log2e,
-    int window) {
+    int window, int tile_rows, const int32_t* __restrict__ item_split, int split_keys, float* __restrict__ part_acc,
+    float* __restrict__ part_ml, int max_splits) {
     // the two tile buffers are two objects (one static, one dynamic): the compiler then sees that the loads
     // into one never touch what is read from the other, and makes no read wait for them
     __shared__ __attribute__((aligned(1024))) unsigned char tile_a[2 * TILE_BYTES];
@@ -328,9 +351,9 @@ __global__ void __launch_bounds__(THREADS, 2) attention_prefill_dma_kernel(
     const int item = work / n_q, head = work % n_q;
     const int kvh = head / (n_q / n_kv);
     const int seq = item_seq[item];
-    const int tile_row0 = item_tile[item] * BM;
+    const int tile_row0 = item_tile[item] * tile_rows;
     const int row0 = q_start[seq] + tile_row0;
-    const int rows_in_tile = min(BM, q_len[seq] - tile_row0);
+    const int rows_in_tile = min(tile_rows, q_len[seq] - tile_row0);
     const int pos0 = positions[row0];
     const int last_pos = pos0 + rows_in_tile - 1;
     const int32_t* table = block_table + (size_t)seq * max_blocks;
@@ -355,10 +378,12 @@ __global__ void __launch_bounds__(THREADS, 2) attention_prefill_dma_kernel(
         for (int v = 0; v < 16; ++v) o[dt][v] = 0.0f;
     float m_run = -INFINITY, l_run = 0.0f;
 
-    const int tile_lo = (window > 0 ? max(0, pos0 - window + 1) : 0) / BN;
-    const int tile_hi = last_pos / BN;
+    // with `split_keys` the keys are cut at multiples of it and this work item takes one cut (windows are not split)
+    const int split = split_keys > 0 ? item_split[item] : 0;
+    const int tile_lo = split_keys > 0 ? split * (split_keys / BN) : (window > 0 ? max(0, pos0 - window + 1) : 0) / BN;
+    const int tile_hi = split_keys > 0 ? min(last_pos / BN, (split + 1) * (split_keys / BN) - 1) : last_pos / BN;
     const int page_shift = __builtin_ctz(page);
-    const int first_block = (tile_lo * BN) >> page_shift, last_block = last_pos >> page_shift;
+    const int first_block = (tile_lo * BN) >> page_shift, last_block = min(last_pos, tile_hi * BN + BN - 1) >> page_shift;
     for (int i = tid; i <= last_block - first_block; i += THREADS) s_page[i] = table[first_block + i];
     __syncthreads();
 
@@ -528,6 +553,24 @@ __global__ void __launch_bounds__(THREADS, 2) attention_prefill_dma_kernel(
         if (kt + 1 <= tile_hi) work_tile(kt + 1, tile_b, tile_a);
     }
     if (!row_valid) return;
+    if (split_keys > 0) {
+        // one cut of the keys: the sums as they are, with their reference maximum (base 2) and their
+        // denominator; attention_prefill_merge_kernel adds the cuts of a row in order
+        const size_t slot = ((size_t)(row0 + my_row) * n_q + head) * max_splits + split;
+        if (hh == 0) {
+            part_ml[slot * 2] = m_run == -INFINITY ? -INFINITY : m_run * scale_log2e;
+            part_ml[slot * 2 + 1] = l_run;
+        }
+        float* p_row = part_acc + slot * HEAD_DIM;
+#pragma unroll
+        for (int dt = 0; dt < DTILES; ++dt)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int dcol = 32 * dt + 8 * g + 4 * hh;
+                if (dcol < HEAD_DIM) *(f32x4*)(p_row + dcol) = (f32x4){o[dt][4 * g + 0], o[dt][4 * g + 1], o[dt][4 * g + 2], o[dt][4 * g + 3]};
+            }
+        return;
+    }
     const float inv = 1.0f / l_run;
     bf16_t* o_row = out + ((size_t)(row0 + my_row) * n_q + head) * HEAD_DIM;
 #pragma unroll
@@ -541,24 +584,61 @@ __global__ void __launch_bounds__(THREADS, 2) attention_prefill_dma_kernel(
 }
 #endif  // HEAD_DIM == 128
 
+// The cuts of a row's keys, added in order: out = sum_s acc_s 2^(m_s - m) / sum_s l_s 2^(m_s - m).  A wave a
+// (row, head).  How many cuts a row has follows from the last position of the tile of query rows it lies in (every
+// row of a tile has the tile's cuts; a cut that begins behind a row's own position holds nothing: m = -inf, l = 0).
+__global__ void __launch_bounds__(KIPP_WAVE) attention_prefill_merge_kernel(
+    const float* __restrict__ part_acc, const float* __restrict__ part_ml, bf16_t* __restrict__ out,
+    const int32_t* __restrict__ merge_rows, const int32_t* __restrict__ merge_cuts, int n_q, int max_splits) {
+    const int head = blockIdx.x, lane = threadIdx.x;
+    const int row = merge_rows[blockIdx.y], cuts = merge_cuts[blockIdx.y];
+    const size_t slot0 = ((size_t)row * n_q + head) * max_splits;
+    float m = -INFINITY;
+    for (int s = 0; s < cuts; ++s) m = fmaxf(m, part_ml[(slot0 + s) * 2]);
+    float denom = 0.0f;
+    for (int s = 0; s < cuts; ++s) {
+        const float ms = part_ml[(slot0 + s) * 2];
+        if (ms != -INFINITY) denom += part_ml[(slot0 + s) * 2 + 1] * exp2f(ms - m);
+    }
+    for (int dcol = lane; dcol < HEAD_DIM; dcol += KIPP_WAVE) {
+        float a = 0.0f;
+        for (int s = 0; s < cuts; ++s) {
+            const float ms = part_ml[(slot0 + s) * 2];
+            if (ms != -INFINITY) a += part_acc[(slot0 + s) * HEAD_DIM + dcol] * exp2f(ms - m);
+        }
+        out[((size_t)row * n_q + head) * HEAD_DIM + dcol] = f32_to_bf16(a / denom);
+    }
+}
+
 extern "C" {
 
 int kipp_attention_prefill_rows() { return BM; }
 
-// `item_seq[i]`, `item_tile[i]`: sequence (row of the block table) and 128-row
-// tile of its portion for work item i; best sorted from the longest key range to the shortest.
+// `item_seq[i]`, `item_tile[i]`: sequence (row of the block table) and tile of `tile_rows` query rows
+// of its portion for work item i; best sorted from the longest key range to the shortest.
+// `tile_rows`: 128, or 64 or 32 where the items of 128 rows would leave compute units idle (a wave takes
+// 32 rows; with fewer rows the other waves of a workgroup only help to bring keys and values in).
 int kipp_attention_prefill(const void* q, const void* k_cache, const void* v_cache, void* out,
                            const int32_t* item_seq, const int32_t* item_tile, const int32_t* q_start,
                            const int32_t* q_len, const int32_t* positions, const int32_t* block_table, int max_blocks,
                            int n_items, int n_q, int n_kv, int head_dim, int page, float scale, int window,
+                           int tile_rows, const int32_t* item_split, int split_keys, float* part_acc, float* part_ml,
+                           int max_splits, const int32_t* merge_rows, const int32_t* merge_cuts, int n_merge,
                            hipStream_t stream) {
     if (n_items <= 0) return 0;
     if (head_dim != HEAD_DIM || n_kv <= 0 || n_q % n_kv) return -1;
+    if (tile_rows != 128 && tile_rows != 64 && tile_rows != 32) return -7;
+    // keys cut at multiples of `split_keys` (0: not cut): work item i then takes cut item_split[i] and writes sums that
+    // are not normalised yet into part_acc [rows, n_q, max_splits, head_dim] / part_ml [.., 2]; rows merge_rows[j] with
+    // merge_cuts[j] cuts are merged afterwards.  Windows are not cut.
+    if (split_keys < 0 || (split_keys % BN) || (split_keys > 0 && (window > 0 || !item_split || !part_acc || !part_ml ||
+                                                                    max_splits <= 0 || !merge_rows || !merge_cuts)))
+        return -8;
     if (page <= 0 || (page & (page - 1))) return -4;   // pages of a power of two only
     if (max_blocks > MAX_PAGES) return -5;             // the table row is staged in LDS
     const float scale_log2e = scale * 1.4426950408889634f;
 #if HEAD_DIM == 128 && PREFILL_DMA
-    {
+    if (true) {
         static bool prepared = false;
         if (!prepared) {
             if (hipFuncSetAttribute((const void*)attention_prefill_dma_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -567,13 +647,17 @@ int kipp_attention_prefill(const void* q, const void* k_cache, const void* v_cac
         }
         hipLaunchKernelGGL(attention_prefill_dma_kernel, dim3(n_items * n_q), dim3(THREADS), DMA_LDS_BYTES + max_blocks * 4,
                            stream, (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, item_seq,
-                           item_tile, q_start, q_len, positions, block_table, max_blocks, n_q, n_kv, page, scale_log2e, window);
-        return KIPP_LAUNCH_CHECK();
-    }
+                           item_tile, q_start, q_len, positions, block_table, max_blocks, n_q, n_kv, page, scale_log2e, window, tile_rows,
+                           item_split, split_keys, part_acc, part_ml, max_splits);
+    } else
 #endif
     hipLaunchKernelGGL(attention_prefill_kernel, dim3(n_items * n_q), dim3(THREADS), 0, stream, (const bf16_t*)q,
                        (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, item_seq, item_tile, q_start, q_len,
-                       positions, block_table, max_blocks, n_q, n_kv, page, scale_log2e, window);
+                       positions, block_table, max_blocks, n_q, n_kv, page, scale_log2e, window, tile_rows, item_split,
+                       split_keys, part_acc, part_ml, max_splits);
+    if (split_keys > 0 && n_merge > 0)
+        hipLaunchKernelGGL(attention_prefill_merge_kernel, dim3(n_q, n_merge), dim3(KIPP_WAVE), 0, stream, part_acc, part_ml,
+                           (bf16_t*)out, merge_rows, merge_cuts, n_q, max_splits);
     return KIPP_LAUNCH_CHECK();
 }
 

@@ -286,7 +286,9 @@ def attention_fast_ok(n_q: int, n_kv: int, page: int, max_blocks: int = 0) -> bo
 
 
 DECODE_SPLIT = 256      # keys per workgroup of the decode kernel (checked against the library at load)
-PREFILL_ROWS = 128      # query rows per workgroup of the prefill kernel
+PREFILL_ROWS = 128      # query rows per workgroup of the prefill kernel (64 or 32 where that fills the GPU better)
+COMPUTE_UNITS = 256     # of the MI355X
+PREFILL_MIN_CUT = 512   # fewest keys of a cut of the prefill kernel's keys (below, the merge costs more than the cut gains)
 
 
 def attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
@@ -406,22 +408,50 @@ def attention_decode_workspace(n_items: int, n_q: int, head_dim: int, max_contex
 def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
                       item_seq: torch.Tensor, item_tile: torch.Tensor, q_start: torch.Tensor, q_len: torch.Tensor,
                       positions: torch.Tensor, block_table: torch.Tensor, n_q: int, n_kv: int, head_dim: int,
-                      scale: float, window: int = 0) -> torch.Tensor:
+                      scale: float, window: int = 0, tile_rows: int = 128, cuts=None) -> torch.Tensor:
     """Attention of prompt portions: work item i is the `item_tile[i]`-th tile
-    of PREFILL_ROWS query rows of sequence `item_seq[i]`."""
+    of `tile_rows` (128, 64 or 32) query rows of sequence `item_seq[i]`.
+
+    `cuts` = (split_keys, item_split, merge_rows, merge_cuts, workspace): the keys are cut at multiples of
+    `split_keys` (a multiple of 64), work item i takes cut `item_split[i]` of its tile's keys, and the rows
+    `merge_rows[j]` (each with `merge_cuts[j]` cuts) are merged afterwards, in the order of the cuts.
+    `workspace` = (part_acc, part_ml) float32 from `attention_prefill_workspace`.  For few, long work items,
+    which alone would leave most compute units idle; not with a window."""
     _dev(q, k_cache, v_cache, out, item_seq, item_tile, q_start, q_len, positions, block_table)
+    _need(tile_rows in (32, 64, 128), "attention_prefill: tiles of 32, 64 or 128 query rows")
     for t, name in ((item_seq, "item_seq"), (item_tile, "item_tile"), (q_start, "q_start"), (q_len, "q_len"),
                     (positions, "positions"), (block_table, "block_table")):
         _i32(t, name)
     _attn_common(q, k_cache, v_cache, out, n_q, n_kv, head_dim, "attention_prefill")
     _need(item_seq.numel() == item_tile.numel(), "attention_prefill: one tile index per work item")
     _need(block_table.shape[1] <= PREFILL_MAX_BLOCKS, "attention_prefill: more pages per sequence than the kernel stages")
+    split_keys, item_split, merge_rows, merge_cuts, part_acc, part_ml, max_splits = 0, None, None, None, None, None, 0
+    if cuts is not None:
+        split_keys, item_split, merge_rows, merge_cuts, (part_acc, part_ml) = cuts
+        _dev(item_split, merge_rows, merge_cuts, part_acc, part_ml)
+        for t, name in ((item_split, "item_split"), (merge_rows, "merge_rows"), (merge_cuts, "merge_cuts")):
+            _i32(t, name)
+        rows = q.shape[0]
+        max_splits = part_ml.numel() // max(1, rows * n_q * 2)
+        _need(window == 0 and split_keys > 0 and split_keys % 64 == 0 and item_split.numel() == item_seq.numel()
+              and merge_rows.numel() == merge_cuts.numel() and part_acc.dtype == torch.float32 and part_ml.dtype == torch.float32
+              and max_splits >= 1 and part_acc.numel() >= rows * n_q * max_splits * head_dim,
+              "attention_prefill: cuts need no window, a multiple of 64 keys, one cut per work item and a workspace for every row")
     fn = _fn("attention_prefill", "kipp_attention_prefill",
-             [_c_ptr] * 10 + [_c_int] * 6 + [_c_float, _c_int, _c_ptr], {"HEAD_DIM": head_dim})
+             [_c_ptr] * 10 + [_c_int] * 6 + [_c_float, _c_int, _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int,
+                                             _c_ptr], {"HEAD_DIM": head_dim})
     _check(fn(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(item_seq), _ptr(item_tile), _ptr(q_start),
               _ptr(q_len), _ptr(positions), _ptr(block_table), block_table.shape[1], item_seq.numel(), n_q, n_kv,
-              head_dim, k_cache.shape[2], float(scale), int(window), _stream()), "attention_prefill")
+              head_dim, k_cache.shape[2], float(scale), int(window), int(tile_rows), _ptr(item_split), int(split_keys),
+              _ptr(part_acc), _ptr(part_ml), int(max_splits), _ptr(merge_rows), _ptr(merge_cuts),
+              merge_rows.numel() if merge_rows is not None else 0, _stream()), "attention_prefill")
     return out
+
+
+def attention_prefill_workspace(rows: int, n_q: int, head_dim: int, max_splits: int, device) -> tuple:
+    """(part_acc, part_ml) for `attention_prefill(..., cuts=...)`: sums and (maximum, denominator) of every cut."""
+    return (torch.empty(rows * n_q * max_splits * head_dim, dtype=torch.float32, device=device),
+            torch.empty(rows * n_q * max_splits * 2, dtype=torch.float32, device=device))
 
 
 # --------------------------------------------------------------------------- matrix products

@@ -129,10 +129,10 @@ class Attention:
         out = rt.empty((n, s.q_dim), rt.act_dtype)
         if fast:
             if batch.n_portions:
-                item_seq, item_tile = self._prefill_work(batch)
+                item_seq, item_tile, cuts = self._prefill_work(batch)
                 rt.ops.attention_prefill(q, cache.k, cache.v, out, item_seq, item_tile, batch.q_start,
                                          batch.q_len, batch.positions, table, s.num_heads, s.num_kv_heads, s.head_dim,
-                                         self.scale, s.window or 0)
+                                         self.scale, s.window or 0, cuts=cuts)
             if batch.n_decode:
                 rt.ops.attention_decode(q, cache.k, cache.v, out, batch.decode_rows, batch.positions, batch.seq_of_token,
                                         table, s.num_heads, s.num_kv_heads, s.head_dim, self.scale, s.window or 0,
@@ -144,22 +144,51 @@ class Attention:
         return rt.linear(out, self.w_o, slabs=True, defer=True)
 
     def _prefill_work(self, batch):
-        """The work list of the prefill kernel: (entry, tile of its kernel's query rows) for every
-        entry that brings a portion, the longest key range first (the kernel folds the list so that
-        workgroups sharing a compute unit carry about the same load).  Made by the first attention
-        layer of a forward pass and shared by the others of the same tile size."""
-        tile = self.rt.ops.PREFILL_ROWS
-        key = ("attention_prefill_work", tile)
+        """The work list of the prefill kernel: (entry, tile of 128 query rows) for every entry that brings a
+        portion, the longest key range first (the kernel folds the list so that workgroups sharing a
+        compute unit carry about the same load).
+
+        A workgroup walks all keys its tile sees, one after the other.  Where the tiles times the heads are
+        fewer workgroups than two a compute unit and the contexts are long (a portion of a few hundred rows
+        behind thousands of keys), the keys are cut as well, at multiples of a length chosen so that the
+        GPU is filled about twice: a work item is then (entry, tile, cut), and the cuts of a row are merged
+        in order afterwards.  The cuts follow from the step's shape, not from a row's place in it, so a row's
+        result may differ in its last bits between steps of different shapes, as between the kernels for
+        portions and for single tokens.  Made by the first attention layer of a forward pass and shared by
+        the others of the same geometry."""
+        s, ops = self.spec, self.rt.ops
+        key = ("attention_prefill_work", s.num_heads, s.head_dim, s.window)
         work = batch.step_cache.get(key)
         if work is None:
-            items = []
-            for i, (n, ctx) in enumerate(zip(batch.host["q_len"], batch.host["ctx_len"])):
-                if n > 1:
-                    start = ctx - n
-                    for t in range((n + tile - 1) // tile):
-                        items.append((-(start + min((t + 1) * tile, n)), i, t))    # keys the tile's last row sees
-            items.sort()
-            work = batch.upload([i for _, i, _ in items], [t for _, _, t in items])
+            tile = ops.PREFILL_ROWS
+            q_start = batch.host["q_start"]
+            portions = [(i, n, ctx) for i, (n, ctx) in enumerate(zip(batch.host["q_len"], batch.host["ctx_len"])) if n > 1]
+            tiles = [(i, t, ctx - n + min((t + 1) * tile, n) - 1, q_start[i] + t * tile, min(tile, n - t * tile))
+                     for i, n, ctx in portions for t in range((n + tile - 1) // tile)]     # (entry, tile, last key, first row, rows)
+            workgroups = len(tiles) * s.num_heads
+            longest = max(last for _, _, last, _, _ in tiles) + 1
+            split_keys = 0
+            if s.window is None and workgroups < 2 * ops.COMPUTE_UNITS:
+                want = -(-2 * ops.COMPUTE_UNITS // workgroups)
+                split_keys = max(ops.PREFILL_MIN_CUT, -(-longest // want // 64) * 64)
+                if longest <= split_keys:
+                    split_keys = 0
+            if not split_keys:
+                items = sorted((-last, i, t) for i, t, last, _, _ in tiles)
+                work = tuple(batch.upload([i for _, i, _ in items], [t for _, _, t in items])) + (None,)
+            else:
+                items, merge_rows, merge_cuts = [], [], []
+                for i, t, last, row0, rows in tiles:
+                    cuts = last // split_keys + 1
+                    items.extend((-(min(last + 1, (c + 1) * split_keys) - c * split_keys), i, t, c) for c in range(cuts))
+                    merge_rows.extend(range(row0, row0 + rows))
+                    merge_cuts.extend([cuts] * rows)
+                items.sort()
+                most = max(merge_cuts)
+                seq, til, cut, rows_d, cuts_d = batch.upload([i for _, i, _, _ in items], [t for _, _, t, _ in items],
+                                                             [c for _, _, _, c in items], merge_rows, merge_cuts)
+                space = ops.attention_prefill_workspace(batch.n_tokens, s.num_heads, s.head_dim, most, self.rt.device)
+                work = (seq, til, (split_keys, cut, rows_d, cuts_d, space))
             batch.step_cache[key] = work
         return work
 

@@ -536,7 +536,10 @@ def _from_the_projection(ops, n_q, n_kv, d, page, window, norm, slabs, write_kv)
 @pytest.mark.parametrize("n_q,n_kv,d,page", [(32, 8, 128, 16), (6, 2, 48, 8), (4, 4, 64, 4), (3, 1, 80, 16), (2, 1, 256, 32), (2, 2, 16, 8),
                                              (4, 2, 128, 4), (5, 1, 128, 64)])
 @pytest.mark.parametrize("window", [0, 100])
-def test_attention_prefill(n_q, n_kv, d, page, window):
+@pytest.mark.parametrize("tile_rows", [128, 64, 32])
+def test_attention_prefill(n_q, n_kv, d, page, window, tile_rows):
+    """Tiles of 128 query rows, and of 64 and 32 (what the mixer asks for where tiles of 128 would leave
+    compute units idle): the same result whichever way a portion is cut into work items."""
     ops = _ops()
     rng = np.random.default_rng(n_q * 11 + d + window)
     seq_lens = [130, 64, 300, 5, 257]      # tokens in the cache after this step
@@ -548,16 +551,63 @@ def test_attention_prefill(n_q, n_kv, d, page, window):
         positions += list(range(n - ql, n))
         seq_of += [s] * ql
     t = len(positions)
-    items = [(s, tile) for s, ql in enumerate(q_lens) for tile in range(-(-ql // ops.PREFILL_ROWS))]
+    items = [(s, tile) for s, ql in enumerate(q_lens) for tile in range(-(-ql // tile_rows))]
     q = torch.tensor(rng.normal(size=(t, n_q * d)), dtype=torch.bfloat16)
     out = ops.attention_prefill(q.to(DEV), k.to(DEV), v.to(DEV), torch.zeros(t, n_q * d, dtype=torch.bfloat16, device=DEV),
                                 _t([i[0] for i in items], torch.int32), _t([i[1] for i in items], torch.int32),
                                 _t(q_start, torch.int32), _t(q_lens, torch.int32), _t(positions, torch.int32),
-                                _t(table, torch.int32), n_q, n_kv, d, 1 / math.sqrt(d), window)
+                                _t(table, torch.int32), n_q, n_kv, d, 1 / math.sqrt(d), window, tile_rows=tile_rows)
     ref = _attention_reference(q, k, v, table, positions, seq_of, n_q, n_kv, d, page, window)
     got = out.float().cpu().numpy().reshape(t, n_q, d)
     for i in range(t):
         assert _rel(got[i], ref[i]) < 2e-5, f"row {i}: position {positions[i]} of sequence {seq_of[i]}"
+
+
+@pytest.mark.parametrize("n_q,n_kv,d,page", [(8, 2, 128, 16), (6, 2, 48, 8), (3, 1, 80, 16), (2, 2, 16, 8)])
+@pytest.mark.parametrize("split_keys", [64, 192, 512])
+def test_attention_prefill_with_the_keys_cut(n_q, n_kv, d, page, split_keys):
+    """The keys of a work item cut at multiples of `split_keys`, the cuts merged afterwards: portions that begin
+    at position 0 and deep in a sequence, a tile whose rows lie on both sides of a cut's edge (rows before the
+    edge have nothing in the cut behind it), a row count that is no multiple of the tile."""
+    ops = _ops()
+    rng = np.random.default_rng(n_q * 7 + d + split_keys)
+    seq_lens = [700, 130, 330, 64]
+    q_lens = [150, 130, 2, 5]
+    table, k, v = _paged_setup(rng, seq_lens, n_kv, d, page, torch.bfloat16)
+    positions, seq_of, q_start = [], [], []
+    for s, (n, ql) in enumerate(zip(seq_lens, q_lens)):
+        q_start.append(len(positions))
+        positions += list(range(n - ql, n))
+        seq_of += [s] * ql
+    t = len(positions)
+    items, merge_rows, merge_cuts = [], [], []
+    for s, (n, ql) in enumerate(zip(seq_lens, q_lens)):
+        for tile in range(-(-ql // 128)):
+            rows = min(128, ql - tile * 128)
+            last = n - ql + tile * 128 + rows - 1
+            cuts = last // split_keys + 1
+            items += [(s, tile, c) for c in range(cuts)]
+            merge_rows += list(range(q_start[s] + tile * 128, q_start[s] + tile * 128 + rows))
+            merge_cuts += [cuts] * rows
+    rng.shuffle(items)                                           # any order of the work items
+    space = ops.attention_prefill_workspace(t, n_q, d, max(merge_cuts), DEV)
+    space[0].fill_(float("nan"))                                 # whatever the workspace held before is never read
+    space[1].fill_(float("nan"))
+    q = torch.tensor(rng.normal(size=(t, n_q * d)), dtype=torch.bfloat16)
+    cuts = (split_keys, _t([i[2] for i in items], torch.int32), _t(merge_rows, torch.int32), _t(merge_cuts, torch.int32), space)
+    out = ops.attention_prefill(q.to(DEV), k.to(DEV), v.to(DEV), torch.zeros(t, n_q * d, dtype=torch.bfloat16, device=DEV),
+                                _t([i[0] for i in items], torch.int32), _t([i[1] for i in items], torch.int32),
+                                _t(q_start, torch.int32), _t(q_lens, torch.int32), _t(positions, torch.int32),
+                                _t(table, torch.int32), n_q, n_kv, d, 1 / math.sqrt(d), 0, cuts=cuts)
+    ref = _attention_reference(q, k, v, table, positions, seq_of, n_q, n_kv, d, page, 0)
+    got = out.float().cpu().numpy().reshape(t, n_q, d)
+    for i in range(t):
+        assert _rel(got[i], ref[i]) < 2e-5, f"row {i}: position {positions[i]} of sequence {seq_of[i]}"
+    with pytest.raises(Exception):                               # a window is not cut
+        ops.attention_prefill(q.to(DEV), k.to(DEV), v.to(DEV), torch.zeros(t, n_q * d, dtype=torch.bfloat16, device=DEV),
+                              _t([i[0] for i in items], torch.int32), _t([i[1] for i in items], torch.int32),
+                              _t(q_start, torch.int32), _t(q_lens, torch.int32), _t(positions, torch.int32),
+                              _t(table, torch.int32), n_q, n_kv, d, 1 / math.sqrt(d), 100, cuts=cuts)
 
 
 @pytest.mark.parametrize("rise", [3.0, 40.0, 400.0, -40.0])

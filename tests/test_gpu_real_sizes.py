@@ -270,3 +270,32 @@ def test_prompt_portions_of_many_rows_by_either_product(real_folder, real_refere
         out = engine.step([StepEntry("b", toks[:300], list(range(300)))])
         H.assert_close(out.float().cpu().numpy(), ref[:300], H.NMSE_BF16["real"], "many rows, timed choice")
         assert len(auto.prompt_product_choices) >= 4       # QKV, output, gate-up, down: each decided
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_portions_behind_a_long_context_cut_their_keys(long_folder, dtype):
+    """A portion of a few hundred rows behind a thousand keys and more is few, long work items for the prefill
+    attention: under bfloat16 their keys are cut over more workgroups and merged (the first portion, from an
+    empty context, is not cut).  Every row of every portion against the plain implementation."""
+    from kipp_amd.engine import Engine, StepEntry
+    cfg, weights = plain.load_folder(long_folder)
+    toks = H.random_tokens(41, 1500, 311)
+    ref = plain.forward_whole(cfg, weights, toks)
+    engine = Engine.from_folder(long_folder, dtype=dtype, page_size=16, max_tokens=1536, max_requests=2, share_prefixes=False)
+    seen = []
+    mixer = engine.model.blocks[0].mixer
+    inner = mixer._prefill_work
+
+    def watching(batch):
+        work = inner(batch)
+        seen.append(work[2] is not None)
+        return work
+    mixer._prefill_work = watching
+    got, at = [], 0
+    for n in (700, 300, 130, 370):
+        got.append(engine.step([StepEntry("long", toks[at:at + n], list(range(n)))]).float().cpu().numpy())
+        at += n
+    tol = H.NMSE_F32 if dtype == "float32" else H.NMSE_BF16["real"]
+    H.assert_close(np.concatenate(got), ref, tol, f"portions behind a long context/{dtype}")
+    if dtype == "bfloat16":
+        assert seen == [True, True, True, True]      # 700 keys already exceed a cut of 512; every portion was cut
