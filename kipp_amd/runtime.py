@@ -174,6 +174,11 @@ class Runtime:
         return ScaledRows(rows_out, sumsq, (w.shape[0] + 15) // 16, eps)
 
     # -- products of prompt portions ------------------------------------------------------------
+    @staticmethod
+    def _rows_class(m: int) -> int:
+        """Rows of a prompt product, in classes of a factor of two (257-512, 513-1024, ...): one decision a class."""
+        return 1 << (max(m, 1) - 1).bit_length()
+
     def _ours_is_faster(self, key, ours, library) -> bool:
         """Which of two ways to compute one product is taken for the shape `key`: decided once, by the
         switch or by timing both on the operands at hand (three runs each after a first one)."""
@@ -221,7 +226,7 @@ class Runtime:
 
         def library():
             return self.ops.swiglu(self._library_product(x, rows), act)
-        if self.ops.gemm_tiles_ok(m, k) and self._ours_is_faster(("gated", -(-m // 128), rows.shape[0], k), ours, library):
+        if self.ops.gemm_tiles_ok(m, k) and self._ours_is_faster(("gated", self._rows_class(m), rows.shape[0], k), ours, library):
             self.tile_products += 1
             return ours()
         self.library_products += 1
@@ -273,7 +278,7 @@ class Runtime:
 
             def library():
                 return self._library_product(x, w)
-            if self._ours_is_faster(("linear", -(-m // 128), n, x.shape[1], most), ours, library):
+            if self._ours_is_faster(("linear", self._rows_class(m), n, x.shape[1], most), ours, library):
                 self.tile_products += 1
                 return ours()
         self.library_products += 1
