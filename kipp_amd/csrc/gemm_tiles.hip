@@ -33,7 +33,6 @@
 #include "common.h"
 
 #define BK 32                                      // columns of a step
-#define STAGES 4
 #define THREADS 256
 #define CHUNKS (BK / 8)                            // 16-byte chunks of a row of a piece
 #define GROUP_ROWS (16 / CHUNKS)                   // rows that share 256 bytes of LDS
@@ -78,10 +77,19 @@ __device__ __forceinline__ void wait_reads(u32x4 (&fa)[WM], u32x4 (&fb)[WN]) {
         asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(fa[0]), "+v"(fa[1]), "+v"(fb[0]), "+v"(fb[1]));
 }
 
+// steps of K that are in LDS or on their way there.  (Three for the smaller tiles, so that three workgroups of
+// the smallest share a compute unit instead of two, was measured and is slower: those tiles are bound by what
+// the DMA brings, not by the matrix cores, and a step less on its way is what they then lack.)
+template <int WM, int WN>
+struct Depth {
+    static constexpr int value = 4;
+};
+
 template <int WM, int WN, int END>
 __global__ void __launch_bounds__(THREADS, 1) gemm_tiles_kernel(
     const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* __restrict__ Y, int M, int N, int K,
     int tiles_m, int tiles_n, int parts, int inner, int col_begin, int col_end) {
+    constexpr int STAGES = Depth<WM, WN>::value;
     constexpr int TM = 64 * WM, TN = 64 * WN;                     // the workgroup's tile
     constexpr int X_PIECE = TM * BK * 2, W_PIECE = TN * BK * 2;   // bytes of a step's pieces
     constexpr int STAGE_BYTES = X_PIECE + W_PIECE;
@@ -368,7 +376,7 @@ static int plan(int M, int N, int K, int end, int max_parts, Cut* cuts) {
 
 template <int WM, int WN, int END>
 static int launch_cut(const void* X, const void* W, void* Y, int M, int N, int K, const Cut& cut, hipStream_t stream) {
-    constexpr int lds_bytes = STAGES * 64 * (WM + WN) * BK * 2;
+    constexpr int lds_bytes = Depth<WM, WN>::value * 64 * (WM + WN) * BK * 2;
     static bool prepared = false;
     if (!prepared) {
         if (hipFuncSetAttribute((const void*)gemm_tiles_kernel<WM, WN, END>, hipFuncAttributeMaxDynamicSharedMemorySize,

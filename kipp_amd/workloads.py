@@ -5,11 +5,16 @@ portions, and requests that share a long beginning (paged prefix reuse).
     python -m kipp_amd.workloads continuous    [--shape qwen3-8b]  [--requests 32] ...
     python -m kipp_amd.workloads shared-prefix [--shape qwen3-32b] [--requests 8]  ...
     python -m kipp_amd.workloads hbm           [--gib 4]
+    python -m kipp_amd.workloads products      [--shape qwen3-4b] [--rows 2048,512]
+    python -m kipp_amd.workloads portion       [--shape qwen3-4b] [--rows 512] [--behind 4096]
 
 One JSON line: generated tokens a second over the whole run, prompt tokens a
 second, time to the first token, and what the cache reused.  `hbm` is no
 workload but the yardstick for the decode kernels: how fast a kernel that only
 reads gets a large buffer out of memory (best of several grids and ring depths).
+`products` times the four matrix products of a layer for prompt portions, our
+kernel beside the library's; `portion` times a prompt portion behind a context
+that is already in the cache (what a step of chunked prefill costs).
 """
 from __future__ import annotations
 
@@ -107,9 +112,96 @@ def hbm_read(gib: float) -> dict:
     return {"workload": "hbm read", "GiB": gib, "compute_units": cus, "best": best, "all": table}
 
 
+def _time(fn, runs: int = 20) -> float:
+    """Microseconds a call, over `runs` calls after three that are not timed."""
+    import torch
+    for _ in range(3):
+        fn()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(runs):
+        fn()
+    end.record()
+    end.synchronize()
+    return start.elapsed_time(end) / runs * 1e3
+
+
+def products(shape: str, rows_list) -> dict:
+    """The matrix products of one layer at `rows` rows: our kernel for prompt portions (SwiGLU in its end for
+    gate/up, K in slabs for the others) beside the library's product (float32 result, SwiGLU a kernel of its own)."""
+    import torch
+    from .config import parse_config, shape_config
+    from .csrc import ops
+    _, cfg = parse_config(shape_config(shape))
+    h, q, kv, inner = cfg.hidden_size, cfg.q_dim, cfg.kv_dim, cfg.intermediate_size
+    sizes = {"qkv": (q + 2 * kv, h, "slabs"), "o": (h, q, "slabs"), "gate_up": (2 * inner, h, "swiglu"), "down": (h, inner, "slabs")}
+    out = {"workload": "products", "shape": shape, "rows": {}}
+    for rows in rows_list:
+        table = {}
+        for name, (n, k, end) in sizes.items():
+            x = torch.randn(rows, k, device="cuda:0", dtype=torch.bfloat16)
+            w = torch.randn(n, k, device="cuda:0", dtype=torch.bfloat16) * 0.02
+            act = torch.empty(rows, n // 2, device="cuda:0", dtype=torch.bfloat16)
+            ours = _time(lambda: ops.gemm_tiles(x, w, end, max_parts=4))
+            if end == "swiglu":
+                library = _time(lambda: ops.swiglu(torch.mm(x, w.t(), out_dtype=torch.float32), act))
+            else:
+                library = _time(lambda: torch.mm(x, w.t(), out_dtype=torch.float32))
+            flops = 2.0 * rows * n * k
+            table[name] = {"ours_us": round(ours, 1), "library_us": round(library, 1), "ours_PFLOPs": round(flops / ours / 1e9, 3),
+                           "library_PFLOPs": round(flops / library / 1e9, 3)}
+            log(f"{rows} rows {name:8s} ours {ours:7.1f} us ({flops / ours / 1e9:.2f} PFLOP/s)   library {library:7.1f} us "
+                f"({flops / library / 1e9:.2f} PFLOP/s)")
+        out["rows"][str(rows)] = table
+    return out
+
+
+def portion(shape: str, layers, rows: int, behind: int, runs: int = 6) -> dict:
+    """A prompt portion of `rows` tokens behind `behind` tokens that are in the cache already: milliseconds a step."""
+    import torch
+    from .engine import StepEntry
+    engine, config, full = build_engine(shape, layers, behind + (runs + 3) * rows + 64, behind + (runs + 3) * rows + 64, 2)
+    gen = torch.Generator().manual_seed(1)
+
+    def feed(n):
+        engine.step([StepEntry("a", torch.randint(0, config["vocab_size"], (n,), generator=gen).tolist(), [])])
+    at = 0
+    while at < behind:
+        n = min(2048, behind - at)
+        feed(n)
+        at += n
+    for _ in range(2):
+        feed(rows)
+    torch.cuda.synchronize()
+    start = time.perf_counter()
+    for _ in range(runs):
+        feed(rows)
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - start) / runs * 1e3
+    log(f"{rows} tokens behind {behind} to {behind + (runs + 2) * rows}: {ms:.2f} ms a step, {rows / ms * 1e3:.0f} tok/s")
+    return {"workload": "portion", "shape": shape, "layers": config["num_hidden_layers"], "rows": rows, "behind": behind,
+            "ms_per_step": round(ms, 3), "tokens_per_s": round(rows / ms * 1e3, 1),
+            "product_choices": {str(k): ("ours" if v else "library") for k, v in engine.rt.prompt_product_choices.items()}}
+
+
 def main(argv=None) -> int:
     if argv is None:
         argv = sys.argv[1:]
+    if argv and argv[0] in ("products", "portion"):
+        ap = argparse.ArgumentParser(prog=f"python -m kipp_amd.workloads {argv[0]}")
+        ap.add_argument("--shape", default="qwen3-4b")
+        ap.add_argument("--layers", type=int, default=0)
+        ap.add_argument("--rows", default="2048,512" if argv[0] == "products" else "512")
+        ap.add_argument("--behind", type=int, default=4096)
+        args = ap.parse_args(argv[1:])
+        import torch
+        if not torch.cuda.is_available():
+            print("workload: no GPU", file=sys.stderr)
+            return 1
+        rows = [int(r) for r in args.rows.split(",") if r]
+        result = products(args.shape, rows) if argv[0] == "products" else portion(args.shape, args.layers, rows[0], args.behind)
+        print(json.dumps(result), flush=True)
+        return 0
     if argv and argv[0] == "hbm":
         ap = argparse.ArgumentParser(prog="python -m kipp_amd.workloads hbm")
         ap.add_argument("--gib", type=float, default=4.0, help="size of the buffer that is read")
