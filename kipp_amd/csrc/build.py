@@ -91,7 +91,9 @@ def _start(name: str, defines: Optional[dict]):
         return out, None, None
     tmp = f"{out}.{os.getpid()}.tmp"
     cmd = [_hipcc()] + FLAGS + dflags + ["-I", HERE, src, "-o", tmp]
-    proc = subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    # what the compiler prints goes to a file: through a pipe that nobody reads before the compiler
+    # ends, a long list of warnings would fill the pipe and the compiler would wait for ever
+    proc = subprocess.Popen(cmd, stdout=open(tmp + ".log", "w"), stderr=subprocess.STDOUT)
     return out, tmp, proc
 
 
@@ -100,7 +102,14 @@ def _say(msg: str) -> None:
 
 
 def _finish(name, out, tmp, proc, started) -> None:
-    log = proc.communicate()[0]
+    proc.wait()
+    log = ""
+    try:
+        with open(tmp + ".log", "r", errors="replace") as f:
+            log = f.read()
+        os.remove(tmp + ".log")
+    except OSError:
+        pass
     if proc.returncode != 0 or not os.path.exists(tmp):
         try:
             os.remove(tmp)

@@ -80,13 +80,23 @@ __device__ __forceinline__ void wait_reads(u32x4 (&fa)[WM], u32x4 (&fb)[WN]) {
 // steps of K that are in LDS or on their way there.  (Three for the smaller tiles, so that three workgroups of
 // the smallest share a compute unit instead of two, was measured and is slower: those tiles are bound by what
 // the DMA brings, not by the matrix cores, and a step less on its way is what they then lack.)
+#ifndef SMALL_DEPTH
+#define SMALL_DEPTH 4
+#endif
+#ifndef SMALL_WGS
+#define SMALL_WGS 1
+#endif
 template <int WM, int WN>
 struct Depth {
-    static constexpr int value = 4;
+    static constexpr int value = WM * WN <= 8 ? SMALL_DEPTH : 4;
 };
 
+#ifdef PROBE_CLOCK
+__device__ long long clock_probe[2048][4];
+#endif
+
 template <int WM, int WN, int END>
-__global__ void __launch_bounds__(THREADS, 1) gemm_tiles_kernel(
+__global__ void __launch_bounds__(THREADS, (WM * WN <= 8 ? SMALL_WGS : 1)) gemm_tiles_kernel(
     const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* __restrict__ Y, int M, int N, int K,
     int tiles_m, int tiles_n, int parts, int inner, int col_begin, int col_end) {
     constexpr int STAGES = Depth<WM, WN>::value;
@@ -127,12 +137,16 @@ __global__ void __launch_bounds__(THREADS, 1) gemm_tiles_kernel(
     const int q4 = lane >> 4, s16 = lane & 15;
     const int in_group = s16 ^ (q4 & (CHUNKS - 1));
     const int lane_row = GROUP_ROWS * q4 + in_group / CHUNKS, col8 = (in_group % CHUNKS) * 8;
-    const unsigned char* x_src[WM];
-    const unsigned char* w_src[WN];
+    // an address is a base that all lanes share (it walks along K in scalar registers) plus a lane's own 32-bit
+    // offset, which never changes: no vector arithmetic for an address inside the walk (the launcher refuses
+    // operands of 4 GiB and more)
+    uint32_t x_src[WM], w_src[WN];
+    const unsigned char* x_base = (const unsigned char*)(X + (size_t)s_begin * BK);
+    const unsigned char* w_base = (const unsigned char*)(W + (size_t)s_begin * BK);
 #pragma unroll
     for (int i = 0; i < WM; ++i) {
         const int r = (TM / 4) * wave + INSTR_ROWS * i + lane_row;
-        x_src[i] = (const unsigned char*)(X + (size_t)min(tm * TM + r, M - 1) * K + (size_t)s_begin * BK + col8);
+        x_src[i] = (uint32_t)(((size_t)min(tm * TM + r, M - 1) * K + col8) * 2);
     }
 #pragma unroll
     for (int i = 0; i < WN; ++i) {
@@ -146,19 +160,32 @@ __global__ void __launch_bounds__(THREADS, 1) gemm_tiles_kernel(
         } else {
             wr = min(col_begin + tn * TN + r, col_end - 1);
         }
-        w_src[i] = (const unsigned char*)(W + (size_t)wr * K + (size_t)s_begin * BK + col8);
+        w_src[i] = (uint32_t)(((size_t)wr * K + col8) * 2);
     }
-    auto issue_one = [&](int step, int stage, int n) {          // DMA instruction n (0 .. LOADS - 1) of a step
-#ifdef ABLATE_DMA
+    // where step `step` of an operand begins, for every lane: pinned to scalar registers (left to itself the
+    // compiler adds the lane's offset first and then walks a 64-bit vector address along K)
+    auto step_base = [&](const unsigned char* base, int step) {
+#if defined(ABLATE_DMA) && ABLATE_DMA == 2
+        step = 0;                                                // measurements only: every step brings the first again
+#endif
+        const unsigned char* at = base + (size_t)step * (BK * 2);
+        asm volatile("" : "+s"(at));
+        return at;
+    };
+    auto issue_one = [&](const unsigned char* x_at, const unsigned char* w_at, int stage, int n) {   // DMA instruction n (0 .. LOADS - 1) of a step
+#if defined(ABLATE_DMA) && ABLATE_DMA == 1
         return;
 #endif
+        // the lane's offset passes through an empty asm here, so that its widening to 64 bits stands beside the
+        // load: the compiler then takes the form "scalar base + 32-bit vector offset" and adds nothing per load
+        // (widened once outside the walk, the offset would cost a 64-bit vector add for every load)
         unsigned char* dst = lds + stage * STAGE_BYTES;
-        const size_t at = (size_t)step * (BK * 2);
+        uint32_t off = n < WM ? x_src[n < WM ? n : 0] : w_src[n < WM ? 0 : n - WM];
+        asm volatile("" : "+v"(off));
         if (n < WM)
-            __builtin_amdgcn_global_load_lds(GLOBAL_PTR(x_src[n < WM ? n : 0] + at), LDS_PTR(dst + wave * (X_PIECE / 4) + 1024 * n), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds(GLOBAL_PTR(x_at + off), LDS_PTR(dst + wave * (X_PIECE / 4) + 1024 * n), 16, 0, 0);
         else
-            __builtin_amdgcn_global_load_lds(GLOBAL_PTR(w_src[n < WM ? 0 : n - WM] + at),
-                                             LDS_PTR(dst + X_PIECE + wave * (W_PIECE / 4) + 1024 * (n - WM)), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds(GLOBAL_PTR(w_at + off), LDS_PTR(dst + X_PIECE + wave * (W_PIECE / 4) + 1024 * (n - WM)), 16, 0, 0);
     };
 
     // ---- a lane's place in the operands: row 32 j + l32 of the wave's rows, chunk 2 t + hh of the step
@@ -206,46 +233,98 @@ __global__ void __launch_bounds__(THREADS, 1) gemm_tiles_kernel(
             __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa.v, fb.v, acc[(M_) / WN][(M_) % WN], 0, 0, 0); \
     } while (0)
 
+    // The DMA instructions of a step go out in two groups, half a step apart: the first LOADS_EARLY of step
+    // kt + STAGES behind the products of the second half of step kt (into the buffer of step kt, which every wave
+    // has left at the barrier in the middle of step kt), the others behind the products of the first half of
+    // step kt + 1.  So a wave asks for 1 KB every third product and not every product for half of the time:
+    // the four waves' requests together then stay under what the compute unit's path to memory takes, and no
+    // wave waits to hand one in (measured: 20 cycles an instruction when they all came behind one another).
+    constexpr int LOADS_EARLY = (LOADS + 1) / 2, LOADS_LATE = LOADS - LOADS_EARLY;
+    // the items of a half step: NR reads of operands, one behind each of the first products, then D DMA
+    // instructions spread over the products that are left (all spread evenly where there are more items than products)
+#define KIPP_ITEMS(D, M_, READ, DMA)                                                          \
+    do {                                                                                      \
+        constexpr int T_ = NR + (D);                                                          \
+        _Pragma("unroll") for (int p_ = 0; p_ < T_; ++p_) {                                   \
+            const int behind_ = T_ > NM ? p_ * NM / T_ : (p_ < NR ? p_ : NR + (p_ - NR) * (NM - NR) / (D)); \
+            if (behind_ != (M_)) continue;                                                    \
+            if (p_ >= NR) { DMA(p_ - NR); }                                                   \
+            else { READ(p_); }                                                                \
+        }                                                                                     \
+    } while (0)
+
 #pragma unroll
-    for (int s = 0; s < STAGES; ++s)
+    for (int s = 0; s < STAGES; ++s) {
+        const unsigned char* x_at = step_base(x_base, min(s, nk - 1));
+        const unsigned char* w_at = step_base(w_base, min(s, nk - 1));
 #pragma unroll
-        for (int n = 0; n < LOADS; ++n) issue_one(min(s, nk - 1), s, n);
-    // the loads of steps 1 .. STAGES - 1 may still be on their way
-    __builtin_amdgcn_s_waitcnt(0x0F70 | (((STAGES - 1) * LOADS) & 15) | ((((STAGES - 1) * LOADS) >> 4) << 14));
-    __syncthreads();
+        for (int n = 0; n < (s == STAGES - 1 ? LOADS_EARLY : LOADS); ++n) issue_one(x_at, w_at, s, n);
+    }
+    // step 0 has arrived when steps 1 .. STAGES - 2 and the early part of step STAGES - 1 may still be on their way
+    constexpr int AFTER_FIRST = (STAGES - 2) * LOADS + LOADS_EARLY;
+    static_assert(AFTER_FIRST < 64, "the wait counts must fit the counter");
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (AFTER_FIRST & 15) | ((AFTER_FIRST >> 4) << 14));
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();                                  // bare, as in the walk below
+    asm volatile("" ::: "memory");
 #pragma unroll
     for (int r = 0; r < NR; ++r) KIPP_READ_ONE(0, 0, 0, r);
+#ifdef PROBE_CLOCK
+    const long long c0 = __builtin_readcyclecounter(), r0 = __builtin_amdgcn_s_memrealtime();
+#endif
     for (int kt = 0; kt < nk; ++kt) {
-        // first half: products of columns 0 .. 15 of the step; the operands of the second half arrive meanwhile
+        // first half: products of columns 0 .. 15 of the step; the operands of the second half arrive meanwhile,
+        // and the late DMA instructions of step kt + STAGES - 1 go out, into the buffer of step kt - 1
         // (the scheduler may not carry instructions over the marks: the order written here is the order meant)
         wait_reads<WM, WN>(a[0], b[0]);
         __builtin_amdgcn_sched_barrier(0);
+        const int late = min(kt + STAGES - 1, nk - 1), late_stage = (kt + STAGES - 1) % STAGES;
+        const unsigned char* x_late = step_base(x_base, late);
+        const unsigned char* w_late = step_base(w_base, late);
+#define KIPP_READ_A(R) KIPP_READ_ONE(1, kt, 1, R)
+#define KIPP_DMA_A(N_) issue_one(x_late, w_late, late_stage, LOADS_EARLY + (N_))
 #pragma unroll
         for (int m = 0; m < NM; ++m) {
             KIPP_PRODUCT(0, m);
-#pragma unroll
-            for (int r = m * NR / NM; r < (m + 1) * NR / NM; ++r) KIPP_READ_ONE(1, kt, 1, r);
+            KIPP_ITEMS(LOADS_LATE, m, KIPP_READ_A, KIPP_DMA_A);
             __builtin_amdgcn_sched_barrier(0);
         }
-        // second half: every wave's part of the next step has arrived, and every wave is done with this step's
-        // buffer (its operands are in registers), which the step STAGES ahead is now asked into
+        // second half: every wave's part of the next step has arrived (what may still be on its way: the steps
+        // behind it), and every wave is done with this step's buffer (its operands are in registers), into which
+        // the early DMA instructions of step kt + STAGES now go
         wait_reads<WM, WN>(a[1], b[1]);
         __builtin_amdgcn_s_waitcnt(0x0F70 | (((STAGES - 2) * LOADS) & 15) | ((((STAGES - 2) * LOADS) >> 4) << 14));
-        __syncthreads();
+        // the bare barrier: __syncthreads() also fences, and the fence waits for EVERY load into LDS that is on
+        // its way (the compiler writes vmcnt(0) for it), which would leave nothing in flight across a step
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
         __builtin_amdgcn_sched_barrier(0);
         const int ahead = min(kt + STAGES, nk - 1);
+        const unsigned char* x_ahead = step_base(x_base, ahead);
+        const unsigned char* w_ahead = step_base(w_base, ahead);
+#define KIPP_READ_B(R) KIPP_READ_ONE(0, kt + 1, 0, R)
+#define KIPP_DMA_B(N_) issue_one(x_ahead, w_ahead, kt % STAGES, N_)
 #pragma unroll
         for (int m = 0; m < NM; ++m) {
             KIPP_PRODUCT(1, m);
-            // NR reads of the next step's first operands, then the LOADS DMA instructions, spread over the products
-#pragma unroll
-            for (int x = m * (NR + LOADS) / NM; x < (m + 1) * (NR + LOADS) / NM; ++x) {
-                if (x < NR) KIPP_READ_ONE(0, kt + 1, 0, x);
-                else issue_one(ahead, kt % STAGES, x - NR);
-            }
+            KIPP_ITEMS(LOADS_EARLY, m, KIPP_READ_B, KIPP_DMA_B);
             __builtin_amdgcn_sched_barrier(0);
         }
     }
+#undef KIPP_READ_A
+#undef KIPP_DMA_A
+#undef KIPP_READ_B
+#undef KIPP_DMA_B
+#undef KIPP_ITEMS
+#ifdef PROBE_CLOCK
+    if (tid == 0 && blockIdx.x < 2048 && blockIdx.z == 0) {
+        clock_probe[blockIdx.x][0] = __builtin_readcyclecounter() - c0;
+        clock_probe[blockIdx.x][1] = __builtin_amdgcn_s_memrealtime() - r0;
+        clock_probe[blockIdx.x][2] = nk;
+        clock_probe[blockIdx.x][3] = r0;
+    }
+#endif
     wait_reads<WM, WN>(a[0], b[0]);
     __builtin_amdgcn_s_waitcnt(0x0F70);      // nothing may still be on its way into LDS when the buffers are used again
 #undef KIPP_READ_ONE
@@ -407,6 +486,11 @@ static int launch_end(const void* X, const void* W, void* Y, int M, int N, int K
 }
 
 extern "C" {
+#ifdef PROBE_CLOCK
+int kipp_gemm_tiles_clock(long long* out, int n) {
+    return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(clock_probe), (size_t)n * 4 * sizeof(long long));
+}
+#endif
 
 // parts that kipp_gemm_tiles cuts K into for these sizes when it may use up to `max_parts` (1 for the ends that are not slabs)
 int kipp_gemm_tiles_parts(int M, int N, int K, int end, int max_parts) {
@@ -425,6 +509,8 @@ int kipp_gemm_tiles(const void* X, const void* W, void* Y, int M, int N, int K, 
     if (K <= 0 || (K % BK) || max_parts <= 0) return -1;
     if (end != END_SLABS && end != END_SWIGLU && end != END_BF16) return -3;
     if (end == END_SWIGLU && (N & 1)) return -4;
+    // a lane's offset into an operand is 32 bits wide
+    if ((unsigned long long)M * K * 2 >= (1ull << 32) || (unsigned long long)N * K * 2 >= (1ull << 32)) return -6;
     Cut cuts[2];
     int n_cuts = plan(M, N, K, end, max_parts, cuts);
     if (force) {

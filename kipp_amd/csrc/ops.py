@@ -643,9 +643,10 @@ def gemm_skinny_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tens
 TILES_END = {"slabs": 0, "swiglu": 1, "bf16": 2}
 
 
-def gemm_tiles_ok(m: int, k: int) -> bool:
-    """Shapes the product for prompt portions takes: K a multiple of 32 (any number of rows; it is built for hundreds)."""
-    return m > 0 and k > 0 and k % 32 == 0
+def gemm_tiles_ok(m: int, k: int, n: int = 1) -> bool:
+    """Shapes the product for prompt portions takes: K a multiple of 32 (any number of rows; it is built for
+    hundreds), each operand under 4 GiB (a lane's offset into it is 32 bits wide)."""
+    return m > 0 and k > 0 and k % 32 == 0 and max(m, n) * k * 2 < 2**32
 
 
 def gemm_tiles(x: torch.Tensor, w: torch.Tensor, end: str = "slabs", max_parts: int = 1, force: int = 0) -> torch.Tensor:
@@ -701,6 +702,22 @@ def stream_read(buffer: torch.Tensor, workgroups: int, depth: int = 8) -> int:
     sink = torch.zeros(1, dtype=torch.int32, device=buffer.device)
     got = fn(_ptr(buffer), buffer.numel() * buffer.element_size(), int(workgroups), int(depth), _ptr(sink), _stream())
     _need(got > 0, "stream_read: buffer too small for this grid")
+    return int(got)
+
+
+def mfma_rate(data: torch.Tensor, workgroups: int, accumulators: int, iters: int) -> int:
+    """Launches the probe that only multiplies (32x32x16 bfloat16 products from registers, `accumulators` = 8 or 16
+    independent sums a wave, `workgroups` of 4 waves); `data`: 16 KiB whose bits are the operands.  Returns the
+    floating-point operations launched."""
+    _dev(data)
+    _need(data.is_contiguous() and data.numel() * data.element_size() == 16384 and accumulators in (8, 16),
+          "mfma_rate: 16 KiB of operand bits, 8 or 16 accumulators")
+    fn = build.library("probe").kipp_probe_mfma_rate
+    fn.restype = ctypes.c_longlong
+    fn.argtypes = [_c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_ptr]
+    sink = torch.zeros(1, dtype=torch.int32, device=data.device)
+    got = fn(_ptr(data), int(workgroups), int(accumulators), int(iters), _ptr(sink), _stream())
+    _need(got > 0, "mfma_rate: refused")
     return int(got)
 
 

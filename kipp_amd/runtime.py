@@ -107,10 +107,11 @@ class Runtime:
         self.library_products = 0   # calls that went to the library (they stay out of HIP graphs)
         self.generic_attention_launches = 0   # bfloat16 attention that fell to the generic kernel (geometry the matrix-core kernels refuse)
         self.fuse_norms = True      # few rows: residual add and norm ride on the products around them
-        # products of more than 256 rows: our own matrix-core kernel or the library's, whichever is faster for the
-        # shape ("auto": both are timed once, at the shape's first use); True / False: always ours / always the library's
+        # products of more than 256 rows: our own matrix-core kernel (as planned, or in one of a few other cuts) or
+        # the library's, whichever is fastest for the shape ("auto": all are timed once, at the shape's first use);
+        # True / False: always ours as planned / always the library's
         self.own_prompt_products = "auto"
-        self.prompt_product_choices = {}     # shape -> True (ours) / False (the library's)
+        self.prompt_product_choices = {}     # shape -> "library", "plan" (our kernel, cut as planned) or a forced cut of ours
         self.tile_products = 0      # products of more than 256 rows that ran on our own kernel
         torch.backends.cuda.matmul.allow_tf32 = False
 
@@ -179,25 +180,36 @@ class Runtime:
         """Rows of a prompt product, in classes of a factor of two (257-512, 513-1024, ...): one decision a class."""
         return 1 << (max(m, 1) - 1).bit_length()
 
-    def _ours_is_faster(self, key, ours, library) -> bool:
-        """Which of two ways to compute one product is taken for the shape `key`: decided once, by the
-        switch or by timing both on the operands at hand (three runs each after a first one)."""
+    # cuts of our kernel that are timed beside the planned one: 100 x (wave tile rows / 32) + 10 x (wave tile
+    # columns / 32) + parts of K.  The plan's cost model is linear; the GPU under its power limit is not (a
+    # round that leaves compute units idle clocks the others higher), so the plan is not always the fastest.
+    TILE_CUTS_SLABS = (441, 442, 444, 431, 432, 421, 422)
+    TILE_CUTS_BF16 = (441, 421, 241)
+
+    def _fastest(self, key, ways: dict):
+        """Which of several ways to compute one product is taken for the shape `key`: decided once, by the
+        switch (True: our planned cut, False: the library's) or by timing all of them on the operands at hand
+        (three runs each after a first one).  `ways`: name -> callable, "library" and "plan" among them."""
         choice = self.prompt_product_choices.get(key)
         if choice is None:
             if self.own_prompt_products != "auto":
-                choice = bool(self.own_prompt_products)
+                choice = "plan" if self.own_prompt_products else "library"
             else:
-                times = []
-                for run in (ours, library):
-                    run()
+                best = None
+                for name, run in ways.items():
+                    try:
+                        run()
+                    except self.ops.KernelError:
+                        continue                      # a cut this shape does not take
                     begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                     begin.record()
                     for _ in range(3):
                         run()
                     end.record()
                     end.synchronize()
-                    times.append(begin.elapsed_time(end))
-                choice = times[0] <= times[1]
+                    ms = begin.elapsed_time(end)
+                    if best is None or ms < best:
+                        best, choice = ms, name
             self.prompt_product_choices[key] = choice
         return choice
 
@@ -221,14 +233,18 @@ class Runtime:
         m, k = x.shape
         rows = w.rows
 
-        def ours():
-            return self.ops.gemm_tiles(x, rows, end="swiglu")
+        def ours(force=0):
+            return self.ops.gemm_tiles(x, rows, end="swiglu", force=force)
 
         def library():
             return self.ops.swiglu(self._library_product(x, rows), act)
-        if self.ops.gemm_tiles_ok(m, k) and self._ours_is_faster(("gated", self._rows_class(m), rows.shape[0], k), ours, library):
-            self.tile_products += 1
-            return ours()
+        if self.ops.gemm_tiles_ok(m, k, rows.shape[0]):
+            ways = {"library": library, "plan": ours}
+            ways.update({cut: (lambda cut=cut: ours(cut)) for cut in self.TILE_CUTS_BF16})
+            choice = self._fastest(("gated", self._rows_class(m), rows.shape[0], k), ways)
+            if choice != "library":
+                self.tile_products += 1
+                return ours(0 if choice == "plan" else choice)
         self.library_products += 1
         return library()
 
@@ -269,17 +285,20 @@ class Runtime:
                 y = self.ops.gemm_rows(x, w, max_parts=1 if most == 0 else (most or 12), tiles=tiles)
             return y if y.shape[0] > 1 else y[0]
         # more than 256 rows (prompt portions): our matrix-core kernel, or the library's product
-        if self.ops.gemm_tiles_ok(m, x.shape[1]):
+        if self.ops.gemm_tiles_ok(m, x.shape[1], n):
             most = 1 if slabs is False else (4 if slabs is True else max(1, min(4, int(slabs))))
 
-            def ours():
-                y = self.ops.gemm_tiles(x, w, end="slabs", max_parts=most)
+            def ours(force=0):
+                y = self.ops.gemm_tiles(x, w, end="slabs", max_parts=most, force=force)
                 return y if y.shape[0] > 1 else y[0]
 
             def library():
                 return self._library_product(x, w)
-            if self._ours_is_faster(("linear", self._rows_class(m), n, x.shape[1], most), ours, library):
+            ways = {"library": library, "plan": ours}
+            ways.update({cut: (lambda cut=cut: ours(cut)) for cut in self.TILE_CUTS_SLABS if cut % 10 <= most})
+            choice = self._fastest(("linear", self._rows_class(m), n, x.shape[1], most), ways)
+            if choice != "library":
                 self.tile_products += 1
-                return ours()
+                return ours(0 if choice == "plan" else choice)
         self.library_products += 1
         return self._library_product(x, w)

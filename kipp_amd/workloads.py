@@ -5,6 +5,7 @@ portions, and requests that share a long beginning (paged prefix reuse).
     python -m kipp_amd.workloads continuous    [--shape qwen3-8b]  [--requests 32] ...
     python -m kipp_amd.workloads shared-prefix [--shape qwen3-32b] [--requests 8]  ...
     python -m kipp_amd.workloads hbm           [--gib 4]
+    python -m kipp_amd.workloads mfma
     python -m kipp_amd.workloads products      [--shape qwen3-4b] [--rows 2048,512]
     python -m kipp_amd.workloads portion       [--shape qwen3-4b] [--rows 512] [--behind 4096]
 
@@ -12,6 +13,8 @@ One JSON line: generated tokens a second over the whole run, prompt tokens a
 second, time to the first token, and what the cache reused.  `hbm` is no
 workload but the yardstick for the decode kernels: how fast a kernel that only
 reads gets a large buffer out of memory (best of several grids and ring depths).
+`mfma` is the yardstick for the prompt products: what the matrix cores sustain on
+operands that never leave the registers.
 `products` times the four matrix products of a layer for prompt portions, our
 kernel beside the library's; `portion` times a prompt portion behind a context
 that is already in the cache (what a step of chunked prefill costs).
@@ -112,6 +115,35 @@ def hbm_read(gib: float) -> dict:
     return {"workload": "hbm read", "GiB": gib, "compute_units": cus, "best": best, "all": table}
 
 
+def mfma_rate() -> dict:
+    """What the matrix cores sustain on operands that stay in registers: by the operands' bits (zeros, values
+    of a normal distribution), the compute units at work, waves a SIMD and the kernel's length."""
+    import torch
+    from .csrc import ops
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    gen = torch.Generator().manual_seed(0)
+    operands = {"zeros": torch.zeros(8192, dtype=torch.bfloat16),
+                "normal": torch.randn(8192, generator=gen).to(torch.bfloat16)}
+    table = []
+    for name, host in operands.items():
+        data = host.to("cuda:0")
+        for groups, acc, what in ((cus, 16, "1 wave a SIMD"), (2 * cus, 8, "2 waves a SIMD"), (80, 16, "80 compute units")):
+            for iters in (400, 4000, 40000):
+                start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                ops.mfma_rate(data, groups, acc, iters)
+                best = 0.0
+                for _ in range(3):
+                    start.record()
+                    flops = ops.mfma_rate(data, groups, acc, iters)
+                    end.record()
+                    torch.cuda.synchronize()
+                    ms = start.elapsed_time(end)
+                    best = max(best, flops / (ms * 1e-3) / 1e15)
+                table.append({"operands": name, "grid": what, "ms": round(ms, 3), "PFLOP_s": round(best, 3)})
+                log(f"{name:6s} {what:17s} kernel of {ms:8.3f} ms: {best:5.3f} PFLOP/s")
+    return {"workload": "mfma rate", "compute_units": cus, "all": table}
+
+
 def _time(fn, runs: int = 20) -> float:
     """Microseconds a call, over `runs` calls after three that are not timed."""
     import torch
@@ -128,10 +160,12 @@ def _time(fn, runs: int = 20) -> float:
 
 def products(shape: str, rows_list) -> dict:
     """The matrix products of one layer at `rows` rows: our kernel for prompt portions (SwiGLU in its end for
-    gate/up, K in slabs for the others) beside the library's product (float32 result, SwiGLU a kernel of its own)."""
+    gate/up, K in slabs for the others), cut as planned and in the best of the cuts the runtime times, beside the
+    library's product (float32 result, SwiGLU a kernel of its own)."""
     import torch
     from .config import parse_config, shape_config
     from .csrc import ops
+    from .runtime import Runtime
     _, cfg = parse_config(shape_config(shape))
     h, q, kv, inner = cfg.hidden_size, cfg.q_dim, cfg.kv_dim, cfg.intermediate_size
     sizes = {"qkv": (q + 2 * kv, h, "slabs"), "o": (h, q, "slabs"), "gate_up": (2 * inner, h, "swiglu"), "down": (h, inner, "slabs")}
@@ -143,15 +177,24 @@ def products(shape: str, rows_list) -> dict:
             w = torch.randn(n, k, device="cuda:0", dtype=torch.bfloat16) * 0.02
             act = torch.empty(rows, n // 2, device="cuda:0", dtype=torch.bfloat16)
             ours = _time(lambda: ops.gemm_tiles(x, w, end, max_parts=4))
+            best_cut, best = "plan", ours
+            for cut in (Runtime.TILE_CUTS_SLABS if end == "slabs" else Runtime.TILE_CUTS_BF16):
+                try:
+                    took = _time(lambda: ops.gemm_tiles(x, w, end, max_parts=4, force=cut))
+                except ops.KernelError:
+                    continue
+                if took < best:
+                    best_cut, best = str(cut), took
             if end == "swiglu":
                 library = _time(lambda: ops.swiglu(torch.mm(x, w.t(), out_dtype=torch.float32), act))
             else:
                 library = _time(lambda: torch.mm(x, w.t(), out_dtype=torch.float32))
             flops = 2.0 * rows * n * k
-            table[name] = {"ours_us": round(ours, 1), "library_us": round(library, 1), "ours_PFLOPs": round(flops / ours / 1e9, 3),
+            table[name] = {"ours_us": round(ours, 1), "ours_best_cut": best_cut, "ours_best_us": round(best, 1),
+                           "library_us": round(library, 1), "ours_PFLOPs": round(flops / best / 1e9, 3),
                            "library_PFLOPs": round(flops / library / 1e9, 3)}
-            log(f"{rows} rows {name:8s} ours {ours:7.1f} us ({flops / ours / 1e9:.2f} PFLOP/s)   library {library:7.1f} us "
-                f"({flops / library / 1e9:.2f} PFLOP/s)")
+            log(f"{rows} rows {name:8s} ours as planned {ours:7.1f} us, best cut {best_cut} {best:7.1f} us ({flops / best / 1e9:.2f} PFLOP/s)   "
+                f"library {library:7.1f} us ({flops / library / 1e9:.2f} PFLOP/s)")
         out["rows"][str(rows)] = table
     return out
 
@@ -181,7 +224,7 @@ def portion(shape: str, layers, rows: int, behind: int, runs: int = 6) -> dict:
     log(f"{rows} tokens behind {behind} to {behind + (runs + 2) * rows}: {ms:.2f} ms a step, {rows / ms * 1e3:.0f} tok/s")
     return {"workload": "portion", "shape": shape, "layers": config["num_hidden_layers"], "rows": rows, "behind": behind,
             "ms_per_step": round(ms, 3), "tokens_per_s": round(rows / ms * 1e3, 1),
-            "product_choices": {str(k): ("ours" if v else "library") for k, v in engine.rt.prompt_product_choices.items()}}
+            "product_choices": {str(k): str(v) for k, v in engine.rt.prompt_product_choices.items()}}
 
 
 def main(argv=None) -> int:
@@ -201,6 +244,13 @@ def main(argv=None) -> int:
         rows = [int(r) for r in args.rows.split(",") if r]
         result = products(args.shape, rows) if argv[0] == "products" else portion(args.shape, args.layers, rows[0], args.behind)
         print(json.dumps(result), flush=True)
+        return 0
+    if argv and argv[0] == "mfma":
+        import torch
+        if not torch.cuda.is_available():
+            print("workload: no GPU", file=sys.stderr)
+            return 1
+        print(json.dumps(mfma_rate()), flush=True)
         return 0
     if argv and argv[0] == "hbm":
         ap = argparse.ArgumentParser(prog="python -m kipp_amd.workloads hbm")

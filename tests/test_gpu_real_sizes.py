@@ -248,8 +248,8 @@ def test_a_long_position_limit_keeps_the_matrix_core_kernels(real_folder, real_r
 def test_prompt_portions_of_many_rows_by_either_product(real_folder, real_reference, ours):
     """Portions of more than 256 rows at the benchmark's layer sizes, with every product of theirs forced to our
     matrix-core kernel (SwiGLU in its end, K split into slabs that the norms add), then to the library's:
-    against the plain implementation, every row; left alone the engine times both once a shape and takes the
-    faster, and says which."""
+    against the plain implementation, every row; left alone the engine times the library's product and a few
+    cuts of ours once a shape, takes the fastest, and says which."""
     from kipp_amd.engine import Engine, StepEntry
     from kipp_amd.engine.model import load_model
     from kipp_amd.runtime import Runtime
@@ -263,7 +263,7 @@ def test_prompt_portions_of_many_rows_by_either_product(real_folder, real_refere
            engine.step([StepEntry("a", toks[300:], list(range(320)))])]
     H.assert_close(torch.cat(got).float().cpu().numpy(), ref, H.NMSE_BF16["real"], f"many rows, ours {ours}")
     assert (rt.tile_products > 0 and rt.library_products == 0) if ours else (rt.tile_products == 0 and rt.library_products > 0)
-    assert set(rt.prompt_product_choices.values()) == {ours}
+    assert set(rt.prompt_product_choices.values()) == {"plan" if ours else "library"}
     if ours:
         auto = Runtime("bfloat16")
         engine = Engine(load_model(real_folder, auto), page_size=16, max_tokens=1024, max_requests=2, share_prefixes=False)
