@@ -6,6 +6,7 @@ portions, and requests that share a long beginning (paged prefix reuse).
     python -m kipp_amd.workloads shared-prefix [--shape qwen3-32b] [--requests 8]  ...
     python -m kipp_amd.workloads hbm           [--gib 4]
     python -m kipp_amd.workloads mfma
+    python -m kipp_amd.workloads walk          [--ablate-dma 1|2] [--ablate-reads]
     python -m kipp_amd.workloads products      [--shape qwen3-4b] [--rows 2048,512]
     python -m kipp_amd.workloads portion       [--shape qwen3-4b] [--rows 512] [--behind 4096]
 
@@ -14,7 +15,8 @@ second, time to the first token, and what the cache reused.  `hbm` is no
 workload but the yardstick for the decode kernels: how fast a kernel that only
 reads gets a large buffer out of memory (best of several grids and ring depths).
 `mfma` is the yardstick for the prompt products: what the matrix cores sustain on
-operands that never leave the registers.
+operands that never leave the registers; `walk` counts the shader cycles a product
+takes inside our prompt-product kernel (a build with clock counters; it compiles at its first call).
 `products` times the four matrix products of a layer for prompt portions, our
 kernel beside the library's; `portion` times a prompt portion behind a context
 that is already in the cache (what a step of chunked prefill costs).
@@ -144,6 +146,49 @@ def mfma_rate() -> dict:
     return {"workload": "mfma rate", "compute_units": cus, "all": table}
 
 
+def walk(ablate_dma: int, ablate_reads: bool, n: int = 8192, k: int = 9728, rows: int = 2048) -> dict:
+    """Shader cycles a product (v_mfma_f32_32x32x16_bf16, 32 cycles of the matrix core) inside the walk over K
+    of the prompt-product kernel, from a build that reads the shader clock and the 100 MHz clock around the
+    walk; optionally with the DMA taken out (1) or made to bring the first step every time (2: it always hits
+    the cache), and with the reads out of LDS taken out.  The ablated builds compute nothing meaningful."""
+    import ctypes
+    import numpy as np
+    import torch
+    from .csrc import build
+    defines = {"PROBE_CLOCK": 1}
+    if ablate_dma:
+        defines["ABLATE_DMA"] = int(ablate_dma)
+    if ablate_reads:
+        defines["ABLATE_READS"] = 1
+    lib = build.library("gemm_tiles", defines)
+    ptr, i32 = ctypes.c_void_p, ctypes.c_int
+    lib.kipp_gemm_tiles.argtypes = [ptr, ptr, ptr, i32, i32, i32, i32, i32, i32, ptr]
+    lib.kipp_gemm_tiles_clock.argtypes = [ptr, i32]
+    x = torch.randn(rows, k, device="cuda:0").bfloat16()
+    w = (torch.randn(n, k, device="cuda:0") * 0.02).bfloat16()
+    out = torch.zeros(rows * n, device="cuda:0", dtype=torch.float32)
+    table = []
+    for launches in (1, 20):
+        for _ in range(launches):
+            rc = lib.kipp_gemm_tiles(x.data_ptr(), w.data_ptr(), out.data_ptr(), rows, n, k, 0, 1, 441, torch.cuda.current_stream().cuda_stream)
+            if rc != 0:
+                raise RuntimeError(f"gemm_tiles refused (code {rc})")
+        torch.cuda.synchronize()
+        groups = min(2048, -(-rows // 256) * -(-n // 256))
+        buf = np.zeros((2048, 4), dtype=np.int64)
+        if lib.kipp_gemm_tiles_clock(buf.ctypes.data, 2048) != 0:
+            raise RuntimeError("the probe's counters could not be read")
+        b = buf[:groups].astype(float)
+        products = b[:, 2] * 32                      # a wave's products in the walk: 32 a step
+        row = {"after_launches": launches, "cycles_per_product": round(float(np.median(b[:, 0] / products)), 2),
+               "ns_per_product": round(float(np.median(b[:, 1] * 10 / products)), 2),
+               "GHz": round(float(np.median(b[:, 0] / (b[:, 1] * 10))), 3)}
+        table.append(row)
+        log(f"{rows} x {n} x {k}, after {launches} launch(es): {row['cycles_per_product']} shader cycles a product, "
+            f"{row['ns_per_product']} ns, clock {row['GHz']} GHz")
+    return {"workload": "walk", "ablate_dma": ablate_dma, "ablate_reads": bool(ablate_reads), "all": table}
+
+
 def _time(fn, runs: int = 20) -> float:
     """Microseconds a call, over `runs` calls after three that are not timed."""
     import torch
@@ -244,6 +289,17 @@ def main(argv=None) -> int:
         rows = [int(r) for r in args.rows.split(",") if r]
         result = products(args.shape, rows) if argv[0] == "products" else portion(args.shape, args.layers, rows[0], args.behind)
         print(json.dumps(result), flush=True)
+        return 0
+    if argv and argv[0] == "walk":
+        ap = argparse.ArgumentParser(prog="python -m kipp_amd.workloads walk")
+        ap.add_argument("--ablate-dma", type=int, default=0, choices=[0, 1, 2])
+        ap.add_argument("--ablate-reads", action="store_true")
+        args = ap.parse_args(argv[1:])
+        import torch
+        if not torch.cuda.is_available():
+            print("workload: no GPU", file=sys.stderr)
+            return 1
+        print(json.dumps(walk(args.ablate_dma, args.ablate_reads)), flush=True)
         return 0
     if argv and argv[0] == "mfma":
         import torch
