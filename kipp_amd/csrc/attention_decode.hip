@@ -41,14 +41,13 @@
 #error "compile with -DGROUP=<query heads per key/value head>"
 #endif
 
-#define SPLIT 256
+#define SPLIT 256                              // keys of a split (the kernel that takes one a workgroup also has longer ones)
+#define SPLIT_MAX 384
 #define WAVES 4
 #define THREADS (WAVES * KIPP_WAVE)
 #define KSTEPS ((HEAD_DIM + 31) / 32)          // MFMA steps of 32 over the head size
 #define CHUNKS (HEAD_DIM / 8)                  // 16-byte chunks of a row
 #define CHUNKS_PER_LANE ((CHUNKS + 15) / 16)
-#define BLOCKS_PER_WAVE (SPLIT / 16 / WAVES)   // 16-key blocks a wave scores
-#define KEYS_PER_GROUP (SPLIT / 16)            // keys a lane group multiplies with values
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
@@ -78,39 +77,47 @@ struct Projected {
     int write_kv;            // 0: the cache is another layer's, keys and values are already there
 };
 
-template <bool FUSED>
+template <bool FUSED, int SPLIT_T>
 __global__ void __launch_bounds__(THREADS) attention_decode_kernel(
     const bf16_t* __restrict__ q, bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache,
     bf16_t* __restrict__ out, float* __restrict__ part_acc, float* __restrict__ part_ml,
     const int32_t* __restrict__ rows, const int32_t* __restrict__ positions, const int32_t* __restrict__ seq_of_token,
     const int32_t* __restrict__ block_table, int max_blocks, int n_q, int n_kv, int page, float scale_log2e,
     int window, int max_splits, Projected pj) {
-    __shared__ float s_scores[GROUP][SPLIT + 4];
+    static_assert(SPLIT_T % (16 * WAVES) == 0 && SPLIT_T <= 2 * THREADS, "whole blocks of 16 keys a wave; at most two pages a thread");
+    constexpr int BPW = SPLIT_T / 16 / WAVES;         // 16-key blocks a wave scores
+    constexpr int KPG = SPLIT_T / 16;                 // keys a lane group multiplies with values
+    __shared__ float s_scores[GROUP][SPLIT_T + 4];
     __shared__ __attribute__((aligned(16))) bf16_t s_new[FUSED ? GROUP + 2 : 1][HEAD_DIM];
     __shared__ float s_red[WAVES][GROUP][HEAD_DIM];
     __shared__ float s_m[GROUP], s_l[GROUP];
-    __shared__ int s_page[SPLIT + 2];                 // page of every key of the split (any page size)
+    __shared__ int s_page[SPLIT_T + 2];                 // page of every key of the split (any page size)
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l16 = lane & 15, h = lane >> 4;
     const int kvh = blockIdx.y;
-    const int row = rows[blockIdx.z];                 // row of this query token in the batch
+    // The grid is (query tokens, key/value heads, splits): workgroups are handed out in that order, so those of
+    // splits beyond a sequence's position, which the grid has for the longest context it was recorded for,
+    // come last and leave at once instead of holding a place that a working one waits for.
+    const int row = rows[blockIdx.x];                 // row of this query token in the batch
     const int pos = positions[row];
     const int lo = window > 0 ? max(0, pos - window + 1) : 0;
-    const int first_split = lo / SPLIT, last_split = pos / SPLIT;
-    const int split = first_split + blockIdx.x;
+    const int first_split = lo / SPLIT_T, last_split = pos / SPLIT_T;
+    const int split = first_split + blockIdx.z;
     if (split > last_split) return;                   // the grid covers the longest sequence
     const int n_splits = last_split - first_split + 1;
-    const int base = split * SPLIT;
+    const int base = split * SPLIT_T;
     const int32_t* table = block_table + (size_t)seq_of_token[row] * max_blocks;
 
     // Pages first, once, into LDS: the loads of keys and values below then depend on
     // nothing that is still in flight and can all be issued back to back.  Keys beyond
     // the query's position read the last valid page (finite values, masked later).
     const int page_shift = __builtin_ctz(page);          // the page size is a power of two (checked by the launcher)
-    int my_page = 0;
-    if (tid < SPLIT) my_page = table[min(base + tid, pos) >> page_shift];
+    int my_page[2] = {0, 0};
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+        if (tid + THREADS * i < SPLIT_T) my_page[i] = table[min(base + tid + THREADS * i, pos) >> page_shift];
 
     // ---- fused: ask for the projected heads this wave prepares, and for what their norm and
     // rotation need, before the keys and values are asked for: they are wanted first
@@ -162,7 +169,9 @@ __global__ void __launch_bounds__(THREADS) attention_decode_kernel(
         }
     }
 #endif
-    if (tid < SPLIT) s_page[tid] = my_page;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+        if (tid + THREADS * i < SPLIT_T) s_page[tid + THREADS * i] = my_page[i];
     __syncthreads();
 
     // ---- the GROUP queries as B operand: lane (slot l16, quarter h) holds q[slot][32 t + 8 h .. + 7]
@@ -175,21 +184,21 @@ __global__ void __launch_bounds__(THREADS) attention_decode_kernel(
         }
     }
 
-    // ---- scores: each wave takes BLOCKS_PER_WAVE blocks of 16 keys; every load is unconditional
-    Frag kf[BLOCKS_PER_WAVE][KSTEPS];
+    // ---- scores: each wave takes BPW blocks of 16 keys; every load is unconditional
+    Frag kf[BPW][KSTEPS];
 #pragma unroll
-    for (int b = 0; b < BLOCKS_PER_WAVE; ++b) {
-        const int kl = (wave * BLOCKS_PER_WAVE + b) * 16 + l16;
+    for (int b = 0; b < BPW; ++b) {
+        const int kl = (wave * BPW + b) * 16 + l16;
         const int s = min(base + kl, pos);
         const bf16_t* k_row = k_cache + (((size_t)s_page[kl] * n_kv + kvh) * page + (s & (page - 1))) * HEAD_DIM;
 #pragma unroll
         for (int t = 0; t < KSTEPS; ++t) kf[b][t].u = *(const u32x4*)(k_row + min(32 * t + 8 * h, HEAD_DIM - 8));
     }
     // ---- values are asked for now, so that they arrive while the scores are worked on
-    Frag vf[KEYS_PER_GROUP][CHUNKS_PER_LANE];
+    Frag vf[KPG][CHUNKS_PER_LANE];
     const int kg = wave * 4 + h;                      // this lane group's keys: base + kg + 16 i
 #pragma unroll
-    for (int i = 0; i < KEYS_PER_GROUP; ++i) {
+    for (int i = 0; i < KPG; ++i) {
         const int kl = kg + 16 * i;
         const int s = min(base + kl, pos);
         const bf16_t* v_row = v_cache + (((size_t)s_page[kl] * n_kv + kvh) * page + (s & (page - 1))) * HEAD_DIM;
@@ -247,14 +256,14 @@ __global__ void __launch_bounds__(THREADS) attention_decode_kernel(
             qf[t].u = *(const u32x4*)(&s_new[min(l16, GROUP - 1)][min(32 * t + 8 * h, HEAD_DIM - 8)]);
         if (owner) {                                  // the token's own key and value come from LDS, not from the cache
 #pragma unroll
-            for (int b = 0; b < BLOCKS_PER_WAVE; ++b)
-                if ((wave * BLOCKS_PER_WAVE + b) * 16 + l16 == own_slot) {
+            for (int b = 0; b < BPW; ++b)
+                if ((wave * BPW + b) * 16 + l16 == own_slot) {
 #pragma unroll
                     for (int t = 0; t < KSTEPS; ++t)
                         kf[b][t].u = *(const u32x4*)(&s_new[GROUP][min(32 * t + 8 * h, HEAD_DIM - 8)]);
                 }
 #pragma unroll
-            for (int i = 0; i < KEYS_PER_GROUP; ++i)
+            for (int i = 0; i < KPG; ++i)
                 if (kg + 16 * i == own_slot) {
 #pragma unroll
                     for (int c = 0; c < CHUNKS_PER_LANE; ++c)
@@ -268,7 +277,7 @@ __global__ void __launch_bounds__(THREADS) attention_decode_kernel(
     for (int t = 0; t < KSTEPS; ++t)
         if (32 * t + 8 * h >= HEAD_DIM || l16 >= GROUP) qf[t].u = (u32x4){0u, 0u, 0u, 0u};
 #pragma unroll
-    for (int b = 0; b < BLOCKS_PER_WAVE; ++b) {
+    for (int b = 0; b < BPW; ++b) {
         f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (int t = 0; t < KSTEPS; ++t) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[b][t].v, qf[t].v, acc, 0, 0, 0);
@@ -276,7 +285,7 @@ __global__ void __launch_bounds__(THREADS) attention_decode_kernel(
         if (l16 < GROUP) {
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
-                const int kl = (wave * BLOCKS_PER_WAVE + b) * 16 + 4 * h + v;
+                const int kl = (wave * BPW + b) * 16 + 4 * h + v;
                 const int s = base + kl;
                 s_scores[l16][kl] = (s >= lo && s <= pos) ? acc[v] * scale_log2e : -INFINITY;
             }
@@ -286,17 +295,17 @@ __global__ void __launch_bounds__(THREADS) attention_decode_kernel(
 
     // ---- softmax over the split's keys, one head per wave at a time
     for (int g = wave; g < GROUP; g += WAVES) {
-        float sc[SPLIT / KIPP_WAVE];
+        float sc[SPLIT_T / KIPP_WAVE];
         float m = -INFINITY;
 #pragma unroll
-        for (int i = 0; i < SPLIT / KIPP_WAVE; ++i) {
+        for (int i = 0; i < SPLIT_T / KIPP_WAVE; ++i) {
             sc[i] = s_scores[g][lane + KIPP_WAVE * i];
             m = fmaxf(m, sc[i]);
         }
         m = wave_max(m);
         float l = 0.0f;
 #pragma unroll
-        for (int i = 0; i < SPLIT / KIPP_WAVE; ++i) {
+        for (int i = 0; i < SPLIT_T / KIPP_WAVE; ++i) {
             const float p = exp2f(sc[i] - m);          // -inf gives 0
             s_scores[g][lane + KIPP_WAVE * i] = p;
             l += p;
@@ -318,7 +327,7 @@ __global__ void __launch_bounds__(THREADS) attention_decode_kernel(
 #pragma unroll
             for (int j = 0; j < 8; ++j) acc[g][c][j] = 0.0f;
 #pragma unroll
-    for (int i = 0; i < KEYS_PER_GROUP; ++i) {
+    for (int i = 0; i < KPG; ++i) {
         const int kl = kg + 16 * i;
         float p[GROUP];
 #pragma unroll
@@ -369,7 +378,7 @@ __global__ void __launch_bounds__(THREADS) attention_decode_kernel(
         if (n_splits == 1) {
             out[((size_t)row * n_q + head) * HEAD_DIM + dcol] = f32_to_bf16(a / s_l[g]);
         } else {
-            const size_t slot = ((size_t)blockIdx.z * n_q + head) * max_splits + blockIdx.x;
+            const size_t slot = ((size_t)blockIdx.x * n_q + head) * max_splits + blockIdx.z;
             part_acc[slot * HEAD_DIM + dcol] = a;
             if (dcol == 0) {
                 part_ml[slot * 2] = s_m[g];
@@ -1075,6 +1084,51 @@ static int launch_ring(const bf16_t* q, bf16_t* k_cache, bf16_t* v_cache, bf16_t
 }
 #endif
 
+// The kernel that takes one split a workgroup, with splits of 256 keys, or of 320 or 384 where splits of 256
+// would be more workgroups than two a compute unit and the longer ones are not: workgroups beyond those that
+// fit at once run as a second round behind the first (measured at 8 sequences of 8 key/value heads: 576
+// workgroups for 2,050 keys cost 0.15 ms a step more than 512 for 2,040).  A function of the launch's shape.
+static int split_keys_for(int n_items, int n_kv, int span_keys, int window, int longest) {
+    const long long pairs = (long long)n_items * n_kv, fit = 2 * 256;
+    const int extra = window > 0 ? 1 : 0;
+    if (pairs * ((span_keys + SPLIT - 1) / SPLIT + extra) <= fit) return SPLIT;
+    for (int keys = SPLIT + 64; keys <= longest; keys += 64)
+        if (pairs * ((span_keys + keys - 1) / keys + extra) <= fit) return keys;
+    return longest;                                   // more than fit at once either way: the fewest workgroups
+}
+
+template <bool FUSED>
+static int launch_split(const bf16_t* q, bf16_t* k_cache, bf16_t* v_cache, bf16_t* out, float* part_acc, float* part_ml,
+                        const int32_t* rows, const int32_t* positions, const int32_t* seq_of_token,
+                        const int32_t* block_table, int max_blocks, int n_items, int n_q, int n_kv, int page,
+                        float scale_log2e, int window, int grid_splits, int max_splits, Projected pj, hipStream_t stream) {
+    const int extra = window > 0 ? 1 : 0;
+    const int span_keys = (grid_splits - extra) * SPLIT;           // the caller counts splits of SPLIT keys
+    // the fused form holds the projected heads as well: with splits of 384 keys it needs more registers than two
+    // workgroups a compute unit leave it (272 of 256)
+    const int keys = split_keys_for(n_items, n_kv, span_keys, window, FUSED ? 320 : SPLIT_MAX);
+    const int splits = keys == SPLIT ? grid_splits : (span_keys + keys - 1) / keys + extra;
+#define KIPP_SPLIT_LAUNCH(KEYS)                                                                                       \
+    hipLaunchKernelGGL((attention_decode_kernel<FUSED, KEYS>), dim3(n_items, n_kv, splits), dim3(THREADS), 0, stream, q, \
+                       k_cache, v_cache, out, part_acc, part_ml, rows, positions, seq_of_token, block_table, max_blocks, \
+                       n_q, n_kv, page, scale_log2e, window, max_splits, pj)
+    switch (keys) {
+        case 256: KIPP_SPLIT_LAUNCH(256); break;
+        case 320: KIPP_SPLIT_LAUNCH(320); break;
+        case 384:
+            if constexpr (!FUSED) {
+                KIPP_SPLIT_LAUNCH(384);
+                break;
+            }
+            return -1;
+        default: return -1;
+    }
+#undef KIPP_SPLIT_LAUNCH
+    int rc = KIPP_LAUNCH_CHECK();
+    if (rc != 0 || splits == 1) return rc;
+    return launch_reduce(part_acc, part_ml, out, rows, positions, n_items, n_q, window, max_splits, keys, splits, stream);
+}
+
 extern "C" {
 
 int kipp_attention_decode_split() { return SPLIT; }
@@ -1123,13 +1177,9 @@ int kipp_attention_decode(const void* q, const void* k_cache, const void* v_cach
         if (rc != 0 || big_splits == 1) return rc;
         return launch_reduce(part_acc, part_ml, (bf16_t*)out, rows, positions, n_items, n_q, window, max_splits, BIG, big_splits, stream);
     }
-    hipLaunchKernelGGL(attention_decode_kernel<false>, dim3(grid_splits, n_kv, n_items), dim3(THREADS), 0, stream,
-                       (const bf16_t*)q, (bf16_t*)k_cache, (bf16_t*)v_cache, (bf16_t*)out, part_acc, part_ml,
-                       rows, positions, seq_of_token, block_table, max_blocks, n_q, n_kv, page, scale_log2e, window,
-                       max_splits, Projected{});
-    int rc = KIPP_LAUNCH_CHECK();
-    if (rc != 0 || grid_splits == 1) return rc;
-    return launch_reduce(part_acc, part_ml, (bf16_t*)out, rows, positions, n_items, n_q, window, max_splits, SPLIT, grid_splits, stream);
+    return launch_split<false>((const bf16_t*)q, (bf16_t*)k_cache, (bf16_t*)v_cache, (bf16_t*)out, part_acc, part_ml, rows, positions,
+                               seq_of_token, block_table, max_blocks, n_items, n_q, n_kv, page, scale_log2e, window, grid_splits,
+                               max_splits, Projected{}, stream);
 }
 
 // 1 if this build has the fused kernel (head sizes that are multiples of 128).
@@ -1164,13 +1214,9 @@ int kipp_attention_decode_fused(const float* qkv, int parts, int n_tokens, const
             return rc;
     }
 #endif
-    hipLaunchKernelGGL(attention_decode_kernel<true>, dim3(grid_splits, n_kv, n_items), dim3(THREADS), 0, stream,
-                       (const bf16_t*)nullptr, (bf16_t*)k_cache, (bf16_t*)v_cache, (bf16_t*)out, part_acc, part_ml,
-                       rows, positions, seq_of_token, block_table, max_blocks, n_q, n_kv, page, scale_log2e, window,
-                       max_splits, pj);
-    int rc = KIPP_LAUNCH_CHECK();
-    if (rc != 0 || grid_splits == 1) return rc;
-    return launch_reduce(part_acc, part_ml, (bf16_t*)out, rows, positions, n_items, n_q, window, max_splits, SPLIT, grid_splits, stream);
+    return launch_split<true>((const bf16_t*)nullptr, (bf16_t*)k_cache, (bf16_t*)v_cache, (bf16_t*)out, part_acc, part_ml, rows,
+                              positions, seq_of_token, block_table, max_blocks, n_items, n_q, n_kv, page, scale_log2e, window,
+                              grid_splits, max_splits, pj, stream);
 #else
     return -5;
 #endif
