@@ -179,13 +179,19 @@ __global__ void __launch_bounds__(THREADS, (WM * WN <= 8 ? SMALL_WGS : 1)) gemm_
         // the lane's offset passes through an empty asm here, so that its widening to 64 bits stands beside the
         // load: the compiler then takes the form "scalar base + 32-bit vector offset" and adds nothing per load
         // (widened once outside the walk, the offset would cost a 64-bit vector add for every load)
+        // (in place: the offset keeps its own register for the whole walk.  A copy in a scratch register could be
+        // handed to a read out of LDS as its destination right behind the DMA instruction, and nothing says how
+        // long the memory pipeline takes to fetch an instruction's address registers)
         unsigned char* dst = lds + stage * STAGE_BYTES;
-        uint32_t off = n < WM ? x_src[n < WM ? n : 0] : w_src[n < WM ? 0 : n - WM];
-        asm volatile("" : "+v"(off));
-        if (n < WM)
+        if (n < WM) {
+            uint32_t& off = x_src[n < WM ? n : 0];
+            asm volatile("" : "+v"(off));
             __builtin_amdgcn_global_load_lds(GLOBAL_PTR(x_at + off), LDS_PTR(dst + wave * (X_PIECE / 4) + 1024 * n), 16, 0, 0);
-        else
+        } else {
+            uint32_t& off = w_src[n < WM ? 0 : n - WM];
+            asm volatile("" : "+v"(off));
             __builtin_amdgcn_global_load_lds(GLOBAL_PTR(w_at + off), LDS_PTR(dst + X_PIECE + wave * (W_PIECE / 4) + 1024 * (n - WM)), 16, 0, 0);
+        }
     };
 
     // ---- a lane's place in the operands: row 32 j + l32 of the wave's rows, chunk 2 t + hh of the step
