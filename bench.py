@@ -216,6 +216,8 @@ def main():
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--repeats", type=int, default=5, help="times the K timed steps are run; the median is reported")
     ap.add_argument("--no-long", action="store_true", help="leave out the points at longer contexts")
+    ap.add_argument("--products", choices=["default", "own", "auto", "library"], default="default",
+                    help="products of more than 256 rows: the runtime's default, our kernel only, the fastest of ours and the library's, the library's")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -241,6 +243,8 @@ def main():
     log(f"building {args.shape} ({layers} of {full_layers} layers) with random bfloat16 weights on the device ...")
     t0 = time.perf_counter()
     rt = Runtime("bfloat16")
+    if args.products != "default":
+        rt.own_prompt_products = {"own": True, "auto": "auto", "library": False}[args.products]
     model = random_model(config, seed=0, runtime=rt)
     # the first requests take part in every batch size: room for all those steps
     repeats = max(1, args.repeats)

@@ -95,15 +95,18 @@ struct Depth {
 __device__ long long clock_probe[2048][4];
 #endif
 
-template <int WM, int WN, int END>
-__global__ void __launch_bounds__(THREADS, (WM * WN <= 8 ? SMALL_WGS : 1)) gemm_tiles_kernel(
+template <int WM, int WN, int END, int WGN = 2>
+__global__ void __launch_bounds__(64 * 2 * WGN, (WM * WN <= 8 && WGN == 2 ? SMALL_WGS : 1)) gemm_tiles_kernel(
     const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* __restrict__ Y, int M, int N, int K,
     int tiles_m, int tiles_n, int parts, int inner, int col_begin, int col_end) {
     constexpr int STAGES = Depth<WM, WN>::value;
-    constexpr int TM = 64 * WM, TN = 64 * WN;                     // the workgroup's tile
+    constexpr int WAVES = 2 * WGN;                                // 2 down, WGN across (2: one wave a SIMD, 4: two)
+    constexpr int TM = 64 * WM, TN = 32 * WN * WGN;               // the workgroup's tile
     constexpr int X_PIECE = TM * BK * 2, W_PIECE = TN * BK * 2;   // bytes of a step's pieces
     constexpr int STAGE_BYTES = X_PIECE + W_PIECE;
-    constexpr int LOADS = WM + WN;                                // DMA instructions a wave issues a step
+    constexpr int XI = TM / INSTR_ROWS / WAVES, WI = TN / INSTR_ROWS / WAVES;   // DMA instructions of a wave for each piece
+    static_assert(XI >= 1 && XI * INSTR_ROWS * WAVES == TM && WI * INSTR_ROWS * WAVES == TN, "the waves share the pieces evenly");
+    constexpr int LOADS = XI + WI;                                // DMA instructions a wave issues a step
     constexpr int NM = WM * WN;                                   // products of a half step
     constexpr int NR = WM + WN;                                   // operand reads of a half step
     constexpr int OUT_N = END == END_SWIGLU ? TN / 2 : TN;        // output columns of a tile
@@ -115,7 +118,7 @@ __global__ void __launch_bounds__(THREADS, (WM * WN <= 8 ? SMALL_WGS : 1)) gemm_
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l32 = lane & 31, hh = lane >> 5;
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave / WGN, wn = wave % WGN;
 
     // ---- which tile: workgroups id, id + 8, id + 16, ... run on one die; each die takes a run of
     //      consecutive tiles, rows of X fastest, so that its tiles share rows of W
@@ -140,20 +143,21 @@ __global__ void __launch_bounds__(THREADS, (WM * WN <= 8 ? SMALL_WGS : 1)) gemm_
     // an address is a base that all lanes share (it walks along K in scalar registers) plus a lane's own 32-bit
     // offset, which never changes: no vector arithmetic for an address inside the walk (the launcher refuses
     // operands of 4 GiB and more)
-    uint32_t x_src[WM], w_src[WN];
+    uint32_t x_src[XI], w_src[WI];
     const unsigned char* x_base = (const unsigned char*)(X + (size_t)s_begin * BK);
     const unsigned char* w_base = (const unsigned char*)(W + (size_t)s_begin * BK);
 #pragma unroll
-    for (int i = 0; i < WM; ++i) {
-        const int r = (TM / 4) * wave + INSTR_ROWS * i + lane_row;
+    for (int i = 0; i < XI; ++i) {
+        const int r = (TM / WAVES) * wave + INSTR_ROWS * i + lane_row;
         x_src[i] = (uint32_t)(((size_t)min(tm * TM + r, M - 1) * K + col8) * 2);
     }
 #pragma unroll
-    for (int i = 0; i < WN; ++i) {
-        const int r = (TN / 4) * wave + INSTR_ROWS * i + lane_row;    // row of the piece
+    for (int i = 0; i < WI; ++i) {
+        const int r = (TN / WAVES) * wave + INSTR_ROWS * i + lane_row;    // row of the piece
         int wr;
         if (END == END_SWIGLU) {
-            // a wave's 32 WN rows of the piece are 16 WN gate rows, then the 16 WN up rows that belong to them
+            // the 32 WN rows of the piece that a wave multiplies are 16 WN gate rows, then the 16 WN up rows that
+            // belong to them (`half`: which of the WGN waves across)
             const int half = r / (32 * WN), within = r % (32 * WN);
             const int c = col_begin + tn * OUT_N + 16 * WN * half + within % (16 * WN);
             wr = min(c, col_end - 1) + (within >= 16 * WN ? inner : 0);
@@ -183,14 +187,14 @@ __global__ void __launch_bounds__(THREADS, (WM * WN <= 8 ? SMALL_WGS : 1)) gemm_
         // handed to a read out of LDS as its destination right behind the DMA instruction, and nothing says how
         // long the memory pipeline takes to fetch an instruction's address registers)
         unsigned char* dst = lds + stage * STAGE_BYTES;
-        if (n < WM) {
-            uint32_t& off = x_src[n < WM ? n : 0];
+        if (n < XI) {
+            uint32_t& off = x_src[n < XI ? n : 0];
             asm volatile("" : "+v"(off));
-            __builtin_amdgcn_global_load_lds(GLOBAL_PTR(x_at + off), LDS_PTR(dst + wave * (X_PIECE / 4) + 1024 * n), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds(GLOBAL_PTR(x_at + off), LDS_PTR(dst + wave * (X_PIECE / WAVES) + 1024 * n), 16, 0, 0);
         } else {
-            uint32_t& off = w_src[n < WM ? 0 : n - WM];
+            uint32_t& off = w_src[n < XI ? 0 : n - XI];
             asm volatile("" : "+v"(off));
-            __builtin_amdgcn_global_load_lds(GLOBAL_PTR(w_at + off), LDS_PTR(dst + X_PIECE + wave * (W_PIECE / 4) + 1024 * (n - WM)), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds(GLOBAL_PTR(w_at + off), LDS_PTR(dst + X_PIECE + wave * (W_PIECE / WAVES) + 1024 * (n - XI)), 16, 0, 0);
         }
     };
 
@@ -201,7 +205,7 @@ __global__ void __launch_bounds__(THREADS, (WM * WN <= 8 ? SMALL_WGS : 1)) gemm_
         const int group = l32 / GROUP_ROWS;
         frag_at[t] = group * 256 + (((CHUNKS * (l32 % GROUP_ROWS) + 2 * t + hh) ^ (group & (CHUNKS - 1))) << 4);
     }
-    const int a_base = wm * (X_PIECE / 2), b_base = X_PIECE + wn * (W_PIECE / 2);
+    const int a_base = wm * (X_PIECE / 2), b_base = X_PIECE + wn * (W_PIECE / WGN);
 
     f32x16 acc[WM][WN];
 #pragma unroll
@@ -361,9 +365,9 @@ __global__ void __launch_bounds__(THREADS, (WM * WN <= 8 ? SMALL_WGS : 1)) gemm_
     // which a lane takes 8 neighbouring columns of one row: 16 bytes a store, whole memory lines a row
     constexpr int WCOLS = END == END_SWIGLU ? 16 * WN : 32 * WN;   // output columns of a wave
     constexpr int PITCH = WCOLS + 8;                               // bf16 elements a staged row (the pad spreads the banks)
-    static_assert(32 * PITCH * 2 <= STAGES * STAGE_BYTES / 4, "a wave's staging fits its quarter of LDS");
+    static_assert(32 * PITCH * 2 <= STAGES * STAGE_BYTES / WAVES, "a wave's staging fits its share of LDS");
     __syncthreads();                                               // every wave is done reading operands
-    bf16_t* stage = (bf16_t*)(lds + wave * (STAGES * STAGE_BYTES / 4));
+    bf16_t* stage = (bf16_t*)(lds + wave * (STAGES * STAGE_BYTES / WAVES));
     bf16_t* out = (bf16_t*)Y;
     const int out_width = END == END_SWIGLU ? inner : N;
     const int col0 = col_begin + tn * OUT_N + wn * WCOLS;
@@ -406,6 +410,7 @@ __global__ void __launch_bounds__(THREADS, (WM * WN <= 8 ? SMALL_WGS : 1)) gemm_
 struct Cut {
     int wm, wn, parts;
     int col_begin, col_end;     // output columns
+    int wgn = 2;                // waves across: 2 (4 waves, one a SIMD) or 4 (8 waves, two a SIMD)
 };
 
 #define N_SHAPES 5
@@ -459,20 +464,20 @@ static int plan(int M, int N, int K, int end, int max_parts, Cut* cuts) {
     return n_cuts;
 }
 
-template <int WM, int WN, int END>
+template <int WM, int WN, int END, int WGN = 2>
 static int launch_cut(const void* X, const void* W, void* Y, int M, int N, int K, const Cut& cut, hipStream_t stream) {
-    constexpr int lds_bytes = Depth<WM, WN>::value * 64 * (WM + WN) * BK * 2;
+    constexpr int lds_bytes = Depth<WM, WN>::value * (64 * WM + 32 * WN * WGN) * BK * 2;
     static bool prepared = false;
     if (!prepared) {
-        if (hipFuncSetAttribute((const void*)gemm_tiles_kernel<WM, WN, END>, hipFuncAttributeMaxDynamicSharedMemorySize,
+        if (hipFuncSetAttribute((const void*)gemm_tiles_kernel<WM, WN, END, WGN>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                 lds_bytes) != hipSuccess)
             return -6;
         prepared = true;
     }
-    const int tm = 64 * WM, tn = END == END_SWIGLU ? 32 * WN : 64 * WN;
+    const int tm = 64 * WM, tn = (END == END_SWIGLU ? 16 : 32) * WN * WGN;
     const int tiles_m = (M + tm - 1) / tm, tiles_n = (cut.col_end - cut.col_begin + tn - 1) / tn;
     const int per_die = (tiles_m * tiles_n + 7) / 8;
-    hipLaunchKernelGGL((gemm_tiles_kernel<WM, WN, END>), dim3(per_die * 8, 1, cut.parts), dim3(THREADS), lds_bytes, stream,
+    hipLaunchKernelGGL((gemm_tiles_kernel<WM, WN, END, WGN>), dim3(per_die * 8, 1, cut.parts), dim3(64 * 2 * WGN), lds_bytes, stream,
                        (const bf16_t*)X, (const bf16_t*)W, Y, M, N, K, tiles_m, tiles_n, cut.parts, N / 2, cut.col_begin,
                        cut.col_end);
     return KIPP_LAUNCH_CHECK();
@@ -480,6 +485,12 @@ static int launch_cut(const void* X, const void* W, void* Y, int M, int N, int K
 
 template <int END>
 static int launch_end(const void* X, const void* W, void* Y, int M, int N, int K, const Cut& cut, hipStream_t stream) {
+    if (cut.wgn == 4) {
+        // 8 waves, two a SIMD: the same workgroup tiles from wave tiles half as wide
+        if (cut.wm == 4 && cut.wn == 2) return launch_cut<4, 2, END, 4>(X, W, Y, M, N, K, cut, stream);
+        if (cut.wm == 2 && cut.wn == 2) return launch_cut<2, 2, END, 4>(X, W, Y, M, N, K, cut, stream);
+        return -5;
+    }
     if (cut.wm == 4 && cut.wn == 4) return launch_cut<4, 4, END>(X, W, Y, M, N, K, cut, stream);
     if (cut.wm == 4 && cut.wn == 2) return launch_cut<4, 2, END>(X, W, Y, M, N, K, cut, stream);
     if (cut.wm == 2 && cut.wn == 4) return launch_cut<2, 4, END>(X, W, Y, M, N, K, cut, stream);
@@ -507,7 +518,7 @@ int kipp_gemm_tiles_parts(int M, int N, int K, int end, int max_parts) {
 }
 
 // Y: float32 [parts, M, N] with parts = kipp_gemm_tiles_parts(...) (end 0), bfloat16 [M, N / 2] = silu(gate) * up for
-// W = [gate; up] (end 1), bfloat16 [M, N] (end 2).  K a multiple of 32.  `force`: 0, or 100 wm + 10 wn + parts to take
+// W = [gate; up] (end 1), bfloat16 [M, N] (end 2).  K a multiple of 32.  `force`: 0, or 100 wm + 10 wn + parts (+ 1000: 8 waves, four across) to take
 // that cut for all columns whatever the plan says (measurements and tests).
 int kipp_gemm_tiles(const void* X, const void* W, void* Y, int M, int N, int K, int end, int max_parts, int force,
                     hipStream_t stream) {
@@ -521,7 +532,7 @@ int kipp_gemm_tiles(const void* X, const void* W, void* Y, int M, int N, int K, 
     int n_cuts = plan(M, N, K, end, max_parts, cuts);
     if (force) {
         n_cuts = 1;
-        cuts[0] = {force / 100, (force / 10) % 10, force % 10, 0, end == END_SWIGLU ? N / 2 : N};
+        cuts[0] = {(force / 100) % 10, (force / 10) % 10, force % 10, 0, end == END_SWIGLU ? N / 2 : N, force >= 1000 ? 4 : 2};
     }
     for (int c = 0; c < n_cuts; ++c) {
         const Cut& cut = cuts[c];

@@ -649,11 +649,17 @@ def gemm_tiles_ok(m: int, k: int, n: int = 1) -> bool:
     return m > 0 and k > 0 and k % 32 == 0 and max(m, n) * k * 2 < 2**32
 
 
+def gemm_tiles_parts(m: int, n: int, k: int, end: str = "slabs", max_parts: int = 1) -> int:
+    """Parts of K the launcher plans for a product of these sizes when it may use up to `max_parts`."""
+    return int(build.library("gemm_tiles").kipp_gemm_tiles_parts(int(m), int(n), int(k), TILES_END[end], int(max_parts)))
+
+
 def gemm_tiles(x: torch.Tensor, w: torch.Tensor, end: str = "slabs", max_parts: int = 1, force: int = 0) -> torch.Tensor:
     """x [M, K] . w [N, K]^T on the matrix cores for many rows, bfloat16 operands, float32 accumulation.
     end "slabs": float32 [parts, M, N] whose sum over parts is the product (parts <= max_parts, chosen from the shape);
     "swiglu": w = [gate; up] of [2 I, K], the result is bfloat16 [M, I] = silu(x . gate^T) * (x . up^T);
-    "bf16": bfloat16 [M, N].  `force` = 100 wm + 10 wn + parts takes that cut instead of the planned one (tests)."""
+    "bf16": bfloat16 [M, N].  `force` = 100 wm + 10 wn + parts (+ 1000: workgroups of 8 waves, four across, wave tiles
+    4 x 2 or 2 x 2) takes that cut instead of the planned one (the runtime's timed choice, tests)."""
     _dev(x, w)
     m, k = x.shape
     n = w.shape[0]

@@ -9,6 +9,8 @@ dtype "float32": everything is widened to float32 and every product is a true
 """
 from __future__ import annotations
 
+import os
+
 import torch
 
 from .csrc import ops
@@ -107,10 +109,12 @@ class Runtime:
         self.library_products = 0   # calls that went to the library (they stay out of HIP graphs)
         self.generic_attention_launches = 0   # bfloat16 attention that fell to the generic kernel (geometry the matrix-core kernels refuse)
         self.fuse_norms = True      # few rows: residual add and norm ride on the products around them
-        # products of more than 256 rows: our own matrix-core kernel (as planned, or in one of a few other cuts) or
-        # the library's, whichever is fastest for the shape ("auto": all are timed once, at the shape's first use);
-        # True / False: always ours as planned / always the library's
-        self.own_prompt_products = "auto"
+        # products of more than 256 rows: "auto" (the default): the fastest of our own matrix-core kernel's cuts and
+        # the library's product, timed once in a process at a shape's first use (another process may choose
+        # otherwise, and its results then differ in their last bits); True: our kernel, in the fastest of the cuts
+        # that give the planned cut's bits (the same bits in every process); False: always the library's.
+        # KIPP_AMD_PRODUCTS=own|auto|library sets it from outside.
+        self.own_prompt_products = {"own": True, "auto": "auto", "library": False}.get(os.environ.get("KIPP_AMD_PRODUCTS", "auto"), "auto")
         self.prompt_product_choices = {}     # shape -> "library", "plan" (our kernel, cut as planned) or a forced cut of ours
         self.tile_products = 0      # products of more than 256 rows that ran on our own kernel
         torch.backends.cuda.matmul.allow_tf32 = False
@@ -180,37 +184,60 @@ class Runtime:
         """Rows of a prompt product, in classes of a factor of two (257-512, 513-1024, ...): one decision a class."""
         return 1 << (max(m, 1) - 1).bit_length()
 
-    # cuts of our kernel that are timed beside the planned one: 100 x (wave tile rows / 32) + 10 x (wave tile
-    # columns / 32) + parts of K.  The plan's cost model is linear; the GPU under its power limit is not (a
-    # round that leaves compute units idle clocks the others higher), so the plan is not always the fastest.
-    TILE_CUTS_SLABS = (441, 442, 444, 431, 432, 421, 422)
-    TILE_CUTS_BF16 = (441, 421, 241)
+    # Cuts of our kernel that are timed beside the planned one: 100 x (wave tile rows / 32) + 10 x (wave tile
+    # columns / 32) + parts of K (+ 1000: workgroups of 8 waves, two a SIMD, on the same 256 x 256 tile).  The
+    # plan's cost model is linear; the GPU under its power limit is not (a round that leaves compute units idle
+    # clocks the others higher), so the plan is not always the fastest.  An output element is summed over K in
+    # the same order whatever the tile, so cuts with the same parts of K give the same bits.
+    _choices_of_process: dict = {}
+    TILE_CUTS_SLABS = (441, 442, 444, 431, 432, 421, 422, 1421, 1422, 1424)
+    TILE_CUTS_BF16 = (441, 421, 241, 1421)
 
-    def _fastest(self, key, ways: dict):
-        """Which of several ways to compute one product is taken for the shape `key`: decided once, by the
-        switch (True: our planned cut, False: the library's) or by timing all of them on the operands at hand
-        (three runs each after a first one).  `ways`: name -> callable, "library" and "plan" among them."""
+    def _fastest(self, key, ways: dict, same_bits):
+        """Which of several ways to compute one product is taken for the shape `key`: decided once, by timing
+        them on the operands at hand (three runs each after a first one).  `ways`: name -> callable, "library"
+        and "plan" among them; `same_bits`: the names whose results are those of "plan" bit for bit.
+        `own_prompt_products` True (the default): only those are timed, so the choice changes how long a
+        product takes and never what it gives; "auto": all of them (the library's product and other parts of K
+        round differently: two runs of one program may then differ in their last bits); False: the library's."""
         choice = self.prompt_product_choices.get(key)
         if choice is None:
-            if self.own_prompt_products != "auto":
-                choice = "plan" if self.own_prompt_products else "library"
+            choice = self._choices_of_process.get((self.own_prompt_products, key))      # every engine of a process decides alike
+        if choice is not None:
+            self.prompt_product_choices[key] = choice
+        if choice is None:
+            if self.own_prompt_products is False:
+                choice = "library"
             else:
-                best = None
+                # The chip is at its power limit while products follow each other, and a product that wins from
+                # a standing start need not win then: every candidate runs a few times first, then they are
+                # timed in turn, twice round, without a pause between them
+                runs = {}
                 for name, run in ways.items():
+                    if self.own_prompt_products != "auto" and name not in same_bits:
+                        continue
                     try:
-                        run()
+                        for _ in range(3):
+                            run()
                     except self.ops.KernelError:
                         continue                      # a cut this shape does not take
-                    begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                    begin.record()
-                    for _ in range(3):
-                        run()
-                    end.record()
-                    end.synchronize()
-                    ms = begin.elapsed_time(end)
-                    if best is None or ms < best:
-                        best, choice = ms, name
+                    runs[name] = run
+                marks = []
+                for _ in range(2):
+                    for name, run in runs.items():
+                        begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                        begin.record()
+                        for _ in range(4):
+                            run()
+                        end.record()
+                        marks.append((name, begin, end))
+                torch.cuda.current_stream().synchronize()
+                took = {}
+                for name, begin, end in marks:
+                    took[name] = took.get(name, 0.0) + begin.elapsed_time(end)
+                choice = min(took, key=took.get) if took else "plan"
             self.prompt_product_choices[key] = choice
+            self._choices_of_process[(self.own_prompt_products, key)] = choice
         return choice
 
     def _library_product(self, x, w):
@@ -241,7 +268,7 @@ class Runtime:
         if self.ops.gemm_tiles_ok(m, k, rows.shape[0]):
             ways = {"library": library, "plan": ours}
             ways.update({cut: (lambda cut=cut: ours(cut)) for cut in self.TILE_CUTS_BF16})
-            choice = self._fastest(("gated", self._rows_class(m), rows.shape[0], k), ways)
+            choice = self._fastest(("gated", self._rows_class(m), rows.shape[0], k), ways, ("plan",) + self.TILE_CUTS_BF16)
             if choice != "library":
                 self.tile_products += 1
                 return ours(0 if choice == "plan" else choice)
@@ -296,7 +323,9 @@ class Runtime:
                 return self._library_product(x, w)
             ways = {"library": library, "plan": ours}
             ways.update({cut: (lambda cut=cut: ours(cut)) for cut in self.TILE_CUTS_SLABS if cut % 10 <= most})
-            choice = self._fastest(("linear", self._rows_class(m), n, x.shape[1], most), ways)
+            planned = self.ops.gemm_tiles_parts(m, n, x.shape[1], "slabs", most)
+            same = ("plan",) + tuple(cut for cut in self.TILE_CUTS_SLABS if cut % 10 == planned)
+            choice = self._fastest(("linear", self._rows_class(m), n, x.shape[1], most), ways, same)
             if choice != "library":
                 self.tile_products += 1
                 return ours(0 if choice == "plan" else choice)

@@ -146,7 +146,7 @@ def mfma_rate() -> dict:
     return {"workload": "mfma rate", "compute_units": cus, "all": table}
 
 
-def walk(ablate_dma: int, ablate_reads: bool, n: int = 8192, k: int = 9728, rows: int = 2048) -> dict:
+def walk(ablate_dma: int, ablate_reads: bool, n: int = 8192, k: int = 9728, rows: int = 2048, cut: int = 441) -> dict:
     """Shader cycles a product (v_mfma_f32_32x32x16_bf16, 32 cycles of the matrix core) inside the walk over K
     of the prompt-product kernel, from a build that reads the shader clock and the 100 MHz clock around the
     walk; optionally with the DMA taken out (1) or made to bring the first step every time (2: it always hits
@@ -170,21 +170,22 @@ def walk(ablate_dma: int, ablate_reads: bool, n: int = 8192, k: int = 9728, rows
     table = []
     for launches in (1, 20):
         for _ in range(launches):
-            rc = lib.kipp_gemm_tiles(x.data_ptr(), w.data_ptr(), out.data_ptr(), rows, n, k, 0, 1, 441, torch.cuda.current_stream().cuda_stream)
+            rc = lib.kipp_gemm_tiles(x.data_ptr(), w.data_ptr(), out.data_ptr(), rows, n, k, 0, 1, cut, torch.cuda.current_stream().cuda_stream)
             if rc != 0:
                 raise RuntimeError(f"gemm_tiles refused (code {rc})")
         torch.cuda.synchronize()
-        groups = min(2048, -(-rows // 256) * -(-n // 256))
+        groups = min(2048, -(-rows // (64 * ((cut // 100) % 10))) * -(-n // (32 * ((cut // 10) % 10) * (4 if cut >= 1000 else 2))))
         buf = np.zeros((2048, 4), dtype=np.int64)
         if lib.kipp_gemm_tiles_clock(buf.ctypes.data, 2048) != 0:
             raise RuntimeError("the probe's counters could not be read")
         b = buf[:groups].astype(float)
-        products = b[:, 2] * 32                      # a wave's products in the walk: 32 a step
+        wm, wn, per_simd = (cut // 100) % 10, (cut // 10) % 10, (2 if cut >= 1000 else 1)
+        products = b[:, 2] * 2 * wm * wn * per_simd  # a SIMD's products in the walk: 2 wm wn a step of each of its waves
         row = {"after_launches": launches, "cycles_per_product": round(float(np.median(b[:, 0] / products)), 2),
                "ns_per_product": round(float(np.median(b[:, 1] * 10 / products)), 2),
                "GHz": round(float(np.median(b[:, 0] / (b[:, 1] * 10))), 3)}
         table.append(row)
-        log(f"{rows} x {n} x {k}, after {launches} launch(es): {row['cycles_per_product']} shader cycles a product, "
+        log(f"{rows} x {n} x {k}, after {launches} launch(es): {row['cycles_per_product']} shader cycles a product of a SIMD, "
             f"{row['ns_per_product']} ns, clock {row['GHz']} GHz")
     return {"workload": "walk", "ablate_dma": ablate_dma, "ablate_reads": bool(ablate_reads), "all": table}
 
@@ -294,12 +295,15 @@ def main(argv=None) -> int:
         ap = argparse.ArgumentParser(prog="python -m kipp_amd.workloads walk")
         ap.add_argument("--ablate-dma", type=int, default=0, choices=[0, 1, 2])
         ap.add_argument("--ablate-reads", action="store_true")
+        ap.add_argument("--cut", type=int, default=441, help="100 wm + 10 wn + parts (+ 1000: 8 waves)")
+        ap.add_argument("--n", type=int, default=8192)
+        ap.add_argument("--k", type=int, default=9728)
         args = ap.parse_args(argv[1:])
         import torch
         if not torch.cuda.is_available():
             print("workload: no GPU", file=sys.stderr)
             return 1
-        print(json.dumps(walk(args.ablate_dma, args.ablate_reads)), flush=True)
+        print(json.dumps(walk(args.ablate_dma, args.ablate_reads, n=args.n, k=args.k, cut=args.cut)), flush=True)
         return 0
     if argv and argv[0] == "mfma":
         import torch

@@ -783,7 +783,7 @@ def test_gemm_rows(m, n, k, max_parts):
                            ops.gemm_rows(x.to(DEV), wd, max_parts))
 
 
-TILE_CUTS = [0, 441, 442, 421, 243, 221, 224, 431, 232]      # 100 wm + 10 wn + parts; 0: what the launcher plans
+TILE_CUTS = [0, 441, 442, 421, 243, 221, 224, 431, 232, 1421, 1422, 1221]      # 100 wm + 10 wn + parts (+ 1000: 8 waves); 0: what the launcher plans
 
 
 @pytest.mark.parametrize("force", TILE_CUTS)
@@ -807,7 +807,7 @@ def test_gemm_tiles_float32_end(m, n, k, force):
     assert np.array_equal(out.cpu().numpy(), xi.float().numpy() @ wi.float().numpy().T)
 
 
-@pytest.mark.parametrize("force", [0, 441, 421, 241, 221])
+@pytest.mark.parametrize("force", [0, 441, 421, 241, 221, 1421, 1221])
 @pytest.mark.parametrize("m,inner,k", [(257, 150, 64), (600, 9728 // 8, 160), (300, 24, 2560), (2050, 1300, 96)])
 def test_gemm_tiles_swiglu_and_bfloat16_ends(m, inner, k, force):
     """W = [gate; up]: silu(x . gate^T) * (x . up^T) rounded once, at the end (gate first: the other way round
@@ -828,6 +828,23 @@ def test_gemm_tiles_swiglu_and_bfloat16_ends(m, inner, k, force):
     # bit for bit what rounding the float32 end gives
     exact = ops.gemm_tiles(x.to(DEV), w.to(DEV), "slabs", force=force)[0]
     assert torch.equal(rounded, exact.to(torch.bfloat16))
+
+
+def test_gemm_tiles_cuts_with_the_same_parts_give_the_same_bits():
+    """An output element is summed over K in the same order whatever the wave tile and the number of waves: every
+    cut with the same parts of K gives the same bits (the runtime relies on it when it takes the fastest of them)."""
+    ops = _ops()
+    rng = np.random.default_rng(3)
+    x = torch.tensor(rng.normal(size=(700, 2560)), dtype=torch.bfloat16).to(DEV)
+    w = torch.tensor(rng.normal(size=(1300, 2560)) * 0.05, dtype=torch.bfloat16).to(DEV)
+    for parts, cuts in ((1, (441, 431, 421, 241, 221, 1421, 1221)), (2, (442, 432, 422, 222, 1422)), (4, (444, 424, 1424))):
+        base = ops.gemm_tiles(x, w, "slabs", max_parts=4, force=cuts[0])
+        assert base.shape[0] == parts
+        for cut in cuts[1:]:
+            assert torch.equal(ops.gemm_tiles(x, w, "slabs", max_parts=4, force=cut), base), cut
+    gated = ops.gemm_tiles(x, w, "swiglu", force=441)
+    for cut in (0, 421, 241, 221, 1421):
+        assert torch.equal(ops.gemm_tiles(x, w, "swiglu", force=cut), gated), cut
 
 
 def test_gemm_tiles_refuses_what_it_cannot_do():
