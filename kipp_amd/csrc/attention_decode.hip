@@ -684,11 +684,11 @@ __global__ void __launch_bounds__(THREADS, 2) attention_decode_ring_kernel(
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l16 = lane & 15, h = lane >> 4;
     const int kvh = blockIdx.y;
-    const int row = rows[blockIdx.z];
+    const int row = rows[blockIdx.x];                 // the grid is (query tokens, key/value heads, ranges): ranges beyond a sequence's position come last
     const int pos = positions[row];
     const int lo = window > 0 ? max(0, pos - window + 1) : 0;
     const int first_split = lo / range, last_split = pos / range;
-    const int split = first_split + blockIdx.x;
+    const int split = first_split + blockIdx.z;
     if (split > last_split) return;
     const int n_splits = last_split - first_split + 1;
     const int base = split * range;
@@ -923,7 +923,7 @@ __global__ void __launch_bounds__(THREADS, 2) attention_decode_ring_kernel(
         if (n_splits == 1) {
             out[((size_t)row * n_q + head) * HEAD_DIM + dcol] = f32_to_bf16(a / l);
         } else {
-            const size_t slot = ((size_t)blockIdx.z * n_q + head) * max_splits + blockIdx.x;
+            const size_t slot = ((size_t)blockIdx.x * n_q + head) * max_splits + blockIdx.z;
             part_acc[slot * HEAD_DIM + dcol] = a;
             if (dcol == 0) {
                 part_ml[slot * 2] = m;
@@ -1041,14 +1041,20 @@ static int launch_reduce(const float* part_acc, const float* part_ml, bf16_t* ou
 
 #if RING_OK
 // Keys a workgroup of the kernel that streams through LDS walks in a launch of this shape; 0: the launch
-// is not for it.  Many sequences: whole contexts (RING_RANGE keys at most).  Few: ranges that give 256
-// workgroups, if those are 1,024 keys and more.  A function of the launch's shape, never of the data.
+// is not for it.  RING_WHOLE_FROM_PAIRS (sequence, key/value head) pairs and more: whole contexts (RING_RANGE
+// keys at most).  Fewer: ranges that give 256 workgroups, if those are 1,024 keys and more; else whole contexts
+// from RING_FROM_PAIRS pairs on.  Measured in the decode step at 2,100 keys, 8 heads: 12 sequences in two ranges
+// (192 workgroups at work instead of 96) 3.24 instead of 3.54 ms; 16 sequences 3.50 to 3.56 either way; 24
+// sequences in two ranges 4.11 instead of 3.97 (the partial results and their merge cost more than the second
+// workgroup on every compute unit brings).  A function of the launch's shape, never of the data.
+#define RING_WHOLE_FROM_PAIRS 128
 static int ring_range(int n_items, int n_kv, int page, int grid_splits) {
     if (page % 16 != 0) return 0;
     const long long pairs = (long long)n_items * n_kv, span = (long long)grid_splits * SPLIT;
-    if (pairs >= RING_FROM_PAIRS) return (int)(span < RING_RANGE ? span : RING_RANGE);
+    const long long whole = span < RING_RANGE ? span : RING_RANGE;
+    if (pairs >= RING_WHOLE_FROM_PAIRS) return (int)whole;
     const long long range = span * pairs / 256 / SPLIT * SPLIT;
-    if (range < 1024) return 0;
+    if (range < 1024) return pairs >= RING_FROM_PAIRS ? (int)whole : 0;
     return (int)(range < RING_RANGE ? range : RING_RANGE);
 }
 
@@ -1074,7 +1080,7 @@ static int launch_ring(const bf16_t* q, bf16_t* k_cache, bf16_t* v_cache, bf16_t
     const int span = grid_splits * SPLIT;
     const int ring_splits = (span + range - 1) / range + (window > 0 ? 1 : 0);   // a window may straddle one more edge
     if (ring_splits > max_splits) return 0;
-    hipLaunchKernelGGL(attention_decode_ring_kernel<FUSED>, dim3(ring_splits, n_kv, n_items), dim3(THREADS), lds, stream, q,
+    hipLaunchKernelGGL(attention_decode_ring_kernel<FUSED>, dim3(n_items, n_kv, ring_splits), dim3(THREADS), lds, stream, q,
                        k_cache, v_cache, out, part_acc, part_ml, rows, positions, seq_of_token, block_table, max_blocks, n_q,
                        n_kv, page, scale_log2e, window, max_splits, range, pj);
     *rc = KIPP_LAUNCH_CHECK();
