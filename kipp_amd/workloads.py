@@ -143,7 +143,22 @@ def mfma_rate() -> dict:
                     best = max(best, flops / (ms * 1e-3) / 1e15)
                 table.append({"operands": name, "grid": what, "ms": round(ms, 3), "PFLOP_s": round(best, 3)})
                 log(f"{name:6s} {what:17s} kernel of {ms:8.3f} ms: {best:5.3f} PFLOP/s")
-    return {"workload": "mfma rate", "compute_units": cus, "all": table}
+    # what a DMA instruction into LDS costs the products of the wave that issues it, and whether a second wave hides it
+    data = operands["normal"].to("cuda:0")
+    src = torch.zeros(cus * 65536, dtype=torch.uint8, device="cuda:0")
+    dma = []
+    for waves in (4, 8):
+        for every in (0, 4, 2):
+            start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            ops.mfma_dma(data, src, cus, waves, every, 2000)
+            start.record()
+            flops = ops.mfma_dma(data, src, cus, waves, every, 2000)
+            end.record()
+            torch.cuda.synchronize()
+            ns = start.elapsed_time(end) * 1e6 / (flops / 32768 / (cus * 4))
+            dma.append({"waves_per_simd": waves // 4, "dma_every": every, "ns_per_product_of_a_simd": round(ns, 2)})
+            log(f"{waves // 4} wave(s) a SIMD, a DMA instruction behind every {every or 'no'} product(s): {ns:6.2f} ns a product of a SIMD")
+    return {"workload": "mfma rate", "compute_units": cus, "all": table, "dma": dma}
 
 
 def walk(ablate_dma: int, ablate_reads: bool, n: int = 8192, k: int = 9728, rows: int = 2048, cut: int = 441) -> dict:
