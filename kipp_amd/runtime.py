@@ -193,10 +193,12 @@ class Runtime:
     TILE_CUTS_SLABS = (441, 442, 444, 431, 432, 421, 422, 1421, 1422, 1424)
     TILE_CUTS_BF16 = (441, 421, 241, 1421)
 
-    def _fastest(self, key, ways: dict, same_bits):
+    def _fastest(self, key, ways: dict, same_bits, extra_ms=None):
         """Which of several ways to compute one product is taken for the shape `key`: decided once, by timing
         them on the operands at hand (three runs each after a first one).  `ways`: name -> callable, "library"
-        and "plan" among them; `same_bits`: the names whose results are those of "plan" bit for bit.
+        and "plan" among them; `same_bits`: the names whose results are those of "plan" bit for bit;
+        `extra_ms`: name -> milliseconds that a way costs its consumer beyond its own kernel (the slabs of a split
+        product are read by the kernel that adds them).
         `own_prompt_products` True (the default): only those are timed, so the choice changes how long a
         product takes and never what it gives; "auto": all of them (the library's product and other parts of K
         round differently: two runs of one program may then differ in their last bits); False: the library's."""
@@ -234,7 +236,9 @@ class Runtime:
                 torch.cuda.current_stream().synchronize()
                 took = {}
                 for name, begin, end in marks:
-                    took[name] = took.get(name, 0.0) + begin.elapsed_time(end)
+                    took[name] = took.get(name, 0.0) + begin.elapsed_time(end) / 4
+                for name in took:
+                    took[name] += 2 * (extra_ms or {}).get(name, 0.0)
                 choice = min(took, key=took.get) if took else "plan"
             self.prompt_product_choices[key] = choice
             self._choices_of_process[(self.own_prompt_products, key)] = choice
@@ -325,7 +329,10 @@ class Runtime:
             ways.update({cut: (lambda cut=cut: ours(cut)) for cut in self.TILE_CUTS_SLABS if cut % 10 <= most})
             planned = self.ops.gemm_tiles_parts(m, n, x.shape[1], "slabs", most)
             same = ("plan",) + tuple(cut for cut in self.TILE_CUTS_SLABS if cut % 10 == planned)
-            choice = self._fastest(("linear", self._rows_class(m), n, x.shape[1], most), ways, same)
+            # every slab beyond the first is read once more by the kernel that adds them (at about 5 TB/s)
+            slab_ms = m * n * 4 / 5e12 * 1e3
+            extra = {name: ((planned if name == "plan" else name % 10) - 1) * slab_ms for name in ways if name != "library"}
+            choice = self._fastest(("linear", self._rows_class(m), n, x.shape[1], most), ways, same, extra)
             if choice != "library":
                 self.tile_products += 1
                 return ours(0 if choice == "plan" else choice)
