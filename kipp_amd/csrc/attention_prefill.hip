@@ -446,18 +446,48 @@ __global__ void __launch_bounds__(THREADS, 2) attention_prefill_dma_kernel(
         if (!wave_active) return;
 
         // ---- S^T = K Q^T for the two 32-key halves of the tile
+        // The key operands of step t + 2 are asked for before the products of step t: a read out of LDS takes
+        // longer than the two products of a step, and asked for right in front of them it is waited for every
+        // step.  Written out, with waits that count: left to the compiler every wait is for all reads on their way.
+        static_assert(QSTEPS == 8, "the waits below are written for eight steps");
         f32x16 s_acc[2];
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
+        for (int j = 0; j < 2; ++j)
 #pragma unroll
             for (int v = 0; v < 16; ++v) s_acc[j][v] = 0.0f;
-#pragma unroll
-            for (int t = 0; t < QSTEPS; ++t) {
-                Frag kf;
-                kf.u = *(const u32x4*)(Ks + k_at[t] + j * (32 * 256));
-                s_acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf.v, qf[t].v, s_acc[j], 0, 0, 0);
-            }
-        }
+        u32x4 kf[3][2];
+        const uint32_t k_lds = (uint32_t)(uintptr_t)LDS_PTR(Ks);
+#define KIPP_K_READ(T)                                                                                              \
+    _Pragma("unroll") for (int j = 0; j < 2; ++j)                                                                   \
+        asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(kf[(T) % 3][j]) : "v"(k_lds + k_at[T]), "i"(j * (32 * 256)))
+#define KIPP_K_STEP(T, N)                                                                                           \
+    do {                                                                                                            \
+        asm volatile("s_waitcnt lgkmcnt(" #N ")" : "+v"(kf[(T) % 3][0]), "+v"(kf[(T) % 3][1]));                      \
+        _Pragma("unroll") for (int j = 0; j < 2; ++j) {                                                             \
+            Frag f;                                                                                                 \
+            f.u = kf[(T) % 3][j];                                                                                   \
+            s_acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.v, qf[T].v, s_acc[j], 0, 0, 0);                    \
+        }                                                                                                           \
+        __builtin_amdgcn_sched_barrier(0);   /* the order written here is the order meant */                       \
+    } while (0)
+        KIPP_K_READ(0);
+        KIPP_K_READ(1);
+        KIPP_K_READ(2);
+        KIPP_K_STEP(0, 4);
+        KIPP_K_READ(3);
+        KIPP_K_STEP(1, 4);
+        KIPP_K_READ(4);
+        KIPP_K_STEP(2, 4);
+        KIPP_K_READ(5);
+        KIPP_K_STEP(3, 4);
+        KIPP_K_READ(6);
+        KIPP_K_STEP(4, 4);
+        KIPP_K_READ(7);
+        KIPP_K_STEP(5, 4);
+        KIPP_K_STEP(6, 2);
+        KIPP_K_STEP(7, 0);
+#undef KIPP_K_READ
+#undef KIPP_K_STEP
         const bool masked = key0 + BN - 1 > pos0 + wave * 32 || window > 0;
         if (masked) {
 #pragma unroll
