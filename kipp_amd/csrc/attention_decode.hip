@@ -42,7 +42,7 @@
 #endif
 
 #define SPLIT 256                              // keys of a split (the kernel that takes one a workgroup also has longer ones)
-#define SPLIT_MAX 384
+#define SPLIT_MAX 320                          // the longest (the fused form has registers for no more with two workgroups a compute unit)
 #define WAVES 4
 #define THREADS (WAVES * KIPP_WAVE)
 #define KSTEPS ((HEAD_DIM + 31) / 32)          // MFMA steps of 32 over the head size
@@ -1090,8 +1090,8 @@ static int launch_ring(const bf16_t* q, bf16_t* k_cache, bf16_t* v_cache, bf16_t
 }
 #endif
 
-// The kernel that takes one split a workgroup, with splits of 256 keys, or of 320 or 384 where splits of 256
-// would be more workgroups than two a compute unit and the longer ones are not: workgroups beyond those that
+// The kernel that takes one split a workgroup, with splits of 256 keys, or of 320 where splits of 256
+// would be more workgroups than two a compute unit: workgroups beyond those that
 // fit at once run as a second round behind the first (measured at 8 sequences of 8 key/value heads: 576
 // workgroups for 2,050 keys cost 0.15 ms a step more than 512 for 2,040).  A function of the launch's shape.
 static int split_keys_for(int n_items, int n_kv, int span_keys, int window, int longest) {
@@ -1110,9 +1110,8 @@ static int launch_split(const bf16_t* q, bf16_t* k_cache, bf16_t* v_cache, bf16_
                         float scale_log2e, int window, int grid_splits, int max_splits, Projected pj, hipStream_t stream) {
     const int extra = window > 0 ? 1 : 0;
     const int span_keys = (grid_splits - extra) * SPLIT;           // the caller counts splits of SPLIT keys
-    // the fused form holds the projected heads as well: with splits of 384 keys it needs more registers than two
-    // workgroups a compute unit leave it (272 of 256)
-    const int keys = split_keys_for(n_items, n_kv, span_keys, window, FUSED ? 320 : SPLIT_MAX);
+    // one rule for both forms, so that they cut alike and give the same bits
+    const int keys = split_keys_for(n_items, n_kv, span_keys, window, SPLIT_MAX);
     const int splits = keys == SPLIT ? grid_splits : (span_keys + keys - 1) / keys + extra;
 #define KIPP_SPLIT_LAUNCH(KEYS)                                                                                       \
     hipLaunchKernelGGL((attention_decode_kernel<FUSED, KEYS>), dim3(n_items, n_kv, splits), dim3(THREADS), 0, stream, q, \
@@ -1121,12 +1120,6 @@ static int launch_split(const bf16_t* q, bf16_t* k_cache, bf16_t* v_cache, bf16_
     switch (keys) {
         case 256: KIPP_SPLIT_LAUNCH(256); break;
         case 320: KIPP_SPLIT_LAUNCH(320); break;
-        case 384:
-            if constexpr (!FUSED) {
-                KIPP_SPLIT_LAUNCH(384);
-                break;
-            }
-            return -1;
         default: return -1;
     }
 #undef KIPP_SPLIT_LAUNCH

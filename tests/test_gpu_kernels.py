@@ -472,6 +472,38 @@ def test_attention_decode_of_few_long_sequences(window):
         assert _rel(got[i], ref[i]) < 1e-5, f"context of {seq_lens[i]} keys"
 
 
+def test_attention_decode_in_longer_splits():
+    """8 sequences of 8 key/value heads behind 2,100 to 2,700 keys: splits of 256 keys would be more workgroups
+    than fit at once, so both forms of the kernel cut the keys every 320 (a recorded graph asks for the longest
+    context of its bucket: the splits beyond a sequence's position leave at once).  Against the plain attention,
+    and the same bits from both forms."""
+    ops = _ops()
+    n_q, n_kv, d, page = 32, 8, 128, 16
+    rng = np.random.default_rng(21)
+    seq_lens = [2100, 2700, 2561, 320, 321, 1, 2239, 2240]
+    table, k, v = _paged_setup(rng, seq_lens, n_kv, d, page, torch.bfloat16)
+    t = len(seq_lens)
+    rows, positions, seq_of = list(range(t)), [n - 1 for n in seq_lens], list(range(t))
+    width = (n_q + 2 * n_kv) * d
+    qkv = _t(rng.normal(size=(t, width)).astype(np.float32))
+    inv_freq = _t(np.power(1e6, -(2.0 * np.arange(d // 2)) / d).astype(np.float32))
+    args = (_t(positions, torch.int32), _t(seq_of, torch.int32), _t(table, torch.int32))
+    longest = 3072                                     # what a graph recorded for this bucket of contexts asks for
+    ws = ops.attention_decode_workspace(t, n_q, d, longest, DEV)
+    k1, v1 = k.to(DEV), v.to(DEV)
+    q = ops.qk_norm_rope_kv_write(qkv, torch.empty(t, n_q * d, dtype=torch.bfloat16, device=DEV), k1, v1, *args, n_q, n_kv, d,
+                                  None, None, 0.0, inv_freq, d, write_kv=True)
+    want = ops.attention_decode(q, k1, v1, torch.zeros(t, n_q * d, dtype=torch.bfloat16, device=DEV), _t(rows, torch.int32),
+                                *args, n_q, n_kv, d, 1 / math.sqrt(d), 0, longest, ws)
+    k2, v2 = k.to(DEV), v.to(DEV)
+    got = ops.attention_decode_fused(qkv, k2, v2, torch.zeros(t, n_q * d, dtype=torch.bfloat16, device=DEV),
+                                     _t(rows, torch.int32), *args, n_q, n_kv, d, None, None, 0.0, inv_freq, d, True,
+                                     1 / math.sqrt(d), 0, longest, ws)
+    assert torch.equal(got, want) and torch.equal(k1, k2) and torch.equal(v1, v2)
+    ref = _attention_reference(q.cpu(), k1.cpu(), v1.cpu(), table, positions, seq_of, n_q, n_kv, d, page, 0)
+    assert _rel(want.float().cpu().numpy().reshape(t, n_q, d), ref) < 1e-5
+
+
 _PROJECTION_GEOMETRIES = [(32, 8, 128, 16), (8, 1, 128, 8), (16, 1, 128, 16), (3, 3, 128, 4), (8, 2, 256, 32), (4, 2, 256, 16)]
 
 
