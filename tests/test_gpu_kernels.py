@@ -447,6 +447,40 @@ def test_attention_decode_over_whole_contexts(n_q, n_kv, d, page, window):
         ops._fn = inner
 
 
+@pytest.mark.parametrize("window", [0, 2500])
+def test_attention_decode_of_a_dozen_sequences_in_ranges(window):
+    """12 sequences of 8 key/value heads are 96 workgroups when each walks a whole context: behind 2,000 to
+    3,000 keys the streaming kernel takes them in ranges that give 256 (here 1,152 keys), merged in order;
+    contexts at the ranges' edges, both forms of the kernel, the same bits from both."""
+    ops = _ops()
+    n_q, n_kv, d, page = 32, 8, 128, 16
+    longest = 3072
+    assert ops.attention_decode_streams(12, n_kv, d, n_q // n_kv, page, longest, window)
+    rng = np.random.default_rng(33 + window)
+    seq_lens = [2100, 3000, 1151, 1152, 1153, 1, 2304, 2305, 500, 3072, 17, 2700]
+    table, k, v = _paged_setup(rng, seq_lens, n_kv, d, page, torch.bfloat16)
+    t = len(seq_lens)
+    rows, positions, seq_of = list(range(t)), [n - 1 for n in seq_lens], list(range(t))
+    qkv = _t(rng.normal(size=(t, (n_q + 2 * n_kv) * d)).astype(np.float32))
+    inv_freq = _t(np.power(1e6, -(2.0 * np.arange(d // 2)) / d).astype(np.float32))
+    args = (_t(positions, torch.int32), _t(seq_of, torch.int32), _t(table, torch.int32))
+    ws = ops.attention_decode_workspace(t, n_q, d, longest, DEV)
+    k1, v1 = k.to(DEV), v.to(DEV)
+    q = ops.qk_norm_rope_kv_write(qkv, torch.empty(t, n_q * d, dtype=torch.bfloat16, device=DEV), k1, v1, *args, n_q, n_kv, d,
+                                  None, None, 0.0, inv_freq, d, write_kv=True)
+    want = ops.attention_decode(q, k1, v1, torch.zeros(t, n_q * d, dtype=torch.bfloat16, device=DEV), _t(rows, torch.int32),
+                                *args, n_q, n_kv, d, 1 / math.sqrt(d), window, longest, ws)
+    k2, v2 = k.to(DEV), v.to(DEV)
+    got = ops.attention_decode_fused(qkv, k2, v2, torch.zeros(t, n_q * d, dtype=torch.bfloat16, device=DEV),
+                                     _t(rows, torch.int32), *args, n_q, n_kv, d, None, None, 0.0, inv_freq, d, True,
+                                     1 / math.sqrt(d), window, longest, ws)
+    assert torch.equal(got, want) and torch.equal(k1, k2) and torch.equal(v1, v2)
+    ref = _attention_reference(q.cpu(), k1.cpu(), v1.cpu(), table, positions, seq_of, n_q, n_kv, d, page, window)
+    out = want.float().cpu().numpy().reshape(t, n_q, d)
+    for i in range(t):
+        assert _rel(out[i], ref[i]) < 1e-5, f"context of {seq_lens[i]} keys"
+
+
 @pytest.mark.parametrize("window", [0, 6000, 8000])
 def test_attention_decode_of_few_long_sequences(window):
     """Four sequences of several thousand keys: the streaming kernel takes them in ranges of 1,024 keys
