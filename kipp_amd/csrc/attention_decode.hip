@@ -1111,7 +1111,8 @@ static int launch_split(const bf16_t* q, bf16_t* k_cache, bf16_t* v_cache, bf16_
     const int extra = window > 0 ? 1 : 0;
     const int span_keys = (grid_splits - extra) * SPLIT;           // the caller counts splits of SPLIT keys
     // one rule for both forms, so that they cut alike and give the same bits
-    const int keys = split_keys_for(n_items, n_kv, span_keys, window, SPLIT_MAX);
+    // (head sizes above 128 stay with 256 keys: a longer split's keys and values would not fit the registers)
+    const int keys = split_keys_for(n_items, n_kv, span_keys, window, HEAD_DIM <= 128 ? SPLIT_MAX : SPLIT);
     const int splits = keys == SPLIT ? grid_splits : (span_keys + keys - 1) / keys + extra;
 #define KIPP_SPLIT_LAUNCH(KEYS)                                                                                       \
     hipLaunchKernelGGL((attention_decode_kernel<FUSED, KEYS>), dim3(n_items, n_kv, splits), dim3(THREADS), 0, stream, q, \
