@@ -2,21 +2,27 @@
 // Y[M, N] = X[M, K] . W[N, K]^T, bfloat16 operands, float32 accumulation on
 // v_mfma_f32_32x32x16_bf16, K a multiple of 32.
 //
-// A workgroup of 4 waves (2 x 2) owns a tile of outputs; a wave holds WM x WN accumulator tiles of
-// 32 x 32 (4 x 4: a workgroup tile of 256 x 256 and 256 accumulator registers a lane; also 4 x 2,
-// 2 x 4 and 2 x 2, chosen by the launcher so that the tiles of a product fill the 256 compute units
-// in whole rounds).  It walks K in steps of 32 columns.  The pieces of X and W of a step go from
+// A workgroup of 4 waves (2 x 2, one a SIMD) or of 8 (2 x 4, two a SIMD) owns a tile of outputs; a wave holds
+// WM x WN accumulator tiles of 32 x 32 (4 waves of 4 x 4, or 8 waves of 4 x 2: a workgroup tile of 256 x 256;
+// also smaller ones, chosen by the launcher so that the tiles of a product fill the 256 compute units in whole
+// rounds, or by the caller).  It walks K in steps of 32 columns.  The pieces of X and W of a step go from
 // global memory straight into LDS (global_load_lds_dwordx4: no registers, no waiting wave), four
 // steps deep.  In LDS four rows of a piece share 256 bytes, whose sixteen 16-byte slots are permuted
 // by the low bits of the group's index: the 16 lanes that read one operand column together then hit
 // sixteen different slots (no bank conflict is counted), and a wave's DMA instruction still writes
 // one contiguous KB.
 //
-// A wave is alone on its SIMD, so whatever holds up its instruction stream idles the matrix cores.
-// Every other instruction of the walk (the reads of the next operands out of LDS, the DMA of the
-// step four ahead) is therefore placed between two products, a few at a time, and the barrier of a
-// step falls between its two halves.  Measured with the DMA and the reads taken out: the walk
-// takes the same time, i.e. it is bound by the matrix cores' own rate.
+// With one wave a SIMD, whatever holds up its instruction stream idles the matrix cores.  Every other
+// instruction of the walk (the reads of the next operands out of LDS, the DMA of the steps ahead) is
+// therefore placed between two products, a few at a time, and the barrier of a step falls between its two
+// halves.  Measured (a build with -DPROBE_CLOCK counts the shader clock around the walk): 37.5 cycles a
+// product where the matrix core needs 32; 33.5 with the DMA taken out (-DABLATE_DMA=1): a wave that issues
+// a DMA instruction cannot issue its next product in time, which a second wave on the SIMD hides.  In the
+// run of a prefill the chip is at its power limit, and the time of a product is set by that, not by the
+// cycles: the cuts differ by a few per cent, and which is fastest for a shape is found by the clock.
+//
+// An output element is summed over K in the same order whatever the tile and the number of waves: cuts
+// with the same parts of K give the same bits.
 //
 // The result leaves through one of three ends:
 //   slabs   float32 [parts, M, N]: K is split over `parts` workgroups (grid.z) where the tiles
@@ -33,7 +39,6 @@
 #include "common.h"
 
 #define BK 32                                      // columns of a step
-#define THREADS 256
 #define CHUNKS (BK / 8)                            // 16-byte chunks of a row of a piece
 #define GROUP_ROWS (16 / CHUNKS)                   // rows that share 256 bytes of LDS
 #define INSTR_ROWS (4 * GROUP_ROWS)                // rows one DMA instruction of a wave brings (1 KB)
