@@ -231,6 +231,18 @@ def _trace(requests, steps):
     return lines
 
 
+def test_trace_run_says_why_it_refuses_a_step(model_folders, tmp_path):
+    """More tokens than --max-tokens gives pages for: one line on standard error, exit code 1, no `done`."""
+    folder = model_folders[("a", "float32")]
+    proc = subprocess.run([os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", "float32", "--out", str(tmp_path / "o"),
+                           "--max-tokens", "64"], input=json.dumps({"step": 0, "entries": [{"id": "x", "tokens": list(range(1, 131)), "want": [129]}],
+                                                                    "end": []}) + "\n",
+                          capture_output=True, text=True, timeout=120)
+    assert proc.returncode == 1 and "done" not in proc.stdout
+    assert "step 0 refused" in proc.stderr and "Traceback" not in proc.stderr
+
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("key,page,cut", [("b", 16, "mixed"), ("a", 16, "portions"), ("b", 8, "portions"), ("a", 32, "tail")])
 def test_trace_run(model_folders, tiny_configs, tmp_path, dtype, key, page, cut):
