@@ -109,7 +109,8 @@ class WrongKernelClass(RuntimeError):
 
 
 def measure_decode(engine, rt, ids, first, steps, warmup, repeats, weight_bytes, kv_per_token):
-    """`repeats` timings of `steps` decode steps (warm-up before the first); the median one is reported.
+    """`repeats` timings of `steps` decode steps (warm-up before the first), each from the same contexts (what a
+    repeat decoded is cut off again); the median one is reported.
     Raises WrongKernelClass unless every timed step was a replay of a recorded graph of our own kernels."""
     timings = []
     again = 0
@@ -119,6 +120,8 @@ def measure_decode(engine, rt, ids, first, steps, warmup, repeats, weight_bytes,
         library, generic, replays = rt.library_products, rt.generic_attention_launches, engine.graphs.replays
         w = warmup if rep == 0 else 0
         seconds = decode_run(engine, ids, first, steps, w)
+        for r, n in zip(ids, lengths):                   # every repeat, and every batch size, decodes behind the prompts alone
+            engine.cache.truncate(engine.cache.requests[r], n)
         if rt.library_products != library or rt.generic_attention_launches != generic:
             raise WrongKernelClass(f"decode batch {len(ids)}: {rt.library_products - library} products went to the library and "
                                    f"{rt.generic_attention_launches - generic} attention launches to the generic kernel")
