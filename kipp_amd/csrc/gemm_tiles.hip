@@ -82,9 +82,10 @@ __device__ __forceinline__ void wait_reads(u32x4 (&fa)[WM], u32x4 (&fb)[WN]) {
         asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(fa[0]), "+v"(fa[1]), "+v"(fb[0]), "+v"(fb[1]));
 }
 
-// steps of K that are in LDS or on their way there.  (Three for the smaller tiles, so that three workgroups of
-// the smallest share a compute unit instead of two, was measured and is slower: those tiles are bound by what
-// the DMA brings, not by the matrix cores, and a step less on its way is what they then lack.)
+// Steps of K that are in LDS or on their way there: four.  (Measurements only: -DSMALL_DEPTH=3 -DSMALL_WGS=2 gives
+// the tiles of half the size three steps and two workgroups a compute unit, i.e. two waves a SIMD from two
+// workgroups.  Measured and no faster: those tiles move half as many bytes again through the DMA for the same
+// products.  Two waves a SIMD on the full tile are the 8-wave cuts.)
 #ifndef SMALL_DEPTH
 #define SMALL_DEPTH 4
 #endif
