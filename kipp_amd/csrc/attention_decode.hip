@@ -42,6 +42,7 @@
 #endif
 
 #define SPLIT 256                              // keys of a split (the kernel that takes one a workgroup also has longer ones)
+#define SPLIT_MIN 192                          // the shortest (few sequences)
 #define SPLIT_MAX 320                          // the longest (the fused form has registers for no more with two workgroups a compute unit)
 #define WAVES 4
 #define THREADS (WAVES * KIPP_WAVE)
@@ -1090,13 +1091,20 @@ static int launch_ring(const bf16_t* q, bf16_t* k_cache, bf16_t* v_cache, bf16_t
 }
 #endif
 
-// The kernel that takes one split a workgroup, with splits of 256 keys, or of 320 where splits of 256
-// would be more workgroups than two a compute unit: workgroups beyond those that
+// The kernel that takes one split a workgroup, with splits of 256 keys, of 192 for one or two sequences, or of 320
+// where splits of 256 would be more workgroups than two a compute unit: workgroups beyond those that
 // fit at once run as a second round behind the first (measured at 8 sequences of 8 key/value heads: 576
 // workgroups for 2,050 keys cost 0.15 ms a step more than 512 for 2,040).  A function of the launch's shape.
-static int split_keys_for(int n_items, int n_kv, int span_keys, int window, int longest) {
+static int split_keys_for(int n_items, int n_kv, int span_keys, int window, int longest, int max_splits) {
     const long long pairs = (long long)n_items * n_kv, fit = 2 * 256;
     const int extra = window > 0 ? 1 : 0;
+    // few pairs: shorter splits, where they still are at most a workgroup a compute unit and the merge takes them
+    // at once (a workgroup's keys and values are what one compute unit has to draw: 96 KB instead of 128; one
+    // and two sequences of 8 heads at 2,100 keys: 1.3 % of the step)
+    {
+        const int n = (span_keys + SPLIT_MIN - 1) / SPLIT_MIN + extra;
+        if (longest > SPLIT && pairs * n <= 256 && n <= 16 && n <= max_splits) return SPLIT_MIN;
+    }
     if (pairs * ((span_keys + SPLIT - 1) / SPLIT + extra) <= fit) return SPLIT;
     for (int keys = SPLIT + 64; keys <= longest; keys += 64)
         if (pairs * ((span_keys + keys - 1) / keys + extra) <= fit) return keys;
@@ -1112,13 +1120,14 @@ static int launch_split(const bf16_t* q, bf16_t* k_cache, bf16_t* v_cache, bf16_
     const int span_keys = (grid_splits - extra) * SPLIT;           // the caller counts splits of SPLIT keys
     // one rule for both forms, so that they cut alike and give the same bits
     // (head sizes above 128 stay with 256 keys: a longer split's keys and values would not fit the registers)
-    const int keys = split_keys_for(n_items, n_kv, span_keys, window, HEAD_DIM <= 128 ? SPLIT_MAX : SPLIT);
+    const int keys = split_keys_for(n_items, n_kv, span_keys, window, HEAD_DIM <= 128 ? SPLIT_MAX : SPLIT, max_splits);
     const int splits = keys == SPLIT ? grid_splits : (span_keys + keys - 1) / keys + extra;
 #define KIPP_SPLIT_LAUNCH(KEYS)                                                                                       \
     hipLaunchKernelGGL((attention_decode_kernel<FUSED, KEYS>), dim3(n_items, n_kv, splits), dim3(THREADS), 0, stream, q, \
                        k_cache, v_cache, out, part_acc, part_ml, rows, positions, seq_of_token, block_table, max_blocks, \
                        n_q, n_kv, page, scale_log2e, window, max_splits, pj)
     switch (keys) {
+        case SPLIT_MIN: KIPP_SPLIT_LAUNCH(SPLIT_MIN); break;
         case 256: KIPP_SPLIT_LAUNCH(256); break;
         case 320: KIPP_SPLIT_LAUNCH(320); break;
         default: return -1;
@@ -1132,6 +1141,8 @@ static int launch_split(const bf16_t* q, bf16_t* k_cache, bf16_t* v_cache, bf16_
 extern "C" {
 
 int kipp_attention_decode_split() { return SPLIT; }
+// The shortest split a launch may be cut into: what the workspace has to hold partial results for.
+int kipp_attention_decode_split_min() { return SPLIT_MIN; }
 
 // 1 if a launch of this shape goes to the kernel that streams through LDS (its fused form has no limit
 // on the rows or the context).

@@ -286,6 +286,7 @@ def attention_fast_ok(n_q: int, n_kv: int, page: int, max_blocks: int = 0) -> bo
 
 
 DECODE_SPLIT = 256      # keys per workgroup of the decode kernel (checked against the library at load)
+DECODE_SPLIT_MIN = 192  # ... and of its shortest splits (few sequences), which size the workspace
 PREFILL_ROWS = 128      # query rows per workgroup of the prefill kernel (64 or 32 where that fills the GPU better)
 COMPUTE_UNITS = 256     # of the MI355X
 PREFILL_MIN_CUT = 512   # fewest keys of a cut of the prefill kernel's keys (below, the merge costs more than the cut gains)
@@ -400,7 +401,7 @@ def attention_decode_fused(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: to
 
 
 def attention_decode_workspace(n_items: int, n_q: int, head_dim: int, max_context: int, device) -> tuple:
-    max_splits = (max_context + DECODE_SPLIT - 1) // DECODE_SPLIT + 1
+    max_splits = (max_context + DECODE_SPLIT_MIN - 1) // DECODE_SPLIT_MIN + 1       # the shortest splits a launch may take
     return (torch.empty(n_items * n_q * max_splits * head_dim, dtype=torch.float32, device=device),
             torch.empty(n_items * n_q * max_splits * 2, dtype=torch.float32, device=device))
 
