@@ -460,6 +460,7 @@ def attention_prefill_workspace(rows: int, n_q: int, head_dim: int, max_splits: 
 SKINNY_MAX_ROWS = 64     # rows the few-rows kernel takes
 SKINNY_BEST_ROWS = 8     # ... and rows up to which it is the faster one (each wave reads its rows of x itself; beyond, x staged in LDS wins)
 ROWS_MAX_ROWS = 256      # rows of the kernel that stages x through LDS
+ROWS_BEST_ROWS = 192     # beyond these the product built for hundreds of rows is faster where it takes the shape (measured)
 
 
 def gemm_rows_ok(m: int, k: int) -> bool:

@@ -131,7 +131,11 @@ class DecodeGraph:
             # kernels keep); if nothing in it went to a library, the same launches are then
             # recorded for the steps to come
             before = engine.rt.library_products
-            logits = engine.model.forward(self.batch, engine.cache)
+            engine.rt.for_a_graph = True        # the products of these rows keep to kernels that can be recorded
+            try:
+                logits = engine.model.forward(self.batch, engine.cache)
+            finally:
+                engine.rt.for_a_graph = False
             self.eager_runs += 1
             if engine.rt.library_products != before or self.eager_runs < 2:
                 return logits[:len(entries)]
@@ -141,10 +145,12 @@ class DecodeGraph:
             # off until the recording ends (it runs once before, inside torch.cuda.graph)
             was_enabled = gc.isenabled()
             gc.disable()
+            engine.rt.for_a_graph = True
             try:
                 with torch.cuda.graph(graph):
                     self.logits = engine.model.forward(self.batch, engine.cache)
             finally:
+                engine.rt.for_a_graph = False
                 if was_enabled:
                     gc.enable()
             self.graph = graph

@@ -48,7 +48,7 @@ class GatedMLP:
         rows, inner = x.shape[0], self.spec.intermediate_size
         act = rt.empty((rows, inner), rt.act_dtype)
         w = self.w_gate_up
-        ours = w.dtype == x.dtype == torch.bfloat16 and rt.ops.gemm_rows_ok(rows, x.shape[1])
+        ours = w.dtype == x.dtype == torch.bfloat16 and rt.streams(rows, x.shape[1], 2 * inner)
         if ours and rows <= rt.ops.SKINNY_BEST_ROWS:
             # both products and the activation in one kernel (and the norm's scale, if it was left to us)
             scaled = isinstance(x, ScaledRows)
@@ -59,7 +59,7 @@ class GatedMLP:
         if ours and w.pairs:
             # streamed from the paired tiles: the columns come out gate tile by gate tile
             rt.ops.swiglu(rt.ops.gemm_rows(x, w.rows, max_parts=12, tiles=w.tiles, pairs=True), act, pairs=True)
-        elif w.dtype == x.dtype == torch.bfloat16 and rows > rt.ops.ROWS_MAX_ROWS:
+        elif w.dtype == x.dtype == torch.bfloat16 and not ours:
             act = rt.gated(x, w, act)       # many rows: both products and the activation, by whichever way is faster
         else:
             rt.ops.swiglu(rt.linear(x, w, slabs=True), act)

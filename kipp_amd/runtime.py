@@ -109,14 +109,15 @@ class Runtime:
         self.library_products = 0   # calls that went to the library (they stay out of HIP graphs)
         self.generic_attention_launches = 0   # bfloat16 attention that fell to the generic kernel (geometry the matrix-core kernels refuse)
         self.fuse_norms = True      # few rows: residual add and norm ride on the products around them
-        # products of more than 256 rows: "auto" (the default): the fastest of our own matrix-core kernel's cuts and
+        # products of more than about 200 rows: "auto" (the default): the fastest of our own matrix-core kernel's cuts and
         # the library's product, timed once in a process at a shape's first use (another process may choose
         # otherwise, and its results then differ in their last bits); True: our kernel, in the fastest of the cuts
         # that give the planned cut's bits (the same bits in every process); False: always the library's.
         # KIPP_AMD_PRODUCTS=own|auto|library sets it from outside.
         self.own_prompt_products = {"own": True, "auto": "auto", "library": False}.get(os.environ.get("KIPP_AMD_PRODUCTS", "auto"), "auto")
         self.prompt_product_choices = {}     # shape -> "library", "plan" (our kernel, cut as planned) or a forced cut of ours
-        self.tile_products = 0      # products of more than 256 rows that ran on our own kernel
+        self.tile_products = 0      # products of many rows that ran on our own kernel
+        self.for_a_graph = False    # set around a step of single tokens that is, or is to be, recorded as a HIP graph
         torch.backends.cuda.matmul.allow_tf32 = False
 
     # -- placement -----------------------------------------------------------
@@ -179,9 +180,14 @@ class Runtime:
         return ScaledRows(rows_out, sumsq, (w.shape[0] + 15) // 16, eps)
 
     # -- products of prompt portions ------------------------------------------------------------
+    def streams(self, m: int, k: int, n: int) -> bool:
+        """Whether a bfloat16 product of m rows takes the kernels that stream the weight once (few rows, or a
+        shape the product for many rows does not take)."""
+        return self.ops.gemm_rows_ok(m, k) and (m <= self.ops.ROWS_BEST_ROWS or not self.ops.gemm_tiles_ok(m, k, n))
+
     @staticmethod
     def _rows_class(m: int) -> int:
-        """Rows of a prompt product, in classes of a factor of two (257-512, 513-1024, ...): one decision a class."""
+        """Rows of a prompt product, in classes of a factor of two (193-256, 257-512, 513-1024, ...): one decision a class."""
         return 1 << (max(m, 1) - 1).bit_length()
 
     # Cuts of our kernel that are timed beside the planned one: 100 x (wave tile rows / 32) + 10 x (wave tile
@@ -202,6 +208,10 @@ class Runtime:
         `own_prompt_products` True (the default): only those are timed, so the choice changes how long a
         product takes and never what it gives; "auto": all of them (the library's product and other parts of K
         round differently: two runs of one program may then differ in their last bits); False: the library's."""
+        if self.for_a_graph:
+            # a step that is to be recorded keeps to our own kernels (the library's calls stay out of HIP graphs)
+            key = key + ("for a graph",)
+            ways = {name: run for name, run in ways.items() if name != "library"}
         choice = self.prompt_product_choices.get(key)
         if choice is None:
             choice = self._choices_of_process.get((self.own_prompt_products, key))      # every engine of a process decides alike
@@ -209,7 +219,7 @@ class Runtime:
             self.prompt_product_choices[key] = choice
         if choice is None:
             if self.own_prompt_products is False:
-                choice = "library"
+                choice = "library" if "library" in ways else "plan"
             else:
                 # The chip is at its power limit while products follow each other, and a product that wins from
                 # a standing start need not win then: every candidate runs a few times first, then they are
@@ -307,15 +317,15 @@ class Runtime:
             return self.ops.gemm_f32(x, w, self.empty((m, n), torch.float32))
         if x.dtype != torch.bfloat16:
             x = self.ops.cast(x, self.empty(x.shape, torch.bfloat16))
-        if self.ops.gemm_rows_ok(m, x.shape[1]):
-            # up to 256 rows: our own kernels stream the weight once
+        if self.streams(m, x.shape[1], n):
+            # up to about 200 rows: our own kernels stream the weight once
             most = 0 if slabs is False else (None if slabs is True else int(slabs))
             if m <= self.ops.SKINNY_BEST_ROWS:
                 y = self.ops.gemm_skinny(x, w, max_parts=1 if most == 0 else (most or 8), tiles=tiles, row_scale=row_scale)
             else:
                 y = self.ops.gemm_rows(x, w, max_parts=1 if most == 0 else (most or 12), tiles=tiles)
             return y if y.shape[0] > 1 else y[0]
-        # more than 256 rows (prompt portions): our matrix-core kernel, or the library's product
+        # more rows (prompt portions): our matrix-core kernel, or the library's product
         if self.ops.gemm_tiles_ok(m, x.shape[1], n):
             most = 1 if slabs is False else (4 if slabs is True else max(1, min(4, int(slabs))))
 

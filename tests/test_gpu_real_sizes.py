@@ -189,7 +189,7 @@ def test_a_batch_whose_size_changes_replays_one_graph(long_folder, dtype):
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_many_decoding_rows_beside_prompt_portions(long_folder, dtype):
     """Steps that hold 20 to 34 single tokens AND two or three prompt portions of changing size (2 to 290
-    tokens; a few steps pass 256 rows and take the library's product), at head size 128: in bfloat16 one
+    tokens; a few steps pass 192 rows and take the products for many rows), at head size 128: in bfloat16 one
     forward pass then runs the rotary kernel, the prefill attention and the split decode attention side
     by side.  The pool holds exactly what live requests need at the peak, so pages are used again while
     others are still read.  Every row of every request against the plain implementation."""
@@ -246,8 +246,8 @@ def test_a_long_position_limit_keeps_the_matrix_core_kernels(real_folder, real_r
 
 @pytest.mark.parametrize("ours", [True, False, "auto"])
 def test_prompt_portions_of_many_rows_by_either_product(real_folder, real_reference, ours):
-    """Portions of more than 256 rows at the benchmark's layer sizes, with every product of theirs on our
-    matrix-core kernel (SwiGLU in its end, K split into slabs that the norms add; the fastest of the cuts that
+    """Portions of 230 and 390 rows (more than the streaming products are best at) at the benchmark's layer
+    sizes, with every product of theirs on our matrix-core kernel (SwiGLU in its end, K split into slabs that the norms add; the fastest of the cuts that
     give the planned cut's bits), then on the library's, then left to the clock among all of them (the
     default): against the plain implementation, every row.  Our kernel alone gives the same bits on a second
     engine, whatever its clock chose."""
@@ -263,8 +263,8 @@ def test_prompt_portions_of_many_rows_by_either_product(real_folder, real_refere
         rt = Runtime("bfloat16")
         rt.own_prompt_products = ours
         engine = Engine(load_model(real_folder, rt), page_size=16, max_tokens=1024, max_requests=2, share_prefixes=False)
-        got = [engine.step([StepEntry("a", toks[:300], list(range(300)))]),
-               engine.step([StepEntry("a", toks[300:], list(range(320)))])]
+        got = [engine.step([StepEntry("a", toks[:230], list(range(230)))]),
+               engine.step([StepEntry("a", toks[230:], list(range(390)))])]
         return rt, torch.cat(got).float().cpu().numpy()
     rt, got = run()
     H.assert_close(got, ref, H.NMSE_BF16["real"], f"many rows, ours {ours}")
