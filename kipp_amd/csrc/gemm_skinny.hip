@@ -370,7 +370,11 @@ static int launch_kw(const bf16_t* X, const bf16_t* W, float* Y, bf16_t* act, in
 #define KIPP_SK(MT, D) \
     hipLaunchKernelGGL((gemm_skinny_kernel<MT, SWIGLU, KW, D, TILED>), grid, block, 0, stream, X, W, Y, act, M, N, K, rs, an)
     switch (mt) {
-        case 1: KIPP_SK(1, 8); break;
+        case 1:
+            // fewer workgroups than compute units: what is in flight is what the busy ones ask for, so they ask for twice as much
+            if (grid.x * grid.y < 256 && K / 32 / 16 >= KW) KIPP_SK(1, 16);
+            else KIPP_SK(1, 8);
+            break;
         case 2: KIPP_SK(2, 8); break;
         case 3: KIPP_SK(3, 4); break;
         case 4: KIPP_SK(4, 4); break;
