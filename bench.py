@@ -220,7 +220,7 @@ def main():
     ap.add_argument("--repeats", type=int, default=5, help="times the K timed steps are run; the median is reported")
     ap.add_argument("--no-long", action="store_true", help="leave out the points at longer contexts")
     ap.add_argument("--products", choices=["default", "own", "auto", "library"], default="default",
-                    help="products of more than 256 rows: the runtime's default, our kernel only, the fastest of ours and the library's, the library's")
+                    help="products of many rows (prompt portions): the runtime's default, our kernel only, the fastest of ours and the library's, the library's")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -318,7 +318,7 @@ def main():
     main_r = results[args.batch]
     achieved = main_r["bytes"] / (main_r["ms"] / 1e3) / 1e9
     line = {
-        "metric": "decode tok/s at batch 8 (Qwen3-4B-shaped, bf16, random weights)",
+        "metric": f"decode tok/s at batch {args.batch} ({args.shape.replace('qwen3-', 'Qwen3-').upper().replace('QWEN3', 'Qwen3')}-shaped, bf16, random weights)",
         "value": round(main_r["tok_s"], 1), "unit": "tok/s", "n_gpus": 1, "steps": main_r["steps"],
         "warmup": main_r["warmup"], "ms_per_step": round(main_r["ms"], 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
