@@ -15,9 +15,19 @@
 //            16th key; products in float32 FMA, summed over the groups in LDS.
 //
 // Split boundaries are multiples of SPLIT in absolute key index, and the merge
-// (attention_decode_reduce_kernel) adds the splits in index order, so the result
-// for a token does not depend on the batch it is in.  A sequence that needs
-// one split only is written normalised at once.
+// adds the splits in index order, so the result for a token does not depend on
+// the batch it is in.  A sequence that needs one split only is written
+// normalised at once.  The merge is done by whichever workgroup of a (token,
+// key/value head) finishes last: every workgroup writes its partial result
+// through to memory (stores of device scope: the dies' L2 caches do not see each
+// other's lines), waits until the stores have arrived, and adds one to the
+// head's count with an atomic of device scope; the one that brings the count to
+// the number of splits reads all partial results from memory (loads of device
+// scope), merges them and sets the count back to zero.  Nobody waits for
+// anybody, no fence is needed (a fence of device scope writes a die's whole L2
+// back: 40 us), and the sums are those of attention_decode_reduce_kernel in the
+// same order, which a caller without the counts still gets as a second launch
+// (4.7 us a layer; merged here a decode step at batch 8 is 1 % shorter).
 //
 // FUSED: the kernel starts from the output of the QKV projection instead of from
 // finished queries.  Each workgroup norms and rotates the GROUP queries of its
@@ -78,13 +88,101 @@ struct Projected {
     int write_kv;            // 0: the cache is another layer's, keys and values are already there
 };
 
+// Values that another workgroup of the same launch reads: written through to memory and read from there (the
+// dies' L2 caches do not see each other's lines).  A store is known to have arrived once the wave's count of
+// outstanding memory operations is back to zero.
+__device__ __forceinline__ void store_through(float* p, float v) {
+    __hip_atomic_store((unsigned*)p, __float_as_uint(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float load_through(const float* p) {
+    return __uint_as_float(__hip_atomic_load((const unsigned*)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+}
+
+// The merge of attention_decode_reduce_kernel (the same sums in the same order) by the workgroup that finished
+// last among the splits of a (token, key/value head): element `dcol` of head `head`.
+__device__ __forceinline__ float merge_splits_here(const float* part_acc, const float* part_ml, size_t slot0, int n_splits, int dcol) {
+    constexpr int AT_ONCE = 16;
+    float m_s[AT_ONCE], l_s[AT_ONCE], a_s[AT_ONCE];
+    // the first 16 splits are asked for together, whatever their number (beyond it: the last again, dropped below)
+#pragma unroll
+    for (int i = 0; i < AT_ONCE; ++i) {
+        const size_t slot = slot0 + min(i, n_splits - 1);
+        m_s[i] = load_through(part_ml + slot * 2);
+        l_s[i] = load_through(part_ml + slot * 2 + 1);
+        a_s[i] = load_through(part_acc + slot * HEAD_DIM + dcol);
+    }
+    float m = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < AT_ONCE; ++i) m = fmaxf(m, i < n_splits ? m_s[i] : -INFINITY);
+    for (int s = AT_ONCE; s < n_splits; ++s) m = fmaxf(m, load_through(part_ml + (slot0 + s) * 2));
+    float denom = 0.0f, a = 0.0f;
+#pragma unroll
+    for (int i = 0; i < AT_ONCE; ++i) {
+        if (i < n_splits) {
+            const float w = exp2f(m_s[i] - m);
+            denom += l_s[i] * w;
+            a += a_s[i] * w;
+        }
+    }
+    for (int s = AT_ONCE; s < n_splits; ++s) {
+        const float w = exp2f(load_through(part_ml + (slot0 + s) * 2) - m);
+        denom += load_through(part_ml + (slot0 + s) * 2 + 1) * w;
+        a += load_through(part_acc + (slot0 + s) * HEAD_DIM + dcol) * w;
+    }
+    return a / denom;
+}
+
+// One element of a split's partial result.  With `arrivals` the splits are merged inside this launch.
+__device__ __forceinline__ void put_partial(const unsigned* arrivals, float* part_acc, float* part_ml, size_t slot, int dcol,
+                                            float a, float m, float l) {
+    if (arrivals != nullptr) {
+        store_through(part_acc + slot * HEAD_DIM + dcol, a);
+        if (dcol == 0) {
+            store_through(part_ml + slot * 2, m);
+            store_through(part_ml + slot * 2 + 1, l);
+        }
+    } else {
+        part_acc[slot * HEAD_DIM + dcol] = a;
+        if (dcol == 0) {
+            part_ml[slot * 2] = m;
+            part_ml[slot * 2 + 1] = l;
+        }
+    }
+}
+
+// The end of a workgroup that has put one of several splits of (token `item`, key/value head `kvh`): it counts
+// itself once what it wrote has arrived, and the one that counts last merges the splits, in split order.  Nobody
+// waits for anybody.  Called by all threads of the workgroup.
+__device__ __forceinline__ void merge_by_the_last(unsigned* arrivals, const float* part_acc, const float* part_ml, bf16_t* out,
+                                                  int item, int row, int kvh, int n_q, int n_kv, int max_splits, int n_splits) {
+    __shared__ int s_last;
+    const int tid = threadIdx.x;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (tid == 0) {
+        unsigned* count = arrivals + (size_t)item * n_kv + kvh;
+        const unsigned before = __hip_atomic_fetch_add(count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const int last = before + 1u == (unsigned)n_splits;
+        if (last) __hip_atomic_store(count, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // as the next launch expects it
+        s_last = last;
+    }
+    __syncthreads();
+    if (!s_last) return;
+    for (int idx = tid; idx < GROUP * HEAD_DIM; idx += THREADS) {
+        const int g = idx / HEAD_DIM, dcol = idx % HEAD_DIM;
+        const int head = kvh * GROUP + g;
+        const size_t slot0 = ((size_t)item * n_q + head) * max_splits;
+        out[((size_t)row * n_q + head) * HEAD_DIM + dcol] = f32_to_bf16(merge_splits_here(part_acc, part_ml, slot0, n_splits, dcol));
+    }
+}
+
 template <bool FUSED, int SPLIT_T>
 __global__ void __launch_bounds__(THREADS) attention_decode_kernel(
     const bf16_t* __restrict__ q, bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache,
     bf16_t* __restrict__ out, float* __restrict__ part_acc, float* __restrict__ part_ml,
     const int32_t* __restrict__ rows, const int32_t* __restrict__ positions, const int32_t* __restrict__ seq_of_token,
     const int32_t* __restrict__ block_table, int max_blocks, int n_q, int n_kv, int page, float scale_log2e,
-    int window, int max_splits, Projected pj) {
+    int window, int max_splits, Projected pj, unsigned* arrivals) {
     static_assert(SPLIT_T % (16 * WAVES) == 0 && SPLIT_T <= 2 * THREADS, "whole blocks of 16 keys a wave; at most two pages a thread");
     constexpr int BPW = SPLIT_T / 16 / WAVES;         // 16-key blocks a wave scores
     constexpr int KPG = SPLIT_T / 16;                 // keys a lane group multiplies with values
@@ -379,14 +477,11 @@ __global__ void __launch_bounds__(THREADS) attention_decode_kernel(
         if (n_splits == 1) {
             out[((size_t)row * n_q + head) * HEAD_DIM + dcol] = f32_to_bf16(a / s_l[g]);
         } else {
-            const size_t slot = ((size_t)blockIdx.x * n_q + head) * max_splits + blockIdx.z;
-            part_acc[slot * HEAD_DIM + dcol] = a;
-            if (dcol == 0) {
-                part_ml[slot * 2] = s_m[g];
-                part_ml[slot * 2 + 1] = s_l[g];
-            }
+            put_partial(arrivals, part_acc, part_ml, ((size_t)blockIdx.x * n_q + head) * max_splits + blockIdx.z, dcol, a, s_m[g], s_l[g]);
         }
     }
+    if (arrivals != nullptr && n_splits > 1)
+        merge_by_the_last(arrivals, part_acc, part_ml, out, blockIdx.x, row, kvh, n_q, n_kv, max_splits, n_splits);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -410,7 +505,7 @@ __global__ void __launch_bounds__(THREADS) attention_decode_stream_kernel(
     bf16_t* __restrict__ out, float* __restrict__ part_acc, float* __restrict__ part_ml,
     const int32_t* __restrict__ rows, const int32_t* __restrict__ positions, const int32_t* __restrict__ seq_of_token,
     const int32_t* __restrict__ block_table, int max_blocks, int n_q, int n_kv, int page, float scale_log2e,
-    int window, int max_splits) {
+    int window, int max_splits, unsigned* arrivals) {
     __shared__ float s_scores[GROUP][SUB + 4];
     __shared__ float s_red[WAVES][GROUP][HEAD_DIM];
     __shared__ float s_m[GROUP], s_l[GROUP], s_alpha[GROUP];
@@ -604,14 +699,11 @@ __global__ void __launch_bounds__(THREADS) attention_decode_stream_kernel(
         if (n_splits == 1) {
             out[((size_t)row * n_q + head) * HEAD_DIM + dcol] = f32_to_bf16(a / s_l[g]);
         } else {
-            const size_t slot = ((size_t)blockIdx.z * n_q + head) * max_splits + blockIdx.x;
-            part_acc[slot * HEAD_DIM + dcol] = a;
-            if (dcol == 0) {
-                part_ml[slot * 2] = s_m[g];
-                part_ml[slot * 2 + 1] = s_l[g];
-            }
+            put_partial(arrivals, part_acc, part_ml, ((size_t)blockIdx.z * n_q + head) * max_splits + blockIdx.x, dcol, a, s_m[g], s_l[g]);
         }
     }
+    if (arrivals != nullptr && n_splits > 1)
+        merge_by_the_last(arrivals, part_acc, part_ml, out, blockIdx.z, row, kvh, n_q, n_kv, max_splits, n_splits);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -678,7 +770,7 @@ __global__ void __launch_bounds__(THREADS, 2) attention_decode_ring_kernel(
     bf16_t* __restrict__ out, float* __restrict__ part_acc, float* __restrict__ part_ml,
     const int32_t* __restrict__ rows, const int32_t* __restrict__ positions, const int32_t* __restrict__ seq_of_token,
     const int32_t* __restrict__ block_table, int max_blocks, int n_q, int n_kv, int page, float scale_log2e,
-    int window, int max_splits, int range, Projected pj) {
+    int window, int max_splits, int range, Projected pj, unsigned* arrivals) {
     extern __shared__ __attribute__((aligned(1024))) unsigned char ring[];
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -924,14 +1016,11 @@ __global__ void __launch_bounds__(THREADS, 2) attention_decode_ring_kernel(
         if (n_splits == 1) {
             out[((size_t)row * n_q + head) * HEAD_DIM + dcol] = f32_to_bf16(a / l);
         } else {
-            const size_t slot = ((size_t)blockIdx.x * n_q + head) * max_splits + blockIdx.z;
-            part_acc[slot * HEAD_DIM + dcol] = a;
-            if (dcol == 0) {
-                part_ml[slot * 2] = m;
-                part_ml[slot * 2 + 1] = l;
-            }
+            put_partial(arrivals, part_acc, part_ml, ((size_t)blockIdx.x * n_q + head) * max_splits + blockIdx.z, dcol, a, m, l);
         }
     }
+    if (arrivals != nullptr && n_splits > 1)
+        merge_by_the_last(arrivals, part_acc, part_ml, out, blockIdx.x, row, kvh, n_q, n_kv, max_splits, n_splits);
 }
 #endif  // RING_OK
 
@@ -1064,8 +1153,8 @@ template <bool FUSED>
 static int launch_ring(const bf16_t* q, bf16_t* k_cache, bf16_t* v_cache, bf16_t* out, float* part_acc, float* part_ml,
                        const int32_t* rows, const int32_t* positions, const int32_t* seq_of_token,
                        const int32_t* block_table, int max_blocks, int n_items, int n_q, int n_kv, int page,
-                       float scale_log2e, int window, int grid_splits, int max_splits, Projected pj, hipStream_t stream,
-                       int* rc) {
+                       float scale_log2e, int window, int grid_splits, int max_splits, Projected pj, unsigned* arrivals,
+                       hipStream_t stream, int* rc) {
     const int range = ring_range(n_items, n_kv, page, grid_splits);
     if (range == 0) return 0;
     const int lds = RING_BYTES + (FUSED ? (GROUP + 2) * HEAD_DIM * 2 : 0);
@@ -1083,9 +1172,9 @@ static int launch_ring(const bf16_t* q, bf16_t* k_cache, bf16_t* v_cache, bf16_t
     if (ring_splits > max_splits) return 0;
     hipLaunchKernelGGL(attention_decode_ring_kernel<FUSED>, dim3(n_items, n_kv, ring_splits), dim3(THREADS), lds, stream, q,
                        k_cache, v_cache, out, part_acc, part_ml, rows, positions, seq_of_token, block_table, max_blocks, n_q,
-                       n_kv, page, scale_log2e, window, max_splits, range, pj);
+                       n_kv, page, scale_log2e, window, max_splits, range, pj, arrivals);
     *rc = KIPP_LAUNCH_CHECK();
-    if (*rc != 0 || ring_splits == 1) return 1;
+    if (*rc != 0 || ring_splits == 1 || arrivals != nullptr) return 1;
     *rc = launch_reduce(part_acc, part_ml, (bf16_t*)out, rows, positions, n_items, n_q, window, max_splits, range, ring_splits, stream);
     return 1;
 }
@@ -1115,7 +1204,8 @@ template <bool FUSED>
 static int launch_split(const bf16_t* q, bf16_t* k_cache, bf16_t* v_cache, bf16_t* out, float* part_acc, float* part_ml,
                         const int32_t* rows, const int32_t* positions, const int32_t* seq_of_token,
                         const int32_t* block_table, int max_blocks, int n_items, int n_q, int n_kv, int page,
-                        float scale_log2e, int window, int grid_splits, int max_splits, Projected pj, hipStream_t stream) {
+                        float scale_log2e, int window, int grid_splits, int max_splits, Projected pj, unsigned* arrivals,
+                        hipStream_t stream) {
     const int extra = window > 0 ? 1 : 0;
     const int span_keys = (grid_splits - extra) * SPLIT;           // the caller counts splits of SPLIT keys
     // one rule for both forms, so that they cut alike and give the same bits
@@ -1125,7 +1215,7 @@ static int launch_split(const bf16_t* q, bf16_t* k_cache, bf16_t* v_cache, bf16_
 #define KIPP_SPLIT_LAUNCH(KEYS)                                                                                       \
     hipLaunchKernelGGL((attention_decode_kernel<FUSED, KEYS>), dim3(n_items, n_kv, splits), dim3(THREADS), 0, stream, q, \
                        k_cache, v_cache, out, part_acc, part_ml, rows, positions, seq_of_token, block_table, max_blocks, \
-                       n_q, n_kv, page, scale_log2e, window, max_splits, pj)
+                       n_q, n_kv, page, scale_log2e, window, max_splits, pj, arrivals)
     switch (keys) {
         case SPLIT_MIN: KIPP_SPLIT_LAUNCH(SPLIT_MIN); break;
         case 256: KIPP_SPLIT_LAUNCH(256); break;
@@ -1134,7 +1224,7 @@ static int launch_split(const bf16_t* q, bf16_t* k_cache, bf16_t* v_cache, bf16_
     }
 #undef KIPP_SPLIT_LAUNCH
     int rc = KIPP_LAUNCH_CHECK();
-    if (rc != 0 || splits == 1) return rc;
+    if (rc != 0 || splits == 1 || arrivals != nullptr) return rc;      // with `arrivals` the last workgroup of a head has merged
     return launch_reduce(part_acc, part_ml, out, rows, positions, n_items, n_q, window, max_splits, keys, splits, stream);
 }
 
@@ -1161,7 +1251,8 @@ int kipp_attention_decode_ring_takes(int n_items, int n_kv, int page, int grid_s
 int kipp_attention_decode(const void* q, const void* k_cache, const void* v_cache, void* out, float* part_acc,
                           float* part_ml, const int32_t* rows, const int32_t* positions, const int32_t* seq_of_token,
                           const int32_t* block_table, int max_blocks, int n_items, int n_q, int n_kv, int head_dim,
-                          int page, float scale, int window, int grid_splits, int max_splits, hipStream_t stream) {
+                          int page, float scale, int window, int grid_splits, int max_splits, int32_t* arrivals,
+                          hipStream_t stream) {
     if (n_items <= 0) return 0;
     if (head_dim != HEAD_DIM || n_kv <= 0 || n_q != n_kv * GROUP) return -1;
     if (grid_splits <= 0 || grid_splits > max_splits) return -3;
@@ -1172,7 +1263,7 @@ int kipp_attention_decode(const void* q, const void* k_cache, const void* v_cach
         int rc = 0;
         if (launch_ring<false>((const bf16_t*)q, (bf16_t*)k_cache, (bf16_t*)v_cache, (bf16_t*)out, part_acc, part_ml, rows,
                                positions, seq_of_token, block_table, max_blocks, n_items, n_q, n_kv, page, scale_log2e, window,
-                               grid_splits, max_splits, Projected{}, stream, &rc))
+                               grid_splits, max_splits, Projected{}, (unsigned*)arrivals, stream, &rc))
             return rc;
     }
 #endif
@@ -1183,14 +1274,14 @@ int kipp_attention_decode(const void* q, const void* k_cache, const void* v_cach
         hipLaunchKernelGGL(attention_decode_stream_kernel, dim3(big_splits, n_kv, n_items), dim3(THREADS), 0, stream,
                            (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, part_acc,
                            part_ml, rows, positions, seq_of_token, block_table, max_blocks, n_q, n_kv, page, scale_log2e,
-                           window, max_splits);
+                           window, max_splits, (unsigned*)arrivals);
         int rc = KIPP_LAUNCH_CHECK();
-        if (rc != 0 || big_splits == 1) return rc;
+        if (rc != 0 || big_splits == 1 || arrivals != nullptr) return rc;
         return launch_reduce(part_acc, part_ml, (bf16_t*)out, rows, positions, n_items, n_q, window, max_splits, BIG, big_splits, stream);
     }
     return launch_split<false>((const bf16_t*)q, (bf16_t*)k_cache, (bf16_t*)v_cache, (bf16_t*)out, part_acc, part_ml, rows, positions,
                                seq_of_token, block_table, max_blocks, n_items, n_q, n_kv, page, scale_log2e, window, grid_splits,
-                               max_splits, Projected{}, stream);
+                               max_splits, Projected{}, (unsigned*)arrivals, stream);
 }
 
 // 1 if this build has the fused kernel (head sizes that are multiples of 128).
@@ -1207,7 +1298,7 @@ int kipp_attention_decode_fused(const float* qkv, int parts, int n_tokens, const
                                 float* part_acc, float* part_ml, const int32_t* rows, const int32_t* positions,
                                 const int32_t* seq_of_token, const int32_t* block_table, int max_blocks, int n_items,
                                 int n_q, int n_kv, int head_dim, int page, float scale, int window, int grid_splits,
-                                int max_splits, hipStream_t stream) {
+                                int max_splits, int32_t* arrivals, hipStream_t stream) {
 #if FUSED_OK
     if (n_items <= 0) return 0;
     if (head_dim != HEAD_DIM || n_kv <= 0 || n_q != n_kv * GROUP || parts <= 0 || parts > MAX_SLABS) return -1;
@@ -1221,13 +1312,13 @@ int kipp_attention_decode_fused(const float* qkv, int parts, int n_tokens, const
         int rc = 0;
         if (launch_ring<true>((const bf16_t*)nullptr, (bf16_t*)k_cache, (bf16_t*)v_cache, (bf16_t*)out, part_acc, part_ml, rows,
                               positions, seq_of_token, block_table, max_blocks, n_items, n_q, n_kv, page, scale_log2e, window,
-                              grid_splits, max_splits, pj, stream, &rc))
+                              grid_splits, max_splits, pj, (unsigned*)arrivals, stream, &rc))
             return rc;
     }
 #endif
     return launch_split<true>((const bf16_t*)nullptr, (bf16_t*)k_cache, (bf16_t*)v_cache, (bf16_t*)out, part_acc, part_ml, rows,
                               positions, seq_of_token, block_table, max_blocks, n_items, n_q, n_kv, page, scale_log2e, window,
-                              grid_splits, max_splits, pj, stream);
+                              grid_splits, max_splits, pj, (unsigned*)arrivals, stream);
 #else
     return -5;
 #endif

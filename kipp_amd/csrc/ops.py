@@ -298,7 +298,8 @@ def attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
                      workspace: tuple, grid_splits: Optional[int] = None) -> torch.Tensor:
     """Attention of single query tokens (batch rows `rows`) over their pages.
     `max_context`: the longest context among them (sizes the grid); `workspace`:
-    (part_acc, part_ml) float32 buffers from `attention_decode_workspace`."""
+    (part_acc, part_ml, arrivals) from `attention_decode_workspace` (without `arrivals`, or with None for it,
+    the splits are merged by a launch of its own instead of by the last workgroup of every head)."""
     _dev(q, k_cache, v_cache, out, rows, positions, seq_of_token, block_table, *workspace)
     for t, name in ((rows, "rows"), (positions, "positions"), (seq_of_token, "seq_of_token"), (block_table, "block_table")):
         _i32(t, name)
@@ -306,7 +307,7 @@ def attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
     group = n_q // n_kv
     _need(group <= 16, "attention_decode: more than 16 query heads per key/value head are refused")
     n_items = rows.numel()
-    part_acc, part_ml = workspace
+    part_acc, part_ml, arrivals = _decode_workspace(workspace, n_items, n_kv, "attention_decode")
     max_splits = part_ml.numel() // max(1, n_items * n_q * 2)
     span = min(max_context, window) if window else max_context
     need = (span + DECODE_SPLIT - 1) // DECODE_SPLIT + (1 if window else 0)
@@ -316,11 +317,21 @@ def attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
           "attention_decode: workspace too small for this context")
     defines = {"HEAD_DIM": head_dim, "GROUP": group}
     fn = _fn("attention_decode", "kipp_attention_decode",
-             [_c_ptr] * 10 + [_c_int] * 6 + [_c_float, _c_int, _c_int, _c_int, _c_ptr], defines)
+             [_c_ptr] * 10 + [_c_int] * 6 + [_c_float, _c_int, _c_int, _c_int, _c_ptr, _c_ptr], defines)
     _check(fn(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(part_acc), _ptr(part_ml), _ptr(rows),
               _ptr(positions), _ptr(seq_of_token), _ptr(block_table), block_table.shape[1], n_items, n_q, n_kv,
-              head_dim, k_cache.shape[2], float(scale), int(window), grid, max_splits, _stream()), "attention_decode")
+              head_dim, k_cache.shape[2], float(scale), int(window), grid, max_splits, _ptr(arrivals), _stream()),
+           "attention_decode")
     return out
+
+
+def _decode_workspace(workspace, n_items: int, n_kv: int, what: str):
+    part_acc, part_ml = workspace[0], workspace[1]
+    arrivals = workspace[2] if len(workspace) > 2 else None
+    if arrivals is not None:
+        _i32(arrivals, "arrivals")
+        _need(arrivals.numel() >= n_items * n_kv, f"{what}: one count per token and key/value head")
+    return part_acc, part_ml, arrivals
 
 
 DECODE_FUSED_SLABS = 4
@@ -379,7 +390,7 @@ def attention_decode_fused(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: to
     group = n_q // n_kv
     _need(group <= 16, "attention_decode_fused: more than 16 query heads per key/value head are refused")
     n_items = rows.numel()
-    part_acc, part_ml = workspace
+    part_acc, part_ml, arrivals = _decode_workspace(workspace, n_items, n_kv, "attention_decode_fused")
     max_splits = part_ml.numel() // max(1, n_items * n_q * 2)
     span = min(max_context, window) if window else max_context
     need = (span + DECODE_SPLIT - 1) // DECODE_SPLIT + (1 if window else 0)
@@ -390,20 +401,25 @@ def attention_decode_fused(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: to
     defines = {"HEAD_DIM": head_dim, "GROUP": group}
     fn = _fn("attention_decode", "kipp_attention_decode_fused",
              [_c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_float, _c_ptr, _c_ptr, _c_int] + [_c_ptr] * 9 + [_c_int] * 6
-             + [_c_float, _c_int, _c_int, _c_int, _c_ptr], defines)
+             + [_c_float, _c_int, _c_int, _c_int, _c_ptr, _c_ptr], defines)
     null = lambda t: _ptr(t) if t is not None else None
     _check(fn(_ptr(qkv), parts, n_tokens, null(q_norm_w), null(k_norm_w), float(eps), null(inv_freq), null(angles),
               1 if write_kv else 0,
               _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(part_acc), _ptr(part_ml), _ptr(rows), _ptr(positions),
               _ptr(seq_of_token), _ptr(block_table), block_table.shape[1], n_items, n_q, n_kv, head_dim,
-              k_cache.shape[2], float(scale), int(window), grid, max_splits, _stream()), "attention_decode_fused")
+              k_cache.shape[2], float(scale), int(window), grid, max_splits, _ptr(arrivals), _stream()),
+           "attention_decode_fused")
     return out
 
 
 def attention_decode_workspace(n_items: int, n_q: int, head_dim: int, max_context: int, device) -> tuple:
+    """(part_acc, part_ml, arrivals): room for every split's partial result, and a count per (token, key/value
+    head) of the splits that have finished, which is zero between launches (the last to finish merges and sets
+    it back).  One launch at a time may use a workspace."""
     max_splits = (max_context + DECODE_SPLIT_MIN - 1) // DECODE_SPLIT_MIN + 1       # the shortest splits a launch may take
     return (torch.empty(n_items * n_q * max_splits * head_dim, dtype=torch.float32, device=device),
-            torch.empty(n_items * n_q * max_splits * 2, dtype=torch.float32, device=device))
+            torch.empty(n_items * n_q * max_splits * 2, dtype=torch.float32, device=device),
+            torch.zeros(n_items * n_q, dtype=torch.int32, device=device))
 
 
 def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,

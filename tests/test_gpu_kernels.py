@@ -362,6 +362,43 @@ def test_attention_decode(n_q, n_kv, d, page, window):
     assert not got[untouched].any()
 
 
+@pytest.mark.parametrize("n_seqs,n_q,n_kv,d,page,window,longest", [
+    (6, 32, 8, 128, 16, 0, 4500), (6, 32, 8, 128, 16, 600, 4500), (6, 6, 2, 48, 8, 0, 4500), (6, 16, 1, 32, 16, 0, 4500),
+    (12, 32, 8, 128, 16, 0, 4500),          # a dozen sequences: the kernel that streams through LDS, in ranges
+    (8, 16, 8, 64, 16, 0, 9500)])           # long contexts at a head size the LDS kernel does not take: long ranges
+def test_attention_decode_merged_by_the_last_workgroup_gives_the_bits_of_the_merge_launch(n_seqs, n_q, n_kv, d, page, window, longest):
+    """The splits of a head are merged by whichever of their workgroups finishes last, from partial results
+    written through to memory, or (without the arrival counts in the workspace) by a launch of its own: the same
+    sums in the same order, so the same bits, in each of the three kernels.  Several launches on one workspace,
+    with other contexts each time (a count that was not set back, or a partial result read before it arrived,
+    would show), one to two dozen splits a head, a sequence of one split among them."""
+    ops = _ops()
+    rng = np.random.default_rng(n_q + d + window + n_seqs)
+    ws = ops.attention_decode_workspace(n_seqs, n_q, d, longest, DEV)
+    assert len(ws) == 3 and ws[2].dtype == torch.int32 and not ws[2].any()
+    for launch in range(4 if longest < 5000 else 2):
+        seq_lens = [int(n) for n in rng.integers(longest // 2, longest, size=n_seqs - 1)] + [int(rng.integers(1, 190))]
+        if launch % 2:
+            seq_lens[0] = int(rng.integers(260, 600))
+        table, k, v = _paged_setup(rng, seq_lens, n_kv, d, page, torch.bfloat16)
+        rows = list(range(n_seqs))
+        positions = [n - 1 for n in seq_lens]
+        q = torch.tensor(rng.normal(size=(n_seqs, n_q * d)), dtype=torch.bfloat16).to(DEV)
+        args = (k.to(DEV), v.to(DEV))
+        idx = (_t(rows, torch.int32), _t(positions, torch.int32), _t(rows, torch.int32), _t(table, torch.int32))
+        here, apart = (torch.zeros(n_seqs, n_q * d, dtype=torch.bfloat16, device=DEV) for _ in range(2))
+        ws[0].fill_(float("nan"))
+        ops.attention_decode(q, *args, here, *idx, n_q, n_kv, d, 1 / math.sqrt(d), window, max(seq_lens), ws)
+        torch.cuda.synchronize()
+        assert not ws[2].any(), f"launch {launch}: a count was not set back"
+        ops.attention_decode(q, *args, apart, *idx, n_q, n_kv, d, 1 / math.sqrt(d), window, max(seq_lens), ws[:2])
+        assert torch.equal(here, apart), f"launch {launch}"
+        if launch == 0:
+            some = [0, n_seqs - 1]
+            ref = _attention_reference(q.cpu()[some], k, v, table, [positions[i] for i in some], some, n_q, n_kv, d, page, window)
+            assert _rel(here.float().cpu().numpy().reshape(n_seqs, n_q, d)[some], ref) < 1e-5
+
+
 @pytest.mark.parametrize("n_q,n_kv,d,page,window", [(32, 8, 128, 16, 0), (32, 8, 128, 16, 1500), (6, 2, 48, 8, 0), (2, 1, 16, 16, 700)])
 def test_attention_decode_of_many_rows(n_q, n_kv, d, page, window):
     """The kernel that walks long ranges of keys with a running maximum (built here so that it
