@@ -205,8 +205,8 @@ class Runtime:
         and "plan" among them; `same_bits`: the names whose results are those of "plan" bit for bit;
         `extra_ms`: name -> milliseconds that a way costs its consumer beyond its own kernel (the slabs of a split
         product are read by the kernel that adds them).
-        `own_prompt_products` True (the default): only those are timed, so the choice changes how long a
-        product takes and never what it gives; "auto": all of them (the library's product and other parts of K
+        `own_prompt_products` True: only those are timed, so the choice changes how long a
+        product takes and never what it gives; "auto" (the default): all of them (the library's product and other parts of K
         round differently: two runs of one program may then differ in their last bits); False: the library's."""
         if self.for_a_graph:
             # a step that is to be recorded keeps to our own kernels (the library's calls stay out of HIP graphs)
