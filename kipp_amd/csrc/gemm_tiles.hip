@@ -524,8 +524,8 @@ int kipp_gemm_tiles_parts(int M, int N, int K, int end, int max_parts) {
 }
 
 // Y: float32 [parts, M, N] with parts = kipp_gemm_tiles_parts(...) (end 0), bfloat16 [M, N / 2] = silu(gate) * up for
-// W = [gate; up] (end 1), bfloat16 [M, N] (end 2).  K a multiple of 32.  `force`: 0, or 100 wm + 10 wn + parts (+ 1000: 8 waves, four across) to take
-// that cut for all columns whatever the plan says (measurements and tests).
+// W = [gate; up] (end 1), bfloat16 [M, N] (end 2).  K a multiple of 32.  `force`: 0, or 100 wm + 10 wn + parts (+ 1000: 8 waves, four across; + 2000: the same for whole rounds of tiles, the
+// rest of the columns in smaller ones, which + 10000 r chooses) to take that cut whatever the plan says (the runtime's timed choice, tests).
 int kipp_gemm_tiles(const void* X, const void* W, void* Y, int M, int N, int K, int end, int max_parts, int force,
                     hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
@@ -537,8 +537,26 @@ int kipp_gemm_tiles(const void* X, const void* W, void* Y, int M, int N, int K, 
     Cut cuts[2];
     int n_cuts = plan(M, N, K, end, max_parts, cuts);
     if (force) {
+        const int cols = end == END_SWIGLU ? N / 2 : N;
         n_cuts = 1;
-        cuts[0] = {(force / 100) % 10, (force / 10) % 10, force % 10, 0, end == END_SWIGLU ? N / 2 : N, force >= 1000 ? 4 : 2};
+        const int rest_code = force / 10000;         // + 10000 r: the tile of the columns that + 2000 leaves (below)
+        force %= 10000;
+        cuts[0] = {(force / 100) % 10, (force / 10) % 10, force % 10, 0, cols, force >= 1000 ? 4 : 2};
+        if (force >= 2000 && end != END_SLABS) {
+            // + 2000: 8 waves as with + 1000, but only the whole rounds of 256 tiles in this cut; the columns that
+            // are left, which would hold every compute unit for a round that few of them have a tile in, go to
+            // smaller tiles: 8 waves on half the rows and columns, or (r = 1, 2, 3) 4 waves on 256 x 64, 128 x 128, 128 x 64
+            const int tm = 64 * cuts[0].wm, tn = (end == END_SWIGLU ? 16 : 32) * cuts[0].wn * 4;
+            const int tiles_m = (M + tm - 1) / tm;
+            const long long whole = ((long long)tiles_m * (cols / tn)) / 256 * 256;
+            const int first_cols = (int)(whole / tiles_m) * tn;
+            if (first_cols > 0 && first_cols < cols) {
+                n_cuts = 2;
+                cuts[0].col_end = first_cols;
+                static const int rest[4][3] = {{2, 2, 4}, {4, 2, 2}, {2, 4, 2}, {2, 2, 2}};
+                cuts[1] = {rest[rest_code & 3][0], rest[rest_code & 3][1], 1, first_cols, cols, rest[rest_code & 3][2]};
+            }
+        }
     }
     for (int c = 0; c < n_cuts; ++c) {
         const Cut& cut = cuts[c];

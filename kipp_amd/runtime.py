@@ -191,13 +191,14 @@ class Runtime:
         return 1 << (max(m, 1) - 1).bit_length()
 
     # Cuts of our kernel that are timed beside the planned one: 100 x (wave tile rows / 32) + 10 x (wave tile
-    # columns / 32) + parts of K (+ 1000: workgroups of 8 waves, two a SIMD, on the same 256 x 256 tile).  The
+    # columns / 32) + parts of K (+ 1000: workgroups of 8 waves, two a SIMD, on the same 256 x 256 tile; + 2000: those for
+    # the whole rounds of 256 tiles and smaller tiles for the columns that are left, + 30000: the smallest for those).  The
     # plan's cost model is linear; the GPU under its power limit is not (a round that leaves compute units idle
     # clocks the others higher), so the plan is not always the fastest.  An output element is summed over K in
     # the same order whatever the tile, so cuts with the same parts of K give the same bits.
     _choices_of_process: dict = {}
     TILE_CUTS_SLABS = (441, 442, 444, 431, 432, 421, 422, 1421, 1422, 1424)
-    TILE_CUTS_BF16 = (441, 421, 241, 1421)
+    TILE_CUTS_BF16 = (441, 421, 241, 1421, 2421, 32421)
 
     def _fastest(self, key, ways: dict, same_bits, extra_ms=None):
         """Which of several ways to compute one product is taken for the shape `key`: decided once, by timing

@@ -886,7 +886,7 @@ def test_gemm_rows(m, n, k, max_parts):
                            ops.gemm_rows(x.to(DEV), wd, max_parts))
 
 
-TILE_CUTS = [0, 441, 442, 421, 243, 221, 224, 431, 232, 1421, 1422, 1221]      # 100 wm + 10 wn + parts (+ 1000: 8 waves); 0: what the launcher plans
+TILE_CUTS = [0, 441, 442, 421, 243, 221, 224, 431, 232, 1421, 1422, 1221]      # 100 wm + 10 wn + parts (+ 1000: 8 waves; + 2000: whole rounds of those, the rest smaller; + 10000 r: the rest's tile); 0: what the launcher plans
 
 
 @pytest.mark.parametrize("force", TILE_CUTS)
@@ -910,12 +910,13 @@ def test_gemm_tiles_float32_end(m, n, k, force):
     assert np.array_equal(out.cpu().numpy(), xi.float().numpy() @ wi.float().numpy().T)
 
 
-@pytest.mark.parametrize("force", [0, 441, 421, 241, 221, 1421, 1221])
-@pytest.mark.parametrize("m,inner,k", [(257, 150, 64), (600, 9728 // 8, 160), (300, 24, 2560), (2050, 1300, 96)])
+@pytest.mark.parametrize("force", [0, 441, 421, 241, 221, 1421, 1221, 2421, 32421])
+@pytest.mark.parametrize("m,inner,k", [(257, 150, 64), (600, 9728 // 8, 160), (300, 24, 2560), (2050, 1300, 96), (2050, 4804, 64)])
 def test_gemm_tiles_swiglu_and_bfloat16_ends(m, inner, k, force):
     """W = [gate; up]: silu(x . gate^T) * (x . up^T) rounded once, at the end (gate first: the other way round
-    gives another result), also where the launcher cuts the columns into two kinds of tiles; and the plain
-    bfloat16 end.  Widths that are no multiple of 8 take the store of single values."""
+    gives another result), also where the launcher cuts the columns into two kinds of tiles (as planned, or
+    forced with + 2000: whole rounds of 8-wave tiles and the rest of the columns in smaller ones, which the
+    last size has); and the plain bfloat16 end.  Widths that are no multiple of 8 take the store of single values."""
     ops = _ops()
     rng = np.random.default_rng(m + inner + force)
     x = torch.tensor(rng.normal(size=(m, k)), dtype=torch.bfloat16)
@@ -947,6 +948,12 @@ def test_gemm_tiles_cuts_with_the_same_parts_give_the_same_bits():
             assert torch.equal(ops.gemm_tiles(x, w, "slabs", max_parts=4, force=cut), base), cut
     gated = ops.gemm_tiles(x, w, "swiglu", force=441)
     for cut in (0, 421, 241, 221, 1421):
+        assert torch.equal(ops.gemm_tiles(x, w, "swiglu", force=cut), gated), cut
+    # wide enough for whole rounds of tiles and a rest
+    x = torch.tensor(rng.normal(size=(2050, 96)), dtype=torch.bfloat16).to(DEV)
+    w = torch.tensor(rng.normal(size=(2 * 4800, 96)) * 0.3, dtype=torch.bfloat16).to(DEV)
+    gated = ops.gemm_tiles(x, w, "swiglu", force=441)
+    for cut in (0, 1421, 2421, 12421, 22421, 32421):
         assert torch.equal(ops.gemm_tiles(x, w, "swiglu", force=cut), gated), cut
 
 
