@@ -677,7 +677,9 @@ def gemm_tiles(x: torch.Tensor, w: torch.Tensor, end: str = "slabs", max_parts: 
     end "slabs": float32 [parts, M, N] whose sum over parts is the product (parts <= max_parts, chosen from the shape);
     "swiglu": w = [gate; up] of [2 I, K], the result is bfloat16 [M, I] = silu(x . gate^T) * (x . up^T);
     "bf16": bfloat16 [M, N].  `force` = 100 wm + 10 wn + parts (+ 1000: workgroups of 8 waves, four across, wave tiles
-    4 x 2 or 2 x 2) takes that cut instead of the planned one (the runtime's timed choice, tests)."""
+    4 x 2 or 2 x 2; + 2000, bfloat16 ends: those for the whole rounds of 256 tiles and smaller tiles for the columns
+    that are left, 8 waves on half the rows or, + 10000 r, 4 waves on 256 x 64, 128 x 128 or 128 x 64 outputs) takes
+    that cut instead of the planned one (the runtime's timed choice, tests)."""
     _dev(x, w)
     m, k = x.shape
     n = w.shape[0]
