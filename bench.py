@@ -5,7 +5,8 @@ bfloat16 weights on one MI355X.
 
 One JSON line: `value` is decoded tokens a second at batch 8 (a step is one
 decode step of the whole batch, tokens chosen greedily on the device and fed
-back), with the prefill of one 2,048-token prompt, the decode step's HBM
+back; by default 256 steps behind prompts of 2,048 tokens, the run from 2,048
+to 2,304 tokens that the workload names), with the prefill of one 2,048-token prompt, the decode step's HBM
 roofline and the batch-1 / batch-64 / batch-128 points beside it, then points at
 longer contexts (decode at batch 8 behind 8,192 and 30,720 tokens, a prompt
 portion of 512 tokens behind 4,096 and 16,384).  Peaks are MI355X's published
@@ -39,19 +40,42 @@ def log(msg):
     print(f"bench: {msg}", file=sys.stderr, flush=True)
 
 
-def model_numbers(cfg, layers):
-    """Weight elements a decode step reads and flops per token of the products."""
-    h, q, kv, i, v = cfg.hidden_size, cfg.q_dim, cfg.kv_dim, cfg.intermediate_size, cfg.vocab_size
-    per_layer = h * (q + 2 * kv) + q * h + 3 * h * i
-    head = v * h
-    kv_bytes_per_token = layers * 2 * kv * 2
-    return per_layer, head, kv_bytes_per_token
+def model_numbers(spec, cache_groups, element_size):
+    """What a step costs, from what the model's parts declare (no architecture's field names): the bytes of weights a
+    decode step reads (every tensor once; the embedding table only where it is also the head, since a step gathers a
+    few rows of it), the elements of the layers' matrices (2 flops a token each), the elements of the head's matrix,
+    the cache bytes a token holds (from the cache groups) and the attention flops per (query, key) pair."""
+    from kipp_amd.engine.model import model_params
+    params = model_params(spec)
+    embedding = spec.embedding.prefix + "weight"
+    head = embedding if spec.head.tied else spec.head.prefix + "weight"
+
+    def numel(p):
+        n = 1
+        for d in p.shape:
+            n *= d
+        return n
+    weight_bytes = element_size * sum(numel(p) for name, p in params.items() if name != embedding or spec.head.tied)
+    matrix_elems = 0
+    per_layer = {}
+    for index, layer in enumerate(spec.layers):
+        names = [spec_.prefix for _, spec_ in layer.parts if hasattr(spec_, "prefix")]
+        per_layer[index] = sum(numel(p) for name, p in params.items()
+                               if len(p.shape) == 2 and any(name.startswith(pre) for pre in names) and name not in (embedding, head))
+    pair_flops = 0.0
+    for run in spec.order:
+        matrix_elems += per_layer[run.layer]
+        mixer = dict(spec.layers[run.layer].parts).get("mixer")
+        pair_flops += 4.0 * getattr(mixer, "q_dim", 0)
+    kv_bytes_per_token = sum(g.bytes_per_token(element_size) for g in cache_groups)
+    return {"weight_bytes": float(weight_bytes), "matrix_elems": matrix_elems, "head_elems": numel(params[head]),
+            "kv_bytes_per_token": kv_bytes_per_token, "pair_flops": pair_flops}
 
 
-def prefill_flops(cfg, layers, n):
-    per_layer, head, _ = model_numbers(cfg, layers)
-    gemm = 2.0 * n * per_layer * layers + 2.0 * head          # the head runs on one row
-    attn = layers * 4.0 * cfg.q_dim * (n * (n + 1) / 2.0)     # causal half of QK^T and PV
+def prefill_flops(numbers, n, behind=0, wanted=1):
+    """Flops of a prompt portion of `n` tokens behind `behind` tokens already in the cache, with `wanted` rows of logits."""
+    gemm = 2.0 * n * numbers["matrix_elems"] + 2.0 * wanted * numbers["head_elems"]
+    attn = numbers["pair_flops"] * (n * behind + n * (n + 1) / 2.0)      # QK^T and PV over the keys each row sees
     return gemm + attn
 
 
@@ -109,30 +133,36 @@ class WrongKernelClass(RuntimeError):
 
 
 def measure_decode(engine, rt, ids, first, steps, warmup, repeats, weight_bytes, kv_per_token):
-    """`repeats` timings of `steps` decode steps (warm-up before the first), each from the same contexts (what a
-    repeat decoded is cut off again); the median one is reported.
+    """`repeats` timings of `steps` decode steps, each from the same contexts (what a repeat, and the warm-up before the
+    first, decoded is cut off again: with 256 steps behind prompts of 2,048 tokens every repeat is the run 2,048 -> 2,304
+    tokens); the median one is reported.
     Raises WrongKernelClass unless every timed step was a replay of a recorded graph of our own kernels."""
     timings = []
+    lengths = [engine.length(r) for r in ids]
+
+    def cut_back():
+        for r, n in zip(ids, lengths):                   # every repeat, and every batch size, decodes behind the prompts alone
+            engine.cache.truncate(engine.cache.requests[r], n)
+    if warmup > 0:
+        decode_run(engine, ids, first, warmup, 0)
+        cut_back()
     again = 0
     rep = 0
     while rep < repeats:
-        lengths = [engine.length(r) for r in ids]
         library, generic, replays = rt.library_products, rt.generic_attention_launches, engine.graphs.replays
-        w = warmup if rep == 0 else 0
-        seconds = decode_run(engine, ids, first, steps, w)
-        for r, n in zip(ids, lengths):                   # every repeat, and every batch size, decodes behind the prompts alone
-            engine.cache.truncate(engine.cache.requests[r], n)
+        seconds = decode_run(engine, ids, first, steps, 0)
+        cut_back()
         if rt.library_products != library or rt.generic_attention_launches != generic:
             raise WrongKernelClass(f"decode batch {len(ids)}: {rt.library_products - library} products went to the library and "
                                    f"{rt.generic_attention_launches - generic} attention launches to the generic kernel")
-        if engine.graphs.replays - replays < steps and again < 2:
-            again += 1         # the contexts passed into the next bucket, whose graph is recorded now: time these steps again
+        if engine.graphs.replays - replays < steps and again < 3:
+            again += 1         # the contexts passed into a bucket whose graph is recorded now: time these steps again
             continue
         if engine.graphs.replays - replays < steps:
-            raise WrongKernelClass(f"decode batch {len(ids)}: only {engine.graphs.replays - replays} of {steps + w + 1} steps "
+            raise WrongKernelClass(f"decode batch {len(ids)}: only {engine.graphs.replays - replays} of {steps + 1} steps "
                                    f"were replays of a recorded graph")
         # bytes a step has to read: every weight once and the cache of the live requests (their lengths mid-way)
-        kv_tokens = sum(n + 1 + w + steps / 2.0 for n in lengths)
+        kv_tokens = sum(n + 1 + (steps + 1) / 2.0 for n in lengths)
         timings.append((seconds / steps, weight_bytes + kv_tokens * kv_per_token))
         rep += 1
     per_step = sorted(t for t, _ in timings)
@@ -140,17 +170,17 @@ def measure_decode(engine, rt, ids, first, steps, warmup, repeats, weight_bytes,
     mad = sorted(abs(t - median) for t in per_step)[len(per_step) // 2]
     nbytes = [b for t, b in timings if t == median][0]
     return {"tok_s": len(ids) / median, "ms": median * 1e3, "mad_ms": mad * 1e3, "steps": steps, "warmup": warmup,
-            "bytes": nbytes, "repeats": repeats}
+            "bytes": nbytes, "repeats": repeats, "context": [lengths[0] + 1, lengths[0] + 1 + steps]}
 
 
-def long_context_points(model, rt, cfg, layers, args, weight_bytes, kv_per_token):
+def long_context_points(model, rt, cfg, numbers, args, weight_bytes, kv_per_token):
     """Decode at batch 8 behind 8,192 and 30,720 tokens and a prompt portion of 512 tokens behind 4,096 and
     16,384: tokens a second, and the fraction of the roofline (HBM for decode, bf16 MFMA for the portion)."""
     import torch
     from kipp_amd.engine import Engine, StepEntry
     batch, page, top = 8, 16, 30720
-    steps, warmup = max(8, args.steps // 2), max(2, args.warmup // 2)
-    room = top + 2 * (steps * 5 + warmup + 2) + 16
+    steps, warmup = max(8, min(64, args.steps // 2)), max(2, args.warmup // 2)
+    room = top + steps + warmup + 32
     engine = Engine(model, page_size=page, num_pages=batch * (-(-room // page)) + 4, max_requests=batch,
                     share_prefixes=False, max_position=room)
     ids = [f"long{i}" for i in range(batch)]
@@ -193,12 +223,11 @@ def long_context_points(model, rt, cfg, layers, args, weight_bytes, kv_per_token
             f"{r['bytes'] / (r['ms'] / 1e3) / 1e9:.0f} GB/s")
         for rid in ids:                              # the tokens of the timed steps are in the cache; go on from a known one
             last[rid] = 0
-    per_layer, _, _ = model_numbers(cfg, layers)
     for behind, times in portion_ms.items():
         if not times:
             continue
         ms = sorted(times)[len(times) // 2]
-        flops = 2.0 * 512 * per_layer * layers + layers * 4.0 * cfg.q_dim * (512 * behind + 512 * 513 / 2.0)
+        flops = prefill_flops(numbers, 512, behind, wanted=0)
         points[f"prefill512_ctx{behind}"] = round(512 / (ms / 1e3), 1)
         fracs[f"prefill512_ctx{behind}"] = round(flops / (ms / 1e3) / PEAK_FLOPS["bf16"], 4)
         log(f"a portion of 512 tokens behind {behind}: {ms:.2f} ms (median of {len(times)}), {512 / (ms / 1e3):.0f} tok/s")
@@ -208,7 +237,8 @@ def long_context_points(model, rt, cfg, layers, args, weight_bytes, kv_per_token
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--steps", type=int, default=256,
+                    help="timed decode steps; 256 behind prompts of 2,048 tokens is the workload's run from 2,048 to 2,304 tokens")
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--shape", default="qwen3-4b")
     ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the shape has (named in config)")
@@ -249,18 +279,19 @@ def main():
     if args.products != "default":
         rt.own_prompt_products = {"own": True, "auto": "auto", "library": False}[args.products]
     model = random_model(config, seed=0, runtime=rt)
-    # the first requests take part in every batch size: room for all those steps
+    # every repeat and every batch size starts from the prompts again: room for one run of steps behind a prompt
     repeats = max(1, args.repeats)
-    decoded = sum((repeats + 2) * (args.steps if b == args.batch else max(8, args.steps // 2)) +
-                  (args.warmup if b == args.batch else max(2, args.warmup // 2)) + 1 for b in batches)
-    tokens_per_request = args.prompt + decoded + 8
+    tokens_per_request = args.prompt + max(args.steps, args.warmup) + 16
+    if tokens_per_request > context:
+        print(f"bench: a prompt of {args.prompt} tokens and {args.steps} steps exceed the context of {context}", file=sys.stderr)
+        return 1
     engine = Engine(model, page_size=page, num_pages=max_batch * (-(-tokens_per_request // page)) + 4,
                     max_requests=max_batch, share_prefixes=False)
     torch.cuda.synchronize()
     log(f"model and cache ready in {time.perf_counter() - t0:.1f} s")
 
-    per_layer, head, kv_per_token = model_numbers(cfg, layers)
-    weight_bytes = 2.0 * (per_layer * layers + head)
+    numbers = model_numbers(model.spec, engine.cache.groups, 2)
+    weight_bytes, kv_per_token = numbers["weight_bytes"], numbers["kv_bytes_per_token"]
 
     # ---- prefill of one 2,048-token prompt (logits of the last place)
     prefill = None
@@ -276,7 +307,7 @@ def main():
             times.append(time.perf_counter() - start)
             engine.close("prefill")
         best = sorted(times[1:])[len(times[1:]) // 2]
-        flops = prefill_flops(cfg, layers, PREFILL_TOKENS)
+        flops = prefill_flops(numbers, PREFILL_TOKENS)
         prefill = {"value": round(PREFILL_TOKENS / best, 1), "tokens": PREFILL_TOKENS, "ms": round(best * 1e3, 3),
                    "frac": round(flops / best / PEAK_FLOPS["bf16"], 4)}
         log(f"prefill {PREFILL_TOKENS} tokens: {best * 1e3:.2f} ms, {PREFILL_TOKENS / best:.0f} tok/s")
@@ -289,8 +320,7 @@ def main():
     log(f"filled in {time.perf_counter() - t0:.1f} s")
     results = {}
     for b in batches:
-        steps = args.steps if b == args.batch else max(8, args.steps // 2)
-        warmup = args.warmup if b == args.batch else max(2, args.warmup // 2)
+        steps, warmup = args.steps, args.warmup
         try:
             results[b] = measure_decode(engine, rt, ids[:b], first, steps, warmup, repeats, weight_bytes, kv_per_token)
         except Exception as exc:          # a further point must not cost the headline: say so and go on
@@ -309,7 +339,7 @@ def main():
         del engine
         torch.cuda.empty_cache()
         try:
-            long_points, long_fracs = long_context_points(model, rt, cfg, layers, args, weight_bytes, kv_per_token)
+            long_points, long_fracs = long_context_points(model, rt, cfg, numbers, args, weight_bytes, kv_per_token)
         except WrongKernelClass:
             raise
         except Exception as exc:
@@ -325,7 +355,8 @@ def main():
         "config": {"model": args.shape, "layers": layers, "layers_of_shape": full_layers, "hidden": cfg.hidden_size,
                    "q_heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
                    "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size, "tied": cfg.tie_word_embeddings,
-                   "global_batch": args.batch, "seq_len": context, "prompt_tokens": args.prompt, "kv_page": page,
+                   "global_batch": args.batch, "seq_len": context, "prompt_tokens": args.prompt,
+                   "decoded_tokens": main_r["steps"], "kv_page": page,
                    "parallelism": "none", "weights": "random N(0,0.02) seed 0"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4)},

@@ -93,7 +93,8 @@ def _start(name: str, defines: Optional[dict]):
     cmd = [_hipcc()] + FLAGS + dflags + ["-I", HERE, src, "-o", tmp]
     # what the compiler prints goes to a file: through a pipe that nobody reads before the compiler
     # ends, a long list of warnings would fill the pipe and the compiler would wait for ever
-    proc = subprocess.Popen(cmd, stdout=open(tmp + ".log", "w"), stderr=subprocess.STDOUT)
+    with open(tmp + ".log", "w") as log:
+        proc = subprocess.Popen(cmd, stdout=log, stderr=subprocess.STDOUT)     # the child keeps its own handle
     return out, tmp, proc
 
 

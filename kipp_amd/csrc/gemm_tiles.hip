@@ -15,8 +15,8 @@
 // With one wave a SIMD, whatever holds up its instruction stream idles the matrix cores.  Every other
 // instruction of the walk (the reads of the next operands out of LDS, the DMA of the steps ahead) is
 // therefore placed between two products, a few at a time, and the barrier of a step falls between its two
-// halves.  Measured (a build with -DPROBE_CLOCK counts the shader clock around the walk): 37.5 cycles a
-// product where the matrix core needs 32; 33.5 with the DMA taken out (-DABLATE_DMA=1): a wave that issues
+// halves.  Measured with the shader clock around the walk: 37.5 cycles a
+// product where the matrix core needs 32; 33.5 with the DMA taken out: a wave that issues
 // a DMA instruction cannot issue its next product in time, which a second wave on the SIMD hides.  In the
 // run of a prefill the chip is at its power limit, and the time of a product is set by that, not by the
 // cycles: the cuts differ by a few per cent, and which is fastest for a shape is found by the clock.
@@ -42,9 +42,6 @@
 #define CHUNKS (BK / 8)                            // 16-byte chunks of a row of a piece
 #define GROUP_ROWS (16 / CHUNKS)                   // rows that share 256 bytes of LDS
 #define INSTR_ROWS (4 * GROUP_ROWS)                // rows one DMA instruction of a wave brings (1 KB)
-#ifndef ABLATE_READS
-#define ABLATE_READS 0                             // measurements only: 1 takes the reads of the operands out
-#endif
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
@@ -82,27 +79,17 @@ __device__ __forceinline__ void wait_reads(u32x4 (&fa)[WM], u32x4 (&fb)[WN]) {
         asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(fa[0]), "+v"(fa[1]), "+v"(fb[0]), "+v"(fb[1]));
 }
 
-// Steps of K that are in LDS or on their way there: four.  (Measurements only: -DSMALL_DEPTH=3 -DSMALL_WGS=2 gives
-// the tiles of half the size three steps and two workgroups a compute unit, i.e. two waves a SIMD from two
-// workgroups.  Measured and no faster: those tiles move half as many bytes again through the DMA for the same
-// products.  Two waves a SIMD on the full tile are the 8-wave cuts.)
-#ifndef SMALL_DEPTH
-#define SMALL_DEPTH 4
-#endif
-#ifndef SMALL_WGS
-#define SMALL_WGS 1
-#endif
+// Steps of K that are in LDS or on their way there: four.  (Tiles of half the size with three steps and two
+// workgroups a compute unit, i.e. two waves a SIMD from two workgroups, were measured and are no faster: those
+// tiles move half as many bytes again through the DMA for the same products.  Two waves a SIMD on the full tile
+// are the 8-wave cuts.)
 template <int WM, int WN>
 struct Depth {
-    static constexpr int value = WM * WN <= 8 ? SMALL_DEPTH : 4;
+    static constexpr int value = 4;
 };
 
-#ifdef PROBE_CLOCK
-__device__ long long clock_probe[2048][4];
-#endif
-
 template <int WM, int WN, int END, int WGN = 2>
-__global__ void __launch_bounds__(64 * 2 * WGN, (WM * WN <= 8 && WGN == 2 ? SMALL_WGS : 1)) gemm_tiles_kernel(
+__global__ void __launch_bounds__(64 * 2 * WGN, 1) gemm_tiles_kernel(
     const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* __restrict__ Y, int M, int N, int K,
     int tiles_m, int tiles_n, int parts, int inner, int col_begin, int col_end) {
     constexpr int STAGES = Depth<WM, WN>::value;
@@ -175,17 +162,11 @@ __global__ void __launch_bounds__(64 * 2 * WGN, (WM * WN <= 8 && WGN == 2 ? SMAL
     // where step `step` of an operand begins, for every lane: pinned to scalar registers (left to itself the
     // compiler adds the lane's offset first and then walks a 64-bit vector address along K)
     auto step_base = [&](const unsigned char* base, int step) {
-#if defined(ABLATE_DMA) && ABLATE_DMA == 2
-        step = 0;                                                // measurements only: every step brings the first again
-#endif
         const unsigned char* at = base + (size_t)step * (BK * 2);
         asm volatile("" : "+s"(at));
         return at;
     };
     auto issue_one = [&](const unsigned char* x_at, const unsigned char* w_at, int stage, int n) {   // DMA instruction n (0 .. LOADS - 1) of a step
-#if defined(ABLATE_DMA) && ABLATE_DMA == 1
-        return;
-#endif
         // the lane's offset passes through an empty asm here, so that its widening to 64 bits stands beside the
         // load: the compiler then takes the form "scalar base + 32-bit vector offset" and adds nothing per load
         // (widened once outside the walk, the offset would cost a 64-bit vector add for every load)
@@ -232,13 +213,11 @@ __global__ void __launch_bounds__(64 * 2 * WGN, (WM * WN <= 8 && WGN == 2 ? SMAL
     do {                                                                                                           \
         const uint32_t st_ = (uint32_t)(uintptr_t)LDS_PTR(lds + ((STEP) % STAGES) * STAGE_BYTES);                  \
         const uint32_t a_at_ = st_ + a_base + frag_at[KS], b_at_ = st_ + b_base + frag_at[KS];                     \
-        if (!ABLATE_READS) {                                                                                       \
-            if ((R) == 0) asm volatile("ds_read_b128 %0, %1" : "=v"(a[T][0]) : "v"(a_at_));                        \
-            else if ((R) <= WN)                                                                                    \
-                asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(b[T][(R) <= WN ? (R) - 1 : 0]) : "v"(b_at_), "i"(((R) - 1) * 32 * BK * 2)); \
-            else                                                                                                   \
-                asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(a[T][(R) > WN ? (R) - WN : 0]) : "v"(a_at_), "i"(((R) - WN) * 32 * BK * 2)); \
-        }                                                                                                          \
+        if ((R) == 0) asm volatile("ds_read_b128 %0, %1" : "=v"(a[T][0]) : "v"(a_at_));                            \
+        else if ((R) <= WN)                                                                                        \
+            asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(b[T][(R) <= WN ? (R) - 1 : 0]) : "v"(b_at_), "i"(((R) - 1) * 32 * BK * 2)); \
+        else                                                                                                       \
+            asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(a[T][(R) > WN ? (R) - WN : 0]) : "v"(a_at_), "i"(((R) - WN) * 32 * BK * 2)); \
     } while (0)
 #define KIPP_PRODUCT(T, M_)                                                                         \
     do {                                                                                            \
@@ -285,9 +264,6 @@ __global__ void __launch_bounds__(64 * 2 * WGN, (WM * WN <= 8 && WGN == 2 ? SMAL
     asm volatile("" ::: "memory");
 #pragma unroll
     for (int r = 0; r < NR; ++r) KIPP_READ_ONE(0, 0, 0, r);
-#ifdef PROBE_CLOCK
-    const long long c0 = __builtin_readcyclecounter(), r0 = __builtin_amdgcn_s_memrealtime();
-#endif
     for (int kt = 0; kt < nk; ++kt) {
         // first half: products of columns 0 .. 15 of the step; the operands of the second half arrive meanwhile,
         // and the late DMA instructions of step kt + STAGES - 1 go out, into the buffer of step kt - 1
@@ -333,14 +309,6 @@ __global__ void __launch_bounds__(64 * 2 * WGN, (WM * WN <= 8 && WGN == 2 ? SMAL
 #undef KIPP_READ_B
 #undef KIPP_DMA_B
 #undef KIPP_ITEMS
-#ifdef PROBE_CLOCK
-    if (tid == 0 && blockIdx.x < 2048 && blockIdx.z == 0) {
-        clock_probe[blockIdx.x][0] = __builtin_readcyclecounter() - c0;
-        clock_probe[blockIdx.x][1] = __builtin_amdgcn_s_memrealtime() - r0;
-        clock_probe[blockIdx.x][2] = nk;
-        clock_probe[blockIdx.x][3] = r0;
-    }
-#endif
     wait_reads<WM, WN>(a[0], b[0]);
     __builtin_amdgcn_s_waitcnt(0x0F70);      // nothing may still be on its way into LDS when the buffers are used again
 #undef KIPP_READ_ONE
@@ -509,12 +477,6 @@ static int launch_end(const void* X, const void* W, void* Y, int M, int N, int K
 }
 
 extern "C" {
-#ifdef PROBE_CLOCK
-int kipp_gemm_tiles_clock(long long* out, int n) {
-    return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(clock_probe), (size_t)n * 4 * sizeof(long long));
-}
-#endif
-
 // parts that kipp_gemm_tiles cuts K into for these sizes when it may use up to `max_parts` (1 for the ends that are not slabs)
 int kipp_gemm_tiles_parts(int M, int N, int K, int end, int max_parts) {
     if (K <= 0 || (K % BK) || M <= 0 || N <= 0) return -1;

@@ -747,21 +747,6 @@ def mfma_rate(data: torch.Tensor, workgroups: int, accumulators: int, iters: int
     return int(got)
 
 
-def mfma_dma(data: torch.Tensor, src: torch.Tensor, workgroups: int, waves: int, every: int, iters: int) -> int:
-    """The probe that multiplies and issues a DMA instruction into LDS behind every `every`-th product (0: none), in
-    workgroups of 4 or 8 waves; `src`: 64 KiB a workgroup.  Returns the floating-point operations launched."""
-    _dev(data, src)
-    _need(data.numel() * data.element_size() == 16384 and src.numel() * src.element_size() >= 65536 * workgroups,
-          "mfma_dma: 16 KiB of operand bits and 64 KiB of source a workgroup")
-    fn = build.library("probe").kipp_probe_mfma_dma
-    fn.restype = ctypes.c_longlong
-    fn.argtypes = [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr]
-    sink = torch.zeros(1, dtype=torch.int32, device=data.device)
-    got = fn(_ptr(data), _ptr(src), int(workgroups), int(waves), int(every), int(iters), _ptr(sink), _stream())
-    _need(got > 0, "mfma_dma: refused")
-    return int(got)
-
-
 # --------------------------------------------------------------------------- sampling
 
 def argmax(logits: torch.Tensor, out: torch.Tensor) -> torch.Tensor:

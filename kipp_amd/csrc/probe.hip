@@ -66,55 +66,6 @@ __global__ void __launch_bounds__(256) mfma_rate_kernel(const u32x4* __restrict_
     if (total == 123.456f) sink[0] = 1;          // keeps the products
 }
 
-// The same with a DMA instruction (global_load_lds_dwordx4: 1 KB from `src` straight into LDS) behind every
-// EVERY-th product: what such an instruction costs the products of the wave that issues it, with one wave a SIMD
-// (256 threads, 16 accumulators) and with two (512 threads, 8 accumulators each), where the other wave's products
-// fill the time.  `src` holds 64 KiB for every workgroup.
-#define PROBE_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
-#define PROBE_GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void*)(p))
-template <int ACC, int EVERY, int THREADS>
-__global__ void __launch_bounds__(THREADS) mfma_dma_kernel(const u32x4* __restrict__ data, const unsigned char* __restrict__ src,
-                                                           int iters, uint32_t* __restrict__ sink) {
-    extern __shared__ __attribute__((aligned(1024))) unsigned char probe_lds[];
-    union {
-        u32x4 u;
-        bf16x8 v;
-    } a[4], b[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        a[i].u = data[(threadIdx.x + 64 * i) & 1023];
-        b[i].u = data[(threadIdx.x * 3 + 17 * i + 512) & 1023];
-    }
-    f32x16 acc[ACC];
-#pragma unroll
-    for (int i = 0; i < ACC; ++i)
-#pragma unroll
-        for (int j = 0; j < 16; ++j) acc[i][j] = 0.0f;
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    uint32_t off = (uint32_t)(wave * 8192 + lane * 16);
-    const unsigned char* base = src + (size_t)blockIdx.x * 65536;
-    unsigned char* dst = probe_lds + wave * 4096;
-    for (int it = 0; it < iters; ++it) {
-#pragma unroll
-        for (int i = 0; i < ACC; ++i) {
-            acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i & 3].v, b[(i >> 2) & 3].v, acc[i], 0, 0, 0);
-            if (EVERY > 0 && i % EVERY == EVERY - 1) {
-                asm volatile("" : "+v"(off));
-                __builtin_amdgcn_global_load_lds(PROBE_GLOBAL_PTR(base + off), PROBE_LDS_PTR(dst + 1024 * ((i / EVERY) & 3)), 16, 0, 0);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-        }
-        if (EVERY > 0 && (it & 3) == 3) __builtin_amdgcn_s_waitcnt(0x0F78);   // at most 8 on their way
-    }
-    __builtin_amdgcn_s_waitcnt(0x0F70);
-    float total = 0.0f;
-#pragma unroll
-    for (int i = 0; i < ACC; ++i)
-#pragma unroll
-        for (int j = 0; j < 16; ++j) total += acc[i][j];
-    if (total == 123.456f) sink[0] = 1 + probe_lds[threadIdx.x];
-}
-
 extern "C" {
 
 // `workgroups` of 4 waves, each wave `iters` rounds over `accumulators` (8 or 16) products of 32x32x16 from
@@ -129,33 +80,6 @@ long long kipp_probe_mfma_rate(const void* data, int workgroups, int accumulator
         return -1;
     if (KIPP_LAUNCH_CHECK() != 0) return -1;
     return (long long)workgroups * 4 * accumulators * iters * 32768LL;
-}
-
-// `workgroups` x (4 or 8) waves, a DMA instruction behind every `every`-th product (0: none).  Returns the
-// floating-point operations launched, or -1.  `src`: 64 KiB a workgroup.
-long long kipp_probe_mfma_dma(const void* data, const void* src, int workgroups, int waves, int every, int iters, void* sink,
-                              hipStream_t stream) {
-    if (workgroups <= 0 || iters <= 0 || (waves != 4 && waves != 8) || (every != 0 && every != 2 && every != 4)) return -1;
-#define KIPP_PROBE_DMA(ACC, EVERY, THREADS)                                                                           \
-    do {                                                                                                               \
-        if (hipFuncSetAttribute((const void*)mfma_dma_kernel<ACC, EVERY, THREADS>, hipFuncAttributeMaxDynamicSharedMemorySize, \
-                                65536) != hipSuccess)                                                                  \
-            return -1;                                                                                                 \
-        hipLaunchKernelGGL((mfma_dma_kernel<ACC, EVERY, THREADS>), dim3(workgroups), dim3(THREADS), 65536, stream,         \
-                           (const u32x4*)data, (const unsigned char*)src, iters, (uint32_t*)sink);                     \
-    } while (0)
-    if (waves == 4) {
-        if (every == 0) KIPP_PROBE_DMA(16, 0, 256);
-        else if (every == 2) KIPP_PROBE_DMA(16, 2, 256);
-        else KIPP_PROBE_DMA(16, 4, 256);
-    } else {
-        if (every == 0) KIPP_PROBE_DMA(8, 0, 512);
-        else if (every == 2) KIPP_PROBE_DMA(8, 2, 512);
-        else KIPP_PROBE_DMA(8, 4, 512);
-    }
-#undef KIPP_PROBE_DMA
-    if (KIPP_LAUNCH_CHECK() != 0) return -1;
-    return (long long)workgroups * waves * (waves == 4 ? 16 : 8) * iters * 32768LL;
 }
 
 // Reads `bytes` (rounded down to what `workgroups` x 4 waves x whole rings cover) once.  Returns the bytes read, or -1.

@@ -55,3 +55,32 @@ def prebuilt() -> List[Spec]:
             _add(out, model_variants(cfg.model_spec(), dtype))
     out.append(("probe", None))
     return out
+
+
+# Kernel builds beyond what the named shapes launch: head sizes and head groupings at which the kernels are checked
+# alone and in small models, and builds of the decode attention whose thresholds are lowered so that a check can
+# reach the kernels for long contexts and many sequences with inputs it can verify.  `build()` compiles them ahead
+# together with `prebuilt()`; whoever finds one missing compiles it then.
+ATTENTION = [(128, 16), (128, 1), (16, 3), (48, 3), (64, 1), (32, 16), (256, 4), (80, 3), (256, 2), (16, 1), (32, 2), (16, 6)]   # (head size, group)
+EARLY_STREAM = [(128, 4), (48, 3), (16, 2)]      # the kernel for long contexts takes over at 1,024 keys
+WHOLE_CONTEXTS = [(128, 4), (128, 16)]           # the whole-context kernel at few sequences
+
+
+def check_builds() -> List[Spec]:
+    """Builds beyond the named shapes' own that the checks of the kernels and of small models launch."""
+    out = []
+    for head_dim, group in ATTENTION:
+        out.append(("attention_prefill", {"HEAD_DIM": head_dim}))
+        out.append(("attention_decode", {"HEAD_DIM": head_dim, "GROUP": group}))
+    for head_dim, group in EARLY_STREAM:
+        out.append(("attention_decode", {"HEAD_DIM": head_dim, "GROUP": group, "STREAM_FROM": 1024}))
+    for head_dim, group in WHOLE_CONTEXTS:
+        out.append(("attention_decode", {"HEAD_DIM": head_dim, "GROUP": group, "RING_FROM_PAIRS": 1}))
+    seen, unique = set(), []
+    for name, defines in out:
+        key = (name, tuple(sorted(defines.items())))
+        if key not in seen:
+            seen.add(key)
+            unique.append((name, defines))
+    return unique
+

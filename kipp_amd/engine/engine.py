@@ -119,6 +119,7 @@ class Engine:
                 batch = build_batch(entries, requests, len(self.cache.groups), self.rt.device)
                 logits = self.model.forward(batch, self.cache)
         except Exception:
+            self._after_failed_launches()
             for r in requests:                  # the step did not happen: its pages go back
                 self.cache.trim(r)
             for rid in opened:
@@ -131,6 +132,23 @@ class Engine:
             for r in requests:
                 self._uncommitted[r.id] = 1
         return logits
+
+    def _after_failed_launches(self) -> None:
+        """A forward pass that stopped half way may have left counts of finished splits above zero in a decode
+        workspace that outlives the step (a recorded shape keeps its own): the next launch on it would merge early or
+        never.  They are set back to zero by a kernel; a recording that was under way is dropped with its shape."""
+        if self.graphs is None:
+            return
+        for key, graph in list(self.graphs.graphs.items()):
+            if graph.graph is None and graph.eager_runs >= 2:
+                del self.graphs.graphs[key]                 # failed while recording: made anew when the shape returns
+                continue
+            for name, space in graph.batch.host.items():
+                if isinstance(name, tuple) and name and name[0] == "decode_workspace" and len(space) > 2 and space[2] is not None:
+                    try:
+                        self.rt.ops.fill_zero(space[2])
+                    except Exception:                       # noqa: BLE001 - the device itself is gone: nothing left to tidy
+                        return
 
     def commit(self, request_id, tokens: Sequence[int]) -> None:
         """The tokens of a step that ran from `device_tokens` are known now."""

@@ -21,6 +21,10 @@ Policy (the reference's server loop lifted out of its HTTP code,
   its last place.
 * A sampled stop token ends the request and is neither kept nor fed back;
   reaching `max_new_tokens` ends it without running the last token.
+* A step that fails (the step function raises) fails as a unit: every request that had
+  tokens in it ends with `finish_reason="failed"` and its error, its pages go back, and
+  the queue moves on (/root/reference/src/kipp_server.c:2081-2088).  The engine has
+  already undone the step's own reservations by then.
 * While every running request decodes and none waits, the scheduler runs one step
   ahead of what it knows (`lookahead`): the next step is launched with the tokens
   still on the device, and the tokens of the step before are read while it runs,
@@ -63,8 +67,10 @@ class Request:
     rng: Optional[XorShift64Star] = None
     recent: Deque[int] = field(default_factory=lambda: deque(maxlen=RECENT_WINDOW))
     arrived: float = 0.0
+    admitted_at: Optional[float] = None
     first_token_at: Optional[float] = None
     finished_at: Optional[float] = None
+    error: Optional[str] = None     # what the step function said when a step with this request in it failed
 
     @property
     def budget_tokens(self) -> int:
@@ -83,6 +89,15 @@ class SchedulerStats:
     steps: int = 0
     waits_for_pages: int = 0
     waits_for_prefix: int = 0
+    # what the reference's server counts beside these (/root/reference/src/kipp_server.c:71-84): requests that a
+    # failed step ended, and sums of seconds with their counts, so that a reader derives averages and rates
+    failed: int = 0
+    failed_steps: int = 0
+    queue_wait_seconds_sum: float = 0.0     # arrival -> admission
+    queue_wait_count: int = 0
+    ttft_seconds_sum: float = 0.0           # arrival -> first token known
+    ttft_count: int = 0
+    decode_seconds_sum: float = 0.0         # first token -> finish, of requests that ended without failing
 
 
 def _rows_on_device(engine, tokens, rows):
@@ -226,6 +241,9 @@ class Scheduler:
                 self.stats.waits_for_pages += 1
                 return
             self.waiting.popleft()
+            req.admitted_at = time.monotonic()
+            self.stats.queue_wait_seconds_sum += req.admitted_at - req.arrived
+            self.stats.queue_wait_count += 1
             req.fed = rc.length
             self.stats.prefix_tokens_reused += rc.length
             req.state = "prefill"
@@ -265,7 +283,11 @@ class Scheduler:
         if not plan:
             return produced
         entries = [StepEntry(req.id, tokens, want) for req, tokens, want in plan]
-        logits = self.engine.step(entries, borrow=True)      # read by `choose` before the next step is launched
+        try:
+            logits = self.engine.step(entries, borrow=True)      # read by `choose` before the next step is launched
+        except Exception as error:                               # noqa: BLE001 - whatever the step function raises fails the batch
+            self._fail([req for req, _, _ in plan], error)
+            return produced
         self.stats.steps += 1
         sampling = [req for req, _, want in plan if want]
         self._tell(sampling, logits)
@@ -302,7 +324,13 @@ class Scheduler:
         if go_on:
             cont = [reqs[i] for i in go_on]
             tokens = picks.device if len(go_on) == len(reqs) else _rows_on_device(self.engine, picks.device, go_on)
-            logits = self.engine.step([StepEntry(req.id, [0], [0]) for req in cont], device_tokens=tokens, borrow=True)
+            try:
+                logits = self.engine.step([StepEntry(req.id, [0], [0]) for req in cont], device_tokens=tokens, borrow=True)
+            except Exception as error:                           # noqa: BLE001
+                # the step before still holds good: its tokens are read and kept, then its requests fail with this one
+                produced = self._drain()
+                self._fail([req for req in cont if req.state != "finished"], error)
+                return produced
             self._tell(cont, logits)
             self.stats.steps += 1
             nxt = (cont, self.engine.choose(logits, cont, wait=False))
@@ -338,6 +366,15 @@ class Scheduler:
                 self._accept(req, int(token), produced)
         return produced
 
+    def _fail(self, requests, error) -> None:
+        """The step these requests had tokens in failed as a unit: each of them ends, failed, and its
+        pages and slot go back; requests that were not in the step go on
+        (/root/reference/src/kipp_server.c:2081-2088)."""
+        self.stats.failed_steps += 1
+        for req in requests:
+            req.error = f"{type(error).__name__}: {error}"
+            self._finish(req, "failed")
+
     def _accept(self, req: Request, token: int, produced) -> None:
         if req.max_new_tokens == 0:
             self._finish(req, "length")
@@ -348,6 +385,8 @@ class Scheduler:
         now = time.monotonic()
         if req.first_token_at is None:
             req.first_token_at = now
+            self.stats.ttft_seconds_sum += now - req.arrived
+            self.stats.ttft_count += 1
         req.output.append(token)
         req.recent.append(token)
         produced.append((req.id, token))
@@ -368,6 +407,10 @@ class Scheduler:
             self.engine.close(req.id)
         self.finished[req.id] = req
         self.stats.finished += 1
+        if reason == "failed":
+            self.stats.failed += 1
+        elif req.first_token_at is not None:
+            self.stats.decode_seconds_sum += req.finished_at - req.first_token_at
         self._common = {k: v for k, v in self._common.items() if req.id not in k}
 
     def run(self, max_steps: Optional[int] = None) -> Dict[object, Request]:

@@ -201,5 +201,7 @@ class Attention:
         if ws is None:
             ws = self.rt.ops.attention_decode_workspace(batch.n_decode, s.num_heads, s.head_dim,
                                                         batch.max_decode_ctx, self.rt.device)
+            if not self.rt.merge_in_kernel:
+                ws = ws[:2]         # without the counts the splits are merged by a launch of its own
             batch.host[key] = ws
         return ws

@@ -109,14 +109,18 @@ class Runtime:
         self.library_products = 0   # calls that went to the library (they stay out of HIP graphs)
         self.generic_attention_launches = 0   # bfloat16 attention that fell to the generic kernel (geometry the matrix-core kernels refuse)
         self.fuse_norms = True      # few rows: residual add and norm ride on the products around them
-        # products of more than about 200 rows: "auto" (the default): the fastest of our own matrix-core kernel's cuts and
-        # the library's product, timed once in a process at a shape's first use (another process may choose
-        # otherwise, and its results then differ in their last bits); True: our kernel, in the fastest of the cuts
-        # that give the planned cut's bits (the same bits in every process); False: always the library's.
+        # products of more than about 200 rows: True (the default): our own matrix-core kernel, in the fastest of the
+        # cuts that give the planned cut's bits, so that every process computes the same bits; "auto": the fastest of
+        # all our cuts and the library's product, timed once in a process at a shape's first use (another process
+        # may choose otherwise, and its results then differ in their last bits); False: always the library's.
         # KIPP_AMD_PRODUCTS=own|auto|library sets it from outside.
-        self.own_prompt_products = {"own": True, "auto": "auto", "library": False}.get(os.environ.get("KIPP_AMD_PRODUCTS", "auto"), "auto")
+        self.own_prompt_products = {"own": True, "auto": "auto", "library": False}.get(os.environ.get("KIPP_AMD_PRODUCTS", "own"), True)
         self.prompt_product_choices = {}     # shape -> "library", "plan" (our kernel, cut as planned) or a forced cut of ours
         self.tile_products = 0      # products of many rows that ran on our own kernel
+        # decode attention: the splits of a head are merged by whichever of their workgroups finishes last (one launch
+        # fewer a layer; ordered by device-scope stores, one device-scope counter a head and device-scope loads); False,
+        # or KIPP_AMD_DECODE_MERGE=launch, merges them in a launch of its own, which needs no ordering between workgroups
+        self.merge_in_kernel = os.environ.get("KIPP_AMD_DECODE_MERGE", "kernel") != "launch"
         self.for_a_graph = False    # set around a step of single tokens that is, or is to be, recorded as a HIP graph
         torch.backends.cuda.matmul.allow_tf32 = False
 

@@ -6,7 +6,6 @@ portions, and requests that share a long beginning (paged prefix reuse).
     python -m kipp_amd.workloads shared-prefix [--shape qwen3-32b] [--requests 8]  ...
     python -m kipp_amd.workloads hbm           [--gib 4]
     python -m kipp_amd.workloads mfma
-    python -m kipp_amd.workloads walk          [--ablate-dma 1|2] [--ablate-reads]
     python -m kipp_amd.workloads products      [--shape qwen3-4b] [--rows 2048,512]
     python -m kipp_amd.workloads portion       [--shape qwen3-4b] [--rows 512] [--behind 4096]
 
@@ -15,8 +14,7 @@ second, time to the first token, and what the cache reused.  `hbm` is no
 workload but the yardstick for the decode kernels: how fast a kernel that only
 reads gets a large buffer out of memory (best of several grids and ring depths).
 `mfma` is the yardstick for the prompt products: what the matrix cores sustain on
-operands that never leave the registers; `walk` counts the shader cycles a product
-takes inside our prompt-product kernel (a build with clock counters; it compiles at its first call).
+operands that never leave the registers.
 `products` times the four matrix products of a layer for prompt portions, our
 kernel beside the library's; `portion` times a prompt portion behind a context
 that is already in the cache (what a step of chunked prefill costs).
@@ -143,66 +141,7 @@ def mfma_rate() -> dict:
                     best = max(best, flops / (ms * 1e-3) / 1e15)
                 table.append({"operands": name, "grid": what, "ms": round(ms, 3), "PFLOP_s": round(best, 3)})
                 log(f"{name:6s} {what:17s} kernel of {ms:8.3f} ms: {best:5.3f} PFLOP/s")
-    # what a DMA instruction into LDS costs the products of the wave that issues it, and whether a second wave hides it
-    data = operands["normal"].to("cuda:0")
-    src = torch.zeros(cus * 65536, dtype=torch.uint8, device="cuda:0")
-    dma = []
-    for waves in (4, 8):
-        for every in (0, 4, 2):
-            start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            ops.mfma_dma(data, src, cus, waves, every, 2000)
-            start.record()
-            flops = ops.mfma_dma(data, src, cus, waves, every, 2000)
-            end.record()
-            torch.cuda.synchronize()
-            ns = start.elapsed_time(end) * 1e6 / (flops / 32768 / (cus * 4))
-            dma.append({"waves_per_simd": waves // 4, "dma_every": every, "ns_per_product_of_a_simd": round(ns, 2)})
-            log(f"{waves // 4} wave(s) a SIMD, a DMA instruction behind every {every or 'no'} product(s): {ns:6.2f} ns a product of a SIMD")
-    return {"workload": "mfma rate", "compute_units": cus, "all": table, "dma": dma}
-
-
-def walk(ablate_dma: int, ablate_reads: bool, n: int = 8192, k: int = 9728, rows: int = 2048, cut: int = 441) -> dict:
-    """Shader cycles a product (v_mfma_f32_32x32x16_bf16, 32 cycles of the matrix core) inside the walk over K
-    of the prompt-product kernel, from a build that reads the shader clock and the 100 MHz clock around the
-    walk; optionally with the DMA taken out (1) or made to bring the first step every time (2: it always hits
-    the cache), and with the reads out of LDS taken out.  The ablated builds compute nothing meaningful."""
-    import ctypes
-    import numpy as np
-    import torch
-    from .csrc import build
-    defines = {"PROBE_CLOCK": 1}
-    if ablate_dma:
-        defines["ABLATE_DMA"] = int(ablate_dma)
-    if ablate_reads:
-        defines["ABLATE_READS"] = 1
-    lib = build.library("gemm_tiles", defines)
-    ptr, i32 = ctypes.c_void_p, ctypes.c_int
-    lib.kipp_gemm_tiles.argtypes = [ptr, ptr, ptr, i32, i32, i32, i32, i32, i32, ptr]
-    lib.kipp_gemm_tiles_clock.argtypes = [ptr, i32]
-    x = torch.randn(rows, k, device="cuda:0").bfloat16()
-    w = (torch.randn(n, k, device="cuda:0") * 0.02).bfloat16()
-    out = torch.zeros(rows * n, device="cuda:0", dtype=torch.float32)
-    table = []
-    for launches in (1, 20):
-        for _ in range(launches):
-            rc = lib.kipp_gemm_tiles(x.data_ptr(), w.data_ptr(), out.data_ptr(), rows, n, k, 0, 1, cut, torch.cuda.current_stream().cuda_stream)
-            if rc != 0:
-                raise RuntimeError(f"gemm_tiles refused (code {rc})")
-        torch.cuda.synchronize()
-        groups = min(2048, -(-rows // (64 * ((cut // 100) % 10))) * -(-n // (32 * ((cut // 10) % 10) * (4 if cut >= 1000 else 2))))
-        buf = np.zeros((2048, 4), dtype=np.int64)
-        if lib.kipp_gemm_tiles_clock(buf.ctypes.data, 2048) != 0:
-            raise RuntimeError("the probe's counters could not be read")
-        b = buf[:groups].astype(float)
-        wm, wn, per_simd = (cut // 100) % 10, (cut // 10) % 10, (2 if cut >= 1000 else 1)
-        products = b[:, 2] * 2 * wm * wn * per_simd  # a SIMD's products in the walk: 2 wm wn a step of each of its waves
-        row = {"after_launches": launches, "cycles_per_product": round(float(np.median(b[:, 0] / products)), 2),
-               "ns_per_product": round(float(np.median(b[:, 1] * 10 / products)), 2),
-               "GHz": round(float(np.median(b[:, 0] / (b[:, 1] * 10))), 3)}
-        table.append(row)
-        log(f"{rows} x {n} x {k}, after {launches} launch(es): {row['cycles_per_product']} shader cycles a product of a SIMD, "
-            f"{row['ns_per_product']} ns, clock {row['GHz']} GHz")
-    return {"workload": "walk", "ablate_dma": ablate_dma, "ablate_reads": bool(ablate_reads), "all": table}
+    return {"workload": "mfma rate", "compute_units": cus, "all": table}
 
 
 def _time(fn, runs: int = 20) -> float:
@@ -305,20 +244,6 @@ def main(argv=None) -> int:
         rows = [int(r) for r in args.rows.split(",") if r]
         result = products(args.shape, rows) if argv[0] == "products" else portion(args.shape, args.layers, rows[0], args.behind)
         print(json.dumps(result), flush=True)
-        return 0
-    if argv and argv[0] == "walk":
-        ap = argparse.ArgumentParser(prog="python -m kipp_amd.workloads walk")
-        ap.add_argument("--ablate-dma", type=int, default=0, choices=[0, 1, 2])
-        ap.add_argument("--ablate-reads", action="store_true")
-        ap.add_argument("--cut", type=int, default=441, help="100 wm + 10 wn + parts (+ 1000: 8 waves)")
-        ap.add_argument("--n", type=int, default=8192)
-        ap.add_argument("--k", type=int, default=9728)
-        args = ap.parse_args(argv[1:])
-        import torch
-        if not torch.cuda.is_available():
-            print("workload: no GPU", file=sys.stderr)
-            return 1
-        print(json.dumps(walk(args.ablate_dma, args.ablate_reads, n=args.n, k=args.k, cut=args.cut)), flush=True)
         return 0
     if argv and argv[0] == "mfma":
         import torch

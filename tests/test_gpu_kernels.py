@@ -886,7 +886,7 @@ def test_gemm_rows(m, n, k, max_parts):
                            ops.gemm_rows(x.to(DEV), wd, max_parts))
 
 
-TILE_CUTS = [0, 441, 442, 421, 243, 221, 224, 431, 232, 1421, 1422, 1221]      # 100 wm + 10 wn + parts (+ 1000: 8 waves; + 2000: whole rounds of those, the rest smaller; + 10000 r: the rest's tile); 0: what the launcher plans
+TILE_CUTS = [0, 441, 442, 444, 421, 422, 243, 221, 224, 431, 432, 232, 1421, 1422, 1424, 1221]      # 100 wm + 10 wn + parts (+ 1000: 8 waves; + 2000: whole rounds of those, the rest smaller; + 10000 r: the rest's tile); 0: what the launcher plans
 
 
 @pytest.mark.parametrize("force", TILE_CUTS)

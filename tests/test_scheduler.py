@@ -224,3 +224,67 @@ def test_a_request_id_names_one_request_at_a_time():
     assert sched.stats.refused == 4
     eng.cache.close("session")
     eng.cache.check()
+
+
+class FailingEngine(FakeEngine):
+    """The step function raises on the calls named in `fail_on` (1-based), after it has undone what it
+    reserved for that step, as the real engine does."""
+
+    def __init__(self, fail_on, **kw):
+        super().__init__(**kw)
+        self.fail_on = set(fail_on)
+        self.tries = 0
+
+    def step(self, entries, borrow=False):
+        self.tries += 1
+        if self.tries in self.fail_on:
+            reqs, opened = [], []
+            for e in entries:
+                if e.request not in self.cache.requests:
+                    self.cache.open(e.request)
+                    opened.append(e.request)
+                reqs.append(self.cache.requests[e.request])
+            self.cache.reserve([(r, len(e.tokens)) for r, e in zip(reqs, entries)])
+            for r in reqs:
+                self.cache.trim(r)
+            for rid in opened:
+                self.cache.close(rid)
+            raise RuntimeError("the device said no")
+        return super().step(entries, borrow)
+
+
+def test_a_failed_step_fails_its_requests_and_the_queue_moves_on():
+    """/root/reference/src/kipp_server.c:2081-2088: the batch fails as a unit.  Requests that had tokens in
+    the failed step end as failed and give everything back; a request that waited is admitted and runs."""
+    eng = FailingEngine(fail_on=[3], num_pages=6, page_size=4)
+    sched = Scheduler(eng, max_step_tokens=8, prefill_chunk=4)
+    sched.add(Request("a", list(range(1, 9)), 4))          # 11 tokens: 3 pages
+    sched.add(Request("b", [7, 8, 9], 6))                  # 8 tokens: 2 pages
+    sched.add(Request("c", [4, 5, 6, 7, 8], 8))            # 12 tokens: 3 pages, waits until a or b has gone
+    done = sched.run(max_steps=50)
+    assert sched.idle
+    assert done["a"].finish_reason == "failed" and done["b"].finish_reason == "failed"
+    assert "the device said no" in done["a"].error and done["a"].error == done["b"].error
+    assert done["c"].finish_reason == "length" and done["c"].output == expected_output([4, 5, 6, 7, 8], 8)
+    st = sched.stats
+    assert (st.failed, st.failed_steps, st.finished, st.requests) == (2, 1, 3, 3)
+    assert st.queue_wait_count == 3 and st.queue_wait_seconds_sum >= 0.0
+    assert st.ttft_count >= 1 and st.ttft_seconds_sum >= 0.0 and st.decode_seconds_sum >= 0.0
+    assert not eng.cache.requests and eng.cache.free_pages() == [6]
+    eng.cache.check()
+
+
+def test_a_failed_step_leaves_requests_outside_it_running():
+    """With a budget of one token a step, the step that fails holds one request only; the other goes on
+    and produces what it would have produced."""
+    eng = FailingEngine(fail_on=[4], num_pages=8, page_size=4)
+    sched = Scheduler(eng, max_step_tokens=1, prefill_chunk=4)
+    sched.add(Request("a", [1, 2], 3))
+    sched.add(Request("b", [3, 4], 3))
+    done = sched.run(max_steps=60)
+    reasons = sorted(r.finish_reason for r in done.values())
+    assert reasons == ["failed", "length"]
+    ok = [r for r in done.values() if r.finish_reason == "length"][0]
+    assert ok.output == expected_output(list(ok.prompt), 3)
+    assert sched.stats.failed == 1 and eng.cache.free_pages() == [8]
+    eng.cache.check()
