@@ -84,9 +84,11 @@ class AttentionSpec:
             raise ConfigError(
                 f"num_attention_heads {self.num_heads} is not a multiple of "
                 f"num_key_value_heads {self.num_kv_heads}")
-        if self.head_dim <= 0 or self.head_dim % 16 or self.head_dim > 256:
+        # any head size up to 256 runs (the float32 path and the generic kernel take it); the matrix-core attention
+        # kernels of the bfloat16 path take multiples of 16 and the mixer falls back to the generic one otherwise
+        if self.head_dim <= 0 or self.head_dim > 256:
             raise ConfigError(
-                f"head_dim {self.head_dim} unsupported: kernels take multiples of 16 up to 256")
+                f"head_dim {self.head_dim} unsupported: the attention kernels take head sizes from 1 to 256")
         if self.window is not None and self.window <= 0:
             raise ConfigError(f"attention window must be positive, got {self.window}")
 

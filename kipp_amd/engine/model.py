@@ -67,10 +67,10 @@ class Model:
         yield "norm", self.spec.final_norm, self.final_norm
         yield "head", self.spec.head, self.head
 
-    def load_tensors(self, tensors: Dict[str, torch.Tensor], where: str = "the given tensors") -> "Model":
-        """Bind tensors by name (checked against what the parts declare) and put
-        them on the device, one part at a time."""
-        check_tensors(where, tensors, model_params(self.spec))
+    def bind(self, tensors) -> "Model":
+        """Give every part its tensors: `tensors[file name]` (a mapping; it may make a tensor when it is asked for it)
+        is put on the device as the part's class says and handed over under the part's local name.  The one place where
+        a part category's tensors reach its part, whatever their source."""
         for category, part_spec, part in self._owners():
             cls = part_class(category, part_spec.kind)
             forced = getattr(cls, "placement", lambda s: {})(part_spec)
@@ -85,6 +85,11 @@ class Model:
                 part.load(local)
         self.loaded = True
         return self
+
+    def load_tensors(self, tensors: Dict[str, torch.Tensor], where: str = "the given tensors") -> "Model":
+        """Bind tensors by name, checked first against what the parts declare."""
+        check_tensors(where, tensors, model_params(self.spec))
+        return self.bind(tensors)
 
     # -- forward ---------------------------------------------------------------------------
     def forward(self, batch, cache) -> Optional[torch.Tensor]:
@@ -134,22 +139,9 @@ def random_model(config: dict, seed: int, runtime) -> Model:
     model = Model(spec, runtime)
     expected = model_params(spec)
 
-    class _Lazy(dict):
+    class _Made(dict):
         def __missing__(self, name):
             return random_tensor(seed, name, expected[name], torch.bfloat16, device=str(runtime.device))
-    lazy = _Lazy()
-    for category, part_spec, part in model._owners():
-        cls = part_class(category, part_spec.kind)
-        forced = getattr(cls, "placement", lambda s: {})(part_spec)
-        prefix = getattr(part_spec, "prefix", "")
-        local = {}
-        for name, p in cls.params(part_spec).items():
-            force = {"float32": torch.float32, None: None}[forced.get(name)]
-            local[name] = runtime.place(lazy[prefix + name], p.kind, force)
-        if category == "head":
-            part.load(local, embedding=model.embedding)
-        else:
-            part.load(local)
-    model.loaded = True
+    model.bind(_Made())
     model.config = cfg
     return model

@@ -66,7 +66,7 @@ class Attention:
         """The builds of its specialised kernels (one per head size; decode also per number of query heads
         that share a key/value head).  Under float32, and for more than 16 heads a group, the generic
         attention kernel runs, which every model has."""
-        if dtype != "bfloat16":
+        if dtype != "bfloat16" or spec.head_dim % 16:
             return []
         group = spec.num_heads // spec.num_kv_heads
         out = [("attention_prefill", {"HEAD_DIM": spec.head_dim})]
@@ -102,7 +102,8 @@ class Attention:
         eps = s.qk_norm_eps if s.qk_norm_eps is not None else 0.0
         pairing = getattr(self.position, "pairing", "half")
         # a table row is as wide as the longest context of this step, so what decides is what the step needs
-        fast = rt.dtype == "bfloat16" and rt.ops.attention_fast_ok(s.num_heads, s.num_kv_heads, cache.page_size, table.shape[1])
+        fast = rt.dtype == "bfloat16" and s.head_dim % 16 == 0 \
+            and rt.ops.attention_fast_ok(s.num_heads, s.num_kv_heads, cache.page_size, table.shape[1])
         if rt.dtype == "bfloat16" and not fast:
             rt.generic_attention_launches += 1      # the slow kernel class: a measurement must know it ran
         # single tokens only: norm, rotation, cache write and attention in one kernel, for a few of them (with

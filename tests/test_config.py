@@ -47,7 +47,8 @@ def test_head_dim_defaults_to_hidden_over_heads(tiny_configs):
     ("use_sliding_window", True, "use_sliding_window"),
     ("model_type", "llama", "model_type"),
     ("num_key_value_heads", 3, "multiple"),
-    ("head_dim", 24, "head_dim"),
+    ("head_dim", 260, "head_dim"),
+    ("head_dim", 23, "rotary_dim"),
     ("vocab_size", "256", "vocab_size"),
     ("num_hidden_layers", 0, "num_hidden_layers"),
     ("rms_norm_eps", -1.0, "rms_norm_eps"),
@@ -98,7 +99,8 @@ def test_eos_token_becomes_stop_tokens(tiny_configs):
 
 def test_part_specs_check_their_sizes():
     with pytest.raises(ConfigError):
-        AttentionSpec(64, 4, 2, 20)
+        AttentionSpec(64, 4, 2, 272)
+    assert AttentionSpec(64, 4, 2, 20).q_dim == 80      # no multiple of 16: the generic attention kernel runs it
     with pytest.raises(ConfigError):
         AttentionSpec(64, 4, 2, 16, window=0)
     with pytest.raises(ConfigError):

@@ -112,3 +112,22 @@ def test_norms_in_kernels_of_their_own(model_folders, tiny_configs, key):
         for rid, toks in requests.items():
             H.assert_close(got[rid], H.plain_logits(folder, toks), H.NMSE_BF16["tiny"], f"{key}/fused norms {fuse}/{rid}")
         assert (calls["delta"] == 0) == fuse, calls
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_head_size_that_is_no_multiple_of_16(tmp_path, tiny_configs, dtype):
+    """Head size 24 (q width 96 beside a hidden width of 80): the float32 path takes any head size up to 256, and
+    under bfloat16 the mixer sends such a geometry to the generic attention kernel, which is counted, instead
+    of the configuration refusing it.  Portions, single tokens and a mixed batch against the plain implementation."""
+    from kipp_amd.engine import Engine
+    from kipp_amd.weights import write_random_model
+    cfg = dict(tiny_configs["b"], head_dim=24, num_attention_heads=4, num_key_value_heads=2)
+    folder = write_random_model(str(tmp_path / "d24"), cfg, seed=77, dtype=dtype)
+    requests = {f"r{i}": H.random_tokens(40 + i, n, cfg["vocab_size"]) for i, n in enumerate([9, 33, 50])}
+    for maker in (H.tail_one_by_one, H.changing_portions, lambda r: H.mixed(r, seed=3)):
+        engine = Engine.from_folder(folder, dtype=dtype, page_size=8, max_tokens=512, share_prefixes=False)
+        got = H.replay(engine, requests, maker(requests))
+        for rid, toks in requests.items():
+            H.assert_close(got[rid], H.plain_logits(folder, toks), H.NMSE_F32 if dtype == "float32" else H.NMSE_BF16["tiny"],
+                           f"head size 24/{dtype}/{rid}")
+        assert (engine.rt.generic_attention_launches > 0) == (dtype == "bfloat16")
