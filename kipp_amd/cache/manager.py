@@ -1,10 +1,10 @@
 """The cache manager: pages of keys and values for every request, per group of
 layers, and slots of fixed-size state.
 
-Runs of the layer order with the same need (heads, head size, window) form a
-group; a group has its own pool of pages, its own block table for every
-request, and one key and one value tensor for each of its runs, laid out
-[page][kv head][slot in page][head_dim].  A group with a window gives pages
+Runs of the layer order with the same need (heads, head size, window, page size)
+form a group; a group has its own pool of pages, of its own page size and its own
+number of pages, its own block table for every request, and one key and one value
+tensor for each of its runs, laid out [page][kv head][slot in page][head_dim].  A group with a window gives pages
 back as soon as the window has passed them; every group gives all pages back
 when the request ends.  Mixers that keep state of fixed size get a slot per
 request instead: a row of a tensor [slots, ...], zeroed when claimed.
@@ -29,6 +29,16 @@ class OutOfPages(RuntimeError):
 
 class OutOfSlots(RuntimeError):
     """Every request slot is taken."""
+
+
+def _per_group(value, n_groups: int, what: str) -> List[int]:
+    """`value` for every group: one integer for all, or a sequence with one entry a group."""
+    if isinstance(value, (int, np.integer)):
+        return [int(value)] * n_groups
+    out = [int(v) for v in value]
+    if len(out) != n_groups:
+        raise ValueError(f"{what}: {len(out)} values for {n_groups} cache groups")
+    return out
 
 
 @dataclass
@@ -74,33 +84,51 @@ class CacheGroup:
 
 class CacheManager:
     def __init__(self, kv_needs: Sequence[Optional[KVNeed]], state_needs: Sequence[Optional[StateNeed]],
-                 page_size: int, num_pages: int, max_requests: int, max_position: int,
+                 page_size: int, num_pages, max_requests: int, max_position: int,
                  runtime=None, share_prefixes: bool = True, page_order=None):
         """`kv_needs[r]` / `state_needs[r]`: what run r of the layer order keeps
-        (None: nothing).  `num_pages` is the size of every group's pool.  With
-        `runtime` None no device memory is made (bookkeeping only).  `page_order`:
+        (None: nothing).  `page_size`: tokens a page for every group whose need names none of
+        its own.  `num_pages`: the pages of a pool, one number for every group (a group whose
+        pages have another size gets as many as hold the same tokens) or a sequence with a number
+        for each group, in the order in which the groups first appear in the run order.
+        With `runtime` None no device memory is made (bookkeeping only).  `page_order`:
         the order in which every group's fresh pool hands out its pages (see `PagePool`)."""
         self.page_size = page_size
         self.max_requests = max_requests
         self.max_position = max_position
-        self.max_blocks = (max_position + page_size - 1) // page_size
         self.rt = runtime
         self.groups: List[CacheGroup] = []
         self.run_group: Dict[int, Tuple[int, int]] = {}
+        needs: List[KVNeed] = []
+        for need in kv_needs:
+            if need is not None and need not in needs:
+                needs.append(need)
+        sizes = [need.page_size or page_size for need in needs]
+        if isinstance(num_pages, (int, np.integer)):
+            pages = [-(-int(num_pages) * page_size // size) for size in sizes]
+        else:
+            pages = _per_group(num_pages, len(needs), "num_pages")
         by_need: Dict[KVNeed, CacheGroup] = {}
         for run, need in enumerate(kv_needs):
             if need is None:
                 continue
             group = by_need.get(need)
             if group is None:
-                group = CacheGroup(len(self.groups), need, [], num_pages, page_size, page_order)
+                at = len(self.groups)
+                order = page_order if page_order is None or len(page_order) == pages[at] else None
+                group = CacheGroup(at, need, [], pages[at], sizes[at], order)
                 by_need[need] = group
                 self.groups.append(group)
             group.runs.append(run)
+        self.max_blocks = max([-(-max_position // g.page_size) for g in self.groups] or [1])
         self.state_needs = {r: n for r, n in enumerate(state_needs) if n is not None}
         self.states: Dict[int, object] = {}
-        # content sharing needs every token of the prefix to be in pages that are kept
-        self.share = share_prefixes and not self.state_needs and all(g.need.window is None for g in self.groups)
+        # content sharing needs every token of the prefix to be in pages that are kept, and pages that
+        # hold the same tokens in every group (one page size)
+        self.share = share_prefixes and not self.state_needs and all(g.need.window is None for g in self.groups) \
+            and len({g.page_size for g in self.groups}) <= 1
+        if self.groups and len({g.page_size for g in self.groups}) == 1:
+            self.page_size = self.groups[0].page_size
         self.free_slots = list(range(max_requests - 1, -1, -1))
         self.requests: Dict[object, RequestCache] = {}
         self._serial = 0
@@ -113,7 +141,7 @@ class CacheManager:
         rt = self.rt
         for g in self.groups:
             # one page more than the pool hands out: `scratch_page`, where rows that only pad a batch write
-            shape = (g.pool.num_pages + 1, g.need.num_kv_heads, self.page_size, g.need.head_dim)
+            shape = (g.pool.num_pages + 1, g.need.num_kv_heads, g.page_size, g.need.head_dim)
             for run in g.runs:
                 # zeroed: masked slots must hold finite values
                 g.k[run] = torch.zeros(shape, dtype=rt.cache_dtype, device=rt.device)
@@ -138,7 +166,7 @@ class CacheManager:
         src = run if reads_run is None else reads_run
         for g in self.groups:
             if src in g.runs:
-                return KVCacheView(g.index, g.k.get(src), g.v.get(src), self.page_size, writable=reads_run is None)
+                return KVCacheView(g.index, g.k.get(src), g.v.get(src), g.page_size, writable=reads_run is None)
         return None
 
     def state(self, run: int):
@@ -167,7 +195,8 @@ class CacheManager:
                 row.zero_()
         self._serial += 1
         req = RequestCache(request_id, slot, tables=[[] for _ in self.groups], adopted=[0 for _ in self.groups],
-                           rows=[np.zeros(self.max_blocks, dtype=np.int32) for _ in self.groups], serial=self._serial)
+                           rows=[np.zeros(-(-self.max_position // g.page_size), dtype=np.int32) for g in self.groups],
+                           serial=self._serial)
         if self.share and prompt is not None and self.groups:
             matches = [g.pool.prefix_match(prompt) for g in self.groups]
             keep = min(len(pages) for pages, _ in matches)
@@ -194,8 +223,24 @@ class CacheManager:
 
     def pages_needed(self, req: RequestCache, new_length: int) -> List[int]:
         """Pages each group still has to claim so that positions < new_length have one."""
-        blocks = (new_length + self.page_size - 1) // self.page_size
-        return [max(0, blocks - len(req.tables[g.index])) for g in self.groups]
+        return [max(0, -(-new_length // g.page_size) - len(req.tables[g.index])) for g in self.groups]
+
+    def pages_bound(self, req: Optional[RequestCache], budget_tokens: int, step_tokens: int) -> List[int]:
+        """The most pages each group may still have to hand the request beyond those it holds now, if it grows to
+        `budget_tokens` in steps of at most `step_tokens` (`req` None: a request that holds nothing yet).  A group
+        that keeps every key: the blocks it has not claimed.  A group with a window gives pages back as the
+        window passes them, so the request never holds more than the pages of window - 1 + step_tokens tokens
+        and one more for where they begin: what a scheduler has to keep free for it is the distance to that."""
+        out = []
+        for g in self.groups:
+            table = req.tables[g.index] if req is not None else []
+            need = max(0, -(-budget_tokens // g.page_size) - len(table))
+            if g.need.window is not None:
+                most = -(-(g.need.window - 1 + step_tokens) // g.page_size) + 1
+                held = sum(1 for page in table if page >= 0)
+                need = min(need, max(0, most - held))
+            out.append(need)
+        return out
 
     def free_pages(self) -> List[int]:
         return [g.pool.free_count for g in self.groups]
@@ -204,12 +249,10 @@ class CacheManager:
         """Claim the pages that every (request, number of new tokens) of a step
         needs, in every group; all or nothing."""
         claimed: List[Tuple[RequestCache, int, int]] = []
-        page_size = self.page_size
         for req, n_new in entries:
             new_length = req.length + n_new
             if n_new > 0 and new_length <= self.max_position:
-                blocks = (new_length + page_size - 1) // page_size
-                if all(len(t) >= blocks for t in req.tables):
+                if all(len(req.tables[g.index]) * g.page_size >= new_length for g in self.groups):
                     continue                                  # every position already has its page
             if n_new <= 0:
                 self._rollback(claimed)
@@ -238,8 +281,8 @@ class CacheManager:
 
     def trim(self, req: RequestCache) -> None:
         """Give back pages that were claimed for a step that did not happen."""
-        blocks = (req.length + self.page_size - 1) // self.page_size
         for g in self.groups:
+            blocks = -(-req.length // g.page_size)
             table = req.tables[g.index]
             while len(table) > blocks:
                 page = table.pop()
@@ -282,7 +325,7 @@ class CacheManager:
                 continue
             first_needed = max(0, req.length - window + 1)
             table = req.tables[g.index]
-            for block in range(min(first_needed // self.page_size, len(table))):
+            for block in range(min(first_needed // g.page_size, len(table))):
                 if table[block] >= 0:
                     g.pool.release(table[block])
                     table[block] = -1

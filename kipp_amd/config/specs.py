@@ -64,7 +64,9 @@ class AttentionSpec:
 
     `window` None keeps every key; W keeps the last W keys (the query's own
     position included).  `qk_norm_eps` None means no per-head norm of q and k.
-    `scale` None means 1/sqrt(head_dim).
+    `scale` None means 1/sqrt(head_dim).  `page_size` None keeps its keys in pages
+    of the engine's size; P asks for pages of P tokens (a short window is served
+    better by small pages), in a pool of their own.
     """
     hidden_size: int
     num_heads: int
@@ -76,6 +78,7 @@ class AttentionSpec:
     scale: Optional[float] = None
     prefix: str = ""
     kind: str = "attention"
+    page_size: Optional[int] = None
 
     def __post_init__(self):
         if self.num_heads <= 0 or self.num_kv_heads <= 0:
@@ -91,6 +94,8 @@ class AttentionSpec:
                 f"head_dim {self.head_dim} unsupported: the attention kernels take head sizes from 1 to 256")
         if self.window is not None and self.window <= 0:
             raise ConfigError(f"attention window must be positive, got {self.window}")
+        if self.page_size is not None and self.page_size <= 0:
+            raise ConfigError(f"attention page_size must be positive, got {self.page_size}")
 
     @property
     def q_dim(self) -> int:

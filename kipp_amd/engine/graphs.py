@@ -57,9 +57,10 @@ class DecodeGraph:
         self.groups = len(cache.groups)
         # a table row is as wide as the contexts of this shape, not as the model's longest possible one:
         # kernels choose by it what they can do, and it is copied whenever a row changes
-        self.max_blocks = max(1, -(-max_context // cache.page_size))
+        self.blocks = [max(1, -(-max_context // g.page_size)) for g in cache.groups]     # of a table row, per group
+        self.table_at = [4 * n + n * sum(self.blocks[:g]) for g in range(self.groups)]     # where a group's tables begin
         self.max_context = max_context
-        table_ints = self.groups * n * self.max_blocks
+        table_ints = n * sum(self.blocks)
         # [tokens | positions | ctx_len | slots | tables | arange | ones]
         self.layout = {"tokens": 0, "positions": n, "ctx_len": 2 * n, "slots": 3 * n, "tables": 4 * n}
         var_ints = 4 * n + table_ints
@@ -74,7 +75,7 @@ class DecodeGraph:
         d = self.dev
         arange = d[var_ints:var_ints + n]
         ones = d[var_ints + n:]
-        tables = {g: d[4 * n + g * n * self.max_blocks:4 * n + (g + 1) * n * self.max_blocks].view(n, self.max_blocks)
+        tables = {g: d[self.table_at[g]:self.table_at[g] + n * self.blocks[g]].view(n, self.blocks[g])
                   for g in range(self.groups)}
         self.batch = StepBatch(
             n_tokens=n, n_seqs=n, n_want=n, tokens=d[0:n], positions=d[n:2 * n], seq_of_token=arange, q_start=arange,
@@ -113,10 +114,9 @@ class DecodeGraph:
             if self.row_marks[i] != mark:
                 self.row_marks[i] = mark
                 changed = True
-                at = 4 * n + i * self.max_blocks
                 for g in range(self.groups):
-                    h[at:at + self.max_blocks] = r.rows[g][:self.max_blocks] if r is not None else self.scratch_pages[g]
-                    at += n * self.max_blocks
+                    at, width = self.table_at[g] + i * self.blocks[g], self.blocks[g]
+                    h[at:at + width] = r.rows[g][:width] if r is not None else self.scratch_pages[g]
         upto = self.var_ints if changed else 4 * n
         self.dev[:upto].copy_(self.host[:upto], non_blocking=True)
         self.copied = torch.cuda.Event()

@@ -148,13 +148,15 @@ class Scheduler:
         self._common: Dict[Tuple[object, object], int] = {}
 
     # -- page arithmetic -----------------------------------------------------------
-    def _pages(self, tokens: int) -> int:
-        return -(-tokens // self.cache.page_size)
+    @property
+    def _largest_step(self) -> int:
+        """Most tokens one request brings in a step."""
+        return min(self.prefill_chunk, self.max_step_tokens)
 
     def _still_to_claim(self, req: Request) -> List[int]:
-        """Pages a running request may still claim in each group."""
+        """Pages a running request may still claim in each group, beyond those it holds."""
         rc = self.cache.requests[req.id]
-        return self.cache.pages_needed(rc, req.budget_tokens)
+        return self.cache.pages_bound(rc, req.budget_tokens, self._largest_step)
 
     # -- interface -------------------------------------------------------------------
     def add(self, req: Request) -> None:
@@ -173,9 +175,10 @@ class Scheduler:
             raise RequestRefused(
                 f"request {req.id!r}: prompt {len(req.prompt)} + max_new_tokens {req.max_new_tokens} "
                 f"exceeds the model's {self.cache.max_position} positions")
-        if any(self._pages(req.budget_tokens) > g.pool.num_pages for g in self.cache.groups):
-            self.stats.refused += 1
-            raise RequestRefused(f"request {req.id!r}: needs {self._pages(req.budget_tokens)} pages, more than the pool has")
+        for g, most in zip(self.cache.groups, self.cache.pages_bound(None, req.budget_tokens, self._largest_step)):
+            if most > g.pool.num_pages:
+                self.stats.refused += 1
+                raise RequestRefused(f"request {req.id!r}: needs {most} pages of group {g.index}, more than its pool's {g.pool.num_pages}")
         for t in req.prompt:
             if not 0 <= int(t) < self.engine.vocab_size:
                 self.stats.refused += 1
@@ -230,7 +233,7 @@ class Scheduler:
                 self.stats.waits_for_prefix += 1
                 return
             rc = self.cache.open(req.id, req.prompt, publish_early=True)   # adopts the longest known beginning
-            need = self.cache.pages_needed(rc, req.budget_tokens)
+            need = self.cache.pages_bound(rc, req.budget_tokens, self._largest_step)
             promised = [0] * len(self.cache.groups)
             for other in self.running:
                 for g, n in enumerate(self._still_to_claim(other)):

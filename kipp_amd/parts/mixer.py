@@ -88,7 +88,7 @@ class Attention:
 
     def cache_need(self):
         s = self.spec
-        return KVNeed(num_kv_heads=s.num_kv_heads, head_dim=s.head_dim, window=s.window)
+        return KVNeed(num_kv_heads=s.num_kv_heads, head_dim=s.head_dim, window=s.window, page_size=s.page_size)
 
     def state_need(self):
         return None

@@ -284,3 +284,40 @@ def test_random_orders_lose_nothing(seed):
         m.close(rid)
     m.check()
     assert m.free_pages() == [g.pool.num_pages for g in m.groups] and len(m.free_slots) == 4
+
+
+def test_groups_with_page_sizes_and_pool_sizes_of_their_own():
+    """Two groups that differ in both: runs that keep every key in pages of 4 tokens, 10 of them, and a run with a
+    window of 6 that asks for pages of 2 tokens and gets a pool of 7.  Each group's tables, claims and returns go
+    by its own page size; content sharing is off (a page does not hold the same tokens in both)."""
+    needs = [KVNeed(2, 16), KVNeed(1, 32, window=6, page_size=2), KVNeed(2, 16)]
+    m = CacheManager(needs, [None, None, None], page_size=4, num_pages=[10, 7], max_requests=3, max_position=40, runtime=None)
+    full, win = m.groups
+    assert (full.page_size, full.pool.num_pages, full.runs) == (4, 10, [0, 2])
+    assert (win.page_size, win.pool.num_pages, win.runs) == (2, 7, [1])
+    assert not m.share and m.view(1).page_size == 2 and m.view(2).page_size == 4
+    # one number for every group: the same tokens in each pool
+    same = CacheManager(needs, [None, None, None], page_size=4, num_pages=10, max_requests=3, max_position=40, runtime=None)
+    assert [g.pool.num_pages for g in same.groups] == [10, 20]
+    r = m.open("r")
+    assert [len(row) for row in r.rows] == [10, 20]
+    for n in (5, 4, 1, 1, 6):
+        m.reserve([(r, n)])
+        m.commit(r, [1] * n)
+        m.check()
+        assert len(r.tables[0]) == -(-r.length // 4) and len(r.tables[1]) == -(-r.length // 2)
+        first_needed = max(0, r.length - 6 + 1)
+        assert all((page < 0) == ((block + 1) * 2 <= first_needed) for block, page in enumerate(r.tables[1]))
+        assert all(page >= 0 for page in r.tables[0])
+    # 17 tokens: 5 pages of 4; of the 9 pages of 2 the window keeps those from position 12 on
+    assert m.free_pages() == [10 - 5, 7 - 3]
+    # what a scheduler must keep free for it up to 40 tokens in steps of at most 4: every block of the first group,
+    # and in the windowed one the distance to the most it ever holds, the pages of 6 - 1 + 4 tokens and one more
+    assert m.pages_bound(r, 40, 4) == [10 - 5, 6 - 3]
+    assert m.pages_bound(None, 40, 4) == [10, 6]
+    with pytest.raises(OutOfPages):
+        m.reserve([(r, 23)])                       # 40 tokens: 20 pages of 2, 12 of them beyond what it has, 4 free
+    assert m.free_pages() == [5, 4]
+    m.close("r")
+    assert m.free_pages() == [10, 7]
+    m.check()

@@ -278,3 +278,60 @@ def test_trace_run(model_folders, tiny_configs, tmp_path, dtype, key, page, cut)
     tol = H.NMSE_F32 if dtype == "float32" else H.NMSE_BF16["tiny"]
     for rid, toks in requests.items():
         H.assert_close(np.concatenate(rows[rid]), H.plain_logits(folder, toks), tol, f"trace {key} page {page} {cut} {dtype} {rid}")
+
+
+def _run_trace(folder, dtype, out, lines, *options):
+    proc = subprocess.run([os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype, "--out", str(out), *options],
+                          input="\n".join(lines) + "\n", capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert proc.stdout.split() == [w for i in range(len(lines)) for w in ("done", str(i))]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_with_requests_that_share_a_beginning(model_folders, tiny_configs, tmp_path, dtype):
+    """--share: a request whose first tokens an earlier request left in the cache adopts those pages (whole pages,
+    none that holds a wanted place) and runs the rest only; the logits at the wanted places are the plain ones.
+    Pages of 24 tokens, which do not divide 64."""
+    folder, vocab = model_folders[("b", dtype)], tiny_configs["b"]["vocab_size"]
+    first = H.random_tokens(1, 70, vocab)
+    second = first[:50] + H.random_tokens(2, 30, vocab)
+    third = first[:50] + H.random_tokens(3, 11, vocab)
+    lines = [json.dumps(rec) for rec in (
+        {"step": 0, "entries": [{"id": "a", "tokens": first[:40], "want": []}], "end": []},
+        {"step": 1, "entries": [{"id": "a", "tokens": first[40:], "want": [25, 29]}], "end": ["a"]},
+        # b adopts two pages (48 of the 50 tokens it has in common with a); c wants a place inside them and adopts one
+        {"step": 2, "entries": [{"id": "b", "tokens": second, "want": list(range(60, 80))},
+                                {"id": "c", "tokens": third[:45], "want": [30, 44]}], "end": []},
+        {"step": 3, "entries": [{"id": "c", "tokens": third[45:], "want": list(range(16))}], "end": ["b", "c"]},
+        # the pages a, b and c left are used again by a request that shares nothing
+        {"step": 4, "entries": [{"id": "d", "tokens": H.random_tokens(4, 128, vocab), "want": [127]}], "end": ["d"]},
+    )]
+    out = tmp_path / "out"
+    _run_trace(folder, dtype, out, lines, "--max-tokens", "192", "--page", "24", "--share")
+    tol = H.NMSE_F32 if dtype == "float32" else H.NMSE_BF16["tiny"]
+
+    def rows(step):
+        return np.fromfile(out / f"{step}.f32", dtype="<f4").reshape(-1, vocab)
+    assert not (out / "0.f32").exists()
+    ref_a, ref_b, ref_c = (H.plain_logits(folder, t) for t in (first, second, third))
+    H.assert_close(rows(1), ref_a[[65, 69]], tol, f"shared trace {dtype} a")
+    got = rows(2)
+    H.assert_close(got[:20], ref_b[60:80], tol, f"shared trace {dtype} b")
+    H.assert_close(got[20:], ref_c[[30, 44]], tol, f"shared trace {dtype} c")
+    H.assert_close(rows(3), ref_c[45:], tol, f"shared trace {dtype} c, second step")
+    H.assert_close(rows(4), H.plain_logits(folder, H.random_tokens(4, 128, vocab))[[127]], tol, f"shared trace {dtype} d")
+
+
+def test_two_bfloat16_replays_write_the_same_bytes(model_folders, tiny_configs, tmp_path):
+    """The products of a portion of some hundred rows run on the engine's own kernel in the cut that gives the planned
+    bits, whichever cut a process finds fastest: two processes write the same bytes."""
+    folder, vocab = model_folders[("b", "bfloat16")], tiny_configs["b"]["vocab_size"]
+    toks = H.random_tokens(9, 240, vocab)
+    lines = [json.dumps({"step": 0, "entries": [{"id": "x", "tokens": toks[:230], "want": [0, 100, 229]}], "end": []}),
+             json.dumps({"step": 1, "entries": [{"id": "x", "tokens": toks[230:], "want": [9]}], "end": ["x"]})]
+    for name in ("one", "two"):
+        _run_trace(folder, "bfloat16", tmp_path / name, lines, "--max-tokens", "256")
+    for step in (0, 1):
+        assert (tmp_path / "one" / f"{step}.f32").read_bytes() == (tmp_path / "two" / f"{step}.f32").read_bytes()
+    H.assert_close(np.fromfile(tmp_path / "one" / "0.f32", dtype="<f4").reshape(-1, vocab), H.plain_logits(folder, toks)[[0, 100, 229]],
+                   H.NMSE_BF16["tiny"], "replayed twice")

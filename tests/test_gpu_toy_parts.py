@@ -557,7 +557,7 @@ def _register_geometries():
             wide = AttentionSpec(G_HIDDEN, 4, 2, 32, position=RopeSpec(32, THETA, pairing="interleaved"), qk_norm_eps=EPS,
                                  prefix="layers.0.attn.")
             narrow = AttentionSpec(G_HIDDEN, 6, 1, 16, position=RopeSpec(16, 50.0, rotary_dim=8), qk_norm_eps=None,
-                                   window=G_WINDOW, prefix="layers.1.attn.")
+                                   window=G_WINDOW, prefix="layers.1.attn.", page_size=self.d.get("narrow_page"))
             return ModelSpec("ToyGeometriesForTests", G_HIDDEN, VOCAB, G_POSITIONS, EmbeddingSpec(VOCAB, G_HIDDEN, "embed."),
                              (layer(0, wide), layer(1, narrow)), (LayerRun(0), LayerRun(1)), RMSNormSpec(G_HIDDEN, EPS, "norm."),
                              HeadSpec(VOCAB, G_HIDDEN, False, "head."),
@@ -641,6 +641,60 @@ def test_two_attention_geometries_a_window_and_a_learned_position(tmp_path, dtyp
         assert cache.free_pages() == [g.pool.num_pages for g in cache.groups]
         if dtype == "bfloat16":
             assert engine.rt.generic_attention_launches == 0                # both geometries ran on the matrix-core kernels
+    finally:
+        unregister_architecture("ToyGeometriesForTests")
+        unregister("position", "toy_learned_position")
+
+
+def _peak_window_pages(requests, steps, page, window):
+    """Most pages a group with `window` holds over `steps`: a step claims a page for every new block first (a portion's
+    early rows still see keys that its late rows have left behind) and gives back, afterwards, the pages that lie wholly
+    behind the window of the next query."""
+    length, blocks, held = {}, {}, {}
+    peak = 0
+    for entries, ends in steps:
+        for rid, n in entries:
+            length[rid] = length.get(rid, 0) + n
+            new_blocks = -(-length[rid] // page)
+            held.setdefault(rid, set()).update(range(blocks.get(rid, 0), new_blocks))
+            blocks[rid] = new_blocks
+        peak = max(peak, sum(len(h) for h in held.values()))
+        for rid, _ in entries:
+            first_needed = max(0, length[rid] - window + 1)
+            held[rid] = {b for b in held[rid] if (b + 1) * page > first_needed}
+        for rid in ends:
+            del length[rid], blocks[rid], held[rid]
+    return peak
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("cut", ["tail", "mixed"])
+def test_cache_groups_with_page_sizes_and_pools_of_their_own(tmp_path, dtype, cut):
+    """The same two-geometry model, the windowed layer asking for pages of 4 tokens where the engine's are 8, and the
+    two pools sized apart: the full-attention group for the contexts of the live requests, the windowed one for
+    their windows only (fewer tokens than the contexts hold).  Block tables, claims and returns go by each group's
+    own page size, in a step that launches both geometries."""
+    from kipp_amd.config import unregister_architecture
+    from kipp_amd.engine import Engine
+    from kipp_amd.parts import unregister
+    from kipp_amd.weights import write_random_model
+    _register_geometries()
+    try:
+        folder = write_random_model(str(tmp_path / "geometries"), {"architectures": ["ToyGeometriesForTests"], "narrow_page": 4},
+                                    seed=15, dtype=dtype)
+        _, weights = plain.load_folder(folder)
+        requests = {f"g{i}": H.random_tokens(80 + i, n, VOCAB) for i, n in enumerate([9, 70, 41, 90, 33])}
+        steps = {"tail": H.tail_one_by_one, "mixed": lambda r: H.mixed(r, seed=8)}[cut](requests)
+        full, windowed = H.peak_pages(requests, steps, 8), _peak_window_pages(requests, steps, 4, G_WINDOW)
+        assert windowed * 4 < full * 8                                      # the windowed pool holds fewer tokens
+        engine = Engine.from_folder(folder, dtype=dtype, page_size=8, num_pages=[full, windowed], max_requests=4)
+        cache = engine.cache
+        assert [(g.page_size, g.pool.num_pages) for g in cache.groups] == [(8, full), (4, windowed)]
+        got = H.replay(engine, requests, steps)
+        tol = H.NMSE_F32 if dtype == "float32" else H.NMSE_BF16["tiny"]
+        for rid, toks in requests.items():
+            H.assert_close(got[rid], _plain_geometries(weights, toks), tol, f"two pools/{dtype}/{cut}/{rid}")
+        assert cache.free_pages() == [full, windowed]
     finally:
         unregister_architecture("ToyGeometriesForTests")
         unregister("position", "toy_learned_position")

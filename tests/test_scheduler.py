@@ -288,3 +288,29 @@ def test_a_failed_step_leaves_requests_outside_it_running():
     assert ok.output == expected_output(list(ok.prompt), 3)
     assert sched.stats.failed == 1 and eng.cache.free_pages() == [8]
     eng.cache.check()
+
+
+def test_a_windowed_group_with_a_small_pool_of_its_own():
+    """A model whose second run keeps a window of 6 keys in pages of 2: its pool is sized for the windows of the
+    running requests, not for their whole contexts, and admission counts what each may still hold there."""
+    class TwoGroups(FakeEngine):
+        def __init__(self):
+            self.cache = CacheManager([KVNeed(1, 16), KVNeed(1, 16, window=6, page_size=2)], [None, None], 4, [24, 14],
+                                      max_requests=4, max_position=64, runtime=None, share_prefixes=False)
+            self.vocab_size = VOCAB
+            self.calls = []
+    eng = TwoGroups()
+    sched = Scheduler(eng, max_step_tokens=8, prefill_chunk=4)
+    # a request holds at most the pages of 6 - 1 + 4 tokens and one more in the windowed group: 6 of 14, so two run and a third waits
+    for name, prompt in (("a", list(range(1, 21))), ("b", list(range(2, 19))), ("c", [5, 6, 7])):
+        sched.add(Request(name, prompt, 12))
+    sched.step()
+    assert [r.id for r in sched.running] == ["a", "b"] and [r.id for r in sched.waiting] == ["c"]
+    done = sched.run(max_steps=200)
+    for name, prompt in (("a", list(range(1, 21))), ("b", list(range(2, 19))), ("c", [5, 6, 7])):
+        assert done[name].output == expected_output(prompt, 12)
+    assert eng.cache.free_pages() == [24, 14] and sched.stats.waits_for_pages > 0
+    with pytest.raises(RequestRefused):
+        big = Scheduler(eng, max_step_tokens=64, prefill_chunk=32)      # steps of 32 tokens: 19 pages of 2 at once
+        big.add(Request("d", list(range(40)), 2))
+    eng.cache.check()
