@@ -150,6 +150,39 @@ def build_all(specs: Iterable[Tuple[str, Optional[dict]]], jobs: int = 8, force:
             if time.time() - last > 10:
                 last = time.time()
                 _say(f"still compiling {', '.join(r[0] for r in running)} ({last - started:.0f} s)")
+    if started != last or force or not os.path.exists(os.path.join(HERE, "_lib", "MANIFEST")):
+        write_manifest()
+
+
+def write_manifest() -> Optional[str]:
+    """`MANIFEST` in the in-tree folder: a line "<name>[.<CONSTANT><value>...] <file>" for every library there that is the
+    current build of its source (a host that is no Python, the C one, finds the kernels by it).  Returns its
+    path, or None where the folder cannot be written."""
+    import re
+    folder = os.path.join(HERE, "_lib")
+    if not os.path.isdir(folder):
+        return None
+    lines = []
+    for f in sorted(os.listdir(folder)):
+        m = re.fullmatch(r"libkipp_([a-z0-9_]+?)((?:\.[A-Z_]+[0-9]+)*)\.([0-9a-f]{10})\.so", f)
+        if not m:
+            continue
+        name, tag = m.group(1), m.group(2)
+        defines = {k: int(v) for k, v in re.findall(r"\.([A-Z_]+?)([0-9]+)(?=\.|$)", tag)} or None
+        try:
+            current = os.path.basename(library_path(name, defines)[0])
+        except BuildError:
+            continue
+        if current == f:
+            lines.append(f"{name}{tag} {f}")
+    try:
+        tmp = os.path.join(folder, f".MANIFEST.{os.getpid()}")
+        with open(tmp, "w") as out:
+            out.write("\n".join(lines) + "\n")
+        os.replace(tmp, os.path.join(folder, "MANIFEST"))
+    except OSError:
+        return None
+    return os.path.join(folder, "MANIFEST")
 
 
 def library(name: str, defines: Optional[dict] = None) -> ctypes.CDLL:

@@ -1,0 +1,679 @@
+/*
+ * The GPU's table of operations: the launchers of the kernel libraries
+ * (csrc/<name>.hip, each built into its own shared library) on buffers from
+ * hipMalloc, one stream of the default priority, in bfloat16 (the kernels that
+ * serving uses) or in true float32 (plain FMA products, the generic attention).
+ * The libraries are opened at their first use; one that is missing, or a launch
+ * that a kernel refuses, is an error with its name: there is no other path
+ * behind any operation.
+ *
+ * Which file holds a kernel: <kernel_dir>/MANIFEST lists "<name>[.<constants>] <file>"
+ * for the current builds (written by kipp_amd.csrc.build); without it the folder
+ * is searched for libkipp_<name>[.<constants>].<10 hex digits>.so and the newest is taken.
+ */
+#define __HIP_PLATFORM_AMD__ 1
+#include <dirent.h>
+#include <dlfcn.h>
+#include <hip/hip_runtime_api.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+#include <sys/stat.h>
+#include <unistd.h>
+
+#include "backend.h"
+
+#define PREFILL_MAX_BLOCKS 4096 /* table entries of one sequence the kernel for portions stages */
+
+typedef int (*fn_embed)(const void *, int, const int32_t *, float *, int, int, hipStream_t);
+typedef int (*fn_rmsnorm)(float *, const void *, int, int, const float *, void *, int, int, int, float, hipStream_t);
+typedef int (*fn_residual_add)(float *, const void *, int, int, size_t, hipStream_t);
+typedef int (*fn_swiglu)(const void *, int, int, void *, int, int, int, int, hipStream_t);
+typedef int (*fn_cast)(const void *, int, void *, int, size_t, hipStream_t);
+typedef int (*fn_gather_rows)(const void *, const int32_t *, void *, int, int, hipStream_t);
+typedef int (*fn_fill_zero)(void *, size_t, hipStream_t);
+typedef int (*fn_rotary_angles)(const int32_t *, const float *, float *, int, int, hipStream_t);
+typedef int (*fn_qk_norm_rope_kv)(const void *, int, void *, int, void *, void *, int, const int32_t *, const int32_t *, const int32_t *, int,
+                                  const float *, const float *, float, const float *, const float *, int, int, int, int, int, int, int, int,
+                                  int, hipStream_t);
+typedef int (*fn_attention_generic)(const void *, int, const void *, const void *, int, void *, int, const int32_t *, const int32_t *,
+                                    const int32_t *, int, int, int, int, int, int, float, int, hipStream_t);
+typedef int (*fn_attention_prefill)(const void *, const void *, const void *, void *, const int32_t *, const int32_t *, const int32_t *,
+                                    const int32_t *, const int32_t *, const int32_t *, int, int, int, int, int, int, float, int, int,
+                                    const int32_t *, int, float *, float *, int, const int32_t *, const int32_t *, int, hipStream_t);
+typedef int (*fn_attention_decode)(const void *, const void *, const void *, void *, float *, float *, const int32_t *, const int32_t *,
+                                   const int32_t *, const int32_t *, int, int, int, int, int, int, float, int, int, int, int32_t *,
+                                   hipStream_t);
+typedef int (*fn_int_void)(void);
+typedef int (*fn_gemm_f32)(const float *, const void *, int, float *, int, int, int, hipStream_t);
+typedef int (*fn_skinny_parts)(int, int, int);
+typedef int (*fn_gemm_skinny)(const void *, const void *, float *, int, int, int, int, int, const float *, int, float, float *, const float *,
+                              void *, float *, hipStream_t);
+typedef int (*fn_rows_parts)(int, int, int, int);
+typedef int (*fn_gemm_rows)(const void *, const void *, float *, int, int, int, int, int, hipStream_t);
+typedef int (*fn_tiles_parts)(int, int, int, int, int);
+typedef int (*fn_gemm_tiles)(const void *, const void *, void *, int, int, int, int, int, int, hipStream_t);
+
+typedef struct {
+    uint32_t head_dim, group;
+    void *prefill_lib, *decode_lib;
+    fn_attention_prefill prefill;
+    fn_attention_decode decode;
+    int prefill_rows, split, split_min;
+} attention_variant;
+
+typedef struct {
+    int device;
+    hipStream_t stream;
+    char kernel_dir[3072];
+    void *libs[8];
+    size_t lib_count;
+    fn_embed embed;
+    fn_rmsnorm rmsnorm;
+    fn_residual_add residual_add;
+    fn_swiglu swiglu;
+    fn_cast cast;
+    fn_gather_rows gather_rows;
+    fn_fill_zero fill_zero;
+    fn_rotary_angles rotary_angles;
+    fn_qk_norm_rope_kv qk_norm_rope_kv;
+    fn_attention_generic attention_generic;
+    fn_gemm_f32 gemm_f32;
+    fn_skinny_parts skinny_parts;
+    fn_gemm_skinny gemm_skinny;
+    fn_rows_parts rows_parts;
+    fn_gemm_rows gemm_rows;
+    fn_tiles_parts tiles_parts;
+    fn_gemm_tiles gemm_tiles;
+    attention_variant variants[8];
+    size_t variant_count;
+    uint64_t generic_attention_launches; /* bfloat16 attention that fell to the generic kernel */
+} hip_state;
+
+static int hip_bad(kipp_error *error, hipError_t code, const char *what) {
+    return kipp_fail(error, code == hipErrorOutOfMemory ? KIPP_ERROR_MEMORY : KIPP_ERROR_INTERNAL, "%s: %s", what, hipGetErrorString(code));
+}
+
+/* ------------------------------------------------------------------ finding and opening the libraries */
+static int find_library(const hip_state *st, const char *key, char *path, size_t path_size, kipp_error *error) {
+    char manifest[4096], line[1024];
+    snprintf(manifest, sizeof(manifest), "%s/MANIFEST", st->kernel_dir);
+    FILE *f = fopen(manifest, "r");
+    if (f != NULL) {
+        size_t key_length = strlen(key);
+        while (fgets(line, sizeof(line), f) != NULL) {
+            if (strncmp(line, key, key_length) == 0 && line[key_length] == ' ') {
+                char *name = line + key_length + 1;
+                name[strcspn(name, "\r\n")] = '\0';
+                snprintf(path, path_size, "%s/%s", st->kernel_dir, name);
+                fclose(f);
+                if (access(path, R_OK) == 0) return 0;
+                return kipp_fail(error, KIPP_ERROR_IO, "%s names %s for %s, which is not there: build the kernels again", manifest, name, key);
+            }
+        }
+        fclose(f);
+    }
+    /* no manifest, or it does not know the key: libkipp_<key>.<10 hex digits>.so, the newest */
+    DIR *dir = opendir(st->kernel_dir);
+    if (dir == NULL) return kipp_fail(error, KIPP_ERROR_IO, "the folder of the kernel libraries, %s, cannot be read", st->kernel_dir);
+    char prefix[256];
+    snprintf(prefix, sizeof(prefix), "libkipp_%s.", key);
+    size_t prefix_length = strlen(prefix);
+    time_t newest = 0;
+    bool any = false;
+    struct dirent *entry;
+    while ((entry = readdir(dir)) != NULL) {
+        const char *name = entry->d_name;
+        if (strncmp(name, prefix, prefix_length) != 0 || strlen(name) != prefix_length + 13 || strcmp(name + prefix_length + 10, ".so") != 0) continue;
+        char candidate[4096];
+        struct stat info;
+        snprintf(candidate, sizeof(candidate), "%s/%s", st->kernel_dir, name);
+        if (stat(candidate, &info) == 0 && (!any || info.st_mtime > newest)) {
+            any = true;
+            newest = info.st_mtime;
+            snprintf(path, path_size, "%s", candidate);
+        }
+    }
+    closedir(dir);
+    if (!any)
+        return kipp_fail(error, KIPP_ERROR_IO, "no kernel library for %s in %s: build it first (python -m kipp_amd.csrc.build)", key, st->kernel_dir);
+    return 0;
+}
+
+static void *open_library(hip_state *st, const char *key, kipp_error *error) {
+    char path[4096];
+    if (find_library(st, key, path, sizeof(path), error) != 0) return NULL;
+    void *lib = dlopen(path, RTLD_NOW | RTLD_LOCAL);
+    if (lib == NULL) kipp_fail(error, KIPP_ERROR_IO, "cannot load %s: %s", path, dlerror());
+    return lib;
+}
+
+static void *symbol(void *lib, const char *name, kipp_error *error) {
+    void *fn = dlsym(lib, name);
+    if (fn == NULL) kipp_fail(error, KIPP_ERROR_INTERNAL, "a kernel library lacks %s", name);
+    return fn;
+}
+
+#define KIPP_SYM(lib, field, name)                                   \
+    do {                                                             \
+        *(void **)(&st->field) = symbol(lib, name, error);           \
+        if (st->field == NULL) return -1;                            \
+    } while (0)
+
+static int open_common(hip_state *st, kipp_error *error) {
+    static const char *const names[] = {"elementwise", "rope_kv", "attention_generic", "gemm_f32", "gemm_skinny", "gemm_rows", "gemm_tiles"};
+    void *libs[7];
+    for (size_t i = 0; i < 7; ++i) {
+        libs[i] = open_library(st, names[i], error);
+        if (libs[i] == NULL) return -1;
+        st->libs[st->lib_count++] = libs[i];
+    }
+    KIPP_SYM(libs[0], embed, "kipp_embed");
+    KIPP_SYM(libs[0], rmsnorm, "kipp_rmsnorm");
+    KIPP_SYM(libs[0], residual_add, "kipp_residual_add");
+    KIPP_SYM(libs[0], swiglu, "kipp_swiglu");
+    KIPP_SYM(libs[0], cast, "kipp_cast");
+    KIPP_SYM(libs[0], gather_rows, "kipp_gather_rows");
+    KIPP_SYM(libs[0], fill_zero, "kipp_fill_zero");
+    KIPP_SYM(libs[1], rotary_angles, "kipp_rotary_angles");
+    KIPP_SYM(libs[1], qk_norm_rope_kv, "kipp_qk_norm_rope_kv");
+    KIPP_SYM(libs[2], attention_generic, "kipp_paged_attention_generic");
+    KIPP_SYM(libs[3], gemm_f32, "kipp_gemm_f32");
+    KIPP_SYM(libs[4], skinny_parts, "kipp_gemm_skinny_parts");
+    KIPP_SYM(libs[4], gemm_skinny, "kipp_gemm_skinny");
+    KIPP_SYM(libs[5], rows_parts, "kipp_gemm_rows_parts");
+    KIPP_SYM(libs[5], gemm_rows, "kipp_gemm_rows");
+    KIPP_SYM(libs[6], tiles_parts, "kipp_gemm_tiles_parts");
+    KIPP_SYM(libs[6], gemm_tiles, "kipp_gemm_tiles");
+    return 0;
+}
+
+static attention_variant *variant_of(hip_state *st, uint32_t head_dim, uint32_t group, kipp_error *error) {
+    for (size_t i = 0; i < st->variant_count; ++i) {
+        if (st->variants[i].head_dim == head_dim && st->variants[i].group == group) return &st->variants[i];
+    }
+    if (st->variant_count == sizeof(st->variants) / sizeof(st->variants[0])) {
+        kipp_fail(error, KIPP_ERROR_UNSUPPORTED, "more attention geometries in one model than this table keeps");
+        return NULL;
+    }
+    attention_variant *v = &st->variants[st->variant_count];
+    char key[96];
+    memset(v, 0, sizeof(*v));
+    v->head_dim = head_dim;
+    v->group = group;
+    snprintf(key, sizeof(key), "attention_prefill.HEAD_DIM%u", head_dim);
+    if ((v->prefill_lib = open_library(st, key, error)) == NULL) return NULL;
+    snprintf(key, sizeof(key), "attention_decode.GROUP%u.HEAD_DIM%u", group, head_dim);
+    if ((v->decode_lib = open_library(st, key, error)) == NULL) return NULL;
+    *(void **)(&v->prefill) = symbol(v->prefill_lib, "kipp_attention_prefill", error);
+    *(void **)(&v->decode) = symbol(v->decode_lib, "kipp_attention_decode", error);
+    fn_int_void rows = NULL, split = NULL, split_min = NULL;
+    *(void **)(&rows) = symbol(v->prefill_lib, "kipp_attention_prefill_rows", error);
+    *(void **)(&split) = symbol(v->decode_lib, "kipp_attention_decode_split", error);
+    *(void **)(&split_min) = symbol(v->decode_lib, "kipp_attention_decode_split_min", error);
+    if (v->prefill == NULL || v->decode == NULL || rows == NULL || split == NULL || split_min == NULL) return NULL;
+    v->prefill_rows = rows();
+    v->split = split();
+    v->split_min = split_min();
+    ++st->variant_count;
+    return v;
+}
+
+/* ------------------------------------------------------------------ memory */
+static void hip_destroy(kipp_runtime *rt) {
+    hip_state *st = rt->state;
+    if (st != NULL) {
+        hipStreamSynchronize(st->stream);
+        if (st->stream != NULL) hipStreamDestroy(st->stream);
+        /* the libraries stay loaded: their kernels may be registered with the HIP runtime until the process ends */
+        free(st);
+    }
+    free(rt);
+}
+
+static void *hip_alloc(kipp_runtime *rt, size_t bytes, kipp_error *error) {
+    hip_state *st = rt->state;
+    void *memory = NULL;
+    hipError_t code = hipMalloc(&memory, bytes ? bytes : 256);
+    if (code != hipSuccess) {
+        hip_bad(error, code, "hipMalloc");
+        return NULL;
+    }
+    code = hipMemsetAsync(memory, 0, bytes ? bytes : 256, st->stream);
+    if (code != hipSuccess) {
+        hipFree(memory);
+        hip_bad(error, code, "hipMemsetAsync");
+        return NULL;
+    }
+    return memory;
+}
+
+static void hip_free(kipp_runtime *rt, void *memory) {
+    hip_state *st = rt->state;
+    hipStreamSynchronize(st->stream); /* nothing in flight may still use it */
+    hipFree(memory);
+}
+
+static int hip_zero(kipp_runtime *rt, void *memory, size_t bytes, kipp_error *error) {
+    hip_state *st = rt->state;
+    hipError_t code = hipMemsetAsync(memory, 0, bytes, st->stream);
+    return code == hipSuccess ? 0 : hip_bad(error, code, "hipMemsetAsync");
+}
+
+static int hip_upload(kipp_runtime *rt, void *to, const void *from_host, size_t bytes, kipp_error *error) {
+    hip_state *st = rt->state;
+    if (bytes == 0) return 0;
+    /* from pageable memory: the call returns once the bytes have left the host buffer */
+    hipError_t code = hipMemcpyAsync(to, from_host, bytes, hipMemcpyHostToDevice, st->stream);
+    return code == hipSuccess ? 0 : hip_bad(error, code, "copy to the GPU");
+}
+
+static int hip_download(kipp_runtime *rt, void *to_host, const void *from, size_t bytes, kipp_error *error) {
+    hip_state *st = rt->state;
+    hipError_t code = hipSuccess;
+    if (bytes != 0) code = hipMemcpyAsync(to_host, from, bytes, hipMemcpyDeviceToHost, st->stream);
+    if (code == hipSuccess) code = hipStreamSynchronize(st->stream);
+    return code == hipSuccess ? 0 : hip_bad(error, code, "copy from the GPU (or a kernel before it)");
+}
+
+static int hip_copy(kipp_runtime *rt, void *to, const void *from, size_t bytes, kipp_error *error) {
+    hip_state *st = rt->state;
+    hipError_t code = hipMemcpyAsync(to, from, bytes, hipMemcpyDeviceToDevice, st->stream);
+    return code == hipSuccess ? 0 : hip_bad(error, code, "copy on the GPU");
+}
+
+/* ------------------------------------------------------------------ placement */
+static float half_to_float(uint16_t bits) {
+    uint32_t sign = (uint32_t)(bits & 0x8000u) << 16, exponent = (bits >> 10) & 0x1f, fraction = bits & 0x3ffu, wide;
+    if (exponent == 0) {
+        if (fraction == 0) wide = sign;
+        else {
+            int shift = 0;
+            while (!(fraction & 0x400u)) {
+                fraction <<= 1;
+                ++shift;
+            }
+            wide = sign | ((uint32_t)(127 - 15 + 1 - shift) << 23) | ((fraction & 0x3ffu) << 13);
+        }
+    } else if (exponent == 31) wide = sign | 0x7f800000u | (fraction << 13);
+    else wide = sign | ((exponent + 127 - 15) << 23) | (fraction << 13);
+    float value;
+    memcpy(&value, &wide, sizeof(value));
+    return value;
+}
+
+/* The tensor's values as float32 in a buffer of the host (freed by the caller). */
+static float *widened(const kipp_tensor *tensor, size_t count, kipp_error *error) {
+    float *wide = malloc(count ? count * sizeof(float) : 4);
+    if (wide == NULL) {
+        kipp_fail(error, KIPP_ERROR_MEMORY, "out of memory widening %s", tensor->name);
+        return NULL;
+    }
+    if (tensor->dtype == KIPP_F32) memcpy(wide, tensor->data, count * sizeof(float));
+    else {
+        const uint16_t *narrow = tensor->data;
+        for (size_t i = 0; i < count; ++i) {
+            if (tensor->dtype == KIPP_BF16) {
+                uint32_t bits = (uint32_t)narrow[i] << 16;
+                memcpy(&wide[i], &bits, sizeof(float));
+            } else {
+                wide[i] = half_to_float(narrow[i]);
+            }
+        }
+    }
+    return wide;
+}
+
+static int hip_place_matrix(kipp_runtime *rt, const kipp_tensor *const *pieces, size_t piece_count, kipp_weight *out, kipp_error *error) {
+    uint64_t rows = 0, columns = pieces[0]->shape[1];
+    bool keep_bf16 = rt->act_dtype == KIPP_BF16;
+    for (size_t p = 0; p < piece_count; ++p) {
+        rows += pieces[p]->shape[0];
+        keep_bf16 = keep_bf16 && pieces[p]->dtype == KIPP_BF16; /* pieces of different types, and everything on the 32-bit path, are widened */
+    }
+    size_t count, bytes;
+    if (rows > INT32_MAX || columns > INT32_MAX || kipp_mul_size((size_t)rows, (size_t)columns, &count) != 0 ||
+        kipp_mul_size(count, keep_bf16 ? 2 : 4, &bytes) != 0)
+        return kipp_fail(error, KIPP_ERROR_RANGE, "a matrix of %llu x %llu is too large", (unsigned long long)rows, (unsigned long long)columns);
+    char *data = hip_alloc(rt, bytes, error);
+    if (data == NULL) return -1;
+    size_t at = 0;
+    for (size_t p = 0; p < piece_count; ++p) {
+        size_t n = (size_t)(pieces[p]->shape[0] * pieces[p]->shape[1]);
+        int rc;
+        if (keep_bf16 || pieces[p]->dtype == KIPP_F32) {
+            rc = hip_upload(rt, data + at, pieces[p]->data, n * (keep_bf16 ? 2 : 4), error); /* straight out of the mapped file */
+        } else {
+            float *wide = widened(pieces[p], n, error);
+            rc = wide == NULL ? -1 : hip_upload(rt, data + at, wide, n * 4, error);
+            if (rc == 0) rc = hip_download(rt, NULL, NULL, 0, error); /* the copy has left the buffer before it is freed */
+            free(wide);
+        }
+        if (rc != 0) {
+            hip_free(rt, data);
+            return -1;
+        }
+        at += n * (keep_bf16 ? 2 : 4);
+    }
+    *out = (kipp_weight){data, keep_bf16 ? KIPP_BF16 : KIPP_F32, (uint32_t)rows, (uint32_t)columns};
+    return 0;
+}
+
+static int hip_place_vector(kipp_runtime *rt, const kipp_tensor *tensor, float **out, kipp_error *error) {
+    size_t n = (size_t)tensor->shape[0];
+    float *wide = widened(tensor, n, error);
+    if (wide == NULL) return -1;
+    float *data = hip_alloc(rt, n * sizeof(float), error);
+    int rc = data == NULL ? -1 : hip_upload(rt, data, wide, n * sizeof(float), error);
+    if (rc == 0) rc = hip_download(rt, NULL, NULL, 0, error);
+    free(wide);
+    if (rc != 0) {
+        if (data != NULL) hip_free(rt, data);
+        return -1;
+    }
+    *out = data;
+    return 0;
+}
+
+static void hip_free_weight(kipp_runtime *rt, kipp_weight *weight) {
+    if (weight->data != NULL) hip_free(rt, weight->data);
+    weight->data = NULL;
+}
+
+/* ------------------------------------------------------------------ operations */
+static int refused(kipp_error *error, const char *what, int code) {
+    return kipp_fail(error, KIPP_ERROR_INTERNAL, "%s: launch failed or arguments refused (code %d)", what, code);
+}
+
+static int hip_embed(kipp_runtime *rt, const kipp_weight *table, const int32_t *tokens, float *out, uint32_t n, kipp_error *error) {
+    hip_state *st = rt->state;
+    int rc = st->embed(table->data, table->dtype, tokens, out, (int)n, (int)table->k, st->stream);
+    return rc == 0 ? 0 : refused(error, "embed", rc);
+}
+
+static int hip_rmsnorm(kipp_runtime *rt, float *x, const kipp_delta *delta, const float *weight, void *out, uint32_t rows, uint32_t width,
+                       float eps, kipp_error *error) {
+    hip_state *st = rt->state;
+    int rc = st->rmsnorm(x, delta != NULL ? delta->data : NULL, KIPP_F32, delta != NULL ? delta->parts : 1, weight, out, rt->act_dtype, (int)rows,
+                         (int)width, eps, st->stream);
+    return rc == 0 ? 0 : refused(error, "rmsnorm", rc);
+}
+
+static int hip_residual_add(kipp_runtime *rt, float *x, const kipp_delta *delta, uint32_t rows, uint32_t width, kipp_error *error) {
+    hip_state *st = rt->state;
+    int rc = st->residual_add(x, delta->data, KIPP_F32, delta->parts, (size_t)rows * width, st->stream);
+    return rc == 0 ? 0 : refused(error, "residual_add", rc);
+}
+
+/* x . w^T.  bfloat16 x bfloat16: up to 8 rows the kernel in which every wave streams its rows of w against all of x, up to
+ * 256 rows the one that stages x through LDS, beyond those the tiled matrix-core kernel (K a multiple of 32) or the staged
+ * one over runs of 256 rows; a shape none of them takes (K no multiple of 8, or below 32) and every float32 weight go
+ * through the plain float32 product. */
+static int hip_linear(kipp_runtime *rt, const void *x, const kipp_weight *w, uint32_t m, int max_parts, kipp_delta *out, kipp_error *error) {
+    hip_state *st = rt->state;
+    const int M = (int)m, N = (int)w->n, K = (int)w->k;
+    size_t count;
+    if (kipp_mul_size(m, w->n, &count) != 0 || count > SIZE_MAX / 64) return kipp_fail(error, KIPP_ERROR_RANGE, "a product's size overflows");
+    if (max_parts < 1) max_parts = 1;
+    int rc;
+    if (w->dtype == KIPP_BF16 && rt->act_dtype == KIPP_BF16 && K % 8 == 0 && K >= 32) {
+        if (M <= 8) {
+            int most = max_parts > 8 ? 8 : max_parts, parts = st->skinny_parts(N, K, most);
+            float *y = parts >= 1 ? kipp_scratch(rt, (size_t)parts * count * 4, error) : NULL;
+            if (y == NULL) return parts >= 1 ? -1 : refused(error, "gemm_skinny (its cut)", parts);
+            rc = st->gemm_skinny(x, w->data, y, M, N, K, most, 0, NULL, 0, 0.0f, NULL, NULL, NULL, NULL, st->stream);
+            *out = (kipp_delta){y, parts};
+            return rc == 0 ? 0 : refused(error, "gemm_skinny", rc);
+        }
+        if (M <= 256) {
+            int most = max_parts > 12 ? 12 : max_parts, parts = st->rows_parts(M, N, K, most);
+            float *y = parts >= 1 ? kipp_scratch(rt, (size_t)parts * count * 4, error) : NULL;
+            if (y == NULL) return parts >= 1 ? -1 : refused(error, "gemm_rows (its cut)", parts);
+            rc = st->gemm_rows(x, w->data, y, M, N, K, most, 0, st->stream);
+            *out = (kipp_delta){y, parts};
+            return rc == 0 ? 0 : refused(error, "gemm_rows", rc);
+        }
+        if (K % 32 == 0 && (uint64_t)(M > N ? M : N) * (uint64_t)K * 2 < ((uint64_t)1 << 32)) {
+            int most = max_parts > 4 ? 4 : max_parts, parts = st->tiles_parts(M, N, K, 0, most);
+            float *y = parts >= 1 ? kipp_scratch(rt, (size_t)parts * count * 4, error) : NULL;
+            if (y == NULL) return parts >= 1 ? -1 : refused(error, "gemm_tiles (its cut)", parts);
+            rc = st->gemm_tiles(x, w->data, y, M, N, K, 0, most, 0, st->stream);
+            *out = (kipp_delta){y, parts};
+            return rc == 0 ? 0 : refused(error, "gemm_tiles", rc);
+        }
+        float *y = kipp_scratch(rt, count * 4, error);
+        if (y == NULL) return -1;
+        for (int row = 0; row < M; row += 256) {
+            int rows = M - row < 256 ? M - row : 256;
+            rc = st->gemm_rows((const char *)x + (size_t)row * K * 2, w->data, y + (size_t)row * N, rows, N, K, 1, 0, st->stream);
+            if (rc != 0) return refused(error, "gemm_rows", rc);
+        }
+        *out = (kipp_delta){y, 1};
+        return 0;
+    }
+    const float *wide = x;
+    if (rt->act_dtype == KIPP_BF16) {
+        float *cast = kipp_scratch(rt, (size_t)m * w->k * 4, error);
+        if (cast == NULL) return -1;
+        rc = st->cast(x, KIPP_BF16, cast, KIPP_F32, (size_t)m * w->k, st->stream);
+        if (rc != 0) return refused(error, "cast", rc);
+        wide = cast;
+    }
+    float *y = kipp_scratch(rt, count * 4, error);
+    if (y == NULL) return -1;
+    rc = st->gemm_f32(wide, w->data, w->dtype, y, M, N, K, st->stream);
+    *out = (kipp_delta){y, 1};
+    return rc == 0 ? 0 : refused(error, "gemm_f32", rc);
+}
+
+static int hip_swiglu(kipp_runtime *rt, const kipp_delta *gate_up, void *out, uint32_t rows, uint32_t inner, kipp_error *error) {
+    hip_state *st = rt->state;
+    int rc = st->swiglu(gate_up->data, KIPP_F32, gate_up->parts, out, rt->act_dtype, (int)rows, (int)inner, 0, st->stream);
+    return rc == 0 ? 0 : refused(error, "swiglu", rc);
+}
+
+static int hip_rotary_angles(kipp_runtime *rt, const int32_t *positions, const float *inv_freq, uint32_t n, uint32_t half,
+                             const float **out_rotation, kipp_error *error) {
+    hip_state *st = rt->state;
+    float *angles = kipp_scratch(rt, (size_t)n * 2 * half * sizeof(float), error);
+    if (angles == NULL) return -1;
+    int rc = st->rotary_angles(positions, inv_freq, angles, (int)n, (int)half, st->stream);
+    *out_rotation = angles;
+    return rc == 0 ? 0 : refused(error, "rotary_angles", rc);
+}
+
+static int hip_qk_norm_rope_kv(kipp_runtime *rt, const kipp_delta *qkv, void *q_out, const kipp_cache_view *cache, const kipp_batch *batch,
+                               const kipp_attention_geometry *g, const float *q_norm_w, const float *k_norm_w, float eps,
+                               const float *rotation, uint32_t rotary_dim, int interleaved, kipp_error *error) {
+    hip_state *st = rt->state;
+    int rc = st->qk_norm_rope_kv(qkv->data, KIPP_F32, q_out, rt->act_dtype, cache->k, cache->v, rt->act_dtype, batch->positions,
+                                 batch->seq_of_token, batch->tables[cache->group], (int)batch->max_blocks, q_norm_w, k_norm_w, eps, NULL, rotation,
+                                 (int)rotary_dim, interleaved, (int)batch->n_tokens, (int)g->n_q, (int)g->n_kv, (int)g->head_dim,
+                                 (int)cache->page_tokens, cache->writable ? 1 : 0, qkv->parts, st->stream);
+    return rc == 0 ? 0 : refused(error, "qk_norm_rope_kv", rc);
+}
+
+static int compare_items(const void *a, const void *b) {
+    const int32_t *x = a, *y = b; /* (last key, entry, tile): the longest key range first, then in order */
+    if (x[0] != y[0]) return x[0] > y[0] ? -1 : 1;
+    if (x[1] != y[1]) return x[1] < y[1] ? -1 : 1;
+    return x[2] < y[2] ? -1 : (x[2] > y[2]);
+}
+
+/* The work list of the kernel for portions: (entry, tile of its query rows) for every entry that brings more than one
+ * token, the longest key range first.  Made by the first attention of a forward pass, shared by the others. */
+static int prefill_work(kipp_runtime *rt, kipp_batch *batch, int tile_rows, kipp_error *error) {
+    if (batch->item_seq != NULL) return 0;
+    size_t count = 0;
+    for (uint32_t i = 0; i < batch->n_seqs; ++i) {
+        if (batch->h_q_len[i] > 1) count += (size_t)(batch->h_q_len[i] + tile_rows - 1) / (size_t)tile_rows;
+    }
+    int32_t *items = malloc((count ? count : 1) * 3 * sizeof(int32_t)), *lists = malloc((count ? count : 1) * 2 * sizeof(int32_t));
+    if (items == NULL || lists == NULL) {
+        free(items);
+        free(lists);
+        return kipp_fail(error, KIPP_ERROR_MEMORY, "out of memory");
+    }
+    size_t at = 0;
+    for (uint32_t i = 0; i < batch->n_seqs; ++i) {
+        int n = batch->h_q_len[i], ctx = batch->h_ctx_len[i];
+        if (n <= 1) continue;
+        for (int t = 0; t * tile_rows < n; ++t, ++at) {
+            int last_row = (t + 1) * tile_rows < n ? (t + 1) * tile_rows : n;
+            items[3 * at] = ctx - n + last_row - 1;
+            items[3 * at + 1] = (int32_t)i;
+            items[3 * at + 2] = t;
+        }
+    }
+    qsort(items, count, 3 * sizeof(int32_t), compare_items);
+    for (size_t i = 0; i < count; ++i) {
+        lists[i] = items[3 * i + 1];
+        lists[count + i] = items[3 * i + 2];
+    }
+    int32_t *device = kipp_scratch(rt, (count ? count : 1) * 2 * sizeof(int32_t), error);
+    int rc = device == NULL ? -1 : hip_upload(rt, device, lists, count * 2 * sizeof(int32_t), error);
+    free(items);
+    free(lists);
+    if (rc != 0) return -1;
+    batch->item_seq = device;
+    batch->item_tile = device + count;
+    batch->n_items = (uint32_t)count;
+    return 0;
+}
+
+static int hip_attention(kipp_runtime *rt, const void *q, const kipp_cache_view *cache, void *out, kipp_batch *batch,
+                         const kipp_attention_geometry *g, kipp_error *error) {
+    hip_state *st = rt->state;
+    const uint32_t group = g->n_q / g->n_kv, page = cache->page_tokens;
+    const int32_t *table = batch->tables[cache->group];
+    int rc;
+    bool fast = rt->act_dtype == KIPP_BF16 && g->head_dim % 16 == 0 && group <= 16 && (page & (page - 1)) == 0 &&
+                batch->max_blocks <= PREFILL_MAX_BLOCKS;
+    if (!fast) {
+        /* the float32 path, and geometries the matrix-core kernels refuse (head sizes that are no multiple of 16, more than
+         * 16 query heads a key/value head, pages that are no power of two) */
+        if (rt->act_dtype == KIPP_BF16) ++st->generic_attention_launches;
+        rc = st->attention_generic(q, rt->act_dtype, cache->k, cache->v, rt->act_dtype, out, rt->act_dtype, batch->positions, batch->seq_of_token,
+                                   table, (int)batch->max_blocks, (int)batch->n_tokens, (int)g->n_q, (int)g->n_kv, (int)g->head_dim, (int)page,
+                                   g->scale, (int)g->window, st->stream);
+        return rc == 0 ? 0 : refused(error, "paged_attention_generic", rc);
+    }
+    attention_variant *v = variant_of(st, g->head_dim, group, error);
+    if (v == NULL) return -1;
+    if (batch->n_portions != 0) {
+        if (prefill_work(rt, batch, v->prefill_rows, error) != 0) return -1;
+        rc = v->prefill(q, cache->k, cache->v, out, batch->item_seq, batch->item_tile, batch->q_start, batch->q_len, batch->positions, table,
+                        (int)batch->max_blocks, (int)batch->n_items, (int)g->n_q, (int)g->n_kv, (int)g->head_dim, (int)page, g->scale,
+                        (int)g->window, v->prefill_rows, NULL, 0, NULL, NULL, 0, NULL, NULL, 0, st->stream);
+        if (rc != 0) return refused(error, "attention_prefill", rc);
+    }
+    if (batch->n_decode != 0) {
+        /* partial results of the splits, shared by the layers of one geometry within the step; without a count of
+         * finished splits the merge is a launch of its own */
+        const size_t max_splits = (batch->max_decode_ctx + (size_t)v->split_min - 1) / (size_t)v->split_min + 1;
+        const size_t key = ((size_t)g->n_q << 32) ^ ((size_t)g->head_dim << 16) ^ max_splits;
+        if (batch->decode_workspace[0] == NULL || batch->decode_workspace_key != key) {
+            size_t rows = (size_t)batch->n_decode * g->n_q * max_splits;
+            batch->decode_workspace[0] = kipp_scratch(rt, rows * g->head_dim * sizeof(float), error);
+            batch->decode_workspace[1] = kipp_scratch(rt, rows * 2 * sizeof(float), error);
+            if (batch->decode_workspace[0] == NULL || batch->decode_workspace[1] == NULL) return -1;
+            batch->decode_workspace_key = key;
+        }
+        uint32_t span = g->window != 0 && g->window < batch->max_decode_ctx ? g->window : batch->max_decode_ctx;
+        size_t need = (span + (size_t)v->split - 1) / (size_t)v->split + (g->window != 0 ? 1 : 0);
+        int grid = (int)(need < 1 ? 1 : (need > max_splits ? max_splits : need));
+        rc = v->decode(q, cache->k, cache->v, out, batch->decode_workspace[0], batch->decode_workspace[1], batch->decode_rows, batch->positions,
+                       batch->seq_of_token, table, (int)batch->max_blocks, (int)batch->n_decode, (int)g->n_q, (int)g->n_kv, (int)g->head_dim,
+                       (int)page, g->scale, (int)g->window, grid, (int)max_splits, NULL, st->stream);
+        if (rc != 0) return refused(error, "attention_decode", rc);
+    }
+    return 0;
+}
+
+static int hip_gather_rows(kipp_runtime *rt, const float *x, const int32_t *index, float *out, uint32_t n, uint32_t width, kipp_error *error) {
+    hip_state *st = rt->state;
+    int rc = st->gather_rows(x, index, out, (int)n, (int)width, st->stream);
+    return rc == 0 ? 0 : refused(error, "gather_rows", rc);
+}
+
+/* ------------------------------------------------------------------ making the table */
+static void default_kernel_dir(char *out, size_t size) {
+    const char *env = getenv("KIPP_AMD_KERNELS");
+    if (env != NULL && env[0] != '\0') {
+        snprintf(out, size, "%s", env);
+        return;
+    }
+    Dl_info info;
+    out[0] = '\0';
+    if (dladdr((void *)default_kernel_dir, &info) != 0 && info.dli_fname != NULL) {
+        /* this library lies in <package>/host/_lib; the kernels in <package>/csrc/_lib */
+        char here[3000];
+        snprintf(here, sizeof(here), "%s", info.dli_fname);
+        char *slash = strrchr(here, '/');
+        if (slash != NULL) {
+            *slash = '\0';
+            snprintf(out, size, "%s/../../csrc/_lib", here);
+        }
+    }
+}
+
+kipp_runtime *kipp_runtime_hip(kipp_path path, int device, const char *kernel_dir, kipp_error *error) {
+    int count = 0;
+    hipError_t code = hipGetDeviceCount(&count);
+    if (code != hipSuccess || count <= 0) {
+        kipp_fail(error, KIPP_ERROR_UNSUPPORTED, "no GPU visible: the paths gpu-bf16 and gpu-fp32 run on a gfx950 GPU only (cpu-fp32 needs none)");
+        return NULL;
+    }
+    if (device < 0 || device >= count) {
+        kipp_fail(error, KIPP_ERROR_ARGUMENT, "GPU %d of %d", device, count);
+        return NULL;
+    }
+    kipp_runtime *rt = calloc(1, sizeof(*rt));
+    hip_state *st = calloc(1, sizeof(*st));
+    if (rt == NULL || st == NULL) {
+        free(rt);
+        free(st);
+        kipp_fail(error, KIPP_ERROR_MEMORY, "out of memory");
+        return NULL;
+    }
+    rt->state = st;
+    st->device = device;
+    if (kernel_dir != NULL && kernel_dir[0] != '\0') snprintf(st->kernel_dir, sizeof(st->kernel_dir), "%s", kernel_dir);
+    else default_kernel_dir(st->kernel_dir, sizeof(st->kernel_dir));
+    if ((code = hipSetDevice(device)) != hipSuccess || (code = hipStreamCreate(&st->stream)) != hipSuccess) {
+        hip_bad(error, code, "hipSetDevice / hipStreamCreate");
+        free(st);
+        free(rt);
+        return NULL;
+    }
+    if (open_common(st, error) != 0) {
+        hipStreamDestroy(st->stream);
+        free(st);
+        free(rt);
+        return NULL;
+    }
+    rt->name = path == KIPP_PATH_GPU_BF16 ? "gpu-bf16" : "gpu-fp32";
+    rt->path = path;
+    rt->act_dtype = path == KIPP_PATH_GPU_BF16 ? KIPP_BF16 : KIPP_F32;
+    rt->on_host = false;
+    rt->destroy = hip_destroy;
+    rt->mem_alloc = hip_alloc;
+    rt->mem_free = hip_free;
+    rt->mem_zero = hip_zero;
+    rt->upload = hip_upload;
+    rt->download = hip_download;
+    rt->copy = hip_copy;
+    rt->place_matrix = hip_place_matrix;
+    rt->place_vector = hip_place_vector;
+    rt->free_weight = hip_free_weight;
+    rt->embed = hip_embed;
+    rt->rmsnorm = hip_rmsnorm;
+    rt->residual_add = hip_residual_add;
+    rt->linear = hip_linear;
+    rt->swiglu = hip_swiglu;
+    rt->rotary_angles = hip_rotary_angles;
+    rt->qk_norm_rope_kv = hip_qk_norm_rope_kv;
+    rt->attention = hip_attention;
+    rt->gather_rows = hip_gather_rows;
+    return rt;
+}

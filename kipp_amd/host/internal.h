@@ -113,6 +113,7 @@ typedef struct {
 #define KIPP_MAX_ROLES 6
 typedef struct {
     char block[24];
+    uint32_t hidden; /* width of the residual stream */
     kipp_role_spec roles[KIPP_MAX_ROLES];
     uint32_t role_count;
 } kipp_layer_spec;
@@ -321,8 +322,8 @@ typedef struct {
     uint32_t n_items;
     size_t capacity; /* ints the two buffers hold */
     /* values of this forward pass that parts share */
-    float *angles;
-    const float *angles_of; /* the table of frequencies they were made from */
+    const float *rotation;    /* what the table's rotary_angles made */
+    const float *rotation_of; /* the frequencies it was made from */
     void *decode_workspace[3];
     size_t decode_workspace_key;
 } kipp_batch;
@@ -414,5 +415,9 @@ struct kipp_model {
 
 int kipp_model_params(const kipp_model_spec *spec, kipp_param_list *out, kipp_error *error);
 int kipp_model_forward(kipp_model *model, kipp_batch *batch, float **out_logits, kipp_error *error);
+int kipp_embedding_forward(void *part, const int32_t *tokens, float *out, uint32_t n, kipp_error *error);
+int kipp_head_forward(void *part, const void *x, uint32_t rows, kipp_delta *out, kipp_error *error);
+uint64_t kipp_weight_bytes(const kipp_weight *w);
+int kipp_check_tensors(const char *where, kipp_tensor_file *found, const kipp_param_list *expected, kipp_error *error);
 
 #endif
