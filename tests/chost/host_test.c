@@ -1,0 +1,316 @@
+/*
+ * The host logic of the C library under AddressSanitizer and UndefinedBehaviorSanitizer
+ * (the reference builds its own host the same way, /root/reference/Makefile): the JSON reader, checked sizes,
+ * the page pool and the cache manager under random orders of sessions, a model folder opened
+ * and stepped on the scalar path under several cuttings with scrambled block tables, the error paths
+ * of the step function, and the sampler.  The GPU's table is not part of this build.
+ *
+ *   host_test MODEL_DIR [MODEL_DIR ...]      exit code 0 and a last line "ok <checks>" on success
+ */
+#include <math.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include "internal.h"
+
+static int checks, failures;
+#define CHECK(cond)                                                            \
+    do {                                                                       \
+        ++checks;                                                              \
+        if (!(cond)) {                                                         \
+            ++failures;                                                        \
+            fprintf(stderr, "FAILED %s:%d: %s\n", __FILE__, __LINE__, #cond); \
+        }                                                                      \
+    } while (0)
+
+static uint64_t rng_state = 0x9e3779b97f4a7c15ull;
+static uint32_t rnd(uint32_t below) {
+    rng_state ^= rng_state >> 12;
+    rng_state ^= rng_state << 25;
+    rng_state ^= rng_state >> 27;
+    return (uint32_t)(((rng_state * 2685821657736338717ull) >> 33) % below);
+}
+
+static void test_json(void) {
+    kj_doc doc;
+    kipp_error error;
+    const char *good = "{\"a\": [1, 2.5, -3e2, true, null], \"b\": {\"c\": \"x\\u00e9\\ud83d\\ude00\\n\"}, \"d\": 9007199254740993}";
+    CHECK(kj_parse(good, strlen(good), &doc, &error) == 0);
+    const kj_node *root = kj_root(&doc), *a = kj_get(&doc, root, "a");
+    CHECK(root->type == KJ_OBJECT && root->count == 3 && a != NULL && a->type == KJ_ARRAY && a->count == 5);
+    const kj_node *item = kj_first(&doc, a);
+    CHECK(item->is_integer && item->integer == 1);
+    item = kj_next(&doc, item);
+    CHECK(!item->is_integer && item->number == 2.5);
+    item = kj_next(&doc, item);
+    CHECK(!item->is_integer && item->number == -300.0);
+    item = kj_next(&doc, item);
+    CHECK(item->type == KJ_BOOL && item->boolean);
+    item = kj_next(&doc, item);
+    CHECK(item->type == KJ_NULL && kj_next(&doc, item) == NULL);
+    const kj_node *c = kj_get(&doc, kj_get(&doc, root, "b"), "c");
+    CHECK(c != NULL && strcmp(c->string, "x\xc3\xa9\xf0\x9f\x98\x80\n") == 0 && c->string_length == 8);
+    CHECK(kj_get(&doc, root, "d")->is_integer && kj_get(&doc, root, "d")->integer == 9007199254740993ll);
+    CHECK(kj_get(&doc, root, "nope") == NULL);
+    kj_free(&doc);
+    static const char *const bad[] = {"", "{", "{\"a\": 1,}", "{\"a\": 1} x", "{\"a\": 1, \"a\": 2}", "[01]", "[1.]", "[.5]", "[1e]", "[NaN]",
+                                      "[Infinity]", "\"\\ud800\"", "\"\\udc00\"", "\"\\u12\"", "\"a\nb\"", "\"\\x\"", "[1 2]", "{1: 2}", "{\"a\" 1}",
+                                      "'a'", "[\"\\u0000\"]", "tru", "[1e999]", "-", "\"abc"};
+    for (size_t i = 0; i < sizeof(bad) / sizeof(bad[0]); ++i) {
+        CHECK(kj_parse(bad[i], strlen(bad[i]), &doc, &error) != 0);
+        CHECK(error.code == KIPP_ERROR_FORMAT);
+    }
+    char deep[200];
+    memset(deep, '[', 70);
+    memset(deep + 70, ']', 70);
+    CHECK(kj_parse(deep, 140, &doc, &error) != 0);
+    memset(deep, '[', 60);
+    memset(deep + 60, ']', 60);
+    CHECK(kj_parse(deep, 120, &doc, &error) == 0);
+    kj_free(&doc);
+    /* a text that is not nul-terminated at its length */
+    char *exact = malloc(7);
+    memcpy(exact, "[1, 23]", 7);
+    CHECK(kj_parse(exact, 7, &doc, &error) == 0 && kj_root(&doc)->count == 2);
+    kj_free(&doc);
+    CHECK(kj_parse(exact, 6, &doc, &error) != 0);
+    free(exact);
+}
+
+static void test_sizes(void) {
+    size_t out = 0;
+    CHECK(kipp_add_size(SIZE_MAX - 1, 1, &out) == 0 && out == SIZE_MAX);
+    CHECK(kipp_add_size(SIZE_MAX, 1, &out) != 0);
+    CHECK(kipp_mul_size(SIZE_MAX / 2, 2, &out) == 0 && kipp_mul_size(SIZE_MAX / 2 + 1, 2, &out) != 0 && kipp_mul_size(0, SIZE_MAX, &out) == 0);
+    CHECK(kipp_test_float_to_bf16(1.0f) == 0x3f80 && kipp_test_float_to_bf16(-2.0f) == 0xc000); /* /root/reference/tests/kipp_test.c:56-62 */
+    CHECK(isinf(kipp_test_bf16_to_float(0x7f80)) && kipp_test_bf16_to_float(kipp_test_float_to_bf16(1.00390625f)) == 1.0f);
+    CHECK(kipp_test_float_to_bf16(1.01171875f) == 0x3f82); /* 1 + 3/256: a tie, to the even neighbour above */
+}
+
+/* /root/reference/tests/kipp_test.c:3092-3392 has the reference's pool scenarios; these are their invariants under random orders */
+static void test_pool(void) {
+    kipp_pool pool;
+    kipp_error error;
+    const uint32_t pages = 13, page_tokens = 4;
+    CHECK(kipp_pool_init(&pool, pages, page_tokens, NULL, &error) == 0);
+    uint32_t held[64], n_held = 0, tokens[4];
+    for (int round = 0; round < 4000; ++round) {
+        uint32_t action = rnd(10);
+        if (action < 4) {
+            uint32_t page = kipp_pool_alloc(&pool);
+            CHECK((page == KIPP_NO_PAGE) == (pool.free_count == 0 && page == KIPP_NO_PAGE));
+            if (page != KIPP_NO_PAGE) held[n_held++] = page;
+        } else if (action < 7 && n_held > 0) {
+            uint32_t at = rnd(n_held);
+            CHECK(kipp_pool_release(&pool, held[at]) == 0);
+            held[at] = held[--n_held];
+        } else if (action < 9 && n_held > 0) {
+            uint32_t at = rnd(n_held);
+            for (int i = 0; i < 4; ++i) tokens[i] = rnd(2);
+            if (!kipp_pool_is_indexed(&pool, held[at]) && pool.pages[held[at]].ref_count == 1) kipp_pool_seal(&pool, held[at], rnd(2), tokens);
+        } else if (n_held < 60) {
+            uint32_t sequence[9], got[2];
+            for (int i = 0; i < 9; ++i) sequence[i] = rnd(2);
+            uint32_t matched = kipp_pool_prefix_match(&pool, sequence, 9, got, 2, NULL);
+            CHECK(matched <= 2);
+            for (uint32_t i = 0; i < matched; ++i) held[n_held++] = got[i];
+        }
+        if (kipp_pool_check(&pool, &error) != 0) {
+            CHECK(0);
+            fprintf(stderr, "%s\n", error.message);
+            break;
+        }
+        uint32_t referenced = 0;
+        for (uint32_t p = 0; p < pages; ++p) referenced += pool.pages[p].ref_count;
+        CHECK(referenced == n_held && pool.free_count <= pages);
+    }
+    CHECK(kipp_pool_release(&pool, 99) != 0);
+    while (n_held > 0) kipp_pool_release(&pool, held[--n_held]);
+    CHECK(pool.free_count == pages);
+    kipp_pool_free(&pool);
+    /* a collision: the same forced hash for different tokens is told apart by the tokens */
+    CHECK(kipp_pool_init(&pool, 4, 2, NULL, &error) == 0);
+    pool.force_hash = true;
+    pool.forced_hash = 7;
+    uint32_t a = kipp_pool_alloc(&pool), b = kipp_pool_alloc(&pool), ta[2] = {1, 2}, tb[2] = {3, 4}, find[3] = {3, 4, 9}, got[1];
+    kipp_pool_seal(&pool, a, 0, ta);
+    kipp_pool_seal(&pool, b, 0, tb);
+    CHECK(kipp_pool_prefix_match(&pool, find, 3, got, 1, NULL) == 1 && got[0] == b);
+    kipp_pool_free(&pool);
+    uint32_t twice[3] = {0, 1, 1};
+    CHECK(kipp_pool_init(&pool, 3, 2, twice, &error) != 0);
+    CHECK(kipp_pool_init(&pool, 0, 2, NULL, &error) != 0);
+}
+
+static int same_bits(const float *a, const float *b, size_t n) { return memcmp(a, b, n * sizeof(float)) == 0; }
+
+/* One model folder on the scalar path: the whole sequence in one step, then the same tokens in portions beside a second
+ * session, with the tables reversed on the way; the logits must be the same bits. */
+static void test_model(const char *folder) {
+    kipp_model *model = NULL;
+    kipp_error error;
+    kipp_model_open_config config;
+    memset(&config, 0, sizeof(config));
+    config.path = KIPP_PATH_CPU_FP32;
+    config.page_tokens = 4;
+    config.kv_pool_pages = 40;
+    config.max_sessions = 3;
+    config.share_prefixes = 1;
+    if (kipp_model_open_ex(folder, &config, &model, &error) != 0) {
+        fprintf(stderr, "cannot open %s: %s\n", folder, error.message);
+        CHECK(0);
+        return;
+    }
+    kipp_model_info info;
+    CHECK(kipp_model_get_info(model, &info) == 0 && info.vocab_size > 0 && info.cache_groups == 1);
+    const uint32_t vocab = info.vocab_size, n = 37;
+    uint32_t tokens[64], other[64], want[64];
+    for (uint32_t i = 0; i < 64; ++i) {
+        tokens[i] = rnd(vocab);
+        other[i] = rnd(vocab);
+        want[i] = i;
+    }
+    float *whole = malloc((size_t)n * vocab * sizeof(float)), *cut = malloc((size_t)n * vocab * sizeof(float)),
+          *spare = malloc((size_t)64 * vocab * sizeof(float));
+    kipp_session *a = NULL, *b = NULL, *c = NULL, *d = NULL;
+    CHECK(kipp_session_create(model, 0, &a, &error) == 0);
+    kipp_step_item item = {a, tokens, n, want, n};
+    CHECK(kipp_step(model, &item, 1, whole, (size_t)n * vocab, &error) == 0);
+    for (size_t i = 0; i < (size_t)n * vocab; ++i) {
+        if (!isfinite(whole[i])) {
+            CHECK(0);
+            break;
+        }
+    }
+    kipp_session_info sinfo;
+    CHECK(kipp_session_get_info(a, &sinfo) == 0 && sinfo.length == n && sinfo.cache_bytes > 0);
+    CHECK(kipp_session_reset(a, &error) == 0); /* publishes 9 full pages */
+    CHECK(kipp_session_create(model, 0, &b, &error) == 0 && kipp_session_create(model, 0, &c, &error) == 0);
+    CHECK(kipp_session_create(model, 0, &d, &error) != 0 && error.code == KIPP_ERROR_RANGE); /* three slots */
+    /* portions of `a` (which adopts nothing: its first portion is run) beside portions and single tokens of `b` */
+    static const uint32_t portions[] = {5, 2, 9, 1, 1, 7, 3, 1, 8};
+    uint32_t fed = 0, fed_b = 0;
+    for (size_t p = 0; p < sizeof(portions) / sizeof(portions[0]); ++p) {
+        uint32_t take_b = 1 + rnd(4);
+        kipp_step_item items[2] = {{b, other + fed_b, take_b, want, p % 2 ? take_b : 0}, {a, tokens + fed, portions[p], want, portions[p]}};
+        size_t rows_b = items[0].want_count;
+        CHECK(kipp_step(model, items, 2, spare, (size_t)64 * vocab, &error) == 0);
+        memcpy(cut + (size_t)fed * vocab, spare + rows_b * vocab, (size_t)portions[p] * vocab * sizeof(float));
+        fed += portions[p];
+        fed_b += take_b;
+        if (p % 3 == 1) CHECK(kipp_test_scramble_session_kv(a, &error) == 0 && kipp_test_scramble_session_kv(b, &error) == 0);
+        CHECK(kipp_cache_check(&model->cache, model->sessions, model->session_count, &error) == 0);
+    }
+    CHECK(fed == n && same_bits(whole, cut, (size_t)n * vocab));
+    /* a session that adopts the published beginning continues with the same bits */
+    uint32_t matched = 0;
+    CHECK(kipp_session_match_prefix(c, tokens, n, &matched, &error) == 0 && matched == 36);
+    CHECK(kipp_test_scramble_session_kv(c, &error) != 0 && error.code == KIPP_ERROR_UNSUPPORTED);
+    CHECK(kipp_session_eval(c, tokens + matched, n - matched, spare, vocab, &error) == 0 && same_bits(spare, whole + (size_t)(n - 1) * vocab, vocab));
+    /* error paths leave everything as it was */
+    kipp_kv_pool_stats_public before, after;
+    kipp_model_kv_pool_stats(model, 0, &before);
+    uint32_t bad_token = vocab, place = 5;
+    kipp_step_item bad = {a, &bad_token, 1, want, 1};
+    CHECK(kipp_step(model, &bad, 1, spare, vocab, &error) != 0 && error.code == KIPP_ERROR_RANGE);
+    bad = (kipp_step_item){a, tokens, 2, &place, 1};
+    CHECK(kipp_step(model, &bad, 1, spare, vocab, &error) != 0);
+    bad = (kipp_step_item){a, tokens, 2, want, 2};
+    CHECK(kipp_step(model, &bad, 1, spare, vocab, &error) != 0 && error.code == KIPP_ERROR_ARGUMENT); /* room for one row only */
+    kipp_step_item twice[2] = {{a, tokens, 1, want, 1}, {a, tokens, 1, want, 1}};
+    CHECK(kipp_step(model, twice, 2, spare, 2 * (size_t)vocab, &error) != 0);
+    kipp_model_kv_pool_stats(model, 0, &after);
+    CHECK(before.free_blocks == after.free_blocks && kipp_session_get_info(a, &sinfo) == 0 && sinfo.length == n);
+    CHECK(kipp_session_truncate(a, 10, &error) == 0 && kipp_session_truncate(a, 11, &error) != 0);
+    CHECK(kipp_session_eval_n(a, tokens + 10, 5, spare, 3, &error) == 0 && same_bits(spare, whole + (size_t)12 * vocab, (size_t)3 * vocab));
+    CHECK(kipp_model_close(model, &error) != 0); /* sessions are alive */
+    kipp_session_destroy(a);
+    kipp_session_destroy(b);
+    kipp_session_destroy(c);
+    kipp_model_kv_pool_stats(model, 0, &after);
+    CHECK(after.free_blocks == after.total_blocks && after.reused_blocks_total >= 9);
+    CHECK(kipp_model_close(model, &error) == 0);
+    free(whole);
+    free(cut);
+    free(spare);
+    /* a folder that is not there, and one without weights */
+    CHECK(kipp_model_open_ex("/nonexistent/kipp", &config, &model, &error) != 0 && error.code == KIPP_ERROR_IO && model == NULL);
+}
+
+static void test_sampler(void) {
+    kipp_error error;
+    uint32_t token = 99;
+    uint64_t state = 1;
+    float logits[5] = {0.5f, 2.0f, 2.0f, -1.0f, 1.5f};
+    CHECK(kipp_sample(logits, 5, 0.0f, 1.0f, NULL, &token, &error) == 0 && token == 1); /* greedy never touches the generator */
+    CHECK(kipp_sample(logits, 5, 1.0f, 1.0f, NULL, &token, &error) != 0 && error.code == KIPP_ERROR_ARGUMENT);
+    CHECK(kipp_sample(logits, 5, 1.0f, 1.5f, &state, &token, &error) != 0);
+    int seen[5] = {0};
+    for (int i = 0; i < 2000; ++i) {
+        CHECK(kipp_sample(logits, 5, 1.0f, 1.0f, &state, &token, &error) == 0 && token < 5);
+        ++seen[token];
+    }
+    CHECK(seen[1] > seen[0] && seen[2] > seen[3] && seen[3] > 0);
+    kipp_sample_params params;
+    memset(&params, 0, sizeof(params));
+    params.temperature = 1.0f;
+    params.top_p = 1.0f;
+    params.top_k = 1;
+    for (int i = 0; i < 50; ++i) CHECK(kipp_sample_ex(logits, 5, &params, &state, &token, &error) == 0 && token == 1); /* top_k = 1 is the argmax */
+    uint32_t recent[3] = {1, 1, 7}, bias_tokens[2] = {3, 9};
+    float bias_values[2] = {10.0f, 1.0f};
+    params.temperature = 0.0f;
+    params.repetition_penalty = 2.0f;
+    params.recent_tokens = recent;
+    params.recent_count = 3;
+    CHECK(kipp_sample_ex(logits, 5, &params, NULL, &token, &error) == 0 && token == 2); /* token 1 halved, tokens beyond the vocabulary ignored */
+    params.logit_bias_tokens = bias_tokens;
+    params.logit_bias_values = bias_values;
+    params.logit_bias_count = 2;
+    CHECK(kipp_sample_ex(logits, 5, &params, NULL, &token, &error) == 0 && token == 3);
+    CHECK(strcmp(kipp_error_code_name(KIPP_ERROR_RANGE), "range") == 0 && strcmp(kipp_path_name(KIPP_PATH_CPU_FP32), "cpu-fp32") == 0);
+}
+
+/* vectors of the reference's own unit tests for the scalar operations (/root/reference/tests/kipp_test.c:88-175) */
+static void test_scalar_operations(void) {
+    float x[2] = {3.0f, 4.0f}, w[2] = {1.0f, 1.0f}, out[2];
+    kipp_test_rms_norm(x, w, out, 2, 0.0f);
+    CHECK(fabsf(out[0] - 3.0f / sqrtf(12.5f)) < 1e-6f && fabsf(out[1] - 4.0f / sqrtf(12.5f)) < 1e-6f);
+    float matrix[6] = {1, 2, 3, -1, 0.5f, 0}, input[3] = {2, -1, 0.5f}, product[2];
+    kipp_test_matvec(matrix, input, product, 2, 3);
+    CHECK(product[0] == 1.5f && product[1] == -2.5f);
+    float head[4] = {1, 2, 3, 4};
+    kipp_test_rope(head, 4, 1, 10000.0f);
+    float c = cosf(1.0f), s = sinf(1.0f), c2 = cosf(0.01f), s2 = sinf(0.01f);
+    CHECK(fabsf(head[0] - (c - 3 * s)) < 1e-6f && fabsf(head[1] - (2 * c2 - 4 * s2)) < 1e-6f && fabsf(head[2] - (3 * c + s)) < 1e-6f &&
+          fabsf(head[3] - (4 * c2 + 2 * s2)) < 1e-6f);
+    float values[3] = {1, 2, 3};
+    kipp_test_softmax(values, 3);
+    CHECK(fabsf(values[0] + values[1] + values[2] - 1.0f) < 1e-6f && values[0] < values[1] && values[1] < values[2]);
+    CHECK(kipp_test_silu(0.0f) == 0.0f && fabsf(kipp_test_silu(1.0f) - 0.7310586f) < 1e-6f);
+    /* two tokens, 32 query heads over 8 key/value heads, q = k = 0, v0 = 1, v1 = 3: 1 then 2 */
+    enum { T = 2, NQ = 32, NKV = 8, D = 128 };
+    static float q[T * NQ * D], k[T * NKV * D], v[T * NKV * D], o[T * NQ * D];
+    for (int i = 0; i < NKV * D; ++i) {
+        v[i] = 1.0f;
+        v[NKV * D + i] = 3.0f;
+    }
+    kipp_test_causal_gqa(q, k, v, o, T, NQ, NKV, D);
+    CHECK(o[0] == 1.0f && o[NQ * D - 1] == 1.0f && o[NQ * D] == 2.0f && o[2 * NQ * D - 1] == 2.0f);
+}
+
+int main(int argc, char **argv) {
+    test_json();
+    test_sizes();
+    test_pool();
+    test_sampler();
+    test_scalar_operations();
+    for (int i = 1; i < argc; ++i) test_model(argv[i]);
+    if (failures != 0) {
+        fprintf(stderr, "%d of %d checks failed\n", failures, checks);
+        return 1;
+    }
+    printf("ok %d\n", checks);
+    return 0;
+}

@@ -194,3 +194,34 @@ def assert_close(got: np.ndarray, ref: np.ndarray, tol: float, what: str) -> Non
         with open(NMSE_LOG, "a") as f:
             f.write(f"{what}\t{worst:.3e}\t{tol:.1e}\n")
     assert worst <= tol, f"{what}: NMSE {worst:.3e} at position {worst_at} exceeds {tol:.1e}"
+
+
+def replay_c(model, requests: Dict[str, Sequence[int]], steps: Sequence[Step], scramble_every: int = 0) -> Dict[str, np.ndarray]:
+    """`replay` through the C host (`kipp_amd.chost.CModel`): the same schedules through kipp_step, asking for
+    the logits of every token.  `scramble_every` N: every N-th step, each live session's block tables are reversed
+    first (the pages' contents moving along)."""
+    fed = {r: 0 for r in requests}
+    rows: Dict[str, List[np.ndarray]] = {r: [] for r in requests}
+    sessions = {}
+    for number, (entries, ends) in enumerate(steps):
+        if scramble_every and number % scramble_every == scramble_every - 1:
+            for s in sessions.values():
+                s.scramble()
+        batch = []
+        for rid, n in entries:
+            if rid not in sessions:
+                sessions[rid] = model.session()
+            toks = list(requests[rid][fed[rid]:fed[rid] + n])
+            assert len(toks) == n, f"schedule feeds more tokens of {rid} than it has"
+            batch.append((sessions[rid], toks, list(range(n))))
+        out = model.step(batch)
+        at = 0
+        for rid, n in entries:
+            rows[rid].append(out[at:at + n])
+            at += n
+            fed[rid] += n
+        for rid in ends:
+            sessions.pop(rid).destroy()
+    for s in sessions.values():
+        s.destroy()
+    return {r: np.concatenate(v, axis=0) for r, v in rows.items() if v}

@@ -1,0 +1,387 @@
+"""The C host (`kipp_amd/host`, through `kipp_amd.chost`) on its scalar float32 path, which needs no GPU: the step
+function under every cutting against the plain implementation and bit for bit against itself, scrambled block
+tables, pages that are used again, shared beginnings, truncation, what happens when pages run out; configuration
+and weight errors; the sampler against the Python one."""
+import json
+import os
+import random
+import shutil
+
+import numpy as np
+import pytest
+
+from kipp_amd.chost import CModel, KippError, Rng, sample
+from tests import helpers as H
+
+PAGE = {"a": 16, "b": 8}
+LENGTHS = {"a": [1, 17, 40, 64], "b": [7, 33, 61, 100]}
+
+
+def _requests(key, cfg, seed=0):
+    return {f"r{i}": H.random_tokens(seed * 100 + i, n, cfg["vocab_size"]) for i, n in enumerate(LENGTHS[key])}
+
+
+def _model(model_folders, key, pages=64, **kw):
+    return CModel(model_folders[(key, "float32")], path="cpu-fp32", page_tokens=PAGE[key], kv_pool_pages=pages, **kw)
+
+
+@pytest.mark.parametrize("key", ["a", "b"])
+@pytest.mark.parametrize("cut", ["whole", "tail", "portions", "mixed"])
+def test_host_path_cuttings_match_plain_and_each_other(model_folders, tiny_configs, key, cut):
+    """Every cutting against the plain implementation, and bit for bit against the whole prompts: on the scalar path
+    every sum runs in an order that its own row and position fix.  The mixed cutting runs with exactly as many pages as
+    the live requests hold at their peak, so pages that were given back are used again, and with every session's block
+    tables reversed every third step."""
+    cfg = tiny_configs[key]
+    requests = _requests(key, cfg)
+    with _model(model_folders, key, share_prefixes=False) as model:
+        base = H.replay_c(model, requests, H.whole(requests))
+    if cut == "mixed":
+        more = {f"s{i}": H.random_tokens(900 + i, n, cfg["vocab_size"]) for i, n in enumerate(LENGTHS[key])}
+        with _model(model_folders, key, share_prefixes=False) as model:
+            base.update(H.replay_c(model, more, H.whole(more)))
+        requests = {**requests, **more}
+        steps = H.mixed(requests, seed=5)
+        pages = H.peak_pages(requests, steps, PAGE[key])
+        assert pages < sum(-(-len(t) // PAGE[key]) for t in requests.values())
+        model = _model(model_folders, key, pages=pages, share_prefixes=False)
+        got = H.replay_c(model, requests, steps, scramble_every=3)
+    else:
+        steps = {"whole": H.whole, "tail": H.tail_one_by_one, "portions": H.changing_portions}[cut](requests)
+        model = _model(model_folders, key, share_prefixes=False)
+        got = H.replay_c(model, requests, steps, scramble_every=2 if cut != "whole" else 0)
+    for rid, toks in requests.items():
+        H.assert_close(got[rid], H.plain_logits(model_folders[(key, "float32")], toks), H.NMSE_F32, f"C host {key}/{cut}/{rid}")
+        assert np.array_equal(got[rid], base[rid]), f"{key}/{cut}/{rid}: bits differ from the whole prompt's"
+    stats = model.pool_stats()
+    assert stats["free_blocks"] == stats["total_blocks"]
+    model.close()
+
+
+def test_a_scrambled_table_is_noticed_when_the_contents_stay(model_folders, tiny_configs):
+    """The scramble hook moves the pages' contents along with the table.  If a step read through a table that does
+    not match where the keys lie, the logits would change: shown by feeding a sequence, swapping two pages'
+    *roles* by hand (evaluating the rest in a second model whose sessions got their pages in another order
+    gives the same bits; evaluating behind pages of another sequence does not)."""
+    cfg = tiny_configs["b"]
+    toks = H.random_tokens(5, 60, cfg["vocab_size"])
+    other = H.random_tokens(6, 60, cfg["vocab_size"])
+    with _model(model_folders, "b", share_prefixes=False) as model:
+        s = model.session()
+        model.step([(s, toks[:40], [])])
+        right = model.step([(s, toks[40:], list(range(20)))])
+    order = list(range(64))
+    random.Random(3).shuffle(order)
+    with _model(model_folders, "b", share_prefixes=False, page_order=order) as model:
+        s = model.session()
+        model.step([(s, toks[:40], [])])
+        assert s.pages() == order[:5]
+        assert np.array_equal(model.step([(s, toks[40:], list(range(20)))]), right)       # where pages lie changes nothing
+    with _model(model_folders, "b", share_prefixes=False) as model:
+        s = model.session()
+        model.step([(s, other[:40], [])])                                                  # another sequence's keys in the pages
+        wrong = model.step([(s, toks[40:], list(range(20)))])
+        assert not np.array_equal(wrong, right)
+
+
+def test_steps_are_all_or_nothing(model_folders, tiny_configs):
+    cfg = tiny_configs["a"]
+    vocab = cfg["vocab_size"]
+    with _model(model_folders, "a", pages=4, share_prefixes=False) as model:
+        a, b = model.session(), model.session()
+        model.step([(a, H.random_tokens(1, 40, vocab), [])])              # 3 of 4 pages
+        before = model.pool_stats()["free_blocks"]
+        with pytest.raises(KippError, match="range: KV pool exhausted"):
+            model.step([(a, [1, 2], [1]), (b, H.random_tokens(2, 20, vocab), [19])])     # a fits, b needs 2 pages: 1 free
+        assert model.pool_stats()["free_blocks"] == before and (a.length, b.length) == (40, 0)
+        with pytest.raises(KippError, match="twice"):
+            model.step([(a, [1], [0]), (a, [2], [0])])
+        with pytest.raises(KippError, match="vocabulary"):
+            model.step([(a, [vocab], [0])])
+        with pytest.raises(KippError, match="wanted place"):
+            model.step([(a, [1, 2], [2])])
+        with pytest.raises(KippError, match="at least one token"):
+            model.step([(a, [], [])])
+        with pytest.raises(KippError, match="capacity"):
+            model.step([(a, H.random_tokens(3, 100, vocab), [])])          # 140 tokens: beyond the model's 128 positions
+        assert model.pool_stats()["free_blocks"] == before and a.length == 40
+        row = model.step([(a, [7], [0])])                                  # and it still works afterwards
+        assert row.shape == (1, vocab) and a.length == 41
+
+
+def test_shared_beginnings_truncation_and_rows_one_by_one(model_folders, tiny_configs):
+    """kipp.h's session calls: a finished session publishes its full pages, a fresh one adopts the longest known beginning
+    (whole pages, at most (n - 1) / page), truncation never goes below it, eval_n and eval_scored give the rows of
+    single-token evaluation (/root/reference/src/kipp.h:172-235, /root/reference/tests/kipp_test.c:3233-3238)."""
+    cfg = tiny_configs["b"]
+    vocab, folder = cfg["vocab_size"], model_folders[("b", "float32")]
+    toks = H.random_tokens(8, 64, vocab)
+    ref = H.plain_logits(folder, toks)
+    with _model(model_folders, "b", pages=24) as model:
+        first = model.session()
+        H.assert_close(first.eval(toks[:50])[None], ref[49:50], H.NMSE_F32, "eval")
+        first.destroy()                                                     # publishes 6 full pages of 8
+        second = model.session()
+        assert second.match_prefix(toks[:48]) == 40                         # an exact multiple adopts one page less: a token is left to run
+        second.destroy()
+        second = model.session()
+        assert second.match_prefix(toks) == 48 and second.adopted_tokens == 48
+        assert model.pool_stats()["reused_blocks_total"] == 5 + 6
+        rows = second.eval_n(toks[48:], 10)
+        H.assert_close(rows, ref[54:], H.NMSE_F32, "eval_n behind an adopted beginning")
+        with pytest.raises(KippError, match="adopted"):
+            second.truncate(40)
+        second.truncate(56)
+        again = second.eval_scored(toks[56:], 8)
+        assert np.array_equal(again, rows[2:])
+        third = model.session()
+        with pytest.raises(KippError, match="fresh"):
+            second.match_prefix(toks)
+        batch = model.eval_batch([(third, toks[:30])])
+        H.assert_close(batch, ref[29:30], H.NMSE_F32, "eval_batch")
+        second.reset()
+        assert second.length == 0
+    with _model(model_folders, "b", share_prefixes=False) as model:
+        s = model.session()
+        with pytest.raises(KippError, match="unsupported"):
+            s.match_prefix(toks)
+        with pytest.raises(KippError, match="alive"):
+            err_model = model
+            lib = err_model.lib
+            from kipp_amd.chost import _Error, _raise
+            import ctypes
+            e = _Error()
+            if lib.kipp_model_close(err_model.handle, ctypes.byref(e)) != 0:
+                _raise(lib, e)
+
+
+def test_model_info_and_stop_tokens(model_folders, tiny_configs, tmp_path):
+    with _model(model_folders, "b") as model:
+        info = model.info
+        cfg = tiny_configs["b"]
+        assert info.architecture == b"Qwen3ForCausalLM" and info.path == 2
+        assert (info.block_count, info.embedding_length, info.feed_forward_length, info.attention_head_count, info.attention_head_count_kv,
+                info.attention_head_dim, info.vocab_size, info.context_length, info.tied_embeddings) == (
+            cfg["num_hidden_layers"], cfg["hidden_size"], cfg["intermediate_size"], cfg["num_attention_heads"], cfg["num_key_value_heads"],
+            cfg["head_dim"], cfg["vocab_size"], cfg["max_position_embeddings"], 0)
+        assert abs(info.rope_theta - cfg["rope_theta"]) < 1 and abs(info.rms_norm_eps - cfg["rms_norm_eps"]) < 1e-12
+        assert info.cache_groups == 1 and info.page_tokens == 8 and info.weight_bytes > 0 and info.cache_bytes > 0
+    folder = str(tmp_path / "stops")
+    shutil.copytree(model_folders[("a", "float32")], folder)
+    cfg = json.load(open(os.path.join(folder, "config.json")))
+    cfg["eos_token_id"] = [7, 200]
+    json.dump(cfg, open(os.path.join(folder, "config.json"), "w"))
+    with CModel(folder, path="cpu-fp32") as model:
+        assert model.is_stop_token(7) and model.is_stop_token(200) and not model.is_stop_token(8)
+
+
+def _edit_config(model_folders, tmp_path, **changes):
+    folder = str(tmp_path / "edited")
+    if os.path.exists(folder):
+        shutil.rmtree(folder)
+    shutil.copytree(model_folders[("a", "float32")], folder)
+    path = os.path.join(folder, "config.json")
+    cfg = json.load(open(path))
+    for key, value in changes.items():
+        if value is ...:
+            cfg.pop(key, None)
+        else:
+            cfg[key] = value
+    json.dump(cfg, open(path, "w"))
+    return folder
+
+
+@pytest.mark.parametrize("changes,code,match", [
+    ({"rope_scaling": {"type": "yarn", "factor": 4}}, "unsupported", "rope_scaling"),
+    ({"attention_bias": True}, "unsupported", "attention_bias"),
+    ({"hidden_act": "gelu"}, "unsupported", "hidden_act"),
+    ({"use_sliding_window": True}, "unsupported", "use_sliding_window"),
+    ({"model_type": "llama"}, "unsupported", "model_type"),
+    ({"architectures": ["LlamaForCausalLM"]}, "unsupported", "not in the registry; known: Qwen3ForCausalLM"),
+    ({"num_key_value_heads": 3}, "format", "multiple"),
+    ({"vocab_size": "256"}, "format", "vocab_size"),
+    ({"num_hidden_layers": 0}, "format", "num_hidden_layers"),
+    ({"rms_norm_eps": -1.0}, "format", "rms_norm_eps"),
+    ({"tie_word_embeddings": "yes"}, "format", "tie_word_embeddings"),
+    ({"eos_token_id": 99999}, "format", "eos_token_id"),
+    ({"rope_theta": ..., "rms_norm_eps": ...}, "format", "rms_norm_eps, rope_theta"),
+])
+def test_configurations_the_host_refuses(model_folders, tmp_path, changes, code, match):
+    folder = _edit_config(model_folders, tmp_path, **changes)
+    with pytest.raises(KippError, match=match) as e:
+        CModel(folder, path="cpu-fp32")
+    assert e.value.code == code
+
+
+def test_config_json_is_read_strictly(model_folders, tmp_path):
+    folder = _edit_config(model_folders, tmp_path)
+    path = os.path.join(folder, "config.json")
+    good = open(path).read()
+    for bad, match in ((good + " x", "something follows"), (good.replace('"vocab_size"', '"hidden_size": 1, "vocab_size"', 1), "duplicate key"),
+                       (good.replace("256", "0256", 1), "leading zero"), ("[" * 70 + "]" * 70, "nested too deeply"),
+                       (good.replace('"qwen3"', '"qw\x01en3"'), "control character"), (good[:-1], "unterminated|expected")):
+        open(path, "w").write(bad)
+        with pytest.raises(KippError, match=match):
+            CModel(folder, path="cpu-fp32")
+
+
+def test_one_error_lists_every_wrong_tensor(model_folders, tmp_path):
+    """Missing, unexpected and wrongly shaped tensors and wrong types together, in one error
+    (the reference stops at the first: /root/reference/src/kipp.c:859-906, 997-1002)."""
+    import torch
+    from kipp_amd.weights.safetensors_io import read_file, write_file
+    folder = str(tmp_path / "broken")
+    shutil.copytree(model_folders[("a", "float32")], folder)
+    tensors = dict(read_file(os.path.join(folder, "model.safetensors")))
+    del tensors["model.layers.1.mlp.up_proj.weight"], tensors["model.norm.weight"]
+    tensors["lm_head.weight"] = torch.zeros(256, 64)                            # tied: the head has no tensor of its own
+    tensors["model.layers.0.self_attn.q_norm.weight"] = torch.zeros(8)
+    tensors["model.layers.0.self_attn.k_proj.weight"] = torch.zeros(32, 64, dtype=torch.int32)
+    write_file(os.path.join(folder, "model.safetensors"), tensors)
+    with pytest.raises(KippError) as e:
+        CModel(folder, path="cpu-fp32")
+    text = e.value.message
+    assert e.value.code == "format" and "do not match the configuration" in text
+    assert "missing tensors (2): model.layers.1.mlp.up_proj.weight, model.norm.weight" in text
+    assert "unexpected tensors (1): lm_head.weight" in text
+    assert "model.layers.0.self_attn.q_norm.weight: shape (8), expected (16)" in text
+    assert "model.layers.0.self_attn.k_proj.weight: type I32" in text
+
+
+def test_safetensors_format_errors(model_folders, tmp_path):
+    """Errors of the file itself: truncation, a header that does not fit, spans that overlap or leave the file, a span
+    that is not product(shape) x element size (/root/reference/src/kipp.c:1032-1061, /root/reference/tools/convert_to_gguf.py:337-340)."""
+    import struct
+    folder = str(tmp_path / "files")
+    shutil.copytree(model_folders[("a", "float32")], folder)
+    path = os.path.join(folder, "model.safetensors")
+    raw = open(path, "rb").read()
+    (n,) = struct.unpack("<Q", raw[:8])
+    header = json.loads(raw[8:8 + n])
+
+    def rewrite(new_header, payload=raw[8 + n:]):
+        text = json.dumps(new_header).encode()
+        open(path, "wb").write(struct.pack("<Q", len(text)) + text + payload)
+
+    def expect(match):
+        with pytest.raises(KippError, match=match) as e:
+            CModel(folder, path="cpu-fp32")
+        assert e.value.code == "format"
+    open(path, "wb").write(raw[:5])
+    expect("truncated before the header length")
+    open(path, "wb").write(struct.pack("<Q", 10**9) + raw[8:])
+    expect("does not fit the file")
+    open(path, "wb").write(raw[:8] + b"[" + raw[9:])
+    expect("not valid JSON")
+    names = sorted(k for k in header if k != "__metadata__")
+    a, b = names[0], names[1]
+    broken = json.loads(json.dumps(header))
+    broken[b]["data_offsets"] = [header[a]["data_offsets"][0], header[a]["data_offsets"][0] + header[b]["data_offsets"][1] - header[b]["data_offsets"][0]]
+    rewrite(broken)
+    expect("overlap")
+    broken = json.loads(json.dumps(header))
+    broken[a]["data_offsets"][1] += 4
+    rewrite(broken)
+    expect("spans .* bytes but its shape")
+    rewrite(header, raw[8 + n:-16])
+    expect("lies outside the file")
+    broken = json.loads(json.dumps(header))
+    broken[a]["dtype"] = "F8_E4M3"
+    rewrite(broken)
+    expect("unsupported dtype")
+    broken = json.loads(json.dumps(header))
+    del broken[a]["shape"]
+    rewrite(broken)
+    expect("malformed")
+
+
+def test_sharded_folders(model_folders, tiny_configs, tmp_path):
+    """model.safetensors.index.json: every tensor from the shard that the weight_map names
+    (/root/reference/tools/convert_to_gguf.py:297-314)."""
+    from kipp_amd.weights.safetensors_io import read_file, write_file
+    src = model_folders[("b", "float32")]
+    folder = str(tmp_path / "sharded")
+    os.makedirs(folder)
+    shutil.copy(os.path.join(src, "config.json"), folder)
+    tensors = dict(read_file(os.path.join(src, "model.safetensors")))
+    names = sorted(tensors)
+    halves = {"model-00001-of-00002.safetensors": names[::2], "model-00002-of-00002.safetensors": names[1::2]}
+    for shard, members in halves.items():
+        write_file(os.path.join(folder, shard), {n: tensors[n] for n in members})
+    json.dump({"weight_map": {n: shard for shard, members in halves.items() for n in members}},
+              open(os.path.join(folder, "model.safetensors.index.json"), "w"))
+    toks = H.random_tokens(4, 21, tiny_configs["b"]["vocab_size"])
+    with CModel(folder, path="cpu-fp32", page_tokens=8) as model:
+        got = model.step([(model.session(), toks, list(range(21)))])
+    H.assert_close(got, H.plain_logits(src, toks), H.NMSE_F32, "sharded")
+    index = json.load(open(os.path.join(folder, "model.safetensors.index.json")))
+    index["weight_map"]["model.ghost.weight"] = "model-00001-of-00002.safetensors"
+    json.dump(index, open(os.path.join(folder, "model.safetensors.index.json"), "w"))
+    with pytest.raises(KippError, match="listed but absent from their shard: model.ghost.weight"):
+        CModel(folder, path="cpu-fp32")
+
+
+def test_bfloat16_weights_are_widened_exactly(model_folders, tiny_configs):
+    """A folder stored in bfloat16 on the float32 path: the same values, widened, as the plain implementation reads them."""
+    toks = H.random_tokens(12, 30, tiny_configs["a"]["vocab_size"])
+    folder = model_folders[("a", "bfloat16")]
+    with CModel(folder, path="cpu-fp32") as model:
+        got = model.step([(model.session(), toks, list(range(30)))])
+    H.assert_close(got, H.plain_logits(folder, toks), H.NMSE_F32, "bfloat16 file, float32 path")
+
+
+def test_the_c_sampler_is_the_python_sampler(tiny_configs):
+    """Same order, same float widths, same generator: the same token and the same generator state for random
+    parameters (vectors of the reference's own tests pin the Python one: tests/test_sampler.py)."""
+    from kipp_amd.sampling import SampleParams, XorShift64Star
+    from kipp_amd.sampling import sample as py_sample
+    rng = np.random.default_rng(5)
+    for case in range(300):
+        vocab = int(rng.integers(2, 400))
+        logits = (rng.normal(size=vocab) * rng.choice([0.5, 3.0, 12.0])).astype(np.float32)
+        if case % 7 == 0:
+            logits[rng.integers(0, vocab, size=3)] = logits.max()               # ties
+        recent = [int(t) for t in rng.integers(0, vocab + 3, size=int(rng.integers(0, 12)))]
+        bias = {int(t): float(rng.normal() * 4) for t in rng.integers(0, vocab + 2, size=int(rng.integers(0, 4)))}
+        p = SampleParams(temperature=float(rng.choice([0.0, 0.3, 1.0, 2.5])), top_p=float(rng.choice([1.0, 0.9, 0.3, 1e-6])),
+                         top_k=int(rng.choice([0, 1, 5, 1000])), min_p=float(rng.choice([0.0, 0.05, 0.5])),
+                         repetition_penalty=float(rng.choice([1.0, 1.3, 0.8])), presence_penalty=float(rng.choice([0.0, 0.7])),
+                         frequency_penalty=float(rng.choice([0.0, 0.2])), logit_bias=bias)
+        seed = int(rng.integers(1, 2**62))
+        py_rng, c_rng = XorShift64Star(seed), Rng(seed)
+        want = py_sample(logits, p, py_rng, recent)
+        got = sample(logits, p.temperature, p.top_p, p.top_k, p.min_p, p.frequency_penalty, p.presence_penalty, p.repetition_penalty,
+                     recent, bias, c_rng)
+        assert got == want, (case, p)
+        assert c_rng.state.value == py_rng.state
+    with pytest.raises(KippError, match="top_p"):
+        sample(np.zeros(4, np.float32), temperature=1.0, top_p=0.0, rng=Rng(1))
+    with pytest.raises(KippError, match="nonzero RNG"):
+        sample(np.zeros(4, np.float32), temperature=1.0, rng=Rng(0))
+    assert sample(np.array([1.0, 3.0, 3.0, 2.0], np.float32)) == 1               # greedy: the lowest index among equals, no generator
+
+
+def test_host_logic_under_the_sanitizers(model_folders, tmp_path):
+    """tests/chost/host_test.c, linked with the host's sources (without the GPU's table) under AddressSanitizer and
+    UndefinedBehaviorSanitizer: JSON, checked sizes, pool and cache manager under random orders, both tiny models
+    opened and stepped on the scalar path under several cuttings with scrambled tables, error paths, the sampler."""
+    import subprocess
+    from kipp_amd.host import build
+    here = os.path.dirname(os.path.abspath(__file__))
+    exe = build.test_program(os.path.join(here, "chost", "host_test.c"), str(tmp_path / "host_test"))
+    env = dict(os.environ, ASAN_OPTIONS="detect_leaks=1:abort_on_error=0", UBSAN_OPTIONS="print_stacktrace=1:halt_on_error=1")
+    proc = subprocess.run([exe, model_folders[("a", "float32")], model_folders[("b", "float32")], model_folders[("b", "bfloat16")]],
+                          capture_output=True, text=True, timeout=300, env=env)
+    assert proc.returncode == 0, proc.stdout[-2000:] + proc.stderr[-6000:]
+    assert proc.stdout.strip().splitlines()[-1].startswith("ok ")
+    assert "runtime error" not in proc.stderr and "AddressSanitizer" not in proc.stderr and "LeakSanitizer" not in proc.stderr
+
+
+def test_the_host_compiles_without_warnings():
+    import subprocess
+    from kipp_amd.host import build
+    for gpu in (False, True):
+        flags, _ = build._flags(gpu, False)
+        for src in build._sources(gpu):
+            proc = subprocess.run([build._compiler()] + flags + ["-fsyntax-only", src], capture_output=True, text=True)
+            assert proc.returncode == 0 and "warning" not in proc.stderr, proc.stderr

@@ -1,0 +1,122 @@
+"""The C host on the GPU (`kipp_amd.chost.CModel`, paths gpu-fp32 and gpu-bf16): the same schedules as the Python
+engine's tests through kipp_step, against the plain implementation, against the library's own scalar path, and in
+float32 bit for bit against the Python engine, which launches the same kernels."""
+import numpy as np
+import pytest
+
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+PAGE = {"a": 16, "b": 8}
+LENGTHS = {"a": [1, 17, 40, 64], "b": [7, 33, 61, 100]}
+PATH = {"float32": "gpu-fp32", "bfloat16": "gpu-bf16"}
+
+
+def _requests(key, cfg, seed=0):
+    return {f"r{i}": H.random_tokens(seed * 100 + i, n, cfg["vocab_size"]) for i, n in enumerate(LENGTHS[key])}
+
+
+def _model(model_folders, key, dtype, pages=64, **kw):
+    from kipp_amd.chost import CModel
+    return CModel(model_folders[(key, dtype)], path=PATH[dtype], page_tokens=PAGE[key], kv_pool_pages=pages, share_prefixes=False, **kw)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("key", ["a", "b"])
+@pytest.mark.parametrize("cut", ["whole", "tail", "portions", "mixed"])
+def test_c_host_cuttings_match_plain(model_folders, tiny_configs, key, dtype, cut):
+    cfg = tiny_configs[key]
+    requests = _requests(key, cfg)
+    tol = H.NMSE_F32 if dtype == "float32" else H.NMSE_BF16["tiny"]
+    if cut == "mixed":
+        more = {f"s{i}": H.random_tokens(900 + i, n, cfg["vocab_size"]) for i, n in enumerate(LENGTHS[key])}
+        requests = {**requests, **more}
+        steps = H.mixed(requests, seed=5)
+        pages = H.peak_pages(requests, steps, PAGE[key])          # pages that were given back are used again
+        model = _model(model_folders, key, dtype, pages=pages)
+        got = H.replay_c(model, requests, steps, scramble_every=3)
+    else:
+        steps = {"whole": H.whole, "tail": H.tail_one_by_one, "portions": H.changing_portions}[cut](requests)
+        model = _model(model_folders, key, dtype)
+        got = H.replay_c(model, requests, steps, scramble_every=4 if cut == "portions" else 0)
+    for rid, toks in requests.items():
+        H.assert_close(got[rid], H.plain_logits(model_folders[(key, dtype)], toks), tol, f"C host {key}/{dtype}/{cut}/{rid}")
+    stats = model.pool_stats()
+    assert stats["free_blocks"] == stats["total_blocks"]
+    model.close()
+
+
+@pytest.mark.parametrize("key", ["a", "b"])
+def test_c_host_float32_is_the_python_engine_bit_for_bit(model_folders, tiny_configs, key):
+    """Both hosts launch the same float32 kernels, whose sums run in an order that a row's own position fixes: the
+    same bits from either host, under different cuttings."""
+    from kipp_amd.engine import Engine
+    cfg = tiny_configs[key]
+    requests = _requests(key, cfg, seed=3)
+    engine = Engine.from_folder(model_folders[(key, "float32")], dtype="float32", page_size=PAGE[key], max_tokens=512, share_prefixes=False)
+    base = H.replay(engine, requests, H.whole(requests))
+    for maker in (H.whole, H.tail_one_by_one, lambda r: H.mixed(r, seed=11)):
+        with _model(model_folders, key, "float32") as model:
+            got = H.replay_c(model, requests, maker(requests))
+        for rid in requests:
+            assert np.array_equal(got[rid], base[rid]), f"{key}/{rid}: the C host's bits differ from the Python engine's"
+
+
+@pytest.mark.parametrize("key", ["a", "b"])
+def test_c_host_gpu_float32_against_its_scalar_path(model_folders, tiny_configs, key):
+    """The GPU's float32 kernels against the scalar C references, through the whole model: same formulas, sums in another
+    order."""
+    from kipp_amd.chost import CModel
+    cfg = tiny_configs[key]
+    requests = _requests(key, cfg, seed=6)
+    steps = H.changing_portions(requests)
+    with _model(model_folders, key, "float32") as gpu, CModel(model_folders[(key, "float32")], path="cpu-fp32", page_tokens=PAGE[key],
+                                                                kv_pool_pages=64, share_prefixes=False) as cpu:
+        got, ref = H.replay_c(gpu, requests, steps), H.replay_c(cpu, requests, steps)
+    for rid in requests:
+        H.assert_close(got[rid], ref[rid].astype(np.float64), 1e-9, f"GPU float32 against the scalar path {key}/{rid}")
+
+
+def test_c_host_sessions_on_the_gpu(model_folders, tiny_configs):
+    """kipp.h's session calls on the bfloat16 path: shared beginnings, eval_n (the wanted tokens one by one) beside
+    eval_scored (one step), truncation, a step that is refused leaves everything as it was."""
+    from kipp_amd.chost import CModel, KippError
+    cfg = tiny_configs["b"]
+    vocab, folder = cfg["vocab_size"], model_folders[("b", "bfloat16")]
+    toks = H.random_tokens(8, 64, vocab)
+    ref = H.plain_logits(folder, toks)
+    with CModel(folder, path="gpu-bf16", page_tokens=8, kv_pool_pages=12) as model:
+        first = model.session()
+        H.assert_close(first.eval(toks[:50])[None], ref[49:50], H.NMSE_BF16["tiny"], "eval")
+        first.destroy()
+        second = model.session()
+        assert second.match_prefix(toks) == 48
+        one_by_one = second.eval_n(toks[48:], 10)
+        H.assert_close(one_by_one, ref[54:], H.NMSE_BF16["tiny"], "eval_n")
+        second.truncate(54)
+        at_once = second.eval_scored(toks[54:], 10)
+        H.assert_close(at_once, ref[54:], H.NMSE_BF16["tiny"], "eval_scored")
+        third = model.session()
+        before = model.pool_stats()["free_blocks"]
+        with pytest.raises(KippError, match="KV pool exhausted"):
+            model.step([(second, [1], [0]), (third, H.random_tokens(1, 40, vocab), [39])])
+        assert model.pool_stats()["free_blocks"] == before and (second.length, third.length) == (64, 0)
+        row = model.step([(third, toks[:20], [19])])
+        H.assert_close(row, ref[19:20], H.NMSE_BF16["tiny"], "a step after a refused one")
+
+
+def test_c_host_products_of_every_row_class(model_folders, tiny_configs):
+    """A prompt of 230 tokens in one step, portions of 9 to 200 rows and single tokens: the bfloat16 products of the C
+    host go to the few-rows kernel, the staged one and the tiled matrix-core kernel by their rows."""
+    cfg = tiny_configs["b"]
+    toks = H.random_tokens(31, 250, cfg["vocab_size"])
+    ref = H.plain_logits(model_folders[("b", "bfloat16")], toks)
+    for cuts in ([230, 1, 1, 18], [9, 200, 40, 1], [3, 5, 130, 110, 2]):
+        with _model(model_folders, "b", "bfloat16") as model:
+            s = model.session()
+            rows = []
+            for n in cuts:
+                at = s.length
+                rows.append(model.step([(s, toks[at:at + n], list(range(n)))]))
+            H.assert_close(np.concatenate(rows), ref, H.NMSE_BF16["tiny"], f"C host, cuts {cuts}")
