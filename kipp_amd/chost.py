@@ -89,6 +89,14 @@ def library(variant: str = "gpu") -> ctypes.CDLL:
     """The loaded C library: "gpu" (every path) or "host-only" (cpu-fp32 alone; needs no HIP to load)."""
     lib = _libs.get(variant)
     if lib is None:
+        if variant == "gpu":
+            # A process has ONE HIP runtime: the first one loaded serves every library that names it.  Where PyTorch
+            # is installed it ships its own, which it must get whether it is imported before or after this library, so
+            # it is loaded first here.  Nothing else of it is used.
+            try:
+                import torch  # noqa: F401
+            except ImportError:
+                pass
         lib = ctypes.CDLL(_build.library_path(variant))
         vp, sz, u32, err = ctypes.c_void_p, ctypes.c_size_t, ctypes.c_uint32, ctypes.POINTER(_Error)
         sigs = {

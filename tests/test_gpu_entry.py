@@ -104,6 +104,47 @@ def test_running_one_step_ahead_changes_nothing(model_folders, dtype):
     assert run(False, stop_of_first=[stop])[0] == stopped
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_one_step_ahead_with_shared_beginnings_and_a_stop_token(model_folders, dtype):
+    """Sharing on: two requests with a common beginning of four pages (the second adopts what the first published early)
+    and a third of its own decode together one step ahead of what the scheduler knows; a stop token ends the first one
+    step late, and its step in vain leaves nothing behind: the same tokens as waiting for every step gives, the plain
+    argmax for the greedy ones, every page back, and a later request still adopts the pages of the one that was stopped."""
+    from kipp_amd.engine import Engine
+    from kipp_amd.engine.scheduler import Request, Scheduler
+    folder = model_folders[("b", dtype)]
+    margin = 1e-5 if dtype == "float32" else 0.03
+    common = H.random_tokens(71, 32, 509)
+    prompts = [common + H.random_tokens(72, 6, 509), common + H.random_tokens(73, 11, 509), H.random_tokens(74, 21, 509)]
+
+    def run(lookahead, stop=()):
+        engine = Engine.from_folder(folder, dtype=dtype, page_size=8, max_tokens=4 * 128, share_prefixes=True)
+        sched = Scheduler(engine, max_step_tokens=32, prefill_chunk=16, lookahead=lookahead)
+        for i, prompt in enumerate(prompts):
+            sched.add(Request(i, prompt, [30, 12, 18][i], stop_tokens=tuple(stop) if i == 0 else ()))
+        done = sched.run()
+        assert sched.stats.prefix_tokens_reused == 32
+        # the one that was stopped published its pages as it went: a request that begins like it adopts them
+        sched.add(Request("late", prompts[0] + done[0].output[:9], 3))
+        late = sched.run()["late"]
+        assert sched.stats.prefix_tokens_reused == 32 + (len(prompts[0]) + min(9, len(done[0].output)) - 1) // 8 * 8
+        engine.cache.check()
+        assert engine.cache.free_pages() == [64] and not engine._uncommitted
+        return {rid: (r.output, r.finish_reason) for rid, r in done.items() if rid != "late"}, late.output, sched.stats.steps
+
+    plainly, late_plainly, _ = run(False)
+    ahead, late_ahead, _ = run(True)
+    assert ahead == plainly and late_ahead == late_plainly
+    for i in range(3):
+        _follows_plain_argmax(folder, prompts[i], ahead[i][0], margin)
+    stop = plainly[0][0][14]
+    first = plainly[0][0].index(stop)
+    stopped, late_stopped, _ = run(True, stop=[stop])
+    assert stopped[0] == (plainly[0][0][:first], "stop") and stopped[1] == plainly[1] and stopped[2] == plainly[2]
+    assert run(False, stop=[stop])[:2] == (stopped, late_stopped)
+    _follows_plain_argmax(folder, prompts[0] + stopped[0][0][:9], late_stopped, margin)
+
+
 def test_the_scheduler_with_many_requests(model_folders):
     """150 requests at once (more than one 128-row product and more than the default of running requests):
     greedy and seeded sampling, lengths of 3 to 20; one step ahead gives what waiting for every step gives,

@@ -38,16 +38,82 @@ def test_benchmark_layer_sizes_match_plain(real_folder, real_reference, dtype):
     from kipp_amd.engine import Engine
     requests, refs = real_reference
     tol = H.NMSE_F32 if dtype == "float32" else H.NMSE_BF16["real"]
-    for cut, maker in (("whole", H.whole), ("tail", lambda r: H.tail_one_by_one(r, 20)), ("mixed", lambda r: H.mixed(r, seed=4))):
+    _cuttings_against_plain(real_folder, requests, refs, dtype, tol, "4B sizes")
+
+
+CUTTINGS = (("whole", H.whole), ("tail", lambda r: H.tail_one_by_one(r, 20)), ("portions", H.changing_portions),
+            ("mixed", lambda r: H.mixed(r, seed=4)))
+
+
+def _cuttings_against_plain(folder, requests, refs, dtype, tol, what):
+    """Whole prompts, the last 20 tokens one by one, portions of changing size down to two tokens, and a mixed batch
+    with as many pages as the live requests hold at their peak."""
+    from kipp_amd.engine import Engine
+    for cut, maker in CUTTINGS:
         steps = maker(requests)
-        engine = Engine.from_folder(real_folder, dtype=dtype, page_size=16, num_pages=H.peak_pages(requests, steps, 16),
+        engine = Engine.from_folder(folder, dtype=dtype, page_size=16, num_pages=H.peak_pages(requests, steps, 16),
                                     max_requests=4, share_prefixes=False)
         got = H.replay(engine, requests, steps)
         for rid in requests:
-            H.assert_close(got[rid], refs[rid], tol, f"4B sizes/{dtype}/{cut}/{rid}")
+            H.assert_close(got[rid], refs[rid], tol, f"{what}/{dtype}/{cut}/{rid}")
             if dtype == "float32":
                 assert np.array_equal(got[rid].argmax(axis=1), refs[rid].argmax(axis=1))
+        if dtype == "bfloat16":
+            assert engine.rt.generic_attention_launches == 0 and engine.rt.library_products == 0
         del engine
+
+
+# The layer sizes of the two larger shapes that the serving workloads run (Qwen3-8B: hidden 4096, SwiGLU 12288, 32 query
+# heads; Qwen3-32B: hidden 5120, SwiGLU 25600, 64 query heads, eight to a key/value head; both with a head of its own),
+# two layers each and a small vocabulary that is no power of two, so that the plain implementation stays affordable.
+LARGER = {"qwen3-8b": {"p": 150, "q": 37, "r": 70}, "qwen3-32b": {"p": 100, "q": 37, "r": 50}}
+
+
+@pytest.fixture(scope="module", params=sorted(LARGER))
+def larger_shape(request, tmp_path_factory):
+    from kipp_amd.config import shape_config
+    from kipp_amd.weights import write_random_model
+    shape = request.param
+    cfg = shape_config(shape)
+    cfg.update(num_hidden_layers=2, vocab_size=2053)
+    folder = str(tmp_path_factory.mktemp("larger") / f"{shape}-2layers")
+    write_random_model(folder, cfg, seed=23, dtype="bfloat16")
+    plain_cfg, weights = plain.load_folder(folder)
+    requests = {rid: H.random_tokens(40 + i, n, 2053) for i, (rid, n) in enumerate(LARGER[shape].items())}
+    refs = {rid: plain.forward_whole(plain_cfg, weights, toks) for rid, toks in requests.items()}
+    del weights
+    return shape, folder, requests, refs
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_the_larger_shapes_layer_sizes_match_plain(larger_shape, dtype):
+    """What the serving workloads run at: products of 4,096 and 5,120 columns against up to 51,200 rows, 64 query heads in
+    groups of eight, the few-rows products that keep their norm's kernel because every workgroup would read too much of x
+    (the 32B sizes), an untied head."""
+    shape, folder, requests, refs = larger_shape
+    tol = H.NMSE_F32 if dtype == "float32" else H.NMSE_BF16["real"]
+    _cuttings_against_plain(folder, requests, refs, dtype, tol, f"{shape} sizes")
+
+
+@pytest.mark.parametrize("fault", ["read-slot", "other-run"])
+def test_the_tolerance_at_these_sizes_notices_a_cache_fault(real_folder, real_reference, fault):
+    """The bound for bfloat16 at the benchmark's layer sizes is wider than at the tiny sizes; it still fails a run in which
+    every read of the cache lands one slot further, or every layer but the first reads the first layer's cache."""
+    from kipp_amd.engine import Engine
+    from tests.test_gpu_adversarial import Faulty
+    requests, refs = real_reference
+    steps = H.tail_one_by_one(requests, 20)
+    engine = Engine.from_folder(real_folder, dtype="bfloat16", page_size=16, num_pages=H.peak_pages(requests, steps, 16) + 2,
+                                max_requests=4, share_prefixes=False, use_graphs=False)
+    faulty = Faulty(engine.rt.ops, fault, engine)
+    engine.rt.ops = faulty
+    got = H.replay(engine, requests, steps)
+    assert faulty.hits > 0
+    worst = max(plain.nmse(got[rid][i], refs[rid][i]) for rid in requests for i in range(len(requests[rid])))
+    assert worst > 10 * H.NMSE_BF16["real"], f"{fault}: worst NMSE {worst:.2e} is no further from the bound than rounding"
+    with pytest.raises(AssertionError):
+        for rid in requests:
+            H.assert_close(got[rid], refs[rid], H.NMSE_BF16["real"], f"4B sizes/{fault}/{rid}")
 
 
 def test_split_products_keep_their_norm_kernels(real_folder, real_reference):
@@ -121,6 +187,35 @@ def test_decoding_across_a_graph_bucket_and_many_splits(long_folder, dtype):
     for rid in seqs:
         first = {"long": 1000, "mid": 240, "short": 10}[rid]
         H.assert_close(np.stack(got[rid]), refs[rid][first:fed[rid]], tol, f"long context/{dtype}/{rid}")
+
+
+def test_the_splits_merged_by_a_launch_of_its_own(long_folder):
+    """`Runtime.merge_in_kernel = False` (KIPP_AMD_DECODE_MERGE=launch) drops the count of finished splits: decode
+    attention then merges a head's splits in a launch of its own, which needs no ordering between workgroups.  The same
+    sums in the same order: behind 700 and 300 tokens (several splits a head) the same bits as merged by the last
+    workgroup, eager and as recorded graphs, and the plain implementation's values."""
+    from kipp_amd.engine import Engine, StepEntry
+    from kipp_amd.engine.model import load_model
+    from kipp_amd.runtime import Runtime
+    cfg, weights = plain.load_folder(long_folder)
+    seqs = {"long": H.random_tokens(41, 720, 311), "mid": H.random_tokens(42, 320, 311)}
+    got = {}
+    for merge in (True, False):
+        rt = Runtime("bfloat16")
+        rt.merge_in_kernel = merge
+        engine = Engine(load_model(long_folder, rt), page_size=16, max_tokens=1152, max_requests=2, share_prefixes=False)
+        for rid, toks in seqs.items():
+            engine.step([StepEntry(rid, toks[:-20], [])])
+        rows = []
+        for i in range(20, 0, -1):
+            rows.append(engine.step([StepEntry(rid, [toks[-i]], [0]) for rid, toks in seqs.items()]).cpu().numpy())
+        got[merge] = np.stack(rows)
+        spaces = [space for graph in engine.graphs.graphs.values() for name, space in graph.batch.host.items()
+                  if isinstance(name, tuple) and name[0] == "decode_workspace"]
+        assert engine.graphs.replays >= 10 and spaces and all((len(space) == 3) == merge for space in spaces)
+    assert np.array_equal(got[True], got[False])
+    for at, (rid, toks) in enumerate(seqs.items()):
+        H.assert_close(got[False][:, at], plain.forward_whole(cfg, weights, toks)[-20:], H.NMSE_BF16["real"], f"merge by a launch/{rid}")
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
