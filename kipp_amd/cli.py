@@ -6,6 +6,12 @@ KIPP_METRIC line.  The prompt is token ids (this engine has no tokenizer).
     python -m kipp_amd.cli --model DIR --tokens 5,17,3 --decode 16
     python -m kipp_amd.cli --model DIR --ppl tokens.u32 --ppl-window 512
     python -m kipp_amd.cli --write-random DIR --random tiny-a --seed-weights 7
+    python -m kipp_amd.cli --random tiny-b --seed-weights 3 --tokens 5,17,3 --decode 8      (a model made for this run)
+    python -m kipp_amd.cli --model DIR --path cpu-fp32 --tokens 5,17,3 --decode 8             (the C host's scalar path)
+
+`--path` names the execution path as the reference's `--backend` names its own (never a fallback): gpu-bf16 and
+gpu-fp32 are `--dtype bfloat16|float32`; cpu-fp32 is the scalar path of the C host, which needs no GPU.  `--host c`
+runs the GPU paths through the C host as well.
 """
 from __future__ import annotations
 
@@ -36,6 +42,12 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--backend", default="hip", help="explicit backend; this engine has one, hip, and never falls back")
     ap.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16",
                     help="execution path (default bfloat16; float32 is the true 32-bit path)")
+    ap.add_argument("--path", choices=["gpu-bf16", "gpu-fp32", "cpu-fp32"], default=None,
+                    help="execution path by name: gpu-bf16, gpu-fp32 (as --dtype), or cpu-fp32, the scalar path of the C host")
+    ap.add_argument("--host", choices=["python", "c"], default="python", help="the host that drives the kernels (cpu-fp32 is the C host's)")
+    ap.add_argument("--max-context", type=int, default=0,
+                    help="most tokens the session may hold (default: the model's positions); prompt + decode beyond it is refused")
+    ap.add_argument("--kv-mib", type=float, default=0.0, help="size of the page pool in MiB (instead of --kv-pages)")
     ap.add_argument("--decode", type=int, default=0, help="greedy/sampled tokens to generate")
     ap.add_argument("--temperature", type=float, default=0.0, help="0 = greedy argmax (default)")
     ap.add_argument("--top-p", type=float, default=1.0, help="nucleus mass, 0 < F <= 1 (default 1)")
@@ -52,7 +64,8 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--kv-pages", type=int, default=None, help="pages in the pool (default: enough for this run)")
     ap.add_argument("--prefill-chunk", type=int, default=512, help="largest portion of a prompt in one step")
     ap.add_argument("--max-step-tokens", type=int, default=2048, help="token budget of one step")
-    ap.add_argument("--random", metavar="SHAPE", help="with --write-random: named shape (tiny-a, tiny-b, qwen3-4b, ...)")
+    ap.add_argument("--random", metavar="SHAPE",
+                    help="named shape (tiny-a, tiny-b, qwen3-4b, ...): with --write-random the folder to write, else the model of this run")
     ap.add_argument("--seed-weights", type=int, default=0, help="seed of the random weights")
     ap.add_argument("--write-random", metavar="DIR", help="write a random-weights model folder and exit")
     ap.add_argument("--weights-dtype", choices=["bfloat16", "float32"], default="bfloat16")
@@ -119,9 +132,105 @@ def main(argv=None) -> int:
         write_random_model(args.write_random, shape_config(args.random), args.seed_weights, args.weights_dtype)
         print(f"kipp: wrote {args.random} (seed {args.seed_weights}, {args.weights_dtype}) to {args.write_random}", file=sys.stderr)
         return 0
+    if args.path is not None:
+        if args.path != "cpu-fp32":
+            args.dtype = "bfloat16" if args.path == "gpu-bf16" else "float32"
+        else:
+            args.host = "c"
+    made = None
+    if not args.model and args.random:
+        # a model with random weights made for this run, in a folder that goes away with it
+        import tempfile
+        from .config import shape_config
+        from .weights import write_random_model
+        made = tempfile.TemporaryDirectory(prefix="kipp-random-")
+        args.model = write_random_model(made.name, shape_config(args.random), args.seed_weights, args.weights_dtype)
     if not args.model:
-        raise SystemExit("kipp: --model is required")
+        raise SystemExit("kipp: --model (or --random SHAPE) is required")
+    try:
+        return _run(args)
+    finally:
+        if made is not None:
+            made.cleanup()
+
+
+def _pool_pages(args, capacity: int, bytes_per_page: int) -> int:
+    """Pages of the pool: --kv-pages, or what --kv-mib holds (/root/reference/src/kipp_server.c:2681-2698), or enough for
+    this run."""
+    if args.kv_mib:
+        pages = int(args.kv_mib * 1024 * 1024) // max(1, bytes_per_page)
+        if pages < 1:
+            raise SystemExit(f"kipp: --kv-mib {args.kv_mib:g} holds no page of {bytes_per_page} bytes")
+        return pages
+    return args.kv_pages or -(-capacity // args.page)
+
+
+def _check_capacity(n_prompt: int, decode: int, limit: int) -> None:
+    """/root/reference/src/kipp_cli.c:1057-1067: the session holds prompt + decode tokens, within the context length."""
+    if n_prompt > limit or decode > limit - n_prompt:
+        raise SystemExit(f"kipp: session: {n_prompt} prompt tokens and {decode} to decode exceed the context of {limit} tokens")
+
+
+def run_c_host(args, tokens) -> int:
+    """The same run through the C host (`kipp_amd/host`): prompt in portions, then one token a step, tokens chosen by
+    the C sampler; `--path cpu-fp32` is its scalar path and needs no GPU."""
+    import numpy as np
+    from .chost import CModel, Rng, sample
+    from .config import load_config
+    path = args.path or ("gpu-bf16" if args.dtype == "bfloat16" else "gpu-fp32")
+    _, cfg = load_config(args.model)
+    spec = cfg.model_spec()
+    limit = min(args.max_context or spec.max_position, spec.max_position)
+    _check_capacity(len(tokens), max(args.decode, 0), limit)
+    capacity = len(tokens) + max(args.decode, 0)
+    from .engine.model import cache_bytes_per_page
+    per_page = cache_bytes_per_page(spec, args.page, 2 if path == "gpu-bf16" else 4) if args.kv_mib else 0
+    pages = _pool_pages(args, capacity, per_page)
+    model = CModel(args.model, path=path, page_tokens=args.page, kv_pool_pages=pages, max_sessions=1,
+                   max_step_tokens=max(args.prefill_chunk, 1), share_prefixes=False)
+    stops = tuple(args.stop_token) if args.stop_token is not None else tuple(spec.stop_tokens)
+    print(f"kipp: evaluating {len(tokens)} token{'s' if len(tokens) != 1 else ''} on {path} (C host)", file=sys.stderr)
+    session = model.session(capacity)
+    rng = Rng(args.seed)
+    started = time.perf_counter()
+    row = None
+    for at in range(0, len(tokens), args.prefill_chunk):
+        chunk = tokens[at:at + args.prefill_chunk]
+        last = at + len(chunk) == len(tokens)
+        out = model.step([(session, chunk, [len(chunk) - 1] if last else [])])
+        row = out[0] if last else row
+    prefill_seconds = time.perf_counter() - started
+    started = time.perf_counter()
+    output = []
+    if args.decode > 0:
+        sys.stdout.write("generated\t")
+        while True:
+            token = sample(row, args.temperature, args.top_p, args.top_k, args.min_p, rng=rng)
+            if token in stops:
+                break
+            sys.stdout.write(("" if not output else " ") + str(token))
+            sys.stdout.flush()
+            output.append(token)
+            if len(output) >= args.decode:
+                break
+            row = model.step([(session, [token], [0])])[0]
+        sys.stdout.write("\n")
+    decode_seconds = time.perf_counter() - started
+    order = sorted(range(len(row)), key=lambda i: (-float(row[i]), i))[:min(args.top, len(row))] if len(row) < 4096 else \
+        sorted(np.argpartition(-row, args.top)[:args.top].tolist(), key=lambda i: (-float(row[i]), i))
+    for rank, i in enumerate(order, 1):
+        print(f"{rank}\t{int(i)}\t{float(row[i]):.9g}")
+    decoded = max(0, len(output) - 1) if args.decode else 0
+    print(f"KIPP_METRIC backend={path} prefill_tokens={len(tokens)} prefill_seconds={prefill_seconds:.9f} "
+          f"decode_tokens={decoded} decode_seconds={decode_seconds:.9f}", file=sys.stderr)
+    model.close()
+    return 0
+
+
+def _run(args) -> int:
     if args.ppl:
+        if args.host == "c":
+            raise SystemExit("kipp: --ppl runs on the Python host")
         return run_perplexity(args)
     if not 1 <= args.top <= 100:
         raise SystemExit("kipp: --top must be between 1 and 100")
@@ -131,14 +240,25 @@ def main(argv=None) -> int:
     if not tokens:
         raise SystemExit("kipp: the prompt is empty")
 
+    if args.host == "c":
+        return run_c_host(args, tokens)
+
     import torch
+    from .config import load_config
     from .engine import Engine, StepEntry
+    from .engine.model import cache_bytes_per_page
     from .engine.scheduler import Request, Scheduler
     from .sampling import SampleParams
 
+    _, cfg = load_config(args.model)
+    spec = cfg.model_spec()
+    limit = min(args.max_context or spec.max_position, spec.max_position)
+    _check_capacity(len(tokens), max(args.decode, 0), limit)
     capacity = len(tokens) + args.decode
-    pages = args.kv_pages or -(-capacity // args.page)
-    engine = Engine.from_folder(args.model, dtype=args.dtype, page_size=args.page, num_pages=pages, max_requests=1)
+    per_page = cache_bytes_per_page(spec, args.page, 2 if args.dtype == "bfloat16" else 4) if args.kv_mib else 0
+    pages = _pool_pages(args, capacity, per_page)
+    engine = Engine.from_folder(args.model, dtype=args.dtype, page_size=args.page, num_pages=pages, max_requests=1,
+                                max_position=limit)
     stops = tuple(args.stop_token) if args.stop_token is not None else tuple(engine.model.spec.stop_tokens)
     backend = f"hip-{args.dtype}"
     print(f"kipp: evaluating {len(tokens)} token{'s' if len(tokens) != 1 else ''} on {backend}", file=sys.stderr)

@@ -36,6 +36,19 @@ def model_params(spec: ModelSpec) -> Dict[str, ParamSpec]:
     return out
 
 
+def cache_bytes_per_page(spec: ModelSpec, page_size: int, element_size: int) -> int:
+    """Bytes one page of every cache group takes together, from what the mixers of the spec declare (`need_of(spec)`, a
+    static method of a mixer class that keeps keys and values); no device is touched.  Sizes a pool given in bytes."""
+    from ..cache import CacheManager
+    needs = []
+    for run in spec.order:
+        mixer = dict(spec.layers[run.layer].parts).get("mixer")
+        need_of = getattr(part_class("mixer", mixer.kind), "need_of", None) if mixer is not None else None
+        needs.append(need_of(mixer) if need_of is not None and run.cache_of is None else None)
+    groups = CacheManager(needs, [None] * len(needs), page_size, 1, 1, spec.max_position, runtime=None).groups
+    return sum(g.bytes_per_token(element_size) * g.page_size for g in groups)
+
+
 class Model:
     def __init__(self, spec: ModelSpec, runtime):
         self.spec = spec

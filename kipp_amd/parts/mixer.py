@@ -86,9 +86,13 @@ class Attention:
             self.q_norm = tensors["q_norm.weight"]
             self.k_norm = tensors["k_norm.weight"]
 
+    @staticmethod
+    def need_of(spec):
+        """What a mixer of this spec keeps per token, known without building it."""
+        return KVNeed(num_kv_heads=spec.num_kv_heads, head_dim=spec.head_dim, window=spec.window, page_size=spec.page_size)
+
     def cache_need(self):
-        s = self.spec
-        return KVNeed(num_kv_heads=s.num_kv_heads, head_dim=s.head_dim, window=s.window, page_size=s.page_size)
+        return self.need_of(self.spec)
 
     def state_need(self):
         return None

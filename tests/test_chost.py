@@ -385,3 +385,39 @@ def test_the_host_compiles_without_warnings():
         for src in build._sources(gpu):
             proc = subprocess.run([build._compiler()] + flags + ["-fsyntax-only", src], capture_output=True, text=True)
             assert proc.returncode == 0 and "warning" not in proc.stderr, proc.stderr
+
+
+def test_command_line_on_the_scalar_path(model_folders, tiny_configs, capsys):
+    """`--path cpu-fp32`: the command line through the C host, no GPU: the greedy tokens are the plain argmax, the top-N
+    table is that of the last token that counts, one KIPP_METRIC line; --max-context and --kv-mib are checked before
+    anything runs (/root/reference/src/kipp_cli.c:1057-1067, 1213-1217)."""
+    from kipp_amd.cli import main
+    from tests.plain import qwen3_plain as plain
+    folder = model_folders[("b", "float32")]
+    prompt = H.random_tokens(17, 11, tiny_configs["b"]["vocab_size"])
+    common = ["--model", folder, "--path", "cpu-fp32", "--tokens", ",".join(map(str, prompt)), "--page", "8"]
+    assert main(common + ["--decode", "7", "--top", "4", "--prefill-chunk", "4"]) == 0
+    out, err = capsys.readouterr()
+    lines = out.strip().splitlines()
+    assert lines[0].startswith("generated\t")
+    generated = [int(t) for t in lines[0].split("\t")[1].split()]
+    cfg, weights = plain.load_folder(folder)
+    logits = plain.forward_whole(cfg, weights, prompt + generated)
+    for i, token in enumerate(generated):
+        assert token == int(np.argmax(logits[len(prompt) - 1 + i]))
+    table = [line.split("\t") for line in lines[1:]]
+    last = logits[len(prompt) + len(generated) - 2]                # the row the last generated token was chosen from
+    assert [int(r[1]) for r in table] == [int(i) for i in np.argsort(-last)[:4]] and [int(r[0]) for r in table] == [1, 2, 3, 4]
+    assert abs(float(table[0][2]) - last.max()) < 1e-4
+    assert f"KIPP_METRIC backend=cpu-fp32 prefill_tokens={len(prompt)}" in err and "decode_tokens=6" in err
+    with pytest.raises(SystemExit, match="exceed the context of 12 tokens"):
+        main(common + ["--decode", "7", "--max-context", "12"])
+    with pytest.raises(SystemExit, match="holds no page"):
+        main(common + ["--decode", "2", "--kv-mib", "0.001"])
+    assert main(common + ["--decode", "5", "--kv-mib", "0.02", "--temperature", "0.8", "--seed", "9"]) == 0    # 3 pages of 6,144 bytes
+    first = capsys.readouterr().out.splitlines()[0]
+    assert main(common + ["--decode", "5", "--kv-mib", "0.02", "--temperature", "0.8", "--seed", "9"]) == 0
+    assert capsys.readouterr().out.splitlines()[0] == first       # seeded
+    with pytest.raises(KippError, match="KV pool exhausted"):
+        main(common + ["--decode", "20", "--kv-mib", "0.02"])      # 31 tokens need 4 pages
+    assert main(["--random", "tiny-a", "--seed-weights", "4", "--path", "cpu-fp32", "--tokens", "1,2,3", "--decode", "2"]) == 0
