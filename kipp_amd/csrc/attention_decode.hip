@@ -14,9 +14,12 @@
 //            at head size 128), the 16 lane groups of the workgroup take every
 //            16th key; products in float32 FMA, summed over the groups in LDS.
 //
-// Split boundaries are multiples of SPLIT in absolute key index, and the merge
-// adds the splits in index order, so the result for a token does not depend on
-// the batch it is in.  A sequence that needs one split only is written
+// Split boundaries are multiples of the split's length in absolute key index, and the
+// merge adds the splits in index order, so within one launch shape the result for a
+// token does not depend on what else is in the batch.  The split's length (192, 256 or
+// 320 keys) and the kernel follow from the launch's shape (rows, key/value heads,
+// longest context), so between shapes, batch 1 and batch 8 say, a token's bits may
+// differ in the last place.  A sequence that needs one split only is written
 // normalised at once.  The merge is done by whichever workgroup of a (token,
 // key/value head) finishes last: every workgroup writes its partial result
 // through to memory (stores of device scope: the dies' L2 caches do not see each
