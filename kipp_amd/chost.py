@@ -76,6 +76,37 @@ class _SampleParams(ctypes.Structure):
                 ("logit_bias_values", _f32p), ("logit_bias_count", ctypes.c_size_t)]
 
 
+class _SchedulerConfig(ctypes.Structure):
+    _fields_ = [("max_step_tokens", ctypes.c_uint32), ("prefill_chunk", ctypes.c_uint32), ("max_running", ctypes.c_uint32),
+                ("keep_last_logits", ctypes.c_int)]
+
+
+class _Request(ctypes.Structure):
+    _fields_ = [("id", ctypes.c_uint64), ("prompt", _u32p), ("prompt_count", ctypes.c_size_t), ("max_new_tokens", ctypes.c_uint32),
+                ("params", _SampleParams), ("seed", ctypes.c_uint64), ("stop_tokens", ctypes.c_uint32 * _MAX_STOP),
+                ("stop_token_count", ctypes.c_uint32)]
+
+
+class _Produced(ctypes.Structure):
+    _fields_ = [("id", ctypes.c_uint64), ("token", ctypes.c_uint32)]
+
+
+class _Result(ctypes.Structure):
+    _fields_ = [("id", ctypes.c_uint64), ("reason", ctypes.c_int), ("output", _u32p), ("output_count", ctypes.c_size_t),
+                ("error", ctypes.c_char_p)]
+
+
+class _SchedulerStats(ctypes.Structure):
+    _fields_ = [(name, ctypes.c_uint64) for name in ("requests", "refused", "finished", "failed", "failed_steps", "prompt_tokens",
+                                                     "generated_tokens", "prefix_tokens_reused", "steps", "waits_for_pages",
+                                                     "waits_for_prefix")] + \
+               [("queue_wait_seconds_sum", ctypes.c_double), ("queue_wait_count", ctypes.c_uint64), ("ttft_seconds_sum", ctypes.c_double),
+                ("ttft_count", ctypes.c_uint64), ("decode_seconds_sum", ctypes.c_double)]
+
+
+FINISH_REASONS = {0: None, 1: "length", 2: "stop", 3: "cancelled", 4: "failed"}
+
+
 class KippError(RuntimeError):
     def __init__(self, code: str, message: str):
         super().__init__(f"{code}: {message}")
@@ -117,11 +148,22 @@ def library(variant: str = "gpu") -> ctypes.CDLL:
             "kipp_step": [vp, ctypes.POINTER(_StepItem), sz, _f32p, sz, err],
             "kipp_sample_ex": [_f32p, sz, ctypes.POINTER(_SampleParams), ctypes.POINTER(ctypes.c_uint64), _u32p, err],
             "kipp_test_scramble_session_kv": [vp, err],
+            "kipp_scheduler_create": [vp, ctypes.POINTER(_SchedulerConfig), ctypes.POINTER(vp), err],
+            "kipp_scheduler_add": [vp, ctypes.POINTER(_Request), err],
+            "kipp_scheduler_cancel": [vp, ctypes.c_uint64, err],
+            "kipp_scheduler_step": [vp, ctypes.POINTER(_Produced), sz, ctypes.POINTER(sz), err],
+            "kipp_scheduler_idle": [vp],
+            "kipp_scheduler_result": [vp, ctypes.c_uint64, ctypes.POINTER(_Result)],
+            "kipp_scheduler_collect": [vp, ctypes.c_uint64],
+            "kipp_scheduler_get_stats": [vp, ctypes.POINTER(_SchedulerStats)],
         }
         for name, argtypes in sigs.items():
             fn = getattr(lib, name)
             fn.argtypes, fn.restype = argtypes, ctypes.c_int
         lib.kipp_session_destroy.argtypes, lib.kipp_session_destroy.restype = [vp], None
+        lib.kipp_scheduler_destroy.argtypes, lib.kipp_scheduler_destroy.restype = [vp], None
+        lib.kipp_scheduler_last_logits.argtypes, lib.kipp_scheduler_last_logits.restype = [vp, ctypes.c_uint64], _f32p
+        lib.kipp_test_fail_forward_after.argtypes, lib.kipp_test_fail_forward_after.restype = [vp, ctypes.c_int], None
         lib.kipp_error_code_name.argtypes, lib.kipp_error_code_name.restype = [ctypes.c_int], ctypes.c_char_p
         lib.kipp_test_session_pages.argtypes = [vp, u32, ctypes.POINTER(ctypes.c_int32), sz]
         lib.kipp_test_session_pages.restype = sz
@@ -301,6 +343,83 @@ class CModel:
 
     def __exit__(self, *exc):
         self.close()
+
+
+class CScheduler:
+    """The C scheduler (`host/scheduler.c`) over a `CModel`: requests in, (request, token) pairs out."""
+
+    def __init__(self, model: CModel, max_step_tokens: int = 2048, prefill_chunk: int = 512, max_running: int = 0,
+                 keep_last_logits: bool = False):
+        self.model, self.lib = model, model.lib
+        config = _SchedulerConfig(max_step_tokens, prefill_chunk, max_running, int(keep_last_logits))
+        handle, error = ctypes.c_void_p(), _Error()
+        if self.lib.kipp_scheduler_create(model.handle, ctypes.byref(config), ctypes.byref(handle), ctypes.byref(error)) != 0:
+            _raise(self.lib, error)
+        self.handle = handle
+        self._produced = (_Produced * 1024)()
+
+    def add(self, request_id: int, prompt: Sequence[int], max_new_tokens: int, temperature: float = 0.0, top_p: float = 1.0,
+            top_k: int = 0, min_p: float = 0.0, frequency_penalty: float = 0.0, presence_penalty: float = 0.0,
+            repetition_penalty: float = 1.0, logit_bias: Optional[dict] = None, seed: int = 1, stop_tokens: Sequence[int] = ()) -> None:
+        p, pp = _u32(prompt)
+        bias = logit_bias or {}
+        bt, btp = _u32(list(bias.keys()))
+        bv = np.ascontiguousarray(np.asarray(list(bias.values()), dtype=np.float32))
+        params = _SampleParams(temperature, top_p, top_k, min_p, frequency_penalty, presence_penalty, repetition_penalty, None, 0,
+                               btp if len(bt) else None, bv.ctypes.data_as(_f32p) if len(bv) else None, len(bt))
+        stops = (ctypes.c_uint32 * _MAX_STOP)(*list(stop_tokens)[:_MAX_STOP])
+        request = _Request(request_id, pp, len(p), max_new_tokens, params, seed, stops, len(stop_tokens))
+        error = _Error()
+        if self.lib.kipp_scheduler_add(self.handle, ctypes.byref(request), ctypes.byref(error)) != 0:
+            _raise(self.lib, error)
+
+    def step(self):
+        """One step; the (request id, token) pairs that became known."""
+        count, error = ctypes.c_size_t(0), _Error()
+        if self.lib.kipp_scheduler_step(self.handle, self._produced, 1024, ctypes.byref(count), ctypes.byref(error)) != 0:
+            _raise(self.lib, error)
+        return [(int(self._produced[i].id), int(self._produced[i].token)) for i in range(min(count.value, 1024))]
+
+    @property
+    def idle(self) -> bool:
+        return bool(self.lib.kipp_scheduler_idle(self.handle))
+
+    def run(self, max_steps: int = 100000) -> None:
+        steps = 0
+        while not self.idle and steps < max_steps:
+            self.step()
+            steps += 1
+
+    def cancel(self, request_id: int) -> None:
+        error = _Error()
+        if self.lib.kipp_scheduler_cancel(self.handle, request_id, ctypes.byref(error)) != 0:
+            _raise(self.lib, error)
+
+    def result(self, request_id: int) -> dict:
+        out = _Result()
+        if self.lib.kipp_scheduler_result(self.handle, request_id, ctypes.byref(out)) != 0:
+            raise KeyError(request_id)
+        return {"id": int(out.id), "finish_reason": FINISH_REASONS[out.reason], "output": [int(out.output[i]) for i in range(out.output_count)],
+                "error": (out.error or b"").decode("utf-8", "replace")}
+
+    def last_logits(self, request_id: int) -> Optional[np.ndarray]:
+        ptr = self.lib.kipp_scheduler_last_logits(self.handle, request_id)
+        return np.ctypeslib.as_array(ptr, shape=(self.model.vocab_size,)).copy() if ptr else None
+
+    def collect(self, request_id: int) -> None:
+        if self.lib.kipp_scheduler_collect(self.handle, request_id) != 0:
+            raise KeyError(request_id)
+
+    @property
+    def stats(self) -> dict:
+        st = _SchedulerStats()
+        self.lib.kipp_scheduler_get_stats(self.handle, ctypes.byref(st))
+        return {name: getattr(st, name) for name, _ in _SchedulerStats._fields_}
+
+    def destroy(self) -> None:
+        if self.handle is not None:
+            self.lib.kipp_scheduler_destroy(self.handle)
+            self.handle = None
 
 
 class Rng:

@@ -20,7 +20,7 @@ from typing import List, Tuple
 HERE = os.path.dirname(os.path.abspath(__file__))
 REF = os.path.join(os.path.dirname(HERE), "csrc", "ref")
 SOURCES = ["error.c", "json.c", "config.c", "safetensors.c", "pool.c", "cache.c", "runtime.c", "backend_cpu.c", "parts.c",
-           "model.c", "step.c", "sampler.c", "hooks.c"]
+           "model.c", "step.c", "scheduler.c", "sampler.c", "hooks.c"]
 GPU_SOURCES = ["backend_hip.c"]
 # -ffp-contract=off: a sum's bits must not depend on how the compiler happened to fuse a loop
 FLAGS = ["-std=c11", "-O2", "-fPIC", "-D_GNU_SOURCE", "-ffp-contract=off", "-Wall", "-Wextra", "-Werror=implicit-function-declaration"]
@@ -115,6 +115,29 @@ def library_path(variant: str = "gpu", force: bool = False) -> str:
     return out
 
 
+def cli_path(force: bool = False) -> str:
+    """The built command line of the C host (`kipp_cli.c` linked against the library's sources): `_lib/kipp.<hash>`."""
+    files = [os.path.join(HERE, "kipp_cli.c")] + _sources(True)
+    compile_flags, link = _flags(True, False)
+    name = f"kipp.{_digest(files, compile_flags + link)}"
+    in_tree = os.path.join(HERE, "_lib", name)
+    if os.path.exists(in_tree) and not force:
+        return in_tree
+    out = os.path.join(_out_dir(), name)
+    if os.path.exists(out) and not force:
+        return out
+    tmp = f"{out}.{os.getpid()}.tmp"
+    _run([_compiler()] + compile_flags + files + ["-o", tmp] + link, "compiling the command line of the C host")
+    os.replace(tmp, out)
+    for stale in os.listdir(os.path.dirname(out)):
+        if stale.startswith("kipp.") and not stale.endswith(".so") and stale != name and ".tmp" not in stale:
+            try:
+                os.remove(os.path.join(os.path.dirname(out), stale))
+            except OSError:
+                pass
+    return out
+
+
 def test_program(source: str, out: str, sanitize: bool = True) -> str:
     """An executable of `source` (a C file with main) linked with the host's sources without the GPU's table,
     by default under AddressSanitizer and UndefinedBehaviorSanitizer."""
@@ -127,5 +150,10 @@ test_program.__test__ = False
 
 
 if __name__ == "__main__":
-    print(library_path("gpu", force=True))
-    print(library_path("host-only", force=True))
+    import sys
+    if "--cli" in sys.argv:
+        print(cli_path())           # what bin/kipp-c runs: built if it is not there
+    else:
+        print(library_path("gpu", force=True))
+        print(library_path("host-only", force=True))
+        print(cli_path(force=True))

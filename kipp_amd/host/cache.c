@@ -211,6 +211,12 @@ int kipp_cache_adopt(kipp_cache *cache, kipp_session *session, const uint32_t *t
     }
     session->adopted_tokens = session->length = keep * cache->page_tokens;
     memcpy(session->tokens, tokens, (size_t)session->length * sizeof(uint32_t));
+    session->published = keep;
+    session->chain = 0;
+    for (uint32_t block = 0; block < keep; ++block) {
+        const kipp_pool *pool = &cache->groups[0].pool;
+        session->chain = pool->force_hash ? pool->forced_hash : kipp_pool_chain_hash(session->chain, tokens + (size_t)block * cache->page_tokens, cache->page_tokens);
+    }
     *matched = session->length;
     return 0;
 }
@@ -249,6 +255,16 @@ void kipp_cache_trim(kipp_cache *cache, kipp_session *session) {
 void kipp_cache_commit(kipp_cache *cache, kipp_session *session, const uint32_t *tokens, size_t count) {
     memcpy(session->tokens + session->length, tokens, count * sizeof(uint32_t));
     session->length += (uint32_t)count;
+    if (session->publish_early && cache->share) {
+        while ((session->published + 1) * cache->page_tokens <= session->length) {
+            const uint32_t *chunk = session->tokens + (size_t)session->published * cache->page_tokens;
+            uint64_t hash = session->chain;
+            for (uint32_t g = 0; g < cache->group_count; ++g)
+                hash = kipp_pool_seal(&cache->groups[g].pool, (uint32_t)session->tables[g][session->published], session->chain, chunk);
+            session->chain = hash;
+            ++session->published;
+        }
+    }
     for (uint32_t g = 0; g < cache->group_count; ++g) {
         kipp_cache_group *group = &cache->groups[g];
         if (group->need.window == 0) continue;
@@ -272,8 +288,8 @@ int kipp_cache_truncate(kipp_cache *cache, kipp_session *session, uint32_t lengt
     for (uint32_t g = 0; g < cache->group_count; ++g) {
         if (cache->groups[g].need.window != 0) return kipp_fail(error, KIPP_ERROR_UNSUPPORTED, "a windowed group cannot be rolled back");
     }
-    if (length < session->adopted_tokens)
-        return kipp_fail(error, KIPP_ERROR_RANGE, "cannot truncate below the %u adopted tokens", session->adopted_tokens);
+    uint32_t floor = session->published * cache->page_tokens > session->adopted_tokens ? session->published * cache->page_tokens : session->adopted_tokens;
+    if (length < floor) return kipp_fail(error, KIPP_ERROR_RANGE, "cannot truncate below the %u adopted or published tokens", floor);
     session->length = length;
     kipp_cache_trim(cache, session);
     return 0;
@@ -301,6 +317,8 @@ void kipp_cache_clear(kipp_cache *cache, kipp_session *session) {
         session->adopted[g] = 0;
     }
     session->length = session->adopted_tokens = 0;
+    session->published = 0;
+    session->chain = 0;
 }
 
 void kipp_cache_close(kipp_cache *cache, kipp_session *session) {

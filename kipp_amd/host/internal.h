@@ -261,6 +261,11 @@ struct kipp_session {
     uint32_t *adopted; /* per group: leading pages taken from the index */
     uint32_t adopted_tokens;
     bool in_step; /* set while a step holds it: a session may appear once in a step */
+    /* a session that will never be truncated below them may publish its full pages as soon as they are written, so that
+     * sessions running beside it can adopt them (a scheduler's requests do) */
+    bool publish_early;
+    uint32_t published; /* leading blocks that are adopted or published */
+    uint64_t chain;     /* chained hash after them */
 };
 
 typedef struct {
@@ -409,8 +414,7 @@ struct kipp_model {
     kipp_session **sessions;
     size_t session_count, session_capacity;
     uint64_t weight_bytes;
-    float *logits_out; /* where the path computes: [max wanted rows][vocab] */
-    size_t logits_rows;
+    int fail_forward_after; /* tests: < 0 never; else the forward pass after that many fails */
 };
 
 int kipp_model_params(const kipp_model_spec *spec, kipp_param_list *out, kipp_error *error);

@@ -185,6 +185,87 @@ typedef struct {
 int kipp_sample_ex(const float *logits, size_t logits_count, const kipp_sample_params *params, uint64_t *rng_state,
                    uint32_t *out_token, kipp_error *error);
 
+/*
+ * The scheduler above the step function: it admits requests, cuts prompts into
+ * portions under a token budget, decodes, finishes and frees (the reference's
+ * server loop lifted out of its HTTP code, /root/reference/src/kipp_server.c:1623-1893
+ * admission, :1900-2125 stepping).  Waiting requests are admitted strictly in
+ * arrival order; pages are reserved at admission, so a running request never
+ * fails for pages and a short pool delays requests, in order; one step is one
+ * call of kipp_step with every decoding request's next token first and portions
+ * of prompts in arrival order behind them; a step that fails fails the requests
+ * that had tokens in it, and the queue moves on.
+ */
+typedef struct kipp_scheduler kipp_scheduler;
+
+typedef struct {
+    uint32_t max_step_tokens; /* token budget of one step; 0: 2048 */
+    uint32_t prefill_chunk;   /* largest portion of a prompt in one step; 0: 512 */
+    uint32_t max_running;     /* requests running at a time; 0: as many as the model has session slots */
+    int keep_last_logits;     /* keep, for every request, the logits row its last token was chosen from (kipp_scheduler_last_logits) */
+} kipp_scheduler_config;
+
+typedef struct {
+    uint64_t id;
+    const uint32_t *prompt;
+    size_t prompt_count;
+    uint32_t max_new_tokens;
+    kipp_sample_params params; /* recent_tokens is ignored: the scheduler keeps the last 64 generated tokens itself */
+    uint64_t seed;             /* of the request's own generator; 0 is taken as 1 */
+    uint32_t stop_tokens[KIPP_MAX_STOP_TOKENS];
+    uint32_t stop_token_count;
+} kipp_request;
+
+typedef enum {
+    KIPP_FINISH_NONE = 0,
+    KIPP_FINISH_LENGTH,    /* max_new_tokens reached */
+    KIPP_FINISH_STOP,      /* a stop token was chosen: neither kept nor fed back */
+    KIPP_FINISH_CANCELLED,
+    KIPP_FINISH_FAILED     /* a step it had tokens in failed */
+} kipp_finish_reason;
+
+typedef struct {
+    uint64_t id;
+    uint32_t token;
+} kipp_produced;
+
+typedef struct {
+    uint64_t id;
+    kipp_finish_reason reason; /* KIPP_FINISH_NONE: still waiting or running */
+    const uint32_t *output;    /* what it has generated so far; valid until the next call on the scheduler */
+    size_t output_count;
+    const char *error;         /* what the failed step said, else "" */
+} kipp_result;
+
+typedef struct {
+    uint64_t requests, refused, finished, failed, failed_steps;
+    uint64_t prompt_tokens, generated_tokens, prefix_tokens_reused, steps, waits_for_pages, waits_for_prefix;
+    /* sums of seconds with their counts, as the reference's server exports them (/root/reference/src/kipp_server.c:71-84) */
+    double queue_wait_seconds_sum;
+    uint64_t queue_wait_count;
+    double ttft_seconds_sum;
+    uint64_t ttft_count;
+    double decode_seconds_sum;
+} kipp_scheduler_stats;
+
+int kipp_scheduler_create(kipp_model *model, const kipp_scheduler_config *config, kipp_scheduler **out_scheduler, kipp_error *error);
+/* Cancels what is waiting or running, then frees. */
+void kipp_scheduler_destroy(kipp_scheduler *scheduler);
+/* Refused (-1) if it can never run: empty prompt, a token outside the vocabulary, prompt + max_new_tokens beyond the
+ * model's positions or the pool, an id that is still known. */
+int kipp_scheduler_add(kipp_scheduler *scheduler, const kipp_request *request, kipp_error *error);
+int kipp_scheduler_cancel(kipp_scheduler *scheduler, uint64_t id, kipp_error *error);
+/* Admit, run one batch, choose tokens.  Writes the (request, token) pairs that became known, at most `capacity`. */
+int kipp_scheduler_step(kipp_scheduler *scheduler, kipp_produced *out, size_t capacity, size_t *out_count, kipp_error *error);
+int kipp_scheduler_idle(const kipp_scheduler *scheduler);
+/* A request by its id, whatever its state; -1 if the id is not known. */
+int kipp_scheduler_result(const kipp_scheduler *scheduler, uint64_t id, kipp_result *out_result);
+/* Forget a finished request (its id may come again). */
+int kipp_scheduler_collect(kipp_scheduler *scheduler, uint64_t id);
+int kipp_scheduler_get_stats(const kipp_scheduler *scheduler, kipp_scheduler_stats *out_stats);
+/* The logits row the last token of request `id` was chosen from (vocab floats), or NULL: for a caller that prints them. */
+const float *kipp_scheduler_last_logits(const kipp_scheduler *scheduler, uint64_t id);
+
 const char *kipp_error_code_name(kipp_error_code code);
 
 /*
@@ -208,6 +289,8 @@ void kipp_test_causal_gqa(const float *query, const float *key, const float *val
 uint64_t kipp_test_chain_hash(uint64_t parent, const uint32_t *tokens, size_t count);
 /* Reverse the block table of a session that holds pages (contents move with it): results must not change. */
 int kipp_test_scramble_session_kv(kipp_session *session, kipp_error *error);
+/* The model's next `skip` forward passes run; the one after them fails with an error of its own.  skip < 0: never. */
+void kipp_test_fail_forward_after(kipp_model *model, int skip);
 /* Pages a session holds in a group, in table order; returns how many were written (at most `capacity`). */
 size_t kipp_test_session_pages(const kipp_session *session, uint32_t group, int32_t *out_pages, size_t capacity);
 

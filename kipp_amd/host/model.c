@@ -141,6 +141,7 @@ int kipp_model_open_ex(const char *model_dir, const kipp_model_open_config *conf
     kipp_model *model = calloc(1, sizeof(*model));
     if (model == NULL) return kipp_fail(error, KIPP_ERROR_MEMORY, "out of memory");
     model->config = *config;
+    model->fail_forward_after = -1;
     if (model->config.page_tokens == 0) model->config.page_tokens = 16;
     if (model->config.max_sessions == 0) model->config.max_sessions = 64;
     if (model->config.max_step_tokens == 0) model->config.max_step_tokens = 2048;
@@ -257,6 +258,8 @@ int kipp_model_get_info(const kipp_model *model, kipp_model_info *out_info) {
     return 0;
 }
 
+void kipp_test_fail_forward_after(kipp_model *model, int skip) { model->fail_forward_after = skip; }
+
 int kipp_model_is_stop_token(const kipp_model *model, uint32_t token) {
     for (uint32_t i = 0; i < model->spec.stop_token_count; ++i) {
         if (model->spec.stop_tokens[i] == token) return 1;
@@ -277,6 +280,7 @@ int kipp_model_forward(kipp_model *model, kipp_batch *batch, float **out_logits,
     const kipp_model_spec *spec = &model->spec;
     const uint32_t n = batch->n_tokens;
     *out_logits = NULL;
+    if (model->fail_forward_after >= 0 && model->fail_forward_after-- == 0) return kipp_fail(error, KIPP_ERROR_INTERNAL, "the forward pass was told to fail (a test's switch)");
     batch->rotation = batch->rotation_of = NULL;
     batch->item_seq = batch->item_tile = NULL;
     batch->n_items = 0;

@@ -3,7 +3,8 @@
  * (the reference builds its own host the same way, /root/reference/Makefile): the JSON reader, checked sizes,
  * the page pool and the cache manager under random orders of sessions, a model folder opened
  * and stepped on the scalar path under several cuttings with scrambled block tables, the error paths
- * of the step function, and the sampler.  The GPU's table is not part of this build.
+ * of the step function, the scheduler over few pages with cancellations and a failed step, and the sampler.
+ * The GPU's table is not part of this build.
  *
  *   host_test MODEL_DIR [MODEL_DIR ...]      exit code 0 and a last line "ok <checks>" on success
  */
@@ -300,6 +301,114 @@ static void test_scalar_operations(void) {
     CHECK(o[0] == 1.0f && o[NQ * D - 1] == 1.0f && o[NQ * D] == 2.0f && o[2 * NQ * D - 1] == 2.0f);
 }
 
+/* The scheduler over few pages: random requests, some sharing a beginning, cancellations and one failed step.  Greedy
+ * output must not depend on the company: each request is run again alone and gives the same tokens. */
+static void test_scheduler(const char *folder) {
+    kipp_model *model = NULL;
+    kipp_error error;
+    kipp_model_open_config config;
+    memset(&config, 0, sizeof(config));
+    config.path = KIPP_PATH_CPU_FP32;
+    config.page_tokens = 4;
+    config.kv_pool_pages = 24;
+    config.max_sessions = 4;
+    config.share_prefixes = 1;
+    if (kipp_model_open_ex(folder, &config, &model, &error) != 0) {
+        CHECK(0);
+        return;
+    }
+    kipp_model_info info;
+    kipp_model_get_info(model, &info);
+    enum { REQUESTS = 14, LONGEST = 40 };
+    static uint32_t prompts[REQUESTS][LONGEST], outputs[REQUESTS][16];
+    size_t lengths[REQUESTS], output_counts[REQUESTS];
+    uint32_t budgets[REQUESTS];
+    kipp_finish_reason reasons[REQUESTS];
+    kipp_scheduler *scheduler = NULL;
+    kipp_scheduler_config sconfig = {11, 6, 0, 1};
+    CHECK(kipp_scheduler_create(model, &sconfig, &scheduler, &error) == 0);
+    kipp_request request;
+    for (int r = 0; r < REQUESTS; ++r) {
+        lengths[r] = 3 + rnd(LONGEST - 3);
+        for (size_t i = 0; i < lengths[r]; ++i) prompts[r][i] = r % 3 == 2 && i < 17 ? prompts[r - 1][i] : rnd(info.vocab_size);
+        if (r % 3 == 2 && lengths[r - 1] < 17) lengths[r] = lengths[r - 1]; /* the copied part must exist */
+        budgets[r] = 1 + rnd(12);
+    }
+    int added = 0, steps = 0;
+    while (added < REQUESTS || !kipp_scheduler_idle(scheduler)) {
+        for (int k = rnd(3); k > 0 && added < REQUESTS; --k, ++added) {
+            memset(&request, 0, sizeof(request));
+            request.id = 100 + added;
+            request.prompt = prompts[added];
+            request.prompt_count = lengths[added];
+            request.max_new_tokens = budgets[added];
+            request.params.repetition_penalty = 1.0f;
+            CHECK(kipp_scheduler_add(scheduler, &request, &error) == 0);
+            CHECK(kipp_scheduler_add(scheduler, &request, &error) != 0); /* the id is known */
+        }
+        if (steps == 9) kipp_test_fail_forward_after(model, 0);
+        if (steps == 5) kipp_scheduler_cancel(scheduler, 100, &error);
+        kipp_produced produced[8];
+        size_t count = 0;
+        CHECK(kipp_scheduler_step(scheduler, produced, 8, &count, &error) == 0 && count <= 4);
+        CHECK(kipp_cache_check(&model->cache, model->sessions, model->session_count, &error) == 0);
+        if (++steps > 2000) {
+            CHECK(0);
+            break;
+        }
+    }
+    kipp_scheduler_stats stats;
+    CHECK(kipp_scheduler_get_stats(scheduler, &stats) == 0 && stats.requests == REQUESTS && stats.failed_steps == 1 && stats.failed >= 1);
+    for (int r = 0; r < REQUESTS; ++r) {
+        kipp_result result;
+        CHECK(kipp_scheduler_result(scheduler, 100 + r, &result) == 0 && result.reason != KIPP_FINISH_NONE);
+        reasons[r] = result.reason;
+        output_counts[r] = result.output_count;
+        CHECK(result.output_count <= budgets[r]);
+        memcpy(outputs[r], result.output, result.output_count * sizeof(uint32_t));
+        if (result.reason == KIPP_FINISH_LENGTH) CHECK(result.output_count == budgets[r] && kipp_scheduler_last_logits(scheduler, 100 + r) != NULL);
+        if (result.reason == KIPP_FINISH_FAILED) CHECK(result.error[0] != '\0');
+        CHECK(kipp_scheduler_collect(scheduler, 100 + r) == 0 && kipp_scheduler_result(scheduler, 100 + r, &result) != 0);
+    }
+    kipp_kv_pool_stats_public pool;
+    kipp_model_kv_pool_stats(model, 0, &pool);
+    CHECK(pool.free_blocks == pool.total_blocks);
+    /* alone, one after the other: the same tokens as far as the first run got */
+    for (int r = 0; r < REQUESTS; ++r) {
+        memset(&request, 0, sizeof(request));
+        request.id = r;
+        request.prompt = prompts[r];
+        request.prompt_count = lengths[r];
+        request.max_new_tokens = budgets[r];
+        request.params.repetition_penalty = 1.0f;
+        CHECK(kipp_scheduler_add(scheduler, &request, &error) == 0);
+        while (!kipp_scheduler_idle(scheduler)) {
+            kipp_produced produced[4];
+            size_t count;
+            CHECK(kipp_scheduler_step(scheduler, produced, 4, &count, &error) == 0);
+        }
+        kipp_result result;
+        CHECK(kipp_scheduler_result(scheduler, r, &result) == 0 && result.reason == KIPP_FINISH_LENGTH && result.output_count >= output_counts[r]);
+        CHECK(memcmp(result.output, outputs[r], output_counts[r] * sizeof(uint32_t)) == 0);
+        if (reasons[r] == KIPP_FINISH_LENGTH) CHECK(result.output_count == output_counts[r]);
+    }
+    /* destroyed with work in hand: what runs is cancelled and its pages come back */
+    memset(&request, 0, sizeof(request));
+    request.id = 999;
+    request.prompt = prompts[0];
+    request.prompt_count = lengths[0];
+    request.max_new_tokens = 5;
+    request.params.repetition_penalty = 1.0f;
+    CHECK(kipp_scheduler_add(scheduler, &request, &error) == 0);
+    kipp_produced one[4];
+    size_t count;
+    CHECK(kipp_scheduler_step(scheduler, one, 4, &count, &error) == 0);
+    kipp_scheduler_destroy(scheduler);
+    kipp_model_kv_pool_stats(model, 0, &pool);
+    CHECK(pool.free_blocks == pool.total_blocks);
+    CHECK(kipp_model_close(model, &error) == 0);
+}
+
 int main(int argc, char **argv) {
     test_json();
     test_sizes();
@@ -307,6 +416,7 @@ int main(int argc, char **argv) {
     test_sampler();
     test_scalar_operations();
     for (int i = 1; i < argc; ++i) test_model(argv[i]);
+    for (int i = 1; i < argc; ++i) test_scheduler(argv[i]);
     if (failures != 0) {
         fprintf(stderr, "%d of %d checks failed\n", failures, checks);
         return 1;

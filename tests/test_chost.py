@@ -421,3 +421,209 @@ def test_command_line_on_the_scalar_path(model_folders, tiny_configs, capsys):
     with pytest.raises(KippError, match="KV pool exhausted"):
         main(common + ["--decode", "20", "--kv-mib", "0.02"])      # 31 tokens need 4 pages
     assert main(["--random", "tiny-a", "--seed-weights", "4", "--path", "cpu-fp32", "--tokens", "1,2,3", "--decode", "2"]) == 0
+
+
+def test_the_c_command_line_matches_the_python_one(model_folders, tiny_configs, capsys, tmp_path):
+    """kipp_cli.c over the C scheduler: the same stdout as `python -m kipp_amd.cli --path cpu-fp32` (tokens and top-N table),
+    one KIPP_METRIC line, a token file, and refusals with exit code 2 or 1 before or after the model is opened."""
+    import subprocess
+    from kipp_amd.cli import main
+    from kipp_amd.host import build
+    exe = build.cli_path()
+    folder = model_folders[("a", "float32")]
+    prompt = H.random_tokens(23, 13, tiny_configs["a"]["vocab_size"])
+    common = ["--model", folder, "--path", "cpu-fp32", "--page", "8", "--decode", "9", "--top", "5", "--prefill-chunk", "5"]
+    for sampling in ([], ["--temperature", "0.9", "--top-k", "12", "--top-p", "0.9", "--seed", "5"]):
+        assert main(common + ["--tokens", ",".join(map(str, prompt))] + sampling) == 0
+        python_out = capsys.readouterr().out
+        proc = subprocess.run([exe] + common + ["--tokens", ",".join(map(str, prompt))] + sampling, capture_output=True, text=True, timeout=60)
+        assert proc.returncode == 0, proc.stderr
+        assert proc.stdout == python_out
+        assert f"KIPP_METRIC backend=cpu-fp32 prefill_tokens={len(prompt)}" in proc.stderr and "decode_tokens=8" in proc.stderr
+    token_file = tmp_path / "prompt.u32"
+    token_file.write_bytes(np.asarray(prompt, "<u4").tobytes())
+    from_file = subprocess.run([exe] + common + ["--tokens-file", str(token_file)], capture_output=True, text=True, timeout=60)
+    greedy = subprocess.run([exe] + common + ["--tokens", ",".join(map(str, prompt))], capture_output=True, text=True, timeout=60)
+    assert from_file.returncode == 0 and greedy.returncode == 0 and from_file.stdout == greedy.stdout
+    for extra, code, words in ((["--tokens", "1,2", "--max-context", "8"], 1, "exceed the context of 8 tokens"),
+                               (["--tokens", "1,x"], 2, "token ids"),
+                               (["--tokens", "1,2", "--path", "metal"], 2, "not built into this engine"),
+                               (["--tokens", "1,2", "--kv-mib", "0.0001"], 1, "holds no page"),
+                               (["--tokens", str(10 ** 6)], 1, "vocabulary"),
+                               (["--tokens", "1,2", "--kv-pages", "1"], 1, "pool")):
+        proc = subprocess.run([exe] + common + extra, capture_output=True, text=True, timeout=60)
+        assert proc.returncode == code and words in proc.stderr, (extra, proc.returncode, proc.stderr)
+    assert subprocess.run([exe, "--help"], capture_output=True, text=True).stdout.startswith("usage: kipp")
+
+
+# ---------------------------------------------------------------------------------------------- the C scheduler
+
+def _greedy(folder, prompt, n, stop=()):
+    """What greedy generation gives by the plain implementation: the argmax at every step (recomputing the whole sequence)."""
+    from tests.plain import qwen3_plain as plain
+    cfg, weights = plain.load_folder(folder)
+    toks, out = list(prompt), []
+    for _ in range(n):
+        t = int(np.argmax(plain.forward_whole(cfg, weights, toks)[-1]))
+        if t in stop:
+            break
+        out.append(t)
+        toks.append(t)
+    return out
+
+
+def test_c_scheduler_portions_decode_first_and_the_budget(model_folders, tiny_configs):
+    """A prompt goes in in portions, its last portion asks for logits, then one token a step; a decoding request's token
+    comes first in a step and portions get what the budget leaves; every generated token is the plain argmax."""
+    from kipp_amd.chost import CScheduler
+    folder, vocab = model_folders[("a", "float32")], tiny_configs["a"]["vocab_size"]
+    a, b = H.random_tokens(1, 11, vocab), H.random_tokens(2, 9, vocab)
+    with _model(model_folders, "a", pages=16) as model:
+        sched = CScheduler(model, max_step_tokens=6, prefill_chunk=4)
+        sched.add(1, a, 5)
+        steps = 0
+        while not sched.idle:
+            produced = sched.step()
+            steps += 1
+            if steps == 3:
+                assert produced and sched.stats["prompt_tokens"] == 11          # portions of 4, 4, 3: the third brings the first token
+                sched.add(2, b, 3)                                               # arrives while request 1 decodes
+            if steps == 4:
+                assert sched.stats["prompt_tokens"] == 11 + 4                    # its first portion, beside request 1's token ...
+                assert [rid for rid, _ in produced] == [1]
+            if steps == 5:
+                assert sched.stats["prompt_tokens"] == 11 + 4 + 4                # ... and so on, 1 + 4 <= 6 a step
+        assert sched.result(1)["output"] == _greedy(folder, a, 5) and sched.result(1)["finish_reason"] == "length"
+        assert sched.result(2)["output"] == _greedy(folder, b, 3)
+        st = sched.stats
+        assert (st["requests"], st["finished"], st["failed"], st["generated_tokens"], st["prompt_tokens"]) == (2, 2, 0, 8, 20)
+        assert st["queue_wait_count"] == 2 and st["ttft_count"] == 2 and st["decode_seconds_sum"] >= 0
+        assert model.pool_stats()["free_blocks"] == 16
+        with pytest.raises(KippError, match="already"):
+            sched.add(1, a, 2)                                                   # finished, its result not collected yet
+        sched.collect(1)
+        sched.add(1, a, 2)
+        sched.run()
+        assert sched.result(1)["output"] == _greedy(folder, a, 2)
+        sched.destroy()
+
+
+def test_c_scheduler_refusals_stop_tokens_and_cancel(model_folders, tiny_configs):
+    from kipp_amd.chost import CScheduler
+    folder, vocab = model_folders[("a", "float32")], tiny_configs["a"]["vocab_size"]
+    prompt = H.random_tokens(3, 7, vocab)
+    free = _greedy(folder, prompt, 6)
+    with _model(model_folders, "a", pages=4) as model:                           # 64 tokens of pages
+        sched = CScheduler(model, max_step_tokens=16, prefill_chunk=8)
+        for bad, match in (((9, [], 2), "empty prompt"), ((9, [vocab], 2), "vocabulary"), ((9, [1] * 100, 40), "positions"),
+                           ((9, [1] * 60, 10), "more than its pool")):
+            with pytest.raises(KippError, match=match):
+                sched.add(*bad)
+        assert sched.stats["refused"] == 4
+        sched.add(1, prompt, 6, stop_tokens=[free[3]])
+        sched.add(2, prompt[:5], 0)                                              # nothing to generate: its prompt runs, then it ends
+        sched.add(3, H.random_tokens(4, 12, vocab), 30)
+        sched.step()
+        sched.cancel(3)
+        sched.run()
+        first = free.index(free[3])
+        assert sched.result(1) == {"id": 1, "finish_reason": "stop", "output": free[:first], "error": ""}   # the stop token is neither kept nor fed back
+        assert sched.result(2)["finish_reason"] == "length" and sched.result(2)["output"] == []
+        assert sched.result(3)["finish_reason"] == "cancelled"
+        with pytest.raises(KippError, match="neither waiting nor running"):
+            sched.cancel(3)
+        assert model.pool_stats()["free_blocks"] == 4
+        sched.destroy()
+
+
+def test_c_scheduler_waits_in_order_when_pages_are_short(model_folders, tiny_configs):
+    """Pressure delays, never corrupts (/root/reference/tests/test_server.py:899): three requests of which two fit the pool at a
+    time; the third waits although a fourth, smaller one behind it would fit (strict arrival order), and every output is what
+    it would be alone."""
+    from kipp_amd.chost import CScheduler
+    folder, vocab = model_folders[("b", "float32")], tiny_configs["b"]["vocab_size"]
+    prompts = {i: H.random_tokens(20 + i, n, vocab) for i, n in ((1, 20), (2, 18), (3, 21), (4, 3))}
+    with _model(model_folders, "b", pages=8, share_prefixes=False) as model:      # pages of 8: a request of 20 + 5 tokens needs 3
+        sched = CScheduler(model, max_step_tokens=32, prefill_chunk=16)
+        for i, p in prompts.items():
+            sched.add(i, p, 5 if i < 4 else 2)
+        sched.step()
+        assert sched.result(3)["finish_reason"] is None and sched.stats["waits_for_pages"] >= 1
+        assert sched.stats["queue_wait_count"] == 2                               # 1 and 2 run; 3 waits, and 4 behind it
+        sched.run()
+        for i, p in prompts.items():
+            assert sched.result(i)["output"] == _greedy(folder, p, 5 if i < 4 else 2)
+        assert model.pool_stats()["free_blocks"] == 8 and sched.stats["finished"] == 4
+        sched.destroy()
+
+
+def test_c_scheduler_requests_that_begin_alike_adopt_pages(model_folders, tiny_configs):
+    """Four requests with a common beginning of five pages arrive together: the later ones wait until the first has
+    published those pages (as soon as each is full) and adopt them; the outputs are still the plain argmax."""
+    from kipp_amd.chost import CScheduler
+    folder, vocab = model_folders[("b", "float32")], tiny_configs["b"]["vocab_size"]
+    common = H.random_tokens(61, 43, vocab)
+    prompts = [common + H.random_tokens(62 + i, n, vocab) for i, n in enumerate([5, 1, 17, 9])]
+    with _model(model_folders, "b", pages=64) as model:
+        sched = CScheduler(model, max_step_tokens=24, prefill_chunk=10)
+        for i, p in enumerate(prompts):
+            sched.add(i, p, 6)
+        sched.run()
+        st = sched.stats
+        assert st["prefix_tokens_reused"] == 3 * 40 and st["prompt_tokens"] == sum(map(len, prompts)) - 120 and st["waits_for_prefix"] > 0
+        for i, p in enumerate(prompts):
+            assert sched.result(i)["output"] == _greedy(folder, p, 6)
+        assert model.pool_stats()["free_blocks"] == 64
+        sched.destroy()
+
+
+def test_c_scheduler_a_failed_step_fails_its_requests_and_the_queue_moves_on(model_folders, tiny_configs):
+    """/root/reference/src/kipp_server.c:2081-2088: the batch fails as a unit.  The third forward pass is told to fail: the two
+    requests that had tokens in it end as failed with the error's text and give everything back; the one that waited is
+    admitted and runs to its end."""
+    from kipp_amd.chost import CScheduler
+    folder, vocab = model_folders[("a", "float32")], tiny_configs["a"]["vocab_size"]
+    prompts = {1: H.random_tokens(31, 30, vocab), 2: H.random_tokens(32, 20, vocab), 3: H.random_tokens(33, 40, vocab)}
+    with _model(model_folders, "a", pages=6, share_prefixes=False) as model:      # 3 + 2 pages run; the third request needs 3
+        sched = CScheduler(model, max_step_tokens=32, prefill_chunk=16)
+        for i, p in prompts.items():
+            sched.add(i, p, 4)
+        model.lib.kipp_test_fail_forward_after(model.handle, 2)
+        sched.run()
+        assert sched.result(1)["finish_reason"] == "failed" and sched.result(2)["finish_reason"] == "failed"
+        assert "told to fail" in sched.result(1)["error"] and sched.result(1)["error"].startswith("internal:")
+        assert sched.result(3) == {"id": 3, "finish_reason": "length", "output": _greedy(folder, prompts[3], 4), "error": ""}
+        st = sched.stats
+        assert (st["failed"], st["failed_steps"], st["finished"]) == (2, 1, 3)
+        assert model.pool_stats()["free_blocks"] == 6
+        sched.destroy()
+
+
+def test_c_scheduler_seeded_sampling_and_penalties(model_folders, tiny_configs):
+    """A temperature request has a generator of its own, seeded by the request; the penalties look back over the tokens it
+    generated: the same tokens as the Python sampler chooses from the plain logits with the same seed."""
+    from kipp_amd.chost import CScheduler
+    from kipp_amd.sampling import SampleParams, XorShift64Star
+    from kipp_amd.sampling import sample as py_sample
+    from tests.plain import qwen3_plain as plain
+    folder, vocab = model_folders[("b", "float32")], tiny_configs["b"]["vocab_size"]
+    prompt = H.random_tokens(9, 12, vocab)
+    with _model(model_folders, "b", pages=16) as model:
+        sched = CScheduler(model, keep_last_logits=True)
+        sched.add(7, prompt, 10, temperature=0.9, top_k=40, top_p=0.95, repetition_penalty=1.3, frequency_penalty=0.2, seed=11)
+        sched.add(8, prompt, 4)                                                  # greedy, beside it
+        sched.run()
+        got = sched.result(7)["output"]
+        assert len(got) == 10 and sched.result(8)["output"] == _greedy(folder, prompt, 4)
+        cfg, weights = plain.load_folder(folder)
+        rng, toks, out = XorShift64Star(11), list(prompt), []
+        params = SampleParams(temperature=0.9, top_k=40, top_p=0.95, repetition_penalty=1.3, frequency_penalty=0.2)
+        for _ in range(10):
+            row = plain.forward_whole(cfg, weights, toks)[-1].astype(np.float32)
+            t = py_sample(row, params, rng, out[-64:])
+            out.append(t)
+            toks.append(t)
+        assert got == out
+        last = sched.last_logits(7)
+        H.assert_close(last[None], plain.forward_whole(cfg, weights, prompt + out[:-1])[-1:], 1e-9, "the logits the last token was chosen from")
+        sched.destroy()
