@@ -120,3 +120,61 @@ def test_c_host_products_of_every_row_class(model_folders, tiny_configs):
                 at = s.length
                 rows.append(model.step([(s, toks[at:at + n], list(range(n)))]))
             H.assert_close(np.concatenate(rows), ref, H.NMSE_BF16["tiny"], f"C host, cuts {cuts}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("key", ["a", "b"])
+def test_c_scheduler_on_the_gpu(model_folders, tiny_configs, key, dtype):
+    """Seven requests through the C scheduler over so few pages that some wait, portions of six tokens beside decoded
+    tokens, two sharing a beginning: every chosen token is the plain implementation's best (within the precision's margin
+    of its row), pages all come back, and the counters add up."""
+    from kipp_amd.chost import CModel, CScheduler
+    cfg = tiny_configs[key]
+    vocab = cfg["vocab_size"]
+    prompts = {i: H.random_tokens(40 + i, n, vocab) for i, n in enumerate([5, 23, 41, 12, 33, 9, 28])}
+    prompts[6] = prompts[2][:2 * PAGE[key] + 3] + prompts[6][:5]
+    budget = {i: 4 + 3 * (i % 4) for i in prompts}
+    margin = 1e-4 if dtype == "float32" else 0.05
+    with CModel(model_folders[(key, dtype)], path=PATH[dtype], page_tokens=PAGE[key], kv_pool_pages=(110 + PAGE[key] - 1) // PAGE[key] + 2,
+                max_sessions=4, share_prefixes=True) as model:
+        sched = CScheduler(model, max_step_tokens=13, prefill_chunk=6)
+        for i, prompt in prompts.items():
+            sched.add(i, prompt, budget[i])
+        sched.run()
+        assert sched.idle
+        for i, prompt in prompts.items():
+            result = sched.result(i)
+            assert result["finish_reason"] == "length" and len(result["output"]) == budget[i]
+            ref = H.plain_logits(model_folders[(key, dtype)], prompt + result["output"])
+            for j, token in enumerate(result["output"]):
+                row = ref[len(prompt) - 1 + j]
+                assert row[token] >= row.max() - margin, (key, dtype, i, j, token, int(row.argmax()))
+        stats = sched.stats
+        assert stats["finished"] == 7 and stats["failed"] == 0 and stats["generated_tokens"] == sum(budget.values())
+        assert stats["prompt_tokens"] + stats["prefix_tokens_reused"] == sum(len(p) for p in prompts.values())
+        assert stats["waits_for_pages"] > 0
+        sched.destroy()
+        pool = model.pool_stats()
+        assert pool["free_blocks"] == pool["total_blocks"]
+
+
+def test_c_command_line_on_the_gpu(model_folders, tiny_configs):
+    """The C program on gpu-bf16 and gpu-fp32, given the folder of the built kernels: greedy tokens that the plain
+    implementation agrees with, and the KIPP_METRIC line naming the path."""
+    import os
+    import subprocess
+    from kipp_amd.csrc import build as kernels
+    from kipp_amd.host import build
+    exe = build.cli_path()
+    prompt = H.random_tokens(77, 19, tiny_configs["b"]["vocab_size"])
+    for dtype, margin in (("float32", 1e-4), ("bfloat16", 0.05)):
+        folder = model_folders[("b", dtype)]
+        proc = subprocess.run([exe, "--model", folder, "--path", PATH[dtype], "--tokens", ",".join(map(str, prompt)), "--decode", "6", "--page", "8",
+                               "--kernels", os.path.join(os.path.dirname(kernels.__file__), "_lib")], capture_output=True, text=True, timeout=120)
+        assert proc.returncode == 0, proc.stderr
+        generated = [int(t) for t in proc.stdout.splitlines()[0].split("\t")[1].split()]
+        assert len(generated) == 6 and f"KIPP_METRIC backend={PATH[dtype]}" in proc.stderr
+        ref = H.plain_logits(folder, prompt + generated)
+        for j, token in enumerate(generated):
+            row = ref[len(prompt) - 1 + j]
+            assert row[token] >= row.max() - margin
