@@ -15,7 +15,7 @@ Errors of the library are raised as `KippError` with the library's code name
 from __future__ import annotations
 
 import ctypes
-from typing import Optional, Sequence, Tuple
+from typing import List, Optional, Sequence, Tuple
 
 import numpy as np
 
@@ -36,7 +36,7 @@ class _Error(ctypes.Structure):
 class _OpenConfig(ctypes.Structure):
     _fields_ = [("path", ctypes.c_int), ("page_tokens", ctypes.c_uint32), ("kv_pool_pages", ctypes.c_uint32),
                 ("max_sessions", ctypes.c_uint32), ("max_step_tokens", ctypes.c_uint32), ("share_prefixes", ctypes.c_int),
-                ("device", ctypes.c_int), ("kernel_dir", ctypes.c_char_p), ("page_order", _u32p)]
+                ("device", ctypes.c_int), ("kernel_dir", ctypes.c_char_p), ("page_order", _u32p), ("eager_steps", ctypes.c_int)]
 
 
 class _ModelInfo(ctypes.Structure):
@@ -146,6 +146,7 @@ def library(variant: str = "gpu") -> ctypes.CDLL:
             "kipp_session_match_prefix": [vp, _u32p, sz, _u32p, err],
             "kipp_eval_batch": [vp, ctypes.POINTER(_BatchItem), sz, err],
             "kipp_step": [vp, ctypes.POINTER(_StepItem), sz, _f32p, sz, err],
+            "kipp_step_argmax": [vp, ctypes.POINTER(_StepItem), sz, _u32p, sz, err],
             "kipp_sample_ex": [_f32p, sz, ctypes.POINTER(_SampleParams), ctypes.POINTER(ctypes.c_uint64), _u32p, err],
             "kipp_test_scramble_session_kv": [vp, err],
             "kipp_scheduler_create": [vp, ctypes.POINTER(_SchedulerConfig), ctypes.POINTER(vp), err],
@@ -165,6 +166,7 @@ def library(variant: str = "gpu") -> ctypes.CDLL:
         lib.kipp_scheduler_last_logits.argtypes, lib.kipp_scheduler_last_logits.restype = [vp, ctypes.c_uint64], _f32p
         lib.kipp_test_fail_forward_after.argtypes, lib.kipp_test_fail_forward_after.restype = [vp, ctypes.c_int], None
         lib.kipp_error_code_name.argtypes, lib.kipp_error_code_name.restype = [ctypes.c_int], ctypes.c_char_p
+        lib.kipp_test_graph_replays.argtypes, lib.kipp_test_graph_replays.restype = [vp], ctypes.c_uint64
         lib.kipp_test_session_pages.argtypes = [vp, u32, ctypes.POINTER(ctypes.c_int32), sz]
         lib.kipp_test_session_pages.restype = sz
         _libs[variant] = lib
@@ -245,7 +247,7 @@ class CSession:
 class CModel:
     def __init__(self, folder: str, path: str = "gpu-bf16", page_tokens: int = 16, kv_pool_pages: int = 0, max_sessions: int = 64,
                  max_step_tokens: int = 4096, share_prefixes: bool = True, device: int = 0, kernel_dir: Optional[str] = None,
-                 page_order: Optional[Sequence[int]] = None, variant: Optional[str] = None):
+                 page_order: Optional[Sequence[int]] = None, variant: Optional[str] = None, eager_steps: bool = False):
         if path not in PATHS:
             raise ValueError(f"path is one of {sorted(PATHS)}")
         self.lib = library(variant or ("host-only" if path == "cpu-fp32" and variant is None else "gpu"))
@@ -260,7 +262,7 @@ class CModel:
             kernel_dir = build._lib_dir()
         order = _u32(page_order) if page_order is not None else (None, None)
         config = _OpenConfig(PATHS[path], page_tokens, kv_pool_pages, max_sessions, max_step_tokens, int(share_prefixes), device,
-                             kernel_dir.encode() if kernel_dir else None, order[1])
+                             kernel_dir.encode() if kernel_dir else None, order[1], int(eager_steps))
         handle, error = ctypes.c_void_p(), _Error()
         if self.lib.kipp_model_open_ex(folder.encode(), ctypes.byref(config), ctypes.byref(handle), ctypes.byref(error)) != 0:
             _raise(self.lib, error)
@@ -270,6 +272,11 @@ class CModel:
         self.lib.kipp_model_get_info(self.handle, ctypes.byref(info))
         self.info = info
         self.vocab_size = info.vocab_size
+
+    @property
+    def graph_replays(self) -> int:
+        """Steps that ran from a recording since the model was opened."""
+        return int(self.lib.kipp_test_graph_replays(self.handle))
 
     def session(self, capacity: int = 0) -> CSession:
         handle, error = ctypes.c_void_p(), _Error()
@@ -295,6 +302,23 @@ class CModel:
         if self.lib.kipp_step(self.handle, items, len(entries), out.ctypes.data_as(_f32p), out.size, ctypes.byref(error)) != 0:
             _raise(self.lib, error)
         return out if wanted else None
+
+    def step_argmax(self, entries: Sequence[Tuple[CSession, Sequence[int], Sequence[int]]]) -> List[int]:
+        """The same batch, answered with the index of the largest logit at every wanted place (found where the path computes)."""
+        items = (_StepItem * len(entries))()
+        keep = []
+        wanted = 0
+        for i, (session, tokens, want) in enumerate(entries):
+            t, tp = _u32(tokens)
+            w, wp = _u32(want)
+            keep.append((t, w))
+            items[i] = _StepItem(session.handle, tp, len(t), wp if len(w) else None, len(w))
+            wanted += len(w)
+        out = np.zeros(max(wanted, 1), dtype=np.uint32)
+        error = _Error()
+        if self.lib.kipp_step_argmax(self.handle, items, len(entries), out.ctypes.data_as(_u32p), wanted, ctypes.byref(error)) != 0:
+            _raise(self.lib, error)
+        return [int(t) for t in out[:wanted]]
 
     def eval_batch(self, entries: Sequence[Tuple[CSession, Sequence[int]]]) -> np.ndarray:
         """kipp.h's batched call: every session's tokens appended, the logits of each one's last token."""

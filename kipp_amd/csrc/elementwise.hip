@@ -133,6 +133,30 @@ __global__ void __launch_bounds__(256) scale_rows_kernel(const bf16_t* __restric
     }
 }
 
+// The streaming layout of a bfloat16 matrix [n, k] (k a multiple of 32) that the few-rows products read:
+// [tile of 16 rows][step of 32 columns][lane][8 values], lane l holding row l % 16 and columns 8 (l / 16) .. + 7
+// of the step, rows padded to whole tiles with zeros.  `inner` > 0: the matrix is [gate; up] of `inner` rows
+// each and tile t holds gate rows 8 t .. 8 t + 7 over up rows 8 t .. 8 t + 7.  A thread moves 16 bytes.
+__global__ void __launch_bounds__(256) tile_weight_kernel(const uint4* __restrict__ rows, uint4* __restrict__ tiles, int n, int k,
+                                                          int inner, size_t units) {
+    const size_t u = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (u >= units) return;
+    const int steps = k / 32, lane = (int)(u & 63), r = lane & 15, h = lane >> 4;
+    const size_t tile = u / ((size_t)steps * 64);
+    const int step = (int)((u >> 6) % (size_t)steps);
+    long long row;
+    if (inner > 0) {
+        const long long i = (long long)tile * 8 + (r & 7);
+        row = i < inner ? (r < 8 ? i : inner + i) : -1;
+    } else {
+        row = (long long)tile * 16 + r;
+        if (row >= n) row = -1;
+    }
+    uint4 v = make_uint4(0u, 0u, 0u, 0u);
+    if (row >= 0) v = rows[((size_t)row * k + 32 * step + 8 * h) / 8];
+    tiles[u] = v;
+}
+
 // x += delta (the last residual add when no norm follows in the same kernel).
 template <typename TD>
 __global__ void residual_add_kernel(float* __restrict__ x, const TD* __restrict__ delta, size_t n, int parts) {
@@ -271,6 +295,17 @@ int kipp_scale_rows(const void* rows, const float* sumsq, void* out, int n_rows,
     if (parts <= 0 || stride < parts) return -1;
     hipLaunchKernelGGL(scale_rows_kernel, dim3(n_rows), dim3(256), 0, stream, (const bf16_t*)rows, sumsq, (bf16_t*)out, width,
                        parts, stride, eps);
+    return KIPP_LAUNCH_CHECK();
+}
+
+// tiles: bfloat16 [ceil(n / 16) 16, k] (`inner` 0) or [ceil(inner / 8) 16, k] (`inner` > 0, n = 2 inner), as above.
+int kipp_tile_weight(const void* rows, void* tiles, int n, int k, int inner, hipStream_t stream) {
+    if (n <= 0 || k <= 0 || (k & 31) || inner < 0 || (inner > 0 && n != 2 * inner)) return -1;
+    const size_t tile_count = inner > 0 ? ((size_t)inner + 7) / 8 : ((size_t)n + 15) / 16;
+    const size_t units = tile_count * (size_t)(k / 32) * 64;
+    if ((units + 255) / 256 > 0x7fffffffu) return -2;
+    hipLaunchKernelGGL(tile_weight_kernel, dim3((unsigned)((units + 255) / 256)), dim3(256), 0, stream, (const uint4*)rows, (uint4*)tiles,
+                       n, k, inner, units);
     return KIPP_LAUNCH_CHECK();
 }
 

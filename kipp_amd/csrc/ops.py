@@ -524,6 +524,21 @@ def tile_weight_pairs(w_gate_up: torch.Tensor) -> torch.Tensor:
     return _tile(torch.cat([gate.view(-1, 8, k), up.view(-1, 8, k)], dim=1).view(-1, k))
 
 
+def tile_weight_device(w: torch.Tensor, gate_up: bool = False) -> torch.Tensor:
+    """`tile_weight(w)` (or `tile_weight_pairs(w)` with `gate_up`) by the kernel that hosts without torch use."""
+    _dev(w)
+    _need(w.dim() == 2 and w.dtype == torch.bfloat16 and w.is_contiguous() and w.shape[1] % 32 == 0,
+          "tile_weight_device: a contiguous bfloat16 matrix, K a multiple of 32")
+    n, k = w.shape
+    _need(not gate_up or n % 2 == 0, "tile_weight_device: gate and up of equal height")
+    inner = n // 2 if gate_up else 0
+    tile_count = (inner + 7) // 8 if gate_up else (n + 15) // 16
+    out = torch.empty(tile_count * 16 * k, dtype=torch.bfloat16, device=w.device)
+    fn = _fn("elementwise", "kipp_tile_weight", [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr])
+    _check(fn(_ptr(w), _ptr(out), n, k, inner, _stream()), "tile_weight_device")
+    return out
+
+
 def pairs_width(inner: int) -> int:
     """Columns of a product from paired tiles: 16 for every 8 outputs."""
     return 16 * ((inner + 7) // 8)

@@ -62,8 +62,10 @@ static float widen(const kipp_tensor *tensor, size_t index) {
     return value;
 }
 
-static int cpu_place_matrix(kipp_runtime *rt, const kipp_tensor *const *pieces, size_t piece_count, kipp_weight *out, kipp_error *error) {
+static int cpu_place_matrix(kipp_runtime *rt, const kipp_tensor *const *pieces, size_t piece_count, kipp_weight_layout layout, kipp_weight *out,
+                            kipp_error *error) {
     (void)rt;
+    (void)layout;
     uint64_t rows = 0, columns = pieces[0]->shape[1];
     for (size_t p = 0; p < piece_count; ++p) rows += pieces[p]->shape[0];
     size_t count;
@@ -76,7 +78,7 @@ static int cpu_place_matrix(kipp_runtime *rt, const kipp_tensor *const *pieces, 
         size_t n = (size_t)(pieces[p]->shape[0] * pieces[p]->shape[1]);
         for (size_t i = 0; i < n; ++i) data[at++] = widen(pieces[p], i);
     }
-    *out = (kipp_weight){data, KIPP_F32, (uint32_t)rows, (uint32_t)columns};
+    *out = (kipp_weight){data, KIPP_F32, (uint32_t)rows, (uint32_t)columns, NULL, false};
     return 0;
 }
 
@@ -110,30 +112,39 @@ static void add_delta(float *x, const kipp_delta *delta, size_t count) {
     }
 }
 
-static int cpu_rmsnorm(kipp_runtime *rt, float *x, const kipp_delta *delta, const float *weight, void *out, uint32_t rows, uint32_t width,
-                       float eps, kipp_error *error) {
-    (void)rt;
-    (void)error;
+static int cpu_rmsnorm(kipp_runtime *rt, float *x, kipp_delta *delta, const float *weight, kipp_rows *out, uint32_t rows, uint32_t width,
+                       float eps, bool may_leave_scale, kipp_error *error) {
+    (void)may_leave_scale; /* this path finishes every row */
+    if (delta != NULL && kipp_settle(rt, delta, error) != 0) return -1;
     if (delta != NULL && delta->parts > 0) add_delta(x, delta, (size_t)rows * width);
-    for (uint32_t r = 0; r < rows; ++r) ref_rms_norm(x + (size_t)r * width, weight, (float *)out + (size_t)r * width, width, eps);
+    for (uint32_t r = 0; r < rows; ++r) ref_rms_norm(x + (size_t)r * width, weight, (float *)out->data + (size_t)r * width, width, eps);
+    out->sumsq = NULL;
     return 0;
 }
 
-static int cpu_residual_add(kipp_runtime *rt, float *x, const kipp_delta *delta, uint32_t rows, uint32_t width, kipp_error *error) {
-    (void)rt;
-    (void)error;
+static int cpu_residual_add(kipp_runtime *rt, float *x, kipp_delta *delta, uint32_t rows, uint32_t width, kipp_error *error) {
+    if (kipp_settle(rt, delta, error) != 0) return -1;
     add_delta(x, delta, (size_t)rows * width);
     return 0;
 }
 
-static int cpu_linear(kipp_runtime *rt, const void *x, const kipp_weight *w, uint32_t m, int max_parts, kipp_delta *out, kipp_error *error) {
+static int cpu_argmax(kipp_runtime *rt, const float *logits, int32_t *out, uint32_t rows, uint32_t vocab, kipp_error *error) {
+    (void)rt;
+    (void)error;
+    for (uint32_t r = 0; r < rows; ++r) out[r] = (int32_t)ref_argmax(logits + (size_t)r * vocab, vocab);
+    return 0;
+}
+
+static int cpu_linear(kipp_runtime *rt, const kipp_rows *rows_in, const kipp_weight *w, uint32_t m, int max_parts, kipp_delta *out, kipp_error *error) {
     (void)max_parts;
+    if (rows_in->sumsq != NULL) return kipp_fail(error, KIPP_ERROR_INTERNAL, "rows without their scale on the host path");
+    const void *x = rows_in->data;
     size_t count;
     if (kipp_mul_size(m, w->n, &count) != 0 || count > SIZE_MAX / 4) return kipp_fail(error, KIPP_ERROR_RANGE, "a product's size overflows");
     float *y = kipp_scratch(rt, count * sizeof(float), error);
     if (y == NULL) return -1;
     for (uint32_t r = 0; r < m; ++r) ref_matvec(w->data, REF_F32, (const float *)x + (size_t)r * w->k, y + (size_t)r * w->n, w->n, w->k);
-    *out = (kipp_delta){y, 1};
+    *out = (kipp_delta){y, 1, NULL, NULL, 0, 0};
     return 0;
 }
 
@@ -233,5 +244,6 @@ kipp_runtime *kipp_runtime_cpu(kipp_error *error) {
     rt->qk_norm_rope_kv = cpu_qk_norm_rope_kv;
     rt->attention = cpu_attention;
     rt->gather_rows = cpu_gather_rows;
+    rt->argmax = cpu_argmax;
     return rt;
 }

@@ -51,6 +51,15 @@ typedef int (*fn_gemm_skinny)(const void *, const void *, float *, int, int, int
                               void *, float *, hipStream_t);
 typedef int (*fn_rows_parts)(int, int, int, int);
 typedef int (*fn_gemm_rows)(const void *, const void *, float *, int, int, int, int, int, hipStream_t);
+typedef int (*fn_skinny_swiglu)(const void *, const void *, void *, int, int, int, int, const float *, int, float, hipStream_t);
+typedef int (*fn_int_int)(int);
+typedef int (*fn_scale_rows)(const void *, const float *, void *, int, int, int, int, float, hipStream_t);
+typedef int (*fn_tile_weight)(const void *, void *, int, int, int, hipStream_t);
+typedef int (*fn_argmax)(const float *, int32_t *, int, int, float *, hipStream_t);
+typedef int (*fn_attention_decode_fused)(const float *, int, int, const float *, const float *, float, const float *, const float *, int, void *,
+                                         void *, void *, float *, float *, const int32_t *, const int32_t *, const int32_t *, const int32_t *, int,
+                                         int, int, int, int, int, float, int, int, int, int32_t *, hipStream_t);
+typedef int (*fn_ring_takes)(int, int, int, int);
 typedef int (*fn_tiles_parts)(int, int, int, int, int);
 typedef int (*fn_gemm_tiles)(const void *, const void *, void *, int, int, int, int, int, int, hipStream_t);
 
@@ -59,14 +68,16 @@ typedef struct {
     void *prefill_lib, *decode_lib;
     fn_attention_prefill prefill;
     fn_attention_decode decode;
-    int prefill_rows, split, split_min;
+    fn_attention_decode_fused decode_fused;
+    fn_ring_takes ring_takes;
+    int prefill_rows, split, split_min, fused_ok, fused_slabs;
 } attention_variant;
 
 typedef struct {
     int device;
     hipStream_t stream;
     char kernel_dir[3072];
-    void *libs[8];
+    void *libs[12];
     size_t lib_count;
     fn_embed embed;
     fn_rmsnorm rmsnorm;
@@ -85,6 +96,16 @@ typedef struct {
     fn_gemm_rows gemm_rows;
     fn_tiles_parts tiles_parts;
     fn_gemm_tiles gemm_tiles;
+    fn_skinny_swiglu gemm_skinny_swiglu;
+    fn_int_int skinny_sumsq_stride;
+    fn_scale_rows scale_rows;
+    fn_tile_weight tile_weight;
+    fn_argmax argmax;
+    fn_int_int argmax_scratch_floats;
+    bool fuse;             /* few rows: residual add and norm ride on the products around them, decode attention starts from the QKV product */
+    bool merge_in_kernel;  /* decode attention: the splits of a head are merged by the last of their workgroups to finish */
+    int32_t *arrivals;     /* its counts of finished splits, zero between launches */
+    size_t arrivals_count;
     attention_variant variants[8];
     size_t variant_count;
     uint64_t generic_attention_launches; /* bfloat16 attention that fell to the generic kernel */
@@ -161,9 +182,9 @@ static void *symbol(void *lib, const char *name, kipp_error *error) {
     } while (0)
 
 static int open_common(hip_state *st, kipp_error *error) {
-    static const char *const names[] = {"elementwise", "rope_kv", "attention_generic", "gemm_f32", "gemm_skinny", "gemm_rows", "gemm_tiles"};
-    void *libs[7];
-    for (size_t i = 0; i < 7; ++i) {
+    static const char *const names[] = {"elementwise", "rope_kv", "attention_generic", "gemm_f32", "gemm_skinny", "gemm_rows", "gemm_tiles", "sampling"};
+    void *libs[8];
+    for (size_t i = 0; i < 8; ++i) {
         libs[i] = open_library(st, names[i], error);
         if (libs[i] == NULL) return -1;
         st->libs[st->lib_count++] = libs[i];
@@ -185,6 +206,12 @@ static int open_common(hip_state *st, kipp_error *error) {
     KIPP_SYM(libs[5], gemm_rows, "kipp_gemm_rows");
     KIPP_SYM(libs[6], tiles_parts, "kipp_gemm_tiles_parts");
     KIPP_SYM(libs[6], gemm_tiles, "kipp_gemm_tiles");
+    KIPP_SYM(libs[0], scale_rows, "kipp_scale_rows");
+    KIPP_SYM(libs[0], tile_weight, "kipp_tile_weight");
+    KIPP_SYM(libs[4], gemm_skinny_swiglu, "kipp_gemm_skinny_swiglu");
+    KIPP_SYM(libs[4], skinny_sumsq_stride, "kipp_gemm_skinny_sumsq_stride");
+    KIPP_SYM(libs[7], argmax, "kipp_argmax");
+    KIPP_SYM(libs[7], argmax_scratch_floats, "kipp_argmax_scratch_floats");
     return 0;
 }
 
@@ -207,14 +234,22 @@ static attention_variant *variant_of(hip_state *st, uint32_t head_dim, uint32_t 
     if ((v->decode_lib = open_library(st, key, error)) == NULL) return NULL;
     *(void **)(&v->prefill) = symbol(v->prefill_lib, "kipp_attention_prefill", error);
     *(void **)(&v->decode) = symbol(v->decode_lib, "kipp_attention_decode", error);
-    fn_int_void rows = NULL, split = NULL, split_min = NULL;
+    *(void **)(&v->decode_fused) = symbol(v->decode_lib, "kipp_attention_decode_fused", error);
+    *(void **)(&v->ring_takes) = symbol(v->decode_lib, "kipp_attention_decode_ring_takes", error);
+    fn_int_void rows = NULL, split = NULL, split_min = NULL, fused_ok = NULL, fused_slabs = NULL;
     *(void **)(&rows) = symbol(v->prefill_lib, "kipp_attention_prefill_rows", error);
     *(void **)(&split) = symbol(v->decode_lib, "kipp_attention_decode_split", error);
     *(void **)(&split_min) = symbol(v->decode_lib, "kipp_attention_decode_split_min", error);
-    if (v->prefill == NULL || v->decode == NULL || rows == NULL || split == NULL || split_min == NULL) return NULL;
+    *(void **)(&fused_ok) = symbol(v->decode_lib, "kipp_attention_decode_fused_ok", error);
+    *(void **)(&fused_slabs) = symbol(v->decode_lib, "kipp_attention_decode_fused_slabs", error);
+    if (v->prefill == NULL || v->decode == NULL || v->decode_fused == NULL || v->ring_takes == NULL || rows == NULL || split == NULL ||
+        split_min == NULL || fused_ok == NULL || fused_slabs == NULL)
+        return NULL;
     v->prefill_rows = rows();
     v->split = split();
     v->split_min = split_min();
+    v->fused_ok = fused_ok();
+    v->fused_slabs = fused_slabs();
     ++st->variant_count;
     return v;
 }
@@ -224,6 +259,7 @@ static void hip_destroy(kipp_runtime *rt) {
     hip_state *st = rt->state;
     if (st != NULL) {
         hipStreamSynchronize(st->stream);
+        if (st->arrivals != NULL) hipFree(st->arrivals);
         if (st->stream != NULL) hipStreamDestroy(st->stream);
         /* the libraries stay loaded: their kernels may be registered with the HIP runtime until the process ends */
         free(st);
@@ -282,6 +318,8 @@ static int hip_copy(kipp_runtime *rt, void *to, const void *from, size_t bytes, 
     return code == hipSuccess ? 0 : hip_bad(error, code, "copy on the GPU");
 }
 
+static int refused(kipp_error *error, const char *what, int code);
+
 /* ------------------------------------------------------------------ placement */
 static float half_to_float(uint16_t bits) {
     uint32_t sign = (uint32_t)(bits & 0x8000u) << 16, exponent = (bits >> 10) & 0x1f, fraction = bits & 0x3ffu, wide;
@@ -324,7 +362,9 @@ static float *widened(const kipp_tensor *tensor, size_t count, kipp_error *error
     return wide;
 }
 
-static int hip_place_matrix(kipp_runtime *rt, const kipp_tensor *const *pieces, size_t piece_count, kipp_weight *out, kipp_error *error) {
+static int hip_place_matrix(kipp_runtime *rt, const kipp_tensor *const *pieces, size_t piece_count, kipp_weight_layout layout, kipp_weight *out,
+                            kipp_error *error) {
+    hip_state *st = rt->state;
     uint64_t rows = 0, columns = pieces[0]->shape[1];
     bool keep_bf16 = rt->act_dtype == KIPP_BF16;
     for (size_t p = 0; p < piece_count; ++p) {
@@ -355,7 +395,29 @@ static int hip_place_matrix(kipp_runtime *rt, const kipp_tensor *const *pieces, 
         }
         at += n * (keep_bf16 ? 2 : 4);
     }
-    *out = (kipp_weight){data, keep_bf16 ? KIPP_BF16 : KIPP_F32, (uint32_t)rows, (uint32_t)columns};
+    *out = (kipp_weight){data, keep_bf16 ? KIPP_BF16 : KIPP_F32, (uint32_t)rows, (uint32_t)columns, NULL, false};
+    /* Decode reads every weight once a step and is bound by that read, which is a fifth faster from the streaming layout;
+     * products of many rows read the rows.  The price is the matrix held twice. */
+    bool pairs = layout == KIPP_LAYOUT_STREAM_PAIRS && piece_count == 2 && pieces[0]->shape[0] == pieces[1]->shape[0];
+    if (keep_bf16 && layout != KIPP_LAYOUT_ROWS && columns % 32 == 0 && columns > 0 && rows > 0) {
+        size_t inner = pairs ? (size_t)(rows / 2) : 0, tile_count = pairs ? (inner + 7) / 8 : ((size_t)rows + 15) / 16, tile_bytes;
+        if (kipp_mul_size(tile_count * 32, (size_t)columns, &tile_bytes) != 0) {
+            hip_free(rt, data);
+            return kipp_fail(error, KIPP_ERROR_RANGE, "a matrix of %llu x %llu is too large", (unsigned long long)rows, (unsigned long long)columns);
+        }
+        void *tiles = hip_alloc(rt, tile_bytes, error);
+        int rc = tiles == NULL ? -1 : st->tile_weight(data, tiles, (int)rows, (int)columns, (int)inner, st->stream);
+        if (rc != 0) {
+            if (tiles != NULL) {
+                hip_free(rt, tiles);
+                refused(error, "tile_weight", rc);
+            }
+            hip_free(rt, data);
+            return -1;
+        }
+        out->tiles = tiles;
+        out->pairs = pairs;
+    }
     return 0;
 }
 
@@ -377,7 +439,8 @@ static int hip_place_vector(kipp_runtime *rt, const kipp_tensor *tensor, float *
 
 static void hip_free_weight(kipp_runtime *rt, kipp_weight *weight) {
     if (weight->data != NULL) hip_free(rt, weight->data);
-    weight->data = NULL;
+    if (weight->tiles != NULL) hip_free(rt, weight->tiles);
+    weight->data = weight->tiles = NULL;
 }
 
 /* ------------------------------------------------------------------ operations */
@@ -391,64 +454,124 @@ static int hip_embed(kipp_runtime *rt, const kipp_weight *table, const int32_t *
     return rc == 0 ? 0 : refused(error, "embed", rc);
 }
 
-static int hip_rmsnorm(kipp_runtime *rt, float *x, const kipp_delta *delta, const float *weight, void *out, uint32_t rows, uint32_t width,
-                       float eps, kipp_error *error) {
+#define FEW_ROWS 8            /* up to these the kernel in which every wave reads its rows of x itself is the faster one, and has the fused ends */
+#define STAGED_ROWS 192       /* up to these the kernel that stages x through LDS; beyond, the one built for hundreds of rows where it takes the shape */
+#define FUSE_NORM_X_BYTES 40e6 /* most bytes of x the workgroups of an unsplit product may read together for the fused norm to pay */
+
+/* The few-rows kernel takes this product (and with it the ends that spare a decode step its norm kernels). */
+static bool few_rows(const kipp_runtime *rt, const kipp_weight *w, uint32_t m) {
+    return rt->act_dtype == KIPP_BF16 && w->dtype == KIPP_BF16 && m <= FEW_ROWS && w->k % 8 == 0 && w->k >= 32;
+}
+
+static bool hip_defers(kipp_runtime *rt, const kipp_rows *x, const kipp_weight *w, uint32_t m) {
+    const hip_state *st = rt->state;
+    return st->fuse && x->sumsq == NULL && few_rows(rt, w, m) && !w->pairs;
+}
+
+static int hip_scale_rows(kipp_runtime *rt, const kipp_rows *in, void *out, uint32_t rows, uint32_t width, kipp_error *error) {
     hip_state *st = rt->state;
-    int rc = st->rmsnorm(x, delta != NULL ? delta->data : NULL, KIPP_F32, delta != NULL ? delta->parts : 1, weight, out, rt->act_dtype, (int)rows,
-                         (int)width, eps, st->stream);
+    int rc = st->scale_rows(in->data, in->sumsq, out, (int)rows, (int)width, in->sumsq_parts, (in->sumsq_parts + 3) / 4 * 4, in->eps, st->stream);
+    return rc == 0 ? 0 : refused(error, "scale_rows", rc);
+}
+
+static int hip_rmsnorm(kipp_runtime *rt, float *x, kipp_delta *delta, const float *weight, kipp_rows *out, uint32_t rows, uint32_t width,
+                       float eps, bool may_leave_scale, kipp_error *error) {
+    hip_state *st = rt->state;
+    out->sumsq = NULL;
+    if (delta != NULL && delta->parts == 0 && delta->w != NULL) {
+        /* A product that has not been launched: its kernel adds it to x and prepares the norm of the new x.  That kernel is
+         * not split over workgroups; where the product alone would be, each of its N / 16 workgroups reads all of its
+         * operand instead of a part, which costs more than the norm's kernel once that is some tens of megabytes. */
+        const kipp_weight *w = delta->w;
+        const int N = (int)w->n, K = (int)w->k, most = delta->max_parts > 8 ? 8 : (delta->max_parts < 1 ? 1 : delta->max_parts);
+        bool fused = st->fuse && few_rows(rt, w, delta->m) && !w->pairs && delta->m == rows && w->n == width &&
+                     !(st->skinny_parts(N, K, most) > 1 && (double)((N + 15) / 16) * rows * K * 2 > FUSE_NORM_X_BYTES);
+        if (fused) {
+            const int stride = st->skinny_sumsq_stride(N);
+            float *sumsq = kipp_scratch(rt, (size_t)rows * (size_t)stride * sizeof(float), error);
+            void *unscaled = may_leave_scale ? out->data : kipp_scratch(rt, (size_t)rows * width * 2, error);
+            if (sumsq == NULL || unscaled == NULL) return -1;
+            const bool tiled = w->tiles != NULL;
+            int rc = st->gemm_skinny(delta->x, tiled ? w->tiles : w->data, NULL, (int)rows, N, K, 1, tiled ? 1 : 0, NULL, 0, 0.0f, x, weight, unscaled,
+                                     sumsq, st->stream);
+            if (rc != 0) return refused(error, "gemm_skinny (with the residual's end)", rc);
+            *delta = (kipp_delta){NULL, 0, NULL, NULL, 0, 0};
+            const kipp_rows left = {unscaled, sumsq, (N + 15) / 16, eps};
+            if (may_leave_scale) {
+                *out = left;
+                return 0;
+            }
+            return hip_scale_rows(rt, &left, out->data, rows, width, error);
+        }
+        if (kipp_settle(rt, delta, error) != 0) return -1;
+    }
+    const bool any = delta != NULL && delta->parts > 0;
+    int rc = st->rmsnorm(x, any ? delta->data : NULL, KIPP_F32, any ? delta->parts : 1, weight, out->data, rt->act_dtype, (int)rows, (int)width, eps,
+                         st->stream);
     return rc == 0 ? 0 : refused(error, "rmsnorm", rc);
 }
 
-static int hip_residual_add(kipp_runtime *rt, float *x, const kipp_delta *delta, uint32_t rows, uint32_t width, kipp_error *error) {
+static int hip_residual_add(kipp_runtime *rt, float *x, kipp_delta *delta, uint32_t rows, uint32_t width, kipp_error *error) {
     hip_state *st = rt->state;
+    if (kipp_settle(rt, delta, error) != 0) return -1;
     int rc = st->residual_add(x, delta->data, KIPP_F32, delta->parts, (size_t)rows * width, st->stream);
     return rc == 0 ? 0 : refused(error, "residual_add", rc);
 }
 
-/* x . w^T.  bfloat16 x bfloat16: up to 8 rows the kernel in which every wave streams its rows of w against all of x, up to
- * 256 rows the one that stages x through LDS, beyond those the tiled matrix-core kernel (K a multiple of 32) or the staged
- * one over runs of 256 rows; a shape none of them takes (K no multiple of 8, or below 32) and every float32 weight go
- * through the plain float32 product. */
-static int hip_linear(kipp_runtime *rt, const void *x, const kipp_weight *w, uint32_t m, int max_parts, kipp_delta *out, kipp_error *error) {
+/* x . w^T.  bfloat16 x bfloat16: up to 8 rows the kernel in which every wave streams its rows of w against all of x (it also
+ * applies a scale that the rows still lack), up to 192 rows the one that stages x through LDS, both from the streaming layout
+ * where the weight has it; beyond those the tiled matrix-core kernel (K a multiple of 32) or the staged one over runs of 256
+ * rows; a shape none of them takes (K no multiple of 8, or below 32) and every float32 weight go through the plain float32
+ * product. */
+static int hip_linear(kipp_runtime *rt, const kipp_rows *rows_in, const kipp_weight *w, uint32_t m, int max_parts, kipp_delta *out, kipp_error *error) {
     hip_state *st = rt->state;
     const int M = (int)m, N = (int)w->n, K = (int)w->k;
     size_t count;
     if (kipp_mul_size(m, w->n, &count) != 0 || count > SIZE_MAX / 64) return kipp_fail(error, KIPP_ERROR_RANGE, "a product's size overflows");
     if (max_parts < 1) max_parts = 1;
+    kipp_rows finished = *rows_in;
+    if (finished.sumsq != NULL && !few_rows(rt, w, m) && kipp_finish_rows(rt, &finished, m, w->k, error) != 0) return -1;
+    const void *x = finished.data;
+    /* paired tiles give the columns in another order: only the product that ends in the activation reads them */
+    const bool tiled = w->tiles != NULL && !w->pairs;
+    const void *streamed = tiled ? w->tiles : w->data;
     int rc;
+#define KIPP_DELTA(y, parts) ((kipp_delta){(y), (parts), NULL, NULL, 0, 0})
     if (w->dtype == KIPP_BF16 && rt->act_dtype == KIPP_BF16 && K % 8 == 0 && K >= 32) {
-        if (M <= 8) {
+        if (M <= FEW_ROWS) {
             int most = max_parts > 8 ? 8 : max_parts, parts = st->skinny_parts(N, K, most);
             float *y = parts >= 1 ? kipp_scratch(rt, (size_t)parts * count * 4, error) : NULL;
             if (y == NULL) return parts >= 1 ? -1 : refused(error, "gemm_skinny (its cut)", parts);
-            rc = st->gemm_skinny(x, w->data, y, M, N, K, most, 0, NULL, 0, 0.0f, NULL, NULL, NULL, NULL, st->stream);
-            *out = (kipp_delta){y, parts};
+            rc = st->gemm_skinny(x, streamed, y, M, N, K, most, tiled ? 1 : 0, finished.sumsq, finished.sumsq_parts, finished.eps, NULL, NULL, NULL,
+                                 NULL, st->stream);
+            *out = KIPP_DELTA(y, parts);
             return rc == 0 ? 0 : refused(error, "gemm_skinny", rc);
         }
-        if (M <= 256) {
+        const bool tiles_take = K % 32 == 0 && (uint64_t)(M > N ? M : N) * (uint64_t)K * 2 < ((uint64_t)1 << 32);
+        if (M <= STAGED_ROWS || (M <= 256 && !tiles_take)) {
             int most = max_parts > 12 ? 12 : max_parts, parts = st->rows_parts(M, N, K, most);
             float *y = parts >= 1 ? kipp_scratch(rt, (size_t)parts * count * 4, error) : NULL;
             if (y == NULL) return parts >= 1 ? -1 : refused(error, "gemm_rows (its cut)", parts);
-            rc = st->gemm_rows(x, w->data, y, M, N, K, most, 0, st->stream);
-            *out = (kipp_delta){y, parts};
+            rc = st->gemm_rows(x, streamed, y, M, N, K, most, tiled ? 1 : 0, st->stream);
+            *out = KIPP_DELTA(y, parts);
             return rc == 0 ? 0 : refused(error, "gemm_rows", rc);
         }
-        if (K % 32 == 0 && (uint64_t)(M > N ? M : N) * (uint64_t)K * 2 < ((uint64_t)1 << 32)) {
+        if (tiles_take) {
             int most = max_parts > 4 ? 4 : max_parts, parts = st->tiles_parts(M, N, K, 0, most);
             float *y = parts >= 1 ? kipp_scratch(rt, (size_t)parts * count * 4, error) : NULL;
             if (y == NULL) return parts >= 1 ? -1 : refused(error, "gemm_tiles (its cut)", parts);
             rc = st->gemm_tiles(x, w->data, y, M, N, K, 0, most, 0, st->stream);
-            *out = (kipp_delta){y, parts};
+            *out = KIPP_DELTA(y, parts);
             return rc == 0 ? 0 : refused(error, "gemm_tiles", rc);
         }
         float *y = kipp_scratch(rt, count * 4, error);
         if (y == NULL) return -1;
         for (int row = 0; row < M; row += 256) {
             int rows = M - row < 256 ? M - row : 256;
-            rc = st->gemm_rows((const char *)x + (size_t)row * K * 2, w->data, y + (size_t)row * N, rows, N, K, 1, 0, st->stream);
+            rc = st->gemm_rows((const char *)x + (size_t)row * K * 2, streamed, y + (size_t)row * N, rows, N, K, 1, tiled ? 1 : 0, st->stream);
             if (rc != 0) return refused(error, "gemm_rows", rc);
         }
-        *out = (kipp_delta){y, 1};
+        *out = KIPP_DELTA(y, 1);
         return 0;
     }
     const float *wide = x;
@@ -462,8 +585,29 @@ static int hip_linear(kipp_runtime *rt, const void *x, const kipp_weight *w, uin
     float *y = kipp_scratch(rt, count * 4, error);
     if (y == NULL) return -1;
     rc = st->gemm_f32(wide, w->data, w->dtype, y, M, N, K, st->stream);
-    *out = (kipp_delta){y, 1};
+    *out = KIPP_DELTA(y, 1);
     return rc == 0 ? 0 : refused(error, "gemm_f32", rc);
+}
+
+/* Few rows against [gate; up]: both products and the activation in one kernel (and the norm's scale, if it was left to us). */
+static int hip_gated(kipp_runtime *rt, const kipp_rows *x, const kipp_weight *w, void *act, uint32_t m, bool *done, kipp_error *error) {
+    hip_state *st = rt->state;
+    *done = false;
+    if (!few_rows(rt, w, m) || w->n % 2 != 0 || (w->tiles != NULL && !w->pairs)) return 0;
+    const bool tiled = w->tiles != NULL;
+    int rc = st->gemm_skinny_swiglu(x->data, tiled ? w->tiles : w->data, act, (int)m, (int)w->n, (int)w->k, tiled ? 1 : 0, x->sumsq, x->sumsq_parts,
+                                    x->eps, st->stream);
+    if (rc != 0) return refused(error, "gemm_skinny_swiglu", rc);
+    *done = true;
+    return 0;
+}
+
+static int hip_argmax(kipp_runtime *rt, const float *logits, int32_t *out, uint32_t rows, uint32_t vocab, kipp_error *error) {
+    hip_state *st = rt->state;
+    float *scratch = kipp_scratch(rt, (size_t)st->argmax_scratch_floats((int)rows) * sizeof(float), error);
+    if (scratch == NULL) return -1;
+    int rc = st->argmax(logits, out, (int)rows, (int)vocab, scratch, st->stream);
+    return rc == 0 ? 0 : refused(error, "argmax", rc);
 }
 
 static int hip_swiglu(kipp_runtime *rt, const kipp_delta *gate_up, void *out, uint32_t rows, uint32_t inner, kipp_error *error) {
@@ -541,14 +685,96 @@ static int prefill_work(kipp_runtime *rt, kipp_batch *batch, int tile_rows, kipp
     return 0;
 }
 
+/* Counts of finished splits for `count` (token, key/value head) pairs: zero between launches (the workgroup that merges sets
+ * its count back), kept from step to step, zeroed again after a step that failed.  NULL: the merge is a launch of its own. */
+static int arrivals_for(kipp_runtime *rt, size_t count, int32_t **out, kipp_error *error) {
+    hip_state *st = rt->state;
+    *out = NULL;
+    if (!st->merge_in_kernel) return 0;
+    if (st->arrivals_count < count) {
+        if (rt->recording) return kipp_fail(error, KIPP_ERROR_MEMORY, "the counts of finished splits would grow while a step is recorded");
+        size_t grown = count < 65536 ? 65536 : count;
+        ++rt->generation; /* recordings hold the old address */
+        hipStreamSynchronize(st->stream);
+        if (st->arrivals != NULL) hipFree(st->arrivals);
+        st->arrivals = NULL;
+        st->arrivals_count = 0;
+        hipError_t code = hipMalloc((void **)&st->arrivals, grown * sizeof(int32_t));
+        if (code != hipSuccess) return hip_bad(error, code, "hipMalloc");
+        int rc = st->fill_zero(st->arrivals, grown, st->stream);
+        if (rc != 0) return refused(error, "fill_zero", rc);
+        st->arrivals_count = grown;
+    }
+    *out = st->arrivals;
+    return 0;
+}
+
+/* Partial results of the splits, shared by the layers of one geometry within the step. */
+static int decode_workspace(kipp_runtime *rt, kipp_batch *batch, const attention_variant *v, const kipp_attention_geometry *g, size_t *max_splits,
+                            int *grid, kipp_error *error) {
+    *max_splits = (batch->max_decode_ctx + (size_t)v->split_min - 1) / (size_t)v->split_min + 1;
+    const size_t key = ((size_t)g->n_q << 32) ^ ((size_t)g->head_dim << 16) ^ *max_splits;
+    if (batch->decode_workspace[0] == NULL || batch->decode_workspace_key != key) {
+        size_t rows = (size_t)batch->n_decode * g->n_q * *max_splits;
+        batch->decode_workspace[0] = kipp_scratch(rt, rows * g->head_dim * sizeof(float), error);
+        batch->decode_workspace[1] = kipp_scratch(rt, rows * 2 * sizeof(float), error);
+        if (batch->decode_workspace[0] == NULL || batch->decode_workspace[1] == NULL) return -1;
+        batch->decode_workspace_key = key;
+    }
+    uint32_t span = g->window != 0 && g->window < batch->max_decode_ctx ? g->window : batch->max_decode_ctx;
+    size_t need = (span + (size_t)v->split - 1) / (size_t)v->split + (g->window != 0 ? 1 : 0);
+    *grid = (int)(need < 1 ? 1 : (need > *max_splits ? *max_splits : need));
+    return 0;
+}
+
+static bool attention_fast(const kipp_runtime *rt, const kipp_attention_geometry *g, const kipp_cache_view *cache, const kipp_batch *batch) {
+    const uint32_t group = g->n_q / g->n_kv, page = cache->page_tokens;
+    return rt->act_dtype == KIPP_BF16 && g->head_dim % 16 == 0 && group <= 16 && (page & (page - 1)) == 0 && batch->max_blocks <= PREFILL_MAX_BLOCKS;
+}
+
+#define FUSED_DECODE_ROWS 16   /* up to this many single tokens take the decode attention that starts from the QKV product ... */
+#define FUSED_DECODE_KEYS 8192 /* ... while their contexts are shorter than this (beyond, every split's workgroup would prepare the queries again) */
+
+/* Single tokens only: the QKV product in at most four slabs, then norm, rotation, cache write and attention in one kernel,
+ * for a few tokens and wherever the kernel that walks whole contexts or long ranges runs. */
+static int hip_decode_attention(kipp_runtime *rt, const kipp_rows *x, const kipp_weight *w_qkv, const kipp_cache_view *cache, void *out,
+                                kipp_batch *batch, const kipp_attention_geometry *g, const float *q_norm_w, const float *k_norm_w, float eps,
+                                const float *rotation, uint32_t rotary_dim, int interleaved, bool *done, kipp_error *error) {
+    hip_state *st = rt->state;
+    *done = false;
+    const uint32_t n = batch->n_tokens;
+    if (!st->fuse || !attention_fast(rt, g, cache, batch) || batch->n_portions != 0 || batch->n_decode != n || interleaved) return 0;
+    if (g->head_dim % 128 != 0 || g->head_dim > 256 || (rotation != NULL && rotary_dim != g->head_dim)) return 0;
+    attention_variant *v = variant_of(st, g->head_dim, g->n_q / g->n_kv, error);
+    if (v == NULL) return -1;
+    if (!v->fused_ok) return 0;
+    size_t max_splits;
+    int grid;
+    uint32_t span = g->window != 0 && g->window < batch->max_decode_ctx ? g->window : batch->max_decode_ctx;
+    int splits = (int)((span + (size_t)v->split - 1) / (size_t)v->split) + (g->window != 0 ? 1 : 0);
+    if (!((n <= FUSED_DECODE_ROWS && batch->max_decode_ctx < FUSED_DECODE_KEYS) ||
+          v->ring_takes((int)n, (int)g->n_kv, (int)cache->page_tokens, splits < 1 ? 1 : splits)))
+        return 0;
+    kipp_delta qkv;
+    if (hip_linear(rt, x, w_qkv, n, v->fused_slabs, &qkv, error) != 0) return -1;
+    int32_t *arrivals;
+    if (decode_workspace(rt, batch, v, g, &max_splits, &grid, error) != 0 || arrivals_for(rt, (size_t)n * g->n_q, &arrivals, error) != 0) return -1;
+    int rc = v->decode_fused(qkv.data, qkv.parts, (int)n, q_norm_w, k_norm_w, eps, NULL, rotation, cache->writable ? 1 : 0, cache->k, cache->v, out,
+                             batch->decode_workspace[0], batch->decode_workspace[1], batch->decode_rows, batch->positions, batch->seq_of_token,
+                             batch->tables[cache->group], (int)batch->max_blocks, (int)n, (int)g->n_q, (int)g->n_kv, (int)g->head_dim,
+                             (int)cache->page_tokens, g->scale, (int)g->window, grid, (int)max_splits, arrivals, st->stream);
+    if (rc != 0) return refused(error, "attention_decode_fused", rc);
+    *done = true;
+    return 0;
+}
+
 static int hip_attention(kipp_runtime *rt, const void *q, const kipp_cache_view *cache, void *out, kipp_batch *batch,
                          const kipp_attention_geometry *g, kipp_error *error) {
     hip_state *st = rt->state;
     const uint32_t group = g->n_q / g->n_kv, page = cache->page_tokens;
     const int32_t *table = batch->tables[cache->group];
     int rc;
-    bool fast = rt->act_dtype == KIPP_BF16 && g->head_dim % 16 == 0 && group <= 16 && (page & (page - 1)) == 0 &&
-                batch->max_blocks <= PREFILL_MAX_BLOCKS;
+    const bool fast = attention_fast(rt, g, cache, batch);
     if (!fast) {
         /* the float32 path, and geometries the matrix-core kernels refuse (head sizes that are no multiple of 16, more than
          * 16 query heads a key/value head, pages that are no power of two) */
@@ -568,26 +794,65 @@ static int hip_attention(kipp_runtime *rt, const void *q, const kipp_cache_view 
         if (rc != 0) return refused(error, "attention_prefill", rc);
     }
     if (batch->n_decode != 0) {
-        /* partial results of the splits, shared by the layers of one geometry within the step; without a count of
-         * finished splits the merge is a launch of its own */
-        const size_t max_splits = (batch->max_decode_ctx + (size_t)v->split_min - 1) / (size_t)v->split_min + 1;
-        const size_t key = ((size_t)g->n_q << 32) ^ ((size_t)g->head_dim << 16) ^ max_splits;
-        if (batch->decode_workspace[0] == NULL || batch->decode_workspace_key != key) {
-            size_t rows = (size_t)batch->n_decode * g->n_q * max_splits;
-            batch->decode_workspace[0] = kipp_scratch(rt, rows * g->head_dim * sizeof(float), error);
-            batch->decode_workspace[1] = kipp_scratch(rt, rows * 2 * sizeof(float), error);
-            if (batch->decode_workspace[0] == NULL || batch->decode_workspace[1] == NULL) return -1;
-            batch->decode_workspace_key = key;
-        }
-        uint32_t span = g->window != 0 && g->window < batch->max_decode_ctx ? g->window : batch->max_decode_ctx;
-        size_t need = (span + (size_t)v->split - 1) / (size_t)v->split + (g->window != 0 ? 1 : 0);
-        int grid = (int)(need < 1 ? 1 : (need > max_splits ? max_splits : need));
+        size_t max_splits;
+        int grid;
+        int32_t *arrivals;
+        if (decode_workspace(rt, batch, v, g, &max_splits, &grid, error) != 0 || arrivals_for(rt, (size_t)batch->n_decode * g->n_q, &arrivals, error) != 0)
+            return -1;
         rc = v->decode(q, cache->k, cache->v, out, batch->decode_workspace[0], batch->decode_workspace[1], batch->decode_rows, batch->positions,
                        batch->seq_of_token, table, (int)batch->max_blocks, (int)batch->n_decode, (int)g->n_q, (int)g->n_kv, (int)g->head_dim,
-                       (int)page, g->scale, (int)g->window, grid, (int)max_splits, NULL, st->stream);
+                       (int)page, g->scale, (int)g->window, grid, (int)max_splits, arrivals, st->stream);
         if (rc != 0) return refused(error, "attention_decode", rc);
     }
     return 0;
+}
+
+/* A step that failed may have left counts of finished splits behind: zero them, so that the next launch merges when it should. */
+static void hip_after_failed_step(kipp_runtime *rt) {
+    hip_state *st = rt->state;
+    hipStreamSynchronize(st->stream);
+    (void)hipGetLastError();
+    if (st->arrivals != NULL) st->fill_zero(st->arrivals, st->arrivals_count, st->stream);
+}
+
+/* ------------------------------------------------------------------ recorded steps (HIP graphs) */
+static int hip_graph_begin(kipp_runtime *rt, kipp_error *error) {
+    hip_state *st = rt->state;
+    hipError_t code = hipStreamBeginCapture(st->stream, hipStreamCaptureModeThreadLocal);
+    if (code != hipSuccess) return hip_bad(error, code, "hipStreamBeginCapture");
+    rt->recording = true;
+    return 0;
+}
+
+static int hip_graph_end(kipp_runtime *rt, bool keep, void **out_graph, kipp_error *error) {
+    hip_state *st = rt->state;
+    hipGraph_t graph = NULL;
+    hipError_t code = hipStreamEndCapture(st->stream, &graph);
+    rt->recording = false;
+    *out_graph = NULL;
+    if (code != hipSuccess || graph == NULL || !keep) {
+        if (graph != NULL) hipGraphDestroy(graph);
+        (void)hipGetLastError();
+        return keep ? hip_bad(error, code, "hipStreamEndCapture") : 0;
+    }
+    hipGraphExec_t exec = NULL;
+    code = hipGraphInstantiate(&exec, graph, NULL, NULL, 0);
+    hipGraphDestroy(graph);
+    if (code != hipSuccess) return hip_bad(error, code, "hipGraphInstantiate");
+    *out_graph = exec;
+    return 0;
+}
+
+static int hip_graph_launch(kipp_runtime *rt, void *graph, kipp_error *error) {
+    hip_state *st = rt->state;
+    hipError_t code = hipGraphLaunch((hipGraphExec_t)graph, st->stream);
+    return code == hipSuccess ? 0 : hip_bad(error, code, "hipGraphLaunch");
+}
+
+static void hip_graph_free(kipp_runtime *rt, void *graph) {
+    hip_state *st = rt->state;
+    hipStreamSynchronize(st->stream);
+    hipGraphExecDestroy((hipGraphExec_t)graph);
 }
 
 static int hip_gather_rows(kipp_runtime *rt, const float *x, const int32_t *index, float *out, uint32_t n, uint32_t width, kipp_error *error) {
@@ -638,6 +903,11 @@ kipp_runtime *kipp_runtime_hip(kipp_path path, int device, const char *kernel_di
     }
     rt->state = st;
     st->device = device;
+    /* KIPP_AMD_FUSE=0: every norm and the rotation as kernels of their own, also for few rows; KIPP_AMD_DECODE_MERGE=launch:
+     * the splits of decode attention are merged by a launch of its own, which needs no ordering between workgroups */
+    const char *fuse = getenv("KIPP_AMD_FUSE"), *merge = getenv("KIPP_AMD_DECODE_MERGE");
+    st->fuse = path == KIPP_PATH_GPU_BF16 && !(fuse != NULL && strcmp(fuse, "0") == 0);
+    st->merge_in_kernel = !(merge != NULL && strcmp(merge, "launch") == 0);
     if (kernel_dir != NULL && kernel_dir[0] != '\0') snprintf(st->kernel_dir, sizeof(st->kernel_dir), "%s", kernel_dir);
     else default_kernel_dir(st->kernel_dir, sizeof(st->kernel_dir));
     if ((code = hipSetDevice(device)) != hipSuccess || (code = hipStreamCreate(&st->stream)) != hipSuccess) {
@@ -675,5 +945,17 @@ kipp_runtime *kipp_runtime_hip(kipp_path path, int device, const char *kernel_di
     rt->qk_norm_rope_kv = hip_qk_norm_rope_kv;
     rt->attention = hip_attention;
     rt->gather_rows = hip_gather_rows;
+    rt->defers = hip_defers;
+    rt->scale_rows = hip_scale_rows;
+    rt->gated = hip_gated;
+    rt->decode_attention = hip_decode_attention;
+    rt->argmax = hip_argmax;
+    rt->after_failed_step = hip_after_failed_step;
+    if (path == KIPP_PATH_GPU_BF16) { /* the 32-bit path is for checking, not for speed: its steps run as they are */
+        rt->graph_begin = hip_graph_begin;
+        rt->graph_end = hip_graph_end;
+        rt->graph_launch = hip_graph_launch;
+        rt->graph_free = hip_graph_free;
+    }
     return rt;
 }

@@ -215,18 +215,43 @@ int kipp_pool_check(const kipp_pool *pool, kipp_error *error);
 struct kipp_backend;
 struct kipp_runtime;
 
-/* A matrix [n, k] where the path computes. */
+/* A matrix [n, k] where the path computes: its rows as stored, and (bfloat16 on the GPU, k a multiple of 32) the same
+ * values once more in the layout that the few-rows products stream fastest, [tile of 16 rows][step of 32 columns][lane][8].
+ * `pairs`: the matrix is [gate; up] and a tile holds 8 gate rows over the 8 matching up rows. */
 typedef struct {
     void *data;
     int dtype;
     uint32_t n, k;
+    void *tiles;
+    bool pairs;
 } kipp_weight;
 
-/* A delta of the residual stream: float32 [parts, rows, width] whose sum over parts is the value. */
+typedef enum { KIPP_LAYOUT_ROWS = 0, KIPP_LAYOUT_STREAM, KIPP_LAYOUT_STREAM_PAIRS } kipp_weight_layout;
+
+/* Rows in the activation type.  With `sumsq` they still lack the scale of their RMS norm: data = rows * norm weight, and
+ * row t's scale is rsqrt(sum(sumsq[t, :sumsq_parts]) / width + eps), sumsq in rows of sumsq_parts rounded up to 4.  A row's
+ * scale commutes with a product over the row, so a product may apply it to its own rows; kipp_finish_rows gives any other
+ * consumer the finished rows. */
+typedef struct {
+    void *data;
+    const float *sumsq;
+    int sumsq_parts;
+    float eps;
+} kipp_rows;
+
+/* A delta of the residual stream: float32 [parts, rows, width] whose sum over parts is the value; or (parts 0, w given) the
+ * product x [m, k] . w^T that has not been launched yet, which the norm that follows may launch together with the residual
+ * add and kipp_settle launches as it is. */
 typedef struct {
     float *data;
     int parts;
+    const void *x;
+    const kipp_weight *w;
+    uint32_t m;
+    int max_parts;
 } kipp_delta;
+
+static inline bool kipp_delta_any(const kipp_delta *delta) { return delta != NULL && (delta->parts > 0 || delta->w != NULL); }
 
 /* What a mixer keeps per token (in pages) and per session (of fixed size). */
 typedef struct {
@@ -315,6 +340,7 @@ bool kipp_cache_view_of(const kipp_cache *cache, uint32_t run, int32_t cache_of,
 /* ------------------------------------------------------------------ one step's batch, flattened (step.c) */
 typedef struct {
     uint32_t n_tokens, n_seqs, n_want, n_decode, n_portions;
+    bool want_every_row; /* the wanted rows are all rows, in order */
     uint32_t max_decode_ctx, max_blocks;
     /* on the host */
     int32_t *h_all;
@@ -328,7 +354,7 @@ typedef struct {
     size_t capacity; /* ints the two buffers hold */
     /* values of this forward pass that parts share */
     const float *rotation;    /* what the table's rotary_angles made */
-    const float *rotation_of; /* the frequencies it was made from */
+    uint64_t rotation_of;     /* the `same_as` of the frequencies it was made from (0: none yet) */
     void *decode_workspace[3];
     size_t decode_workspace_key;
 } kipp_batch;
@@ -360,25 +386,29 @@ typedef struct kipp_part_kind {
 } kipp_part_kind;
 
 typedef struct {
-    /* out = norm(x [+ delta]) in the activation type; with a delta, x += delta in place first */
-    int (*forward)(void *part, float *x, const kipp_delta *delta, void *out, uint32_t rows, kipp_error *error);
+    /* out->data (given by the caller) = norm(x [+ delta]) in the activation type; with a delta, x += delta in place first.
+     * `may_leave_scale`: the consumer takes rows that lack their scale (out->sumsq then says so). */
+    int (*forward)(void *part, float *x, kipp_delta *delta, kipp_rows *out, uint32_t rows, bool may_leave_scale, kipp_error *error);
 } kipp_norm_fn;
 
 typedef struct {
-    /* frequencies where the path computes (NULL: no rotation), the dims they turn, the pairing */
-    int (*table)(void *part, const float **inv_freq, uint32_t *rotary_dim, int *interleaved);
+    /* frequencies where the path computes (NULL: no rotation), the dims they turn, the pairing, and a number that two parts
+     * share exactly if they turn alike (0: no rotation) */
+    int (*table)(void *part, const float **inv_freq, uint32_t *rotary_dim, int *interleaved, uint64_t *same_as);
 } kipp_position_fn;
 
 typedef struct {
     void (*cache_need)(const void *spec, kipp_kv_need *out);
     void (*state_need)(const void *spec, kipp_state_need *out);
-    /* x: [tokens, hidden] in the activation type; out: the delta, in workspace of the step */
-    int (*forward)(void *part, const void *x, kipp_batch *batch, const kipp_cache_view *cache, void *state, kipp_delta *out,
+    /* x: [tokens, hidden] in the activation type; out: the delta, in workspace of the step (or a product not yet launched) */
+    int (*forward)(void *part, const kipp_rows *x, kipp_batch *batch, const kipp_cache_view *cache, void *state, kipp_delta *out,
                    kipp_error *error);
+    bool takes_scaled_rows; /* false: the block finishes rows that lack their scale before it calls */
 } kipp_mixer_fn;
 
 typedef struct {
-    int (*forward)(void *part, const void *x, kipp_batch *batch, kipp_delta *out, kipp_error *error);
+    int (*forward)(void *part, const kipp_rows *x, kipp_batch *batch, kipp_delta *out, kipp_error *error);
+    bool takes_scaled_rows;
 } kipp_ffn_fn;
 
 typedef struct {
@@ -415,12 +445,28 @@ struct kipp_model {
     size_t session_count, session_capacity;
     uint64_t weight_bytes;
     int fail_forward_after; /* tests: < 0 never; else the forward pass after that many fails */
+    /* steps of single tokens, recorded once a shape has come twice and run again as a graph (step.c) */
+    struct kipp_step_graph *graphs;
+    size_t graph_count, graph_capacity;
+    uint64_t graph_replays;
 };
+
+/* One recorded shape: rows, the width of the block tables, the longest context (both rounded up), logits or their largest. */
+typedef struct kipp_step_graph {
+    uint64_t key;
+    uint32_t seen;
+    bool refused;          /* recording it failed once: it runs as it is */
+    void *graph;
+    const void *batch_base; /* what the recording read its integers from: valid while the batch's buffer has not moved */
+    uint64_t generation;    /* ... and while the table of operations has not moved its own buffers */
+    float *logits;
+    int32_t *chosen;
+} kipp_step_graph;
 
 int kipp_model_params(const kipp_model_spec *spec, kipp_param_list *out, kipp_error *error);
 int kipp_model_forward(kipp_model *model, kipp_batch *batch, float **out_logits, kipp_error *error);
 int kipp_embedding_forward(void *part, const int32_t *tokens, float *out, uint32_t n, kipp_error *error);
-int kipp_head_forward(void *part, const void *x, uint32_t rows, kipp_delta *out, kipp_error *error);
+int kipp_head_forward(void *part, const kipp_rows *x, uint32_t rows, kipp_delta *out, kipp_error *error);
 uint64_t kipp_weight_bytes(const kipp_weight *w);
 int kipp_check_tensors(const char *where, kipp_tensor_file *found, const kipp_param_list *expected, kipp_error *error);
 

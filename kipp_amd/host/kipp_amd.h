@@ -65,6 +65,7 @@ typedef struct {
     int device;               /* GPU ordinal */
     const char *kernel_dir;   /* folder of the built kernel libraries; NULL: $KIPP_AMD_KERNELS, else beside this library */
     const uint32_t *page_order; /* NULL, or kv_pool_pages page ids: the order in which a fresh pool hands out its pages */
+    int eager_steps;          /* nonzero: no step is recorded and run again as a graph (gpu-bf16 records its steps of single tokens) */
 } kipp_model_open_config;
 
 typedef struct {
@@ -163,6 +164,11 @@ typedef struct {
  */
 int kipp_step(kipp_model *model, const kipp_step_item *items, size_t item_count, float *logits, size_t logits_capacity,
               kipp_error *error);
+/* The same step, answered with the index of the largest logit at every wanted place (the lowest index among equals,
+ * /root/reference/src/kipp.c:3459-3464), found where the path computes: greedy decoding then reads back one number a
+ * place instead of a row of logits. */
+int kipp_step_argmax(kipp_model *model, const kipp_step_item *items, size_t item_count, uint32_t *tokens, size_t token_capacity,
+                     kipp_error *error);
 
 int kipp_sample(const float *logits, size_t logits_count, float temperature, float top_p, uint64_t *rng_state, uint32_t *out_token,
                 kipp_error *error);

@@ -106,6 +106,10 @@ static void model_free(kipp_model *model) {
     if (model == NULL) return;
     free(model->batch.h_all);
     if (model->rt != NULL) {
+        for (size_t i = 0; i < model->graph_count; ++i) {
+            if (model->graphs[i].graph != NULL) model->rt->graph_free(model->rt, model->graphs[i].graph);
+        }
+        free(model->graphs);
         if (model->batch.d_all != NULL && !model->rt->on_host) model->rt->mem_free(model->rt, model->batch.d_all);
         if (model->batch.d_all != NULL && model->rt->on_host) free(model->batch.d_all);
         free(model->batch.tables);
@@ -170,7 +174,7 @@ int kipp_model_open_ex(const char *model_dir, const kipp_model_open_config *conf
     }
     model->embedding.kind = kipp_part_kind_of("embedding", "embedding", error);
     if (model->embedding.kind == NULL || (model->embedding.part = model->embedding.kind->create(&spec->embedding, rt, error)) == NULL) goto fail;
-    if (model->embedding.kind->load(model->embedding.part, &model->tensors, NULL, error) != 0) goto fail;
+    if (model->embedding.kind->load(model->embedding.part, &model->tensors, (void *)&spec->head, error) != 0) goto fail;
     for (uint32_t l = 0; l < spec->layer_count; ++l) {
         model->blocks[l].kind = kipp_part_kind_of("block", spec->layers[l].block, error);
         if (model->blocks[l].kind == NULL || (model->blocks[l].part = model->blocks[l].kind->create(&spec->layers[l], rt, error)) == NULL) goto fail;
@@ -280,14 +284,14 @@ int kipp_model_forward(kipp_model *model, kipp_batch *batch, float **out_logits,
     const kipp_model_spec *spec = &model->spec;
     const uint32_t n = batch->n_tokens;
     *out_logits = NULL;
-    if (model->fail_forward_after >= 0 && model->fail_forward_after-- == 0) return kipp_fail(error, KIPP_ERROR_INTERNAL, "the forward pass was told to fail (a test's switch)");
-    batch->rotation = batch->rotation_of = NULL;
+    batch->rotation = NULL;
+    batch->rotation_of = 0;
     batch->item_seq = batch->item_tile = NULL;
     batch->n_items = 0;
     batch->decode_workspace[0] = NULL;
     float *x = kipp_scratch(rt, (size_t)n * spec->hidden * sizeof(float), error);
     if (x == NULL || kipp_embedding_forward(model->embedding.part, batch->tokens, x, n, error) != 0) return -1;
-    kipp_delta pending = {NULL, 0};
+    kipp_delta pending = {NULL, 0, NULL, NULL, 0, 0};
     for (uint32_t run = 0; run < spec->run_count; ++run) {
         const kipp_built_part *block = &model->blocks[spec->order[run].layer];
         kipp_cache_view view;
@@ -296,14 +300,22 @@ int kipp_model_forward(kipp_model *model, kipp_batch *batch, float **out_logits,
             return -1;
     }
     if (batch->n_want == 0) return 0; /* a portion of a prompt whose logits nobody needs: no final norm, no head */
-    if (pending.parts > 0 && rt->residual_add(rt, x, &pending, n, spec->hidden, error) != 0) return -1;
-    float *rows = kipp_scratch(rt, (size_t)batch->n_want * spec->hidden * sizeof(float), error);
-    void *normed = kipp_scratch(rt, (size_t)batch->n_want * spec->hidden * kipp_dtype_bytes(rt->act_dtype), error);
-    if (rows == NULL || normed == NULL) return -1;
-    if (rt->gather_rows(rt, x, batch->want_rows, rows, batch->n_want, spec->hidden, error) != 0) return -1;
-    if (((const kipp_norm_fn *)model->final_norm.kind->fn)->forward(model->final_norm.part, rows, NULL, normed, batch->n_want, error) != 0) return -1;
+    const kipp_norm_fn *final_norm = model->final_norm.kind->fn;
+    kipp_rows normed = {kipp_scratch(rt, (size_t)batch->n_want * spec->hidden * kipp_dtype_bytes(rt->act_dtype), error), NULL, 0, 0.0f};
+    if (normed.data == NULL) return -1;
+    if (batch->want_every_row) {
+        /* every row in order (a step of single tokens): no gather, the last delta is added inside the norm, and the head's
+         * product may apply the norm's scale */
+        if (final_norm->forward(model->final_norm.part, x, kipp_delta_any(&pending) ? &pending : NULL, &normed, n, true, error) != 0) return -1;
+    } else {
+        if (kipp_delta_any(&pending) && rt->residual_add(rt, x, &pending, n, spec->hidden, error) != 0) return -1;
+        float *rows = kipp_scratch(rt, (size_t)batch->n_want * spec->hidden * sizeof(float), error);
+        if (rows == NULL) return -1;
+        if (rt->gather_rows(rt, x, batch->want_rows, rows, batch->n_want, spec->hidden, error) != 0) return -1;
+        if (final_norm->forward(model->final_norm.part, rows, NULL, &normed, batch->n_want, true, error) != 0) return -1;
+    }
     kipp_delta logits;
-    if (kipp_head_forward(model->head.part, normed, batch->n_want, &logits, error) != 0) return -1;
+    if (kipp_head_forward(model->head.part, &normed, batch->n_want, &logits, error) != 0) return -1;
     if (logits.parts != 1) return kipp_fail(error, KIPP_ERROR_INTERNAL, "the head's product came in %d parts", logits.parts);
     *out_logits = logits.data;
     return 0;

@@ -116,9 +116,9 @@ static void rms_norm_destroy(void *part_) {
 }
 
 /* y = x * rsqrt(mean(x^2) + eps) * w  (/root/reference/src/kipp.c:2221-2231) */
-static int rms_norm_forward(void *part_, float *x, const kipp_delta *delta, void *out, uint32_t rows, kipp_error *error) {
+static int rms_norm_forward(void *part_, float *x, kipp_delta *delta, kipp_rows *out, uint32_t rows, bool may_leave_scale, kipp_error *error) {
     rms_norm_part *part = part_;
-    return part->rt->rmsnorm(part->rt, x, delta, part->weight, out, rows, part->spec.width, part->spec.eps, error);
+    return part->rt->rmsnorm(part->rt, x, delta, part->weight, out, rows, part->spec.width, part->spec.eps, may_leave_scale, error);
 }
 
 static const kipp_norm_fn rms_norm_fn = {rms_norm_forward};
@@ -130,6 +130,7 @@ typedef struct {
     kipp_rope_spec spec;
     kipp_runtime *rt;
     float *inv_freq; /* where the path computes */
+    uint64_t same_as; /* a hash of the frequencies' bits: layers that turn alike share one step's angles */
 } rope_part;
 
 static int no_params(const void *spec, kipp_param_list *out, kipp_error *error) {
@@ -160,6 +161,13 @@ static void *rope_create(const void *spec_, kipp_runtime *rt, kipp_error *error)
     part->spec = *spec;
     part->rt = rt;
     for (uint32_t i = 0; i < half; ++i) host[i] = (float)pow(spec->theta, -(2.0 * (double)i) / (double)spec->rotary_dim);
+    part->same_as = 1469598103934665603ull ^ spec->rotary_dim;
+    for (uint32_t i = 0; i < half; ++i) {
+        uint32_t bits;
+        memcpy(&bits, &host[i], sizeof(bits));
+        part->same_as = (part->same_as ^ bits) * 1099511628211ull;
+    }
+    if (part->same_as == 0) part->same_as = 1;
     part->inv_freq = rt->mem_alloc(rt, half * sizeof(float), error);
     if (part->inv_freq == NULL || rt->upload(rt, part->inv_freq, host, half * sizeof(float), error) != 0) {
         if (part->inv_freq != NULL) rt->mem_free(rt, part->inv_freq);
@@ -185,11 +193,12 @@ static void rope_destroy(void *part_) {
     free(part);
 }
 
-static int rope_table(void *part_, const float **inv_freq, uint32_t *rotary_dim, int *interleaved) {
+static int rope_table(void *part_, const float **inv_freq, uint32_t *rotary_dim, int *interleaved, uint64_t *same_as) {
     rope_part *part = part_;
     *inv_freq = part->inv_freq;
     *rotary_dim = part->spec.rotary_dim;
     *interleaved = part->spec.interleaved;
+    *same_as = part->same_as;
     return 0;
 }
 
@@ -205,11 +214,12 @@ static void *none_create(const void *spec, kipp_runtime *rt, kipp_error *error) 
     return part;
 }
 
-static int none_table(void *part, const float **inv_freq, uint32_t *rotary_dim, int *interleaved) {
+static int none_table(void *part, const float **inv_freq, uint32_t *rotary_dim, int *interleaved, uint64_t *same_as) {
     (void)part;
     *inv_freq = NULL;
     *rotary_dim = 0;
     *interleaved = 0;
+    *same_as = 0;
     return 0;
 }
 
@@ -283,7 +293,8 @@ static int attention_load(void *part_, const kipp_tensor_file *tensors, void *co
     const kipp_tensor *o = tensor_of(tensors, part->spec.prefix, "o_proj.weight", error);
     if (qkv[0] == NULL || qkv[1] == NULL || qkv[2] == NULL || o == NULL) return -1;
     /* rows one under the other: one product serves q, k and v, and no output element changes */
-    if (rt->place_matrix(rt, qkv, 3, &part->w_qkv, error) != 0 || rt->place_matrix(rt, &o, 1, &part->w_o, error) != 0) return -1;
+    if (rt->place_matrix(rt, qkv, 3, KIPP_LAYOUT_STREAM, &part->w_qkv, error) != 0 || rt->place_matrix(rt, &o, 1, KIPP_LAYOUT_STREAM, &part->w_o, error) != 0)
+        return -1;
     if (part->spec.qk_norm) {
         const kipp_tensor *qn = tensor_of(tensors, part->spec.prefix, "q_norm.weight", error);
         const kipp_tensor *kn = tensor_of(tensors, part->spec.prefix, "k_norm.weight", error);
@@ -305,7 +316,7 @@ static void no_state(const void *spec, kipp_state_need *out) {
 
 /* Causal grouped-query attention with optional per-head q/k norm, a position part and an optional window over the
  * paged cache; query head h reads key/value head h / (n_q / n_kv)  (/root/reference/src/kipp.c:2950-2993). */
-static int attention_forward(void *part_, const void *x, kipp_batch *batch, const kipp_cache_view *cache, void *state, kipp_delta *out,
+static int attention_forward(void *part_, const kipp_rows *x, kipp_batch *batch, const kipp_cache_view *cache, void *state, kipp_delta *out,
                              kipp_error *error) {
     attention_part *part = part_;
     kipp_runtime *rt = part->rt;
@@ -315,31 +326,42 @@ static int attention_forward(void *part_, const void *x, kipp_batch *batch, cons
     const float *inv_freq;
     uint32_t rotary_dim;
     int interleaved;
-    ((const kipp_position_fn *)part->position.kind->fn)->table(part->position.part, &inv_freq, &rotary_dim, &interleaved);
+    uint64_t same_as;
+    ((const kipp_position_fn *)part->position.kind->fn)->table(part->position.part, &inv_freq, &rotary_dim, &interleaved, &same_as);
     const float *rotation = NULL;
     if (inv_freq != NULL) {
         /* made by the first layer of a forward pass that turns with these frequencies, shared by the others */
-        if (batch->rotation_of != inv_freq) {
+        if (batch->rotation_of != same_as) {
             if (rt->rotary_angles(rt, batch->positions, inv_freq, batch->n_tokens, rotary_dim / 2, &batch->rotation, error) != 0) return -1;
-            batch->rotation_of = inv_freq;
+            batch->rotation_of = same_as;
         }
         rotation = batch->rotation;
     }
     const uint32_t n = batch->n_tokens;
     const size_t q_dim = (size_t)s->n_heads * s->head_dim, act = kipp_dtype_bytes(rt->act_dtype);
     const kipp_attention_geometry geometry = {s->n_heads, s->n_kv_heads, s->head_dim, s->window, part->scale};
+    const float eps = s->qk_norm ? s->qk_norm_eps : 0.0f;
+    void *mixed = kipp_scratch(rt, n * q_dim * act, error);
+    if (mixed == NULL) return -1;
+    if (rt->decode_attention != NULL && batch->n_portions == 0) {
+        /* single tokens only: a table may have fewer kernels for the way from x to the mixed heads */
+        bool done = false;
+        if (rt->decode_attention(rt, x, &part->w_qkv, cache, mixed, batch, &geometry, part->q_norm, part->k_norm, eps, rotation, rotary_dim,
+                                 interleaved, &done, error) != 0)
+            return -1;
+        if (done) return kipp_linear_defer(rt, &(kipp_rows){mixed, NULL, 0, 0.0f}, &part->w_o, n, 8, out, error);
+    }
     kipp_delta qkv;
     if (rt->linear(rt, x, &part->w_qkv, n, 4, &qkv, error) != 0) return -1;
-    void *q = kipp_scratch(rt, n * q_dim * act, error), *mixed = kipp_scratch(rt, n * q_dim * act, error);
-    if (q == NULL || mixed == NULL) return -1;
-    if (rt->qk_norm_rope_kv(rt, &qkv, q, cache, batch, &geometry, part->q_norm, part->k_norm, s->qk_norm ? s->qk_norm_eps : 0.0f, rotation,
-                            rotary_dim, interleaved, error) != 0)
+    void *q = kipp_scratch(rt, n * q_dim * act, error);
+    if (q == NULL) return -1;
+    if (rt->qk_norm_rope_kv(rt, &qkv, q, cache, batch, &geometry, part->q_norm, part->k_norm, eps, rotation, rotary_dim, interleaved, error) != 0)
         return -1;
     if (rt->attention(rt, q, cache, mixed, batch, &geometry, error) != 0) return -1;
-    return rt->linear(rt, mixed, &part->w_o, n, 8, out, error);
+    return kipp_linear_defer(rt, &(kipp_rows){mixed, NULL, 0, 0.0f}, &part->w_o, n, 8, out, error);
 }
 
-static const kipp_mixer_fn attention_fn = {attention_cache_need, no_state, attention_forward};
+static const kipp_mixer_fn attention_fn = {attention_cache_need, no_state, attention_forward, true};
 static const kipp_part_kind attention_kind = {"mixer",        "attention",      sizeof(kipp_attention_spec), attention_params, attention_create,
                                               attention_load, attention_destroy, &attention_fn};
 
@@ -377,8 +399,8 @@ static int gated_mlp_load(void *part_, const kipp_tensor_file *tensors, void *co
                                      tensor_of(tensors, part->spec.prefix, "up_proj.weight", error)};
     const kipp_tensor *down = tensor_of(tensors, part->spec.prefix, "down_proj.weight", error);
     if (gate_up[0] == NULL || gate_up[1] == NULL || down == NULL) return -1;
-    if (part->rt->place_matrix(part->rt, gate_up, 2, &part->w_gate_up, error) != 0) return -1;
-    return part->rt->place_matrix(part->rt, &down, 1, &part->w_down, error);
+    if (part->rt->place_matrix(part->rt, gate_up, 2, KIPP_LAYOUT_STREAM_PAIRS, &part->w_gate_up, error) != 0) return -1;
+    return part->rt->place_matrix(part->rt, &down, 1, KIPP_LAYOUT_STREAM, &part->w_down, error);
 }
 
 static void gated_mlp_destroy(void *part_) {
@@ -389,18 +411,22 @@ static void gated_mlp_destroy(void *part_) {
 }
 
 /* delta = W_down (silu(W_gate x) * (W_up x))  (/root/reference/src/kipp.c:2633-2653) */
-static int gated_mlp_forward(void *part_, const void *x, kipp_batch *batch, kipp_delta *out, kipp_error *error) {
+static int gated_mlp_forward(void *part_, const kipp_rows *x, kipp_batch *batch, kipp_delta *out, kipp_error *error) {
     gated_mlp_part *part = part_;
     kipp_runtime *rt = part->rt;
     const uint32_t n = batch->n_tokens;
-    kipp_delta gate_up;
-    if (rt->linear(rt, x, &part->w_gate_up, n, 8, &gate_up, error) != 0) return -1;
     void *act = kipp_scratch(rt, (size_t)n * part->spec.inner * kipp_dtype_bytes(rt->act_dtype), error);
-    if (act == NULL || rt->swiglu(rt, &gate_up, act, n, part->spec.inner, error) != 0) return -1;
-    return rt->linear(rt, act, &part->w_down, n, 8, out, error);
+    if (act == NULL) return -1;
+    bool done = false;
+    if (rt->gated != NULL && rt->gated(rt, x, &part->w_gate_up, act, n, &done, error) != 0) return -1; /* both products and the activation in one kernel */
+    if (!done) {
+        kipp_delta gate_up;
+        if (rt->linear(rt, x, &part->w_gate_up, n, 8, &gate_up, error) != 0 || rt->swiglu(rt, &gate_up, act, n, part->spec.inner, error) != 0) return -1;
+    }
+    return kipp_linear_defer(rt, &(kipp_rows){act, NULL, 0, 0.0f}, &part->w_down, n, 8, out, error);
 }
 
-static const kipp_ffn_fn gated_mlp_fn = {gated_mlp_forward};
+static const kipp_ffn_fn gated_mlp_fn = {gated_mlp_forward, true};
 static const kipp_part_kind gated_mlp_kind = {"feed_forward", "gated_mlp",      sizeof(kipp_gated_mlp_spec), gated_mlp_params, gated_mlp_create,
                                               gated_mlp_load, gated_mlp_destroy, &gated_mlp_fn};
 
@@ -484,15 +510,23 @@ static int pre_norm_forward(void *block_, float *x, kipp_delta *pending, kipp_ba
                             kipp_error *error) {
     pre_norm_block *block = block_;
     kipp_runtime *rt = block->rt;
-    const size_t bytes = (size_t)batch->n_tokens * block->hidden * kipp_dtype_bytes(rt->act_dtype);
-    void *h = kipp_scratch(rt, bytes, error);
-    if (h == NULL) return -1;
+    const uint32_t n = batch->n_tokens;
+    const size_t bytes = (size_t)n * block->hidden * kipp_dtype_bytes(rt->act_dtype);
     const kipp_norm_fn *norm1 = block->mixer_norm.kind->fn, *norm2 = block->ffn_norm.kind->fn;
-    if (norm1->forward(block->mixer_norm.part, x, pending->parts > 0 ? pending : NULL, h, batch->n_tokens, error) != 0) return -1;
+    const kipp_mixer_fn *mixer = block->mixer.kind->fn;
+    const kipp_ffn_fn *ffn = block->ffn.kind->fn;
+    /* a part that does not take rows without their scale gets finished ones: the norm is told, and what it leaves all the same is finished here */
+    kipp_rows h = {kipp_scratch(rt, bytes, error), NULL, 0, 0.0f};
+    if (h.data == NULL) return -1;
+    if (norm1->forward(block->mixer_norm.part, x, kipp_delta_any(pending) ? pending : NULL, &h, n, mixer->takes_scaled_rows, error) != 0) return -1;
+    if (!mixer->takes_scaled_rows && kipp_finish_rows(rt, &h, n, block->hidden, error) != 0) return -1;
     kipp_delta delta;
-    if (((const kipp_mixer_fn *)block->mixer.kind->fn)->forward(block->mixer.part, h, batch, cache, state, &delta, error) != 0) return -1;
-    if (norm2->forward(block->ffn_norm.part, x, &delta, h, batch->n_tokens, error) != 0) return -1;
-    return ((const kipp_ffn_fn *)block->ffn.kind->fn)->forward(block->ffn.part, h, batch, pending, error);
+    if (mixer->forward(block->mixer.part, &h, batch, cache, state, &delta, error) != 0) return -1;
+    kipp_rows h2 = {kipp_scratch(rt, bytes, error), NULL, 0, 0.0f};
+    if (h2.data == NULL) return -1;
+    if (norm2->forward(block->ffn_norm.part, x, &delta, &h2, n, ffn->takes_scaled_rows, error) != 0) return -1;
+    if (!ffn->takes_scaled_rows && kipp_finish_rows(rt, &h2, n, block->hidden, error) != 0) return -1;
+    return ffn->forward(block->ffn.part, &h2, batch, pending, error);
 }
 
 static void *pre_norm_mixer_of(void *block_, const kipp_part_kind **kind, const void **spec) {
@@ -529,11 +563,13 @@ static void *embedding_create(const void *spec, kipp_runtime *rt, kipp_error *er
     return part;
 }
 
+/* `context`: the head's spec (or NULL); a table that a tied head multiplies with is placed as the products want it */
 static int embedding_load(void *part_, const kipp_tensor_file *tensors, void *context, kipp_error *error) {
     embedding_part *part = part_;
-    (void)context;
+    const kipp_head_spec *head = context;
     const kipp_tensor *table = tensor_of(tensors, part->spec.prefix, "weight", error);
-    return table == NULL ? -1 : part->rt->place_matrix(part->rt, &table, 1, &part->table, error);
+    return table == NULL ? -1
+                         : part->rt->place_matrix(part->rt, &table, 1, head != NULL && head->tied ? KIPP_LAYOUT_STREAM : KIPP_LAYOUT_ROWS, &part->table, error);
 }
 
 static void embedding_destroy(void *part_) {
@@ -576,7 +612,7 @@ static int head_load(void *part_, const kipp_tensor_file *tensors, void *context
         return 0;
     }
     const kipp_tensor *w = tensor_of(tensors, part->spec.prefix, "weight", error);
-    if (w == NULL || part->rt->place_matrix(part->rt, &w, 1, &part->weight, error) != 0) return -1;
+    if (w == NULL || part->rt->place_matrix(part->rt, &w, 1, KIPP_LAYOUT_STREAM, &part->weight, error) != 0) return -1;
     part->owns = true;
     return 0;
 }
@@ -596,7 +632,7 @@ int kipp_embedding_forward(void *part_, const int32_t *tokens, float *out, uint3
 }
 
 /* logits = W x, float32, no bias (/root/reference/src/kipp.c:2660-2661) */
-int kipp_head_forward(void *part_, const void *x, uint32_t rows, kipp_delta *out, kipp_error *error) {
+int kipp_head_forward(void *part_, const kipp_rows *x, uint32_t rows, kipp_delta *out, kipp_error *error) {
     head_part *part = part_;
     return part->rt->linear(part->rt, x, &part->weight, rows, 1, out, error);
 }

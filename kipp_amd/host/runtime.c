@@ -22,6 +22,11 @@ void *kipp_scratch(kipp_runtime *rt, size_t bytes, kipp_error *error) {
         ++rt->workspace.current;
         rt->workspace.used = 0;
     }
+    if (rt->recording) {
+        /* memory cannot be made while operations are recorded: the caller drops the recording and runs the step as it is */
+        kipp_fail(error, KIPP_ERROR_MEMORY, "the step's workspace would grow while a step is recorded");
+        return NULL;
+    }
     size_t size = bytes > KIPP_CHUNK ? bytes : KIPP_CHUNK;
     void **chunks = realloc(rt->workspace.chunks, (rt->workspace.count + 1) * sizeof(void *));
     if (chunks != NULL) rt->workspace.chunks = chunks;
@@ -43,6 +48,31 @@ void *kipp_scratch(kipp_runtime *rt, size_t bytes, kipp_error *error) {
 void kipp_scratch_reset(kipp_runtime *rt) {
     rt->workspace.current = 0;
     rt->workspace.used = 0;
+}
+
+int kipp_settle(kipp_runtime *rt, kipp_delta *delta, kipp_error *error) {
+    if (delta->parts > 0 || delta->w == NULL) return 0;
+    const kipp_rows x = {(void *)delta->x, NULL, 0, 0.0f};
+    const kipp_weight *w = delta->w;
+    delta->w = NULL; /* what linear writes is a delta that has been launched */
+    return rt->linear(rt, &x, w, delta->m, delta->max_parts, delta, error);
+}
+
+int kipp_finish_rows(kipp_runtime *rt, kipp_rows *rows, uint32_t m, uint32_t width, kipp_error *error) {
+    if (rows->sumsq == NULL) return 0;
+    if (rt->scale_rows == NULL) return kipp_fail(error, KIPP_ERROR_INTERNAL, "rows without their scale on a path that leaves none");
+    void *out = kipp_scratch(rt, (size_t)m * width * kipp_dtype_bytes(rt->act_dtype), error);
+    if (out == NULL || rt->scale_rows(rt, rows, out, m, width, error) != 0) return -1;
+    *rows = (kipp_rows){out, NULL, 0, 0.0f};
+    return 0;
+}
+
+int kipp_linear_defer(kipp_runtime *rt, const kipp_rows *x, const kipp_weight *w, uint32_t m, int max_parts, kipp_delta *out, kipp_error *error) {
+    if (rt->defers != NULL && x->sumsq == NULL && rt->defers(rt, x, w, m)) {
+        *out = (kipp_delta){NULL, 0, x->data, w, m, max_parts};
+        return 0;
+    }
+    return rt->linear(rt, x, w, m, max_parts, out, error);
 }
 
 void kipp_runtime_destroy(kipp_runtime *rt) {

@@ -61,6 +61,7 @@ struct kipp_scheduler {
     request **item_requests;
     uint32_t *wants;
     float *logits;
+    uint32_t *chosen;
     size_t logits_rows;
 };
 
@@ -121,7 +122,8 @@ int kipp_scheduler_create(kipp_model *model, const kipp_scheduler_config *config
     s->wants = calloc(s->max_running, sizeof(uint32_t));
     s->logits_rows = s->max_running;
     s->logits = malloc(s->logits_rows * (size_t)model->spec.vocab * sizeof(float));
-    if (s->items == NULL || s->item_requests == NULL || s->wants == NULL || s->logits == NULL) {
+    s->chosen = malloc(s->logits_rows * sizeof(uint32_t));
+    if (s->items == NULL || s->item_requests == NULL || s->wants == NULL || s->logits == NULL || s->chosen == NULL) {
         kipp_scheduler_destroy(s);
         return kipp_fail(error, KIPP_ERROR_MEMORY, "out of memory for the scheduler's step");
     }
@@ -143,6 +145,7 @@ void kipp_scheduler_destroy(kipp_scheduler *s) {
     free(s->item_requests);
     free(s->wants);
     free(s->logits);
+    free(s->chosen);
     free(s);
 }
 
@@ -396,8 +399,17 @@ int kipp_scheduler_step(kipp_scheduler *s, kipp_produced *out, size_t capacity, 
         wanted += last;
     }
     if (n == 0) return 0;
+    /* where every wanted place is chosen by the largest logit alone, the choice is made beside the logits */
+    bool greedy = !s->keep_last_logits;
+    for (uint32_t i = 0; i < n && greedy; ++i) {
+        const kipp_sample_params *p = &s->item_requests[i]->params;
+        greedy = s->items[i].want_count == 0 || (p->temperature <= 0.0f && p->frequency_penalty == 0.0f && p->presence_penalty == 0.0f &&
+                                                 (p->repetition_penalty == 1.0f || p->repetition_penalty == 0.0f) && p->logit_bias_count == 0);
+    }
     kipp_error step_error;
-    if (kipp_step(s->model, s->items, n, s->logits, s->logits_rows * (size_t)s->model->spec.vocab, &step_error) != 0) {
+    int step_rc = greedy ? kipp_step_argmax(s->model, s->items, n, s->chosen, s->logits_rows, &step_error)
+                         : kipp_step(s->model, s->items, n, s->logits, s->logits_rows * (size_t)s->model->spec.vocab, &step_error);
+    if (step_rc != 0) {
         /* the batch failed as a unit: every request that had tokens in it fails; those that were not in it go on */
         ++s->stats.failed_steps;
         for (uint32_t i = 0; i < n; ++i) {
@@ -416,6 +428,10 @@ int kipp_scheduler_step(kipp_scheduler *s, kipp_produced *out, size_t capacity, 
             s->stats.prompt_tokens += s->items[i].token_count;
         }
         if (s->items[i].want_count == 0) continue;
+        if (greedy) {
+            accept(s, r, s->chosen[row++], out, capacity, &produced);
+            continue;
+        }
         const float *logits = s->logits + (size_t)row++ * vocab;
         if (r->last_logits != NULL) memcpy(r->last_logits, logits, (size_t)vocab * sizeof(float));
         kipp_sample_params params = r->params;

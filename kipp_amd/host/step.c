@@ -106,6 +106,10 @@ int kipp_session_match_prefix(kipp_session *session, const uint32_t *tokens, siz
 }
 
 /* ------------------------------------------------------------------ the batch */
+#define KIPP_GRAPH_CONTEXT 1024u /* contexts of recorded steps are rounded up to multiples of this */
+#define KIPP_GRAPH_ROWS 64u      /* most single tokens of a recorded step */
+#define KIPP_GRAPH_SHAPES 64u    /* recordings kept */
+
 static int batch_room(kipp_model *model, size_t ints, kipp_error *error) {
     kipp_batch *batch = &model->batch;
     kipp_runtime *rt = model->rt;
@@ -133,7 +137,7 @@ static int batch_room(kipp_model *model, size_t ints, kipp_error *error) {
 
 /* Flattens the items: the tokens of every item one after the other, with what each operation needs to find a token's
  * sequence, position and pages; all integers go to where the path computes in one copy. */
-static int build_batch(kipp_model *model, const kipp_step_item *items, size_t item_count, kipp_error *error) {
+static int build_batch(kipp_model *model, const kipp_step_item *items, size_t item_count, bool rounded, kipp_error *error) {
     kipp_batch *batch = &model->batch;
     const kipp_cache *cache = &model->cache;
     size_t n_tokens = 0, n_want = 0, n_decode = 0;
@@ -148,6 +152,15 @@ static int build_batch(kipp_model *model, const kipp_step_item *items, size_t it
         for (uint32_t g = 0; g < cache->group_count; ++g) {
             if (items[i].session->table_lengths[g] > max_blocks) max_blocks = items[i].session->table_lengths[g];
         }
+    }
+    if (rounded) {
+        /* a step that may be recorded: the width of the tables and the longest context are rounded up, so that the launches'
+         * shapes, and with them the recording, serve every step of the same class (a row's own position still bounds what
+         * it reads) */
+        uint32_t width = 16;
+        while (width < max_blocks) width *= 2;
+        max_blocks = width;
+        max_decode_ctx = (max_decode_ctx + KIPP_GRAPH_CONTEXT - 1) / KIPP_GRAPH_CONTEXT * KIPP_GRAPH_CONTEXT;
     }
     size_t n = item_count, tables = (size_t)cache->group_count * n * max_blocks;
     size_t ints = 3 * n_tokens + 4 * n + n_want + n_decode + tables;
@@ -199,6 +212,8 @@ static int build_batch(kipp_model *model, const kipp_step_item *items, size_t it
     batch->n_tokens = (uint32_t)n_tokens;
     batch->n_seqs = (uint32_t)n;
     batch->n_want = (uint32_t)n_want;
+    batch->want_every_row = n_want == n_tokens;
+    for (size_t w = 0; w < n_want && batch->want_every_row; ++w) batch->want_every_row = h_want[w] == (int32_t)w;
     batch->n_decode = (uint32_t)n_decode;
     batch->n_portions = (uint32_t)(n - n_decode);
     batch->max_decode_ctx = max_decode_ctx;
@@ -207,8 +222,98 @@ static int build_batch(kipp_model *model, const kipp_step_item *items, size_t it
 }
 
 /* ------------------------------------------------------------------ the step */
+/* The forward pass of the batch, and with `choose` the index of the largest logit of every wanted row beside it (the lowest
+ * among equals): what comes back is then one number a row. */
+static int forward_and_choose(kipp_model *model, bool choose, float **logits, int32_t **chosen, kipp_error *error) {
+    kipp_scratch_reset(model->rt);
+    *chosen = NULL;
+    if (kipp_model_forward(model, &model->batch, logits, error) != 0) return -1;
+    if (!choose || model->batch.n_want == 0) return 0;
+    *chosen = kipp_scratch(model->rt, (size_t)model->batch.n_want * sizeof(int32_t), error);
+    if (*chosen == NULL) return -1;
+    return model->rt->argmax(model->rt, *logits, *chosen, model->batch.n_want, model->spec.vocab, error);
+}
+
+/* Runs the batch.  `single` (tokens one a session, all wanted, their shape rounded by build_batch): a shape that has come
+ * before is recorded, and from then on run again from the recording.  Every buffer a recording names keeps its place:
+ * weights, pages and state slots for the model's life, the step's workspace because a step takes it in the same order from
+ * the same start, the batch's integers and the table's own buffers until they grow (then the recording is made again). */
+static int run_step(kipp_model *model, bool single, bool choose, float **logits, int32_t **chosen, kipp_error *error) {
+    kipp_runtime *rt = model->rt;
+    const kipp_batch *batch = &model->batch;
+    if (!single) return forward_and_choose(model, choose, logits, chosen, error);
+    const uint64_t key = ((uint64_t)batch->n_tokens << 48) | ((uint64_t)batch->max_blocks << 24) | ((uint64_t)(batch->max_decode_ctx / KIPP_GRAPH_CONTEXT) << 1) |
+                         (choose ? 1u : 0u);
+    kipp_step_graph *entry = NULL;
+    for (size_t i = 0; i < model->graph_count && entry == NULL; ++i) {
+        if (model->graphs[i].key == key) entry = &model->graphs[i];
+    }
+    if (entry == NULL) {
+        if (model->graph_count == KIPP_GRAPH_SHAPES) return forward_and_choose(model, choose, logits, chosen, error); /* more shapes than are kept */
+        if (model->graph_count == model->graph_capacity) {
+            size_t capacity = model->graph_capacity == 0 ? 8 : model->graph_capacity * 2;
+            kipp_step_graph *grown = realloc(model->graphs, capacity * sizeof(kipp_step_graph));
+            if (grown == NULL) return forward_and_choose(model, choose, logits, chosen, error);
+            model->graphs = grown;
+            model->graph_capacity = capacity;
+        }
+        entry = &model->graphs[model->graph_count++];
+        *entry = (kipp_step_graph){key, 0, false, NULL, NULL, 0, NULL, NULL};
+    }
+    if (entry->graph != NULL && (entry->batch_base != batch->d_all || entry->generation != rt->generation)) {
+        rt->graph_free(rt, entry->graph); /* a buffer it names has moved */
+        entry->graph = NULL;
+    }
+    if (entry->graph == NULL && entry->seen >= 1 && !entry->refused) {
+        /* the shape has run once as it is (whatever it needed to make is made): record it now */
+        kipp_error why;
+        void *graph = NULL;
+        if (rt->graph_begin(rt, &why) == 0) {
+            int rc = forward_and_choose(model, choose, logits, chosen, &why);
+            if (rt->graph_end(rt, rc == 0, &graph, &why) != 0) graph = NULL;
+        }
+        if (graph == NULL) {
+            entry->refused = true; /* run as it is, now and from now on */
+            if (rt->after_failed_step != NULL) rt->after_failed_step(rt);
+        } else {
+            entry->graph = graph;
+            entry->batch_base = batch->d_all;
+            entry->generation = rt->generation;
+            entry->logits = *logits;
+            entry->chosen = *chosen;
+        }
+    }
+    if (entry->graph != NULL) {
+        *logits = entry->logits;
+        *chosen = entry->chosen;
+        ++model->graph_replays;
+        return rt->graph_launch(rt, entry->graph, error);
+    }
+    ++entry->seen;
+    return forward_and_choose(model, choose, logits, chosen, error);
+}
+
+uint64_t kipp_test_graph_replays(const kipp_model *model) { return model != NULL ? model->graph_replays : 0; }
+
+static int step_common(kipp_model *model, const kipp_step_item *items, size_t item_count, float *logits, size_t logits_capacity, uint32_t *best,
+                       kipp_error *error);
+
 int kipp_step(kipp_model *model, const kipp_step_item *items, size_t item_count, float *logits, size_t logits_capacity,
               kipp_error *error) {
+    return step_common(model, items, item_count, logits, logits_capacity, NULL, error);
+}
+
+int kipp_step_argmax(kipp_model *model, const kipp_step_item *items, size_t item_count, uint32_t *tokens, size_t token_capacity,
+                     kipp_error *error) {
+    uint32_t none; /* a step that wants nothing may come without room */
+    if (tokens == NULL && token_capacity != 0) return kipp_fail(error, KIPP_ERROR_ARGUMENT, "no room for the tokens");
+    return step_common(model, items, item_count, NULL, tokens != NULL ? token_capacity : 0, tokens != NULL ? tokens : &none, error);
+}
+
+/* `best` NULL: the wanted rows of logits go to `logits` (room for `capacity` floats); else the index of the largest logit of
+ * every wanted row goes to `best` (room for `capacity` indices), found where the path computes. */
+static int step_common(kipp_model *model, const kipp_step_item *items, size_t item_count, float *logits, size_t logits_capacity, uint32_t *best,
+                       kipp_error *error) {
     kipp_error_clear(error);
     if (model == NULL || (items == NULL && item_count != 0)) return kipp_fail(error, KIPP_ERROR_ARGUMENT, "model and items must be given");
     if (item_count == 0) return 0;
@@ -251,7 +356,13 @@ int kipp_step(kipp_model *model, const kipp_step_item *items, size_t item_count,
         goto unmark;
     }
     size_t floats;
-    if (kipp_mul_size(wanted, vocab, &floats) != 0 || floats > logits_capacity || (wanted != 0 && logits == NULL)) {
+    if (best != NULL) {
+        if (wanted > logits_capacity || wanted > INT32_MAX) {
+            kipp_fail(error, KIPP_ERROR_ARGUMENT, "%zu wanted places do not fit the %zu indices given", wanted, logits_capacity);
+            goto unmark;
+        }
+        floats = 0;
+    } else if (kipp_mul_size(wanted, vocab, &floats) != 0 || floats > logits_capacity || (wanted != 0 && logits == NULL)) {
         kipp_fail(error, KIPP_ERROR_ARGUMENT, "%zu wanted rows of %u logits do not fit the %zu floats given", wanted, vocab, logits_capacity);
         goto unmark;
     }
@@ -259,16 +370,28 @@ int kipp_step(kipp_model *model, const kipp_step_item *items, size_t item_count,
     for (; claimed < item_count; ++claimed) {
         if (kipp_cache_reserve_one(&model->cache, items[claimed].session, items[claimed].token_count, error) != 0) goto unclaim;
     }
-    kipp_scratch_reset(model->rt);
+    if (model->fail_forward_after >= 0 && model->fail_forward_after-- == 0) {
+        kipp_fail(error, KIPP_ERROR_INTERNAL, "the forward pass was told to fail (a test's switch)");
+        goto unclaim;
+    }
+    /* single tokens that all want their logits: the shape comes again and again, so it is recorded once and run as a graph */
+    bool single = model->rt->graph_begin != NULL && item_count <= KIPP_GRAPH_ROWS && wanted == item_count;
+    for (size_t i = 0; i < item_count && single; ++i) single = items[i].token_count == 1;
+    if (build_batch(model, items, item_count, single, error) != 0) goto unclaim; /* rounded whether or not steps are recorded: the same launches either way */
     float *device_logits = NULL;
-    if (build_batch(model, items, item_count, error) != 0) goto unclaim;
-    if (kipp_model_forward(model, &model->batch, &device_logits, error) != 0) goto unclaim;
+    int32_t *chosen = NULL;
+    if (run_step(model, single && !model->config.eager_steps, best != NULL, &device_logits, &chosen, error) != 0) goto unclaim;
     /* reading back (even nothing) waits for the step's work: what it wrote into the pages is there when it returns */
-    if (model->rt->download(model->rt, logits, device_logits, floats * sizeof(float), error) != 0) goto unclaim;
+    if (best != NULL && wanted != 0) {
+        if (model->rt->download(model->rt, best, chosen, wanted * sizeof(int32_t), error) != 0) goto unclaim;
+    } else if (model->rt->download(model->rt, logits, device_logits, floats * sizeof(float), error) != 0) {
+        goto unclaim;
+    }
     for (size_t i = 0; i < item_count; ++i) kipp_cache_commit(&model->cache, items[i].session, items[i].tokens, items[i].token_count);
     rc = 0;
     goto unmark;
 unclaim:
+    if (model->rt->after_failed_step != NULL) model->rt->after_failed_step(model->rt);
     for (size_t i = 0; i < claimed; ++i) kipp_cache_trim(&model->cache, items[i].session); /* the step did not happen: its pages go back */
 unmark:
     for (size_t i = 0; i < item_count; ++i) {

@@ -456,6 +456,29 @@ def test_the_c_command_line_matches_the_python_one(model_folders, tiny_configs, 
     assert subprocess.run([exe, "--help"], capture_output=True, text=True).stdout.startswith("usage: kipp")
 
 
+def test_step_argmax_is_the_argmax_of_step(model_folders, tiny_configs):
+    """kipp_step_argmax: the same step answered with one index a wanted place, the lowest among equal logits; room is checked."""
+    cfg = tiny_configs["a"]
+    with CModel(model_folders[("a", "float32")], path="cpu-fp32", page_tokens=4, kv_pool_pages=32, share_prefixes=False) as model:
+        a, b, c, d = (model.session() for _ in range(4))
+        pa, pb = H.random_tokens(1, 13, cfg["vocab_size"]), H.random_tokens(2, 7, cfg["vocab_size"])
+        rows = model.step([(a, pa, [3, 12]), (b, pb, [6])])
+        assert model.step_argmax([(c, pa, [3, 12]), (d, pb, [6])]) == [int(np.argmax(r)) for r in rows]
+        assert model.step_argmax([(c, [5], [])]) == []
+        with pytest.raises(KippError, match="do not fit"):
+            import ctypes
+            from kipp_amd import chost
+            items = (chost._StepItem * 1)()
+            t, tp = chost._u32([7, 8])
+            w, wp = chost._u32([0, 1])
+            items[0] = chost._StepItem(d.handle, tp, 2, wp, 2)
+            one = np.zeros(1, np.uint32)
+            error = chost._Error()
+            if model.lib.kipp_step_argmax(model.handle, items, 1, one.ctypes.data_as(chost._u32p), 1, ctypes.byref(error)) != 0:
+                chost._raise(model.lib, error)
+        assert d.length == 7                                          # the refused step left the session as it was
+
+
 # ---------------------------------------------------------------------------------------------- the C scheduler
 
 def _greedy(folder, prompt, n, stop=()):

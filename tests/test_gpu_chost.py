@@ -178,3 +178,51 @@ def test_c_command_line_on_the_gpu(model_folders, tiny_configs):
         for j, token in enumerate(generated):
             row = ref[len(prompt) - 1 + j]
             assert row[token] >= row.max() - margin
+
+
+@pytest.mark.parametrize("key", ["a", "b"])
+def test_c_host_recorded_steps_give_the_bits_of_steps_run_as_they_are(model_folders, tiny_configs, key):
+    """Steps of single tokens are recorded once their shape has come twice and run again from the recording.  Two models
+    walk the same schedule, one with recording switched off: three requests decode one token a step, prompts of a fourth and
+    fifth come in between (steps that are never recorded, and that use the same workspace), tables are scrambled on the
+    way, one request leaves.  Every row of every step has the same bits from both, many steps did run from recordings, and
+    the rows are the plain implementation's."""
+    from kipp_amd.chost import CModel
+    cfg = tiny_configs[key]
+    vocab = cfg["vocab_size"]
+    prompts = [H.random_tokens(60 + i, n, vocab) for i, n in enumerate([45, 21, 33])]
+    late = [H.random_tokens(70 + i, n, vocab) for i, n in enumerate([27, 40])]
+    models = [CModel(model_folders[(key, "bfloat16")], path="gpu-bf16", page_tokens=PAGE[key], kv_pool_pages=80, max_sessions=8,
+                     share_prefixes=False, eager_steps=eager) for eager in (True, False)]
+    got = [[], []]
+    for which, model in enumerate(models):
+        rows = got[which]
+        sessions = [model.session() for _ in prompts]
+        for s, p in zip(sessions, prompts):
+            rows.append(model.step([(s, p[:-12], [len(p) - 13])]))
+        extra = []
+        for step in range(12):
+            live = [(s, [p[len(p) - 12 + step]], [0]) for s, p in zip(sessions, prompts)]
+            if step >= 9:
+                live = live[:2]                                     # a shape of two rows from here on
+            rows.append(model.step(live))
+            if step in (3, 6):                                      # a prompt in between: a step that is not recorded
+                extra.append(model.session())
+                rows.append(model.step([(extra[-1], late[len(extra) - 1], [0, 5])]))
+            if step == 5:
+                for s in sessions:
+                    s.scramble()
+            if step == 7:
+                rows.append(model.step_argmax(live))                # the other kind of answer has a recording of its own
+                for s, _, _ in live:
+                    s.truncate(s.length - 1)
+    assert models[0].graph_replays == 0 and models[1].graph_replays >= 8
+    for a, b in zip(*got):
+        assert np.array_equal(np.asarray(a), np.asarray(b))
+    ref = [H.plain_logits(model_folders[(key, "bfloat16")], p) for p in prompts]
+    for step in range(9):
+        at = len(prompts) + step + (1 if step > 3 else 0) + (1 if step > 6 else 0) + (1 if step > 7 else 0)
+        for i, p in enumerate(prompts):
+            H.assert_close(got[1][at][i:i + 1], ref[i][len(p) - 12 + step:len(p) - 11 + step], H.NMSE_BF16["tiny"], f"recorded step {step}, request {i}")
+    for model in models:
+        model.close()

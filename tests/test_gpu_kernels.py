@@ -842,6 +842,16 @@ def test_gemm_skinny_adds_the_residual_and_prepares_the_norm(m, n, k, tiled):
         assert _rel(act.float().cpu().numpy(), plain.silu(ref) * ref) < 3e-5
 
 
+@pytest.mark.parametrize("n,k", [(20, 64), (16, 32), (151, 96), (2560, 4096), (38, 2560)])
+def test_tile_weight_by_the_kernel(n, k):
+    """The kernel that lays a matrix out for streaming (what the C host calls at load) against the torch form."""
+    ops = _ops()
+    w = torch.randn(n, k).bfloat16().to(DEV)
+    assert torch.equal(ops.tile_weight_device(w), ops.tile_weight(w))
+    if n % 2 == 0:
+        assert torch.equal(ops.tile_weight_device(w, gate_up=True), ops.tile_weight_pairs(w))
+
+
 def test_tile_weight_layout():
     ops = _ops()
     w = torch.arange(20 * 64, dtype=torch.float32).reshape(20, 64).bfloat16()          # 20 rows: the second tile is padded

@@ -63,6 +63,21 @@ def _cuttings_against_plain(folder, requests, refs, dtype, tol, what):
         del engine
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_benchmark_layer_sizes_through_the_c_host(real_folder, real_reference, dtype):
+    """The same four cuttings through kipp_step of the C host at the 4B layer sizes, against the same plain rows."""
+    from kipp_amd.chost import CModel
+    requests, refs = real_reference
+    tol = H.NMSE_F32 if dtype == "float32" else H.NMSE_BF16["real"]
+    for cut, maker in CUTTINGS:
+        steps = maker(requests)
+        with CModel(real_folder, path={"float32": "gpu-fp32", "bfloat16": "gpu-bf16"}[dtype], page_tokens=16,
+                    kv_pool_pages=H.peak_pages(requests, steps, 16), max_sessions=4, share_prefixes=False) as model:
+            got = H.replay_c(model, requests, steps, scramble_every=5 if cut == "mixed" else 0)
+            for rid in requests:
+                H.assert_close(got[rid], refs[rid], tol, f"C host, 4B sizes/{dtype}/{cut}/{rid}")
+
+
 # The layer sizes of the two larger shapes that the serving workloads run (Qwen3-8B: hidden 4096, SwiGLU 12288, 32 query
 # heads; Qwen3-32B: hidden 5120, SwiGLU 25600, 64 query heads, eight to a key/value head; both with a head of its own),
 # two layers each and a small vocabulary that is no power of two, so that the plain implementation stays affordable.
