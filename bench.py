@@ -391,7 +391,7 @@ def main():
     c_points = {}
     if not args.no_c_host:
         try:
-            c_points = c_host_points(config, sorted(set([1, args.batch]) & set(batches)) or [args.batch], args.prompt, args.steps, args.warmup)
+            c_points = c_host_points(config, sorted(set([1, args.batch, 64]) & set(batches)) or [args.batch], args.prompt, args.steps, args.warmup)
         except Exception as exc:
             log(f"the points through the C host failed and are left out: {type(exc).__name__}: {exc}")
 

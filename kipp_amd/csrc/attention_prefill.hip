@@ -620,8 +620,9 @@ __global__ void __launch_bounds__(THREADS, 2) attention_prefill_dma_kernel(
 __global__ void __launch_bounds__(KIPP_WAVE) attention_prefill_merge_kernel(
     const float* __restrict__ part_acc, const float* __restrict__ part_ml, bf16_t* __restrict__ out,
     const int32_t* __restrict__ merge_rows, const int32_t* __restrict__ merge_cuts, int n_q, int max_splits) {
-    const int head = blockIdx.x, lane = threadIdx.x;
-    const int row = merge_rows[blockIdx.y], cuts = merge_cuts[blockIdx.y];
+    // rows on the grid's x, which takes as many as a step has (y ends at 65,535)
+    const int head = blockIdx.y, lane = threadIdx.x;
+    const int row = merge_rows[blockIdx.x], cuts = merge_cuts[blockIdx.x];
     const size_t slot0 = ((size_t)row * n_q + head) * max_splits;
     float m = -INFINITY;
     for (int s = 0; s < cuts; ++s) m = fmaxf(m, part_ml[(slot0 + s) * 2]);
@@ -686,7 +687,7 @@ int kipp_attention_prefill(const void* q, const void* k_cache, const void* v_cac
                        positions, block_table, max_blocks, n_q, n_kv, page, scale_log2e, window, tile_rows, item_split,
                        split_keys, part_acc, part_ml, max_splits);
     if (split_keys > 0 && n_merge > 0)
-        hipLaunchKernelGGL(attention_prefill_merge_kernel, dim3(n_q, n_merge), dim3(KIPP_WAVE), 0, stream, part_acc, part_ml,
+        hipLaunchKernelGGL(attention_prefill_merge_kernel, dim3(n_merge, n_q), dim3(KIPP_WAVE), 0, stream, part_acc, part_ml,
                            (bf16_t*)out, merge_rows, merge_cuts, n_q, max_splits);
     return KIPP_LAUNCH_CHECK();
 }

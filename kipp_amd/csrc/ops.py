@@ -288,8 +288,15 @@ def attention_fast_ok(n_q: int, n_kv: int, page: int, max_blocks: int = 0) -> bo
 DECODE_SPLIT = 256      # keys per workgroup of the decode kernel (checked against the library at load)
 DECODE_SPLIT_MIN = 192  # ... and of its shortest splits (few sequences), which size the workspace
 PREFILL_ROWS = 128      # query rows per workgroup of the prefill kernel (64 or 32 where that fills the GPU better)
-COMPUTE_UNITS = 256     # of the MI355X
+COMPUTE_UNITS = 256     # of the MI355X (what the kernels' own plans assume); `compute_units()` asks the device
 PREFILL_MIN_CUT = 512   # fewest keys of a cut of the prefill kernel's keys (below, the merge costs more than the cut gains)
+
+
+def compute_units(device=None) -> int:
+    """Compute units of the device at hand (the MI355X has 256), for host-side plans that fill the GPU."""
+    if torch.cuda.is_available():
+        return int(torch.cuda.get_device_properties(device if device is not None else torch.cuda.current_device()).multi_processor_count)
+    return COMPUTE_UNITS
 
 
 def attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,

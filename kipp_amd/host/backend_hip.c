@@ -589,15 +589,33 @@ static int hip_linear(kipp_runtime *rt, const kipp_rows *rows_in, const kipp_wei
     return rc == 0 ? 0 : refused(error, "gemm_f32", rc);
 }
 
-/* Few rows against [gate; up]: both products and the activation in one kernel (and the norm's scale, if it was left to us). */
+/* Few rows against [gate; up]: both products and the activation in one kernel (and the norm's scale, if it was left to us).
+ * Up to 192 rows: the product streamed from the paired tiles, whose columns come out gate tile by gate tile, then the activation
+ * over those pairs. */
 static int hip_gated(kipp_runtime *rt, const kipp_rows *x, const kipp_weight *w, void *act, uint32_t m, bool *done, kipp_error *error) {
     hip_state *st = rt->state;
     *done = false;
-    if (!few_rows(rt, w, m) || w->n % 2 != 0 || (w->tiles != NULL && !w->pairs)) return 0;
+    if (rt->act_dtype != KIPP_BF16 || w->dtype != KIPP_BF16 || w->n % 2 != 0 || w->k % 8 != 0 || w->k < 32 || (w->tiles != NULL && !w->pairs)) return 0;
     const bool tiled = w->tiles != NULL;
-    int rc = st->gemm_skinny_swiglu(x->data, tiled ? w->tiles : w->data, act, (int)m, (int)w->n, (int)w->k, tiled ? 1 : 0, x->sumsq, x->sumsq_parts,
-                                    x->eps, st->stream);
-    if (rc != 0) return refused(error, "gemm_skinny_swiglu", rc);
+    const int M = (int)m, K = (int)w->k, inner = (int)(w->n / 2);
+    if (m <= FEW_ROWS) {
+        int rc = st->gemm_skinny_swiglu(x->data, tiled ? w->tiles : w->data, act, M, (int)w->n, K, tiled ? 1 : 0, x->sumsq, x->sumsq_parts, x->eps,
+                                        st->stream);
+        if (rc != 0) return refused(error, "gemm_skinny_swiglu", rc);
+        *done = true;
+        return 0;
+    }
+    if (!tiled || m > STAGED_ROWS) return 0;
+    kipp_rows finished = *x;
+    if (kipp_finish_rows(rt, &finished, m, w->k, error) != 0) return -1;
+    const int width = 16 * ((inner + 7) / 8); /* columns of the product from paired tiles: 16 for every 8 outputs */
+    int parts = st->rows_parts(M, width, K, 12);
+    float *y = parts >= 1 ? kipp_scratch(rt, (size_t)parts * m * (size_t)width * sizeof(float), error) : NULL;
+    if (y == NULL) return parts >= 1 ? -1 : refused(error, "gemm_rows (its cut)", parts);
+    int rc = st->gemm_rows(finished.data, w->tiles, y, M, width, K, 12, 1, st->stream);
+    if (rc != 0) return refused(error, "gemm_rows (paired tiles)", rc);
+    rc = st->swiglu(y, KIPP_F32, parts, act, rt->act_dtype, M, inner, 1, st->stream);
+    if (rc != 0) return refused(error, "swiglu (pairs)", rc);
     *done = true;
     return 0;
 }

@@ -49,7 +49,7 @@ class GatedMLP:
         act = rt.empty((rows, inner), rt.act_dtype)
         w = self.w_gate_up
         ours = w.dtype == x.dtype == torch.bfloat16 and rt.streams(rows, x.shape[1], 2 * inner)
-        if ours and rows <= rt.ops.SKINNY_BEST_ROWS:
+        if ours and rows <= rt.few_rows:
             # both products and the activation in one kernel (and the norm's scale, if it was left to us)
             scaled = isinstance(x, ScaledRows)
             rt.ops.gemm_skinny_swiglu(x.rows if scaled else x, w.rows, act, tiles=w.tiles,

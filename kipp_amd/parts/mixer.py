@@ -23,9 +23,6 @@ from ..cache.needs import KVNeed
 from .base import ParamSpec, build_part, register
 
 
-FUSED_DECODE_ROWS = 16      # up to this many single tokens take the fused decode attention ...
-FUSED_DECODE_KEYS = 8192    # ... while their contexts are shorter than this
-
 
 @register("mixer", "attention")
 class Attention:
@@ -115,7 +112,7 @@ class Attention:
         # than the rotary kernel it saves) and wherever the kernel that walks whole contexts or long ranges runs
         fused = fast and not batch.n_portions and batch.n_decode == n and pairing == "half" \
             and rt.ops.attention_decode_fused_ok(s.head_dim, rotary_dim, inv_freq is not None) \
-            and ((n <= FUSED_DECODE_ROWS and batch.max_decode_ctx < FUSED_DECODE_KEYS)
+            and ((n <= rt.fused_decode_rows and batch.max_decode_ctx < rt.fused_decode_keys)
                  or rt.ops.attention_decode_streams(n, s.num_kv_heads, s.head_dim, s.num_heads // s.num_kv_heads,
                                                     cache.page_size, batch.max_decode_ctx, s.window or 0))
         qkv = rt.linear(x, self.w_qkv, slabs=rt.ops.DECODE_FUSED_SLABS if fused else True)
@@ -173,8 +170,9 @@ class Attention:
             workgroups = len(tiles) * s.num_heads
             longest = max(last for _, _, last, _, _ in tiles) + 1
             split_keys = 0
-            if s.window is None and workgroups < 2 * ops.COMPUTE_UNITS:
-                want = -(-2 * ops.COMPUTE_UNITS // workgroups)
+            units = ops.compute_units(self.rt.device)
+            if s.window is None and workgroups < 2 * units:
+                want = -(-2 * units // workgroups)
                 split_keys = max(ops.PREFILL_MIN_CUT, -(-longest // want // 64) * 64)
                 if longest <= split_keys:
                     split_keys = 0

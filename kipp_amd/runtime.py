@@ -109,6 +109,13 @@ class Runtime:
         self.library_products = 0   # calls that went to the library (they stay out of HIP graphs)
         self.generic_attention_launches = 0   # bfloat16 attention that fell to the generic kernel (geometry the matrix-core kernels refuse)
         self.fuse_norms = True      # few rows: residual add and norm ride on the products around them
+        # Where one kernel hands over to the next, measured at the 4B shape on an MI355X; another width or device may
+        # move them, so they are the runtime's and can be set on it
+        self.few_rows = ops.SKINNY_BEST_ROWS        # rows up to which every wave reads its rows of x itself (the kernel with the fused ends)
+        self.staged_rows = ops.ROWS_BEST_ROWS       # rows up to which x is staged through LDS; beyond, the product built for hundreds of rows
+        self.fused_decode_rows = 16                 # single tokens up to which decode attention starts from the QKV product ...
+        self.fused_decode_keys = 8192               # ... while their contexts are shorter than this
+        self.fuse_norm_x_bytes = self.FUSE_NORM_X_BYTES
         # products of more than about 200 rows: True (the default): our own matrix-core kernel, in the fastest of the
         # cuts that give the planned cut's bits, so that every process computes the same bits; "auto": the fastest of
         # all our cuts and the library's product, timed once in a process at a shape's first use (another process
@@ -150,7 +157,7 @@ class Runtime:
     # -- matrix product ------------------------------------------------------
     def _few_rows(self, m: int, k: int, w) -> bool:
         """The product goes to the few-rows kernel (the one with the fused ends, which take up to 16 rows)."""
-        return w.dtype == torch.bfloat16 and self.ops.gemm_rows_ok(m, k) and m <= min(self.ops.SKINNY_BEST_ROWS, 16)
+        return w.dtype == torch.bfloat16 and self.ops.gemm_rows_ok(m, k) and m <= min(self.few_rows, 16)
 
     def settle(self, delta):
         """The tensor of a delta, launched now if it was deferred."""
@@ -178,7 +185,7 @@ class Runtime:
         # each against 4.6 saved; at 4 rows and for narrower weights the fused form wins).
         most = 1 if delta.slabs is False else (8 if delta.slabs is True else int(delta.slabs))
         n_out = w.shape[0]
-        if self.ops.gemm_skinny_parts(n_out, k, most) > 1 and ((n_out + 15) // 16) * rows * k * 2 > self.FUSE_NORM_X_BYTES:
+        if self.ops.gemm_skinny_parts(n_out, k, most) > 1 and ((n_out + 15) // 16) * rows * k * 2 > self.fuse_norm_x_bytes:
             return None
         rows_out, sumsq = self.ops.gemm_skinny(delta.x, w.rows, tiles=w.tiles, add_norm=(x, norm_weight))
         return ScaledRows(rows_out, sumsq, (w.shape[0] + 15) // 16, eps)
@@ -187,7 +194,7 @@ class Runtime:
     def streams(self, m: int, k: int, n: int) -> bool:
         """Whether a bfloat16 product of m rows takes the kernels that stream the weight once (few rows, or a
         shape the product for many rows does not take)."""
-        return self.ops.gemm_rows_ok(m, k) and (m <= self.ops.ROWS_BEST_ROWS or not self.ops.gemm_tiles_ok(m, k, n))
+        return self.ops.gemm_rows_ok(m, k) and (m <= self.staged_rows or not self.ops.gemm_tiles_ok(m, k, n))
 
     @staticmethod
     def _rows_class(m: int) -> int:
@@ -325,7 +332,7 @@ class Runtime:
         if self.streams(m, x.shape[1], n):
             # up to about 200 rows: our own kernels stream the weight once
             most = 0 if slabs is False else (None if slabs is True else int(slabs))
-            if m <= self.ops.SKINNY_BEST_ROWS:
+            if m <= self.few_rows:
                 y = self.ops.gemm_skinny(x, w, max_parts=1 if most == 0 else (most or 8), tiles=tiles, row_scale=row_scale)
             else:
                 y = self.ops.gemm_rows(x, w, max_parts=1 if most == 0 else (most or 12), tiles=tiles)

@@ -144,7 +144,7 @@ def test_split_products_keep_their_norm_kernels(real_folder, real_reference):
     for limit in (0, None):
         rt = Runtime("bfloat16")
         if limit is not None:
-            rt.FUSE_NORM_X_BYTES = limit
+            rt.fuse_norm_x_bytes = limit
         fused = {"yes": 0, "no": 0}
         inner = rt.product_add_norm
 
