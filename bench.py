@@ -234,47 +234,6 @@ def long_context_points(model, rt, cfg, numbers, args, weight_bytes, kv_per_toke
     return points, fracs
 
 
-def c_host_points(config, batches, prompt, steps, warmup):
-    """Decode through the C host (`kipp_amd/host`, no Python between the launches of a step): the same shape written to a
-    folder with random weights, prompts filled through kipp_step, then `steps` greedy steps timed on the host's clock
-    around kipp_step_argmax, everything a serving loop pays included (the batch's integers up, the tokens back)."""
-    import shutil
-    import tempfile
-
-    import numpy as np
-    from kipp_amd.chost import CModel
-    from kipp_amd.weights import write_random_model
-    tmp = tempfile.mkdtemp(prefix="kipp_bench_")
-    points = {}
-    try:
-        t0 = time.perf_counter()
-        folder = write_random_model(os.path.join(tmp, "model"), config, seed=0, dtype="bfloat16")
-        log(f"C host: wrote the model folder in {time.perf_counter() - t0:.1f} s")
-        most = max(batches)
-        per_request = -(-(prompt + steps + warmup + 16) // 16)
-        rng = np.random.default_rng(3)
-        with CModel(folder, path="gpu-bf16", page_tokens=16, kv_pool_pages=most * per_request, max_sessions=most,
-                    max_step_tokens=max(4096, prompt), share_prefixes=False) as model:
-            sessions = [model.session() for _ in range(most)]
-            for s in sessions:
-                model.step([(s, rng.integers(0, config["vocab_size"], prompt).tolist(), [])])
-            for b in batches:
-                tokens = [1 + i for i in range(b)]
-                for _ in range(warmup):
-                    tokens = model.step_argmax([(s, [t], [0]) for s, t in zip(sessions[:b], tokens)])
-                start = time.perf_counter()
-                for _ in range(steps):
-                    tokens = model.step_argmax([(s, [t], [0]) for s, t in zip(sessions[:b], tokens)])
-                took = time.perf_counter() - start
-                points[f"decode_b{b}_c_host"] = round(b * steps / took, 1)
-                log(f"C host: decode batch {b}: {took / steps * 1e3:.3f} ms/step, {b * steps / took:.0f} tok/s ({model.graph_replays} steps so far ran from recordings)")
-                for s in sessions[:b]:
-                    s.truncate(prompt)
-    finally:
-        shutil.rmtree(tmp, ignore_errors=True)
-    return points
-
-
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -391,7 +350,8 @@ def main():
     c_points = {}
     if not args.no_c_host:
         try:
-            c_points = c_host_points(config, sorted(set([1, args.batch, 64]) & set(batches)) or [args.batch], args.prompt, args.steps, args.warmup)
+            from kipp_amd.workloads import c_host_decode
+            c_points = c_host_decode(config, sorted(set([1, args.batch, 64]) & set(batches)) or [args.batch], args.prompt, args.steps, args.warmup)
         except Exception as exc:
             log(f"the points through the C host failed and are left out: {type(exc).__name__}: {exc}")
 

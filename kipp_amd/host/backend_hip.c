@@ -591,7 +591,7 @@ static int hip_linear(kipp_runtime *rt, const kipp_rows *rows_in, const kipp_wei
 
 /* Few rows against [gate; up]: both products and the activation in one kernel (and the norm's scale, if it was left to us).
  * Up to 192 rows: the product streamed from the paired tiles, whose columns come out gate tile by gate tile, then the activation
- * over those pairs. */
+ * over those pairs.  Beyond: the matrix-core kernel with the activation as its end. */
 static int hip_gated(kipp_runtime *rt, const kipp_rows *x, const kipp_weight *w, void *act, uint32_t m, bool *done, kipp_error *error) {
     hip_state *st = rt->state;
     *done = false;
@@ -605,8 +605,17 @@ static int hip_gated(kipp_runtime *rt, const kipp_rows *x, const kipp_weight *w,
         *done = true;
         return 0;
     }
-    if (!tiled || m > STAGED_ROWS) return 0;
     kipp_rows finished = *x;
+    if (m > STAGED_ROWS) {
+        /* many rows: both products and the activation in one pass of the matrix-core kernel (one rounding, after the activation) */
+        if (K % 32 != 0 || (uint64_t)(M > (int)w->n ? M : (int)w->n) * (uint64_t)K * 2 >= ((uint64_t)1 << 32)) return 0;
+        if (kipp_finish_rows(rt, &finished, m, w->k, error) != 0) return -1;
+        int rc = st->gemm_tiles(finished.data, w->data, act, M, (int)w->n, K, 1, 1, 0, st->stream);
+        if (rc != 0) return refused(error, "gemm_tiles (with the activation's end)", rc);
+        *done = true;
+        return 0;
+    }
+    if (!tiled) return 0;
     if (kipp_finish_rows(rt, &finished, m, w->k, error) != 0) return -1;
     const int width = 16 * ((inner + 7) / 8); /* columns of the product from paired tiles: 16 for every 8 outputs */
     int parts = st->rows_parts(M, width, K, 12);

@@ -8,6 +8,7 @@ portions, and requests that share a long beginning (paged prefix reuse).
     python -m kipp_amd.workloads mfma
     python -m kipp_amd.workloads products      [--shape qwen3-4b] [--rows 2048,512]
     python -m kipp_amd.workloads portion       [--shape qwen3-4b] [--rows 512] [--behind 4096]
+    python -m kipp_amd.workloads c-host        [--shape qwen3-4b] [--batches 8] [--steps 256]
 
 One JSON line: generated tokens a second over the whole run, prompt tokens a
 second, time to the first token, and what the cache reused.  `hbm` is no
@@ -18,11 +19,13 @@ operands that never leave the registers.
 `products` times the four matrix products of a layer for prompt portions, our
 kernel beside the library's; `portion` times a prompt portion behind a context
 that is already in the cache (what a step of chunked prefill costs).
+`c-host` decodes through the C host (`kipp_amd/host`), host work included.
 """
 from __future__ import annotations
 
 import argparse
 import json
+import os
 import sys
 import time
 
@@ -227,6 +230,47 @@ def portion(shape: str, layers, rows: int, behind: int, runs: int = 6) -> dict:
             "product_choices": {str(k): str(v) for k, v in engine.rt.prompt_product_choices.items()}}
 
 
+def c_host_decode(config, batches, prompt, steps, warmup):
+    """Decode through the C host (`kipp_amd/host`, no Python between the launches of a step): the same shape written to a
+    folder with random weights, prompts filled through kipp_step, then `steps` greedy steps timed on the host's clock
+    around kipp_step_argmax, everything a serving loop pays included (the batch's integers up, the tokens back)."""
+    import shutil
+    import tempfile
+
+    import numpy as np
+    from kipp_amd.chost import CModel
+    from kipp_amd.weights import write_random_model
+    tmp = tempfile.mkdtemp(prefix="kipp_bench_")
+    points = {}
+    try:
+        t0 = time.perf_counter()
+        folder = write_random_model(os.path.join(tmp, "model"), config, seed=0, dtype="bfloat16")
+        log(f"C host: wrote the model folder in {time.perf_counter() - t0:.1f} s")
+        most = max(batches)
+        per_request = -(-(prompt + steps + warmup + 16) // 16)
+        rng = np.random.default_rng(3)
+        with CModel(folder, path="gpu-bf16", page_tokens=16, kv_pool_pages=most * per_request, max_sessions=most,
+                    max_step_tokens=max(4096, prompt), share_prefixes=False) as model:
+            sessions = [model.session() for _ in range(most)]
+            for s in sessions:
+                model.step([(s, rng.integers(0, config["vocab_size"], prompt).tolist(), [])])
+            for b in batches:
+                tokens = [1 + i for i in range(b)]
+                for _ in range(warmup):
+                    tokens = model.step_argmax([(s, [t], [0]) for s, t in zip(sessions[:b], tokens)])
+                start = time.perf_counter()
+                for _ in range(steps):
+                    tokens = model.step_argmax([(s, [t], [0]) for s, t in zip(sessions[:b], tokens)])
+                took = time.perf_counter() - start
+                points[f"decode_b{b}_c_host"] = round(b * steps / took, 1)
+                log(f"C host: decode batch {b}: {took / steps * 1e3:.3f} ms/step, {b * steps / took:.0f} tok/s ({model.graph_replays} steps so far ran from recordings)")
+                for s in sessions[:b]:
+                    s.truncate(prompt)
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)
+    return points
+
+
 def main(argv=None) -> int:
     if argv is None:
         argv = sys.argv[1:]
@@ -244,6 +288,23 @@ def main(argv=None) -> int:
         rows = [int(r) for r in args.rows.split(",") if r]
         result = products(args.shape, rows) if argv[0] == "products" else portion(args.shape, args.layers, rows[0], args.behind)
         print(json.dumps(result), flush=True)
+        return 0
+    if argv and argv[0] == "c-host":
+        ap = argparse.ArgumentParser(prog="python -m kipp_amd.workloads c-host")
+        ap.add_argument("--shape", default="qwen3-4b")
+        ap.add_argument("--layers", type=int, default=0)
+        ap.add_argument("--batches", default="8")
+        ap.add_argument("--prompt", type=int, default=2048)
+        ap.add_argument("--steps", type=int, default=256)
+        ap.add_argument("--warmup", type=int, default=8)
+        args = ap.parse_args(argv[1:])
+        from .config import shape_config
+        config = shape_config(args.shape)
+        if args.layers:
+            config["num_hidden_layers"] = args.layers
+        points = c_host_decode(config, [int(b) for b in args.batches.split(",") if b], args.prompt, args.steps, args.warmup)
+        print(json.dumps({"workload": "c-host", "shape": args.shape, "layers": config["num_hidden_layers"], "prompt": args.prompt,
+                          "steps": args.steps, "tokens_per_s": points}), flush=True)
         return 0
     if argv and argv[0] == "mfma":
         import torch

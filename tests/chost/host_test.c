@@ -6,13 +6,16 @@
  * of the step function, the scheduler over few pages with cancellations and a failed step, and the sampler.
  * The GPU's table is not part of this build.
  *
- *   host_test MODEL_DIR [MODEL_DIR ...]      exit code 0 and a last line "ok <checks>" on success
+ *   host_test MODEL_DIR [MODEL_DIR ...] [--toy TOY_DIR]      exit code 0 and a last line "ok <checks>" on success
+ *
+ * TOY_DIR holds a model of an architecture that this file defines and registers itself (a mixer with state of its own).
  */
 #include <math.h>
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
 
+#include "backend.h"
 #include "internal.h"
 
 static int checks, failures;
@@ -409,14 +412,242 @@ static void test_scheduler(const char *folder) {
     CHECK(kipp_model_close(model, &error) == 0);
 }
 
+/* ------------------------------------------------------------------------------------------------------------------
+ * A toy architecture that exists in this file alone: every second layer mixes by the mean of what its session has seen
+ * so far, which it keeps as state of fixed size (no pages).  Registered from here, built, loaded and stepped by the
+ * library as it is: nothing in the library knows it. */
+typedef struct {
+    uint32_t hidden;
+    char prefix[KIPP_NAME];
+} toy_mean_spec;
+
+typedef struct {
+    toy_mean_spec spec;
+    kipp_runtime *rt;
+    kipp_weight w;
+} toy_mean_part;
+
+static int toy_mean_params(const void *spec_, kipp_param_list *out, kipp_error *error) {
+    const toy_mean_spec *spec = spec_;
+    return kipp_params_add(out, spec->prefix, "w.weight", 2, spec->hidden, spec->hidden, error);
+}
+
+static void *toy_mean_create(const void *spec, struct kipp_runtime *rt, kipp_error *error) {
+    toy_mean_part *part = calloc(1, sizeof(*part));
+    if (part == NULL) {
+        kipp_fail(error, KIPP_ERROR_MEMORY, "out of memory");
+        return NULL;
+    }
+    part->spec = *(const toy_mean_spec *)spec;
+    part->rt = rt;
+    return part;
+}
+
+static int toy_mean_load(void *part_, const kipp_tensor_file *tensors, void *context, kipp_error *error) {
+    toy_mean_part *part = part_;
+    char name[KIPP_NAME + 32];
+    (void)context;
+    snprintf(name, sizeof(name), "%sw.weight", part->spec.prefix);
+    const kipp_tensor *w = kipp_tensors_find(tensors, name);
+    if (w == NULL) return kipp_fail(error, KIPP_ERROR_FORMAT, "missing tensor '%s'", name);
+    return part->rt->place_matrix(part->rt, &w, 1, KIPP_LAYOUT_ROWS, &part->w, error);
+}
+
+static void toy_mean_destroy(void *part_) {
+    toy_mean_part *part = part_;
+    part->rt->free_weight(part->rt, &part->w);
+    free(part);
+}
+
+static void toy_mean_cache_need(const void *spec, kipp_kv_need *out) {
+    (void)spec;
+    memset(out, 0, sizeof(*out)); /* no pages */
+}
+
+static void toy_mean_state_need(const void *spec_, kipp_state_need *out) {
+    const toy_mean_spec *spec = spec_;
+    *out = (kipp_state_need){true, ((uint64_t)spec->hidden + 1) * sizeof(float)}; /* the sum of its inputs, and their number */
+}
+
+/* delta[t] = W mean(x[0..t] of the session); the sums live in the session's slot and go on from step to step */
+static int toy_mean_forward(void *part_, const kipp_rows *x, kipp_batch *batch, const kipp_cache_view *cache, void *state, kipp_delta *out,
+                            kipp_error *error) {
+    toy_mean_part *part = part_;
+    kipp_runtime *rt = part->rt;
+    const uint32_t h = part->spec.hidden;
+    (void)cache;
+    if (!rt->on_host || state == NULL) return kipp_fail(error, KIPP_ERROR_UNSUPPORTED, "the toy mixer computes on the host path only");
+    float *mean = kipp_scratch(rt, (size_t)batch->n_tokens * h * sizeof(float), error);
+    if (mean == NULL) return -1;
+    const float *rows = x->data;
+    for (uint32_t i = 0; i < batch->n_seqs; ++i) {
+        float *slot = (float *)state + (size_t)batch->slots[i] * (h + 1);
+        for (int32_t t = batch->q_start[i]; t < batch->q_start[i] + batch->q_len[i]; ++t) {
+            slot[h] += 1.0f;
+            for (uint32_t c = 0; c < h; ++c) {
+                slot[c] += rows[(size_t)t * h + c];
+                mean[(size_t)t * h + c] = slot[c] / slot[h];
+            }
+        }
+    }
+    return rt->linear(rt, &(kipp_rows){mean, NULL, 0, 0.0f}, &part->w, batch->n_tokens, 1, out, error);
+}
+
+static const kipp_mixer_fn toy_mean_fn = {toy_mean_cache_need, toy_mean_state_need, toy_mean_forward, false};
+static const kipp_part_kind toy_mean_kind = {"mixer", "toy_mean", sizeof(toy_mean_spec), toy_mean_params, toy_mean_create, toy_mean_load,
+                                             toy_mean_destroy, &toy_mean_fn};
+
+static uint32_t toy_uint(const kj_doc *doc, const char *key) {
+    const kj_node *v = kj_get(doc, kj_root(doc), key);
+    return v != NULL && v->type == KJ_NUMBER && v->is_integer && v->integer > 0 ? (uint32_t)v->integer : 0;
+}
+
+/* config.json of "ToyMeanForCausalLM": even layers attend (two heads, rotary), odd layers take the toy mixer */
+static int parse_toy(const kj_doc *doc, kipp_model_spec *spec, kipp_error *error) {
+    uint32_t vocab = toy_uint(doc, "vocab_size"), hidden = toy_uint(doc, "hidden_size"), inner = toy_uint(doc, "intermediate_size"),
+             layers = toy_uint(doc, "num_hidden_layers"), positions = toy_uint(doc, "max_position_embeddings");
+    if (vocab == 0 || hidden == 0 || inner == 0 || layers == 0 || positions == 0 || hidden % 2 != 0)
+        return kipp_fail(error, KIPP_ERROR_FORMAT, "config.json of the toy architecture lacks a size");
+    spec->hidden = hidden;
+    spec->vocab = vocab;
+    spec->max_position = positions;
+    spec->embedding = (kipp_embedding_spec){vocab, hidden, "model.embed_tokens."};
+    spec->head = (kipp_head_spec){vocab, hidden, true, "lm_head."};
+    spec->layers = calloc(layers, sizeof(kipp_layer_spec));
+    spec->order = calloc(layers, sizeof(kipp_layer_run));
+    kipp_rms_norm_spec *final_norm = calloc(1, sizeof(kipp_rms_norm_spec));
+    if (spec->layers == NULL || spec->order == NULL || final_norm == NULL) {
+        free(final_norm);
+        return kipp_fail(error, KIPP_ERROR_MEMORY, "out of memory");
+    }
+    spec->layer_count = spec->run_count = layers;
+    *final_norm = (kipp_rms_norm_spec){hidden, 1e-5f, "model.norm."};
+    spec->final_norm = final_norm;
+    snprintf(spec->final_norm_kind, sizeof(spec->final_norm_kind), "rms_norm");
+    for (uint32_t l = 0; l < layers; ++l) {
+        kipp_layer_spec *layer = &spec->layers[l];
+        kipp_rms_norm_spec norm = {hidden, 1e-5f, ""};
+        kipp_gated_mlp_spec mlp = {hidden, inner, ""};
+        snprintf(layer->block, sizeof(layer->block), "pre_norm");
+        layer->hidden = hidden;
+        snprintf(norm.prefix, sizeof(norm.prefix), "model.layers.%u.input_layernorm.", l);
+        if (kipp_spec_add_role(layer, "mixer_norm", "norm", "rms_norm", &norm, sizeof(norm), error) != 0) return -1;
+        if (l % 2 == 1) {
+            toy_mean_spec toy = {hidden, ""};
+            snprintf(toy.prefix, sizeof(toy.prefix), "model.layers.%u.mixer.", l);
+            if (kipp_spec_add_role(layer, "mixer", "mixer", "toy_mean", &toy, sizeof(toy), error) != 0) return -1;
+        } else {
+            kipp_attention_spec attn;
+            memset(&attn, 0, sizeof(attn));
+            attn.hidden = hidden;
+            attn.n_heads = 2;
+            attn.n_kv_heads = 1;
+            attn.head_dim = hidden / 2;
+            snprintf(attn.position_kind, sizeof(attn.position_kind), "rope");
+            attn.rope = (kipp_rope_spec){hidden / 2, 10000.0, hidden / 2, 0};
+            snprintf(attn.prefix, sizeof(attn.prefix), "model.layers.%u.self_attn.", l);
+            if (kipp_spec_add_role(layer, "mixer", "mixer", "attention", &attn, sizeof(attn), error) != 0) return -1;
+        }
+        snprintf(norm.prefix, sizeof(norm.prefix), "model.layers.%u.post_attention_layernorm.", l);
+        if (kipp_spec_add_role(layer, "ffn_norm", "norm", "rms_norm", &norm, sizeof(norm), error) != 0) return -1;
+        snprintf(mlp.prefix, sizeof(mlp.prefix), "model.layers.%u.mlp.", l);
+        if (kipp_spec_add_role(layer, "ffn", "feed_forward", "gated_mlp", &mlp, sizeof(mlp), error) != 0) return -1;
+        spec->order[l] = (kipp_layer_run){l, -1};
+    }
+    spec->info.block_count = layers;
+    spec->info.embedding_length = hidden;
+    spec->info.vocab_size = vocab;
+    spec->info.context_length = positions;
+    spec->info.tied_embeddings = true;
+    return 0;
+}
+
+/* The toy model's folder (written by the caller: config.json with architectures ["ToyMeanForCausalLM"], tensors by the names
+ * the parts declare): whole prompts, portions beside another session's, and a slot taken again all give the same bits; what
+ * the state cannot do is refused. */
+static void test_toy_architecture(const char *folder) {
+    kipp_model *model = NULL;
+    kipp_error error;
+    kipp_model_open_config config;
+    memset(&config, 0, sizeof(config));
+    config.path = KIPP_PATH_CPU_FP32;
+    config.page_tokens = 4;
+    config.kv_pool_pages = 24;
+    config.max_sessions = 2;
+    config.share_prefixes = 1; /* asked for, and switched off by the model itself: state cannot be adopted */
+    CHECK(kipp_model_open_ex(folder, &config, &model, &error) != 0 && error.code == KIPP_ERROR_UNSUPPORTED); /* nobody knows the architecture yet */
+    CHECK(kipp_register_part(&toy_mean_kind) == 0 && kipp_register_architecture("ToyMeanForCausalLM", parse_toy) == 0);
+    if (kipp_model_open_ex(folder, &config, &model, &error) != 0) {
+        fprintf(stderr, "cannot open the toy model %s: %s\n", folder, error.message);
+        CHECK(0);
+        return;
+    }
+    kipp_model_info info;
+    CHECK(kipp_model_get_info(model, &info) == 0 && info.cache_groups == 1 && strcmp(info.architecture, "ToyMeanForCausalLM") == 0);
+    const uint32_t vocab = info.vocab_size, n = 21;
+    uint32_t tokens[32], other[32], want[32];
+    for (uint32_t i = 0; i < 32; ++i) {
+        tokens[i] = rnd(vocab);
+        other[i] = rnd(vocab);
+        want[i] = i;
+    }
+    float *whole = malloc((size_t)n * vocab * sizeof(float)), *cut = malloc((size_t)n * vocab * sizeof(float)),
+          *spare = malloc((size_t)32 * vocab * sizeof(float));
+    kipp_session *a = NULL, *b = NULL, *c = NULL;
+    CHECK(kipp_session_create(model, 0, &a, &error) == 0);
+    kipp_step_item item = {a, tokens, n, want, n};
+    CHECK(kipp_step(model, &item, 1, whole, (size_t)n * vocab, &error) == 0);
+    uint32_t matched = 7;
+    CHECK(kipp_session_truncate(a, 5, &error) != 0 && error.code == KIPP_ERROR_UNSUPPORTED);                    /* state cannot be rolled back */
+    CHECK(kipp_session_match_prefix(a, tokens, n, &matched, &error) != 0 && error.code == KIPP_ERROR_UNSUPPORTED); /* nor adopted */
+    kipp_session_destroy(a);
+    /* portions of b beside portions of c: each session's sums stay its own */
+    CHECK(kipp_session_create(model, 0, &b, &error) == 0 && kipp_session_create(model, 0, &c, &error) == 0);
+    static const uint32_t portions[] = {5, 1, 1, 7, 2, 5};
+    uint32_t fed = 0, fed_c = 0;
+    for (size_t p = 0; p < sizeof(portions) / sizeof(portions[0]); ++p) {
+        uint32_t take_c = 1 + rnd(3);
+        kipp_step_item items[2] = {{c, other + fed_c, take_c, want, 0}, {b, tokens + fed, portions[p], want, portions[p]}};
+        CHECK(kipp_step(model, items, 2, spare, (size_t)32 * vocab, &error) == 0);
+        memcpy(cut + (size_t)fed * vocab, spare, (size_t)portions[p] * vocab * sizeof(float));
+        fed += portions[p];
+        fed_c += take_c;
+    }
+    CHECK(fed == n && same_bits(whole, cut, (size_t)n * vocab));
+    /* the slot that b leaves is c's successor's: it starts from zero again */
+    kipp_session_destroy(b);
+    CHECK(kipp_session_create(model, 0, &b, &error) == 0);
+    item = (kipp_step_item){b, tokens, n, want, n};
+    CHECK(kipp_step(model, &item, 1, cut, (size_t)n * vocab, &error) == 0 && same_bits(whole, cut, (size_t)n * vocab));
+    /* the mixer does count: the same last token behind another beginning has other logits */
+    kipp_session_destroy(b);
+    CHECK(kipp_session_create(model, 0, &b, &error) == 0);
+    other[n - 1] = tokens[n - 1];
+    item = (kipp_step_item){b, other, n, want + n - 1, 1};
+    CHECK(kipp_step(model, &item, 1, spare, vocab, &error) == 0 && !same_bits(spare, whole + (size_t)(n - 1) * vocab, vocab));
+    kipp_session_destroy(b);
+    kipp_session_destroy(c);
+    CHECK(kipp_model_close(model, &error) == 0);
+    free(whole);
+    free(cut);
+    free(spare);
+}
+
 int main(int argc, char **argv) {
     test_json();
     test_sizes();
     test_pool();
     test_sampler();
     test_scalar_operations();
-    for (int i = 1; i < argc; ++i) test_model(argv[i]);
-    for (int i = 1; i < argc; ++i) test_scheduler(argv[i]);
+    int models = argc;
+    for (int i = 1; i < argc; ++i) {
+        if (strcmp(argv[i], "--toy") == 0 && i + 1 < argc) {
+            test_toy_architecture(argv[i + 1]);
+            models = i;
+        }
+    }
+    for (int i = 1; i < models; ++i) test_model(argv[i]);
+    for (int i = 1; i < models; ++i) test_scheduler(argv[i]);
     if (failures != 0) {
         fprintf(stderr, "%d of %d checks failed\n", failures, checks);
         return 1;

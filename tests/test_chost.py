@@ -361,16 +361,49 @@ def test_the_c_sampler_is_the_python_sampler(tiny_configs):
     assert sample(np.array([1.0, 3.0, 3.0, 2.0], np.float32)) == 1               # greedy: the lowest index among equals, no generator
 
 
+def _toy_mean_folder(folder):
+    """A model folder of the architecture that tests/chost/host_test.c defines and registers itself: attention in the even
+    layers, a mixer that keeps a running mean as per-session state in the odd ones.  Tensors by the names its parts declare."""
+    import json
+    import torch
+    from kipp_amd.weights.safetensors_io import write_file
+    hidden, inner, layers, vocab = 24, 40, 4, 61
+    os.makedirs(folder, exist_ok=True)
+    with open(os.path.join(folder, "config.json"), "w", encoding="utf-8") as f:
+        json.dump({"architectures": ["ToyMeanForCausalLM"], "vocab_size": vocab, "hidden_size": hidden, "intermediate_size": inner,
+                   "num_hidden_layers": layers, "max_position_embeddings": 64}, f)
+    gen = torch.Generator().manual_seed(5)
+    normal = lambda *shape: torch.randn(*shape, generator=gen) * 0.3
+    tensors = {"model.embed_tokens.weight": normal(vocab, hidden), "model.norm.weight": 1 + 0.1 * normal(hidden)}
+    for l in range(layers):
+        p = f"model.layers.{l}."
+        tensors[p + "input_layernorm.weight"] = 1 + 0.1 * normal(hidden)
+        tensors[p + "post_attention_layernorm.weight"] = 1 + 0.1 * normal(hidden)
+        for name, shape in (("gate_proj", (inner, hidden)), ("up_proj", (inner, hidden)), ("down_proj", (hidden, inner))):
+            tensors[p + f"mlp.{name}.weight"] = normal(*shape)
+        if l % 2 == 1:
+            tensors[p + "mixer.w.weight"] = normal(hidden, hidden)
+        else:
+            for name, rows in (("q_proj", hidden), ("k_proj", hidden // 2), ("v_proj", hidden // 2)):
+                tensors[p + f"self_attn.{name}.weight"] = normal(rows, hidden)
+            tensors[p + "self_attn.o_proj.weight"] = normal(hidden, hidden)
+    write_file(os.path.join(folder, "model.safetensors"), tensors)
+    return folder
+
+
 def test_host_logic_under_the_sanitizers(model_folders, tmp_path):
     """tests/chost/host_test.c, linked with the host's sources (without the GPU's table) under AddressSanitizer and
     UndefinedBehaviorSanitizer: JSON, checked sizes, pool and cache manager under random orders, both tiny models
-    opened and stepped on the scalar path under several cuttings with scrambled tables, error paths, the sampler."""
+    opened and stepped on the scalar path under several cuttings with scrambled tables, error paths, the sampler; and an
+    architecture that the test program defines itself (a mixer with per-session state of fixed size), registered, built,
+    loaded and stepped by the library as it is."""
     import subprocess
     from kipp_amd.host import build
     here = os.path.dirname(os.path.abspath(__file__))
     exe = build.test_program(os.path.join(here, "chost", "host_test.c"), str(tmp_path / "host_test"))
     env = dict(os.environ, ASAN_OPTIONS="detect_leaks=1:abort_on_error=0", UBSAN_OPTIONS="print_stacktrace=1:halt_on_error=1")
-    proc = subprocess.run([exe, model_folders[("a", "float32")], model_folders[("b", "float32")], model_folders[("b", "bfloat16")]],
+    toy = _toy_mean_folder(str(tmp_path / "toy"))
+    proc = subprocess.run([exe, model_folders[("a", "float32")], model_folders[("b", "float32")], model_folders[("b", "bfloat16")], "--toy", toy],
                           capture_output=True, text=True, timeout=300, env=env)
     assert proc.returncode == 0, proc.stdout[-2000:] + proc.stderr[-6000:]
     assert proc.stdout.strip().splitlines()[-1].startswith("ok ")

@@ -76,6 +76,13 @@ def test_benchmark_layer_sizes_through_the_c_host(real_folder, real_reference, d
             got = H.replay_c(model, requests, steps, scramble_every=5 if cut == "mixed" else 0)
             for rid in requests:
                 H.assert_close(got[rid], refs[rid], tol, f"C host, 4B sizes/{dtype}/{cut}/{rid}")
+    # the three prompts in one step: 257 rows, which go to the products built for hundreds of rows (the activation as their end)
+    together = [([(rid, len(toks)) for rid, toks in requests.items()], list(requests))]
+    with CModel(real_folder, path={"float32": "gpu-fp32", "bfloat16": "gpu-bf16"}[dtype], page_tokens=16,
+                kv_pool_pages=H.peak_pages(requests, together, 16), max_sessions=4, share_prefixes=False) as model:
+        got = H.replay_c(model, requests, together)
+        for rid in requests:
+            H.assert_close(got[rid], refs[rid], tol, f"C host, 4B sizes/{dtype}/together/{rid}")
 
 
 # The layer sizes of the two larger shapes that the serving workloads run (Qwen3-8B: hidden 4096, SwiGLU 12288, 32 query
