@@ -120,8 +120,10 @@ __global__ void __launch_bounds__(256) rmsnorm_rows_kernel(float* __restrict__ x
 
 // out[t, :] = rows[t, :] * rsqrt(sum_p sumsq[t, p] / width + eps), sumsq in rows of `stride`: the normalized rows, for a consumer that
 // does not apply the scale itself (rows = bfloat16(x * norm weight), sumsq = partial sums of x^2).
+// `steps_major`: `rows` come as [width / 32][rows][32] (what the few-rows products write for each other); out is [rows][width].
 __global__ void __launch_bounds__(256) scale_rows_kernel(const bf16_t* __restrict__ rows, const float* __restrict__ sumsq,
-                                                         bf16_t* __restrict__ out, int width, int parts, int stride, float eps) {
+                                                         bf16_t* __restrict__ out, int width, int parts, int stride, float eps,
+                                                         int steps_major) {
     __shared__ float scratch[16];
     float a = 0.0f;
     for (int p = threadIdx.x; p < parts; p += 256) a += sumsq[(size_t)blockIdx.x * stride + p];
@@ -129,7 +131,8 @@ __global__ void __launch_bounds__(256) scale_rows_kernel(const bf16_t* __restric
     const float scale = 1.0f / sqrtf(a / (float)width + eps);
     for (int i = threadIdx.x; i < width; i += 256) {
         const size_t at = (size_t)blockIdx.x * width + i;
-        out[at] = f32_to_bf16(bf16_to_f32(rows[at]) * scale);
+        const size_t from = steps_major ? ((size_t)(i >> 5) * gridDim.x + blockIdx.x) * 32 + (i & 31) : at;
+        out[at] = f32_to_bf16(bf16_to_f32(rows[from]) * scale);
     }
 }
 
@@ -290,11 +293,11 @@ int kipp_rmsnorm(float* x, const void* delta, int delta_dtype, int parts, const 
 }
 
 int kipp_scale_rows(const void* rows, const float* sumsq, void* out, int n_rows, int width, int parts, int stride, float eps,
-                    hipStream_t stream) {
+                    int steps_major, hipStream_t stream) {
     if (n_rows <= 0 || width <= 0) return 0;
-    if (parts <= 0 || stride < parts) return -1;
+    if (parts <= 0 || stride < parts || (steps_major && (width & 31))) return -1;
     hipLaunchKernelGGL(scale_rows_kernel, dim3(n_rows), dim3(256), 0, stream, (const bf16_t*)rows, sumsq, (bf16_t*)out, width,
-                       parts, stride, eps);
+                       parts, stride, eps, steps_major);
     return KIPP_LAUNCH_CHECK();
 }
 

@@ -66,14 +66,20 @@ struct AddNorm {                // residual == nullptr: none
     bf16_t* rows_out;           // [M, N] = bfloat16(residual * norm_w)
     float* sumsq_out;           // [M, stride]: ceil(N / 16) sums a row, stride as in RowScale
     int stride;
+    int steps_major;            // rows_out as [N / 32][M][32] (N a multiple of 32)
 };
+
+// Where element (row, column) of bfloat16 rows lies: [row][width], or [column / 32][row][32] for `rows` rows.
+__device__ __forceinline__ size_t rows_at(int row, int col, int width, int rows, int steps_major) {
+    return steps_major ? ((size_t)(col >> 5) * rows + row) * 32 + (col & 31) : (size_t)row * width + col;
+}
 
 #define SCALE_LOADS 10          // 16-byte loads of partial sums a lane has in flight: 160 sums of a row, what 2,560 columns give
 
 template <int MT, bool SWIGLU, int KW, int DEPTH, bool TILED>
 __global__ void __launch_bounds__(THREADS) gemm_skinny_kernel(
     const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, float* Y, bf16_t* __restrict__ act,
-    int M, int N, int K, RowScale rs, AddNorm an) {
+    int M, int N, int K, RowScale rs, AddNorm an, int x_major, int act_major) {
     constexpr bool PAIRS = SWIGLU && TILED;          // gate and up rows share a tile
     constexpr int NT = SWIGLU && !TILED ? 2 : 1;
     constexpr int TW = WAVES / KW;                   // row tiles of a workgroup
@@ -110,7 +116,8 @@ __global__ void __launch_bounds__(THREADS) gemm_skinny_kernel(
     }
     const bf16_t* x_row[MT];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) x_row[mt] = X + (size_t)min(16 * mt + l16, M - 1) * K + 8 * h;
+    for (int mt = 0; mt < MT; ++mt) x_row[mt] = X + (size_t)min(16 * mt + l16, M - 1) * (x_major ? 32 : K) + 8 * h;
+    const int x_step = x_major ? 32 * M : 32;        // from one step's columns of a row to the next step's
 
     // the partial sums of the rows' scales, asked for first, all at once, and added once the first
     // weights are on their way (up to 16 rows): lane group h takes every fourth run of four sums of token l % 16.
@@ -164,7 +171,7 @@ __global__ void __launch_bounds__(THREADS) gemm_skinny_kernel(
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) wf[u][nt].u = *(const u32x4*)(w_row[nt] + (TILED ? 512 * step : k));
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) xf[u][mt].u = *(const u32x4*)(x_row[mt] + k);
+        for (int mt = 0; mt < MT; ++mt) xf[u][mt].u = *(const u32x4*)(x_row[mt] + (size_t)step * x_step);
     };
     auto multiply = [&](int u) {
 #pragma unroll
@@ -304,14 +311,13 @@ __global__ void __launch_bounds__(THREADS) gemm_skinny_kernel(
                 uint2 packed;
                 packed.x = (uint32_t)f32_to_bf16(x[0] * norm_w[0]) | ((uint32_t)f32_to_bf16(x[1] * norm_w[1]) << 16);
                 packed.y = (uint32_t)f32_to_bf16(x[2] * norm_w[2]) | ((uint32_t)f32_to_bf16(x[3] * norm_w[3]) << 16);
-                *(uint2*)(an.rows_out + at) = packed;
+                *(uint2*)(an.rows_out + rows_at(token, n, N, M, an.steps_major)) = packed;   // four columns of one run of 32
             } else if (token < M) {
 #pragma unroll
                 for (int v = 0; v < 4; ++v) {
                     if (n + v < N) {
-                        const size_t at = (size_t)token * N + n + v;
-                        an.residual[at] = x[v];
-                        an.rows_out[at] = f32_to_bf16(x[v] * norm_w[v]);
+                        an.residual[(size_t)token * N + n + v] = x[v];
+                        an.rows_out[rows_at(token, n + v, N, M, an.steps_major)] = f32_to_bf16(x[v] * norm_w[v]);
                     }
                 }
             }
@@ -331,7 +337,7 @@ __global__ void __launch_bounds__(THREADS) gemm_skinny_kernel(
             for (int v = 0; v < 4; ++v) {
                 const float g = sum[0][mt][v], up = __shfl_xor(g, 32, KIPP_WAVE);
                 const int o = out0 + 4 * h + v;
-                if (h < 2 && token < M && o < inner) act[(size_t)token * inner + o] = f32_to_bf16(g / (1.0f + expf(-g)) * up);
+                if (h < 2 && token < M && o < inner) act[rows_at(token, o, inner, M, act_major)] = f32_to_bf16(g / (1.0f + expf(-g)) * up);
             }
             continue;
         }
@@ -341,7 +347,7 @@ __global__ void __launch_bounds__(THREADS) gemm_skinny_kernel(
             for (int v = 0; v < 4; ++v) {
                 if (n + v < inner) {
                     const float g = sum[0][mt][v], up = sum[NT - 1][mt][v];
-                    act[(size_t)token * inner + n + v] = f32_to_bf16(g / (1.0f + expf(-g)) * up);
+                    act[rows_at(token, n + v, inner, M, act_major)] = f32_to_bf16(g / (1.0f + expf(-g)) * up);
                 }
             }
         } else {
@@ -359,7 +365,7 @@ __global__ void __launch_bounds__(THREADS) gemm_skinny_kernel(
 
 template <bool SWIGLU, int KW, bool TILED>
 static int launch_kw(const bf16_t* X, const bf16_t* W, float* Y, bf16_t* act, int M, int N, int K, int parts,
-                     RowScale rs, AddNorm an, hipStream_t stream) {
+                     RowScale rs, AddNorm an, int x_major, int act_major, hipStream_t stream) {
     const int inner = SWIGLU ? N / 2 : N;
     const int tiles = SWIGLU && TILED ? (inner + 7) / 8 : (inner + 15) / 16;
     constexpr int TW = WAVES / KW;
@@ -368,7 +374,8 @@ static int launch_kw(const bf16_t* X, const bf16_t* W, float* Y, bf16_t* act, in
     if (rs.sumsq != nullptr && M > 16) return -1;
     const int mt = (M + 15) / 16;
 #define KIPP_SK(MT, D) \
-    hipLaunchKernelGGL((gemm_skinny_kernel<MT, SWIGLU, KW, D, TILED>), grid, block, 0, stream, X, W, Y, act, M, N, K, rs, an)
+    hipLaunchKernelGGL((gemm_skinny_kernel<MT, SWIGLU, KW, D, TILED>), grid, block, 0, stream, X, W, Y, act, M, N, K, rs, an, x_major, \
+                       act_major)
     switch (mt) {
         case 1:
             // fewer workgroups than compute units: what is in flight is what the busy ones ask for, so they ask for twice as much
@@ -386,11 +393,14 @@ static int launch_kw(const bf16_t* X, const bf16_t* W, float* Y, bf16_t* act, in
 
 template <bool SWIGLU>
 static int launch(const bf16_t* X, const bf16_t* W, float* Y, bf16_t* act, int M, int N, int K, int parts, int kw,
-                  int tiled, RowScale rs, AddNorm an, hipStream_t stream) {
+                  int tiled, RowScale rs, AddNorm an, int x_major, int act_major, hipStream_t stream) {
     if (tiled && (K & 31)) return -1;
+    if (x_major && (K & 31)) return -1;              // whole runs of 32 columns only
+    if (an.residual != nullptr && an.steps_major && (N & 31)) return -1;
+    if (act_major && ((N / 2) & 31)) return -1;
 #define KIPP_KW(KW)                                                                          \
-    return tiled ? launch_kw<SWIGLU, KW, true>(X, W, Y, act, M, N, K, parts, rs, an, stream)         \
-                 : launch_kw<SWIGLU, KW, false>(X, W, Y, act, M, N, K, parts, rs, an, stream)
+    return tiled ? launch_kw<SWIGLU, KW, true>(X, W, Y, act, M, N, K, parts, rs, an, x_major, act_major, stream)         \
+                 : launch_kw<SWIGLU, KW, false>(X, W, Y, act, M, N, K, parts, rs, an, x_major, act_major, stream)
     switch (kw) {
         case 1: KIPP_KW(1);
         case 2: KIPP_KW(2);
@@ -453,37 +463,40 @@ int kipp_gemm_skinny_sumsq_stride(int N) { return sumsq_stride((N + 15) / 16); }
 // streaming layout (K a multiple of 32), else [N, K] rows.
 // `sumsq` [M, sumsq_parts rounded up to a multiple of 4] (or null; M <= 16 then): every row of the product is multiplied by
 // rsqrt(sum of the row's sumsq / K + eps).
+// `x_steps_major`: X comes as [K / 32][M][32] (K a multiple of 32); `rows_out_steps_major`: rows_out is written as
+// [N / 32][M][32] (N a multiple of 32).
 // `residual` [M, N] (or null): the product is added to it in place (Y is not written and there is
 // one part), `rows_out` [M, N] = bfloat16(residual * norm_w) and `sumsq_out`
 // [M, kipp_gemm_skinny_sumsq_stride(N)] = every row's sums of squares of the new residual over each 16 columns
 // (M <= 16 with a residual).
 int kipp_gemm_skinny(const void* X, const void* W, float* Y, int M, int N, int K, int max_parts, int tiled,
                      const float* sumsq, int sumsq_parts, float eps, float* residual, const float* norm_w, void* rows_out,
-                     float* sumsq_out, hipStream_t stream) {
+                     float* sumsq_out, int x_steps_major, int rows_out_steps_major, hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
     if (M > 64 || K <= 0 || (K & 7) || max_parts <= 0) return -1;
     if (sumsq != nullptr && (sumsq_parts <= 0 || M > 16)) return -1;
     if (residual != nullptr && (norm_w == nullptr || rows_out == nullptr || sumsq_out == nullptr || M > 16)) return -1;
     int kw, parts;
     plan((N + 15) / 16, K, residual != nullptr ? 1 : max_parts, &kw, &parts);
-    AddNorm an = {residual, norm_w, (bf16_t*)rows_out, sumsq_out, sumsq_stride((N + 15) / 16)};
+    AddNorm an = {residual, norm_w, (bf16_t*)rows_out, sumsq_out, sumsq_stride((N + 15) / 16), rows_out_steps_major};
     return launch<false>((const bf16_t*)X, (const bf16_t*)W, Y, nullptr, M, N, K, parts, kw, tiled,
-                         row_scale_of(sumsq, sumsq_parts, K, eps), an, stream);
+                         row_scale_of(sumsq, sumsq_parts, K, eps), an, x_steps_major, 0, stream);
 }
 
 // W: [2 I, K] = [gate; up] (tiled: tiles of 8 gate rows over the 8 matching up rows); act: bfloat16 [M, I].
 // The contraction is cut the same way from both layouts, so both give the same bits.
-// `sumsq`, `sumsq_parts`, `eps`: as above.
+// `sumsq`, `sumsq_parts`, `eps`, `x_steps_major`: as above; `act_steps_major`: act is written as [I / 32][M][32] (I a multiple of 32).
 int kipp_gemm_skinny_swiglu(const void* X, const void* W, void* act, int M, int two_inner, int K, int tiled,
-                            const float* sumsq, int sumsq_parts, float eps, hipStream_t stream) {
+                            const float* sumsq, int sumsq_parts, float eps, int x_steps_major, int act_steps_major,
+                            hipStream_t stream) {
     if (M <= 0 || two_inner <= 0) return 0;
     if (M > 64 || K <= 0 || (K & 7) || (two_inner & 1)) return -1;
     if (sumsq != nullptr && (sumsq_parts <= 0 || M > 16)) return -1;
     int kw, parts;
     plan((two_inner / 2 + 7) / 8, K, 1, &kw, &parts);
-    AddNorm none = {nullptr, nullptr, nullptr, nullptr, 4};
+    AddNorm none = {nullptr, nullptr, nullptr, nullptr, 4, 0};
     return launch<true>((const bf16_t*)X, (const bf16_t*)W, nullptr, (bf16_t*)act, M, two_inner, K, 1, kw, tiled,
-                        row_scale_of(sumsq, sumsq_parts, K, eps), none, stream);
+                        row_scale_of(sumsq, sumsq_parts, K, eps), none, x_steps_major, act_steps_major, stream);
 }
 
 }  // extern "C"

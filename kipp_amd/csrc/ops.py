@@ -576,8 +576,22 @@ def gemm_skinny_parts(n: int, k: int, max_parts: int) -> int:
     return build.library("gemm_skinny").kipp_gemm_skinny_parts(int(n), int(k), int(max_parts))
 
 
+def steps_major(rows: torch.Tensor) -> torch.Tensor:
+    """bfloat16 rows [M, K] (K a multiple of 32) as [K / 32][M][32], the order the few-rows products may read and write
+    their rows in (`x_steps_major`, `out_steps_major`): what a wave reads of x in one step is then one run of memory."""
+    m, k = rows.shape
+    _need(k % 32 == 0, "steps_major: whole runs of 32 columns")
+    return rows.view(m, k // 32, 32).transpose(0, 1).contiguous().view(m, k)
+
+
+def from_steps_major(rows: torch.Tensor) -> torch.Tensor:
+    """The inverse of `steps_major`: [K / 32][M][32] (held as a tensor of shape [M, K]) back to [M, K]."""
+    m, k = rows.shape
+    return rows.view(k // 32, m, 32).transpose(0, 1).contiguous().view(m, k)
+
+
 def gemm_skinny(x: torch.Tensor, w: torch.Tensor, max_parts: int = 1, tiles: torch.Tensor = None,
-                row_scale=None, add_norm=None):
+                row_scale=None, add_norm=None, x_steps_major: bool = False, out_steps_major: bool = False):
     """float32 [parts, M, N] whose sum over parts is x . w^T, for M <= 64 rows of
     bfloat16 x against bfloat16 w [N, K].  parts <= max_parts is chosen from the
     shape (1 when the weight has many rows).  With `tiles` (tile_weight(w)) the
@@ -590,13 +604,17 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, max_parts: int = 1, tiles: tor
     (in one part) is added to `residual` in place by the kernel itself and the
     call returns (rows, sumsq) instead: rows = bfloat16(residual * norm_weight)
     and sumsq [M, P rounded up to 4] with P = ceil(N / 16) sums a row: (sumsq, P, eps)
-    is the `row_scale` of the next product."""
+    is the `row_scale` of the next product.
+    `x_steps_major`: x holds its values as `steps_major` orders them; `out_steps_major`: so do the rows that
+    `add_norm` returns (both need the width in question to be a multiple of 32)."""
     _dev(x, w)
     m, k = x.shape
     n = w.shape[0]
     _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm_skinny: bfloat16 operands")
     _need(w.shape == (n, k), "gemm_skinny: shapes do not match")
     _need(gemm_skinny_ok(m, k), "gemm_skinny: at most 64 rows, K a multiple of 8 and at least 32")
+    _need(not x_steps_major or k % 32 == 0, "gemm_skinny: rows in steps-major order need K a multiple of 32")
+    _need(not out_steps_major or (add_norm is not None and n % 32 == 0), "gemm_skinny: steps-major rows come from add_norm, N a multiple of 32")
     lib = build.library("gemm_skinny")
     tiled = _tiles_ok(tiles, n, k, "gemm_skinny")
     sumsq, sumsq_parts, eps = _row_scale_args(row_scale, m, "gemm_skinny")
@@ -614,22 +632,26 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, max_parts: int = 1, tiles: tor
         sumsq_out = torch.empty((m, ((n + 15) // 16 + 3) // 4 * 4), dtype=torch.float32, device=x.device)
     fn = _fn("gemm_skinny", "kipp_gemm_skinny",
              [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_int, _c_float,
-              _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr])
+              _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr])
     _check(fn(_ptr(x), _ptr(tiles if tiled else w), _ptr(out), m, n, k, int(max_parts), tiled, sumsq, sumsq_parts, eps,
-              _ptr(residual), _ptr(norm_w), _ptr(rows), _ptr(sumsq_out), _stream()), "gemm_skinny")
+              _ptr(residual), _ptr(norm_w), _ptr(rows), _ptr(sumsq_out), int(bool(x_steps_major)), int(bool(out_steps_major)),
+              _stream()), "gemm_skinny")
     return out if add_norm is None else (rows, sumsq_out)
 
 
-def scale_rows(rows: torch.Tensor, sumsq: torch.Tensor, parts: int, eps: float, out: torch.Tensor) -> torch.Tensor:
+def scale_rows(rows: torch.Tensor, sumsq: torch.Tensor, parts: int, eps: float, out: torch.Tensor,
+               steps_major: bool = False) -> torch.Tensor:
     """out[t] = rows[t] * rsqrt(sum(sumsq[t, :parts]) / width + eps), bfloat16: the rows of an RMS norm
-    from what `gemm_skinny(..., add_norm=...)` returns, for a consumer that does not take `row_scale`."""
+    from what `gemm_skinny(..., add_norm=...)` returns, for a consumer that does not take `row_scale`
+    (`steps_major`: `rows` were written in that order; `out` is [M, width] rows all the same)."""
     _dev(rows, sumsq, out)
     m, width = rows.shape
     _need(rows.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and out.shape == rows.shape
           and sumsq.dtype == torch.float32 and sumsq.dim() == 2 and sumsq.shape[0] == m and 0 < parts <= sumsq.shape[1]
           and sumsq.is_contiguous(), "scale_rows: shapes or types differ")
-    fn = _fn("elementwise", "kipp_scale_rows", [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_float, _c_ptr])
-    _check(fn(_ptr(rows), _ptr(sumsq), _ptr(out), m, width, int(parts), sumsq.shape[1], float(eps), _stream()), "scale_rows")
+    fn = _fn("elementwise", "kipp_scale_rows", [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_ptr])
+    _check(fn(_ptr(rows), _ptr(sumsq), _ptr(out), m, width, int(parts), sumsq.shape[1], float(eps), int(bool(steps_major)), _stream()),
+           "scale_rows")
     return out
 
 
@@ -659,10 +681,11 @@ def gemm_rows(x: torch.Tensor, w: torch.Tensor, max_parts: int = 1, tiles: torch
 
 
 def gemm_skinny_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor, tiles: torch.Tensor = None,
-                       row_scale=None) -> torch.Tensor:
+                       row_scale=None, x_steps_major: bool = False, out_steps_major: bool = False) -> torch.Tensor:
     """out[M, I] (bfloat16) = silu(x . w_gate^T) * (x . w_up^T), w_gate_up = [gate; up] of [2 I, K];
     `tiles` = tile_weight_pairs(w_gate_up).  The same bits from both layouts.
-    `row_scale`: as in `gemm_skinny` (both products are scaled before the activation)."""
+    `row_scale`, `x_steps_major`: as in `gemm_skinny` (both products are scaled before the activation);
+    `out_steps_major`: `out` is written in the order of `steps_major` (I a multiple of 32)."""
     _dev(x, w_gate_up, out)
     m, k = x.shape
     two_inner = w_gate_up.shape[0]
@@ -671,12 +694,14 @@ def gemm_skinny_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tens
     _need(w_gate_up.shape == (two_inner, k) and two_inner % 2 == 0 and out.shape == (m, two_inner // 2),
           "gemm_skinny_swiglu: shapes do not match")
     _need(gemm_skinny_ok(m, k), "gemm_skinny_swiglu: at most 64 rows, K a multiple of 8 and at least 32")
+    _need((not x_steps_major or k % 32 == 0) and (not out_steps_major or (two_inner // 2) % 32 == 0),
+          "gemm_skinny_swiglu: rows in steps-major order need their width to be a multiple of 32")
     tiled = _tiles_ok(tiles, pairs_width(two_inner // 2), k, "gemm_skinny_swiglu")
     sumsq, sumsq_parts, eps = _row_scale_args(row_scale, m, "gemm_skinny_swiglu")
     fn = _fn("gemm_skinny", "kipp_gemm_skinny_swiglu",
-             [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_int, _c_float, _c_ptr])
+             [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_int, _c_float, _c_int, _c_int, _c_ptr])
     _check(fn(_ptr(x), _ptr(tiles if tiled else w_gate_up), _ptr(out), m, two_inner, k, tiled, sumsq, sumsq_parts, eps,
-              _stream()), "gemm_skinny_swiglu")
+              int(bool(x_steps_major)), int(bool(out_steps_major)), _stream()), "gemm_skinny_swiglu")
     return out
 
 

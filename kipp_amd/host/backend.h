@@ -62,8 +62,11 @@ struct kipp_runtime {
     /* out = in's rows with their scale applied (only a table that leaves scales has it) */
     int (*scale_rows)(kipp_runtime *rt, const kipp_rows *in, void *out, uint32_t rows, uint32_t width, kipp_error *error);
     /* Optional (NULL: none).  act[t, i] = silu(x . gate_i) * (x . up_i) for w = [gate; up], in one kernel where the table has
-     * one for this shape: *done says whether it ran (else the caller takes linear and swiglu). */
-    int (*gated)(kipp_runtime *rt, const kipp_rows *x, const kipp_weight *w_gate_up, void *act, uint32_t m, bool *done, kipp_error *error);
+     * one for this shape: *done says whether it ran (else the caller takes linear and swiglu).  act->data is given; `reader` is
+     * the matrix that act is multiplied with next (the table may write act in the order that product reads fastest, and says so
+     * in act->steps_major). */
+    int (*gated)(kipp_runtime *rt, const kipp_rows *x, const kipp_weight *w_gate_up, const kipp_weight *reader, kipp_rows *act, uint32_t m,
+                 bool *done, kipp_error *error);
     /* out[t, i] = silu(gate_up[t, i]) * gate_up[t, inner + i] in the activation type */
     int (*swiglu)(kipp_runtime *rt, const kipp_delta *gate_up, void *out, uint32_t rows, uint32_t inner, kipp_error *error);
     /* The rotation of a step's positions in the form this table's `qk_norm_rope_kv` rotates from, made once for every layer

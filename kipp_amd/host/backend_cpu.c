@@ -137,14 +137,14 @@ static int cpu_argmax(kipp_runtime *rt, const float *logits, int32_t *out, uint3
 
 static int cpu_linear(kipp_runtime *rt, const kipp_rows *rows_in, const kipp_weight *w, uint32_t m, int max_parts, kipp_delta *out, kipp_error *error) {
     (void)max_parts;
-    if (rows_in->sumsq != NULL) return kipp_fail(error, KIPP_ERROR_INTERNAL, "rows without their scale on the host path");
+    if (rows_in->sumsq != NULL || rows_in->steps_major) return kipp_fail(error, KIPP_ERROR_INTERNAL, "rows without their scale on the host path");
     const void *x = rows_in->data;
     size_t count;
     if (kipp_mul_size(m, w->n, &count) != 0 || count > SIZE_MAX / 4) return kipp_fail(error, KIPP_ERROR_RANGE, "a product's size overflows");
     float *y = kipp_scratch(rt, count * sizeof(float), error);
     if (y == NULL) return -1;
     for (uint32_t r = 0; r < m; ++r) ref_matvec(w->data, REF_F32, (const float *)x + (size_t)r * w->k, y + (size_t)r * w->n, w->n, w->k);
-    *out = (kipp_delta){y, 1, NULL, NULL, 0, 0};
+    *out = (kipp_delta){y, 1, NULL, NULL, 0, 0, false};
     return 0;
 }
 

@@ -48,12 +48,12 @@ typedef int (*fn_int_void)(void);
 typedef int (*fn_gemm_f32)(const float *, const void *, int, float *, int, int, int, hipStream_t);
 typedef int (*fn_skinny_parts)(int, int, int);
 typedef int (*fn_gemm_skinny)(const void *, const void *, float *, int, int, int, int, int, const float *, int, float, float *, const float *,
-                              void *, float *, hipStream_t);
+                              void *, float *, int, int, hipStream_t);
 typedef int (*fn_rows_parts)(int, int, int, int);
 typedef int (*fn_gemm_rows)(const void *, const void *, float *, int, int, int, int, int, hipStream_t);
-typedef int (*fn_skinny_swiglu)(const void *, const void *, void *, int, int, int, int, const float *, int, float, hipStream_t);
+typedef int (*fn_skinny_swiglu)(const void *, const void *, void *, int, int, int, int, const float *, int, float, int, int, hipStream_t);
 typedef int (*fn_int_int)(int);
-typedef int (*fn_scale_rows)(const void *, const float *, void *, int, int, int, int, float, hipStream_t);
+typedef int (*fn_scale_rows)(const void *, const float *, void *, int, int, int, int, float, int, hipStream_t);
 typedef int (*fn_tile_weight)(const void *, void *, int, int, int, hipStream_t);
 typedef int (*fn_argmax)(const float *, int32_t *, int, int, float *, hipStream_t);
 typedef int (*fn_attention_decode_fused)(const float *, int, int, const float *, const float *, float, const float *, const float *, int, void *,
@@ -103,6 +103,7 @@ typedef struct {
     fn_argmax argmax;
     fn_int_int argmax_scratch_floats;
     bool fuse;             /* few rows: residual add and norm ride on the products around them, decode attention starts from the QKV product */
+    bool steps_major;      /* rows that one few-rows product writes for the next: in the order that product reads fastest */
     bool merge_in_kernel;  /* decode attention: the splits of a head are merged by the last of their workgroups to finish */
     int32_t *arrivals;     /* its counts of finished splits, zero between launches */
     size_t arrivals_count;
@@ -470,7 +471,8 @@ static bool hip_defers(kipp_runtime *rt, const kipp_rows *x, const kipp_weight *
 
 static int hip_scale_rows(kipp_runtime *rt, const kipp_rows *in, void *out, uint32_t rows, uint32_t width, kipp_error *error) {
     hip_state *st = rt->state;
-    int rc = st->scale_rows(in->data, in->sumsq, out, (int)rows, (int)width, in->sumsq_parts, (in->sumsq_parts + 3) / 4 * 4, in->eps, st->stream);
+    int rc = st->scale_rows(in->data, in->sumsq, out, (int)rows, (int)width, in->sumsq_parts, (in->sumsq_parts + 3) / 4 * 4, in->eps,
+                            in->steps_major ? 1 : 0, st->stream);
     return rc == 0 ? 0 : refused(error, "scale_rows", rc);
 }
 
@@ -492,11 +494,13 @@ static int hip_rmsnorm(kipp_runtime *rt, float *x, kipp_delta *delta, const floa
             void *unscaled = may_leave_scale ? out->data : kipp_scratch(rt, (size_t)rows * width * 2, error);
             if (sumsq == NULL || unscaled == NULL) return -1;
             const bool tiled = w->tiles != NULL;
+            /* the rows go to a few-rows product (or to the kernel that finishes them): in the order those read fastest */
+            const bool major = st->steps_major && N % 32 == 0 && rows > 1;
             int rc = st->gemm_skinny(delta->x, tiled ? w->tiles : w->data, NULL, (int)rows, N, K, 1, tiled ? 1 : 0, NULL, 0, 0.0f, x, weight, unscaled,
-                                     sumsq, st->stream);
+                                     sumsq, delta->x_steps_major ? 1 : 0, major ? 1 : 0, st->stream);
             if (rc != 0) return refused(error, "gemm_skinny (with the residual's end)", rc);
-            *delta = (kipp_delta){NULL, 0, NULL, NULL, 0, 0};
-            const kipp_rows left = {unscaled, sumsq, (N + 15) / 16, eps};
+            *delta = (kipp_delta){NULL, 0, NULL, NULL, 0, 0, false};
+            const kipp_rows left = {unscaled, sumsq, (N + 15) / 16, eps, major};
             if (may_leave_scale) {
                 *out = left;
                 return 0;
@@ -531,19 +535,20 @@ static int hip_linear(kipp_runtime *rt, const kipp_rows *rows_in, const kipp_wei
     if (max_parts < 1) max_parts = 1;
     kipp_rows finished = *rows_in;
     if (finished.sumsq != NULL && !few_rows(rt, w, m) && kipp_finish_rows(rt, &finished, m, w->k, error) != 0) return -1;
+    if (finished.steps_major && !few_rows(rt, w, m)) return kipp_fail(error, KIPP_ERROR_INTERNAL, "rows in steps-major order for a product that does not read it");
     const void *x = finished.data;
     /* paired tiles give the columns in another order: only the product that ends in the activation reads them */
     const bool tiled = w->tiles != NULL && !w->pairs;
     const void *streamed = tiled ? w->tiles : w->data;
     int rc;
-#define KIPP_DELTA(y, parts) ((kipp_delta){(y), (parts), NULL, NULL, 0, 0})
+#define KIPP_DELTA(y, parts) ((kipp_delta){(y), (parts), NULL, NULL, 0, 0, false})
     if (w->dtype == KIPP_BF16 && rt->act_dtype == KIPP_BF16 && K % 8 == 0 && K >= 32) {
         if (M <= FEW_ROWS) {
             int most = max_parts > 8 ? 8 : max_parts, parts = st->skinny_parts(N, K, most);
             float *y = parts >= 1 ? kipp_scratch(rt, (size_t)parts * count * 4, error) : NULL;
             if (y == NULL) return parts >= 1 ? -1 : refused(error, "gemm_skinny (its cut)", parts);
             rc = st->gemm_skinny(x, streamed, y, M, N, K, most, tiled ? 1 : 0, finished.sumsq, finished.sumsq_parts, finished.eps, NULL, NULL, NULL,
-                                 NULL, st->stream);
+                                 NULL, finished.steps_major ? 1 : 0, 0, st->stream);
             *out = KIPP_DELTA(y, parts);
             return rc == 0 ? 0 : refused(error, "gemm_skinny", rc);
         }
@@ -592,16 +597,20 @@ static int hip_linear(kipp_runtime *rt, const kipp_rows *rows_in, const kipp_wei
 /* Few rows against [gate; up]: both products and the activation in one kernel (and the norm's scale, if it was left to us).
  * Up to 192 rows: the product streamed from the paired tiles, whose columns come out gate tile by gate tile, then the activation
  * over those pairs.  Beyond: the matrix-core kernel with the activation as its end. */
-static int hip_gated(kipp_runtime *rt, const kipp_rows *x, const kipp_weight *w, void *act, uint32_t m, bool *done, kipp_error *error) {
+static int hip_gated(kipp_runtime *rt, const kipp_rows *x, const kipp_weight *w, const kipp_weight *reader, kipp_rows *act, uint32_t m, bool *done,
+                     kipp_error *error) {
     hip_state *st = rt->state;
     *done = false;
     if (rt->act_dtype != KIPP_BF16 || w->dtype != KIPP_BF16 || w->n % 2 != 0 || w->k % 8 != 0 || w->k < 32 || (w->tiles != NULL && !w->pairs)) return 0;
     const bool tiled = w->tiles != NULL;
     const int M = (int)m, K = (int)w->k, inner = (int)(w->n / 2);
     if (m <= FEW_ROWS) {
-        int rc = st->gemm_skinny_swiglu(x->data, tiled ? w->tiles : w->data, act, M, (int)w->n, K, tiled ? 1 : 0, x->sumsq, x->sumsq_parts, x->eps,
-                                        st->stream);
+        /* the activation goes to `reader` alone: in the order its product reads fastest, if that is a few-rows product too */
+        const bool major = st->steps_major && reader != NULL && few_rows(rt, reader, m) && !reader->pairs && inner % 32 == 0 && m > 1;
+        int rc = st->gemm_skinny_swiglu(x->data, tiled ? w->tiles : w->data, act->data, M, (int)w->n, K, tiled ? 1 : 0, x->sumsq, x->sumsq_parts, x->eps,
+                                        x->steps_major ? 1 : 0, major ? 1 : 0, st->stream);
         if (rc != 0) return refused(error, "gemm_skinny_swiglu", rc);
+        act->steps_major = major;
         *done = true;
         return 0;
     }
@@ -610,7 +619,7 @@ static int hip_gated(kipp_runtime *rt, const kipp_rows *x, const kipp_weight *w,
         /* many rows: both products and the activation in one pass of the matrix-core kernel (one rounding, after the activation) */
         if (K % 32 != 0 || (uint64_t)(M > (int)w->n ? M : (int)w->n) * (uint64_t)K * 2 >= ((uint64_t)1 << 32)) return 0;
         if (kipp_finish_rows(rt, &finished, m, w->k, error) != 0) return -1;
-        int rc = st->gemm_tiles(finished.data, w->data, act, M, (int)w->n, K, 1, 1, 0, st->stream);
+        int rc = st->gemm_tiles(finished.data, w->data, act->data, M, (int)w->n, K, 1, 1, 0, st->stream);
         if (rc != 0) return refused(error, "gemm_tiles (with the activation's end)", rc);
         *done = true;
         return 0;
@@ -623,7 +632,7 @@ static int hip_gated(kipp_runtime *rt, const kipp_rows *x, const kipp_weight *w,
     if (y == NULL) return parts >= 1 ? -1 : refused(error, "gemm_rows (its cut)", parts);
     int rc = st->gemm_rows(finished.data, w->tiles, y, M, width, K, 12, 1, st->stream);
     if (rc != 0) return refused(error, "gemm_rows (paired tiles)", rc);
-    rc = st->swiglu(y, KIPP_F32, parts, act, rt->act_dtype, M, inner, 1, st->stream);
+    rc = st->swiglu(y, KIPP_F32, parts, act->data, rt->act_dtype, M, inner, 1, st->stream);
     if (rc != 0) return refused(error, "swiglu (pairs)", rc);
     *done = true;
     return 0;
@@ -935,6 +944,8 @@ kipp_runtime *kipp_runtime_hip(kipp_path path, int device, const char *kernel_di
     const char *fuse = getenv("KIPP_AMD_FUSE"), *merge = getenv("KIPP_AMD_DECODE_MERGE");
     st->fuse = path == KIPP_PATH_GPU_BF16 && !(fuse != NULL && strcmp(fuse, "0") == 0);
     st->merge_in_kernel = !(merge != NULL && strcmp(merge, "launch") == 0);
+    const char *major = getenv("KIPP_AMD_STEPS_MAJOR");
+    st->steps_major = st->fuse && !(major != NULL && strcmp(major, "0") == 0);
     if (kernel_dir != NULL && kernel_dir[0] != '\0') snprintf(st->kernel_dir, sizeof(st->kernel_dir), "%s", kernel_dir);
     else default_kernel_dir(st->kernel_dir, sizeof(st->kernel_dir));
     if ((code = hipSetDevice(device)) != hipSuccess || (code = hipStreamCreate(&st->stream)) != hipSuccess) {

@@ -231,12 +231,14 @@ typedef enum { KIPP_LAYOUT_ROWS = 0, KIPP_LAYOUT_STREAM, KIPP_LAYOUT_STREAM_PAIR
 /* Rows in the activation type.  With `sumsq` they still lack the scale of their RMS norm: data = rows * norm weight, and
  * row t's scale is rsqrt(sum(sumsq[t, :sumsq_parts]) / width + eps), sumsq in rows of sumsq_parts rounded up to 4.  A row's
  * scale commutes with a product over the row, so a product may apply it to its own rows; kipp_finish_rows gives any other
- * consumer the finished rows. */
+ * consumer the finished rows.  Rows that one few-rows product writes for the next may be in steps-major order (below):
+ * only those products read it, and whoever makes such rows knows that their reader is one. */
 typedef struct {
     void *data;
     const float *sumsq;
     int sumsq_parts;
     float eps;
+    bool steps_major; /* data is [width / 32][rows][32], the order the few-rows products read fastest, not [rows][width] */
 } kipp_rows;
 
 /* A delta of the residual stream: float32 [parts, rows, width] whose sum over parts is the value; or (parts 0, w given) the
@@ -249,6 +251,7 @@ typedef struct {
     const kipp_weight *w;
     uint32_t m;
     int max_parts;
+    bool x_steps_major;
 } kipp_delta;
 
 static inline bool kipp_delta_any(const kipp_delta *delta) { return delta != NULL && (delta->parts > 0 || delta->w != NULL); }

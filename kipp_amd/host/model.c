@@ -291,7 +291,7 @@ int kipp_model_forward(kipp_model *model, kipp_batch *batch, float **out_logits,
     batch->decode_workspace[0] = NULL;
     float *x = kipp_scratch(rt, (size_t)n * spec->hidden * sizeof(float), error);
     if (x == NULL || kipp_embedding_forward(model->embedding.part, batch->tokens, x, n, error) != 0) return -1;
-    kipp_delta pending = {NULL, 0, NULL, NULL, 0, 0};
+    kipp_delta pending = {NULL, 0, NULL, NULL, 0, 0, false};
     for (uint32_t run = 0; run < spec->run_count; ++run) {
         const kipp_built_part *block = &model->blocks[spec->order[run].layer];
         kipp_cache_view view;
@@ -301,7 +301,7 @@ int kipp_model_forward(kipp_model *model, kipp_batch *batch, float **out_logits,
     }
     if (batch->n_want == 0) return 0; /* a portion of a prompt whose logits nobody needs: no final norm, no head */
     const kipp_norm_fn *final_norm = model->final_norm.kind->fn;
-    kipp_rows normed = {kipp_scratch(rt, (size_t)batch->n_want * spec->hidden * kipp_dtype_bytes(rt->act_dtype), error), NULL, 0, 0.0f};
+    kipp_rows normed = {kipp_scratch(rt, (size_t)batch->n_want * spec->hidden * kipp_dtype_bytes(rt->act_dtype), error), NULL, 0, 0.0f, false};
     if (normed.data == NULL) return -1;
     if (batch->want_every_row) {
         /* every row in order (a step of single tokens): no gather, the last delta is added inside the norm, and the head's

@@ -349,7 +349,7 @@ static int attention_forward(void *part_, const kipp_rows *x, kipp_batch *batch,
         if (rt->decode_attention(rt, x, &part->w_qkv, cache, mixed, batch, &geometry, part->q_norm, part->k_norm, eps, rotation, rotary_dim,
                                  interleaved, &done, error) != 0)
             return -1;
-        if (done) return kipp_linear_defer(rt, &(kipp_rows){mixed, NULL, 0, 0.0f}, &part->w_o, n, 8, out, error);
+        if (done) return kipp_linear_defer(rt, &(kipp_rows){mixed, NULL, 0, 0.0f, false}, &part->w_o, n, 8, out, error);
     }
     kipp_delta qkv;
     if (rt->linear(rt, x, &part->w_qkv, n, 4, &qkv, error) != 0) return -1;
@@ -358,7 +358,7 @@ static int attention_forward(void *part_, const kipp_rows *x, kipp_batch *batch,
     if (rt->qk_norm_rope_kv(rt, &qkv, q, cache, batch, &geometry, part->q_norm, part->k_norm, eps, rotation, rotary_dim, interleaved, error) != 0)
         return -1;
     if (rt->attention(rt, q, cache, mixed, batch, &geometry, error) != 0) return -1;
-    return kipp_linear_defer(rt, &(kipp_rows){mixed, NULL, 0, 0.0f}, &part->w_o, n, 8, out, error);
+    return kipp_linear_defer(rt, &(kipp_rows){mixed, NULL, 0, 0.0f, false}, &part->w_o, n, 8, out, error);
 }
 
 static const kipp_mixer_fn attention_fn = {attention_cache_need, no_state, attention_forward, true};
@@ -415,15 +415,16 @@ static int gated_mlp_forward(void *part_, const kipp_rows *x, kipp_batch *batch,
     gated_mlp_part *part = part_;
     kipp_runtime *rt = part->rt;
     const uint32_t n = batch->n_tokens;
-    void *act = kipp_scratch(rt, (size_t)n * part->spec.inner * kipp_dtype_bytes(rt->act_dtype), error);
-    if (act == NULL) return -1;
+    kipp_rows act = {kipp_scratch(rt, (size_t)n * part->spec.inner * kipp_dtype_bytes(rt->act_dtype), error), NULL, 0, 0.0f, false};
+    if (act.data == NULL) return -1;
     bool done = false;
-    if (rt->gated != NULL && rt->gated(rt, x, &part->w_gate_up, act, n, &done, error) != 0) return -1; /* both products and the activation in one kernel */
+    /* both products and the activation in one kernel where the table has one */
+    if (rt->gated != NULL && rt->gated(rt, x, &part->w_gate_up, &part->w_down, &act, n, &done, error) != 0) return -1;
     if (!done) {
         kipp_delta gate_up;
-        if (rt->linear(rt, x, &part->w_gate_up, n, 8, &gate_up, error) != 0 || rt->swiglu(rt, &gate_up, act, n, part->spec.inner, error) != 0) return -1;
+        if (rt->linear(rt, x, &part->w_gate_up, n, 8, &gate_up, error) != 0 || rt->swiglu(rt, &gate_up, act.data, n, part->spec.inner, error) != 0) return -1;
     }
-    return kipp_linear_defer(rt, &(kipp_rows){act, NULL, 0, 0.0f}, &part->w_down, n, 8, out, error);
+    return kipp_linear_defer(rt, &act, &part->w_down, n, 8, out, error);
 }
 
 static const kipp_ffn_fn gated_mlp_fn = {gated_mlp_forward, true};
@@ -516,13 +517,13 @@ static int pre_norm_forward(void *block_, float *x, kipp_delta *pending, kipp_ba
     const kipp_mixer_fn *mixer = block->mixer.kind->fn;
     const kipp_ffn_fn *ffn = block->ffn.kind->fn;
     /* a part that does not take rows without their scale gets finished ones: the norm is told, and what it leaves all the same is finished here */
-    kipp_rows h = {kipp_scratch(rt, bytes, error), NULL, 0, 0.0f};
+    kipp_rows h = {kipp_scratch(rt, bytes, error), NULL, 0, 0.0f, false};
     if (h.data == NULL) return -1;
     if (norm1->forward(block->mixer_norm.part, x, kipp_delta_any(pending) ? pending : NULL, &h, n, mixer->takes_scaled_rows, error) != 0) return -1;
     if (!mixer->takes_scaled_rows && kipp_finish_rows(rt, &h, n, block->hidden, error) != 0) return -1;
     kipp_delta delta;
     if (mixer->forward(block->mixer.part, &h, batch, cache, state, &delta, error) != 0) return -1;
-    kipp_rows h2 = {kipp_scratch(rt, bytes, error), NULL, 0, 0.0f};
+    kipp_rows h2 = {kipp_scratch(rt, bytes, error), NULL, 0, 0.0f, false};
     if (h2.data == NULL) return -1;
     if (norm2->forward(block->ffn_norm.part, x, &delta, &h2, n, ffn->takes_scaled_rows, error) != 0) return -1;
     if (!ffn->takes_scaled_rows && kipp_finish_rows(rt, &h2, n, block->hidden, error) != 0) return -1;

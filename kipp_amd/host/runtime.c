@@ -52,7 +52,7 @@ void kipp_scratch_reset(kipp_runtime *rt) {
 
 int kipp_settle(kipp_runtime *rt, kipp_delta *delta, kipp_error *error) {
     if (delta->parts > 0 || delta->w == NULL) return 0;
-    const kipp_rows x = {(void *)delta->x, NULL, 0, 0.0f};
+    const kipp_rows x = {(void *)delta->x, NULL, 0, 0.0f, delta->x_steps_major};
     const kipp_weight *w = delta->w;
     delta->w = NULL; /* what linear writes is a delta that has been launched */
     return rt->linear(rt, &x, w, delta->m, delta->max_parts, delta, error);
@@ -63,13 +63,13 @@ int kipp_finish_rows(kipp_runtime *rt, kipp_rows *rows, uint32_t m, uint32_t wid
     if (rt->scale_rows == NULL) return kipp_fail(error, KIPP_ERROR_INTERNAL, "rows without their scale on a path that leaves none");
     void *out = kipp_scratch(rt, (size_t)m * width * kipp_dtype_bytes(rt->act_dtype), error);
     if (out == NULL || rt->scale_rows(rt, rows, out, m, width, error) != 0) return -1;
-    *rows = (kipp_rows){out, NULL, 0, 0.0f};
+    *rows = (kipp_rows){out, NULL, 0, 0.0f, false};
     return 0;
 }
 
 int kipp_linear_defer(kipp_runtime *rt, const kipp_rows *x, const kipp_weight *w, uint32_t m, int max_parts, kipp_delta *out, kipp_error *error) {
     if (rt->defers != NULL && x->sumsq == NULL && rt->defers(rt, x, w, m)) {
-        *out = (kipp_delta){NULL, 0, x->data, w, m, max_parts};
+        *out = (kipp_delta){NULL, 0, x->data, w, m, max_parts, x->steps_major};
         return 0;
     }
     return rt->linear(rt, x, w, m, max_parts, out, error);

@@ -52,9 +52,12 @@ class GatedMLP:
         if ours and rows <= rt.few_rows:
             # both products and the activation in one kernel (and the norm's scale, if it was left to us)
             scaled = isinstance(x, ScaledRows)
+            # the activation goes to the down projection alone: written in the order that product reads fastest
+            major = rt.steps_major_rows and inner % 32 == 0 and rows > 1 and rt._few_rows(rows, inner, self.w_down)
             rt.ops.gemm_skinny_swiglu(x.rows if scaled else x, w.rows, act, tiles=w.tiles,
-                                      row_scale=x.scale if scaled else None)
-            return rt.linear(act, self.w_down, slabs=True, defer=True)
+                                      row_scale=x.scale if scaled else None,
+                                      x_steps_major=scaled and x.steps_major, out_steps_major=major)
+            return rt.linear(act, self.w_down, slabs=True, defer=True, x_steps_major=major)
         x = rt.rows_of(x)
         if ours and w.pairs:
             # streamed from the paired tiles: the columns come out gate tile by gate tile

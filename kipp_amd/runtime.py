@@ -57,11 +57,12 @@ class ScaledRows:
     weight) and `sumsq` [M, >= parts], `parts` partial sums of x^2 a row whose total gives
     row t's scale rsqrt(sum(sumsq[t, :parts]) / width + eps).  A row's scale commutes with a product over
     the row, so `Runtime.linear` applies it to the product's rows; any other
-    consumer asks `Runtime.rows_of` for the finished rows."""
-    __slots__ = ("rows", "sumsq", "parts", "eps")
+    consumer asks `Runtime.rows_of` for the finished rows.  `steps_major`: `rows` holds its values as
+    [width / 32][M][32] (what the few-rows products read fastest, `ops.steps_major`), not as [M][width]."""
+    __slots__ = ("rows", "sumsq", "parts", "eps", "steps_major")
 
-    def __init__(self, rows: torch.Tensor, sumsq: torch.Tensor, parts: int, eps: float):
-        self.rows, self.sumsq, self.parts, self.eps = rows, sumsq, parts, eps
+    def __init__(self, rows: torch.Tensor, sumsq: torch.Tensor, parts: int, eps: float, steps_major: bool = False):
+        self.rows, self.sumsq, self.parts, self.eps, self.steps_major = rows, sumsq, parts, eps, steps_major
 
     @property
     def scale(self):
@@ -81,14 +82,14 @@ class Deferred:
     """A product `x . w^T` that `Runtime.linear(..., defer=True)` has not launched
     yet: the delta of a mixer or a feed-forward, which a norm that follows may
     launch together with the residual add (`Runtime.product_add_norm`); `run()`
-    launches it as it is."""
-    __slots__ = ("rt", "x", "w", "slabs")
+    launches it as it is.  `x_steps_major`: x holds its values in the order of `ops.steps_major`."""
+    __slots__ = ("rt", "x", "w", "slabs", "x_steps_major")
 
-    def __init__(self, rt, x, w, slabs):
-        self.rt, self.x, self.w, self.slabs = rt, x, w, slabs
+    def __init__(self, rt, x, w, slabs, x_steps_major=False):
+        self.rt, self.x, self.w, self.slabs, self.x_steps_major = rt, x, w, slabs, x_steps_major
 
     def run(self) -> torch.Tensor:
-        return self.rt.linear(self.x, self.w, slabs=self.slabs)
+        return self.rt.linear(self.x, self.w, slabs=self.slabs, x_steps_major=self.x_steps_major)
 
 
 class Runtime:
@@ -116,6 +117,9 @@ class Runtime:
         self.fused_decode_rows = 16                 # single tokens up to which decode attention starts from the QKV product ...
         self.fused_decode_keys = 8192               # ... while their contexts are shorter than this
         self.fuse_norm_x_bytes = self.FUSE_NORM_X_BYTES
+        # rows that one few-rows product writes for the next (a norm's rows, the activation) in the order that product
+        # reads fastest, [width / 32][rows][32]: half the memory requests for x at 8 rows (3 % of a decode step at batch 8)
+        self.steps_major_rows = os.environ.get("KIPP_AMD_STEPS_MAJOR", "1") != "0"
         # products of more than about 200 rows: True (the default): our own matrix-core kernel, in the fastest of the
         # cuts that give the planned cut's bits, so that every process computes the same bits; "auto": the fastest of
         # all our cuts and the library's product, timed once in a process at a shape's first use (another process
@@ -167,7 +171,7 @@ class Runtime:
         """The tensor of norm output, scaled now if the scale was left to a product."""
         if not isinstance(h, ScaledRows):
             return h
-        return self.ops.scale_rows(h.rows, h.sumsq, h.parts, h.eps, self.empty(h.rows.shape, torch.bfloat16))
+        return self.ops.scale_rows(h.rows, h.sumsq, h.parts, h.eps, self.empty(h.rows.shape, torch.bfloat16), steps_major=h.steps_major)
 
     def product_add_norm(self, delta: Deferred, x: torch.Tensor, norm_weight: torch.Tensor, eps: float):
         """x += delta's product, in the product's own kernel, which also prepares the
@@ -187,8 +191,10 @@ class Runtime:
         n_out = w.shape[0]
         if self.ops.gemm_skinny_parts(n_out, k, most) > 1 and ((n_out + 15) // 16) * rows * k * 2 > self.fuse_norm_x_bytes:
             return None
-        rows_out, sumsq = self.ops.gemm_skinny(delta.x, w.rows, tiles=w.tiles, add_norm=(x, norm_weight))
-        return ScaledRows(rows_out, sumsq, (w.shape[0] + 15) // 16, eps)
+        major = self.steps_major_rows and n_out % 32 == 0 and rows > 1       # one row is one run either way
+        rows_out, sumsq = self.ops.gemm_skinny(delta.x, w.rows, tiles=w.tiles, add_norm=(x, norm_weight),
+                                               x_steps_major=delta.x_steps_major, out_steps_major=major)
+        return ScaledRows(rows_out, sumsq, (w.shape[0] + 15) // 16, eps, steps_major=major)
 
     # -- products of prompt portions ------------------------------------------------------------
     def streams(self, m: int, k: int, n: int) -> bool:
@@ -301,22 +307,25 @@ class Runtime:
         self.library_products += 1
         return library()
 
-    def linear(self, x, w, slabs: bool = False, defer: bool = False):
+    def linear(self, x, w, slabs: bool = False, defer: bool = False, x_steps_major: bool = False):
         """float32 [M, N] = x [M, K] . w [N, K]^T.  With `slabs` the result may come
         as [parts, M, N] whose sum over parts is the product (few rows against a
         weight with few output rows: the contraction is split over workgroups and
         the consumer adds the slabs in order); an integer is the most slabs the
         consumer takes.  `x` may be ScaledRows.  With
         `defer` the product may come back as a `Deferred` (for a delta of the
-        residual stream, which the next norm launches or `settle` does)."""
+        residual stream, which the next norm launches or `settle` does).  `x_steps_major`: a plain x
+        holds its values in the order of `ops.steps_major` (few rows only)."""
         if defer and self.fuse_norms and not isinstance(x, ScaledRows) and self._few_rows(x.shape[0], x.shape[1], w):
-            return Deferred(self, x, w, slabs)
+            return Deferred(self, x, w, slabs, x_steps_major)
         row_scale = None
         if isinstance(x, ScaledRows):
             if self._few_rows(x.shape[0], x.shape[1], w):
-                row_scale, x = x.scale, x.rows
+                row_scale, x_steps_major, x = x.scale, x.steps_major, x.rows
             else:
                 x = self.rows_of(x)
+        if x_steps_major and not (isinstance(w, Weight) and self._few_rows(x.shape[0], x.shape[1], w) and self.streams(x.shape[0], x.shape[1], w.shape[0])):
+            x, x_steps_major = self.ops.from_steps_major(x), False       # only the few-rows kernel reads that order
         tiles = None
         if isinstance(w, Weight):
             # paired tiles give the columns in another order: only the feed-forward asks for that
@@ -333,7 +342,8 @@ class Runtime:
             # up to about 200 rows: our own kernels stream the weight once
             most = 0 if slabs is False else (None if slabs is True else int(slabs))
             if m <= self.few_rows:
-                y = self.ops.gemm_skinny(x, w, max_parts=1 if most == 0 else (most or 8), tiles=tiles, row_scale=row_scale)
+                y = self.ops.gemm_skinny(x, w, max_parts=1 if most == 0 else (most or 8), tiles=tiles, row_scale=row_scale,
+                                         x_steps_major=x_steps_major)
             else:
                 y = self.ops.gemm_rows(x, w, max_parts=1 if most == 0 else (most or 12), tiles=tiles)
             return y if y.shape[0] > 1 else y[0]

@@ -490,7 +490,7 @@ static int toy_mean_forward(void *part_, const kipp_rows *x, kipp_batch *batch, 
             }
         }
     }
-    return rt->linear(rt, &(kipp_rows){mean, NULL, 0, 0.0f}, &part->w, batch->n_tokens, 1, out, error);
+    return rt->linear(rt, &(kipp_rows){mean, NULL, 0, 0.0f, false}, &part->w, batch->n_tokens, 1, out, error);
 }
 
 static const kipp_mixer_fn toy_mean_fn = {toy_mean_cache_need, toy_mean_state_need, toy_mean_forward, false};

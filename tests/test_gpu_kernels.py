@@ -852,6 +852,45 @@ def test_tile_weight_by_the_kernel(n, k):
         assert torch.equal(ops.tile_weight_device(w, gate_up=True), ops.tile_weight_pairs(w))
 
 
+@pytest.mark.parametrize("m", [1, 2, 5, 8])
+@pytest.mark.parametrize("n,k", [(96, 64), (2560, 4096), (160, 320)])
+def test_few_rows_products_with_rows_in_steps_major_order(m, n, k):
+    """The few-rows products read x, and write the rows they make for the next product, as [width / 32][rows][32] when told
+    so: the same bits as from and to [rows][width], for the plain product, the residual's end, the activation's end and the
+    kernel that finishes a norm's rows."""
+    ops = _ops()
+    torch.manual_seed(m * 1000 + n)
+    x = torch.randn(m, k).bfloat16().to(DEV)
+    w = (torch.randn(n, k) * 0.1).bfloat16().to(DEV)
+    tiles = ops.tile_weight(w)
+    xm = ops.steps_major(x)
+    assert torch.equal(ops.from_steps_major(xm), x)
+    for t in (None, tiles):
+        assert torch.equal(ops.gemm_skinny(xm, w, 4, tiles=t, x_steps_major=True), ops.gemm_skinny(x, w, 4, tiles=t))
+    # the residual's end: rows and sums from either order of x, into either order of the rows
+    norm_w = (1 + 0.1 * torch.randn(n)).to(DEV)
+    res = torch.randn(m, n).to(DEV)
+    want_res = res.clone()
+    want_rows, want_ss = ops.gemm_skinny(x, w, tiles=tiles, add_norm=(want_res, norm_w))
+    for x_major, out_major in ((True, False), (False, True), (True, True)):
+        got_res = res.clone()
+        rows, ss = ops.gemm_skinny(xm if x_major else x, w, tiles=tiles, add_norm=(got_res, norm_w), x_steps_major=x_major, out_steps_major=out_major)
+        parts = (n + 15) // 16                                     # the sums a row has (its stride is rounded up to 4)
+        assert torch.equal(got_res, want_res) and torch.equal(ss[:, :parts], want_ss[:, :parts])
+        assert torch.equal(ops.from_steps_major(rows) if out_major else rows, want_rows)
+        fin = ops.scale_rows(rows, ss, parts, 1e-6, torch.empty(m, n, dtype=torch.bfloat16, device=DEV), steps_major=out_major)
+        assert torch.equal(fin, ops.scale_rows(want_rows, want_ss, parts, 1e-6, torch.empty(m, n, dtype=torch.bfloat16, device=DEV)))
+    # the activation's end ([gate; up] of n / 2 rows each, when n / 2 is a multiple of 32)
+    if (n // 2) % 32 == 0:
+        for t in (None, ops.tile_weight_pairs(w)):
+            want = ops.gemm_skinny_swiglu(x, w, torch.empty(m, n // 2, dtype=torch.bfloat16, device=DEV), tiles=t)
+            got = ops.gemm_skinny_swiglu(xm, w, torch.empty(m, n // 2, dtype=torch.bfloat16, device=DEV), tiles=t, x_steps_major=True,
+                                         out_steps_major=True)
+            assert torch.equal(ops.from_steps_major(got), want)
+    with pytest.raises(ops.KernelError):
+        ops.gemm_skinny(torch.zeros(2, 40, dtype=torch.bfloat16, device=DEV), torch.zeros(16, 40, dtype=torch.bfloat16, device=DEV), x_steps_major=True)
+
+
 def test_tile_weight_layout():
     ops = _ops()
     w = torch.arange(20 * 64, dtype=torch.float32).reshape(20, 64).bfloat16()          # 20 rows: the second tile is padded
