@@ -451,7 +451,7 @@ struct kipp_model {
     /* steps of single tokens, recorded once a shape has come twice and run again as a graph (step.c) */
     struct kipp_step_graph *graphs;
     size_t graph_count, graph_capacity;
-    uint64_t graph_replays;
+    uint64_t graph_replays, graph_clock;
 };
 
 /* One recorded shape: rows, the width of the block tables, the longest context (both rounded up), logits or their largest. */
@@ -464,6 +464,7 @@ typedef struct kipp_step_graph {
     uint64_t generation;    /* ... and while the table of operations has not moved its own buffers */
     float *logits;
     int32_t *chosen;
+    uint64_t used; /* the model's graph_clock when it last ran */
 } kipp_step_graph;
 
 int kipp_model_params(const kipp_model_spec *spec, kipp_param_list *out, kipp_error *error);

@@ -234,6 +234,13 @@ static int forward_and_choose(kipp_model *model, bool choose, float **logits, in
     return model->rt->argmax(model->rt, *logits, *chosen, model->batch.n_want, model->spec.vocab, error);
 }
 
+/* Recordings kept: KIPP_GRAPH_SHAPES, or what KIPP_AMD_GRAPH_SHAPES says (tests make it small). */
+static size_t graph_shapes(void) {
+    const char *text = getenv("KIPP_AMD_GRAPH_SHAPES");
+    long n = text != NULL ? strtol(text, NULL, 10) : 0;
+    return n >= 1 && n <= 4096 ? (size_t)n : KIPP_GRAPH_SHAPES;
+}
+
 /* Runs the batch.  `single` (tokens one a session, all wanted, their shape rounded by build_batch): a shape that has come
  * before is recorded, and from then on run again from the recording.  Every buffer a recording names keeps its place:
  * weights, pages and state slots for the model's life, the step's workspace because a step takes it in the same order from
@@ -248,8 +255,16 @@ static int run_step(kipp_model *model, bool single, bool choose, float **logits,
     for (size_t i = 0; i < model->graph_count && entry == NULL; ++i) {
         if (model->graphs[i].key == key) entry = &model->graphs[i];
     }
+    if (entry == NULL && model->graph_count >= graph_shapes()) {
+        /* more shapes than are kept: the one used longest ago makes room */
+        entry = &model->graphs[0];
+        for (size_t i = 1; i < model->graph_count; ++i) {
+            if (model->graphs[i].used < entry->used) entry = &model->graphs[i];
+        }
+        if (entry->graph != NULL) rt->graph_free(rt, entry->graph);
+        *entry = (kipp_step_graph){key, 0, false, NULL, NULL, 0, NULL, NULL, 0};
+    }
     if (entry == NULL) {
-        if (model->graph_count == KIPP_GRAPH_SHAPES) return forward_and_choose(model, choose, logits, chosen, error); /* more shapes than are kept */
         if (model->graph_count == model->graph_capacity) {
             size_t capacity = model->graph_capacity == 0 ? 8 : model->graph_capacity * 2;
             kipp_step_graph *grown = realloc(model->graphs, capacity * sizeof(kipp_step_graph));
@@ -258,8 +273,9 @@ static int run_step(kipp_model *model, bool single, bool choose, float **logits,
             model->graph_capacity = capacity;
         }
         entry = &model->graphs[model->graph_count++];
-        *entry = (kipp_step_graph){key, 0, false, NULL, NULL, 0, NULL, NULL};
+        *entry = (kipp_step_graph){key, 0, false, NULL, NULL, 0, NULL, NULL, 0};
     }
+    entry->used = ++model->graph_clock;
     if (entry->graph != NULL && (entry->batch_base != batch->d_all || entry->generation != rt->generation)) {
         rt->graph_free(rt, entry->graph); /* a buffer it names has moved */
         entry->graph = NULL;

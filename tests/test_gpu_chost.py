@@ -226,3 +226,30 @@ def test_c_host_recorded_steps_give_the_bits_of_steps_run_as_they_are(model_fold
             H.assert_close(got[1][at][i:i + 1], ref[i][len(p) - 12 + step:len(p) - 11 + step], H.NMSE_BF16["tiny"], f"recorded step {step}, request {i}")
     for model in models:
         model.close()
+
+
+def test_c_host_keeps_a_bounded_number_of_recordings(model_folders, tiny_configs, monkeypatch):
+    """With room for two recordings, runs of steps of one, two and three rows push each other out (the one used longest
+    ago goes) and are recorded again: every step still has the bits of the model that records nothing."""
+    from kipp_amd.chost import CModel
+    monkeypatch.setenv("KIPP_AMD_GRAPH_SHAPES", "2")
+    vocab = tiny_configs["a"]["vocab_size"]
+    prompts = [H.random_tokens(80 + i, 30, vocab) for i in range(3)]
+    got = []
+    for eager in (True, False):
+        rows = []
+        with CModel(model_folders[("a", "bfloat16")], path="gpu-bf16", page_tokens=16, kv_pool_pages=12, max_sessions=3,
+                    share_prefixes=False, eager_steps=eager) as model:
+            sessions = [model.session() for _ in prompts]
+            for s, p in zip(sessions, prompts):
+                model.step([(s, p[:6], [])])
+            for step in range(18):
+                live = 1 + (step // 3) % 3                           # three steps of one row, of two, of three, and again
+                rows.append(model.step([(s, [p[6 + step]], [0]) for s, p in list(zip(sessions, prompts))[:live]]))
+                for s in sessions[live:]:                            # the others keep pace without being asked for logits
+                    model.step([(s, [prompts[sessions.index(s)][6 + step]], [])])
+            replays = model.graph_replays
+        got.append(rows)
+        assert replays == 0 if eager else replays > 0
+    for a, b in zip(*got):
+        assert np.array_equal(a, b)
