@@ -63,6 +63,9 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--page", type=int, default=16, help="tokens per cache page")
     ap.add_argument("--kv-pages", type=int, default=None, help="pages in the pool (default: enough for this run)")
     ap.add_argument("--prefill-chunk", type=int, default=512, help="largest portion of a prompt in one step")
+    ap.add_argument("--warm-up", action="store_true",
+                    help="run one portion of the prompt's first step's size before the clock starts: what a shape decides once a process "
+                         "(the cut of a prompt product) then does not count as prefill time")
     ap.add_argument("--max-step-tokens", type=int, default=2048, help="token budget of one step")
     ap.add_argument("--random", metavar="SHAPE",
                     help="named shape (tiny-a, tiny-b, qwen3-4b, ...): with --write-random the folder to write, else the model of this run")
@@ -259,6 +262,8 @@ def _run(args) -> int:
     pages = _pool_pages(args, capacity, per_page)
     engine = Engine.from_folder(args.model, dtype=args.dtype, page_size=args.page, num_pages=pages, max_requests=1,
                                 max_position=limit)
+    if args.warm_up:
+        engine.warm_up((min(len(tokens), args.prefill_chunk, args.max_step_tokens),))
     stops = tuple(args.stop_token) if args.stop_token is not None else tuple(engine.model.spec.stop_tokens)
     backend = f"hip-{args.dtype}"
     print(f"kipp: evaluating {len(tokens)} token{'s' if len(tokens) != 1 else ''} on {backend}", file=sys.stderr)

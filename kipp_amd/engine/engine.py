@@ -57,6 +57,25 @@ class Engine:
         self._uncommitted.pop(request_id, None)     # a step that was never recorded leaves nothing behind
         self.cache.close(request_id)
 
+    def warm_up(self, rows: Sequence[int] = (2048, 512, 256)) -> None:
+        """Run a prompt portion of each of these sizes on a request of its own and forget it: what a shape decides at
+        its first use (the cut of a prompt product is timed once a process) is decided now, not inside a request's
+        first step.  Sizes that the pools or the positions cannot hold are left out; nothing is published."""
+        share, self.cache.share = self.cache.share, False
+        try:
+            for n in rows:
+                fits = 0 < n <= self.cache.max_position and all(-(-n // g.page_size) <= g.pool.free_count for g in self.cache.groups)
+                if not fits or not self.cache.free_slots:
+                    continue
+                name = ("warm-up", n)
+                try:
+                    self.step([StepEntry(name, [0] * n, [n - 1])])
+                finally:
+                    if name in self.cache.requests:
+                        self.close(name)
+        finally:
+            self.cache.share = share
+
     def length(self, request_id) -> int:
         return self.cache.requests[request_id].length
 

@@ -422,3 +422,24 @@ def test_portions_behind_a_long_context_cut_their_keys(long_folder, dtype):
     H.assert_close(np.concatenate(got), ref, tol, f"portions behind a long context/{dtype}")
     if dtype == "bfloat16":
         assert seen == [True, True, True, True]      # 700 keys already exceed a cut of 512; every portion was cut
+
+
+def test_warm_up_decides_before_the_first_request(real_folder, real_reference):
+    """`Engine.warm_up` runs portions of the given sizes on a request of its own: the products' cuts for those sizes are
+    decided then (not in a request's first step), the pool is as empty as before, nothing was published, and a prompt
+    afterwards has the bits it has on an engine that was never warmed up."""
+    from kipp_amd.engine import Engine, StepEntry
+    requests, _ = real_reference
+    toks = requests["p"]
+    warm = Engine.from_folder(real_folder, dtype="bfloat16", page_size=16, max_tokens=512, max_requests=2)
+    assert not warm.rt.prompt_product_choices
+    warm.warm_up((256, 100000))                                   # the second neither fits the pool nor the positions: left out
+    assert warm.rt.prompt_product_choices and not warm.cache.requests
+    for g in warm.cache.groups:
+        assert g.pool.free_count == g.pool.num_pages and all(c is None for c in g.pool.content)
+    decided = dict(warm.rt.prompt_product_choices)
+    got = warm.step([StepEntry("p", toks, list(range(len(toks))))]).float().cpu()
+    cold = Engine.from_folder(real_folder, dtype="bfloat16", page_size=16, max_tokens=512, max_requests=2)
+    want = cold.step([StepEntry("p", toks, list(range(len(toks))))]).float().cpu()
+    assert torch.equal(got, want)
+    assert all(warm.rt.prompt_product_choices[k] == v for k, v in decided.items())
