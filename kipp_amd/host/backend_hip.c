@@ -455,7 +455,7 @@ static int hip_embed(kipp_runtime *rt, const kipp_weight *table, const int32_t *
     return rc == 0 ? 0 : refused(error, "embed", rc);
 }
 
-#define FEW_ROWS 8            /* up to these the kernel in which every wave reads its rows of x itself is the faster one, and has the fused ends */
+#define FEW_ROWS 12           /* up to these the kernel in which every wave reads its rows of x itself is the faster one, and has the fused ends */
 #define STAGED_ROWS 192       /* up to these the kernel that stages x through LDS; beyond, the one built for hundreds of rows where it takes the shape */
 #define FUSE_NORM_X_BYTES 40e6 /* most bytes of x the workgroups of an unsplit product may read together for the fused norm to pay */
 
@@ -522,7 +522,7 @@ static int hip_residual_add(kipp_runtime *rt, float *x, kipp_delta *delta, uint3
     return rc == 0 ? 0 : refused(error, "residual_add", rc);
 }
 
-/* x . w^T.  bfloat16 x bfloat16: up to 8 rows the kernel in which every wave streams its rows of w against all of x (it also
+/* x . w^T.  bfloat16 x bfloat16: up to 12 rows the kernel in which every wave streams its rows of w against all of x (it also
  * applies a scale that the rows still lack), up to 192 rows the one that stages x through LDS, both from the streaming layout
  * where the weight has it; beyond those the tiled matrix-core kernel (K a multiple of 32) or the staged one over runs of 256
  * rows; a shape none of them takes (K no multiple of 8, or below 32) and every float32 weight go through the plain float32

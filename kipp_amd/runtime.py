@@ -112,7 +112,7 @@ class Runtime:
         self.fuse_norms = True      # few rows: residual add and norm ride on the products around them
         # Where one kernel hands over to the next, measured at the 4B shape on an MI355X; another width or device may
         # move them, so they are the runtime's and can be set on it
-        self.few_rows = ops.SKINNY_BEST_ROWS        # rows up to which every wave reads its rows of x itself (the kernel with the fused ends)
+        self.few_rows = int(os.environ.get("KIPP_AMD_FEW_ROWS", ops.SKINNY_BEST_ROWS))   # rows up to which every wave reads its rows of x itself (the kernel with the fused ends)
         self.staged_rows = ops.ROWS_BEST_ROWS       # rows up to which x is staged through LDS; beyond, the product built for hundreds of rows
         self.fused_decode_rows = 16                 # single tokens up to which decode attention starts from the QKV product ...
         self.fused_decode_keys = 8192               # ... while their contexts are shorter than this
