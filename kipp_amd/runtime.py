@@ -116,7 +116,7 @@ class Runtime:
         self.staged_rows = ops.ROWS_BEST_ROWS       # rows up to which x is staged through LDS; beyond, the product built for hundreds of rows
         self.fused_decode_rows = 16                 # single tokens up to which decode attention starts from the QKV product ...
         self.fused_decode_keys = 8192               # ... while their contexts are shorter than this
-        self.fuse_norm_x_bytes = self.FUSE_NORM_X_BYTES
+        self.fuse_norm_x_bytes = float(os.environ.get("KIPP_AMD_FUSE_NORM_X_BYTES", self.FUSE_NORM_X_BYTES))
         # rows that one few-rows product writes for the next (a norm's rows, the activation) in the order that product
         # reads fastest, [width / 32][rows][32]: half the memory requests for x at 8 rows (3 % of a decode step at batch 8)
         self.steps_major_rows = os.environ.get("KIPP_AMD_STEPS_MAJOR", "1") != "0"
