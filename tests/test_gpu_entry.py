@@ -285,8 +285,9 @@ def test_trace_run_says_why_it_refuses_a_step(model_folders, tmp_path):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("key,page,cut", [("b", 16, "mixed"), ("a", 16, "portions"), ("b", 8, "portions"), ("a", 32, "tail")])
-def test_trace_run(model_folders, tiny_configs, tmp_path, dtype, key, page, cut):
+@pytest.mark.parametrize("key,page,cut,host", [("b", 16, "mixed", "python"), ("a", 16, "portions", "python"), ("b", 8, "portions", "python"),
+                                               ("a", 32, "tail", "python"), ("b", 16, "mixed", "c"), ("a", 16, "tail", "c")])
+def test_trace_run(model_folders, tiny_configs, tmp_path, dtype, key, page, cut, host):
     folder = model_folders[(key, dtype)]
     vocab = tiny_configs[key]["vocab_size"]
     requests = {f"r{i}": H.random_tokens(300 + i, n, vocab) for i, n in enumerate([70, 33, 100, 7, 61, 90])}
@@ -301,7 +302,8 @@ def test_trace_run(model_folders, tiny_configs, tmp_path, dtype, key, page, cut)
             del fed[rid]
     out = tmp_path / "out"
     proc = subprocess.Popen([os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype, "--out", str(out),
-                             "--max-tokens", str(peak), "--page", str(page)], stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True)
+                             "--max-tokens", str(peak), "--page", str(page), "--host", host], stdin=subprocess.PIPE, stdout=subprocess.PIPE,
+                            text=True)
     for i, line in enumerate(_trace(requests, steps)):
         proc.stdin.write(line + "\n")
         proc.stdin.flush()
@@ -318,7 +320,7 @@ def test_trace_run(model_folders, tiny_configs, tmp_path, dtype, key, page, cut)
         assert at == data.shape[0]
     tol = H.NMSE_F32 if dtype == "float32" else H.NMSE_BF16["tiny"]
     for rid, toks in requests.items():
-        H.assert_close(np.concatenate(rows[rid]), H.plain_logits(folder, toks), tol, f"trace {key} page {page} {cut} {dtype} {rid}")
+        H.assert_close(np.concatenate(rows[rid]), H.plain_logits(folder, toks), tol, f"trace {key} page {page} {cut} {dtype} {host} {rid}")
 
 
 def _run_trace(folder, dtype, out, lines, *options):
@@ -328,8 +330,9 @@ def _run_trace(folder, dtype, out, lines, *options):
     assert proc.stdout.split() == [w for i in range(len(lines)) for w in ("done", str(i))]
 
 
+@pytest.mark.parametrize("host", ["python", "c"])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_trace_run_with_requests_that_share_a_beginning(model_folders, tiny_configs, tmp_path, dtype):
+def test_trace_run_with_requests_that_share_a_beginning(model_folders, tiny_configs, tmp_path, dtype, host):
     """--share: a request whose first tokens an earlier request left in the cache adopts those pages (whole pages,
     none that holds a wanted place) and runs the rest only; the logits at the wanted places are the plain ones.
     Pages of 24 tokens, which do not divide 64."""
@@ -348,7 +351,7 @@ def test_trace_run_with_requests_that_share_a_beginning(model_folders, tiny_conf
         {"step": 4, "entries": [{"id": "d", "tokens": H.random_tokens(4, 128, vocab), "want": [127]}], "end": ["d"]},
     )]
     out = tmp_path / "out"
-    _run_trace(folder, dtype, out, lines, "--max-tokens", "192", "--page", "24", "--share")
+    _run_trace(folder, dtype, out, lines, "--max-tokens", "192", "--page", "24", "--share", "--host", host)
     tol = H.NMSE_F32 if dtype == "float32" else H.NMSE_BF16["tiny"]
 
     def rows(step):
