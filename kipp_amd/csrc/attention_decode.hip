@@ -89,7 +89,14 @@ struct Projected {
     const float* inv_freq;   // null (and angles null): no rotation
     const float* angles;     // [tokens][HEAD_DIM]: cosines then sines of every token's angles, or null: computed here
     int write_kv;            // 0: the cache is another layer's, keys and values are already there
+    int out_rows;            // > 0: `out` is written as [n_q HEAD_DIM / 32][out_rows][32] for the product that reads it next (below)
 };
+
+// Where element `col` of row `row` of the mixed heads lies: [row][width], or with `out_rows` > 0 in the order the
+// few-rows products read their rows fastest, [width / 32][out_rows][32] (a wave's 64 bytes of each row are then one run).
+__device__ __forceinline__ size_t out_at(int row, int col, int width, int out_rows) {
+    return out_rows > 0 ? ((size_t)(col >> 5) * out_rows + row) * 32 + (col & 31) : (size_t)row * width + col;
+}
 
 // Values that another workgroup of the same launch reads: written through to memory and read from there (the
 // dies' L2 caches do not see each other's lines).  A store is known to have arrived once the wave's count of
@@ -157,7 +164,8 @@ __device__ __forceinline__ void put_partial(const unsigned* arrivals, float* par
 // itself once what it wrote has arrived, and the one that counts last merges the splits, in split order.  Nobody
 // waits for anybody.  Called by all threads of the workgroup.
 __device__ __forceinline__ void merge_by_the_last(unsigned* arrivals, const float* part_acc, const float* part_ml, bf16_t* out,
-                                                  int item, int row, int kvh, int n_q, int n_kv, int max_splits, int n_splits) {
+                                                  int item, int row, int kvh, int n_q, int n_kv, int max_splits, int n_splits,
+                                                  int out_rows = 0) {
     __shared__ int s_last;
     const int tid = threadIdx.x;
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -175,7 +183,7 @@ __device__ __forceinline__ void merge_by_the_last(unsigned* arrivals, const floa
         const int g = idx / HEAD_DIM, dcol = idx % HEAD_DIM;
         const int head = kvh * GROUP + g;
         const size_t slot0 = ((size_t)item * n_q + head) * max_splits;
-        out[((size_t)row * n_q + head) * HEAD_DIM + dcol] = f32_to_bf16(merge_splits_here(part_acc, part_ml, slot0, n_splits, dcol));
+        out[out_at(row, head * HEAD_DIM + dcol, n_q * HEAD_DIM, out_rows)] = f32_to_bf16(merge_splits_here(part_acc, part_ml, slot0, n_splits, dcol));
     }
 }
 
@@ -478,13 +486,13 @@ __global__ void __launch_bounds__(THREADS) attention_decode_kernel(
         for (int w = 0; w < WAVES; ++w) a += s_red[w][g][dcol];
         const int head = kvh * GROUP + g;
         if (n_splits == 1) {
-            out[((size_t)row * n_q + head) * HEAD_DIM + dcol] = f32_to_bf16(a / s_l[g]);
+            out[out_at(row, head * HEAD_DIM + dcol, n_q * HEAD_DIM, FUSED ? pj.out_rows : 0)] = f32_to_bf16(a / s_l[g]);
         } else {
             put_partial(arrivals, part_acc, part_ml, ((size_t)blockIdx.x * n_q + head) * max_splits + blockIdx.z, dcol, a, s_m[g], s_l[g]);
         }
     }
     if (arrivals != nullptr && n_splits > 1)
-        merge_by_the_last(arrivals, part_acc, part_ml, out, blockIdx.x, row, kvh, n_q, n_kv, max_splits, n_splits);
+        merge_by_the_last(arrivals, part_acc, part_ml, out, blockIdx.x, row, kvh, n_q, n_kv, max_splits, n_splits, FUSED ? pj.out_rows : 0);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -1017,13 +1025,13 @@ __global__ void __launch_bounds__(THREADS, 2) attention_decode_ring_kernel(
         }
         const int head = kvh * GROUP + g;
         if (n_splits == 1) {
-            out[((size_t)row * n_q + head) * HEAD_DIM + dcol] = f32_to_bf16(a / l);
+            out[out_at(row, head * HEAD_DIM + dcol, n_q * HEAD_DIM, FUSED ? pj.out_rows : 0)] = f32_to_bf16(a / l);
         } else {
             put_partial(arrivals, part_acc, part_ml, ((size_t)blockIdx.x * n_q + head) * max_splits + blockIdx.z, dcol, a, m, l);
         }
     }
     if (arrivals != nullptr && n_splits > 1)
-        merge_by_the_last(arrivals, part_acc, part_ml, out, blockIdx.x, row, kvh, n_q, n_kv, max_splits, n_splits);
+        merge_by_the_last(arrivals, part_acc, part_ml, out, blockIdx.x, row, kvh, n_q, n_kv, max_splits, n_splits, FUSED ? pj.out_rows : 0);
 }
 #endif  // RING_OK
 
@@ -1033,7 +1041,7 @@ __global__ void __launch_bounds__(THREADS, 2) attention_decode_ring_kernel(
 __global__ void attention_decode_reduce_kernel(
     const float* __restrict__ part_acc, const float* __restrict__ part_ml, bf16_t* __restrict__ out,
     const int32_t* __restrict__ rows, const int32_t* __restrict__ positions, int n_q, int window, int max_splits,
-    int split_keys) {
+    int split_keys, int out_rows) {
     const int head = blockIdx.x, item = blockIdx.y;
     const int row = rows[item];
     const int pos = positions[row];
@@ -1061,7 +1069,7 @@ __global__ void attention_decode_reduce_kernel(
             a += a3 * exp2f(part_ml[(slot0 + s + 3) * 2] - m);
         }
         for (; s < n_splits; ++s) a += part_acc[(slot0 + s) * HEAD_DIM + dcol] * exp2f(part_ml[(slot0 + s) * 2] - m);
-        out[((size_t)row * n_q + head) * HEAD_DIM + dcol] = f32_to_bf16(a / denom);
+        out[out_at(row, head * HEAD_DIM + dcol, n_q * HEAD_DIM, out_rows)] = f32_to_bf16(a / denom);
     }
 }
 
@@ -1073,7 +1081,7 @@ template <int MAXS>
 __global__ void __launch_bounds__(KIPP_WAVE) attention_decode_reduce_few_kernel(
     const float* __restrict__ part_acc, const float* __restrict__ part_ml, bf16_t* __restrict__ out,
     const int32_t* __restrict__ rows, const int32_t* __restrict__ positions, int n_q, int window, int max_splits,
-    int split_keys, int grid_splits) {
+    int split_keys, int grid_splits, int out_rows) {
     constexpr int COLS = (HEAD_DIM + KIPP_WAVE - 1) / KIPP_WAVE;     // columns of a head a lane merges
     const int head = blockIdx.x, item = blockIdx.y, lane = threadIdx.x;
     const size_t slot0 = ((size_t)item * n_q + head) * max_splits;
@@ -1110,24 +1118,24 @@ __global__ void __launch_bounds__(KIPP_WAVE) attention_decode_reduce_few_kernel(
 #pragma unroll
     for (int c = 0; c < COLS; ++c) {
         const int dcol = lane + KIPP_WAVE * c;
-        if (dcol < HEAD_DIM) out[((size_t)row * n_q + head) * HEAD_DIM + dcol] = f32_to_bf16(a[c] / denom);
+        if (dcol < HEAD_DIM) out[out_at(row, head * HEAD_DIM + dcol, n_q * HEAD_DIM, out_rows)] = f32_to_bf16(a[c] / denom);
     }
 }
 
 // The merge of a launch's splits (`grid_splits` of `split_keys` keys each at most).
 static int launch_reduce(const float* part_acc, const float* part_ml, bf16_t* out, const int32_t* rows,
                          const int32_t* positions, int n_items, int n_q, int window, int max_splits, int split_keys,
-                         int grid_splits, hipStream_t stream) {
+                         int grid_splits, hipStream_t stream, int out_rows = 0) {
     const dim3 grid(n_q, n_items);
     if (grid_splits <= 8)
         hipLaunchKernelGGL(attention_decode_reduce_few_kernel<8>, grid, dim3(KIPP_WAVE), 0, stream, part_acc, part_ml, out,
-                           rows, positions, n_q, window, max_splits, split_keys, grid_splits);
+                           rows, positions, n_q, window, max_splits, split_keys, grid_splits, out_rows);
     else if (grid_splits <= 16)
         hipLaunchKernelGGL(attention_decode_reduce_few_kernel<16>, grid, dim3(KIPP_WAVE), 0, stream, part_acc, part_ml, out,
-                           rows, positions, n_q, window, max_splits, split_keys, grid_splits);
+                           rows, positions, n_q, window, max_splits, split_keys, grid_splits, out_rows);
     else
         hipLaunchKernelGGL(attention_decode_reduce_kernel, grid, dim3(HEAD_DIM >= 64 ? 64 : HEAD_DIM), 0, stream, part_acc,
-                           part_ml, out, rows, positions, n_q, window, max_splits, split_keys);
+                           part_ml, out, rows, positions, n_q, window, max_splits, split_keys, out_rows);
     return KIPP_LAUNCH_CHECK();
 }
 
@@ -1178,7 +1186,8 @@ static int launch_ring(const bf16_t* q, bf16_t* k_cache, bf16_t* v_cache, bf16_t
                        n_kv, page, scale_log2e, window, max_splits, range, pj, arrivals);
     *rc = KIPP_LAUNCH_CHECK();
     if (*rc != 0 || ring_splits == 1 || arrivals != nullptr) return 1;
-    *rc = launch_reduce(part_acc, part_ml, (bf16_t*)out, rows, positions, n_items, n_q, window, max_splits, range, ring_splits, stream);
+    *rc = launch_reduce(part_acc, part_ml, (bf16_t*)out, rows, positions, n_items, n_q, window, max_splits, range, ring_splits, stream,
+                        FUSED ? pj.out_rows : 0);
     return 1;
 }
 #endif
@@ -1228,7 +1237,7 @@ static int launch_split(const bf16_t* q, bf16_t* k_cache, bf16_t* v_cache, bf16_
 #undef KIPP_SPLIT_LAUNCH
     int rc = KIPP_LAUNCH_CHECK();
     if (rc != 0 || splits == 1 || arrivals != nullptr) return rc;      // with `arrivals` the last workgroup of a head has merged
-    return launch_reduce(part_acc, part_ml, out, rows, positions, n_items, n_q, window, max_splits, keys, splits, stream);
+    return launch_reduce(part_acc, part_ml, out, rows, positions, n_items, n_q, window, max_splits, keys, splits, stream, FUSED ? pj.out_rows : 0);
 }
 
 extern "C" {
@@ -1294,14 +1303,15 @@ int kipp_attention_decode_fused_slabs() { return MAX_SLABS; }
 // The same from the output of the QKV projection: `qkv` float32 [parts][tokens][(n_q + 2 n_kv) head_dim];
 // norm weights, `inv_freq` and `angles` may be null (no norm; no rotation if both are null; a rotation covers
 // the whole head; `angles` [tokens][head_dim] holds every token's cosines, then sines);
-// with `write_kv` the token's key and value are written into the cache as well.
+// with `write_kv` the token's key and value are written into the cache as well; with `out_steps_major` `out` is written
+// as [n_q head_dim / 32][n_tokens][32], the order in which the few-rows product that follows reads its rows fastest.
 int kipp_attention_decode_fused(const float* qkv, int parts, int n_tokens, const float* q_norm_w, const float* k_norm_w,
                                 float eps, const float* inv_freq, const float* angles, int write_kv, void* k_cache,
                                 void* v_cache, void* out,
                                 float* part_acc, float* part_ml, const int32_t* rows, const int32_t* positions,
                                 const int32_t* seq_of_token, const int32_t* block_table, int max_blocks, int n_items,
                                 int n_q, int n_kv, int head_dim, int page, float scale, int window, int grid_splits,
-                                int max_splits, int32_t* arrivals, hipStream_t stream) {
+                                int max_splits, int32_t* arrivals, int out_steps_major, hipStream_t stream) {
 #if FUSED_OK
     if (n_items <= 0) return 0;
     if (head_dim != HEAD_DIM || n_kv <= 0 || n_q != n_kv * GROUP || parts <= 0 || parts > MAX_SLABS) return -1;
@@ -1309,7 +1319,7 @@ int kipp_attention_decode_fused(const float* qkv, int parts, int n_tokens, const
     if (page <= 0 || (page & (page - 1))) return -4;
     const float scale_log2e = scale * 1.4426950408889634f;
     Projected pj{qkv, parts, (size_t)n_tokens * (n_q + 2 * n_kv) * HEAD_DIM, q_norm_w, k_norm_w, eps, inv_freq, angles,
-                 write_kv};
+                 write_kv, out_steps_major ? n_tokens : 0};
 #if RING_OK
     {
         int rc = 0;

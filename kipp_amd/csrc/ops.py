@@ -371,11 +371,12 @@ def attention_decode_fused(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: to
                            q_norm_w: Optional[torch.Tensor], k_norm_w: Optional[torch.Tensor], eps: float,
                            inv_freq: Optional[torch.Tensor], rotary_dim: int, write_kv: bool, scale: float, window: int,
                            max_context: int, workspace: tuple, grid_splits: Optional[int] = None,
-                           angles: Optional[torch.Tensor] = None) -> torch.Tensor:
+                           angles: Optional[torch.Tensor] = None, out_steps_major: bool = False) -> torch.Tensor:
     """Decode attention straight from the QKV projection: per-head q/k RMSNorm,
     rotation, the write of the token's key and value into its page and the
     attention over the pages in one kernel (plus the merge of the splits).
-    `qkv`: float32 [tokens, width] or slabs [parts, tokens, width]."""
+    `qkv`: float32 [tokens, width] or slabs [parts, tokens, width].  `out_steps_major`: `out` is written in the
+    order of `steps_major` (for the few-rows product that reads it next)."""
     _dev(qkv, k_cache, v_cache, out, rows, positions, seq_of_token, block_table, angles, *workspace)
     for t, name in ((rows, "rows"), (positions, "positions"), (seq_of_token, "seq_of_token"), (block_table, "block_table")):
         _i32(t, name)
@@ -408,13 +409,13 @@ def attention_decode_fused(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: to
     defines = {"HEAD_DIM": head_dim, "GROUP": group}
     fn = _fn("attention_decode", "kipp_attention_decode_fused",
              [_c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_float, _c_ptr, _c_ptr, _c_int] + [_c_ptr] * 9 + [_c_int] * 6
-             + [_c_float, _c_int, _c_int, _c_int, _c_ptr, _c_ptr], defines)
+             + [_c_float, _c_int, _c_int, _c_int, _c_ptr, _c_int, _c_ptr], defines)
     null = lambda t: _ptr(t) if t is not None else None
     _check(fn(_ptr(qkv), parts, n_tokens, null(q_norm_w), null(k_norm_w), float(eps), null(inv_freq), null(angles),
               1 if write_kv else 0,
               _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(part_acc), _ptr(part_ml), _ptr(rows), _ptr(positions),
               _ptr(seq_of_token), _ptr(block_table), block_table.shape[1], n_items, n_q, n_kv, head_dim,
-              k_cache.shape[2], float(scale), int(window), grid, max_splits, _ptr(arrivals), _stream()),
+              k_cache.shape[2], float(scale), int(window), grid, max_splits, _ptr(arrivals), int(bool(out_steps_major)), _stream()),
            "attention_decode_fused")
     return out
 

@@ -83,10 +83,12 @@ struct kipp_runtime {
                      const kipp_attention_geometry *geometry, kipp_error *error);
     /* Optional (NULL: none).  A step of single tokens: the QKV product, the per-head norms, the rotation, the write of the new
      * keys and values and the attention over the pages, with as few kernels as the table has for this shape; *done says
-     * whether it ran (else the caller takes linear, qk_norm_rope_kv and attention). */
-    int (*decode_attention)(kipp_runtime *rt, const kipp_rows *x, const kipp_weight *w_qkv, const kipp_cache_view *cache, void *out,
-                            kipp_batch *batch, const kipp_attention_geometry *geometry, const float *q_norm_w, const float *k_norm_w,
-                            float eps, const float *rotation, uint32_t rotary_dim, int interleaved, bool *done, kipp_error *error);
+     * whether it ran (else the caller takes linear, qk_norm_rope_kv and attention).  out->data is given; `reader` is the matrix
+     * that the mixed heads are multiplied with next (as for `gated`). */
+    int (*decode_attention)(kipp_runtime *rt, const kipp_rows *x, const kipp_weight *w_qkv, const kipp_cache_view *cache,
+                            const kipp_weight *reader, kipp_rows *out, kipp_batch *batch, const kipp_attention_geometry *geometry,
+                            const float *q_norm_w, const float *k_norm_w, float eps, const float *rotation, uint32_t rotary_dim,
+                            int interleaved, bool *done, kipp_error *error);
     int (*gather_rows)(kipp_runtime *rt, const float *x, const int32_t *index, float *out, uint32_t n, uint32_t width, kipp_error *error);
     /* out[r] = the index of the largest of logits[r, :vocab], the lowest among equals (/root/reference/src/kipp.c:3459-3464) */
     int (*argmax)(kipp_runtime *rt, const float *logits, int32_t *out, uint32_t rows, uint32_t vocab, kipp_error *error);

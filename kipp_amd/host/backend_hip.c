@@ -58,7 +58,7 @@ typedef int (*fn_tile_weight)(const void *, void *, int, int, int, hipStream_t);
 typedef int (*fn_argmax)(const float *, int32_t *, int, int, float *, hipStream_t);
 typedef int (*fn_attention_decode_fused)(const float *, int, int, const float *, const float *, float, const float *, const float *, int, void *,
                                          void *, void *, float *, float *, const int32_t *, const int32_t *, const int32_t *, const int32_t *, int,
-                                         int, int, int, int, int, float, int, int, int, int32_t *, hipStream_t);
+                                         int, int, int, int, int, float, int, int, int, int32_t *, int, hipStream_t);
 typedef int (*fn_ring_takes)(int, int, int, int);
 typedef int (*fn_tiles_parts)(int, int, int, int, int);
 typedef int (*fn_gemm_tiles)(const void *, const void *, void *, int, int, int, int, int, int, hipStream_t);
@@ -773,9 +773,10 @@ static bool attention_fast(const kipp_runtime *rt, const kipp_attention_geometry
 
 /* Single tokens only: the QKV product in at most four slabs, then norm, rotation, cache write and attention in one kernel,
  * for a few tokens and wherever the kernel that walks whole contexts or long ranges runs. */
-static int hip_decode_attention(kipp_runtime *rt, const kipp_rows *x, const kipp_weight *w_qkv, const kipp_cache_view *cache, void *out,
-                                kipp_batch *batch, const kipp_attention_geometry *g, const float *q_norm_w, const float *k_norm_w, float eps,
-                                const float *rotation, uint32_t rotary_dim, int interleaved, bool *done, kipp_error *error) {
+static int hip_decode_attention(kipp_runtime *rt, const kipp_rows *x, const kipp_weight *w_qkv, const kipp_cache_view *cache,
+                                const kipp_weight *reader, kipp_rows *out, kipp_batch *batch, const kipp_attention_geometry *g,
+                                const float *q_norm_w, const float *k_norm_w, float eps, const float *rotation, uint32_t rotary_dim,
+                                int interleaved, bool *done, kipp_error *error) {
     hip_state *st = rt->state;
     *done = false;
     const uint32_t n = batch->n_tokens;
@@ -795,11 +796,15 @@ static int hip_decode_attention(kipp_runtime *rt, const kipp_rows *x, const kipp
     if (hip_linear(rt, x, w_qkv, n, v->fused_slabs, &qkv, error) != 0) return -1;
     int32_t *arrivals;
     if (decode_workspace(rt, batch, v, g, &max_splits, &grid, error) != 0 || arrivals_for(rt, (size_t)n * g->n_q, &arrivals, error) != 0) return -1;
-    int rc = v->decode_fused(qkv.data, qkv.parts, (int)n, q_norm_w, k_norm_w, eps, NULL, rotation, cache->writable ? 1 : 0, cache->k, cache->v, out,
-                             batch->decode_workspace[0], batch->decode_workspace[1], batch->decode_rows, batch->positions, batch->seq_of_token,
-                             batch->tables[cache->group], (int)batch->max_blocks, (int)n, (int)g->n_q, (int)g->n_kv, (int)g->head_dim,
-                             (int)cache->page_tokens, g->scale, (int)g->window, grid, (int)max_splits, arrivals, st->stream);
+    /* the mixed heads go to `reader` alone: in the order its product reads fastest, if that is a few-rows product */
+    const bool major = st->steps_major && reader != NULL && few_rows(rt, reader, n) && !reader->pairs && n > 1;
+    int rc = v->decode_fused(qkv.data, qkv.parts, (int)n, q_norm_w, k_norm_w, eps, NULL, rotation, cache->writable ? 1 : 0, cache->k, cache->v,
+                             out->data, batch->decode_workspace[0], batch->decode_workspace[1], batch->decode_rows, batch->positions,
+                             batch->seq_of_token, batch->tables[cache->group], (int)batch->max_blocks, (int)n, (int)g->n_q, (int)g->n_kv,
+                             (int)g->head_dim, (int)cache->page_tokens, g->scale, (int)g->window, grid, (int)max_splits, arrivals, major ? 1 : 0,
+                             st->stream);
     if (rc != 0) return refused(error, "attention_decode_fused", rc);
+    out->steps_major = major;
     *done = true;
     return 0;
 }

@@ -346,10 +346,11 @@ static int attention_forward(void *part_, const kipp_rows *x, kipp_batch *batch,
     if (rt->decode_attention != NULL && batch->n_portions == 0) {
         /* single tokens only: a table may have fewer kernels for the way from x to the mixed heads */
         bool done = false;
-        if (rt->decode_attention(rt, x, &part->w_qkv, cache, mixed, batch, &geometry, part->q_norm, part->k_norm, eps, rotation, rotary_dim,
-                                 interleaved, &done, error) != 0)
+        kipp_rows heads = {mixed, NULL, 0, 0.0f, false};
+        if (rt->decode_attention(rt, x, &part->w_qkv, cache, &part->w_o, &heads, batch, &geometry, part->q_norm, part->k_norm, eps, rotation,
+                                 rotary_dim, interleaved, &done, error) != 0)
             return -1;
-        if (done) return kipp_linear_defer(rt, &(kipp_rows){mixed, NULL, 0, 0.0f, false}, &part->w_o, n, 8, out, error);
+        if (done) return kipp_linear_defer(rt, &heads, &part->w_o, n, 8, out, error);
     }
     kipp_delta qkv;
     if (rt->linear(rt, x, &part->w_qkv, n, 4, &qkv, error) != 0) return -1;

@@ -118,12 +118,14 @@ class Attention:
         qkv = rt.linear(x, self.w_qkv, slabs=rt.ops.DECODE_FUSED_SLABS if fused else True)
         if fused:
             out = rt.empty((n, s.q_dim), rt.act_dtype)
+            # the mixed heads go to the output projection alone: in the order that product reads fastest, if it is a few-rows one
+            major = rt.steps_major_rows and n > 1 and rt._few_rows(n, s.q_dim, self.w_o)
             rt.ops.attention_decode_fused(qkv, cache.k, cache.v, out, batch.decode_rows, batch.positions,
                                           batch.seq_of_token, table, s.num_heads, s.num_kv_heads, s.head_dim,
                                           self.q_norm, self.k_norm, eps, inv_freq, rotary_dim, cache.writable,
                                           self.scale, s.window or 0, batch.max_decode_ctx, self._workspace(batch),
-                                          angles=angles)
-            return rt.linear(out, self.w_o, slabs=True, defer=True)
+                                          angles=angles, out_steps_major=major)
+            return rt.linear(out, self.w_o, slabs=True, defer=True, x_steps_major=major)
         q = rt.ops.qk_norm_rope_kv_write(
             qkv, rt.empty((n, s.q_dim), rt.act_dtype), cache.k, cache.v,
             batch.positions, batch.seq_of_token, table, s.num_heads, s.num_kv_heads, s.head_dim,

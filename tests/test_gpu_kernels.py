@@ -512,6 +512,10 @@ def test_attention_decode_of_a_dozen_sequences_in_ranges(window):
                                      _t(rows, torch.int32), *args, n_q, n_kv, d, None, None, 0.0, inv_freq, d, True,
                                      1 / math.sqrt(d), window, longest, ws)
     assert torch.equal(got, want) and torch.equal(k1, k2) and torch.equal(v1, v2)
+    major = ops.attention_decode_fused(qkv, k.to(DEV), v.to(DEV), torch.zeros(t, n_q * d, dtype=torch.bfloat16, device=DEV),
+                                       _t(rows, torch.int32), *args, n_q, n_kv, d, None, None, 0.0, inv_freq, d, True,
+                                       1 / math.sqrt(d), window, longest, ws, out_steps_major=True)
+    assert torch.equal(ops.from_steps_major(major), want)
     ref = _attention_reference(q.cpu(), k1.cpu(), v1.cpu(), table, positions, seq_of, n_q, n_kv, d, page, window)
     out = want.float().cpu().numpy().reshape(t, n_q, d)
     for i in range(t):
@@ -571,6 +575,10 @@ def test_attention_decode_in_longer_splits():
                                      _t(rows, torch.int32), *args, n_q, n_kv, d, None, None, 0.0, inv_freq, d, True,
                                      1 / math.sqrt(d), 0, longest, ws)
     assert torch.equal(got, want) and torch.equal(k1, k2) and torch.equal(v1, v2)
+    major = ops.attention_decode_fused(qkv, k.to(DEV), v.to(DEV), torch.zeros(t, n_q * d, dtype=torch.bfloat16, device=DEV),
+                                       _t(rows, torch.int32), *args, n_q, n_kv, d, None, None, 0.0, inv_freq, d, True,
+                                       1 / math.sqrt(d), 0, longest, ws, out_steps_major=True)
+    assert torch.equal(ops.from_steps_major(major), want)
     ref = _attention_reference(q.cpu(), k1.cpu(), v1.cpu(), table, positions, seq_of, n_q, n_kv, d, page, 0)
     assert _rel(want.float().cpu().numpy().reshape(t, n_q, d), ref) < 1e-5
 
@@ -632,6 +640,14 @@ def _from_the_projection(ops, n_q, n_kv, d, page, window, norm, slabs, write_kv)
     assert torch.equal(again, got) and torch.equal(k3, k2) and torch.equal(v3, v2)
     assert write_kv != torch.equal(k2.cpu(), k)            # the cache changed exactly when it was to be written
     assert torch.equal(got, want)
+    # the rows in the order a few-rows product reads them in: the same values, merged by the last split's workgroup
+    # or by a launch of its own
+    for workspace in (ws, ws[:2]):
+        k4, v4 = k.to(DEV), v.to(DEV)
+        major = ops.attention_decode_fused(qkv, k4, v4, torch.zeros(t, n_q * d, dtype=torch.bfloat16, device=DEV),
+                                           _t(rows, torch.int32), *args, n_q, n_kv, d, qw, kw, 1e-6, inv_freq, d, write_kv,
+                                           1 / math.sqrt(d), window, max(seq_lens), workspace, out_steps_major=True)
+        assert torch.equal(ops.from_steps_major(major), want) and torch.equal(k4, k2) and torch.equal(v4, v2)
     assert not ops.attention_decode_fused_ok(64, 64, True) and not ops.attention_decode_fused_ok(128, 64, True)
     assert ops.attention_decode_fused_ok(128, 64, False)
 
