@@ -12,6 +12,13 @@
 // K is split over `parts` workgroups (grid.y): part p writes slab p of
 // Y[parts, M, N]; the consumer adds the slabs in order.
 //
+// A workgroup has 4 to 8 waves (its size is the launch's, not the kernel's), so that the tiles of W can be
+// dealt out to about as many workgroups as there are compute units without splitting K: the SwiGLU end
+// (W = [gate; up] in paired tiles, act = silu(gate) * up written straight from the sums) needs the whole of K
+// in one workgroup.  `RowScale`: X holds the rows of an RMS norm without their scale (bfloat16(x * norm
+// weight)) and the partial sums of x^2 beside them; every row of the product is multiplied by
+// rsqrt(sum / K + eps), which is the product of the normalized row.
+//
 // v_mfma_f32_16x16x32_bf16: A = W tile (lane: row l % 16, k = 8 (l / 16) + j),
 // B = X^T from LDS (lane: token l % 16, same k), D: lane holds features
 // 4 (l / 16) + v of token l % 16.
@@ -28,26 +35,38 @@ union Frag {
     bf16x8 v;
 };
 
+struct RowScale {               // sumsq == nullptr: none
+    const float* sumsq;         // [M, stride]: `parts` partial sums of squares of each row X was made from
+    int parts, stride;          // stride: parts rounded up to a multiple of 4, so that a lane loads four sums at once
+    float inv_width, eps;
+};
+
 // TILED: W in the streaming layout [tile of 16 rows][step of 32 columns][lane][8 values]
 // (rows padded to whole tiles with zeros, K a multiple of 32), in which a wave's load is
 // one contiguous KB.
 // DEPTH: steps of 32 columns in one chunk.  NTW: 16-row tiles of W a wave streams (every fragment of X
 // read from LDS then serves NTW products, and a workgroup's staging of X serves NTW times the rows).
-template <int MT, int TW, bool TILED, int DEPTH, int NTW>
-__global__ void __launch_bounds__(TW * KIPP_WAVE) gemm_rows_kernel(
-    const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, float* __restrict__ Y, int M, int N, int K) {
+// END 1: W is [gate; up] in paired tiles (8 gate rows over the 8 matching up rows), N = 16 tiles' columns, K is not split and
+// act[M, inner] = bfloat16(silu(gate) * up) is written instead of Y.
+#define MIN_WAVES 4
+#define MAX_WAVES 8
+
+template <int MT, bool TILED, int DEPTH, int NTW, int END>
+__global__ void __launch_bounds__(MAX_WAVES * KIPP_WAVE) gemm_rows_kernel(
+    const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, float* __restrict__ Y, bf16_t* __restrict__ act, int M, int N, int K,
+    int inner, RowScale rs) {
     constexpr int CHUNK = 32 * DEPTH;                          // columns of X staged at a time
     constexpr int X_PITCH = CHUNK + 8;                         // bf16 elements per staged row (the pad spreads the banks)
-    constexpr int THREADS = TW * KIPP_WAVE;
     constexpr int UNITS = MT * 16 * (CHUNK / 8);              // 16-byte units of one staged chunk
-    constexpr int XR = UNITS / THREADS;                        // units a thread moves
-    static_assert(UNITS % THREADS == 0, "every thread stages the same number of units");
+    constexpr int XR = UNITS / (MIN_WAVES * KIPP_WAVE);        // units a thread of the smallest workgroup moves
+    static_assert(UNITS % (MIN_WAVES * KIPP_WAVE) == 0, "whole waves stage whole runs of units");
     __shared__ __attribute__((aligned(16))) bf16_t xs[2][MT * 16 * X_PITCH];
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int threads = blockDim.x, tw = threads >> 6;         // MIN_WAVES to MAX_WAVES waves
     const int l16 = lane & 15, h = lane >> 4;
-    const int n0 = (blockIdx.x * TW + wave) * (16 * NTW);
+    const int n0 = (blockIdx.x * tw + wave) * (16 * NTW);
     const int part = blockIdx.y, parts = gridDim.y;
     const int groups = K / CHUNK;                              // whole chunks; the rest of K goes to the last part
     const int g_begin = (int)((long long)groups * part / parts);
@@ -59,16 +78,52 @@ __global__ void __launch_bounds__(TW * KIPP_WAVE) gemm_rows_kernel(
         w_row[i] = TILED ? W + (size_t)min((n0 >> 4) + i, (N + 15) / 16 - 1) * (K / 32) * 512 + lane * 8
                          : W + (size_t)min(n0 + 16 * i + l16, N - 1) * K + 8 * h;
 
-    // the units of X this thread stages: unit -> (row, 8-column chunk)
+    // the units of X this thread stages: unit -> (row, 8-column chunk); a larger workgroup has fewer a thread
     const bf16_t* x_src[XR];
     int x_dst[XR];
+    bool x_mine[XR];
 #pragma unroll
     for (int i = 0; i < XR; ++i) {
-        const int unit = tid + i * THREADS;
-        const int r = unit / (CHUNK / 8), c = unit % (CHUNK / 8);
+        const int unit = tid + i * threads;
+        x_mine[i] = unit < UNITS;
+        const int r = min(unit, UNITS - 1) / (CHUNK / 8), c = unit % (CHUNK / 8);
         x_src[i] = X + (size_t)min(r, M - 1) * K + c * 8;
         x_dst[i] = r * X_PITCH + c * 8;
     }
+
+    // the partial sums of the rows' scales, asked for before everything else (they arrive first and are added once
+    // the first weights are on their way): lane group h takes the h-th run of four sums of its tokens
+    // (up to 64 rows; beyond, the kernel is long, registers are short and the sums are fetched at the end)
+    constexpr bool EARLY = MT <= 4;
+    float4 scale_part[EARLY ? MT : 1];
+    if (EARLY && rs.sumsq != nullptr) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+            scale_part[mt] = *(const float4*)(rs.sumsq + (size_t)min(16 * mt + l16, M - 1) * rs.stride + min(4 * h, rs.stride - 4));
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    float row_scale[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) row_scale[mt] = 1.0f;
+    auto finish_scale = [&](bool early) {
+        if (rs.sumsq == nullptr || early != EARLY) return;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const int p = 4 * h;
+            if (!EARLY) scale_part[0] = *(const float4*)(rs.sumsq + (size_t)min(16 * mt + l16, M - 1) * rs.stride + min(4 * h, rs.stride - 4));
+            const float4 part4 = scale_part[EARLY ? mt : 0];
+            float t = 0.0f;
+            t += p < rs.parts ? part4.x : 0.0f;
+            t += p + 1 < rs.parts ? part4.y : 0.0f;
+            t += p + 2 < rs.parts ? part4.z : 0.0f;
+            t += p + 3 < rs.parts ? part4.w : 0.0f;
+            const float* more = rs.sumsq + (size_t)min(16 * mt + l16, M - 1) * rs.stride;
+            for (int q = 16 + h; q < rs.parts; q += 4) t += more[q];        // rows wider than 16 partial sums
+            t += __shfl_xor(t, 16, KIPP_WAVE);     // the four lane groups of a token
+            t += __shfl_xor(t, 32, KIPP_WAVE);
+            row_scale[mt] = 1.0f / sqrtf(t * rs.inv_width + rs.eps);
+        }
+    };
 
     f32x4 acc[NTW][MT];
 #pragma unroll
@@ -84,11 +139,13 @@ __global__ void __launch_bounds__(TW * KIPP_WAVE) gemm_rows_kernel(
     };
     auto fetch_x = [&](int g) {
 #pragma unroll
-        for (int i = 0; i < XR; ++i) xr[i] = *(const u32x4*)(x_src[i] + (size_t)g * CHUNK);
+        for (int i = 0; i < XR; ++i)
+            if (x_mine[i]) xr[i] = *(const u32x4*)(x_src[i] + (size_t)g * CHUNK);
     };
     auto stage_x = [&](int buf) {
 #pragma unroll
-        for (int i = 0; i < XR; ++i) *(u32x4*)(xs[buf] + x_dst[i]) = xr[i];
+        for (int i = 0; i < XR; ++i)
+            if (x_mine[i]) *(u32x4*)(xs[buf] + x_dst[i]) = xr[i];
     };
     auto multiply = [&](int u, int buf) {
 #pragma unroll
@@ -107,6 +164,7 @@ __global__ void __launch_bounds__(TW * KIPP_WAVE) gemm_rows_kernel(
 #pragma unroll
         for (int u = 0; u < DEPTH; ++u) fetch_w(u, g_begin * DEPTH + u);
         stage_x(0);
+        finish_scale(true);
         __syncthreads();
         int buf = 0;
         for (int g = g_begin; g + 1 < g_end; ++g) {
@@ -123,6 +181,8 @@ __global__ void __launch_bounds__(TW * KIPP_WAVE) gemm_rows_kernel(
         }
 #pragma unroll
         for (int u = 0; u < DEPTH; ++u) multiply(u, buf);
+    } else {
+        finish_scale(true);
     }
     // the rest of K (less than a chunk), by the last part, straight from global memory
     if (part == parts - 1) {
@@ -144,6 +204,37 @@ __global__ void __launch_bounds__(TW * KIPP_WAVE) gemm_rows_kernel(
             }
         }
     }
+    finish_scale(false);
+    if (END == 1) {
+        // rows 0..7 of a tile are gates, rows 8..15 the matching ups: they sit 32 lanes apart
+#pragma unroll
+        for (int i = 0; i < NTW; ++i) {
+            const int o = (n0 / 2) + 8 * i + 4 * h;                // first of this lane's four features (lane groups 0 and 1)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                const int token = 16 * mt + l16;
+                float a[4];
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const float g = acc[i][mt][v] * row_scale[mt], up = __shfl_xor(g, 32, KIPP_WAVE);
+                    a[v] = g / (1.0f + expf(-g)) * up;
+                }
+                if (h >= 2 || token >= M) continue;
+                bf16_t* out = act + (size_t)token * inner + o;
+                if (o + 3 < inner && (inner & 3) == 0) {
+                    uint2 packed;
+                    packed.x = (uint32_t)f32_to_bf16(a[0]) | ((uint32_t)f32_to_bf16(a[1]) << 16);
+                    packed.y = (uint32_t)f32_to_bf16(a[2]) | ((uint32_t)f32_to_bf16(a[3]) << 16);
+                    *(uint2*)out = packed;
+                } else {
+#pragma unroll
+                    for (int v = 0; v < 4; ++v)
+                        if (o + v < inner) out[v] = f32_to_bf16(a[v]);
+                }
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < NTW; ++i) {
         const int n = n0 + 16 * i + 4 * h;
@@ -152,18 +243,19 @@ __global__ void __launch_bounds__(TW * KIPP_WAVE) gemm_rows_kernel(
             const int token = 16 * mt + l16;
             if (token >= M) continue;
             float* y = Y + ((size_t)part * M + token) * N + n;
+            const float sc = row_scale[mt];
             if (n + 3 < N && (N & 3) == 0) {
-                *(float4*)y = make_float4(acc[i][mt][0], acc[i][mt][1], acc[i][mt][2], acc[i][mt][3]);
+                *(float4*)y = make_float4(acc[i][mt][0] * sc, acc[i][mt][1] * sc, acc[i][mt][2] * sc, acc[i][mt][3] * sc);
             } else {
 #pragma unroll
                 for (int v = 0; v < 4; ++v)
-                    if (n + v < N) y[v] = acc[i][mt][v];
+                    if (n + v < N) y[v] = acc[i][mt][v] * sc;
             }
         }
     }
 }
 
-// Tiles of 16 rows of W per workgroup (4 or 8 waves with one tile each, or 8 waves with two) and parts of
+// Tiles of 16 rows of W per workgroup (4 to 8 waves with one tile each, or 5 to 8 waves with two) and parts of
 // K, from the shape only.  A compute unit draws a bounded number of bytes a second, so the workgroups run
 // in rounds of 256 and a round costs what one workgroup reads, its rows of W and (from L2, at about a
 // quarter of the price a row) all rows of X, plus a fixed start; the plan takes the cheapest rounds, with a
@@ -171,26 +263,90 @@ __global__ void __launch_bounds__(TW * KIPP_WAVE) gemm_rows_kernel(
 // sweeps over these splits at 32, 64 and 128 rows: the more rows X has, the larger the workgroups.)
 static int chunk_of(int M) { return M > 128 ? 64 : (M > 64 ? 128 : 256); }
 
-static void plan(int M, int N, int K, int max_parts, int* tw, int* ntw, int* parts) {
+static double plan(int M, int N, int K, int max_parts, int* tw, int* ntw, int* parts) {
+    static const int tiles_of_a_workgroup[] = {4, 5, 6, 7, 8, 10, 12, 14, 16};
     const int tiles = (N + 15) / 16;
     const int groups = K / chunk_of(M) > 0 ? K / chunk_of(M) : 1;
     double best = 1e300;
     *tw = 4;
     *ntw = 1;
     *parts = 1;
-    for (int t = 4; t <= 16; t *= 2) {
+    for (int t : tiles_of_a_workgroup) {
         const int cols = (tiles + t - 1) / t;
         for (int p = 1; p <= max_parts && p <= groups; ++p) {
             const int rounds = (cols * p + 255) / 256;
             const double cost = rounds * ((t + 0.27 * M / 16.0) * (double)K / p + 150.0 * t) * (1.0 + 0.02 * p);
             if (cost < best * 0.999) {
                 best = cost;
-                *tw = t > 8 ? 8 : t;
+                *tw = t > 8 ? t / 2 : t;
                 *ntw = t > 8 ? 2 : 1;
                 *parts = p;
             }
         }
     }
+    return best;
+}
+
+// `cut` (for measurements and tests): 10 x waves + tiles a wave, with exactly max_parts parts of K (as many as K has chunks).
+static int cut_or_plan(int M, int N, int K, int max_parts, int cut, int* tw, int* ntw, int* parts) {
+    if (cut == 0) {
+        plan(M, N, K, max_parts, tw, ntw, parts);
+        return 0;
+    }
+    *tw = cut / 10;
+    *ntw = cut % 10;
+    const int groups = K / chunk_of(M) > 0 ? K / chunk_of(M) : 1;
+    *parts = max_parts < groups ? max_parts : groups;
+    return (*tw < MIN_WAVES || *tw > MAX_WAVES || *ntw < 1 || *ntw > 2) ? -1 : 0;
+}
+
+static int sumsq_stride(int parts) { return (parts + 3) / 4 * 4; }
+
+template <int END>
+static int launch(const void* X, const void* W, float* Y, void* act, int M, int N, int K, int inner, int tw, int ntw, int parts,
+                  int tiled, RowScale rs, hipStream_t stream) {
+    const int tiles = (N + 15) / 16;
+    dim3 grid((tiles + tw * ntw - 1) / (tw * ntw), parts), block(tw * KIPP_WAVE);
+    const int mt = (M + 15) / 16;       // from 65 rows on an even number of 16-row tiles is staged (whole waves move whole runs of units)
+#define KIPP_GR(MT, DEPTH, NTW)                                                                                          \
+    do {                                                                                                                 \
+        if (tiled)                                                                                                       \
+            hipLaunchKernelGGL((gemm_rows_kernel<MT, true, DEPTH, NTW, END>), grid, block, 0, stream, (const bf16_t*)X,  \
+                               (const bf16_t*)W, Y, (bf16_t*)act, M, N, K, inner, rs);                                   \
+        else if (END == 0)                                                                                               \
+            hipLaunchKernelGGL((gemm_rows_kernel<MT, false, DEPTH, NTW, 0>), grid, block, 0, stream, (const bf16_t*)X,   \
+                               (const bf16_t*)W, Y, (bf16_t*)act, M, N, K, inner, rs);                                   \
+        else                                                                                                             \
+            return -1;                                                                                                   \
+    } while (0)
+#define KIPP_GR_NTW(NTW)                   \
+    switch (mt) {                          \
+        case 1: KIPP_GR(1, 8, NTW); break; \
+        case 2: KIPP_GR(2, 8, NTW); break; \
+        case 3: KIPP_GR(3, 8, NTW); break; \
+        case 4: KIPP_GR(4, 8, NTW); break; \
+        case 5:                            \
+        case 6: KIPP_GR(6, 4, NTW); break; \
+        case 7:                            \
+        case 8: KIPP_GR(8, 4, NTW); break; \
+        case 9:                            \
+        case 10:                           \
+        case 11:                           \
+        case 12: KIPP_GR(12, 2, NTW); break; \
+        case 13:                           \
+        case 14:                           \
+        case 15:                           \
+        case 16: KIPP_GR(16, 2, NTW); break; \
+        default: return -1;                \
+    }
+    if (ntw == 2) {
+        KIPP_GR_NTW(2)
+    } else {
+        KIPP_GR_NTW(1)
+    }
+#undef KIPP_GR_NTW
+#undef KIPP_GR
+    return KIPP_LAUNCH_CHECK();
 }
 
 extern "C" {
@@ -205,54 +361,46 @@ int kipp_gemm_rows_parts(int M, int N, int K, int max_parts) {
 
 // Y: float32 [parts, M, N] with parts = kipp_gemm_rows_parts(M, N, K, max_parts).
 // M <= 256, K a multiple of 8; `tiled`: W in the streaming layout (K a multiple of 32).
+// `sumsq` [M, sumsq_parts rounded up to a multiple of 4] (or null): every row of the product is multiplied by
+// rsqrt(sum of the row's sumsq / K + eps).
 int kipp_gemm_rows(const void* X, const void* W, float* Y, int M, int N, int K, int max_parts, int tiled,
-                   hipStream_t stream) {
+                   const float* sumsq, int sumsq_parts, float eps, int cut, hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
     if (M > MAX_ROWS || K <= 0 || (K & 7) || max_parts <= 0 || (tiled && (K & 31))) return -1;
+    if (sumsq != nullptr && sumsq_parts <= 0) return -1;
     int tw, ntw, parts;
-    plan(M, N, K, max_parts, &tw, &ntw, &parts);
-    const int tiles = (N + 15) / 16;
-    dim3 grid((tiles + tw * ntw - 1) / (tw * ntw), parts), block(tw * KIPP_WAVE);
-    const int mt = (M + 15) / 16;       // from 65 rows on an even number of 16-row tiles is staged (every thread moves whole units)
-#define KIPP_GR(MT, TW, DEPTH, NTW)                                                                                     \
-    do {                                                                                                                \
-        if (tiled)                                                                                                      \
-            hipLaunchKernelGGL((gemm_rows_kernel<MT, TW, true, DEPTH, NTW>), grid, block, 0, stream, (const bf16_t*)X,  \
-                               (const bf16_t*)W, Y, M, N, K);                                                           \
-        else                                                                                                            \
-            hipLaunchKernelGGL((gemm_rows_kernel<MT, TW, false, DEPTH, NTW>), grid, block, 0, stream, (const bf16_t*)X, \
-                               (const bf16_t*)W, Y, M, N, K);                                                           \
-    } while (0)
-#define KIPP_GR_TW(TW, NTW)                    \
-    switch (mt) {                              \
-        case 1: KIPP_GR(1, TW, 8, NTW); break; \
-        case 2: KIPP_GR(2, TW, 8, NTW); break; \
-        case 3: KIPP_GR(3, TW, 8, NTW); break; \
-        case 4: KIPP_GR(4, TW, 8, NTW); break; \
-        case 5:                                \
-        case 6: KIPP_GR(6, TW, 4, NTW); break; \
-        case 7:                                \
-        case 8: KIPP_GR(8, TW, 4, NTW); break; \
-        case 9:                                \
-        case 10:                               \
-        case 11:                               \
-        case 12: KIPP_GR(12, TW, 2, NTW); break; \
-        case 13:                               \
-        case 14:                               \
-        case 15:                               \
-        case 16: KIPP_GR(16, TW, 2, NTW); break; \
-        default: return -1;                    \
-    }
-    if (tw == 8 && ntw == 2) {
-        KIPP_GR_TW(8, 2)
-    } else if (tw == 8) {
-        KIPP_GR_TW(8, 1)
-    } else {
-        KIPP_GR_TW(4, 1)
-    }
-#undef KIPP_GR_TW
-#undef KIPP_GR
-    return KIPP_LAUNCH_CHECK();
+    if (cut_or_plan(M, N, K, max_parts, cut, &tw, &ntw, &parts) != 0) return -1;
+    RowScale rs = {sumsq, sumsq_parts, sumsq_stride(sumsq_parts), 1.0f / (float)K, eps};
+    return launch<0>(X, W, Y, nullptr, M, N, K, 0, tw, ntw, parts, tiled, rs, stream);
+}
+
+// Whether the product that ends in SwiGLU is taken for this shape: K is not split there, and where the tiles of W are
+// too few for that (or leave most of a round of workgroups idle) the split product and an activation kernel are faster.
+int kipp_gemm_rows_swiglu_pays(int M, int two_inner, int K) {
+    if (M <= 0 || M > MAX_ROWS || two_inner <= 0 || (two_inner & 1) || K <= 0 || (K & 31)) return 0;
+    // beyond 64 rows the activation's arithmetic at the end of every workgroup costs what the second launch does (measured at
+    // 2560 x 19456: 2 to 3 us saved of 23 to 27 up to 64 rows, nothing from 80 rows on)
+    if (M > 64) return 0;
+    const int N = 16 * ((two_inner / 2 + 7) / 8);
+    int tw, ntw, parts;
+    const double whole = plan(M, N, K, 1, &tw, &ntw, &parts), split = plan(M, N, K, 12, &tw, &ntw, &parts);
+    // the split product's slabs are written, read again and the activation is a launch of its own: about a fifth of its time
+    return whole <= 1.2 * split;
+}
+
+// act: bfloat16 [M, I] = silu(X . gate^T) * (X . up^T); W: the paired tiles of [gate; up] ([2 I, K], tiles of 8 gate rows
+// over the 8 matching up rows, K a multiple of 32).  `sumsq`, `sumsq_parts`, `eps`: as above (both products are scaled
+// before the activation).
+int kipp_gemm_rows_swiglu(const void* X, const void* W, void* act, int M, int two_inner, int K, const float* sumsq,
+                          int sumsq_parts, float eps, int cut, hipStream_t stream) {
+    if (M <= 0 || two_inner <= 0) return 0;
+    if (M > MAX_ROWS || K <= 0 || (K & 31) || (two_inner & 1)) return -1;
+    if (sumsq != nullptr && sumsq_parts <= 0) return -1;
+    const int inner = two_inner / 2, N = 16 * ((inner + 7) / 8);
+    int tw, ntw, parts;
+    if (cut_or_plan(M, N, K, 1, cut, &tw, &ntw, &parts) != 0 || parts != 1) return -1;
+    RowScale rs = {sumsq, sumsq_parts, sumsq_stride(sumsq_parts), 1.0f / (float)K, eps};
+    return launch<1>(X, W, nullptr, act, M, N, K, inner, tw, ntw, 1, 1, rs, stream);
 }
 
 }  // extern "C"

@@ -50,9 +50,11 @@ typedef int (*fn_skinny_parts)(int, int, int);
 typedef int (*fn_gemm_skinny)(const void *, const void *, float *, int, int, int, int, int, const float *, int, float, float *, const float *,
                               void *, float *, int, int, hipStream_t);
 typedef int (*fn_rows_parts)(int, int, int, int);
-typedef int (*fn_gemm_rows)(const void *, const void *, float *, int, int, int, int, int, hipStream_t);
+typedef int (*fn_gemm_rows)(const void *, const void *, float *, int, int, int, int, int, const float *, int, float, int, hipStream_t);
+typedef int (*fn_gemm_rows_swiglu)(const void *, const void *, void *, int, int, int, const float *, int, float, int, hipStream_t);
 typedef int (*fn_skinny_swiglu)(const void *, const void *, void *, int, int, int, int, const float *, int, float, int, int, hipStream_t);
 typedef int (*fn_int_int)(int);
+typedef int (*fn_int3)(int, int, int);
 typedef int (*fn_scale_rows)(const void *, const float *, void *, int, int, int, int, float, int, hipStream_t);
 typedef int (*fn_tile_weight)(const void *, void *, int, int, int, hipStream_t);
 typedef int (*fn_argmax)(const float *, int32_t *, int, int, float *, hipStream_t);
@@ -94,6 +96,8 @@ typedef struct {
     fn_gemm_skinny gemm_skinny;
     fn_rows_parts rows_parts;
     fn_gemm_rows gemm_rows;
+    fn_gemm_rows_swiglu gemm_rows_swiglu;
+    fn_int3 rows_swiglu_pays;
     fn_tiles_parts tiles_parts;
     fn_gemm_tiles gemm_tiles;
     fn_skinny_swiglu gemm_skinny_swiglu;
@@ -205,6 +209,8 @@ static int open_common(hip_state *st, kipp_error *error) {
     KIPP_SYM(libs[4], gemm_skinny, "kipp_gemm_skinny");
     KIPP_SYM(libs[5], rows_parts, "kipp_gemm_rows_parts");
     KIPP_SYM(libs[5], gemm_rows, "kipp_gemm_rows");
+    KIPP_SYM(libs[5], gemm_rows_swiglu, "kipp_gemm_rows_swiglu");
+    KIPP_SYM(libs[5], rows_swiglu_pays, "kipp_gemm_rows_swiglu_pays");
     KIPP_SYM(libs[6], tiles_parts, "kipp_gemm_tiles_parts");
     KIPP_SYM(libs[6], gemm_tiles, "kipp_gemm_tiles");
     KIPP_SYM(libs[0], scale_rows, "kipp_scale_rows");
@@ -557,7 +563,7 @@ static int hip_linear(kipp_runtime *rt, const kipp_rows *rows_in, const kipp_wei
             int most = max_parts > 12 ? 12 : max_parts, parts = st->rows_parts(M, N, K, most);
             float *y = parts >= 1 ? kipp_scratch(rt, (size_t)parts * count * 4, error) : NULL;
             if (y == NULL) return parts >= 1 ? -1 : refused(error, "gemm_rows (its cut)", parts);
-            rc = st->gemm_rows(x, streamed, y, M, N, K, most, tiled ? 1 : 0, st->stream);
+            rc = st->gemm_rows(x, streamed, y, M, N, K, most, tiled ? 1 : 0, NULL, 0, 0.0f, 0, st->stream);
             *out = KIPP_DELTA(y, parts);
             return rc == 0 ? 0 : refused(error, "gemm_rows", rc);
         }
@@ -573,7 +579,7 @@ static int hip_linear(kipp_runtime *rt, const kipp_rows *rows_in, const kipp_wei
         if (y == NULL) return -1;
         for (int row = 0; row < M; row += 256) {
             int rows = M - row < 256 ? M - row : 256;
-            rc = st->gemm_rows((const char *)x + (size_t)row * K * 2, streamed, y + (size_t)row * N, rows, N, K, 1, tiled ? 1 : 0, st->stream);
+            rc = st->gemm_rows((const char *)x + (size_t)row * K * 2, streamed, y + (size_t)row * N, rows, N, K, 1, tiled ? 1 : 0, NULL, 0, 0.0f, 0, st->stream);
             if (rc != 0) return refused(error, "gemm_rows", rc);
         }
         *out = KIPP_DELTA(y, 1);
@@ -626,11 +632,18 @@ static int hip_gated(kipp_runtime *rt, const kipp_rows *x, const kipp_weight *w,
     }
     if (!tiled) return 0;
     if (kipp_finish_rows(rt, &finished, m, w->k, error) != 0) return -1;
+    if (K % 32 == 0 && st->rows_swiglu_pays(M, (int)w->n, K)) {
+        /* a few dozen rows against a weight with rows enough for every compute unit: the activation at the product's end */
+        int rc = st->gemm_rows_swiglu(finished.data, w->tiles, act->data, M, (int)w->n, K, NULL, 0, 0.0f, 0, st->stream);
+        if (rc != 0) return refused(error, "gemm_rows_swiglu", rc);
+        *done = true;
+        return 0;
+    }
     const int width = 16 * ((inner + 7) / 8); /* columns of the product from paired tiles: 16 for every 8 outputs */
     int parts = st->rows_parts(M, width, K, 12);
     float *y = parts >= 1 ? kipp_scratch(rt, (size_t)parts * m * (size_t)width * sizeof(float), error) : NULL;
     if (y == NULL) return parts >= 1 ? -1 : refused(error, "gemm_rows (its cut)", parts);
-    int rc = st->gemm_rows(finished.data, w->tiles, y, M, width, K, 12, 1, st->stream);
+    int rc = st->gemm_rows(finished.data, w->tiles, y, M, width, K, 12, 1, NULL, 0, 0.0f, 0, st->stream);
     if (rc != 0) return refused(error, "gemm_rows (paired tiles)", rc);
     rc = st->swiglu(y, KIPP_F32, parts, act->data, rt->act_dtype, M, inner, 1, st->stream);
     if (rc != 0) return refused(error, "swiglu (pairs)", rc);

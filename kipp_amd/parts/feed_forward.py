@@ -59,7 +59,10 @@ class GatedMLP:
                                       x_steps_major=scaled and x.steps_major, out_steps_major=major)
             return rt.linear(act, self.w_down, slabs=True, defer=True, x_steps_major=major)
         x = rt.rows_of(x)
-        if ours and w.pairs:
+        if ours and w.pairs and rt.ops.gemm_rows_swiglu_pays(rows, 2 * inner, x.shape[1]):
+            # a few dozen rows against a weight with rows enough for every compute unit: the activation at the product's end
+            rt.ops.gemm_rows_swiglu(x, w.tiles, act)
+        elif ours and w.pairs:
             # streamed from the paired tiles: the columns come out gate tile by gate tile
             rt.ops.swiglu(rt.ops.gemm_rows(x, w.rows, max_parts=12, tiles=w.tiles, pairs=True), act, pairs=True)
         elif w.dtype == x.dtype == torch.bfloat16 and not ours:

@@ -951,6 +951,73 @@ def test_gemm_rows(m, n, k, max_parts):
                            ops.gemm_rows(x.to(DEV), wd, max_parts))
 
 
+ROWS_CUTS = [41, 51, 61, 71, 81, 52, 62, 72, 82]        # 10 x waves of a workgroup + tiles of 16 rows a wave
+
+
+@pytest.mark.parametrize("m", [13, 16, 40, 64, 100, 200])
+@pytest.mark.parametrize("n,k,parts", [(77, 544, 1), (2560, 1024, 3), (509, 2560, 2), (1200, 320, 1)])
+def test_gemm_rows_workgroups_of_any_size(m, n, k, parts):
+    """A workgroup of 4 to 8 waves, one or two tiles of 16 rows of W a wave: an output element is summed over K in the
+    same order whatever the workgroup, so every cut with the same parts of K gives the same bits; with the rows'
+    scales (partial sums of squares, fewer and more than the 16 a lane group takes at once) every row is multiplied
+    by rsqrt(sum / K + eps)."""
+    ops = _ops()
+    rng = np.random.default_rng(m + n + parts)
+    x = torch.tensor(rng.normal(size=(m, k)), dtype=torch.bfloat16).to(DEV)
+    w = torch.tensor(rng.normal(size=(n, k)), dtype=torch.bfloat16).to(DEV)
+    tiles = ops.tile_weight(w)
+    ref = x.double().cpu().numpy() @ w.double().cpu().numpy().T
+    first = None
+    for cut in ROWS_CUTS:
+        out = ops.gemm_rows(x, w, parts, tiles=tiles, cut=cut)
+        assert out.shape == (parts, m, n)
+        if first is None:
+            first = out
+            assert _rel(out.sum(dim=0).cpu().numpy(), ref) < 1e-11
+        assert torch.equal(out, first), f"cut {cut}"
+        assert torch.equal(ops.gemm_rows(x, w, parts, cut=cut), first), f"cut {cut}, from rows"
+    for n_sums in (3, 16, 37):
+        sumsq = torch.tensor(rng.uniform(0.5, 2.0, size=(m, (n_sums + 3) // 4 * 4)), dtype=torch.float32).to(DEV)
+        scale = 1.0 / np.sqrt(sumsq[:, :n_sums].double().cpu().numpy().sum(axis=1) / k + 1e-5)
+        for cut in (0, 51, 82):
+            out = ops.gemm_rows(x, w, parts, tiles=tiles, row_scale=(sumsq, n_sums, 1e-5), cut=cut)
+            assert _rel(out.sum(dim=0).cpu().numpy(), ref * scale[:, None]) < 1e-6, f"{n_sums} sums, cut {cut}"
+    with pytest.raises(ops.KernelError):
+        ops.gemm_rows(x, w, parts, tiles=tiles, cut=31)
+    with pytest.raises(ops.KernelError):
+        ops.gemm_rows(x, w, parts, tiles=tiles, cut=83)
+
+
+@pytest.mark.parametrize("m", [13, 16, 33, 64, 90, 256])
+@pytest.mark.parametrize("inner,k", [(16, 32), (77, 96), (9728, 2560), (1001, 512), (300, 1056)])
+def test_gemm_rows_swiglu(m, inner, k):
+    """The gate and up products of a few dozen rows with the activation at their end, from the paired tiles, K not split:
+    against the plain activation of the exact products, the same bits as the product in one slab followed by the activation
+    kernel, the same from every workgroup size, and with the rows' scales."""
+    ops = _ops()
+    rng = np.random.default_rng(m + inner)
+    x = torch.tensor(rng.normal(size=(m, k)), dtype=torch.bfloat16).to(DEV)
+    w = torch.tensor(rng.normal(size=(2 * inner, k)) / math.sqrt(k), dtype=torch.bfloat16).to(DEV)
+    tiles = ops.tile_weight_pairs(w)
+    gu = x.double().cpu().numpy() @ w.double().cpu().numpy().T
+    ref = plain.silu(gu[:, :inner]) * gu[:, inner:]
+    new = lambda: torch.full((m, inner), 7.0, dtype=torch.bfloat16, device=DEV)
+    got = ops.gemm_rows_swiglu(x, tiles, new())
+    assert _rel(got.float().cpu().numpy(), ref) < 1e-5
+    two = ops.swiglu(ops.gemm_rows(x, w, 1, tiles=tiles, pairs=True), new(), pairs=True)
+    assert torch.equal(got, two)
+    for cut in ROWS_CUTS:
+        assert torch.equal(ops.gemm_rows_swiglu(x, tiles, new(), cut=cut), got), f"cut {cut}"
+    n_sums = 5
+    sumsq = torch.tensor(rng.uniform(0.5, 2.0, size=(m, 8)), dtype=torch.float32).to(DEV)
+    scale = 1.0 / np.sqrt(sumsq[:, :n_sums].double().cpu().numpy().sum(axis=1) / k + 1e-6)
+    gu = gu * scale[:, None]
+    scaled = ops.gemm_rows_swiglu(x, tiles, new(), row_scale=(sumsq, n_sums, 1e-6))
+    assert _rel(scaled.float().cpu().numpy(), plain.silu(gu[:, :inner]) * gu[:, inner:]) < 1e-5
+    assert ops.gemm_rows_swiglu_pays(64, 2 * 9728, 2560) and not ops.gemm_rows_swiglu_pays(128, 2 * 9728, 2560)
+    assert not ops.gemm_rows_swiglu_pays(64, 2 * 512, 2560)          # too few rows of W to go round without splitting K
+
+
 TILE_CUTS = [0, 441, 442, 444, 421, 422, 243, 221, 224, 431, 432, 232, 1421, 1422, 1424, 1221]      # 100 wm + 10 wn + parts (+ 1000: 8 waves; + 2000: whole rounds of those, the rest smaller; + 10000 r: the rest's tile); 0: what the launcher plans
 
 
