@@ -15,9 +15,7 @@
 // A workgroup has 4 to 8 waves (its size is the launch's, not the kernel's), so that the tiles of W can be
 // dealt out to about as many workgroups as there are compute units without splitting K: the SwiGLU end
 // (W = [gate; up] in paired tiles, act = silu(gate) * up written straight from the sums) needs the whole of K
-// in one workgroup.  `RowScale`: X holds the rows of an RMS norm without their scale (bfloat16(x * norm
-// weight)) and the partial sums of x^2 beside them; every row of the product is multiplied by
-// rsqrt(sum / K + eps), which is the product of the normalized row.
+// in one workgroup.
 //
 // v_mfma_f32_16x16x32_bf16: A = W tile (lane: row l % 16, k = 8 (l / 16) + j),
 // B = X^T from LDS (lane: token l % 16, same k), D: lane holds features
@@ -35,12 +33,6 @@ union Frag {
     bf16x8 v;
 };
 
-struct RowScale {               // sumsq == nullptr: none
-    const float* sumsq;         // [M, stride]: `parts` partial sums of squares of each row X was made from
-    int parts, stride;          // stride: parts rounded up to a multiple of 4, so that a lane loads four sums at once
-    float inv_width, eps;
-};
-
 // TILED: W in the streaming layout [tile of 16 rows][step of 32 columns][lane][8 values]
 // (rows padded to whole tiles with zeros, K a multiple of 32), in which a wave's load is
 // one contiguous KB.
@@ -54,7 +46,7 @@ struct RowScale {               // sumsq == nullptr: none
 template <int MT, bool TILED, int DEPTH, int NTW, int END>
 __global__ void __launch_bounds__(MAX_WAVES * KIPP_WAVE) gemm_rows_kernel(
     const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, float* __restrict__ Y, bf16_t* __restrict__ act, int M, int N, int K,
-    int inner, RowScale rs) {
+    int inner) {
     constexpr int CHUNK = 32 * DEPTH;                          // columns of X staged at a time
     constexpr int X_PITCH = CHUNK + 8;                         // bf16 elements per staged row (the pad spreads the banks)
     constexpr int UNITS = MT * 16 * (CHUNK / 8);              // 16-byte units of one staged chunk
@@ -90,40 +82,6 @@ __global__ void __launch_bounds__(MAX_WAVES * KIPP_WAVE) gemm_rows_kernel(
         x_src[i] = X + (size_t)min(r, M - 1) * K + c * 8;
         x_dst[i] = r * X_PITCH + c * 8;
     }
-
-    // the partial sums of the rows' scales, asked for before everything else (they arrive first and are added once
-    // the first weights are on their way): lane group h takes the h-th run of four sums of its tokens
-    // (up to 64 rows; beyond, the kernel is long, registers are short and the sums are fetched at the end)
-    constexpr bool EARLY = MT <= 4;
-    float4 scale_part[EARLY ? MT : 1];
-    if (EARLY && rs.sumsq != nullptr) {
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-            scale_part[mt] = *(const float4*)(rs.sumsq + (size_t)min(16 * mt + l16, M - 1) * rs.stride + min(4 * h, rs.stride - 4));
-        __builtin_amdgcn_sched_barrier(0);
-    }
-    float row_scale[MT];
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) row_scale[mt] = 1.0f;
-    auto finish_scale = [&](bool early) {
-        if (rs.sumsq == nullptr || early != EARLY) return;
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-            const int p = 4 * h;
-            if (!EARLY) scale_part[0] = *(const float4*)(rs.sumsq + (size_t)min(16 * mt + l16, M - 1) * rs.stride + min(4 * h, rs.stride - 4));
-            const float4 part4 = scale_part[EARLY ? mt : 0];
-            float t = 0.0f;
-            t += p < rs.parts ? part4.x : 0.0f;
-            t += p + 1 < rs.parts ? part4.y : 0.0f;
-            t += p + 2 < rs.parts ? part4.z : 0.0f;
-            t += p + 3 < rs.parts ? part4.w : 0.0f;
-            const float* more = rs.sumsq + (size_t)min(16 * mt + l16, M - 1) * rs.stride;
-            for (int q = 16 + h; q < rs.parts; q += 4) t += more[q];        // rows wider than 16 partial sums
-            t += __shfl_xor(t, 16, KIPP_WAVE);     // the four lane groups of a token
-            t += __shfl_xor(t, 32, KIPP_WAVE);
-            row_scale[mt] = 1.0f / sqrtf(t * rs.inv_width + rs.eps);
-        }
-    };
 
     f32x4 acc[NTW][MT];
 #pragma unroll
@@ -164,7 +122,6 @@ __global__ void __launch_bounds__(MAX_WAVES * KIPP_WAVE) gemm_rows_kernel(
 #pragma unroll
         for (int u = 0; u < DEPTH; ++u) fetch_w(u, g_begin * DEPTH + u);
         stage_x(0);
-        finish_scale(true);
         __syncthreads();
         int buf = 0;
         for (int g = g_begin; g + 1 < g_end; ++g) {
@@ -181,8 +138,6 @@ __global__ void __launch_bounds__(MAX_WAVES * KIPP_WAVE) gemm_rows_kernel(
         }
 #pragma unroll
         for (int u = 0; u < DEPTH; ++u) multiply(u, buf);
-    } else {
-        finish_scale(true);
     }
     // the rest of K (less than a chunk), by the last part, straight from global memory
     if (part == parts - 1) {
@@ -204,7 +159,6 @@ __global__ void __launch_bounds__(MAX_WAVES * KIPP_WAVE) gemm_rows_kernel(
             }
         }
     }
-    finish_scale(false);
     if (END == 1) {
         // rows 0..7 of a tile are gates, rows 8..15 the matching ups: they sit 32 lanes apart
 #pragma unroll
@@ -216,7 +170,7 @@ __global__ void __launch_bounds__(MAX_WAVES * KIPP_WAVE) gemm_rows_kernel(
                 float a[4];
 #pragma unroll
                 for (int v = 0; v < 4; ++v) {
-                    const float g = acc[i][mt][v] * row_scale[mt], up = __shfl_xor(g, 32, KIPP_WAVE);
+                    const float g = acc[i][mt][v], up = __shfl_xor(g, 32, KIPP_WAVE);
                     a[v] = g / (1.0f + expf(-g)) * up;
                 }
                 if (h >= 2 || token >= M) continue;
@@ -243,13 +197,12 @@ __global__ void __launch_bounds__(MAX_WAVES * KIPP_WAVE) gemm_rows_kernel(
             const int token = 16 * mt + l16;
             if (token >= M) continue;
             float* y = Y + ((size_t)part * M + token) * N + n;
-            const float sc = row_scale[mt];
             if (n + 3 < N && (N & 3) == 0) {
-                *(float4*)y = make_float4(acc[i][mt][0] * sc, acc[i][mt][1] * sc, acc[i][mt][2] * sc, acc[i][mt][3] * sc);
+                *(float4*)y = make_float4(acc[i][mt][0], acc[i][mt][1], acc[i][mt][2], acc[i][mt][3]);
             } else {
 #pragma unroll
                 for (int v = 0; v < 4; ++v)
-                    if (n + v < N) y[v] = acc[i][mt][v] * sc;
+                    if (n + v < N) y[v] = acc[i][mt][v];
             }
         }
     }
@@ -300,11 +253,9 @@ static int cut_or_plan(int M, int N, int K, int max_parts, int cut, int* tw, int
     return (*tw < MIN_WAVES || *tw > MAX_WAVES || *ntw < 1 || *ntw > 2) ? -1 : 0;
 }
 
-static int sumsq_stride(int parts) { return (parts + 3) / 4 * 4; }
-
 template <int END>
 static int launch(const void* X, const void* W, float* Y, void* act, int M, int N, int K, int inner, int tw, int ntw, int parts,
-                  int tiled, RowScale rs, hipStream_t stream) {
+                  int tiled, hipStream_t stream) {
     const int tiles = (N + 15) / 16;
     dim3 grid((tiles + tw * ntw - 1) / (tw * ntw), parts), block(tw * KIPP_WAVE);
     const int mt = (M + 15) / 16;       // from 65 rows on an even number of 16-row tiles is staged (whole waves move whole runs of units)
@@ -312,10 +263,10 @@ static int launch(const void* X, const void* W, float* Y, void* act, int M, int 
     do {                                                                                                                 \
         if (tiled)                                                                                                       \
             hipLaunchKernelGGL((gemm_rows_kernel<MT, true, DEPTH, NTW, END>), grid, block, 0, stream, (const bf16_t*)X,  \
-                               (const bf16_t*)W, Y, (bf16_t*)act, M, N, K, inner, rs);                                   \
+                               (const bf16_t*)W, Y, (bf16_t*)act, M, N, K, inner);                                       \
         else if (END == 0)                                                                                               \
             hipLaunchKernelGGL((gemm_rows_kernel<MT, false, DEPTH, NTW, 0>), grid, block, 0, stream, (const bf16_t*)X,   \
-                               (const bf16_t*)W, Y, (bf16_t*)act, M, N, K, inner, rs);                                   \
+                               (const bf16_t*)W, Y, (bf16_t*)act, M, N, K, inner);                                       \
         else                                                                                                             \
             return -1;                                                                                                   \
     } while (0)
@@ -361,17 +312,13 @@ int kipp_gemm_rows_parts(int M, int N, int K, int max_parts) {
 
 // Y: float32 [parts, M, N] with parts = kipp_gemm_rows_parts(M, N, K, max_parts).
 // M <= 256, K a multiple of 8; `tiled`: W in the streaming layout (K a multiple of 32).
-// `sumsq` [M, sumsq_parts rounded up to a multiple of 4] (or null): every row of the product is multiplied by
-// rsqrt(sum of the row's sumsq / K + eps).
-int kipp_gemm_rows(const void* X, const void* W, float* Y, int M, int N, int K, int max_parts, int tiled,
-                   const float* sumsq, int sumsq_parts, float eps, int cut, hipStream_t stream) {
+int kipp_gemm_rows(const void* X, const void* W, float* Y, int M, int N, int K, int max_parts, int tiled, int cut,
+                   hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
     if (M > MAX_ROWS || K <= 0 || (K & 7) || max_parts <= 0 || (tiled && (K & 31))) return -1;
-    if (sumsq != nullptr && sumsq_parts <= 0) return -1;
     int tw, ntw, parts;
     if (cut_or_plan(M, N, K, max_parts, cut, &tw, &ntw, &parts) != 0) return -1;
-    RowScale rs = {sumsq, sumsq_parts, sumsq_stride(sumsq_parts), 1.0f / (float)K, eps};
-    return launch<0>(X, W, Y, nullptr, M, N, K, 0, tw, ntw, parts, tiled, rs, stream);
+    return launch<0>(X, W, Y, nullptr, M, N, K, 0, tw, ntw, parts, tiled, stream);
 }
 
 // Whether the product that ends in SwiGLU is taken for this shape: K is not split there, and where the tiles of W are
@@ -389,18 +336,14 @@ int kipp_gemm_rows_swiglu_pays(int M, int two_inner, int K) {
 }
 
 // act: bfloat16 [M, I] = silu(X . gate^T) * (X . up^T); W: the paired tiles of [gate; up] ([2 I, K], tiles of 8 gate rows
-// over the 8 matching up rows, K a multiple of 32).  `sumsq`, `sumsq_parts`, `eps`: as above (both products are scaled
-// before the activation).
-int kipp_gemm_rows_swiglu(const void* X, const void* W, void* act, int M, int two_inner, int K, const float* sumsq,
-                          int sumsq_parts, float eps, int cut, hipStream_t stream) {
+// over the 8 matching up rows, K a multiple of 32).
+int kipp_gemm_rows_swiglu(const void* X, const void* W, void* act, int M, int two_inner, int K, int cut, hipStream_t stream) {
     if (M <= 0 || two_inner <= 0) return 0;
     if (M > MAX_ROWS || K <= 0 || (K & 31) || (two_inner & 1)) return -1;
-    if (sumsq != nullptr && sumsq_parts <= 0) return -1;
     const int inner = two_inner / 2, N = 16 * ((inner + 7) / 8);
     int tw, ntw, parts;
     if (cut_or_plan(M, N, K, 1, cut, &tw, &ntw, &parts) != 0 || parts != 1) return -1;
-    RowScale rs = {sumsq, sumsq_parts, sumsq_stride(sumsq_parts), 1.0f / (float)K, eps};
-    return launch<1>(X, W, nullptr, act, M, N, K, inner, tw, ntw, 1, 1, rs, stream);
+    return launch<1>(X, W, nullptr, act, M, N, K, inner, tw, ntw, 1, 1, stream);
 }
 
 }  // extern "C"

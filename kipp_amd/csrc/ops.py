@@ -561,15 +561,15 @@ def _tiles_ok(tiles, n: int, k: int, what: str) -> int:
     return 1
 
 
-def _row_scale_args(row_scale, m: int, what: str, most_rows: int = 16):
+def _row_scale_args(row_scale, m: int, what: str):
     """(sumsq pointer, parts, eps) of `row_scale` = (sumsq, parts, eps), sumsq float32 [M, parts rounded up to 4]."""
     if row_scale is None:
         return None, 0, 0.0
     sumsq, parts, eps = row_scale
     _dev(sumsq)
-    _need(m <= most_rows and sumsq.dtype == torch.float32 and sumsq.dim() == 2 and parts > 0
+    _need(m <= 16 and sumsq.dtype == torch.float32 and sumsq.dim() == 2 and parts > 0
           and tuple(sumsq.shape) == (m, (parts + 3) // 4 * 4) and sumsq.is_contiguous(),
-          f"{what}: row_scale is (float32 [M, parts rounded up to 4], parts, eps), for at most {most_rows} rows")
+          f"{what}: row_scale is (float32 [M, parts rounded up to 4], parts, eps), for at most 16 rows")
     return _ptr(sumsq), int(parts), float(eps)
 
 
@@ -658,12 +658,12 @@ def scale_rows(rows: torch.Tensor, sumsq: torch.Tensor, parts: int, eps: float, 
 
 
 def gemm_rows(x: torch.Tensor, w: torch.Tensor, max_parts: int = 1, tiles: torch.Tensor = None,
-              pairs: bool = False, row_scale=None, cut: int = 0) -> torch.Tensor:
+              pairs: bool = False, cut: int = 0) -> torch.Tensor:
     """float32 [parts, M, N] whose sum over parts is x . w^T, for 8 < M <= 256 rows
     (any M <= 256 is taken): the rows of x are staged through LDS and shared by
     the waves of a workgroup.  `pairs`: `tiles` is tile_weight_pairs(w), w = [gate; up];
     the product then has `pairs_width(inner)` columns in the order of those tiles
-    (what `swiglu(..., pairs=True)` takes).  `row_scale`: as in `gemm_skinny`, for any number of rows.
+    (what `swiglu(..., pairs=True)` takes).
     `cut` (measurements and tests): 10 x waves of a workgroup (4 to 8) + tiles of 16 rows a wave (1 or 2),
     with exactly `max_parts` parts of K."""
     _dev(x, w)
@@ -679,11 +679,8 @@ def gemm_rows(x: torch.Tensor, w: torch.Tensor, max_parts: int = 1, tiles: torch
     parts = lib.kipp_gemm_rows_parts(m, n, k, int(max_parts)) if not cut else min(int(max_parts), max(1, k // rows_chunk(m)))
     out = torch.empty((parts, m, n), dtype=torch.float32, device=x.device)
     tiled = _tiles_ok(tiles, n, k, "gemm_rows")
-    sumsq, sumsq_parts, eps = _row_scale_args(row_scale, m, "gemm_rows", ROWS_MAX_ROWS)
-    fn = _fn("gemm_rows", "kipp_gemm_rows", [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_int, _c_float,
-                                            _c_int, _c_ptr])
-    _check(fn(_ptr(x), _ptr(tiles if tiled else w), _ptr(out), m, n, k, int(max_parts), tiled, sumsq, sumsq_parts, eps, int(cut),
-              _stream()), "gemm_rows")
+    fn = _fn("gemm_rows", "kipp_gemm_rows", [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr])
+    _check(fn(_ptr(x), _ptr(tiles if tiled else w), _ptr(out), m, n, k, int(max_parts), tiled, int(cut), _stream()), "gemm_rows")
     return out
 
 
@@ -698,9 +695,9 @@ def gemm_rows_swiglu_pays(m: int, two_inner: int, k: int) -> bool:
     return bool(build.library("gemm_rows").kipp_gemm_rows_swiglu_pays(int(m), int(two_inner), int(k)))
 
 
-def gemm_rows_swiglu(x: torch.Tensor, tiles: torch.Tensor, out: torch.Tensor, row_scale=None, cut: int = 0) -> torch.Tensor:
+def gemm_rows_swiglu(x: torch.Tensor, tiles: torch.Tensor, out: torch.Tensor, cut: int = 0) -> torch.Tensor:
     """out[M, I] (bfloat16) = silu(x . w_gate^T) * (x . w_up^T) for up to 256 rows; `tiles` = tile_weight_pairs([gate; up]).
-    `row_scale`, `cut`: as in `gemm_rows`."""
+    `cut`: as in `gemm_rows`."""
     _dev(x, tiles, out)
     m, k = x.shape
     inner = out.shape[1]
@@ -708,9 +705,8 @@ def gemm_rows_swiglu(x: torch.Tensor, tiles: torch.Tensor, out: torch.Tensor, ro
           and x.is_contiguous(), "gemm_rows_swiglu: bfloat16 operands and output")
     _need(0 < m <= ROWS_MAX_ROWS and k % 32 == 0 and out.shape[0] == m, "gemm_rows_swiglu: at most 256 rows and K a multiple of 32")
     _tiles_ok(tiles, pairs_width(inner), k, "gemm_rows_swiglu")
-    sumsq, sumsq_parts, eps = _row_scale_args(row_scale, m, "gemm_rows_swiglu", ROWS_MAX_ROWS)
-    fn = _fn("gemm_rows", "kipp_gemm_rows_swiglu", [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_int, _c_float, _c_int, _c_ptr])
-    _check(fn(_ptr(x), _ptr(tiles), _ptr(out), m, 2 * inner, k, sumsq, sumsq_parts, eps, int(cut), _stream()), "gemm_rows_swiglu")
+    fn = _fn("gemm_rows", "kipp_gemm_rows_swiglu", [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr])
+    _check(fn(_ptr(x), _ptr(tiles), _ptr(out), m, 2 * inner, k, int(cut), _stream()), "gemm_rows_swiglu")
     return out
 
 

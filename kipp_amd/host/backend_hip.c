@@ -50,8 +50,8 @@ typedef int (*fn_skinny_parts)(int, int, int);
 typedef int (*fn_gemm_skinny)(const void *, const void *, float *, int, int, int, int, int, const float *, int, float, float *, const float *,
                               void *, float *, int, int, hipStream_t);
 typedef int (*fn_rows_parts)(int, int, int, int);
-typedef int (*fn_gemm_rows)(const void *, const void *, float *, int, int, int, int, int, const float *, int, float, int, hipStream_t);
-typedef int (*fn_gemm_rows_swiglu)(const void *, const void *, void *, int, int, int, const float *, int, float, int, hipStream_t);
+typedef int (*fn_gemm_rows)(const void *, const void *, float *, int, int, int, int, int, int, hipStream_t);
+typedef int (*fn_gemm_rows_swiglu)(const void *, const void *, void *, int, int, int, int, hipStream_t);
 typedef int (*fn_skinny_swiglu)(const void *, const void *, void *, int, int, int, int, const float *, int, float, int, int, hipStream_t);
 typedef int (*fn_int_int)(int);
 typedef int (*fn_int3)(int, int, int);
@@ -563,7 +563,7 @@ static int hip_linear(kipp_runtime *rt, const kipp_rows *rows_in, const kipp_wei
             int most = max_parts > 12 ? 12 : max_parts, parts = st->rows_parts(M, N, K, most);
             float *y = parts >= 1 ? kipp_scratch(rt, (size_t)parts * count * 4, error) : NULL;
             if (y == NULL) return parts >= 1 ? -1 : refused(error, "gemm_rows (its cut)", parts);
-            rc = st->gemm_rows(x, streamed, y, M, N, K, most, tiled ? 1 : 0, NULL, 0, 0.0f, 0, st->stream);
+            rc = st->gemm_rows(x, streamed, y, M, N, K, most, tiled ? 1 : 0, 0, st->stream);
             *out = KIPP_DELTA(y, parts);
             return rc == 0 ? 0 : refused(error, "gemm_rows", rc);
         }
@@ -579,7 +579,7 @@ static int hip_linear(kipp_runtime *rt, const kipp_rows *rows_in, const kipp_wei
         if (y == NULL) return -1;
         for (int row = 0; row < M; row += 256) {
             int rows = M - row < 256 ? M - row : 256;
-            rc = st->gemm_rows((const char *)x + (size_t)row * K * 2, streamed, y + (size_t)row * N, rows, N, K, 1, tiled ? 1 : 0, NULL, 0, 0.0f, 0, st->stream);
+            rc = st->gemm_rows((const char *)x + (size_t)row * K * 2, streamed, y + (size_t)row * N, rows, N, K, 1, tiled ? 1 : 0, 0, st->stream);
             if (rc != 0) return refused(error, "gemm_rows", rc);
         }
         *out = KIPP_DELTA(y, 1);
@@ -634,7 +634,7 @@ static int hip_gated(kipp_runtime *rt, const kipp_rows *x, const kipp_weight *w,
     if (kipp_finish_rows(rt, &finished, m, w->k, error) != 0) return -1;
     if (K % 32 == 0 && st->rows_swiglu_pays(M, (int)w->n, K)) {
         /* a few dozen rows against a weight with rows enough for every compute unit: the activation at the product's end */
-        int rc = st->gemm_rows_swiglu(finished.data, w->tiles, act->data, M, (int)w->n, K, NULL, 0, 0.0f, 0, st->stream);
+        int rc = st->gemm_rows_swiglu(finished.data, w->tiles, act->data, M, (int)w->n, K, 0, st->stream);
         if (rc != 0) return refused(error, "gemm_rows_swiglu", rc);
         *done = true;
         return 0;
@@ -643,7 +643,7 @@ static int hip_gated(kipp_runtime *rt, const kipp_rows *x, const kipp_weight *w,
     int parts = st->rows_parts(M, width, K, 12);
     float *y = parts >= 1 ? kipp_scratch(rt, (size_t)parts * m * (size_t)width * sizeof(float), error) : NULL;
     if (y == NULL) return parts >= 1 ? -1 : refused(error, "gemm_rows (its cut)", parts);
-    int rc = st->gemm_rows(finished.data, w->tiles, y, M, width, K, 12, 1, NULL, 0, 0.0f, 0, st->stream);
+    int rc = st->gemm_rows(finished.data, w->tiles, y, M, width, K, 12, 1, 0, st->stream);
     if (rc != 0) return refused(error, "gemm_rows (paired tiles)", rc);
     rc = st->swiglu(y, KIPP_F32, parts, act->data, rt->act_dtype, M, inner, 1, st->stream);
     if (rc != 0) return refused(error, "swiglu (pairs)", rc);

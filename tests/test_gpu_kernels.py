@@ -958,9 +958,7 @@ ROWS_CUTS = [41, 51, 61, 71, 81, 52, 62, 72, 82]        # 10 x waves of a workgr
 @pytest.mark.parametrize("n,k,parts", [(77, 544, 1), (2560, 1024, 3), (509, 2560, 2), (1200, 320, 1)])
 def test_gemm_rows_workgroups_of_any_size(m, n, k, parts):
     """A workgroup of 4 to 8 waves, one or two tiles of 16 rows of W a wave: an output element is summed over K in the
-    same order whatever the workgroup, so every cut with the same parts of K gives the same bits; with the rows'
-    scales (partial sums of squares, fewer and more than the 16 a lane group takes at once) every row is multiplied
-    by rsqrt(sum / K + eps)."""
+    same order whatever the workgroup, so every cut with the same parts of K gives the same bits."""
     ops = _ops()
     rng = np.random.default_rng(m + n + parts)
     x = torch.tensor(rng.normal(size=(m, k)), dtype=torch.bfloat16).to(DEV)
@@ -976,12 +974,6 @@ def test_gemm_rows_workgroups_of_any_size(m, n, k, parts):
             assert _rel(out.sum(dim=0).cpu().numpy(), ref) < 1e-11
         assert torch.equal(out, first), f"cut {cut}"
         assert torch.equal(ops.gemm_rows(x, w, parts, cut=cut), first), f"cut {cut}, from rows"
-    for n_sums in (3, 16, 37):
-        sumsq = torch.tensor(rng.uniform(0.5, 2.0, size=(m, (n_sums + 3) // 4 * 4)), dtype=torch.float32).to(DEV)
-        scale = 1.0 / np.sqrt(sumsq[:, :n_sums].double().cpu().numpy().sum(axis=1) / k + 1e-5)
-        for cut in (0, 51, 82):
-            out = ops.gemm_rows(x, w, parts, tiles=tiles, row_scale=(sumsq, n_sums, 1e-5), cut=cut)
-            assert _rel(out.sum(dim=0).cpu().numpy(), ref * scale[:, None]) < 1e-6, f"{n_sums} sums, cut {cut}"
     with pytest.raises(ops.KernelError):
         ops.gemm_rows(x, w, parts, tiles=tiles, cut=31)
     with pytest.raises(ops.KernelError):
@@ -993,7 +985,7 @@ def test_gemm_rows_workgroups_of_any_size(m, n, k, parts):
 def test_gemm_rows_swiglu(m, inner, k):
     """The gate and up products of a few dozen rows with the activation at their end, from the paired tiles, K not split:
     against the plain activation of the exact products, the same bits as the product in one slab followed by the activation
-    kernel, the same from every workgroup size, and with the rows' scales."""
+    kernel, and the same from every workgroup size."""
     ops = _ops()
     rng = np.random.default_rng(m + inner)
     x = torch.tensor(rng.normal(size=(m, k)), dtype=torch.bfloat16).to(DEV)
@@ -1008,12 +1000,6 @@ def test_gemm_rows_swiglu(m, inner, k):
     assert torch.equal(got, two)
     for cut in ROWS_CUTS:
         assert torch.equal(ops.gemm_rows_swiglu(x, tiles, new(), cut=cut), got), f"cut {cut}"
-    n_sums = 5
-    sumsq = torch.tensor(rng.uniform(0.5, 2.0, size=(m, 8)), dtype=torch.float32).to(DEV)
-    scale = 1.0 / np.sqrt(sumsq[:, :n_sums].double().cpu().numpy().sum(axis=1) / k + 1e-6)
-    gu = gu * scale[:, None]
-    scaled = ops.gemm_rows_swiglu(x, tiles, new(), row_scale=(sumsq, n_sums, 1e-6))
-    assert _rel(scaled.float().cpu().numpy(), plain.silu(gu[:, :inner]) * gu[:, inner:]) < 1e-5
     assert ops.gemm_rows_swiglu_pays(64, 2 * 9728, 2560) and not ops.gemm_rows_swiglu_pays(128, 2 * 9728, 2560)
     assert not ops.gemm_rows_swiglu_pays(64, 2 * 512, 2560)          # too few rows of W to go round without splitting K
 
