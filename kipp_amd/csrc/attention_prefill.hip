@@ -614,31 +614,52 @@ __global__ void __launch_bounds__(THREADS, 2) attention_prefill_dma_kernel(
 }
 #endif  // HEAD_DIM == 128
 
-// The cuts of a row's keys, added in order: out = sum_s acc_s 2^(m_s - m) / sum_s l_s 2^(m_s - m).  A wave a
-// (row, head).  How many cuts a row has follows from the last position of the tile of query rows it lies in (every
-// row of a tile has the tile's cuts; a cut that begins behind a row's own position holds nothing: m = -inf, l = 0).
-__global__ void __launch_bounds__(KIPP_WAVE) attention_prefill_merge_kernel(
+// The cuts of a row's keys, added in order: out = sum_s acc_s 2^(m_s - m) / sum_s l_s 2^(m_s - m).  A workgroup takes
+// MERGE_HEADS heads of a row, a thread four neighbouring elements of one of them; the cuts are read four at a time, all
+// asked for before the first is added.  How many cuts a row has follows from the last position of the tile of query
+// rows it lies in (every row of a tile has the tile's cuts; a cut that begins behind a row's own position holds
+// nothing: m = -inf, l = 0).
+#define MERGE_LANES (HEAD_DIM / 4)               // threads of a head
+#define MERGE_HEADS (256 / MERGE_LANES > 0 ? 256 / MERGE_LANES : 1)
+__global__ void __launch_bounds__(MERGE_HEADS * MERGE_LANES) attention_prefill_merge_kernel(
     const float* __restrict__ part_acc, const float* __restrict__ part_ml, bf16_t* __restrict__ out,
     const int32_t* __restrict__ merge_rows, const int32_t* __restrict__ merge_cuts, int n_q, int max_splits) {
     // rows on the grid's x, which takes as many as a step has (y ends at 65,535)
-    const int head = blockIdx.y, lane = threadIdx.x;
+    const int head = blockIdx.y * MERGE_HEADS + threadIdx.x / MERGE_LANES, dcol = 4 * (threadIdx.x % MERGE_LANES);
+    if (head >= n_q) return;
     const int row = merge_rows[blockIdx.x], cuts = merge_cuts[blockIdx.x];
     const size_t slot0 = ((size_t)row * n_q + head) * max_splits;
+    const float2* ml = (const float2*)part_ml + slot0;
     float m = -INFINITY;
-    for (int s = 0; s < cuts; ++s) m = fmaxf(m, part_ml[(slot0 + s) * 2]);
+    for (int s0 = 0; s0 < cuts; s0 += 4) {
+        float ms[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) ms[q] = s0 + q < cuts ? ml[s0 + q].x : -INFINITY;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) m = fmaxf(m, ms[q]);
+    }
     float denom = 0.0f;
-    for (int s = 0; s < cuts; ++s) {
-        const float ms = part_ml[(slot0 + s) * 2];
-        if (ms != -INFINITY) denom += part_ml[(slot0 + s) * 2 + 1] * exp2f(ms - m);
-    }
-    for (int dcol = lane; dcol < HEAD_DIM; dcol += KIPP_WAVE) {
-        float a = 0.0f;
-        for (int s = 0; s < cuts; ++s) {
-            const float ms = part_ml[(slot0 + s) * 2];
-            if (ms != -INFINITY) a += part_acc[(slot0 + s) * HEAD_DIM + dcol] * exp2f(ms - m);
+    f32x4 a = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
+    for (int s0 = 0; s0 < cuts; s0 += 4) {
+        float2 one[4];
+        f32x4 acc[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int s = min(s0 + q, cuts - 1);
+            one[q] = ml[s];
+            acc[q] = *(const f32x4*)(part_acc + (slot0 + s) * HEAD_DIM + dcol);
         }
-        out[((size_t)row * n_q + head) * HEAD_DIM + dcol] = f32_to_bf16(a / denom);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            if (s0 + q < cuts && one[q].x != -INFINITY) {
+                const float w = exp2f(one[q].x - m);
+                denom += one[q].y * w;
+                a += acc[q] * w;
+            }
+        }
     }
+    bf16_t* o = out + ((size_t)row * n_q + head) * HEAD_DIM + dcol;
+    *(u32x2*)o = (u32x2){pack_bf16(a[0] / denom, a[1] / denom), pack_bf16(a[2] / denom, a[3] / denom)};
 }
 
 extern "C" {
@@ -687,7 +708,7 @@ int kipp_attention_prefill(const void* q, const void* k_cache, const void* v_cac
                        positions, block_table, max_blocks, n_q, n_kv, page, scale_log2e, window, tile_rows, item_split,
                        split_keys, part_acc, part_ml, max_splits);
     if (split_keys > 0 && n_merge > 0)
-        hipLaunchKernelGGL(attention_prefill_merge_kernel, dim3(n_merge, n_q), dim3(KIPP_WAVE), 0, stream, part_acc, part_ml,
+        hipLaunchKernelGGL(attention_prefill_merge_kernel, dim3(n_merge, (n_q + MERGE_HEADS - 1) / MERGE_HEADS), dim3(MERGE_HEADS * MERGE_LANES), 0, stream, part_acc, part_ml,
                            (bf16_t*)out, merge_rows, merge_cuts, n_q, max_splits);
     return KIPP_LAUNCH_CHECK();
 }

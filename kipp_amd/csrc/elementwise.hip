@@ -166,7 +166,13 @@ __global__ void residual_add_kernel(float* __restrict__ x, const TD* __restrict_
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) {
         float v = x[i];
-        for (int p = 0; p < parts; ++p) v += load_f(delta, p * n + i);
+        for (int p0 = 0; p0 < parts; p0 += 4) {   // slabs in order; four at a time, all asked for before the first is added
+            float d[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) d[q] = p0 + q < parts ? load_f(delta, (p0 + q) * n + i) : 0.0f;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) v += d[q];
+        }
         x[i] = v;
     }
 }
@@ -185,9 +191,18 @@ __global__ void swiglu_kernel(const TI* __restrict__ gu, TO* __restrict__ out, i
     const size_t slab = (total / inner) * width;
     const size_t at_g = t * width + (pairs ? 16 * (i >> 3) + (i & 7) : i), at_u = at_g + (pairs ? 8 : inner);
     float g = 0.0f, u = 0.0f;
-    for (int p = 0; p < parts; ++p) {   // slabs of a split product, in order
-        g += load_f(gu, p * slab + at_g);
-        u += load_f(gu, p * slab + at_u);
+    for (int p0 = 0; p0 < parts; p0 += 4) {   // slabs of a split product, in order; four at a time, all asked for before the first is added
+        float gs[4], us[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            gs[q] = p0 + q < parts ? load_f(gu, (p0 + q) * slab + at_g) : 0.0f;
+            us[q] = p0 + q < parts ? load_f(gu, (p0 + q) * slab + at_u) : 0.0f;
+        }
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            g += gs[q];
+            u += us[q];
+        }
     }
     store_f(out, idx, g / (1.0f + expf(-g)) * u);
 }

@@ -167,10 +167,28 @@ __global__ void __launch_bounds__(HEADS_PER_BLOCK * KIPP_WAVE) qk_norm_rope_kv_r
             const int slot = min(s0 + u * waves, n_slots - 1);
             const TI* src = qkv + row + (size_t)slot * D + lane;
 #pragma unroll
-            for (int c = 0; c < NC; ++c) {
-                v[u][c] = load_f(src, c * KIPP_WAVE);
-                if (SLABS)
-                    for (int p = 1; p < parts; ++p) v[u][c] += load_f(src, p * part_stride + c * KIPP_WAVE);
+            for (int c = 0; c < NC; ++c) v[u][c] = load_f(src, c * KIPP_WAVE);
+        }
+        if (SLABS) {
+            // the other slabs, four at a time: all their loads are asked for before the first is added (slabs in order)
+            for (int p0 = 1; p0 < parts; p0 += 4) {
+                float more[4][BATCH][NC];
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+#pragma unroll
+                    for (int u = 0; u < BATCH; ++u) {
+                        const int slot = min(s0 + u * waves, n_slots - 1);
+                        const TI* src = qkv + row + (size_t)slot * D + lane;
+#pragma unroll
+                        for (int c = 0; c < NC; ++c)
+                            more[q][u][c] = p0 + q < parts ? load_f(src, (size_t)(p0 + q) * part_stride + c * KIPP_WAVE) : 0.0f;
+                    }
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+#pragma unroll
+                    for (int u = 0; u < BATCH; ++u)
+#pragma unroll
+                        for (int c = 0; c < NC; ++c) v[u][c] += more[q][u][c];
             }
         }
 #pragma unroll
