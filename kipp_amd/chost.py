@@ -167,6 +167,7 @@ def library(variant: str = "gpu") -> ctypes.CDLL:
         lib.kipp_test_fail_forward_after.argtypes, lib.kipp_test_fail_forward_after.restype = [vp, ctypes.c_int], None
         lib.kipp_error_code_name.argtypes, lib.kipp_error_code_name.restype = [ctypes.c_int], ctypes.c_char_p
         lib.kipp_test_graph_replays.argtypes, lib.kipp_test_graph_replays.restype = [vp], ctypes.c_uint64
+        lib.kipp_test_cut_attention_steps.argtypes, lib.kipp_test_cut_attention_steps.restype = [vp], ctypes.c_uint64
         lib.kipp_test_session_pages.argtypes = [vp, u32, ctypes.POINTER(ctypes.c_int32), sz]
         lib.kipp_test_session_pages.restype = sz
         _libs[variant] = lib
@@ -277,6 +278,11 @@ class CModel:
     def graph_replays(self) -> int:
         """Steps that ran from a recording since the model was opened."""
         return int(self.lib.kipp_test_graph_replays(self.handle))
+
+    @property
+    def cut_attention_steps(self) -> int:
+        """Work lists of prompt portions whose keys were cut over more workgroups since the model was opened."""
+        return int(self.lib.kipp_test_cut_attention_steps(self.handle))
 
     def session(self, capacity: int = 0) -> CSession:
         handle, error = ctypes.c_void_p(), _Error()

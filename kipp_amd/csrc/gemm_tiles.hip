@@ -399,6 +399,23 @@ static double cut_cost(int M, int cols, int steps, int end, int shape, int parts
     return rounds * (kFixed[shape] + kStep[shape] * ((steps + parts - 1) / parts)) + 1.0 * (parts - 1);
 }
 
+// Workgroups of 8 waves (wave tiles of 4 x 2, four across: the 256 x 256 tile with two waves a SIMD) for the whole rounds of
+// 256 tiles, and the columns that are left, which would hold every compute unit for a round that few of them have a tile
+// in, in smaller tiles: 8 waves on half the rows and columns, or (`rest` = 1, 2, 3) 4 waves on 256 x 64, 128 x 128, 128 x 64.
+// Without whole rounds, or with nothing left, one cut of the 8-wave tile.
+static int whole_rounds_then_rest(int M, int cols, int end, int rest, Cut* cuts) {
+    cuts[0] = {4, 2, 1, 0, cols, 4};
+    const int tm = 256, tn = (end == END_SWIGLU ? 16 : 32) * 2 * 4;
+    const int tiles_m = (M + tm - 1) / tm;
+    const long long whole = ((long long)tiles_m * (cols / tn)) / 256 * 256;
+    const int first_cols = (int)(whole / tiles_m) * tn;
+    if (first_cols <= 0 || first_cols >= cols) return 1;
+    cuts[0].col_end = first_cols;
+    static const int tiles[4][3] = {{2, 2, 4}, {4, 2, 2}, {2, 4, 2}, {2, 2, 2}};
+    cuts[1] = {tiles[rest & 3][0], tiles[rest & 3][1], 1, first_cols, cols, tiles[rest & 3][2]};
+    return 2;
+}
+
 // Up to two cuts, side by side in the output's columns.  The float32 end takes one cut, whose parts of K may be
 // more than one.  The bfloat16 ends cannot split K; where whole rounds of the largest tile leave a rest of tiles
 // that would hold the 256 units for another whole round, the rest of the columns is cut into smaller tiles.
@@ -416,6 +433,11 @@ static int plan(int M, int N, int K, int end, int max_parts, Cut* cuts) {
                 cuts[0] = {kShapes[s][0], kShapes[s][1], parts, 0, cols};
             }
         }
+    }
+    if (end == END_SWIGLU && M >= 512) {
+        // from 512 rows on the 8-wave tile is the faster one for this end, measured at 512, 1,024 and 2,048 rows of the 4B
+        // shape (57 against 65 us, 115 against 114, 196 against 209); an element's sum does not depend on the tile
+        return whole_rounds_then_rest(M, cols, end, 0, cuts);
     }
     if (end != END_SLABS) {
         // whole rounds of the largest tile first, the rest of the columns in smaller tiles
@@ -504,21 +526,7 @@ int kipp_gemm_tiles(const void* X, const void* W, void* Y, int M, int N, int K, 
         const int rest_code = force / 10000;         // + 10000 r: the tile of the columns that + 2000 leaves (below)
         force %= 10000;
         cuts[0] = {(force / 100) % 10, (force / 10) % 10, force % 10, 0, cols, force >= 1000 ? 4 : 2};
-        if (force >= 2000 && end != END_SLABS) {
-            // + 2000: 8 waves as with + 1000, but only the whole rounds of 256 tiles in this cut; the columns that
-            // are left, which would hold every compute unit for a round that few of them have a tile in, go to
-            // smaller tiles: 8 waves on half the rows and columns, or (r = 1, 2, 3) 4 waves on 256 x 64, 128 x 128, 128 x 64
-            const int tm = 64 * cuts[0].wm, tn = (end == END_SWIGLU ? 16 : 32) * cuts[0].wn * 4;
-            const int tiles_m = (M + tm - 1) / tm;
-            const long long whole = ((long long)tiles_m * (cols / tn)) / 256 * 256;
-            const int first_cols = (int)(whole / tiles_m) * tn;
-            if (first_cols > 0 && first_cols < cols) {
-                n_cuts = 2;
-                cuts[0].col_end = first_cols;
-                static const int rest[4][3] = {{2, 2, 4}, {4, 2, 2}, {2, 4, 2}, {2, 2, 2}};
-                cuts[1] = {rest[rest_code & 3][0], rest[rest_code & 3][1], 1, first_cols, cols, rest[rest_code & 3][2]};
-            }
-        }
+        if (force >= 2000 && end != END_SLABS) n_cuts = whole_rounds_then_rest(M, cols, end, rest_code, cuts);   // + 2000 (above)
     }
     for (int c = 0; c < n_cuts; ++c) {
         const Cut& cut = cuts[c];

@@ -102,6 +102,7 @@ struct kipp_runtime {
     void (*graph_free)(kipp_runtime *rt, void *graph);
     bool recording;
     uint64_t generation; /* counts moves of buffers that recordings hold addresses of */
+    uint64_t cut_attention_steps; /* work lists of portions whose keys were cut over more workgroups (for tests) */
 
     /* Optional (NULL: none): what a table has to put right after a step that failed. */
     void (*after_failed_step)(kipp_runtime *rt);

@@ -114,6 +114,7 @@ typedef struct {
     attention_variant variants[8];
     size_t variant_count;
     uint64_t generic_attention_launches; /* bfloat16 attention that fell to the generic kernel */
+    int compute_units;     /* of the device, for plans that fill it */
 } hip_state;
 
 static int hip_bad(kipp_error *error, hipError_t code, const char *what) {
@@ -687,50 +688,110 @@ static int hip_qk_norm_rope_kv(kipp_runtime *rt, const kipp_delta *qkv, void *q_
 }
 
 static int compare_items(const void *a, const void *b) {
-    const int32_t *x = a, *y = b; /* (last key, entry, tile): the longest key range first, then in order */
+    const int32_t *x = a, *y = b; /* (keys, entry, tile, cut): the longest key range first, then in order */
     if (x[0] != y[0]) return x[0] > y[0] ? -1 : 1;
     if (x[1] != y[1]) return x[1] < y[1] ? -1 : 1;
-    return x[2] < y[2] ? -1 : (x[2] > y[2]);
+    if (x[2] != y[2]) return x[2] < y[2] ? -1 : 1;
+    return x[3] < y[3] ? -1 : (x[3] > y[3]);
 }
 
+#define PREFILL_MIN_CUT 512 /* fewest keys of a cut of the keys (below, the merge costs more than the cut gains) */
+
 /* The work list of the kernel for portions: (entry, tile of its query rows) for every entry that brings more than one
- * token, the longest key range first.  Made by the first attention of a forward pass, shared by the others. */
-static int prefill_work(kipp_runtime *rt, kipp_batch *batch, int tile_rows, kipp_error *error) {
-    if (batch->item_seq != NULL) return 0;
-    size_t count = 0;
+ * token, the longest key range first.  A workgroup walks all keys its tile sees.  Where the tiles times the heads are
+ * fewer workgroups than two a compute unit and the contexts are long (a portion of a few hundred rows behind thousands of
+ * keys), the keys are cut as well, at multiples of a length chosen so that the GPU is filled about twice: an item is then
+ * (entry, tile, cut), and the cuts of a row are merged in order afterwards.  Made by the first attention of a forward pass,
+ * shared by the others of the same geometry. */
+static int prefill_work(kipp_runtime *rt, kipp_batch *batch, int tile_rows, const kipp_attention_geometry *g, kipp_error *error) {
+    hip_state *st = rt->state;
+    const uint64_t made_for = ((uint64_t)g->n_q << 40) ^ ((uint64_t)g->head_dim << 24) ^ ((uint64_t)g->window << 1) ^ 1u;
+    if (batch->item_seq != NULL && batch->items_of == made_for) return 0;
+    size_t tiles = 0;
+    int longest = 0;
     for (uint32_t i = 0; i < batch->n_seqs; ++i) {
-        if (batch->h_q_len[i] > 1) count += (size_t)(batch->h_q_len[i] + tile_rows - 1) / (size_t)tile_rows;
+        if (batch->h_q_len[i] <= 1) continue;
+        tiles += (size_t)(batch->h_q_len[i] + tile_rows - 1) / (size_t)tile_rows;
+        if (batch->h_ctx_len[i] > longest) longest = batch->h_ctx_len[i]; /* the last tile's last key + 1 */
     }
-    int32_t *items = malloc((count ? count : 1) * 3 * sizeof(int32_t)), *lists = malloc((count ? count : 1) * 2 * sizeof(int32_t));
+    int cut_keys = 0;
+    const size_t workgroups = tiles * g->n_q, units = (size_t)st->compute_units;
+    if (g->window == 0 && tiles != 0 && workgroups < 2 * units) {
+        const size_t want = (2 * units + workgroups - 1) / workgroups;
+        cut_keys = (int)((((size_t)longest + want - 1) / want + 63) / 64 * 64);
+        if (cut_keys < PREFILL_MIN_CUT) cut_keys = PREFILL_MIN_CUT;
+        if (longest <= cut_keys) cut_keys = 0;
+    }
+    size_t count = 0, merged = 0;
+    for (uint32_t i = 0; i < batch->n_seqs; ++i) {
+        int n = batch->h_q_len[i], ctx = batch->h_ctx_len[i];
+        if (n <= 1) continue;
+        for (int t = 0; t * tile_rows < n; ++t) {
+            int last_row = (t + 1) * tile_rows < n ? (t + 1) * tile_rows : n;
+            count += cut_keys ? (size_t)((ctx - n + last_row - 1) / cut_keys + 1) : 1;
+            merged += (size_t)(last_row - t * tile_rows);
+        }
+    }
+    const size_t ints = (count ? count : 1) * 3 + (merged ? merged : 1) * 2;
+    int32_t *items = malloc((count ? count : 1) * 4 * sizeof(int32_t)), *lists = malloc(ints * sizeof(int32_t));
     if (items == NULL || lists == NULL) {
         free(items);
         free(lists);
         return kipp_fail(error, KIPP_ERROR_MEMORY, "out of memory");
     }
-    size_t at = 0;
+    int32_t *rows_of = lists + 3 * count, *cuts_of = rows_of + merged;
+    size_t at = 0, row_at = 0;
+    uint32_t most = 1;
     for (uint32_t i = 0; i < batch->n_seqs; ++i) {
         int n = batch->h_q_len[i], ctx = batch->h_ctx_len[i];
         if (n <= 1) continue;
-        for (int t = 0; t * tile_rows < n; ++t, ++at) {
+        for (int t = 0; t * tile_rows < n; ++t) {
             int last_row = (t + 1) * tile_rows < n ? (t + 1) * tile_rows : n;
-            items[3 * at] = ctx - n + last_row - 1;
-            items[3 * at + 1] = (int32_t)i;
-            items[3 * at + 2] = t;
+            int last = ctx - n + last_row - 1; /* the last key the tile sees */
+            int cuts = cut_keys ? last / cut_keys + 1 : 1;
+            for (int c = 0; c < cuts; ++c, ++at) {
+                int end = cut_keys && (c + 1) * cut_keys < last + 1 ? (c + 1) * cut_keys : last + 1;
+                items[4 * at] = cut_keys ? end - c * cut_keys : last; /* the keys it walks (uncut: the last key, as good an order) */
+                items[4 * at + 1] = (int32_t)i;
+                items[4 * at + 2] = t;
+                items[4 * at + 3] = c;
+            }
+            if ((uint32_t)cuts > most) most = (uint32_t)cuts;
+            for (int r = t * tile_rows; r < last_row; ++r, ++row_at) {
+                rows_of[row_at] = batch->h_q_start[i] + r;
+                cuts_of[row_at] = cuts;
+            }
         }
     }
-    qsort(items, count, 3 * sizeof(int32_t), compare_items);
+    qsort(items, count, 4 * sizeof(int32_t), compare_items);
     for (size_t i = 0; i < count; ++i) {
-        lists[i] = items[3 * i + 1];
-        lists[count + i] = items[3 * i + 2];
+        lists[i] = items[4 * i + 1];
+        lists[count + i] = items[4 * i + 2];
+        lists[2 * count + i] = items[4 * i + 3];
     }
-    int32_t *device = kipp_scratch(rt, (count ? count : 1) * 2 * sizeof(int32_t), error);
-    int rc = device == NULL ? -1 : hip_upload(rt, device, lists, count * 2 * sizeof(int32_t), error);
+    int32_t *device = kipp_scratch(rt, ints * sizeof(int32_t), error);
+    int rc = device == NULL ? -1 : hip_upload(rt, device, lists, ints * sizeof(int32_t), error);
     free(items);
     free(lists);
     if (rc != 0) return -1;
     batch->item_seq = device;
     batch->item_tile = device + count;
+    batch->item_cut = device + 2 * count;
+    batch->merge_rows = device + 3 * count;
+    batch->merge_cuts = batch->merge_rows + merged;
     batch->n_items = (uint32_t)count;
+    batch->n_merge = (uint32_t)merged;
+    batch->cut_keys = (uint32_t)cut_keys;
+    batch->most_cuts = most;
+    batch->cut_acc = batch->cut_ml = NULL;
+    if (cut_keys) {
+        ++rt->cut_attention_steps;
+        const size_t slots = (size_t)batch->n_tokens * g->n_q * most;
+        batch->cut_acc = kipp_scratch(rt, slots * g->head_dim * sizeof(float), error);
+        batch->cut_ml = kipp_scratch(rt, slots * 2 * sizeof(float), error);
+        if (batch->cut_acc == NULL || batch->cut_ml == NULL) return -1;
+    }
+    batch->items_of = made_for;
     return 0;
 }
 
@@ -841,10 +902,13 @@ static int hip_attention(kipp_runtime *rt, const void *q, const kipp_cache_view 
     attention_variant *v = variant_of(st, g->head_dim, group, error);
     if (v == NULL) return -1;
     if (batch->n_portions != 0) {
-        if (prefill_work(rt, batch, v->prefill_rows, error) != 0) return -1;
+        if (prefill_work(rt, batch, v->prefill_rows, g, error) != 0) return -1;
+        const bool cut = batch->cut_keys != 0;
         rc = v->prefill(q, cache->k, cache->v, out, batch->item_seq, batch->item_tile, batch->q_start, batch->q_len, batch->positions, table,
                         (int)batch->max_blocks, (int)batch->n_items, (int)g->n_q, (int)g->n_kv, (int)g->head_dim, (int)page, g->scale,
-                        (int)g->window, v->prefill_rows, NULL, 0, NULL, NULL, 0, NULL, NULL, 0, st->stream);
+                        (int)g->window, v->prefill_rows, cut ? batch->item_cut : NULL, (int)batch->cut_keys, batch->cut_acc, batch->cut_ml,
+                        cut ? (int)batch->most_cuts : 0, cut ? batch->merge_rows : NULL, cut ? batch->merge_cuts : NULL,
+                        cut ? (int)batch->n_merge : 0, st->stream);
         if (rc != 0) return refused(error, "attention_prefill", rc);
     }
     if (batch->n_decode != 0) {
@@ -972,6 +1036,8 @@ kipp_runtime *kipp_runtime_hip(kipp_path path, int device, const char *kernel_di
         free(rt);
         return NULL;
     }
+    if (hipDeviceGetAttribute(&st->compute_units, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || st->compute_units <= 0)
+        st->compute_units = 256;
     if (open_common(st, error) != 0) {
         hipStreamDestroy(st->stream);
         free(st);

@@ -354,6 +354,11 @@ typedef struct {
     int32_t **tables; /* per group: [n_seqs][max_blocks] */
     int32_t *item_seq, *item_tile; /* work list of the kernel for portions: (entry, tile of query rows), longest key range first */
     uint32_t n_items;
+    uint64_t items_of; /* the attention geometry the list was made for (0: none yet) */
+    /* where the list alone would leave compute units idle its keys are cut as well: an item is then (entry, tile, cut) */
+    int32_t *item_cut, *merge_rows, *merge_cuts; /* the cut of every item; the rows to merge afterwards and how many cuts each has */
+    uint32_t cut_keys, n_merge, most_cuts;       /* keys of a cut (0: not cut) */
+    float *cut_acc, *cut_ml;                     /* the cuts' sums, and their maxima and denominators */
     size_t capacity; /* ints the two buffers hold */
     /* values of this forward pass that parts share */
     const float *rotation;    /* what the table's rotary_angles made */

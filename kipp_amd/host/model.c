@@ -287,6 +287,7 @@ int kipp_model_forward(kipp_model *model, kipp_batch *batch, float **out_logits,
     batch->rotation = NULL;
     batch->rotation_of = 0;
     batch->item_seq = batch->item_tile = NULL;
+    batch->items_of = 0;
     batch->n_items = 0;
     batch->decode_workspace[0] = NULL;
     float *x = kipp_scratch(rt, (size_t)n * spec->hidden * sizeof(float), error);

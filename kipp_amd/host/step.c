@@ -311,6 +311,9 @@ static int run_step(kipp_model *model, bool single, bool choose, float **logits,
 
 uint64_t kipp_test_graph_replays(const kipp_model *model) { return model != NULL ? model->graph_replays : 0; }
 
+/* For tests: work lists of prompt portions whose keys were cut over more workgroups since the model was opened. */
+uint64_t kipp_test_cut_attention_steps(const kipp_model *model) { return model != NULL ? model->rt->cut_attention_steps : 0; }
+
 static int step_common(kipp_model *model, const kipp_step_item *items, size_t item_count, float *logits, size_t logits_capacity, uint32_t *best,
                        kipp_error *error);
 

@@ -424,6 +424,24 @@ def test_portions_behind_a_long_context_cut_their_keys(long_folder, dtype):
         assert seen == [True, True, True, True]      # 700 keys already exceed a cut of 512; every portion was cut
 
 
+def test_the_c_host_cuts_the_keys_of_such_portions_too(long_folder):
+    """The same portions through the C host: from the second on their keys are cut (700 keys already exceed a cut of
+    512) and merged; every row against the plain implementation."""
+    from kipp_amd.chost import CModel
+    cfg, weights = plain.load_folder(long_folder)
+    toks = H.random_tokens(41, 1500, 311)
+    ref = plain.forward_whole(cfg, weights, toks)
+    with CModel(long_folder, path="gpu-bf16", page_tokens=16, kv_pool_pages=96, max_sessions=2, max_step_tokens=1024,
+                share_prefixes=False) as model:
+        session = model.session()
+        got, at = [], 0
+        for n in (700, 300, 130, 370):
+            got.append(model.step([(session, toks[at:at + n], list(range(n)))]))
+            at += n
+        assert model.cut_attention_steps == 4
+    H.assert_close(np.concatenate(got), ref, H.NMSE_BF16["real"], "portions behind a long context/C host")
+
+
 def test_warm_up_decides_before_the_first_request(real_folder, real_reference):
     """`Engine.warm_up` runs portions of the given sizes on a request of its own: the products' cuts for those sizes are
     decided then (not in a request's first step), the pool is as empty as before, nothing was published, and a prompt
