@@ -92,6 +92,41 @@ def serve(engine, prompts, new_tokens: int, chunk: int, max_step_tokens: int):
     return sched, seconds, first
 
 
+def serve_c(config, prompts, new_tokens: int, chunk: int, max_step_tokens: int, share: bool):
+    """The same through the C host (`kipp_amd/host`: its scheduler over kipp_step, no Python inside a step): the shape is
+    written to a folder with random weights first.  Returns (the scheduler's counters, seconds)."""
+    import shutil
+    import tempfile
+
+    from .chost import CModel, CScheduler
+    from .weights import write_random_model
+    tmp = tempfile.mkdtemp(prefix="kipp_workload_")
+    try:
+        start = time.perf_counter()
+        folder = write_random_model(os.path.join(tmp, "model"), config, seed=0, dtype="bfloat16")
+        log(f"C host: wrote the model folder in {time.perf_counter() - start:.1f} s")
+        pages = sum(-(-(len(p) + new_tokens + 16) // 16) for p in prompts) + 8
+        with CModel(folder, path="gpu-bf16", page_tokens=16, kv_pool_pages=pages, max_sessions=len(prompts) + 2,
+                    max_step_tokens=max_step_tokens, share_prefixes=share) as model:
+            vocab = config["vocab_size"]
+            warm = CScheduler(model, max_step_tokens=max_step_tokens, prefill_chunk=chunk, max_running=2)
+            for i, p in enumerate(prompts[:2]):          # other tokens: nothing of it is adopted later
+                warm.add(i, [(t + 1) % vocab for t in p[:chunk + 3]], 4)
+            warm.run()
+            warm.destroy()
+            sched = CScheduler(model, max_step_tokens=max_step_tokens, prefill_chunk=chunk, max_running=len(prompts))
+            for i, p in enumerate(prompts):
+                sched.add(i, p, new_tokens)
+            start = time.perf_counter()
+            sched.run()
+            seconds = time.perf_counter() - start
+            stats = sched.stats
+            sched.destroy()
+        return stats, seconds
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)
+
+
 def hbm_read(gib: float) -> dict:
     """Read bandwidth of a buffer far larger than every cache, one pass a launch, over
     grids of 1 to 8 workgroups a compute unit and rings of 4 to 16 loads a lane."""
@@ -341,6 +376,7 @@ def main(argv=None) -> int:
     ap.add_argument("--context", type=int, default=None)
     ap.add_argument("--seed", type=int, default=1)
     ap.add_argument("--no-sharing", action="store_true", help="shared-prefix: compute every prompt in full, for comparison")
+    ap.add_argument("--host", choices=["python", "c"], default="python", help="which host serves: the Python engine or the C library")
     args = ap.parse_args(argv)
 
     import torch
@@ -357,6 +393,29 @@ def main(argv=None) -> int:
         print(f"workload: prompt {longest} + {new} new tokens exceed the context {context}", file=sys.stderr)
         return 1
     per_request = -(-(longest + new) // 64) * 64
+    if args.host == "c":
+        from .config import shape_config
+        config = shape_config(shape)
+        full_layers = config["num_hidden_layers"]
+        if args.layers:
+            config["num_hidden_layers"] = min(args.layers, full_layers)
+        config["max_position_embeddings"] = max(context, 64)
+        vocab = config["vocab_size"]
+        prompts = (continuous_prompts(n, args.min_prompt, args.max_prompt, vocab, args.seed) if cont
+                   else shared_prefix_prompts(n, args.prefix, args.suffix, vocab, args.seed))
+        st, seconds = serve_c(config, prompts, new, args.prefill_chunk, args.max_step_tokens, not args.no_sharing)
+        prompt_tokens = sum(len(p) for p in prompts)
+        print(json.dumps({
+            "workload": args.workload, "host": "c", "value": st["generated_tokens"] / seconds, "unit": "generated tokens/s",
+            "seconds": seconds, "requests": n, "generated_tokens": st["generated_tokens"], "prompt_tokens": prompt_tokens,
+            "prompt_tokens_run": st["prompt_tokens"], "prefix_tokens_reused": st["prefix_tokens_reused"],
+            "total_tokens_per_s": (prompt_tokens + st["generated_tokens"]) / seconds, "steps": st["steps"],
+            "first_token_s_mean": st["ttft_seconds_sum"] / max(1, st["ttft_count"]), "dtype": "bf16",
+            "data": "synthetic uniform-random tokens, random weights",
+            "config": {"model": shape, "layers": config["num_hidden_layers"], "layers_full": full_layers, "context": context,
+                       "prefill_chunk": args.prefill_chunk, "max_step_tokens": args.max_step_tokens, "new_tokens": new,
+                       "kv_page": 16, "sharing": not args.no_sharing}}), flush=True)
+        return 0
     engine, config, full_layers = build_engine(shape, args.layers, context, n * per_request, n, args.seed)
     if args.no_sharing:
         engine.cache.share = False
