@@ -442,6 +442,36 @@ def test_the_c_host_cuts_the_keys_of_such_portions_too(long_folder):
     H.assert_close(np.concatenate(got), ref, H.NMSE_BF16["real"], "portions behind a long context/C host")
 
 
+@pytest.mark.parametrize("host", ["python", "c"])
+def test_portions_of_several_requests_behind_long_contexts(long_folder, host):
+    """Three requests of 1,400, 900 and 620 tokens fed together in portions of 40 to 260 tokens, then one by one: once a
+    context passes 512 keys the portions' keys are cut, with a different number of cuts for every request (and for the
+    tiles of one portion), beside portions that are not cut and single tokens.  Every row of every request against
+    the plain implementation, through either host."""
+    cfg, weights = plain.load_folder(long_folder)
+    requests = {"x": H.random_tokens(61, 1400, 311), "y": H.random_tokens(62, 900, 311), "z": H.random_tokens(63, 620, 311)}
+    steps = H.mixed(requests, seed=9, max_live=3, prefill_portion=(40, 260), decode_tail=6)
+    assert sum(1 for entries, _ in steps if sum(1 for _, n in entries if n > 1) >= 2) >= 5
+    pages = H.peak_pages(requests, steps, 16) + 2
+    if host == "python":
+        from kipp_amd.engine import Engine
+        engine = Engine.from_folder(long_folder, dtype="bfloat16", page_size=16, num_pages=pages, max_requests=4, share_prefixes=False)
+        cut = []
+        mixer = engine.model.blocks[0].mixer
+        inner = mixer._prefill_work
+        mixer._prefill_work = lambda batch: (lambda work: (cut.append(work[2] is not None), work)[1])(inner(batch))
+        got = H.replay(engine, requests, steps)
+        assert sum(cut) >= 5
+    else:
+        from kipp_amd.chost import CModel
+        with CModel(long_folder, path="gpu-bf16", page_tokens=16, kv_pool_pages=pages, max_sessions=4, max_step_tokens=1024,
+                    share_prefixes=False) as model:
+            got = H.replay_c(model, requests, steps)
+            assert model.cut_attention_steps >= 5
+    for rid, toks in requests.items():
+        H.assert_close(got[rid], plain.forward_whole(cfg, weights, toks), H.NMSE_BF16["real"], f"portions behind long contexts/{host}/{rid}")
+
+
 def test_warm_up_decides_before_the_first_request(real_folder, real_reference):
     """`Engine.warm_up` runs portions of the given sizes on a request of its own: the products' cuts for those sizes are
     decided then (not in a request's first step), the pool is as empty as before, nothing was published, and a prompt
