@@ -326,6 +326,10 @@ class CModel:
             _raise(self.lib, error)
         return [int(t) for t in out[:wanted]]
 
+    def singles(self, sessions: Sequence[CSession]) -> "CSingles":
+        """A step of one token a session, made ready once: `CSingles.step` then costs one call into the library."""
+        return CSingles(self, sessions)
+
     def eval_batch(self, entries: Sequence[Tuple[CSession, Sequence[int]]]) -> np.ndarray:
         """kipp.h's batched call: every session's tokens appended, the logits of each one's last token."""
         out = np.empty((len(entries), self.vocab_size), dtype=np.float32)
@@ -373,6 +377,31 @@ class CModel:
 
     def __exit__(self, *exc):
         self.close()
+
+
+class CSingles:
+    """Sessions that each bring one token a step and want its largest logit's index (greedy decoding): the items of
+    kipp_step_argmax are built once, so a step is `tokens` in, one call, `out` back, with no Python for every session."""
+
+    def __init__(self, model: CModel, sessions: Sequence[CSession]):
+        self.model, self.n = model, len(sessions)
+        self.tokens = np.zeros(self.n, dtype=np.uint32)       # what the next step feeds
+        self.out = np.zeros(max(self.n, 1), dtype=np.uint32)  # what the last step chose
+        self._want = np.zeros(1, dtype=np.uint32)
+        self._items = (_StepItem * self.n)()
+        base = self.tokens.ctypes.data
+        for i, session in enumerate(sessions):
+            self._items[i] = _StepItem(session.handle, ctypes.cast(base + 4 * i, _u32p), 1, self._want.ctypes.data_as(_u32p), 1)
+
+    def step(self, feed_back: bool = False) -> np.ndarray:
+        """One step from `self.tokens`; returns `self.out`.  `feed_back`: the chosen tokens are the next step's."""
+        error = _Error()
+        if self.model.lib.kipp_step_argmax(self.model.handle, self._items, self.n, self.out.ctypes.data_as(_u32p), self.n,
+                                           ctypes.byref(error)) != 0:
+            _raise(self.model.lib, error)
+        if feed_back:
+            self.tokens[:] = self.out[:self.n]
+        return self.out
 
 
 class CScheduler:

@@ -270,7 +270,8 @@ def portion(shape: str, layers, rows: int, behind: int, runs: int = 6) -> dict:
 def c_host_decode(config, batches, prompt, steps, warmup):
     """Decode through the C host (`kipp_amd/host`, no Python between the launches of a step): the same shape written to a
     folder with random weights, prompts filled through kipp_step, then `steps` greedy steps timed on the host's clock
-    around kipp_step_argmax, everything a serving loop pays included (the batch's integers up, the tokens back)."""
+    around kipp_step_argmax, everything a serving loop pays included (the batch's integers up, the tokens back); the
+    call's arguments are made once (`CModel.singles`), so a step is one call into the library."""
     import shutil
     import tempfile
 
@@ -292,12 +293,13 @@ def c_host_decode(config, batches, prompt, steps, warmup):
             for s in sessions:
                 model.step([(s, rng.integers(0, config["vocab_size"], prompt).tolist(), [])])
             for b in batches:
-                tokens = [1 + i for i in range(b)]
+                batch = model.singles(sessions[:b])
+                batch.tokens[:] = [1 + i for i in range(b)]
                 for _ in range(warmup):
-                    tokens = model.step_argmax([(s, [t], [0]) for s, t in zip(sessions[:b], tokens)])
+                    batch.step(feed_back=True)
                 start = time.perf_counter()
                 for _ in range(steps):
-                    tokens = model.step_argmax([(s, [t], [0]) for s, t in zip(sessions[:b], tokens)])
+                    batch.step(feed_back=True)
                 took = time.perf_counter() - start
                 points[f"decode_b{b}_c_host"] = round(b * steps / took, 1)
                 log(f"C host: decode batch {b}: {took / steps * 1e3:.3f} ms/step, {b * steps / took:.0f} tok/s ({model.graph_replays} steps so far ran from recordings)")

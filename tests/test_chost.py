@@ -512,6 +512,25 @@ def test_step_argmax_is_the_argmax_of_step(model_folders, tiny_configs):
         assert d.length == 7                                          # the refused step left the session as it was
 
 
+def test_single_tokens_made_ready_once_decode_like_step_argmax(model_folders, tiny_configs):
+    """`CModel.singles`: the items of kipp_step_argmax built once and fed from one buffer; six greedy steps of three sessions
+    give the tokens that step_argmax gives entry by entry."""
+    cfg = tiny_configs["b"]
+    prompts = [H.random_tokens(10 + i, 5 + 3 * i, cfg["vocab_size"]) for i in range(3)]
+    with CModel(model_folders[("b", "float32")], path="cpu-fp32", page_tokens=8, kv_pool_pages=24, share_prefixes=False) as model:
+        one, two = [model.session() for _ in prompts], [model.session() for _ in prompts]
+        first = model.step_argmax([(s, p, [len(p) - 1]) for s, p in zip(one, prompts)])
+        assert model.step_argmax([(s, p, [len(p) - 1]) for s, p in zip(two, prompts)]) == first
+        batch = model.singles(two)
+        batch.tokens[:] = first
+        tokens, seen, want = list(first), [], []
+        for _ in range(6):
+            tokens = model.step_argmax([(s, [t], [0]) for s, t in zip(one, tokens)])
+            want.append(tokens)
+            seen.append([int(t) for t in batch.step(feed_back=True)[:3]])
+        assert seen == want and [s.length for s in two] == [s.length for s in one]
+
+
 # ---------------------------------------------------------------------------------------------- the C scheduler
 
 def _greedy(folder, prompt, n, stop=()):
