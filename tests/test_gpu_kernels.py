@@ -36,9 +36,11 @@ def test_embed(dtype):
     assert torch.equal(out.cpu(), table.float()[tokens])
 
 
-@pytest.mark.parametrize("width,rows", [(2, 1), (72, 5), (2560, 3), (5000, 2)])
+@pytest.mark.parametrize("width,rows", [(2, 1), (72, 5), (2560, 3), (5000, 2), (1536, 4), (8192, 2), (8196, 2), (2560, 300), (1028, 256)])
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
 def test_rmsnorm(width, rows, out_dtype):
+    """Rows of every width class: up to 256 rows of more than 1,024 columns take a workgroup of 512 or 1,024 threads under
+    bfloat16 (1,536; 2,560 and 1,028; 5,000 and 8,192 in two passes), more rows or wider ones the workgroups of 256."""
     ops = _ops()
     rng = np.random.default_rng(width)
     x = rng.normal(size=(rows, width)).astype(np.float32)
@@ -1176,19 +1178,22 @@ def test_gate_up_product_from_paired_tiles(m, inner, k, max_parts):
     assert _rel(y.sum(dim=0).cpu().numpy()[:, keep], plain_y.numpy()[:, [order[c] for c in keep]]) < 1e-10
 
 
-def test_rmsnorm_adds_slabs_in_order():
+@pytest.mark.parametrize("rows,width,n_parts,out_dtype", [(3, 80, 4, torch.float32), (20, 2560, 7, torch.bfloat16), (5, 1536, 2, torch.bfloat16),
+                                                       (4, 5120, 9, torch.bfloat16), (300, 2560, 3, torch.bfloat16)])
+def test_rmsnorm_adds_slabs_in_order(rows, width, n_parts, out_dtype):
+    """The slabs of a split product are added to the residual one after the other, whatever the workgroup's size."""
     ops = _ops()
-    rng = np.random.default_rng(8)
-    x = rng.normal(size=(3, 80)).astype(np.float32)
-    parts = rng.normal(size=(4, 3, 80)).astype(np.float32)
-    w = np.ones(80, dtype=np.float32)
+    rng = np.random.default_rng(8 + rows)
+    x = rng.normal(size=(rows, width)).astype(np.float32)
+    parts = rng.normal(size=(n_parts, rows, width)).astype(np.float32)
+    w = (1 + 0.1 * rng.normal(size=width)).astype(np.float32)
     xd = _t(x)
-    got = ops.rmsnorm(xd, _t(w), 1e-6, torch.empty(3, 80, device=DEV), delta=_t(parts))
+    got = ops.rmsnorm(xd, _t(w), 1e-6, torch.empty(rows, width, dtype=out_dtype, device=DEV), delta=_t(parts))
     total = x.copy()
     for p in parts:
         total = total + p
     assert np.array_equal(xd.cpu().numpy(), total)
-    assert _rel(got.cpu().numpy(), plain.rms_norm(total, w, 1e-6)) < 1e-12
+    assert _rel(got.float().cpu().numpy(), plain.rms_norm(total, w, 1e-6)) < (1e-12 if out_dtype == torch.float32 else 1e-5)
 
 
 @pytest.mark.parametrize("vocab", [509, 151936])
