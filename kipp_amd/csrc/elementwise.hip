@@ -207,9 +207,13 @@ __global__ void swiglu_kernel(const TI* __restrict__ gu, TO* __restrict__ out, i
     store_f(out, idx, g / (1.0f + expf(-g)) * u);
 }
 
-// The same, eight columns a thread with 16-byte accesses (inner a multiple of 8, one slab).
+// The same, eight columns a thread with 16-byte accesses (inner a multiple of 8); the slabs of a split product are added
+// in order, four at a time with all their loads asked for before the first is added.
+__device__ __forceinline__ float4 add4(float4 a, float4 b) { return make_float4(a.x + b.x, a.y + b.y, a.z + b.z, a.w + b.w); }
+
 template <typename TI, typename TO>
-__global__ void swiglu_vec_kernel(const TI* __restrict__ gu, TO* __restrict__ out, int inner, size_t total8, int pairs) {
+__global__ void swiglu_vec_kernel(const TI* __restrict__ gu, TO* __restrict__ out, int inner, size_t total8, int pairs, int parts,
+                                  size_t slab4) {
     const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= total8) return;
     const int per_row = inner / 8;
@@ -217,8 +221,28 @@ __global__ void swiglu_vec_kernel(const TI* __restrict__ gu, TO* __restrict__ ou
     const int i4 = (int)(idx - t * per_row) * 2;              // in units of 4 columns
     const size_t row4 = t * 2 * (size_t)inner / 4;
     const size_t g4 = row4 + (pairs ? 2 * i4 : i4), u4 = g4 + (pairs ? 2 : inner / 4);
-    const float4 g0 = load4(gu, g4), g1 = load4(gu, g4 + 1);
-    const float4 u0 = load4(gu, u4), u1 = load4(gu, u4 + 1);
+    float4 g0 = load4(gu, g4), g1 = load4(gu, g4 + 1);
+    float4 u0 = load4(gu, u4), u1 = load4(gu, u4 + 1);
+    for (int p0 = 1; p0 < parts; p0 += 4) {
+        float4 more[4][4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const size_t at = (size_t)min(p0 + q, parts - 1) * slab4;
+            more[q][0] = load4(gu, at + g4);
+            more[q][1] = load4(gu, at + g4 + 1);
+            more[q][2] = load4(gu, at + u4);
+            more[q][3] = load4(gu, at + u4 + 1);
+        }
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            if (p0 + q < parts) {
+                g0 = add4(g0, more[q][0]);
+                g1 = add4(g1, more[q][1]);
+                u0 = add4(u0, more[q][2]);
+                u1 = add4(u1, more[q][3]);
+            }
+        }
+    }
     const size_t o4 = t * (size_t)inner / 4 + i4;
     store4(out, o4, make_float4(g0.x / (1.0f + expf(-g0.x)) * u0.x, g0.y / (1.0f + expf(-g0.y)) * u0.y,
                                 g0.z / (1.0f + expf(-g0.z)) * u0.z, g0.w / (1.0f + expf(-g0.w)) * u0.w));
@@ -352,10 +376,11 @@ int kipp_swiglu(const void* gu, int in_dtype, int parts, void* out, int out_dtyp
                 hipStream_t stream) {
     size_t total = (size_t)rows * inner;
     if (total == 0) return 0;
-    if (parts == 1 && (inner & 7) == 0) {
+    if (parts >= 1 && (inner & 7) == 0) {
         const size_t total8 = total / 8;
+        const size_t slab4 = (size_t)rows * 2 * inner / 4;       // a slab in units of four values (paired tiles are as wide: 16 columns for 8 outputs)
         dim3 grid8((unsigned)((total8 + 255) / 256)), block8(256);
-#define KIPP_SV(TI, TO) hipLaunchKernelGGL((swiglu_vec_kernel<TI, TO>), grid8, block8, 0, stream, (const TI*)gu, (TO*)out, inner, total8, pairs)
+#define KIPP_SV(TI, TO) hipLaunchKernelGGL((swiglu_vec_kernel<TI, TO>), grid8, block8, 0, stream, (const TI*)gu, (TO*)out, inner, total8, pairs, parts, slab4)
         if (in_dtype == KIPP_BF16) {
             if (out_dtype == KIPP_BF16) KIPP_SV(bf16_t, bf16_t); else KIPP_SV(bf16_t, float);
         } else {
