@@ -108,38 +108,68 @@ __device__ __forceinline__ float load_through(const float* p) {
     return __uint_as_float(__hip_atomic_load((const unsigned*)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
 }
 
+// two neighbouring values at an address that 8 divides
+__device__ __forceinline__ float2 load_through2(const float* p) {
+    const unsigned long long bits = __hip_atomic_load((const unsigned long long*)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return make_float2(__uint_as_float((unsigned)bits), __uint_as_float((unsigned)(bits >> 32)));
+}
+
 // The merge of attention_decode_reduce_kernel (the same sums in the same order) by the workgroup that finished
-// last among the splits of a (token, key/value head): element `dcol` of head `head`.
-__device__ __forceinline__ float merge_splits_here(const float* part_acc, const float* part_ml, size_t slot0, int n_splits, int dcol) {
+// last among the splits of a (token, key/value head): elements `dcol` and `dcol` + 1 (dcol even) of head `head`.
+// A split costs a thread two loads of 8 bytes: its maximum with its denominator, and the two sums.
+__device__ __forceinline__ float2 merge_splits_here(const float* part_acc, const float* part_ml, size_t slot0, int n_splits, int dcol) {
     constexpr int AT_ONCE = 16;
-    float m_s[AT_ONCE], l_s[AT_ONCE], a_s[AT_ONCE];
-    // the first 16 splits are asked for together, whatever their number (beyond it: the last again, dropped below)
+    float2 ml_s[AT_ONCE], a_s[AT_ONCE];
+    // the first 16 splits are asked for together
 #pragma unroll
     for (int i = 0; i < AT_ONCE; ++i) {
-        const size_t slot = slot0 + min(i, n_splits - 1);
-        m_s[i] = load_through(part_ml + slot * 2);
-        l_s[i] = load_through(part_ml + slot * 2 + 1);
-        a_s[i] = load_through(part_acc + slot * HEAD_DIM + dcol);
+        ml_s[i] = make_float2(-INFINITY, 0.0f);
+        a_s[i] = make_float2(0.0f, 0.0f);
+        if (i < n_splits) {
+            ml_s[i] = load_through2(part_ml + (slot0 + i) * 2);
+            a_s[i] = load_through2(part_acc + (slot0 + i) * HEAD_DIM + dcol);
+        }
     }
     float m = -INFINITY;
 #pragma unroll
-    for (int i = 0; i < AT_ONCE; ++i) m = fmaxf(m, i < n_splits ? m_s[i] : -INFINITY);
+    for (int i = 0; i < AT_ONCE; ++i) m = fmaxf(m, ml_s[i].x);
     for (int s = AT_ONCE; s < n_splits; ++s) m = fmaxf(m, load_through(part_ml + (slot0 + s) * 2));
-    float denom = 0.0f, a = 0.0f;
+    float denom = 0.0f;
+    float2 a = make_float2(0.0f, 0.0f);
 #pragma unroll
     for (int i = 0; i < AT_ONCE; ++i) {
         if (i < n_splits) {
-            const float w = exp2f(m_s[i] - m);
-            denom += l_s[i] * w;
-            a += a_s[i] * w;
+            const float w = exp2f(ml_s[i].x - m);
+            denom += ml_s[i].y * w;
+            a.x += a_s[i].x * w;
+            a.y += a_s[i].y * w;
         }
     }
     for (int s = AT_ONCE; s < n_splits; ++s) {
-        const float w = exp2f(load_through(part_ml + (slot0 + s) * 2) - m);
-        denom += load_through(part_ml + (slot0 + s) * 2 + 1) * w;
-        a += load_through(part_acc + (slot0 + s) * HEAD_DIM + dcol) * w;
+        const float2 ml = load_through2(part_ml + (slot0 + s) * 2), more = load_through2(part_acc + (slot0 + s) * HEAD_DIM + dcol);
+        const float w = exp2f(ml.x - m);
+        denom += ml.y * w;
+        a.x += more.x * w;
+        a.y += more.y * w;
     }
-    return a / denom;
+    return make_float2(a.x / denom, a.y / denom);
+}
+
+__device__ __forceinline__ void store_through2(float* p, float a, float b) {
+    __hip_atomic_store((unsigned long long*)p, (unsigned long long)__float_as_uint(a) | ((unsigned long long)__float_as_uint(b) << 32),
+                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Two neighbouring elements (dcol even) of a split's partial result.  With `arrivals` the splits are merged inside this launch.
+__device__ __forceinline__ void put_partial2(const unsigned* arrivals, float* part_acc, float* part_ml, size_t slot, int dcol,
+                                             float a0, float a1, float m, float l) {
+    if (arrivals != nullptr) {
+        store_through2(part_acc + slot * HEAD_DIM + dcol, a0, a1);
+        if (dcol == 0) store_through2(part_ml + slot * 2, m, l);
+    } else {
+        *(float2*)(part_acc + slot * HEAD_DIM + dcol) = make_float2(a0, a1);
+        if (dcol == 0) *(float2*)(part_ml + slot * 2) = make_float2(m, l);
+    }
 }
 
 // One element of a split's partial result.  With `arrivals` the splits are merged inside this launch.
@@ -179,11 +209,14 @@ __device__ __forceinline__ void merge_by_the_last(unsigned* arrivals, const floa
     }
     __syncthreads();
     if (!s_last) return;
-    for (int idx = tid; idx < GROUP * HEAD_DIM; idx += THREADS) {
-        const int g = idx / HEAD_DIM, dcol = idx % HEAD_DIM;
+    for (int idx = tid; idx < GROUP * HEAD_DIM / 2; idx += THREADS) {
+        const int g = idx / (HEAD_DIM / 2), dcol = 2 * (idx % (HEAD_DIM / 2));
         const int head = kvh * GROUP + g;
         const size_t slot0 = ((size_t)item * n_q + head) * max_splits;
-        out[out_at(row, head * HEAD_DIM + dcol, n_q * HEAD_DIM, out_rows)] = f32_to_bf16(merge_splits_here(part_acc, part_ml, slot0, n_splits, dcol));
+        const float2 merged = merge_splits_here(part_acc, part_ml, slot0, n_splits, dcol);
+        // two neighbouring columns lie side by side in either order of the rows (runs of 32 columns)
+        *(uint32_t*)(out + out_at(row, head * HEAD_DIM + dcol, n_q * HEAD_DIM, out_rows)) =
+            (uint32_t)f32_to_bf16(merged.x) | ((uint32_t)f32_to_bf16(merged.y) << 16);
     }
 }
 
@@ -479,16 +512,20 @@ __global__ void __launch_bounds__(THREADS) attention_decode_kernel(
             }
     }
     __syncthreads();
-    for (int idx = tid; idx < GROUP * HEAD_DIM; idx += THREADS) {
-        const int g = idx / HEAD_DIM, dcol = idx % HEAD_DIM;
-        float a = 0.0f;
+    for (int idx = tid; idx < GROUP * HEAD_DIM / 2; idx += THREADS) {      // two neighbouring columns a thread
+        const int g = idx / (HEAD_DIM / 2), dcol = 2 * (idx % (HEAD_DIM / 2));
+        float a0 = 0.0f, a1 = 0.0f;
 #pragma unroll
-        for (int w = 0; w < WAVES; ++w) a += s_red[w][g][dcol];
+        for (int w = 0; w < WAVES; ++w) {
+            a0 += s_red[w][g][dcol];
+            a1 += s_red[w][g][dcol + 1];
+        }
         const int head = kvh * GROUP + g;
         if (n_splits == 1) {
-            out[out_at(row, head * HEAD_DIM + dcol, n_q * HEAD_DIM, FUSED ? pj.out_rows : 0)] = f32_to_bf16(a / s_l[g]);
+            *(uint32_t*)(out + out_at(row, head * HEAD_DIM + dcol, n_q * HEAD_DIM, FUSED ? pj.out_rows : 0)) =
+                (uint32_t)f32_to_bf16(a0 / s_l[g]) | ((uint32_t)f32_to_bf16(a1 / s_l[g]) << 16);
         } else {
-            put_partial(arrivals, part_acc, part_ml, ((size_t)blockIdx.x * n_q + head) * max_splits + blockIdx.z, dcol, a, s_m[g], s_l[g]);
+            put_partial2(arrivals, part_acc, part_ml, ((size_t)blockIdx.x * n_q + head) * max_splits + blockIdx.z, dcol, a0, a1, s_m[g], s_l[g]);
         }
     }
     if (arrivals != nullptr && n_splits > 1)
@@ -1011,23 +1048,25 @@ __global__ void __launch_bounds__(THREADS, 2) attention_decode_ring_kernel(
         }
     }
     __syncthreads();
-    for (int idx = tid; idx < GROUP * HEAD_DIM; idx += THREADS) {
-        const int g = idx / HEAD_DIM, dcol = idx % HEAD_DIM;
+    for (int idx = tid; idx < GROUP * HEAD_DIM / 2; idx += THREADS) {      // two neighbouring columns a thread
+        const int g = idx / (HEAD_DIM / 2), dcol = 2 * (idx % (HEAD_DIM / 2));
         float m = -INFINITY;
 #pragma unroll
         for (int w = 0; w < WAVES; ++w) m = fmaxf(m, s_ml[(w * GROUP + g) * 2]);
-        float a = 0.0f, l = 0.0f;
+        float a0 = 0.0f, a1 = 0.0f, l = 0.0f;
 #pragma unroll
         for (int w = 0; w < WAVES; ++w) {
             const float f = exp2f(__fsub_rn(s_ml[(w * GROUP + g) * 2], m));    // a wave without keys: 2^-inf = 0
-            a = fmaf(s_red[((size_t)w * GROUP + g) * HEAD_DIM + dcol], f, a);
+            a0 = fmaf(s_red[((size_t)w * GROUP + g) * HEAD_DIM + dcol], f, a0);
+            a1 = fmaf(s_red[((size_t)w * GROUP + g) * HEAD_DIM + dcol + 1], f, a1);
             l = fmaf(s_ml[(w * GROUP + g) * 2 + 1], f, l);
         }
         const int head = kvh * GROUP + g;
         if (n_splits == 1) {
-            out[out_at(row, head * HEAD_DIM + dcol, n_q * HEAD_DIM, FUSED ? pj.out_rows : 0)] = f32_to_bf16(a / l);
+            *(uint32_t*)(out + out_at(row, head * HEAD_DIM + dcol, n_q * HEAD_DIM, FUSED ? pj.out_rows : 0)) =
+                (uint32_t)f32_to_bf16(a0 / l) | ((uint32_t)f32_to_bf16(a1 / l) << 16);
         } else {
-            put_partial(arrivals, part_acc, part_ml, ((size_t)blockIdx.x * n_q + head) * max_splits + blockIdx.z, dcol, a, m, l);
+            put_partial2(arrivals, part_acc, part_ml, ((size_t)blockIdx.x * n_q + head) * max_splits + blockIdx.z, dcol, a0, a1, m, l);
         }
     }
     if (arrivals != nullptr && n_splits > 1)
