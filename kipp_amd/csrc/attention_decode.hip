@@ -1184,10 +1184,11 @@ static int launch_reduce(const float* part_acc, const float* part_ml, bf16_t* ou
 // is not for it.  RING_WHOLE_FROM_PAIRS (sequence, key/value head) pairs and more: whole contexts (RING_RANGE
 // keys at most).  Fewer: ranges that give 256 workgroups, if those are 1,024 keys and more; else whole contexts
 // from RING_FROM_PAIRS pairs on.  Measured in the decode step at 2,100 keys, 8 heads: 12 sequences in two ranges
-// (192 workgroups at work instead of 96) 3.24 instead of 3.54 ms; 16 sequences 3.50 to 3.56 either way; 24
-// sequences in two ranges 4.11 instead of 3.97 (the partial results and their merge cost more than the second
-// workgroup on every compute unit brings).  A function of the launch's shape, never of the data.
-#define RING_WHOLE_FROM_PAIRS 128
+// (192 workgroups at work instead of 96) 3.24 instead of 3.54 ms; 16 sequences 3.31 instead of 3.39 (they were
+// level while the merge asked for its partial results four bytes at a time); 24 sequences in two ranges 4.11
+// instead of 3.97 (the partial results and their merge cost more than the second workgroup on every compute
+// unit brings).  A function of the launch's shape, never of the data.
+#define RING_WHOLE_FROM_PAIRS 160
 static int ring_range(int n_items, int n_kv, int page, int grid_splits) {
     if (page % 16 != 0) return 0;
     const long long pairs = (long long)n_items * n_kv, span = (long long)grid_splits * SPLIT;
