@@ -1232,24 +1232,36 @@ static int launch_ring(const bf16_t* q, bf16_t* k_cache, bf16_t* v_cache, bf16_t
 }
 #endif
 
-// The kernel that takes one split a workgroup, with splits of 256 keys, of 192 for one or two sequences, or of 320
-// where splits of 256 would be more workgroups than two a compute unit: workgroups beyond those that
-// fit at once run as a second round behind the first (measured at 8 sequences of 8 key/value heads: 576
-// workgroups for 2,050 keys cost 0.15 ms a step more than 512 for 2,040).  A function of the launch's shape.
+// The kernel that takes one split a workgroup, with splits of 192, 256 or 320 keys (head sizes above 128: 256): the
+// length whose workgroups take the fewest keys one after the other on a compute unit.  The workgroups of a launch run in
+// rounds of 256, and a round costs what one split reads, so a length is priced as rounds x keys, with the rounds of the
+// splits that contexts really have: a recorded step is launched for the longest context of its class of 1,024, and the
+// splits beyond a sequence's position leave at once, so the price is the mean over the contexts of that class.
+// Measured in the decode step behind 2,048 to 2,304 keys (a class up to 3,072), 32 query over 8 key/value heads, for
+// 192 / 256 / 320 keys: 4 sequences 2.353 / 2.416 / 2.340 ms, 5: 2.394 / 2.454 / 2.531, 6: 2.550 / 2.493 / 2.575,
+// 8: 2.620 / 2.741 / 2.648; every order is the price's.  (While the merge of the splits asked for its partial results
+// four bytes at a time the shorter splits' merges cost more than that, and 8 sequences took 320.)  A function of the
+// launch's shape, never of the data.
 static int split_keys_for(int n_items, int n_kv, int span_keys, int window, int longest, int max_splits) {
-    const long long pairs = (long long)n_items * n_kv, fit = 2 * 256;
+    const long long pairs = (long long)n_items * n_kv;
     const int extra = window > 0 ? 1 : 0;
-    // few pairs: shorter splits, where they still are at most a workgroup a compute unit and the merge takes them
-    // at once (a workgroup's keys and values are what one compute unit has to draw: 96 KB instead of 128; one
-    // and two sequences of 8 heads at 2,100 keys: 1.3 % of the step)
-    {
-        const int n = (span_keys + SPLIT_MIN - 1) / SPLIT_MIN + extra;
-        if (longest > SPLIT && pairs * n <= 256 && n <= 16 && n <= max_splits) return SPLIT_MIN;
+    static const int lengths[] = {SPLIT_MAX, SPLIT, SPLIT_MIN};          // of equal price the longest: fewer partial results
+    const bool a_class = span_keys > 1024 && span_keys % 1024 == 0;      // every context of the last 1,024 keys may come
+    long long best = -1;
+    int keys = 0;
+    for (int length : lengths) {
+        if (length > longest || (span_keys + length - 1) / length + extra > max_splits) continue;
+        long long price = 0;
+        for (int i = a_class ? 1 : 16; i <= 16; ++i) {
+            const int context = span_keys - (16 - i) * 64;
+            price += (pairs * ((context + length - 1) / length + extra) + 255) / 256 * length;
+        }
+        if (best < 0 || price < best) {
+            best = price;
+            keys = length;
+        }
     }
-    if (pairs * ((span_keys + SPLIT - 1) / SPLIT + extra) <= fit) return SPLIT;
-    for (int keys = SPLIT + 64; keys <= longest; keys += 64)
-        if (pairs * ((span_keys + keys - 1) / keys + extra) <= fit) return keys;
-    return longest;                                   // more than fit at once either way: the fewest workgroups
+    return keys != 0 ? keys : longest;                // (no length fits the room for partial results: the launcher refuses)
 }
 
 template <bool FUSED>
