@@ -11,7 +11,7 @@ A graph holds our own kernels only: nothing that reads back to the host, no
 library call, no memset node.  A model with a part that does not declare
 `graph_safe`, or a step that went to a library product, runs eagerly instead.
 
-The number of rows is rounded up to one of a few sizes (exact up to 12, then 16, 24, 32,
+The number of rows is rounded up to one of a few sizes (exact up to 16, then 24, 32,
 48, ... 256), so that a batch whose size changes from step to step still finds its
 graph: the rows that fill up bring token 0 at position 0 of a sequence of their own,
 whose block table names the cache's scratch page and whose state is the scratch slot;
@@ -39,7 +39,7 @@ MAX_GRAPHS = 48              # shapes kept (each holds its recorded launches and
 MAX_GRAPH_ENTRIES = 256     # rows up to which every product of a step is one of our own kernels (none goes to a library)
 
 
-GRAPH_SIZES = [1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 16, 24, 32, 48, 64, 96, 128, 192, 256]   # exact while the few-rows products run (every row costs there)
+GRAPH_SIZES = [1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15, 16, 24, 32, 48, 64, 96, 128, 192, 256]   # exact up to 16 rows (every row costs there: 13 rows on a recording of 16 took 3.23 ms, of 13 rows 3.12)
 
 
 def padded_size(n: int) -> int:

@@ -274,21 +274,21 @@ def test_many_requests_decode_together(long_folder, dtype, n_requests):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_a_batch_whose_size_changes_replays_one_graph(long_folder, dtype):
-    """13 to 16 requests decode together, another number in every step (the others wait): all those steps
-    are one recorded shape of 16 rows, the rows that fill up write to the cache's scratch page; a request
+    """17 to 24 requests decode together, another number in every step (the others wait): all those steps
+    are one recorded shape of 24 rows, the rows that fill up write to the cache's scratch page; a request
     that joined late and the ones that paused give the logits of the plain implementation."""
     from kipp_amd.engine import Engine, StepEntry
     from kipp_amd.engine.graphs import padded_size
-    assert [padded_size(n) for n in (1, 8, 9, 12, 13, 100, 129, 256)] == [1, 8, 9, 12, 16, 128, 192, 256]
+    assert [padded_size(n) for n in (1, 8, 9, 12, 13, 16, 17, 100, 129, 256)] == [1, 8, 9, 12, 13, 16, 24, 128, 192, 256]
     cfg, weights = plain.load_folder(long_folder)
-    seqs = {f"r{i}": H.random_tokens(300 + i, 20 + 3 * i + 14, 311) for i in range(16)}
-    engine = Engine.from_folder(long_folder, dtype=dtype, page_size=16, max_tokens=16 * 128, max_requests=16, share_prefixes=False)
+    seqs = {f"r{i}": H.random_tokens(300 + i, 20 + 3 * i + 14, 311) for i in range(24)}
+    engine = Engine.from_folder(long_folder, dtype=dtype, page_size=16, max_tokens=24 * 128, max_requests=24, share_prefixes=False)
     fed = {rid: len(toks) - 14 for rid, toks in seqs.items()}
     engine.step([StepEntry(rid, seqs[rid][:fed[rid]], []) for rid in seqs])
     got = {rid: [] for rid in seqs}
     order = list(seqs)
-    for step, n in enumerate([16, 14, 15, 13, 16, 14, 13, 15, 16, 13, 14, 16, 15, 16]):
-        live = [rid for rid in (order[step % 16:] + order[:step % 16]) if fed[rid] < len(seqs[rid])][:n]
+    for step, n in enumerate([24, 19, 21, 17, 24, 20, 18, 23, 24, 17, 22, 24, 19, 24]):
+        live = [rid for rid in (order[step % 24:] + order[:step % 24]) if fed[rid] < len(seqs[rid])][:n]
         logits = engine.step([StepEntry(rid, [seqs[rid][fed[rid]]], [0]) for rid in live]).cpu().numpy()
         assert logits.shape[0] == len(live)
         for row, rid in zip(logits, live):
