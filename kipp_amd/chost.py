@@ -145,6 +145,7 @@ def library(variant: str = "gpu") -> ctypes.CDLL:
             "kipp_session_eval_scored": [vp, _u32p, sz, _f32p, u32, err],
             "kipp_session_match_prefix": [vp, _u32p, sz, _u32p, err],
             "kipp_eval_batch": [vp, ctypes.POINTER(_BatchItem), sz, err],
+            "kipp_model_eval": [vp, _u32p, sz, _f32p, sz, err],
             "kipp_step": [vp, ctypes.POINTER(_StepItem), sz, _f32p, sz, err],
             "kipp_step_argmax": [vp, ctypes.POINTER(_StepItem), sz, _u32p, sz, err],
             "kipp_sample_ex": [_f32p, sz, ctypes.POINTER(_SampleParams), ctypes.POINTER(ctypes.c_uint64), _u32p, err],
@@ -329,6 +330,15 @@ class CModel:
     def singles(self, sessions: Sequence[CSession]) -> "CSingles":
         """A step of one token a session, made ready once: `CSingles.step` then costs one call into the library."""
         return CSingles(self, sessions)
+
+    def eval(self, tokens: Sequence[int]) -> np.ndarray:
+        """kipp.h's evaluation without a session: the logits of the last of up to 256 tokens."""
+        t, tp = _u32(tokens)
+        out = np.empty(self.vocab_size, dtype=np.float32)
+        error = _Error()
+        if self.lib.kipp_model_eval(self.handle, tp, len(t), out.ctypes.data_as(_f32p), out.size, ctypes.byref(error)) != 0:
+            _raise(self.lib, error)
+        return out
 
     def eval_batch(self, entries: Sequence[Tuple[CSession, Sequence[int]]]) -> np.ndarray:
         """kipp.h's batched call: every session's tokens appended, the logits of each one's last token."""

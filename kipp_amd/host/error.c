@@ -60,6 +60,8 @@ const char *kipp_path_name(kipp_path path) {
     return "unknown";
 }
 
+const char *kipp_backend_name(kipp_path path) { return kipp_path_name(path); }
+
 void kipp_text_add(kipp_text *text, const char *format, ...) {
     if (text->failed) return;
     for (;;) {

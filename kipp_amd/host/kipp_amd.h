@@ -100,11 +100,23 @@ typedef struct {
 
 int kipp_model_open(const char *model_dir, kipp_model **out_model, kipp_error *error);
 int kipp_model_open_ex(const char *model_dir, const kipp_model_open_config *config, kipp_model **out_model, kipp_error *error);
+/* Every other field as kipp_model_open leaves it, on the given path (/root/reference/src/kipp.h:110-111). */
+int kipp_model_open_backend(const char *model_dir, kipp_path path, kipp_model **out_model, kipp_error *error);
+/* The same with a pool of `kv_pool_pages` pages (not 0) for every cache group, shared by all sessions, which publish and
+ * adopt beginnings (/root/reference/src/kipp.h:112-122). */
+int kipp_model_open_pooled(const char *model_dir, kipp_path path, uint32_t kv_pool_pages, kipp_model **out_model, kipp_error *error);
 /* Refuses while sessions are alive (/root/reference/src/kipp.c:1340-1344). */
 int kipp_model_close(kipp_model *model, kipp_error *error);
 int kipp_model_get_info(const kipp_model *model, kipp_model_info *out_info);
 int kipp_model_is_stop_token(const kipp_model *model, uint32_t token);
 const char *kipp_path_name(kipp_path path);
+const char *kipp_backend_name(kipp_path path); /* the reference's name for the same (/root/reference/src/kipp.h:145) */
+/* Evaluation without a session of the caller's: up to KIPP_MODEL_EVAL_LIMIT tokens through a session of its own, which
+ * is destroyed before the call returns (it needs one free session and the pages for the tokens; where sharing is on its
+ * full pages stay published like any ended session's); the logits of the last token, `logits_count` at least the
+ * vocabulary (/root/reference/src/kipp.h:159-166). */
+#define KIPP_MODEL_EVAL_LIMIT 256u
+int kipp_model_eval(kipp_model *model, const uint32_t *tokens, size_t token_count, float *logits, size_t logits_count, kipp_error *error);
 
 /* A session holds up to `capacity` tokens (0: the model's context length). */
 int kipp_session_create(kipp_model *model, uint32_t capacity, kipp_session **out_session, kipp_error *error);

@@ -138,6 +138,25 @@ int kipp_model_open(const char *model_dir, kipp_model **out_model, kipp_error *e
     return kipp_model_open_ex(model_dir, &config, out_model, error);
 }
 
+int kipp_model_open_backend(const char *model_dir, kipp_path path, kipp_model **out_model, kipp_error *error) {
+    kipp_model_open_config config;
+    memset(&config, 0, sizeof(config));
+    config.share_prefixes = 1;
+    config.path = path;
+    return kipp_model_open_ex(model_dir, &config, out_model, error);
+}
+
+int kipp_model_open_pooled(const char *model_dir, kipp_path path, uint32_t kv_pool_pages, kipp_model **out_model, kipp_error *error) {
+    kipp_error_clear(error);
+    if (kv_pool_pages == 0) return kipp_fail(error, KIPP_ERROR_ARGUMENT, "a pool of no pages");
+    kipp_model_open_config config;
+    memset(&config, 0, sizeof(config));
+    config.share_prefixes = 1;
+    config.path = path;
+    config.kv_pool_pages = kv_pool_pages;
+    return kipp_model_open_ex(model_dir, &config, out_model, error);
+}
+
 int kipp_model_open_ex(const char *model_dir, const kipp_model_open_config *config, kipp_model **out_model, kipp_error *error) {
     kipp_error_clear(error);
     if (model_dir == NULL || config == NULL || out_model == NULL) return kipp_fail(error, KIPP_ERROR_ARGUMENT, "model folder, configuration and result must be given");

@@ -468,6 +468,19 @@ int kipp_session_eval(kipp_session *session, const uint32_t *tokens, size_t toke
     return kipp_session_eval_scored(session, tokens, token_count, logits, 1, error);
 }
 
+int kipp_model_eval(kipp_model *model, const uint32_t *tokens, size_t token_count, float *logits, size_t logits_count, kipp_error *error) {
+    kipp_error_clear(error);
+    if (model == NULL || tokens == NULL || logits == NULL) return kipp_fail(error, KIPP_ERROR_ARGUMENT, "model, tokens and logits must be given");
+    if (token_count == 0 || token_count > KIPP_MODEL_EVAL_LIMIT)
+        return kipp_fail(error, KIPP_ERROR_RANGE, "between 1 and %u tokens, not %zu", KIPP_MODEL_EVAL_LIMIT, token_count);
+    if (logits_count < model->spec.vocab) return kipp_fail(error, KIPP_ERROR_RANGE, "logits must hold %u floats", model->spec.vocab);
+    kipp_session *session = NULL;
+    if (kipp_session_create(model, (uint32_t)token_count, &session, error) != 0) return -1;
+    const int rc = kipp_session_eval_scored(session, tokens, token_count, logits, 1, error);
+    kipp_session_destroy(session);
+    return rc;
+}
+
 int kipp_eval_batch(kipp_model *model, kipp_batch_item *items, size_t item_count, kipp_error *error) {
     kipp_error_clear(error);
     if (model == NULL || (items == NULL && item_count != 0)) return kipp_fail(error, KIPP_ERROR_ARGUMENT, "model and items must be given");

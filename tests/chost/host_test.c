@@ -234,7 +234,29 @@ static void test_model(const char *folder) {
     kipp_session_destroy(c);
     kipp_model_kv_pool_stats(model, 0, &after);
     CHECK(after.free_blocks == after.total_blocks && after.reused_blocks_total >= 9);
+    /* evaluation through a session of its own: the bits of the whole sequence, nothing held afterwards, three slots free again */
+    CHECK(kipp_model_eval(model, tokens, n, spare, vocab, &error) == 0 && same_bits(spare, whole + (size_t)(n - 1) * vocab, vocab));
+    CHECK(kipp_model_eval(model, tokens, n, spare, vocab - 1, &error) != 0 && error.code == KIPP_ERROR_RANGE);
+    CHECK(kipp_model_eval(model, tokens, 0, spare, vocab, &error) != 0 && error.code == KIPP_ERROR_RANGE);
+    CHECK(kipp_model_eval(model, tokens, KIPP_MODEL_EVAL_LIMIT + 1, spare, vocab, &error) != 0 && error.code == KIPP_ERROR_RANGE);
+    kipp_model_kv_pool_stats(model, 0, &after);
+    CHECK(after.free_blocks == after.total_blocks && model->session_count == 0);
     CHECK(kipp_model_close(model, &error) == 0);
+    /* the short ways to open: a path alone, a path and a pool */
+    CHECK(strcmp(kipp_backend_name(KIPP_PATH_CPU_FP32), kipp_path_name(KIPP_PATH_CPU_FP32)) == 0);
+    CHECK(kipp_model_open_pooled(folder, KIPP_PATH_CPU_FP32, 0, &model, &error) != 0 && error.code == KIPP_ERROR_ARGUMENT);
+    CHECK(kipp_model_open_pooled(folder, KIPP_PATH_CPU_FP32, 7, &model, &error) == 0);
+    if (model != NULL) {
+        kipp_model_kv_pool_stats(model, 0, &after);
+        CHECK(after.total_blocks == 7 && kipp_model_get_info(model, &info) == 0 && info.path == KIPP_PATH_CPU_FP32);
+        CHECK(kipp_model_eval(model, tokens, n, spare, vocab, &error) == 0 && same_bits(spare, whole + (size_t)(n - 1) * vocab, vocab));
+        CHECK(kipp_model_close(model, &error) == 0);
+    }
+    CHECK(kipp_model_open_backend(folder, KIPP_PATH_CPU_FP32, &model, &error) == 0);
+    if (model != NULL) {
+        CHECK(kipp_model_get_info(model, &info) == 0 && info.path == KIPP_PATH_CPU_FP32 && info.page_tokens == 16);
+        CHECK(kipp_model_close(model, &error) == 0);
+    }
     free(whole);
     free(cut);
     free(spare);

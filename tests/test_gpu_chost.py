@@ -104,6 +104,13 @@ def test_c_host_sessions_on_the_gpu(model_folders, tiny_configs):
         assert model.pool_stats()["free_blocks"] == before and (second.length, third.length) == (64, 0)
         row = model.step([(third, toks[:20], [19])])
         H.assert_close(row, ref[19:20], H.NMSE_BF16["tiny"], "a step after a refused one")
+        second.destroy()
+        third.destroy()
+        # evaluation without a session (a session of its own, gone afterwards; a published beginning is not adopted)
+        H.assert_close(model.eval(toks[:30])[None], ref[29:30], H.NMSE_BF16["tiny"], "model eval")
+        assert model.pool_stats()["free_blocks"] == model.pool_stats()["total_blocks"]
+        with pytest.raises(KippError, match="between 1 and 256"):
+            model.eval(list(toks) * 5)
 
 
 def test_c_host_products_of_every_row_class(model_folders, tiny_configs):
