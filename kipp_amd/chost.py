@@ -274,6 +274,7 @@ class CModel:
         self.lib.kipp_model_get_info(self.handle, ctypes.byref(info))
         self.info = info
         self.vocab_size = info.vocab_size
+        self.context_length = info.context_length
 
     @property
     def graph_replays(self) -> int:

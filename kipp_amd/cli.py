@@ -75,12 +75,7 @@ def build_parser() -> argparse.ArgumentParser:
     return ap
 
 
-def run_perplexity(args) -> int:
-    """Windows of `--ppl-window` tokens that do not overlap, each from an empty
-    context, no burn-in; a window of W tokens scores its W - 1 targets
-    (/root/reference/src/kipp_cli.c:646-801: the protocol and the lines printed)."""
-    import torch
-    from .engine import Engine, StepEntry
+def _ppl_stream(args) -> list:
     with open(args.ppl, "rb") as f:
         raw = f.read()
     if len(raw) % 4:
@@ -90,6 +85,56 @@ def run_perplexity(args) -> int:
         stream = stream[:args.ppl_limit]
     if len(stream) < 2:
         raise SystemExit("kipp: ppl: need at least two tokens to score")
+    return stream
+
+
+def run_perplexity_c(args, stream) -> int:
+    """The same protocol through the C host: one session, reset before every window, every portion's rows from one step."""
+    import numpy as np
+    from .chost import CModel
+    path = args.path or ("gpu-bf16" if args.dtype == "bfloat16" else "gpu-fp32")
+    window = args.ppl_window
+    with CModel(args.model, path=path, page_tokens=args.page, kv_pool_pages=args.kv_pages or -(-window // args.page), max_sessions=1,
+                max_step_tokens=max(args.prefill_chunk, 1), share_prefixes=False) as model:
+        if not 2 <= window <= model.context_length:
+            raise SystemExit(f"kipp: --ppl-window must be between 2 and {model.context_length}")
+        for index, token in enumerate(stream):
+            if not 0 <= token < model.vocab_size:
+                raise SystemExit(f"kipp: ppl: token {index} is out of range")
+        windows = -(-len(stream) // window)
+        nll, scored = 0.0, 0
+        started = time.perf_counter()
+        session = model.session(window)
+        for w in range(windows):
+            tokens = stream[w * window:(w + 1) * window]
+            if len(tokens) < 2:
+                break
+            session.reset()
+            for at in range(0, len(tokens), args.prefill_chunk):
+                chunk = tokens[at:at + args.prefill_chunk]
+                wide = session.eval_scored(chunk, len(chunk)).astype(np.float64)
+                rows = [r for r in range(len(chunk)) if at + r + 1 < len(tokens)]
+                if rows:
+                    wide = wide[rows]
+                    top = wide.max(axis=-1)
+                    targets = np.asarray([tokens[at + r + 1] for r in rows])
+                    nll += float((top + np.log(np.exp(wide - top[:, None]).sum(axis=-1)) - wide[np.arange(len(rows)), targets]).sum())
+                    scored += len(rows)
+            print(f"ppl: window {w + 1}/{windows} ppl={math.exp(nll / scored):.4f}", file=sys.stderr)
+        print(f"KIPP_PPL backend={path} tokens={len(stream)} scored={scored} window={window} nll={nll:.9f} "
+              f"ppl={math.exp(nll / scored):.6f} seconds={time.perf_counter() - started:.3f}", file=sys.stderr)
+    return 0
+
+
+def run_perplexity(args) -> int:
+    """Windows of `--ppl-window` tokens that do not overlap, each from an empty
+    context, no burn-in; a window of W tokens scores its W - 1 targets
+    (/root/reference/src/kipp_cli.c:646-801: the protocol and the lines printed)."""
+    stream = _ppl_stream(args)
+    if args.host == "c":
+        return run_perplexity_c(args, stream)
+    import torch
+    from .engine import Engine, StepEntry
     window = args.ppl_window
     engine = Engine.from_folder(args.model, dtype=args.dtype, page_size=args.page,
                                 num_pages=args.kv_pages or -(-window // args.page), max_requests=1, share_prefixes=False)
@@ -232,8 +277,6 @@ def run_c_host(args, tokens) -> int:
 
 def _run(args) -> int:
     if args.ppl:
-        if args.host == "c":
-            raise SystemExit("kipp: --ppl runs on the Python host")
         return run_perplexity(args)
     if not 1 <= args.top <= 100:
         raise SystemExit("kipp: --top must be between 1 and 100")

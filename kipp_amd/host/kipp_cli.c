@@ -6,8 +6,10 @@
  * engine has no tokenizer).
  *
  *   kipp --model DIR --tokens 5,17,3 --decode 16 [--path gpu-bf16|gpu-fp32|cpu-fp32]
+ *   kipp --model DIR --ppl tokens.u32 --ppl-window 512        perplexity over a token file (:646-801)
  */
 #include <errno.h>
+#include <math.h>
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
@@ -16,7 +18,7 @@
 #include "kipp_amd.h"
 
 static void usage(FILE *out) {
-    fputs("usage: kipp --model DIR (--tokens 5,17,3 | --tokens-file F.u32) [options]\n"
+    fputs("usage: kipp --model DIR (--tokens 5,17,3 | --tokens-file F.u32 | --ppl F.u32) [options]\n"
           "  --path gpu-bf16|gpu-fp32|cpu-fp32   execution path, never a fallback (default gpu-bf16)\n"
           "  --decode N          tokens to generate (default 0)\n"
           "  --temperature F     0 = greedy argmax (default)\n"
@@ -32,6 +34,9 @@ static void usage(FILE *out) {
           "  --kv-mib F          size of the pool in MiB instead\n"
           "  --prefill-chunk N   largest portion of a prompt in one step (default 512)\n"
           "  --max-step-tokens N token budget of one step (default 2048)\n"
+          "  --ppl FILE          perplexity over a file of little-endian uint32 tokens\n"
+          "  --ppl-window N      tokens of one window; each starts from an empty context (default 2048)\n"
+          "  --ppl-limit N       score at most N tokens of the file (0 = all)\n"
           "  --kernels DIR       folder of the built kernel libraries\n",
           out);
 }
@@ -100,8 +105,65 @@ static int read_token_file(const char *path, uint32_t **out, size_t *count) {
     return 0;
 }
 
+/* Perplexity: windows of `window` tokens that do not overlap, each from an empty session, no burn-in; a window of W tokens
+ * scores its W - 1 targets.  Portions of `chunk` tokens, every row's logits from one step (eval_scored); the sums in double. */
+static int run_perplexity(kipp_model *model, const kipp_model_info *info, const uint32_t *stream, size_t token_count, size_t window,
+                          size_t chunk) {
+    int status = 1;
+    kipp_error error;
+    kipp_session *session = NULL;
+    const uint32_t vocab = info->vocab_size;
+    float *logits = malloc(chunk * (size_t)vocab * sizeof(float));
+    if (logits == NULL) {
+        fprintf(stderr, "kipp: ppl: unable to allocate logits\n");
+        return 1;
+    }
+    if (kipp_session_create(model, (uint32_t)window, &session, &error) != 0) {
+        fprintf(stderr, "kipp: ppl: session: %s\n", error.message);
+        goto done;
+    }
+    const size_t windows = (token_count + window - 1) / window;
+    size_t scored = 0;
+    double nll = 0.0;
+    const double started = seconds();
+    for (size_t w = 0; w < windows; ++w) {
+        const uint32_t *tokens = stream + w * window;
+        const size_t length = token_count - w * window < window ? token_count - w * window : window;
+        if (length < 2) break; /* a tail of one token has nothing to score */
+        if (kipp_session_reset(session, &error) != 0) {
+            fprintf(stderr, "kipp: ppl: reset: %s\n", error.message);
+            goto done;
+        }
+        for (size_t at = 0; at < length; at += chunk) {
+            const size_t n = length - at < chunk ? length - at : chunk;
+            if (kipp_session_eval_scored(session, tokens + at, n, logits, (uint32_t)n, &error) != 0) {
+                fprintf(stderr, "kipp: ppl: eval: %s\n", error.message);
+                goto done;
+            }
+            for (size_t r = 0; r < n && at + r + 1 < length; ++r) { /* row r predicts the token behind it, inside the window */
+                const float *row = logits + r * (size_t)vocab;
+                float top = row[0];
+                for (uint32_t t = 1; t < vocab; ++t) top = row[t] > top ? row[t] : top;
+                double sum = 0.0;
+                for (uint32_t t = 0; t < vocab; ++t) sum += exp((double)row[t] - (double)top);
+                nll += (double)top + log(sum) - (double)row[tokens[at + r + 1]];
+                ++scored;
+            }
+        }
+        fprintf(stderr, "ppl: window %zu/%zu ppl=%.4f\n", w + 1, windows, exp(nll / (double)scored));
+    }
+    fprintf(stderr, "KIPP_PPL backend=%s tokens=%zu scored=%zu window=%zu nll=%.9f ppl=%.6f seconds=%.3f\n", kipp_path_name(info->path),
+            token_count, scored, window, nll, exp(nll / (double)scored), seconds() - started);
+    status = 0;
+done:
+    kipp_session_destroy(session);
+    free(logits);
+    return status;
+}
+
 int main(int argc, char **argv) {
-    const char *model_dir = NULL, *tokens_text = NULL, *tokens_file = NULL, *kernels = NULL, *path_name = "gpu-bf16";
+    const char *model_dir = NULL, *tokens_text = NULL, *tokens_file = NULL, *kernels = NULL, *path_name = "gpu-bf16", *ppl_file = NULL;
+    unsigned long ppl_window = 2048, ppl_limit = 0;
     unsigned long decode = 0, top_k = 0, top_n = 10, page = 16, kv_pages = 0, prefill_chunk = 512, max_step_tokens = 2048, max_context = 0;
     unsigned long long seed = 1;
     double temperature = 0.0, top_p = 1.0, min_p = 0.0, kv_mib = 0.0;
@@ -124,6 +186,9 @@ int main(int argc, char **argv) {
         else if (strcmp(arg, "--tokens-file") == 0) tokens_file = value;
         else if (strcmp(arg, "--path") == 0 || strcmp(arg, "--backend") == 0) path_name = value;
         else if (strcmp(arg, "--kernels") == 0) kernels = value;
+        else if (strcmp(arg, "--ppl") == 0) ppl_file = value;
+        else if (strcmp(arg, "--ppl-window") == 0) ppl_window = strtoul(value, NULL, 10);
+        else if (strcmp(arg, "--ppl-limit") == 0) ppl_limit = strtoul(value, NULL, 10);
         else if (strcmp(arg, "--decode") == 0) decode = strtoul(value, NULL, 10);
         else if (strcmp(arg, "--temperature") == 0) temperature = strtod(value, NULL);
         else if (strcmp(arg, "--top-p") == 0) top_p = strtod(value, NULL);
@@ -176,11 +241,29 @@ int main(int argc, char **argv) {
     }
     uint32_t *tokens = NULL;
     size_t token_count = 0;
-    if ((tokens_text == NULL) == (tokens_file == NULL)) {
+    if (ppl_file != NULL) {
+        if (tokens_text != NULL || tokens_file != NULL || decode != 0) {
+            fprintf(stderr, "kipp: --ppl cannot be combined with --tokens, --tokens-file or --decode\n");
+            return 2;
+        }
+        if (ppl_window < 2) {
+            fprintf(stderr, "kipp: --ppl-window must be at least 2\n");
+            return 2;
+        }
+        if (read_token_file(ppl_file, &tokens, &token_count) != 0) {
+            fprintf(stderr, "kipp: ppl: '%s' is not a uint32 token file\n", ppl_file);
+            return 2;
+        }
+        if (ppl_limit != 0 && ppl_limit < token_count) token_count = ppl_limit;
+        if (token_count < 2) {
+            fprintf(stderr, "kipp: ppl: need at least two tokens to score\n");
+            free(tokens);
+            return 2;
+        }
+    } else if ((tokens_text == NULL) == (tokens_file == NULL)) {
         fprintf(stderr, "kipp: give --tokens or --tokens-file\n");
         return 2;
-    }
-    if ((tokens_text != NULL ? parse_tokens(tokens_text, &tokens, &token_count) : read_token_file(tokens_file, &tokens, &token_count)) != 0) {
+    } else if ((tokens_text != NULL ? parse_tokens(tokens_text, &tokens, &token_count) : read_token_file(tokens_file, &tokens, &token_count)) != 0) {
         fprintf(stderr, "kipp: the prompt must be token ids (5,17,3, or a file of little-endian uint32)\n");
         return 2;
     }
@@ -201,7 +284,8 @@ int main(int argc, char **argv) {
     config.max_sessions = 1;
     config.max_step_tokens = (uint32_t)max_step_tokens;
     config.kernel_dir = kernels;
-    size_t capacity = token_count + decode;
+    size_t capacity = ppl_file != NULL ? ppl_window : token_count + decode;
+    if (ppl_file != NULL && max_step_tokens < prefill_chunk) config.max_step_tokens = (uint32_t)prefill_chunk;
     config.kv_pool_pages = kv_pages != 0 ? (uint32_t)kv_pages : (uint32_t)((capacity + page - 1) / page);
     if (kv_mib > 0.0) {
         /* what a page takes is asked of a model with a pool of one page: bytes of all groups' slabs for that page and its spare */
@@ -230,6 +314,20 @@ int main(int argc, char **argv) {
     }
     kipp_model_info info;
     kipp_model_get_info(model, &info);
+    if (ppl_file != NULL) {
+        if (ppl_window > info.context_length) {
+            fprintf(stderr, "kipp: --ppl-window must be between 2 and %u\n", info.context_length);
+            goto done;
+        }
+        for (size_t i = 0; i < token_count; ++i) {
+            if (tokens[i] >= info.vocab_size) {
+                fprintf(stderr, "kipp: ppl: token %zu is out of range\n", i);
+                goto done;
+            }
+        }
+        rc = run_perplexity(model, &info, tokens, token_count, ppl_window, prefill_chunk);
+        goto done;
+    }
     /* the session holds prompt + decode tokens, within the context length (/root/reference/src/kipp_cli.c:1057-1067) */
     size_t limit = max_context != 0 && max_context < info.context_length ? max_context : info.context_length;
     if (token_count > limit || decode > limit - token_count) {

@@ -489,6 +489,53 @@ def test_the_c_command_line_matches_the_python_one(model_folders, tiny_configs, 
     assert subprocess.run([exe, "--help"], capture_output=True, text=True).stdout.startswith("usage: kipp")
 
 
+def test_perplexity_through_the_c_command_lines(model_folders, tiny_configs, capsys, tmp_path):
+    """--ppl on the scalar path, by kipp_cli.c and by `python -m kipp_amd.cli --host c`: windows that do not overlap, each
+    from an empty session, a window of W tokens scores W - 1 targets (/root/reference/src/kipp_cli.c:722-790); against
+    the plain implementation, and the refusals."""
+    import subprocess
+    from kipp_amd.cli import main
+    from kipp_amd.host import build
+    from tests.plain import qwen3_plain as plain
+    exe = build.cli_path()
+    folder = model_folders[("b", "float32")]
+    vocab = tiny_configs["b"]["vocab_size"]
+    stream = H.random_tokens(55, 75, vocab)
+    path = tmp_path / "tokens.u32"
+    path.write_bytes(np.asarray(stream, "<u4").tobytes())
+    cfg, weights = plain.load_folder(folder)
+    nll, scored = 0.0, 0
+    for at in range(0, 75, 32):
+        tokens = stream[at:at + 32]
+        logits = plain.forward_whole(cfg, weights, tokens)
+        for r in range(len(tokens) - 1):
+            row = logits[r]
+            nll += row.max() + np.log(np.exp(row - row.max()).sum()) - row[tokens[r + 1]]
+            scored += 1
+    common = ["--model", folder, "--path", "cpu-fp32", "--page", "8", "--ppl", str(path), "--ppl-window", "32", "--prefill-chunk", "10"]
+    proc = subprocess.run([exe] + common, capture_output=True, text=True, timeout=120)
+    assert proc.returncode == 0, proc.stderr
+    assert main(common + ["--host", "c"]) == 0
+    for stderr in (proc.stderr, capsys.readouterr().err):
+        line = [l for l in stderr.splitlines() if l.startswith("KIPP_PPL")][0]
+        fields = dict(f.split("=") for f in line.split()[1:])
+        assert fields["backend"] == "cpu-fp32" and int(fields["tokens"]) == 75 and int(fields["scored"]) == scored == 72
+        assert int(fields["window"]) == 32 and abs(float(fields["nll"]) - nll) < 1e-3 and abs(float(fields["ppl"]) - np.exp(nll / scored)) < 1e-3
+        assert "ppl: window 3/3" in stderr
+    limited = subprocess.run([exe] + common + ["--ppl-limit", "33"], capture_output=True, text=True, timeout=120)
+    assert limited.returncode == 0 and "tokens=33 scored=31" in limited.stderr          # the second window's one token scores nothing
+    (tmp_path / "odd.u32").write_bytes(b"12345")
+    (tmp_path / "far.u32").write_bytes(np.asarray([1, vocab], "<u4").tobytes())
+    for extra, code, words in ((["--decode", "3"], 2, "cannot be combined"),
+                               (["--ppl-window", "1"], 2, "at least 2"),
+                               (["--ppl-window", "100000"], 1, "--ppl-window must be between 2 and"),
+                               (["--ppl", str(tmp_path / "odd.u32")], 2, "not a uint32 token file"),
+                               (["--ppl", str(tmp_path / "far.u32")], 1, "token 1 is out of range"),
+                               (["--ppl-limit", "1"], 2, "at least two tokens")):
+        bad = subprocess.run([exe] + common + extra, capture_output=True, text=True, timeout=120)
+        assert bad.returncode == code and words in bad.stderr, (extra, bad.returncode, bad.stderr)
+
+
 def test_step_argmax_is_the_argmax_of_step(model_folders, tiny_configs):
     """kipp_step_argmax: the same step answered with one index a wanted place, the lowest among equal logits; room is checked."""
     cfg = tiny_configs["a"]

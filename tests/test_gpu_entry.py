@@ -255,6 +255,13 @@ def test_command_line_perplexity(model_folders, tmp_path):
     assert fields["backend"] == "hip-float32" and int(fields["tokens"]) == 75 and int(fields["scored"]) == scored == 72
     assert abs(float(fields["nll"]) - nll) < 1e-3 and abs(float(fields["ppl"]) - np.exp(nll / scored)) < 1e-3
     assert "ppl: window 3/3" in run.stderr
+    through_c = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "kipp"), "--model", folder, "--host", "c", "--path", "gpu-fp32",
+                                "--page", "8", "--ppl", str(path), "--ppl-window", "32", "--prefill-chunk", "10"],
+                               capture_output=True, text=True, timeout=300)
+    assert through_c.returncode == 0, through_c.stderr
+    line = [l for l in through_c.stderr.splitlines() if l.startswith("KIPP_PPL")][0]
+    fields = dict(f.split("=") for f in line.split()[1:])
+    assert fields["backend"] == "gpu-fp32" and int(fields["scored"]) == 72 and abs(float(fields["nll"]) - nll) < 1e-3
     bad = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "kipp"), "--model", folder, "--backend", "metal", "--tokens", "1"],
                          capture_output=True, text=True, timeout=300)
     assert bad.returncode != 0 and "only hip" in bad.stderr
