@@ -65,6 +65,11 @@ class _StepItem(ctypes.Structure):
                 ("want_count", ctypes.c_size_t)]
 
 
+class _RowChoice(ctypes.Structure):
+    _fields_ = [("temperature", ctypes.c_float), ("top_p", ctypes.c_float), ("top_k", ctypes.c_uint32), ("min_p", ctypes.c_float),
+                ("uniform", ctypes.c_double)]
+
+
 class _BatchItem(ctypes.Structure):
     _fields_ = [("session", ctypes.c_void_p), ("tokens", _u32p), ("token_count", ctypes.c_size_t), ("logits", _f32p)]
 
@@ -148,6 +153,7 @@ def library(variant: str = "gpu") -> ctypes.CDLL:
             "kipp_model_eval": [vp, _u32p, sz, _f32p, sz, err],
             "kipp_step": [vp, ctypes.POINTER(_StepItem), sz, _f32p, sz, err],
             "kipp_step_argmax": [vp, ctypes.POINTER(_StepItem), sz, _u32p, sz, err],
+            "kipp_step_sample": [vp, ctypes.POINTER(_StepItem), sz, ctypes.POINTER(_RowChoice), _u32p, sz, err],
             "kipp_sample_ex": [_f32p, sz, ctypes.POINTER(_SampleParams), ctypes.POINTER(ctypes.c_uint64), _u32p, err],
             "kipp_test_scramble_session_kv": [vp, err],
             "kipp_scheduler_create": [vp, ctypes.POINTER(_SchedulerConfig), ctypes.POINTER(vp), err],
@@ -163,6 +169,7 @@ def library(variant: str = "gpu") -> ctypes.CDLL:
             fn = getattr(lib, name)
             fn.argtypes, fn.restype = argtypes, ctypes.c_int
         lib.kipp_session_destroy.argtypes, lib.kipp_session_destroy.restype = [vp], None
+        lib.kipp_rng_uniform.argtypes, lib.kipp_rng_uniform.restype = [ctypes.POINTER(ctypes.c_uint64)], ctypes.c_double
         lib.kipp_scheduler_destroy.argtypes, lib.kipp_scheduler_destroy.restype = [vp], None
         lib.kipp_scheduler_last_logits.argtypes, lib.kipp_scheduler_last_logits.restype = [vp, ctypes.c_uint64], _f32p
         lib.kipp_test_fail_forward_after.argtypes, lib.kipp_test_fail_forward_after.restype = [vp, ctypes.c_int], None
@@ -325,6 +332,27 @@ class CModel:
         out = np.zeros(max(wanted, 1), dtype=np.uint32)
         error = _Error()
         if self.lib.kipp_step_argmax(self.handle, items, len(entries), out.ctypes.data_as(_u32p), wanted, ctypes.byref(error)) != 0:
+            _raise(self.lib, error)
+        return [int(t) for t in out[:wanted]]
+
+    def step_sample(self, entries: Sequence[Tuple[CSession, Sequence[int], Sequence[int]]], choices: Sequence[tuple]) -> List[int]:
+        """The same batch, answered with one token for every wanted place, chosen where the path computes: `choices` has
+        (temperature, top_p, top_k, min_p, uniform) for each wanted place in order; temperature <= 0 takes the largest logit."""
+        items = (_StepItem * len(entries))()
+        keep = []
+        wanted = 0
+        for i, (session, tokens, want) in enumerate(entries):
+            t, tp = _u32(tokens)
+            w, wp = _u32(want)
+            keep.append((t, w))
+            items[i] = _StepItem(session.handle, tp, len(t), wp if len(w) else None, len(w))
+            wanted += len(w)
+        if len(choices) != wanted:
+            raise ValueError("one choice for every wanted place")
+        rows = (_RowChoice * max(wanted, 1))(*[_RowChoice(float(t), float(p), int(k), float(m), float(u)) for t, p, k, m, u in choices])
+        out = np.zeros(max(wanted, 1), dtype=np.uint32)
+        error = _Error()
+        if self.lib.kipp_step_sample(self.handle, items, len(entries), rows, out.ctypes.data_as(_u32p), wanted, ctypes.byref(error)) != 0:
             _raise(self.lib, error)
         return [int(t) for t in out[:wanted]]
 
@@ -497,6 +525,10 @@ class Rng:
 
     def __init__(self, seed: int):
         self.state = ctypes.c_uint64(seed)
+
+    def uniform(self, variant: str = "host-only") -> float:
+        """The next draw in [0, 1), as kipp_sample_ex takes it."""
+        return float(library(variant).kipp_rng_uniform(ctypes.byref(self.state)))
 
 
 def sample(logits: np.ndarray, temperature: float = 0.0, top_p: float = 1.0, top_k: int = 0, min_p: float = 0.0,

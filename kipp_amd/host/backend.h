@@ -92,6 +92,10 @@ struct kipp_runtime {
     int (*gather_rows)(kipp_runtime *rt, const float *x, const int32_t *index, float *out, uint32_t n, uint32_t width, kipp_error *error);
     /* out[r] = the index of the largest of logits[r, :vocab], the lowest among equals (/root/reference/src/kipp.c:3459-3464) */
     int (*argmax)(kipp_runtime *rt, const float *logits, int32_t *out, uint32_t rows, uint32_t vocab, kipp_error *error);
+    /* Optional (NULL: the caller samples on the host).  *out = memory of the path's own with one token a row, each chosen as
+     * its kipp_row_choice (host memory) says; it takes nothing from the step's workspace, so it may follow a recorded step. */
+    int (*sample)(kipp_runtime *rt, const float *logits, const kipp_row_choice *choices, int32_t **out, uint32_t rows, uint32_t vocab,
+                  kipp_error *error);
 
     /* Optional (NULL: none).  Recording: between graph_begin and graph_end the operations above are recorded instead of run
      * (no memory may be made meanwhile: the step's workspace says so, and the recording is dropped); graph_end with `keep`

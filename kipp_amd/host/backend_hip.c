@@ -58,6 +58,8 @@ typedef int (*fn_int3)(int, int, int);
 typedef int (*fn_scale_rows)(const void *, const float *, void *, int, int, int, int, float, int, hipStream_t);
 typedef int (*fn_tile_weight)(const void *, void *, int, int, int, hipStream_t);
 typedef int (*fn_argmax)(const float *, int32_t *, int, int, float *, hipStream_t);
+typedef int (*fn_sample)(const float *, int, int, const float *, const int32_t *, const float *, const float *, const double *, int32_t *,
+                         hipStream_t);
 typedef int (*fn_attention_decode_fused)(const float *, int, int, const float *, const float *, float, const float *, const float *, int, void *,
                                          void *, void *, float *, float *, const int32_t *, const int32_t *, const int32_t *, const int32_t *, int,
                                          int, int, int, int, int, float, int, int, int, int32_t *, int, hipStream_t);
@@ -106,6 +108,10 @@ typedef struct {
     fn_tile_weight tile_weight;
     fn_argmax argmax;
     fn_int_int argmax_scratch_floats;
+    fn_sample sample;
+    unsigned char *sample_host; /* a step's kipp_row_choices, packed by field */
+    void *sample_device;        /* the same on the GPU, and behind them the tokens chosen */
+    uint32_t sample_rows;       /* rows both have room for */
     bool fuse;             /* few rows: residual add and norm ride on the products around them, decode attention starts from the QKV product */
     bool steps_major;      /* rows that one few-rows product writes for the next: in the order that product reads fastest */
     bool merge_in_kernel;  /* decode attention: the splits of a head are merged by the last of their workgroups to finish */
@@ -220,6 +226,7 @@ static int open_common(hip_state *st, kipp_error *error) {
     KIPP_SYM(libs[4], skinny_sumsq_stride, "kipp_gemm_skinny_sumsq_stride");
     KIPP_SYM(libs[7], argmax, "kipp_argmax");
     KIPP_SYM(libs[7], argmax_scratch_floats, "kipp_argmax_scratch_floats");
+    KIPP_SYM(libs[7], sample, "kipp_sample");
     return 0;
 }
 
@@ -268,6 +275,8 @@ static void hip_destroy(kipp_runtime *rt) {
     if (st != NULL) {
         hipStreamSynchronize(st->stream);
         if (st->arrivals != NULL) hipFree(st->arrivals);
+        if (st->sample_device != NULL) hipFree(st->sample_device);
+        free(st->sample_host);
         if (st->stream != NULL) hipStreamDestroy(st->stream);
         /* the libraries stay loaded: their kernels may be registered with the HIP runtime until the process ends */
         free(st);
@@ -650,6 +659,50 @@ static int hip_gated(kipp_runtime *rt, const kipp_rows *x, const kipp_weight *w,
     if (rc != 0) return refused(error, "swiglu (pairs)", rc);
     *done = true;
     return 0;
+}
+
+/* The device sampler over the rows of a step.  Its parameters go up in one copy, packed by field
+ * ([temperature | top_p | min_p | top_k] of 4 bytes a row, then the draws of 8), into memory of its own that is made once for
+ * the most rows a step can want and stays where it is: the step's workspace is not touched (a recorded step's logits lie
+ * there), and a call that follows a recording allocates nothing. */
+static int hip_sample(kipp_runtime *rt, const float *logits, const kipp_row_choice *choices, int32_t **out, uint32_t rows, uint32_t vocab,
+                      kipp_error *error) {
+    hip_state *st = rt->state;
+    if (rows == 0) return 0;
+    if (vocab >= (1u << 24)) return kipp_fail(error, KIPP_ERROR_UNSUPPORTED, "the device sampler takes vocabularies below 2^24");
+    if (rows > st->sample_rows) {
+        uint32_t room = rows > 256 ? rows : 256;
+        unsigned char *host = realloc(st->sample_host, (size_t)room * 24);
+        if (host == NULL) return kipp_fail(error, KIPP_ERROR_MEMORY, "out of memory");
+        st->sample_host = host;
+        st->sample_rows = 0;
+        if (st->sample_device != NULL) {
+            hipStreamSynchronize(st->stream);
+            hipFree(st->sample_device);
+            st->sample_device = NULL;
+        }
+        hipError_t code = hipMalloc(&st->sample_device, (size_t)room * 28);
+        if (code != hipSuccess) return hip_bad(error, code, "hipMalloc");
+        st->sample_rows = room;
+    }
+    float *f32 = (float *)st->sample_host;
+    int32_t *i32 = (int32_t *)(st->sample_host + (size_t)rows * 12);
+    double *f64 = (double *)(st->sample_host + (size_t)rows * 16);
+    for (uint32_t r = 0; r < rows; ++r) {
+        const bool sampled = choices[r].temperature > 0.0f;
+        f32[r] = sampled ? choices[r].temperature : 0.0f;
+        f32[rows + r] = sampled ? choices[r].top_p : 1.0f;
+        f32[2 * rows + r] = sampled ? choices[r].min_p : 0.0f;
+        i32[r] = sampled ? (int32_t)(choices[r].top_k < (uint32_t)INT32_MAX ? choices[r].top_k : 0) : 0;
+        f64[r] = sampled ? choices[r].uniform : 0.0;
+    }
+    unsigned char *d = st->sample_device;
+    hipError_t code = hipMemcpyAsync(d, st->sample_host, (size_t)rows * 24, hipMemcpyHostToDevice, st->stream);
+    if (code != hipSuccess) return hip_bad(error, code, "copy to the GPU");
+    *out = (int32_t *)(d + (size_t)st->sample_rows * 24);
+    int rc = st->sample(logits, (int)rows, (int)vocab, (const float *)d, (const int32_t *)(d + (size_t)rows * 12), (const float *)d + rows,
+                        (const float *)d + 2 * rows, (const double *)(d + (size_t)rows * 16), *out, st->stream);
+    return rc == 0 ? 0 : refused(error, "sample", rc);
 }
 
 static int hip_argmax(kipp_runtime *rt, const float *logits, int32_t *out, uint32_t rows, uint32_t vocab, kipp_error *error) {
@@ -1072,6 +1125,7 @@ kipp_runtime *kipp_runtime_hip(kipp_path path, int device, const char *kernel_di
     rt->gated = hip_gated;
     rt->decode_attention = hip_decode_attention;
     rt->argmax = hip_argmax;
+    rt->sample = hip_sample;
     rt->after_failed_step = hip_after_failed_step;
     if (path == KIPP_PATH_GPU_BF16) { /* the 32-bit path is for checking, not for speed: its steps run as they are */
         rt->graph_begin = hip_graph_begin;

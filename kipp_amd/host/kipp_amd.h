@@ -182,6 +182,25 @@ int kipp_step(kipp_model *model, const kipp_step_item *items, size_t item_count,
 int kipp_step_argmax(kipp_model *model, const kipp_step_item *items, size_t item_count, uint32_t *tokens, size_t token_capacity,
                      kipp_error *error);
 
+/* How one wanted row of a step is chosen where the path computes (kipp_step_sample): the largest logit where
+ * temperature <= 0, else temperature sampling with top-k (0: off), min-p (0: off) and top-p in the order of
+ * kipp_sample_ex, with `uniform` in [0, 1) as the one draw that kipp_sample_ex would take from its generator. */
+typedef struct {
+    float temperature;
+    float top_p;
+    uint32_t top_k;
+    float min_p;
+    double uniform;
+} kipp_row_choice;
+
+/* kipp_step with one token for every wanted place, chosen beside the logits: `choices` has one entry a wanted place, in the
+ * order of the items and their places.  Only a number a row comes back.  KIPP_ERROR_UNSUPPORTED on a path that has no
+ * sampler of its own (the scalar one: take kipp_step and kipp_sample_ex). */
+int kipp_step_sample(kipp_model *model, const kipp_step_item *items, size_t item_count, const kipp_row_choice *choices, uint32_t *tokens,
+                     size_t token_capacity, kipp_error *error);
+/* The next draw of a generator, as kipp_sample_ex takes it (/root/reference/src/kipp.c:3322-3333): in [0, 1); the state must not be 0. */
+double kipp_rng_uniform(uint64_t *rng_state);
+
 int kipp_sample(const float *logits, size_t logits_count, float temperature, float top_p, uint64_t *rng_state, uint32_t *out_token,
                 kipp_error *error);
 

@@ -16,7 +16,7 @@
 #include "internal.h"
 
 /* /root/reference/src/kipp.c:3322-3333 */
-static double uniform_unit(uint64_t *state) {
+double kipp_rng_uniform(uint64_t *state) {
     uint64_t x = *state;
     x ^= x >> 12;
     x ^= x << 25;
@@ -155,7 +155,7 @@ int kipp_sample_ex(const float *logits, size_t logits_count, const kipp_sample_p
             nucleus = 1;
             kept = items[0].logit;
         }
-        double draw = uniform_unit(rng_state) * kept, cumulative = 0.0;
+        double draw = kipp_rng_uniform(rng_state) * kept, cumulative = 0.0;
         uint32_t token = items[nucleus - 1].token;
         for (size_t i = 0; i < nucleus; ++i) {
             cumulative += items[i].logit;

@@ -18,6 +18,7 @@
 #include <time.h>
 
 #include "internal.h"
+#include "backend.h"
 
 #define RECENT_WINDOW 64 /* tokens the penalties look back over (/root/reference/src/kipp_server.c:848) */
 
@@ -62,7 +63,9 @@ struct kipp_scheduler {
     uint32_t *wants;
     float *logits;
     uint32_t *chosen;
+    kipp_row_choice *choices;
     size_t logits_rows;
+    bool device_sampler; /* the path has a sampler of its own and KIPP_AMD_SAMPLER does not say "host" */
 };
 
 static double now_seconds(void) {
@@ -123,7 +126,10 @@ int kipp_scheduler_create(kipp_model *model, const kipp_scheduler_config *config
     s->logits_rows = s->max_running;
     s->logits = malloc(s->logits_rows * (size_t)model->spec.vocab * sizeof(float));
     s->chosen = malloc(s->logits_rows * sizeof(uint32_t));
-    if (s->items == NULL || s->item_requests == NULL || s->wants == NULL || s->logits == NULL || s->chosen == NULL) {
+    s->choices = malloc(s->logits_rows * sizeof(kipp_row_choice));
+    const char *sampler = getenv("KIPP_AMD_SAMPLER");
+    s->device_sampler = model->rt->sample != NULL && !(sampler != NULL && strcmp(sampler, "host") == 0);
+    if (s->items == NULL || s->item_requests == NULL || s->wants == NULL || s->logits == NULL || s->chosen == NULL || s->choices == NULL) {
         kipp_scheduler_destroy(s);
         return kipp_fail(error, KIPP_ERROR_MEMORY, "out of memory for the scheduler's step");
     }
@@ -146,6 +152,7 @@ void kipp_scheduler_destroy(kipp_scheduler *s) {
     free(s->wants);
     free(s->logits);
     free(s->chosen);
+    free(s->choices);
     free(s);
 }
 
@@ -406,9 +413,29 @@ int kipp_scheduler_step(kipp_scheduler *s, kipp_produced *out, size_t capacity, 
         greedy = s->items[i].want_count == 0 || (p->temperature <= 0.0f && p->frequency_penalty == 0.0f && p->presence_penalty == 0.0f &&
                                                  (p->repetition_penalty == 1.0f || p->repetition_penalty == 0.0f) && p->logit_bias_count == 0);
     }
+    /* else, where no row's logits are changed first (bias, penalties) and the path has a sampler of its own, every row is
+     * chosen there as well, a sampled row with the draw that kipp_sample_ex would take from the request's generator now
+     * (parameters it would refuse go to it, so that it does) */
+    bool beside = !greedy && !s->keep_last_logits && s->device_sampler;
+    uint32_t rows = 0;
+    for (uint32_t i = 0; i < n && beside; ++i) {
+        const kipp_sample_params *p = &s->item_requests[i]->params;
+        if (s->items[i].want_count == 0) continue;
+        beside = p->frequency_penalty == 0.0f && p->presence_penalty == 0.0f && (p->repetition_penalty == 1.0f || p->repetition_penalty == 0.0f) &&
+                 p->logit_bias_count == 0 &&
+                 (p->temperature <= 0.0f || (p->top_p > 0.0f && p->top_p <= 1.0f && p->min_p >= 0.0f && p->min_p <= 1.0f && s->item_requests[i]->rng != 0));
+    }
+    for (uint32_t i = 0; i < n && beside; ++i) {
+        request *r = s->item_requests[i];
+        if (s->items[i].want_count == 0) continue;
+        s->choices[rows++] = (kipp_row_choice){r->params.temperature, r->params.top_p, r->params.top_k, r->params.min_p,
+                                               r->params.temperature > 0.0f ? kipp_rng_uniform(&r->rng) : 0.0};
+    }
+    greedy = greedy || beside; /* from here on: the tokens are in s->chosen */
     kipp_error step_error;
-    int step_rc = greedy ? kipp_step_argmax(s->model, s->items, n, s->chosen, s->logits_rows, &step_error)
-                         : kipp_step(s->model, s->items, n, s->logits, s->logits_rows * (size_t)s->model->spec.vocab, &step_error);
+    int step_rc = beside   ? kipp_step_sample(s->model, s->items, n, s->choices, s->chosen, s->logits_rows, &step_error)
+                  : greedy ? kipp_step_argmax(s->model, s->items, n, s->chosen, s->logits_rows, &step_error)
+                           : kipp_step(s->model, s->items, n, s->logits, s->logits_rows * (size_t)s->model->spec.vocab, &step_error);
     if (step_rc != 0) {
         /* the batch failed as a unit: every request that had tokens in it fails; those that were not in it go on */
         ++s->stats.failed_steps;

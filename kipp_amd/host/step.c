@@ -315,24 +315,35 @@ uint64_t kipp_test_graph_replays(const kipp_model *model) { return model != NULL
 uint64_t kipp_test_cut_attention_steps(const kipp_model *model) { return model != NULL ? model->rt->cut_attention_steps : 0; }
 
 static int step_common(kipp_model *model, const kipp_step_item *items, size_t item_count, float *logits, size_t logits_capacity, uint32_t *best,
-                       kipp_error *error);
+                       const kipp_row_choice *choices, kipp_error *error);
 
 int kipp_step(kipp_model *model, const kipp_step_item *items, size_t item_count, float *logits, size_t logits_capacity,
               kipp_error *error) {
-    return step_common(model, items, item_count, logits, logits_capacity, NULL, error);
+    return step_common(model, items, item_count, logits, logits_capacity, NULL, NULL, error);
+}
+
+int kipp_step_sample(kipp_model *model, const kipp_step_item *items, size_t item_count, const kipp_row_choice *choices, uint32_t *tokens,
+                     size_t token_capacity, kipp_error *error) {
+    uint32_t none;
+    kipp_error_clear(error);
+    if (model != NULL && model->rt->sample == NULL) return kipp_fail(error, KIPP_ERROR_UNSUPPORTED, "this path has no sampler of its own");
+    if (choices == NULL) return kipp_fail(error, KIPP_ERROR_ARGUMENT, "no choices");
+    if (tokens == NULL && token_capacity != 0) return kipp_fail(error, KIPP_ERROR_ARGUMENT, "no room for the tokens");
+    return step_common(model, items, item_count, NULL, tokens != NULL ? token_capacity : 0, tokens != NULL ? tokens : &none, choices, error);
 }
 
 int kipp_step_argmax(kipp_model *model, const kipp_step_item *items, size_t item_count, uint32_t *tokens, size_t token_capacity,
                      kipp_error *error) {
     uint32_t none; /* a step that wants nothing may come without room */
     if (tokens == NULL && token_capacity != 0) return kipp_fail(error, KIPP_ERROR_ARGUMENT, "no room for the tokens");
-    return step_common(model, items, item_count, NULL, tokens != NULL ? token_capacity : 0, tokens != NULL ? tokens : &none, error);
+    return step_common(model, items, item_count, NULL, tokens != NULL ? token_capacity : 0, tokens != NULL ? tokens : &none, NULL, error);
 }
 
-/* `best` NULL: the wanted rows of logits go to `logits` (room for `capacity` floats); else the index of the largest logit of
- * every wanted row goes to `best` (room for `capacity` indices), found where the path computes. */
+/* `best` NULL: the wanted rows of logits go to `logits` (room for `capacity` floats); else one token for every wanted row goes
+ * to `best` (room for `capacity` of them), found where the path computes: the index of the largest logit, or with `choices`
+ * what each row's choice says. */
 static int step_common(kipp_model *model, const kipp_step_item *items, size_t item_count, float *logits, size_t logits_capacity, uint32_t *best,
-                       kipp_error *error) {
+                       const kipp_row_choice *choices, kipp_error *error) {
     kipp_error_clear(error);
     if (model == NULL || (items == NULL && item_count != 0)) return kipp_fail(error, KIPP_ERROR_ARGUMENT, "model and items must be given");
     if (item_count == 0) return 0;
@@ -399,7 +410,8 @@ static int step_common(kipp_model *model, const kipp_step_item *items, size_t it
     if (build_batch(model, items, item_count, single, error) != 0) goto unclaim; /* rounded whether or not steps are recorded: the same launches either way */
     float *device_logits = NULL;
     int32_t *chosen = NULL;
-    if (run_step(model, single && !model->config.eager_steps, best != NULL, &device_logits, &chosen, error) != 0) goto unclaim;
+    if (run_step(model, single && !model->config.eager_steps, best != NULL && choices == NULL, &device_logits, &chosen, error) != 0) goto unclaim;
+    if (choices != NULL && wanted != 0 && model->rt->sample(model->rt, device_logits, choices, &chosen, (uint32_t)wanted, vocab, error) != 0) goto unclaim;
     /* reading back (even nothing) waits for the step's work: what it wrote into the pages is there when it returns */
     if (best != NULL && wanted != 0) {
         if (model->rt->download(model->rt, best, chosen, wanted * sizeof(int32_t), error) != 0) goto unclaim;
