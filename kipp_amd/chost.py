@@ -65,11 +65,6 @@ class _StepItem(ctypes.Structure):
                 ("want_count", ctypes.c_size_t)]
 
 
-class _RowChoice(ctypes.Structure):
-    _fields_ = [("temperature", ctypes.c_float), ("top_p", ctypes.c_float), ("top_k", ctypes.c_uint32), ("min_p", ctypes.c_float),
-                ("uniform", ctypes.c_double)]
-
-
 class _BatchItem(ctypes.Structure):
     _fields_ = [("session", ctypes.c_void_p), ("tokens", _u32p), ("token_count", ctypes.c_size_t), ("logits", _f32p)]
 
@@ -153,7 +148,7 @@ def library(variant: str = "gpu") -> ctypes.CDLL:
             "kipp_model_eval": [vp, _u32p, sz, _f32p, sz, err],
             "kipp_step": [vp, ctypes.POINTER(_StepItem), sz, _f32p, sz, err],
             "kipp_step_argmax": [vp, ctypes.POINTER(_StepItem), sz, _u32p, sz, err],
-            "kipp_step_sample": [vp, ctypes.POINTER(_StepItem), sz, ctypes.POINTER(_RowChoice), _u32p, sz, err],
+            "kipp_step_sample": [vp, ctypes.POINTER(_StepItem), sz, ctypes.POINTER(_SampleParams), ctypes.POINTER(ctypes.c_double), _u32p, sz, err],
             "kipp_sample_ex": [_f32p, sz, ctypes.POINTER(_SampleParams), ctypes.POINTER(ctypes.c_uint64), _u32p, err],
             "kipp_test_scramble_session_kv": [vp, err],
             "kipp_scheduler_create": [vp, ctypes.POINTER(_SchedulerConfig), ctypes.POINTER(vp), err],
@@ -335,9 +330,10 @@ class CModel:
             _raise(self.lib, error)
         return [int(t) for t in out[:wanted]]
 
-    def step_sample(self, entries: Sequence[Tuple[CSession, Sequence[int], Sequence[int]]], choices: Sequence[tuple]) -> List[int]:
-        """The same batch, answered with one token for every wanted place, chosen where the path computes: `choices` has
-        (temperature, top_p, top_k, min_p, uniform) for each wanted place in order; temperature <= 0 takes the largest logit."""
+    def step_sample(self, entries: Sequence[Tuple[CSession, Sequence[int], Sequence[int]]], choices: Sequence[dict]) -> List[int]:
+        """The same batch, answered with one token for every wanted place, chosen where the path computes as kipp_sample_ex
+        would: `choices` has, for each wanted place in order, the sampler's parameters by name (temperature, top_p, top_k,
+        min_p, frequency_penalty, presence_penalty, repetition_penalty, recent, logit_bias) and `uniform`, the draw."""
         items = (_StepItem * len(entries))()
         keep = []
         wanted = 0
@@ -349,10 +345,22 @@ class CModel:
             wanted += len(w)
         if len(choices) != wanted:
             raise ValueError("one choice for every wanted place")
-        rows = (_RowChoice * max(wanted, 1))(*[_RowChoice(float(t), float(p), int(k), float(m), float(u)) for t, p, k, m, u in choices])
+        params = (_SampleParams * max(wanted, 1))()
+        draws = (ctypes.c_double * max(wanted, 1))()
+        for r, c in enumerate(choices):
+            recent, rp = _u32(c.get("recent", ()))
+            bias = c.get("logit_bias") or {}
+            bt, btp = _u32(list(bias.keys()))
+            bv = np.ascontiguousarray(np.asarray(list(bias.values()), dtype=np.float32))
+            keep.append((recent, bt, bv))
+            params[r] = _SampleParams(c.get("temperature", 0.0), c.get("top_p", 1.0), c.get("top_k", 0), c.get("min_p", 0.0),
+                                      c.get("frequency_penalty", 0.0), c.get("presence_penalty", 0.0), c.get("repetition_penalty", 1.0),
+                                      rp if len(recent) else None, len(recent), btp if len(bt) else None,
+                                      bv.ctypes.data_as(_f32p) if len(bv) else None, len(bt))
+            draws[r] = c.get("uniform", 0.0)
         out = np.zeros(max(wanted, 1), dtype=np.uint32)
         error = _Error()
-        if self.lib.kipp_step_sample(self.handle, items, len(entries), rows, out.ctypes.data_as(_u32p), wanted, ctypes.byref(error)) != 0:
+        if self.lib.kipp_step_sample(self.handle, items, len(entries), params, draws, out.ctypes.data_as(_u32p), wanted, ctypes.byref(error)) != 0:
             _raise(self.lib, error)
         return [int(t) for t in out[:wanted]]
 

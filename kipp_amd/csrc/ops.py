@@ -838,6 +838,28 @@ def argmax(logits: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     return out
 
 
+def adjust_logits(logits: torch.Tensor, begin: torch.Tensor, biases: torch.Tensor, token: torch.Tensor, value: torch.Tensor,
+                  repetition: torch.Tensor, presence: torch.Tensor, frequency: torch.Tensor) -> torch.Tensor:
+    """Logit bias and the penalties over recent tokens, applied to rows of float32 logits in place, in the host
+    sampler's order and with its float operations: row r's entries are begin[r] .. begin[r + 1], the first biases[r]
+    of them biases (value: the bias), the others distinct recent tokens (value: how often each occurs); tokens lie
+    inside the vocabulary."""
+    _dev(logits, begin, biases, token, value, repetition, presence, frequency)
+    _i32(begin, "begin")
+    _i32(biases, "biases")
+    _i32(token, "token")
+    rows = logits.shape[0]
+    _need(logits.dtype == torch.float32 and logits.dim() == 2 and logits.is_contiguous(), "adjust_logits: float32 [rows, vocab]")
+    _need(begin.numel() == rows + 1 and all(t.numel() == rows for t in (biases, repetition, presence, frequency)),
+          "adjust_logits: one value per row, rows + 1 begins")
+    _need(token.numel() == value.numel() and all(t.dtype == torch.float32 for t in (value, repetition, presence, frequency)),
+          "adjust_logits: one float32 value per entry, float32 penalties")
+    fn = _fn("sampling", "kipp_adjust_logits", [_c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr])
+    _check(fn(_ptr(logits), rows, logits.shape[1], _ptr(begin), _ptr(biases), _ptr(token), _ptr(value), _ptr(repetition),
+              _ptr(presence), _ptr(frequency), _stream()), "adjust_logits")
+    return logits
+
+
 def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
            min_p: torch.Tensor, uniform: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     """One token for each row of float32 logits: greedy where temperature <= 0,

@@ -168,6 +168,48 @@ extern "C" int kipp_argmax_static(const float* logits, int32_t* out, int rows, i
 }
 
 // ---------------------------------------------------------------------------------------
+// Logit bias and the penalties over a request's recent tokens, applied to rows of logits where
+// they lie, before a token is chosen from them (/root/reference/src/kipp.c:3386-3431): first every
+// bias entry in its order, l[token] += bias; then, for every distinct recent token with its count,
+// l = l > 0 ? l / repetition : l * repetition (unless repetition is 0 or 1), l -= presence,
+// l -= frequency * count.  A row's entries are few (its biases, at most 64 recent tokens) and
+// their order counts, so one lane walks them; every operation is one IEEE float operation as on
+// the host (the kernel is compiled without contraction into fused multiply-adds).
+// `begin` [rows + 1]: a row's entries are begin[r] .. begin[r + 1]; the first `biases[r]` of them
+// are biases (`value`: the bias), the rest penalties (`value`: the token's count).  The host has
+// dropped tokens outside the vocabulary and recent tokens that came before.
+__global__ void adjust_logits_kernel(float* __restrict__ logits, int rows, int vocab, const int32_t* __restrict__ begin,
+                                     const int32_t* __restrict__ biases, const int32_t* __restrict__ token,
+                                     const float* __restrict__ value, const float* __restrict__ repetition,
+                                     const float* __restrict__ presence, const float* __restrict__ frequency) {
+#pragma clang fp contract(off)   // the product freq * count is rounded before it is taken off, as on the host
+    const int r = blockIdx.x * blockDim.x + threadIdx.x;
+    if (r >= rows) return;
+    float* row = logits + (size_t)r * vocab;
+    const int first = begin[r], last = begin[r + 1], first_penalty = first + biases[r];
+    for (int e = first; e < first_penalty && e < last; ++e) row[token[e]] = row[token[e]] + value[e];
+    const float rep = repetition[r], pres = presence[r], freq = frequency[r];
+    for (int e = first_penalty; e < last; ++e) {
+        float v = row[token[e]];
+        if (rep != 0.0f && rep != 1.0f) v = v > 0.0f ? v / rep : v * rep;
+        v = v - pres;
+        const float off = freq * value[e];
+        v = v - off;
+        row[token[e]] = v;
+    }
+}
+
+extern "C" int kipp_adjust_logits(float* logits, int rows, int vocab, const int32_t* begin, const int32_t* biases,
+                                  const int32_t* token, const float* value, const float* repetition, const float* presence,
+                                  const float* frequency, hipStream_t stream) {
+    if (rows <= 0) return 0;
+    if (vocab <= 0) return -1;
+    hipLaunchKernelGGL(adjust_logits_kernel, dim3((rows + 63) / 64), dim3(64), 0, stream, logits, rows, vocab, begin, biases, token,
+                       value, repetition, presence, frequency);
+    return KIPP_LAUNCH_CHECK();
+}
+
+// ---------------------------------------------------------------------------------------
 // Temperature sampling with top-k, min-p and top-p, one workgroup per row, with the
 // meaning of the host sampler (/root/reference/src/kipp.c:3433-3559): scale by 1/T,
 // keep candidates within 20 of the maximum, order them by descending logit (ties: lower

@@ -181,17 +181,19 @@ class Engine:
         sampling parameters, generator and recent tokens.  Rows are chosen on the
         device in one launch (greedy and temperature rows alike; the uniform draw
         of a temperature row comes from its request's generator on the host).
-        Only rows whose logits are changed first (bias, penalties) go through the
-        host sampler.  With `wait` false the choice is not waited for: the result
+        Rows whose logits are changed first (bias, penalties over the request's
+        recent tokens) are changed where they lie, by a kernel that walks each
+        row's few entries in the host sampler's order (`logits` is overwritten
+        there).  With `wait` false the choice is not waited for: the result
         is a `Picks` whose `device` tensor can feed the next step at once and whose
-        `result()` gives the tokens when the host needs them."""
-        from ..sampling import sample
+        `result()` gives the tokens when the host needs them (the recent tokens
+        of a row with penalties must then be known: the scheduler waits for them)."""
+        from ..sampling import logit_change_entries
         rows = logits.shape[0]
         if rows != len(requests):
             raise ValueError("one request for each row of logits")
-        on_host = [i for i, r in enumerate(requests) if r.params.changes_logits]
-        if on_host and not wait:
-            raise ValueError("rows whose logits are changed on the host cannot be chosen without waiting")
+        if any(r.params.changes_logits for r in requests):
+            self._adjust_logits(logits, requests, logit_change_entries)
         picked = self.rt.empty((rows,), torch.int32)
         if all(r.params.greedy for r in requests):
             self.rt.ops.argmax(logits, picked)
@@ -203,7 +205,7 @@ class Engine:
             f64 = pack[rows * 16:].view(torch.float64)
             for i, req in enumerate(requests):
                 p = req.params
-                sampled = not p.greedy and i not in on_host
+                sampled = not p.greedy
                 if sampled:
                     p.validate()
                 f32[i] = float(p.temperature) if sampled else 0.0
@@ -217,11 +219,36 @@ class Engine:
                                d32[2 * rows:], dev[rows * 16:].view(torch.float64), picked)
         if not wait:
             return Picks(picked)
-        out = picked.cpu().tolist()
-        for i in on_host:
-            req = requests[i]
-            out[i] = sample(logits[i].cpu().numpy(), req.params, req.rng, list(req.recent))
-        return out
+        return picked.cpu().tolist()
+
+    def _adjust_logits(self, logits: torch.Tensor, requests: Sequence[object], entries_of) -> None:
+        """Bias and penalties of every row that has them, in one launch: the rows' entries and parameters go up in one
+        pinned buffer of 4-byte words [begin (rows + 1) | biases | tokens | values | repetition | presence | frequency]."""
+        rows, vocab = logits.shape
+        per_row = [entries_of(r.params, list(r.recent), vocab) if r.params.changes_logits else ([], [], 0) for r in requests]
+        total = sum(len(tokens) for tokens, _, _ in per_row)
+        words = 2 * rows + 1 + 2 * total + 3 * rows
+        pack = torch.empty(words, dtype=torch.int32).pin_memory()
+        as_float = pack.view(torch.float32)
+        begin, biases, token = pack[:rows + 1], pack[rows + 1:2 * rows + 1], pack[2 * rows + 1:2 * rows + 1 + total]
+        at_value = 2 * rows + 1 + total
+        value = as_float[at_value:at_value + total]
+        penalties = as_float[at_value + total:].view(3, rows)
+        at = 0
+        for i, (req, (tokens, values, n_bias)) in enumerate(zip(requests, per_row)):
+            begin[i], biases[i] = at, n_bias
+            if tokens:
+                token[at:at + len(tokens)] = torch.tensor(tokens, dtype=torch.int32)
+                value[at:at + len(tokens)] = torch.tensor(values, dtype=torch.float32)
+            at += len(tokens)
+            p = req.params
+            penalties[0, i], penalties[1, i], penalties[2, i] = float(p.repetition_penalty), float(p.presence_penalty), float(p.frequency_penalty)
+        begin[rows] = at
+        dev = pack.to(self.rt.device, non_blocking=True)
+        dev_float = dev.view(torch.float32)
+        self.rt.ops.adjust_logits(logits, dev[:rows + 1], dev[rows + 1:2 * rows + 1], dev[2 * rows + 1:at_value],
+                                  dev_float[at_value:at_value + total], dev_float[at_value + total:at_value + total + rows],
+                                  dev_float[at_value + total + rows:at_value + total + 2 * rows], dev_float[at_value + total + 2 * rows:])
 
 
 class Picks:

@@ -93,9 +93,10 @@ struct kipp_runtime {
     /* out[r] = the index of the largest of logits[r, :vocab], the lowest among equals (/root/reference/src/kipp.c:3459-3464) */
     int (*argmax)(kipp_runtime *rt, const float *logits, int32_t *out, uint32_t rows, uint32_t vocab, kipp_error *error);
     /* Optional (NULL: the caller samples on the host).  *out = memory of the path's own with one token a row, each chosen as
-     * its kipp_row_choice (host memory) says; it takes nothing from the step's workspace, so it may follow a recorded step. */
-    int (*sample)(kipp_runtime *rt, const float *logits, const kipp_row_choice *choices, int32_t **out, uint32_t rows, uint32_t vocab,
-                  kipp_error *error);
+     * kipp_sample_ex would choose it with `params[r]` (host memory; bias and penalties change the row of logits where it
+     * lies) and the draw `uniform[r]`; it takes nothing from the step's workspace, so it may follow a recorded step. */
+    int (*sample)(kipp_runtime *rt, float *logits, const kipp_sample_params *params, const double *uniform, int32_t **out, uint32_t rows,
+                  uint32_t vocab, kipp_error *error);
 
     /* Optional (NULL: none).  Recording: between graph_begin and graph_end the operations above are recorded instead of run
      * (no memory may be made meanwhile: the step's workspace says so, and the recording is dropped); graph_end with `keep`

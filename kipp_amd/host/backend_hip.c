@@ -60,6 +60,8 @@ typedef int (*fn_tile_weight)(const void *, void *, int, int, int, hipStream_t);
 typedef int (*fn_argmax)(const float *, int32_t *, int, int, float *, hipStream_t);
 typedef int (*fn_sample)(const float *, int, int, const float *, const int32_t *, const float *, const float *, const double *, int32_t *,
                          hipStream_t);
+typedef int (*fn_adjust_logits)(float *, int, int, const int32_t *, const int32_t *, const int32_t *, const float *, const float *,
+                                const float *, const float *, hipStream_t);
 typedef int (*fn_attention_decode_fused)(const float *, int, int, const float *, const float *, float, const float *, const float *, int, void *,
                                          void *, void *, float *, float *, const int32_t *, const int32_t *, const int32_t *, const int32_t *, int,
                                          int, int, int, int, int, float, int, int, int, int32_t *, int, hipStream_t);
@@ -109,9 +111,10 @@ typedef struct {
     fn_argmax argmax;
     fn_int_int argmax_scratch_floats;
     fn_sample sample;
-    unsigned char *sample_host; /* a step's kipp_row_choices, packed by field */
-    void *sample_device;        /* the same on the GPU, and behind them the tokens chosen */
-    uint32_t sample_rows;       /* rows both have room for */
+    fn_adjust_logits adjust_logits;
+    unsigned char *sample_host; /* what the sampler of a step is told, packed by field */
+    unsigned char *sample_device; /* the same on the GPU, behind the tokens chosen */
+    size_t sample_bytes;        /* room of both */
     bool fuse;             /* few rows: residual add and norm ride on the products around them, decode attention starts from the QKV product */
     bool steps_major;      /* rows that one few-rows product writes for the next: in the order that product reads fastest */
     bool merge_in_kernel;  /* decode attention: the splits of a head are merged by the last of their workgroups to finish */
@@ -227,6 +230,7 @@ static int open_common(hip_state *st, kipp_error *error) {
     KIPP_SYM(libs[7], argmax, "kipp_argmax");
     KIPP_SYM(libs[7], argmax_scratch_floats, "kipp_argmax_scratch_floats");
     KIPP_SYM(libs[7], sample, "kipp_sample");
+    KIPP_SYM(libs[7], adjust_logits, "kipp_adjust_logits");
     return 0;
 }
 
@@ -661,45 +665,94 @@ static int hip_gated(kipp_runtime *rt, const kipp_rows *x, const kipp_weight *w,
     return 0;
 }
 
-/* The device sampler over the rows of a step.  Its parameters go up in one copy, packed by field
- * ([temperature | top_p | min_p | top_k] of 4 bytes a row, then the draws of 8), into memory of its own that is made once for
- * the most rows a step can want and stays where it is: the step's workspace is not touched (a recorded step's logits lie
- * there), and a call that follows a recording allocates nothing. */
-static int hip_sample(kipp_runtime *rt, const float *logits, const kipp_row_choice *choices, int32_t **out, uint32_t rows, uint32_t vocab,
-                      kipp_error *error) {
+/* The device sampler over the rows of a step.  What it is told goes up in one copy, packed by field: the sampler's
+ * parameters ([temperature | top_p | min_p | top_k] of 4 bytes a row, then the draws of 8), and, where a row has a bias or
+ * penalties, the entries that the kernel before it walks ([begin (rows + 1) | biases | repetition | presence | frequency |
+ * tokens | values]: a row's biases in their order, then its distinct recent tokens with their counts, as kipp_sample_ex
+ * goes through them).  All of it lies in memory of its own that stays where it is until it must grow: the step's workspace is
+ * not touched (a recorded step's logits lie there), and a call that follows a recording allocates nothing. */
+static int hip_sample(kipp_runtime *rt, float *logits, const kipp_sample_params *params, const double *uniform, int32_t **out, uint32_t rows,
+                      uint32_t vocab, kipp_error *error) {
     hip_state *st = rt->state;
     if (rows == 0) return 0;
     if (vocab >= (1u << 24)) return kipp_fail(error, KIPP_ERROR_UNSUPPORTED, "the device sampler takes vocabularies below 2^24");
-    if (rows > st->sample_rows) {
-        uint32_t room = rows > 256 ? rows : 256;
-        unsigned char *host = realloc(st->sample_host, (size_t)room * 24);
+    size_t entries = 0;
+    for (uint32_t r = 0; r < rows; ++r) {
+        const kipp_sample_params *p = &params[r];
+        const bool penalties = p->frequency_penalty != 0.0f || p->presence_penalty != 0.0f || (p->repetition_penalty != 0.0f && p->repetition_penalty != 1.0f);
+        entries += p->logit_bias_count + (penalties ? p->recent_count : 0); /* at most: tokens outside the vocabulary and repeated ones drop out */
+    }
+    const size_t out_bytes = ((size_t)rows * 4 + 15) / 16 * 16, pack_bytes = (size_t)rows * 24;
+    const size_t adjust_words = entries != 0 ? 5 * (size_t)rows + 1 + 2 * entries : 0;
+    const size_t bytes = out_bytes + pack_bytes + adjust_words * 4;
+    if (bytes > st->sample_bytes) {
+        size_t room = bytes < 16384 ? 16384 : 2 * bytes;
+        unsigned char *host = realloc(st->sample_host, room);
         if (host == NULL) return kipp_fail(error, KIPP_ERROR_MEMORY, "out of memory");
         st->sample_host = host;
-        st->sample_rows = 0;
+        st->sample_bytes = 0;
         if (st->sample_device != NULL) {
             hipStreamSynchronize(st->stream);
             hipFree(st->sample_device);
             st->sample_device = NULL;
         }
-        hipError_t code = hipMalloc(&st->sample_device, (size_t)room * 28);
+        hipError_t code = hipMalloc((void **)&st->sample_device, room);
         if (code != hipSuccess) return hip_bad(error, code, "hipMalloc");
-        st->sample_rows = room;
+        st->sample_bytes = room;
     }
-    float *f32 = (float *)st->sample_host;
-    int32_t *i32 = (int32_t *)(st->sample_host + (size_t)rows * 12);
-    double *f64 = (double *)(st->sample_host + (size_t)rows * 16);
+    /* host and device hold the same layout; nothing of the first out_bytes goes up */
+    unsigned char *h = st->sample_host + out_bytes, *d = st->sample_device + out_bytes;
+    float *f32 = (float *)h;
+    int32_t *i32 = (int32_t *)(h + (size_t)rows * 12);
+    double *f64 = (double *)(h + (size_t)rows * 16);
+    int32_t *begin = (int32_t *)(h + pack_bytes), *biases = begin + rows + 1;
+    float *penalty = (float *)(biases + rows); /* [repetition | presence | frequency] */
+    int32_t *token = (int32_t *)(penalty + 3 * (size_t)rows);
+    float *value = (float *)(token + entries);
+    size_t at = 0;
     for (uint32_t r = 0; r < rows; ++r) {
-        const bool sampled = choices[r].temperature > 0.0f;
-        f32[r] = sampled ? choices[r].temperature : 0.0f;
-        f32[rows + r] = sampled ? choices[r].top_p : 1.0f;
-        f32[2 * rows + r] = sampled ? choices[r].min_p : 0.0f;
-        i32[r] = sampled ? (int32_t)(choices[r].top_k < (uint32_t)INT32_MAX ? choices[r].top_k : 0) : 0;
-        f64[r] = sampled ? choices[r].uniform : 0.0;
+        const kipp_sample_params *p = &params[r];
+        const bool sampled = p->temperature > 0.0f;
+        f32[r] = sampled ? p->temperature : 0.0f;
+        f32[rows + r] = sampled ? p->top_p : 1.0f;
+        f32[2 * rows + r] = sampled ? p->min_p : 0.0f;
+        i32[r] = sampled && p->top_k < (uint32_t)INT32_MAX ? (int32_t)p->top_k : 0;
+        f64[r] = sampled ? uniform[r] : 0.0;
+        if (entries == 0) continue;
+        begin[r] = (int32_t)at;
+        for (size_t b = 0; b < p->logit_bias_count; ++b) {
+            if (p->logit_bias_tokens[b] >= vocab) continue;
+            token[at] = (int32_t)p->logit_bias_tokens[b];
+            value[at++] = p->logit_bias_values[b];
+        }
+        biases[r] = (int32_t)at - begin[r];
+        penalty[r] = p->repetition_penalty;
+        penalty[rows + r] = p->presence_penalty;
+        penalty[2 * (size_t)rows + r] = p->frequency_penalty;
+        const bool penalties = p->frequency_penalty != 0.0f || p->presence_penalty != 0.0f || (p->repetition_penalty != 0.0f && p->repetition_penalty != 1.0f);
+        for (size_t i = 0; penalties && i < p->recent_count; ++i) {
+            const uint32_t t = p->recent_tokens[i];
+            bool seen = t >= vocab;
+            for (size_t j = 0; j < i && !seen; ++j) seen = p->recent_tokens[j] == t;
+            if (seen) continue; /* each distinct token once */
+            size_t count = 0;
+            for (size_t j = 0; j < p->recent_count; ++j) count += p->recent_tokens[j] == t;
+            token[at] = (int32_t)t;
+            value[at++] = (float)count;
+        }
     }
-    unsigned char *d = st->sample_device;
-    hipError_t code = hipMemcpyAsync(d, st->sample_host, (size_t)rows * 24, hipMemcpyHostToDevice, st->stream);
+    if (entries != 0) begin[rows] = (int32_t)at;
+    hipError_t code = hipMemcpyAsync(d, h, pack_bytes + adjust_words * 4, hipMemcpyHostToDevice, st->stream);
     if (code != hipSuccess) return hip_bad(error, code, "copy to the GPU");
-    *out = (int32_t *)(d + (size_t)st->sample_rows * 24);
+    if (at != 0) {
+        const int32_t *d_begin = (const int32_t *)(d + pack_bytes), *d_biases = d_begin + rows + 1;
+        const float *d_penalty = (const float *)(d_biases + rows);
+        const int32_t *d_token = (const int32_t *)(d_penalty + 3 * (size_t)rows);
+        int rc = st->adjust_logits(logits, (int)rows, (int)vocab, d_begin, d_biases, d_token, (const float *)(d_token + entries), d_penalty,
+                                   d_penalty + rows, d_penalty + 2 * (size_t)rows, st->stream);
+        if (rc != 0) return refused(error, "adjust_logits", rc);
+    }
+    *out = (int32_t *)st->sample_device;
     int rc = st->sample(logits, (int)rows, (int)vocab, (const float *)d, (const int32_t *)(d + (size_t)rows * 12), (const float *)d + rows,
                         (const float *)d + 2 * rows, (const double *)(d + (size_t)rows * 16), *out, st->stream);
     return rc == 0 ? 0 : refused(error, "sample", rc);

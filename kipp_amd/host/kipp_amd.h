@@ -182,25 +182,6 @@ int kipp_step(kipp_model *model, const kipp_step_item *items, size_t item_count,
 int kipp_step_argmax(kipp_model *model, const kipp_step_item *items, size_t item_count, uint32_t *tokens, size_t token_capacity,
                      kipp_error *error);
 
-/* How one wanted row of a step is chosen where the path computes (kipp_step_sample): the largest logit where
- * temperature <= 0, else temperature sampling with top-k (0: off), min-p (0: off) and top-p in the order of
- * kipp_sample_ex, with `uniform` in [0, 1) as the one draw that kipp_sample_ex would take from its generator. */
-typedef struct {
-    float temperature;
-    float top_p;
-    uint32_t top_k;
-    float min_p;
-    double uniform;
-} kipp_row_choice;
-
-/* kipp_step with one token for every wanted place, chosen beside the logits: `choices` has one entry a wanted place, in the
- * order of the items and their places.  Only a number a row comes back.  KIPP_ERROR_UNSUPPORTED on a path that has no
- * sampler of its own (the scalar one: take kipp_step and kipp_sample_ex). */
-int kipp_step_sample(kipp_model *model, const kipp_step_item *items, size_t item_count, const kipp_row_choice *choices, uint32_t *tokens,
-                     size_t token_capacity, kipp_error *error);
-/* The next draw of a generator, as kipp_sample_ex takes it (/root/reference/src/kipp.c:3322-3333): in [0, 1); the state must not be 0. */
-double kipp_rng_uniform(uint64_t *rng_state);
-
 int kipp_sample(const float *logits, size_t logits_count, float temperature, float top_p, uint64_t *rng_state, uint32_t *out_token,
                 kipp_error *error);
 
@@ -221,6 +202,17 @@ typedef struct {
 
 int kipp_sample_ex(const float *logits, size_t logits_count, const kipp_sample_params *params, uint64_t *rng_state,
                    uint32_t *out_token, kipp_error *error);
+
+/* kipp_step with one token for every wanted place, chosen where the path computes, with the meaning of kipp_sample_ex:
+ * `params` has one entry a wanted place, in the order of the items and their places (bias and recent tokens included:
+ * they change the row where it lies, in kipp_sample_ex's order and with its float operations), `uniform` for each the
+ * one draw in [0, 1) that kipp_sample_ex would take from its generator (not looked at where temperature <= 0: the
+ * largest logit).  Only a number a row comes back.  KIPP_ERROR_UNSUPPORTED on a path that has no sampler of its own
+ * (the scalar one: take kipp_step and kipp_sample_ex). */
+int kipp_step_sample(kipp_model *model, const kipp_step_item *items, size_t item_count, const kipp_sample_params *params,
+                     const double *uniform, uint32_t *tokens, size_t token_capacity, kipp_error *error);
+/* The next draw of a generator, as kipp_sample_ex takes it (/root/reference/src/kipp.c:3322-3333): in [0, 1); the state must not be 0. */
+double kipp_rng_uniform(uint64_t *rng_state);
 
 /*
  * The scheduler above the step function: it admits requests, cuts prompts into

@@ -63,7 +63,8 @@ struct kipp_scheduler {
     uint32_t *wants;
     float *logits;
     uint32_t *chosen;
-    kipp_row_choice *choices;
+    kipp_sample_params *choices; /* with the device sampler: every wanted row's parameters, */
+    double *draws;               /* and its draw */
     size_t logits_rows;
     bool device_sampler; /* the path has a sampler of its own and KIPP_AMD_SAMPLER does not say "host" */
 };
@@ -126,10 +127,11 @@ int kipp_scheduler_create(kipp_model *model, const kipp_scheduler_config *config
     s->logits_rows = s->max_running;
     s->logits = malloc(s->logits_rows * (size_t)model->spec.vocab * sizeof(float));
     s->chosen = malloc(s->logits_rows * sizeof(uint32_t));
-    s->choices = malloc(s->logits_rows * sizeof(kipp_row_choice));
+    s->choices = malloc(s->logits_rows * sizeof(kipp_sample_params));
+    s->draws = malloc(s->logits_rows * sizeof(double));
     const char *sampler = getenv("KIPP_AMD_SAMPLER");
     s->device_sampler = model->rt->sample != NULL && !(sampler != NULL && strcmp(sampler, "host") == 0);
-    if (s->items == NULL || s->item_requests == NULL || s->wants == NULL || s->logits == NULL || s->chosen == NULL || s->choices == NULL) {
+    if (s->items == NULL || s->item_requests == NULL || s->wants == NULL || s->logits == NULL || s->chosen == NULL || s->choices == NULL || s->draws == NULL) {
         kipp_scheduler_destroy(s);
         return kipp_fail(error, KIPP_ERROR_MEMORY, "out of memory for the scheduler's step");
     }
@@ -153,6 +155,7 @@ void kipp_scheduler_destroy(kipp_scheduler *s) {
     free(s->logits);
     free(s->chosen);
     free(s->choices);
+    free(s->draws);
     free(s);
 }
 
@@ -413,27 +416,27 @@ int kipp_scheduler_step(kipp_scheduler *s, kipp_produced *out, size_t capacity, 
         greedy = s->items[i].want_count == 0 || (p->temperature <= 0.0f && p->frequency_penalty == 0.0f && p->presence_penalty == 0.0f &&
                                                  (p->repetition_penalty == 1.0f || p->repetition_penalty == 0.0f) && p->logit_bias_count == 0);
     }
-    /* else, where no row's logits are changed first (bias, penalties) and the path has a sampler of its own, every row is
-     * chosen there as well, a sampled row with the draw that kipp_sample_ex would take from the request's generator now
+    /* else, where the path has a sampler of its own, every row is chosen there as well: a row's bias and penalties change it
+     * where it lies, and a sampled row gets the draw that kipp_sample_ex would take from the request's generator now
      * (parameters it would refuse go to it, so that it does) */
     bool beside = !greedy && !s->keep_last_logits && s->device_sampler;
     uint32_t rows = 0;
     for (uint32_t i = 0; i < n && beside; ++i) {
         const kipp_sample_params *p = &s->item_requests[i]->params;
         if (s->items[i].want_count == 0) continue;
-        beside = p->frequency_penalty == 0.0f && p->presence_penalty == 0.0f && (p->repetition_penalty == 1.0f || p->repetition_penalty == 0.0f) &&
-                 p->logit_bias_count == 0 &&
-                 (p->temperature <= 0.0f || (p->top_p > 0.0f && p->top_p <= 1.0f && p->min_p >= 0.0f && p->min_p <= 1.0f && s->item_requests[i]->rng != 0));
+        beside = p->temperature <= 0.0f || (p->top_p > 0.0f && p->top_p <= 1.0f && p->min_p >= 0.0f && p->min_p <= 1.0f && s->item_requests[i]->rng != 0);
     }
     for (uint32_t i = 0; i < n && beside; ++i) {
         request *r = s->item_requests[i];
         if (s->items[i].want_count == 0) continue;
-        s->choices[rows++] = (kipp_row_choice){r->params.temperature, r->params.top_p, r->params.top_k, r->params.min_p,
-                                               r->params.temperature > 0.0f ? kipp_rng_uniform(&r->rng) : 0.0};
+        s->choices[rows] = r->params;
+        s->choices[rows].recent_tokens = r->recent;
+        s->choices[rows].recent_count = r->recent_count;
+        s->draws[rows++] = r->params.temperature > 0.0f ? kipp_rng_uniform(&r->rng) : 0.0;
     }
     greedy = greedy || beside; /* from here on: the tokens are in s->chosen */
     kipp_error step_error;
-    int step_rc = beside   ? kipp_step_sample(s->model, s->items, n, s->choices, s->chosen, s->logits_rows, &step_error)
+    int step_rc = beside   ? kipp_step_sample(s->model, s->items, n, s->choices, s->draws, s->chosen, s->logits_rows, &step_error)
                   : greedy ? kipp_step_argmax(s->model, s->items, n, s->chosen, s->logits_rows, &step_error)
                            : kipp_step(s->model, s->items, n, s->logits, s->logits_rows * (size_t)s->model->spec.vocab, &step_error);
     if (step_rc != 0) {

@@ -315,35 +315,35 @@ uint64_t kipp_test_graph_replays(const kipp_model *model) { return model != NULL
 uint64_t kipp_test_cut_attention_steps(const kipp_model *model) { return model != NULL ? model->rt->cut_attention_steps : 0; }
 
 static int step_common(kipp_model *model, const kipp_step_item *items, size_t item_count, float *logits, size_t logits_capacity, uint32_t *best,
-                       const kipp_row_choice *choices, kipp_error *error);
+                       const kipp_sample_params *choices, const double *uniform, kipp_error *error);
 
 int kipp_step(kipp_model *model, const kipp_step_item *items, size_t item_count, float *logits, size_t logits_capacity,
               kipp_error *error) {
-    return step_common(model, items, item_count, logits, logits_capacity, NULL, NULL, error);
+    return step_common(model, items, item_count, logits, logits_capacity, NULL, NULL, NULL, error);
 }
 
-int kipp_step_sample(kipp_model *model, const kipp_step_item *items, size_t item_count, const kipp_row_choice *choices, uint32_t *tokens,
-                     size_t token_capacity, kipp_error *error) {
+int kipp_step_sample(kipp_model *model, const kipp_step_item *items, size_t item_count, const kipp_sample_params *params,
+                     const double *uniform, uint32_t *tokens, size_t token_capacity, kipp_error *error) {
     uint32_t none;
     kipp_error_clear(error);
     if (model != NULL && model->rt->sample == NULL) return kipp_fail(error, KIPP_ERROR_UNSUPPORTED, "this path has no sampler of its own");
-    if (choices == NULL) return kipp_fail(error, KIPP_ERROR_ARGUMENT, "no choices");
+    if (params == NULL || uniform == NULL) return kipp_fail(error, KIPP_ERROR_ARGUMENT, "parameters and draws must be given");
     if (tokens == NULL && token_capacity != 0) return kipp_fail(error, KIPP_ERROR_ARGUMENT, "no room for the tokens");
-    return step_common(model, items, item_count, NULL, tokens != NULL ? token_capacity : 0, tokens != NULL ? tokens : &none, choices, error);
+    return step_common(model, items, item_count, NULL, tokens != NULL ? token_capacity : 0, tokens != NULL ? tokens : &none, params, uniform, error);
 }
 
 int kipp_step_argmax(kipp_model *model, const kipp_step_item *items, size_t item_count, uint32_t *tokens, size_t token_capacity,
                      kipp_error *error) {
     uint32_t none; /* a step that wants nothing may come without room */
     if (tokens == NULL && token_capacity != 0) return kipp_fail(error, KIPP_ERROR_ARGUMENT, "no room for the tokens");
-    return step_common(model, items, item_count, NULL, tokens != NULL ? token_capacity : 0, tokens != NULL ? tokens : &none, NULL, error);
+    return step_common(model, items, item_count, NULL, tokens != NULL ? token_capacity : 0, tokens != NULL ? tokens : &none, NULL, NULL, error);
 }
 
 /* `best` NULL: the wanted rows of logits go to `logits` (room for `capacity` floats); else one token for every wanted row goes
  * to `best` (room for `capacity` of them), found where the path computes: the index of the largest logit, or with `choices`
- * what each row's choice says. */
+ * what kipp_sample_ex would choose with each row's parameters and draw. */
 static int step_common(kipp_model *model, const kipp_step_item *items, size_t item_count, float *logits, size_t logits_capacity, uint32_t *best,
-                       const kipp_row_choice *choices, kipp_error *error) {
+                       const kipp_sample_params *choices, const double *uniform, kipp_error *error) {
     kipp_error_clear(error);
     if (model == NULL || (items == NULL && item_count != 0)) return kipp_fail(error, KIPP_ERROR_ARGUMENT, "model and items must be given");
     if (item_count == 0) return 0;
@@ -411,7 +411,16 @@ static int step_common(kipp_model *model, const kipp_step_item *items, size_t it
     float *device_logits = NULL;
     int32_t *chosen = NULL;
     if (run_step(model, single && !model->config.eager_steps, best != NULL && choices == NULL, &device_logits, &chosen, error) != 0) goto unclaim;
-    if (choices != NULL && wanted != 0 && model->rt->sample(model->rt, device_logits, choices, &chosen, (uint32_t)wanted, vocab, error) != 0) goto unclaim;
+    if (choices != NULL && wanted != 0) {
+        for (size_t w = 0; w < wanted; ++w) { /* what kipp_sample_ex refuses */
+            const kipp_sample_params *p = &choices[w];
+            if (p->temperature > 0.0f && !(p->top_p > 0.0f && p->top_p <= 1.0f && p->min_p >= 0.0f && p->min_p <= 1.0f && uniform[w] >= 0.0 && uniform[w] < 1.0)) {
+                kipp_fail(error, KIPP_ERROR_ARGUMENT, "wanted place %zu: top_p in (0, 1], min_p in [0, 1] and a draw in [0, 1)", w);
+                goto unclaim;
+            }
+        }
+        if (model->rt->sample(model->rt, device_logits, choices, uniform, &chosen, (uint32_t)wanted, vocab, error) != 0) goto unclaim;
+    }
     /* reading back (even nothing) waits for the step's work: what it wrote into the pages is there when it returns */
     if (best != NULL && wanted != 0) {
         if (model->rt->download(model->rt, best, chosen, wanted * sizeof(int32_t), error) != 0) goto unclaim;

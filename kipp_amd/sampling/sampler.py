@@ -100,6 +100,27 @@ def apply_bias_and_penalties(logits: np.ndarray, params: SampleParams, recent: S
     return out
 
 
+def logit_change_entries(params: SampleParams, recent: Sequence[int], vocab: int):
+    """What `apply_bias_and_penalties` does to one row, as the entries the device kernel walks (`ops.adjust_logits`):
+    (tokens, values, how many of them are biases).  A bias entry's value is the bias; the others are the distinct recent
+    tokens in their order, each with its count.  Tokens outside the vocabulary are dropped, as there."""
+    tokens, values = [], []
+    for token, bias in params.logit_bias.items():
+        if 0 <= token < vocab:
+            tokens.append(int(token))
+            values.append(float(np.float32(bias)))
+    biases = len(tokens)
+    if params.has_penalty and recent:
+        seen = set()
+        for token in recent:
+            if token >= vocab or token < 0 or token in seen:
+                continue
+            seen.add(token)
+            tokens.append(int(token))
+            values.append(float(sum(1 for other in recent if other == token)))
+    return tokens, values, biases
+
+
 def argmax(values: np.ndarray) -> int:
     """Strict '>' in index order: the lowest index among equals (kipp.c:3459-3464)."""
     return int(np.argmax(values))

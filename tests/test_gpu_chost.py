@@ -182,27 +182,34 @@ def test_c_host_tokens_chosen_beside_the_logits(model_folders, tiny_configs, dty
             twins.append(sessions)
         portion = H.random_tokens(70, 11, vocab)
         entries = lambda ss: [(ss[0], [3], [0]), (ss[3], portion, [2, 10]), (ss[1], [7], [0]), (ss[2], [11], [0])]
-        settings = [(0.0, 1.0, 0, 0.0), (0.8, 0.9, 0, 0.0), (1.3, 1.0, 5, 0.0), (0.7, 0.95, 40, 0.05), (1.0, 1.0, 0, 0.0)]
+        recent = [5, 9, 5, 5, 77, vocab + 4, 9]
+        settings = [dict(), dict(temperature=0.8, top_p=0.9), dict(temperature=1.3, top_k=5, repetition_penalty=1.4, recent=recent),
+                    dict(temperature=0.7, top_p=0.95, top_k=40, min_p=0.05, logit_bias={3: 4.0, 100: -2.0, 3 + vocab: 1.0}),
+                    dict(presence_penalty=0.5, frequency_penalty=0.2, recent=recent, logit_bias={9: 6.0})]
         for round_ in range(6):                                  # every round other draws; the sessions grow by their tokens
             logits = model.step(entries(twins[0]))
             seeds = [1000 * round_ + 17 * r + 1 for r in range(5)]
-            choices = [(t, p, k, m, Rng(seed).uniform()) for (t, p, k, m), seed in zip(settings, seeds)]
+            choices = [dict(kw, uniform=Rng(seed).uniform()) for kw, seed in zip(settings, seeds)]
             chosen = model.step_sample(entries(twins[1]), choices)
-            expect = [sample(logits[r], t, p, k, m, rng=Rng(seed)) for r, ((t, p, k, m), seed) in enumerate(zip(settings, seeds))]
+            expect = [sample(logits[r], rng=Rng(seed), **kw) for r, (kw, seed) in enumerate(zip(settings, seeds))]
             assert chosen == expect, (round_, chosen, expect)    # (the twins' steps are the same launches: the same bits of logits)
             assert chosen[0] == int(np.argmax(logits[0]))
         with pytest.raises(ValueError):
             model.step_sample(entries(twins[1]), choices[:2])
+        before = [s.length for s in twins[1]]
+        with pytest.raises(KippError, match="top_p in"):
+            model.step_sample(entries(twins[1]), [dict(c, top_p=1.5) for c in choices])
+        assert [s.length for s in twins[1]] == before            # refused as a whole: nothing was appended
     with CModel(model_folders[("b", "float32")], path="cpu-fp32", page_tokens=8, kv_pool_pages=8) as scalar:
         with pytest.raises(KippError, match="no sampler of its own"):
-            scalar.step_sample([(scalar.session(), [1], [0])], [(0.0, 1.0, 0, 0.0, 0.0)])
+            scalar.step_sample([(scalar.session(), [1], [0])], [dict()])
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_c_scheduler_samples_on_the_device_as_on_the_host(model_folders, tiny_configs, dtype, monkeypatch):
     """Requests with temperature, top-k, top-p and min-p beside greedy ones through the C scheduler: chosen by the device
     sampler, with the draws of each request's generator, they are the tokens that KIPP_AMD_SAMPLER=host (every row's
-    logits read back and given to kipp_sample_ex) chooses; a request with a penalty takes the host's way in both."""
+    logits read back and given to kipp_sample_ex) chooses, also where requests have penalties and a bias."""
     from kipp_amd.chost import CModel, CScheduler
     cfg = tiny_configs["a"]
     vocab = cfg["vocab_size"]
@@ -210,20 +217,24 @@ def test_c_scheduler_samples_on_the_device_as_on_the_host(model_folders, tiny_co
     how = {0: dict(temperature=0.9, top_p=0.9, seed=11), 1: dict(temperature=1.2, top_k=8, seed=12), 2: dict(),
            3: dict(temperature=0.7, min_p=0.1, top_p=0.95, seed=14), 4: dict(temperature=1.0, seed=15)}
     outputs = {}
-    for sampler in ("device", "host", "penalty"):
-        monkeypatch.setenv("KIPP_AMD_SAMPLER", "host" if sampler == "host" else "device")
+    for sampler in ("device", "host", "penalty", "penalty on the host"):
+        monkeypatch.setenv("KIPP_AMD_SAMPLER", "host" if sampler.endswith("host") else "device")
         with CModel(model_folders[("a", dtype)], path=PATH[dtype], page_tokens=PAGE["a"], kv_pool_pages=64, max_sessions=5,
                     share_prefixes=False) as model:
             sched = CScheduler(model, max_step_tokens=24, prefill_chunk=8)
             for i, prompt in prompts.items():
-                extra = dict(repetition_penalty=1.3) if sampler == "penalty" and i == 4 else {}
+                extra = {}
+                if sampler.startswith("penalty"):
+                    extra = {4: dict(repetition_penalty=1.3), 2: dict(frequency_penalty=0.4, logit_bias={5: 1.5, 11: -3.0}),
+                             0: dict(presence_penalty=0.6)}.get(i, {})
                 sched.add(i, prompt, 12, **how[i], **extra)
             sched.run()
             outputs[sampler] = {i: sched.result(i)["output"] for i in prompts}
             assert all(len(o) == 12 for o in outputs[sampler].values())
             sched.destroy()
     assert outputs["device"] == outputs["host"]
-    assert outputs["penalty"][4] != outputs["device"][4] and all(outputs["penalty"][i] == outputs["device"][i] for i in range(4))
+    assert outputs["penalty"] == outputs["penalty on the host"]
+    assert outputs["penalty"][4] != outputs["device"][4] and all(outputs["penalty"][i] == outputs["device"][i] for i in (1, 3))
     ref = H.plain_logits(model_folders[("a", dtype)], prompts[2] + outputs["device"][2])
     margin = 1e-4 if dtype == "float32" else 0.05
     for j, token in enumerate(outputs["device"][2]):             # the greedy request among them

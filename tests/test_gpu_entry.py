@@ -105,6 +105,44 @@ def test_running_one_step_ahead_changes_nothing(model_folders, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_bias_and_penalties_are_applied_where_the_logits_lie(model_folders, dtype):
+    """Requests with penalties over their recent tokens and a bias, greedy and sampled, beside plain ones: the scheduler
+    changes their rows on the device and chooses there; every token is what the host sampler chooses from the step's
+    logits (read through `on_logits` before they are changed) with the request's parameters, recent tokens and draw."""
+    from kipp_amd.engine import Engine
+    from kipp_amd.engine.scheduler import Request, Scheduler
+    from kipp_amd.sampling import SampleParams, XorShift64Star, sample
+    folder = model_folders[("a", dtype)]
+    prompts = [H.random_tokens(190 + i, n, 256) for i, n in enumerate([6, 21, 3, 14])]
+    how = [SampleParams(repetition_penalty=1.5, frequency_penalty=0.3),
+           SampleParams(temperature=0.9, top_p=0.9, presence_penalty=0.8, logit_bias={5: 2.0, 40: -4.0}),
+           SampleParams(temperature=1.1, top_k=20),
+           SampleParams(logit_bias={17: 0.7}, repetition_penalty=0.7)]
+    engine = Engine.from_folder(folder, dtype=dtype, page_size=16, max_tokens=4 * 128, share_prefixes=False)
+    seen = []
+
+    def keep(requests, logits):
+        seen.append(([r.id for r in requests], logits.cpu().numpy().copy(), [list(r.recent) for r in requests]))
+
+    sched = Scheduler(engine, max_step_tokens=32, prefill_chunk=8, on_logits=keep)
+    for i, prompt in enumerate(prompts):
+        sched.add(Request(i, prompt, 14, params=how[i], seed=70 + i))
+    while not sched.idle:
+        sched.step()
+    outputs = {rid: r.output for rid, r in sched.finished.items()}
+    assert all(len(o) == 14 for o in outputs.values())
+    twins = {i: XorShift64Star(70 + i) for i in range(4)}
+    at = {i: 0 for i in range(4)}
+    for ids, logits, recents in seen:
+        for row, (rid, recent) in enumerate(zip(ids, recents)):
+            want = sample(logits[row], how[rid], twins[rid], recent)
+            assert outputs[rid][at[rid]] == want, (rid, at[rid])
+            at[rid] += 1
+    assert at == {i: 14 for i in range(4)}
+    assert len(set(outputs[0])) > 3                              # the penalties keep a greedy request from repeating itself
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_one_step_ahead_with_shared_beginnings_and_a_stop_token(model_folders, dtype):
     """Sharing on: two requests with a common beginning of four pages (the second adopts what the first published early)
     and a third of its own decode together one step ahead of what the scheduler knows; a stop token ends the first one

@@ -1224,6 +1224,46 @@ def test_device_sampler_agrees_with_the_host_sampler(vocab):
         assert got[i] == want, f"row {i}: T={temperature} top_k={top_k} top_p={top_p} min_p={min_p}: {got[i]} != {want}"
 
 
+@pytest.mark.parametrize("vocab", [509, 151936])
+def test_bias_and_penalties_on_the_device_are_the_host_sampler_s(vocab):
+    """Rows with a bias, with every penalty alone and together, with recent tokens that repeat and that lie outside the
+    vocabulary, beside rows with nothing: the changed logits are the host sampler's bit for bit (each step one IEEE
+    operation, in its order), and so is the token then chosen for the same draw."""
+    from kipp_amd.sampling import SampleParams, XorShift64Star, apply_bias_and_penalties, logit_change_entries, sample
+    ops = _ops()
+    rng = np.random.default_rng(vocab + 1)
+    recents = [[], [3, 7, 3, 3, 100, 7], list(rng.integers(0, vocab, 64)), [5, vocab + 3, 5, 9], [vocab - 1] * 64]
+    settings = [dict(), dict(logit_bias={4: 2.5, 100: -7.0, vocab + 9: 1.0}), dict(repetition_penalty=1.3), dict(presence_penalty=0.7),
+                dict(frequency_penalty=0.31), dict(repetition_penalty=0.8, presence_penalty=-0.2, frequency_penalty=0.05, logit_bias={3: 1.1, 7: -0.3}),
+                dict(repetition_penalty=0.0, frequency_penalty=1e-3)]
+    cases = [(SampleParams(temperature=t, top_p=0.9, **kw), recent) for kw in settings for recent in recents for t in (0.0, 0.9)]
+    rows = len(cases)
+    logits = (rng.normal(size=(rows, vocab)) * 3.0).astype(np.float32)
+    begin, biases, tokens, values = [0], [], [], []
+    for params, recent in cases:
+        t, v, n_bias = logit_change_entries(params, recent, vocab) if params.changes_logits else ([], [], 0)
+        tokens += t
+        values += v
+        biases.append(n_bias)
+        begin.append(len(tokens))
+    device = _t(logits)
+    ops.adjust_logits(device, _t(begin, torch.int32), _t(biases, torch.int32), _t(tokens or [0], torch.int32)[:len(tokens)],
+                      _t(values or [0.0])[:len(tokens)], _t([p.repetition_penalty for p, _ in cases]),
+                      _t([p.presence_penalty for p, _ in cases]), _t([p.frequency_penalty for p, _ in cases]))
+    got = device.cpu().numpy()
+    changed = 0
+    for i, (params, recent) in enumerate(cases):
+        want = apply_bias_and_penalties(logits[i], params, recent)
+        assert np.array_equal(got[i], want), f"row {i}: {params} recent {recent[:8]}: {np.flatnonzero(got[i] != want)[:5]}"
+        changed += int(not np.array_equal(want, logits[i]))
+    assert changed >= rows // 2
+    seeds = rng.integers(1, 2 ** 62, size=rows)
+    picked = ops.sample(device, _t([p.temperature for p, _ in cases]), _t([0] * rows, torch.int32), _t([0.9] * rows), _t([0.0] * rows),
+                        _t([XorShift64Star(int(s)).uniform() for s in seeds], torch.float64), torch.empty(rows, dtype=torch.int32, device=DEV)).cpu().tolist()
+    for i, (params, recent) in enumerate(cases):
+        assert picked[i] == sample(logits[i], params, XorShift64Star(int(seeds[i])), recent), i
+
+
 def test_device_sampler_follows_the_distribution():
     ops = _ops()
     from kipp_amd.sampling import XorShift64Star
