@@ -149,6 +149,8 @@ def library(variant: str = "gpu") -> ctypes.CDLL:
             "kipp_step": [vp, ctypes.POINTER(_StepItem), sz, _f32p, sz, err],
             "kipp_step_argmax": [vp, ctypes.POINTER(_StepItem), sz, _u32p, sz, err],
             "kipp_step_sample": [vp, ctypes.POINTER(_StepItem), sz, ctypes.POINTER(_SampleParams), ctypes.POINTER(ctypes.c_double), _u32p, sz, err],
+            "kipp_step_sample_logits": [vp, ctypes.POINTER(_StepItem), sz, ctypes.POINTER(_SampleParams), ctypes.POINTER(ctypes.c_double), _u32p, sz,
+                                        _f32p, sz, err],
             "kipp_sample_ex": [_f32p, sz, ctypes.POINTER(_SampleParams), ctypes.POINTER(ctypes.c_uint64), _u32p, err],
             "kipp_test_scramble_session_kv": [vp, err],
             "kipp_scheduler_create": [vp, ctypes.POINTER(_SchedulerConfig), ctypes.POINTER(vp), err],
@@ -330,10 +332,11 @@ class CModel:
             _raise(self.lib, error)
         return [int(t) for t in out[:wanted]]
 
-    def step_sample(self, entries: Sequence[Tuple[CSession, Sequence[int], Sequence[int]]], choices: Sequence[dict]) -> List[int]:
+    def step_sample(self, entries: Sequence[Tuple[CSession, Sequence[int], Sequence[int]]], choices: Sequence[dict], logits: bool = False):
         """The same batch, answered with one token for every wanted place, chosen where the path computes as kipp_sample_ex
         would: `choices` has, for each wanted place in order, the sampler's parameters by name (temperature, top_p, top_k,
-        min_p, frequency_penalty, presence_penalty, repetition_penalty, recent, logit_bias) and `uniform`, the draw."""
+        min_p, frequency_penalty, presence_penalty, repetition_penalty, recent, logit_bias) and `uniform`, the draw.
+        With `logits` the result is (tokens, the wanted rows of logits as the model left them)."""
         items = (_StepItem * len(entries))()
         keep = []
         wanted = 0
@@ -360,6 +363,12 @@ class CModel:
             draws[r] = c.get("uniform", 0.0)
         out = np.zeros(max(wanted, 1), dtype=np.uint32)
         error = _Error()
+        if logits:
+            rows = np.empty((wanted, self.vocab_size), dtype=np.float32)
+            if self.lib.kipp_step_sample_logits(self.handle, items, len(entries), params, draws, out.ctypes.data_as(_u32p), wanted,
+                                                rows.ctypes.data_as(_f32p), rows.size, ctypes.byref(error)) != 0:
+                _raise(self.lib, error)
+            return [int(t) for t in out[:wanted]], rows
         if self.lib.kipp_step_sample(self.handle, items, len(entries), params, draws, out.ctypes.data_as(_u32p), wanted, ctypes.byref(error)) != 0:
             _raise(self.lib, error)
         return [int(t) for t in out[:wanted]]

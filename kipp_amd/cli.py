@@ -240,28 +240,38 @@ def run_c_host(args, tokens) -> int:
     print(f"kipp: evaluating {len(tokens)} token{'s' if len(tokens) != 1 else ''} on {path} (C host)", file=sys.stderr)
     session = model.session(capacity)
     rng = Rng(args.seed)
+    beside = path != "cpu-fp32" and args.decode > 0          # the GPU paths choose the token beside the logits
+
+    def step_and_choose(chunk, place):
+        """One step of the session; the token chosen from the row at `place`, and that row."""
+        if beside:
+            how = dict(temperature=args.temperature, top_p=args.top_p, top_k=args.top_k, min_p=args.min_p,
+                       uniform=rng.uniform() if args.temperature > 0 else 0.0)
+            chosen, rows = model.step_sample([(session, chunk, [place])], [how], logits=True)
+            return chosen[0], rows[0]
+        row = model.step([(session, chunk, [place])])[0]
+        return (sample(row, args.temperature, args.top_p, args.top_k, args.min_p, rng=rng) if args.decode > 0 else None), row
+
     started = time.perf_counter()
-    row = None
+    row = token = None
     for at in range(0, len(tokens), args.prefill_chunk):
         chunk = tokens[at:at + args.prefill_chunk]
-        last = at + len(chunk) == len(tokens)
-        out = model.step([(session, chunk, [len(chunk) - 1] if last else [])])
-        row = out[0] if last else row
+        if at + len(chunk) == len(tokens):
+            token, row = step_and_choose(chunk, len(chunk) - 1)
+        else:
+            model.step([(session, chunk, [])])
     prefill_seconds = time.perf_counter() - started
     started = time.perf_counter()
     output = []
     if args.decode > 0:
         sys.stdout.write("generated\t")
-        while True:
-            token = sample(row, args.temperature, args.top_p, args.top_k, args.min_p, rng=rng)
-            if token in stops:
-                break
+        while token not in stops:
             sys.stdout.write(("" if not output else " ") + str(token))
             sys.stdout.flush()
             output.append(token)
             if len(output) >= args.decode:
                 break
-            row = model.step([(session, [token], [0])])[0]
+            token, row = step_and_choose([token], 0)
         sys.stdout.write("\n")
     decode_seconds = time.perf_counter() - started
     order = sorted(range(len(row)), key=lambda i: (-float(row[i]), i))[:min(args.top, len(row))] if len(row) < 4096 else \

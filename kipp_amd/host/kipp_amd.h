@@ -211,6 +211,10 @@ int kipp_sample_ex(const float *logits, size_t logits_count, const kipp_sample_p
  * (the scalar one: take kipp_step and kipp_sample_ex). */
 int kipp_step_sample(kipp_model *model, const kipp_step_item *items, size_t item_count, const kipp_sample_params *params,
                      const double *uniform, uint32_t *tokens, size_t token_capacity, kipp_error *error);
+/* The same, and the wanted rows of logits as the model left them (before a bias or a penalty changed them) as well. */
+int kipp_step_sample_logits(kipp_model *model, const kipp_step_item *items, size_t item_count, const kipp_sample_params *params,
+                            const double *uniform, uint32_t *tokens, size_t token_capacity, float *logits, size_t logits_capacity,
+                            kipp_error *error);
 /* The next draw of a generator, as kipp_sample_ex takes it (/root/reference/src/kipp.c:3322-3333): in [0, 1); the state must not be 0. */
 double kipp_rng_uniform(uint64_t *rng_state);
 

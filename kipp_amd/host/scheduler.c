@@ -419,7 +419,7 @@ int kipp_scheduler_step(kipp_scheduler *s, kipp_produced *out, size_t capacity, 
     /* else, where the path has a sampler of its own, every row is chosen there as well: a row's bias and penalties change it
      * where it lies, and a sampled row gets the draw that kipp_sample_ex would take from the request's generator now
      * (parameters it would refuse go to it, so that it does) */
-    bool beside = !greedy && !s->keep_last_logits && s->device_sampler;
+    bool beside = !greedy && s->device_sampler;
     uint32_t rows = 0;
     for (uint32_t i = 0; i < n && beside; ++i) {
         const kipp_sample_params *p = &s->item_requests[i]->params;
@@ -436,7 +436,8 @@ int kipp_scheduler_step(kipp_scheduler *s, kipp_produced *out, size_t capacity, 
     }
     greedy = greedy || beside; /* from here on: the tokens are in s->chosen */
     kipp_error step_error;
-    int step_rc = beside   ? kipp_step_sample(s->model, s->items, n, s->choices, s->draws, s->chosen, s->logits_rows, &step_error)
+    int step_rc = beside   ? kipp_step_sample_logits(s->model, s->items, n, s->choices, s->draws, s->chosen, s->logits_rows,
+                                                     s->keep_last_logits ? s->logits : NULL, s->logits_rows * (size_t)s->model->spec.vocab, &step_error)
                   : greedy ? kipp_step_argmax(s->model, s->items, n, s->chosen, s->logits_rows, &step_error)
                            : kipp_step(s->model, s->items, n, s->logits, s->logits_rows * (size_t)s->model->spec.vocab, &step_error);
     if (step_rc != 0) {
@@ -459,6 +460,7 @@ int kipp_scheduler_step(kipp_scheduler *s, kipp_produced *out, size_t capacity, 
         }
         if (s->items[i].want_count == 0) continue;
         if (greedy) {
+            if (r->last_logits != NULL) memcpy(r->last_logits, s->logits + (size_t)row * vocab, (size_t)vocab * sizeof(float));
             accept(s, r, s->chosen[row++], out, capacity, &produced);
             continue;
         }

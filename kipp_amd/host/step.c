@@ -315,35 +315,43 @@ uint64_t kipp_test_graph_replays(const kipp_model *model) { return model != NULL
 uint64_t kipp_test_cut_attention_steps(const kipp_model *model) { return model != NULL ? model->rt->cut_attention_steps : 0; }
 
 static int step_common(kipp_model *model, const kipp_step_item *items, size_t item_count, float *logits, size_t logits_capacity, uint32_t *best,
-                       const kipp_sample_params *choices, const double *uniform, kipp_error *error);
+                       size_t best_capacity, const kipp_sample_params *choices, const double *uniform, kipp_error *error);
 
 int kipp_step(kipp_model *model, const kipp_step_item *items, size_t item_count, float *logits, size_t logits_capacity,
               kipp_error *error) {
-    return step_common(model, items, item_count, logits, logits_capacity, NULL, NULL, NULL, error);
+    return step_common(model, items, item_count, logits, logits_capacity, NULL, 0, NULL, NULL, error);
 }
 
-int kipp_step_sample(kipp_model *model, const kipp_step_item *items, size_t item_count, const kipp_sample_params *params,
-                     const double *uniform, uint32_t *tokens, size_t token_capacity, kipp_error *error) {
+int kipp_step_sample_logits(kipp_model *model, const kipp_step_item *items, size_t item_count, const kipp_sample_params *params,
+                            const double *uniform, uint32_t *tokens, size_t token_capacity, float *logits, size_t logits_capacity,
+                            kipp_error *error) {
     uint32_t none;
     kipp_error_clear(error);
     if (model != NULL && model->rt->sample == NULL) return kipp_fail(error, KIPP_ERROR_UNSUPPORTED, "this path has no sampler of its own");
     if (params == NULL || uniform == NULL) return kipp_fail(error, KIPP_ERROR_ARGUMENT, "parameters and draws must be given");
     if (tokens == NULL && token_capacity != 0) return kipp_fail(error, KIPP_ERROR_ARGUMENT, "no room for the tokens");
-    return step_common(model, items, item_count, NULL, tokens != NULL ? token_capacity : 0, tokens != NULL ? tokens : &none, params, uniform, error);
+    return step_common(model, items, item_count, logits, logits != NULL ? logits_capacity : 0, tokens != NULL ? tokens : &none,
+                       tokens != NULL ? token_capacity : 0, params, uniform, error);
+}
+
+int kipp_step_sample(kipp_model *model, const kipp_step_item *items, size_t item_count, const kipp_sample_params *params,
+                     const double *uniform, uint32_t *tokens, size_t token_capacity, kipp_error *error) {
+    return kipp_step_sample_logits(model, items, item_count, params, uniform, tokens, token_capacity, NULL, 0, error);
 }
 
 int kipp_step_argmax(kipp_model *model, const kipp_step_item *items, size_t item_count, uint32_t *tokens, size_t token_capacity,
                      kipp_error *error) {
     uint32_t none; /* a step that wants nothing may come without room */
     if (tokens == NULL && token_capacity != 0) return kipp_fail(error, KIPP_ERROR_ARGUMENT, "no room for the tokens");
-    return step_common(model, items, item_count, NULL, tokens != NULL ? token_capacity : 0, tokens != NULL ? tokens : &none, NULL, NULL, error);
+    return step_common(model, items, item_count, NULL, 0, tokens != NULL ? tokens : &none, tokens != NULL ? token_capacity : 0, NULL, NULL, error);
 }
 
-/* `best` NULL: the wanted rows of logits go to `logits` (room for `capacity` floats); else one token for every wanted row goes
- * to `best` (room for `capacity` of them), found where the path computes: the index of the largest logit, or with `choices`
- * what kipp_sample_ex would choose with each row's parameters and draw. */
+/* `best` NULL: the wanted rows of logits go to `logits` (room for `logits_capacity` floats); else one token for every wanted
+ * row goes to `best` (room for `best_capacity` of them), found where the path computes: the index of the largest logit, or
+ * with `choices` what kipp_sample_ex would choose with each row's parameters and draw, and then `logits`, if given, gets the
+ * rows as the model left them (before a bias or a penalty changed them) as well. */
 static int step_common(kipp_model *model, const kipp_step_item *items, size_t item_count, float *logits, size_t logits_capacity, uint32_t *best,
-                       const kipp_sample_params *choices, const double *uniform, kipp_error *error) {
+                       size_t best_capacity, const kipp_sample_params *choices, const double *uniform, kipp_error *error) {
     kipp_error_clear(error);
     if (model == NULL || (items == NULL && item_count != 0)) return kipp_fail(error, KIPP_ERROR_ARGUMENT, "model and items must be given");
     if (item_count == 0) return 0;
@@ -385,12 +393,12 @@ static int step_common(kipp_model *model, const kipp_step_item *items, size_t it
         kipp_fail(error, KIPP_ERROR_RANGE, "a step of %zu tokens exceeds max_step_tokens = %u", total, model->config.max_step_tokens);
         goto unmark;
     }
-    size_t floats;
-    if (best != NULL) {
-        if (wanted > logits_capacity || wanted > INT32_MAX) {
-            kipp_fail(error, KIPP_ERROR_ARGUMENT, "%zu wanted places do not fit the %zu indices given", wanted, logits_capacity);
-            goto unmark;
-        }
+    size_t floats = 0;
+    if (best != NULL && (wanted > best_capacity || wanted > INT32_MAX)) {
+        kipp_fail(error, KIPP_ERROR_ARGUMENT, "%zu wanted places do not fit the %zu indices given", wanted, best_capacity);
+        goto unmark;
+    }
+    if (best != NULL && logits == NULL) {
         floats = 0;
     } else if (kipp_mul_size(wanted, vocab, &floats) != 0 || floats > logits_capacity || (wanted != 0 && logits == NULL)) {
         kipp_fail(error, KIPP_ERROR_ARGUMENT, "%zu wanted rows of %u logits do not fit the %zu floats given", wanted, vocab, logits_capacity);
@@ -411,6 +419,7 @@ static int step_common(kipp_model *model, const kipp_step_item *items, size_t it
     float *device_logits = NULL;
     int32_t *chosen = NULL;
     if (run_step(model, single && !model->config.eager_steps, best != NULL && choices == NULL, &device_logits, &chosen, error) != 0) goto unclaim;
+    if (best != NULL && logits != NULL && model->rt->download(model->rt, logits, device_logits, floats * sizeof(float), error) != 0) goto unclaim;
     if (choices != NULL && wanted != 0) {
         for (size_t w = 0; w < wanted; ++w) { /* what kipp_sample_ex refuses */
             const kipp_sample_params *p = &choices[w];

@@ -262,6 +262,21 @@ def test_c_command_line_on_the_gpu(model_folders, tiny_configs):
         for j, token in enumerate(generated):
             row = ref[len(prompt) - 1 + j]
             assert row[token] >= row.max() - margin
+        # sampled: the tokens are chosen on the device and the last row of logits still comes back for the table: the
+        # same output as with every row read back and chosen by kipp_sample_ex, from kipp_cli.c and from `bin/kipp --host c`
+        import sys
+        sampled = ["--model", folder, "--path", PATH[dtype], "--tokens", ",".join(map(str, prompt)), "--decode", "9", "--page", "8",
+                   "--temperature", "0.9", "--top-k", "30", "--top-p", "0.9", "--seed", "21", "--top", "5"]
+        outs = []
+        for command in ([exe, "--kernels", os.path.join(os.path.dirname(kernels.__file__), "_lib")],
+                        [sys.executable, os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "bin", "kipp"), "--host", "c"]):
+            for sampler in ("device", "host"):
+                if sampler == "host" and command[0] != exe:
+                    continue                                     # the Python command line has no switch: it is held to kipp_cli.c's output
+                run = subprocess.run(command + sampled, capture_output=True, text=True, timeout=300, env=dict(os.environ, KIPP_AMD_SAMPLER=sampler))
+                assert run.returncode == 0, run.stderr
+                outs.append(run.stdout)
+        assert outs[0] == outs[1] == outs[2] and len(outs[0].splitlines()) == 6 and len(outs[0].splitlines()[0].split("\t")[1].split()) == 9
 
 
 @pytest.mark.parametrize("key", ["a", "b"])
