@@ -148,6 +148,7 @@ def library(variant: str = "gpu") -> ctypes.CDLL:
             "kipp_model_eval": [vp, _u32p, sz, _f32p, sz, err],
             "kipp_step": [vp, ctypes.POINTER(_StepItem), sz, _f32p, sz, err],
             "kipp_step_argmax": [vp, ctypes.POINTER(_StepItem), sz, _u32p, sz, err],
+            "kipp_step_nll": [vp, ctypes.POINTER(_StepItem), sz, _u32p, ctypes.POINTER(ctypes.c_double), sz, err],
             "kipp_step_sample": [vp, ctypes.POINTER(_StepItem), sz, ctypes.POINTER(_SampleParams), ctypes.POINTER(ctypes.c_double), _u32p, sz, err],
             "kipp_step_sample_logits": [vp, ctypes.POINTER(_StepItem), sz, ctypes.POINTER(_SampleParams), ctypes.POINTER(ctypes.c_double), _u32p, sz,
                                         _f32p, sz, err],
@@ -331,6 +332,28 @@ class CModel:
         if self.lib.kipp_step_argmax(self.handle, items, len(entries), out.ctypes.data_as(_u32p), wanted, ctypes.byref(error)) != 0:
             _raise(self.lib, error)
         return [int(t) for t in out[:wanted]]
+
+    def step_nll(self, entries: Sequence[Tuple[CSession, Sequence[int], Sequence[int]]], targets: Sequence[int]) -> np.ndarray:
+        """The same batch, answered with -log softmax(row)[target] (float64) for every wanted place, computed where the
+        path computes: `targets` has one token a wanted place, in order."""
+        items = (_StepItem * len(entries))()
+        keep = []
+        wanted = 0
+        for i, (session, tokens, want) in enumerate(entries):
+            t, tp = _u32(tokens)
+            w, wp = _u32(want)
+            keep.append((t, w))
+            items[i] = _StepItem(session.handle, tp, len(t), wp if len(w) else None, len(w))
+            wanted += len(w)
+        if len(targets) != wanted:
+            raise ValueError("one target for every wanted place")
+        tg, tgp = _u32(targets if wanted else [0])
+        out = np.zeros(max(wanted, 1), dtype=np.float64)
+        error = _Error()
+        if self.lib.kipp_step_nll(self.handle, items, len(entries), tgp, out.ctypes.data_as(ctypes.POINTER(ctypes.c_double)), wanted,
+                                  ctypes.byref(error)) != 0:
+            _raise(self.lib, error)
+        return out[:wanted]
 
     def step_sample(self, entries: Sequence[Tuple[CSession, Sequence[int], Sequence[int]]], choices: Sequence[dict], logits: bool = False):
         """The same batch, answered with one token for every wanted place, chosen where the path computes as kipp_sample_ex

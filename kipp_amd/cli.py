@@ -90,7 +90,6 @@ def _ppl_stream(args) -> list:
 
 def run_perplexity_c(args, stream) -> int:
     """The same protocol through the C host: one session, reset before every window, every portion's rows from one step."""
-    import numpy as np
     from .chost import CModel
     path = args.path or ("gpu-bf16" if args.dtype == "bfloat16" else "gpu-fp32")
     window = args.ppl_window
@@ -112,14 +111,10 @@ def run_perplexity_c(args, stream) -> int:
             session.reset()
             for at in range(0, len(tokens), args.prefill_chunk):
                 chunk = tokens[at:at + args.prefill_chunk]
-                wide = session.eval_scored(chunk, len(chunk)).astype(np.float64)
                 rows = [r for r in range(len(chunk)) if at + r + 1 < len(tokens)]
-                if rows:
-                    wide = wide[rows]
-                    top = wide.max(axis=-1)
-                    targets = np.asarray([tokens[at + r + 1] for r in rows])
-                    nll += float((top + np.log(np.exp(wide - top[:, None]).sum(axis=-1)) - wide[np.arange(len(rows)), targets]).sum())
-                    scored += len(rows)
+                # every row is scored in the step that makes it: only a number a row comes back
+                nll += float(model.step_nll([(session, chunk, rows)], [tokens[at + r + 1] for r in rows]).sum())
+                scored += len(rows)
             print(f"ppl: window {w + 1}/{windows} ppl={math.exp(nll / scored):.4f}", file=sys.stderr)
         print(f"KIPP_PPL backend={path} tokens={len(stream)} scored={scored} window={window} nll={nll:.9f} "
               f"ppl={math.exp(nll / scored):.6f} seconds={time.perf_counter() - started:.3f}", file=sys.stderr)
@@ -156,9 +151,11 @@ def run_perplexity(args) -> int:
             rows = [r for r in range(len(chunk)) if at + r + 1 < len(tokens)]
             logits = engine.step([StepEntry("ppl", chunk, rows)])
             if rows:
-                targets = torch.tensor([tokens[at + r + 1] for r in rows], device=logits.device)
-                wide = logits.double()
-                nll += float((torch.logsumexp(wide, dim=-1) - wide.gather(1, targets[:, None])[:, 0]).sum())
+                # every row's -log softmax at its target by the kernel that the C host scores with (the maximum in float32,
+                # exponentials and their sum in float64): only a number a row comes back
+                targets = torch.tensor([tokens[at + r + 1] for r in rows], dtype=torch.int32, device=logits.device)
+                each = torch.empty(len(rows), dtype=torch.float64, device=logits.device)
+                nll += float(engine.rt.ops.row_nll(logits.contiguous(), targets, each).sum())
                 scored += len(rows)
         engine.close("ppl")
         print(f"ppl: window {w + 1}/{windows} ppl={math.exp(nll / scored):.4f}", file=sys.stderr)

@@ -838,6 +838,19 @@ def argmax(logits: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     return out
 
 
+def row_nll(logits: torch.Tensor, targets: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[r] = -log softmax(logits[r])[targets[r]] in float64 (the maximum in float32, exponentials and their sum in
+    float64): what a perplexity run adds up."""
+    _dev(logits, targets, out)
+    _i32(targets, "targets")
+    rows = logits.shape[0]
+    _need(logits.dtype == torch.float32 and logits.dim() == 2 and logits.is_contiguous(), "row_nll: float32 [rows, vocab]")
+    _need(targets.numel() == rows and out.numel() == rows and out.dtype == torch.float64, "row_nll: one target and one float64 a row")
+    fn = _fn("sampling", "kipp_row_nll", [_c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr])
+    _check(fn(_ptr(logits), rows, logits.shape[1], _ptr(targets), _ptr(out), _stream()), "row_nll")
+    return out
+
+
 def adjust_logits(logits: torch.Tensor, begin: torch.Tensor, biases: torch.Tensor, token: torch.Tensor, value: torch.Tensor,
                   repetition: torch.Tensor, presence: torch.Tensor, frequency: torch.Tensor) -> torch.Tensor:
     """Logit bias and the penalties over recent tokens, applied to rows of float32 logits in place, in the host

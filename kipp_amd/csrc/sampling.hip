@@ -168,6 +168,45 @@ extern "C" int kipp_argmax_static(const float* logits, int32_t* out, int rows, i
 }
 
 // ---------------------------------------------------------------------------------------
+// What a row of logits gives for its target token: -log softmax(row)[target], as the
+// reference's perplexity run computes it (/root/reference/src/kipp_cli.c:759-778): the row's
+// maximum in float32, the exponentials of (logit - maximum) and their sum in float64,
+// maximum + log(sum) - logit[target].  One workgroup a row; the sum is added in a fixed tree
+// (every lane its stride, then lanes, then waves), so a row gives the same bits every time.
+#define NLL_THREADS 256
+__global__ void __launch_bounds__(NLL_THREADS) row_nll_kernel(const float* __restrict__ logits, int vocab,
+                                                               const int32_t* __restrict__ targets, double* __restrict__ out) {
+    __shared__ float s_max[NLL_THREADS / KIPP_WAVE];
+    __shared__ double s_sum[NLL_THREADS / KIPP_WAVE];
+    const float* row = logits + (size_t)blockIdx.x * vocab;
+    float top = -INFINITY;
+    for (int i = threadIdx.x; i < vocab; i += NLL_THREADS) top = fmaxf(top, row[i]);
+    top = wave_max(top);
+    if ((threadIdx.x & (KIPP_WAVE - 1)) == 0) s_max[threadIdx.x / KIPP_WAVE] = top;
+    __syncthreads();
+    top = s_max[0];
+    for (int w = 1; w < NLL_THREADS / KIPP_WAVE; ++w) top = fmaxf(top, s_max[w]);
+    double sum = 0.0;
+    for (int i = threadIdx.x; i < vocab; i += NLL_THREADS) sum += exp((double)row[i] - (double)top);
+    for (int off = KIPP_WAVE / 2; off > 0; off >>= 1) sum += __shfl_xor(sum, off, KIPP_WAVE);
+    if ((threadIdx.x & (KIPP_WAVE - 1)) == 0) s_sum[threadIdx.x / KIPP_WAVE] = sum;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        double total = s_sum[0];
+        for (int w = 1; w < NLL_THREADS / KIPP_WAVE; ++w) total += s_sum[w];
+        out[blockIdx.x] = (double)top + log(total) - (double)row[targets[blockIdx.x]];
+    }
+}
+
+// out[r] = -log softmax(logits[r, :])[targets[r]] (float64); every target inside the vocabulary.
+extern "C" int kipp_row_nll(const float* logits, int rows, int vocab, const int32_t* targets, double* out, hipStream_t stream) {
+    if (rows <= 0) return 0;
+    if (vocab <= 0) return -1;
+    hipLaunchKernelGGL(row_nll_kernel, dim3(rows), dim3(NLL_THREADS), 0, stream, logits, vocab, targets, out);
+    return KIPP_LAUNCH_CHECK();
+}
+
+// ---------------------------------------------------------------------------------------
 // Logit bias and the penalties over a request's recent tokens, applied to rows of logits where
 // they lie, before a token is chosen from them (/root/reference/src/kipp.c:3386-3431): first every
 // bias entry in its order, l[token] += bias; then, for every distinct recent token with its count,

@@ -92,6 +92,10 @@ struct kipp_runtime {
     int (*gather_rows)(kipp_runtime *rt, const float *x, const int32_t *index, float *out, uint32_t n, uint32_t width, kipp_error *error);
     /* out[r] = the index of the largest of logits[r, :vocab], the lowest among equals (/root/reference/src/kipp.c:3459-3464) */
     int (*argmax)(kipp_runtime *rt, const float *logits, int32_t *out, uint32_t rows, uint32_t vocab, kipp_error *error);
+    /* out[r] (host memory, float64) = -log softmax(logits[r, :vocab])[targets[r]] (`targets`: host memory, inside the
+     * vocabulary): the row's maximum in float32, exponentials and their sum in float64 (/root/reference/src/kipp_cli.c:759-778).
+     * It waits for the result, and takes nothing from the step's workspace. */
+    int (*row_nll)(kipp_runtime *rt, const float *logits, const uint32_t *targets, double *out, uint32_t rows, uint32_t vocab, kipp_error *error);
     /* Optional (NULL: the caller samples on the host).  *out = memory of the path's own with one token a row, each chosen as
      * kipp_sample_ex would choose it with `params[r]` (host memory; bias and penalties change the row of logits where it
      * lies) and the draw `uniform[r]`; it takes nothing from the step's workspace, so it may follow a recorded step. */

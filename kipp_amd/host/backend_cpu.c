@@ -5,6 +5,7 @@
  * host path, /root/reference/src/kipp.c:2588-2661 and :2882-3020) and needs no GPU.
  * Weights are widened to float32 when placed; the cache is float32.
  */
+#include <math.h>
 #include <stdlib.h>
 #include <string.h>
 
@@ -135,6 +136,20 @@ static int cpu_argmax(kipp_runtime *rt, const float *logits, int32_t *out, uint3
     return 0;
 }
 
+static int cpu_row_nll(kipp_runtime *rt, const float *logits, const uint32_t *targets, double *out, uint32_t rows, uint32_t vocab, kipp_error *error) {
+    (void)rt;
+    (void)error;
+    for (uint32_t r = 0; r < rows; ++r) {
+        const float *row = logits + (size_t)r * vocab;
+        float top = row[0];
+        for (uint32_t t = 1; t < vocab; ++t) top = row[t] > top ? row[t] : top;
+        double sum = 0.0;
+        for (uint32_t t = 0; t < vocab; ++t) sum += exp((double)row[t] - (double)top);
+        out[r] = (double)top + log(sum) - (double)row[targets[r]];
+    }
+    return 0;
+}
+
 static int cpu_linear(kipp_runtime *rt, const kipp_rows *rows_in, const kipp_weight *w, uint32_t m, int max_parts, kipp_delta *out, kipp_error *error) {
     (void)max_parts;
     if (rows_in->sumsq != NULL || rows_in->steps_major) return kipp_fail(error, KIPP_ERROR_INTERNAL, "rows without their scale on the host path");
@@ -245,5 +260,6 @@ kipp_runtime *kipp_runtime_cpu(kipp_error *error) {
     rt->attention = cpu_attention;
     rt->gather_rows = cpu_gather_rows;
     rt->argmax = cpu_argmax;
+    rt->row_nll = cpu_row_nll;
     return rt;
 }

@@ -60,6 +60,7 @@ typedef int (*fn_tile_weight)(const void *, void *, int, int, int, hipStream_t);
 typedef int (*fn_argmax)(const float *, int32_t *, int, int, float *, hipStream_t);
 typedef int (*fn_sample)(const float *, int, int, const float *, const int32_t *, const float *, const float *, const double *, int32_t *,
                          hipStream_t);
+typedef int (*fn_row_nll)(const float *, int, int, const int32_t *, double *, hipStream_t);
 typedef int (*fn_adjust_logits)(float *, int, int, const int32_t *, const int32_t *, const int32_t *, const float *, const float *,
                                 const float *, const float *, hipStream_t);
 typedef int (*fn_attention_decode_fused)(const float *, int, int, const float *, const float *, float, const float *, const float *, int, void *,
@@ -112,6 +113,7 @@ typedef struct {
     fn_int_int argmax_scratch_floats;
     fn_sample sample;
     fn_adjust_logits adjust_logits;
+    fn_row_nll row_nll;
     unsigned char *sample_host; /* what the sampler of a step is told, packed by field */
     unsigned char *sample_device; /* the same on the GPU, behind the tokens chosen */
     size_t sample_bytes;        /* room of both */
@@ -231,6 +233,7 @@ static int open_common(hip_state *st, kipp_error *error) {
     KIPP_SYM(libs[7], argmax_scratch_floats, "kipp_argmax_scratch_floats");
     KIPP_SYM(libs[7], sample, "kipp_sample");
     KIPP_SYM(libs[7], adjust_logits, "kipp_adjust_logits");
+    KIPP_SYM(libs[7], row_nll, "kipp_row_nll");
     return 0;
 }
 
@@ -665,6 +668,41 @@ static int hip_gated(kipp_runtime *rt, const kipp_rows *x, const kipp_weight *w,
     return 0;
 }
 
+/* Memory of its own for what follows a step's logits (the sampler's parameters and tokens, targets and their results): host
+ * and GPU hold `bytes` each, and keep their place until more is asked for. */
+static int sample_room(hip_state *st, size_t bytes, kipp_error *error) {
+    if (bytes <= st->sample_bytes) return 0;
+    size_t room = bytes < 16384 ? 16384 : 2 * bytes;
+    unsigned char *host = realloc(st->sample_host, room);
+    if (host == NULL) return kipp_fail(error, KIPP_ERROR_MEMORY, "out of memory");
+    st->sample_host = host;
+    st->sample_bytes = 0;
+    if (st->sample_device != NULL) {
+        hipStreamSynchronize(st->stream);
+        hipFree(st->sample_device);
+        st->sample_device = NULL;
+    }
+    hipError_t code = hipMalloc((void **)&st->sample_device, room);
+    if (code != hipSuccess) return hip_bad(error, code, "hipMalloc");
+    st->sample_bytes = room;
+    return 0;
+}
+
+static int hip_row_nll(kipp_runtime *rt, const float *logits, const uint32_t *targets, double *out, uint32_t rows, uint32_t vocab, kipp_error *error) {
+    hip_state *st = rt->state;
+    if (rows == 0) return 0;
+    const size_t result_bytes = (size_t)rows * 8, target_bytes = (size_t)rows * 4;
+    if (sample_room(st, result_bytes + target_bytes, error) != 0) return -1;
+    memcpy(st->sample_host + result_bytes, targets, target_bytes);
+    hipError_t code = hipMemcpyAsync(st->sample_device + result_bytes, st->sample_host + result_bytes, target_bytes, hipMemcpyHostToDevice, st->stream);
+    if (code != hipSuccess) return hip_bad(error, code, "copy to the GPU");
+    int rc = st->row_nll(logits, (int)rows, (int)vocab, (const int32_t *)(st->sample_device + result_bytes), (double *)st->sample_device, st->stream);
+    if (rc != 0) return refused(error, "row_nll", rc);
+    code = hipMemcpyAsync(out, st->sample_device, result_bytes, hipMemcpyDeviceToHost, st->stream);
+    if (code == hipSuccess) code = hipStreamSynchronize(st->stream);
+    return code == hipSuccess ? 0 : hip_bad(error, code, "copy from the GPU (or a kernel before it)");
+}
+
 /* The device sampler over the rows of a step.  What it is told goes up in one copy, packed by field: the sampler's
  * parameters ([temperature | top_p | min_p | top_k] of 4 bytes a row, then the draws of 8), and, where a row has a bias or
  * penalties, the entries that the kernel before it walks ([begin (rows + 1) | biases | repetition | presence | frequency |
@@ -685,21 +723,7 @@ static int hip_sample(kipp_runtime *rt, float *logits, const kipp_sample_params 
     const size_t out_bytes = ((size_t)rows * 4 + 15) / 16 * 16, pack_bytes = (size_t)rows * 24;
     const size_t adjust_words = entries != 0 ? 5 * (size_t)rows + 1 + 2 * entries : 0;
     const size_t bytes = out_bytes + pack_bytes + adjust_words * 4;
-    if (bytes > st->sample_bytes) {
-        size_t room = bytes < 16384 ? 16384 : 2 * bytes;
-        unsigned char *host = realloc(st->sample_host, room);
-        if (host == NULL) return kipp_fail(error, KIPP_ERROR_MEMORY, "out of memory");
-        st->sample_host = host;
-        st->sample_bytes = 0;
-        if (st->sample_device != NULL) {
-            hipStreamSynchronize(st->stream);
-            hipFree(st->sample_device);
-            st->sample_device = NULL;
-        }
-        hipError_t code = hipMalloc((void **)&st->sample_device, room);
-        if (code != hipSuccess) return hip_bad(error, code, "hipMalloc");
-        st->sample_bytes = room;
-    }
+    if (sample_room(st, bytes, error) != 0) return -1;
     /* host and device hold the same layout; nothing of the first out_bytes goes up */
     unsigned char *h = st->sample_host + out_bytes, *d = st->sample_device + out_bytes;
     float *f32 = (float *)h;
@@ -1179,6 +1203,7 @@ kipp_runtime *kipp_runtime_hip(kipp_path path, int device, const char *kernel_di
     rt->decode_attention = hip_decode_attention;
     rt->argmax = hip_argmax;
     rt->sample = hip_sample;
+    rt->row_nll = hip_row_nll;
     rt->after_failed_step = hip_after_failed_step;
     if (path == KIPP_PATH_GPU_BF16) { /* the 32-bit path is for checking, not for speed: its steps run as they are */
         rt->graph_begin = hip_graph_begin;

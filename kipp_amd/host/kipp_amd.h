@@ -215,6 +215,12 @@ int kipp_step_sample(kipp_model *model, const kipp_step_item *items, size_t item
 int kipp_step_sample_logits(kipp_model *model, const kipp_step_item *items, size_t item_count, const kipp_sample_params *params,
                             const double *uniform, uint32_t *tokens, size_t token_capacity, float *logits, size_t logits_capacity,
                             kipp_error *error);
+/* kipp_step with, for every wanted place, what its row of logits gives for a target token: nll[w] = -log softmax(row)[targets[w]]
+ * (the row's maximum in float32, the exponentials and their sum in float64: what a perplexity run adds up,
+ * /root/reference/src/kipp_cli.c:759-778), computed where the path computes; `targets` has one token a wanted place, in the
+ * order of the items and their places.  Only a number a row comes back. */
+int kipp_step_nll(kipp_model *model, const kipp_step_item *items, size_t item_count, const uint32_t *targets, double *nll, size_t nll_capacity,
+                  kipp_error *error);
 /* The next draw of a generator, as kipp_sample_ex takes it (/root/reference/src/kipp.c:3322-3333): in [0, 1); the state must not be 0. */
 double kipp_rng_uniform(uint64_t *rng_state);
 

@@ -106,18 +106,22 @@ static int read_token_file(const char *path, uint32_t **out, size_t *count) {
 }
 
 /* Perplexity: windows of `window` tokens that do not overlap, each from an empty session, no burn-in; a window of W tokens
- * scores its W - 1 targets.  Portions of `chunk` tokens, every row's logits from one step (eval_scored); the sums in double. */
+ * scores its W - 1 targets.  Portions of `chunk` tokens, every row scored in the step that makes it (kipp_step_nll); sums in double. */
 static int run_perplexity(kipp_model *model, const kipp_model_info *info, const uint32_t *stream, size_t token_count, size_t window,
                           size_t chunk) {
     int status = 1;
     kipp_error error;
     kipp_session *session = NULL;
-    const uint32_t vocab = info->vocab_size;
-    float *logits = malloc(chunk * (size_t)vocab * sizeof(float));
-    if (logits == NULL) {
-        fprintf(stderr, "kipp: ppl: unable to allocate logits\n");
+    (void)info;
+    double *nll_of = malloc(chunk * sizeof(double));
+    uint32_t *want = malloc(chunk * sizeof(uint32_t));
+    if (nll_of == NULL || want == NULL) {
+        fprintf(stderr, "kipp: ppl: unable to allocate a portion's results\n");
+        free(nll_of);
+        free(want);
         return 1;
     }
+    for (size_t r = 0; r < chunk; ++r) want[r] = (uint32_t)r;
     if (kipp_session_create(model, (uint32_t)window, &session, &error) != 0) {
         fprintf(stderr, "kipp: ppl: session: %s\n", error.message);
         goto done;
@@ -136,19 +140,16 @@ static int run_perplexity(kipp_model *model, const kipp_model_info *info, const 
         }
         for (size_t at = 0; at < length; at += chunk) {
             const size_t n = length - at < chunk ? length - at : chunk;
-            if (kipp_session_eval_scored(session, tokens + at, n, logits, (uint32_t)n, &error) != 0) {
+            /* row r predicts the token behind it, if that lies inside the window: the rows wanted are the first `rows`, their
+             * targets the tokens from at + 1 on; each row's -log softmax at its target is computed where the logits lie */
+            const size_t rows = at + n < length ? n : n - 1;
+            kipp_step_item item = {session, tokens + at, n, want, rows};
+            if (kipp_step_nll(model, &item, 1, tokens + at + 1, nll_of, chunk, &error) != 0) {
                 fprintf(stderr, "kipp: ppl: eval: %s\n", error.message);
                 goto done;
             }
-            for (size_t r = 0; r < n && at + r + 1 < length; ++r) { /* row r predicts the token behind it, inside the window */
-                const float *row = logits + r * (size_t)vocab;
-                float top = row[0];
-                for (uint32_t t = 1; t < vocab; ++t) top = row[t] > top ? row[t] : top;
-                double sum = 0.0;
-                for (uint32_t t = 0; t < vocab; ++t) sum += exp((double)row[t] - (double)top);
-                nll += (double)top + log(sum) - (double)row[tokens[at + r + 1]];
-                ++scored;
-            }
+            for (size_t r = 0; r < rows; ++r) nll += nll_of[r];
+            scored += rows;
         }
         fprintf(stderr, "ppl: window %zu/%zu ppl=%.4f\n", w + 1, windows, exp(nll / (double)scored));
     }
@@ -157,7 +158,8 @@ static int run_perplexity(kipp_model *model, const kipp_model_info *info, const 
     status = 0;
 done:
     kipp_session_destroy(session);
-    free(logits);
+    free(nll_of);
+    free(want);
     return status;
 }
 

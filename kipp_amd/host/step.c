@@ -314,12 +314,17 @@ uint64_t kipp_test_graph_replays(const kipp_model *model) { return model != NULL
 /* For tests: work lists of prompt portions whose keys were cut over more workgroups since the model was opened. */
 uint64_t kipp_test_cut_attention_steps(const kipp_model *model) { return model != NULL ? model->rt->cut_attention_steps : 0; }
 
+typedef struct {
+    const uint32_t *targets; /* one a wanted place */
+    double *nll;
+    size_t capacity;
+} nll_request;
 static int step_common(kipp_model *model, const kipp_step_item *items, size_t item_count, float *logits, size_t logits_capacity, uint32_t *best,
-                       size_t best_capacity, const kipp_sample_params *choices, const double *uniform, kipp_error *error);
+                       size_t best_capacity, const kipp_sample_params *choices, const double *uniform, const nll_request *scored, kipp_error *error);
 
 int kipp_step(kipp_model *model, const kipp_step_item *items, size_t item_count, float *logits, size_t logits_capacity,
               kipp_error *error) {
-    return step_common(model, items, item_count, logits, logits_capacity, NULL, 0, NULL, NULL, error);
+    return step_common(model, items, item_count, logits, logits_capacity, NULL, 0, NULL, NULL, NULL, error);
 }
 
 int kipp_step_sample_logits(kipp_model *model, const kipp_step_item *items, size_t item_count, const kipp_sample_params *params,
@@ -331,7 +336,7 @@ int kipp_step_sample_logits(kipp_model *model, const kipp_step_item *items, size
     if (params == NULL || uniform == NULL) return kipp_fail(error, KIPP_ERROR_ARGUMENT, "parameters and draws must be given");
     if (tokens == NULL && token_capacity != 0) return kipp_fail(error, KIPP_ERROR_ARGUMENT, "no room for the tokens");
     return step_common(model, items, item_count, logits, logits != NULL ? logits_capacity : 0, tokens != NULL ? tokens : &none,
-                       tokens != NULL ? token_capacity : 0, params, uniform, error);
+                       tokens != NULL ? token_capacity : 0, params, uniform, NULL, error);
 }
 
 int kipp_step_sample(kipp_model *model, const kipp_step_item *items, size_t item_count, const kipp_sample_params *params,
@@ -339,19 +344,28 @@ int kipp_step_sample(kipp_model *model, const kipp_step_item *items, size_t item
     return kipp_step_sample_logits(model, items, item_count, params, uniform, tokens, token_capacity, NULL, 0, error);
 }
 
+int kipp_step_nll(kipp_model *model, const kipp_step_item *items, size_t item_count, const uint32_t *targets, double *nll, size_t nll_capacity,
+                  kipp_error *error) {
+    kipp_error_clear(error);
+    if (targets == NULL || nll == NULL) return kipp_fail(error, KIPP_ERROR_ARGUMENT, "targets and room for the results must be given");
+    const nll_request scored = {targets, nll, nll_capacity};
+    return step_common(model, items, item_count, NULL, 0, NULL, 0, NULL, NULL, &scored, error);
+}
+
 int kipp_step_argmax(kipp_model *model, const kipp_step_item *items, size_t item_count, uint32_t *tokens, size_t token_capacity,
                      kipp_error *error) {
     uint32_t none; /* a step that wants nothing may come without room */
     if (tokens == NULL && token_capacity != 0) return kipp_fail(error, KIPP_ERROR_ARGUMENT, "no room for the tokens");
-    return step_common(model, items, item_count, NULL, 0, tokens != NULL ? tokens : &none, tokens != NULL ? token_capacity : 0, NULL, NULL, error);
+    return step_common(model, items, item_count, NULL, 0, tokens != NULL ? tokens : &none, tokens != NULL ? token_capacity : 0, NULL, NULL, NULL, error);
 }
 
 /* `best` NULL: the wanted rows of logits go to `logits` (room for `logits_capacity` floats); else one token for every wanted
  * row goes to `best` (room for `best_capacity` of them), found where the path computes: the index of the largest logit, or
  * with `choices` what kipp_sample_ex would choose with each row's parameters and draw, and then `logits`, if given, gets the
- * rows as the model left them (before a bias or a penalty changed them) as well. */
+ * rows as the model left them (before a bias or a penalty changed them) as well.  With `scored` neither: every wanted row's
+ * -log softmax at its target goes there. */
 static int step_common(kipp_model *model, const kipp_step_item *items, size_t item_count, float *logits, size_t logits_capacity, uint32_t *best,
-                       size_t best_capacity, const kipp_sample_params *choices, const double *uniform, kipp_error *error) {
+                       size_t best_capacity, const kipp_sample_params *choices, const double *uniform, const nll_request *scored, kipp_error *error) {
     kipp_error_clear(error);
     if (model == NULL || (items == NULL && item_count != 0)) return kipp_fail(error, KIPP_ERROR_ARGUMENT, "model and items must be given");
     if (item_count == 0) return 0;
@@ -398,7 +412,18 @@ static int step_common(kipp_model *model, const kipp_step_item *items, size_t it
         kipp_fail(error, KIPP_ERROR_ARGUMENT, "%zu wanted places do not fit the %zu indices given", wanted, best_capacity);
         goto unmark;
     }
-    if (best != NULL && logits == NULL) {
+    if (scored != NULL) {
+        if (wanted > scored->capacity || wanted > INT32_MAX) {
+            kipp_fail(error, KIPP_ERROR_ARGUMENT, "%zu wanted places do not fit the %zu results given", wanted, scored->capacity);
+            goto unmark;
+        }
+        for (size_t w = 0; w < wanted; ++w) {
+            if (scored->targets[w] >= vocab) {
+                kipp_fail(error, KIPP_ERROR_RANGE, "wanted place %zu: target %u is outside the vocabulary of %u", w, scored->targets[w], vocab);
+                goto unmark;
+            }
+        }
+    } else if (best != NULL && logits == NULL) {
         floats = 0;
     } else if (kipp_mul_size(wanted, vocab, &floats) != 0 || floats > logits_capacity || (wanted != 0 && logits == NULL)) {
         kipp_fail(error, KIPP_ERROR_ARGUMENT, "%zu wanted rows of %u logits do not fit the %zu floats given", wanted, vocab, logits_capacity);
@@ -431,7 +456,9 @@ static int step_common(kipp_model *model, const kipp_step_item *items, size_t it
         if (model->rt->sample(model->rt, device_logits, choices, uniform, &chosen, (uint32_t)wanted, vocab, error) != 0) goto unclaim;
     }
     /* reading back (even nothing) waits for the step's work: what it wrote into the pages is there when it returns */
-    if (best != NULL && wanted != 0) {
+    if (scored != NULL && wanted != 0) {
+        if (model->rt->row_nll(model->rt, device_logits, scored->targets, scored->nll, (uint32_t)wanted, vocab, error) != 0) goto unclaim;
+    } else if (best != NULL && wanted != 0) {
         if (model->rt->download(model->rt, best, chosen, wanted * sizeof(int32_t), error) != 0) goto unclaim;
     } else if (model->rt->download(model->rt, logits, device_logits, floats * sizeof(float), error) != 0) {
         goto unclaim;

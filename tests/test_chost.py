@@ -536,6 +536,26 @@ def test_perplexity_through_the_c_command_lines(model_folders, tiny_configs, cap
         assert bad.returncode == code and words in bad.stderr, (extra, bad.returncode, bad.stderr)
 
 
+def test_step_nll_is_the_row_s_log_softmax_at_its_target(model_folders, tiny_configs):
+    """kipp_step_nll: a mixed step answered with one float64 a wanted place, -log softmax(row)[target], from the logits
+    that kipp_step gives for the same step; targets outside the vocabulary and too little room are refused before anything runs."""
+    cfg = tiny_configs["a"]
+    vocab = cfg["vocab_size"]
+    with CModel(model_folders[("a", "float32")], path="cpu-fp32", page_tokens=4, kv_pool_pages=32, share_prefixes=False) as model:
+        a, b, c, d = (model.session() for _ in range(4))
+        pa, pb = H.random_tokens(1, 13, vocab), H.random_tokens(2, 7, vocab)
+        rows = model.step([(a, pa, [0, 3, 12]), (b, pb, [6])]).astype(np.float64)
+        targets = [5, vocab - 1, 0, 9]
+        got = model.step_nll([(c, pa, [0, 3, 12]), (d, pb, [6])], targets)
+        top = rows.max(axis=1)
+        want = top + np.log(np.exp(rows - top[:, None]).sum(axis=1)) - rows[np.arange(4), targets]
+        assert np.allclose(got, want, rtol=1e-12, atol=1e-12)
+        assert len(model.step_nll([(c, [5], [])], [])) == 0 and c.length == 14
+        with pytest.raises(KippError, match="outside the vocabulary"):
+            model.step_nll([(c, [1], [0])], [vocab])
+        assert c.length == 14
+
+
 def test_step_argmax_is_the_argmax_of_step(model_folders, tiny_configs):
     """kipp_step_argmax: the same step answered with one index a wanted place, the lowest among equal logits; room is checked."""
     cfg = tiny_configs["a"]

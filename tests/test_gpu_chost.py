@@ -206,6 +206,29 @@ def test_c_host_tokens_chosen_beside_the_logits(model_folders, tiny_configs, dty
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_c_host_rows_scored_beside_the_logits(model_folders, tiny_configs, dtype):
+    """kipp_step_nll on the GPU paths: -log softmax at a target for every wanted row of a mixed step, against float64 over
+    the logits that the same step gives a twin session (the same launches, so the same bits of logits)."""
+    from kipp_amd.chost import CModel
+    cfg = tiny_configs["b"]
+    vocab, folder = cfg["vocab_size"], model_folders[("b", dtype)]
+    with CModel(folder, path=PATH[dtype], page_tokens=8, kv_pool_pages=24, share_prefixes=False) as model:
+        a, b, c, d = (model.session() for _ in range(4))
+        pa, pb = H.random_tokens(31, 29, vocab), H.random_tokens(32, 3, vocab)
+        want_a = list(range(0, 29, 3))
+        rows = model.step([(a, pa, want_a), (b, pb, [2])]).astype(np.float64)
+        targets = H.random_tokens(33, len(want_a) + 1, vocab)
+        got = model.step_nll([(c, pa, want_a), (d, pb, [2])], targets)
+        top = rows.max(axis=1)
+        want = top + np.log(np.exp(rows - top[:, None]).sum(axis=1)) - rows[np.arange(len(targets)), targets]
+        assert np.allclose(got, want, rtol=1e-12, atol=1e-12), np.abs(got - want).max()
+        one = model.step_nll([(c, [4], [0]), (d, [9], [0])], [1, 2])          # single tokens: the recorded kind of step
+        again = model.step([(a, [4], [0]), (b, [9], [0])]).astype(np.float64)
+        top = again.max(axis=1)
+        assert np.allclose(one, top + np.log(np.exp(again - top[:, None]).sum(axis=1)) - again[[0, 1], [1, 2]], rtol=1e-12, atol=1e-12)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_c_scheduler_samples_on_the_device_as_on_the_host(model_folders, tiny_configs, dtype, monkeypatch):
     """Requests with temperature, top-k, top-p and min-p beside greedy ones through the C scheduler: chosen by the device
     sampler, with the draws of each request's generator, they are the tokens that KIPP_AMD_SAMPLER=host (every row's

@@ -1264,6 +1264,26 @@ def test_bias_and_penalties_on_the_device_are_the_host_sampler_s(vocab):
         assert picked[i] == sample(logits[i], params, XorShift64Star(int(seeds[i])), recent), i
 
 
+@pytest.mark.parametrize("vocab", [509, 151936])
+def test_row_nll_against_float64(vocab):
+    """-log softmax at a target: the maximum in float32, exponentials and sum in float64, as the perplexity run of the
+    reference adds it up; rows with a far outlier and with equal values."""
+    ops = _ops()
+    rng = np.random.default_rng(vocab + 5)
+    rows = 9
+    logits = (rng.normal(size=(rows, vocab)) * rng.choice([0.5, 4.0, 12.0], size=(rows, 1))).astype(np.float32)
+    logits[1, 7] = 80.0
+    logits[2] = 0.25
+    targets = rng.integers(0, vocab, rows)
+    targets[1] = 7
+    got = ops.row_nll(_t(logits), _t(targets, torch.int32), torch.empty(rows, dtype=torch.float64, device=DEV)).cpu().numpy()
+    wide = logits.astype(np.float64)
+    top = wide.max(axis=1)
+    want = top + np.log(np.exp(wide - top[:, None]).sum(axis=1)) - wide[np.arange(rows), targets]
+    assert np.allclose(got, want, rtol=1e-13, atol=1e-13), np.abs(got - want).max()
+    assert abs(got[2] - np.log(vocab)) < 1e-12 and got[1] < 1e-6
+
+
 def test_device_sampler_follows_the_distribution():
     ops = _ops()
     from kipp_amd.sampling import XorShift64Star
