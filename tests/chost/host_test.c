@@ -234,6 +234,38 @@ static void test_model(const char *folder) {
     kipp_session_destroy(c);
     kipp_model_kv_pool_stats(model, 0, &after);
     CHECK(after.free_blocks == after.total_blocks && after.reused_blocks_total >= 9);
+    /* rows scored in the step that makes them: -log softmax at the next token, from the logits of the whole sequence */
+    {
+        kipp_session *e = NULL;
+        double each[64], sum = 0.0, want_sum = 0.0;
+        CHECK(kipp_session_create(model, 0, &e, &error) == 0);
+        kipp_step_item scored_item = {e, tokens, n, want, n - 1};
+        CHECK(kipp_step_nll(model, &scored_item, 1, tokens + 1, each, 64, &error) == 0);
+        for (uint32_t r = 0; r + 1 < n; ++r) {
+            const float *row = whole + (size_t)r * vocab;
+            float top = row[0];
+            double total = 0.0;
+            for (uint32_t t = 1; t < vocab; ++t) top = row[t] > top ? row[t] : top;
+            for (uint32_t t = 0; t < vocab; ++t) total += exp((double)row[t] - (double)top);
+            want_sum += (double)top + log(total) - (double)row[tokens[r + 1]];
+            sum += each[r];
+        }
+        CHECK(fabs(sum - want_sum) < 1e-9 && sum > 0.0);
+        CHECK(kipp_step_nll(model, &scored_item, 1, tokens + 1, each, 3, &error) != 0 && error.code == KIPP_ERROR_ARGUMENT);
+        uint32_t far_target = vocab;
+        kipp_step_item one = {e, tokens, 1, want, 1};
+        CHECK(kipp_step_nll(model, &one, 1, &far_target, each, 64, &error) != 0 && error.code == KIPP_ERROR_RANGE);
+        /* the scalar path has no sampler of its own; the generator's draws are kipp_sample_ex's */
+        kipp_sample_params greedy_params;
+        memset(&greedy_params, 0, sizeof(greedy_params));
+        double draw = 0.0;
+        uint32_t token = 0;
+        CHECK(kipp_step_sample(model, &one, 1, &greedy_params, &draw, &token, 1, &error) != 0 && error.code == KIPP_ERROR_UNSUPPORTED);
+        uint64_t state = 88172645463325252ull, twin = state;
+        double u = kipp_rng_uniform(&state);
+        CHECK(u >= 0.0 && u < 1.0 && state != twin);
+        kipp_session_destroy(e);
+    }
     /* evaluation through a session of its own: the bits of the whole sequence, nothing held afterwards, three slots free again */
     CHECK(kipp_model_eval(model, tokens, n, spare, vocab, &error) == 0 && same_bits(spare, whole + (size_t)(n - 1) * vocab, vocab));
     CHECK(kipp_model_eval(model, tokens, n, spare, vocab - 1, &error) != 0 && error.code == KIPP_ERROR_RANGE);
