@@ -271,6 +271,14 @@ __device__ __forceinline__ uint32_t float_order(float x) {
     return (b & 0x80000000u) ? ~b : (b | 0x80000000u);   // larger float, larger integer
 }
 
+// The float whose order is `o`, for the ends of a range of orders: orders beyond the infinities (the patterns of NaN)
+// give the infinity on their side, so that a comparison with the end never turns false for a number inside the range.
+__device__ __forceinline__ float float_of_order(uint32_t o) {
+    if (o > 0xff800000u) return INFINITY;
+    if (o < 0x007fffffu) return -INFINITY;
+    return __uint_as_float((o & 0x80000000u) ? (o & 0x7fffffffu) : ~o);
+}
+
 struct SampleRow {
     const float* row;
     int vocab;
@@ -278,70 +286,250 @@ struct SampleRow {
     unsigned long long key_floor;   // candidates of the top-k cut have key >= key_floor
     double min_weight;              // ... and weight >= min_weight (0: no min-p)
 
-    __device__ __forceinline__ bool member(int i, unsigned long long* key, float* weight) const {
-        const float scaled = row[i] * inv_t;
-        if (!(scaled >= cutoff)) return false;
-        *key = ((unsigned long long)float_order(scaled) << 32) | (uint32_t)(0xffffffffu - (uint32_t)i);
-        if (*key < key_floor) return false;
+    // a candidate by its logit and the top-k cut alone (no exponential yet): its key and its scaled logit
+    __device__ __forceinline__ bool candidate(int i, float logit, unsigned long long* key, float* scaled) const {
+        *scaled = logit * inv_t;
+        if (!(*scaled >= cutoff)) return false;
+        *key = ((unsigned long long)float_order(*scaled) << 32) | (uint32_t)(0xffffffffu - (uint32_t)i);
+        return *key >= key_floor;
+    }
+    // its weight, and whether min-p keeps it
+    __device__ __forceinline__ bool weighs(float scaled, float* weight) const {
         *weight = expf(scaled - scaled_max);
         return (double)*weight >= min_weight;
     }
+    __device__ __forceinline__ bool member(int i, float logit, unsigned long long* key, float* weight) const {
+        float scaled;
+        return candidate(i, logit, key, &scaled) && weighs(scaled, weight);
+    }
 };
+
+// f(i, row[i]) for every logit of a row, a lane's in ascending order, eight loads asked for before the first is used (a pass
+// over a row is a chain of loads otherwise, each waiting for the one before); loads of 16 bytes where the row allows them
+// (a vocabulary that is a multiple of four: a quarter of the loads, and of the waits).
+#define SAMPLE_AHEAD 8
+template <typename F>
+__device__ __forceinline__ void for_each_logit(const float* __restrict__ row, int vocab, F f) {
+    if ((vocab & 3) == 0 && ((size_t)row & 15) == 0) {
+        const float4* __restrict__ row4 = (const float4*)row;
+        const int quads = vocab >> 2;
+        for (int base = threadIdx.x; base < quads; base += SAMPLE_AHEAD * blockDim.x) {
+            float4 v[SAMPLE_AHEAD];
+#pragma unroll
+            for (int j = 0; j < SAMPLE_AHEAD; ++j) {
+                const int q = base + j * blockDim.x;
+                v[j] = q < quads ? row4[q] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            }
+#pragma unroll
+            for (int j = 0; j < SAMPLE_AHEAD; ++j) {
+                const int q = base + j * blockDim.x;
+                if (q < quads) {
+                    f(4 * q, v[j].x);
+                    f(4 * q + 1, v[j].y);
+                    f(4 * q + 2, v[j].z);
+                    f(4 * q + 3, v[j].w);
+                }
+            }
+        }
+        return;
+    }
+    for (int base = threadIdx.x; base < vocab; base += SAMPLE_AHEAD * blockDim.x) {
+        float v[SAMPLE_AHEAD];
+#pragma unroll
+        for (int j = 0; j < SAMPLE_AHEAD; ++j) {
+            const int i = base + j * blockDim.x;
+            v[j] = i < vocab ? row[i] : 0.0f;
+        }
+#pragma unroll
+        for (int j = 0; j < SAMPLE_AHEAD; ++j) {
+            const int i = base + j * blockDim.x;
+            if (i < vocab) f(i, v[j]);
+        }
+    }
+}
+
+// The histogram of one level: for each value of the key's byte the measure of the candidates that have it (masses or
+// counts), how many they are, and the key of one of them (the key of the only one, where there is one).
+struct Bins {
+    unsigned long long measure[256];
+    unsigned long long key[256];
+    unsigned int count[256];
+};
+
+// What a lane has gathered for one bin goes to the workgroup's histogram: where all lanes of the wave mean the same bin (the
+// usual case: neighbouring logits share their leading bits) the wave adds up first and one lane goes to memory.  Integer
+// sums: the order of the additions changes nothing.
+__device__ __forceinline__ void add_to_bin(Bins* bins, int bin, unsigned long long m, unsigned int n, unsigned long long key) {
+    const int first = __builtin_amdgcn_readfirstlane(bin);
+    if (__all(bin == first)) {
+        if (n != 0) bins->key[first] = key;       // any of them: the key is only looked at where the bin holds one candidate
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            m += __shfl_xor(m, off, KIPP_WAVE);
+            n += __shfl_xor(n, off, KIPP_WAVE);
+        }
+        if ((threadIdx.x & (KIPP_WAVE - 1)) == 0 && n != 0) {
+            atomicAdd(&bins->measure[first], m);
+            atomicAdd(&bins->count[first], n);
+        }
+    } else if (n != 0) {
+        atomicAdd(&bins->measure[bin], m);
+        atomicAdd(&bins->count[bin], n);
+        bins->key[bin] = key;
+    }
+}
+
+// One pass over the row: the candidates whose key begins with `prefix` above `level` (level 7: all; `only_byte` >= 0: those
+// with that top byte alone) go into `bins` by the key's byte at `level`.  A lane keeps what it has gathered for the bin it met
+// last and goes to the histogram only when the bin changes; the exponential is taken only of candidates under the prefix.
+template <bool MASS>
+__device__ __forceinline__ void gather(const SampleRow& r, int level, unsigned long long prefix, int only_byte, Bins* bins) {
+    int at_bin = 0;
+    unsigned int n = 0;
+    unsigned long long sum = 0, last_key = 0;
+    // Most logits of a pass fall to a comparison of two floats: the key's upper half is a monotone image of the scaled logit,
+    // so the keys at or above the floor, under a prefix that lies within that half (levels 6 to 4), or with one top byte, are
+    // the scaled logits of a range, and only what lies in it goes through the exact tests below.
+    uint32_t order_lo = (uint32_t)(r.key_floor >> 32), order_hi = 0xffffffffu;
+    if (level >= 4 && level < 7) {
+        const int free_bits = 8 * (level + 1) - 32;
+        const uint32_t first = (uint32_t)(prefix << free_bits);
+        order_lo = first > order_lo ? first : order_lo;
+        order_hi = first | ((1u << free_bits) - 1u);
+    } else if (level == 7 && only_byte >= 0) {
+        const uint32_t first = (uint32_t)only_byte << 24;
+        order_lo = first > order_lo ? first : order_lo;
+        order_hi = first | 0x00ffffffu;
+    }
+    const float range_lo = fmaxf(float_of_order(order_lo), r.cutoff), range_hi = float_of_order(order_hi);
+    for_each_logit(r.row, r.vocab, [&](int i, float logit) {
+        unsigned long long key;
+        float scaled, w = 1.0f;
+        if (!(logit * r.inv_t >= range_lo && logit * r.inv_t <= range_hi)) return;
+        if (!r.candidate(i, logit, &key, &scaled)) return;
+        if (level < 7 && (key >> (8 * (level + 1))) != prefix) return;
+        if (only_byte >= 0 && (int)(key >> 56) != only_byte) return;
+        if ((MASS || r.min_weight > 0.0) && !r.weighs(scaled, &w)) return;
+        const int bin = (int)((key >> (8 * level)) & 0xff);
+        if (bin != at_bin && n != 0) {
+            atomicAdd(&bins->measure[at_bin], sum);
+            atomicAdd(&bins->count[at_bin], n);
+            bins->key[at_bin] = last_key;
+            sum = 0;
+            n = 0;
+        }
+        at_bin = bin;
+        sum += MASS ? (unsigned long long)(w * MASS_SCALE) : 1ull;
+        n += 1;
+        last_key = key;
+    });
+    add_to_bin(bins, at_bin, sum, n, last_key);
+}
 
 // Walk down the key bytes.  With MASS the measure of a candidate is its fixed-point weight,
 // else 1.  Finds the first candidate in key order (descending) at which the running measure
 // reaches `target` (STRICT: exceeds it).  Returns its key; *before gets the measure of the
 // candidates ahead of it, *own its own measure.  If the target is beyond the total, the
-// last candidate is returned.
+// last candidate is returned.  The walk ends at the level whose chosen byte one candidate alone
+// has: that candidate is the answer, and the levels below would add nothing ahead of it.
+// `fraction` (not null): the target is *fraction times the measure of all candidates, which the
+// top level's histogram adds up to.  `top` (not null) with `keep`: the top level's histogram is
+// left there; without `keep`: it is taken from there for the bytes above the floor's (their
+// candidates have not changed since: only the floor was raised), and the floor's own byte is
+// gathered again.
 template <bool MASS, bool STRICT>
-__device__ unsigned long long descend(const SampleRow& r, double target, unsigned long long* hist,
+__device__ unsigned long long descend(const SampleRow& r, double target, const double* fraction, Bins* bins, Bins* top, bool keep,
                                       unsigned long long* shared, double* before, double* own) {
     unsigned long long prefix = 0;      // the key bytes fixed so far, right-aligned
-    double ahead = 0.0;
+    unsigned long long ahead = 0;       // the measure of the candidates ahead of the prefix: an integer, exact
     for (int level = 7; level >= 0; --level) {
         if (level == 3) {               // byte 3 is the top byte of the inverted index: always 0xff (vocab < 2^24)
             prefix = (prefix << 8) | 0xffull;
             continue;
         }
-        for (int b = threadIdx.x; b < 256; b += blockDim.x) hist[b] = 0;
-        __syncthreads();
-        for (int i = threadIdx.x; i < r.vocab; i += blockDim.x) {
-            unsigned long long key;
-            float w;
-            if (!r.member(i, &key, &w)) continue;
-            if (level < 7 && (key >> (8 * (level + 1))) != prefix) continue;
-            const unsigned long long m = MASS ? (unsigned long long)(w * MASS_SCALE) : 1ull;
-            atomicAdd(&hist[(key >> (8 * level)) & 0xff], m);
+        const int floor_byte = (int)(r.key_floor >> 56);
+        const bool reuse = level == 7 && top != nullptr && !keep;
+        for (int b = threadIdx.x; b < 256; b += blockDim.x) {
+            const bool from_top = reuse && b > floor_byte;
+            bins->measure[b] = from_top ? top->measure[b] : 0;
+            bins->count[b] = from_top ? top->count[b] : 0;
+            if (from_top) bins->key[b] = top->key[b];
         }
         __syncthreads();
-        if (threadIdx.x == 0) {
-            int chosen = -1, lowest = 0;
-            double run = ahead;
-            for (int b = 255; b >= 0; --b) {
-                if (hist[b] == 0) continue;
-                lowest = b;
-                const double next = run + (double)hist[b];
-                if (STRICT ? next > target : next >= target) {
-                    chosen = b;
-                    break;
+        gather<MASS>(r, level, prefix, reuse ? floor_byte : -1, bins);
+        __syncthreads();
+        if (level == 7 && top != nullptr && keep) {
+            for (int b = threadIdx.x; b < 256; b += blockDim.x) {
+                top->measure[b] = bins->measure[b];
+                top->count[b] = bins->count[b];
+                top->key[b] = bins->key[b];
+            }
+        }
+        // The byte at which the running measure reaches the target, found by the first wave: a lane takes four bins (the
+        // highest bytes first), the lanes' sums are scanned across the wave, and every lane looks for the place among its own.
+        if (threadIdx.x < KIPP_WAVE) {
+            const int l = threadIdx.x;
+            unsigned long long h[4], mine = 0;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                h[q] = bins->measure[255 - 4 * l - q];
+                mine += h[q];
+            }
+            unsigned long long through = mine;                     // of this lane's bins and of all lanes before it
+#pragma unroll
+            for (int off = 1; off < KIPP_WAVE; off <<= 1) {
+                const unsigned long long other = __shfl_up(through, off, KIPP_WAVE);
+                if (l >= off) through += other;
+            }
+            const unsigned long long total = __shfl(through, KIPP_WAVE - 1, KIPP_WAVE);
+            if (level == 7 && fraction != nullptr) target = *fraction * (double)total;
+            unsigned long long run = ahead + (through - mine), run_there = 0;
+            int found = -1, low = -1;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                if (h[q] == 0) continue;
+                low = 255 - 4 * l - q;
+                if (found >= 0) continue;
+                const unsigned long long next = run + h[q];
+                if (STRICT ? (double)next > target : (double)next >= target) {
+                    found = 255 - 4 * l - q;
+                    run_there = run;
+                } else {
+                    run = next;
                 }
-                run = next;
             }
-            if (chosen < 0) {           // the target lies beyond everything: the last candidate
-                chosen = lowest;
-                run -= (double)hist[lowest];
+            const unsigned long long reached = __ballot(found >= 0), filled = __ballot(mine != 0);
+            int chosen = 0;
+            unsigned long long chosen_run = ahead;
+            if (reached != 0) {
+                const int from = __ffsll((long long)reached) - 1;
+                chosen = __shfl(found, from, KIPP_WAVE);
+                chosen_run = __shfl(run_there, from, KIPP_WAVE);
+            } else if (filled != 0) {   // the target lies beyond everything: the last candidate
+                chosen = __shfl(low, 63 - __clzll((long long)filled), KIPP_WAVE);
+                chosen_run = ahead + total - bins->measure[chosen];
             }
-            shared[0] = (unsigned long long)chosen;
-            shared[1] = (unsigned long long)__double_as_longlong(run);
-            shared[2] = hist[chosen];
+            if (l == 0) {
+                shared[0] = (unsigned long long)chosen;
+                shared[1] = chosen_run;
+                shared[2] = bins->measure[chosen];
+                shared[3] = bins->count[chosen] == 1 ? bins->key[chosen] : 0;       // (no key is 0: byte 3 is 0xff)
+                shared[4] = (unsigned long long)__double_as_longlong(target);
+            }
         }
         __syncthreads();
         prefix = (prefix << 8) | shared[0];
-        ahead = __longlong_as_double((long long)shared[1]);
+        ahead = shared[1];
         *own = (double)shared[2];
+        const unsigned long long alone = shared[3];
+        target = __longlong_as_double((long long)shared[4]);
         __syncthreads();
+        if (alone != 0) {
+            prefix = alone;
+            break;
+        }
     }
-    *before = ahead;
+    *before = (double)ahead;
     return prefix;
 }
 
@@ -349,8 +537,8 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) sample_kernel(
     const float* __restrict__ logits, int vocab, const float* __restrict__ temperature, const int32_t* __restrict__ top_k,
     const float* __restrict__ top_p, const float* __restrict__ min_p, const double* __restrict__ uniform,
     int32_t* __restrict__ out) {
-    __shared__ unsigned long long hist[256];
-    __shared__ unsigned long long shared[4];
+    __shared__ Bins bins, top;
+    __shared__ unsigned long long shared[5];
     __shared__ float best_v[16];
     __shared__ int best_i[16];
     const int rowi = blockIdx.x;
@@ -358,13 +546,12 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) sample_kernel(
     // ---- the maximum, the lowest index among equals
     float bv = -INFINITY;
     int bi = 0x7fffffff;
-    for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
-        const float v = row[i];
+    for_each_logit(row, vocab, [&](int i, float v) {
         if (v > bv || (bi == 0x7fffffff && !(v != v))) {
             bv = v;
             bi = i;
         }
-    }
+    });
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {
         const float ov = __shfl_xor(bv, off, KIPP_WAVE);
@@ -403,28 +590,17 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) sample_kernel(
     double before, own;
     // ---- top-k: the key of the k-th candidate is the floor of what stays
     const int k = top_k[rowi];
-    if (k > 0) r.key_floor = descend<false, false>(r, (double)k, hist, shared, &before, &own);
+    if (k > 0) r.key_floor = descend<false, false>(r, (double)k, nullptr, &bins, nullptr, false, shared, &before, &own);
     // ---- min-p relative to the top weight, which is exp(0) = 1
     const float mp = min_p[rowi];
     if (mp > 0.0f) r.min_weight = (double)mp;
-    // ---- top-p: the shortest prefix whose mass reaches top_p of the total
-    for (int b = threadIdx.x; b < 4; b += blockDim.x) shared[b] = 0;
-    __syncthreads();
-    unsigned long long mine = 0;
-    for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
-        unsigned long long key;
-        float w;
-        if (r.member(i, &key, &w)) mine += (unsigned long long)(w * MASS_SCALE);
-    }
-    atomicAdd(&shared[3], mine);
-    __syncthreads();
-    const double total = (double)shared[3];
-    __syncthreads();
-    const unsigned long long last = descend<true, false>(r, (double)top_p[rowi] * total, hist, shared, &before, &own);
+    // ---- top-p: the shortest prefix whose mass reaches top_p of the total (the total: what the top level's histogram adds up to)
+    const double share = (double)top_p[rowi];
+    const unsigned long long last = descend<true, false>(r, 0.0, &share, &bins, &top, true, shared, &before, &own);
     if (last > r.key_floor) r.key_floor = last;
     const double kept = before + own;
-    // ---- the draw
-    const unsigned long long pick = descend<true, true>(r, uniform[rowi] * kept, hist, shared, &before, &own);
+    // ---- the draw, among what is kept: above the floor's byte the top level's histogram still holds
+    const unsigned long long pick = descend<true, true>(r, uniform[rowi] * kept, nullptr, &bins, &top, false, shared, &before, &own);
     if (threadIdx.x == 0) out[rowi] = (int32_t)(0xffffffffu - (uint32_t)(pick & 0xffffffffu));
 }
 

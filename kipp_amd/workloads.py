@@ -68,13 +68,15 @@ def shared_prefix_prompts(n: int, prefix: int, suffix: int, vocab: int, seed: in
     return [head + torch.randint(0, vocab, (suffix,), generator=gen).tolist() for _ in range(n)]
 
 
-def serve(engine, prompts, new_tokens: int, chunk: int, max_step_tokens: int):
-    """All requests arrive at once; runs until every one has finished."""
+def serve(engine, prompts, new_tokens: int, chunk: int, max_step_tokens: int, sampling: dict = None):
+    """All requests arrive at once; runs until every one has finished.  `sampling`: the sampler's parameters by name for
+    every request (none: greedy); request i draws from seed 100 + i."""
     import torch
     from .engine.scheduler import Request, Scheduler
+    from .sampling import SampleParams
     sched = Scheduler(engine, max_step_tokens=max_step_tokens, prefill_chunk=chunk, max_running=len(prompts))
     for i, prompt in enumerate(prompts):
-        sched.add(Request(i, prompt, new_tokens))
+        sched.add(Request(i, prompt, new_tokens, params=SampleParams(**sampling), seed=100 + i) if sampling else Request(i, prompt, new_tokens))
     torch.cuda.synchronize()
     start = time.perf_counter()
     last = start
@@ -92,7 +94,7 @@ def serve(engine, prompts, new_tokens: int, chunk: int, max_step_tokens: int):
     return sched, seconds, first
 
 
-def serve_c(config, prompts, new_tokens: int, chunk: int, max_step_tokens: int, share: bool):
+def serve_c(config, prompts, new_tokens: int, chunk: int, max_step_tokens: int, share: bool, sampling: dict = None):
     """The same through the C host (`kipp_amd/host`: its scheduler over kipp_step, no Python inside a step): the shape is
     written to a folder with random weights first.  Returns (the scheduler's counters, seconds)."""
     import shutil
@@ -116,7 +118,7 @@ def serve_c(config, prompts, new_tokens: int, chunk: int, max_step_tokens: int, 
             warm.destroy()
             sched = CScheduler(model, max_step_tokens=max_step_tokens, prefill_chunk=chunk, max_running=len(prompts))
             for i, p in enumerate(prompts):
-                sched.add(i, p, new_tokens)
+                sched.add(i, p, new_tokens, seed=100 + i, **(sampling or {}))
             start = time.perf_counter()
             sched.run()
             seconds = time.perf_counter() - start
@@ -379,6 +381,10 @@ def main(argv=None) -> int:
     ap.add_argument("--seed", type=int, default=1)
     ap.add_argument("--no-sharing", action="store_true", help="shared-prefix: compute every prompt in full, for comparison")
     ap.add_argument("--host", choices=["python", "c"], default="python", help="which host serves: the Python engine or the C library")
+    ap.add_argument("--temperature", type=float, default=0.0, help="above 0: every request samples (seeded), with the options below")
+    ap.add_argument("--top-p", type=float, default=1.0)
+    ap.add_argument("--top-k", type=int, default=0)
+    ap.add_argument("--repetition-penalty", type=float, default=1.0)
     args = ap.parse_args(argv)
 
     import torch
@@ -395,6 +401,9 @@ def main(argv=None) -> int:
         print(f"workload: prompt {longest} + {new} new tokens exceed the context {context}", file=sys.stderr)
         return 1
     per_request = -(-(longest + new) // 64) * 64
+    sampling = None
+    if args.temperature > 0.0 or args.repetition_penalty != 1.0:
+        sampling = dict(temperature=args.temperature, top_p=args.top_p, top_k=args.top_k, repetition_penalty=args.repetition_penalty)
     if args.host == "c":
         from .config import shape_config
         config = shape_config(shape)
@@ -405,7 +414,7 @@ def main(argv=None) -> int:
         vocab = config["vocab_size"]
         prompts = (continuous_prompts(n, args.min_prompt, args.max_prompt, vocab, args.seed) if cont
                    else shared_prefix_prompts(n, args.prefix, args.suffix, vocab, args.seed))
-        st, seconds = serve_c(config, prompts, new, args.prefill_chunk, args.max_step_tokens, not args.no_sharing)
+        st, seconds = serve_c(config, prompts, new, args.prefill_chunk, args.max_step_tokens, not args.no_sharing, sampling)
         prompt_tokens = sum(len(p) for p in prompts)
         print(json.dumps({
             "workload": args.workload, "host": "c", "value": st["generated_tokens"] / seconds, "unit": "generated tokens/s",
@@ -416,7 +425,7 @@ def main(argv=None) -> int:
             "data": "synthetic uniform-random tokens, random weights",
             "config": {"model": shape, "layers": config["num_hidden_layers"], "layers_full": full_layers, "context": context,
                        "prefill_chunk": args.prefill_chunk, "max_step_tokens": args.max_step_tokens, "new_tokens": new,
-                       "kv_page": 16, "sharing": not args.no_sharing}}), flush=True)
+                       "kv_page": 16, "sharing": not args.no_sharing, "sampling": json.dumps(sampling) if sampling else "greedy"}}), flush=True)
         return 0
     engine, config, full_layers = build_engine(shape, args.layers, context, n * per_request, n, args.seed)
     if args.no_sharing:
@@ -429,7 +438,7 @@ def main(argv=None) -> int:
 
     warm = [p[:args.prefill_chunk + 3] for p in prompts[:2]]            # other tokens: nothing of it is adopted later
     serve(engine, [[(t + 1) % vocab for t in p] for p in warm], 4, args.prefill_chunk, args.max_step_tokens)
-    sched, seconds, first = serve(engine, prompts, new, args.prefill_chunk, args.max_step_tokens)
+    sched, seconds, first = serve(engine, prompts, new, args.prefill_chunk, args.max_step_tokens, sampling)
     st = sched.stats
     prompt_tokens = sum(len(p) for p in prompts)
     out = {
@@ -445,7 +454,8 @@ def main(argv=None) -> int:
                    "heads": config["num_attention_heads"], "kv_heads": config["num_key_value_heads"],
                    "head_dim": config["head_dim"], "vocab": vocab, "context": context,
                    "prefill_chunk": args.prefill_chunk, "max_step_tokens": args.max_step_tokens,
-                   "new_tokens": new, "kv_page": 16, "sharing": not args.no_sharing},
+                   "new_tokens": new, "kv_page": 16, "sharing": not args.no_sharing,
+                   "sampling": json.dumps(sampling) if sampling else "greedy"},
     }
     print(json.dumps(out), flush=True)
     return 0
