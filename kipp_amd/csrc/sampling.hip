@@ -264,6 +264,7 @@ extern "C" int kipp_adjust_logits(float* logits, int rows, int vocab, const int3
 // atomics: the sums are exact and do not depend on the order of the additions.
 
 #define SAMPLE_THREADS 1024
+#define SAMPLE_LIST SAMPLE_THREADS       // candidates that are finished in LDS, a lane each
 #define MASS_SCALE 17592186044416.0f   // 2^44
 
 __device__ __forceinline__ uint32_t float_order(float x) {
@@ -539,6 +540,8 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) sample_kernel(
     int32_t* __restrict__ out) {
     __shared__ Bins bins, top;
     __shared__ unsigned long long shared[5];
+    __shared__ unsigned long long list_key[SAMPLE_LIST], list_mass[SAMPLE_LIST];
+    __shared__ unsigned int list_n;
     __shared__ float best_v[16];
     __shared__ int best_i[16];
     const int rowi = blockIdx.x;
@@ -594,8 +597,65 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) sample_kernel(
     // ---- min-p relative to the top weight, which is exp(0) = 1
     const float mp = min_p[rowi];
     if (mp > 0.0f) r.min_weight = (double)mp;
-    // ---- top-p: the shortest prefix whose mass reaches top_p of the total (the total: what the top level's histogram adds up to)
     const double share = (double)top_p[rowi];
+    if (k > 0 && k <= SAMPLE_LIST) {
+        // ---- few candidates are left (at most k): one pass gathers them, key and mass, into LDS, a lane a candidate; each
+        //      adds up the masses of those ahead of it in key order, and the two questions (where does the mass reach
+        //      top_p of the total; where does it exceed the draw's share of what is kept) are answered by the one candidate
+        //      at which the running mass crosses the target: the answers of the two walks below, without their passes
+        if (threadIdx.x == 0) list_n = 0;
+        __syncthreads();
+        for_each_logit(row, vocab, [&](int i, float logit) {
+            unsigned long long key;
+            float w;
+            if (!r.member(i, logit, &key, &w)) return;
+            const unsigned int at = atomicAdd(&list_n, 1u);
+            if (at < SAMPLE_LIST) {
+                list_key[at] = key;
+                list_mass[at] = (unsigned long long)(w * MASS_SCALE);
+            }
+        });
+        __syncthreads();
+        const int n = (int)(list_n < SAMPLE_LIST ? list_n : SAMPLE_LIST);
+        const bool have = (int)threadIdx.x < n;
+        const unsigned long long my_key = have ? list_key[threadIdx.x] : 0, my_mass = have ? list_mass[threadIdx.x] : 0;
+        unsigned long long ahead_of_me = 0, total = 0;
+        int rank = 0;
+        for (int j = 0; j < n; ++j) {
+            const unsigned long long other = list_key[j], mass = list_mass[j];
+            total += mass;
+            if (other > my_key) {
+                ahead_of_me += mass;
+                ++rank;
+            }
+        }
+        if (threadIdx.x == 0) shared[0] = 0;
+        __syncthreads();
+        const double reach = share * (double)total;
+        if (have && (double)(ahead_of_me + my_mass) >= reach && (rank == 0 || !((double)ahead_of_me >= reach))) {
+            shared[0] = my_key;                                                     // the last candidate that top-p keeps
+            shared[1] = (unsigned long long)__double_as_longlong((double)ahead_of_me + (double)my_mass);
+        }
+        __syncthreads();
+        if (shared[0] == 0 && have && rank == n - 1) {                              // (beyond everything: the last candidate)
+            shared[0] = my_key;
+            shared[1] = (unsigned long long)__double_as_longlong((double)ahead_of_me + (double)my_mass);
+        }
+        __syncthreads();
+        const unsigned long long last_kept = shared[0];
+        const double kept_mass = __longlong_as_double((long long)shared[1]), draw = uniform[rowi] * kept_mass;
+        __syncthreads();
+        if (threadIdx.x == 0) shared[2] = 0;
+        __syncthreads();
+        const bool kept_one = have && my_key >= last_kept;
+        if (kept_one && (double)(ahead_of_me + my_mass) > draw && (rank == 0 || !((double)ahead_of_me > draw))) shared[2] = my_key;
+        __syncthreads();
+        if (shared[2] == 0 && kept_one && my_key == last_kept) shared[2] = my_key;  // (beyond everything: the last one kept)
+        __syncthreads();
+        if (threadIdx.x == 0) out[rowi] = (int32_t)(0xffffffffu - (uint32_t)(shared[2] & 0xffffffffu));
+        return;
+    }
+    // ---- top-p: the shortest prefix whose mass reaches top_p of the total (the total: what the top level's histogram adds up to)
     const unsigned long long last = descend<true, false>(r, 0.0, &share, &bins, &top, true, shared, &before, &own);
     if (last > r.key_floor) r.key_floor = last;
     const double kept = before + own;
