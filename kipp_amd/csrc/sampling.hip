@@ -598,8 +598,27 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) sample_kernel(
     const float mp = min_p[rowi];
     if (mp > 0.0f) r.min_weight = (double)mp;
     const double share = (double)top_p[rowi];
-    if (k > 0 && k <= SAMPLE_LIST) {
-        // ---- few candidates are left (at most k): one pass gathers them, key and mass, into LDS, a lane a candidate; each
+    bool few = k > 0 && k <= SAMPLE_LIST;
+    if (!few) {
+        // how many candidates there are (logits within 20 of the largest, after the temperature: a few hundred of a trained
+        // model's 150,000): a pass that takes no exponential
+        if (threadIdx.x == 0) list_n = 0;
+        __syncthreads();
+        unsigned int mine = 0;
+        for_each_logit(row, vocab, [&](int i, float logit) {
+            unsigned long long key;
+            float scaled;
+            if (logit * r.inv_t >= r.cutoff && r.candidate(i, logit, &key, &scaled)) ++mine;
+        });
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) mine += __shfl_xor(mine, off, KIPP_WAVE);
+        if ((threadIdx.x & (KIPP_WAVE - 1)) == 0 && mine != 0) atomicAdd(&list_n, mine);
+        __syncthreads();
+        few = list_n <= SAMPLE_LIST;
+        __syncthreads();
+    }
+    if (few) {
+        // ---- few candidates are left: one pass gathers them, key and mass, into LDS, a lane a candidate; each
         //      adds up the masses of those ahead of it in key order, and the two questions (where does the mass reach
         //      top_p of the total; where does it exceed the draw's share of what is kept) are answered by the one candidate
         //      at which the running mass crosses the target: the answers of the two walks below, without their passes
