@@ -1284,6 +1284,31 @@ def test_row_nll_against_float64(vocab):
     assert abs(got[2] - np.log(vocab)) < 1e-12 and got[1] < 1e-6
 
 
+@pytest.mark.parametrize("vocab", [509, 151936])
+def test_device_sampler_at_the_ends_of_the_draw(vocab):
+    """A draw of 0 takes the first candidate (the largest logit, the lowest id among equals); a draw just under 1 the last
+    one that is kept: the smallest logit within 20 of the largest after the temperature (the highest id among equals), or the
+    k-th largest under top-k.  Rows of many candidates (walked level by level) and of few (finished in LDS)."""
+    ops = _ops()
+    rng = np.random.default_rng(vocab + 9)
+    rows = 8
+    logits = (rng.normal(size=(rows, vocab)) * np.array([0.05, 0.05, 3.0, 3.0, 9.0, 9.0, 0.05, 9.0])[:, None]).astype(np.float32)
+    logits[1, 5] = logits[1, 77] = logits[1].max() + 1.0          # equal maxima
+    logits[3, 100:110] = logits[3].min()                           # equal minima
+    temperature = np.array([0.8, 1.0, 0.8, 1.3, 0.5, 0.9, 0.8, 0.9], dtype=np.float32)
+    top_k = np.array([0, 0, 0, 0, 0, 0, 7, 7], dtype=np.int32)
+    for draw in (0.0, 1.0 - 2.0 ** -53):
+        got = ops.sample(_t(logits), _t(temperature), _t(top_k, torch.int32), _t([1.0] * rows), _t([0.0] * rows),
+                         _t([draw] * rows, torch.float64), torch.empty(rows, dtype=torch.int32, device=DEV)).cpu().tolist()
+        for r in range(rows):
+            scaled = logits[r] * (np.float32(1.0) / temperature[r])
+            order = sorted(range(vocab), key=lambda i: (-float(scaled[i]), i))
+            kept = [i for i in order if scaled[i] >= scaled.max() - np.float32(20.0)]
+            if top_k[r]:
+                kept = kept[:top_k[r]]
+            assert got[r] == (kept[0] if draw == 0.0 else kept[-1]), (r, draw, got[r], kept[0], kept[-1], len(kept))
+
+
 def test_device_sampler_follows_the_distribution():
     ops = _ops()
     from kipp_amd.sampling import XorShift64Star
