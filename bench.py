@@ -96,17 +96,27 @@ def fill(engine, ids, prompt_len, vocab, seed, chunk=2048):
     return first
 
 
-def decode_run(engine, ids, tokens, steps, warmup):
+SAMPLED = dict(temperature=0.8, top_k=50, top_p=0.9)         # the sampled points: every request draws with these, seeded
+
+
+def decode_run(engine, ids, tokens, steps, warmup, sampled=False):
     """`warmup` untimed and `steps` timed decode steps of all `ids` together, as the
-    scheduler runs them: tokens are chosen greedily on the device and feed the next
-    step from there; the host reads them one step behind, while that step runs."""
+    scheduler runs them: tokens are chosen on the device (greedily, or with `sampled`
+    by the device sampler from each request's own generator) and feed the next step
+    from there; the host reads them one step behind, while that step runs."""
     import torch
     from kipp_amd.engine import StepEntry
-    from kipp_amd.sampling import SampleParams
+    from kipp_amd.sampling import SampleParams, XorShift64Star
 
     class Greedy:
         params, rng, recent = SampleParams(), None, ()
-    rows = [Greedy()] * len(ids)
+
+    class Sampled:
+        recent = ()
+
+        def __init__(self, seed):
+            self.params, self.rng = SampleParams(**SAMPLED), XorShift64Star(seed)
+    rows = [Sampled(100 + i) for i in range(len(ids))] if sampled else [Greedy()] * len(ids)
     logits = engine.step([StepEntry(r, [tokens[r]], [0]) for r in ids])
     picks = engine.choose(logits, rows, wait=False)
     entries = [StepEntry(r, [0], [0]) for r in ids]
@@ -132,7 +142,7 @@ class WrongKernelClass(RuntimeError):
     """The timed steps did not run on the kernels the measurement is about."""
 
 
-def measure_decode(engine, rt, ids, first, steps, warmup, repeats, weight_bytes, kv_per_token):
+def measure_decode(engine, rt, ids, first, steps, warmup, repeats, weight_bytes, kv_per_token, sampled=False):
     """`repeats` timings of `steps` decode steps, each from the same contexts (what a repeat, and the warm-up before the
     first, decoded is cut off again: with 256 steps behind prompts of 2,048 tokens every repeat is the run 2,048 -> 2,304
     tokens); the median one is reported.
@@ -144,13 +154,13 @@ def measure_decode(engine, rt, ids, first, steps, warmup, repeats, weight_bytes,
         for r, n in zip(ids, lengths):                   # every repeat, and every batch size, decodes behind the prompts alone
             engine.cache.truncate(engine.cache.requests[r], n)
     if warmup > 0:
-        decode_run(engine, ids, first, warmup, 0)
+        decode_run(engine, ids, first, warmup, 0, sampled)
         cut_back()
     again = 0
     rep = 0
     while rep < repeats:
         library, generic, replays = rt.library_products, rt.generic_attention_launches, engine.graphs.replays
-        seconds = decode_run(engine, ids, first, steps, 0)
+        seconds = decode_run(engine, ids, first, steps, 0, sampled)
         cut_back()
         if rt.library_products != library or rt.generic_attention_launches != generic:
             raise WrongKernelClass(f"decode batch {len(ids)}: {rt.library_products - library} products went to the library and "
@@ -249,6 +259,7 @@ def main():
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--repeats", type=int, default=5, help="times the K timed steps are run; the median is reported")
     ap.add_argument("--no-long", action="store_true", help="leave out the points at longer contexts")
+    ap.add_argument("--no-sampled", action="store_true", help="leave out the points with sampling requests")
     ap.add_argument("--no-c-host", action="store_true", help="leave out the points measured through the C host")
     ap.add_argument("--products", choices=["default", "own", "auto", "library"], default="default",
                     help="products of many rows (prompt portions): the runtime's default, our kernel only, the fastest of ours and the library's, the library's")
@@ -333,6 +344,17 @@ def main():
         log(f"decode batch {b}: {r['ms']:.3f} ms/step (median of {repeats}, MAD {r['mad_ms']:.3f}), {r['tok_s']:.0f} tok/s, "
             f"{r['bytes'] / (r['ms'] / 1e3) / 1e9:.0f} GB/s")
         # the requests beyond this batch keep their caches; the first ones simply go on
+    # ---- the same steps with every request sampling (temperature, top-k, top-p): the step plus the device sampler
+    sampled_points = {}
+    for b in (b for b in batches if b in (args.batch, 64) and not args.no_sampled):
+        try:
+            r = measure_decode(engine, rt, ids[:b], first, args.steps, args.warmup, min(repeats, 3), weight_bytes, kv_per_token, sampled=True)
+        except Exception as exc:          # noqa: BLE001
+            log(f"sampled decode at batch {b} failed and is left out: {type(exc).__name__}: {exc}")
+            continue
+        sampled_points[f"decode_b{b}_sampled"] = round(r["tok_s"], 1)
+        log(f"decode batch {b}, sampled (T {SAMPLED['temperature']}, top-k {SAMPLED['top_k']}, top-p {SAMPLED['top_p']}): "
+            f"{r['ms']:.3f} ms/step, {r['tok_s']:.0f} tok/s")
 
     # ---- longer contexts, on a cache of their own behind the same weights
     long_points, long_fracs = {}, {}
@@ -374,6 +396,7 @@ def main():
         "protocol": {"repeats": main_r["repeats"], "reported": "median", "mad_ms_per_step": round(main_r["mad_ms"], 4),
                      "timed_steps_are_graph_replays_of_own_kernels": True},
     }
+    line["points"].update(sampled_points)
     line["points"].update(long_points)
     line["points"].update(c_points)
     line["points_roofline_frac"] = {f"decode_b{b}": round(results[b]["bytes"] / (results[b]["ms"] / 1e3) / 1e9 / HBM_PEAK_GBS, 4)
