@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define KIPP_AMD_VERSION "0.3.0"
+#define KIPP_AMD_VERSION "0.4.0"
 #define KIPP_MAX_STOP_TOKENS 8u
 #define KIPP_EVAL_BATCH_LIMIT 256u
 
