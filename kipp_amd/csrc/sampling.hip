@@ -262,6 +262,11 @@ extern "C" int kipp_adjust_logits(float* logits, int rows, int vocab, const int3
 // walking down the key one byte at a time with a 256-bin histogram of counts or of
 // masses.  Masses are weights exp(l - max) in 44-bit fixed point, added with integer
 // atomics: the sums are exact and do not depend on the order of the additions.
+// A walk ends where the chosen byte has one candidate alone; the total mass is what the
+// top level's histogram adds up to; and where few candidates are left (at most
+// SAMPLE_LIST: after top-k, or counted) they are gathered into LDS once and the two
+// mass questions are answered there, by the candidate at which the running mass
+// crosses the target.
 
 #define SAMPLE_THREADS 1024
 #define SAMPLE_LIST SAMPLE_THREADS       // candidates that are finished in LDS, a lane each
