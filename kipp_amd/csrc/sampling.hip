@@ -319,15 +319,16 @@ __device__ __forceinline__ void for_each_logit(const float* __restrict__ row, in
     if ((vocab & 3) == 0 && ((size_t)row & 15) == 0) {
         const float4* __restrict__ row4 = (const float4*)row;
         const int quads = vocab >> 2;
-        for (int base = threadIdx.x; base < quads; base += SAMPLE_AHEAD * blockDim.x) {
-            float4 v[SAMPLE_AHEAD];
+        constexpr int QUADS_AHEAD = SAMPLE_AHEAD / 2;               // as many bytes on their way as fit the registers of 1,024 lanes
+        for (int base = threadIdx.x; base < quads; base += QUADS_AHEAD * blockDim.x) {
+            float4 v[QUADS_AHEAD];
 #pragma unroll
-            for (int j = 0; j < SAMPLE_AHEAD; ++j) {
+            for (int j = 0; j < QUADS_AHEAD; ++j) {
                 const int q = base + j * blockDim.x;
                 v[j] = q < quads ? row4[q] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
             }
 #pragma unroll
-            for (int j = 0; j < SAMPLE_AHEAD; ++j) {
+            for (int j = 0; j < QUADS_AHEAD; ++j) {
                 const int q = base + j * blockDim.x;
                 if (q < quads) {
                     f(4 * q, v[j].x);
@@ -677,6 +678,13 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) sample_kernel(
         if (shared[2] == 0 && kept_one && my_key == last_kept) shared[2] = my_key;  // (beyond everything: the last one kept)
         __syncthreads();
         if (threadIdx.x == 0) out[rowi] = (int32_t)(0xffffffffu - (uint32_t)(shared[2] & 0xffffffffu));
+        return;
+    }
+    if (!(share < 1.0)) {
+        // ---- top-p keeps everything: the draw's share of the total mass, in one walk
+        const double part = uniform[rowi];
+        const unsigned long long pick = descend<true, true>(r, 0.0, &part, &bins, nullptr, false, shared, &before, &own);
+        if (threadIdx.x == 0) out[rowi] = (int32_t)(0xffffffffu - (uint32_t)(pick & 0xffffffffu));
         return;
     }
     // ---- top-p: the shortest prefix whose mass reaches top_p of the total (the total: what the top level's histogram adds up to)
