@@ -114,6 +114,7 @@ typedef struct {
     fn_sample sample;
     fn_adjust_logits adjust_logits;
     fn_row_nll row_nll;
+    void *pinned;               /* SMALL_DOWNLOAD bytes of pinned host memory */
     unsigned char *sample_host; /* what the sampler of a step is told, packed by field */
     unsigned char *sample_device; /* the same on the GPU, behind the tokens chosen */
     size_t sample_bytes;        /* room of both */
@@ -283,6 +284,7 @@ static void hip_destroy(kipp_runtime *rt) {
         hipStreamSynchronize(st->stream);
         if (st->arrivals != NULL) hipFree(st->arrivals);
         if (st->sample_device != NULL) hipFree(st->sample_device);
+        if (st->pinned != NULL) hipHostFree(st->pinned);
         free(st->sample_host);
         if (st->stream != NULL) hipStreamDestroy(st->stream);
         /* the libraries stay loaded: their kernels may be registered with the HIP runtime until the process ends */
@@ -328,11 +330,19 @@ static int hip_upload(kipp_runtime *rt, void *to, const void *from_host, size_t 
     return code == hipSuccess ? 0 : hip_bad(error, code, "copy to the GPU");
 }
 
+#define SMALL_DOWNLOAD 4096 /* bytes that come back through pinned memory of the runtime's own (a step's chosen tokens) */
+
 static int hip_download(kipp_runtime *rt, void *to_host, const void *from, size_t bytes, kipp_error *error) {
     hip_state *st = rt->state;
     hipError_t code = hipSuccess;
-    if (bytes != 0) code = hipMemcpyAsync(to_host, from, bytes, hipMemcpyDeviceToHost, st->stream);
+    /* a copy into pageable memory is staged by the runtime and waited for inside the call; the few bytes of a decode step
+     * come through a pinned buffer instead: the copy is queued behind the step and one wait covers both */
+    if (bytes != 0 && bytes <= SMALL_DOWNLOAD && st->pinned == NULL && hipHostMalloc(&st->pinned, SMALL_DOWNLOAD, hipHostMallocDefault) != hipSuccess)
+        st->pinned = NULL; /* without it: straight to the caller's memory, as for the large copies */
+    void *target = bytes != 0 && bytes <= SMALL_DOWNLOAD && st->pinned != NULL ? st->pinned : to_host;
+    if (bytes != 0) code = hipMemcpyAsync(target, from, bytes, hipMemcpyDeviceToHost, st->stream);
     if (code == hipSuccess) code = hipStreamSynchronize(st->stream);
+    if (code == hipSuccess && target != to_host) memcpy(to_host, target, bytes);
     return code == hipSuccess ? 0 : hip_bad(error, code, "copy from the GPU (or a kernel before it)");
 }
 
