@@ -273,7 +273,8 @@ extern "C" int kipp_adjust_logits(float* logits, int rows, int vocab, const int3
 #define MASS_SCALE 17592186044416.0f   // 2^44
 
 __device__ __forceinline__ uint32_t float_order(float x) {
-    const uint32_t b = __float_as_uint(x);
+    uint32_t b = __float_as_uint(x);
+    if (b == 0x80000000u) b = 0u;                        // -0 is 0: equal logits are ordered by their ids alone, as on the host
     return (b & 0x80000000u) ? ~b : (b | 0x80000000u);   // larger float, larger integer
 }
 

@@ -1284,6 +1284,27 @@ def test_row_nll_against_float64(vocab):
     assert abs(got[2] - np.log(vocab)) < 1e-12 and got[1] < 1e-6
 
 
+def test_device_sampler_orders_equal_logits_by_their_ids():
+    """Rows of many equal logits, zeros of both signs among them (-0.0 equals 0.0: such candidates are ordered by their ids
+    alone, as the host sampler's comparison orders them), quantized values, and every sampling option: the host's token."""
+    from kipp_amd.sampling import SampleParams, XorShift64Star, sample
+    ops = _ops()
+    rng = np.random.default_rng(77)
+    vocab, rows = 4096, 192
+    logits = (np.round(rng.normal(size=(rows, vocab)) * rng.choice([0.05, 0.5, 2.0], size=(rows, 1)) * 4) / 4).astype(np.float32)
+    assert (np.signbit(logits) & (logits == 0)).any() and ((~np.signbit(logits)) & (logits == 0)).any()
+    t = rng.choice([0.2, 0.7, 1.0, 1.6], size=rows).astype(np.float32)
+    k = rng.choice([0, 0, 1, 3, 50, 900, 2000], size=rows).astype(np.int32)
+    p = rng.choice([1.0, 1.0, 0.95, 0.5, 0.1], size=rows).astype(np.float32)
+    m = rng.choice([0.0, 0.0, 0.02, 0.3], size=rows).astype(np.float32)
+    seeds = rng.integers(1, 2 ** 62, size=rows)
+    got = ops.sample(_t(logits), _t(t), _t(k, torch.int32), _t(p), _t(m), _t([XorShift64Star(int(s)).uniform() for s in seeds], torch.float64),
+                     torch.empty(rows, dtype=torch.int32, device=DEV)).cpu().tolist()
+    for i in range(rows):
+        want = sample(logits[i], SampleParams(temperature=float(t[i]), top_k=int(k[i]), top_p=float(p[i]), min_p=float(m[i])), XorShift64Star(int(seeds[i])))
+        assert got[i] == want, f"row {i}: T={t[i]} top_k={k[i]} top_p={p[i]} min_p={m[i]}: {got[i]} != {want}"
+
+
 @pytest.mark.parametrize("vocab", [509, 151936])
 def test_device_sampler_at_the_ends_of_the_draw(vocab):
     """A draw of 0 takes the first candidate (the largest logit, the lowest id among equals); a draw just under 1 the last
