@@ -265,6 +265,40 @@ def test_c_scheduler_samples_on_the_device_as_on_the_host(model_folders, tiny_co
         assert row[token] >= row.max() - margin
 
 
+@pytest.mark.parametrize("key", ["a", "b"])
+def test_both_schedulers_choose_the_same_sampled_tokens(model_folders, tiny_configs, key):
+    """On the float32 path the two hosts' logits are the same bits, their generators are the same and both choose on the
+    device: requests with every sampling option (temperature, top-k, top-p, min-p, the three penalties, a bias, greedy ones
+    among them) get the same tokens from the Python scheduler and from the C one."""
+    from kipp_amd.chost import CModel, CScheduler
+    from kipp_amd.engine import Engine
+    from kipp_amd.engine.scheduler import Request, Scheduler
+    from kipp_amd.sampling import SampleParams
+    cfg = tiny_configs[key]
+    vocab, folder = cfg["vocab_size"], model_folders[(key, "float32")]
+    rng = np.random.default_rng(5)
+    prompts = [H.random_tokens(300 + i, int(rng.integers(2, 30)), vocab) for i in range(7)]
+    how = [dict(), dict(temperature=0.9), dict(temperature=1.3, top_k=12, top_p=0.9), dict(temperature=0.7, min_p=0.05, repetition_penalty=1.4),
+           dict(presence_penalty=0.6, frequency_penalty=0.3), dict(temperature=1.0, top_p=0.8, logit_bias={3: 2.0, 17: -5.0}, frequency_penalty=0.2),
+           dict(temperature=0.5, top_k=3, presence_penalty=-0.3)]
+    new = 20
+    engine = Engine.from_folder(folder, dtype="float32", page_size=PAGE[key], max_tokens=7 * 64, share_prefixes=False)
+    sched = Scheduler(engine, max_step_tokens=24, prefill_chunk=8)
+    for i, prompt in enumerate(prompts):
+        sched.add(Request(i, prompt, new, params=SampleParams(**how[i]), seed=40 + i))
+    while not sched.idle:
+        sched.step()
+    by_python = {rid: list(r.output) for rid, r in sched.finished.items()}
+    with CModel(folder, path="gpu-fp32", page_tokens=PAGE[key], kv_pool_pages=7 * 64 // PAGE[key] + 8, max_sessions=7, share_prefixes=False) as model:
+        csched = CScheduler(model, max_step_tokens=24, prefill_chunk=8)
+        for i, prompt in enumerate(prompts):
+            csched.add(i, prompt, new, seed=40 + i, **how[i])
+        csched.run()
+        by_c = {i: csched.result(i)["output"] for i in range(7)}
+        csched.destroy()
+    assert by_python == by_c and all(len(o) == new for o in by_c.values())
+
+
 def test_c_command_line_on_the_gpu(model_folders, tiny_configs):
     """The C program on gpu-bf16 and gpu-fp32, given the folder of the built kernels: greedy tokens that the plain
     implementation agrees with, and the KIPP_METRIC line naming the path."""
